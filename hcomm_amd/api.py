@@ -1,0 +1,247 @@
+"""ctypes binding of include/hcomm_gfx.h.
+
+Every function here is a one-line call into libhcomm_gfx.so; there is no Python or CPU implementation of
+any operation.  If the library is missing, importing this module raises - it never falls back.
+"""
+import ctypes as C
+import os
+
+__all__ = [
+    "lib", "LIB_PATH", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
+    "LaunchRecord", "PlanInfo", "SchedOp", "Slice", "HcommError", "check",
+    "HcommLocalCopyOnThread", "HcommLocalReduceOnThread", "HcommThreadAlloc", "HcommThreadFree",
+    "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
+    "HcommThreadNotifyWaitOnThread", "HcommMemAlloc", "HcommMemFree", "HcommBatchModeStart", "HcommBatchModeEnd",
+    "HcommGfxThreadSynchronize", "HcommGfxReduceKOnThread", "HcommGfxRecorderThreadAlloc", "launch_log",
+    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion",
+    "DTYPE_SIZE",
+]
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libhcomm_gfx.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'` or "
+        "`make -C hcomm_amd/csrc`" % LIB_PATH)
+lib = C.CDLL(LIB_PATH)
+
+
+class HcclResult:
+    SUCCESS, E_PARA, E_PTR, E_MEMORY, E_INTERNAL, E_NOT_SUPPORT, E_NOT_FOUND, E_UNAVAIL = range(8)
+    E_TIMEOUT = 9
+    E_RUNTIME = 15
+
+
+class HcommReduceOp:
+    SUM, PROD, MAX, MIN = 0, 1, 2, 3
+    RESERVED = 255
+
+
+class HcommDataType:
+    INT8, INT16, INT32, FP16, FP32, INT64, UINT64, UINT8, UINT16, UINT32, FP64, BFP16, INT128 = range(13)
+    HIF8, FP8E4M3, FP8E5M2, FP8E8M0 = 14, 15, 16, 17
+    RESERVED = 255
+
+
+DTYPE_SIZE = {HcommDataType.INT8: 1, HcommDataType.INT16: 2, HcommDataType.INT32: 4, HcommDataType.FP16: 2,
+              HcommDataType.FP32: 4, HcommDataType.BFP16: 2}
+
+
+class CommEngine:
+    RESERVED, CPU, CPU_TS, AICPU, AICPU_TS, AIV, CCU = -1, 0, 1, 2, 3, 4, 5
+
+
+class Alg:
+    ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
+        REDUCE_SCATTER_RING_STANDALONE = range(6)
+
+
+class Lowering:
+    STEPWISE, FUSED = 0, 1
+
+
+class Kernel:
+    COPY, REDUCE2, CHAIN, TREE, BYTEWISE = range(5)
+
+
+class LaunchRecord(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("dtype", C.c_uint32), ("op", C.c_uint32), ("nseg", C.c_uint32),
+                ("bytes", C.c_uint64), ("blocks", C.c_uint64)]
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [("launches", C.c_uint32), ("steps", C.c_uint32), ("algorithmicBytes", C.c_uint64),
+                ("movedBytes", C.c_uint64)]
+
+
+class SchedOp(C.Structure):
+    _fields_ = [("step", C.c_uint32), ("kind", C.c_uint32), ("rank", C.c_uint32), ("dstBuf", C.c_uint32),
+                ("srcRank", C.c_uint32), ("srcBuf", C.c_uint32), ("dstOff", C.c_uint64), ("srcOff", C.c_uint64),
+                ("bytes", C.c_uint64)]
+
+    def astuple(self):
+        return (self.step, self.kind, self.rank, self.dstBuf, self.dstOff, self.srcRank, self.srcBuf, self.srcOff,
+                self.bytes)
+
+
+class Slice(C.Structure):
+    _fields_ = [("offset", C.c_uint64), ("size", C.c_uint64)]
+
+
+class HcommError(RuntimeError):
+    def __init__(self, code, what):
+        super().__init__("%s failed with HcclResult %d" % (what, code))
+        self.code = code
+
+
+def check(code, what="call"):
+    if code != 0:
+        raise HcommError(code, what)
+    return code
+
+
+def _sig(name, restype, *argtypes):
+    f = getattr(lib, name)
+    f.restype = restype
+    f.argtypes = list(argtypes)
+    return f
+
+
+_u64, _u32, _i32, _vp = C.c_uint64, C.c_uint32, C.c_int32, C.c_void_p
+
+HcommLocalCopyOnThread = _sig("HcommLocalCopyOnThread", _i32, _u64, _vp, _vp, _u64)
+HcommLocalReduceOnThread = _sig("HcommLocalReduceOnThread", _i32, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
+_thread_alloc = _sig("HcommThreadAlloc", _i32, C.c_int, _u32, C.POINTER(_u32), C.POINTER(_u64))
+_thread_free = _sig("HcommThreadFree", _i32, C.POINTER(_u64), _u32)
+_thread_alloc_stream = _sig("HcommThreadAllocWithStream", _i32, C.c_int, _vp, _u32, C.POINTER(_u64))
+_thread_free_stream = _sig("HcommThreadFreeWithStream", _i32, C.POINTER(_u64), _u32)
+HcommThreadNotifyRecordOnThread = _sig("HcommThreadNotifyRecordOnThread", _i32, _u64, _u64, _u32)
+HcommThreadNotifyWaitOnThread = _sig("HcommThreadNotifyWaitOnThread", _i32, _u64, _u32, _u32)
+_mem_alloc = _sig("HcommMemAlloc", _i32, C.POINTER(_vp), C.c_size_t)
+HcommMemFree = _sig("HcommMemFree", _i32, _vp)
+HcommBatchModeStart = _sig("HcommBatchModeStart", _i32, C.c_char_p)
+HcommBatchModeEnd = _sig("HcommBatchModeEnd", _i32, C.c_char_p)
+HcommGfxThreadSynchronize = _sig("HcommGfxThreadSynchronize", _i32, _u64)
+_reduce_k = _sig("HcommGfxReduceKOnThread", _i32, _u64, _vp, C.POINTER(_vp), _u32, _u64, C.c_int, C.c_int)
+_recorder_alloc = _sig("HcommGfxRecorderThreadAlloc", _i32, C.POINTER(_u64))
+_log_read = _sig("HcommGfxLaunchLogRead", _i32, _u64, C.POINTER(LaunchRecord), _u32, C.POINTER(_u32))
+HcommGfxLaunchLogClear = _sig("HcommGfxLaunchLogClear", _i32, _u64)
+_calc_slices = _sig("HcommGfxCalcSlices", _i32, _u64, _u32, _u32, C.POINTER(Slice))
+HcommGfxDataTypeSize = _sig("HcommGfxDataTypeSize", _u32, C.c_int)
+_plan_create = _sig("HcommGfxPlanCreate", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
+                    C.c_int, C.POINTER(_vp))
+_plan_run = _sig("HcommGfxPlanRun", _i32, _vp, _u64)
+_plan_run_range = _sig("HcommGfxPlanRunRange", _i32, _vp, _u64, _u32, _u32)
+_plan_destroy = _sig("HcommGfxPlanDestroy", _i32, _vp)
+_plan_info = _sig("HcommGfxPlanGetInfo", _i32, _vp, C.POINTER(PlanInfo))
+_plan_launch = _sig("HcommGfxPlanGetLaunch", _i32, _vp, _u32, C.POINTER(LaunchRecord))
+_sched_emit = _sig("HcommGfxScheduleEmit", _i32, C.c_int, _u32, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+                   C.POINTER(_u64))
+_version = _sig("HcommGfxVersion", C.c_char_p)
+
+
+def HcommGfxVersion():
+    return _version().decode()
+
+
+def HcommThreadAlloc(engine=CommEngine.CPU_TS, thread_num=1, notify_num=0):
+    """Returns (code, [handles])."""
+    handles = (_u64 * max(thread_num, 1))()
+    notif = (_u32 * 1)(notify_num)
+    code = _thread_alloc(engine, thread_num, notif, handles)
+    return code, list(handles)[:thread_num]
+
+
+def HcommThreadFree(handles):
+    arr = (_u64 * max(len(handles), 1))(*handles)
+    return _thread_free(arr, len(handles))
+
+
+def HcommThreadAllocWithStream(stream_ptr, notify_num=0, engine=CommEngine.CPU_TS):
+    """stream_ptr: integer value of a hipStream_t (0 = default stream).  Returns (code, handle)."""
+    h = _u64(0)
+    code = _thread_alloc_stream(engine, _vp(stream_ptr), notify_num, C.byref(h))
+    return code, h.value
+
+
+def HcommThreadFreeWithStream(handles):
+    arr = (_u64 * max(len(handles), 1))(*handles)
+    return _thread_free_stream(arr, len(handles))
+
+
+def HcommMemAlloc(size):
+    p = _vp(0)
+    code = _mem_alloc(C.byref(p), size)
+    return code, (p.value or 0)
+
+
+def HcommGfxReduceKOnThread(thread, dst, srcs, count, dtype, op):
+    arr = (_vp * max(len(srcs), 1))(*srcs)
+    return _reduce_k(thread, dst, arr, len(srcs), count, dtype, op)
+
+
+def HcommGfxRecorderThreadAlloc():
+    h = _u64(0)
+    code = _recorder_alloc(C.byref(h))
+    return code, h.value
+
+
+def launch_log(thread):
+    n = _u32(0)
+    check(_log_read(thread, None, 0, C.byref(n)), "HcommGfxLaunchLogRead")
+    recs = (LaunchRecord * max(n.value, 1))()
+    check(_log_read(thread, recs, n.value, C.byref(n)), "HcommGfxLaunchLogRead")
+    return [recs[i] for i in range(n.value)]
+
+
+def calc_slices(count, unit, n):
+    sl = (Slice * n)()
+    check(_calc_slices(count, unit, n, sl), "HcommGfxCalcSlices")
+    return [(s.offset, s.size) for s in sl]
+
+
+def schedule_emit(alg, n_ranks, count, dtype):
+    n = _u64(0)
+    check(_sched_emit(alg, n_ranks, count, dtype, None, 0, C.byref(n)), "HcommGfxScheduleEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_sched_emit(alg, n_ranks, count, dtype, ops, n.value, C.byref(n)), "HcommGfxScheduleEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+class Plan:
+    """HcommGfxPlan: build once, run many."""
+
+    def __init__(self, alg, lowering, in_ptrs, out_ptrs, count, dtype, op):
+        n = len(in_ptrs)
+        self._in = (_vp * n)(*in_ptrs)
+        self._out = (_vp * n)(*out_ptrs) if out_ptrs is not None else None
+        p = _vp(0)
+        check(_plan_create(alg, lowering, n, self._in, self._out, count, dtype, op, C.byref(p)), "HcommGfxPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+    def run(self, thread):
+        return _plan_run(self._p, thread)
+
+    def run_range(self, thread, first, n):
+        return _plan_run_range(self._p, thread, first, n)
+
+    def launches(self):
+        out = []
+        for i in range(self.info.launches):
+            r = LaunchRecord()
+            check(_plan_launch(self._p, i, C.byref(r)), "HcommGfxPlanGetLaunch")
+            out.append(r)
+        return out
+
+    def destroy(self):
+        if self._p is not None:
+            _plan_destroy(self._p)
+            self._p = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

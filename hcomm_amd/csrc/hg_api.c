@@ -1,0 +1,448 @@
+/*
+ * hg_api.c - the exported primitives: threads, local copy / reduce, notifies, memory, batch mode.
+ *
+ * Mirrors the host adapter of the reference (src/base_comm/primitives/api_c_adpt/cpu_primitives_c_adpt.cc,
+ * hcomm_thread_c_adpt.cc) in names, argument meaning, check order and return codes.  A ThreadHandle is an
+ * opaque pointer to a library-owned object, as in the reference (cpu_primitives_c_adpt.cc:66).
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "hg_host.h"
+
+#define HG_LOG_MAX (1u << 16)
+#define HG_TOUCHED_MAX 64u
+
+static int g_allow_prod = -1;
+
+static int allow_prod(void)
+{
+    if (g_allow_prod < 0) {
+        const char* e = getenv("HCOMM_GFX_ALLOW_PROD");
+        g_allow_prod = (e && e[0] == '1') ? 1 : 0;
+    }
+    return g_allow_prod;
+}
+
+/* thread_local launch context of the calling host thread (cpu_primitives_c_adpt.cc:27) */
+static _Thread_local struct {
+    int batching;
+    HgThread* touched[HG_TOUCHED_MAX];
+    uint32_t ntouched;
+} g_ctx;
+
+const char* HcommGfxVersion(void) { return "hcomm_gfx 0.1 gfx950"; }
+
+uint32_t HcommGfxDataTypeSize(HcommDataType dataType)
+{
+    /* SIZE_TABLE, pkg_inc/legacy/hccl/dtype_common.h:18-36 */
+    switch ((int)dataType) {
+        case HCOMM_DATA_TYPE_INT8: return 1;
+        case HCOMM_DATA_TYPE_INT16: return 2;
+        case HCOMM_DATA_TYPE_INT32: return 4;
+        case HCOMM_DATA_TYPE_FP16: return 2;
+        case HCOMM_DATA_TYPE_FP32: return 4;
+        case HCOMM_DATA_TYPE_INT64: return 8;
+        case HCOMM_DATA_TYPE_UINT64: return 8;
+        case HCOMM_DATA_TYPE_UINT8: return 1;
+        case HCOMM_DATA_TYPE_UINT16: return 2;
+        case HCOMM_DATA_TYPE_UINT32: return 4;
+        case HCOMM_DATA_TYPE_FP64: return 8;
+        case HCOMM_DATA_TYPE_BFP16: return 2;
+        case HCOMM_DATA_TYPE_INT128: return 16;
+        case 13: return 2;
+        case HCOMM_DATA_TYPE_HIF8: return 1;
+        case HCOMM_DATA_TYPE_FP8E4M3: return 1;
+        case HCOMM_DATA_TYPE_FP8E5M2: return 1;
+        case HCOMM_DATA_TYPE_FP8E8M0: return 1;
+        default: return 0;
+    }
+}
+
+int hg_dtype_supported(int dtype)
+{
+    return dtype == HCOMM_DATA_TYPE_FP32 || dtype == HCOMM_DATA_TYPE_FP16 || dtype == HCOMM_DATA_TYPE_INT8 ||
+           dtype == HCOMM_DATA_TYPE_INT16 || dtype == HCOMM_DATA_TYPE_INT32 || dtype == HCOMM_DATA_TYPE_BFP16;
+}
+
+int hg_reduce_supported(int dtype, int op, int prod_ok)
+{
+    if (!hg_dtype_supported(dtype)) return 0;
+    if (op == HCOMM_REDUCE_SUM || op == HCOMM_REDUCE_MAX || op == HCOMM_REDUCE_MIN) return 1;
+    /* PROD: collective-level matrix of the reference excludes int16 (param_check.cc:327-343) */
+    if (op == HCOMM_REDUCE_PROD && prod_ok) return dtype != HCOMM_DATA_TYPE_INT16;
+    return 0;
+}
+
+HgThread* hg_thread_from_handle(ThreadHandle h)
+{
+    HgThread* t = (HgThread*)(uintptr_t)h;
+    if (!t || t->magic != HG_THREAD_MAGIC) return NULL;
+    return t;
+}
+
+/* ---- threads ---------------------------------------------------------------------------------- */
+
+static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_t notify_num)
+{
+    HgThread* t = (HgThread*)calloc(1, sizeof(HgThread));
+    if (!t) return NULL;
+    t->magic = HG_THREAD_MAGIC;
+    t->recorder = recorder;
+    t->stream = stream;
+    t->owns_stream = owns_stream;
+    t->notify_num = notify_num;
+    t->log_enabled = 1;
+    if (notify_num) {
+        t->notifies = (void**)calloc(notify_num, sizeof(void*));
+        if (!t->notifies) {
+            free(t);
+            return NULL;
+        }
+        if (!recorder) {
+            for (uint32_t i = 0; i < notify_num; ++i) {
+                if (hg_rt_event_create(&t->notifies[i]) != HCCL_SUCCESS) {
+                    for (uint32_t j = 0; j < i; ++j) hg_rt_event_destroy(t->notifies[j]);
+                    free(t->notifies);
+                    free(t);
+                    return NULL;
+                }
+            }
+        }
+    }
+    return t;
+}
+
+static void thread_delete(HgThread* t)
+{
+    if (!t) return;
+    if (!t->recorder) {
+        for (uint32_t i = 0; i < t->notify_num; ++i)
+            if (t->notifies[i]) hg_rt_event_destroy(t->notifies[i]);
+        if (t->owns_stream && t->stream) {
+            hg_rt_stream_sync(t->stream);
+            hg_rt_stream_destroy(t->stream);
+        }
+    }
+    free(t->notifies);
+    free(t->pending);
+    free(t->log);
+    t->magic = 0;
+    free(t);
+}
+
+HcommResult
+HcommThreadAlloc(CommEngine engine, uint32_t threadNum, const uint32_t* notifyNumPerThread, ThreadHandle* threads)
+{
+    (void)engine;
+    if (!threads) return HCCL_E_PTR;
+    if (!notifyNumPerThread) return HCCL_E_PTR;
+    if (threadNum == 0) return HCCL_E_PARA;
+    if (hg_rt_device_count() <= 0) return HCCL_E_UNAVAIL;
+    const uint32_t notify_num = notifyNumPerThread[0]; /* only [0] is used (hcomm_thread_c_adpt.cc:44-49) */
+    for (uint32_t i = 0; i < threadNum; ++i) {
+        void* stream = NULL;
+        HgThread* t = NULL;
+        if (hg_rt_stream_create(&stream) == HCCL_SUCCESS) t = thread_new(0, stream, 1, notify_num);
+        if (!t) {
+            if (stream) hg_rt_stream_destroy(stream);
+            for (uint32_t j = 0; j < i; ++j) thread_delete(hg_thread_from_handle(threads[j]));
+            return HCCL_E_INTERNAL;
+        }
+        threads[i] = (ThreadHandle)(uintptr_t)t;
+    }
+    return HCCL_SUCCESS;
+}
+
+HcommResult HcommThreadFree(const ThreadHandle* threads, uint32_t threadNum)
+{
+    if (!threads) return HCCL_E_PTR;
+    HcommResult ret = HCCL_SUCCESS;
+    for (uint32_t i = 0; i < threadNum; ++i) {
+        HgThread* t = hg_thread_from_handle(threads[i]);
+        if (!t) {
+            ret = HCCL_E_NOT_FOUND;
+            continue;
+        }
+        thread_delete(t);
+    }
+    return ret;
+}
+
+HcommResult HcommThreadAllocWithStream(CommEngine engine, void* stream, uint32_t notifyNum, ThreadHandle* thread)
+{
+    (void)engine;
+    if (!thread) return HCCL_E_PTR;
+    if (hg_rt_device_count() <= 0) return HCCL_E_UNAVAIL;
+    HgThread* t = thread_new(0, stream, 0, notifyNum);
+    if (!t) return HCCL_E_PTR;
+    *thread = (ThreadHandle)(uintptr_t)t;
+    return HCCL_SUCCESS;
+}
+
+HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t threadNum)
+{
+    if (!threads) return HCCL_E_PTR;
+    if (threadNum == 0) return HCCL_E_PARA; /* hcomm_thread_c_adpt.cc:190-193 */
+    return HcommThreadFree(threads, threadNum);
+}
+
+HcommResult HcommGfxRecorderThreadAlloc(ThreadHandle* thread)
+{
+    if (!thread) return HCCL_E_PTR;
+    HgThread* t = thread_new(1, NULL, 0, 0);
+    if (!t) return HCCL_E_MEMORY;
+    *thread = (ThreadHandle)(uintptr_t)t;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxThreadSynchronize(ThreadHandle thread)
+{
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (t->recorder) return HCCL_SUCCESS;
+    return hg_rt_stream_sync(t->stream);
+}
+
+/* ---- launch log and submission ---------------------------------------------------------------------- */
+
+static void log_launch(HgThread* t, const HgLaunch* l)
+{
+    if (!t->log_enabled || t->log_n >= HG_LOG_MAX) return;
+    if (t->log_n == t->log_cap) {
+        uint32_t cap = t->log_cap ? t->log_cap * 2 : 64;
+        HcommGfxLaunchRecord* p = (HcommGfxLaunchRecord*)realloc(t->log, cap * sizeof(*p));
+        if (!p) return;
+        t->log = p;
+        t->log_cap = cap;
+    }
+    HcommGfxLaunchRecord* r = &t->log[t->log_n++];
+    r->kind = l->kind;
+    r->dtype = l->dtype;
+    r->op = l->op;
+    r->nseg = l->nseg;
+    r->bytes = l->bytes;
+    r->blocks = l->blocks;
+}
+
+int hg_submit(HgThread* t, const HgLaunch* l)
+{
+    log_launch(t, l);
+    if (t->recorder) return HCCL_SUCCESS;
+    switch (l->kind) {
+        case HCOMM_GFX_KERNEL_COPY: return hg_launch_copy(t->stream, &l->tab.seg2, l->blocks);
+        case HCOMM_GFX_KERNEL_REDUCE2:
+            return hg_launch_reduce2(t->stream, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks);
+        case HCOMM_GFX_KERNEL_BYTEWISE:
+            return hg_launch_bytewise(t->stream, l->op != 255u, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks);
+        case HCOMM_GFX_KERNEL_CHAIN:
+        case HCOMM_GFX_KERNEL_TREE:
+            return hg_launch_fold(t->stream, (int)l->dtype, (int)l->op, (int)l->acc_is_dst, &l->tab.fold, l->blocks);
+        default: return HCCL_E_INTERNAL;
+    }
+}
+
+int32_t HcommGfxLaunchLogRead(ThreadHandle thread, HcommGfxLaunchRecord* out, uint32_t cap, uint32_t* n)
+{
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t || !n) return HCCL_E_PTR;
+    *n = t->log_n;
+    if (out) {
+        const uint32_t m = t->log_n < cap ? t->log_n : cap;
+        if (m) memcpy(out, t->log, m * sizeof(*out));
+    }
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxLaunchLogClear(ThreadHandle thread)
+{
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    t->log_n = 0;
+    return HCCL_SUCCESS;
+}
+
+/* ---- eager / batch submission of primitive calls -------------------------------------------------------- */
+
+static int emit_to_thread(const HgLaunch* l, void* ctx) { return hg_submit((HgThread*)ctx, l); }
+
+static int record_or_run(HgThread* t, const HgOp* o)
+{
+    if (!g_ctx.batching) return hg_coalesce(o, 1, emit_to_thread, t);
+    if (t->pending_n == t->pending_cap) {
+        uint32_t cap = t->pending_cap ? t->pending_cap * 2 : 64;
+        HgOp* p = (HgOp*)realloc(t->pending, cap * sizeof(*p));
+        if (!p) return HCCL_E_MEMORY;
+        t->pending = p;
+        t->pending_cap = cap;
+    }
+    t->pending[t->pending_n++] = *o;
+    uint32_t i = 0;
+    while (i < g_ctx.ntouched && g_ctx.touched[i] != t) ++i;
+    if (i == g_ctx.ntouched) {
+        if (g_ctx.ntouched == HG_TOUCHED_MAX) return HCCL_E_UNAVAIL;
+        g_ctx.touched[g_ctx.ntouched++] = t;
+    }
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommLocalCopyOnThread(ThreadHandle thread, void* dst, const void* src, uint64_t len)
+{
+    if (!dst) return HCCL_E_PTR;
+    if (!src) return HCCL_E_PTR;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    HgOp o;
+    memset(&o, 0, sizeof(o));
+    o.is_reduce = 0;
+    o.dtype = 255;
+    o.op = 255;
+    o.dst = dst;
+    o.src = src;
+    o.bytes = len;
+    return record_or_run(t, &o);
+}
+
+int32_t HcommLocalReduceOnThread(
+    ThreadHandle thread, void* dst, const void* src, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp)
+{
+    if (!dst) return HCCL_E_PTR;
+    if (!src) return HCCL_E_PTR;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, allow_prod())) return HCCL_E_PARA;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    HgOp o;
+    memset(&o, 0, sizeof(o));
+    o.is_reduce = 1;
+    o.dtype = (uint8_t)dataType;
+    o.op = (uint8_t)reduceOp;
+    o.dst = dst;
+    o.src = src;
+    o.bytes = count * HcommGfxDataTypeSize(dataType); /* cpu_primitives_c_adpt.cc:109 */
+    return record_or_run(t, &o);
+}
+
+int32_t HcommBatchModeStart(const char* batchTag)
+{
+    (void)batchTag;
+    if (g_ctx.batching) return HCCL_E_PARA;
+    g_ctx.batching = 1;
+    g_ctx.ntouched = 0;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommBatchModeEnd(const char* batchTag)
+{
+    (void)batchTag;
+    if (!g_ctx.batching) return HCCL_E_PARA;
+    g_ctx.batching = 0;
+    int32_t ret = HCCL_SUCCESS;
+    for (uint32_t i = 0; i < g_ctx.ntouched; ++i) {
+        HgThread* t = g_ctx.touched[i];
+        if (ret == HCCL_SUCCESS) ret = hg_coalesce(t->pending, t->pending_n, emit_to_thread, t);
+        t->pending_n = 0;
+    }
+    g_ctx.ntouched = 0;
+    return ret;
+}
+
+/* ---- k-way fused reduce -------------------------------------------------------------------------- */
+
+int32_t HcommGfxReduceKOnThread(
+    ThreadHandle thread, void* dst, const void* const* srcs, uint32_t k, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp)
+{
+    if (!dst) return HCCL_E_PTR;
+    if (!srcs) return HCCL_E_PTR;
+    if (k == 0 || k > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    for (uint32_t j = 0; j < k; ++j)
+        if (!srcs[j]) return HCCL_E_PTR;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    const uint64_t bytes = count * HcommGfxDataTypeSize(dataType);
+    if (bytes == 0) return HCCL_SUCCESS;
+    uintptr_t align = (uintptr_t)dst;
+    for (uint32_t j = 0; j < k; ++j) align |= (uintptr_t)srcs[j];
+    if (align & (HG_VEC_BYTES - 1)) {
+        /* unaligned operands: the same chain as k-1 two-input element-wise launches */
+        HgOp o;
+        memset(&o, 0, sizeof(o));
+        o.dst = dst;
+        o.src = srcs[0];
+        o.bytes = bytes;
+        o.dtype = 255;
+        o.op = 255;
+        int32_t ret = hg_coalesce(&o, 1, emit_to_thread, t);
+        for (uint32_t j = 1; j < k && ret == HCCL_SUCCESS; ++j) {
+            o.is_reduce = 1;
+            o.dtype = (uint8_t)dataType;
+            o.op = (uint8_t)reduceOp;
+            o.src = srcs[j];
+            ret = hg_coalesce(&o, 1, emit_to_thread, t);
+        }
+        return ret;
+    }
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    l->kind = HCOMM_GFX_KERNEL_CHAIN;
+    l->dtype = (uint32_t)dataType;
+    l->op = (uint32_t)reduceOp;
+    l->acc_is_dst = 1;
+    HgFoldTable* f = &l->tab.fold;
+    for (uint32_t j = 0; j < k; ++j) f->in[j] = srcs[j];
+    f->out[0] = dst;
+    f->nseg = 1;
+    f->k = k;
+    f->nranks = k;
+    f->stride = 1;
+    f->out_mode = 1;
+    f->bytes[0] = bytes;
+    hg_finish_fold(l);
+    int32_t ret = hg_submit(t, l);
+    free(l);
+    return ret;
+}
+
+/* ---- notifies ------------------------------------------------------------------------------------ */
+
+int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx)
+{
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    HgThread* d = hg_thread_from_handle(dstThread);
+    if (!d) return HCCL_E_PTR;
+    if (dstNotifyIdx >= d->notify_num) return HCCL_E_PARA;
+    if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    if (t->recorder || d->recorder) return HCCL_SUCCESS;
+    return hg_rt_event_record(d->notifies[dstNotifyIdx], t->stream);
+}
+
+int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut)
+{
+    (void)timeOut;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (notifyIdx >= t->notify_num) return HCCL_E_PARA;
+    if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    if (t->recorder) return HCCL_SUCCESS;
+    return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
+}
+
+/* ---- memory -------------------------------------------------------------------------------------- */
+
+HcommResult HcommMemAlloc(void** ptr, size_t size)
+{
+    if (!ptr) return HCCL_E_PTR;
+    if (size == 0) return HCCL_E_PARA;
+    *ptr = NULL;
+    return hg_rt_malloc(ptr, size);
+}
+
+HcommResult HcommMemFree(void* ptr)
+{
+    if (!ptr) return HCCL_E_PTR;
+    return hg_rt_free(ptr);
+}

@@ -1,0 +1,141 @@
+/*
+ * hg_batch.c - turning recorded primitive calls into kernel launches.
+ *
+ * The reference's batch mode only records between HcommBatchModeStart and HcommBatchModeEnd and submits
+ * once at End (src/base_comm/primitives/launch_context.cc:23-43,139-174).  Here "submitting" additionally
+ * merges runs of operations that cannot observe each other into one launch, which is how all N simulated
+ * ranks of a collective step end up in a single kernel.  The independence test is the memory-conflict rule
+ * of the reference's schedule checker (test/st/algorithm/README_en.md:202-231): within one launch no
+ * written range may overlap any other range that is read or written.
+ */
+#include <stdlib.h>
+#include <string.h>
+
+#include "hg_host.h"
+
+static uint64_t g_grid_cap = 0;
+
+uint64_t hg_grid_blocks(uint64_t total_tiles)
+{
+    if (g_grid_cap == 0) {
+        const char* e = getenv("HCOMM_GFX_GRID_CAP");
+        uint64_t cap = e ? strtoull(e, NULL, 10) : 0;
+        if (cap == 0) {
+            int cus = hg_rt_num_cus();
+            if (cus <= 0) cus = 256;
+            cap = (uint64_t)cus * 8u; /* 8 workgroups x 4 wavefronts fill a CU's 32 wavefront slots */
+        }
+        g_grid_cap = cap;
+    }
+    return total_tiles < g_grid_cap ? total_tiles : g_grid_cap;
+}
+
+static uint64_t tiles_of(uint64_t bytes) { return (bytes + HG_TILE_BYTES - 1) / HG_TILE_BYTES; }
+
+void hg_finish_seg2(HgLaunch* l)
+{
+    HgSeg2Table* t = &l->tab.seg2;
+    uint64_t tiles = 0, bytes = 0;
+    /* the bytewise kernel walks elements, not vectors: one "tile" is HG_TILE_VECS elements */
+    uint32_t es = 1;
+    if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE && l->op != 255u) es = HcommGfxDataTypeSize((HcommDataType)l->dtype);
+    for (uint32_t s = 0; s < t->nseg; ++s) {
+        t->tile_begin[s] = (uint32_t)tiles;
+        if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE)
+            tiles += (t->bytes[s] / es + HG_TILE_VECS - 1) / HG_TILE_VECS;
+        else
+            tiles += tiles_of(t->bytes[s]);
+        bytes += t->bytes[s];
+    }
+    t->tile_begin[t->nseg] = (uint32_t)tiles;
+    l->nseg = t->nseg;
+    l->bytes = bytes;
+    l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
+    l->blocks = hg_grid_blocks(tiles);
+}
+
+void hg_finish_fold(HgLaunch* l)
+{
+    HgFoldTable* t = &l->tab.fold;
+    uint64_t tiles = 0, bytes = 0;
+    for (uint32_t s = 0; s < t->nseg; ++s) {
+        t->tile_begin[s] = (uint32_t)tiles;
+        tiles += tiles_of(t->bytes[s]);
+        bytes += t->bytes[s];
+    }
+    t->tile_begin[t->nseg] = (uint32_t)tiles;
+    l->nseg = t->nseg;
+    l->bytes = bytes;
+    uint64_t per = t->k; /* reads */
+    if (t->store_partials) per += t->k - 1;
+    if (t->store_final_first) per += 1;
+    if (t->out_mode == 1) per += 1;
+    if (t->out_mode == 2) per += t->nranks;
+    l->moved_bytes = bytes * per;
+    l->blocks = hg_grid_blocks(tiles);
+}
+
+static int overlaps(const void* a, uint64_t an, const void* b, uint64_t bn)
+{
+    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+    return a0 < b0 + bn && b0 < a0 + an;
+}
+
+static int aligned16(const HgOp* o) { return (((uintptr_t)o->dst | (uintptr_t)o->src) & (HG_VEC_BYTES - 1)) == 0; }
+
+static uint32_t kind_of(const HgOp* o)
+{
+    if (!aligned16(o)) return HCOMM_GFX_KERNEL_BYTEWISE;
+    return o->is_reduce ? HCOMM_GFX_KERNEL_REDUCE2 : HCOMM_GFX_KERNEL_COPY;
+}
+
+static int conflicts(const HgLaunch* l, const HgOp* o)
+{
+    const HgSeg2Table* t = &l->tab.seg2;
+    for (uint32_t s = 0; s < t->nseg; ++s) {
+        if (overlaps(o->dst, o->bytes, t->dst[s], t->bytes[s])) return 1;
+        if (overlaps(o->dst, o->bytes, t->src[s], t->bytes[s])) return 1;
+        if (overlaps(o->src, o->bytes, t->dst[s], t->bytes[s])) return 1;
+    }
+    return 0;
+}
+
+int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
+{
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    int rc = HCCL_SUCCESS;
+    int open = 0;
+    for (uint64_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
+        const HgOp* o = &ops[i];
+        if (o->bytes == 0) continue;                   /* count == 0: nothing to do (dispatcher.cc:719-722) */
+        if (!o->is_reduce && o->dst == o->src) continue; /* copy onto itself (dispatcher.cc:495-498) */
+        const uint32_t kind = kind_of(o);
+        const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
+        if (open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG ||
+                     conflicts(l, o))) {
+            hg_finish_seg2(l);
+            rc = emit(l, ctx);
+            open = 0;
+            if (rc != HCCL_SUCCESS) break;
+        }
+        if (!open) {
+            memset(l, 0, sizeof(*l));
+            l->kind = kind;
+            l->dtype = dt;
+            l->op = op;
+            open = 1;
+        }
+        HgSeg2Table* t = &l->tab.seg2;
+        t->dst[t->nseg] = o->dst;
+        t->src[t->nseg] = o->src;
+        t->bytes[t->nseg] = o->bytes;
+        t->nseg++;
+    }
+    if (open && rc == HCCL_SUCCESS) {
+        hg_finish_seg2(l);
+        rc = emit(l, ctx);
+    }
+    free(l);
+    return rc;
+}

@@ -1,0 +1,71 @@
+/*
+ * hg_host.h - host-side objects of libhcomm_gfx.so shared by hg_api.c, hg_batch.c, hg_sched.c and hg_plan.c.
+ */
+#ifndef HG_HOST_H
+#define HG_HOST_H
+
+#include "hg_internal.h"
+
+#define HG_THREAD_MAGIC 0x48474654u /* "HGFT" */
+#define HG_PLAN_MAGIC 0x4847504cu   /* "HGPL" */
+
+/* One recorded primitive call (also the unit the batch coalescer works on). */
+typedef struct {
+    uint8_t is_reduce;
+    uint8_t dtype; /* HcommDataType (255 for copies) */
+    uint8_t op;    /* HcommReduceOp (255 for copies) */
+    void* dst;
+    const void* src;
+    uint64_t bytes;
+} HgOp;
+
+/* One kernel launch, fully prepared on the host. */
+typedef struct {
+    uint32_t kind; /* HcommGfxKernelKind */
+    uint32_t dtype;
+    uint32_t op;
+    uint32_t acc_is_dst; /* fold kernels only */
+    uint64_t blocks;
+    uint64_t bytes;       /* output bytes covered */
+    uint64_t moved_bytes; /* bytes read + written */
+    uint32_t nseg;
+    union {
+        HgSeg2Table seg2;
+        HgFoldTable fold;
+    } tab;
+} HgLaunch;
+
+typedef struct HgThread {
+    uint32_t magic;
+    int recorder;     /* 1: log launches, never touch the GPU */
+    int owns_stream;
+    void* stream;     /* hipStream_t */
+    uint32_t notify_num;
+    void** notifies;  /* hipEvent_t per slot */
+    /* operations recorded in batch mode, in call order */
+    HgOp* pending;
+    uint32_t pending_n, pending_cap;
+    /* launch log */
+    HcommGfxLaunchRecord* log;
+    uint32_t log_n, log_cap;
+    int log_enabled;
+} HgThread;
+
+HgThread* hg_thread_from_handle(ThreadHandle h);
+
+/* Turn a list of operations (stream order) into launches: consecutive independent operations of equal
+ * kind / dtype / op share one launch.  Calls emit(launch, ctx) for each; stops at the first error. */
+typedef int (*HgEmitFn)(const HgLaunch* launch, void* ctx);
+int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
+
+/* Fill tile_begin / blocks / bytes of a launch whose segment pointers and sizes are set. */
+void hg_finish_seg2(HgLaunch* l);
+void hg_finish_fold(HgLaunch* l);
+
+/* Execute (or, on a recorder thread, log) one prepared launch. */
+int hg_submit(HgThread* t, const HgLaunch* l);
+
+int hg_dtype_supported(int dtype);
+int hg_reduce_supported(int dtype, int op, int allow_prod);
+
+#endif

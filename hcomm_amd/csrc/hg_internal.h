@@ -1,0 +1,83 @@
+/*
+ * hg_internal.h - interface between the C host code of libhcomm_gfx.so and its HIP launchers.
+ * Plain C; included by the .c host files and by hg_kernels.hip.
+ */
+#ifndef HG_INTERNAL_H
+#define HG_INTERNAL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "hcomm_gfx.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HG_MAX_SEG 32u          /* segments per launch */
+#define HG_VEC_BYTES 16u        /* one lane moves 128 bits per access */
+#define HG_BLOCK 256u           /* threads per workgroup = 4 wavefronts of 64 */
+#define HG_UNROLL 4u            /* 128-bit accesses in flight per lane and operand */
+#define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
+#define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
+
+/* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
+typedef struct {
+    void* dst[HG_MAX_SEG];
+    const void* src[HG_MAX_SEG];
+    uint64_t bytes[HG_MAX_SEG];
+    uint32_t tile_begin[HG_MAX_SEG + 1]; /* prefix sum of tiles per segment */
+    uint32_t nseg;
+} HgSeg2Table;
+
+/*
+ * k-way fold table.  Segment s folds K values per element, position j = 0..K-1 being read from
+ *   in[(first[s] + j * stride) mod nranks] + off[s]
+ * (a rotation of the rank buffers, which is what every ring / mesh schedule uses), or, when
+ * tree != 0, from in[first[s] XOR bitrev(j)] + off[s] (recursive halving).
+ */
+typedef struct {
+    const void* in[HCOMM_GFX_MAX_RANKS];
+    void* out[HCOMM_GFX_MAX_RANKS];
+    uint64_t off[HG_MAX_SEG];     /* byte offset applied to every in[] (and out[] in fan-out mode) */
+    uint64_t out_off[HG_MAX_SEG]; /* byte offset into out[owner[s]] in single-output mode */
+    uint64_t bytes[HG_MAX_SEG];
+    uint32_t tile_begin[HG_MAX_SEG + 1];
+    uint32_t nseg;
+    uint32_t k;              /* values folded per element */
+    uint32_t nranks;         /* modulus of the rotation */
+    int32_t stride;          /* +1 or -1 */
+    uint32_t store_partials; /* store the running value to position j's buffer after fold step j >= 1 */
+    uint32_t store_final_first; /* store the final value to position 0's buffer */
+    uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
+    uint32_t tree;           /* 0 chain, 1 binary tree (k must be a power of two) */
+    uint8_t first[HG_MAX_SEG];
+    uint8_t owner[HG_MAX_SEG];
+} HgFoldTable;
+
+/* Launch geometry decided on the host so that recorder threads can report it without a GPU. */
+uint64_t hg_grid_blocks(uint64_t total_tiles);
+
+/* Launchers.  stream is a hipStream_t.  Return a HcclResult-compatible code. */
+int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks);
+int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks);
+int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks);
+int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks);
+
+/* Thin wrappers over the HIP runtime so that the C files need no HIP headers. */
+int hg_rt_device_count(void);
+int hg_rt_stream_create(void** stream);
+int hg_rt_stream_destroy(void* stream);
+int hg_rt_stream_sync(void* stream);
+int hg_rt_event_create(void** ev);
+int hg_rt_event_destroy(void* ev);
+int hg_rt_event_record(void* ev, void* stream);
+int hg_rt_stream_wait_event(void* stream, void* ev);
+int hg_rt_malloc(void** p, size_t n);
+int hg_rt_free(void* p);
+int hg_rt_num_cus(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

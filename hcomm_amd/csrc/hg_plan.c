@@ -1,0 +1,267 @@
+/*
+ * hg_plan.c - lowering a schedule to a fixed list of kernel launches ("prepare once, run many", the
+ * Prepare / RunAsync split of the reference's templates,
+ * src/legacy/ascend910/algorithm/base/alg_template/alg_template_base_pub.h:237-253).
+ *
+ * STEPWISE lowering feeds the op list through the same coalescer batch mode uses, so every launch is one
+ * schedule step over all ranks.  FUSED lowering uses the k-way fold kernel where the data flow of a whole
+ * phase is element-wise (every ring and mesh schedule): each input is read once, and every value the
+ * step-wise replay would leave in a buffer is still stored, so both lowerings end in identical memory.
+ */
+#include <stdlib.h>
+#include <string.h>
+
+#include "hg_host.h"
+#include "hg_sched.h"
+
+struct HcommGfxPlan {
+    uint32_t magic;
+    uint32_t nlaunch, cap;
+    HgLaunch* launches;
+    HcommGfxPlanInfo info;
+};
+
+static int plan_push(const HgLaunch* l, void* ctx)
+{
+    HcommGfxPlan* p = (HcommGfxPlan*)ctx;
+    if (p->nlaunch == p->cap) {
+        uint32_t cap = p->cap ? p->cap * 2 : 16;
+        HgLaunch* q = (HgLaunch*)realloc(p->launches, (size_t)cap * sizeof(*q));
+        if (!q) return HCCL_E_MEMORY;
+        p->launches = q;
+        p->cap = cap;
+    }
+    p->launches[p->nlaunch++] = *l;
+    p->info.movedBytes += l->moved_bytes;
+    return HCCL_SUCCESS;
+}
+
+static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, void* const* out, int dtype, int op)
+{
+    HgOp* ops = (HgOp*)calloc(ol->n ? ol->n : 1, sizeof(HgOp));
+    if (!ops) return HCCL_E_MEMORY;
+    for (uint64_t i = 0; i < ol->n; ++i) {
+        const HcommGfxSchedOp* s = &ol->ops[i];
+        HgOp* o = &ops[i];
+        o->is_reduce = (uint8_t)s->kind;
+        o->dtype = s->kind ? (uint8_t)dtype : 255;
+        o->op = s->kind ? (uint8_t)op : 255;
+        o->dst = (char*)(s->dstBuf ? out[s->rank] : in[s->rank]) + s->dstOff;
+        o->src = (const char*)(s->srcBuf ? out[s->srcRank] : in[s->srcRank]) + s->srcOff;
+        o->bytes = s->bytes;
+    }
+    int rc = hg_coalesce(ops, ol->n, plan_push, p);
+    free(ops);
+    return rc;
+}
+
+static HgLaunch* new_fold(int dtype, int op, int acc_is_dst, uint32_t n, void* const* in, void* const* out)
+{
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return NULL;
+    l->kind = HCOMM_GFX_KERNEL_CHAIN;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    l->acc_is_dst = (uint32_t)acc_is_dst;
+    HgFoldTable* f = &l->tab.fold;
+    for (uint32_t r = 0; r < n; ++r) {
+        f->in[r] = in[r];
+        f->out[r] = out ? out[r] : NULL;
+    }
+    f->k = n;
+    f->nranks = n;
+    f->stride = 1;
+    return l;
+}
+
+static int single_copy(HcommGfxPlan* p, void* dst, const void* src, uint64_t bytes)
+{
+    HgOp o;
+    memset(&o, 0, sizeof(o));
+    o.dtype = 255;
+    o.op = 255;
+    o.dst = dst;
+    o.src = src;
+    o.bytes = bytes;
+    return hg_coalesce(&o, 1, plan_push, p);
+}
+
+/* ring allreduce / reduce-scatter: slice c travels c+1 -> c+2 -> ... -> c, every hop storing its partial */
+static int fused_ring(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype,
+                      int op, int out_mode, int standalone)
+{
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    if (standalone) {
+        for (uint32_t i = 0; i < n; ++i) {
+            sl[i].offset = (uint64_t)i * count * unit;
+            sl[i].size = count * unit;
+        }
+    } else {
+        int rc = HcommGfxCalcSlices(count, unit, n, sl);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    HgLaunch* l = new_fold(dtype, op, 0, n, in, out);
+    if (!l) return HCCL_E_MEMORY;
+    HgFoldTable* f = &l->tab.fold;
+    f->store_partials = 1;
+    f->out_mode = (uint32_t)out_mode;
+    for (uint32_t c = 0; c < n; ++c) {
+        if (sl[c].size == 0) continue;
+        const uint32_t s = f->nseg++;
+        f->off[s] = sl[c].offset;
+        f->bytes[s] = sl[c].size;
+        f->first[s] = (uint8_t)((c + 1) % n);
+        f->owner[s] = (uint8_t)c;
+        f->out_off[s] = 0;
+    }
+    int rc = HCCL_SUCCESS;
+    if (f->nseg) {
+        hg_finish_fold(l);
+        rc = plan_push(l, p);
+    }
+    free(l);
+    return rc;
+}
+
+static int fused_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype,
+                      int op, int scatter)
+{
+    const uint64_t sz = count * HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (sz == 0) return HCCL_SUCCESS;
+    HgLaunch* l = new_fold(dtype, op, 1, n, in, out);
+    if (!l) return HCCL_E_MEMORY;
+    HgFoldTable* f = &l->tab.fold;
+    f->out_mode = 1;
+    f->stride = scatter ? -1 : 1;     /* reduce-scatter visits r-1, r-2, ...; one-shot visits r+1, r+2, ... */
+    f->store_final_first = scatter ? 1 : 0; /* reduce-scatter accumulates in in[r][slice r] before copying out */
+    f->nseg = n;
+    for (uint32_t r = 0; r < n; ++r) {
+        f->off[r] = scatter ? (uint64_t)r * sz : 0;
+        f->bytes[r] = sz;
+        f->first[r] = (uint8_t)r;
+        f->owner[r] = (uint8_t)r;
+        f->out_off[r] = 0;
+    }
+    hg_finish_fold(l);
+    int rc = plan_push(l, p);
+    free(l);
+    return rc;
+}
+
+static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
+                       int dtype, int op)
+{
+    const uint64_t total = count * HcommGfxDataTypeSize((HcommDataType)dtype);
+    switch (alg) {
+        case HCOMM_GFX_ALG_ALLREDUCE_RING:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_ring(p, n, in, out, count, dtype, op, 2, 0);
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING:
+            if (n == 1) return HCCL_SUCCESS;
+            return fused_ring(p, n, in, out, count, dtype, op, 0, 0);
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_ring(p, n, in, out, count, dtype, op, 1, 1);
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: return fused_mesh(p, n, in, out, count, dtype, op, 0);
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_mesh(p, n, in, out, count, dtype, op, 1);
+        default: return HCCL_E_NOT_SUPPORT;
+    }
+}
+
+static int in_place(int alg) { return alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING; }
+
+int32_t HcommGfxPlanCreate(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!in) return HCCL_E_PTR;
+    if (!out && !in_place((int)alg)) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    if (lowering != HCOMM_GFX_LOWER_STEPWISE && lowering != HCOMM_GFX_LOWER_FUSED) return HCCL_E_PARA;
+    for (uint32_t r = 0; r < nRanks; ++r) {
+        if (!in[r]) return HCCL_E_PTR;
+        if (((uintptr_t)in[r]) & 127u) return HCCL_E_PARA;
+        if (!in_place((int)alg)) {
+            if (!out[r]) return HCCL_E_PTR;
+            if (((uintptr_t)out[r]) & 127u) return HCCL_E_PARA;
+        }
+    }
+    HgOpList ol;
+    int rc = hg_schedule(&ol, (int)alg, nRanks, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
+    if (!p) {
+        hg_oplist_free(&ol);
+        return HCCL_E_MEMORY;
+    }
+    p->magic = HG_PLAN_MAGIC;
+    p->info.steps = ol.steps;
+    for (uint64_t i = 0; i < ol.n; ++i) p->info.algorithmicBytes += ol.ops[i].bytes * (ol.ops[i].kind ? 3u : 2u);
+    if (lowering == HCOMM_GFX_LOWER_STEPWISE)
+        rc = lower_stepwise(p, &ol, in, out, (int)dataType, (int)reduceOp);
+    else
+        rc = lower_fused(p, (int)alg, nRanks, in, out, count, (int)dataType, (int)reduceOp);
+    hg_oplist_free(&ol);
+    if (rc != HCCL_SUCCESS) {
+        HcommGfxPlanDestroy(p);
+        return rc;
+    }
+    p->info.launches = p->nlaunch;
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (first > plan->nlaunch || n > plan->nlaunch - first) return HCCL_E_PARA;
+    for (uint32_t i = first; i < first + n; ++i) {
+        int rc = hg_submit(t, &plan->launches[i]);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
+    return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+}
+
+int32_t HcommGfxPlanDestroy(HcommGfxPlan* plan)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
+    plan->magic = 0;
+    free(plan->launches);
+    free(plan);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanGetInfo(const HcommGfxPlan* plan, HcommGfxPlanInfo* info)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC || !info) return HCCL_E_PTR;
+    *info = plan->info;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaunchRecord* rec)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC || !rec) return HCCL_E_PTR;
+    if (i >= plan->nlaunch) return HCCL_E_PARA;
+    const HgLaunch* l = &plan->launches[i];
+    rec->kind = l->kind;
+    rec->dtype = l->dtype;
+    rec->op = l->op;
+    rec->nseg = l->nseg;
+    rec->bytes = l->bytes;
+    rec->blocks = l->blocks;
+    return HCCL_SUCCESS;
+}

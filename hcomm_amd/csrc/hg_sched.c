@@ -1,0 +1,250 @@
+/*
+ * hg_sched.c - slice tables and the step lists of the ring, recursive halving-doubling and mesh schedules.
+ *
+ * Each generator states the schedule in closed form per step t (all ranks act in parallel inside a step)
+ * and emits the two-input operations the reference's templates hand to the dispatcher: a copy
+ * (HcclD2DMemcpyAsync) or a reduce dst = dst (op) src (HcclReduceAsync) - src/legacy/ascend910/platform/task/
+ * dispatcher_common.cc:114-147.  Paths below are relative to
+ * src/legacy/ascend910/algorithm/base/alg_template/.  The reduce operand roles follow the inline-reduce branch
+ * of Reducer::run (component/reducer.cc:199-222): dst is the local buffer, src the peer's.
+ */
+#include <stdlib.h>
+#include <string.h>
+
+#include "hg_host.h"
+#include "hg_sched.h"
+
+#define HG_SLICE_ALIGN 128u /* HCCL_MIN_SLICE_ALIGN, alg_template_base_pub.h:43 */
+
+int32_t HcommGfxCalcSlices(uint64_t count, uint32_t unitSize, uint32_t n, HcommGfxSlice* slices)
+{
+    if (!slices) return HCCL_E_PTR;
+    if (unitSize == 0 || n == 0) return HCCL_E_PARA;
+    /* temp_all_reduce/all_reduce_ring.cc:142-153; RoundUpWithDivisor(0, 128) is 128 (alg_template_base_pub.h:609-616) */
+    const uint64_t total = count * unitSize;
+    const uint64_t per_raw = (total + (n - 1)) / n;
+    const uint64_t per = (per_raw == 0) ? HG_SLICE_ALIGN : ((per_raw + HG_SLICE_ALIGN - 1) / HG_SLICE_ALIGN) * HG_SLICE_ALIGN;
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < n; ++i) {
+        slices[i].size = residue > per ? per : residue;
+        slices[i].offset = total - residue;
+        residue -= slices[i].size;
+    }
+    return HCCL_SUCCESS;
+}
+
+void hg_oplist_free(HgOpList* l)
+{
+    free(l->ops);
+    memset(l, 0, sizeof(*l));
+}
+
+static int push(HgOpList* l, uint32_t step, uint32_t kind, uint32_t rank, uint32_t dst_buf, uint64_t dst_off,
+                uint32_t src_rank, uint32_t src_buf, uint64_t src_off, uint64_t bytes)
+{
+    if (step + 1 > l->steps) l->steps = step + 1;
+    if (bytes == 0) return HCCL_SUCCESS; /* zero-size slices produce no work (dispatcher.cc:495-498, 719-722) */
+    if (l->n == l->cap) {
+        uint64_t cap = l->cap ? l->cap * 2 : 256;
+        HcommGfxSchedOp* p = (HcommGfxSchedOp*)realloc(l->ops, cap * sizeof(*p));
+        if (!p) return HCCL_E_MEMORY;
+        l->ops = p;
+        l->cap = cap;
+    }
+    HcommGfxSchedOp* o = &l->ops[l->n++];
+    o->step = step;
+    o->kind = kind;
+    o->rank = rank;
+    o->dstBuf = dst_buf;
+    o->srcRank = src_rank;
+    o->srcBuf = src_buf;
+    o->dstOff = dst_off;
+    o->srcOff = src_off;
+    o->bytes = bytes;
+    return HCCL_SUCCESS;
+}
+
+#define IN 0u
+#define OUT 1u
+#define COPY 0u
+#define REDUCE 1u
+#define CHK(x)                                \
+    do {                                      \
+        int rc_ = (x);                        \
+        if (rc_ != HCCL_SUCCESS) return rc_;  \
+    } while (0)
+
+static uint32_t modn(int64_t v, uint32_t n)
+{
+    int64_t r = v % (int64_t)n;
+    return (uint32_t)(r < 0 ? r + n : r);
+}
+
+/* Ring reduce-scatter over `sl` in the input buffers: step t, rank r reduces slice (r-2-t) from its left
+ * neighbour (temp_reduce_scatter/reduce_scatter_ring.cc:207,214,260,268; last step :288-304). */
+static int ring_rs(HgOpList* l, uint32_t n, const HcommGfxSlice* sl, uint32_t step0)
+{
+    for (uint32_t t = 0; t + 1 < n; ++t)
+        for (uint32_t r = 0; r < n; ++r) {
+            const uint32_t c = modn((int64_t)r - 2 - t, n);
+            CHK(push(l, step0 + t, REDUCE, r, IN, sl[c].offset, modn((int64_t)r - 1, n), IN, sl[c].offset, sl[c].size));
+        }
+    return HCCL_SUCCESS;
+}
+
+static int sched_allreduce_ring(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit, int with_gather)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) /* temp_all_reduce/all_reduce_ring.cc:132-140; the staged reduce-scatter does nothing (:73-76) */
+        return with_gather ? push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total) : HCCL_SUCCESS;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    CHK(HcommGfxCalcSlices(count, unit, n, sl));
+    CHK(ring_rs(l, n, sl, 0));
+    if (!with_gather) return HCCL_SUCCESS;
+    /* temp_all_gather/all_gather_ring.cc:116-121: own slice input -> output */
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, n - 1, COPY, r, OUT, sl[r].offset, r, IN, sl[r].offset, sl[r].size));
+    /* all_gather_ring.cc:143-206: round i receives slice (r-1-i) from the left neighbour's output */
+    for (uint32_t i = 0; i + 1 < n; ++i)
+        for (uint32_t r = 0; r < n; ++r) {
+            const uint32_t c = modn((int64_t)r - 1 - i, n);
+            CHK(push(l, n + i, COPY, r, OUT, sl[c].offset, modn((int64_t)r - 1, n), OUT, sl[c].offset, sl[c].size));
+        }
+    return HCCL_SUCCESS;
+}
+
+static int sched_rs_ring_standalone(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz); /* reduce_scatter_ring.cc:103-109 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    for (uint32_t i = 0; i < n; ++i) { /* reduce_scatter_ring.cc:140-157; the output holds one slice, so offset 0 */
+        sl[i].offset = (uint64_t)i * sz;
+        sl[i].size = sz;
+    }
+    CHK(ring_rs(l, n, sl, 0));
+    /* last step reduces into the input slice, then copies it to the output (reducer.cc:209-218) */
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, n - 1, COPY, r, OUT, 0, r, IN, sl[r].offset, sz));
+    return HCCL_SUCCESS;
+}
+
+static uint32_t floor_pow2(uint32_t n)
+{
+    uint32_t b = 1;
+    while ((b << 1) <= n) b <<= 1;
+    return b;
+}
+
+static uint64_t sum_sizes(const HcommGfxSlice* sl, uint32_t first, uint32_t m)
+{
+    uint64_t s = 0;
+    for (uint32_t i = 0; i < m; ++i) s += sl[first + i].size;
+    return s;
+}
+
+static int sched_allreduce_rhd(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* all_reduce_recursive_hd.cc:103-108 */
+    /* recursive_halvingdoubling_base.cc:23-37 */
+    const uint32_t block = floor_pow2(n);
+    const uint32_t part1 = (n - block) * 2;
+    uint32_t levels = 0;
+    while ((1u << (levels + 1)) <= block) ++levels;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    CHK(HcommGfxCalcSlices(count, unit, block, sl)); /* recursive_halvingdoubling_base.cc:64-94 */
+    uint32_t real[HCOMM_GFX_MAX_RANKS]; /* block rank -> rank (recursive_halvingdoubling_base.cc:39-62) */
+    for (uint32_t b = 0; b < block; ++b) real[b] = (b < part1 / 2) ? 2 * b : b + part1 / 2;
+    uint32_t step = 0;
+    if (part1 > 0) { /* fold: even ranks of part one absorb their odd neighbour (all_reduce_recursive_hd.cc:133-203) */
+        for (uint32_t r = 0; r < part1; r += 2) CHK(push(l, step, REDUCE, r, IN, 0, r + 1, IN, 0, total));
+        ++step;
+    }
+    /* halving reduce-scatter (temp_reduce_scatter/reduce_scatter_halving_doubling.cc:65-92,196-257) */
+    for (uint32_t s = 0; s < levels; ++s, ++step) {
+        const uint32_t m = 1u << (levels - 1 - s);
+        for (uint32_t b = 0; b < block; ++b) {
+            const uint32_t p = b ^ m, first = b & ~(m - 1);
+            CHK(push(l, step, REDUCE, real[b], IN, sl[first].offset, real[p], IN, sl[first].offset, sum_sizes(sl, first, m)));
+        }
+    }
+    /* reduce_scatter_halving_doubling.cc:251-254: the slice received last goes input -> output */
+    for (uint32_t b = 0; b < block; ++b)
+        CHK(push(l, step, COPY, real[b], OUT, sl[b].offset, real[b], IN, sl[b].offset, sl[b].size));
+    ++step;
+    /* doubling all-gather in the outputs (temp_all_gather/all_gather_halving_doubling.cc:42-66,164-206) */
+    for (uint32_t s = 0; s < levels; ++s, ++step) {
+        const uint32_t m = 1u << s;
+        for (uint32_t b = 0; b < block; ++b) {
+            const uint32_t p = b ^ m, first = p & ~(m - 1);
+            CHK(push(l, step, COPY, real[b], OUT, sl[first].offset, real[p], OUT, sl[first].offset, sum_sizes(sl, first, m)));
+        }
+    }
+    if (part1 > 0) { /* unfold: even -> odd, whole output (all_reduce_recursive_hd.cc:277-343) */
+        for (uint32_t r = 1; r < part1; r += 2) CHK(push(l, step, COPY, r, OUT, 0, r - 1, OUT, 0, total));
+        ++step;
+    }
+    return HCCL_SUCCESS;
+}
+
+static int sched_allreduce_mesh_oneshot(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    /* temp_all_reduce/all_reduce_mesh_oneshot.cc:78-121: out = in, then reduce the peers' copies in the
+     * order r+1, r+2, ..., r-1.  A peer's communication buffer holds a copy of its input (:96-100), which
+     * the simulation reads as in[peer] directly. */
+    const uint64_t total = count * unit;
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, 0, COPY, r, OUT, 0, r, IN, 0, total));
+    for (uint32_t k = 1; k < n; ++k)
+        for (uint32_t r = 0; r < n; ++r) CHK(push(l, k, REDUCE, r, OUT, 0, (r + k) % n, IN, 0, total));
+    return HCCL_SUCCESS;
+}
+
+static int sched_rs_mesh(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    /* temp_reduce_scatter/reduce_scatter_mesh.cc:51-128 (stream 0): round k receives slice r from rank r-k
+     * (ForwardRank, base/inc/reduce_scatter_mesh_pub.h:31-37) and reduces it into in[r][slice r]; then
+     * :199-211 copies that slice to the output. */
+    const uint64_t sz = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz);
+    for (uint32_t k = 1; k < n; ++k)
+        for (uint32_t r = 0; r < n; ++r)
+            CHK(push(l, k - 1, REDUCE, r, IN, (uint64_t)r * sz, modn((int64_t)r - k, n), IN, (uint64_t)r * sz, sz));
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, n - 1, COPY, r, OUT, 0, r, IN, (uint64_t)r * sz, sz));
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0) return HCCL_E_PARA;
+    int rc;
+    switch (alg) {
+        case HCOMM_GFX_ALG_ALLREDUCE_RING: rc = sched_allreduce_ring(l, n, count, unit, 1); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING: rc = sched_allreduce_ring(l, n, count, unit, 0); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_RHD: rc = sched_allreduce_rhd(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: rc = sched_allreduce_mesh_oneshot(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH: rc = sched_rs_mesh(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, unit); break;
+        default: rc = HCCL_E_PARA;
+    }
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxScheduleEmit(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType, HcommGfxSchedOp* ops,
+    uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule(&l, (int)alg, nRanks, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}

@@ -1,0 +1,330 @@
+/*
+ * hcomm_gfx.h - C ABI of libhcomm_gfx.so: HCOMM's local copy / local reduce data plane and the
+ * collective schedules built from it, executed by hand-written HIP kernels on one MI355X (gfx950).
+ *
+ * Plain C (C99).  Every type and enumerator that also exists in the reference keeps the reference's
+ * name and numeric value, so a caller compiled against the reference headers can bind these symbols
+ * unchanged.  Citations are paths relative to the reference tree.
+ *
+ * Three groups of entry points:
+ *   1. drop-in primitives      - same names, argument meaning and return codes as the reference;
+ *   2. HcommGfx* extensions    - k-way fused reduce, stream sync, launch log (no reference counterpart);
+ *   3. HcommGfxPlan*           - build once / run many replay of the ring, recursive halving-doubling
+ *                                and mesh schedules over N simulated ranks (N pairs of HBM buffers).
+ */
+#ifndef HCOMM_GFX_H
+#define HCOMM_GFX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------------------------------------
+ * Types shared with the reference
+ * ------------------------------------------------------------------------------------------- */
+
+/* include/hcomm_res_defs.h:26 */
+typedef int32_t HcommResult;
+
+/* include/hcomm_primitives.h:30,38 */
+#ifndef CHANNEL_HANDLE_DEFINED
+#define CHANNEL_HANDLE_DEFINED
+typedef uint64_t ChannelHandle;
+#endif
+#ifndef THREAD_HANDLE_DEFINED
+#define THREAD_HANDLE_DEFINED
+typedef uint64_t ThreadHandle;
+#endif
+
+/* include/hccl/hccl_types.h:23-51 (HcclResult); only the codes this library can return */
+enum {
+    HCCL_SUCCESS = 0,
+    HCCL_E_PARA = 1,
+    HCCL_E_PTR = 2,
+    HCCL_E_MEMORY = 3,
+    HCCL_E_INTERNAL = 4,
+    HCCL_E_NOT_SUPPORT = 5,
+    HCCL_E_NOT_FOUND = 6,
+    HCCL_E_UNAVAIL = 7,
+    HCCL_E_TIMEOUT = 9,
+    HCCL_E_RUNTIME = 15
+};
+
+/* include/hcomm_primitives.h:45-51 (identical to HcclReduceOp, include/hccl/hccl_types.h:71-77) */
+typedef enum {
+    HCOMM_REDUCE_SUM = 0,
+    HCOMM_REDUCE_PROD = 1,
+    HCOMM_REDUCE_MAX = 2,
+    HCOMM_REDUCE_MIN = 3,
+    HCOMM_REDUCE_RESERVED = 255
+} HcommReduceOp;
+
+/* include/hcomm_primitives.h:53-72 (identical to HcclDataType, include/hccl/hccl_types.h:82-101) */
+typedef enum {
+    HCOMM_DATA_TYPE_INT8 = 0,
+    HCOMM_DATA_TYPE_INT16 = 1,
+    HCOMM_DATA_TYPE_INT32 = 2,
+    HCOMM_DATA_TYPE_FP16 = 3,
+    HCOMM_DATA_TYPE_FP32 = 4,
+    HCOMM_DATA_TYPE_INT64 = 5,
+    HCOMM_DATA_TYPE_UINT64 = 6,
+    HCOMM_DATA_TYPE_UINT8 = 7,
+    HCOMM_DATA_TYPE_UINT16 = 8,
+    HCOMM_DATA_TYPE_UINT32 = 9,
+    HCOMM_DATA_TYPE_FP64 = 10,
+    HCOMM_DATA_TYPE_BFP16 = 11,
+    HCOMM_DATA_TYPE_INT128 = 12,
+    HCOMM_DATA_TYPE_HIF8 = 14,
+    HCOMM_DATA_TYPE_FP8E4M3 = 15,
+    HCOMM_DATA_TYPE_FP8E5M2 = 16,
+    HCOMM_DATA_TYPE_FP8E8M0 = 17,
+    HCOMM_DATA_TYPE_RESERVED = 255
+} HcommDataType;
+
+/* include/hcomm_res_defs.h:106-114 */
+typedef enum {
+    COMM_ENGINE_RESERVED = -1,
+    COMM_ENGINE_CPU = 0,
+    COMM_ENGINE_CPU_TS = 1,
+    COMM_ENGINE_AICPU = 2,
+    COMM_ENGINE_AICPU_TS = 3,
+    COMM_ENGINE_AIV = 4,
+    COMM_ENGINE_CCU = 5
+} CommEngine;
+
+/* ---------------------------------------------------------------------------------------------
+ * 1. Drop-in primitives
+ * ------------------------------------------------------------------------------------------- */
+
+/*
+ * dst[0..len) = src[0..len) on the thread's stream.  Replaces include/hcomm_primitives.h:152
+ * (host adapter src/base_comm/primitives/api_c_adpt/cpu_primitives_c_adpt.cc:58-86).
+ * Check order: dst NULL -> HCCL_E_PTR, src NULL -> HCCL_E_PTR, thread 0 -> HCCL_E_PTR.
+ * len == 0 or src == dst succeed without doing anything
+ * (src/legacy/ascend910/platform/task/dispatcher.cc:495-498).  len may exceed 4 GiB.
+ * Asynchronous: returns once the work is enqueued (or, in batch mode, recorded).
+ */
+int32_t HcommLocalCopyOnThread(ThreadHandle thread, void* dst, const void* src, uint64_t len);
+
+/*
+ * dst[i] = dst[i] (op) src[i] for i < count, result stored in the element type.  Replaces
+ * include/hcomm_primitives.h:164-165 (host adapter cpu_primitives_c_adpt.cc:88-130).
+ * Check order: dst NULL -> HCCL_E_PTR, src NULL -> HCCL_E_PTR, unsupported dataType/reduceOp ->
+ * HCCL_E_PARA, thread 0 -> HCCL_E_PTR.  Supported exactly as the reference
+ * (cpu_primitives_c_adpt.cc:31-39): {INT8, INT16, INT32, FP16, FP32, BFP16} x {SUM, MAX, MIN};
+ * PROD is rejected here (it exists only at collective level in the reference) unless the
+ * environment variable HCOMM_GFX_ALLOW_PROD=1 is set when the library is loaded.
+ * count == 0 succeeds without doing anything (dispatcher.cc:719-722).  count may exceed 2^32.
+ */
+int32_t HcommLocalReduceOnThread(
+    ThreadHandle thread, void* dst, const void* src, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp);
+
+/*
+ * Thread = one in-order execution queue (a HIP stream) plus notifyNum local notifies.
+ * Replaces include/hcomm_res.h:57-60 (src/base_comm/primitives/api_c_adpt/hcomm_thread_c_adpt.cc:38-86,157).
+ * threads NULL or notifyNumPerThread NULL -> HCCL_E_PTR; threadNum == 0 -> HCCL_E_PARA.
+ * Only notifyNumPerThread[0] is used, as in the reference.  Every engine value maps to the GPU.
+ */
+HcommResult
+HcommThreadAlloc(CommEngine engine, uint32_t threadNum, const uint32_t* notifyNumPerThread, ThreadHandle* threads);
+HcommResult HcommThreadFree(const ThreadHandle* threads, uint32_t threadNum);
+
+/*
+ * Bind a thread to a caller-owned stream (a hipStream_t passed as void*; NULL = the default stream).
+ * Replaces hcomm_thread_c_adpt.cc:164-187 (declared at src/base_comm/primitives/api_c_adpt/hcomm_c_adpt.h:108,113).
+ * The stream is never destroyed by the library.
+ */
+HcommResult HcommThreadAllocWithStream(CommEngine engine, void* stream, uint32_t notifyNum, ThreadHandle* thread);
+HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t threadNum);
+
+/*
+ * Cross-thread ordering.  Replaces include/hcomm_primitives.h:181,191.  Record marks, on dstThread's
+ * notify slot dstNotifyIdx, the point `thread` has reached; Wait makes `thread` wait for the most recent
+ * record on its own slot notifyIdx.  timeOut is accepted and ignored (stream-order wait).
+ */
+int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
+int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);
+
+/* Device memory.  Replaces include/hcomm_res.h:69-71.  ptr NULL -> HCCL_E_PTR, size 0 -> HCCL_E_PARA. */
+HcommResult HcommMemAlloc(void** ptr, size_t size);
+HcommResult HcommMemFree(void* ptr);
+
+/*
+ * Batch mode.  Replaces include/hcomm_primitives.h:498,506 (src/base_comm/primitives/launch_context.cc:139-174).
+ * Between Start and End, on the calling host thread, primitives only record.  End submits everything
+ * recorded, per ThreadHandle in call order, after merging runs of mutually independent operations of the
+ * same kind / type / op into single kernel launches (one launch for all N ranks of a collective step).
+ * Two operations are independent when neither writes memory the other reads or writes.
+ * Start while already batching, or End without Start -> HCCL_E_PARA.  batchTag may be NULL.
+ */
+int32_t HcommBatchModeStart(const char* batchTag);
+int32_t HcommBatchModeEnd(const char* batchTag);
+
+/* ---------------------------------------------------------------------------------------------
+ * 2. Extensions (no reference counterpart)
+ * ------------------------------------------------------------------------------------------- */
+
+#define HCOMM_GFX_MAX_RANKS 32u /* most simulated ranks per plan / most inputs of a fused k-way reduce */
+
+/* Block the host until everything enqueued on the thread has finished. */
+int32_t HcommGfxThreadSynchronize(ThreadHandle thread);
+
+/*
+ * Fused k-way reduce: dst[i] = (..((srcs[0][i] (op) srcs[1][i]) (op) srcs[2][i]) .. (op) srcs[k-1][i]),
+ * left to right with the running value in the "dst" role of the op, rounded to the element type after
+ * every step - i.e. the result of one copy followed by k-1 HcommLocalReduceOnThread calls
+ * (the chain of src/legacy/ascend910/algorithm/base/alg_template/temp_all_reduce/all_reduce_mesh_oneshot.cc:94-119)
+ * in a single pass that reads each input once.  1 <= k <= HCOMM_GFX_MAX_RANKS.  dst may alias srcs[0].
+ * PROD is allowed for the types the reference allows at collective level
+ * (src/legacy/ascend910/framework/common/src/param_check.cc:327-343): INT8, INT32, FP16, FP32; and BFP16.
+ */
+int32_t HcommGfxReduceKOnThread(
+    ThreadHandle thread, void* dst, const void* const* srcs, uint32_t k, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp);
+
+/*
+ * A recorder thread never touches the GPU: every launch it would make is appended to a log instead.
+ * It exists so that argument checking, batching and schedule lowering can be tested on a host without a
+ * GPU (the reference's unit tests mock the engine the same way,
+ * test/ut/framework/communicator/impl/independent_op/data_api/ut_aicpu_ts_HcommLocalReduceOnThread.cc:26-30).
+ */
+HcommResult HcommGfxRecorderThreadAlloc(ThreadHandle* thread);
+
+typedef struct {
+    uint32_t kind;   /* HcommGfxKernelKind */
+    uint32_t dtype;  /* HcommDataType, 255 for copies */
+    uint32_t op;     /* HcommReduceOp, 255 for copies */
+    uint32_t nseg;   /* segments merged into this launch */
+    uint64_t bytes;  /* sum of segment output bytes */
+    uint64_t blocks; /* grid size */
+} HcommGfxLaunchRecord;
+
+typedef enum {
+    HCOMM_GFX_KERNEL_COPY = 0,     /* batched vector copy */
+    HCOMM_GFX_KERNEL_REDUCE2 = 1,  /* batched dst = dst (op) src */
+    HCOMM_GFX_KERNEL_CHAIN = 2,    /* k inputs folded in sequence, optional partial stores, fan-out stores */
+    HCOMM_GFX_KERNEL_TREE = 3,     /* k = 2^j inputs folded as a binary tree with partial stores, fan-out */
+    HCOMM_GFX_KERNEL_BYTEWISE = 4  /* element-at-a-time fallback for pointers not 16-byte aligned */
+} HcommGfxKernelKind;
+
+/* Copy up to `cap` records of the thread's launch log into `out`; *n receives the total logged. */
+int32_t HcommGfxLaunchLogRead(ThreadHandle thread, HcommGfxLaunchRecord* out, uint32_t cap, uint32_t* n);
+int32_t HcommGfxLaunchLogClear(ThreadHandle thread);
+
+/* ---------------------------------------------------------------------------------------------
+ * 3. Collective schedules over N simulated ranks
+ * ------------------------------------------------------------------------------------------- */
+
+typedef enum {
+    /* AllReduceRing: temp_all_reduce/all_reduce_ring.cc:26-62 = ring reduce-scatter + ring all-gather */
+    HCOMM_GFX_ALG_ALLREDUCE_RING = 0,
+    /* reduce-scatter stage of AllReduceRing (RunAsyncStaged(RUN_REDUCE_SCATTER), all_reduce_ring.cc:82-92):
+       in place in the input buffers, S1 slice table; rank r ends up owning slice r in in[r] */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_RING = 1,
+    /* AllReduceRecursiveHalvingDoubling: temp_all_reduce/all_reduce_recursive_hd.cc:28-50 */
+    HCOMM_GFX_ALG_ALLREDUCE_RHD = 2,
+    /* AllReduceMeshDirectOneshot: temp_all_reduce/all_reduce_mesh_oneshot.cc:78-121 */
+    HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT = 3,
+    /* ReduceScatterMesh: temp_reduce_scatter/reduce_scatter_mesh.cc:51-215; count = per-rank OUTPUT count */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_MESH = 4,
+    /* stand-alone ReduceScatterRing: temp_reduce_scatter/reduce_scatter_ring.cc:96-180; count = per-rank
+       OUTPUT count, input holds N*count, result written to out[r][0..count) */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE = 5
+} HcommGfxAlgorithm;
+
+typedef enum {
+    /* one kernel launch per schedule step, all ranks of the step in that launch; every reduce is a
+       two-input dst = dst (op) src exactly as the reference emits it */
+    HCOMM_GFX_LOWER_STEPWISE = 0,
+    /* steps whose data dependences are element-wise are folded into k-way kernels that read every input
+       once and still store every intermediate value the step-wise replay stores, so the final contents
+       of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE */
+    HCOMM_GFX_LOWER_FUSED = 1
+} HcommGfxLowering;
+
+typedef struct {
+    uint64_t offset; /* bytes from the buffer base */
+    uint64_t size;   /* bytes */
+} HcommGfxSlice;     /* struct Slice, base/alg_template/template_v1_utils.h:50-53 */
+
+/*
+ * Slice table of the allreduce templates: total = count * unit; per = roundup(ceil(total / n), 128);
+ * slice i takes min(per, what is left) (temp_all_reduce/all_reduce_ring.cc:142-153,
+ * alg_template_base.cc:787-820, recursive_halvingdoubling_base.cc:64-94).  Writes n entries.
+ * unitSize 0, n 0 or slices NULL -> error.
+ */
+int32_t HcommGfxCalcSlices(uint64_t count, uint32_t unitSize, uint32_t n, HcommGfxSlice* slices);
+
+/* Element size in bytes (SIZE_TABLE, pkg_inc/legacy/hccl/dtype_common.h:18-36); 0 for unknown values. */
+uint32_t HcommGfxDataTypeSize(HcommDataType dataType);
+
+typedef struct HcommGfxPlan HcommGfxPlan;
+
+/*
+ * Build the launch list for one collective over nRanks simulated ranks.
+ *   in[r], out[r] : rank r's input and output buffer (device pointers, 128-byte aligned, not overlapping
+ *                   each other or any other rank's buffers).  Algorithms that run in place ignore out.
+ *   count         : elements per rank (see the algorithm's note for its exact meaning).
+ * Dtypes: INT8, INT16, INT32, FP16, FP32, BFP16.  Ops: SUM, MAX, MIN, and PROD where the reference allows it
+ * at collective level (param_check.cc:327-343: not INT16) plus BFP16.
+ * Returns HCCL_SUCCESS and *plan, or an error code and *plan = NULL.  nRanks in [1, HCOMM_GFX_MAX_RANKS].
+ * Building a plan allocates nothing on the device and launches nothing.
+ */
+int32_t HcommGfxPlanCreate(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+
+/* Enqueue every launch of the plan on the thread, in order.  May be called any number of times. */
+int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread);
+
+/* Enqueue launches [first, first + n) only (used to time one phase of a plan). */
+int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n);
+
+int32_t HcommGfxPlanDestroy(HcommGfxPlan* plan);
+
+typedef struct {
+    uint32_t launches;        /* kernel launches per run */
+    uint32_t steps;           /* schedule steps of the reference algorithm */
+    uint64_t algorithmicBytes; /* sum over all two-input steps of 3*b (reduce) or 2*b (copy) */
+    uint64_t movedBytes;      /* bytes the launches of this lowering actually read + write */
+} HcommGfxPlanInfo;
+
+int32_t HcommGfxPlanGetInfo(const HcommGfxPlan* plan, HcommGfxPlanInfo* info);
+
+/* Per-launch description (same record as the launch log), i in [0, launches). */
+int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaunchRecord* rec);
+
+/*
+ * The schedule as the reference's templates emit it, one two-input operation per record, for inspection
+ * and for checking a plan against an independent replay.
+ */
+typedef struct {
+    uint32_t step;    /* schedule step (ranks act in parallel within a step) */
+    uint32_t kind;    /* 0 = copy, 1 = reduce */
+    uint32_t rank;    /* rank that executes the operation (owner of dst) */
+    uint32_t dstBuf;  /* 0 = in[rank], 1 = out[rank] */
+    uint32_t srcRank; /* rank whose buffer is read */
+    uint32_t srcBuf;  /* 0 = in[srcRank], 1 = out[srcRank] */
+    uint64_t dstOff;  /* bytes */
+    uint64_t srcOff;  /* bytes */
+    uint64_t bytes;
+} HcommGfxSchedOp;
+
+/*
+ * Emit the op list of an algorithm without any pointers.  Writes up to cap records; *n receives the total.
+ * Records are ordered by step, then by rank.
+ */
+int32_t HcommGfxScheduleEmit(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType, HcommGfxSchedOp* ops,
+    uint64_t cap, uint64_t* n);
+
+/* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */
+const char* HcommGfxVersion(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCOMM_GFX_H */

@@ -1,0 +1,179 @@
+"""ctypes loader for the CPU oracle (oracle/hcomm_oracle.c) and the compiled reference code (oracle/_ref).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of
+bench.py - never by the hcomm_amd package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liboracle.so")
+REF_PATH = os.path.join(HERE, "_ref", "libhcomm_ref.so")
+
+SUM, PROD, MAX, MIN = 0, 1, 2, 3
+I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
+ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
+    ALG_RS_RING_STANDALONE = range(6)
+
+# storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
+NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
+
+
+def build(force=False):
+    """Compile liboracle.so (and oracle/_ref when the reference tree is present)."""
+    cmd = ["make", "-C", HERE]
+    if force:
+        cmd.insert(1, "-B")
+    subprocess.run(cmd, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+
+
+class OrcOp(C.Structure):
+    _fields_ = [("step", C.c_uint32), ("kind", C.c_uint32), ("rank", C.c_uint32), ("dst_buf", C.c_uint32),
+                ("src_rank", C.c_uint32), ("src_buf", C.c_uint32), ("dst_off", C.c_uint64), ("src_off", C.c_uint64),
+                ("bytes", C.c_uint64)]
+
+    def astuple(self):
+        return (self.step, self.kind, self.rank, self.dst_buf, self.dst_off, self.src_rank, self.src_buf,
+                self.src_off, self.bytes)
+
+
+class OrcSlice(C.Structure):
+    _fields_ = [("offset", C.c_uint64), ("size", C.c_uint64)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = C.CDLL(LIB_PATH)
+        L.orc_set_threads.argtypes = [C.c_int]
+        L.orc_get_threads.restype = C.c_int
+        L.orc_f16_to_f32.restype = C.c_float
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [C.c_float]
+        L.orc_bf16_to_f32.restype = C.c_float
+        L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_bf16.restype = C.c_uint16
+        L.orc_f32_to_bf16.argtypes = [C.c_float]
+        L.orc_dtype_size.restype = C.c_uint32
+        L.orc_dtype_size.argtypes = [C.c_int]
+        L.orc_reduce.restype = C.c_int
+        L.orc_reduce.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int]
+        L.orc_copy.restype = None
+        L.orc_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64]
+        L.orc_slices_ring.restype = None
+        L.orc_slices_ring.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.POINTER(OrcSlice)]
+        L.orc_slices_rhd.restype = None
+        L.orc_slices_rhd.argtypes = [C.c_uint64, C.c_uint32, C.POINTER(OrcSlice)]
+        L.orc_trace.restype = C.c_int64
+        L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
+        L.orc_run.restype = C.c_int
+        L.orc_run.argtypes = [C.c_int, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_uint64, C.c_int,
+                              C.c_int]
+        L.orc_algorithmic_bytes.restype = C.c_int64
+        L.orc_algorithmic_bytes.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int]
+        L.orc_reduce_k.restype = C.c_int
+        L.orc_reduce_k.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.c_uint64, C.c_int, C.c_int]
+        _lib = L
+    return _lib
+
+
+def have_ref():
+    return os.path.exists(REF_PATH)
+
+
+_ref = None
+
+
+def ref():
+    """The reference's own CPU reduce code, compiled from its sources (None when it was never built)."""
+    global _ref
+    if _ref is None and have_ref():
+        R = C.CDLL(REF_PATH)
+        for name in ("ref_mem_reduce_sum", "ref_mem_reduce_min", "ref_mem_reduce_max"):
+            f = getattr(R, name)
+            f.restype = None
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
+        R.ref_fp16_from_float.restype = C.c_uint16
+        R.ref_fp16_from_float.argtypes = [C.c_float]
+        R.ref_fp16_to_float.restype = C.c_float
+        R.ref_fp16_to_float.argtypes = [C.c_uint16]
+        for name in ("ref_fp16_add", "ref_fp16_mul"):
+            f = getattr(R, name)
+            f.restype = C.c_uint16
+            f.argtypes = [C.c_uint16, C.c_uint16]
+        for name in ("ref_fp16_gt", "ref_fp16_lt"):
+            f = getattr(R, name)
+            f.restype = C.c_int
+            f.argtypes = [C.c_uint16, C.c_uint16]
+        R.ref_fp16_from_float_n.restype = None
+        R.ref_fp16_from_float_n.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64]
+        R.ref_fp16_to_float_n.restype = None
+        R.ref_fp16_to_float_n.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64]
+        _ref = R
+    return _ref
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def reduce(dst, src, dtype, op):
+    """dst = dst (op) src in place on numpy arrays holding the storage type."""
+    assert dst.flags.c_contiguous and src.flags.c_contiguous and dst.size == src.size
+    rc = lib().orc_reduce(_ptr(dst), _ptr(src), dst.size, dtype, op)
+    if rc:
+        raise ValueError("orc_reduce rc=%d" % rc)
+    return dst
+
+
+def reduce_k(srcs, dtype, op):
+    dst = np.empty_like(srcs[0])
+    arr = (C.c_void_p * len(srcs))(*[s.ctypes.data for s in srcs])
+    rc = lib().orc_reduce_k(_ptr(dst), arr, len(srcs), dst.size, dtype, op)
+    if rc:
+        raise ValueError("orc_reduce_k rc=%d" % rc)
+    return dst
+
+
+def slices_ring(count, unit, n):
+    sl = (OrcSlice * n)()
+    lib().orc_slices_ring(count, unit, n, sl)
+    return [(s.offset, s.size) for s in sl]
+
+
+def slices_rhd(data_bytes, block):
+    sl = (OrcSlice * block)()
+    lib().orc_slices_rhd(data_bytes, block, sl)
+    return [(s.offset, s.size) for s in sl]
+
+
+def trace(alg, n, count, dtype):
+    total = lib().orc_trace(alg, n, count, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace(alg, n, count, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run(alg, ins, outs, count, dtype, op):
+    """Execute a collective in place on lists of numpy arrays (one per rank)."""
+    n = len(ins)
+    a = (C.c_void_p * n)(*[x.ctypes.data for x in ins])
+    b = (C.c_void_p * n)(*[x.ctypes.data for x in outs])
+    rc = lib().orc_run(alg, n, a, b, count, dtype, op)
+    if rc:
+        raise ValueError("orc_run rc=%d" % rc)
+
+
+def algorithmic_bytes(alg, n, count, dtype):
+    return lib().orc_algorithmic_bytes(alg, n, count, dtype)

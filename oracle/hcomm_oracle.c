@@ -1,0 +1,640 @@
+/*
+ * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics and of the ring, recursive
+ * halving-doubling and mesh schedules, used ONLY to check libhcomm_gfx.so.
+ *
+ * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
+ * suite, the smoke check and the CPU-baseline leg of the benchmark do.
+ *
+ * Every function cites the reference file:line it restates (paths relative to the reference tree; "tpl/"
+ * abbreviates src/legacy/ascend910/algorithm/base/alg_template/).  The schedules are written the way the
+ * reference writes them - one program per rank, with the running slice indices of the original loops -
+ * and then executed in lock step, which is deliberately a different formulation from the closed-form,
+ * step-major generator inside the product.
+ *
+ * Pinning status (what fixes each function besides its own formula; see tests/test_oracle_*.py):
+ *   integer SUM/PROD/MAX/MIN ........ exhaustive int8 pairs + numpy wrap-around arithmetic; pinned
+ *   fp32 ops ........................ one IEEE-754 operation, checked against numpy float32; pinned
+ *   fp16 conversions and ops ........ exhaustive against numpy float16 and against the reference's own
+ *                                     FP16 class compiled from its sources (oracle/_ref); pinned
+ *   int8/16/32, fp16, fp32 loops .... against the reference's MemReduceSum/Min/Max compiled from its
+ *                                     sources (oracle/_ref); pinned
+ *   bf16 conversions and ops ........ PARITY UNPINNED against the reference: it has no bf16 arithmetic on
+ *                                     any CPU path (hccl_task_reduce_process.cc:57-84 has no BFP16 case).
+ *                                     Defined by analogy with fp16 (fp32 operation + round to nearest even)
+ *                                     and checked against torch.bfloat16 only.
+ *   NaN payloads, int overflow ...... of the real SDMA / vector engines: PARITY UNPINNED (hardware
+ *                                     behaviour outside the reference tree); integers wrap as in the
+ *                                     reference's CPU witnesses.
+ *   slice tables .................... the reference's hand-computable values for the benchmark configs +
+ *                                     invariants; pinned
+ *   schedules ....................... hand-derived step chains for N = 4 (tests/golden), the reference's
+ *                                     own acceptance rule (every output range receives every rank exactly
+ *                                     once, allreduce_semantics_checker.cc:59-96), non-associative fp
+ *                                     inputs, and agreement with the product's independent generator; pinned
+ */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_MAX_RANKS 32
+
+enum { ORC_SUM = 0, ORC_PROD = 1, ORC_MAX = 2, ORC_MIN = 3 };
+enum { ORC_I8 = 0, ORC_I16 = 1, ORC_I32 = 2, ORC_F16 = 3, ORC_F32 = 4, ORC_BF16 = 11 };
+
+static int g_threads = 1;
+
+void orc_set_threads(int n) { g_threads = n > 0 ? n : 1; }
+int orc_get_threads(void) { return g_threads; }
+
+/* ---- 16-bit float conversions --------------------------------------------------------------------- */
+
+static uint32_t f2u(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static float u2f(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* binary16 -> binary32, exact (restates half_to_float, ccu_fp16.h:102-111) */
+float orc_f16_to_f32(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    if (e == 0x1f) return u2f(sign | 0x7f800000u | (m << 13)); /* inf / NaN */
+    if (e == 0) {
+        if (m == 0) return u2f(sign);
+        /* subnormal: renormalise */
+        int shift = 0;
+        while (!(m & 0x400u)) {
+            m <<= 1;
+            ++shift;
+        }
+        m &= 0x3ffu;
+        e = (uint32_t)(1 - shift);
+        return u2f(sign | ((e + 112u) << 23) | (m << 13));
+    }
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* binary32 -> binary16, round to nearest even; NaN -> sign | 0x7e00 (restates float_to_half, ccu_fp16.h:114-135) */
+uint16_t orc_f32_to_f16(float f)
+{
+    const uint32_t x = f2u(f);
+    const uint32_t sign = (x >> 16) & 0x8000u, ax = x & 0x7fffffffu;
+    if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+    if (ax >= 0x47800000u) return (uint16_t)(sign | 0x7c00u); /* >= 65536 or inf */
+    const int32_t e = (int32_t)(ax >> 23) - 127 + 15;
+    uint32_t m = ax & 0x7fffffu;
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign; /* below half of the smallest subnormal */
+        m |= 0x800000u;
+        const uint32_t shift = (uint32_t)(14 - e);
+        uint32_t hm = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (hm & 1u))) ++hm;
+        return (uint16_t)(sign | hm);
+    }
+    uint32_t hv = ((uint32_t)e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (hv & 1u))) ++hv; /* a carry into the exponent is the right answer */
+    return (uint16_t)(sign | hv);
+}
+
+/* bfloat16: the upper half of a binary32.  No reference witness; by analogy with fp16. */
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+uint16_t orc_f32_to_bf16(float f)
+{
+    const uint32_t x = f2u(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)(((x >> 16) & 0x8000u) | 0x7fc0u);
+    return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+
+/* ---- element operation: returns d (op) s with d in the dst role ------------------------------------------
+ * SUM a+b, PROD a*b (reduce_op, test/ut/stub/llt_hccl_stub.cc:4077-4101; AicpuReduceTemplate,
+ * src/legacy/ascend950/service/collective/instruction/instruction.cc:472-493);
+ * MAX (src > dst) ? src : dst, MIN (src < dst) ? src : dst - the stub is called with src1 = src, src2 = dst
+ * (llt_hccl_stub.cc:2374), and MemReduceMax/MinTemplate overwrite dst only when the comparison holds
+ * (test/hccl_vm/src/plugin/runner/runner_utils/hccl_task_reduce_process.cc:30-55), so dst survives ties
+ * and unordered comparisons.  Integers wrap (native C++ arithmetic on the typed value in both witnesses). */
+
+#define INT_OP(T, U)                                                  \
+    static T op_##T(T d, T s, int op)                                 \
+    {                                                                 \
+        switch (op) {                                                 \
+            case ORC_SUM: return (T)(U)((U)d + (U)s);                 \
+            case ORC_PROD: return (T)(U)((U)d * (U)s);                \
+            case ORC_MAX: return (s > d) ? s : d;                     \
+            default: return (s < d) ? s : d;                          \
+        }                                                             \
+    }
+INT_OP(int8_t, uint8_t)
+INT_OP(int16_t, uint16_t)
+INT_OP(int32_t, uint32_t)
+
+static float op_f32(float d, float s, int op)
+{
+    switch (op) {
+        case ORC_SUM: return d + s;
+        case ORC_PROD: return d * s;
+        case ORC_MAX: return (s > d) ? s : d;
+        default: return (s < d) ? s : d;
+    }
+}
+
+/* fp16: widen both, operate in fp32, round back (FP16::operator+=, ccu_fp16.h:60-66); MAX/MIN compare the
+ * widened values and move the raw 16 bits (FP16::operator>, :69-74 with MemReduceMaxTemplate) */
+static uint16_t op_f16(uint16_t d, uint16_t s, int op)
+{
+    const float fd = orc_f16_to_f32(d), fs = orc_f16_to_f32(s);
+    switch (op) {
+        case ORC_SUM: return orc_f32_to_f16(fd + fs);
+        case ORC_PROD: return orc_f32_to_f16(fd * fs);
+        case ORC_MAX: return (fs > fd) ? s : d;
+        default: return (fs < fd) ? s : d;
+    }
+}
+
+static uint16_t op_bf16(uint16_t d, uint16_t s, int op)
+{
+    const float fd = orc_bf16_to_f32(d), fs = orc_bf16_to_f32(s);
+    switch (op) {
+        case ORC_SUM: return orc_f32_to_bf16(fd + fs);
+        case ORC_PROD: return orc_f32_to_bf16(fd * fs);
+        case ORC_MAX: return (fs > fd) ? s : d;
+        default: return (fs < fd) ? s : d;
+    }
+}
+
+uint32_t orc_dtype_size(int dtype)
+{
+    /* SIZE_TABLE, pkg_inc/legacy/hccl/dtype_common.h:18-36 */
+    static const uint32_t table[18] = {1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1};
+    return (dtype >= 0 && dtype < 18) ? table[dtype] : 0;
+}
+
+/* dst[i] = dst[i] (op) src[i], i < count (HcommLocalReduceOnThread, include/hcomm_primitives.h:164-165;
+ * loop shape of vector_reduce, llt_hccl_stub.cc:4159-4201).  Returns 0, or -1 for an unsupported type. */
+int orc_reduce(void* dst, const void* src, uint64_t count, int dtype, int op)
+{
+    if (op < ORC_SUM || op > ORC_MIN) return -1;
+    const int nt = (count >= (1u << 16)) ? g_threads : 1;
+    (void)nt;
+    int64_t i;
+    const int64_t n = (int64_t)count;
+    switch (dtype) {
+        case ORC_I8: {
+            int8_t* d = (int8_t*)dst;
+            const int8_t* s = (const int8_t*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_int8_t(d[i], s[i], op);
+            return 0;
+        }
+        case ORC_I16: {
+            int16_t* d = (int16_t*)dst;
+            const int16_t* s = (const int16_t*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_int16_t(d[i], s[i], op);
+            return 0;
+        }
+        case ORC_I32: {
+            int32_t* d = (int32_t*)dst;
+            const int32_t* s = (const int32_t*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_int32_t(d[i], s[i], op);
+            return 0;
+        }
+        case ORC_F32: {
+            float* d = (float*)dst;
+            const float* s = (const float*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_f32(d[i], s[i], op);
+            return 0;
+        }
+        case ORC_F16: {
+            uint16_t* d = (uint16_t*)dst;
+            const uint16_t* s = (const uint16_t*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_f16(d[i], s[i], op);
+            return 0;
+        }
+        case ORC_BF16: {
+            uint16_t* d = (uint16_t*)dst;
+            const uint16_t* s = (const uint16_t*)src;
+#pragma omp parallel for num_threads(nt) schedule(static)
+            for (i = 0; i < n; ++i) d[i] = op_bf16(d[i], s[i], op);
+            return 0;
+        }
+        default: return -1;
+    }
+}
+
+/* dst[0..len) = src[0..len); nothing when len == 0 or src == dst (HcommLocalCopyOnThread,
+ * include/hcomm_primitives.h:152; src/legacy/ascend910/platform/task/dispatcher.cc:495-498) */
+void orc_copy(void* dst, const void* src, uint64_t len)
+{
+    if (len == 0 || dst == src) return;
+    const int nt = (len >= (1u << 20)) ? g_threads : 1;
+    if (nt == 1) {
+        memmove(dst, src, len);
+        return;
+    }
+    const uint64_t chunk = (len + (uint64_t)nt - 1) / (uint64_t)nt;
+    int t;
+#pragma omp parallel for num_threads(nt) schedule(static)
+    for (t = 0; t < nt; ++t) {
+        const uint64_t b = (uint64_t)t * chunk;
+        if (b < len) memcpy((char*)dst + b, (const char*)src + b, (len - b < chunk) ? len - b : chunk);
+    }
+}
+
+/* ---- slice tables ----------------------------------------------------------------------------------- */
+
+typedef struct {
+    uint64_t offset, size;
+} OrcSlice;
+
+/* AllReduceRing::PrepareRunAsync, tpl/temp_all_reduce/all_reduce_ring.cc:142-153 (same arithmetic as
+ * ExecutorBase::PrepareSliceData, tpl/alg_template_base.cc:787-820) */
+void orc_slices_ring(uint64_t count, uint32_t unit, uint32_t n, OrcSlice* sl)
+{
+    const uint64_t total = count * unit;
+    const uint64_t calc = (total + (n - 1)) / n;
+    /* RoundUpWithDivisor(value, 128): value == 0 gives 128 (tpl/alg_template_base_pub.h:609-616) */
+    const uint64_t aligned = (calc == 0) ? 128 : ((calc + 127) / 128) * 128;
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < n; ++i) {
+        sl[i].size = (residue > aligned) ? aligned : residue;
+        sl[i].offset = total - residue;
+        residue -= sl[i].size;
+    }
+}
+
+/* RecursiveHalvingDoublingBase::CalculateSlices, tpl/recursive_halvingdoubling_base.cc:64-94 */
+void orc_slices_rhd(uint64_t data_bytes, uint32_t block, OrcSlice* sl)
+{
+    uint64_t per = data_bytes / block;
+    if (data_bytes % block != 0) per++;
+    per = ((per + 127) / 128) * 128;
+    uint64_t left = data_bytes;
+    uint32_t i = 0;
+    while (left > 0) {
+        sl[i].size = per < left ? per : left;
+        sl[i].offset = data_bytes - left;
+        left -= sl[i].size;
+        i++;
+    }
+    while (i < block) {
+        sl[i].offset = data_bytes;
+        sl[i].size = 0;
+        i++;
+    }
+}
+
+/* ---- schedules as per-rank programs ------------------------------------------------------------------ */
+
+typedef struct {
+    uint32_t step;
+    uint32_t kind; /* 0 copy, 1 reduce */
+    uint32_t rank;
+    uint32_t dst_buf; /* 0 in, 1 out */
+    uint32_t src_rank;
+    uint32_t src_buf;
+    uint64_t dst_off, src_off, bytes;
+} OrcOp;
+
+typedef struct {
+    OrcOp* ops;
+    uint64_t n, cap;
+    int oom;
+} OrcTrace;
+
+static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint32_t dst_buf, uint64_t dst_off,
+                 uint32_t src_rank, uint32_t src_buf, uint64_t src_off, uint64_t bytes)
+{
+    if (bytes == 0) return; /* a zero-length task does nothing (dispatcher.cc:495-498, 719-722) */
+    if (t->n == t->cap) {
+        uint64_t cap = t->cap ? t->cap * 2 : 256;
+        OrcOp* p = (OrcOp*)realloc(t->ops, cap * sizeof(OrcOp));
+        if (!p) {
+            t->oom = 1;
+            return;
+        }
+        t->ops = p;
+        t->cap = cap;
+    }
+    OrcOp* o = &t->ops[t->n++];
+    o->step = step;
+    o->kind = kind;
+    o->rank = rank;
+    o->dst_buf = dst_buf;
+    o->src_rank = src_rank;
+    o->src_buf = src_buf;
+    o->dst_off = dst_off;
+    o->src_off = src_off;
+    o->bytes = bytes;
+}
+
+enum { B_IN = 0, B_OUT = 1, K_COPY = 0, K_REDUCE = 1 };
+
+/* ReduceScatterRing::RunReduceScatter for one rank, tpl/temp_reduce_scatter/reduce_scatter_ring.cc:182-312.
+ * `out_sl` NULL: the allreduce case, where the template's output memory IS the input memory
+ * (all_reduce_ring.cc:186-187) so the last step reduces in place; otherwise the stand-alone case, where
+ * the inline-reduce branch reduces into the input slice and then copies it to the output
+ * (tpl/component/reducer.cc:199-218). */
+static void prog_ring_rs(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, const OrcSlice* out_sl)
+{
+    const uint32_t left = (rank + n - 1) % n;        /* ringPrevRank, :121 */
+    uint32_t rx = (rank + n - 2) % n;                /* rxSliceIndex, :207 */
+    uint32_t step = 0;
+    for (uint32_t i = 0; i < n - 2; i++) {           /* :232 */
+        emit(t, step++, K_REDUCE, rank, B_IN, sl[rx].offset, left, B_IN, sl[rx].offset, sl[rx].size); /* :245, RunVectorDestRducer :44-62 */
+        rx = (rx + n - 1) % n;                       /* :260 */
+    }
+    /* final receive: slice index == rank, :288-304 */
+    emit(t, step++, K_REDUCE, rank, B_IN, sl[rank].offset, left, B_IN, sl[rank].offset, sl[rank].size);
+    if (out_sl) emit(t, step, K_COPY, rank, B_OUT, out_sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size);
+}
+
+/* AllGatherRing::RunAsync + RunAllGather for one rank, tpl/temp_all_gather/all_gather_ring.cc:116-121,143-206 */
+static void prog_ring_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t step)
+{
+    const uint32_t left = (rank + n - 1) % n;
+    emit(t, step++, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size); /* :116-121 */
+    uint32_t rx = (rank + n - 1) % n; /* ForwordRank(rank, n, 1), :152 */
+    for (uint32_t i = 0; i < n - 1; i++) {
+        emit(t, step++, K_COPY, rank, B_OUT, sl[rx].offset, left, B_OUT, sl[rx].offset, sl[rx].size); /* RxVector :34-45 */
+        rx = (rx + n - 1) % n; /* :196 */
+    }
+}
+
+static void prog_allreduce_ring(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit, int gather)
+{
+    if (n == 1) { /* all_reduce_ring.cc:132-140; staged reduce-scatter: nothing (:73-76) */
+        if (gather) emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, count * unit);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS];
+    orc_slices_ring(count, unit, n, sl);
+    prog_ring_rs(t, rank, n, sl, NULL);
+    if (gather) prog_ring_ag(t, rank, n, sl, n - 1);
+}
+
+static void prog_rs_ring_standalone(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) { /* reduce_scatter_ring.cc:103-109 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, sz);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS], osl[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) { /* :140-157; input larger than output -> output offset 0 */
+        sl[i].size = sz;
+        sl[i].offset = (uint64_t)i * sz;
+        osl[i].size = sz;
+        osl[i].offset = 0;
+    }
+    prog_ring_rs(t, rank, n, sl, osl);
+}
+
+/* AllReduceRecursiveHalvingDoubling for one rank, tpl/temp_all_reduce/all_reduce_recursive_hd.cc:28-50 */
+static void prog_allreduce_rhd(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) { /* :103-108 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
+        return;
+    }
+    /* CalcPartOneSizeAndBlockSize, tpl/recursive_halvingdoubling_base.cc:23-37 */
+    uint32_t round = 0;
+    while ((1u << round) <= n) round++;
+    if (round >= 1) round -= 1;
+    const uint32_t block = 1u << round;
+    const uint32_t part1 = (n - block) * 2;
+    OrcSlice sl[ORC_MAX_RANKS];
+    orc_slices_rhd(total, block, sl);
+
+    uint32_t step = 0;
+    /* ReduceInPartOne, :133-203: even ranks of part one reduce the odd neighbour's whole input into theirs */
+    if (part1 > 0) {
+        if (rank < part1 && rank % 2 == 0) emit(t, step, K_REDUCE, rank, B_IN, 0, rank + 1, B_IN, 0, total);
+        step++;
+    }
+    const int idle = (rank < part1 && rank % 2 == 1); /* :208-210, :243-245 */
+    uint32_t rib = 0;                                 /* rankInBlock */
+    if (!idle) rib = (rank < part1) ? rank / 2 : rank - part1 / 2;
+    /* block rank -> real rank: inverse of BuildSubLinks, tpl/recursive_halvingdoubling_base.cc:39-62 */
+#define REAL(b) (((b) < part1 / 2) ? 2 * (b) : (b) + part1 / 2)
+    uint32_t steps = 0; /* GetBlockStep / Log2 */
+    while ((block >> (steps + 1)) != 0) steps++;
+
+    /* ReduceScatterHalvingDoubling, tpl/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:65-92,196-257 */
+    uint32_t last_rx = 0;
+    for (uint32_t s = 0; s < steps; s++) {
+        if (!idle) {
+            const uint32_t mask = 1u << (steps - s - 1); /* halvingBitmask :72 */
+            const uint32_t peer = rib ^ mask;
+            const uint32_t id = rib & (~(mask - 1)); /* rx slice id :76-77 */
+            uint64_t sz = 0;
+            uint32_t num = mask; /* Sum(), tpl/alg_template_base.cc:1079-1096 */
+            while (num > 0) {
+                num--;
+                sz += sl[id + num].size;
+            }
+            emit(t, step, K_REDUCE, rank, B_IN, sl[id].offset, REAL(peer), B_IN, sl[id].offset, sz);
+            last_rx = id;
+        }
+        step++;
+    }
+    /* :251-254 copy of the last received range (one slice) input -> output */
+    if (!idle) emit(t, step, K_COPY, rank, B_OUT, sl[last_rx].offset, rank, B_IN, sl[last_rx].offset, sl[last_rx].size);
+    step++;
+    /* AllGatherHalvingDoubling in the outputs, tpl/temp_all_gather/all_gather_halving_doubling.cc:42-66,164-206 */
+    for (uint32_t s = 0; s < steps; s++) {
+        if (!idle) {
+            const uint32_t mask = 1u << s;
+            const uint32_t peer = rib ^ mask;
+            const uint32_t id = peer & (~(mask - 1)); /* rx: the peer's aligned group */
+            uint64_t sz = 0;
+            for (uint32_t k = 0; k < mask; k++) sz += sl[id + k].size;
+            emit(t, step, K_COPY, rank, B_OUT, sl[id].offset, REAL(peer), B_OUT, sl[id].offset, sz);
+        }
+        step++;
+    }
+    /* GatherInPartOne, :277-343: odd ranks of part one receive the even neighbour's whole output */
+    if (part1 > 0) {
+        if (rank < part1 && rank % 2 == 1) emit(t, step, K_COPY, rank, B_OUT, 0, rank - 1, B_OUT, 0, total);
+        step++;
+    }
+#undef REAL
+}
+
+/* AllReduceMeshDirectOneshot::RunAllReduceOne, tpl/temp_all_reduce/all_reduce_mesh_oneshot.cc:78-121.  The
+ * remote buffer read at :108-115 is the peer's communication buffer, filled with the peer's input at :96-100;
+ * with two buffers per rank that is in[peer]. */
+static void prog_allreduce_mesh_oneshot(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    emit(t, 0, K_COPY, rank, B_OUT, 0, rank, B_IN, 0, total); /* :92-94 (also the n == 1 path, :53-62) */
+    for (uint32_t round = 1; round < n; round++) {
+        const uint32_t peer = (round + rank) % n; /* :103 */
+        emit(t, round, K_REDUCE, rank, B_OUT, 0, peer, B_IN, 0, total);
+    }
+}
+
+/* ReduceScatterMesh, tpl/temp_reduce_scatter/reduce_scatter_mesh.cc:51-128 (stream index 0), :131-215 */
+static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) { /* :152-157 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, sz);
+        return;
+    }
+    uint32_t step = 0;
+    for (uint32_t round = 1; round < n; round++) {
+        const uint32_t src = (rank + n - round) % n; /* ForwardRank, tpl/../inc/reduce_scatter_mesh_pub.h:31-37 */
+        /* RunDestRducer :35-49: dst = own input slice `rank`, remote offset = same slice */
+        emit(t, step++, K_REDUCE, rank, B_IN, (uint64_t)rank * sz, src, B_IN, (uint64_t)rank * sz, sz);
+    }
+    emit(t, step, K_COPY, rank, B_OUT, 0, rank, B_IN, (uint64_t)rank * sz, sz); /* :199-211 */
+}
+
+enum {
+    ORC_ALG_ALLREDUCE_RING = 0,
+    ORC_ALG_RS_RING_STAGE = 1,
+    ORC_ALG_ALLREDUCE_RHD = 2,
+    ORC_ALG_ALLREDUCE_MESH_ONESHOT = 3,
+    ORC_ALG_RS_MESH = 4,
+    ORC_ALG_RS_RING_STANDALONE = 5
+};
+
+static int cmp_ops(const void* a, const void* b)
+{
+    const OrcOp* x = (const OrcOp*)a;
+    const OrcOp* y = (const OrcOp*)b;
+    if (x->step != y->step) return x->step < y->step ? -1 : 1;
+    if (x->rank != y->rank) return x->rank < y->rank ? -1 : 1;
+    return 0;
+}
+
+static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (n == 0 || n > ORC_MAX_RANKS || unit == 0) return -1;
+    for (uint32_t r = 0; r < n; r++) {
+        switch (alg) {
+            case ORC_ALG_ALLREDUCE_RING: prog_allreduce_ring(t, r, n, count, unit, 1); break;
+            case ORC_ALG_RS_RING_STAGE: prog_allreduce_ring(t, r, n, count, unit, 0); break;
+            case ORC_ALG_ALLREDUCE_RHD: prog_allreduce_rhd(t, r, n, count, unit); break;
+            case ORC_ALG_ALLREDUCE_MESH_ONESHOT: prog_allreduce_mesh_oneshot(t, r, n, count, unit); break;
+            case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, unit); break;
+            case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, unit); break;
+            default: free(t->ops); return -1;
+        }
+    }
+    if (t->oom) {
+        free(t->ops);
+        return -2;
+    }
+    /* lock step: order by step, then rank (stable within a rank because a rank emits one op per step) */
+    qsort(t->ops, t->n, sizeof(OrcOp), cmp_ops);
+    return 0;
+}
+
+/* Write the lock-step op list (ordered by step, then rank).  Returns the total number of ops, or < 0. */
+int64_t orc_trace(int alg, uint32_t n, uint64_t count, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace(&t, alg, n, count, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+static int ranges_overlap(uintptr_t a, uint64_t an, uintptr_t b, uint64_t bn) { return a < b + bn && b < a + an; }
+
+/*
+ * Execute a collective on host buffers in[r] / out[r].  Ranks act in lock step; inside a step the
+ * operations must not observe each other (the memory-conflict rule of the reference's schedule checker,
+ * test/st/algorithm/README_en.md:202-231), which is verified before the step runs, so executing them one
+ * after another equals executing them concurrently.  Returns 0, -1 bad argument, -2 out of memory,
+ * -3 conflict inside a step.
+ */
+int orc_run(int alg, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace(&t, alg, n, count, dtype);
+    if (rc) return rc;
+    const uint32_t unit = orc_dtype_size(dtype);
+    uint64_t i = 0;
+    while (i < t.n) {
+        uint64_t j = i;
+        while (j < t.n && t.ops[j].step == t.ops[i].step) j++;
+        for (uint64_t a = i; a < j; a++) {
+            const OrcOp* x = &t.ops[a];
+            const uintptr_t xd = (uintptr_t)(x->dst_buf ? out[x->rank] : in[x->rank]) + x->dst_off;
+            for (uint64_t b = i; b < j; b++) {
+                if (a == b) continue;
+                const OrcOp* y = &t.ops[b];
+                const uintptr_t yd = (uintptr_t)(y->dst_buf ? out[y->rank] : in[y->rank]) + y->dst_off;
+                const uintptr_t ys = (uintptr_t)(y->src_buf ? out[y->src_rank] : in[y->src_rank]) + y->src_off;
+                if (ranges_overlap(xd, x->bytes, yd, y->bytes) || ranges_overlap(xd, x->bytes, ys, y->bytes)) {
+                    free(t.ops);
+                    return -3;
+                }
+            }
+        }
+        for (uint64_t a = i; a < j; a++) {
+            const OrcOp* x = &t.ops[a];
+            char* d = (char*)(x->dst_buf ? out[x->rank] : in[x->rank]) + x->dst_off;
+            const char* s = (const char*)(x->src_buf ? out[x->src_rank] : in[x->src_rank]) + x->src_off;
+            if (x->kind == K_COPY)
+                orc_copy(d, s, x->bytes);
+            else if (orc_reduce(d, s, x->bytes / unit, dtype, op) != 0) {
+                free(t.ops);
+                return -1;
+            }
+        }
+        i = j;
+    }
+    free(t.ops);
+    return 0;
+}
+
+/* Bytes moved by the two-input model: 3b per reduce, 2b per copy. */
+int64_t orc_algorithmic_bytes(int alg, uint32_t n, uint64_t count, int dtype)
+{
+    OrcTrace t;
+    int rc = build_trace(&t, alg, n, count, dtype);
+    if (rc) return rc;
+    int64_t total = 0;
+    for (uint64_t i = 0; i < t.n; i++) total += (int64_t)t.ops[i].bytes * (t.ops[i].kind ? 3 : 2);
+    free(t.ops);
+    return total;
+}
+
+/* k-way chain on host memory: dst = (((s0 (op) s1) (op) s2) ...), running value in the dst role - the result
+ * of one copy and k-1 reduces (tpl/temp_all_reduce/all_reduce_mesh_oneshot.cc:94-119). */
+int orc_reduce_k(void* dst, const void* const* srcs, uint32_t k, uint64_t count, int dtype, int op)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (k == 0 || unit == 0) return -1;
+    orc_copy(dst, srcs[0], count * unit);
+    for (uint32_t j = 1; j < k; j++)
+        if (orc_reduce(dst, srcs[j], count, dtype, op) != 0) return -1;
+    return 0;
+}

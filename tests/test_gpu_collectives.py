@@ -1,0 +1,206 @@
+"""GPU parity of the schedule replays (both lowerings) against the CPU oracle: every one of the 2N rank
+buffers is compared bit-for-bit after the run, so intermediate partials left in the input buffers count."""
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+import hcomm_amd as h
+from util import DT, OPS, UNIT, assert_same, from_dev, gen, to_dev
+
+pytestmark = pytest.mark.gpu
+
+ALGS = {
+    "ring_ar": (h.Alg.ALLREDUCE_RING, oracle.ALG_ALLREDUCE_RING),
+    "ring_rs_stage": (h.Alg.REDUCE_SCATTER_RING, oracle.ALG_RS_RING_STAGE),
+    "rhd_ar": (h.Alg.ALLREDUCE_RHD, oracle.ALG_ALLREDUCE_RHD),
+    "mesh_oneshot": (h.Alg.ALLREDUCE_MESH_ONESHOT, oracle.ALG_ALLREDUCE_MESH_ONESHOT),
+    "mesh_rs": (h.Alg.REDUCE_SCATTER_MESH, oracle.ALG_RS_MESH),
+    "ring_rs": (h.Alg.REDUCE_SCATTER_RING_STANDALONE, oracle.ALG_RS_RING_STANDALONE),
+}
+FUSABLE = {"ring_ar", "ring_rs_stage", "mesh_oneshot", "mesh_rs", "ring_rs"}
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def buffer_counts(alg, n, count):
+    """(elements in each input buffer, elements in each output buffer)."""
+    if alg in ("mesh_rs", "ring_rs"):
+        return n * count, count
+    return count, count
+
+
+def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None):
+    dt, o = DT[dtype], OPS[op]
+    in_count, out_count = buffer_counts(alg, n, count)
+    kind = kind or ("prod" if op == "prod" else "default")
+    host_in = [gen(dt, in_count, seed * 1000 + r, kind) for r in range(n)]
+    sentinel = gen(dt, out_count, 999, "wide")
+    want_in = [x.copy() for x in host_in]
+    want_out = [sentinel.copy() for _ in range(n)]
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    # zero-length tensors have a null data_ptr; give the plan a real (unused) address instead
+    pad = to_dev(np.zeros(256, np.uint8))
+    ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
+    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+    try:
+        assert plan.run(thread) == 0
+        assert h.HcommGfxThreadSynchronize(thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt, "in[%d]" % r)
+            assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+        return plan.info.launches, plan.info.algorithmicBytes, plan.info.movedBytes
+    finally:
+        plan.destroy()
+
+
+CASES = [
+    # alg, n, count, dtype, op
+    ("ring_ar", 8, 1 << 20, "fp32", "sum"),        # benchmark config 1
+    ("ring_ar", 8, 1000003, "bf16", "sum"),
+    ("ring_ar", 7, 100003, "fp16", "sum"),
+    ("ring_ar", 3, 5, "int8", "sum"),              # most slices empty
+    ("ring_ar", 2, 4099, "int32", "max"),
+    ("ring_ar", 1, 777, "fp32", "sum"),
+    ("ring_ar", 5, 0, "fp32", "sum"),
+    ("ring_ar", 16, 70001, "int16", "min"),
+    ("ring_ar", 32, 300007, "bf16", "max"),
+    ("ring_ar", 4, 65536, "fp32", "prod"),
+    ("ring_rs_stage", 7, 1000003, "fp32", "prod"),  # benchmark config 5a, scaled down
+    ("ring_rs_stage", 7, 1000003, "int8", "sum"),   # benchmark config 5b, scaled down (odd last slice)
+    ("ring_rs_stage", 8, 123457, "bf16", "sum"),
+    ("rhd_ar", 16, 1 << 18, "int32", "sum"),       # benchmark config 3, scaled down
+    ("rhd_ar", 16, 1 << 18, "int32", "max"),
+    ("rhd_ar", 16, 1 << 18, "int32", "min"),
+    ("rhd_ar", 8, 100003, "fp32", "sum"),
+    ("rhd_ar", 6, 100003, "fp16", "sum"),          # part one: ranks 0..3 fold in pairs
+    ("rhd_ar", 7, 50001, "bf16", "sum"),
+    ("rhd_ar", 5, 33, "int8", "sum"),
+    ("rhd_ar", 3, 1 << 16, "fp32", "max"),
+    ("rhd_ar", 2, 12345, "int16", "sum"),
+    ("rhd_ar", 1, 100, "int32", "sum"),
+    ("rhd_ar", 12, 77777, "fp32", "sum"),
+    ("mesh_oneshot", 8, 2048, "fp16", "sum"),      # benchmark config 4, 4 KiB
+    ("mesh_oneshot", 8, 1 << 21, "fp16", "sum"),   # benchmark config 4, 4 MiB
+    ("mesh_oneshot", 8, 100003, "fp32", "sum"),
+    ("mesh_oneshot", 5, 4097, "bf16", "max"),
+    ("mesh_oneshot", 2, 1, "int8", "sum"),
+    ("mesh_oneshot", 1, 1000, "fp32", "sum"),
+    ("mesh_rs", 8, 40001, "fp32", "sum"),
+    ("mesh_rs", 4, 4096, "fp16", "min"),
+    ("mesh_rs", 7, 999, "int32", "sum"),
+    ("ring_rs", 8, 40001, "fp32", "sum"),
+    ("ring_rs", 7, 5000, "bf16", "sum"),
+    ("ring_rs", 2, 64, "int8", "max"),
+]
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
+def test_stepwise_replay_matches_oracle(gpu_thread, alg, n, count, dtype, op):
+    say("stepwise", alg, n, count, dtype, op)
+    launches, algo, moved = run_case(gpu_thread, alg, h.Lowering.STEPWISE, n, count, dtype, op)
+    assert algo == oracle.algorithmic_bytes(ALGS[alg][1], n, count, DT[dtype])
+    assert moved == algo, "the step-wise lowering moves exactly the two-input model's bytes"
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", [c for c in CASES if c[0] in FUSABLE])
+def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype, op):
+    say("fused", alg, n, count, dtype, op)
+    launches, algo, moved = run_case(gpu_thread, alg, h.Lowering.FUSED, n, count, dtype, op)
+    assert launches <= 1
+    assert moved <= algo
+
+
+def test_non_associative_inputs_expose_order(gpu_thread):
+    """fp32 values for which (a+b)+c != a+(b+c): a replay in any other association order fails here."""
+    n, count = 4, 4096
+    base = np.array([1e8, 1.0, -1e8, 1.0], np.float32)
+    for alg in ("ring_ar", "rhd_ar", "mesh_oneshot"):
+        for lowering in ((h.Lowering.STEPWISE, h.Lowering.FUSED) if alg in FUSABLE else (h.Lowering.STEPWISE,)):
+            host_in = [np.full(count, base[(r + i) % 4], np.float32) for i, r in enumerate(range(n))]
+            for r in range(n):
+                host_in[r][1::2] = base[(r + 1) % 4]
+            want_in = [x.copy() for x in host_in]
+            want_out = [np.zeros(count, np.float32) for _ in range(n)]
+            oracle.run(ALGS[alg][1], want_in, want_out, count, oracle.F32, oracle.SUM)
+            d_in = [to_dev(x) for x in host_in]
+            d_out = [to_dev(np.zeros(count, np.float32)) for _ in range(n)]
+            plan = h.Plan(ALGS[alg][0], lowering, [t.data_ptr() for t in d_in], [t.data_ptr() for t in d_out], count,
+                          oracle.F32, oracle.SUM)
+            assert plan.run(gpu_thread) == 0
+            h.HcommGfxThreadSynchronize(gpu_thread)
+            for r in range(n):
+                assert_same(from_dev(d_out[r], host_in[r]), want_out[r], oracle.F32, "%s out[%d]" % (alg, r))
+            plan.destroy()
+
+
+def test_plan_can_run_repeatedly_and_by_range(gpu_thread):
+    """A plan is reusable: re-uploading inputs and running again gives the same result; RunRange over all
+    launches one at a time equals Run."""
+    n, count, dt = 8, 100003, oracle.F32
+    host_in = [gen(dt, count, 50 + r) for r in range(n)]
+    want_in = [x.copy() for x in host_in]
+    want_out = [np.zeros(count, np.float32) for _ in range(n)]
+    oracle.run(oracle.ALG_ALLREDUCE_RING, want_in, want_out, count, dt, oracle.SUM)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(np.zeros(count, np.float32)) for _ in range(n)]
+    plan = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, [t.data_ptr() for t in d_in],
+                  [t.data_ptr() for t in d_out], count, dt, oracle.SUM)
+    import torch
+    for attempt in range(3):
+        for r in range(n):
+            d_in[r].copy_(torch.from_numpy(host_in[r].view(np.uint8)))
+        torch.cuda.synchronize()
+        if attempt == 2:
+            for i in range(plan.info.launches):
+                assert plan.run_range(gpu_thread, i, 1) == 0
+        else:
+            assert plan.run(gpu_thread) == 0
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        for r in range(n):
+            assert_same(from_dev(d_out[r], host_in[r]), want_out[r], dt)
+            assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt)
+    assert plan.run_range(gpu_thread, plan.info.launches, 1) == h.HcclResult.E_PARA
+    plan.destroy()
+
+
+def test_ring_via_public_primitives_in_batch_mode(gpu_thread):
+    """Replay the oracle's op list through HcommLocalCopy/ReduceOnThread with one BatchModeStart/End per
+    step - the way an external operator library would drive the data plane - and get one launch per step."""
+    n, count, dt = 8, 65539, oracle.BF16
+    host_in = [gen(dt, count, 70 + r) for r in range(n)]
+    want_in = [x.copy() for x in host_in]
+    want_out = [np.zeros(count, np.uint16) for _ in range(n)]
+    oracle.run(oracle.ALG_ALLREDUCE_RING, want_in, want_out, count, dt, oracle.SUM)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(np.zeros(count, np.uint16)) for _ in range(n)]
+    bufs = (d_in, d_out)
+    ops = oracle.trace(oracle.ALG_ALLREDUCE_RING, n, count, dt)
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    h.HcommGfxLaunchLogClear(gpu_thread)
+    steps = sorted(set(o[0] for o in ops))
+    for s in steps:
+        assert h.HcommBatchModeStart(None) == 0
+        for (step, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes) in ops:
+            if step != s:
+                continue
+            dst = bufs[dbuf][rank].data_ptr() + doff
+            src = bufs[sbuf][srank].data_ptr() + soff
+            if kind == 0:
+                assert h.HcommLocalCopyOnThread(gpu_thread, dst, src, nbytes) == 0
+            else:
+                assert h.HcommLocalReduceOnThread(gpu_thread, dst, src, nbytes // 2, dt, oracle.SUM) == 0
+        assert h.HcommBatchModeEnd(None) == 0
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    log = h.launch_log(gpu_thread)
+    assert len(log) == len(steps) == 15
+    assert all(r.nseg == n for r in log)
+    for r in range(n):
+        assert_same(from_dev(d_out[r], host_in[r]), want_out[r], dt)
+        assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt)

@@ -1,0 +1,238 @@
+"""GPU parity of the exported primitives against the CPU oracle (bit-exact), through the C ABI.
+
+Shaped after the reference's own API tests
+(test/ut/framework/communicator/impl/independent_op/data_api/ut_aicpu_ts_HcommLocalReduceOnThread.cc,
+ut_aicpu_ts_HcommLocalCopyOnThread.cc) with real data instead of a mocked engine.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+import hcomm_amd as h
+from util import DT, OPS, UNIT, assert_same, from_dev, gen, to_dev
+
+pytestmark = pytest.mark.gpu
+
+# counts chosen to hit: empty, sub-vector, exact vector, one tile +- 1 element, several tiles + tail
+COUNTS = [0, 1, 7, 16, 4099, 16384, 16385, 1 << 20, (1 << 20) + 13]
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("nbytes", [0, 1, 15, 16, 17, 16384, 16400, 3 * 16384 + 5, (1 << 22) + 3])
+def test_local_copy(gpu_thread, nbytes):
+    say("copy", nbytes)
+    src = np.random.default_rng(nbytes).integers(0, 256, nbytes + 64, dtype=np.uint8)
+    d_src, d_dst = to_dev(src), to_dev(np.full(nbytes + 64, 0xAB, np.uint8))
+    assert h.HcommLocalCopyOnThread(gpu_thread, d_dst.data_ptr(), d_src.data_ptr(), nbytes) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    got = d_dst.cpu().numpy()
+    assert np.array_equal(got[:nbytes], src[:nbytes])
+    assert (got[nbytes:] == 0xAB).all(), "copy wrote past len"
+
+
+@pytest.mark.parametrize("dst_off,src_off", [(1, 1), (3, 8), (16, 5), (2, 0)])
+def test_local_copy_unaligned(gpu_thread, dst_off, src_off):
+    nbytes = 100003
+    say("copy unaligned", dst_off, src_off)
+    src = np.random.default_rng(7).integers(0, 256, nbytes + 64, dtype=np.uint8)
+    d_src, d_dst = to_dev(src), to_dev(np.full(nbytes + 64, 0xCD, np.uint8))
+    assert h.HcommLocalCopyOnThread(gpu_thread, d_dst.data_ptr() + dst_off, d_src.data_ptr() + src_off, nbytes) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    got = d_dst.cpu().numpy()
+    assert np.array_equal(got[dst_off:dst_off + nbytes], src[src_off:src_off + nbytes])
+    assert (got[:dst_off] == 0xCD).all() and (got[dst_off + nbytes:] == 0xCD).all()
+
+
+def test_local_copy_same_pointer_is_noop(gpu_thread):
+    d = to_dev(np.arange(64, dtype=np.uint8))
+    h.HcommGfxLaunchLogClear(gpu_thread)
+    assert h.HcommLocalCopyOnThread(gpu_thread, d.data_ptr(), d.data_ptr(), 64) == 0
+    assert len(h.launch_log(gpu_thread)) == 0
+
+
+@pytest.mark.parametrize("dtype", ["int8", "int16", "int32", "fp16", "fp32", "bf16"])
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_local_reduce(gpu_thread, dtype, op):
+    dt, o = DT[dtype], OPS[op]
+    for count in COUNTS:
+        for kind in ("default", "wide"):
+            say("reduce", dtype, op, count, kind)
+            a, b = gen(dt, count + 8, 11 + count, kind), gen(dt, count + 8, 29 + count, kind)
+            want = a.copy()
+            oracle.reduce(want[:count], b[:count].copy(), dt, o)
+            d_a, d_b = to_dev(a), to_dev(b)
+            assert h.HcommLocalReduceOnThread(gpu_thread, d_a.data_ptr(), d_b.data_ptr(), count, dt, o) == 0
+            assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+            got = from_dev(d_a, a)
+            assert_same(got[:count], want[:count], dt, "%s %s %d %s" % (dtype, op, count, kind))
+            assert np.array_equal(got[count:], a[count:]), "reduce wrote past count"
+            assert np.array_equal(from_dev(d_b, b), b), "reduce modified src"
+
+
+@pytest.mark.parametrize("dtype", ["int8", "int32", "fp16", "fp32", "bf16"])
+def test_local_reduce_prod_needs_opt_in(gpu_thread, dtype):
+    """PROD is rejected by the primitive exactly as the reference does (cpu_primitives_c_adpt.cc:37)."""
+    d = to_dev(np.zeros(64, np.uint8))
+    assert h.HcommLocalReduceOnThread(gpu_thread, d.data_ptr(), d.data_ptr(), 4, DT[dtype], OPS["prod"]) == \
+        h.HcclResult.E_PARA
+
+
+@pytest.mark.parametrize("dtype", ["int8", "int16", "fp16", "fp32", "bf16"])
+@pytest.mark.parametrize("op", ["sum", "max"])
+@pytest.mark.parametrize("dst_el,src_el", [(1, 1), (1, 0), (3, 2)])
+def test_local_reduce_unaligned(gpu_thread, dtype, op, dst_el, src_el):
+    """Pointers offset by whole elements but not by 16 bytes take the element-wise kernel."""
+    dt, o, count = DT[dtype], OPS[op], 70001
+    say("reduce unaligned", dtype, op, dst_el, src_el)
+    a, b = gen(dt, count + 16, 3), gen(dt, count + 16, 4)
+    want = a.copy()
+    oracle.reduce(want[dst_el:dst_el + count], b[src_el:src_el + count].copy(), dt, o)
+    d_a, d_b = to_dev(a), to_dev(b)
+    u = UNIT[dt]
+    h.HcommGfxLaunchLogClear(gpu_thread)
+    assert h.HcommLocalReduceOnThread(gpu_thread, d_a.data_ptr() + dst_el * u, d_b.data_ptr() + src_el * u, count,
+                                      dt, o) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    assert [r.kind for r in h.launch_log(gpu_thread)] == [h.Kernel.BYTEWISE]
+    assert_same(from_dev(d_a, a), want, dt)
+
+
+def test_local_reduce_dst_equals_src(gpu_thread):
+    """The reference's UT passes the same pointer for both operands; the result is x (op) x."""
+    a = gen(oracle.F32, 5000, 5)
+    d = to_dev(a)
+    assert h.HcommLocalReduceOnThread(gpu_thread, d.data_ptr(), d.data_ptr(), 5000, oracle.F32, oracle.SUM) == 0
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    assert_same(from_dev(d, a), a + a, oracle.F32)
+
+
+SPECIAL_F32 = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.17549435e-38, 3.4028235e38,
+                        -3.4028235e38, 65504.0, 65520.0, 2.0 ** -24, 2.0 ** -25, 1.0009765625, 0.333333343],
+                       dtype=np.float32)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "fp32", "bf16"])
+@pytest.mark.parametrize("op", ["sum", "max", "min"])
+def test_local_reduce_special_values(gpu_thread, dtype, op):
+    """All pairs of special values: signed zeros, infinities, NaN, denormals, overflow to inf.
+    MAX / MIN keep dst on ties and unordered comparisons; SUM of 16-bit types stores a canonical NaN."""
+    dt, o = DT[dtype], OPS[op]
+    if dt == oracle.F32:
+        vals = SPECIAL_F32
+    elif dt == oracle.F16:
+        with np.errstate(over="ignore"):
+            vals = SPECIAL_F32.astype(np.float16).view(np.uint16)
+        vals = np.concatenate([vals, np.array([0x0001, 0x8001, 0x03FF, 0x7BFF, 0xFBFF, 0x7E01, 0xFE00], np.uint16)])
+    else:
+        vals = np.concatenate([(SPECIAL_F32.view(np.uint32) >> 16).astype(np.uint16),
+                               np.array([0x0001, 0x8001, 0x007F, 0x7F7F, 0xFF7F, 0x7FC1, 0xFFC0], np.uint16)])
+    a = np.repeat(vals, vals.size).copy()
+    b = np.tile(vals, vals.size).copy()
+    want = a.copy()
+    with np.errstate(all="ignore"):
+        oracle.reduce(want, b.copy(), dt, o)
+    d_a, d_b = to_dev(a), to_dev(b)
+    assert h.HcommLocalReduceOnThread(gpu_thread, d_a.data_ptr(), d_b.data_ptr(), a.size, dt, o) == 0
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    assert_same(from_dev(d_a, a), want, dt, "%s %s specials" % (dtype, op))
+
+
+def test_fp16_sum_exhaustive_against_oracle(gpu_thread):
+    """Every fp16 bit pattern added to 512 partners (33.5 M pairs): conversions and rounding agree everywhere."""
+    allh = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    partners = np.random.default_rng(3).integers(0, 1 << 16, 512, dtype=np.uint32).astype(np.uint16)
+    a = np.tile(allh, partners.size)
+    b = np.repeat(partners, allh.size)
+    for dt in (oracle.F16, oracle.BF16):
+        for o in (oracle.SUM, oracle.PROD):
+            say("exhaustive", dt, o)
+            want = a.copy()
+            with np.errstate(all="ignore"):
+                oracle.reduce(want, b.copy(), dt, o)
+            d_a, d_b, d_o = to_dev(a), to_dev(b), to_dev(np.zeros_like(a))
+            assert h.HcommGfxReduceKOnThread(gpu_thread, d_o.data_ptr(), [d_a.data_ptr(), d_b.data_ptr()], a.size, dt,
+                                             o) == 0
+            h.HcommGfxThreadSynchronize(gpu_thread)
+            assert_same(from_dev(d_o, a), want, dt, "dt %d op %d" % (dt, o))
+
+
+def test_batch_mode_merges_independent_ops(gpu_thread):
+    """Eight reduces on disjoint buffers between Start and End become ONE launch; a dependent op splits."""
+    dt, count = oracle.F32, 50000
+    bufs = [gen(dt, count, 100 + i) for i in range(16)]
+    dev = [to_dev(x) for x in bufs]
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    h.HcommGfxLaunchLogClear(gpu_thread)
+    assert h.HcommBatchModeStart(b"step") == 0
+    for i in range(8):
+        assert h.HcommLocalReduceOnThread(gpu_thread, dev[i].data_ptr(), dev[8 + i].data_ptr(), count, dt,
+                                          oracle.SUM) == 0
+    # depends on the first group's result: must not share its launch
+    assert h.HcommLocalReduceOnThread(gpu_thread, dev[15].data_ptr(), dev[0].data_ptr(), count, dt, oracle.SUM) == 0
+    assert len(h.launch_log(gpu_thread)) == 0, "batch mode must not launch before End"
+    assert h.HcommBatchModeEnd(b"step") == 0
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    log = h.launch_log(gpu_thread)
+    assert [(r.kind, r.nseg) for r in log] == [(h.Kernel.REDUCE2, 8), (h.Kernel.REDUCE2, 1)]
+    want = [x.copy() for x in bufs]
+    for i in range(8):
+        oracle.reduce(want[i], want[8 + i], dt, oracle.SUM)
+    oracle.reduce(want[15], want[0], dt, oracle.SUM)
+    for i in range(16):
+        assert_same(from_dev(dev[i], bufs[i]), want[i], dt, "buf %d" % i)
+
+
+@pytest.mark.parametrize("dtype,op", [("fp16", "sum"), ("bf16", "sum"), ("fp32", "prod"), ("int32", "max"),
+                                      ("int8", "sum"), ("fp32", "min"), ("int16", "min")])
+@pytest.mark.parametrize("k", [1, 2, 3, 8, 16, 32])
+def test_reduce_k(gpu_thread, dtype, op, k):
+    dt, o = DT[dtype], OPS[op]
+    for count in (1, 4099, 300007):
+        say("reduce_k", dtype, op, k, count)
+        srcs = [gen(dt, count, 1000 + j, "prod" if op == "prod" else "default") for j in range(k)]
+        want = oracle.reduce_k(srcs, dt, o)
+        dev = [to_dev(s) for s in srcs]
+        d_o = to_dev(np.zeros_like(srcs[0]))
+        assert h.HcommGfxReduceKOnThread(gpu_thread, d_o.data_ptr(), [d.data_ptr() for d in dev], count, dt, o) == 0
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        assert_same(from_dev(d_o, srcs[0]), want, dt)
+        for j in range(k):
+            assert np.array_equal(from_dev(dev[j], srcs[j]), srcs[j]), "input %d modified" % j
+
+
+def test_notify_orders_two_threads(gpu_thread):
+    """Record on thread A / wait on thread B: B's reduce sees A's copy (include/hcomm_primitives.h:181-191)."""
+    code, (tb,) = h.HcommThreadAlloc(h.CommEngine.CPU_TS, 1, 1)
+    assert code == 0
+    try:
+        count = 1 << 20
+        x, y = gen(oracle.I32, count, 1), gen(oracle.I32, count, 2)
+        d_x, d_y, d_t = to_dev(x), to_dev(y), to_dev(np.zeros_like(x))
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        assert h.HcommLocalCopyOnThread(gpu_thread, d_t.data_ptr(), d_x.data_ptr(), count * 4) == 0
+        assert h.HcommThreadNotifyRecordOnThread(gpu_thread, tb, 0) == 0
+        assert h.HcommThreadNotifyWaitOnThread(tb, 0, 10) == 0
+        assert h.HcommLocalReduceOnThread(tb, d_y.data_ptr(), d_t.data_ptr(), count, oracle.I32, oracle.SUM) == 0
+        assert h.HcommGfxThreadSynchronize(tb) == 0
+        assert_same(from_dev(d_y, y), (x + y), oracle.I32)
+        assert h.HcommThreadNotifyWaitOnThread(tb, 1, 0) == h.HcclResult.E_PARA
+    finally:
+        h.HcommThreadFree([tb])
+
+
+def test_mem_alloc_roundtrip(gpu_thread):
+    code, p = h.HcommMemAlloc(1 << 20)
+    assert code == 0 and p != 0 and p % 256 == 0
+    src = np.random.default_rng(0).integers(0, 256, 1 << 20, dtype=np.uint8)
+    d_src, d_back = to_dev(src), to_dev(np.zeros_like(src))
+    assert h.HcommLocalCopyOnThread(gpu_thread, p, d_src.data_ptr(), src.size) == 0
+    assert h.HcommLocalCopyOnThread(gpu_thread, d_back.data_ptr(), p, src.size) == 0
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    assert np.array_equal(d_back.cpu().numpy(), src)
+    assert h.HcommMemFree(p) == 0
