@@ -6,6 +6,13 @@ any operation.  If the library is missing, importing this module raises - it nev
 import ctypes as C
 import os
 
+try:
+    # A process can hold only one HIP runtime.  PyTorch-ROCm ships its own libamdhip64 (same soname as the one
+    # under /opt/rocm), and the dynamic loader shares it with this library only when torch was loaded first.
+    import torch  # noqa: F401
+except ImportError:  # a pure C / ctypes caller without torch uses the system runtime
+    pass
+
 __all__ = [
     "lib", "LIB_PATH", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
     "LaunchRecord", "PlanInfo", "SchedOp", "Slice", "HcommError", "check",
