@@ -7,8 +7,9 @@ resident in HBM before the timed region.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--lowering stepwise|fused|both]
                     [--workload ring_ar_bf16_n8_128MiB|ring_ar_fp32_n8_4MiB] [--no-cpu]
 
-`value` is algorithmic GB/s of the whole allreduce: (5(N-1)S + 2S) bytes / wall time of a step - the two-input
-byte model every collective library is priced with.  `roofline` prices the dominant kernel from HIP-event
+`value` is algorithmic GB/s of the whole allreduce, (5(N-1)S + 2S) bytes / wall time of a step, for the
+step-wise replay (one launch per schedule step; bytes moved == algorithmic bytes).  The fused lowering, which
+leaves identical memory while moving 23/37 of those bytes, is reported under "fused".  `roofline` prices the dominant kernel from HIP-event
 timings taken on the stream the kernels run on.  `cpu_baseline` times the CPU oracle (a C restatement of
 the same schedule) on the host cores of this machine, on the same inputs, and its result is used to verify
 the GPU output bit for bit.
@@ -24,6 +25,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+
+# HBM-side bytes per launch on the 128 MiB workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch; FETCH_SIZE scaled by 2.0, the factor that makes k_copy's 128 MiB read come out right; WRITE_SIZE by
+# 1.0).  Summaries: profiles/k_reduce2_bf16_ring_ar_n8_128MiB.md, profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md.
+MEASURED_TRAFFIC = {
+    ("ring_ar_bf16_n8_128MiB", "stepwise"): (131115.7 * 2.0 + 131072.0) * 1024,
+    ("ring_ar_bf16_n8_128MiB", "fused"): (524352.3 * 2.0 + 1966080.0) * 1024,
+}
 
 WORKLOADS = {
     # name: (ranks, elements per rank, dtype name)
@@ -144,7 +153,10 @@ def main():
         }
         plan.destroy()
 
-    best = max(results, key=lambda k: results[k]["gbs"])
+    # The headline is the step-wise replay: every launch is one schedule step of two-input reduces / copies, so
+    # the bytes it moves ARE the algorithmic bytes.  The fused lowering (same final memory, fewer bytes moved) is
+    # reported beside it under "fused".
+    best = "stepwise" if "stepwise" in results else lowerings[0]
     res = results[best]
 
     cpu = None
@@ -157,12 +169,19 @@ def main():
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         host_out = [np.zeros(count, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
-        t0 = time.perf_counter()
-        oracle.run(oracle.ALG_ALLREDUCE_RING, host_in, host_out, count, odt, oracle.SUM)
-        cpu_s = time.perf_counter() - t0
         alg_bytes = oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_RING, n, count, odt)
-        cpu = {"value": alg_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": "the full workload, one pass (%.2f s), OpenMP static over elements" % cpu_s}
+        passes, cpu_s = 0, 0.0
+        while passes < 1 or (cpu_s < 8.0 and passes < 64):
+            # every pass starts from the pristine inputs (the copy is not timed)
+            work_in = [x.copy() for x in host_in]
+            t0 = time.perf_counter()
+            oracle.run(oracle.ALG_ALLREDUCE_RING, work_in, host_out, count, odt, oracle.SUM)
+            cpu_s += time.perf_counter() - t0
+            passes += 1
+        host_in = work_in
+        cpu = {"value": round(alg_bytes * passes / cpu_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+               "sample": "the full workload, %d passes, %.2f s of CPU work in total; OpenMP static over elements"
+                         % (passes, cpu_s)}
         # verification: one GPU pass per lowering from pristine inputs must equal the oracle bit for bit
         verified = True
         for name in lowerings:
@@ -195,14 +214,15 @@ def main():
         "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": "sum",
                    "algorithm": "ring allreduce (reduce-scatter + all-gather, 8 slices)", "lowering": best},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, best)),
                      "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
                      "algorithmic_bytes_per_launch": res["kernel_alg_bytes"],
                      "moved_gbs": round(res["kernel_moved_gbs"], 2)},
         "cpu_baseline": cpu,
         "verified_bit_exact_vs_oracle": verified,
-        "lowerings": {k: {kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in v.items()}
-                      for k, v in results.items()},
+        "fused": ({kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in results["fused"].items()}
+                  if "fused" in results else None),
     }
     print(json.dumps(out))
 

@@ -5,6 +5,7 @@
  * hcomm_thread_c_adpt.cc) in names, argument meaning, check order and return codes.  A ThreadHandle is an
  * opaque pointer to a library-owned object, as in the reference (cpu_primitives_c_adpt.cc:66).
  */
+#include <pthread.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -75,11 +76,45 @@ int hg_reduce_supported(int dtype, int op, int prod_ok)
     return 0;
 }
 
+/* Live thread objects.  A handle is only dereferenced after it was found here, so a stale or made-up handle
+ * is refused instead of followed (the reference keeps the same kind of map, hcomm_thread_c_adpt.cc:31-35). */
+#define HG_THREADS_MAX 1024u
+static HgThread* g_threads[HG_THREADS_MAX];
+static uint32_t g_threads_hi = 0;
+static pthread_mutex_t g_threads_mtx = PTHREAD_MUTEX_INITIALIZER;
+
+static int registry_add(HgThread* t)
+{
+    int ok = 0;
+    pthread_mutex_lock(&g_threads_mtx);
+    for (uint32_t i = 0; i < HG_THREADS_MAX; ++i) {
+        if (!g_threads[i]) {
+            g_threads[i] = t;
+            if (i + 1 > g_threads_hi) g_threads_hi = i + 1;
+            ok = 1;
+            break;
+        }
+    }
+    pthread_mutex_unlock(&g_threads_mtx);
+    return ok;
+}
+
+static void registry_remove(HgThread* t)
+{
+    pthread_mutex_lock(&g_threads_mtx);
+    for (uint32_t i = 0; i < g_threads_hi; ++i)
+        if (g_threads[i] == t) g_threads[i] = NULL;
+    pthread_mutex_unlock(&g_threads_mtx);
+}
+
 HgThread* hg_thread_from_handle(ThreadHandle h)
 {
     HgThread* t = (HgThread*)(uintptr_t)h;
-    if (!t || t->magic != HG_THREAD_MAGIC) return NULL;
-    return t;
+    if (!t) return NULL;
+    const uint32_t hi = __atomic_load_n(&g_threads_hi, __ATOMIC_ACQUIRE);
+    for (uint32_t i = 0; i < hi; ++i)
+        if (__atomic_load_n(&g_threads[i], __ATOMIC_ACQUIRE) == t) return (t->magic == HG_THREAD_MAGIC) ? t : NULL;
+    return NULL;
 }
 
 /* ---- threads ---------------------------------------------------------------------------------- */
@@ -111,12 +146,20 @@ static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_
             }
         }
     }
+    if (!registry_add(t)) {
+        if (!recorder)
+            for (uint32_t i = 0; i < notify_num; ++i) hg_rt_event_destroy(t->notifies[i]);
+        free(t->notifies);
+        free(t);
+        return NULL;
+    }
     return t;
 }
 
 static void thread_delete(HgThread* t)
 {
     if (!t) return;
+    registry_remove(t);
     if (!t->recorder) {
         for (uint32_t i = 0; i < t->notify_num; ++i)
             if (t->notifies[i]) hg_rt_event_destroy(t->notifies[i]);

@@ -23,7 +23,7 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
         if (cap == 0) {
             int cus = hg_rt_num_cus();
             if (cus <= 0) cus = 256;
-            cap = (uint64_t)cus * 8u; /* 8 workgroups x 4 wavefronts fill a CU's 32 wavefront slots */
+            cap = (uint64_t)cus * 32u; /* measured: a grid of about one 16 KiB tile per workgroup streams best */
         }
         g_grid_cap = cap;
     }

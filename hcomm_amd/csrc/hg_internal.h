@@ -16,8 +16,12 @@ extern "C" {
 
 #define HG_MAX_SEG 32u          /* segments per launch */
 #define HG_VEC_BYTES 16u        /* one lane moves 128 bits per access */
+#ifndef HG_BLOCK
 #define HG_BLOCK 256u           /* threads per workgroup = 4 wavefronts of 64 */
+#endif
+#ifndef HG_UNROLL
 #define HG_UNROLL 4u            /* 128-bit accesses in flight per lane and operand */
+#endif
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
 

@@ -129,8 +129,30 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
     else *(uint32_t*)p = v;
 }
 
-__device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec) { return ((const u32x4*)base)[vec]; }
-__device__ __forceinline__ void stv(void* base, uint64_t vec, u32x4 v) { ((u32x4*)base)[vec] = v; }
+// Cache hints.  A ring step reads what the neighbouring rank's previous step wrote, so plain stores are left
+// to be kept by the memory-side cache while every load is marked non-temporal (each value is read once).
+#ifndef HG_NT_LD_DST
+#define HG_NT_LD_DST 1 /* the operand that is overwritten */
+#endif
+#ifndef HG_NT_LD_SRC
+#define HG_NT_LD_SRC 1 /* the peer's operand */
+#endif
+#ifndef HG_NT_ST
+#define HG_NT_ST 0
+#endif
+#ifndef HG_NT_FOLD_ST
+#define HG_NT_FOLD_ST 1 /* nothing a fold launch stores is read again by it */
+#endif
+template <bool NT> __device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec)
+{
+    if (NT) return __builtin_nontemporal_load((const u32x4*)base + vec);
+    return ((const u32x4*)base)[vec];
+}
+template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec, u32x4 v)
+{
+    if (NT) __builtin_nontemporal_store(v, (u32x4*)base + vec);
+    else ((u32x4*)base)[vec] = v;
+}
 
 // segment that owns a tile (uniform across the workgroup; nseg <= 32)
 __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
@@ -156,14 +178,14 @@ __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
         if (v0 - tid + HG_TILE_VECS <= nvec) {
             u32x4 a[HG_UNROLL];
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv(p, v0 + u * HG_BLOCK);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv(d, v0 + u * HG_BLOCK, a[u]);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<HG_NT_ST>(d, v0 + u * HG_BLOCK, a[u]);
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv(d, v, ldv(p, v));
+                if (v < nvec) stv<HG_NT_ST>(d, v, ldv<HG_NT_LD_SRC>(p, v));
             }
             const uint64_t b = (nvec << 4) + tid; // this tile is the segment's last one: byte tail
             if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
@@ -188,16 +210,16 @@ template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(
         if (v0 - tid + HG_TILE_VECS <= nvec) {
             u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv(d, v0 + u * HG_BLOCK);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_DST>(d, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv(p, v0 + u * HG_BLOCK);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<HG_NT_ST>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv(d, v, vec_op<DT, OP>(ldv(d, v), ldv(p, v)));
+                if (v < nvec) stv<HG_NT_ST>(d, v, vec_op<DT, OP>(ldv<HG_NT_LD_DST>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -248,8 +270,8 @@ __device__ __forceinline__ uint32_t fold_rank(const HgFoldTable& t, uint32_t s, 
 template <int DT, int OP> struct VecItem {
     typedef u32x4 V;
     static __device__ __forceinline__ V zero() { return V{0u, 0u, 0u, 0u}; }
-    static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ldv(p, i); }
-    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stv(p, i, v); }
+    static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ldv<HG_NT_LD_SRC>(p, i); }
+    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stv<HG_NT_FOLD_ST>(p, i, v); }
     static __device__ __forceinline__ V op(V d, V s) { return vec_op<DT, OP>(d, s); }
 };
 

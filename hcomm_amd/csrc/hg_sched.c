@@ -117,6 +117,7 @@ static int sched_rs_ring_standalone(HgOpList* l, uint32_t n, uint64_t count, uin
     const uint64_t sz = count * unit;
     if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz); /* reduce_scatter_ring.cc:103-109 */
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    memset(sl, 0, sizeof(sl));
     for (uint32_t i = 0; i < n; ++i) { /* reduce_scatter_ring.cc:140-157; the output holds one slice, so offset 0 */
         sl[i].offset = (uint64_t)i * sz;
         sl[i].size = sz;

@@ -1,0 +1,279 @@
+"""Host-side behaviour of libhcomm_gfx.so that needs no GPU: exported symbols, argument checks in the
+reference's order, batch-mode coalescing and schedule lowering, observed through a recorder thread (every
+launch it would make is logged instead of executed - the role the mocked engine plays in the reference's
+test/ut/framework/communicator/impl/independent_op/data_api/ut_aicpu_ts_HcommLocalReduceOnThread.cc)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import hcomm_amd as h
+from hcomm_amd import api as raw
+from hcomm_amd import HcclResult as R, HcommDataType as DT, HcommReduceOp as OP
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture()
+def rec():
+    code, t = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    yield t
+    h.HcommThreadFree([t])
+
+
+def test_library_exports_every_declared_symbol():
+    text = open(os.path.join(ROOT, "include", "hcomm_gfx.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b(Hcomm\w+)\s*\(", text))
+    assert {"HcommLocalCopyOnThread", "HcommLocalReduceOnThread", "HcommThreadAlloc", "HcommThreadFree",
+            "HcommBatchModeStart", "HcommBatchModeEnd", "HcommMemAlloc", "HcommMemFree",
+            "HcommGfxPlanCreate", "HcommGfxReduceKOnThread"} <= names
+    for n in sorted(names):
+        assert hasattr(h.lib, n), "libhcomm_gfx.so does not export " + n
+    assert len(names) >= 27
+
+
+def test_enum_values_match_the_reference_headers():
+    """include/hcomm_primitives.h:45-72, include/hccl/hccl_types.h:23-51."""
+    assert (OP.SUM, OP.PROD, OP.MAX, OP.MIN, OP.RESERVED) == (0, 1, 2, 3, 255)
+    assert (DT.INT8, DT.INT16, DT.INT32, DT.FP16, DT.FP32, DT.INT64, DT.UINT64, DT.UINT8, DT.UINT16, DT.UINT32,
+            DT.FP64, DT.BFP16, DT.INT128, DT.HIF8, DT.FP8E4M3, DT.FP8E5M2, DT.FP8E8M0) == \
+        (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14, 15, 16, 17)
+    assert (R.SUCCESS, R.E_PARA, R.E_PTR, R.E_NOT_SUPPORT, R.E_TIMEOUT) == (0, 1, 2, 5, 9)
+    sizes = [1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1]
+    assert [h.HcommGfxDataTypeSize(i) for i in range(18)] == sizes and h.HcommGfxDataTypeSize(255) == 0
+
+
+# ---- argument checks, in the reference's order (cpu_primitives_c_adpt.cc:58-130 and its unit tests) ------
+
+DST, SRC = 0x100000, 0x200000
+
+
+def test_local_reduce_checks(rec):
+    f = h.HcommLocalReduceOnThread
+    assert f(rec, DST, SRC, 1, DT.FP16, OP.SUM) == R.SUCCESS
+    assert f(0, DST, SRC, 1, DT.FP16, OP.SUM) == R.E_PTR           # thread null
+    assert f(rec, None, SRC, 1, DT.FP16, OP.SUM) == R.E_PTR        # dst null
+    assert f(rec, DST, None, 1, DT.FP16, OP.SUM) == R.E_PTR        # src null
+    # null pointers are reported before an unsupported type, an unsupported type before a null thread
+    assert f(rec, None, SRC, 1, DT.FP64, OP.SUM) == R.E_PTR
+    assert f(0, DST, SRC, 1, DT.FP64, OP.SUM) == R.E_PARA
+    for bad in (DT.INT64, DT.UINT64, DT.UINT8, DT.UINT16, DT.UINT32, DT.FP64, DT.INT128, DT.HIF8, DT.FP8E4M3, 255, 13):
+        assert f(rec, DST, SRC, 1, bad, OP.SUM) == R.E_PARA
+    for good in (DT.INT8, DT.INT16, DT.INT32, DT.FP16, DT.FP32, DT.BFP16):
+        for op in (OP.SUM, OP.MAX, OP.MIN):
+            assert f(rec, DST, SRC, 1, good, op) == R.SUCCESS
+        assert f(rec, DST, SRC, 1, good, OP.PROD) == R.E_PARA       # PROD only at collective level
+        assert f(rec, DST, SRC, 1, good, OP.RESERVED) == R.E_PARA
+
+
+def test_local_copy_checks(rec):
+    f = h.HcommLocalCopyOnThread
+    assert f(rec, DST, SRC, 1) == R.SUCCESS
+    assert f(0, DST, SRC, 1) == R.E_PTR
+    assert f(rec, None, SRC, 1) == R.E_PTR
+    assert f(rec, DST, None, 1) == R.E_PTR
+
+
+def test_counts_of_4gib_and_more_succeed(rec):
+    """ut_aicpu_ts_HcommLocalReduceOnThread.cc:71-89, ut_aicpu_ts_HcommLocalCopyOnThread.cc (4 GB, 4 GB + 1)."""
+    big, bigger = 0x100000000, 0x100000001
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommLocalReduceOnThread(rec, DST, SRC, big, DT.FP16, OP.SUM) == R.SUCCESS
+    assert h.HcommLocalReduceOnThread(rec, DST, SRC, bigger, DT.FP16, OP.SUM) == R.SUCCESS
+    assert h.HcommLocalCopyOnThread(rec, DST, SRC + (1 << 40), big) == R.SUCCESS
+    assert h.HcommLocalCopyOnThread(rec, DST, SRC + (1 << 40), bigger) == R.SUCCESS
+    log = h.launch_log(rec)
+    assert [r.bytes for r in log] == [2 * big, 2 * bigger, big, bigger]    # no 32-bit truncation anywhere
+    assert all(r.blocks > 0 for r in log)
+
+
+def test_zero_length_and_self_copy_do_nothing(rec):
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommLocalReduceOnThread(rec, DST, SRC, 0, DT.FP32, OP.SUM) == R.SUCCESS
+    assert h.HcommLocalCopyOnThread(rec, DST, SRC, 0) == R.SUCCESS
+    assert h.HcommLocalCopyOnThread(rec, DST, DST, 4096) == R.SUCCESS
+    assert h.launch_log(rec) == []
+
+
+def test_thread_and_memory_argument_checks():
+    assert raw._thread_alloc(h.CommEngine.CPU_TS, 1, (C.c_uint32 * 1)(0), None) == R.E_PTR
+    assert raw._thread_alloc(h.CommEngine.CPU_TS, 1, None, (C.c_uint64 * 1)()) == R.E_PTR
+    assert raw._thread_alloc(h.CommEngine.CPU_TS, 0, (C.c_uint32 * 1)(0), (C.c_uint64 * 1)()) == R.E_PARA
+    assert raw._thread_free(None, 1) == R.E_PTR
+    assert raw._thread_free_stream(None, 1) == R.E_PTR
+    assert raw._thread_free_stream((C.c_uint64 * 1)(0), 0) == R.E_PARA
+    assert raw._thread_alloc_stream(h.CommEngine.CPU_TS, None, 0, None) == R.E_PTR
+    assert raw._mem_alloc(None, 16) == R.E_PTR
+    assert raw._mem_alloc(C.byref(C.c_void_p()), 0) == R.E_PARA
+    assert h.HcommMemFree(None) == R.E_PTR
+    assert h.HcommGfxThreadSynchronize(0) == R.E_PTR
+    assert h.HcommThreadFree([12345]) == R.E_NOT_FOUND             # not a live handle: refused, never dereferenced
+    assert h.HcommLocalCopyOnThread(12345, DST, SRC, 1) == R.E_PTR
+
+
+def test_notify_argument_checks(rec):
+    assert h.HcommThreadNotifyRecordOnThread(0, rec, 0) == R.E_PTR
+    assert h.HcommThreadNotifyRecordOnThread(rec, 0, 0) == R.E_PTR
+    assert h.HcommThreadNotifyRecordOnThread(rec, rec, 0) == R.E_PARA   # recorder threads own no notifies
+    assert h.HcommThreadNotifyWaitOnThread(0, 0, 1) == R.E_PTR
+    assert h.HcommThreadNotifyWaitOnThread(rec, 0, 1) == R.E_PARA
+
+
+# ---- batch mode --------------------------------------------------------------------------------------------
+
+def test_batch_mode_state_machine(rec):
+    assert h.HcommBatchModeEnd(b"x") == R.E_PARA                   # End without Start
+    assert h.HcommBatchModeStart(b"x") == R.SUCCESS
+    assert h.HcommBatchModeStart(b"x") == R.E_PARA                 # nested Start
+    assert h.HcommBatchModeEnd(b"x") == R.SUCCESS
+    assert h.HcommBatchModeStart(None) == R.SUCCESS                # default tag
+    assert h.HcommBatchModeEnd(None) == R.SUCCESS
+
+
+def test_batch_mode_records_then_merges(rec):
+    mib = 1 << 20
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommBatchModeStart(b"step0") == 0
+    for r in range(8):   # eight independent reduces: one launch
+        assert h.HcommLocalReduceOnThread(rec, DST + 2 * r * mib, DST + (2 * r + 1) * mib, mib // 2, DT.BFP16, OP.SUM) == 0
+    assert h.launch_log(rec) == []                                 # nothing is submitted before End
+    assert h.HcommBatchModeEnd(b"step0") == 0
+    log = h.launch_log(rec)
+    assert [(r.kind, r.nseg, r.bytes, r.dtype, r.op) for r in log] == [(h.Kernel.REDUCE2, 8, 8 * mib, DT.BFP16, OP.SUM)]
+
+
+def test_batch_mode_splits_on_conflict_kind_type_and_capacity(rec):
+    mib = 1 << 20
+    A, B, Cc, D = DST, DST + 4 * mib, DST + 8 * mib, DST + 12 * mib
+
+    def run(calls):
+        h.HcommGfxLaunchLogClear(rec)
+        assert h.HcommBatchModeStart(None) == 0
+        for c in calls:
+            assert c() == 0
+        assert h.HcommBatchModeEnd(None) == 0
+        return [(r.kind, r.nseg) for r in h.launch_log(rec)]
+
+    red = lambda d, s, dt=DT.FP32, op=OP.SUM: (lambda: h.HcommLocalReduceOnThread(rec, d, s, mib // 4, dt, op))
+    cp = lambda d, s: (lambda: h.HcommLocalCopyOnThread(rec, d, s, mib))
+    K = h.Kernel
+    assert run([red(A, B), red(Cc, D)]) == [(K.REDUCE2, 2)]
+    assert run([red(A, B), red(Cc, A)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]      # reads what the first writes
+    assert run([red(A, B), red(B, Cc)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]      # writes what the first reads
+    assert run([red(A, B), red(A + mib // 2, D)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]  # overlapping destinations
+    assert run([red(A, B), red(Cc, B)]) == [(K.REDUCE2, 2)]                      # a shared source is fine
+    assert run([red(A, B), cp(Cc, D)]) == [(K.REDUCE2, 1), (K.COPY, 1)]          # different kernels
+    assert run([red(A, B), red(Cc, D, DT.INT32)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]
+    assert run([red(A, B), red(Cc, D, DT.FP32, OP.MAX)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]
+    assert run([cp(A, B), cp(Cc, D), cp(D + 2 * mib, A)]) == [(K.COPY, 2), (K.COPY, 1)]
+    assert run([red(A + 4, B + 4)]) == [(K.BYTEWISE, 1)]                          # not 16-byte aligned
+    many = [cp(DST + (2 * i) * mib, DST + (2 * i + 1) * mib) for i in range(70)]
+    assert run(many) == [(K.COPY, 32), (K.COPY, 32), (K.COPY, 6)]                 # 32 segments per launch
+
+
+def test_batch_mode_spans_several_threads(rec):
+    code, other = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    for t in (rec, other):
+        h.HcommGfxLaunchLogClear(t)
+    assert h.HcommBatchModeStart(b"two") == 0
+    assert h.HcommLocalCopyOnThread(rec, DST, SRC, 4096) == 0
+    assert h.HcommLocalCopyOnThread(other, DST, SRC, 8192) == 0
+    assert h.HcommLocalCopyOnThread(rec, DST + 65536, SRC + 65536, 4096) == 0
+    assert h.HcommBatchModeEnd(b"two") == 0
+    assert [(r.nseg, r.bytes) for r in h.launch_log(rec)] == [(2, 8192)]
+    assert [(r.nseg, r.bytes) for r in h.launch_log(other)] == [(1, 8192)]
+    h.HcommThreadFree([other])
+
+
+def test_reduce_k_checks(rec):
+    f = h.HcommGfxReduceKOnThread
+    assert f(rec, DST, [SRC, SRC + 4096], 100, DT.FP16, OP.SUM) == R.SUCCESS
+    assert f(rec, DST, [SRC], 100, DT.FP32, OP.PROD) == R.SUCCESS            # PROD allowed here
+    assert f(rec, DST, [SRC], 100, DT.INT16, OP.PROD) == R.E_PARA            # not for int16 (param_check.cc:327-343)
+    assert f(rec, None, [SRC], 100, DT.FP16, OP.SUM) == R.E_PTR
+    assert f(rec, DST, [SRC, 0], 100, DT.FP16, OP.SUM) == R.E_PTR
+    assert f(rec, DST, [], 100, DT.FP16, OP.SUM) == R.E_PARA
+    assert f(rec, DST, [SRC] * 33, 100, DT.FP16, OP.SUM) == R.E_PARA
+    assert f(0, DST, [SRC], 100, DT.FP16, OP.SUM) == R.E_PTR
+    h.HcommGfxLaunchLogClear(rec)
+    assert f(rec, DST, [SRC + i * 4096 for i in range(8)], 2048, DT.FP16, OP.SUM) == 0
+    assert [(r.kind, r.nseg, r.bytes) for r in h.launch_log(rec)] == [(h.Kernel.CHAIN, 1, 4096)]
+    h.HcommGfxLaunchLogClear(rec)
+    assert f(rec, DST + 2, [SRC, SRC + 4096, SRC + 8192], 100, DT.FP16, OP.SUM) == 0   # unaligned: copy + 2 reduces
+    assert [r.kind for r in h.launch_log(rec)] == [h.Kernel.BYTEWISE] * 3
+
+
+# ---- plans ---------------------------------------------------------------------------------------------------
+
+def ptrs(n, size, base=0x10000000):
+    stride = (size + 255) // 256 * 256 + 256
+    return [base + i * stride for i in range(n)], [base + (n + i) * stride for i in range(n)]
+
+
+def test_plan_argument_checks():
+    i, o = ptrs(4, 4096)
+    mk = lambda **k: h.Plan(k.get("alg", h.Alg.ALLREDUCE_RING), k.get("low", h.Lowering.STEPWISE), k.get("i", i),
+                            k.get("o", o), 1024, k.get("dt", DT.FP32), k.get("op", OP.SUM))
+    mk().destroy()
+    for kwargs, code in (({"dt": DT.FP64}, R.E_PARA), ({"op": OP.RESERVED}, R.E_PARA), ({"alg": 77}, R.E_PARA),
+                         ({"low": 5}, R.E_PARA), ({"i": [i[0] + 64] + i[1:]}, R.E_PARA),
+                         ({"i": [0] + i[1:]}, R.E_PTR), ({"dt": DT.INT16, "op": OP.PROD}, R.E_PARA),
+                         ({"i": i * 9, "o": o * 9}, R.E_PARA)):
+        with pytest.raises(h.HcommError) as e:
+            mk(**kwargs)
+        assert e.value.code == code, kwargs
+    mk(dt=DT.BFP16, op=OP.PROD).destroy()
+    with pytest.raises(h.HcommError) as e:
+        mk(alg=h.Alg.ALLREDUCE_RHD, low=h.Lowering.FUSED)
+    assert e.value.code == R.E_NOT_SUPPORT
+
+
+@pytest.mark.parametrize("name,alg,n,count,dt,launches,algo_bytes,moved_fused", [
+    # the five benchmark configurations at full size: launch structure and byte accounting, no memory touched
+    ("cfg1", h.Alg.ALLREDUCE_RING, 8, 1048576, DT.FP32, 15, 155189248, 23 * 4194304),
+    ("cfg2", h.Alg.ALLREDUCE_RING, 8, 67108864, DT.BFP16, 15, 4966055936, 23 * 134217728),
+    ("cfg3", h.Alg.ALLREDUCE_RHD, 16, 33554432, DT.INT32, 9, 10334765056, None),
+    ("cfg4", h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 2097152, DT.FP16, 8, 8 * 23 * 4194304, 72 * 4194304),
+    ("cfg5a", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.FP32, 6, 7200000216, 13 * 400000012),
+    ("cfg5b", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.INT8, 6, 1800000054, 13 * 100000003),
+])
+def test_plan_structure_of_benchmark_configs(rec, name, alg, n, count, dt, launches, algo_bytes, moved_fused):
+    size = count * h.DTYPE_SIZE[dt]
+    i, o = ptrs(n, size)
+    op = OP.PROD if name == "cfg5a" else OP.SUM
+    p = h.Plan(alg, h.Lowering.STEPWISE, i, o, count, dt, op)
+    assert (p.info.launches, p.info.algorithmicBytes, p.info.movedBytes) == (launches, algo_bytes, algo_bytes)
+    assert all(r.nseg == n for r in p.launches())                  # one launch = one step of all ranks
+    h.HcommGfxLaunchLogClear(rec)
+    assert p.run(rec) == 0
+    assert [(r.kind, r.nseg, r.bytes) for r in h.launch_log(rec)] == [(r.kind, r.nseg, r.bytes) for r in p.launches()]
+    p.destroy()
+    if moved_fused is not None:
+        p = h.Plan(alg, h.Lowering.FUSED, i, o, count, dt, op)
+        assert (p.info.launches, p.info.algorithmicBytes, p.info.movedBytes) == (1, algo_bytes, moved_fused)
+        assert [r.kind for r in p.launches()] == [h.Kernel.CHAIN]
+        p.destroy()
+
+
+def test_plan_run_checks(rec):
+    i, o = ptrs(2, 4096)
+    p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, i, o, 1024, DT.FP32, OP.SUM)
+    assert p.run(0) == R.E_PTR
+    assert p.run_range(rec, 0, p.info.launches + 1) == R.E_PARA
+    assert p.run_range(rec, p.info.launches, 0) == R.SUCCESS
+    assert raw._plan_run(None, rec) == R.E_PTR
+    p.destroy()
+
+
+def test_thread_alloc_without_gpu_is_unavailable():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    code, _ = h.HcommThreadAlloc(h.CommEngine.CPU_TS, 1, 0)
+    assert code == R.E_UNAVAIL                                      # fails loudly, no CPU fallback
+    code, _ = h.HcommThreadAllocWithStream(0, 0)
+    assert code == R.E_UNAVAIL

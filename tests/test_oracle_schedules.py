@@ -1,0 +1,257 @@
+"""Pins the oracle's slice tables and schedules against hand-derived fixtures (tests/golden), against what
+the mathematics fixes (exact integer sums prove every rank contributes exactly once - the reference's own
+acceptance rule, test/st/algorithm/utils/checker/semantics_check/allreduce_semantics_checker.cc:59-96),
+and against the product's independently written generator."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+import hcomm_amd as h
+
+GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "schedules_hand_derived.json")))
+
+ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
+        oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE]
+SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE)
+
+
+# ---- slice tables ---------------------------------------------------------------------------------------
+
+def test_slice_tables_hand_computed():
+    for case in GOLD["slice_tables"]["cases"]:
+        got = oracle.slices_ring(case["count"], case["unit"], case["n"])
+        if "slices" in case:
+            assert got == [tuple(x) for x in case["slices"]], case
+        else:
+            sz = case["slices_all_equal"]
+            assert got == [(i * sz, sz) for i in range(case["n"])], case
+        # the recursive-halving formula (recursive_halvingdoubling_base.cc:64-94) agrees wherever both apply
+        total = case["count"] * case["unit"]
+        rhd = oracle.slices_rhd(total, case["n"])
+        assert [s for _, s in rhd] == [s for _, s in got]
+        assert [o for (o, s) in rhd if s] == [o for (o, s) in got if s]
+        # and so does the product
+        assert h.calc_slices(case["count"], case["unit"], case["n"]) == got
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 7, 8, 16, 31, 32])
+def test_slice_table_invariants(n):
+    rng = np.random.default_rng(n)
+    counts = [0, 1, 127, 128, 129, 1000, 100000003] + rng.integers(0, 1 << 30, 40).tolist()
+    for count in counts:
+        for unit in (1, 2, 4):
+            sl = oracle.slices_ring(count, unit, n)
+            total = count * unit
+            assert sum(s for _, s in sl) == total
+            pos = 0
+            for off, size in sl:
+                assert off == pos and off % 128 == 0 or size == 0 and off == total
+                pos += size
+            sizes = [s for _, s in sl]
+            assert sizes == sorted(sizes, reverse=True)           # full slices first, one ragged, then empties
+            assert all(s % 128 == 0 for s in sizes if s == sizes[0]) or n == 1 or sizes[0] == total
+
+
+# ---- which slice each rank receives at each step (hand-derived) ----------------------------------------
+
+def rx_table(alg, n, count, kind):
+    """{rank: [slice index received per step]} for the ops of `kind` addressing the given buffer role."""
+    sl = oracle.slices_ring(count, 4, n)
+    index = {off: i for i, (off, _) in enumerate(sl)}
+    out = {r: [] for r in range(n)}
+    for (step, k, rank, dbuf, doff, srank, sbuf, soff, nbytes) in oracle.trace(alg, n, count, oracle.F32):
+        if (k, dbuf, sbuf) == kind and srank != rank:
+            out[rank].append(index[doff])
+    return out
+
+
+def test_ring_rx_slices_hand_derived():
+    for n_s, table in GOLD["ring_rs_rx_slices"].items():
+        n = int(n_s)
+        got = rx_table(oracle.ALG_ALLREDUCE_RING, n, 128 * n, (1, 0, 0))
+        assert [got[r] for r in range(n)] == table
+    for n_s, table in GOLD["ring_ag_rx_slices"].items():
+        n = int(n_s)
+        got = rx_table(oracle.ALG_ALLREDUCE_RING, n, 128 * n, (0, 1, 1))
+        assert [got[r] for r in range(n)] == table
+
+
+def test_rhd_steps_hand_derived():
+    n, count = 4, 4 * 32  # four 128-byte slices of fp32
+    ops = oracle.trace(oracle.ALG_ALLREDUCE_RHD, n, count, oracle.F32)
+    rs = {r: [] for r in range(n)}
+    ag = {r: [] for r in range(n)}
+    for (step, k, rank, dbuf, doff, srank, sbuf, soff, nbytes) in ops:
+        if k == 1:
+            rs[rank].append((srank, doff // 128, nbytes // 128))
+        elif srank != rank:
+            ag[rank].append((srank, doff // 128, nbytes // 128))
+    g = GOLD["rhd_rs_steps"]["4"]
+    assert [[p for p, _, _ in rs[r]] for r in range(n)] == g["peers"]
+    assert [[f for _, f, _ in rs[r]] for r in range(n)] == g["rx_first_slice"]
+    assert [[m for _, _, m in rs[r]] for r in range(n)] == g["rx_num_slices"]
+    g = GOLD["rhd_ag_steps"]["4"]
+    assert [[p for p, _, _ in ag[r]] for r in range(n)] == g["peers"]
+    assert [[f for _, f, _ in ag[r]] for r in range(n)] == g["rx_first_slice"]
+    assert [[m for _, _, m in ag[r]] for r in range(n)] == g["rx_num_slices"]
+
+
+# ---- association order and operand roles (hand-derived expression trees) -------------------------------
+
+def eval_tree(tree, leaves, op):
+    """[dst, src] -> dst (op) src in float32, with the reference's MAX / MIN tie rule."""
+    if isinstance(tree, int):
+        return leaves[tree]
+    d, s = eval_tree(tree[0], leaves, op), eval_tree(tree[1], leaves, op)
+    with np.errstate(all="ignore"):
+        if op == oracle.SUM:
+            return (d + s).astype(np.float32)
+        if op == oracle.PROD:
+            return (d * s).astype(np.float32)
+        if op == oracle.MAX:
+            return np.where(s > d, s, d)
+        return np.where(s < d, s, d)
+
+
+def order_sensitive_inputs(n, count, op, seed):
+    """Inputs for which a different association order or swapped operand roles changes the bits."""
+    rng = np.random.default_rng(seed)
+    if op in (oracle.MAX, oracle.MIN):
+        # many signed-zero ties: the winner's sign bit reveals which operand was dst
+        return [rng.choice(np.array([0.0, -0.0, 1.0, -1.0], np.float32), count) for _ in range(n)]
+    if op == oracle.PROD:
+        return [(1 + rng.standard_normal(count) * 0.3).astype(np.float32) for _ in range(n)]
+    base = np.array([1e8, 1.0, -1e8, 1.0, 3e-3, -7.5], np.float32)
+    return [(rng.choice(base, count) * rng.uniform(0.5, 2.0, count)).astype(np.float32) for _ in range(n)]
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_ring_and_rhd_trees_hand_derived(op):
+    for key, alg, slicer in (("ring_allreduce_slice_tree", oracle.ALG_ALLREDUCE_RING, None),
+                             ("rhd_allreduce_slice_tree", oracle.ALG_ALLREDUCE_RHD, "block")):
+        for n_s, trees in GOLD[key].items():
+            n = int(n_s)
+            nsl = n if slicer is None else 1 << (n.bit_length() - 1)
+            count = nsl * 96 + 5  # ragged last slice
+            ins = order_sensitive_inputs(n, count, op, seed=n)
+            work_in = [x.copy() for x in ins]
+            outs = [np.zeros(count, np.float32) for _ in range(n)]
+            oracle.run(alg, work_in, outs, count, oracle.F32, op)
+            sl = oracle.slices_ring(count, 4, nsl)
+            for c_s, tree in trees.items():
+                if c_s.startswith("_"):
+                    continue
+                off, size = sl[int(c_s)]
+                lo, hi = off // 4, (off + size) // 4
+                want = eval_tree(tree, [x[lo:hi] for x in ins], op)
+                for r in range(n):  # allreduce: every rank ends with the same bits
+                    assert np.array_equal(outs[r][lo:hi].view(np.uint32), want.view(np.uint32)), (key, n, c_s, r, op)
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])
+def test_mesh_trees_hand_derived(op):
+    n, count = 4, 1001
+    ins = order_sensitive_inputs(n, count, op, seed=9)
+    outs = [np.zeros(count, np.float32) for _ in range(n)]
+    oracle.run(oracle.ALG_ALLREDUCE_MESH_ONESHOT, [x.copy() for x in ins], outs, count, oracle.F32, op)
+    results = set()
+    for r_s, tree in GOLD["mesh_oneshot_rank_tree"]["4"].items():
+        want = eval_tree(tree, ins, op)
+        assert np.array_equal(outs[int(r_s)].view(np.uint32), want.view(np.uint32))
+        results.add(want.tobytes())
+    if op == oracle.SUM:
+        assert len(results) > 1, "inputs were meant to make the per-rank orders visible"
+    big = [np.concatenate([order_sensitive_inputs(n, count, op, seed=20 + r)[0] for _ in range(n)]) for r in range(n)]
+    outs = [np.zeros(count, np.float32) for _ in range(n)]
+    oracle.run(oracle.ALG_RS_MESH, [x.copy() for x in big], outs, count, oracle.F32, op)
+    for r_s, tree in GOLD["mesh_rs_rank_tree"]["4"].items():
+        r = int(r_s)
+        want = eval_tree(tree, [x[r * count:(r + 1) * count] for x in big], op)
+        assert np.array_equal(outs[r].view(np.uint32), want.view(np.uint32))
+
+
+# ---- every rank contributes exactly once (exact integer arithmetic) -------------------------------------
+
+@pytest.mark.parametrize("alg", ALGS)
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 6, 7, 8, 12, 16])
+def test_every_rank_contributes_exactly_once(alg, n):
+    """Rank r contributes 4^r per element (+ a position code in the low part for scatter variants); the
+    int32 sum has base-4 digit 1 for every rank iff each was folded in exactly once (no carries: digits <= 3
+    for up to 3 repeats).  MAX / MIN give the closed forms n-1 / 0 on a second pass."""
+    count = 777
+    per_in = n * count if alg in SCATTER_OUT else count
+    ins = [np.full(per_in, 4 ** r, np.int32) for r in range(n)]
+    outs = [np.full(count, -1, np.int32) for _ in range(n)]
+    oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM)
+    total = sum(4 ** r for r in range(n))
+    if alg == oracle.ALG_RS_RING_STAGE:
+        sl = oracle.slices_ring(count, 4, n)
+        for r in range(n):
+            lo, hi = sl[r][0] // 4, (sl[r][0] + sl[r][1]) // 4
+            assert (ins[r][lo:hi] == total).all()
+    else:
+        for r in range(n):
+            assert (outs[r] == total).all(), (alg, n, r)
+    for op, want in ((oracle.MAX, n - 1), (oracle.MIN, 0)):
+        ins = [np.full(per_in, r, np.int32) for r in range(n)]
+        outs = [np.full(count, -1, np.int32) for _ in range(n)]
+        oracle.run(alg, ins, outs, count, oracle.I32, op)
+        if alg != oracle.ALG_RS_RING_STAGE:
+            assert all((o == want).all() for o in outs)
+
+
+def test_scatter_variants_deliver_the_right_slice():
+    """out[r] of a reduce-scatter is the sum of everybody's slice r, not of some other slice."""
+    n, count = 5, 300
+    for alg in SCATTER_OUT:
+        ins = [(np.arange(n * count, dtype=np.int32) * 10 + r) for r in range(n)]
+        outs = [np.zeros(count, np.int32) for _ in range(n)]
+        want = sum(x.astype(np.int64) for x in ins)
+        oracle.run(alg, [x.copy() for x in ins], outs, count, oracle.I32, oracle.SUM)
+        for r in range(n):
+            assert np.array_equal(outs[r], want[r * count:(r + 1) * count].astype(np.int32))
+
+
+# ---- two independently written generators agree ----------------------------------------------------------
+
+@pytest.mark.parametrize("alg", ALGS)
+def test_product_generator_equals_oracle_trace(alg):
+    for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32):
+        for count, dt in ((0, oracle.F32), (1, oracle.I8), (5, oracle.I8), (1000, oracle.F16), (100003, oracle.F32),
+                          (100000003, oracle.I8)):
+            a = oracle.trace(alg, n, count, dt)
+            b = h.schedule_emit(alg, n, count, dt)
+            assert a == b, (alg, n, count, dt)
+
+
+def test_algorithmic_bytes_of_benchmark_configs():
+    """5(N-1)S + 2S for ring / RHD allreduce, 3(N-1)S for the reduce-scatter stage."""
+    mib = 1 << 20
+    assert oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_RING, 8, 1048576, oracle.F32) == 148 * mib
+    assert oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_RING, 8, 67108864, oracle.BF16) == 4736 * mib
+    assert oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_RHD, 16, 33554432, oracle.I32) == 9856 * mib
+    assert oracle.algorithmic_bytes(oracle.ALG_RS_RING_STAGE, 7, 100000003, oracle.F32) == 7200000216
+    assert oracle.algorithmic_bytes(oracle.ALG_RS_RING_STAGE, 7, 100000003, oracle.I8) == 1800000054
+    m = 4096
+    assert oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_MESH_ONESHOT, 8, m // 2, oracle.F16) == 8 * (2 * m + 3 * 7 * m)
+
+
+def test_steps_are_conflict_free_and_errors_are_reported():
+    """orc_run refuses a step whose operations could observe each other; every schedule passes that check
+    for every rank count, and bad arguments are reported."""
+    for alg in ALGS:
+        for n in range(1, 18):
+            count = 100
+            per_in = n * count if alg in SCATTER_OUT else count
+            ins = [np.ones(per_in, np.int32) for _ in range(n)]
+            outs = [np.zeros(count, np.int32) for _ in range(n)]
+            oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM)  # raises on rc != 0
+    with pytest.raises(ValueError):
+        oracle.trace(99, 4, 10, oracle.F32)
+    with pytest.raises(ValueError):
+        oracle.trace(0, 0, 10, oracle.F32)
+    with pytest.raises(ValueError):
+        oracle.trace(0, 33, 10, oracle.F32)
