@@ -1,18 +1,19 @@
 #!/usr/bin/env python3
-"""Benchmark of the hot path on one MI355X: simulated 8-rank bf16 ring allreduce, 128 MiB per rank.
+"""Benchmark of the hot path on one MI355X.  Default: simulated 8-rank bf16 ring allreduce, 128 MiB per rank.
 
-One "step" is one complete allreduce over the 8 simulated ranks (16 HBM buffers of 128 MiB).  Inputs are
-resident in HBM before the timed region.  Prints ONE JSON line.
+One "step" is one complete collective over the N simulated ranks (2N HBM buffers).  Inputs are resident in
+HBM before the timed region.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--lowering stepwise|fused|both]
-                    [--workload ring_ar_bf16_n8_128MiB|ring_ar_fp32_n8_4MiB] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--lowering stepwise|fused|both]
+                    [--no-cpu] [--cpu-threads T]
 
-`value` is algorithmic GB/s of the whole allreduce, (5(N-1)S + 2S) bytes / wall time of a step, for the
-step-wise replay (one launch per schedule step; bytes moved == algorithmic bytes).  The fused lowering, which
-leaves identical memory while moving 23/37 of those bytes, is reported under "fused".  `roofline` prices the dominant kernel from HIP-event
-timings taken on the stream the kernels run on.  `cpu_baseline` times the CPU oracle (a C restatement of
-the same schedule) on the host cores of this machine, on the same inputs, and its result is used to verify
-the GPU output bit for bit.
+`value` is algorithmic GB/s of the whole collective - the two-input byte model, 3b per reduce and 2b per copy,
+(5(N-1)S + 2S for an allreduce) divided by the wall time of a step - for the step-wise replay (one launch per
+schedule step; bytes moved == algorithmic bytes).  The fused lowering, which leaves identical memory while
+moving fewer bytes, is reported under "fused".  `roofline` prices the dominant kernel from HIP-event timings
+taken on the stream the kernels run on.  `cpu_baseline` times the CPU oracle (a C restatement of the same
+schedule) on the host cores of this machine, on the same inputs, and its result is used to verify the GPU
+output bit for bit.  Workload `mesh_oneshot_fp16_n8_sweep` reports latency and GB/s per message size.
 """
 import argparse
 import json
@@ -26,19 +27,52 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM-side bytes per launch on the 128 MiB workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
-# dispatch; FETCH_SIZE scaled by 2.0, the factor that makes k_copy's 128 MiB read come out right; WRITE_SIZE by
-# 1.0).  Summaries: profiles/k_reduce2_bf16_ring_ar_n8_128MiB.md, profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md.
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch; FETCH_SIZE scaled by 2.0, the factor that makes k_copy's known 128 MiB read come out right;
+# WRITE_SIZE by 1.0).  Summaries: profiles/k_reduce2_bf16_ring_ar_n8_128MiB.md,
+# profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md.
 MEASURED_TRAFFIC = {
     ("ring_ar_bf16_n8_128MiB", "stepwise"): (131115.7 * 2.0 + 131072.0) * 1024,
-    ("ring_ar_bf16_n8_128MiB", "fused"): (524352.3 * 2.0 + 1966080.0) * 1024,
+    ("ring_ar_bf16_n8_128MiB", "fused"): (524348.6 * 2.0 + 1966281.4) * 1024,
 }
 
+# name: (algorithm, ranks, elements per rank, dtype, op, data distribution)
 WORKLOADS = {
-    # name: (ranks, elements per rank, dtype name)
-    "ring_ar_bf16_n8_128MiB": (8, 67108864, "bf16"),
-    "ring_ar_fp32_n8_4MiB": (8, 1048576, "fp32"),
+    "ring_ar_bf16_n8_128MiB": ("ring_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "ring_ar_fp32_n8_4MiB": ("ring_ar", 8, 1048576, "fp32", "sum", "uniform[-1,1)"),
+    "rhd_ar_int32_n16_128MiB_sum": ("rhd_ar", 16, 33554432, "int32", "sum", "ints[-2^20,2^20]"),
+    "rhd_ar_int32_n16_128MiB_max": ("rhd_ar", 16, 33554432, "int32", "max", "ints[-2^20,2^20]"),
+    "rhd_ar_int32_n16_128MiB_min": ("rhd_ar", 16, 33554432, "int32", "min", "ints[-2^20,2^20]"),
+    "ring_rs_fp32_prod_n7_100M": ("ring_rs_stage", 7, 100000003, "fp32", "prod", "uniform[0.99,1.01]"),
+    "ring_rs_int8_sum_n7_100M": ("ring_rs_stage", 7, 100000003, "int8", "sum", "ints[-8,8]"),
+    "mesh_oneshot_fp16_n8_4MiB": ("mesh_oneshot", 8, 2097152, "fp16", "sum", "uniform[-1,1)"),
+    "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
+
+
+def make_inputs(torch, dev, n, count, dtname, seed=1234):
+    """Seeded synthetic inputs on the GPU, returned as uint8 byte tensors (one per rank)."""
+    gen = torch.Generator(device=dev)
+    out = []
+    for r in range(n):
+        gen.manual_seed(seed + r)
+        if dtname == "bf16":
+            x = (torch.randn(count, generator=gen, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+        elif dtname == "fp16":
+            x = (torch.rand(count, generator=gen, device=dev, dtype=torch.float32) * 2 - 1).to(torch.float16)
+        elif dtname == "fp32":
+            x = torch.rand(count, generator=gen, device=dev, dtype=torch.float32) * 2 - 1
+        elif dtname == "fp32prod":
+            x = torch.rand(count, generator=gen, device=dev, dtype=torch.float32) * 0.02 + 0.99
+        elif dtname == "int32":
+            x = torch.randint(-(1 << 20), (1 << 20) + 1, (count,), generator=gen, device=dev, dtype=torch.int32)
+        elif dtname == "int8":
+            x = torch.randint(-8, 9, (count,), generator=gen, device=dev, dtype=torch.int8)
+        else:
+            raise ValueError(dtname)
+        out.append(x.view(torch.uint8).clone())
+        del x
+    return out
 
 
 def main():
@@ -63,42 +97,49 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    n, count, dtname = WORKLOADS[args.workload]
-    dt = {"bf16": h.HcommDataType.BFP16, "fp32": h.HcommDataType.FP32}[dtname]
+    alg_name, n, count, dtname, opname, dist = WORKLOADS[args.workload]
+    DT = {"bf16": h.HcommDataType.BFP16, "fp32": h.HcommDataType.FP32, "fp16": h.HcommDataType.FP16,
+          "int32": h.HcommDataType.INT32, "int8": h.HcommDataType.INT8}
+    ALG = {"ring_ar": h.Alg.ALLREDUCE_RING, "rhd_ar": h.Alg.ALLREDUCE_RHD, "ring_rs_stage": h.Alg.REDUCE_SCATTER_RING,
+           "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT}
+    OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
+          "min": h.HcommReduceOp.MIN}
+    dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
     unit = h.DTYPE_SIZE[dt]
-    nbytes = count * unit
-
-    # seeded synthetic inputs: normal(0,1)*1e-3 rounded to bf16 (gradient-like) / uniform[-1,1) fp32
-    gen = torch.Generator(device=dev)
-    pristine, d_in, d_out = [], [], []
-    for r in range(n):
-        gen.manual_seed(1234 + r)
-        if dtname == "bf16":
-            x = (torch.randn(count, generator=gen, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
-        else:
-            x = torch.rand(count, generator=gen, device=dev, dtype=torch.float32) * 2 - 1
-        pristine.append(x.view(torch.uint8).clone())
-        d_in.append(torch.empty(nbytes, dtype=torch.uint8, device=dev))
-        d_out.append(torch.empty(nbytes, dtype=torch.uint8, device=dev))
-        del x
-
-    def restore():
-        for r in range(n):
-            d_in[r].copy_(pristine[r])
-            d_out[r].zero_()
-        torch.cuda.synchronize()
+    in_place = alg_name == "ring_rs_stage"
 
     stream = torch.cuda.Stream(device=dev)  # default priority
     code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 0)
     h.check(code, "HcommThreadAllocWithStream")
+
+    if count is None:
+        out = mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit)
+        h.HcommThreadFreeWithStream([thread])
+        print(json.dumps(out))
+        return
+
+    nbytes = count * unit
+    pristine = make_inputs(torch, dev, n, count, "fp32prod" if opname == "prod" else dtname)
+    d_in = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
+    d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
+
+    def restore():
+        for r in range(n):
+            d_in[r].copy_(pristine[r])
+            if d_out is not None:
+                d_out[r].zero_()
+        torch.cuda.synchronize()
+
     in_ptrs = [t.data_ptr() for t in d_in]
-    out_ptrs = [t.data_ptr() for t in d_out]
+    out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
+    kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
+             h.Kernel.COPY: "k_copy"}
 
     lowerings = ["stepwise", "fused"] if args.lowering == "both" else [args.lowering]
     results = {}
     for name in lowerings:
         low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-        plan = h.Plan(h.Alg.ALLREDUCE_RING, low, in_ptrs, out_ptrs, count, dt, h.HcommReduceOp.SUM)
+        plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op)
         launches = plan.launches()
         restore()
         for _ in range(args.warmup):
@@ -113,13 +154,16 @@ def main():
         wall = time.perf_counter() - t0
         ms_step = wall * 1e3 / args.steps
 
-        # dominant kernel: the reduce launches (step-wise) or the single fold launch (fused), timed with
-        # HIP events recorded on the stream the kernels run on
-        kinds = [r.kind for r in launches]
-        dom_kind = h.Kernel.REDUCE2 if name == "stepwise" else h.Kernel.CHAIN
-        dom = [i for i, k in enumerate(kinds) if k == dom_kind]
-        first, cnt = dom[0], len(dom)
-        assert dom == list(range(first, first + cnt))
+        # dominant kernel = the kind with the most bytes; its first contiguous run of launches is timed as a
+        # group with HIP events recorded on the stream the kernels run on
+        by_kind = {}
+        for r in launches:
+            by_kind[r.kind] = by_kind.get(r.kind, 0) + r.bytes * (2 if r.kind == h.Kernel.COPY else 3)
+        dom_kind = max(by_kind, key=by_kind.get)
+        first = [i for i, r in enumerate(launches) if r.kind == dom_kind][0]
+        cnt = 1
+        while first + cnt < len(launches) and launches[first + cnt].kind == dom_kind:
+            cnt += 1
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
         for a, b in ev:
             if first:
@@ -132,30 +176,29 @@ def main():
                 h.check(plan.run_range(thread, first + cnt, rest), "run_range")
         stream.synchronize()
         dom_ms = sum(a.elapsed_time(b) for a, b in ev) / (args.steps * cnt)
-        # algorithmic bytes of one dominant launch: 3 x slice bytes x ranks for a reduce step; the whole
-        # allreduce (5(N-1)S + 2S) for the fused launch
         if name == "stepwise":
-            dom_bytes = 3 * launches[first].bytes
+            # average launch of the run: 3 x (bytes it writes) for a reduce step of all ranks
+            dom_bytes = sum(launches[i].bytes for i in range(first, first + cnt)) * 3 // cnt
+            dom_moved = dom_bytes
         else:
-            dom_bytes = plan.info.algorithmicBytes
+            dom_bytes = plan.info.algorithmicBytes  # the single launch is the whole collective
+            dom_moved = plan.info.movedBytes
         results[name] = {
             "ms_per_step": ms_step,
             "gbs": plan.info.algorithmicBytes / (ms_step * 1e-3) / 1e9,
             "launches": plan.info.launches,
             "algorithmic_bytes": plan.info.algorithmicBytes,
             "moved_bytes": plan.info.movedBytes,
-            "kernel": "k_reduce2<bf16,SUM>" if name == "stepwise" else "k_fold_chain<bf16,SUM>",
+            "kernel": "%s<%s,%s>" % (kname[dom_kind], dtname, opname.upper()),
             "kernel_ms": dom_ms,
             "kernel_alg_bytes": dom_bytes,
             "kernel_gbs": dom_bytes / (dom_ms * 1e-3) / 1e9,
-            "kernel_moved_gbs": (3 * launches[first].bytes if name == "stepwise" else plan.info.movedBytes)
-            / (dom_ms * 1e-3) / 1e9,
+            "kernel_moved_gbs": dom_moved / (dom_ms * 1e-3) / 1e9,
         }
         plan.destroy()
 
     # The headline is the step-wise replay: every launch is one schedule step of two-input reduces / copies, so
-    # the bytes it moves ARE the algorithmic bytes.  The fused lowering (same final memory, fewer bytes moved) is
-    # reported beside it under "fused".
+    # the bytes it moves ARE the algorithmic bytes.
     best = "stepwise" if "stepwise" in results else lowerings[0]
     res = results[best]
 
@@ -164,18 +207,21 @@ def main():
     if not args.no_cpu:
         import oracle
         threads = args.cpu_threads or min(16, os.cpu_count() or 1)
-        odt = {"bf16": oracle.BF16, "fp32": oracle.F32}[dtname]
-        npdt = np.uint16 if dtname == "bf16" else np.float32
+        odt = {"bf16": oracle.BF16, "fp32": oracle.F32, "fp16": oracle.F16, "int32": oracle.I32,
+               "int8": oracle.I8}[dtname]
+        oalg = {"ring_ar": oracle.ALG_ALLREDUCE_RING, "rhd_ar": oracle.ALG_ALLREDUCE_RHD,
+                "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT}[alg_name]
+        oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
+        npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
-        host_out = [np.zeros(count, npdt) for _ in range(n)]
+        host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
-        alg_bytes = oracle.algorithmic_bytes(oracle.ALG_ALLREDUCE_RING, n, count, odt)
+        alg_bytes = oracle.algorithmic_bytes(oalg, n, count, odt)
         passes, cpu_s = 0, 0.0
         while passes < 1 or (cpu_s < 8.0 and passes < 64):
-            # every pass starts from the pristine inputs (the copy is not timed)
-            work_in = [x.copy() for x in host_in]
+            work_in = [x.copy() for x in host_in]  # every pass starts from the pristine inputs (copy not timed)
             t0 = time.perf_counter()
-            oracle.run(oracle.ALG_ALLREDUCE_RING, work_in, host_out, count, odt, oracle.SUM)
+            oracle.run(oalg, work_in, host_out, count, odt, oop)
             cpu_s += time.perf_counter() - t0
             passes += 1
         host_in = work_in
@@ -186,19 +232,23 @@ def main():
         verified = True
         for name in lowerings:
             low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-            plan = h.Plan(h.Alg.ALLREDUCE_RING, low, in_ptrs, out_ptrs, count, dt, h.HcommReduceOp.SUM)
+            plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op)
             restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
             stream.synchronize()
             for r in range(n):
-                ok = np.array_equal(d_out[r].cpu().numpy().view(npdt).view(np.uint8), host_out[r].view(np.uint8)) and \
-                    np.array_equal(d_in[r].cpu().numpy().view(npdt).view(np.uint8), host_in[r].view(np.uint8))
+                ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
+                if not in_place:
+                    ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
                 verified = verified and bool(ok)
             plan.destroy()
 
     h.HcommThreadFreeWithStream([thread])
+    metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
+    if args.workload != "ring_ar_bf16_n8_128MiB":
+        metric = "HBM GB/s (% of peak) for simulated %d-rank %s %s %s" % (n, dtname, alg_name, opname)
     out = {
-        "metric": "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank",
+        "metric": metric,
         "value": round(res["gbs"], 2),
         "unit": "GB/s",
         "pct_of_peak": round(100.0 * res["gbs"] / HBM_PEAK_GBS, 2),
@@ -211,20 +261,66 @@ def main():
         "vs_baseline": None,
         "dtype": dtname,
         "data": "synthetic",
-        "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": "sum",
-                   "algorithm": "ring allreduce (reduce-scatter + all-gather, 8 slices)", "lowering": best},
+        "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": opname,
+                   "algorithm": alg_name, "values": dist, "lowering": best},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),
                      "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
-                     "algorithmic_bytes_per_launch": res["kernel_alg_bytes"],
-                     "moved_gbs": round(res["kernel_moved_gbs"], 2)},
+                     "algorithmic_bytes_per_launch": res["kernel_alg_bytes"]},
         "cpu_baseline": cpu,
         "verified_bit_exact_vs_oracle": verified,
         "fused": ({kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in results["fused"].items()}
-                  if "fused" in results else None),
+                  if "fused" in results and best != "fused" else None),
     }
     print(json.dumps(out))
+
+
+def mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit):
+    """Mesh one-shot allreduce SUM fp16, 8 ranks, 4 KiB .. 4 MiB per rank: latency (median of per-collective
+    HIP-event times) and algorithmic GB/s (N(N+1)M bytes) for the fused single launch; the step-wise replay
+    (N launches) is listed beside it."""
+    points = []
+    reps = max(args.steps, 100)
+    for m in [1 << s for s in range(12, 23)]:
+        count = m // unit
+        ins = make_inputs(torch, dev, n, count, "fp16")
+        outs = [torch.zeros(m, dtype=torch.uint8, device=dev) for _ in range(n)]
+        row = {"bytes_per_rank": m}
+        for name, low in (("fused", h.Lowering.FUSED), ("stepwise", h.Lowering.STEPWISE)):
+            plan = h.Plan(h.Alg.ALLREDUCE_MESH_ONESHOT, low, [t.data_ptr() for t in ins], [t.data_ptr() for t in outs],
+                          count, dt, h.HcommReduceOp.SUM)
+            for _ in range(10):
+                plan.run(thread)
+            stream.synchronize()
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            for a, b in ev:
+                a.record(stream)
+                plan.run(thread)
+                b.record(stream)
+            stream.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+            row[name + "_us"] = round(ts[len(ts) // 2], 2)
+            row[name + "_launches"] = plan.info.launches
+            # back-to-back throughput: reps collectives between one pair of events
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(reps):
+                plan.run(thread)
+            b.record(stream)
+            stream.synchronize()
+            per = a.elapsed_time(b) * 1e3 / reps
+            row[name + "_pipelined_us"] = round(per, 2)
+            row[name + "_gbs"] = round(n * (n + 1) * m / (per * 1e-6) / 1e9, 1)
+            plan.destroy()
+        points.append(row)
+    top = points[-1]
+    return {"metric": "mesh one-shot allreduce SUM fp16, 8 simulated ranks: latency (us) and GB/s per message size",
+            "value": top["fused_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": reps, "warmup": 10,
+            "ms_per_step": top["fused_pipelined_us"] / 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+            "config": {"workload": args.workload, "ranks": n, "algorithmic_bytes": "N(N+1)M = 72 M"},
+            "sweep": points}
 
 
 if __name__ == "__main__":

@@ -58,19 +58,36 @@ void hg_finish_fold(HgLaunch* l)
 {
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
+    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES : HG_TILE_BYTES;
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
-        tiles += tiles_of(t->bytes[s]);
+        tiles += (t->bytes[s] + tile_bytes - 1) / tile_bytes;
         bytes += t->bytes[s];
     }
     t->tile_begin[t->nseg] = (uint32_t)tiles;
     l->nseg = t->nseg;
     l->bytes = bytes;
     uint64_t per = t->k; /* reads */
-    if (t->store_partials) per += t->k - 1;
-    if (t->store_final_first) per += 1;
-    if (t->out_mode == 1) per += 1;
-    if (t->out_mode == 2) per += t->nranks;
+    if (t->tree) {
+        /* per element: k leaf reads, one read per absorbed neighbour, one store per even position, one per odd
+         * position that absorbed a neighbour (which block ranks sit on odd positions depends on the slice), and
+         * nout outputs */
+        uint64_t moved = 0;
+        for (uint32_t s = 0; s < t->nseg; ++s) {
+            uint64_t n = t->k + t->k / 2 + t->nout;
+            for (uint32_t b = 0; b < t->k; ++b)
+                if (t->in2[b]) n += 1 + (((b ^ t->first[s]) & (t->k / 2)) ? 1 : 0);
+            moved += n * t->bytes[s];
+        }
+        l->moved_bytes = moved;
+        l->blocks = hg_grid_blocks(tiles);
+        return;
+    } else {
+        if (t->store_partials) per += t->k - 1;
+        if (t->store_final_first) per += 1;
+        if (t->out_mode == 1) per += 1;
+        if (t->out_mode == 2) per += t->nranks;
+    }
     l->moved_bytes = bytes * per;
     l->blocks = hg_grid_blocks(tiles);
 }

@@ -24,6 +24,7 @@ extern "C" {
 #endif
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
+#define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree kernel: one access per lane and input */
 
 /* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
 typedef struct {
@@ -42,6 +43,7 @@ typedef struct {
  */
 typedef struct {
     const void* in[HCOMM_GFX_MAX_RANKS];
+    const void* in2[HCOMM_GFX_MAX_RANKS]; /* tree only: buffer folded into in[b] before the tree, or NULL */
     void* out[HCOMM_GFX_MAX_RANKS];
     uint64_t off[HG_MAX_SEG];     /* byte offset applied to every in[] (and out[] in fan-out mode) */
     uint64_t out_off[HG_MAX_SEG]; /* byte offset into out[owner[s]] in single-output mode */
@@ -55,6 +57,7 @@ typedef struct {
     uint32_t store_final_first; /* store the final value to position 0's buffer */
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
     uint32_t tree;           /* 0 chain, 1 binary tree (k must be a power of two) */
+    uint32_t nout;           /* tree only: number of out[] entries that receive the result */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
 } HgFoldTable;

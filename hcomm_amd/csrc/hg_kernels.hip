@@ -373,6 +373,69 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     }
 }
 
+// ---- k-way tree fold (recursive halving) ---------------------------------------------------------
+//
+// K = 2^L block ranks.  For slice c, position q holds block rank c XOR bitrev(q); level l combines position q
+// (dst role) with q + 2^l - exactly the reduce every halving step performs (peer = rank XOR mask, mask from K/2
+// down to 1); each buffer receives the last value the step-wise replay would leave in it, and the root value
+// goes to every output.
+// A block rank with in2 != NULL first absorbs in2 (the odd neighbour folded in before the halving steps).
+
+template <int L> __device__ __forceinline__ constexpr uint32_t bitrev(uint32_t q)
+{
+    uint32_t r = 0;
+    for (int i = 0; i < L; ++i) r |= ((q >> i) & 1u) << (L - 1 - i);
+    return r;
+}
+
+template <class Item, int L>
+__device__ __forceinline__ void fold_tree_item(const HgFoldTable& tab, uint32_t s, uint64_t idx)
+{
+    typedef typename Item::V V;
+    constexpr uint32_t K = 1u << L;
+    const uint64_t off = tab.off[s];
+    const uint32_t c = tab.first[s];
+    V x[K];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) x[q] = Item::ld((const uint8_t*)tab.in[c ^ bitrev<L>(q)] + off, idx);
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint32_t b = c ^ bitrev<L>(q);
+        if (tab.in2[b]) x[q] = Item::op(x[q], Item::ld((const uint8_t*)tab.in2[b] + off, idx));
+    }
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (uint32_t q = 0; q < K; q += (2u << l)) x[q] = Item::op(x[q], x[q + (1u << l)]);
+    }
+    // What the step-wise replay leaves in each input buffer: an even position is overwritten at every level it
+    // takes part in and keeps the last result; an odd position only changes when it absorbed a neighbour.
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint32_t b = c ^ bitrev<L>(q);
+        if ((q & 1u) == 0u || tab.in2[b]) Item::st((uint8_t*)tab.in[b] + off, idx, x[q]);
+    }
+    for (uint32_t r = 0; r < tab.nout; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, x[0]);
+}
+
+template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    const uint32_t total = tab.tile_begin[tab.nseg];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
+        const uint64_t bytes = tab.bytes[s];
+        const uint64_t nvec = bytes >> 4;
+        if (v < nvec) fold_tree_item<VecItem<DT, OP>, L>(tab, s, v);
+        if (v - tid + HG_BLOCK > nvec) { // the segment's last tile also owns its element tail
+            const uint64_t e = (nvec << 4) / ES + tid;
+            if ((e + 1) * ES <= bytes) fold_tree_item<ElemItem<DT, OP>, L>(tab, s, e);
+        }
+    }
+}
+
 // ---- dispatch -----------------------------------------------------------------------------------
 
 int rc(hipError_t e) { return e == hipSuccess ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
@@ -411,6 +474,30 @@ template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFo
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
+}
+
+template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+{
+    switch (op) {
+        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        default: return HCCL_E_PARA;
+    }
+    return rc(hipGetLastError());
+}
+
+template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+{
+    switch (tab->k) {
+        case 2: return launch_tree_dt_l<DT, 1>(st, op, tab, blocks);
+        case 4: return launch_tree_dt_l<DT, 2>(st, op, tab, blocks);
+        case 8: return launch_tree_dt_l<DT, 3>(st, op, tab, blocks);
+        case 16: return launch_tree_dt_l<DT, 4>(st, op, tab, blocks);
+        case 32: return launch_tree_dt_l<DT, 5>(st, op, tab, blocks);
+        default: return HCCL_E_PARA;
+    }
 }
 
 #define HG_DISPATCH_DT(dtype, CALL)                   \
@@ -459,7 +546,11 @@ int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgS
 int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-    if (tab->tree) return HCCL_E_NOT_SUPPORT;
+    if (tab->tree) {
+#define CALL(DT) launch_tree_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks)
+        HG_DISPATCH_DT(dtype, CALL)
+#undef CALL
+    }
     if (acc_is_dst) {
 #define CALL(DT) launch_fold_dt<DT, true>((hipStream_t)stream, op, tab, (uint32_t)blocks)
         HG_DISPATCH_DT(dtype, CALL)

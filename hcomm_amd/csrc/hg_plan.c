@@ -149,6 +149,48 @@ static int fused_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const*
     return rc;
 }
 
+/* recursive halving-doubling allreduce as one tree launch (block ranks in the table, real ranks as outputs) */
+static int fused_rhd(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype, int op)
+{
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    uint32_t block = 1;
+    while ((block << 1) <= n) block <<= 1;
+    const uint32_t part1 = (n - block) * 2;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    int rc = HcommGfxCalcSlices(count, unit, block, sl);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    l->kind = HCOMM_GFX_KERNEL_TREE;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    HgFoldTable* f = &l->tab.fold;
+    f->tree = 1;
+    f->k = block;
+    f->nranks = block;
+    f->nout = n;
+    for (uint32_t b = 0; b < block; ++b) { /* block rank -> rank, recursive_halvingdoubling_base.cc:39-62 */
+        const uint32_t real = (b < part1 / 2) ? 2 * b : b + part1 / 2;
+        f->in[b] = in[real];
+        f->in2[b] = (b < part1 / 2) ? in[real + 1] : NULL;
+    }
+    for (uint32_t r = 0; r < n; ++r) f->out[r] = out[r];
+    for (uint32_t c = 0; c < block; ++c) {
+        if (sl[c].size == 0) continue;
+        const uint32_t s = f->nseg++;
+        f->off[s] = sl[c].offset;
+        f->bytes[s] = sl[c].size;
+        f->first[s] = (uint8_t)c;
+        f->owner[s] = (uint8_t)c;
+    }
+    if (f->nseg) {
+        hg_finish_fold(l);
+        rc = plan_push(l, p);
+    }
+    free(l);
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
                        int dtype, int op)
 {
@@ -163,6 +205,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_ring(p, n, in, out, count, dtype, op, 1, 1);
+        case HCOMM_GFX_ALG_ALLREDUCE_RHD:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_rhd(p, n, in, out, count, dtype, op);
         case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: return fused_mesh(p, n, in, out, count, dtype, op, 0);
         case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH:
             if (n == 1) return single_copy(p, out[0], in[0], total);

@@ -240,8 +240,8 @@ typedef enum {
        two-input dst = dst (op) src exactly as the reference emits it */
     HCOMM_GFX_LOWER_STEPWISE = 0,
     /* steps whose data dependences are element-wise are folded into k-way kernels that read every input
-       once and still store every intermediate value the step-wise replay stores, so the final contents
-       of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE */
+       once and store every value the step-wise replay leaves in a buffer (partials included), so the final
+       contents of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE */
     HCOMM_GFX_LOWER_FUSED = 1
 } HcommGfxLowering;
 

@@ -19,7 +19,7 @@ ALGS = {
     "mesh_rs": (h.Alg.REDUCE_SCATTER_MESH, oracle.ALG_RS_MESH),
     "ring_rs": (h.Alg.REDUCE_SCATTER_RING_STANDALONE, oracle.ALG_RS_RING_STANDALONE),
 }
-FUSABLE = {"ring_ar", "ring_rs_stage", "mesh_oneshot", "mesh_rs", "ring_rs"}
+FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs"}
 
 
 def say(*a):
@@ -86,6 +86,10 @@ CASES = [
     ("rhd_ar", 2, 12345, "int16", "sum"),
     ("rhd_ar", 1, 100, "int32", "sum"),
     ("rhd_ar", 12, 77777, "fp32", "sum"),
+    ("rhd_ar", 32, 100003, "bf16", "sum"),
+    ("rhd_ar", 31, 4099, "int16", "max"),
+    ("rhd_ar", 17, 100003, "fp32", "min"),
+    ("rhd_ar", 4, 65536, "fp32", "prod"),
     ("mesh_oneshot", 8, 2048, "fp16", "sum"),      # benchmark config 4, 4 KiB
     ("mesh_oneshot", 8, 1 << 21, "fp16", "sum"),   # benchmark config 4, 4 MiB
     ("mesh_oneshot", 8, 100003, "fp32", "sum"),

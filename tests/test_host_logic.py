@@ -227,16 +227,16 @@ def test_plan_argument_checks():
             mk(**kwargs)
         assert e.value.code == code, kwargs
     mk(dt=DT.BFP16, op=OP.PROD).destroy()
-    with pytest.raises(h.HcommError) as e:
-        mk(alg=h.Alg.ALLREDUCE_RHD, low=h.Lowering.FUSED)
-    assert e.value.code == R.E_NOT_SUPPORT
+    p = mk(alg=h.Alg.ALLREDUCE_RHD, low=h.Lowering.FUSED)
+    assert [r.kind for r in p.launches()] == [h.Kernel.TREE]
+    p.destroy()
 
 
 @pytest.mark.parametrize("name,alg,n,count,dt,launches,algo_bytes,moved_fused", [
     # the five benchmark configurations at full size: launch structure and byte accounting, no memory touched
     ("cfg1", h.Alg.ALLREDUCE_RING, 8, 1048576, DT.FP32, 15, 155189248, 23 * 4194304),
     ("cfg2", h.Alg.ALLREDUCE_RING, 8, 67108864, DT.BFP16, 15, 4966055936, 23 * 134217728),
-    ("cfg3", h.Alg.ALLREDUCE_RHD, 16, 33554432, DT.INT32, 9, 10334765056, None),
+    ("cfg3", h.Alg.ALLREDUCE_RHD, 16, 33554432, DT.INT32, 9, 10334765056, 40 * 134217728),
     ("cfg4", h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 2097152, DT.FP16, 8, 8 * 23 * 4194304, 72 * 4194304),
     ("cfg5a", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.FP32, 6, 7200000216, 13 * 400000012),
     ("cfg5b", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.INT8, 6, 1800000054, 13 * 100000003),
@@ -255,8 +255,19 @@ def test_plan_structure_of_benchmark_configs(rec, name, alg, n, count, dt, launc
     if moved_fused is not None:
         p = h.Plan(alg, h.Lowering.FUSED, i, o, count, dt, op)
         assert (p.info.launches, p.info.algorithmicBytes, p.info.movedBytes) == (1, algo_bytes, moved_fused)
-        assert [r.kind for r in p.launches()] == [h.Kernel.CHAIN]
+        assert [r.kind for r in p.launches()] == [h.Kernel.TREE if alg == h.Alg.ALLREDUCE_RHD else h.Kernel.CHAIN]
         p.destroy()
+
+
+def test_fused_rhd_byte_accounting_with_fold():
+    """6 ranks: block of 4, block ranks 0 and 1 (ranks 0, 2) absorb ranks 1, 3.  Per element: 4 leaf reads + 2
+    neighbour reads + 2 stores on even positions + 6 outputs = 14 transfers, + 1 for each absorbing block rank
+    that sits on an odd position for the slice (block rank b is odd-positioned for slice c iff (b^c) & 2):
+    slices 0, 1 -> none; slices 2, 3 -> both."""
+    i, o = ptrs(6, 4096)
+    p = h.Plan(h.Alg.ALLREDUCE_RHD, h.Lowering.FUSED, i, o, 1024, DT.FP32, OP.SUM)
+    assert p.info.movedBytes == 2 * 1024 * 14 + 2 * 1024 * 16
+    p.destroy()
 
 
 def test_plan_run_checks(rec):
