@@ -246,7 +246,7 @@ def main():
     h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
-        metric = "HBM GB/s (% of peak) for simulated %d-rank %s %s %s" % (n, dtname, alg_name, opname)
+        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, alg_name, opname)
     out = {
         "metric": metric,
         "value": round(res["gbs"], 2),

@@ -14,6 +14,7 @@
 #include "hg_host.h"
 
 static uint64_t g_grid_cap = 0;
+static uint64_t g_small_bytes = 0;
 
 uint64_t hg_grid_blocks(uint64_t total_tiles)
 {
@@ -58,7 +59,22 @@ void hg_finish_fold(HgLaunch* l)
 {
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
-    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES : HG_TILE_BYTES;
+    if (!t->tree) {
+        /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
+        if (g_small_bytes == 0) {
+            const char* e = getenv("HCOMM_GFX_SMALL_BYTES");
+            g_small_bytes = e ? strtoull(e, NULL, 10) : 0;
+            if (g_small_bytes == 0) g_small_bytes = 1u << 20;
+        }
+        uint64_t largest = 0;
+        for (uint32_t s = 0; s < t->nseg; ++s)
+            if (t->bytes[s] > largest) largest = t->bytes[s];
+        /* measured cross-over with 8 ranks: 1 MiB per segment for read-only chains (mesh, k-way reduce), a
+         * quarter of that when every position also stores its partial (ring) */
+        const uint64_t limit = t->store_partials ? g_small_bytes / 4 : g_small_bytes;
+        t->small = (largest <= limit) ? 1u : 0u;
+    }
+    const uint64_t tile_bytes = (t->tree || t->small) ? HG_TREE_TILE_BYTES : HG_TILE_BYTES;
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
         tiles += (t->bytes[s] + tile_bytes - 1) / tile_bytes;

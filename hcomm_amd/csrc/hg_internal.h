@@ -24,7 +24,7 @@ extern "C" {
 #endif
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
-#define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree kernel: one access per lane and input */
+#define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree / small-message kernels: one access per lane and input */
 
 /* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
 typedef struct {
@@ -58,6 +58,7 @@ typedef struct {
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
     uint32_t tree;           /* 0 chain, 1 binary tree (k must be a power of two) */
     uint32_t nout;           /* tree only: number of out[] entries that receive the result */
+    uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
 } HgFoldTable;

@@ -373,6 +373,68 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     }
 }
 
+// ---- k-way chain fold, small messages ------------------------------------------------------------------
+//
+// Same result as k_fold_chain, shaped for latency instead of bandwidth: a 4 KiB tile per workgroup (more
+// workgroups for the same bytes) and the loads of eight inputs issued together, so that a launch costs about
+// one memory round trip per eight inputs instead of one per input.  The rank buffers of a plan never overlap,
+// which is what allows a load to be issued ahead of the partial stores of earlier positions.
+
+template <class Item, bool ACC_IS_DST>
+__device__ __forceinline__ void fold_chain_grouped(const HgFoldTable& tab, uint32_t s, uint64_t idx)
+{
+    typedef typename Item::V V;
+    constexpr uint32_t G = 8;
+    const uint64_t off = tab.off[s];
+    const uint32_t k = tab.k;
+    V acc = Item::zero();
+    for (uint32_t j0 = 0; j0 < k; j0 += G) {
+        V buf[G];
+#pragma unroll
+        for (uint32_t jj = 0; jj < G; ++jj) {
+            buf[jj] = Item::zero();
+            if (j0 + jj < k) buf[jj] = Item::ld((const uint8_t*)tab.in[fold_rank(tab, s, j0 + jj)] + off, idx);
+        }
+#pragma unroll
+        for (uint32_t jj = 0; jj < G; ++jj) {
+            const uint32_t j = j0 + jj;
+            if (j < k) {
+                if (j == 0) {
+                    acc = buf[0];
+                } else {
+                    acc = ACC_IS_DST ? Item::op(acc, buf[jj]) : Item::op(buf[jj], acc);
+                    if (tab.store_partials) Item::st((uint8_t*)tab.in[fold_rank(tab, s, j)] + off, idx, acc);
+                }
+            }
+        }
+    }
+    if (tab.store_final_first) Item::st((uint8_t*)tab.in[fold_rank(tab, s, 0)] + off, idx, acc);
+    if (tab.out_mode == 1) {
+        Item::st((uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s], idx, acc);
+    } else if (tab.out_mode == 2) {
+        for (uint32_t r = 0; r < tab.nranks; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, acc);
+    }
+}
+
+template <int DT, int OP, bool ACC_IS_DST>
+__global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    const uint32_t total = tab.tile_begin[tab.nseg];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
+        const uint64_t bytes = tab.bytes[s];
+        const uint64_t nvec = bytes >> 4;
+        if (v < nvec) fold_chain_grouped<VecItem<DT, OP>, ACC_IS_DST>(tab, s, v);
+        if (v - tid + HG_BLOCK > nvec) { // the segment's last tile also owns its element tail
+            const uint64_t e = (nvec << 4) / ES + tid;
+            if ((e + 1) * ES <= bytes) fold_chain_grouped<ElemItem<DT, OP>, ACC_IS_DST>(tab, s, e);
+        }
+    }
+}
+
 // ---- k-way tree fold (recursive halving) ---------------------------------------------------------
 //
 // K = 2^L block ranks.  For slice c, position q holds block rank c XOR bitrev(q); level l combines position q
@@ -466,11 +528,22 @@ template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Tab
 
 template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
 {
+    const dim3 g(blocks), b(HG_BLOCK);
+    if (tab->small) {
+        switch (op) {
+            case OP_SUM: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_SUM, AD>), g, b, 0, st, *tab); break;
+            case OP_PROD: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_PROD, AD>), g, b, 0, st, *tab); break;
+            case OP_MAX: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MAX, AD>), g, b, 0, st, *tab); break;
+            case OP_MIN: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MIN, AD>), g, b, 0, st, *tab); break;
+            default: return HCCL_E_PARA;
+        }
+        return rc(hipGetLastError());
+    }
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_fold_chain<DT, OP_SUM, AD>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_fold_chain<DT, OP_PROD, AD>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_fold_chain<DT, OP_MAX, AD>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_fold_chain<DT, OP_MIN, AD>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_fold_chain<DT, OP_SUM, AD>), g, b, 0, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_chain<DT, OP_PROD, AD>), g, b, 0, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_chain<DT, OP_MAX, AD>), g, b, 0, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_chain<DT, OP_MIN, AD>), g, b, 0, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
