@@ -21,7 +21,8 @@ __all__ = [
     "HcommThreadNotifyWaitOnThread", "HcommMemAlloc", "HcommMemFree", "HcommBatchModeStart", "HcommBatchModeEnd",
     "HcommGfxThreadSynchronize", "HcommGfxReduceKOnThread", "HcommGfxRecorderThreadAlloc", "launch_log",
     "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion",
-    "DTYPE_SIZE",
+    "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
+    "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
@@ -59,7 +60,7 @@ class CommEngine:
 
 class Alg:
     ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
-        REDUCE_SCATTER_RING_STANDALONE = range(6)
+        REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING = range(7)
 
 
 class Lowering:
@@ -88,6 +89,29 @@ class SchedOp(C.Structure):
     def astuple(self):
         return (self.step, self.kind, self.rank, self.dstBuf, self.dstOff, self.srcRank, self.srcBuf, self.srcOff,
                 self.bytes)
+
+
+class _DescRW(C.Structure):
+    _fields_ = [("len", C.c_uint64), ("dst", C.c_void_p), ("src", C.c_void_p)]
+
+
+class _DescReduce(C.Structure):
+    _fields_ = [("count", C.c_uint64), ("dst", C.c_void_p), ("src", C.c_void_p), ("reduceOp", C.c_int),
+                ("dataType", C.c_int)]
+
+
+class _DescInfo(C.Union):
+    _fields_ = [("raws", C.c_uint8 * 56), ("write", _DescRW), ("read", _DescRW), ("reduce", _DescReduce)]
+
+
+class BatchTransferDesc(C.Structure):
+    """HcommBatchTransferDesc (64 bytes)."""
+    _fields_ = [("transType", C.c_int), ("reserved", C.c_uint8 * 4), ("transferInfo", _DescInfo)]
+
+
+class TransferType:
+    INVALID, WRITE, WRITE_REDUCE, WRITE_WITH_NOTIFY, WRITE_REDUCE_WITH_NOTIFY, READ, READ_REDUCE, NOTIFY_RECORD = \
+        -1, 0, 1, 2, 3, 4, 5, 6
 
 
 class Slice(C.Structure):
@@ -134,16 +158,41 @@ _log_read = _sig("HcommGfxLaunchLogRead", _i32, _u64, C.POINTER(LaunchRecord), _
 HcommGfxLaunchLogClear = _sig("HcommGfxLaunchLogClear", _i32, _u64)
 _calc_slices = _sig("HcommGfxCalcSlices", _i32, _u64, _u32, _u32, C.POINTER(Slice))
 HcommGfxDataTypeSize = _sig("HcommGfxDataTypeSize", _u32, C.c_int)
-_plan_create = _sig("HcommGfxPlanCreate", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
-                    C.c_int, C.POINTER(_vp))
+_plan_create = _sig("HcommGfxPlanCreateStrided", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64,
+                    _u64, C.c_int, C.c_int, C.POINTER(_vp))
 _plan_run = _sig("HcommGfxPlanRun", _i32, _vp, _u64)
 _plan_run_range = _sig("HcommGfxPlanRunRange", _i32, _vp, _u64, _u32, _u32)
 _plan_destroy = _sig("HcommGfxPlanDestroy", _i32, _vp)
 _plan_info = _sig("HcommGfxPlanGetInfo", _i32, _vp, C.POINTER(PlanInfo))
 _plan_launch = _sig("HcommGfxPlanGetLaunch", _i32, _vp, _u32, C.POINTER(LaunchRecord))
-_sched_emit = _sig("HcommGfxScheduleEmit", _i32, C.c_int, _u32, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+_sched_emit = _sig("HcommGfxScheduleEmitStrided", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
                    C.POINTER(_u64))
+HcommWriteOnThread = _sig("HcommWriteOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
+HcommReadOnThread = _sig("HcommReadOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
+HcommWriteReduceOnThread = _sig("HcommWriteReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
+HcommReadReduceOnThread = _sig("HcommReadReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
+_batch_transfer = _sig("HcommBatchTransferOnThread", _i32, _u64, _u64, C.POINTER(BatchTransferDesc), _u32)
 _version = _sig("HcommGfxVersion", C.c_char_p)
+
+
+def HcommBatchTransferOnThread(thread, channel, descs):
+    arr = (BatchTransferDesc * max(len(descs), 1))(*descs)
+    return _batch_transfer(thread, channel, arr if descs else None, len(descs))
+
+
+def desc_copy(dst, src, nbytes, read=False):
+    d = BatchTransferDesc()
+    d.transType = TransferType.READ if read else TransferType.WRITE
+    d.transferInfo.write.len, d.transferInfo.write.dst, d.transferInfo.write.src = nbytes, dst, src
+    return d
+
+
+def desc_reduce(dst, src, count, dtype, op, read=False):
+    d = BatchTransferDesc()
+    d.transType = TransferType.READ_REDUCE if read else TransferType.WRITE_REDUCE
+    r = d.transferInfo.reduce
+    r.count, r.dst, r.src, r.reduceOp, r.dataType = count, dst, src, op, dtype
+    return d
 
 
 def HcommGfxVersion():
@@ -206,23 +255,24 @@ def calc_slices(count, unit, n):
     return [(s.offset, s.size) for s in sl]
 
 
-def schedule_emit(alg, n_ranks, count, dtype):
+def schedule_emit(alg, n_ranks, count, dtype, stride=0):
     n = _u64(0)
-    check(_sched_emit(alg, n_ranks, count, dtype, None, 0, C.byref(n)), "HcommGfxScheduleEmit")
+    check(_sched_emit(alg, n_ranks, count, stride, dtype, None, 0, C.byref(n)), "HcommGfxScheduleEmit")
     ops = (SchedOp * max(n.value, 1))()
-    check(_sched_emit(alg, n_ranks, count, dtype, ops, n.value, C.byref(n)), "HcommGfxScheduleEmit")
+    check(_sched_emit(alg, n_ranks, count, stride, dtype, ops, n.value, C.byref(n)), "HcommGfxScheduleEmit")
     return [ops[i].astuple() for i in range(n.value)]
 
 
 class Plan:
     """HcommGfxPlan: build once, run many."""
 
-    def __init__(self, alg, lowering, in_ptrs, out_ptrs, count, dtype, op):
+    def __init__(self, alg, lowering, in_ptrs, out_ptrs, count, dtype, op, stride=0):
         n = len(in_ptrs)
         self._in = (_vp * n)(*in_ptrs)
         self._out = (_vp * n)(*out_ptrs) if out_ptrs is not None else None
         p = _vp(0)
-        check(_plan_create(alg, lowering, n, self._in, self._out, count, dtype, op, C.byref(p)), "HcommGfxPlanCreate")
+        check(_plan_create(alg, lowering, n, self._in, self._out, count, stride, dtype, op, C.byref(p)),
+              "HcommGfxPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

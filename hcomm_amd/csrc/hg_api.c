@@ -12,6 +12,8 @@
 
 #include "hg_host.h"
 
+_Static_assert(sizeof(HcommBatchTransferDesc) == 64, "HcommBatchTransferDesc must keep the reference's 64-byte layout");
+
 #define HG_LOG_MAX (1u << 16)
 #define HG_TOUCHED_MAX 64u
 
@@ -364,6 +366,107 @@ int32_t HcommLocalReduceOnThread(
     o.src = src;
     o.bytes = count * HcommGfxDataTypeSize(dataType); /* cpu_primitives_c_adpt.cc:109 */
     return record_or_run(t, &o);
+}
+
+/* ---- inter-rank twins: the same two operations with one operand in a peer's buffer -------------------- */
+
+static int32_t channel_op(ThreadHandle thread, ChannelHandle channel, int is_reduce, void* dst, const void* src,
+                          uint64_t n, HcommDataType dataType, HcommReduceOp reduceOp)
+{
+    if (!dst) return HCCL_E_PTR;
+    if (!src) return HCCL_E_PTR;
+    if (is_reduce && !hg_reduce_supported((int)dataType, (int)reduceOp, allow_prod())) return HCCL_E_PARA;
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (!channel) return HCCL_E_PTR;
+    HgOp o;
+    memset(&o, 0, sizeof(o));
+    o.is_reduce = (uint8_t)is_reduce;
+    o.dtype = is_reduce ? (uint8_t)dataType : 255;
+    o.op = is_reduce ? (uint8_t)reduceOp : 255;
+    o.dst = dst;
+    o.src = src;
+    o.bytes = is_reduce ? n * HcommGfxDataTypeSize(dataType) : n;
+    return record_or_run(t, &o);
+}
+
+int32_t HcommWriteOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len)
+{
+    return channel_op(thread, channel, 0, dst, src, len, HCOMM_DATA_TYPE_RESERVED, HCOMM_REDUCE_RESERVED);
+}
+
+int32_t HcommReadOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len)
+{
+    return channel_op(thread, channel, 0, dst, src, len, HCOMM_DATA_TYPE_RESERVED, HCOMM_REDUCE_RESERVED);
+}
+
+int32_t HcommWriteReduceOnThread(
+    ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp)
+{
+    return channel_op(thread, channel, 1, dst, src, count, dataType, reduceOp);
+}
+
+int32_t HcommReadReduceOnThread(
+    ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp)
+{
+    return channel_op(thread, channel, 1, dst, src, count, dataType, reduceOp);
+}
+
+int32_t HcommBatchTransferOnThread(
+    ThreadHandle thread, ChannelHandle channel, const HcommBatchTransferDesc* transferDescs, uint32_t transferDescNum)
+{
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    if (!channel) return HCCL_E_PTR;
+    if (transferDescNum == 0) return HCCL_SUCCESS;
+    if (!transferDescs) return HCCL_E_PTR;
+    HgOp* ops = (HgOp*)calloc(transferDescNum, sizeof(HgOp));
+    if (!ops) return HCCL_E_MEMORY;
+    int32_t ret = HCCL_SUCCESS;
+    for (uint32_t i = 0; i < transferDescNum && ret == HCCL_SUCCESS; ++i) {
+        const HcommBatchTransferDesc* d = &transferDescs[i];
+        HgOp* o = &ops[i];
+        switch (d->transType) {
+            case HCOMM_TRANSFER_TYPE_WRITE:
+            case HCOMM_TRANSFER_TYPE_READ:
+                o->dtype = 255;
+                o->op = 255;
+                o->dst = d->transferInfo.write.dst;
+                o->src = d->transferInfo.write.src;
+                o->bytes = d->transferInfo.write.len;
+                break;
+            case HCOMM_TRANSFER_TYPE_WRITE_REDUCE:
+            case HCOMM_TRANSFER_TYPE_READ_REDUCE:
+                if (!hg_reduce_supported((int)d->transferInfo.reduce.dataType, (int)d->transferInfo.reduce.reduceOp,
+                                         allow_prod())) {
+                    ret = HCCL_E_PARA;
+                    break;
+                }
+                o->is_reduce = 1;
+                o->dtype = (uint8_t)d->transferInfo.reduce.dataType;
+                o->op = (uint8_t)d->transferInfo.reduce.reduceOp;
+                o->dst = d->transferInfo.reduce.dst;
+                o->src = d->transferInfo.reduce.src;
+                o->bytes = d->transferInfo.reduce.count * HcommGfxDataTypeSize(d->transferInfo.reduce.dataType);
+                break;
+            case HCOMM_TRANSFER_TYPE_WRITE_WITH_NOTIFY:
+            case HCOMM_TRANSFER_TYPE_WRITE_REDUCE_WITH_NOTIFY:
+            case HCOMM_TRANSFER_TYPE_NOTIFY_RECORD: ret = HCCL_E_NOT_SUPPORT; break;
+            default: ret = HCCL_E_PARA; break;
+        }
+        if (ret == HCCL_SUCCESS && (!o->dst || !o->src)) ret = HCCL_E_PTR;
+    }
+    if (ret == HCCL_SUCCESS) {
+        if (g_ctx.batching) {
+            for (uint32_t i = 0; i < transferDescNum && ret == HCCL_SUCCESS; ++i) ret = record_or_run(t, &ops[i]);
+        } else {
+            ret = hg_coalesce(ops, transferDescNum, emit_to_thread, t);
+        }
+    }
+    free(ops);
+    return ret;
 }
 
 int32_t HcommBatchModeStart(const char* batchTag)

@@ -58,6 +58,7 @@ typedef struct {
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
     uint32_t tree;           /* 0 chain, 1 binary tree (k must be a power of two) */
     uint32_t nout;           /* tree only: number of out[] entries that receive the result */
+    uint32_t ascending;      /* chain only: position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s] */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];

@@ -260,6 +260,10 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 
 __device__ __forceinline__ uint32_t fold_rank(const HgFoldTable& t, uint32_t s, uint32_t j)
 {
+    if (t.ascending) {
+        if (j == 0) return t.first[s];
+        return (j - 1 < t.first[s]) ? j - 1 : j;
+    }
     int32_t r = (int32_t)t.first[s] + (int32_t)j * t.stride;
     const int32_t n = (int32_t)t.nranks;
     r %= n;

@@ -87,14 +87,14 @@ static int single_copy(HcommGfxPlan* p, void* dst, const void* src, uint64_t byt
 }
 
 /* ring allreduce / reduce-scatter: slice c travels c+1 -> c+2 -> ... -> c, every hop storing its partial */
-static int fused_ring(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype,
-                      int op, int out_mode, int standalone)
+static int fused_ring(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count,
+                      uint64_t stride, int dtype, int op, int out_mode, int standalone)
 {
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
     if (standalone) {
         for (uint32_t i = 0; i < n; ++i) {
-            sl[i].offset = (uint64_t)i * count * unit;
+            sl[i].offset = (uint64_t)i * stride * unit;
             sl[i].size = count * unit;
         }
     } else {
@@ -124,10 +124,11 @@ static int fused_ring(HcommGfxPlan* p, uint32_t n, void* const* in, void* const*
     return rc;
 }
 
-static int fused_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype,
-                      int op, int scatter)
+static int fused_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count,
+                      uint64_t stride, int dtype, int op, int scatter, int ascending)
 {
-    const uint64_t sz = count * HcommGfxDataTypeSize((HcommDataType)dtype);
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    const uint64_t sz = count * unit;
     if (sz == 0) return HCCL_SUCCESS;
     HgLaunch* l = new_fold(dtype, op, 1, n, in, out);
     if (!l) return HCCL_E_MEMORY;
@@ -135,9 +136,10 @@ static int fused_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const*
     f->out_mode = 1;
     f->stride = scatter ? -1 : 1;     /* reduce-scatter visits r-1, r-2, ...; one-shot visits r+1, r+2, ... */
     f->store_final_first = scatter ? 1 : 0; /* reduce-scatter accumulates in in[r][slice r] before copying out */
+    f->ascending = ascending ? 1u : 0u;
     f->nseg = n;
     for (uint32_t r = 0; r < n; ++r) {
-        f->off[r] = scatter ? (uint64_t)r * sz : 0;
+        f->off[r] = scatter ? (uint64_t)r * stride * unit : 0;
         f->bytes[r] = sz;
         f->first[r] = (uint8_t)r;
         f->owner[r] = (uint8_t)r;
@@ -192,26 +194,28 @@ static int fused_rhd(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* 
 }
 
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
-                       int dtype, int op)
+                       uint64_t stride, int dtype, int op)
 {
     const uint64_t total = count * HcommGfxDataTypeSize((HcommDataType)dtype);
     switch (alg) {
         case HCOMM_GFX_ALG_ALLREDUCE_RING:
             if (n == 1) return single_copy(p, out[0], in[0], total);
-            return fused_ring(p, n, in, out, count, dtype, op, 2, 0);
+            return fused_ring(p, n, in, out, count, count, dtype, op, 2, 0);
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING:
             if (n == 1) return HCCL_SUCCESS;
-            return fused_ring(p, n, in, out, count, dtype, op, 0, 0);
+            return fused_ring(p, n, in, out, count, count, dtype, op, 0, 0);
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
-            return fused_ring(p, n, in, out, count, dtype, op, 1, 1);
+            return fused_ring(p, n, in, out, count, stride, dtype, op, 1, 1);
         case HCOMM_GFX_ALG_ALLREDUCE_RHD:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rhd(p, n, in, out, count, dtype, op);
-        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: return fused_mesh(p, n, in, out, count, dtype, op, 0);
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: return fused_mesh(p, n, in, out, count, count, dtype, op, 0, 0);
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING:
+            return fused_mesh(p, n, in, out, count, count, dtype, op, 0, 1);
         case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH:
             if (n == 1) return single_copy(p, out[0], in[0], total);
-            return fused_mesh(p, n, in, out, count, dtype, op, 1);
+            return fused_mesh(p, n, in, out, count, stride, dtype, op, 1, 0);
         default: return HCCL_E_NOT_SUPPORT;
     }
 }
@@ -221,6 +225,13 @@ static int in_place(int alg) { return alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING; 
 int32_t HcommGfxPlanCreate(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
     uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    return HcommGfxPlanCreateStrided(alg, lowering, nRanks, in, out, count, 0, dataType, reduceOp, plan);
+}
+
+int32_t HcommGfxPlanCreateStrided(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
 {
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
@@ -238,7 +249,8 @@ int32_t HcommGfxPlanCreate(
         }
     }
     HgOpList ol;
-    int rc = hg_schedule(&ol, (int)alg, nRanks, count, (int)dataType);
+    if (strideCount == 0) strideCount = count;
+    int rc = hg_schedule(&ol, (int)alg, nRanks, count, strideCount, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
     if (!p) {
@@ -251,7 +263,7 @@ int32_t HcommGfxPlanCreate(
     if (lowering == HCOMM_GFX_LOWER_STEPWISE)
         rc = lower_stepwise(p, &ol, in, out, (int)dataType, (int)reduceOp);
     else
-        rc = lower_fused(p, (int)alg, nRanks, in, out, count, (int)dataType, (int)reduceOp);
+        rc = lower_fused(p, (int)alg, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
     hg_oplist_free(&ol);
     if (rc != HCCL_SUCCESS) {
         HcommGfxPlanDestroy(p);

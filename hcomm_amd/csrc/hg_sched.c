@@ -112,14 +112,17 @@ static int sched_allreduce_ring(HgOpList* l, uint32_t n, uint64_t count, uint32_
     return HCCL_SUCCESS;
 }
 
-static int sched_rs_ring_standalone(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+/* Input slice i of the scatter algorithms starts stride elements after slice i-1
+ * (displs[i] = strideLen * i * unitSize, src/legacy/ascend910/framework/device/aicpu_kfc/algorithm/
+ * aicpu_reduce_scatter.cc:78-80); stride == count is the dense layout of reduce_scatter_ring.cc:140-157. */
+static int sched_rs_ring_standalone(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
 {
     const uint64_t sz = count * unit;
     if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz); /* reduce_scatter_ring.cc:103-109 */
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
     memset(sl, 0, sizeof(sl));
     for (uint32_t i = 0; i < n; ++i) { /* reduce_scatter_ring.cc:140-157; the output holds one slice, so offset 0 */
-        sl[i].offset = (uint64_t)i * sz;
+        sl[i].offset = (uint64_t)i * stride * unit;
         sl[i].size = sz;
     }
     CHK(ring_rs(l, n, sl, 0));
@@ -187,19 +190,27 @@ static int sched_allreduce_rhd(HgOpList* l, uint32_t n, uint64_t count, uint32_t
     return HCCL_SUCCESS;
 }
 
-static int sched_allreduce_mesh_oneshot(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+static int sched_allreduce_mesh_oneshot(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit, int ascending)
 {
     /* temp_all_reduce/all_reduce_mesh_oneshot.cc:78-121: out = in, then reduce the peers' copies in the
      * order r+1, r+2, ..., r-1.  A peer's communication buffer holds a copy of its input (:96-100), which
      * the simulation reads as in[peer] directly. */
     const uint64_t total = count * unit;
     for (uint32_t r = 0; r < n; ++r) CHK(push(l, 0, COPY, r, OUT, 0, r, IN, 0, total));
+    if (ascending) {
+        /* src/legacy/ascend950/service/collective/alg/coll_alg_factory/alg_template/ins_alg_template/
+         * ins_temp_all_reduce_mesh_1D_one_shot.cc:102,148-161: out = in, then every other rank's input in
+         * ascending rank order (the gathered scratch copies are read as in[peer] directly) */
+        for (uint32_t k = 1; k < n; ++k)
+            for (uint32_t r = 0; r < n; ++r) CHK(push(l, k, REDUCE, r, OUT, 0, (k - 1 < r) ? k - 1 : k, IN, 0, total));
+        return HCCL_SUCCESS;
+    }
     for (uint32_t k = 1; k < n; ++k)
         for (uint32_t r = 0; r < n; ++r) CHK(push(l, k, REDUCE, r, OUT, 0, (r + k) % n, IN, 0, total));
     return HCCL_SUCCESS;
 }
 
-static int sched_rs_mesh(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+static int sched_rs_mesh(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
 {
     /* temp_reduce_scatter/reduce_scatter_mesh.cc:51-128 (stream 0): round k receives slice r from rank r-k
      * (ForwardRank, base/inc/reduce_scatter_mesh_pub.h:31-37) and reduces it into in[r][slice r]; then
@@ -208,15 +219,20 @@ static int sched_rs_mesh(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
     if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz);
     for (uint32_t k = 1; k < n; ++k)
         for (uint32_t r = 0; r < n; ++r)
-            CHK(push(l, k - 1, REDUCE, r, IN, (uint64_t)r * sz, modn((int64_t)r - k, n), IN, (uint64_t)r * sz, sz));
-    for (uint32_t r = 0; r < n; ++r) CHK(push(l, n - 1, COPY, r, OUT, 0, r, IN, (uint64_t)r * sz, sz));
+            CHK(push(l, k - 1, REDUCE, r, IN, (uint64_t)r * stride * unit, modn((int64_t)r - k, n), IN,
+                     (uint64_t)r * stride * unit, sz));
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, n - 1, COPY, r, OUT, 0, r, IN, (uint64_t)r * stride * unit, sz));
     return HCCL_SUCCESS;
 }
 
-int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, int dtype)
+int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
     if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (stride == 0) stride = count;
+    if (stride < count) return HCCL_E_PARA;
+    if (stride != count && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_MESH && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE)
+        return HCCL_E_PARA;
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
     if (unit == 0) return HCCL_E_PARA;
     int rc;
@@ -224,9 +240,10 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, int dtype)
         case HCOMM_GFX_ALG_ALLREDUCE_RING: rc = sched_allreduce_ring(l, n, count, unit, 1); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING: rc = sched_allreduce_ring(l, n, count, unit, 0); break;
         case HCOMM_GFX_ALG_ALLREDUCE_RHD: rc = sched_allreduce_rhd(l, n, count, unit); break;
-        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: rc = sched_allreduce_mesh_oneshot(l, n, count, unit); break;
-        case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH: rc = sched_rs_mesh(l, n, count, unit); break;
-        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT: rc = sched_allreduce_mesh_oneshot(l, n, count, unit, 0); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING: rc = sched_allreduce_mesh_oneshot(l, n, count, unit, 1); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH: rc = sched_rs_mesh(l, n, count, stride, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, stride, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
@@ -237,9 +254,16 @@ int32_t HcommGfxScheduleEmit(
     HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType, HcommGfxSchedOp* ops,
     uint64_t cap, uint64_t* n)
 {
+    return HcommGfxScheduleEmitStrided(alg, nRanks, count, 0, dataType, ops, cap, n);
+}
+
+int32_t HcommGfxScheduleEmitStrided(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t strideCount, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
     if (!n) return HCCL_E_PTR;
     HgOpList l;
-    int rc = hg_schedule(&l, (int)alg, nRanks, count, (int)dataType);
+    int rc = hg_schedule(&l, (int)alg, nRanks, count, strideCount, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     *n = l.n;
     if (ops) {

@@ -13,7 +13,8 @@ typedef struct {
 } HgOpList;
 
 /* Fill `l` with the op list of `alg`; the caller releases it with hg_oplist_free. */
-int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, int dtype);
+/* stride: elements between consecutive ranks' slices in the input of the scatter algorithms (0 = count). */
+int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype);
 void hg_oplist_free(HgOpList* l);
 
 #endif

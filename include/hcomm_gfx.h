@@ -148,6 +148,90 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);
 
+/*
+ * Inter-rank twins of the two local primitives.  Replace include/hcomm_primitives.h:231-246,291-306 (host
+ * adapter cpu_primitives_c_adpt.cc:284-318,332-384,490-565).  Same arithmetic with one operand on a peer:
+ *   Write        peer dst[0..len) = local src          WriteReduce  peer dst[i] = dst[i] (op) local src[i]
+ *   Read         local dst[0..len) = peer src          ReadReduce   local dst[i] = dst[i] (op) peer src[i]
+ * With every simulated rank in the HBM of one GPU, a peer buffer is directly addressable and the channel is an
+ * opaque non-zero token.  Check order as the reference: dst NULL, src NULL -> HCCL_E_PTR; unsupported
+ * type / op -> HCCL_E_PARA; thread 0 -> HCCL_E_PTR; then channel 0 -> HCCL_E_PTR.  Batch mode applies.
+ */
+int32_t HcommWriteOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len);
+int32_t HcommReadOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len);
+int32_t HcommWriteReduceOnThread(
+    ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp);
+int32_t HcommReadReduceOnThread(
+    ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp);
+
+/* include/hcomm_primitives.h:77-86 */
+typedef enum {
+    HCOMM_TRANSFER_TYPE_INVALID = -1,
+    HCOMM_TRANSFER_TYPE_WRITE = 0,
+    HCOMM_TRANSFER_TYPE_WRITE_REDUCE = 1,
+    HCOMM_TRANSFER_TYPE_WRITE_WITH_NOTIFY = 2,
+    HCOMM_TRANSFER_TYPE_WRITE_REDUCE_WITH_NOTIFY = 3,
+    HCOMM_TRANSFER_TYPE_READ = 4,
+    HCOMM_TRANSFER_TYPE_READ_REDUCE = 5,
+    HCOMM_TRANSFER_TYPE_NOTIFY_RECORD = 6
+} HcommTransferType;
+
+/* include/hcomm_primitives.h:91-131: 64 bytes = type, 4 reserved, 56-byte union; identical layout */
+typedef struct {
+    HcommTransferType transType;
+    uint8_t reserved[4];
+    union {
+        uint8_t raws[56];
+        struct {
+            uint64_t len;
+            void* dst;
+            void* src;
+        } write;
+        struct {
+            uint64_t len;
+            void* dst;
+            void* src;
+        } read;
+        struct {
+            uint64_t count;
+            void* dst;
+            void* src;
+            HcommReduceOp reduceOp;
+            HcommDataType dataType;
+        } reduce;
+        struct {
+            uint32_t notifyIdx;
+        } notifyRecord;
+        struct {
+            uint64_t len;
+            void* dst;
+            void* src;
+            uint32_t notifyIdx;
+        } writeWithNotify;
+        struct {
+            uint64_t count;
+            void* dst;
+            void* src;
+            HcommReduceOp reduceOp;
+            HcommDataType dataType;
+            uint32_t notifyIdx;
+        } writeReduceWithNotify;
+    } transferInfo;
+} HcommBatchTransferDesc;
+
+/*
+ * Submit an array of descriptors as one batch.  Replaces include/hcomm_primitives.h:393-394.  The reference's
+ * host adapter forwards this call to NIC plugins only and otherwise returns HCCL_E_NOT_SUPPORT
+ * (cpu_primitives_c_adpt.cc:320-330); here WRITE / READ / WRITE_REDUCE / READ_REDUCE descriptors are executed,
+ * in array order, with the same merging of independent operations into single launches as batch mode.
+ * The three notify-carrying types -> HCCL_E_NOT_SUPPORT (nothing is submitted).  transferDescs NULL with a
+ * non-zero count -> HCCL_E_PTR.  Every descriptor is validated before anything is enqueued.
+ */
+int32_t HcommBatchTransferOnThread(
+    ThreadHandle thread, ChannelHandle channel, const HcommBatchTransferDesc* transferDescs, uint32_t transferDescNum);
+
 /* Device memory.  Replaces include/hcomm_res.h:69-71.  ptr NULL -> HCCL_E_PTR, size 0 -> HCCL_E_PARA. */
 HcommResult HcommMemAlloc(void** ptr, size_t size);
 HcommResult HcommMemFree(void* ptr);
@@ -232,7 +316,11 @@ typedef enum {
     HCOMM_GFX_ALG_REDUCE_SCATTER_MESH = 4,
     /* stand-alone ReduceScatterRing: temp_reduce_scatter/reduce_scatter_ring.cc:96-180; count = per-rank
        OUTPUT count, input holds N*count, result written to out[r][0..count) */
-    HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE = 5
+    HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE = 5,
+    /* InsTempAllReduceMesh1DOneShot: src/legacy/ascend950/service/collective/alg/coll_alg_factory/alg_template/
+       ins_alg_template/ins_temp_all_reduce_mesh_1D_one_shot.cc:86-164 - out = in[r], then the other ranks'
+       inputs in ascending rank order (the legacy one-shot folds them in the order r+1, r+2, ...) */
+    HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING = 6
 } HcommGfxAlgorithm;
 
 typedef enum {
@@ -277,6 +365,17 @@ int32_t HcommGfxPlanCreate(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
     uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
+/*
+ * As HcommGfxPlanCreate, for the two stand-alone reduce-scatter algorithms with a strided input: rank i's
+ * slice starts strideCount elements after rank i-1's (displs[i] = strideLen * i * unitSize,
+ * src/legacy/ascend910/framework/device/aicpu_kfc/algorithm/aicpu_reduce_scatter.cc:78-80), so the input
+ * buffer holds (nRanks-1)*strideCount + count elements.  strideCount 0 means count (dense);
+ * strideCount < count, or a stride with any other algorithm -> HCCL_E_PARA.
+ */
+int32_t HcommGfxPlanCreateStrided(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+
 /* Enqueue every launch of the plan on the thread, in order.  May be called any number of times. */
 int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread);
 
@@ -320,6 +419,10 @@ typedef struct {
 int32_t HcommGfxScheduleEmit(
     HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType, HcommGfxSchedOp* ops,
     uint64_t cap, uint64_t* n);
+
+int32_t HcommGfxScheduleEmitStrided(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t strideCount, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
 
 /* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */
 const char* HcommGfxVersion(void);

@@ -16,7 +16,7 @@ REF_PATH = os.path.join(HERE, "_ref", "libhcomm_ref.so")
 SUM, PROD, MAX, MIN = 0, 1, 2, 3
 I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
 ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
-    ALG_RS_RING_STANDALONE = range(6)
+    ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING = range(7)
 
 # storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
 NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
@@ -54,6 +54,8 @@ def lib():
             build()
         L = C.CDLL(LIB_PATH)
         L.orc_set_threads.argtypes = [C.c_int]
+        L.orc_set_stride.argtypes = [C.c_uint64]
+        L.orc_set_stride.restype = None
         L.orc_get_threads.restype = C.c_int
         L.orc_f16_to_f32.restype = C.c_float
         L.orc_f16_to_f32.argtypes = [C.c_uint16]
@@ -156,21 +158,30 @@ def slices_rhd(data_bytes, block):
     return [(s.offset, s.size) for s in sl]
 
 
-def trace(alg, n, count, dtype):
-    total = lib().orc_trace(alg, n, count, dtype, None, 0)
-    if total < 0:
-        raise ValueError("orc_trace rc=%d" % total)
-    ops = (OrcOp * max(total, 1))()
-    lib().orc_trace(alg, n, count, dtype, ops, total)
+def trace(alg, n, count, dtype, stride=0):
+    lib().orc_set_stride(stride)
+    try:
+        total = lib().orc_trace(alg, n, count, dtype, None, 0)
+        if total < 0:
+            raise ValueError("orc_trace rc=%d" % total)
+        ops = (OrcOp * max(total, 1))()
+        lib().orc_trace(alg, n, count, dtype, ops, total)
+    finally:
+        lib().orc_set_stride(0)
     return [ops[i].astuple() for i in range(total)]
 
 
-def run(alg, ins, outs, count, dtype, op):
-    """Execute a collective in place on lists of numpy arrays (one per rank)."""
+def run(alg, ins, outs, count, dtype, op, stride=0):
+    """Execute a collective in place on lists of numpy arrays (one per rank).  stride: elements between the
+    input slices of the scatter algorithms (0 = dense)."""
     n = len(ins)
     a = (C.c_void_p * n)(*[x.ctypes.data for x in ins])
     b = (C.c_void_p * n)(*[x.ctypes.data for x in outs])
-    rc = lib().orc_run(alg, n, a, b, count, dtype, op)
+    lib().orc_set_stride(stride)
+    try:
+        rc = lib().orc_run(alg, n, a, b, count, dtype, op)
+    finally:
+        lib().orc_set_stride(0)
     if rc:
         raise ValueError("orc_run rc=%d" % rc)
 

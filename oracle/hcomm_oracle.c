@@ -390,7 +390,7 @@ static void prog_allreduce_ring(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t
     if (gather) prog_ring_ag(t, rank, n, sl, n - 1);
 }
 
-static void prog_rs_ring_standalone(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+static void prog_rs_ring_standalone(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
 {
     const uint64_t sz = count * unit;
     if (n == 1) { /* reduce_scatter_ring.cc:103-109 */
@@ -398,9 +398,12 @@ static void prog_rs_ring_standalone(OrcTrace* t, uint32_t rank, uint32_t n, uint
         return;
     }
     OrcSlice sl[ORC_MAX_RANKS], osl[ORC_MAX_RANKS];
-    for (uint32_t i = 0; i < n; i++) { /* :140-157; input larger than output -> output offset 0 */
+    /* :140-157 (input larger than output -> output offset 0), with the strided input layout of the MC2 path:
+     * displs[i] = strideLen * i * unitSize (src/legacy/ascend910/framework/device/aicpu_kfc/algorithm/
+     * aicpu_reduce_scatter.cc:78-80); stride == count is the dense default */
+    for (uint32_t i = 0; i < n; i++) {
         sl[i].size = sz;
-        sl[i].offset = (uint64_t)i * sz;
+        sl[i].offset = (uint64_t)i * stride * unit;
         osl[i].size = sz;
         osl[i].offset = 0;
     }
@@ -492,8 +495,24 @@ static void prog_allreduce_mesh_oneshot(OrcTrace* t, uint32_t rank, uint32_t n, 
     }
 }
 
-/* ReduceScatterMesh, tpl/temp_reduce_scatter/reduce_scatter_mesh.cc:51-128 (stream index 0), :131-215 */
-static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+/* InsTempAllReduceMesh1DOneShot::RunAllReduce, src/legacy/ascend950/service/collective/alg/coll_alg_factory/
+ * alg_template/ins_alg_template/ins_temp_all_reduce_mesh_1D_one_shot.cc:86-164: copy input to output (:102), gather
+ * every peer's input into scratch slots (:105-141), then reduce the slots into the output in ascending rank
+ * order, skipping the own rank (:148-161).  With two buffers per rank slot[peer] is read as in[peer]. */
+static void prog_allreduce_mesh_ascending(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    emit(t, 0, K_COPY, rank, B_OUT, 0, rank, B_IN, 0, total);
+    uint32_t step = 1;
+    for (uint32_t cur = 0; cur < n; cur++) {
+        if (cur == rank) continue;
+        emit(t, step++, K_REDUCE, rank, B_OUT, 0, cur, B_IN, 0, total);
+    }
+}
+
+/* ReduceScatterMesh, tpl/temp_reduce_scatter/reduce_scatter_mesh.cc:51-128 (stream index 0), :131-215; the
+ * input slice of rank i starts at i * stride elements (aicpu_reduce_scatter.cc:78-80), stride == count by default */
+static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
 {
     const uint64_t sz = count * unit;
     if (n == 1) { /* :152-157 */
@@ -504,9 +523,9 @@ static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count,
     for (uint32_t round = 1; round < n; round++) {
         const uint32_t src = (rank + n - round) % n; /* ForwardRank, tpl/../inc/reduce_scatter_mesh_pub.h:31-37 */
         /* RunDestRducer :35-49: dst = own input slice `rank`, remote offset = same slice */
-        emit(t, step++, K_REDUCE, rank, B_IN, (uint64_t)rank * sz, src, B_IN, (uint64_t)rank * sz, sz);
+        emit(t, step++, K_REDUCE, rank, B_IN, (uint64_t)rank * stride * unit, src, B_IN, (uint64_t)rank * stride * unit, sz);
     }
-    emit(t, step, K_COPY, rank, B_OUT, 0, rank, B_IN, (uint64_t)rank * sz, sz); /* :199-211 */
+    emit(t, step, K_COPY, rank, B_OUT, 0, rank, B_IN, (uint64_t)rank * stride * unit, sz); /* :199-211 */
 }
 
 enum {
@@ -515,7 +534,8 @@ enum {
     ORC_ALG_ALLREDUCE_RHD = 2,
     ORC_ALG_ALLREDUCE_MESH_ONESHOT = 3,
     ORC_ALG_RS_MESH = 4,
-    ORC_ALG_RS_RING_STANDALONE = 5
+    ORC_ALG_RS_RING_STANDALONE = 5,
+    ORC_ALG_ALLREDUCE_MESH_ASCENDING = 6
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -527,19 +547,27 @@ static int cmp_ops(const void* a, const void* b)
     return 0;
 }
 
+static uint64_t g_stride = 0; /* elements between input slices of the scatter algorithms; 0 = dense */
+
+/* Applies to the next orc_trace / orc_run / orc_algorithmic_bytes calls (scatter algorithms only). */
+void orc_set_stride(uint64_t stride) { g_stride = stride; }
+
 static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dtype)
 {
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
     if (n == 0 || n > ORC_MAX_RANKS || unit == 0) return -1;
+    const uint64_t stride = g_stride ? g_stride : count;
+    if (stride < count) return -1;
     for (uint32_t r = 0; r < n; r++) {
         switch (alg) {
             case ORC_ALG_ALLREDUCE_RING: prog_allreduce_ring(t, r, n, count, unit, 1); break;
             case ORC_ALG_RS_RING_STAGE: prog_allreduce_ring(t, r, n, count, unit, 0); break;
             case ORC_ALG_ALLREDUCE_RHD: prog_allreduce_rhd(t, r, n, count, unit); break;
             case ORC_ALG_ALLREDUCE_MESH_ONESHOT: prog_allreduce_mesh_oneshot(t, r, n, count, unit); break;
-            case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, unit); break;
-            case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, unit); break;
+            case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, stride, unit); break;
+            case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, stride, unit); break;
+            case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
             default: free(t->ops); return -1;
         }
     }

@@ -18,8 +18,9 @@ ALGS = {
     "mesh_oneshot": (h.Alg.ALLREDUCE_MESH_ONESHOT, oracle.ALG_ALLREDUCE_MESH_ONESHOT),
     "mesh_rs": (h.Alg.REDUCE_SCATTER_MESH, oracle.ALG_RS_MESH),
     "ring_rs": (h.Alg.REDUCE_SCATTER_RING_STANDALONE, oracle.ALG_RS_RING_STANDALONE),
+    "mesh_ascending": (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, oracle.ALG_ALLREDUCE_MESH_ASCENDING),
 }
-FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs"}
+FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
 
 
 def say(*a):
@@ -27,28 +28,28 @@ def say(*a):
     sys.stdout.flush()
 
 
-def buffer_counts(alg, n, count):
+def buffer_counts(alg, n, count, stride=0):
     """(elements in each input buffer, elements in each output buffer)."""
     if alg in ("mesh_rs", "ring_rs"):
-        return n * count, count
+        return ((n - 1) * stride + count if stride else n * count), count
     return count, count
 
 
-def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None):
+def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None, stride=0):
     dt, o = DT[dtype], OPS[op]
-    in_count, out_count = buffer_counts(alg, n, count)
+    in_count, out_count = buffer_counts(alg, n, count, stride)
     kind = kind or ("prod" if op == "prod" else "default")
     host_in = [gen(dt, in_count, seed * 1000 + r, kind) for r in range(n)]
     sentinel = gen(dt, out_count, 999, "wide")
     want_in = [x.copy() for x in host_in]
     want_out = [sentinel.copy() for _ in range(n)]
-    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o)
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o, stride)
     d_in = [to_dev(x) for x in host_in]
     d_out = [to_dev(sentinel) for _ in range(n)]
     # zero-length tensors have a null data_ptr; give the plan a real (unused) address instead
     pad = to_dev(np.zeros(256, np.uint8))
     ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
-    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o, stride)
     try:
         assert plan.run(thread) == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
@@ -102,6 +103,9 @@ CASES = [
     ("ring_rs", 8, 40001, "fp32", "sum"),
     ("ring_rs", 7, 5000, "bf16", "sum"),
     ("ring_rs", 2, 64, "int8", "max"),
+    ("mesh_ascending", 8, 100003, "fp16", "sum"),
+    ("mesh_ascending", 5, 4097, "fp32", "max"),
+    ("mesh_ascending", 1, 10, "int8", "sum"),
 ]
 
 
@@ -119,6 +123,15 @@ def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype
     launches, algo, moved = run_case(gpu_thread, alg, h.Lowering.FUSED, n, count, dtype, op)
     assert launches <= 1
     assert moved <= algo
+
+
+@pytest.mark.parametrize("alg", ["mesh_rs", "ring_rs"])
+@pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
+def test_strided_reduce_scatter(gpu_thread, alg, lowering):
+    """Input slices spaced strideLen elements apart (aicpu_reduce_scatter.cc:78-80); the gaps keep their bytes."""
+    for n, count, stride, dtype in ((7, 5000, 5000 + 37, "bf16"), (4, 1 << 16, 3 << 16, "fp32"), (3, 33, 64, "int8")):
+        say("strided", alg, lowering, n, count, stride, dtype)
+        run_case(gpu_thread, alg, lowering, n, count, dtype, "sum", stride=stride)
 
 
 def test_non_associative_inputs_expose_order(gpu_thread):

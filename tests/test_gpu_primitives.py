@@ -236,3 +236,65 @@ def test_mem_alloc_roundtrip(gpu_thread):
     h.HcommGfxThreadSynchronize(gpu_thread)
     assert np.array_equal(d_back.cpu().numpy(), src)
     assert h.HcommMemFree(p) == 0
+
+
+def test_inter_rank_twins_and_descriptor_batch(gpu_thread):
+    """Write / Read / WriteReduce / ReadReduce give the same bytes as their local twins, and a descriptor
+    array submitted with HcommBatchTransferOnThread runs as one merged launch per kind."""
+    dt, count, n = oracle.BF16, 40001, 6
+    a = [gen(dt, count, 300 + i) for i in range(n)]
+    b = [gen(dt, count, 400 + i) for i in range(n)]
+    d_a, d_b = [to_dev(x) for x in a], [to_dev(x) for x in b]
+    d_c = [to_dev(np.zeros_like(x)) for x in a]
+    h.HcommGfxThreadSynchronize(gpu_thread)
+    CH = 1
+    assert h.HcommWriteReduceOnThread(gpu_thread, CH, d_a[0].data_ptr(), d_b[0].data_ptr(), count, dt, oracle.SUM) == 0
+    assert h.HcommReadReduceOnThread(gpu_thread, CH, d_a[1].data_ptr(), d_b[1].data_ptr(), count, dt, oracle.MAX) == 0
+    assert h.HcommWriteOnThread(gpu_thread, CH, d_c[0].data_ptr(), d_a[0].data_ptr(), count * 2) == 0
+    assert h.HcommReadOnThread(gpu_thread, CH, d_c[1].data_ptr(), d_a[1].data_ptr(), count * 2) == 0
+    descs = [h.desc_reduce(d_a[i].data_ptr(), d_b[i].data_ptr(), count, dt, oracle.SUM, read=(i % 2 == 0))
+             for i in range(2, n)]
+    descs += [h.desc_copy(d_c[i].data_ptr(), d_a[i].data_ptr(), count * 2, read=(i % 2 == 1)) for i in range(2, n)]
+    h.HcommGfxLaunchLogClear(gpu_thread)
+    assert h.HcommBatchTransferOnThread(gpu_thread, CH, descs) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    assert [(r.kind, r.nseg) for r in h.launch_log(gpu_thread)] == [(h.Kernel.REDUCE2, n - 2), (h.Kernel.COPY, n - 2)]
+    for i in range(n):
+        want = oracle.reduce(a[i].copy(), b[i], dt, oracle.MAX if i == 1 else oracle.SUM)
+        assert_same(from_dev(d_a[i], a[i]), want, dt, "a[%d]" % i)
+        assert_same(from_dev(d_c[i], a[i]), want, dt, "c[%d]" % i)
+
+
+def test_more_than_4gib_in_one_call(gpu_thread):
+    """Lengths beyond 2^32 bytes / elements (the reference's API tests pass 4 GB and 4 GB + 1,
+    ut_aicpu_ts_HcommLocalCopyOnThread.cc, ut_aicpu_ts_HcommLocalReduceOnThread.cc:71-89): 64-bit indexing end
+    to end, checked on the GPU against torch."""
+    import torch
+    n = (1 << 32) + 5
+    say("4GiB copy")
+    src = torch.empty(n + 16, dtype=torch.int8, device="cuda")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    src.random_(-100, 100, generator=g)
+    dst = torch.zeros(n + 16, dtype=torch.int8, device="cuda")
+    torch.cuda.synchronize()
+    assert h.HcommLocalCopyOnThread(gpu_thread, dst.data_ptr(), src.data_ptr(), n) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    assert torch.equal(dst[:n], src[:n]) and int(dst[n:].abs().max()) == 0
+    say("4GiB reduce")
+    want = (dst[n - 4096:n].to(torch.int16) + src[n - 4096:n].to(torch.int16)).to(torch.int8)   # wraps like int8
+    head = (dst[:4096].to(torch.int16) + src[:4096].to(torch.int16)).to(torch.int8)
+    mid0 = (1 << 32) - 2048
+    mid = (dst[mid0:n].to(torch.int16) + src[mid0:n].to(torch.int16)).to(torch.int8)   # straddles 2^32
+    torch.cuda.synchronize()   # torch computed the expectations on its own stream
+    assert h.HcommLocalReduceOnThread(gpu_thread, dst.data_ptr(), src.data_ptr(), n, oracle.I8, oracle.SUM) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    assert torch.equal(dst[:4096], head) and torch.equal(dst[n - 4096:n], want) and torch.equal(dst[mid0:n], mid)
+    assert int(dst[n:].abs().max()) == 0, "reduce wrote past count"
+    # whole-buffer check without a second 4 GiB temporary: dst == 2 * src in wrapping int8 arithmetic
+    chunk = 1 << 28
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        assert torch.equal(dst[lo:hi], src[lo:hi] * 2), "chunk at %d" % lo
+    del src, dst
+    torch.cuda.empty_cache()

@@ -122,6 +122,67 @@ def test_notify_argument_checks(rec):
     assert h.HcommThreadNotifyWaitOnThread(rec, 0, 1) == R.E_PARA
 
 
+def test_inter_rank_twins_checks_and_launches(rec):
+    """HcommWrite/Read[Reduce]OnThread: same arithmetic with a channel argument
+    (cpu_primitives_c_adpt.cc:284-318,332-384,490-565)."""
+    CH = 0x77
+    for f in (h.HcommWriteOnThread, h.HcommReadOnThread):
+        assert f(rec, CH, DST, SRC, 4096) == R.SUCCESS
+        assert f(rec, CH, None, SRC, 4096) == R.E_PTR
+        assert f(rec, CH, DST, None, 4096) == R.E_PTR
+        assert f(0, CH, DST, SRC, 4096) == R.E_PTR
+        assert f(rec, 0, DST, SRC, 4096) == R.E_PTR
+    for f in (h.HcommWriteReduceOnThread, h.HcommReadReduceOnThread):
+        assert f(rec, CH, DST, SRC, 1024, DT.FP16, OP.SUM) == R.SUCCESS
+        assert f(rec, CH, None, SRC, 1024, DT.FP16, OP.SUM) == R.E_PTR
+        assert f(rec, CH, DST, SRC, 1024, DT.FP64, OP.SUM) == R.E_PARA
+        assert f(rec, CH, DST, SRC, 1024, DT.FP16, OP.PROD) == R.E_PARA
+        assert f(0, CH, DST, SRC, 1024, DT.FP64, OP.SUM) == R.E_PARA     # type check precedes the thread check
+        assert f(0, CH, DST, SRC, 1024, DT.FP16, OP.SUM) == R.E_PTR
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommBatchModeStart(None) == 0
+    for r in range(4):
+        assert h.HcommReadReduceOnThread(rec, CH, DST + r * 65536, SRC + r * 65536, 1024, DT.BFP16, OP.MAX) == 0
+    assert h.HcommBatchModeEnd(None) == 0
+    assert [(x.kind, x.nseg, x.op) for x in h.launch_log(rec)] == [(h.Kernel.REDUCE2, 4, OP.MAX)]
+
+
+def test_batch_transfer_descriptors(rec):
+    """HcommBatchTransferDesc[] is one batch: independent descriptors share a launch, order is kept."""
+    CH, K = 5, 65536
+    descs = [h.desc_reduce(DST + r * K, SRC + r * K, 1024, DT.FP32, OP.SUM, read=True) for r in range(8)]
+    descs += [h.desc_copy(DST + (20 + r) * K, DST + r * K, 4096) for r in range(8)]   # depend on the reduces
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommBatchTransferOnThread(rec, CH, descs) == R.SUCCESS
+    assert [(x.kind, x.nseg) for x in h.launch_log(rec)] == [(h.Kernel.REDUCE2, 8), (h.Kernel.COPY, 8)]
+    assert h.HcommBatchTransferOnThread(rec, CH, []) == R.SUCCESS
+    assert h.HcommBatchTransferOnThread(0, CH, descs) == R.E_PTR
+    assert h.HcommBatchTransferOnThread(rec, 0, descs) == R.E_PTR
+    assert raw._batch_transfer(rec, CH, None, 3) == R.E_PTR
+    h.HcommGfxLaunchLogClear(rec)
+    bad = h.desc_reduce(DST, SRC, 16, DT.FP64, OP.SUM)
+    assert h.HcommBatchTransferOnThread(rec, CH, descs[:2] + [bad]) == R.E_PARA
+    notify = h.BatchTransferDesc()
+    notify.transType = h.TransferType.NOTIFY_RECORD
+    assert h.HcommBatchTransferOnThread(rec, CH, descs[:2] + [notify]) == R.E_NOT_SUPPORT
+    null = h.desc_copy(0, SRC, 16)
+    assert h.HcommBatchTransferOnThread(rec, CH, [null]) == R.E_PTR
+    assert h.launch_log(rec) == []                     # validated as a whole before anything is enqueued
+    import ctypes
+    assert ctypes.sizeof(h.BatchTransferDesc) == 64    # include/hcomm_primitives.h:91-131
+
+
+def test_strided_plan_checks():
+    i, o = ptrs(4, 1 << 20)
+    p = h.Plan(h.Alg.REDUCE_SCATTER_MESH, h.Lowering.FUSED, i, o, 1000, DT.FP32, OP.SUM, stride=1500)
+    assert p.info.launches == 1
+    p.destroy()
+    for alg, stride, code in ((h.Alg.REDUCE_SCATTER_MESH, 999, R.E_PARA), (h.Alg.ALLREDUCE_RING, 1500, R.E_PARA)):
+        with pytest.raises(h.HcommError) as e:
+            h.Plan(alg, h.Lowering.STEPWISE, i, o, 1000, DT.FP32, OP.SUM, stride=stride)
+        assert e.value.code == code
+
+
 # ---- batch mode --------------------------------------------------------------------------------------------
 
 def test_batch_mode_state_machine(rec):

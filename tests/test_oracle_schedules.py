@@ -14,7 +14,8 @@ import hcomm_amd as h
 GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "schedules_hand_derived.json")))
 
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
-        oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE]
+        oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
+        oracle.ALG_ALLREDUCE_MESH_ASCENDING]
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE)
 
 
@@ -164,6 +165,11 @@ def test_mesh_trees_hand_derived(op):
         results.add(want.tobytes())
     if op == oracle.SUM:
         assert len(results) > 1, "inputs were meant to make the per-rank orders visible"
+    outs = [np.zeros(count, np.float32) for _ in range(n)]
+    oracle.run(oracle.ALG_ALLREDUCE_MESH_ASCENDING, [x.copy() for x in ins], outs, count, oracle.F32, op)
+    for r_s, tree in GOLD["mesh_ascending_rank_tree"]["4"].items():
+        want = eval_tree(tree, ins, op)
+        assert np.array_equal(outs[int(r_s)].view(np.uint32), want.view(np.uint32))
     big = [np.concatenate([order_sensitive_inputs(n, count, op, seed=20 + r)[0] for _ in range(n)]) for r in range(n)]
     outs = [np.zeros(count, np.float32) for _ in range(n)]
     oracle.run(oracle.ALG_RS_MESH, [x.copy() for x in big], outs, count, oracle.F32, op)
@@ -215,6 +221,28 @@ def test_scatter_variants_deliver_the_right_slice():
             assert np.array_equal(outs[r], want[r * count:(r + 1) * count].astype(np.int32))
 
 
+def test_strided_scatter_input_layout():
+    """Input slice i starts strideLen * i elements into the buffer (aicpu_reduce_scatter.cc:78-80); the gaps
+    between slices are never read or written."""
+    g = GOLD["strided_rs"]
+    n, count, stride = g["n"], g["count"], g["stride"]
+    for alg in SCATTER_OUT:
+        ops = oracle.trace(alg, n, count, oracle.F32, stride)
+        offs = sorted(set(o[4] for o in ops if o[3] == 0) | set(o[7] for o in ops if o[6] == 0))
+        assert offs == g["slice_byte_offsets"]
+        ins = [np.arange(g["input_elements"], dtype=np.int32) * 100 + r for r in range(n)]
+        before = [x.copy() for x in ins]
+        outs = [np.zeros(count, np.int32) for _ in range(n)]
+        oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM, stride)
+        for r in range(n):
+            lo = r * stride
+            assert np.array_equal(outs[r], sum(b[lo:lo + count] for b in before))
+            for i in range(n):  # gaps untouched
+                assert np.array_equal(ins[r][i * stride + count:(i + 1) * stride], before[r][i * stride + count:(i + 1) * stride])
+    with pytest.raises(ValueError):
+        oracle.trace(oracle.ALG_RS_MESH, 3, 10, oracle.F32, 5)      # stride < count
+
+
 # ---- two independently written generators agree ----------------------------------------------------------
 
 @pytest.mark.parametrize("alg", ALGS)
@@ -225,6 +253,8 @@ def test_product_generator_equals_oracle_trace(alg):
             a = oracle.trace(alg, n, count, dt)
             b = h.schedule_emit(alg, n, count, dt)
             assert a == b, (alg, n, count, dt)
+            if alg in SCATTER_OUT:
+                assert oracle.trace(alg, n, count, dt, count + 13) == h.schedule_emit(alg, n, count, dt, count + 13)
 
 
 def test_algorithmic_bytes_of_benchmark_configs():
