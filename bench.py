@@ -225,9 +225,25 @@ def main():
             cpu_s += time.perf_counter() - t0
             passes += 1
         host_in = work_in
+        # the same schedule on ONE thread (the scalar loop shape of the reference's CPU witnesses), one pass
+        oracle.lib().orc_set_threads(1)
+        one_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
+        one_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
+        t0 = time.perf_counter()
+        oracle.run(oalg, one_in, one_out, count, odt, oop)
+        one_s = time.perf_counter() - t0
+        del one_in, one_out
+        model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                model = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")][0]
+        except Exception:
+            pass
         cpu = {"value": round(alg_bytes * passes / cpu_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": "the full workload, %d passes, %.2f s of CPU work in total; OpenMP static over elements"
-                         % (passes, cpu_s)}
+                         % (passes, cpu_s),
+               "single_thread_value": round(alg_bytes / one_s / 1e9, 2), "cpu_model": model,
+               "host_cores": os.cpu_count()}
         # verification: one GPU pass per lowering from pristine inputs must equal the oracle bit for bit
         verified = True
         for name in lowerings:

@@ -23,6 +23,7 @@ __all__ = [
     "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion",
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
+    "CheckReport", "Expect", "oplist_check", "schedule_check",
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
@@ -172,6 +173,35 @@ HcommReadOnThread = _sig("HcommReadOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
 HcommWriteReduceOnThread = _sig("HcommWriteReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
 HcommReadReduceOnThread = _sig("HcommReadReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
 _batch_transfer = _sig("HcommBatchTransferOnThread", _i32, _u64, _u64, C.POINTER(BatchTransferDesc), _u32)
+class CheckReport(C.Structure):
+    _fields_ = [("conflicts", C.c_uint32), ("semanticErrors", C.c_uint32), ("message", C.c_char * 248)]
+
+
+class Expect:
+    ALLREDUCE, REDUCE_SCATTER_IN_PLACE, REDUCE_SCATTER_OUT = 0, 1, 2
+
+
+_oplist_check = _sig("HcommGfxOpListCheck", _i32, C.POINTER(SchedOp), _u64, _u32, C.c_int, _u64, _u64, _u32,
+                     C.POINTER(CheckReport))
+_sched_check = _sig("HcommGfxScheduleCheck", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+
+
+def oplist_check(ops, n_ranks, expect, count, unit, stride=0):
+    """ops: tuples as returned by schedule_emit.  Returns (conflicts, semantic_errors, message)."""
+    arr = (SchedOp * max(len(ops), 1))()
+    for i, (step, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes) in enumerate(ops):
+        arr[i] = SchedOp(step, kind, rank, dbuf, srank, sbuf, doff, soff, nbytes)
+    rep = CheckReport()
+    check(_oplist_check(arr, len(ops), n_ranks, expect, count, stride, unit, C.byref(rep)), "HcommGfxOpListCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+def schedule_check(alg, n_ranks, count, dtype, stride=0):
+    rep = CheckReport()
+    check(_sched_check(alg, n_ranks, count, stride, dtype, C.byref(rep)), "HcommGfxScheduleCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
 _version = _sig("HcommGfxVersion", C.c_char_p)
 
 

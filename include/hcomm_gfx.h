@@ -424,6 +424,36 @@ int32_t HcommGfxScheduleEmitStrided(
     HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t strideCount, HcommDataType dataType,
     HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
 
+/*
+ * Symbolic check of an op list (no data is moved, no GPU needed) - a miniature of the reference's algorithm
+ * checker (test/st/algorithm/README_en.md:13-15,202-231;
+ * test/st/algorithm/utils/checker/semantics_check/allreduce_semantics_checker.cc:59-96):
+ *   conflicts      - operations of one step that write a range another operation of the step reads or writes;
+ *   semanticErrors - bytes of the expected result that do not hold exactly one contribution from every rank,
+ *                    taken from the matching offset of that rank's input.
+ * message describes the first finding.  The call itself returns HCCL_SUCCESS when the check ran.
+ */
+typedef enum {
+    HCOMM_GFX_EXPECT_ALLREDUCE = 0,               /* out[r][0, count*unit) for every r */
+    HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE = 1, /* in[r][slice r], slices from HcommGfxCalcSlices(count, unit, n) */
+    HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT = 2       /* out[r][0, count*unit) = sum of in[k][r*stride*unit + ...] */
+} HcommGfxExpectation;
+
+typedef struct {
+    uint32_t conflicts;
+    uint32_t semanticErrors;
+    char message[248];
+} HcommGfxCheckReport;
+
+int32_t HcommGfxOpListCheck(
+    const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, HcommGfxExpectation expect, uint64_t count,
+    uint64_t strideCount, uint32_t unitSize, HcommGfxCheckReport* report);
+
+/* Generate the op list of alg and check it against the expectation that belongs to the algorithm. */
+int32_t HcommGfxScheduleCheck(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t strideCount, HcommDataType dataType,
+    HcommGfxCheckReport* report);
+
 /* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */
 const char* HcommGfxVersion(void);
 
