@@ -271,6 +271,8 @@ static void log_launch(HgThread* t, const HgLaunch* l)
     r->blocks = l->blocks;
 }
 
+void hg_log_only(HgThread* t, const HgLaunch* l) { log_launch(t, l); }
+
 int hg_submit(HgThread* t, const HgLaunch* l)
 {
     log_launch(t, l);

@@ -64,6 +64,8 @@ void hg_finish_fold(HgLaunch* l);
 
 /* Execute (or, on a recorder thread, log) one prepared launch. */
 int hg_submit(HgThread* t, const HgLaunch* l);
+/* Append one prepared launch to the thread's log without executing it. */
+void hg_log_only(HgThread* t, const HgLaunch* l);
 
 int hg_dtype_supported(int dtype);
 int hg_reduce_supported(int dtype, int op, int allow_prod);

@@ -85,6 +85,12 @@ int hg_rt_stream_wait_event(void* stream, void* ev);
 int hg_rt_malloc(void** p, size_t n);
 int hg_rt_free(void* p);
 int hg_rt_num_cus(void);
+/* Graph replay of a fixed launch list: capture between begin/end on `stream`, then launch the executable. */
+int hg_rt_stream_is_capturing(void* stream);
+int hg_rt_capture_begin(void* stream);
+int hg_rt_capture_end(void* stream, void** graph_exec);
+int hg_rt_graph_launch(void* graph_exec, void* stream);
+int hg_rt_graph_destroy(void* graph_exec);
 
 #ifdef __cplusplus
 }

@@ -656,6 +656,27 @@ int hg_rt_event_record(void* ev, void* stream) { return rc(hipEventRecord((hipEv
 int hg_rt_stream_wait_event(void* stream, void* ev) { return rc(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)ev, 0)); }
 int hg_rt_malloc(void** p, size_t n) { return hipMalloc(p, n) == hipSuccess ? HCCL_SUCCESS : HCCL_E_MEMORY; }
 int hg_rt_free(void* p) { return rc(hipFree(p)); }
+int hg_rt_stream_is_capturing(void* stream)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess) return 1; /* unknown: treat as busy */
+    return st != hipStreamCaptureStatusNone;
+}
+int hg_rt_capture_begin(void* stream) { return rc(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal)); }
+int hg_rt_capture_end(void* stream, void** graph_exec)
+{
+    hipGraph_t g = nullptr;
+    *graph_exec = nullptr;
+    if (hipStreamEndCapture((hipStream_t)stream, &g) != hipSuccess || !g) return HCCL_E_RUNTIME;
+    hipGraphExec_t e = nullptr;
+    const hipError_t err = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (err != hipSuccess) return HCCL_E_RUNTIME;
+    *graph_exec = e;
+    return HCCL_SUCCESS;
+}
+int hg_rt_graph_launch(void* graph_exec, void* stream) { return rc(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream)); }
+int hg_rt_graph_destroy(void* graph_exec) { return rc(hipGraphExecDestroy((hipGraphExec_t)graph_exec)); }
 int hg_rt_num_cus(void)
 {
     int dev = 0, n = 0;

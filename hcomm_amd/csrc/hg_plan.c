@@ -19,7 +19,25 @@ struct HcommGfxPlan {
     uint32_t nlaunch, cap;
     HgLaunch* launches;
     HcommGfxPlanInfo info;
+    /* graph replay of the whole launch list: built at the first full run on a stream, rebuilt when the stream
+     * changes, never used when the caller's stream is itself being captured */
+    void* graph_exec;
+    void* graph_stream;
+    int graph_state; /* 0 not built, 1 ready, -1 unavailable */
 };
+
+static int g_use_graph = -1;
+
+static int use_graph(void)
+{
+    if (g_use_graph < 0) {
+        const char* e = getenv("HCOMM_GFX_GRAPH");
+        /* measured on ROCm 7: replaying 15 small kernels as a graph takes 60 us against 54 us launched one by
+         * one, so graph replay is opt-in */
+        g_use_graph = (e && e[0] == '1') ? 1 : 0;
+    }
+    return g_use_graph;
+}
 
 static int plan_push(const HgLaunch* l, void* ctx)
 {
@@ -290,13 +308,45 @@ int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint
 int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread)
 {
     if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
-    return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    HcommGfxPlan* p = (HcommGfxPlan*)plan; /* the graph is a cache, not part of the plan's meaning */
+    if (t->recorder || p->nlaunch < 2 || !use_graph() || p->graph_state < 0 || hg_rt_stream_is_capturing(t->stream))
+        return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+    if (p->graph_state == 1 && p->graph_stream != t->stream) {
+        hg_rt_graph_destroy(p->graph_exec);
+        p->graph_exec = NULL;
+        p->graph_state = 0;
+    }
+    if (p->graph_state == 0) {
+        if (hg_rt_capture_begin(t->stream) != HCCL_SUCCESS) {
+            p->graph_state = -1;
+            return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+        }
+        const int saved = t->log_enabled;
+        t->log_enabled = 0;
+        int rc = HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+        t->log_enabled = saved;
+        void* exec = NULL;
+        const int rc2 = hg_rt_capture_end(t->stream, &exec);
+        if (rc != HCCL_SUCCESS || rc2 != HCCL_SUCCESS) {
+            if (exec) hg_rt_graph_destroy(exec);
+            p->graph_state = -1;
+            return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
+        }
+        p->graph_exec = exec;
+        p->graph_stream = t->stream;
+        p->graph_state = 1;
+    }
+    for (uint32_t i = 0; i < p->nlaunch; ++i) hg_log_only(t, &p->launches[i]);
+    return hg_rt_graph_launch(p->graph_exec, t->stream);
 }
 
 int32_t HcommGfxPlanDestroy(HcommGfxPlan* plan)
 {
     if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
     plan->magic = 0;
+    if (plan->graph_exec) hg_rt_graph_destroy(plan->graph_exec);
     free(plan->launches);
     free(plan);
     return HCCL_SUCCESS;

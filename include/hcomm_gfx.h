@@ -376,7 +376,13 @@ int32_t HcommGfxPlanCreateStrided(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
     uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
-/* Enqueue every launch of the plan on the thread, in order.  May be called any number of times. */
+/*
+ * Enqueue every launch of the plan on the thread, in order.  May be called any number of times, from one host
+ * thread at a time.  With HCOMM_GFX_GRAPH=1 in the environment a plan of two or more launches is replayed as a
+ * HIP graph captured at its first run on the thread's stream (off by default: it measured slower than
+ * launching kernel by kernel); when the caller's stream is itself being captured the launches are always
+ * issued individually and become part of the caller's graph.
+ */
 int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread);
 
 /* Enqueue launches [first, first + n) only (used to time one phase of a plan). */
