@@ -46,6 +46,7 @@ WORKLOADS = {
     "ring_rs_fp32_prod_n7_100M": ("ring_rs_stage", 7, 100000003, "fp32", "prod", "uniform[0.99,1.01]"),
     "ring_rs_int8_sum_n7_100M": ("ring_rs_stage", 7, 100000003, "int8", "sum", "ints[-8,8]"),
     "mesh_oneshot_fp16_n8_4MiB": ("mesh_oneshot", 8, 2097152, "fp16", "sum", "uniform[-1,1)"),
+    "local_reduce_ar_bf16_n8_128MiB": ("local_reduce", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
 
@@ -101,7 +102,7 @@ def main():
     DT = {"bf16": h.HcommDataType.BFP16, "fp32": h.HcommDataType.FP32, "fp16": h.HcommDataType.FP16,
           "int32": h.HcommDataType.INT32, "int8": h.HcommDataType.INT8}
     ALG = {"ring_ar": h.Alg.ALLREDUCE_RING, "rhd_ar": h.Alg.ALLREDUCE_RHD, "ring_rs_stage": h.Alg.REDUCE_SCATTER_RING,
-           "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT}
+           "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT, "local_reduce": h.Alg.ALLREDUCE_LOCAL_REDUCE}
     OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
           "min": h.HcommReduceOp.MIN}
     dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
@@ -132,6 +133,11 @@ def main():
 
     in_ptrs = [t.data_ptr() for t in d_in]
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
+    scratch_bytes = h.scratch_bytes(alg, n, count, dt)
+    d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
+    scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
+    if alg_name == "local_reduce" and args.lowering == "both":
+        args.lowering = "stepwise"  # this schedule has no fused lowering
     kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
              h.Kernel.COPY: "k_copy"}
 
@@ -139,7 +145,7 @@ def main():
     results = {}
     for name in lowerings:
         low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-        plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op)
+        plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
         launches = plan.launches()
         restore()
         for _ in range(args.warmup):
@@ -177,8 +183,9 @@ def main():
         stream.synchronize()
         dom_ms = sum(a.elapsed_time(b) for a, b in ev) / (args.steps * cnt)
         if name == "stepwise":
-            # average launch of the run: 3 x (bytes it writes) for a reduce step of all ranks
-            dom_bytes = sum(launches[i].bytes for i in range(first, first + cnt)) * 3 // cnt
+            # average launch of the run: 3 x (bytes it writes) for a reduce step of all ranks, 2 x for a copy step
+            per_byte = 2 if dom_kind == h.Kernel.COPY else 3
+            dom_bytes = sum(launches[i].bytes for i in range(first, first + cnt)) * per_byte // cnt
             dom_moved = dom_bytes
         else:
             dom_bytes = plan.info.algorithmicBytes  # the single launch is the whole collective
@@ -189,7 +196,7 @@ def main():
             "launches": plan.info.launches,
             "algorithmic_bytes": plan.info.algorithmicBytes,
             "moved_bytes": plan.info.movedBytes,
-            "kernel": "%s<%s,%s>" % (kname[dom_kind], dtname, opname.upper()),
+            "kernel": "k_copy" if dom_kind == h.Kernel.COPY else "%s<%s,%s>" % (kname[dom_kind], dtname, opname.upper()),
             "kernel_ms": dom_ms,
             "kernel_alg_bytes": dom_bytes,
             "kernel_gbs": dom_bytes / (dom_ms * 1e-3) / 1e9,
@@ -210,18 +217,20 @@ def main():
         odt = {"bf16": oracle.BF16, "fp32": oracle.F32, "fp16": oracle.F16, "int32": oracle.I32,
                "int8": oracle.I8}[dtname]
         oalg = {"ring_ar": oracle.ALG_ALLREDUCE_RING, "rhd_ar": oracle.ALG_ALLREDUCE_RHD,
-                "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT}[alg_name]
+                "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT,
+                "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
+        host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
         alg_bytes = oracle.algorithmic_bytes(oalg, n, count, odt)
         passes, cpu_s = 0, 0.0
         while passes < 1 or (cpu_s < 8.0 and passes < 64):
             work_in = [x.copy() for x in host_in]  # every pass starts from the pristine inputs (copy not timed)
             t0 = time.perf_counter()
-            oracle.run(oalg, work_in, host_out, count, odt, oop)
+            oracle.run(oalg, work_in, host_out, count, odt, oop, scratch=host_scr)
             cpu_s += time.perf_counter() - t0
             passes += 1
         host_in = work_in
@@ -230,7 +239,7 @@ def main():
         one_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         one_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         t0 = time.perf_counter()
-        oracle.run(oalg, one_in, one_out, count, odt, oop)
+        oracle.run(oalg, one_in, one_out, count, odt, oop, scratch=host_scr)
         one_s = time.perf_counter() - t0
         del one_in, one_out
         model = "unknown"
@@ -248,7 +257,7 @@ def main():
         verified = True
         for name in lowerings:
             low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-            plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op)
+            plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
             restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
             stream.synchronize()

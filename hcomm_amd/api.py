@@ -23,7 +23,7 @@ __all__ = [
     "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion",
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
-    "CheckReport", "Expect", "oplist_check", "schedule_check",
+    "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
@@ -61,7 +61,7 @@ class CommEngine:
 
 class Alg:
     ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
-        REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING = range(7)
+        REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING, ALLREDUCE_LOCAL_REDUCE = range(8)
 
 
 class Lowering:
@@ -159,11 +159,19 @@ _log_read = _sig("HcommGfxLaunchLogRead", _i32, _u64, C.POINTER(LaunchRecord), _
 HcommGfxLaunchLogClear = _sig("HcommGfxLaunchLogClear", _i32, _u64)
 _calc_slices = _sig("HcommGfxCalcSlices", _i32, _u64, _u32, _u32, C.POINTER(Slice))
 HcommGfxDataTypeSize = _sig("HcommGfxDataTypeSize", _u32, C.c_int)
-_plan_create = _sig("HcommGfxPlanCreateStrided", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64,
-                    _u64, C.c_int, C.c_int, C.POINTER(_vp))
+_plan_create = _sig("HcommGfxPlanCreateEx", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                    C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+_scratch_bytes = _sig("HcommGfxScratchBytes", _i32, C.c_int, _u32, _u64, C.c_int, C.POINTER(_u64))
+
+
+def scratch_bytes(alg, n_ranks, count, dtype):
+    b = _u64(0)
+    check(_scratch_bytes(alg, n_ranks, count, dtype, C.byref(b)), "HcommGfxScratchBytes")
+    return b.value
 _plan_run = _sig("HcommGfxPlanRun", _i32, _vp, _u64)
 _plan_run_range = _sig("HcommGfxPlanRunRange", _i32, _vp, _u64, _u32, _u32)
 _plan_destroy = _sig("HcommGfxPlanDestroy", _i32, _vp)
+_plan_graph = _sig("HcommGfxPlanSetGraphReplay", _i32, _vp, _i32)
 _plan_info = _sig("HcommGfxPlanGetInfo", _i32, _vp, C.POINTER(PlanInfo))
 _plan_launch = _sig("HcommGfxPlanGetLaunch", _i32, _vp, _u32, C.POINTER(LaunchRecord))
 _sched_emit = _sig("HcommGfxScheduleEmitStrided", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
@@ -296,12 +304,13 @@ def schedule_emit(alg, n_ranks, count, dtype, stride=0):
 class Plan:
     """HcommGfxPlan: build once, run many."""
 
-    def __init__(self, alg, lowering, in_ptrs, out_ptrs, count, dtype, op, stride=0):
+    def __init__(self, alg, lowering, in_ptrs, out_ptrs, count, dtype, op, stride=0, scratch_ptrs=None):
         n = len(in_ptrs)
         self._in = (_vp * n)(*in_ptrs)
         self._out = (_vp * n)(*out_ptrs) if out_ptrs is not None else None
+        self._scratch = (_vp * n)(*scratch_ptrs) if scratch_ptrs is not None else None
         p = _vp(0)
-        check(_plan_create(alg, lowering, n, self._in, self._out, count, stride, dtype, op, C.byref(p)),
+        check(_plan_create(alg, lowering, n, self._in, self._out, self._scratch, count, stride, dtype, op, C.byref(p)),
               "HcommGfxPlanCreate")
         self._p = p
         info = PlanInfo()
@@ -310,6 +319,9 @@ class Plan:
 
     def run(self, thread):
         return _plan_run(self._p, thread)
+
+    def set_graph_replay(self, enable):
+        return _plan_graph(self._p, 1 if enable else 0)
 
     def run_range(self, thread, first, n):
         return _plan_run_range(self._p, thread, first, n)

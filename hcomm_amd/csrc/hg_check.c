@@ -82,7 +82,7 @@ int32_t HcommGfxOpListCheck(
     if (strideCount == 0) strideCount = count;
     const uint64_t total = count * unitSize;
     for (uint64_t i = 0; i < nOps; ++i)
-        if (ops[i].rank >= nRanks || ops[i].srcRank >= nRanks || ops[i].dstBuf > 1 || ops[i].srcBuf > 1 || ops[i].kind > 1)
+        if (ops[i].rank >= nRanks || ops[i].srcRank >= nRanks || ops[i].dstBuf > 2 || ops[i].srcBuf > 2 || ops[i].kind > 1)
             return HCCL_E_PARA;
 
     /* 1. interval boundaries, closed under the translations the operations perform */
@@ -117,17 +117,18 @@ int32_t HcommGfxOpListCheck(
     }
     if (rc != HCCL_SUCCESS) { free(bs.b); return rc; }
 
-    /* 2. state: 2 buffers per rank x intervals */
+    /* 2. state: 3 buffers per rank (input, output, communication buffer) x intervals */
     const size_t ni = bs.n - 1;
-    Cell* st = (Cell*)calloc((size_t)2 * nRanks * (ni ? ni : 1), sizeof(Cell));
+    Cell* st = (Cell*)calloc((size_t)3 * nRanks * (ni ? ni : 1), sizeof(Cell));
     Cell* tmp = (Cell*)calloc(ni ? ni : 1, sizeof(Cell));
     if (!st || !tmp) { free(st); free(tmp); free(bs.b); return HCCL_E_MEMORY; }
-#define CELL(rank, buf, iv) st[((size_t)(rank) * 2 + (buf)) * ni + (iv)]
+#define CELL(rank, buf, iv) st[((size_t)(rank) * 3 + (buf)) * ni + (iv)]
     for (uint32_t r = 0; r < nRanks; ++r)
         for (size_t iv = 0; iv < ni; ++iv) {
             for (uint32_t k = 0; k < nRanks; ++k) {
                 CELL(r, 0, iv).delta[k] = NO_DELTA;
                 CELL(r, 1, iv).delta[k] = NO_DELTA;
+                CELL(r, 2, iv).delta[k] = NO_DELTA;
             }
             CELL(r, 0, iv).cnt[r] = 1; /* an input holds its own rank's data from the same offset */
             CELL(r, 0, iv).delta[r] = 0;

@@ -24,6 +24,7 @@ struct HcommGfxPlan {
     void* graph_exec;
     void* graph_stream;
     int graph_state; /* 0 not built, 1 ready, -1 unavailable */
+    int graph_wanted;
 };
 
 static int g_use_graph = -1;
@@ -54,8 +55,10 @@ static int plan_push(const HgLaunch* l, void* ctx)
     return HCCL_SUCCESS;
 }
 
-static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, void* const* out, int dtype, int op)
+static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, void* const* out,
+                          void* const* scratch, int dtype, int op)
 {
+    void* const* bufs[3] = {in, out, scratch};
     HgOp* ops = (HgOp*)calloc(ol->n ? ol->n : 1, sizeof(HgOp));
     if (!ops) return HCCL_E_MEMORY;
     for (uint64_t i = 0; i < ol->n; ++i) {
@@ -64,8 +67,12 @@ static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, 
         o->is_reduce = (uint8_t)s->kind;
         o->dtype = s->kind ? (uint8_t)dtype : 255;
         o->op = s->kind ? (uint8_t)op : 255;
-        o->dst = (char*)(s->dstBuf ? out[s->rank] : in[s->rank]) + s->dstOff;
-        o->src = (const char*)(s->srcBuf ? out[s->srcRank] : in[s->srcRank]) + s->srcOff;
+        if (s->dstBuf > 2 || s->srcBuf > 2 || !bufs[s->dstBuf] || !bufs[s->srcBuf]) {
+            free(ops);
+            return HCCL_E_PTR;
+        }
+        o->dst = (char*)bufs[s->dstBuf][s->rank] + s->dstOff;
+        o->src = (const char*)bufs[s->srcBuf][s->srcRank] + s->srcOff;
         o->bytes = s->bytes;
     }
     int rc = hg_coalesce(ops, ol->n, plan_push, p);
@@ -251,6 +258,23 @@ int32_t HcommGfxPlanCreateStrided(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
     uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
 {
+    return HcommGfxPlanCreateEx(alg, lowering, nRanks, in, out, NULL, count, strideCount, dataType, reduceOp, plan);
+}
+
+int32_t HcommGfxScratchBytes(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType,
+                             uint64_t* bytes)
+{
+    if (!bytes) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS || HcommGfxDataTypeSize(dataType) == 0) return HCCL_E_PARA;
+    *bytes = hg_scratch_bytes((int)alg, nRanks, count, (int)dataType);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanCreateEx(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    void* const* scratch, uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp,
+    HcommGfxPlan** plan)
+{
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
     if (!in) return HCCL_E_PTR;
@@ -266,6 +290,13 @@ int32_t HcommGfxPlanCreateStrided(
             if (((uintptr_t)out[r]) & 127u) return HCCL_E_PARA;
         }
     }
+    if (nRanks > 1 && hg_scratch_bytes((int)alg, nRanks, count, (int)dataType) > 0) {
+        if (!scratch) return HCCL_E_PTR;
+        for (uint32_t r = 0; r < nRanks; ++r) {
+            if (!scratch[r]) return HCCL_E_PTR;
+            if (((uintptr_t)scratch[r]) & 127u) return HCCL_E_PARA;
+        }
+    }
     HgOpList ol;
     if (strideCount == 0) strideCount = count;
     int rc = hg_schedule(&ol, (int)alg, nRanks, count, strideCount, (int)dataType);
@@ -276,10 +307,11 @@ int32_t HcommGfxPlanCreateStrided(
         return HCCL_E_MEMORY;
     }
     p->magic = HG_PLAN_MAGIC;
+    p->graph_wanted = use_graph();
     p->info.steps = ol.steps;
     for (uint64_t i = 0; i < ol.n; ++i) p->info.algorithmicBytes += ol.ops[i].bytes * (ol.ops[i].kind ? 3u : 2u);
     if (lowering == HCOMM_GFX_LOWER_STEPWISE)
-        rc = lower_stepwise(p, &ol, in, out, (int)dataType, (int)reduceOp);
+        rc = lower_stepwise(p, &ol, in, out, scratch, (int)dataType, (int)reduceOp);
     else
         rc = lower_fused(p, (int)alg, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
     hg_oplist_free(&ol);
@@ -311,7 +343,7 @@ int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread)
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     HcommGfxPlan* p = (HcommGfxPlan*)plan; /* the graph is a cache, not part of the plan's meaning */
-    if (t->recorder || p->nlaunch < 2 || !use_graph() || p->graph_state < 0 || hg_rt_stream_is_capturing(t->stream))
+    if (t->recorder || p->nlaunch < 2 || !p->graph_wanted || p->graph_state < 0 || hg_rt_stream_is_capturing(t->stream))
         return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
     if (p->graph_state == 1 && p->graph_stream != t->stream) {
         hg_rt_graph_destroy(p->graph_exec);
@@ -340,6 +372,14 @@ int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread)
     }
     for (uint32_t i = 0; i < p->nlaunch; ++i) hg_log_only(t, &p->launches[i]);
     return hg_rt_graph_launch(p->graph_exec, t->stream);
+}
+
+int32_t HcommGfxPlanSetGraphReplay(HcommGfxPlan* plan, int32_t enable)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;
+    plan->graph_wanted = enable ? 1 : 0;
+    if (plan->graph_state < 0) plan->graph_state = 0;
+    return HCCL_SUCCESS;
 }
 
 int32_t HcommGfxPlanDestroy(HcommGfxPlan* plan)

@@ -225,6 +225,116 @@ static int sched_rs_mesh(HgOpList* l, uint32_t n, uint64_t count, uint64_t strid
     return HCCL_SUCCESS;
 }
 
+#define SCR 2u
+
+/* Slot size of the deterministic mesh allreduce: ceil(total / n) rounded up to 16 KiB, or to 512 B, or to the
+ * element size, whichever is the first to keep n-1 slots within the message
+ * (AllReduceLocalReduce::PrepareSlice, temp_all_reduce/all_reduce_local_reduce.cc:69-92, with the communication
+ * buffer distinct from the user output so that sizeLimit = totalSize). */
+static uint64_t local_reduce_slot(uint64_t total, uint32_t n, uint32_t unit)
+{
+    const uint64_t ori = (total + n - 1) / n;
+    const uint64_t align[3] = {16384, 512, unit};
+    uint64_t per = 0;
+    for (int a = 0; a < 3; ++a) {
+        per = (ori == 0) ? align[a] : ((ori + align[a] - 1) / align[a]) * align[a];
+        if (per * (n - 1) <= total) break;
+    }
+    return per;
+}
+
+static void local_reduce_slices(uint64_t total, uint32_t n, uint32_t unit, HcommGfxSlice* sl, uint64_t* per_out)
+{
+    const uint64_t per = local_reduce_slot(total, n, unit);
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < n; ++i) {
+        sl[i].size = residue > per ? per : residue;
+        sl[i].offset = residue ? total - residue : total;
+        residue -= sl[i].size;
+    }
+    *per_out = per;
+}
+
+uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype)
+{
+    if (alg != HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE || n < 2) return 0;
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    return (uint64_t)n * local_reduce_slot(count * unit, n, unit);
+}
+
+/* AllReduceLocalReduce, temp_all_reduce/all_reduce_local_reduce.cc.  Stated per destination rank d: its window
+ * of n-1 slots starts at slot 0 (slot 1 for the last rank), slot w of the window is filled by rank d - k where
+ * k is the round that maps to w (:225-229), the neighbour d + 1 reduces straight onto d's own copy (:230-247),
+ * the slots are folded towards the slot at d's natural offset (:301-364), and everybody fetches that slot
+ * (:417-424). */
+static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* :154-163 */
+    if (n & (n - 1)) return HCCL_E_PARA;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    uint64_t per;
+    local_reduce_slices(total, n, unit, sl, &per);
+    const uint32_t half_n = n / 2; /* 2^floor(log2(n-1)) for a power-of-two n */
+    uint32_t step = 0;
+    for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, COPY, d, SCR, sl[d].offset, d, IN, sl[d].offset, sl[d].size));
+    ++step;
+    for (uint32_t k = 1; k < n; ++k, ++step)
+        for (uint32_t d = 0; d < n; ++d) {
+            const uint64_t base = (d == n - 1) ? per : 0;
+            const uint32_t sender = modn((int64_t)d - k, n);
+            if (k == n - 1) {
+                const uint32_t own = (d == n - 1) ? d - 1 : d;
+                CHK(push(l, step, REDUCE, d, SCR, base + (uint64_t)own * per, sender, IN, sl[d].offset, sl[d].size));
+            } else {
+                uint32_t w = (d + k) % (n - 1);
+                if (d == n - 1) w = (w + n - 2) % (n - 1);
+                CHK(push(l, step, COPY, d, SCR, base + (uint64_t)w * per, sender, IN, sl[d].offset, sl[d].size));
+            }
+        }
+    /* fold the n-1 slots: first the slots beyond the power-of-two block onto (or from) the first ones ... */
+    for (uint32_t d = 0; d < n; ++d) {
+        const uint64_t base = (d == n - 1) ? per : 0;
+        for (uint32_t i = 0; i + 1 < half_n; ++i) {
+            const uint64_t lo = base + (uint64_t)i * per, hi = base + (uint64_t)(half_n + i) * per;
+            if (d < half_n) CHK(push(l, step, REDUCE, d, SCR, lo, d, SCR, hi, sl[d].size));
+            else CHK(push(l, step, REDUCE, d, SCR, hi, d, SCR, lo, sl[d].size));
+        }
+    }
+    ++step;
+    /* ... then halve the block of half_n slots towards the slot that holds d's natural offset */
+    uint32_t levels = 0;
+    while ((1u << (levels + 1)) <= half_n) ++levels;
+    for (uint32_t q = 0; q < levels; ++q, ++step)
+        for (uint32_t d = 0; d < n; ++d) {
+            const uint64_t base = (d == n - 1) ? per : 0;
+            uint32_t target = (d < half_n) ? d : ((d - half_n + 1 < half_n - 1) ? d - half_n + 1 : half_n - 1);
+            uint32_t first = (d < half_n) ? 0 : half_n - 1;
+            for (uint32_t z = 0; z < q; ++z) { /* replay the earlier rounds' choice of half */
+                const uint32_t h = half_n >> (z + 1);
+                if (target >= h) {
+                    first += h;
+                    target -= h;
+                }
+            }
+            const uint32_t h = half_n >> (q + 1);
+            for (uint32_t i = 0; i < h; ++i) {
+                const uint64_t lo = base + (uint64_t)(first + i) * per, hi = base + (uint64_t)(first + h + i) * per;
+                if (target < h) CHK(push(l, step, REDUCE, d, SCR, lo, d, SCR, hi, sl[d].size));
+                else CHK(push(l, step, REDUCE, d, SCR, hi, d, SCR, lo, sl[d].size));
+            }
+        }
+    /* gather: own slice from the own window, every other slice from its owner's window (:405-424) */
+    for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, COPY, d, OUT, sl[d].offset, d, SCR, sl[d].offset, sl[d].size));
+    ++step;
+    for (uint32_t k = 1; k < n; ++k, ++step)
+        for (uint32_t d = 0; d < n; ++d) {
+            const uint32_t p = modn((int64_t)d - k, n);
+            CHK(push(l, step, COPY, d, OUT, sl[p].offset, p, SCR, (uint64_t)p * sl[0].size, sl[p].size));
+        }
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
@@ -244,6 +354,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING: rc = sched_allreduce_mesh_oneshot(l, n, count, unit, 1); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH: rc = sched_rs_mesh(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, stride, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE: rc = sched_allreduce_local_reduce(l, n, count, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

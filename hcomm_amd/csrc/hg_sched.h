@@ -16,5 +16,7 @@ typedef struct {
 /* stride: elements between consecutive ranks' slices in the input of the scatter algorithms (0 = count). */
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype);
 void hg_oplist_free(HgOpList* l);
+/* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
+uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);
 
 #endif

@@ -320,7 +320,14 @@ typedef enum {
     /* InsTempAllReduceMesh1DOneShot: src/legacy/ascend950/service/collective/alg/coll_alg_factory/alg_template/
        ins_alg_template/ins_temp_all_reduce_mesh_1D_one_shot.cc:86-164 - out = in[r], then the other ranks'
        inputs in ascending rank order (the legacy one-shot folds them in the order r+1, r+2, ...) */
-    HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING = 6
+    HCOMM_GFX_ALG_ALLREDUCE_MESH_ONESHOT_ASCENDING = 6,
+    /* AllReduceLocalReduce (the deterministic mesh allreduce): src/legacy/ascend910/algorithm/base/alg_template/
+       temp_all_reduce/all_reduce_local_reduce.cc:139-436.  Every rank gathers the other ranks' copies of its
+       slice into N-1 slots of its communication buffer, folds the slots in a fixed tree order, and the ranks
+       then gather the results.  Needs a third buffer per rank (HcommGfxPlanCreateEx, HcommGfxScratchBytes) and a
+       power-of-two rank count: the template's slot arithmetic puts the result where the gather reads it only
+       when N = 2 * 2^floor(log2(N-1)).  Step-wise lowering only. */
+    HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE = 7
 } HcommGfxAlgorithm;
 
 typedef enum {
@@ -377,6 +384,20 @@ int32_t HcommGfxPlanCreateStrided(
     uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
 /*
+ * As HcommGfxPlanCreateStrided, with a per-rank communication ("scratch") buffer for the algorithms that stage
+ * data in one (the CCL buffer of the reference).  scratch[r] must be 128-byte aligned and hold
+ * HcommGfxScratchBytes() bytes; scratch may be NULL for algorithms that need none.
+ */
+int32_t HcommGfxPlanCreateEx(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* in, void* const* out,
+    void* const* scratch, uint64_t count, uint64_t strideCount, HcommDataType dataType, HcommReduceOp reduceOp,
+    HcommGfxPlan** plan);
+
+/* Bytes of communication buffer each rank needs for alg (0 for algorithms that stage nothing). */
+int32_t HcommGfxScratchBytes(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, HcommDataType dataType,
+                             uint64_t* bytes);
+
+/*
  * Enqueue every launch of the plan on the thread, in order.  May be called any number of times, from one host
  * thread at a time.  With HCOMM_GFX_GRAPH=1 in the environment a plan of two or more launches is replayed as a
  * HIP graph captured at its first run on the thread's stream (off by default: it measured slower than
@@ -384,6 +405,9 @@ int32_t HcommGfxPlanCreateStrided(
  * issued individually and become part of the caller's graph.
  */
 int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread);
+
+/* Switch graph replay of HcommGfxPlanRun on or off for this plan (default: HCOMM_GFX_GRAPH in the environment). */
+int32_t HcommGfxPlanSetGraphReplay(HcommGfxPlan* plan, int32_t enable);
 
 /* Enqueue launches [first, first + n) only (used to time one phase of a plan). */
 int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n);
@@ -410,9 +434,9 @@ typedef struct {
     uint32_t step;    /* schedule step (ranks act in parallel within a step) */
     uint32_t kind;    /* 0 = copy, 1 = reduce */
     uint32_t rank;    /* rank that executes the operation (owner of dst) */
-    uint32_t dstBuf;  /* 0 = in[rank], 1 = out[rank] */
+    uint32_t dstBuf;  /* 0 = in[rank], 1 = out[rank], 2 = scratch[rank] (communication buffer) */
     uint32_t srcRank; /* rank whose buffer is read */
-    uint32_t srcBuf;  /* 0 = in[srcRank], 1 = out[srcRank] */
+    uint32_t srcBuf;  /* 0 = in[srcRank], 1 = out[srcRank], 2 = scratch[srcRank] */
     uint64_t dstOff;  /* bytes */
     uint64_t srcOff;  /* bytes */
     uint64_t bytes;

@@ -16,7 +16,7 @@ REF_PATH = os.path.join(HERE, "_ref", "libhcomm_ref.so")
 SUM, PROD, MAX, MIN = 0, 1, 2, 3
 I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
 ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
-    ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING = range(7)
+    ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING, ALG_ALLREDUCE_LOCAL_REDUCE = range(8)
 
 # storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
 NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
@@ -56,6 +56,8 @@ def lib():
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_set_stride.argtypes = [C.c_uint64]
         L.orc_set_stride.restype = None
+        L.orc_set_scratch.argtypes = [C.POINTER(C.c_void_p)]
+        L.orc_set_scratch.restype = None
         L.orc_get_threads.restype = C.c_int
         L.orc_f16_to_f32.restype = C.c_float
         L.orc_f16_to_f32.argtypes = [C.c_uint16]
@@ -171,17 +173,21 @@ def trace(alg, n, count, dtype, stride=0):
     return [ops[i].astuple() for i in range(total)]
 
 
-def run(alg, ins, outs, count, dtype, op, stride=0):
+def run(alg, ins, outs, count, dtype, op, stride=0, scratch=None):
     """Execute a collective in place on lists of numpy arrays (one per rank).  stride: elements between the
-    input slices of the scatter algorithms (0 = dense)."""
+    input slices of the scatter algorithms (0 = dense).  scratch: per-rank communication buffers (uint8 arrays)
+    for the algorithms that stage data."""
     n = len(ins)
     a = (C.c_void_p * n)(*[x.ctypes.data for x in ins])
     b = (C.c_void_p * n)(*[x.ctypes.data for x in outs])
+    sc = (C.c_void_p * n)(*[x.ctypes.data for x in scratch]) if scratch is not None else None
     lib().orc_set_stride(stride)
+    lib().orc_set_scratch(sc)
     try:
         rc = lib().orc_run(alg, n, a, b, count, dtype, op)
     finally:
         lib().orc_set_stride(0)
+        lib().orc_set_scratch(None)
     if rc:
         raise ValueError("orc_run rc=%d" % rc)
 

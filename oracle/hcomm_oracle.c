@@ -345,7 +345,7 @@ static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint3
     o->bytes = bytes;
 }
 
-enum { B_IN = 0, B_OUT = 1, K_COPY = 0, K_REDUCE = 1 };
+enum { B_IN = 0, B_OUT = 1, B_SCR = 2, K_COPY = 0, K_REDUCE = 1 };
 
 /* ReduceScatterRing::RunReduceScatter for one rank, tpl/temp_reduce_scatter/reduce_scatter_ring.cc:182-312.
  * `out_sl` NULL: the allreduce case, where the template's output memory IS the input memory
@@ -528,6 +528,103 @@ static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count,
     emit(t, step, K_COPY, rank, B_OUT, 0, rank, B_IN, (uint64_t)rank * stride * unit, sz); /* :199-211 */
 }
 
+/* AllReduceLocalReduce for one rank, tpl/temp_all_reduce/all_reduce_local_reduce.cc:139-436 - the deterministic
+ * mesh allreduce.  Three buffers per rank: user input (B_IN), the communication buffer commMemOut (B_SCR) and
+ * user output (B_OUT).  An op is recorded under the rank that OWNS the destination; the rank that issues it is
+ * the src rank.  Rounds that the reference runs concurrently on sub-streams get one step each.
+ * The slot arithmetic of RunLocalReduce leaves the result at the offset the gather reads (:419) only for a
+ * power-of-two rank count; other counts are refused. */
+static int prog_allreduce_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) { /* :154-163 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
+        return 0;
+    }
+    if (n & (n - 1)) return -1;
+    /* PrepareSlice :69-120; the communication buffer is not the user output, so sizeLimit = totalSize (:84-88) */
+    OrcSlice sl[ORC_MAX_RANKS], start[ORC_MAX_RANKS];
+    const uint64_t ori = (total + n - 1) / n;
+#define ROUNDUP(v, d) (((v) == 0) ? (uint64_t)(d) : ((((v) + (d) - 1) / (d)) * (d))) /* RoundUpWithDivisor */
+    uint64_t per = ROUNDUP(ori, 16384);                              /* HCCL_MIN_SLICE_ALIGN_910B */
+    if (per * (n - 1) > total) per = ROUNDUP(ori, 512);              /* HCCL_MIN_SLICE_ALIGN_ONCHIP */
+    if (per * (n - 1) > total) per = ROUNDUP(ori, unit);
+#undef ROUNDUP
+    uint64_t residue = total;
+    uint32_t i = 0;
+    while (residue > 0) {
+        const uint64_t sz = per < residue ? per : residue;
+        sl[i].size = sz;
+        sl[i].offset = total - residue;
+        i++;
+        residue -= sz;
+        start[i - 1].size = per;
+        start[i - 1].offset = (i != n) ? 0 : per; /* :102-110: the last rank's window starts one slot later */
+    }
+    while (i < n) {
+        sl[i].size = 0;
+        sl[i].offset = total;
+        start[i].size = 0;
+        start[i].offset = 0;
+        i++;
+    }
+    uint32_t step = 0;
+    /* RunReduceScatter :197-199: own slice, user input -> communication buffer at its natural offset */
+    emit(t, step++, K_COPY, rank, B_SCR, sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size);
+    for (uint32_t round = 1; round < n; round++) { /* :222-266 */
+        const uint32_t dst_rank = (rank + round) % n;
+        uint32_t dst_slice = (dst_rank + round) % (n - 1);
+        if (dst_rank == n - 1) dst_slice = (dst_slice + n - 1 - 1) % (n - 1);
+        if (round == n - 1) {
+            dst_slice = (dst_rank == n - 1) ? (dst_rank - 1) : dst_rank; /* :233 */
+            emit(t, step++, K_REDUCE, dst_rank, B_SCR, start[dst_rank].offset + dst_slice * start[dst_rank].size, rank,
+                 B_IN, sl[dst_rank].offset, sl[dst_rank].size);
+        } else {
+            emit(t, step++, K_COPY, dst_rank, B_SCR, start[dst_rank].offset + dst_slice * start[dst_rank].size, rank,
+                 B_IN, sl[dst_rank].offset, sl[dst_rank].size);
+        }
+    }
+    /* RunLocalReduce :301-364 */
+    uint32_t power = 0;
+    while ((2u << power) <= n - 1) power++; /* floor(log2(n - 1)) */
+    const uint32_t rank_power = 1u << power;
+    const uint64_t align = start[rank].size;
+    const uint64_t size = sl[rank].size;
+    for (uint32_t k = 0; k < n - rank_power - 1; ++k) { /* :311-327, all in one step */
+        if (rank < rank_power)
+            emit(t, step, K_REDUCE, rank, B_SCR, start[rank].offset + k * align, rank, B_SCR,
+                 start[rank].offset + (rank_power + k) * align, size);
+        else
+            emit(t, step, K_REDUCE, rank, B_SCR, start[rank].offset + (rank_power + k) * align, rank, B_SCR,
+                 start[rank].offset + k * align, size);
+    }
+    step++;
+    uint32_t center = rank < rank_power ? rank : (rank - rank_power + 1);
+    if (center > rank_power - 1) center = rank_power - 1;
+    uint64_t offset = rank < rank_power ? 0 : ((n - rank_power - 1) * align);
+    offset += start[rank].offset;
+    for (uint32_t round = 0; round < power; round++) { /* :333-362 */
+        const uint32_t slices_num = rank_power >> (round + 1);
+        if (center < slices_num) {
+            for (uint32_t k = 0; k < slices_num; ++k)
+                emit(t, step, K_REDUCE, rank, B_SCR, offset + k * align, rank, B_SCR, offset + (slices_num + k) * align, size);
+        } else {
+            for (uint32_t k = 0; k < slices_num; ++k)
+                emit(t, step, K_REDUCE, rank, B_SCR, offset + (slices_num + k) * align, rank, B_SCR, offset + k * align, size);
+            offset = offset + slices_num * align;
+            center -= slices_num;
+        }
+        step++;
+    }
+    /* RunAllGather :366-436 */
+    emit(t, step++, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_SCR, sl[rank].offset, sl[rank].size); /* :405-409 */
+    for (uint32_t round = 1; round < n; round++) {
+        const uint32_t peer = (rank + n - round) % n; /* BackwardRank, tpl/inc_all_reduce_deter/all_reduce_local_reduce_pub.h:44-50 */
+        emit(t, step++, K_COPY, rank, B_OUT, sl[peer].offset, peer, B_SCR, (uint64_t)peer * sl[0].size, sl[peer].size); /* :419-423 */
+    }
+    return 0;
+}
+
 enum {
     ORC_ALG_ALLREDUCE_RING = 0,
     ORC_ALG_RS_RING_STAGE = 1,
@@ -535,7 +632,8 @@ enum {
     ORC_ALG_ALLREDUCE_MESH_ONESHOT = 3,
     ORC_ALG_RS_MESH = 4,
     ORC_ALG_RS_RING_STANDALONE = 5,
-    ORC_ALG_ALLREDUCE_MESH_ASCENDING = 6
+    ORC_ALG_ALLREDUCE_MESH_ASCENDING = 6,
+    ORC_ALG_ALLREDUCE_LOCAL_REDUCE = 7
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -568,6 +666,12 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, stride, unit); break;
             case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
+            case ORC_ALG_ALLREDUCE_LOCAL_REDUCE:
+                if (prog_allreduce_local_reduce(t, r, n, count, unit) != 0) {
+                    free(t->ops);
+                    return -1;
+                }
+                break;
             default: free(t->ops); return -1;
         }
     }
@@ -575,8 +679,26 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
         free(t->ops);
         return -2;
     }
-    /* lock step: order by step, then rank (stable within a rank because a rank emits one op per step) */
-    qsort(t->ops, t->n, sizeof(OrcOp), cmp_ops);
+    /* lock step: order by step, then by the rank that owns the destination; emission order is kept among equals */
+    if (t->n > 1) {
+        OrcOp* tmp = (OrcOp*)malloc(t->n * sizeof(OrcOp));
+        if (!tmp) {
+            free(t->ops);
+            return -2;
+        }
+        for (uint64_t width = 1; width < t->n; width *= 2) { /* bottom-up merge sort: stable */
+            for (uint64_t lo = 0; lo < t->n; lo += 2 * width) {
+                const uint64_t mid = lo + width < t->n ? lo + width : t->n;
+                const uint64_t hi = lo + 2 * width < t->n ? lo + 2 * width : t->n;
+                uint64_t a = lo, b = mid, k = lo;
+                while (a < mid && b < hi) tmp[k++] = (cmp_ops(&t->ops[b], &t->ops[a]) < 0) ? t->ops[b++] : t->ops[a++];
+                while (a < mid) tmp[k++] = t->ops[a++];
+                while (b < hi) tmp[k++] = t->ops[b++];
+            }
+            memcpy(t->ops, tmp, t->n * sizeof(OrcOp));
+        }
+        free(tmp);
+    }
     return 0;
 }
 
@@ -602,11 +724,22 @@ static int ranges_overlap(uintptr_t a, uint64_t an, uintptr_t b, uint64_t bn) { 
  * after another equals executing them concurrently.  Returns 0, -1 bad argument, -2 out of memory,
  * -3 conflict inside a step.
  */
+static void* const* g_scratch = NULL; /* per-rank communication buffers for the next orc_run (or NULL) */
+
+void orc_set_scratch(void* const* scratch) { g_scratch = scratch; }
+
+#define BUFPTR(buf, rank) ((buf) == B_SCR ? g_scratch[rank] : ((buf) ? out[rank] : in[rank]))
+
 int orc_run(int alg, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype, int op)
 {
     OrcTrace t;
     int rc = build_trace(&t, alg, n, count, dtype);
     if (rc) return rc;
+    for (uint64_t q = 0; q < t.n; q++)
+        if ((t.ops[q].dst_buf == B_SCR || t.ops[q].src_buf == B_SCR) && !g_scratch) {
+            free(t.ops);
+            return -1;
+        }
     const uint32_t unit = orc_dtype_size(dtype);
     uint64_t i = 0;
     while (i < t.n) {
@@ -614,12 +747,12 @@ int orc_run(int alg, uint32_t n, void* const* in, void* const* out, uint64_t cou
         while (j < t.n && t.ops[j].step == t.ops[i].step) j++;
         for (uint64_t a = i; a < j; a++) {
             const OrcOp* x = &t.ops[a];
-            const uintptr_t xd = (uintptr_t)(x->dst_buf ? out[x->rank] : in[x->rank]) + x->dst_off;
+            const uintptr_t xd = (uintptr_t)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
             for (uint64_t b = i; b < j; b++) {
                 if (a == b) continue;
                 const OrcOp* y = &t.ops[b];
-                const uintptr_t yd = (uintptr_t)(y->dst_buf ? out[y->rank] : in[y->rank]) + y->dst_off;
-                const uintptr_t ys = (uintptr_t)(y->src_buf ? out[y->src_rank] : in[y->src_rank]) + y->src_off;
+                const uintptr_t yd = (uintptr_t)BUFPTR(y->dst_buf, y->rank) + y->dst_off;
+                const uintptr_t ys = (uintptr_t)BUFPTR(y->src_buf, y->src_rank) + y->src_off;
                 if (ranges_overlap(xd, x->bytes, yd, y->bytes) || ranges_overlap(xd, x->bytes, ys, y->bytes)) {
                     free(t.ops);
                     return -3;
@@ -628,8 +761,8 @@ int orc_run(int alg, uint32_t n, void* const* in, void* const* out, uint64_t cou
         }
         for (uint64_t a = i; a < j; a++) {
             const OrcOp* x = &t.ops[a];
-            char* d = (char*)(x->dst_buf ? out[x->rank] : in[x->rank]) + x->dst_off;
-            const char* s = (const char*)(x->src_buf ? out[x->src_rank] : in[x->src_rank]) + x->src_off;
+            char* d = (char*)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
+            const char* s = (const char*)BUFPTR(x->src_buf, x->src_rank) + x->src_off;
             if (x->kind == K_COPY)
                 orc_copy(d, s, x->bytes);
             else if (orc_reduce(d, s, x->bytes / unit, dtype, op) != 0) {

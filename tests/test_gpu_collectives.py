@@ -19,6 +19,7 @@ ALGS = {
     "mesh_rs": (h.Alg.REDUCE_SCATTER_MESH, oracle.ALG_RS_MESH),
     "ring_rs": (h.Alg.REDUCE_SCATTER_RING_STANDALONE, oracle.ALG_RS_RING_STANDALONE),
     "mesh_ascending": (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, oracle.ALG_ALLREDUCE_MESH_ASCENDING),
+    "local_reduce": (h.Alg.ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_LOCAL_REDUCE),
 }
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
 
@@ -43,19 +44,26 @@ def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None, stri
     sentinel = gen(dt, out_count, 999, "wide")
     want_in = [x.copy() for x in host_in]
     want_out = [sentinel.copy() for _ in range(n)]
-    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o, stride)
+    sb = h.scratch_bytes(ALGS[alg][0], n, count, dt)
+    junk = np.random.default_rng(5).integers(0, 256, sb, dtype=np.uint8) if sb else None
+    want_scr = [junk.copy() for _ in range(n)] if sb else None
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o, stride, scratch=want_scr)
     d_in = [to_dev(x) for x in host_in]
     d_out = [to_dev(sentinel) for _ in range(n)]
+    d_scr = [to_dev(junk) for _ in range(n)] if sb else None
     # zero-length tensors have a null data_ptr; give the plan a real (unused) address instead
     pad = to_dev(np.zeros(256, np.uint8))
     ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
-    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o, stride)
+    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o, stride,
+                  [ptr(t) for t in d_scr] if sb else None)
     try:
         assert plan.run(thread) == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
         for r in range(n):
             assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt, "in[%d]" % r)
             assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+            if sb:  # the communication buffer too, slot by slot (bytes never written keep their junk)
+                assert np.array_equal(d_scr[r].cpu().numpy(), want_scr[r]), "scratch[%d]" % r
         return plan.info.launches, plan.info.algorithmicBytes, plan.info.movedBytes
     finally:
         plan.destroy()
@@ -106,6 +114,14 @@ CASES = [
     ("mesh_ascending", 8, 100003, "fp16", "sum"),
     ("mesh_ascending", 5, 4097, "fp32", "max"),
     ("mesh_ascending", 1, 10, "int8", "sum"),
+    ("local_reduce", 8, 1 << 20, "bf16", "sum"),
+    ("local_reduce", 4, 100003, "fp32", "sum"),
+    ("local_reduce", 16, 70001, "fp16", "max"),
+    ("local_reduce", 32, 300007, "int32", "sum"),
+    ("local_reduce", 2, 4099, "int8", "min"),
+    ("local_reduce", 8, 1001, "int16", "sum"),     # slots fall back to 512-byte / element alignment
+    ("local_reduce", 8, 7, "fp32", "sum"),
+    ("local_reduce", 1, 100, "fp32", "sum"),
 ]
 
 
@@ -159,9 +175,9 @@ def test_non_associative_inputs_expose_order(gpu_thread):
 
 def test_plan_can_run_repeatedly_and_by_range(gpu_thread):
     """A plan is reusable: re-uploading inputs and running again gives the same result; RunRange over all
-    launches one at a time equals Run.  With HCOMM_GFX_GRAPH=1 in the environment Run replays the 15 launches
-    as a HIP graph, and this test then checks several graph replays, with eager work and synchronisation in
-    between, against the kernel-by-kernel result."""
+    launches one at a time equals Run.  From the fourth attempt on Run replays the 15 launches as a HIP graph:
+    several replays, with eager work and synchronisation in between, are checked against the same result as
+    the kernel-by-kernel runs."""
     n, count, dt = 8, 100003, oracle.F32
     host_in = [gen(dt, count, 50 + r) for r in range(n)]
     want_in = [x.copy() for x in host_in]
@@ -172,12 +188,14 @@ def test_plan_can_run_repeatedly_and_by_range(gpu_thread):
     plan = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, [t.data_ptr() for t in d_in],
                   [t.data_ptr() for t in d_out], count, dt, oracle.SUM)
     import torch
-    for attempt in range(6):
+    for attempt in range(8):
         for r in range(n):
             d_in[r].copy_(torch.from_numpy(host_in[r].view(np.uint8)))
             d_out[r].zero_()
         torch.cuda.synchronize()
-        if attempt in (2, 5):
+        if attempt == 3:
+            assert plan.set_graph_replay(True) == 0
+        if attempt in (2, 7):
             for i in range(plan.info.launches):
                 assert plan.run_range(gpu_thread, i, 1) == 0
         else:

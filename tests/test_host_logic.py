@@ -172,6 +172,30 @@ def test_batch_transfer_descriptors(rec):
     assert ctypes.sizeof(h.BatchTransferDesc) == 64    # include/hcomm_primitives.h:91-131
 
 
+def test_local_reduce_plan_needs_scratch_and_power_of_two(rec):
+    i, o = ptrs(8, 1 << 22)
+    sc, _ = ptrs(8, 1 << 23, base=0x90000000)
+    count = 1 << 20
+    assert h.scratch_bytes(h.Alg.ALLREDUCE_LOCAL_REDUCE, 8, count, DT.FP32) == 8 * (count * 4 // 8)
+    assert h.scratch_bytes(h.Alg.ALLREDUCE_RING, 8, count, DT.FP32) == 0
+    with pytest.raises(h.HcommError) as e:
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i, o, count, DT.FP32, OP.SUM)
+    assert e.value.code == R.E_PTR                                   # no communication buffers given
+    with pytest.raises(h.HcommError) as e:
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i[:6], o[:6], count, DT.FP32, OP.SUM, 0, sc[:6])
+    assert e.value.code == R.E_PARA                                  # 6 ranks
+    with pytest.raises(h.HcommError) as e:
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM, 0, sc)
+    assert e.value.code == R.E_NOT_SUPPORT
+    p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i, o, count, DT.FP32, OP.SUM, 0, sc)
+    # own copy | 6 gather rounds merged | neighbour reduce | fold + 2 halving rounds | own gather + 7 rounds merged
+    kinds = [(r.kind, r.nseg) for r in p.launches()]
+    assert kinds[0] == (h.Kernel.COPY, 32) and sum(ns for k, ns in kinds if k == h.Kernel.COPY) == 8 + 48 + 8 + 56
+    assert sum(ns for k, ns in kinds if k == h.Kernel.REDUCE2) == 8 + 8 * 3 + 8 * 2 + 8 * 1
+    assert p.info.movedBytes == p.info.algorithmicBytes
+    p.destroy()
+
+
 def test_strided_plan_checks():
     i, o = ptrs(4, 1 << 20)
     p = h.Plan(h.Alg.REDUCE_SCATTER_MESH, h.Lowering.FUSED, i, o, 1000, DT.FP32, OP.SUM, stride=1500)

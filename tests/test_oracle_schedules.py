@@ -15,8 +15,13 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
-        oracle.ALG_ALLREDUCE_MESH_ASCENDING]
+        oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE]
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE)
+
+
+def scratch_for(alg, n, count, dt):
+    sb = h.scratch_bytes(alg, n, count, dt)
+    return [np.zeros(sb, np.uint8) for _ in range(n)] if sb else None
 
 
 # ---- slice tables ---------------------------------------------------------------------------------------
@@ -187,11 +192,13 @@ def test_every_rank_contributes_exactly_once(alg, n):
     """Rank r contributes 4^r per element (+ a position code in the low part for scatter variants); the
     int32 sum has base-4 digit 1 for every rank iff each was folded in exactly once (no carries: digits <= 3
     for up to 3 repeats).  MAX / MIN give the closed forms n-1 / 0 on a second pass."""
+    if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+        pytest.skip("power-of-two rank counts only")
     count = 777
     per_in = n * count if alg in SCATTER_OUT else count
     ins = [np.full(per_in, 4 ** r, np.int32) for r in range(n)]
     outs = [np.full(count, -1, np.int32) for _ in range(n)]
-    oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM)
+    oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM, scratch=scratch_for(alg, n, count, oracle.I32))
     total = sum(4 ** r for r in range(n))
     if alg == oracle.ALG_RS_RING_STAGE:
         sl = oracle.slices_ring(count, 4, n)
@@ -204,7 +211,7 @@ def test_every_rank_contributes_exactly_once(alg, n):
     for op, want in ((oracle.MAX, n - 1), (oracle.MIN, 0)):
         ins = [np.full(per_in, r, np.int32) for r in range(n)]
         outs = [np.full(count, -1, np.int32) for _ in range(n)]
-        oracle.run(alg, ins, outs, count, oracle.I32, op)
+        oracle.run(alg, ins, outs, count, oracle.I32, op, scratch=scratch_for(alg, n, count, oracle.I32))
         if alg != oracle.ALG_RS_RING_STAGE:
             assert all((o == want).all() for o in outs)
 
@@ -219,6 +226,29 @@ def test_scatter_variants_deliver_the_right_slice():
         oracle.run(alg, [x.copy() for x in ins], outs, count, oracle.I32, oracle.SUM)
         for r in range(n):
             assert np.array_equal(outs[r], want[r * count:(r + 1) * count].astype(np.int32))
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])
+def test_local_reduce_trees_hand_derived(op):
+    """The deterministic mesh allreduce (three buffers per rank): fold order per slice worked out by hand."""
+    for n_s, trees in GOLD["local_reduce_slice_tree"].items():
+        n = int(n_s)
+        count = n * 4096 * 4 + 5000       # 16 KiB-aligned slots, ragged last slice
+        ins = order_sensitive_inputs(n, count, op, seed=30 + n)
+        outs = [np.zeros(count, np.float32) for _ in range(n)]
+        sb = h.scratch_bytes(h.Alg.ALLREDUCE_LOCAL_REDUCE, n, count, oracle.F32)
+        per = sb // n
+        assert per % 16384 == 0 and per * (n - 1) <= count * 4 < per * n
+        scr = [np.zeros(sb, np.uint8) for _ in range(n)]
+        oracle.run(oracle.ALG_ALLREDUCE_LOCAL_REDUCE, [x.copy() for x in ins], outs, count, oracle.F32, op, scratch=scr)
+        for d_s, tree in trees.items():
+            lo = int(d_s) * per // 4
+            hi = min(count, lo + per // 4)
+            want = eval_tree(tree, [x[lo:hi] for x in ins], op)
+            for r in range(n):
+                assert np.array_equal(outs[r][lo:hi].view(np.uint32), want.view(np.uint32)), (n, d_s, r)
+    with pytest.raises(ValueError):        # the slot arithmetic only closes for a power-of-two rank count
+        oracle.trace(oracle.ALG_ALLREDUCE_LOCAL_REDUCE, 6, 1000, oracle.F32)
 
 
 def test_strided_scatter_input_layout():
@@ -248,6 +278,8 @@ def test_strided_scatter_input_layout():
 @pytest.mark.parametrize("alg", ALGS)
 def test_product_generator_equals_oracle_trace(alg):
     for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32):
+        if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+            continue
         for count, dt in ((0, oracle.F32), (1, oracle.I8), (5, oracle.I8), (1000, oracle.F16), (100003, oracle.F32),
                           (100000003, oracle.I8)):
             a = oracle.trace(alg, n, count, dt)
@@ -274,11 +306,14 @@ def test_steps_are_conflict_free_and_errors_are_reported():
     for every rank count, and bad arguments are reported."""
     for alg in ALGS:
         for n in range(1, 18):
+            if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+                continue
             count = 100
             per_in = n * count if alg in SCATTER_OUT else count
             ins = [np.ones(per_in, np.int32) for _ in range(n)]
             outs = [np.zeros(count, np.int32) for _ in range(n)]
-            oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM)  # raises on rc != 0
+            oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM,
+                       scratch=scratch_for(alg, n, count, oracle.I32))  # raises on rc != 0
     with pytest.raises(ValueError):
         oracle.trace(99, 4, 10, oracle.F32)
     with pytest.raises(ValueError):

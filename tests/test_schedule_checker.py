@@ -10,12 +10,15 @@ ALL = [(h.Alg.ALLREDUCE_RING, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_RING, Exp
        (h.Alg.ALLREDUCE_RHD, Expect.ALLREDUCE), (h.Alg.ALLREDUCE_MESH_ONESHOT, Expect.ALLREDUCE),
        (h.Alg.REDUCE_SCATTER_MESH, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.REDUCE_SCATTER_RING_STANDALONE, Expect.REDUCE_SCATTER_OUT),
-       (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, Expect.ALLREDUCE)]
+       (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, Expect.ALLREDUCE),
+       (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE)]
 
 
 @pytest.mark.parametrize("alg,expect", ALL)
 def test_generated_schedules_pass(alg, expect):
     for n in list(range(1, 18)) + [24, 31, 32]:
+        if alg == h.Alg.ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+            continue
         for count, dt, unit in ((0, h.HcommDataType.FP32, 4), (1, h.HcommDataType.INT8, 1),
                                 (1000, h.HcommDataType.FP16, 2), (100003, h.HcommDataType.FP32, 4)):
             assert h.schedule_check(alg, n, count, dt)[:2] == (0, 0), (alg, n, count)
