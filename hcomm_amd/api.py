@@ -61,7 +61,8 @@ class CommEngine:
 
 class Alg:
     ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
-        REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING, ALLREDUCE_LOCAL_REDUCE = range(8)
+        REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING, ALLREDUCE_LOCAL_REDUCE, \
+        ALLREDUCE_CHUNK_MESH = range(9)
 
 
 class Lowering:

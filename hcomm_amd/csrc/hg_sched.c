@@ -257,9 +257,42 @@ static void local_reduce_slices(uint64_t total, uint32_t n, uint32_t unit, Hcomm
 
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype)
 {
-    if (alg != HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE || n < 2) return 0;
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (n < 2) return 0;
+    if (alg == HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH) return count * unit;
+    if (alg != HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE) return 0;
     return (uint64_t)n * local_reduce_slot(count * unit, n, unit);
+}
+
+/* AllReduceChunkMesh, temp_all_reduce/all_reduce_chunk_mesh.cc (the communication buffer is not the user output:
+ * the "single operator" branches).  Stated per sub-chunk: sub-chunk q of rank r's slice folds the peers' copies in
+ * the rotation r+q+1, r+q+2, ..., wrapping from r+n-1 back to r+1 (:234-236), one peer per round. */
+static int sched_allreduce_chunk_mesh(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* :137-146 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS], sub[HCOMM_GFX_MAX_RANKS];
+    CHK(HcommGfxCalcSlices(count, unit, n, sl)); /* PrepareSlice :69-102 = the 128-byte-aligned table */
+    uint32_t step = 0;
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, step, COPY, r, SCR, 0, r, IN, 0, total)); /* :188-193 */
+    ++step;
+    for (uint32_t round = 1; round < n; ++round, ++step)
+        for (uint32_t r = 0; r < n; ++r) {
+            CHK(HcommGfxCalcSlices(sl[r].size / unit, unit, n - 1, sub)); /* :108-113 */
+            for (uint32_t q = 0; q + 1 < n; ++q) {
+                const uint32_t hop = (q + round - 1) % (n - 1) + 1; /* 1 .. n-1, starting at q+1 */
+                const uint64_t off = sl[r].offset + sub[q].offset;
+                CHK(push(l, step, REDUCE, r, SCR, off, (r + hop) % n, SCR, off, sub[q].size));
+            }
+        }
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, step, COPY, r, OUT, sl[r].offset, r, SCR, sl[r].offset, sl[r].size));
+    ++step;
+    for (uint32_t k = 1; k < n; ++k, ++step)
+        for (uint32_t r = 0; r < n; ++r) {
+            const uint32_t p = modn((int64_t)r - k, n);
+            CHK(push(l, step, COPY, r, OUT, sl[p].offset, p, SCR, sl[p].offset, sl[p].size));
+        }
+    return HCCL_SUCCESS;
 }
 
 /* AllReduceLocalReduce, temp_all_reduce/all_reduce_local_reduce.cc.  Stated per destination rank d: its window
@@ -355,6 +388,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH: rc = sched_rs_mesh(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE: rc = sched_allreduce_local_reduce(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH: rc = sched_allreduce_chunk_mesh(l, n, count, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

@@ -327,7 +327,13 @@ typedef enum {
        then gather the results.  Needs a third buffer per rank (HcommGfxPlanCreateEx, HcommGfxScratchBytes) and a
        power-of-two rank count: the template's slot arithmetic puts the result where the gather reads it only
        when N = 2 * 2^floor(log2(N-1)).  Step-wise lowering only. */
-    HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE = 7
+    HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE = 7,
+    /* AllReduceChunkMesh (two-shot mesh, what the legacy one-shot executor instantiates for more than two
+       ranks): temp_all_reduce/all_reduce_chunk_mesh.cc:104-345.  Each rank copies its input into its
+       communication buffer, reduces its own slice there in N-1 rounds - sub-chunk p-1 of the slice takes peer
+       r+p, r+p+1, ..., r+N-1, r+1, ..., r+p-1 in that order (a Latin square over links and rounds) - and the
+       ranks gather the slices.  Needs the third buffer (count * unit bytes).  Step-wise lowering only. */
+    HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH = 8
 } HcommGfxAlgorithm;
 
 typedef enum {

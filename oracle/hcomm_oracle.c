@@ -625,6 +625,38 @@ static int prog_allreduce_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, u
     return 0;
 }
 
+/* AllReduceChunkMesh for one rank, tpl/temp_all_reduce/all_reduce_chunk_mesh.cc:104-345, in the configuration
+ * where the communication buffer (B_SCR) is not the user output (the "single operator" branches :186-193,
+ * :239-243).  Slices: PrepareSlice :69-102 over n ranks, then each slice again over n-1 sub-chunks (:104-116). */
+static void prog_allreduce_chunk_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) { /* :137-146 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS], sub[ORC_MAX_RANKS];
+    orc_slices_ring(count, unit, n, sl);                     /* same arithmetic as PrepareSlice :69-102 */
+    orc_slices_ring(sl[rank].size / unit, unit, n - 1, sub); /* sliceMap[rank] :108-113 */
+    uint32_t step = 0;
+    emit(t, step++, K_COPY, rank, B_SCR, 0, rank, B_IN, 0, total); /* :188-193 whole input -> communication buffer */
+    for (uint32_t round = 1; round < n; round++) {                 /* :213-253 */
+        for (uint32_t peer = 1; peer < n; peer++) {
+            const uint32_t gap = (peer + round) > n ? (peer + round - 1) % (n - 1) : (peer + round - 1); /* :235 */
+            const uint32_t dst_rank = (gap + rank) % n;
+            const uint32_t dst_slice = peer - 1;
+            const uint64_t off = sl[rank].offset + sub[dst_slice].offset;
+            emit(t, step, K_REDUCE, rank, B_SCR, off, dst_rank, B_SCR, off, sub[dst_slice].size); /* :245-252 */
+        }
+        step++;
+    }
+    emit(t, step++, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_SCR, sl[rank].offset, sl[rank].size); /* :316-320 */
+    for (uint32_t round = 1; round < n; round++) { /* :322-333 */
+        const uint32_t peer = (rank + n - round) % n; /* BackwardRank, tpl/inc_all_reduce_deter/all_reduce_chunk_mesh_pub.h:45 */
+        emit(t, step++, K_COPY, rank, B_OUT, sl[peer].offset, peer, B_SCR, sl[peer].offset, sl[peer].size);
+    }
+}
+
 enum {
     ORC_ALG_ALLREDUCE_RING = 0,
     ORC_ALG_RS_RING_STAGE = 1,
@@ -633,7 +665,8 @@ enum {
     ORC_ALG_RS_MESH = 4,
     ORC_ALG_RS_RING_STANDALONE = 5,
     ORC_ALG_ALLREDUCE_MESH_ASCENDING = 6,
-    ORC_ALG_ALLREDUCE_LOCAL_REDUCE = 7
+    ORC_ALG_ALLREDUCE_LOCAL_REDUCE = 7,
+    ORC_ALG_ALLREDUCE_CHUNK_MESH = 8
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -666,6 +699,7 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, stride, unit); break;
             case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
+            case ORC_ALG_ALLREDUCE_CHUNK_MESH: prog_allreduce_chunk_mesh(t, r, n, count, unit); break;
             case ORC_ALG_ALLREDUCE_LOCAL_REDUCE:
                 if (prog_allreduce_local_reduce(t, r, n, count, unit) != 0) {
                     free(t->ops);

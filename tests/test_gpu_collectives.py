@@ -20,6 +20,7 @@ ALGS = {
     "ring_rs": (h.Alg.REDUCE_SCATTER_RING_STANDALONE, oracle.ALG_RS_RING_STANDALONE),
     "mesh_ascending": (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, oracle.ALG_ALLREDUCE_MESH_ASCENDING),
     "local_reduce": (h.Alg.ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_LOCAL_REDUCE),
+    "chunk_mesh": (h.Alg.ALLREDUCE_CHUNK_MESH, oracle.ALG_ALLREDUCE_CHUNK_MESH),
 }
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
 
@@ -122,6 +123,13 @@ CASES = [
     ("local_reduce", 8, 1001, "int16", "sum"),     # slots fall back to 512-byte / element alignment
     ("local_reduce", 8, 7, "fp32", "sum"),
     ("local_reduce", 1, 100, "fp32", "sum"),
+    ("chunk_mesh", 8, 1 << 20, "bf16", "sum"),
+    ("chunk_mesh", 7, 100003, "fp32", "sum"),
+    ("chunk_mesh", 3, 4099, "fp16", "max"),
+    ("chunk_mesh", 2, 70001, "int8", "sum"),
+    ("chunk_mesh", 16, 300007, "int32", "min"),
+    ("chunk_mesh", 5, 9, "int16", "sum"),
+    ("chunk_mesh", 1, 100, "fp32", "sum"),
 ]
 
 

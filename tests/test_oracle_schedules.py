@@ -15,7 +15,7 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
-        oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE]
+        oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH]
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE)
 
 
@@ -249,6 +249,36 @@ def test_local_reduce_trees_hand_derived(op):
                 assert np.array_equal(outs[r][lo:hi].view(np.uint32), want.view(np.uint32)), (n, d_s, r)
     with pytest.raises(ValueError):        # the slot arithmetic only closes for a power-of-two rank count
         oracle.trace(oracle.ALG_ALLREDUCE_LOCAL_REDUCE, 6, 1000, oracle.F32)
+
+
+def test_chunk_mesh_fold_order_hand_derived():
+    """Two-shot chunk mesh: sub-chunk q of rank r's slice folds the ranks in a rotation that starts at r+q+1."""
+    for n_s, table in GOLD["chunk_mesh_fold_order"].items():
+        n = int(n_s)
+        count = n * max(n - 1, 1) * 32 * 3 + 45
+        ins = order_sensitive_inputs(n, count, oracle.SUM, seed=50 + n)
+        outs = [np.zeros(count, np.float32) for _ in range(n)]
+        scr = [np.zeros(count * 4, np.uint8) for _ in range(n)]
+        oracle.run(oracle.ALG_ALLREDUCE_CHUNK_MESH, [x.copy() for x in ins], outs, count, oracle.F32, oracle.SUM, scratch=scr)
+        sl = oracle.slices_ring(count, 4, n)
+        for r_s, orders in table.items():
+            r = int(r_s)
+            sub = oracle.slices_ring(sl[r][1] // 4, 4, n - 1)
+            for q, order in enumerate(orders):
+                tree = order[0]
+                for x in order[1:]:
+                    tree = [tree, x]
+                lo = (sl[r][0] + sub[q][0]) // 4
+                hi = lo + sub[q][1] // 4
+                want = eval_tree(tree, [x[lo:hi] for x in ins], oracle.SUM)
+                for k in range(n):
+                    assert np.array_equal(outs[k][lo:hi].view(np.uint32), want.view(np.uint32)), (n, r, q, k)
+            # the rest of the communication buffer is the plain copy of the input
+            got = scr[r].view(np.float32)
+            for k in range(n):
+                if k != r:
+                    lo, hi = sl[k][0] // 4, (sl[k][0] + sl[k][1]) // 4
+                    assert np.array_equal(got[lo:hi], ins[r][lo:hi])
 
 
 def test_strided_scatter_input_layout():

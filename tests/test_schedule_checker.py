@@ -11,7 +11,7 @@ ALL = [(h.Alg.ALLREDUCE_RING, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_RING, Exp
        (h.Alg.REDUCE_SCATTER_MESH, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.REDUCE_SCATTER_RING_STANDALONE, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, Expect.ALLREDUCE),
-       (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE)]
+       (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE), (h.Alg.ALLREDUCE_CHUNK_MESH, Expect.ALLREDUCE)]
 
 
 @pytest.mark.parametrize("alg,expect", ALL)
