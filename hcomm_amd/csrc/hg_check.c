@@ -221,7 +221,8 @@ int32_t HcommGfxScheduleCheck(
     if (rc != HCCL_SUCCESS) return rc;
     HcommGfxExpectation e = HCOMM_GFX_EXPECT_ALLREDUCE;
     if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE;
-    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_MESH || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE)
+    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_MESH || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE ||
+        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
         e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT;
     rc = HcommGfxOpListCheck(l.ops, l.n, nRanks, e, count, strideCount, HcommGfxDataTypeSize(dataType), rep);
     hg_oplist_free(&l);

@@ -368,13 +368,221 @@ static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count,
     return HCCL_SUCCESS;
 }
 
+/* ---- NHR (nonuniform hierarchical ring) and NB (nonuniform Bruck): ceil(log2 N) steps for any N ------------- */
+
+static uint32_t ceil_log2(uint32_t n) /* nonuniform_hierarchical_ring_base.cc:139-147, nonuniform_bruck_base.cc:19-25 */
+{
+    uint32_t s = 0;
+    while ((1u << s) < n) ++s;
+    return s;
+}
+
+/* Slice order of the NHR tree (nonuniform_hierarchical_ring_base.cc:20-91, temp_reduce_scatter/
+ * reduce_scatter_nhr.cc:97-162), stated recursively: a block of logical slices is split into its even and odd
+ * positions, evens first; both halves are split again one level down while a rank still exchanges more than
+ * one slice at that level and the block length was even.  dst receives the block in tree order. */
+static void nhr_tree_order(uint32_t* dst, const uint32_t* src, uint32_t m, uint32_t n, uint32_t level)
+{
+    if (((n - 1 + (1u << level)) >> (level + 1)) <= 1) {
+        memcpy(dst, src, m * sizeof(uint32_t));
+        return;
+    }
+    uint32_t ev[HCOMM_GFX_MAX_RANKS], od[HCOMM_GFX_MAX_RANKS];
+    const uint32_t ne = (m + 1) / 2, no = m / 2;
+    for (uint32_t i = 0; i < m; ++i) {
+        if (i & 1) od[i / 2] = src[i]; else ev[i / 2] = src[i];
+    }
+    if (m & 1) {
+        memcpy(dst, ev, ne * sizeof(uint32_t));
+        memcpy(dst + ne, od, no * sizeof(uint32_t));
+        return;
+    }
+    nhr_tree_order(dst, ev, ne, n, level + 1);
+    nhr_tree_order(dst + ne, od, no, n, level + 1);
+}
+
+/* map[logical slice] = position in the buffer; the identity when the order must be kept (stand-alone
+ * reduce-scatter: reduce_scatter_nhr.cc:86-88) */
+static void nhr_slice_map(uint32_t n, int keep_order, uint32_t* map)
+{
+    uint32_t ident[HCOMM_GFX_MAX_RANKS], tree[HCOMM_GFX_MAX_RANKS];
+    for (uint32_t i = 0; i < n; ++i) ident[i] = i;
+    if (keep_order) {
+        memcpy(map, ident, n * sizeof(uint32_t));
+        return;
+    }
+    nhr_tree_order(tree, ident, n, n, 0);
+    for (uint32_t i = 0; i < n; ++i) map[tree[i]] = i;
+}
+
+/* Ascending by offset, neighbours that touch become one slice (NHRBase::MergeSlices,
+ * nonuniform_hierarchical_ring_base.cc:94-136).  Returns the new number of slices. */
+static uint32_t merge_touching(HcommGfxSlice* v, uint32_t m)
+{
+    if (m <= 1) return m;
+    for (uint32_t i = 1; i < m; ++i) { /* insertion sort by (offset, size) */
+        HcommGfxSlice x = v[i];
+        uint32_t j = i;
+        while (j > 0 && (v[j - 1].offset > x.offset || (v[j - 1].offset == x.offset && v[j - 1].size > x.size))) {
+            v[j] = v[j - 1];
+            --j;
+        }
+        v[j] = x;
+    }
+    uint32_t w = 0;
+    for (uint32_t i = 1; i < m; ++i) {
+        if (v[w].offset + v[w].size == v[i].offset) v[w].size += v[i].size;
+        else v[++w] = v[i];
+    }
+    return w + 1;
+}
+
+/* NHR reduce-scatter over `sl` in the input buffers (reduce_scatter_nhr.cc:408-488 with the step table of
+ * :552-593 and the inline-reduce receive of :197-259): step s, rank r reads rank r + 2^s and folds the logical
+ * slices r, r - 2^(s+1), r - 2*2^(s+1), ... ((N-1+2^s) >> (s+1) of them) into its own copies. */
+static int nhr_rs(HgOpList* l, uint32_t n, const HcommGfxSlice* sl, const uint32_t* map, int merge)
+{
+    const uint32_t steps = ceil_log2(n);
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t cnt = (n - 1 + (1u << s)) >> (s + 1);
+        for (uint32_t r = 0; r < n; ++r) {
+            HcommGfxSlice v[HCOMM_GFX_MAX_RANKS];
+            for (uint32_t i = 0; i < cnt; ++i) v[i] = sl[map[modn((int64_t)r - ((int64_t)i << (s + 1)), n)]];
+            /* the last step handles its single slice unmerged (:239-259) */
+            const uint32_t m = (merge && s + 1 < steps) ? merge_touching(v, cnt) : cnt;
+            for (uint32_t i = 0; i < m; ++i)
+                CHK(push(l, s, REDUCE, r, IN, v[i].offset, (r + (1u << s)) % n, IN, v[i].offset, v[i].size));
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+/* AllReduceNHR (temp_all_reduce/all_reduce_nhr.cc:25-77,133-173): tree-ordered NHR reduce-scatter in place on
+ * the inputs, own slice input -> output, NHR all-gather on the outputs (temp_all_gather/all_gather_nhr.cc:
+ * 75-81,141-195, step table :228-268): step s (delta = 2^(S-1-s)), rank r reads rank r - delta and fetches the
+ * logical slices r - delta, r - delta - 2 delta, ... */
+static int sched_allreduce_nhr(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* all_reduce_nhr.cc:35-44 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    uint32_t map[HCOMM_GFX_MAX_RANKS];
+    CHK(HcommGfxCalcSlices(count, unit, n, sl)); /* all_reduce_nhr.cc:104-121: the ring's slice table */
+    nhr_slice_map(n, 0, map);
+    CHK(nhr_rs(l, n, sl, map, 1));
+    const uint32_t steps = ceil_log2(n);
+    for (uint32_t r = 0; r < n; ++r)
+        CHK(push(l, steps, COPY, r, OUT, sl[map[r]].offset, r, IN, sl[map[r]].offset, sl[map[r]].size));
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t delta = 1u << (steps - 1 - s);
+        const uint32_t cnt = (n - 1 + delta) / (2 * delta);
+        for (uint32_t r = 0; r < n; ++r) {
+            HcommGfxSlice v[HCOMM_GFX_MAX_RANKS];
+            for (uint32_t i = 0; i < cnt; ++i)
+                v[i] = sl[map[modn((int64_t)r - delta - (int64_t)i * 2 * delta, n)]];
+            const uint32_t m = merge_touching(v, cnt);
+            for (uint32_t i = 0; i < m; ++i)
+                CHK(push(l, steps + 1 + s, COPY, r, OUT, v[i].offset, modn((int64_t)r - delta, n), OUT, v[i].offset, v[i].size));
+        }
+    }
+    return HCCL_SUCCESS;
+}
+
+/* Stand-alone ReduceScatterNHR (reduce_scatter_nhr.cc:27-95): slice i of the input at i * stride elements, slice
+ * order kept, nothing merged; the last step reduces into the input slice and copies it to the output, which
+ * holds one slice (:57-75, :239-259, :208-217). */
+static int sched_rs_nhr(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz); /* :41-46 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    uint32_t map[HCOMM_GFX_MAX_RANKS];
+    memset(sl, 0, sizeof(sl));
+    for (uint32_t i = 0; i < n; ++i) {
+        sl[i].offset = (uint64_t)i * stride * unit;
+        sl[i].size = sz;
+    }
+    nhr_slice_map(n, 1, map);
+    CHK(nhr_rs(l, n, sl, map, 0));
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, ceil_log2(n), COPY, r, OUT, 0, r, IN, sl[r].offset, sz));
+    return HCCL_SUCCESS;
+}
+
+/* NB reduce-scatter over `sl` in the input buffers (temp_reduce_scatter/reduce_scatter_nb.cc:119-230,260-311):
+ * step s, rank r reads rank r - 2^s and folds slices r, r + 2^(s+1), r + 2*2^(s+1), ... into its own copies. */
+static int nb_rs(HgOpList* l, uint32_t n, const HcommGfxSlice* sl)
+{
+    const uint32_t steps = ceil_log2(n);
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t cnt = (n - 1 + (1u << s)) >> (s + 1);
+        for (uint32_t r = 0; r < n; ++r)
+            for (uint32_t i = 0; i < cnt; ++i) {
+                const uint32_t c = (uint32_t)((r + ((uint64_t)i << (s + 1))) % n);
+                CHK(push(l, s, REDUCE, r, IN, sl[c].offset, modn((int64_t)r - (1 << s), n), IN, sl[c].offset, sl[c].size));
+            }
+    }
+    return HCCL_SUCCESS;
+}
+
+/* AllReduceNB (temp_all_reduce/all_reduce_nb.cc:26-61,139-150,162-201): slices of ceil(total/N) rounded up to
+ * 128 bytes when larger than 128 KiB, else rounded up to 128 KiB (:203-219: small messages are not cut); NB
+ * reduce-scatter in place; own slice input -> output; NB all-gather on the outputs (temp_all_gather/
+ * all_gather_nb.cc:88-92,101-188): step s, rank r reads rank r - 2^s and fetches slices r - 2^s - i,
+ * i < 2^s (the last step only the N - 2^s that are still missing). */
+static int sched_allreduce_nb(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* all_reduce_nb.cc:130-137 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    const uint64_t small = 128u * 1024u; /* NB_ALLREDUCE_SMALL_SIZE, nonuniform_bruck_base_pub.h:19 */
+    const uint64_t raw = (total + n - 1) / n;
+    const uint64_t gran = raw > small ? HG_SLICE_ALIGN : small;
+    const uint64_t per = raw == 0 ? gran : (raw + gran - 1) / gran * gran;
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < n; ++i) {
+        sl[i].size = residue > per ? per : residue;
+        sl[i].offset = total - residue;
+        residue -= sl[i].size;
+    }
+    CHK(nb_rs(l, n, sl));
+    const uint32_t steps = ceil_log2(n);
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, steps, COPY, r, OUT, sl[r].offset, r, IN, sl[r].offset, sl[r].size));
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t cnt = (s + 1 == steps && n != (1u << steps)) ? n - (1u << s) : (1u << s);
+        for (uint32_t r = 0; r < n; ++r)
+            for (uint32_t i = 0; i < cnt; ++i) {
+                const uint32_t c = modn((int64_t)r - (1 << s) - i, n);
+                CHK(push(l, steps + 1 + s, COPY, r, OUT, sl[c].offset, modn((int64_t)r - (1 << s), n), OUT, sl[c].offset, sl[c].size));
+            }
+    }
+    return HCCL_SUCCESS;
+}
+
+/* Stand-alone ReduceScatterNB (reduce_scatter_nb.cc:27-86): as the stand-alone NHR variant, other direction. */
+static int sched_rs_nb(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, sz); /* :35-40 */
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    memset(sl, 0, sizeof(sl));
+    for (uint32_t i = 0; i < n; ++i) {
+        sl[i].offset = (uint64_t)i * stride * unit;
+        sl[i].size = sz;
+    }
+    CHK(nb_rs(l, n, sl));
+    /* last step: reduce into the input slice, then input slice -> output (:267-289, component/reducer.cc:209-218) */
+    for (uint32_t r = 0; r < n; ++r) CHK(push(l, ceil_log2(n), COPY, r, OUT, 0, r, IN, sl[r].offset, sz));
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
     if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (stride == 0) stride = count;
     if (stride < count) return HCCL_E_PARA;
-    if (stride != count && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_MESH && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE)
+    if (stride != count && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_MESH && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE &&
+        alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
         return HCCL_E_PARA;
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
     if (unit == 0) return HCCL_E_PARA;
@@ -389,6 +597,10 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE: rc = sched_rs_ring_standalone(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE: rc = sched_allreduce_local_reduce(l, n, count, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH: rc = sched_allreduce_chunk_mesh(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_NHR: rc = sched_allreduce_nhr(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_NHR: rc = sched_rs_nhr(l, n, count, stride, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_NB: rc = sched_allreduce_nb(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_NB: rc = sched_rs_nb(l, n, count, stride, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

@@ -333,7 +333,23 @@ typedef enum {
        communication buffer, reduces its own slice there in N-1 rounds - sub-chunk p-1 of the slice takes peer
        r+p, r+p+1, ..., r+N-1, r+1, ..., r+p-1 in that order (a Latin square over links and rounds) - and the
        ranks gather the slices.  Needs the third buffer (count * unit bytes).  Step-wise lowering only. */
-    HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH = 8
+    HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH = 8,
+    /* AllReduceNHR (nonuniform hierarchical ring, ceil(log2 N) steps for any N): temp_all_reduce/
+       all_reduce_nhr.cc:25-77 = ReduceScatterNHR in place on the inputs (temp_reduce_scatter/
+       reduce_scatter_nhr.cc:408-488, step table :552-593: step s, rank r folds from rank r + 2^s) over the
+       tree-ordered slice map (nonuniform_hierarchical_ring_base.cc:20-75) with touching slices merged (:94-136),
+       own slice input -> output, AllGatherNHR on the outputs (temp_all_gather/all_gather_nhr.cc:141-195,228-268) */
+    HCOMM_GFX_ALG_ALLREDUCE_NHR = 9,
+    /* stand-alone ReduceScatterNHR (reduce_scatter_nhr.cc:27-95): input holds N slices of count elements (slice i
+       at i * strideCount), slice order kept, result in out[r][0..count) */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_NHR = 10,
+    /* AllReduceNB (nonuniform Bruck): temp_all_reduce/all_reduce_nb.cc:26-61 = ReduceScatterNB in place
+       (temp_reduce_scatter/reduce_scatter_nb.cc:119-230: step s, rank r folds from rank r - 2^s), own slice
+       input -> output, AllGatherNB (temp_all_gather/all_gather_nb.cc:101-188).  Slices are not cut below
+       128 KiB (all_reduce_nb.cc:203-219) */
+    HCOMM_GFX_ALG_ALLREDUCE_NB = 11,
+    /* stand-alone ReduceScatterNB (reduce_scatter_nb.cc:27-86), layout as HCOMM_GFX_ALG_REDUCE_SCATTER_NHR */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_NB = 12
 } HcommGfxAlgorithm;
 
 typedef enum {

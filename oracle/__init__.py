@@ -16,7 +16,8 @@ REF_PATH = os.path.join(HERE, "_ref", "libhcomm_ref.so")
 SUM, PROD, MAX, MIN = 0, 1, 2, 3
 I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
 ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
-    ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING, ALG_ALLREDUCE_LOCAL_REDUCE, ALG_ALLREDUCE_CHUNK_MESH = range(9)
+    ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING, ALG_ALLREDUCE_LOCAL_REDUCE, ALG_ALLREDUCE_CHUNK_MESH, \
+    ALG_ALLREDUCE_NHR, ALG_RS_NHR, ALG_ALLREDUCE_NB, ALG_RS_NB = range(13)
 
 # storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
 NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
@@ -77,6 +78,10 @@ def lib():
         L.orc_slices_ring.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.POINTER(OrcSlice)]
         L.orc_slices_rhd.restype = None
         L.orc_slices_rhd.argtypes = [C.c_uint64, C.c_uint32, C.POINTER(OrcSlice)]
+        L.orc_slices_nb.restype = None
+        L.orc_slices_nb.argtypes = [C.c_uint64, C.c_uint32, C.POINTER(OrcSlice)]
+        L.orc_nhr_slice_map.restype = None
+        L.orc_nhr_slice_map.argtypes = [C.c_uint32, C.POINTER(C.c_uint32)]
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run.restype = C.c_int
@@ -158,6 +163,18 @@ def slices_rhd(data_bytes, block):
     sl = (OrcSlice * block)()
     lib().orc_slices_rhd(data_bytes, block, sl)
     return [(s.offset, s.size) for s in sl]
+
+
+def slices_nb(total_bytes, n):
+    sl = (OrcSlice * n)()
+    lib().orc_slices_nb(total_bytes, n, sl)
+    return [(s.offset, s.size) for s in sl]
+
+
+def nhr_slice_map(n):
+    m = (C.c_uint32 * n)()
+    lib().orc_nhr_slice_map(n, m)
+    return list(m)
 
 
 def trace(alg, n, count, dtype, stride=0):

@@ -657,6 +657,280 @@ static void prog_allreduce_chunk_mesh(OrcTrace* t, uint32_t rank, uint32_t n, ui
     }
 }
 
+/* ---- NHR and NB: per-rank programs --------------------------------------------------------------------- */
+
+/* NHRBase::GetStepNumInterServer, tpl/nonuniform_hierarchical_ring_base.cc:139-147 = NBBase::CalcCeilLog2,
+ * tpl/nonuniform_bruck_base.cc:19-25 */
+static uint32_t nhr_steps(uint32_t n)
+{
+    uint32_t s = 0;
+    for (uint32_t tmp = n - 1; tmp != 0; tmp >>= 1) s++;
+    return s;
+}
+
+/* NHRBase::GetRankMapping + ReorderSequence, tpl/nonuniform_hierarchical_ring_base.cc:20-91 (the same loop is
+ * ReduceScatterNHR::GetSliceMap + Reorder, tpl/temp_reduce_scatter/reduce_scatter_nhr.cc:97-162), with the
+ * reference's tree / tmp arrays and its part loop. */
+static void nhr_rank_mapping(uint32_t n, int keep_order, uint32_t* slice_map)
+{
+    uint32_t tree[ORC_MAX_RANKS], tmp[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) tree[i] = i;
+    if (keep_order) { /* :27-31 */
+        for (uint32_t i = 0; i < n; i++) slice_map[i] = tree[i];
+        return;
+    }
+    const uint32_t n_steps = nhr_steps(n);
+    uint32_t len = n;
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t n_slices = (n - 1 + (1u << step)) / (1u << (step + 1)); /* :40 */
+        if (n_slices <= 1) break;
+        int end_flag = 0;
+        for (uint32_t part = 0; part * len < n; part++) {
+            const uint32_t start = part * len;
+            const uint32_t end = (start + len < n) ? start + len : n;
+            for (uint32_t i = start; i < end; i++) { /* ReorderSequence, :79-91 */
+                const uint32_t offset = i - start;
+                if ((offset & 1) == 0) tmp[start + offset / 2] = tree[i];
+                else tmp[start + (offset + len) / 2] = tree[i];
+            }
+            if (((end - start) & 1) == 1) end_flag = 1;
+        }
+        for (uint32_t i = 0; i < n; i++) tree[i] = tmp[i];
+        if (end_flag) break;
+        len >>= 1;
+    }
+    for (uint32_t i = 0; i < n; i++) slice_map[tree[i]] = i; /* :69-72 */
+}
+
+static int cmp_slices(const void* a, const void* b)
+{
+    const OrcSlice* x = (const OrcSlice*)a;
+    const OrcSlice* y = (const OrcSlice*)b;
+    if (x->offset != y->offset) return x->offset < y->offset ? -1 : 1;
+    if (x->size != y->size) return x->size < y->size ? -1 : 1;
+    return 0;
+}
+
+/* NHRBase::MergeSlices, tpl/nonuniform_hierarchical_ring_base.cc:94-136 */
+static uint32_t nhr_merge_slices(OrcSlice* v, uint32_t m, int need_merge)
+{
+    if (!need_merge || m <= 1) return m;
+    qsort(v, m, sizeof(OrcSlice), cmp_slices);
+    uint32_t merged = 0;
+    uint64_t off = v[0].offset, size = v[0].size;
+    for (uint32_t i = 1; i < m; i++) {
+        if (off + size == v[i].offset) {
+            size += v[i].size;
+        } else {
+            v[merged].size = size;
+            v[merged].offset = off;
+            merged++;
+            size = v[i].size;
+            off = v[i].offset;
+        }
+    }
+    v[merged].size = size;
+    v[merged].offset = off;
+    return merged + 1;
+}
+
+/* ReduceScatterNHR::RunReduceScatterNHR for one rank on the SDMA / inline-reduce path,
+ * tpl/temp_reduce_scatter/reduce_scatter_nhr.cc:408-488 -> SdmaReducer :383-406 -> InlineReduceRx :222-237 /
+ * InlineReduceRxLastStep :239-259 -> InlineReducer :197-220; step table GetStepInfo :552-593.
+ * out_sl NULL: called from the allreduce, output memory == input memory, so the last step copies nothing. */
+static void prog_nhr_rs(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, const OrcSlice* out_sl,
+                        const uint32_t* slice_map, int need_merge)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << step;                       /* :562 */
+        const uint32_t recv_from = (rank + delta_rank) % n;           /* :564 */
+        const uint32_t n_slices = (n - 1 + (1u << step)) / (1u << (step + 1)); /* :567 */
+        const uint32_t delta_slice = 1u << (step + 1);
+        uint32_t rx_idx = rank;                                       /* :570 */
+        uint32_t rx_idxs[ORC_MAX_RANKS];
+        for (uint32_t i = 0; i < n_slices; i++) {
+            rx_idxs[i] = slice_map[rx_idx];                           /* :577-578 */
+            rx_idx = (rx_idx + n - delta_slice) % n;                  /* :586, u32 arithmetic as in the original */
+        }
+        if (step == n_steps - 1) { /* InlineReduceRxLastStep: per slice, unmerged */
+            for (uint32_t i = 0; i < n_slices; i++) {
+                const OrcSlice s = sl[rx_idxs[i]];
+                emit(t, step, K_REDUCE, rank, B_IN, s.offset, recv_from, B_IN, s.offset, s.size); /* :203-207 */
+                if (out_sl) /* localsrc != localdst, :208-217 */
+                    emit(t, step + 1, K_COPY, rank, B_OUT, out_sl[rx_idxs[i]].offset, rank, B_IN, s.offset, s.size);
+            }
+        } else { /* GetRxSlices :357-381 + InlineReduceRx */
+            OrcSlice rx[ORC_MAX_RANKS];
+            for (uint32_t i = 0; i < n_slices; i++) rx[i] = sl[rx_idxs[i]];
+            const uint32_t m = nhr_merge_slices(rx, n_slices, need_merge);
+            for (uint32_t i = 0; i < m; i++)
+                emit(t, step, K_REDUCE, rank, B_IN, rx[i].offset, recv_from, B_IN, rx[i].offset, rx[i].size);
+        }
+    }
+}
+
+/* AllGatherNHR::RunAllGather for one rank on the SDMA path, tpl/temp_all_gather/all_gather_nhr.cc:141-195 ->
+ * SdmaRx :90-108; step table GetStepInfo :228-268 */
+static void prog_nhr_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, const uint32_t* slice_map,
+                        int need_merge, uint32_t step0)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << (n_steps - 1 - step);                         /* :237 */
+        const uint32_t recv_from = (rank + n - delta_rank) % n;                         /* :238 */
+        const uint32_t n_slices = (n - 1 + (1u << (n_steps - 1 - step))) / (1u << (n_steps - step)); /* :242 */
+        const uint32_t delta_slice = 1u << (n_steps - step);
+        uint32_t rx_idx = (rank - (1u << (n_steps - 1 - step)) + n) % n;                /* :245 */
+        OrcSlice rx[ORC_MAX_RANKS];
+        for (uint32_t i = 0; i < n_slices; i++) {
+            rx[i] = sl[slice_map[rx_idx]];
+            rx_idx = (rx_idx + n - delta_slice) % n;                                    /* :265, u32 arithmetic */
+        }
+        const uint32_t m = nhr_merge_slices(rx, n_slices, need_merge);                  /* :184 */
+        for (uint32_t i = 0; i < m; i++)
+            emit(t, step0 + step, K_COPY, rank, B_OUT, rx[i].offset, recv_from, B_OUT, rx[i].offset, rx[i].size);
+    }
+}
+
+/* AllReduceNHR::RunAsync for one rank, tpl/temp_all_reduce/all_reduce_nhr.cc:25-77: slices :104-121 (the ring's
+ * table), RunReduceScatter :133-154 (input, input, output-as-scratch; needMerge = true), RunAllGather :156-173
+ * (input, output, output; needMerge = true), whose RunAsync first copies the own slice (all_gather_nhr.cc:75-81). */
+static void prog_allreduce_nhr(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    if (n == 1) { /* :35-44 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, count * unit);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS];
+    uint32_t slice_map[ORC_MAX_RANKS];
+    orc_slices_ring(count, unit, n, sl);
+    nhr_rank_mapping(n, 0, slice_map);
+    prog_nhr_rs(t, rank, n, sl, NULL, slice_map, 1);
+    const uint32_t n_steps = nhr_steps(n);
+    const uint32_t target = slice_map[rank];
+    emit(t, n_steps, K_COPY, rank, B_OUT, sl[target].offset, rank, B_IN, sl[target].offset, sl[target].size);
+    prog_nhr_ag(t, rank, n, sl, slice_map, 1, n_steps + 1);
+}
+
+/* Stand-alone ReduceScatterNHR::RunAsync, tpl/temp_reduce_scatter/reduce_scatter_nhr.cc:27-95: slices :57-75
+ * (input larger than output -> output offset 0; input slice i at i * stride elements as in the strided scatter
+ * layout), order kept (:86-88), no merging (isNeedMerge defaults to false,
+ * tpl/nonuniform_hierarchical_ring_base_pub.h:54). */
+static void prog_rs_nhr(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) { /* :41-46 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, sz);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS], osl[ORC_MAX_RANKS];
+    uint32_t slice_map[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) {
+        sl[i].size = sz;
+        sl[i].offset = (uint64_t)i * stride * unit;
+        osl[i].size = sz;
+        osl[i].offset = 0;
+    }
+    nhr_rank_mapping(n, 1, slice_map);
+    prog_nhr_rs(t, rank, n, sl, osl, slice_map, 0);
+}
+
+/* ReduceScatterNB::RunReduceScatterNB for one rank, tpl/temp_reduce_scatter/reduce_scatter_nb.cc:119-230 ->
+ * RunDestReducerNB :260-311 -> Reducer::run inline branch (tpl/component/reducer.cc:199-222). */
+static void prog_nb_rs(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, const OrcSlice* out_sl)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << step;                                /* :149 */
+        const uint32_t recv_from = (n + rank - delta_rank) % n;                /* :150 */
+        const uint32_t n_slices = (n - 1 + (1u << step)) / (1u << (step + 1)); /* :154 */
+        const uint32_t delta_slice = 1u << (step + 1);
+        uint32_t rx_idx = rank;                                                /* :157 */
+        for (uint32_t i = 0; i < n_slices; i++) {
+            if (sl[rx_idx].size > 0) {
+                emit(t, step, K_REDUCE, rank, B_IN, sl[rx_idx].offset, recv_from, B_IN, sl[rx_idx].offset, sl[rx_idx].size);
+                if (step == n_steps - 1 && out_sl) /* :267-289: dst is the output, src the input slice */
+                    emit(t, step + 1, K_COPY, rank, B_OUT, out_sl[rx_idx].offset, rank, B_IN, sl[rx_idx].offset, sl[rx_idx].size);
+            }
+            rx_idx = (rx_idx + delta_slice) % n;
+        }
+    }
+}
+
+/* AllGatherNB::RunAllGather for one rank, tpl/temp_all_gather/all_gather_nb.cc:101-188 */
+static void prog_nb_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t step0)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << step;
+        const uint32_t recv_from = (n + rank - delta_rank) % n; /* :119 */
+        uint32_t n_slices = 1u << step;                          /* :124-127 */
+        if (step == n_steps - 1 && n != (1u << n_steps)) n_slices = n - (1u << step);
+        for (uint32_t i = 0; i < n_slices; i++) {
+            const uint32_t rx = (rank - (1u << step) + n - i) % n; /* :138 */
+            if (sl[rx].size > 0)
+                emit(t, step0 + step, K_COPY, rank, B_OUT, sl[rx].offset, recv_from, B_OUT, sl[rx].offset, sl[rx].size);
+        }
+    }
+}
+
+/* GetSliceSizeOfNB, tpl/temp_all_reduce/all_reduce_nb.cc:203-219 + the slice loop of :139-150 */
+void orc_slices_nb(uint64_t total, uint32_t n, OrcSlice* sl)
+{
+    const uint64_t small = 128u * 1024u; /* NB_ALLREDUCE_SMALL_SIZE, tpl/nonuniform_bruck_base_pub.h:19 */
+    const uint64_t calc = (total + (n - 1)) / n;
+    const uint64_t div = (calc > small) ? 128u : small;
+    const uint64_t aligned = (calc == 0) ? div : ((calc + div - 1) / div) * div; /* RoundUpWithDivisor */
+    uint64_t residue = total;
+    for (uint32_t i = 0; i < n; i++) {
+        sl[i].size = (residue > aligned) ? aligned : residue;
+        sl[i].offset = total - residue;
+        residue -= sl[i].size;
+    }
+}
+
+/* AllReduceNB::RunAsync for one rank, tpl/temp_all_reduce/all_reduce_nb.cc:26-61 (RunReduceScatter :162-180,
+ * RunAllGather :182-201; the own-slice copy is AllGatherNB::RunAsync, tpl/temp_all_gather/all_gather_nb.cc:88-92) */
+static void prog_allreduce_nb(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    if (n == 1) { /* PrepareRunAsync :130-137 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, count * unit);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS];
+    orc_slices_nb(count * unit, n, sl);
+    prog_nb_rs(t, rank, n, sl, NULL);
+    const uint32_t n_steps = nhr_steps(n);
+    emit(t, n_steps, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size);
+    prog_nb_ag(t, rank, n, sl, n_steps + 1);
+}
+
+/* Stand-alone ReduceScatterNB::RunAsync, tpl/temp_reduce_scatter/reduce_scatter_nb.cc:27-86 (slices :50-70) */
+static void prog_rs_nb(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    if (n == 1) { /* :35-40 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, sz);
+        return;
+    }
+    OrcSlice sl[ORC_MAX_RANKS], osl[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) {
+        sl[i].size = sz;
+        sl[i].offset = (uint64_t)i * stride * unit;
+        osl[i].size = sz;
+        osl[i].offset = 0;
+    }
+    prog_nb_rs(t, rank, n, sl, osl);
+}
+
+/* The NHR slice map, exported for the hand-derived fixtures. */
+void orc_nhr_slice_map(uint32_t n, uint32_t* slice_map)
+{
+    if (n == 0 || n > ORC_MAX_RANKS) return;
+    nhr_rank_mapping(n, 0, slice_map);
+}
+
 enum {
     ORC_ALG_ALLREDUCE_RING = 0,
     ORC_ALG_RS_RING_STAGE = 1,
@@ -666,7 +940,11 @@ enum {
     ORC_ALG_RS_RING_STANDALONE = 5,
     ORC_ALG_ALLREDUCE_MESH_ASCENDING = 6,
     ORC_ALG_ALLREDUCE_LOCAL_REDUCE = 7,
-    ORC_ALG_ALLREDUCE_CHUNK_MESH = 8
+    ORC_ALG_ALLREDUCE_CHUNK_MESH = 8,
+    ORC_ALG_ALLREDUCE_NHR = 9,
+    ORC_ALG_RS_NHR = 10,
+    ORC_ALG_ALLREDUCE_NB = 11,
+    ORC_ALG_RS_NB = 12
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -700,6 +978,10 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
             case ORC_ALG_ALLREDUCE_CHUNK_MESH: prog_allreduce_chunk_mesh(t, r, n, count, unit); break;
+            case ORC_ALG_ALLREDUCE_NHR: prog_allreduce_nhr(t, r, n, count, unit); break;
+            case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, stride, unit); break;
+            case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
+            case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_LOCAL_REDUCE:
                 if (prog_allreduce_local_reduce(t, r, n, count, unit) != 0) {
                     free(t->ops);

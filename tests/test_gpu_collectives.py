@@ -21,7 +21,12 @@ ALGS = {
     "mesh_ascending": (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, oracle.ALG_ALLREDUCE_MESH_ASCENDING),
     "local_reduce": (h.Alg.ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_LOCAL_REDUCE),
     "chunk_mesh": (h.Alg.ALLREDUCE_CHUNK_MESH, oracle.ALG_ALLREDUCE_CHUNK_MESH),
+    "nhr_ar": (h.Alg.ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NHR),
+    "nhr_rs": (h.Alg.REDUCE_SCATTER_NHR, oracle.ALG_RS_NHR),
+    "nb_ar": (h.Alg.ALLREDUCE_NB, oracle.ALG_ALLREDUCE_NB),
+    "nb_rs": (h.Alg.REDUCE_SCATTER_NB, oracle.ALG_RS_NB),
 }
+SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
 
 
@@ -32,7 +37,7 @@ def say(*a):
 
 def buffer_counts(alg, n, count, stride=0):
     """(elements in each input buffer, elements in each output buffer)."""
-    if alg in ("mesh_rs", "ring_rs"):
+    if alg in SCATTER:
         return ((n - 1) * stride + count if stride else n * count), count
     return count, count
 
@@ -130,6 +135,28 @@ CASES = [
     ("chunk_mesh", 16, 300007, "int32", "min"),
     ("chunk_mesh", 5, 9, "int16", "sum"),
     ("chunk_mesh", 1, 100, "fp32", "sum"),
+    ("nhr_ar", 8, 1 << 20, "bf16", "sum"),
+    ("nhr_ar", 7, 100003, "fp32", "sum"),
+    ("nhr_ar", 5, 4099, "fp16", "max"),            # step 0 of rank 0 folds two slices that do not touch
+    ("nhr_ar", 3, 70001, "int8", "sum"),
+    ("nhr_ar", 16, 300007, "int32", "min"),
+    ("nhr_ar", 31, 4099, "int16", "max"),
+    ("nhr_ar", 12, 1000, "fp32", "prod"),
+    ("nhr_ar", 2, 9, "bf16", "sum"),
+    ("nhr_ar", 1, 100, "fp32", "sum"),
+    ("nhr_rs", 8, 40001, "fp32", "sum"),
+    ("nhr_rs", 7, 5000, "bf16", "sum"),
+    ("nhr_rs", 5, 64, "int8", "max"),
+    ("nhr_rs", 32, 1001, "int32", "sum"),           # 16 unmerged slices per rank at step 0: several launches
+    ("nb_ar", 8, 1 << 20, "bf16", "sum"),
+    ("nb_ar", 7, 100003, "fp32", "sum"),            # below 128 KiB per rank: cut in 128 KiB granules, not in 7
+    ("nb_ar", 6, 300007, "int32", "min"),
+    ("nb_ar", 16, 1 << 21, "fp16", "max"),
+    ("nb_ar", 3, 70001, "int8", "sum"),
+    ("nb_ar", 1, 100, "fp32", "sum"),
+    ("nb_rs", 8, 40001, "fp32", "sum"),
+    ("nb_rs", 7, 5000, "bf16", "sum"),
+    ("nb_rs", 12, 999, "int32", "sum"),
 ]
 
 
@@ -149,10 +176,12 @@ def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype
     assert moved <= algo
 
 
-@pytest.mark.parametrize("alg", ["mesh_rs", "ring_rs"])
+@pytest.mark.parametrize("alg", SCATTER)
 @pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
 def test_strided_reduce_scatter(gpu_thread, alg, lowering):
     """Input slices spaced strideLen elements apart (aicpu_reduce_scatter.cc:78-80); the gaps keep their bytes."""
+    if lowering == h.Lowering.FUSED and alg not in FUSABLE:
+        pytest.skip("step-wise lowering only")
     for n, count, stride, dtype in ((7, 5000, 5000 + 37, "bf16"), (4, 1 << 16, 3 << 16, "fp32"), (3, 33, 64, "int8")):
         say("strided", alg, lowering, n, count, stride, dtype)
         run_case(gpu_thread, alg, lowering, n, count, dtype, "sum", stride=stride)

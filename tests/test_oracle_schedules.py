@@ -15,8 +15,9 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
-        oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH]
-SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE)
+        oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
+        oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB]
+SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB)
 
 
 def scratch_for(alg, n, count, dt):
@@ -279,6 +280,91 @@ def test_chunk_mesh_fold_order_hand_derived():
                 if k != r:
                     lo, hi = sl[k][0] // 4, (sl[k][0] + sl[k][1]) // 4
                     assert np.array_equal(got[lo:hi], ins[r][lo:hi])
+
+
+# ---- NHR / NB (hand-derived) ------------------------------------------------------------------------------
+
+def test_nhr_slice_map_hand_derived():
+    for n_s, want in GOLD["nhr_slice_map"].items():
+        if not n_s.startswith("_"):
+            assert oracle.nhr_slice_map(int(n_s)) == want, n_s
+    for n in range(1, 33):  # a permutation for every N; a bit reversal for powers of two
+        m = oracle.nhr_slice_map(n)
+        assert sorted(m) == list(range(n))
+        if n & (n - 1) == 0 and n > 1:
+            bits = n.bit_length() - 1
+            assert m == [int(format(i, "0%db" % bits)[::-1], 2) for i in range(n)]
+
+
+def test_nb_slice_tables_hand_computed():
+    for case in GOLD["nb_slice_tables"]["cases"]:
+        assert oracle.slices_nb(case["total"], case["n"]) == [tuple(x) for x in case["slices"]]
+    for total in (0, 1, 131072 * 8, 131072 * 8 + 1, 1 << 30):
+        for n in (2, 7, 8):
+            sl = oracle.slices_nb(total, n)
+            assert sum(s for _, s in sl) == total
+            assert all(o == sum(s for _, s in sl[:i]) for i, (o, _) in enumerate(sl))
+
+
+def test_nhr_merged_rx_runs_hand_derived():
+    for n_s, table in GOLD["nhr_rs_rx_positions"].items():
+        if n_s.startswith("_"):
+            continue
+        n = int(n_s)
+        got = [[[] for _ in table[0]] for _ in range(n)]
+        for (step, k, rank, dbuf, doff, srank, sbuf, soff, nbytes) in oracle.trace(oracle.ALG_ALLREDUCE_NHR, n, 32 * n, oracle.F32):
+            if k == 1:
+                assert srank == (rank + (1 << step)) % n and doff == soff and (dbuf, sbuf) == (0, 0)
+                got[rank][step].append([doff // 128, nbytes // 128])
+        assert got == table
+
+
+def test_nb_ag_rx_slices_hand_derived():
+    for n_s, table in GOLD["nb_ag_rx_slices"].items():
+        if n_s.startswith("_"):
+            continue
+        n = int(n_s)
+        count = n * 40000  # > 128 KiB per slice, so the message is cut into N slices
+        sl = oracle.slices_nb(count * 4, n)
+        index = {off: i for i, (off, _) in enumerate(sl)}
+        steps = len(table[0])
+        got = [[[] for _ in range(steps)] for _ in range(n)]
+        for (step, k, rank, dbuf, doff, srank, sbuf, soff, nbytes) in oracle.trace(oracle.ALG_ALLREDUCE_NB, n, count, oracle.F32):
+            if k == 0 and srank != rank:
+                ag = step - steps - 1
+                assert srank == (rank - (1 << ag)) % n and (dbuf, sbuf) == (1, 1)
+                got[rank][ag].append(index[doff])
+        assert got == table
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_nhr_and_nb_trees_hand_derived(op):
+    for key, alg in (("nhr_allreduce_position_tree", oracle.ALG_ALLREDUCE_NHR), ("nb_allreduce_slice_tree", oracle.ALG_ALLREDUCE_NB)):
+        for n_s, trees in GOLD[key].items():
+            if n_s.startswith("_"):
+                continue
+            n = int(n_s)
+            count = n * 96 - 3 if alg == oracle.ALG_ALLREDUCE_NHR else n * 33000 + 5  # ragged last slice, none empty
+            ins = order_sensitive_inputs(n, count, op, seed=70 + n)
+            outs = [np.zeros(count, np.float32) for _ in range(n)]
+            oracle.run(alg, [x.copy() for x in ins], outs, count, oracle.F32, op)
+            sl = oracle.slices_ring(count, 4, n) if alg == oracle.ALG_ALLREDUCE_NHR else oracle.slices_nb(count * 4, n)
+            assert all(s for _, s in sl)
+            for c_s, tree in trees.items():
+                off, size = sl[int(c_s)]
+                lo, hi = off // 4, (off + size) // 4
+                want = eval_tree(tree, [x[lo:hi] for x in ins], op)
+                for r in range(n):
+                    assert np.array_equal(outs[r][lo:hi].view(np.uint32), want.view(np.uint32)), (key, n, c_s, r, op)
+
+
+def test_nb_small_message_is_not_cut():
+    """Up to 128 KiB per rank share the whole message is slice 0 (all_reduce_nb.cc:203-219): only the ranks whose
+    slice list of the step contains slice 0 reduce - 0,2,4,6 then 0,4 then 0 - and everything moves whole."""
+    n, count = 8, 1000
+    ops = oracle.trace(oracle.ALG_ALLREDUCE_NB, n, count, oracle.F32)
+    assert [sorted(o[2] for o in ops if o[1] == 1 and o[0] == s) for s in range(3)] == [[0, 2, 4, 6], [0, 4], [0]]
+    assert all(o[8] == count * 4 and o[4] == 0 and o[7] == 0 for o in ops)
 
 
 def test_strided_scatter_input_layout():

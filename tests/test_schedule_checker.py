@@ -11,7 +11,9 @@ ALL = [(h.Alg.ALLREDUCE_RING, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_RING, Exp
        (h.Alg.REDUCE_SCATTER_MESH, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.REDUCE_SCATTER_RING_STANDALONE, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.ALLREDUCE_MESH_ONESHOT_ASCENDING, Expect.ALLREDUCE),
-       (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE), (h.Alg.ALLREDUCE_CHUNK_MESH, Expect.ALLREDUCE)]
+       (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE), (h.Alg.ALLREDUCE_CHUNK_MESH, Expect.ALLREDUCE),
+       (h.Alg.ALLREDUCE_NHR, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_NHR, Expect.REDUCE_SCATTER_OUT),
+       (h.Alg.ALLREDUCE_NB, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_NB, Expect.REDUCE_SCATTER_OUT)]
 
 
 @pytest.mark.parametrize("alg,expect", ALL)
@@ -20,7 +22,8 @@ def test_generated_schedules_pass(alg, expect):
         if alg == h.Alg.ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
             continue
         for count, dt, unit in ((0, h.HcommDataType.FP32, 4), (1, h.HcommDataType.INT8, 1),
-                                (1000, h.HcommDataType.FP16, 2), (100003, h.HcommDataType.FP32, 4)):
+                                (1000, h.HcommDataType.FP16, 2), (100003, h.HcommDataType.FP32, 4),
+                                (1200007, h.HcommDataType.FP32, 4)):
             assert h.schedule_check(alg, n, count, dt)[:2] == (0, 0), (alg, n, count)
             ops = oracle.trace(alg, n, count, dt)        # the oracle's per-rank programs pass the same check
             assert h.oplist_check(ops, n, expect, count, unit)[:2] == (0, 0), (alg, n, count)
