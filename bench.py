@@ -50,6 +50,7 @@ WORKLOADS = {
     "chunk_mesh_ar_bf16_n8_128MiB": ("chunk_mesh", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nhr_ar_bf16_n8_128MiB": ("nhr", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nb_ar_bf16_n8_128MiB": ("nb", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "local_reduce_rs_bf16_n8_16MiB": ("local_reduce_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
 
@@ -106,7 +107,8 @@ def main():
           "int32": h.HcommDataType.INT32, "int8": h.HcommDataType.INT8}
     ALG = {"ring_ar": h.Alg.ALLREDUCE_RING, "rhd_ar": h.Alg.ALLREDUCE_RHD, "ring_rs_stage": h.Alg.REDUCE_SCATTER_RING,
            "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT, "local_reduce": h.Alg.ALLREDUCE_LOCAL_REDUCE,
-           "chunk_mesh": h.Alg.ALLREDUCE_CHUNK_MESH, "nhr": h.Alg.ALLREDUCE_NHR, "nb": h.Alg.ALLREDUCE_NB}
+           "chunk_mesh": h.Alg.ALLREDUCE_CHUNK_MESH, "nhr": h.Alg.ALLREDUCE_NHR, "nb": h.Alg.ALLREDUCE_NB,
+           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE}
     OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
           "min": h.HcommReduceOp.MIN}
     dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
@@ -124,8 +126,9 @@ def main():
         return
 
     nbytes = count * unit
-    pristine = make_inputs(torch, dev, n, count, "fp32prod" if opname == "prod" else dtname)
-    d_in = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
+    in_count = n * count if alg_name == "local_reduce_rs" else count  # a scatter's input holds N slices of count
+    pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
+    d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
 
     def restore():
@@ -140,7 +143,7 @@ def main():
     scratch_bytes = h.scratch_bytes(alg, n, count, dt)
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
-    if alg_name in ("local_reduce", "chunk_mesh", "nhr", "nb") and args.lowering == "both":
+    if alg_name in ("local_reduce", "chunk_mesh", "nhr", "nb", "local_reduce_rs") and args.lowering == "both":
         args.lowering = "stepwise"  # this schedule has no fused lowering
     kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
              h.Kernel.COPY: "k_copy"}
@@ -223,7 +226,8 @@ def main():
         oalg = {"ring_ar": oracle.ALG_ALLREDUCE_RING, "rhd_ar": oracle.ALG_ALLREDUCE_RHD,
                 "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT,
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
-                "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB}[alg_name]
+                "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
+                "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]

@@ -3,7 +3,9 @@
  *
  * A miniature of the reference's algorithm checker (test/st/algorithm/README_en.md:13-15,202-231): no data is
  * moved; every byte range of every rank buffer carries the set of (rank, origin offset) contributions folded
- * into it.  Two verdicts:
+ * into it.  Each buffer is cut into intervals at the ends of the ranges operations touch in it, and at the images
+ * of those cuts under the operations' source <-> destination translations, so that one operation always maps whole
+ * intervals onto whole intervals.  Two verdicts:
  *   memory conflicts - inside one step no operation may write a range another operation of the step reads or
  *                      writes (test/st/algorithm/README_en.md:202-231);
  *   semantics        - at the end, every byte of the expected result ranges holds exactly one contribution from
@@ -71,6 +73,31 @@ static void report(HcommGfxCheckReport* r, int is_conflict, const char* fmt, uin
 
 static int ranges_overlap(uint64_t a, uint64_t an, uint64_t b, uint64_t bn) { return a < b + bn && b < a + an; }
 
+#define MAX_BOUNDS_PER_BUFFER (1u << 20)
+
+/* Copy the boundaries of `from` that lie strictly inside (lo, lo + len) into `to`, moved by to_off - lo.
+ * Returns 1 when `to` grew, 0 when not, -1 when out of memory. */
+static int translate_bounds(const Bounds* from, uint64_t lo, uint64_t len, Bounds* to, uint64_t to_off)
+{
+    size_t k0 = bounds_find(from, lo + 1), k1 = bounds_find(from, lo + len);
+    if (k1 <= k0) return 0;
+    const size_t m = k1 - k0;
+    uint64_t* v = (uint64_t*)malloc(m * sizeof(uint64_t)); /* `to` may be `from` itself: take a snapshot first */
+    if (!v) return -1;
+    memcpy(v, &from->b[k0], m * sizeof(uint64_t));
+    int grew = 0;
+    for (size_t k = 0; k < m; ++k) {
+        const int a = bounds_add(to, v[k] - lo + to_off);
+        if (a < 0 || to->n > MAX_BOUNDS_PER_BUFFER) {
+            free(v);
+            return -1;
+        }
+        grew |= a;
+    }
+    free(v);
+    return grew;
+}
+
 int32_t HcommGfxOpListCheck(
     const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, HcommGfxExpectation expect, uint64_t count,
     uint64_t strideCount, uint32_t unitSize, HcommGfxCheckReport* rep)
@@ -79,64 +106,90 @@ int32_t HcommGfxOpListCheck(
     memset(rep, 0, sizeof(*rep));
     if (nOps && !ops) return HCCL_E_PTR;
     if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS || unitSize == 0) return HCCL_E_PARA;
+    if (expect != HCOMM_GFX_EXPECT_ALLREDUCE && expect != HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE &&
+        expect != HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT)
+        return HCCL_E_PARA;
     if (strideCount == 0) strideCount = count;
     const uint64_t total = count * unitSize;
     for (uint64_t i = 0; i < nOps; ++i)
         if (ops[i].rank >= nRanks || ops[i].srcRank >= nRanks || ops[i].dstBuf > 2 || ops[i].srcBuf > 2 || ops[i].kind > 1)
             return HCCL_E_PARA;
 
-    /* 1. interval boundaries, closed under the translations the operations perform */
-    Bounds bs = {0};
-    int rc = HCCL_SUCCESS;
+    /* 1. interval boundaries, one set per rank buffer (input, output, communication buffer), closed under the
+     *    translations the operations perform between their source and destination buffers */
+    const uint32_t nbuf = 3 * nRanks;
+    Bounds* bs = (Bounds*)calloc(nbuf, sizeof(Bounds));
+    size_t* first = (size_t*)calloc((size_t)nbuf + 1, sizeof(size_t));
+    Cell *st = NULL, *tmp = NULL;
+    int rc = (bs && first) ? HCCL_SUCCESS : HCCL_E_MEMORY;
+#define BS(rank, buf) bs[(size_t)(rank) * 3 + (buf)]
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
     HcommGfxCalcSlices(count, unitSize, nRanks, sl);
-    if (bounds_add(&bs, 0) < 0 || bounds_add(&bs, total) < 0) rc = HCCL_E_MEMORY;
-    for (uint32_t r = 0; r < nRanks && rc == HCCL_SUCCESS; ++r) {
-        if (bounds_add(&bs, sl[r].offset) < 0 || bounds_add(&bs, sl[r].offset + sl[r].size) < 0) rc = HCCL_E_MEMORY;
-        if (bounds_add(&bs, (uint64_t)r * strideCount * unitSize) < 0 ||
-            bounds_add(&bs, (uint64_t)r * strideCount * unitSize + total) < 0) rc = HCCL_E_MEMORY;
+    uint64_t res_lo[HCOMM_GFX_MAX_RANKS], res_hi[HCOMM_GFX_MAX_RANKS], res_origin[HCOMM_GFX_MAX_RANKS];
+    uint32_t res_buf = 1;
+    for (uint32_t r = 0; r < nRanks && rc == HCCL_SUCCESS; ++r) { /* the expected result ranges */
+        res_lo[r] = 0;
+        res_hi[r] = total;
+        res_origin[r] = 0;
+        if (expect == HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE) {
+            res_buf = 0;
+            res_lo[r] = sl[r].offset;
+            res_hi[r] = sl[r].offset + sl[r].size;
+        } else if (expect == HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT) {
+            res_origin[r] = (uint64_t)r * strideCount * unitSize; /* out[r][x] comes from everybody's in[..][origin + x] */
+        }
+        if (bounds_add(&BS(r, res_buf), res_lo[r]) < 0 || bounds_add(&BS(r, res_buf), res_hi[r]) < 0) rc = HCCL_E_MEMORY;
     }
     for (uint64_t i = 0; i < nOps && rc == HCCL_SUCCESS; ++i) {
-        if (bounds_add(&bs, ops[i].dstOff) < 0 || bounds_add(&bs, ops[i].dstOff + ops[i].bytes) < 0 ||
-            bounds_add(&bs, ops[i].srcOff) < 0 || bounds_add(&bs, ops[i].srcOff + ops[i].bytes) < 0) rc = HCCL_E_MEMORY;
+        const HcommGfxSchedOp* o = &ops[i];
+        if (bounds_add(&BS(o->rank, o->dstBuf), o->dstOff) < 0 || bounds_add(&BS(o->rank, o->dstBuf), o->dstOff + o->bytes) < 0 ||
+            bounds_add(&BS(o->srcRank, o->srcBuf), o->srcOff) < 0 || bounds_add(&BS(o->srcRank, o->srcBuf), o->srcOff + o->bytes) < 0)
+            rc = HCCL_E_MEMORY;
     }
-    for (int changed = 1, guard = 0; changed && rc == HCCL_SUCCESS && guard < 64; ++guard) {
+    for (int changed = 1; changed && rc == HCCL_SUCCESS;) {
         changed = 0;
         for (uint64_t i = 0; i < nOps && rc == HCCL_SUCCESS; ++i) {
             const HcommGfxSchedOp* o = &ops[i];
-            if (o->dstOff == o->srcOff) continue;
-            for (size_t k = 0; k < bs.n; ++k) {
-                const uint64_t v = bs.b[k];
-                int a = 0, b = 0;
-                if (v > o->srcOff && v < o->srcOff + o->bytes) a = bounds_add(&bs, v - o->srcOff + o->dstOff);
-                if (v > o->dstOff && v < o->dstOff + o->bytes) b = bounds_add(&bs, v - o->dstOff + o->srcOff);
-                if (a < 0 || b < 0) { rc = HCCL_E_MEMORY; break; }
-                if (a > 0 || b > 0) changed = 1;
-            }
+            if (o->bytes == 0) continue;
+            Bounds* s = &BS(o->srcRank, o->srcBuf);
+            Bounds* d = &BS(o->rank, o->dstBuf);
+            const int a = translate_bounds(s, o->srcOff, o->bytes, d, o->dstOff);
+            const int b = a < 0 ? -1 : translate_bounds(d, o->dstOff, o->bytes, s, o->srcOff);
+            if (a < 0 || b < 0) rc = HCCL_E_MEMORY;
+            else if (a || b) changed = 1;
         }
     }
-    if (rc != HCCL_SUCCESS) { free(bs.b); return rc; }
 
-    /* 2. state: 3 buffers per rank (input, output, communication buffer) x intervals */
-    const size_t ni = bs.n - 1;
-    Cell* st = (Cell*)calloc((size_t)3 * nRanks * (ni ? ni : 1), sizeof(Cell));
-    Cell* tmp = (Cell*)calloc(ni ? ni : 1, sizeof(Cell));
-    if (!st || !tmp) { free(st); free(tmp); free(bs.b); return HCCL_E_MEMORY; }
-#define CELL(rank, buf, iv) st[((size_t)(rank) * 3 + (buf)) * ni + (iv)]
+    /* 2. state: one cell per interval of every buffer */
+    size_t ncell = 0, widest = 1;
+    for (uint32_t q = 0; q < nbuf && rc == HCCL_SUCCESS; ++q) {
+        first[q] = ncell;
+        const size_t ni = bs[q].n ? bs[q].n - 1 : 0;
+        ncell += ni;
+        if (ni > widest) widest = ni;
+    }
+    if (rc == HCCL_SUCCESS) {
+        first[nbuf] = ncell;
+        st = (Cell*)calloc(ncell ? ncell : 1, sizeof(Cell));
+        tmp = (Cell*)calloc(widest, sizeof(Cell));
+        if (!st || !tmp) rc = HCCL_E_MEMORY;
+    }
+    if (rc != HCCL_SUCCESS) goto done;
+#define CELL(rank, buf, iv) st[first[(size_t)(rank) * 3 + (buf)] + (iv)]
     for (uint32_t r = 0; r < nRanks; ++r)
-        for (size_t iv = 0; iv < ni; ++iv) {
-            for (uint32_t k = 0; k < nRanks; ++k) {
-                CELL(r, 0, iv).delta[k] = NO_DELTA;
-                CELL(r, 1, iv).delta[k] = NO_DELTA;
-                CELL(r, 2, iv).delta[k] = NO_DELTA;
+        for (uint32_t buf = 0; buf < 3; ++buf) {
+            const size_t ni = first[(size_t)r * 3 + buf + 1] - first[(size_t)r * 3 + buf];
+            for (size_t iv = 0; iv < ni; ++iv) {
+                for (uint32_t k = 0; k < nRanks; ++k) CELL(r, buf, iv).delta[k] = NO_DELTA;
+                if (buf == 0) { /* an input holds its own rank's data from the same offset */
+                    CELL(r, 0, iv).cnt[r] = 1;
+                    CELL(r, 0, iv).delta[r] = 0;
+                }
             }
-            CELL(r, 0, iv).cnt[r] = 1; /* an input holds its own rank's data from the same offset */
-            CELL(r, 0, iv).delta[r] = 0;
         }
 
     /* 3. replay step by step */
-    uint64_t i = 0;
-    while (i < nOps) {
+    for (uint64_t i = 0; i < nOps;) {
         uint64_t j = i;
         while (j < nOps && ops[j].step == ops[i].step) ++j;
         for (uint64_t a = i; a < j; ++a)
@@ -152,9 +205,12 @@ int32_t HcommGfxOpListCheck(
         for (uint64_t a = i; a < j; ++a) {
             const HcommGfxSchedOp* o = &ops[a];
             if (o->bytes == 0) continue;
-            const size_t s0 = bounds_find(&bs, o->srcOff), s1 = bounds_find(&bs, o->srcOff + o->bytes);
-            const size_t d0 = bounds_find(&bs, o->dstOff);
+            const Bounds* sb = &BS(o->srcRank, o->srcBuf);
+            const Bounds* db = &BS(o->rank, o->dstBuf);
+            const size_t s0 = bounds_find(sb, o->srcOff), s1 = bounds_find(sb, o->srcOff + o->bytes);
+            const size_t d0 = bounds_find(db, o->dstOff);
             const int64_t shift = (int64_t)o->srcOff - (int64_t)o->dstOff;
+            /* closure makes the two ranges cut at the same relative positions: s1 - s0 intervals on both sides */
             for (size_t k = 0; k < s1 - s0; ++k) tmp[k] = CELL(o->srcRank, o->srcBuf, s0 + k); /* pre-step value */
             for (size_t k = 0; k < s1 - s0; ++k) {
                 Cell* d = &CELL(o->rank, o->dstBuf, d0 + k);
@@ -179,35 +235,29 @@ int32_t HcommGfxOpListCheck(
 
     /* 4. the expected result ranges */
     for (uint32_t r = 0; r < nRanks; ++r) {
-        uint64_t lo = 0, hi = total, origin = 0;
-        uint32_t buf = 1;
-        if (expect == HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE) {
-            buf = 0;
-            lo = sl[r].offset;
-            hi = sl[r].offset + sl[r].size;
-        } else if (expect == HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT) {
-            origin = (uint64_t)r * strideCount * unitSize; /* out[r][x] comes from everybody's in[..][origin + x] */
-        } else if (expect != HCOMM_GFX_EXPECT_ALLREDUCE) {
-            rc = HCCL_E_PARA;
-            break;
-        }
-        if (hi <= lo) continue;
-        const size_t i0 = bounds_find(&bs, lo), i1 = bounds_find(&bs, hi);
+        if (res_hi[r] <= res_lo[r]) continue;
+        const Bounds* b = &BS(r, res_buf);
+        const size_t i0 = bounds_find(b, res_lo[r]), i1 = bounds_find(b, res_hi[r]);
         for (size_t iv = i0; iv < i1; ++iv) {
-            const Cell* c = &CELL(r, buf, iv);
-            if (c->bad) report(rep, 0, "result of rank %llu at offset %llu mixes one rank's data from two different offsets (buffer %llu)", r, bs.b[iv], buf);
+            const Cell* c = &CELL(r, res_buf, iv);
+            if (c->bad) report(rep, 0, "result of rank %llu at offset %llu mixes one rank's data from two different offsets (buffer %llu)", r, b->b[iv], res_buf);
             for (uint32_t q = 0; q < nRanks; ++q) {
                 if (c->cnt[q] != 1)
-                    report(rep, 0, "result of rank %llu at offset %llu holds rank %llu's data a wrong number of times", r, bs.b[iv], q);
-                else if (c->delta[q] != (int64_t)origin)
-                    report(rep, 0, "result of rank %llu at offset %llu took rank %llu's data from a different offset", r, bs.b[iv], q);
+                    report(rep, 0, "result of rank %llu at offset %llu holds rank %llu's data a wrong number of times", r, b->b[iv], q);
+                else if (c->delta[q] != (int64_t)res_origin[r])
+                    report(rep, 0, "result of rank %llu at offset %llu took rank %llu's data from a different offset", r, b->b[iv], q);
             }
         }
     }
 #undef CELL
+#undef BS
+done:
     free(st);
     free(tmp);
-    free(bs.b);
+    if (bs)
+        for (uint32_t q = 0; q < nbuf; ++q) free(bs[q].b);
+    free(bs);
+    free(first);
     return rc;
 }
 
@@ -222,7 +272,8 @@ int32_t HcommGfxScheduleCheck(
     HcommGfxExpectation e = HCOMM_GFX_EXPECT_ALLREDUCE;
     if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE;
     if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_MESH || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE ||
-        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
+        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB ||
+        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE)
         e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT;
     rc = HcommGfxOpListCheck(l.ops, l.n, nRanks, e, count, strideCount, HcommGfxDataTypeSize(dataType), rep);
     hg_oplist_free(&l);

@@ -255,11 +255,30 @@ static void local_reduce_slices(uint64_t total, uint32_t n, uint32_t unit, Hcomm
     *per_out = per;
 }
 
+/* ReduceScatterLocalReduce: where rank i's receive window starts inside its communication buffer
+ * (temp_reduce_scatter/reduce_scatter_local_reduce.cc:102-123: staggered by the slice's position in the user input
+ * modulo 16 KiB once a slice exceeds 32 KiB) and the distance between the N-1 slots of the window (:162-178: the
+ * slice size rounded up to 16 KiB; the communication buffer is sized so that this first choice always fits). */
+static uint64_t rs_local_reduce_window(uint64_t total, uint32_t i)
+{
+    return total > 32u * 1024u ? ((uint64_t)i * total) % 16384u : 0;
+}
+
+static uint64_t rs_local_reduce_slot(uint64_t total) { return total == 0 ? 16384u : (total + 16383u) / 16384u * 16384u; }
+
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype)
 {
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
     if (n < 2) return 0;
     if (alg == HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH) return count * unit;
+    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE) {
+        uint64_t max_off = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            const uint64_t o = rs_local_reduce_window(count * unit, i);
+            if (o > max_off) max_off = o;
+        }
+        return max_off + (uint64_t)(n - 1) * rs_local_reduce_slot(count * unit);
+    }
     if (alg != HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE) return 0;
     return (uint64_t)n * local_reduce_slot(count * unit, n, unit);
 }
@@ -467,6 +486,7 @@ static int sched_allreduce_nhr(HgOpList* l, uint32_t n, uint64_t count, uint32_t
     if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* all_reduce_nhr.cc:35-44 */
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
     uint32_t map[HCOMM_GFX_MAX_RANKS];
+    memset(map, 0, sizeof(map));
     CHK(HcommGfxCalcSlices(count, unit, n, sl)); /* all_reduce_nhr.cc:104-121: the ring's slice table */
     nhr_slice_map(n, 0, map);
     CHK(nhr_rs(l, n, sl, map, 1));
@@ -539,6 +559,7 @@ static int sched_allreduce_nb(HgOpList* l, uint32_t n, uint64_t count, uint32_t 
     const uint64_t gran = raw > small ? HG_SLICE_ALIGN : small;
     const uint64_t per = raw == 0 ? gran : (raw + gran - 1) / gran * gran;
     uint64_t residue = total;
+    memset(sl, 0, sizeof(sl));
     for (uint32_t i = 0; i < n; ++i) {
         sl[i].size = residue > per ? per : residue;
         sl[i].offset = total - residue;
@@ -575,6 +596,39 @@ static int sched_rs_nb(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride,
     return HCCL_SUCCESS;
 }
 
+/* ReduceScatterLocalReduce, the deterministic mesh reduce-scatter (temp_reduce_scatter/
+ * reduce_scatter_local_reduce.cc:125-160).  Stated per destination d: think of the row V[0] = d's user output,
+ * V[j] = slot j-1 of d's receive window.  Rank d-j writes its copy of slice d into V[j] and d copies its own into
+ * V[0], all at once (:218-243); then the tail beyond the largest power of two P <= N is folded onto the front,
+ * V[a] (op)= V[a+P] (:266-283), and the front is halved, V[a] (op)= V[a+h] for h = P/2, P/4, ..., 1 (:286-301). */
+static int sched_rs_local_reduce(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t sz = count * unit;
+    const uint64_t slot = rs_local_reduce_slot(sz);
+    for (uint32_t d = 0; d < n; ++d)
+        for (uint32_t r = 0; r < n; ++r) {
+            if (r == d) CHK(push(l, 0, COPY, d, OUT, 0, d, IN, (uint64_t)d * sz, sz));
+            else CHK(push(l, 0, COPY, d, SCR, rs_local_reduce_window(sz, d) + slot * (modn((int64_t)d - r, n) - 1), r, IN, (uint64_t)d * sz, sz));
+        }
+#define V_BUF(j) ((j) == 0 ? OUT : SCR)
+#define V_OFF(d, j) ((j) == 0 ? 0 : rs_local_reduce_window(sz, d) + slot * ((j) - 1))
+    const uint32_t p2 = floor_pow2(n);
+    uint32_t step = 1;
+    if (p2 < n) {
+        for (uint32_t d = 0; d < n; ++d)
+            for (uint32_t a = 0; a < n - p2; ++a)
+                CHK(push(l, step, REDUCE, d, V_BUF(a), V_OFF(d, a), d, SCR, V_OFF(d, a + p2), sz));
+        ++step;
+    }
+    for (uint32_t h = p2 / 2; h >= 1; h /= 2, ++step)
+        for (uint32_t d = 0; d < n; ++d)
+            for (uint32_t a = 0; a < h; ++a)
+                CHK(push(l, step, REDUCE, d, V_BUF(a), V_OFF(d, a), d, SCR, V_OFF(d, a + h), sz));
+#undef V_BUF
+#undef V_OFF
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
@@ -601,6 +655,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_REDUCE_SCATTER_NHR: rc = sched_rs_nhr(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_NB: rc = sched_allreduce_nb(l, n, count, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_NB: rc = sched_rs_nb(l, n, count, stride, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE: rc = sched_rs_local_reduce(l, n, count, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

@@ -349,7 +349,13 @@ typedef enum {
        128 KiB (all_reduce_nb.cc:203-219) */
     HCOMM_GFX_ALG_ALLREDUCE_NB = 11,
     /* stand-alone ReduceScatterNB (reduce_scatter_nb.cc:27-86), layout as HCOMM_GFX_ALG_REDUCE_SCATTER_NHR */
-    HCOMM_GFX_ALG_REDUCE_SCATTER_NB = 12
+    HCOMM_GFX_ALG_REDUCE_SCATTER_NB = 12,
+    /* ReduceScatterLocalReduce (the deterministic mesh reduce-scatter, any N): temp_reduce_scatter/
+       reduce_scatter_local_reduce.cc:125-160.  Every rank writes its copy of slice d into a slot of rank d's
+       communication buffer (:218-243), rank d folds the slots and its own copy pairwise in a fixed order into
+       out[d][0..count) (:252-304).  Input holds N dense slices of count elements; needs the third buffer
+       (HcommGfxScratchBytes).  Step-wise lowering only. */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE = 13
 } HcommGfxAlgorithm;
 
 typedef enum {

@@ -924,6 +924,64 @@ static void prog_rs_nb(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, u
     prog_nb_rs(t, rank, n, sl, osl);
 }
 
+/* ReduceScatterLocalReduce::RunAsync for one rank, tpl/temp_reduce_scatter/reduce_scatter_local_reduce.cc:125-160,
+ * in the single-pass configuration (count_ == opInfo->count; the template's "output memory" is the communication
+ * buffer, sized so that CalAlign's first choice fits).  Returns the bytes of communication buffer a rank needs
+ * when t is NULL. */
+static uint64_t prog_rs_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;            /* totalSize, :187 */
+    const uint64_t offset = count * unit;           /* (opInfo_->count) * unitSize, :192 */
+    uint64_t sl_off[ORC_MAX_RANKS], max_off = 0;
+    for (uint32_t i = 0; i < n; i++) {              /* PrepareOffset, :113-121 */
+        sl_off[i] = (total > 32u * 1024u) ? ((uint64_t)i * offset) % 16384u : 0;
+        if (sl_off[i] > max_off) max_off = sl_off[i];
+    }
+    /* CalAlign, :162-178, first choice: RoundUpWithDivisor(totalSize, HCCL_MIN_SLICE_ALIGN_910B), which is the
+     * divisor itself for 0 (tpl/alg_template_base_pub.h:609-616) */
+    const uint64_t align = (total == 0) ? 16384u : ((total + 16383u) / 16384u) * 16384u;
+    const uint64_t need = max_off + align * (n - 1);
+    if (!t || n == 0) return n > 1 ? need : 0;
+    /* RunReduceScatter, :218-243: all rounds run at once, each on a stream of its own */
+    for (uint32_t round = 1; round < n; round++) {
+        const uint32_t dst_rank = (round + rank) % n;
+        emit(t, 0, K_COPY, dst_rank, B_SCR, align * (round - 1) + sl_off[dst_rank], rank, B_IN, offset * dst_rank, total);
+    }
+    emit(t, 0, K_COPY, rank, B_OUT, 0, rank, B_IN, offset * rank, total); /* :238-241 */
+    /* RunLocalReduce, :252-304; the window starts at slices_[rank].offset (:262) */
+    uint32_t power = 0;
+    while ((2u << power) <= n) power++;             /* static_cast<u32>(log2(rankSize)) */
+    uint32_t rank_power = 1u << power;
+    const uint64_t win = sl_off[rank];
+    uint32_t step = 1;
+    if (rank_power < n) {
+        for (uint32_t add = 0; add < n - rank_power; add++) { /* :270-282 */
+            const uint64_t src = win + align * (add + rank_power - 1);
+            if (add == 0) emit(t, step, K_REDUCE, rank, B_OUT, 0, rank, B_SCR, src, total);
+            else emit(t, step, K_REDUCE, rank, B_SCR, win + align * (add - 1), rank, B_SCR, src, total);
+        }
+        step++;
+    }
+    for (uint32_t round = 0; round < power; round++) { /* :286-301 */
+        rank_power = 1u << (power - round - 1);
+        for (uint32_t add = 0; add < rank_power; add++) {
+            const uint64_t src = win + align * (add + rank_power - 1);
+            if (add == 0) emit(t, step, K_REDUCE, rank, B_OUT, 0, rank, B_SCR, src, total);
+            else emit(t, step, K_REDUCE, rank, B_SCR, win + align * (add - 1), rank, B_SCR, src, total);
+        }
+        step++;
+    }
+    return need;
+}
+
+/* Bytes of communication buffer per rank for the deterministic mesh reduce-scatter. */
+uint64_t orc_rs_local_reduce_scratch_bytes(uint32_t n, uint64_t count, int dtype)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (n == 0 || n > ORC_MAX_RANKS || unit == 0) return 0;
+    return prog_rs_local_reduce(NULL, 0, n, count, unit);
+}
+
 /* The NHR slice map, exported for the hand-derived fixtures. */
 void orc_nhr_slice_map(uint32_t n, uint32_t* slice_map)
 {
@@ -944,7 +1002,8 @@ enum {
     ORC_ALG_ALLREDUCE_NHR = 9,
     ORC_ALG_RS_NHR = 10,
     ORC_ALG_ALLREDUCE_NB = 11,
-    ORC_ALG_RS_NB = 12
+    ORC_ALG_RS_NB = 12,
+    ORC_ALG_RS_LOCAL_REDUCE = 13
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -982,6 +1041,13 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
             case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, stride, unit); break;
+            case ORC_ALG_RS_LOCAL_REDUCE:
+                if (stride != count) {
+                    free(t->ops);
+                    return -1;
+                }
+                prog_rs_local_reduce(t, r, n, count, unit);
+                break;
             case ORC_ALG_ALLREDUCE_LOCAL_REDUCE:
                 if (prog_allreduce_local_reduce(t, r, n, count, unit) != 0) {
                     free(t->ops);

@@ -25,6 +25,7 @@ ALGS = {
     "nhr_rs": (h.Alg.REDUCE_SCATTER_NHR, oracle.ALG_RS_NHR),
     "nb_ar": (h.Alg.ALLREDUCE_NB, oracle.ALG_ALLREDUCE_NB),
     "nb_rs": (h.Alg.REDUCE_SCATTER_NB, oracle.ALG_RS_NB),
+    "local_reduce_rs": (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, oracle.ALG_RS_LOCAL_REDUCE),
 }
 SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
@@ -37,7 +38,7 @@ def say(*a):
 
 def buffer_counts(alg, n, count, stride=0):
     """(elements in each input buffer, elements in each output buffer)."""
-    if alg in SCATTER:
+    if alg in SCATTER or alg == "local_reduce_rs":
         return ((n - 1) * stride + count if stride else n * count), count
     return count, count
 
@@ -157,6 +158,14 @@ CASES = [
     ("nb_rs", 8, 40001, "fp32", "sum"),
     ("nb_rs", 7, 5000, "bf16", "sum"),
     ("nb_rs", 12, 999, "int32", "sum"),
+    ("local_reduce_rs", 8, 1 << 20, "bf16", "sum"),
+    ("local_reduce_rs", 7, 100003, "fp32", "sum"),  # receive windows start at i*400012 mod 16384: 4-byte aligned only
+    ("local_reduce_rs", 6, 16384, "fp16", "max"),
+    ("local_reduce_rs", 5, 70001, "int8", "sum"),   # odd byte offsets
+    ("local_reduce_rs", 16, 40000, "int32", "min"),
+    ("local_reduce_rs", 3, 1001, "int16", "sum"),   # up to 32 KiB: windows not staggered
+    ("local_reduce_rs", 2, 9, "fp32", "prod"),
+    ("local_reduce_rs", 1, 100, "fp32", "sum"),
 ]
 
 

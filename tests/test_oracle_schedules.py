@@ -16,8 +16,11 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUCE_RHD,
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
         oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
-        oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB]
-SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB)
+        oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB,
+        oracle.ALG_RS_LOCAL_REDUCE]
+SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
+               oracle.ALG_RS_LOCAL_REDUCE)
+STRIDED = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB)
 
 
 def scratch_for(alg, n, count, dt):
@@ -224,7 +227,7 @@ def test_scatter_variants_deliver_the_right_slice():
         ins = [(np.arange(n * count, dtype=np.int32) * 10 + r) for r in range(n)]
         outs = [np.zeros(count, np.int32) for _ in range(n)]
         want = sum(x.astype(np.int64) for x in ins)
-        oracle.run(alg, [x.copy() for x in ins], outs, count, oracle.I32, oracle.SUM)
+        oracle.run(alg, [x.copy() for x in ins], outs, count, oracle.I32, oracle.SUM, scratch=scratch_for(alg, n, count, oracle.I32))
         for r in range(n):
             assert np.array_equal(outs[r], want[r * count:(r + 1) * count].astype(np.int32))
 
@@ -367,12 +370,43 @@ def test_nb_small_message_is_not_cut():
     assert all(o[8] == count * 4 and o[4] == 0 and o[7] == 0 for o in ops)
 
 
+def test_rs_local_reduce_hand_derived():
+    """Deterministic mesh reduce-scatter: window / slot arithmetic and the pairwise fold order, by hand."""
+    for case in GOLD["rs_local_reduce_layout"]["cases"]:
+        n, count = case["n"], case["count"]
+        assert h.scratch_bytes(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, n, count, oracle.F32) == case["scratch_bytes"]
+        assert oracle.lib().orc_rs_local_reduce_scratch_bytes(n, count, oracle.F32) == case["scratch_bytes"]
+        ops = oracle.trace(oracle.ALG_RS_LOCAL_REDUCE, n, count, oracle.F32)
+        for d in range(n):
+            slots = sorted(o[4] for o in ops if o[0] == 0 and o[2] == d and o[3] == 2)
+            assert slots == [case["windows"][d] + j * case["slot"] for j in range(n - 1)]
+    for n in range(1, 33):
+        for count in (0, 1, 8192, 8193, 100003):
+            assert h.scratch_bytes(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, n, count, oracle.F32) == \
+                oracle.lib().orc_rs_local_reduce_scratch_bytes(n, count, oracle.F32)
+    for op in (oracle.SUM, oracle.MAX):
+        for n_s, trees in GOLD["rs_local_reduce_rank_tree"].items():
+            if n_s.startswith("_"):
+                continue
+            n, count = int(n_s), 9001
+            big = [np.concatenate([order_sensitive_inputs(n, count, op, seed=90 + r * 7 + i)[0] for i in range(n)]) for r in range(n)]
+            outs = [np.zeros(count, np.float32) for _ in range(n)]
+            scr = scratch_for(oracle.ALG_RS_LOCAL_REDUCE, n, count, oracle.F32)
+            oracle.run(oracle.ALG_RS_LOCAL_REDUCE, [x.copy() for x in big], outs, count, oracle.F32, op, scratch=scr)
+            for d_s, tree in trees.items():
+                d = int(d_s)
+                want = eval_tree(tree, [x[d * count:(d + 1) * count] for x in big], op)
+                assert np.array_equal(outs[d].view(np.uint32), want.view(np.uint32)), (n, d, op)
+    with pytest.raises(ValueError):
+        oracle.trace(oracle.ALG_RS_LOCAL_REDUCE, 4, 100, oracle.F32, 200)   # dense input slices only
+
+
 def test_strided_scatter_input_layout():
     """Input slice i starts strideLen * i elements into the buffer (aicpu_reduce_scatter.cc:78-80); the gaps
     between slices are never read or written."""
     g = GOLD["strided_rs"]
     n, count, stride = g["n"], g["count"], g["stride"]
-    for alg in SCATTER_OUT:
+    for alg in STRIDED:
         ops = oracle.trace(alg, n, count, oracle.F32, stride)
         offs = sorted(set(o[4] for o in ops if o[3] == 0) | set(o[7] for o in ops if o[6] == 0))
         assert offs == g["slice_byte_offsets"]
@@ -401,7 +435,7 @@ def test_product_generator_equals_oracle_trace(alg):
             a = oracle.trace(alg, n, count, dt)
             b = h.schedule_emit(alg, n, count, dt)
             assert a == b, (alg, n, count, dt)
-            if alg in SCATTER_OUT:
+            if alg in STRIDED:
                 assert oracle.trace(alg, n, count, dt, count + 13) == h.schedule_emit(alg, n, count, dt, count + 13)
 
 
