@@ -262,6 +262,32 @@ def main():
                          % (passes, cpu_s),
                "single_thread_value": round(alg_bytes / one_s / 1e9, 2), "cpu_model": model,
                "host_cores": os.cpu_count()}
+        # the reference's own CPU reduce loop (VirtualRunTime::MemReduceSum, test/hccl_vm/src/plugin/runner/
+        # runner_utils/hccl_task_reduce_process.cc:57-84, compiled from where it lies into oracle/_ref) on one
+        # thread, for the element types it has (no bf16 there): dst = dst + src over a bounded sample, 3 bytes
+        # of traffic per byte of dst
+        if oracle.have_ref():
+            R = oracle.ref()
+            rng = np.random.default_rng(7)
+            witness = {}
+            for rname, rdt, elems in (("fp32", oracle.F32, 1 << 24), ("fp16", oracle.F16, 1 << 22), ("int32", oracle.I32, 1 << 24)):
+                if rdt == oracle.F16:
+                    d_ = rng.uniform(-1, 1, elems).astype(np.float16).view(np.uint16)
+                    s_ = rng.uniform(-1, 1, elems).astype(np.float16).view(np.uint16)
+                elif rdt == oracle.F32:
+                    d_, s_ = (rng.uniform(-1, 1, elems).astype(np.float32) for _ in range(2))
+                else:
+                    d_, s_ = (rng.integers(-1 << 20, 1 << 20, elems).astype(np.int32) for _ in range(2))
+                reps, t_ref = 0, 0.0
+                while reps < 1 or (t_ref < 1.0 and reps < 64):
+                    t0 = time.perf_counter()
+                    R.ref_mem_reduce_sum(s_.ctypes.data, d_.ctypes.data, d_.nbytes, rdt)
+                    t_ref += time.perf_counter() - t0
+                    reps += 1
+                witness[rname] = round(3.0 * d_.nbytes * reps / t_ref / 1e9, 2)
+            cpu["reference_reduce"] = {"kind": "reference", "function": "VirtualRunTime::MemReduceSum", "cores": 1,
+                                       "unit": "GB/s", "value_by_dtype": witness,
+                                       "sample": "dst += src over 2^24 fp32 / int32 and 2^22 fp16 elements, >= 1 s each"}
         # verification: one GPU pass per lowering from pristine inputs must equal the oracle bit for bit
         verified = True
         for name in lowerings:
