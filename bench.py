@@ -30,10 +30,15 @@ HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
 # dispatch; FETCH_SIZE scaled by 2.0, the factor that makes k_copy's known 128 MiB read come out right;
 # WRITE_SIZE by 1.0).  Summaries: profiles/k_reduce2_bf16_ring_ar_n8_128MiB.md,
-# profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md.
+# profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md, profiles/k_fold_tree_int32_rhd_ar_n16_128MiB.md,
+# profiles/k_reduce2_bf16_nhr_ar_n8_128MiB.md.
 MEASURED_TRAFFIC = {
     ("ring_ar_bf16_n8_128MiB", "stepwise"): (131115.7 * 2.0 + 131072.0) * 1024,
     ("ring_ar_bf16_n8_128MiB", "fused"): (524348.6 * 2.0 + 1966281.4) * 1024,
+    # averages over the launches of the dominant kernel in one collective (they differ in size per step)
+    ("rhd_ar_int32_n16_128MiB_sum", "stepwise"): (491539.0 * 2.0 + 491520.0) * 1024,
+    ("rhd_ar_int32_n16_128MiB_sum", "fused"): (1048633.4 * 2.0 + 3147325.6) * 1024,
+    ("nhr_ar_bf16_n8_128MiB", "stepwise"): (305878.8 * 2.0 + 305834.7) * 1024,
 }
 
 # name: (algorithm, ranks, elements per rank, dtype, op, data distribution)
