@@ -89,6 +89,14 @@ void hg_finish_fold(HgLaunch* l)
          * position that absorbed a neighbour (which block ranks sit on odd positions depends on the slice), and
          * nout outputs */
         uint64_t moved = 0;
+        if (t->tree != 1u) {
+            /* truncated rotation trees: nranks leaf reads, one store per even position that has a right neighbour,
+             * and the root to one output or to all of them */
+            const uint64_t n = (uint64_t)t->nranks + t->nranks / 2 + (t->out_mode == 1u ? 1u : t->nout);
+            l->moved_bytes = n * bytes;
+            l->blocks = hg_grid_blocks(tiles);
+            return;
+        }
         for (uint32_t s = 0; s < t->nseg; ++s) {
             uint64_t n = t->k + t->k / 2 + t->nout;
             for (uint32_t b = 0; b < t->k; ++b)

@@ -484,6 +484,44 @@ __device__ __forceinline__ void fold_tree_item(const HgFoldTable& tab, uint32_t 
     for (uint32_t r = 0; r < tab.nout; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, x[0]);
 }
 
+// The trees of the nonuniform hierarchical ring and of the nonuniform Bruck schedule: n <= K = 2^L ranks, position
+// q of slice c holds rank c + q (tree == 2) or c - q (tree == 3) mod n, and level l combines position q (dst role,
+// q a multiple of 2^(l+1)) with q + 2^l wherever that position exists - the fold rank (c +- q) performs at step l
+// from rank (c +- q) +- 2^l.  An even position that had a right neighbour keeps the last value it computed; the
+// root goes to every output (allreduce) or to the owner's output (reduce-scatter).
+template <class Item, int L>
+__device__ __forceinline__ void fold_tree_item_rot(const HgFoldTable& tab, uint32_t s, uint64_t idx)
+{
+    typedef typename Item::V V;
+    constexpr uint32_t K = 1u << L;
+    const uint64_t off = tab.off[s];
+    const uint32_t c = tab.first[s];
+    const uint32_t n = tab.nranks;
+    const bool plus = tab.tree == 2u;
+    V x[K];
+    uint32_t b[K];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        b[q] = plus ? c + q : c + n - q;
+        if (b[q] >= n) b[q] -= n;
+        if (q < n) x[q] = Item::ld((const uint8_t*)tab.in[b[q]] + off, idx);
+    }
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (uint32_t q = 0; q < K; q += (2u << l))
+            if (q + (1u << l) < n) x[q] = Item::op(x[q], x[q + (1u << l)]);
+    }
+#pragma unroll
+    for (uint32_t q = 0; q < K; q += 2)
+        if (q + 1 < n) Item::st((uint8_t*)tab.in[b[q]] + off, idx, x[q]);
+    if (tab.out_mode == 1u) {
+        Item::st((uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s], idx, x[0]);
+    } else {
+        for (uint32_t r = 0; r < tab.nout; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, x[0]);
+    }
+}
+
 template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
@@ -494,10 +532,17 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
-        if (v < nvec) fold_tree_item<VecItem<DT, OP>, L>(tab, s, v);
+        if (tab.tree == 1u) {
+            if (v < nvec) fold_tree_item<VecItem<DT, OP>, L>(tab, s, v);
+        } else {
+            if (v < nvec) fold_tree_item_rot<VecItem<DT, OP>, L>(tab, s, v);
+        }
         if (v - tid + HG_BLOCK > nvec) { // the segment's last tile also owns its element tail
             const uint64_t e = (nvec << 4) / ES + tid;
-            if ((e + 1) * ES <= bytes) fold_tree_item<ElemItem<DT, OP>, L>(tab, s, e);
+            if ((e + 1) * ES <= bytes) {
+                if (tab.tree == 1u) fold_tree_item<ElemItem<DT, OP>, L>(tab, s, e);
+                else fold_tree_item_rot<ElemItem<DT, OP>, L>(tab, s, e);
+            }
         }
     }
 }

@@ -218,6 +218,59 @@ static int fused_rhd(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* 
     return rc;
 }
 
+/* NHR / NB as one tree launch: slice c is folded over the truncated balanced tree whose position q holds rank
+ * c + q (NHR, the tree-ordered slice map decides where slice c lies) or c - q (NB); see k_fold_tree.  scatter: the
+ * stand-alone reduce-scatter, whose input slice i lies at i * stride elements and whose result goes to out[c][0..). */
+static int fused_rot_tree(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
+                          uint64_t stride, int dtype, int op)
+{
+    HgOpList ol;
+    /* the slice geometry is whatever the schedule's own-slice copy (allreduce) or final copy (reduce-scatter)
+     * says: one copy per rank at step ceil(log2 n), from the input slice that rank owns */
+    int rc = hg_schedule(&ol, alg, n, count, stride, dtype);
+    if (rc != HCCL_SUCCESS) return rc;
+    uint32_t steps = 0;
+    while ((1u << steps) < n) ++steps;
+    const int scatter = (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB);
+    const int plus = (alg == HCOMM_GFX_ALG_ALLREDUCE_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR);
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) {
+        hg_oplist_free(&ol);
+        return HCCL_E_MEMORY;
+    }
+    l->kind = HCOMM_GFX_KERNEL_TREE;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    HgFoldTable* f = &l->tab.fold;
+    f->tree = plus ? 2u : 3u;
+    f->k = 1u << steps;
+    f->nranks = n;
+    f->nout = scatter ? 0 : n;
+    f->out_mode = scatter ? 1u : 2u;
+    for (uint32_t r = 0; r < n; ++r) {
+        f->in[r] = in[r];
+        f->out[r] = out[r];
+    }
+    for (uint64_t i = 0; i < ol.n; ++i) {
+        const HcommGfxSchedOp* o = &ol.ops[i];
+        if (o->step != steps || o->kind != 0 || o->srcBuf != 0 || o->dstBuf != 1 || o->srcRank != o->rank) continue;
+        const uint32_t s = f->nseg++;
+        f->off[s] = o->srcOff;
+        f->out_off[s] = o->dstOff;
+        f->bytes[s] = o->bytes;
+        f->first[s] = (uint8_t)o->rank;
+        f->owner[s] = (uint8_t)o->rank;
+    }
+    hg_oplist_free(&ol);
+    rc = HCCL_SUCCESS;
+    if (f->nseg) {
+        hg_finish_fold(l);
+        rc = plan_push(l, p);
+    }
+    free(l);
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
                        uint64_t stride, int dtype, int op)
 {
@@ -241,6 +294,12 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_REDUCE_SCATTER_MESH:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_mesh(p, n, in, out, count, stride, dtype, op, 1, 0);
+        case HCOMM_GFX_ALG_ALLREDUCE_NHR:
+        case HCOMM_GFX_ALG_ALLREDUCE_NB:
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_NHR:
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_NB:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_rot_tree(p, alg, n, in, out, count, stride, dtype, op);
         default: return HCCL_E_NOT_SUPPORT;
     }
 }

@@ -364,7 +364,9 @@ typedef enum {
     HCOMM_GFX_LOWER_STEPWISE = 0,
     /* steps whose data dependences are element-wise are folded into k-way kernels that read every input
        once and store every value the step-wise replay leaves in a buffer (partials included), so the final
-       contents of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE */
+       contents of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE.  Available for the ring, mesh,
+       recursive halving-doubling, NHR and NB algorithms; the algorithms that stage through a communication
+       buffer return HCCL_E_NOT_SUPPORT */
     HCOMM_GFX_LOWER_FUSED = 1
 } HcommGfxLowering;
 

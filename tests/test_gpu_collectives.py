@@ -28,7 +28,8 @@ ALGS = {
     "local_reduce_rs": (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, oracle.ALG_RS_LOCAL_REDUCE),
 }
 SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
-FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending"}
+FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending",
+           "nhr_ar", "nhr_rs", "nb_ar", "nb_rs"}
 
 
 def say(*a):
@@ -200,7 +201,7 @@ def test_non_associative_inputs_expose_order(gpu_thread):
     """fp32 values for which (a+b)+c != a+(b+c): a replay in any other association order fails here."""
     n, count = 4, 4096
     base = np.array([1e8, 1.0, -1e8, 1.0], np.float32)
-    for alg in ("ring_ar", "rhd_ar", "mesh_oneshot"):
+    for alg in ("ring_ar", "rhd_ar", "mesh_oneshot", "nhr_ar", "nb_ar"):
         for lowering in ((h.Lowering.STEPWISE, h.Lowering.FUSED) if alg in FUSABLE else (h.Lowering.STEPWISE,)):
             host_in = [np.full(count, base[(r + i) % 4], np.float32) for i, r in enumerate(range(n))]
             for r in range(n):
