@@ -91,8 +91,8 @@ static int registry_add(HgThread* t)
     pthread_mutex_lock(&g_threads_mtx);
     for (uint32_t i = 0; i < HG_THREADS_MAX; ++i) {
         if (!g_threads[i]) {
-            g_threads[i] = t;
-            if (i + 1 > g_threads_hi) g_threads_hi = i + 1;
+            __atomic_store_n(&g_threads[i], t, __ATOMIC_RELEASE); /* readers look up without the mutex */
+            if (i + 1 > g_threads_hi) __atomic_store_n(&g_threads_hi, i + 1, __ATOMIC_RELEASE);
             ok = 1;
             break;
         }
@@ -105,7 +105,7 @@ static void registry_remove(HgThread* t)
 {
     pthread_mutex_lock(&g_threads_mtx);
     for (uint32_t i = 0; i < g_threads_hi; ++i)
-        if (g_threads[i] == t) g_threads[i] = NULL;
+        if (g_threads[i] == t) __atomic_store_n(&g_threads[i], (HgThread*)NULL, __ATOMIC_RELEASE);
     pthread_mutex_unlock(&g_threads_mtx);
 }
 
@@ -162,6 +162,9 @@ static void thread_delete(HgThread* t)
 {
     if (!t) return;
     registry_remove(t);
+    /* a thread freed between HcommBatchModeStart and End takes its recorded operations with it */
+    for (uint32_t i = 0; i < g_ctx.ntouched; ++i)
+        if (g_ctx.touched[i] == t) g_ctx.touched[i] = NULL;
     if (!t->recorder) {
         for (uint32_t i = 0; i < t->notify_num; ++i)
             if (t->notifies[i]) hg_rt_event_destroy(t->notifies[i]);
@@ -221,7 +224,7 @@ HcommResult HcommThreadAllocWithStream(CommEngine engine, void* stream, uint32_t
     if (!thread) return HCCL_E_PTR;
     if (hg_rt_device_count() <= 0) return HCCL_E_UNAVAIL;
     HgThread* t = thread_new(0, stream, 0, notifyNum);
-    if (!t) return HCCL_E_PTR;
+    if (!t) return HCCL_E_INTERNAL;
     *thread = (ThreadHandle)(uintptr_t)t;
     return HCCL_SUCCESS;
 }
@@ -488,6 +491,7 @@ int32_t HcommBatchModeEnd(const char* batchTag)
     int32_t ret = HCCL_SUCCESS;
     for (uint32_t i = 0; i < g_ctx.ntouched; ++i) {
         HgThread* t = g_ctx.touched[i];
+        if (!t) continue; /* freed inside the batch */
         if (ret == HCCL_SUCCESS) ret = hg_coalesce(t->pending, t->pending_n, emit_to_thread, t);
         t->pending_n = 0;
     }

@@ -274,6 +274,19 @@ def test_batch_mode_spans_several_threads(rec):
     h.HcommThreadFree([other])
 
 
+def test_thread_freed_inside_a_batch_is_dropped_from_it(rec):
+    code, other = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommBatchModeStart(b"gone") == 0
+    assert h.HcommLocalCopyOnThread(other, DST, SRC, 8192) == 0
+    assert h.HcommLocalCopyOnThread(rec, DST, SRC, 4096) == 0
+    assert h.HcommThreadFree([other]) == 0
+    assert h.HcommBatchModeEnd(b"gone") == 0          # the freed thread's operations went with it
+    assert [(r.nseg, r.bytes) for r in h.launch_log(rec)] == [(1, 4096)]
+    assert h.HcommLocalCopyOnThread(other, DST, SRC, 8192) == R.E_PTR
+
+
 def test_reduce_k_checks(rec):
     f = h.HcommGfxReduceKOnThread
     assert f(rec, DST, [SRC, SRC + 4096], 100, DT.FP16, OP.SUM) == R.SUCCESS
