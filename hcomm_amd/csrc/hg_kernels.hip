@@ -154,6 +154,33 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
     else ((u32x4*)base)[vec] = v;
 }
 
+// Workgroups are dealt to the 8 XCDs round-robin by their index.  REMAP renumbers them so that each XCD walks runs
+// of HG_XCD_RUN consecutive tiles (2 MiB) - or, when the grid does not divide that way, one contiguous eighth of the
+// tiles - instead of every eighth tile.  Measured on the 8 x 128 MiB ring steps (TB/s; plain, runs of 2 / 8 / 32 /
+// 128 tiles, contiguous eighth): copy 6.68, 6.69, 6.65, 6.84, 6.93, 6.87; two-input reduce 6.47, 6.49, 6.53, 6.35,
+// 6.51, 6.17; k-way fold 5.50, 5.44, 5.56, 5.59, 5.15, 4.84.  Only the copy gains beyond run-to-run noise, so only
+// k_copy renumbers.
+#ifndef HG_XCD_REMAP_COPY
+#define HG_XCD_REMAP_COPY 1
+#endif
+#ifndef HG_XCD_REMAP
+#define HG_XCD_REMAP 0
+#endif
+#ifndef HG_XCD_RUN
+#define HG_XCD_RUN 128u
+#endif
+template <bool REMAP> __device__ __forceinline__ uint32_t block_id()
+{
+    const uint32_t g = gridDim.x, b = blockIdx.x;
+    if (!REMAP) return b;
+    if ((g % (8u * HG_XCD_RUN)) == 0u) {
+        const uint32_t i = b >> 3;
+        return (i / HG_XCD_RUN) * 8u * HG_XCD_RUN + (b & 7u) * HG_XCD_RUN + i % HG_XCD_RUN;
+    }
+    if ((g & 7u) == 0u) return (b & 7u) * (g >> 3) + (b >> 3);
+    return b;
+}
+
 // segment that owns a tile (uniform across the workgroup; nseg <= 32)
 __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
 {
@@ -168,7 +195,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP_COPY>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -200,7 +227,7 @@ template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -236,7 +263,7 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 {
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
     const uint32_t total = tab.tile_begin[tab.nseg];
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t e0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + threadIdx.x;
         const uint64_t nelem = tab.bytes[s] / ES;
@@ -355,7 +382,7 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -426,7 +453,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -527,7 +554,7 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];
