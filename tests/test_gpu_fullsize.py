@@ -174,3 +174,34 @@ def test_config4_mesh_oneshot_fp16_sweep(gpu_thread):
             for r in range(n):
                 assert_same(from_dev(d_out[r], want_out[r]), want_out[r], oracle.F16, "m=%d out[%d]" % (m, r))
                 assert_same(from_dev(d_in[r], host_in[r]), host_in[r], oracle.F16, "inputs untouched")
+
+
+@pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
+@pytest.mark.parametrize("n,count", [(16, 33554432), (7, 25000003)])
+@pytest.mark.parametrize("algname", ["nhr", "nb"])
+def test_nhr_and_nb_int32_full_size_closed_form(gpu_thread, algname, n, count, lowering):
+    """NHR / NB allreduce at benchmark size (16 x 128 MiB) and at a ragged non-power-of-two shape: exact int32
+    sums computed independently by torch; every rank's output identical."""
+    import torch
+    say("full", algname, n, count, lowering)
+    g = torch.Generator(device="cuda")
+    ins = []
+    want = torch.zeros(count, dtype=torch.int32, device="cuda")
+    for r in range(n):
+        g.manual_seed(700 + r)
+        ins.append(torch.randint(-(1 << 20), (1 << 20) + 1, (count,), generator=g, device="cuda", dtype=torch.int32))
+        want += ins[-1]
+    outs = [torch.full((count,), -7, dtype=torch.int32, device="cuda") for _ in range(n)]
+    alg = h.Alg.ALLREDUCE_NHR if algname == "nhr" else h.Alg.ALLREDUCE_NB
+    info = run_plan(gpu_thread, alg, lowering, ins, outs, count, oracle.I32, oracle.SUM)
+    steps = (n - 1).bit_length()
+    if lowering == h.Lowering.FUSED:
+        assert info.launches == 1
+    elif algname == "nhr":      # touching slices are merged: one segment or two per rank, one launch per step
+        assert info.launches == 2 * steps + 1
+    else:                       # NB keeps its slices apart: a step of 16 ranks x 8 slices needs 4 launches of 32 segments
+        assert info.launches >= 2 * steps + 1
+    for r in range(n):
+        assert torch.equal(outs[r], want), "out[%d]" % r
+    del ins, outs, want
+    torch.cuda.empty_cache()
