@@ -56,6 +56,9 @@ WORKLOADS = {
     "nhr_ar_bf16_n8_128MiB": ("nhr", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nb_ar_bf16_n8_128MiB": ("nb", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "local_reduce_rs_bf16_n8_16MiB": ("local_reduce_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the executors' op-base loop around the ring template: user buffers <-> 200 MiB CCL buffers (the default size)
+    "opbase_ring_ar_bf16_n8_128MiB": ("opbase_ring_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "opbase_ring_ar_bf16_n8_512MiB": ("opbase_ring_ar", 8, 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
 
@@ -116,6 +119,10 @@ def main():
            "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE}
     OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
           "min": h.HcommReduceOp.MIN}
+    opbase = alg_name.startswith("opbase_")  # the template inside the op-base loop of its executor
+    if opbase:
+        alg_name = alg_name[len("opbase_"):]
+    ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
     unit = h.DTYPE_SIZE[dt]
     in_place = alg_name == "ring_rs_stage"
@@ -146,6 +153,11 @@ def main():
     in_ptrs = [t.data_ptr() for t in d_in]
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
     scratch_bytes = h.scratch_bytes(alg, n, count, dt)
+    d_ccl = None
+    if opbase:
+        d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
+        if args.lowering == "both":
+            args.lowering = "stepwise"
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
     if alg_name in ("local_reduce", "chunk_mesh", "local_reduce_rs") and args.lowering == "both":
@@ -153,11 +165,17 @@ def main():
     kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
              h.Kernel.COPY: "k_copy"}
 
+    def make_plan(low):
+        if opbase:
+            return h.OpBasePlan(alg, low, in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
+                                [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, scr_ptrs)
+        return h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
+
     lowerings = ["stepwise", "fused"] if args.lowering == "both" else [args.lowering]
     results = {}
     for name in lowerings:
         low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-        plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
+        plan = make_plan(low)
         launches = plan.launches()
         restore()
         for _ in range(args.warmup):
@@ -239,12 +257,21 @@ def main():
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
         host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
-        alg_bytes = oracle.algorithmic_bytes(oalg, n, count, odt)
+        alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
+                     else oracle.algorithmic_bytes(oalg, n, count, odt))
+        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if opbase else None
+
+        def cpu_run(ins, outs):
+            if opbase:
+                oracle.run_opbase(oalg, ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop, scratch=host_scr)
+            else:
+                oracle.run(oalg, ins, outs, count, odt, oop, scratch=host_scr)
+
         passes, cpu_s = 0, 0.0
         while passes < 1 or (cpu_s < 8.0 and passes < 64):
             work_in = [x.copy() for x in host_in]  # every pass starts from the pristine inputs (copy not timed)
             t0 = time.perf_counter()
-            oracle.run(oalg, work_in, host_out, count, odt, oop, scratch=host_scr)
+            cpu_run(work_in, host_out)
             cpu_s += time.perf_counter() - t0
             passes += 1
         host_in = work_in
@@ -253,7 +280,7 @@ def main():
         one_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         one_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         t0 = time.perf_counter()
-        oracle.run(oalg, one_in, one_out, count, odt, oop, scratch=host_scr)
+        cpu_run(one_in, one_out)
         one_s = time.perf_counter() - t0
         del one_in, one_out
         model = "unknown"
@@ -297,7 +324,7 @@ def main():
         verified = True
         for name in lowerings:
             low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
-            plan = h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
+            plan = make_plan(low)
             restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
             stream.synchronize()
@@ -305,6 +332,9 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
+                if opbase:  # what the last chunk left in the CCL buffers
+                    ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
+                    ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
             plan.destroy()
 
@@ -327,7 +357,8 @@ def main():
         "dtype": dtname,
         "data": "synthetic",
         "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": opname,
-                   "algorithm": alg_name, "values": dist, "lowering": best},
+                   "algorithm": alg_name, "values": dist, "lowering": best,
+                   **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

@@ -24,6 +24,7 @@ __all__ = [
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
+    "OpBasePlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
@@ -188,7 +189,7 @@ class CheckReport(C.Structure):
 
 
 class Expect:
-    ALLREDUCE, REDUCE_SCATTER_IN_PLACE, REDUCE_SCATTER_OUT = 0, 1, 2
+    ALLREDUCE, REDUCE_SCATTER_IN_PLACE, REDUCE_SCATTER_OUT, ALLREDUCE_USER, REDUCE_SCATTER_USER = 0, 1, 2, 3, 4
 
 
 _oplist_check = _sig("HcommGfxOpListCheck", _i32, C.POINTER(SchedOp), _u64, _u32, C.c_int, _u64, _u64, _u32,
@@ -346,3 +347,50 @@ class Plan:
             self.destroy()
         except Exception:
             pass
+
+
+# ---- the op-base loop around a template ------------------------------------------------------------------
+
+BUF_USER_IN, BUF_USER_OUT = 3, 4
+_opbase_emit = _sig("HcommGfxOpBaseEmit", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+                    C.POINTER(_u64))
+_opbase_check = _sig("HcommGfxOpBaseCheck", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_opbase_max = _sig("HcommGfxOpBaseMaxCount", _i32, C.c_int, _u32, _u64, C.c_int, C.POINTER(_u64))
+_opbase_plan = _sig("HcommGfxOpBasePlanCreate", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                    C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def opbase_emit(alg, n_ranks, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_opbase_emit(alg, n_ranks, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxOpBaseEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_opbase_emit(alg, n_ranks, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxOpBaseEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def opbase_check(alg, n_ranks, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_opbase_check(alg, n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxOpBaseCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+def opbase_max_count(alg, n_ranks, ccl_bytes, dtype):
+    m = _u64(0)
+    check(_opbase_max(alg, n_ranks, ccl_bytes, dtype, C.byref(m)), "HcommGfxOpBaseMaxCount")
+    return m.value
+
+
+class OpBasePlan(Plan):
+    """HcommGfxOpBasePlanCreate: the chunked loop user buffers -> CCL buffers -> template -> user buffers."""
+
+    def __init__(self, alg, lowering, user_in, user_out, ccl_in, ccl_out, ccl_bytes, count, dtype, op,
+                 scratch_ptrs=None):
+        n = len(user_in)
+        self._keep = [(_vp * n)(*x) if x is not None else None for x in (user_in, user_out, ccl_in, ccl_out, scratch_ptrs)]
+        p = _vp(0)
+        check(_opbase_plan(alg, lowering, n, self._keep[0], self._keep[1], self._keep[2], self._keep[3], self._keep[4],
+                           ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxOpBasePlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info

@@ -55,19 +55,19 @@ static int plan_push(const HgLaunch* l, void* ctx)
     return HCCL_SUCCESS;
 }
 
-static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, void* const* out,
-                          void* const* scratch, int dtype, int op)
+/* bufs[role][rank]: the buffer behind each role an op list may name (HCOMM_GFX_NUM_BUFS roles) */
+static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
+                     int op)
 {
-    void* const* bufs[3] = {in, out, scratch};
-    HgOp* ops = (HgOp*)calloc(ol->n ? ol->n : 1, sizeof(HgOp));
+    HgOp* ops = (HgOp*)calloc(n ? n : 1, sizeof(HgOp));
     if (!ops) return HCCL_E_MEMORY;
-    for (uint64_t i = 0; i < ol->n; ++i) {
-        const HcommGfxSchedOp* s = &ol->ops[i];
+    for (uint64_t i = 0; i < n; ++i) {
+        const HcommGfxSchedOp* s = &list[i];
         HgOp* o = &ops[i];
         o->is_reduce = (uint8_t)s->kind;
         o->dtype = s->kind ? (uint8_t)dtype : 255;
         o->op = s->kind ? (uint8_t)op : 255;
-        if (s->dstBuf > 2 || s->srcBuf > 2 || !bufs[s->dstBuf] || !bufs[s->srcBuf]) {
+        if (s->dstBuf >= HCOMM_GFX_NUM_BUFS || s->srcBuf >= HCOMM_GFX_NUM_BUFS || !bufs[s->dstBuf] || !bufs[s->srcBuf]) {
             free(ops);
             return HCCL_E_PTR;
         }
@@ -75,9 +75,16 @@ static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, 
         o->src = (const char*)bufs[s->srcBuf][s->srcRank] + s->srcOff;
         o->bytes = s->bytes;
     }
-    int rc = hg_coalesce(ops, ol->n, plan_push, p);
+    int rc = hg_coalesce(ops, n, plan_push, p);
     free(ops);
     return rc;
+}
+
+static int lower_stepwise(HcommGfxPlan* p, const HgOpList* ol, void* const* in, void* const* out,
+                          void* const* scratch, int dtype, int op)
+{
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {in, out, scratch, NULL, NULL};
+    return lower_ops(p, ol->ops, ol->n, bufs, dtype, op);
 }
 
 static HgLaunch* new_fold(int dtype, int op, int acc_is_dst, uint32_t n, void* const* in, void* const* out)
@@ -373,6 +380,83 @@ int32_t HcommGfxPlanCreateEx(
         rc = lower_stepwise(p, &ol, in, out, scratch, (int)dataType, (int)reduceOp);
     else
         rc = lower_fused(p, (int)alg, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
+    hg_oplist_free(&ol);
+    if (rc != HCCL_SUCCESS) {
+        HcommGfxPlanDestroy(p);
+        return rc;
+    }
+    p->info.launches = p->nlaunch;
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
+static int check_bufs(void* const* b, uint32_t n)
+{
+    if (!b) return HCCL_E_PTR;
+    for (uint32_t r = 0; r < n; ++r) {
+        if (!b[r]) return HCCL_E_PTR;
+        if (((uintptr_t)b[r]) & 127u) return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxOpBasePlanCreate(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* userIn, void* const* userOut,
+    void* const* cclIn, void* const* cclOut, void* const* scratch, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!userIn || !userOut || !cclIn || !cclOut) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    if (lowering != HCOMM_GFX_LOWER_STEPWISE && lowering != HCOMM_GFX_LOWER_FUSED) return HCCL_E_PARA;
+    for (uint32_t r = 0; r < nRanks; ++r)
+        if (!userIn[r] || !userOut[r]) return HCCL_E_PTR;
+    int rc = check_bufs(cclIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclOut, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t unit = HcommGfxDataTypeSize(dataType);
+    const uint64_t maxc = hg_opbase_max_count((int)alg, nRanks, cclBytes, unit);
+    const uint64_t chunk = count < maxc ? count : maxc;
+    if (nRanks > 1 && chunk > 0 && hg_scratch_bytes((int)alg, nRanks, chunk, (int)dataType) > 0) {
+        rc = check_bufs(scratch, nRanks);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    HgOpList ol;
+    rc = hg_schedule_opbase(&ol, (int)alg, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
+    if (!p) {
+        hg_oplist_free(&ol);
+        return HCCL_E_MEMORY;
+    }
+    p->magic = HG_PLAN_MAGIC;
+    p->graph_wanted = use_graph();
+    p->info.steps = ol.steps;
+    for (uint64_t i = 0; i < ol.n; ++i) p->info.algorithmicBytes += ol.ops[i].bytes * (ol.ops[i].kind ? 3u : 2u);
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {cclIn, cclOut, scratch, userIn, userOut};
+    if (lowering == HCOMM_GFX_LOWER_STEPWISE) {
+        rc = lower_ops(p, ol.ops, ol.n, bufs, (int)dataType, (int)reduceOp);
+    } else {
+        /* per chunk: the copies in, the template part fused as a stand-alone plan would be, the copies out.  The
+         * list is ordered by step, and inside a chunk every op that names a user buffer is one of its copies. */
+        uint64_t i = 0, done = 0;
+        while (i < ol.n && rc == HCCL_SUCCESS) {
+            uint64_t j = i;
+            while (j < ol.n && ol.ops[j].srcBuf == HCOMM_GFX_BUF_USER_IN) ++j;
+            rc = lower_ops(p, &ol.ops[i], j - i, bufs, (int)dataType, (int)reduceOp);
+            uint64_t k = j;
+            while (k < ol.n && ol.ops[k].dstBuf != HCOMM_GFX_BUF_USER_OUT) ++k;
+            const uint64_t cur = count - done > maxc ? maxc : count - done;
+            if (rc == HCCL_SUCCESS) rc = lower_fused(p, (int)alg, nRanks, cclIn, cclOut, cur, cur, (int)dataType, (int)reduceOp);
+            uint64_t m = k;
+            while (m < ol.n && ol.ops[m].dstBuf == HCOMM_GFX_BUF_USER_OUT) ++m;
+            if (rc == HCCL_SUCCESS) rc = lower_ops(p, &ol.ops[k], m - k, bufs, (int)dataType, (int)reduceOp);
+            done += cur;
+            i = m;
+        }
+    }
     hg_oplist_free(&ol);
     if (rc != HCCL_SUCCESS) {
         HcommGfxPlanDestroy(p);

@@ -685,3 +685,98 @@ int32_t HcommGfxScheduleEmitStrided(
     hg_oplist_free(&l);
     return HCCL_SUCCESS;
 }
+
+/* ---- the op-base loop around a template (the templates' immediate caller) ------------------------------------ */
+
+static int is_scatter_alg(int alg)
+{
+    return alg == HCOMM_GFX_ALG_REDUCE_SCATTER_MESH || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE ||
+           alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB ||
+           alg == HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE;
+}
+
+uint64_t hg_opbase_max_count(int alg, uint32_t n, uint64_t ccl_bytes, uint32_t unit)
+{
+    if (unit == 0 || n == 0) return 0;
+    /* allreduce: CCLBuffSize / unitSize (coll_all_reduce_executor.cc:129-138); reduce-scatter: the input buffer
+     * holds N slices, each a multiple of 128 bytes (coll_reduce_scatter_executor.cc:124-134) */
+    if (!is_scatter_alg(alg)) return ccl_bytes / unit;
+    return ccl_bytes / n / HG_SLICE_ALIGN * HG_SLICE_ALIGN / unit;
+}
+
+/* One pass per chunk of at most maxCountPerLoop elements: user input -> CCL input, the template on the CCL
+ * buffers, CCL output -> user output.  Paths relative to src/legacy/ascend910/algorithm/impl/coll_executor/:
+ * allreduce coll_all_reduce/coll_all_reduce_executor.cc:199-262 (loop), :304-309 and :326-331 (copies);
+ * reduce-scatter coll_reduce_scatter/coll_reduce_scatter_executor.cc:149-220 (loop), :257-275 (one copy per input
+ * slice, or a single copy when one pass takes everything, :616-620), :292-297 (copy out). */
+int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) return HCCL_E_PARA;
+    const int scatter = is_scatter_alg(alg);
+    const uint64_t maxc = hg_opbase_max_count(alg, n, ccl_bytes, unit);
+    if (maxc == 0) return scatter ? HCCL_E_INTERNAL : HCCL_E_PARA; /* :213-218 / :163-165 */
+    uint32_t step = 0;
+    int rc = HCCL_SUCCESS;
+    for (uint64_t done = 0; done < count && rc == HCCL_SUCCESS;) {
+        const uint64_t cur = count - done > maxc ? maxc : count - done;
+        const uint64_t cur_bytes = cur * unit, off = done * unit;
+        for (uint32_t r = 0; r < n && rc == HCCL_SUCCESS; ++r) {
+            if (!scatter) {
+                rc = push(l, step, COPY, r, IN, 0, r, HCOMM_GFX_BUF_USER_IN, off, cur_bytes);
+            } else if (cur == count) {
+                rc = push(l, step, COPY, r, IN, 0, r, HCOMM_GFX_BUF_USER_IN, 0, count * unit * n);
+            } else {
+                for (uint32_t i = 0; i < n && rc == HCCL_SUCCESS; ++i)
+                    rc = push(l, step, COPY, r, IN, cur_bytes * i, r, HCOMM_GFX_BUF_USER_IN, count * unit * i + off, cur_bytes);
+            }
+        }
+        ++step;
+        HgOpList sub;
+        if (rc == HCCL_SUCCESS) rc = hg_schedule(&sub, alg, n, cur, cur, dtype);
+        if (rc != HCCL_SUCCESS) break;
+        uint32_t used = 0; /* steps of the template that do anything */
+        for (uint64_t i = 0; i < sub.n && rc == HCCL_SUCCESS; ++i) {
+            const HcommGfxSchedOp* o = &sub.ops[i];
+            if (o->step + 1 > used) used = o->step + 1;
+            rc = push(l, step + o->step, o->kind, o->rank, o->dstBuf, o->dstOff, o->srcRank, o->srcBuf, o->srcOff, o->bytes);
+        }
+        hg_oplist_free(&sub);
+        step += used;
+        for (uint32_t r = 0; r < n && rc == HCCL_SUCCESS; ++r)
+            rc = push(l, step, COPY, r, HCOMM_GFX_BUF_USER_OUT, off, r, OUT, 0, cur_bytes);
+        ++step;
+        done += cur;
+    }
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOpBaseEmit(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_opbase(&l, (int)alg, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxOpBaseMaxCount(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t cclBytes, HcommDataType dataType,
+                               uint64_t* maxCountPerLoop)
+{
+    if (!maxCountPerLoop) return HCCL_E_PTR;
+    const uint32_t unit = HcommGfxDataTypeSize(dataType);
+    if (unit == 0 || nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    *maxCountPerLoop = hg_opbase_max_count((int)alg, nRanks, cclBytes, unit);
+    return HCCL_SUCCESS;
+}

@@ -15,6 +15,10 @@ typedef struct {
 /* Fill `l` with the op list of `alg`; the caller releases it with hg_oplist_free. */
 /* stride: elements between consecutive ranks' slices in the input of the scatter algorithms (0 = count). */
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype);
+/* The op-base loop around alg: chunks of at most hg_opbase_max_count elements, each copied from the user input
+ * into the CCL input buffer, run through the template, and copied from the CCL output to the user output. */
+int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
+uint64_t hg_opbase_max_count(int alg, uint32_t n, uint64_t ccl_bytes, uint32_t unit);
 void hg_oplist_free(HgOpList* l);
 /* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);

@@ -464,13 +464,20 @@ typedef struct {
     uint32_t step;    /* schedule step (ranks act in parallel within a step) */
     uint32_t kind;    /* 0 = copy, 1 = reduce */
     uint32_t rank;    /* rank that executes the operation (owner of dst) */
-    uint32_t dstBuf;  /* 0 = in[rank], 1 = out[rank], 2 = scratch[rank] (communication buffer) */
+    uint32_t dstBuf;  /* 0 = in[rank], 1 = out[rank], 2 = scratch[rank] (communication buffer); op-base lists
+                         also use HCOMM_GFX_BUF_USER_IN / HCOMM_GFX_BUF_USER_OUT */
     uint32_t srcRank; /* rank whose buffer is read */
-    uint32_t srcBuf;  /* 0 = in[srcRank], 1 = out[srcRank], 2 = scratch[srcRank] */
+    uint32_t srcBuf;  /* as dstBuf, of srcRank */
     uint64_t dstOff;  /* bytes */
     uint64_t srcOff;  /* bytes */
     uint64_t bytes;
 } HcommGfxSchedOp;
+
+/* Buffer roles of an op-base op list: the template runs on the CCL buffers (roles 0, 1, 2), the loop around it
+   moves chunks between them and the caller's own buffers. */
+#define HCOMM_GFX_BUF_USER_IN 3u
+#define HCOMM_GFX_BUF_USER_OUT 4u
+#define HCOMM_GFX_NUM_BUFS 5u
 
 /*
  * Emit the op list of an algorithm without any pointers.  Writes up to cap records; *n receives the total.
@@ -496,7 +503,10 @@ int32_t HcommGfxScheduleEmitStrided(
 typedef enum {
     HCOMM_GFX_EXPECT_ALLREDUCE = 0,               /* out[r][0, count*unit) for every r */
     HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE = 1, /* in[r][slice r], slices from HcommGfxCalcSlices(count, unit, n) */
-    HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT = 2       /* out[r][0, count*unit) = sum of in[k][r*stride*unit + ...] */
+    HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT = 2,      /* out[r][0, count*unit) = sum of in[k][r*stride*unit + ...] */
+    /* op-base lists: the data starts in the user inputs and the result is looked for in the user outputs */
+    HCOMM_GFX_EXPECT_ALLREDUCE_USER = 3,
+    HCOMM_GFX_EXPECT_REDUCE_SCATTER_USER = 4
 } HcommGfxExpectation;
 
 typedef struct {
@@ -512,6 +522,38 @@ int32_t HcommGfxOpListCheck(
 /* Generate the op list of alg and check it against the expectation that belongs to the algorithm. */
 int32_t HcommGfxScheduleCheck(
     HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t strideCount, HcommDataType dataType,
+    HcommGfxCheckReport* report);
+
+/*
+ * The op-base loop around a template - what the reference's executors do with a caller's buffers when the collective
+ * runs through the communicator's CCL buffers (src/legacy/ascend910/algorithm/impl/coll_executor/
+ * coll_all_reduce/coll_all_reduce_executor.cc:199-339, coll_reduce_scatter/coll_reduce_scatter_executor.cc:149-306):
+ * the message is cut into chunks of at most maxCountPerLoop elements (allreduce: cclBytes / unit; reduce-scatter:
+ * cclBytes / N rounded down to 128 bytes, / unit), and every chunk is copied user input -> CCL input, run through
+ * the template on the CCL buffers, and copied CCL output -> user output.  A reduce-scatter copies one piece per
+ * input slice (a single copy when one chunk takes the whole message).  No counterpart for the in-place ring stage.
+ *
+ * userIn / userOut: the caller's buffers (allreduce: count elements each; reduce-scatter: N * count in, count out).
+ * cclIn / cclOut: cclBytes each, 128-byte aligned.  scratch: as HcommGfxPlanCreateEx, sized for
+ * min(count, maxCountPerLoop) elements.  FUSED lowers the template part of every chunk as HcommGfxPlanCreate would.
+ */
+int32_t HcommGfxOpBasePlanCreate(
+    HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* userIn, void* const* userOut,
+    void* const* cclIn, void* const* cclOut, void* const* scratch, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+
+/* Elements per chunk of the op-base loop. */
+int32_t HcommGfxOpBaseMaxCount(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t cclBytes, HcommDataType dataType,
+                               uint64_t* maxCountPerLoop);
+
+/* The op list HcommGfxOpBasePlanCreate replays (buffer roles 0-2 are the CCL buffers, 3 and 4 the caller's). */
+int32_t HcommGfxOpBaseEmit(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+
+/* Generate the op-base op list and check it (HCOMM_GFX_EXPECT_ALLREDUCE_USER / _REDUCE_SCATTER_USER). */
+int32_t HcommGfxOpBaseCheck(
+    HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType,
     HcommGfxCheckReport* report);
 
 /* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */

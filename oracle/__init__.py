@@ -84,6 +84,14 @@ def lib():
         L.orc_nhr_slice_map.argtypes = [C.c_uint32, C.POINTER(C.c_uint32)]
         L.orc_rs_local_reduce_scratch_bytes.restype = C.c_uint64
         L.orc_rs_local_reduce_scratch_bytes.argtypes = [C.c_uint32, C.c_uint64, C.c_int]
+        L.orc_trace_opbase.restype = C.c_int64
+        L.orc_trace_opbase.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
+        L.orc_run_opbase.restype = C.c_int
+        L.orc_run_opbase.argtypes = [C.c_int, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
+        L.orc_opbase_max_count.restype = C.c_uint64
+        L.orc_opbase_max_count.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int]
+        L.orc_algorithmic_bytes_opbase.restype = C.c_int64
+        L.orc_algorithmic_bytes_opbase.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int]
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run.restype = C.c_int
@@ -213,3 +221,36 @@ def run(alg, ins, outs, count, dtype, op, stride=0, scratch=None):
 
 def algorithmic_bytes(alg, n, count, dtype):
     return lib().orc_algorithmic_bytes(alg, n, count, dtype)
+
+
+# ---- the op-base loop (user buffers -> CCL buffers -> template -> user buffers) ---------------------------
+
+def opbase_max_count(alg, n, ccl_bytes, dtype):
+    return lib().orc_opbase_max_count(alg, n, ccl_bytes, dtype)
+
+
+def trace_opbase(alg, n, count, ccl_bytes, dtype):
+    total = lib().orc_trace_opbase(alg, n, count, ccl_bytes, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_opbase rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_opbase(alg, n, count, ccl_bytes, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_opbase(alg, user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype, op, scratch=None):
+    """Execute the op-base loop on lists of numpy arrays (one per rank and role)."""
+    n = len(user_in)
+    arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in lst]) for lst in (user_in, user_out, ccl_in, ccl_out)]
+    sc = (C.c_void_p * n)(*[x.ctypes.data for x in scratch]) if scratch is not None else None
+    lib().orc_set_scratch(sc)
+    try:
+        rc = lib().orc_run_opbase(alg, n, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
+    finally:
+        lib().orc_set_scratch(None)
+    if rc:
+        raise ValueError("orc_run_opbase rc=%d" % rc)
+
+
+def algorithmic_bytes_opbase(alg, n, count, ccl_bytes, dtype):
+    return lib().orc_algorithmic_bytes_opbase(alg, n, count, ccl_bytes, dtype)

@@ -319,6 +319,8 @@ typedef struct {
     int oom;
 } OrcTrace;
 
+static uint32_t g_step_base = 0; /* added to every emitted step: where the current chunk of an op-base loop starts */
+
 static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint32_t dst_buf, uint64_t dst_off,
                  uint32_t src_rank, uint32_t src_buf, uint64_t src_off, uint64_t bytes)
 {
@@ -334,7 +336,7 @@ static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint3
         t->cap = cap;
     }
     OrcOp* o = &t->ops[t->n++];
-    o->step = step;
+    o->step = g_step_base + step;
     o->kind = kind;
     o->rank = rank;
     o->dst_buf = dst_buf;
@@ -345,7 +347,7 @@ static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint3
     o->bytes = bytes;
 }
 
-enum { B_IN = 0, B_OUT = 1, B_SCR = 2, K_COPY = 0, K_REDUCE = 1 };
+enum { B_IN = 0, B_OUT = 1, B_SCR = 2, B_UIN = 3, B_UOUT = 4, K_COPY = 0, K_REDUCE = 1 };
 
 /* ReduceScatterRing::RunReduceScatter for one rank, tpl/temp_reduce_scatter/reduce_scatter_ring.cc:182-312.
  * `out_sl` NULL: the allreduce case, where the template's output memory IS the input memory
@@ -1015,6 +1017,31 @@ static int cmp_ops(const void* a, const void* b)
     return 0;
 }
 
+/* lock step: order by step, then by the rank that owns the destination; emission order is kept among equals */
+static int sort_trace(OrcTrace* t)
+{
+    if (t->n > 1) {
+        OrcOp* tmp = (OrcOp*)malloc(t->n * sizeof(OrcOp));
+        if (!tmp) {
+            free(t->ops);
+            return -2;
+        }
+        for (uint64_t width = 1; width < t->n; width *= 2) { /* bottom-up merge sort: stable */
+            for (uint64_t lo = 0; lo < t->n; lo += 2 * width) {
+                const uint64_t mid = lo + width < t->n ? lo + width : t->n;
+                const uint64_t hi = lo + 2 * width < t->n ? lo + 2 * width : t->n;
+                uint64_t a = lo, b = mid, k = lo;
+                while (a < mid && b < hi) tmp[k++] = (cmp_ops(&t->ops[b], &t->ops[a]) < 0) ? t->ops[b++] : t->ops[a++];
+                while (a < mid) tmp[k++] = t->ops[a++];
+                while (b < hi) tmp[k++] = t->ops[b++];
+            }
+            memcpy(t->ops, tmp, t->n * sizeof(OrcOp));
+        }
+        free(tmp);
+    }
+    return 0;
+}
+
 static uint64_t g_stride = 0; /* elements between input slices of the scatter algorithms; 0 = dense */
 
 /* Applies to the next orc_trace / orc_run / orc_algorithmic_bytes calls (scatter algorithms only). */
@@ -1061,27 +1088,7 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
         free(t->ops);
         return -2;
     }
-    /* lock step: order by step, then by the rank that owns the destination; emission order is kept among equals */
-    if (t->n > 1) {
-        OrcOp* tmp = (OrcOp*)malloc(t->n * sizeof(OrcOp));
-        if (!tmp) {
-            free(t->ops);
-            return -2;
-        }
-        for (uint64_t width = 1; width < t->n; width *= 2) { /* bottom-up merge sort: stable */
-            for (uint64_t lo = 0; lo < t->n; lo += 2 * width) {
-                const uint64_t mid = lo + width < t->n ? lo + width : t->n;
-                const uint64_t hi = lo + 2 * width < t->n ? lo + 2 * width : t->n;
-                uint64_t a = lo, b = mid, k = lo;
-                while (a < mid && b < hi) tmp[k++] = (cmp_ops(&t->ops[b], &t->ops[a]) < 0) ? t->ops[b++] : t->ops[a++];
-                while (a < mid) tmp[k++] = t->ops[a++];
-                while (b < hi) tmp[k++] = t->ops[b++];
-            }
-            memcpy(t->ops, tmp, t->n * sizeof(OrcOp));
-        }
-        free(tmp);
-    }
-    return 0;
+    return sort_trace(t);
 }
 
 /* Write the lock-step op list (ordered by step, then rank).  Returns the total number of ops, or < 0. */
@@ -1110,52 +1117,207 @@ static void* const* g_scratch = NULL; /* per-rank communication buffers for the 
 
 void orc_set_scratch(void* const* scratch) { g_scratch = scratch; }
 
-#define BUFPTR(buf, rank) ((buf) == B_SCR ? g_scratch[rank] : ((buf) ? out[rank] : in[rank]))
+/* Execute a lock-step op list on host memory; bufs[role][rank], roles B_IN .. B_UOUT.  Refuses a step in which
+ * one operation writes what another reads or writes (test/st/algorithm/README_en.md:202-231). */
+static int exec_trace(OrcTrace* t, void* const* const* bufs, int dtype, int op)
+{
+#define BUFPTR(buf, rank) (bufs[buf][rank])
+    for (uint64_t q = 0; q < t->n; q++)
+        if (!bufs[t->ops[q].dst_buf] || !bufs[t->ops[q].src_buf]) return -1;
+    const uint32_t unit = orc_dtype_size(dtype);
+    uint64_t i = 0;
+    while (i < t->n) {
+        uint64_t j = i;
+        while (j < t->n && t->ops[j].step == t->ops[i].step) j++;
+        for (uint64_t a = i; a < j; a++) {
+            const OrcOp* x = &t->ops[a];
+            const uintptr_t xd = (uintptr_t)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
+            for (uint64_t b = i; b < j; b++) {
+                if (a == b) continue;
+                const OrcOp* y = &t->ops[b];
+                const uintptr_t yd = (uintptr_t)BUFPTR(y->dst_buf, y->rank) + y->dst_off;
+                const uintptr_t ys = (uintptr_t)BUFPTR(y->src_buf, y->src_rank) + y->src_off;
+                if (ranges_overlap(xd, x->bytes, yd, y->bytes) || ranges_overlap(xd, x->bytes, ys, y->bytes)) return -3;
+            }
+        }
+        for (uint64_t a = i; a < j; a++) {
+            const OrcOp* x = &t->ops[a];
+            char* d = (char*)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
+            const char* s = (const char*)BUFPTR(x->src_buf, x->src_rank) + x->src_off;
+            if (x->kind == K_COPY)
+                orc_copy(d, s, x->bytes);
+            else if (orc_reduce(d, s, x->bytes / unit, dtype, op) != 0)
+                return -1;
+        }
+        i = j;
+    }
+    return 0;
+#undef BUFPTR
+}
 
 int orc_run(int alg, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype, int op)
 {
     OrcTrace t;
     int rc = build_trace(&t, alg, n, count, dtype);
     if (rc) return rc;
-    for (uint64_t q = 0; q < t.n; q++)
-        if ((t.ops[q].dst_buf == B_SCR || t.ops[q].src_buf == B_SCR) && !g_scratch) {
-            free(t.ops);
-            return -1;
-        }
+    void* const* bufs[5] = {in, out, g_scratch, NULL, NULL};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+/* ---- the op-base loop of the executors, per rank ------------------------------------------------------------ */
+
+static int is_scatter(int alg)
+{
+    return alg == ORC_ALG_RS_MESH || alg == ORC_ALG_RS_RING_STANDALONE || alg == ORC_ALG_RS_NHR || alg == ORC_ALG_RS_NB ||
+           alg == ORC_ALG_RS_LOCAL_REDUCE;
+}
+
+/* "exec/" abbreviates src/legacy/ascend910/algorithm/impl/coll_executor/.
+ * CollAllReduceExecutor::CalcLoopMaxCount, exec/coll_all_reduce/coll_all_reduce_executor.cc:129-138;
+ * CollReduceScatterExecutor::CalcLoopMaxCount, exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:124-134 */
+uint64_t orc_opbase_max_count(int alg, uint32_t n, uint64_t ccl_bytes, int dtype)
+{
     const uint32_t unit = orc_dtype_size(dtype);
-    uint64_t i = 0;
-    while (i < t.n) {
-        uint64_t j = i;
-        while (j < t.n && t.ops[j].step == t.ops[i].step) j++;
-        for (uint64_t a = i; a < j; a++) {
-            const OrcOp* x = &t.ops[a];
-            const uintptr_t xd = (uintptr_t)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
-            for (uint64_t b = i; b < j; b++) {
-                if (a == b) continue;
-                const OrcOp* y = &t.ops[b];
-                const uintptr_t yd = (uintptr_t)BUFPTR(y->dst_buf, y->rank) + y->dst_off;
-                const uintptr_t ys = (uintptr_t)BUFPTR(y->src_buf, y->src_rank) + y->src_off;
-                if (ranges_overlap(xd, x->bytes, yd, y->bytes) || ranges_overlap(xd, x->bytes, ys, y->bytes)) {
-                    free(t.ops);
-                    return -3;
-                }
-            }
-        }
-        for (uint64_t a = i; a < j; a++) {
-            const OrcOp* x = &t.ops[a];
-            char* d = (char*)BUFPTR(x->dst_buf, x->rank) + x->dst_off;
-            const char* s = (const char*)BUFPTR(x->src_buf, x->src_rank) + x->src_off;
-            if (x->kind == K_COPY)
-                orc_copy(d, s, x->bytes);
-            else if (orc_reduce(d, s, x->bytes / unit, dtype, op) != 0) {
-                free(t.ops);
-                return -1;
-            }
-        }
-        i = j;
+    if (unit == 0 || n == 0) return 0;
+    if (!is_scatter(alg)) return ccl_bytes / unit;
+    return ccl_bytes / n / 128u * 128u / unit;
+}
+
+static void run_template(OrcTrace* t, int alg, uint32_t r, uint32_t n, uint64_t count, uint32_t unit)
+{
+    switch (alg) {
+        case ORC_ALG_ALLREDUCE_RING: prog_allreduce_ring(t, r, n, count, unit, 1); break;
+        case ORC_ALG_ALLREDUCE_RHD: prog_allreduce_rhd(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_MESH_ONESHOT: prog_allreduce_mesh_oneshot(t, r, n, count, unit); break;
+        case ORC_ALG_RS_MESH: prog_rs_mesh(t, r, n, count, count, unit); break;
+        case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, count, unit); break;
+        case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_CHUNK_MESH: prog_allreduce_chunk_mesh(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_LOCAL_REDUCE: prog_allreduce_local_reduce(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_NHR: prog_allreduce_nhr(t, r, n, count, unit); break;
+        case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, count, unit); break;
+        case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
+        case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, count, unit); break;
+        case ORC_ALG_RS_LOCAL_REDUCE: prog_rs_local_reduce(t, r, n, count, unit); break;
+        default: break;
     }
+}
+
+/* Steps of the template that do anything for `count` elements (the ranks run in lock step, so the copy back to
+ * the user buffer of a chunk sits one step after the template's last one on every rank). */
+static int template_steps(int alg, uint32_t n, uint64_t count, int dtype, uint32_t* steps)
+{
+    OrcTrace t;
+    const uint64_t keep = g_stride;
+    const uint32_t keep_base = g_step_base;
+    g_stride = 0;
+    g_step_base = 0;
+    const int rc = build_trace(&t, alg, n, count, dtype);
+    g_stride = keep;
+    g_step_base = keep_base;
+    if (rc) return rc;
+    *steps = t.n ? t.ops[t.n - 1].step + 1 : 0;
     free(t.ops);
     return 0;
+}
+
+/* CollAllReduceExecutor::RunLoop + RunLoopInner for one rank (exec/coll_all_reduce/coll_all_reduce_executor.cc:
+ * 199-262, 264-339) and CollReduceScatterExecutor::RunLoop + RunLoopInner
+ * (exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:149-220, 222-306), both in the buffer-copy mode
+ * (DMAReduceFlag_ false): B_IN / B_OUT are the CCL buffers the template runs on. */
+static int prog_opbase(OrcTrace* t, int alg, uint32_t rank, uint32_t n, uint64_t total_count, uint64_t max_count,
+                       int dtype)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    const int scatter = is_scatter(alg);
+    uint64_t cur_in = 0, cur_out = 0;             /* curInputPtr, curOutputPtr as offsets */
+    uint64_t cur_count = 0, input_offset = 0, output_offset = 0;
+    uint32_t step = 0;
+    for (uint64_t count_left = total_count; count_left > 0; count_left -= cur_count) {
+        cur_in += input_offset;                   /* :236-237 / :172-173 */
+        cur_out += output_offset;
+        cur_count = (count_left > max_count) ? max_count : count_left;
+        const uint64_t cur_size = cur_count * unit;
+        g_step_base = step;
+        if (!scatter) {
+            emit(t, 0, K_COPY, rank, B_IN, 0, rank, B_UIN, cur_in, cur_size);              /* :304-309 */
+        } else if (total_count == cur_count) {                                              /* preloadCopyOpt, :616-620 */
+            emit(t, 0, K_COPY, rank, B_IN, 0, rank, B_UIN, cur_in, total_count * unit * n); /* :260-265 */
+        } else {
+            for (uint32_t i = 0; i < n; i++)                                                /* :267-273 */
+                emit(t, 0, K_COPY, rank, B_IN, cur_size * i, rank, B_UIN, cur_in + total_count * unit * i, cur_size);
+        }
+        uint32_t used = 0;
+        const int rc = template_steps(alg, n, cur_count, dtype, &used);
+        if (rc) {
+            g_step_base = 0;
+            return rc;
+        }
+        g_step_base = step + 1;
+        run_template(t, alg, rank, n, cur_count, unit);                                     /* KernelRun */
+        g_step_base = step + 1 + used;
+        emit(t, 0, K_COPY, rank, B_UOUT, cur_out, rank, B_OUT, 0, cur_size);                /* :326-331 / :292-297 */
+        g_step_base = 0;
+        step += used + 2;
+        input_offset = cur_size;
+        output_offset = cur_size;
+    }
+    return 0;
+}
+
+static int build_trace_opbase(OrcTrace* t, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (n == 0 || n > ORC_MAX_RANKS || unit == 0 || alg == ORC_ALG_RS_RING_STAGE) return -1;
+    const uint64_t max_count = orc_opbase_max_count(alg, n, ccl_bytes, dtype);
+    if (max_count == 0) return -1; /* :213-218 / :163-165 */
+    if (alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE && (n & (n - 1))) return -1;
+    for (uint32_t r = 0; r < n; r++) {
+        const int rc = prog_opbase(t, alg, r, n, count, max_count, dtype);
+        if (rc || t->oom) {
+            free(t->ops);
+            return rc ? rc : -2;
+        }
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_opbase(int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_opbase(&t, alg, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_opbase(int alg, uint32_t n, void* const* user_in, void* const* user_out, void* const* ccl_in,
+                   void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_opbase(&t, alg, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, g_scratch, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+int64_t orc_algorithmic_bytes_opbase(int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    OrcTrace t;
+    int rc = build_trace_opbase(&t, alg, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    int64_t total = 0;
+    for (uint64_t i = 0; i < t.n; i++) total += (int64_t)t.ops[i].bytes * (t.ops[i].kind ? 3 : 2);
+    free(t.ops);
+    return total;
 }
 
 /* Bytes moved by the two-input model: 3b per reduce, 2b per copy. */
