@@ -14,21 +14,28 @@
 #include "hg_host.h"
 
 static uint64_t g_grid_cap = 0;
+static int g_grid_forced = 0;
 static uint64_t g_small_bytes = 0;
 
-uint64_t hg_grid_blocks(uint64_t total_tiles)
+uint64_t hg_grid_blocks(uint64_t total_tiles, int capped)
 {
     if (g_grid_cap == 0) {
         const char* e = getenv("HCOMM_GFX_GRID_CAP");
-        uint64_t cap = e ? strtoull(e, NULL, 10) : 0;
-        if (cap == 0) {
-            int cus = hg_rt_num_cus();
-            if (cus <= 0) cus = 256;
-            cap = (uint64_t)cus * 32u; /* measured: a grid of about one 16 KiB tile per workgroup streams best */
-        }
-        g_grid_cap = cap;
+        g_grid_cap = e ? strtoull(e, NULL, 10) : 0;
+        if (g_grid_cap == 0) g_grid_cap = UINT64_MAX; /* not set */
+        else g_grid_forced = 1;
     }
-    return total_tiles < g_grid_cap ? total_tiles : g_grid_cap;
+    if (g_grid_forced) return total_tiles < g_grid_cap ? total_tiles : g_grid_cap; /* experiments: every kernel */
+    /* Measured over the benchmark configurations: one tile per workgroup, however many that makes, streams best for
+     * the copy and the k-way fold kernels (a 2 GiB copy: 5.84 against 5.38 TB/s with the grid held at 32 workgroups
+     * per CU; the fused 16-rank tree: 0.95 against 1.05 ms).  The two-input reduce is the exception: on the ragged
+     * 7-rank reduce-scatter it loses 6 % without the limit, so it keeps it (its 128 MiB ring step has exactly
+     * 32 workgroups per CU worth of tiles either way). */
+    if (!capped) return total_tiles;
+    int cus = hg_rt_num_cus();
+    if (cus <= 0) cus = 256;
+    const uint64_t cap = (uint64_t)cus * 32u;
+    return total_tiles < cap ? total_tiles : cap;
 }
 
 static uint64_t tiles_of(uint64_t bytes) { return (bytes + HG_TILE_BYTES - 1) / HG_TILE_BYTES; }
@@ -52,7 +59,7 @@ void hg_finish_seg2(HgLaunch* l)
     l->nseg = t->nseg;
     l->bytes = bytes;
     l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
-    l->blocks = hg_grid_blocks(tiles);
+    l->blocks = hg_grid_blocks(tiles, l->kind != HCOMM_GFX_KERNEL_COPY);
 }
 
 void hg_finish_fold(HgLaunch* l)
@@ -94,7 +101,7 @@ void hg_finish_fold(HgLaunch* l)
              * and the root to one output or to all of them */
             const uint64_t n = (uint64_t)t->nranks + t->nranks / 2 + (t->out_mode == 1u ? 1u : t->nout);
             l->moved_bytes = n * bytes;
-            l->blocks = hg_grid_blocks(tiles);
+            l->blocks = hg_grid_blocks(tiles, 0);
             return;
         }
         for (uint32_t s = 0; s < t->nseg; ++s) {
@@ -104,7 +111,7 @@ void hg_finish_fold(HgLaunch* l)
             moved += n * t->bytes[s];
         }
         l->moved_bytes = moved;
-        l->blocks = hg_grid_blocks(tiles);
+        l->blocks = hg_grid_blocks(tiles, 0);
         return;
     } else {
         if (t->store_partials) per += t->k - 1;
@@ -113,7 +120,7 @@ void hg_finish_fold(HgLaunch* l)
         if (t->out_mode == 2) per += t->nranks;
     }
     l->moved_bytes = bytes * per;
-    l->blocks = hg_grid_blocks(tiles);
+    l->blocks = hg_grid_blocks(tiles, 0);
 }
 
 static int overlaps(const void* a, uint64_t an, const void* b, uint64_t bn)

@@ -67,7 +67,7 @@ typedef struct {
 } HgFoldTable;
 
 /* Launch geometry decided on the host so that recorder threads can report it without a GPU. */
-uint64_t hg_grid_blocks(uint64_t total_tiles);
+uint64_t hg_grid_blocks(uint64_t total_tiles, int capped);
 
 /* Launchers.  stream is a hipStream_t.  Return a HcclResult-compatible code. */
 int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks);
