@@ -163,6 +163,9 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
 #ifndef HG_STREAM_COPY_BYTES
 #define HG_STREAM_COPY_BYTES (256ull << 20) /* the 256 MB memory-side cache */
 #endif
+#ifndef HG_STREAM_REDUCE_BYTES
+#define HG_STREAM_REDUCE_BYTES (256ull << 20)
+#endif
 #ifndef HG_XCD_REMAP_COPY
 #define HG_XCD_REMAP_COPY 1
 #endif
@@ -227,7 +230,7 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 
 // ---- batched dst = dst (op) src -----------------------------------------------------------------
 
-template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(const HgSeg2Table tab)
+template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(const HgSeg2Table tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
@@ -246,12 +249,12 @@ template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<HG_NT_ST>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM || HG_NT_ST>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv<HG_NT_ST>(d, v, vec_op<DT, OP>(ldv<HG_NT_LD_DST>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+                if (v < nvec) stv<STREAM || HG_NT_ST>(d, v, vec_op<DT, OP>(ldv<HG_NT_LD_DST>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -583,16 +586,24 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
 
 int rc(hipError_t e) { return e == hipSuccess ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
 
-template <int DT> int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
+template <int DT, bool STREAM> int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
 {
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_reduce2<DT, OP_PROD>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_reduce2<DT, OP_MAX>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_reduce2<DT, OP_MIN>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_reduce2<DT, OP_PROD, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_reduce2<DT, OP_MAX, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_reduce2<DT, OP_MIN, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
+}
+
+template <int DT> int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
+{
+    uint64_t bytes = 0; /* what the launch writes */
+    for (uint32_t s = 0; s < tab->nseg; ++s) bytes += tab->bytes[s];
+    if (bytes > HG_STREAM_REDUCE_BYTES) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks);
+    return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks);
 }
 
 template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
