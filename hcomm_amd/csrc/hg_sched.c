@@ -629,6 +629,28 @@ static int sched_rs_local_reduce(HgOpList* l, uint32_t n, uint64_t count, uint32
     return HCCL_SUCCESS;
 }
 
+/* AllReduceDoubling (temp_all_reduce/all_reduce_doubling.cc:91-128), power-of-two rank counts only (:81-88): the
+ * whole message every step.  Step s: first every rank refreshes the buffer its partner will read - input -> output
+ * at s = 0 (:105-106), output -> input afterwards (:107-108) - then folds the partner's input (rank XOR 2^s) into its
+ * own output (:113-121).  The two halves of a step are separated by the ack exchange, hence two schedule steps. */
+static int sched_allreduce_doubling(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* :38-41 */
+    if (n & (n - 1)) return HCCL_E_PARA;
+    uint32_t step = 0;
+    for (uint32_t bit = 1; bit < n; bit <<= 1) {
+        for (uint32_t r = 0; r < n; ++r) {
+            if (bit == 1) CHK(push(l, step, COPY, r, OUT, 0, r, IN, 0, total));
+            else CHK(push(l, step, COPY, r, IN, 0, r, OUT, 0, total));
+        }
+        ++step;
+        for (uint32_t r = 0; r < n; ++r) CHK(push(l, step, REDUCE, r, OUT, 0, r ^ bit, IN, 0, total));
+        ++step;
+    }
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
@@ -656,6 +678,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_ALLREDUCE_NB: rc = sched_allreduce_nb(l, n, count, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_NB: rc = sched_rs_nb(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE: rc = sched_rs_local_reduce(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_DOUBLING: rc = sched_allreduce_doubling(l, n, count, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

@@ -355,7 +355,12 @@ typedef enum {
        communication buffer (:218-243), rank d folds the slots and its own copy pairwise in a fixed order into
        out[d][0..count) (:252-304).  Input holds N dense slices of count elements; needs the third buffer
        (HcommGfxScratchBytes).  Step-wise lowering only. */
-    HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE = 13
+    HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE = 13,
+    /* AllReduceDoubling (recursive doubling on the whole message, the intra-server small-message allreduce):
+       temp_all_reduce/all_reduce_doubling.cc:91-128.  Power-of-two rank counts; step s copies the running value
+       to the buffer the partner reads (input -> output first, output -> input afterwards) and folds the input of
+       rank XOR 2^s into the own output.  The inputs are overwritten.  Step-wise lowering only. */
+    HCOMM_GFX_ALG_ALLREDUCE_DOUBLING = 14
 } HcommGfxAlgorithm;
 
 typedef enum {

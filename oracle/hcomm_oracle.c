@@ -659,6 +659,28 @@ static void prog_allreduce_chunk_mesh(OrcTrace* t, uint32_t rank, uint32_t n, ui
     }
 }
 
+/* AllReduceDoubling::RunAllReduce for one rank, tpl/temp_all_reduce/all_reduce_doubling.cc:91-128 (n == 1: :38-41;
+ * the power-of-two check is SimpleCheck's, :81-88).  The copy and the reduce of one round are separated by the
+ * TxAck / RxAck exchange (:111-112), so they occupy two lock-step steps. */
+static int prog_allreduce_doubling(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) {
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
+        return 0;
+    }
+    if ((n & (n - 1)) != 0) return -1;
+    uint32_t n_steps = 0;
+    while ((1u << (n_steps + 1)) <= n) n_steps++; /* static_cast<u32>(log2(rankSize)), :97 */
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t neighbor = rank ^ (1u << step); /* :100 */
+        if (step == 0) emit(t, 2 * step, K_COPY, rank, B_OUT, 0, rank, B_IN, 0, total);  /* :105-106 */
+        else emit(t, 2 * step, K_COPY, rank, B_IN, 0, rank, B_OUT, 0, total);            /* :107-108 */
+        emit(t, 2 * step + 1, K_REDUCE, rank, B_OUT, 0, neighbor, B_IN, 0, total);       /* :113-121 */
+    }
+    return 0;
+}
+
 /* ---- NHR and NB: per-rank programs --------------------------------------------------------------------- */
 
 /* NHRBase::GetStepNumInterServer, tpl/nonuniform_hierarchical_ring_base.cc:139-147 = NBBase::CalcCeilLog2,
@@ -1005,7 +1027,8 @@ enum {
     ORC_ALG_RS_NHR = 10,
     ORC_ALG_ALLREDUCE_NB = 11,
     ORC_ALG_RS_NB = 12,
-    ORC_ALG_RS_LOCAL_REDUCE = 13
+    ORC_ALG_RS_LOCAL_REDUCE = 13,
+    ORC_ALG_ALLREDUCE_DOUBLING = 14
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -1068,6 +1091,12 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
             case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, stride, unit); break;
+            case ORC_ALG_ALLREDUCE_DOUBLING:
+                if (prog_allreduce_doubling(t, r, n, count, unit) != 0) {
+                    free(t->ops);
+                    return -1;
+                }
+                break;
             case ORC_ALG_RS_LOCAL_REDUCE:
                 if (stride != count) {
                     free(t->ops);
@@ -1201,6 +1230,7 @@ static void run_template(OrcTrace* t, int alg, uint32_t r, uint32_t n, uint64_t 
         case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
         case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, count, unit); break;
         case ORC_ALG_RS_LOCAL_REDUCE: prog_rs_local_reduce(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_DOUBLING: prog_allreduce_doubling(t, r, n, count, unit); break;
         default: break;
     }
 }
@@ -1274,7 +1304,7 @@ static int build_trace_opbase(OrcTrace* t, int alg, uint32_t n, uint64_t count, 
     if (n == 0 || n > ORC_MAX_RANKS || unit == 0 || alg == ORC_ALG_RS_RING_STAGE) return -1;
     const uint64_t max_count = orc_opbase_max_count(alg, n, ccl_bytes, dtype);
     if (max_count == 0) return -1; /* :213-218 / :163-165 */
-    if (alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE && (n & (n - 1))) return -1;
+    if ((alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE || alg == ORC_ALG_ALLREDUCE_DOUBLING) && (n & (n - 1))) return -1;
     for (uint32_t r = 0; r < n; r++) {
         const int rc = prog_opbase(t, alg, r, n, count, max_count, dtype);
         if (rc || t->oom) {

@@ -26,6 +26,7 @@ ALGS = {
     "nb_ar": (h.Alg.ALLREDUCE_NB, oracle.ALG_ALLREDUCE_NB),
     "nb_rs": (h.Alg.REDUCE_SCATTER_NB, oracle.ALG_RS_NB),
     "local_reduce_rs": (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, oracle.ALG_RS_LOCAL_REDUCE),
+    "doubling": (h.Alg.ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_DOUBLING),
 }
 SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending",
@@ -167,6 +168,11 @@ CASES = [
     ("local_reduce_rs", 3, 1001, "int16", "sum"),   # up to 32 KiB: windows not staggered
     ("local_reduce_rs", 2, 9, "fp32", "prod"),
     ("local_reduce_rs", 1, 100, "fp32", "sum"),
+    ("doubling", 8, 2048, "fp16", "sum"),           # its use: small messages inside a server
+    ("doubling", 16, 100003, "fp32", "max"),
+    ("doubling", 4, 1 << 20, "bf16", "sum"),
+    ("doubling", 2, 9, "int8", "min"),
+    ("doubling", 1, 100, "int32", "sum"),
 ]
 
 

@@ -15,7 +15,8 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 ALG = {"ring_ar": oracle.ALG_ALLREDUCE_RING, "mesh_rs": oracle.ALG_RS_MESH}
 ALLREDUCE = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_ALLREDUCE_RHD, oracle.ALG_ALLREDUCE_MESH_ONESHOT,
              oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
-             oracle.ALG_ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NB]
+             oracle.ALG_ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_ALLREDUCE_DOUBLING]
+POW2_ONLY = (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING)
 SCATTER = [oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
            oracle.ALG_RS_LOCAL_REDUCE]
 UIN, UOUT = 3, 4
@@ -52,7 +53,7 @@ CONFIGS = [(1000, oracle.F32, 2048), (1000, oracle.F32, 1 << 20), (100003, oracl
 def test_product_generator_equals_oracle_trace_and_passes_the_checker(alg):
     expect = Expect.REDUCE_SCATTER_USER if alg in SCATTER else Expect.ALLREDUCE_USER
     for n in (1, 2, 3, 4, 5, 8, 16):
-        if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+        if alg in POW2_ONLY and n & (n - 1):
             continue
         for count, dt, ccl in CONFIGS + [(5, oracle.F16, 128 * n)]:
             if oracle.opbase_max_count(alg, n, ccl, dt) == 0:              # the executors refuse such a buffer
@@ -87,7 +88,7 @@ def scratch_for(alg, n, count, ccl, dt):
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 7, 8])
 def test_exact_integer_results_through_the_loop(alg, n):
     """Chunked or not, every element of the user output is the exact int32 sum (MAX) over the ranks."""
-    if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+    if alg in POW2_ONLY and n & (n - 1):
         pytest.skip("power-of-two rank counts only")
     count = 5003
     scatter = alg in SCATTER

@@ -17,7 +17,8 @@ ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUC
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
         oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
         oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB,
-        oracle.ALG_RS_LOCAL_REDUCE]
+        oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING]
+POW2_ONLY = (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING)
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
                oracle.ALG_RS_LOCAL_REDUCE)
 STRIDED = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB)
@@ -196,7 +197,7 @@ def test_every_rank_contributes_exactly_once(alg, n):
     """Rank r contributes 4^r per element (+ a position code in the low part for scatter variants); the
     int32 sum has base-4 digit 1 for every rank iff each was folded in exactly once (no carries: digits <= 3
     for up to 3 repeats).  MAX / MIN give the closed forms n-1 / 0 on a second pass."""
-    if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+    if alg in POW2_ONLY and n & (n - 1):
         pytest.skip("power-of-two rank counts only")
     count = 777
     per_in = n * count if alg in SCATTER_OUT else count
@@ -401,6 +402,24 @@ def test_rs_local_reduce_hand_derived():
         oracle.trace(oracle.ALG_RS_LOCAL_REDUCE, 4, 100, oracle.F32, 200)   # dense input slices only
 
 
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.MAX])
+def test_doubling_trees_hand_derived(op):
+    for n_s, want in GOLD["doubling_rank_tree"].items():
+        if n_s.startswith("_"):
+            continue
+        n, count = int(n_s), 1003
+        ins = order_sensitive_inputs(n, count, op, seed=110 + n)
+        work = [x.copy() for x in ins]
+        outs = [np.zeros(count, np.float32) for _ in range(n)]
+        oracle.run(oracle.ALG_ALLREDUCE_DOUBLING, work, outs, count, oracle.F32, op)
+        for r_s, tree in want["out"].items():
+            assert np.array_equal(outs[int(r_s)].view(np.uint32), eval_tree(tree, ins, op).view(np.uint32)), (n, r_s)
+        for r_s, tree in want["in"].items():
+            assert np.array_equal(work[int(r_s)].view(np.uint32), eval_tree(tree, ins, op).view(np.uint32)), (n, r_s)
+    with pytest.raises(ValueError):
+        oracle.trace(oracle.ALG_ALLREDUCE_DOUBLING, 6, 100, oracle.F32)
+
+
 def test_strided_scatter_input_layout():
     """Input slice i starts strideLen * i elements into the buffer (aicpu_reduce_scatter.cc:78-80); the gaps
     between slices are never read or written."""
@@ -428,7 +447,7 @@ def test_strided_scatter_input_layout():
 @pytest.mark.parametrize("alg", ALGS)
 def test_product_generator_equals_oracle_trace(alg):
     for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32):
-        if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+        if alg in POW2_ONLY and n & (n - 1):
             continue
         for count, dt in ((0, oracle.F32), (1, oracle.I8), (5, oracle.I8), (1000, oracle.F16), (100003, oracle.F32),
                           (100000003, oracle.I8)):
@@ -456,7 +475,7 @@ def test_steps_are_conflict_free_and_errors_are_reported():
     for every rank count, and bad arguments are reported."""
     for alg in ALGS:
         for n in range(1, 18):
-            if alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and n & (n - 1):
+            if alg in POW2_ONLY and n & (n - 1):
                 continue
             count = 100
             per_in = n * count if alg in SCATTER_OUT else count
