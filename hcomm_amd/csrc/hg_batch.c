@@ -81,7 +81,7 @@ void hg_finish_fold(HgLaunch* l)
         const uint64_t limit = t->store_partials ? g_small_bytes / 4 : g_small_bytes;
         t->small = (largest <= limit) ? 1u : 0u;
     }
-    const uint64_t tile_bytes = (t->tree || t->small) ? HG_TREE_TILE_BYTES : HG_TILE_BYTES;
+    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
         tiles += (t->bytes[s] + tile_bytes - 1) / tile_bytes;

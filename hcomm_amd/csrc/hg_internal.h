@@ -25,6 +25,9 @@ extern "C" {
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
 #define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree / small-message kernels: one access per lane and input */
+/* vectors a lane of the tree kernel handles when it folds k values per element, and the tile that makes */
+#define HG_TREE_NU(k) ((k) <= 8u ? 2u : 1u)
+#define HG_TREE_TILE_BYTES_K(k) (HG_TREE_TILE_BYTES * HG_TREE_NU(k))
 
 /* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
 typedef struct {

@@ -489,34 +489,59 @@ template <int L> __device__ __forceinline__ constexpr uint32_t bitrev(uint32_t q
     return r;
 }
 
-template <class Item, int L>
-__device__ __forceinline__ void fold_tree_item(const HgFoldTable& tab, uint32_t s, uint64_t idx)
+// NU items (128-bit vectors or single elements) per lane, all loads of a lane issued before any of its stores;
+// live[u] guards every access of item u.
+template <class Item, int L, uint32_t NU>
+__device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
+                                                const uint64_t (&idx)[NU])
 {
     typedef typename Item::V V;
     constexpr uint32_t K = 1u << L;
     const uint64_t off = tab.off[s];
     const uint32_t c = tab.first[s];
-    V x[K];
+    V x[K][NU];
 #pragma unroll
-    for (uint32_t q = 0; q < K; ++q) x[q] = Item::ld((const uint8_t*)tab.in[c ^ bitrev<L>(q)] + off, idx);
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint8_t* p = (const uint8_t*)tab.in[c ^ bitrev<L>(q)] + off;
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u) x[q][u] = live[u] ? Item::ld(p, idx[u]) : Item::zero();
+    }
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         const uint32_t b = c ^ bitrev<L>(q);
-        if (tab.in2[b]) x[q] = Item::op(x[q], Item::ld((const uint8_t*)tab.in2[b] + off, idx));
+        if (tab.in2[b]) {
+            const uint8_t* p = (const uint8_t*)tab.in2[b] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) x[q][u] = Item::op(x[q][u], Item::ld(p, idx[u]));
+        }
     }
 #pragma unroll
     for (int l = 0; l < L; ++l) {
 #pragma unroll
-        for (uint32_t q = 0; q < K; q += (2u << l)) x[q] = Item::op(x[q], x[q + (1u << l)]);
+        for (uint32_t q = 0; q < K; q += (2u << l)) {
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u) x[q][u] = Item::op(x[q][u], x[q + (1u << l)][u]);
+        }
     }
     // What the step-wise replay leaves in each input buffer: an even position is overwritten at every level it
     // takes part in and keeps the last result; an odd position only changes when it absorbed a neighbour.
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         const uint32_t b = c ^ bitrev<L>(q);
-        if ((q & 1u) == 0u || tab.in2[b]) Item::st((uint8_t*)tab.in[b] + off, idx, x[q]);
+        if ((q & 1u) == 0u || tab.in2[b]) {
+            uint8_t* p = (uint8_t*)tab.in[b] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[q][u]);
+        }
     }
-    for (uint32_t r = 0; r < tab.nout; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, x[0]);
+    for (uint32_t r = 0; r < tab.nout; ++r) {
+        uint8_t* p = (uint8_t*)tab.out[r] + off;
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u)
+            if (live[u]) Item::st(p, idx[u], x[0][u]);
+    }
 }
 
 // The trees of the nonuniform hierarchical ring and of the nonuniform Bruck schedule: n <= K = 2^L ranks, position
@@ -524,8 +549,9 @@ __device__ __forceinline__ void fold_tree_item(const HgFoldTable& tab, uint32_t 
 // q a multiple of 2^(l+1)) with q + 2^l wherever that position exists - the fold rank (c +- q) performs at step l
 // from rank (c +- q) +- 2^l.  An even position that had a right neighbour keeps the last value it computed; the
 // root goes to every output (allreduce) or to the owner's output (reduce-scatter).
-template <class Item, int L>
-__device__ __forceinline__ void fold_tree_item_rot(const HgFoldTable& tab, uint32_t s, uint64_t idx)
+template <class Item, int L, uint32_t NU>
+__device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
+                                                    const uint64_t (&idx)[NU])
 {
     typedef typename Item::V V;
     constexpr uint32_t K = 1u << L;
@@ -533,51 +559,76 @@ __device__ __forceinline__ void fold_tree_item_rot(const HgFoldTable& tab, uint3
     const uint32_t c = tab.first[s];
     const uint32_t n = tab.nranks;
     const bool plus = tab.tree == 2u;
-    V x[K];
+    V x[K][NU];
     uint32_t b[K];
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         b[q] = plus ? c + q : c + n - q;
         if (b[q] >= n) b[q] -= n;
-        if (q < n) x[q] = Item::ld((const uint8_t*)tab.in[b[q]] + off, idx);
+        if (q < n) {
+            const uint8_t* p = (const uint8_t*)tab.in[b[q]] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u) x[q][u] = live[u] ? Item::ld(p, idx[u]) : Item::zero();
+        }
     }
 #pragma unroll
     for (int l = 0; l < L; ++l) {
 #pragma unroll
         for (uint32_t q = 0; q < K; q += (2u << l))
-            if (q + (1u << l) < n) x[q] = Item::op(x[q], x[q + (1u << l)]);
+            if (q + (1u << l) < n) {
+#pragma unroll
+                for (uint32_t u = 0; u < NU; ++u) x[q][u] = Item::op(x[q][u], x[q + (1u << l)][u]);
+            }
     }
 #pragma unroll
     for (uint32_t q = 0; q < K; q += 2)
-        if (q + 1 < n) Item::st((uint8_t*)tab.in[b[q]] + off, idx, x[q]);
+        if (q + 1 < n) {
+            uint8_t* p = (uint8_t*)tab.in[b[q]] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[q][u]);
+        }
     if (tab.out_mode == 1u) {
-        Item::st((uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s], idx, x[0]);
+        uint8_t* p = (uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s];
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u)
+            if (live[u]) Item::st(p, idx[u], x[0][u]);
     } else {
-        for (uint32_t r = 0; r < tab.nout; ++r) Item::st((uint8_t*)tab.out[r] + off, idx, x[0]);
+        for (uint32_t r = 0; r < tab.nout; ++r) {
+            uint8_t* p = (uint8_t*)tab.out[r] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[0][u]);
+        }
     }
 }
 
+// A lane handles HG_TREE_NU(K) vectors: two while the 2 x K values fit comfortably in registers (K <= 8), else one.
 template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
+    constexpr uint32_t NU = HG_TREE_NU(1u << L);
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
-        const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
+        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * NU) + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
-        if (tab.tree == 1u) {
-            if (v < nvec) fold_tree_item<VecItem<DT, OP>, L>(tab, s, v);
-        } else {
-            if (v < nvec) fold_tree_item_rot<VecItem<DT, OP>, L>(tab, s, v);
+        uint64_t idx[NU];
+        bool live[NU];
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u) {
+            idx[u] = v0 + u * HG_BLOCK;
+            live[u] = idx[u] < nvec;
         }
-        if (v - tid + HG_BLOCK > nvec) { // the segment's last tile also owns its element tail
-            const uint64_t e = (nvec << 4) / ES + tid;
-            if ((e + 1) * ES <= bytes) {
-                if (tab.tree == 1u) fold_tree_item<ElemItem<DT, OP>, L>(tab, s, e);
-                else fold_tree_item_rot<ElemItem<DT, OP>, L>(tab, s, e);
-            }
+        if (tab.tree == 1u) fold_tree_items<VecItem<DT, OP>, L, NU>(tab, s, live, idx);
+        else fold_tree_items_rot<VecItem<DT, OP>, L, NU>(tab, s, live, idx);
+        if (v0 - tid + HG_BLOCK * NU > nvec) { // the segment's last tile also owns its element tail
+            const uint64_t ti[1] = {(nvec << 4) / ES + tid};
+            const bool tl[1] = {(ti[0] + 1) * ES <= bytes};
+            if (tab.tree == 1u) fold_tree_items<ElemItem<DT, OP>, L, 1>(tab, s, tl, ti);
+            else fold_tree_items_rot<ElemItem<DT, OP>, L, 1>(tab, s, tl, ti);
         }
     }
 }
