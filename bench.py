@@ -36,9 +36,10 @@ MEASURED_TRAFFIC = {
     ("ring_ar_bf16_n8_128MiB", "stepwise"): (131115.7 * 2.0 + 131072.0) * 1024,
     ("ring_ar_bf16_n8_128MiB", "fused"): (524348.6 * 2.0 + 1966281.4) * 1024,
     # averages over the launches of the dominant kernel in one collective (they differ in size per step)
-    ("rhd_ar_int32_n16_128MiB_sum", "stepwise"): (491539.0 * 2.0 + 491520.0) * 1024,
-    ("rhd_ar_int32_n16_128MiB_sum", "fused"): (1048633.4 * 2.0 + 3147325.6) * 1024,
-    ("nhr_ar_bf16_n8_128MiB", "stepwise"): (305878.8 * 2.0 + 305834.7) * 1024,
+    ("rhd_ar_int32_n16_128MiB_sum", "stepwise"): (491541.9 * 2.0 + 491520.2) * 1024,
+    ("rhd_ar_int32_n16_128MiB_sum", "fused"): (1048645.9 * 2.0 + 3145988.9) * 1024,
+    ("nhr_ar_bf16_n8_128MiB", "stepwise"): (305877.2 * 2.0 + 305834.7) * 1024,
+    ("nhr_ar_bf16_n8_128MiB", "fused"): (524407.5 * 2.0 + 1574742.8) * 1024,
 }
 
 # name: (algorithm, ranks, elements per rank, dtype, op, data distribution)
