@@ -148,42 +148,75 @@ static int conflicts(const HgLaunch* l, const HgOp* o)
     return 0;
 }
 
+typedef struct {
+    HgLaunch* l;
+    int open;
+    HgEmitFn emit;
+    void* ctx;
+} Coalescer;
+
+static int coalesce_one(Coalescer* c, const HgOp* o)
+{
+    HgLaunch* l = c->l;
+    const uint32_t kind = kind_of(o);
+    const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
+    if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG || conflicts(l, o))) {
+        hg_finish_seg2(l);
+        c->open = 0;
+        const int rc = c->emit(l, c->ctx);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    if (!c->open) {
+        memset(l, 0, sizeof(*l));
+        l->kind = kind;
+        l->dtype = dt;
+        l->op = op;
+        c->open = 1;
+    }
+    HgSeg2Table* t = &l->tab.seg2;
+    t->dst[t->nseg] = o->dst;
+    t->src[t->nseg] = o->src;
+    t->bytes[t->nseg] = o->bytes;
+    t->nseg++;
+    return HCCL_SUCCESS;
+}
+
+/* Both operands equally far from a 16-byte boundary (a rank buffer addressed at an odd element offset): the few
+ * bytes up to that boundary go to the element-wise kernel and the rest runs at full width.  Below this size the
+ * extra launch costs more than it saves. */
+#define HG_SPLIT_MIN_BYTES (64u * 1024u)
+
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
 {
-    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
-    if (!l) return HCCL_E_MEMORY;
+    Coalescer c;
+    c.l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!c.l) return HCCL_E_MEMORY;
+    c.open = 0;
+    c.emit = emit;
+    c.ctx = ctx;
     int rc = HCCL_SUCCESS;
-    int open = 0;
     for (uint64_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
         const HgOp* o = &ops[i];
         if (o->bytes == 0) continue;                   /* count == 0: nothing to do (dispatcher.cc:719-722) */
         if (!o->is_reduce && o->dst == o->src) continue; /* copy onto itself (dispatcher.cc:495-498) */
-        const uint32_t kind = kind_of(o);
-        const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
-        if (open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG ||
-                     conflicts(l, o))) {
-            hg_finish_seg2(l);
-            rc = emit(l, ctx);
-            open = 0;
-            if (rc != HCCL_SUCCESS) break;
+        const uintptr_t md = (uintptr_t)o->dst & (HG_VEC_BYTES - 1), ms = (uintptr_t)o->src & (HG_VEC_BYTES - 1);
+        const uint32_t es = o->is_reduce ? HcommGfxDataTypeSize((HcommDataType)o->dtype) : 1u;
+        if (md != 0 && md == ms && o->bytes >= HG_SPLIT_MIN_BYTES && es != 0 && md % es == 0) {
+            HgOp head = *o, body = *o;
+            head.bytes = HG_VEC_BYTES - md;
+            body.dst = (char*)o->dst + head.bytes;
+            body.src = (const char*)o->src + head.bytes;
+            body.bytes = o->bytes - head.bytes;
+            rc = coalesce_one(&c, &head);
+            if (rc == HCCL_SUCCESS) rc = coalesce_one(&c, &body);
+        } else {
+            rc = coalesce_one(&c, o);
         }
-        if (!open) {
-            memset(l, 0, sizeof(*l));
-            l->kind = kind;
-            l->dtype = dt;
-            l->op = op;
-            open = 1;
-        }
-        HgSeg2Table* t = &l->tab.seg2;
-        t->dst[t->nseg] = o->dst;
-        t->src[t->nseg] = o->src;
-        t->bytes[t->nseg] = o->bytes;
-        t->nseg++;
     }
-    if (open && rc == HCCL_SUCCESS) {
-        hg_finish_seg2(l);
-        rc = emit(l, ctx);
+    if (c.open && rc == HCCL_SUCCESS) {
+        hg_finish_seg2(c.l);
+        rc = emit(c.l, ctx);
     }
-    free(l);
+    free(c.l);
     return rc;
 }

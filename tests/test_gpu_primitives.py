@@ -87,7 +87,8 @@ def test_local_reduce_prod_needs_opt_in(gpu_thread, dtype):
 @pytest.mark.parametrize("op", ["sum", "max"])
 @pytest.mark.parametrize("dst_el,src_el", [(1, 1), (1, 0), (3, 2)])
 def test_local_reduce_unaligned(gpu_thread, dtype, op, dst_el, src_el):
-    """Pointers offset by whole elements but not by 16 bytes take the element-wise kernel."""
+    """Pointers offset by whole elements but not by 16 bytes take the element-wise kernel (only for the bytes up to
+    the next 16-byte boundary when both operands are equally far from one)."""
     dt, o, count = DT[dtype], OPS[op], 70001
     say("reduce unaligned", dtype, op, dst_el, src_el)
     a, b = gen(dt, count + 16, 3), gen(dt, count + 16, 4)
@@ -99,7 +100,10 @@ def test_local_reduce_unaligned(gpu_thread, dtype, op, dst_el, src_el):
     assert h.HcommLocalReduceOnThread(gpu_thread, d_a.data_ptr() + dst_el * u, d_b.data_ptr() + src_el * u, count,
                                       dt, o) == 0
     assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
-    assert [r.kind for r in h.launch_log(gpu_thread)] == [h.Kernel.BYTEWISE]
+    if dst_el == src_el and count * u >= 65536:  # equally misaligned and large: element-wise head, full-width body
+        assert [r.kind for r in h.launch_log(gpu_thread)] == [h.Kernel.BYTEWISE, h.Kernel.REDUCE2]
+    else:
+        assert [r.kind for r in h.launch_log(gpu_thread)] == [h.Kernel.BYTEWISE]
     assert_same(from_dev(d_a, a), want, dt)
 
 

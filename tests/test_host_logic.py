@@ -254,7 +254,13 @@ def test_batch_mode_splits_on_conflict_kind_type_and_capacity(rec):
     assert run([red(A, B), red(Cc, D, DT.INT32)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]
     assert run([red(A, B), red(Cc, D, DT.FP32, OP.MAX)]) == [(K.REDUCE2, 1), (K.REDUCE2, 1)]
     assert run([cp(A, B), cp(Cc, D), cp(D + 2 * mib, A)]) == [(K.COPY, 2), (K.COPY, 1)]
-    assert run([red(A + 4, B + 4)]) == [(K.BYTEWISE, 1)]                          # not 16-byte aligned
+    # both operands 4 bytes past a 16-byte boundary: 12 bytes element-wise, the rest at full width
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommLocalReduceOnThread(rec, A + 4, B + 4, mib // 4, DT.FP32, OP.SUM) == 0
+    assert [(r.kind, r.bytes) for r in h.launch_log(rec)] == [(K.BYTEWISE, 12), (K.REDUCE2, mib - 12)]
+    assert run([red(A + 4, B + 8)]) == [(K.BYTEWISE, 1)]                          # different misalignment
+    small = lambda: h.HcommLocalReduceOnThread(rec, A + 4, B + 4, 1000, DT.FP32, OP.SUM)
+    assert run([small]) == [(K.BYTEWISE, 1)]                                      # too small to be worth two launches
     many = [cp(DST + (2 * i) * mib, DST + (2 * i + 1) * mib) for i in range(70)]
     assert run(many) == [(K.COPY, 32), (K.COPY, 32), (K.COPY, 6)]                 # 32 segments per launch
 
