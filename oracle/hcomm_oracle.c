@@ -1,6 +1,7 @@
 /*
- * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics and of the ring, recursive
- * halving-doubling and mesh schedules, used ONLY to check libhcomm_gfx.so.
+ * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics, of the ring, recursive
+ * halving-doubling, mesh, NHR, NB, local-reduce, chunk-mesh and doubling schedules and of the executors' op-base
+ * loop around them, used ONLY to check libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -31,6 +32,17 @@
  *                                     own acceptance rule (every output range receives every rank exactly
  *                                     once, allreduce_semantics_checker.cc:59-96), non-associative fp
  *                                     inputs, and agreement with the product's independent generator; pinned
+ *   ring, RHD, mesh (both orders) ... hand-derived receive tables and expression trees, N = 2, 3, 4, 6; pinned
+ *   local-reduce allreduce, chunk
+ *   mesh ............................ hand-derived fold trees / fold orders, N = 2, 4; pinned
+ *   NHR ............................. slice maps N = 3..12, merged receive runs N = 5, fold trees N = 3..6, all
+ *                                     by hand; bit reversal for powers of two; pinned
+ *   NB .............................. slice tables, gather order N = 6, fold trees N = 3, 4, 5 by hand; pinned
+ *   local-reduce reduce-scatter ..... window / slot layout and fold trees N = 3..6 by hand; pinned
+ *   recursive doubling .............. per-rank trees and final input contents N = 2, 4, 8 by hand; pinned
+ *   op-base loop .................... chunk tables (offsets, sizes, per-slice copies, single-copy case) and
+ *                                     maxCountPerLoop values by hand; exact integer results; pinned
+ *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
 #include <stdlib.h>
