@@ -24,7 +24,7 @@ __all__ = [
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
-    "OpBasePlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
+    "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
@@ -390,6 +390,28 @@ class OpBasePlan(Plan):
         p = _vp(0)
         check(_opbase_plan(alg, lowering, n, self._keep[0], self._keep[1], self._keep[2], self._keep[3], self._keep[4],
                            ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxOpBasePlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_plan_from_ops = _sig("HcommGfxPlanCreateFromOps", _i32, C.POINTER(SchedOp), _u64, _u32, C.POINTER(C.POINTER(_vp)), C.c_int,
+                      C.c_int, C.POINTER(_vp))
+
+
+class OpListPlan(Plan):
+    """HcommGfxPlanCreateFromOps: replay a caller's own op list.  ops: tuples as schedule_emit returns them;
+    buffers: {role: [pointer per rank]} for the roles the list names."""
+
+    def __init__(self, ops, n_ranks, buffers, dtype, op):
+        arr = (SchedOp * max(len(ops), 1))()
+        for i, (step, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes) in enumerate(ops):
+            arr[i] = SchedOp(step, kind, rank, dbuf, srank, sbuf, doff, soff, nbytes)
+        self._rows = [(_vp * n_ranks)(*buffers[role]) if role in buffers else None for role in range(5)]
+        table = (C.POINTER(_vp) * 5)(*[C.cast(r, C.POINTER(_vp)) if r is not None else None for r in self._rows])
+        p = _vp(0)
+        check(_plan_from_ops(arr, len(ops), n_ranks, table, dtype, op, C.byref(p)), "HcommGfxPlanCreateFromOps")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -467,6 +467,44 @@ int32_t HcommGfxOpBasePlanCreate(
     return HCCL_SUCCESS;
 }
 
+int32_t HcommGfxPlanCreateFromOps(
+    const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, void* const* const* buffers, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if ((nOps && !ops) || !buffers) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    const uint32_t unit = HcommGfxDataTypeSize(dataType);
+    uint32_t steps = 0;
+    for (uint64_t i = 0; i < nOps; ++i) {
+        const HcommGfxSchedOp* o = &ops[i];
+        if (o->kind > 1 || o->rank >= nRanks || o->srcRank >= nRanks || o->dstBuf >= HCOMM_GFX_NUM_BUFS ||
+            o->srcBuf >= HCOMM_GFX_NUM_BUFS)
+            return HCCL_E_PARA;
+        if (o->kind == 1 && o->bytes % unit) return HCCL_E_PARA; /* a reduce moves whole elements */
+        if (i && o->step < ops[i - 1].step) return HCCL_E_PARA;   /* ordered by step */
+        if (!buffers[o->dstBuf] || !buffers[o->srcBuf] || !buffers[o->dstBuf][o->rank] || !buffers[o->srcBuf][o->srcRank])
+            return HCCL_E_PTR;
+        if (o->step + 1 > steps) steps = o->step + 1;
+    }
+    HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
+    if (!p) return HCCL_E_MEMORY;
+    p->magic = HG_PLAN_MAGIC;
+    p->graph_wanted = use_graph();
+    p->info.steps = steps;
+    for (uint64_t i = 0; i < nOps; ++i) p->info.algorithmicBytes += ops[i].bytes * (ops[i].kind ? 3u : 2u);
+    const int rc = lower_ops(p, ops, nOps, buffers, (int)dataType, (int)reduceOp);
+    if (rc != HCCL_SUCCESS) {
+        HcommGfxPlanDestroy(p);
+        return rc;
+    }
+    p->info.launches = p->nlaunch;
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
 int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n)
 {
     if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;

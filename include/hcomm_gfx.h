@@ -547,6 +547,18 @@ int32_t HcommGfxOpBasePlanCreate(
     void* const* cclIn, void* const* cclOut, void* const* scratch, uint64_t cclBytes, uint64_t count,
     HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
+/*
+ * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand
+ * to the dispatcher (HcclD2DMemcpyAsync / HcclReduceAsync, src/legacy/ascend910/platform/task/
+ * dispatcher_common.cc:114-147), ordered by step.  buffers[role][rank] gives the device buffer behind each of the
+ * HCOMM_GFX_NUM_BUFS roles an operation may name (a role no operation names may be NULL).  Operations of a step
+ * are merged into single launches exactly as batch mode merges primitive calls (no written range may overlap
+ * another range the launch reads or writes); HcommGfxOpListCheck verifies such a list without a GPU.
+ */
+int32_t HcommGfxPlanCreateFromOps(
+    const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, void* const* const* buffers, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan);
+
 /* Elements per chunk of the op-base loop. */
 int32_t HcommGfxOpBaseMaxCount(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t cclBytes, HcommDataType dataType,
                                uint64_t* maxCountPerLoop);

@@ -295,3 +295,50 @@ def test_ring_via_public_primitives_in_batch_mode(gpu_thread):
     for r in range(n):
         assert_same(from_dev(d_out[r], host_in[r]), want_out[r], dt)
         assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt)
+
+
+def test_plan_from_a_callers_op_list(gpu_thread):
+    """HcommGfxPlanCreateFromOps: the oracle's own per-rank programs, handed over as an op list, replay to the oracle's
+    result; so does a schedule written by hand here (a two-rank exchange through the communication buffers)."""
+    for name, n, count, dtype in (("nhr_ar", 6, 70001, "fp32"), ("chunk_mesh", 4, 40009, "bf16"), ("nb_rs", 5, 9999, "int32")):
+        dt = DT[dtype]
+        say("op list", name, n, count, dtype)
+        in_count, out_count = buffer_counts(name, n, count)
+        host_in = [gen(dt, in_count, 7000 + r) for r in range(n)]
+        want_in = [x.copy() for x in host_in]
+        want_out = [np.zeros(out_count, host_in[0].dtype) for _ in range(n)]
+        sb = h.scratch_bytes(ALGS[name][0], n, count, dt)
+        want_scr = [np.zeros(sb, np.uint8) for _ in range(n)] if sb else None
+        oracle.run(ALGS[name][1], want_in, want_out, count, dt, oracle.SUM, scratch=want_scr)
+        d_in = [to_dev(x) for x in host_in]
+        d_out = [to_dev(np.zeros(out_count, host_in[0].dtype)) for _ in range(n)]
+        d_scr = [to_dev(np.zeros(sb, np.uint8)) for _ in range(n)] if sb else None
+        bufs = {0: [t.data_ptr() for t in d_in], 1: [t.data_ptr() for t in d_out]}
+        if sb:
+            bufs[2] = [t.data_ptr() for t in d_scr]
+        plan = h.OpListPlan(oracle.trace(ALGS[name][1], n, count, dt), n, bufs, dt, oracle.SUM)
+        assert plan.run(gpu_thread) == 0
+        assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_out[r], want_out[r]), want_out[r], dt, "%s out[%d]" % (name, r))
+            assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt, "%s in[%d]" % (name, r))
+        plan.destroy()
+    # by hand: each of two ranks parks its input in the other's communication buffer, then folds it into its output
+    count, dt = 50001, oracle.F32
+    nb = count * 4
+    a, b = gen(dt, count, 1), gen(dt, count, 2)
+    ops = [(0, 0, 0, 1, 0, 0, 0, 0, nb), (0, 0, 1, 1, 0, 1, 0, 0, nb),          # out[r] = in[r]
+           (0, 0, 0, 2, 0, 1, 0, 0, nb), (0, 0, 1, 2, 0, 0, 0, 0, nb),          # scratch[r] = in[peer]
+           (1, 1, 0, 1, 0, 0, 2, 0, nb), (1, 1, 1, 1, 0, 1, 2, 0, nb)]          # out[r] += scratch[r]
+    assert h.oplist_check(ops, 2, h.Expect.ALLREDUCE, count, 4)[:2] == (0, 0)
+    d_in = [to_dev(a), to_dev(b)]
+    d_out = [to_dev(np.zeros(count, np.float32)) for _ in range(2)]
+    d_scr = [to_dev(np.zeros(count, np.float32)) for _ in range(2)]
+    plan = h.OpListPlan(ops, 2, {0: [t.data_ptr() for t in d_in], 1: [t.data_ptr() for t in d_out],
+                                 2: [t.data_ptr() for t in d_scr]}, dt, oracle.SUM)
+    assert plan.info.launches == 2
+    assert plan.run(gpu_thread) == 0
+    assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+    assert_same(from_dev(d_out[0], a), a + b, dt, "out[0]")
+    assert_same(from_dev(d_out[1], a), b + a, dt, "out[1]")
+    plan.destroy()

@@ -374,6 +374,31 @@ def test_fused_rhd_byte_accounting_with_fold():
     p.destroy()
 
 
+def test_plan_from_a_callers_op_list(rec):
+    """A caller's own op list lowers exactly like the built-in schedule it was taken from; malformed lists are refused."""
+    n, count, dt = 5, 4099, DT.FP32
+    ins = [DST + (i << 22) for i in range(n)]
+    outs = [SRC + (i << 22) for i in range(n)]
+    ops = h.schedule_emit(h.Alg.ALLREDUCE_NHR, n, count, dt)
+    mine = h.OpListPlan(ops, n, {0: ins, 1: outs}, dt, OP.SUM)
+    ref = h.Plan(h.Alg.ALLREDUCE_NHR, h.Lowering.STEPWISE, ins, outs, count, dt, OP.SUM)
+    assert [(l.kind, l.nseg, l.bytes, l.blocks) for l in mine.launches()] == \
+        [(l.kind, l.nseg, l.bytes, l.blocks) for l in ref.launches()]
+    assert (mine.info.steps, mine.info.algorithmicBytes) == (ref.info.steps, ref.info.algorithmicBytes)
+    assert mine.run(rec) == 0
+    for bad, code in ((ops[::-1], R.E_PARA),                                        # not ordered by step
+                      ([(0, 1, 0, 0, 0, 1, 0, 0, 6)], R.E_PARA),                     # a reduce of 1.5 elements
+                      ([(0, 2, 0, 0, 0, 1, 0, 0, 8)], R.E_PARA),                     # unknown kind
+                      ([(0, 0, 7, 0, 0, 1, 0, 0, 8)], R.E_PARA),                     # rank out of range
+                      ([(0, 0, 0, 5, 0, 1, 0, 0, 8)], R.E_PARA),                     # buffer role out of range
+                      ([(0, 0, 0, 2, 0, 1, 0, 0, 8)], R.E_PTR)):                     # role without buffers
+        with pytest.raises(h.HcommError) as e:
+            h.OpListPlan(bad, n, {0: ins, 1: outs}, dt, OP.SUM)
+        assert e.value.code == code
+    empty = h.OpListPlan([], n, {0: ins}, dt, OP.SUM)
+    assert empty.info.launches == 0 and empty.run(rec) == 0
+
+
 def test_plan_run_checks(rec):
     i, o = ptrs(2, 4096)
     p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, i, o, 1024, DT.FP32, OP.SUM)
