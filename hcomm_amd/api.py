@@ -24,6 +24,9 @@ __all__ = [
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
+    "HcommWriteNbiOnThread", "HcommReadNbiOnThread", "HcommSetNotifyWaitTimeOut",
+    "HcommThreadNotifyWaitOnThreadWithDefaultTimeout", "HcommThreadResAcquireTimeOut", "HcommFenceOnThread",
+    "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -183,6 +186,14 @@ HcommWriteOnThread = _sig("HcommWriteOnThread", _i32, _u64, _u64, _vp, _vp, _u64
 HcommReadOnThread = _sig("HcommReadOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
 HcommWriteReduceOnThread = _sig("HcommWriteReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
 HcommReadReduceOnThread = _sig("HcommReadReduceOnThread", _i32, _u64, _u64, _vp, _vp, _u64, C.c_int, C.c_int)
+HcommWriteNbiOnThread = _sig("HcommWriteNbiOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
+HcommReadNbiOnThread = _sig("HcommReadNbiOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
+HcommSetNotifyWaitTimeOut = _sig("HcommSetNotifyWaitTimeOut", _i32, C.c_float)
+HcommThreadNotifyWaitOnThreadWithDefaultTimeout = _sig("HcommThreadNotifyWaitOnThreadWithDefaultTimeout", _i32, _u64, _u32)
+HcommThreadResAcquireTimeOut = _sig("HcommThreadResAcquireTimeOut", _i32, C.c_float)
+HcommFenceOnThread = _sig("HcommFenceOnThread", _i32, _u64)
+HcommChannelFenceOnThread = _sig("HcommChannelFenceOnThread", _i32, _u64, _u64)
+HcommChannelDrainOnThread = _sig("HcommChannelDrainOnThread", _i32, _u64, _u64)
 _batch_transfer = _sig("HcommBatchTransferOnThread", _i32, _u64, _u64, C.POINTER(BatchTransferDesc), _u32)
 class CheckReport(C.Structure):
     _fields_ = [("conflicts", C.c_uint32), ("semanticErrors", C.c_uint32), ("message", C.c_char * 248)]

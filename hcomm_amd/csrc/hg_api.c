@@ -405,6 +405,16 @@ int32_t HcommReadOnThread(ThreadHandle thread, ChannelHandle channel, void* dst,
     return channel_op(thread, channel, 0, dst, src, len, HCOMM_DATA_TYPE_RESERVED, HCOMM_REDUCE_RESERVED);
 }
 
+int32_t HcommWriteNbiOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len)
+{
+    return channel_op(thread, channel, 0, dst, src, len, HCOMM_DATA_TYPE_RESERVED, HCOMM_REDUCE_RESERVED);
+}
+
+int32_t HcommReadNbiOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len)
+{
+    return channel_op(thread, channel, 0, dst, src, len, HCOMM_DATA_TYPE_RESERVED, HCOMM_REDUCE_RESERVED);
+}
+
 int32_t HcommWriteReduceOnThread(
     ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
     HcommReduceOp reduceOp)
@@ -581,6 +591,47 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
     if (t->recorder) return HCCL_SUCCESS;
     return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
+}
+
+/* default notify-wait time-out of the calling host thread, seconds: NOTIFY_WAIT_TIMEOUT_DEFAULT,
+ * src/base_comm/primitives/launch_context.h:24 (kept per host thread there too, cpu_primitives_c_adpt.cc:26) */
+static _Thread_local uint32_t g_notify_timeout = 1836u;
+
+int32_t HcommSetNotifyWaitTimeOut(float timeOut)
+{
+    if (timeOut != timeOut || timeOut < 0.0f || timeOut > (float)UINT32_MAX) return HCCL_E_PARA;
+    g_notify_timeout = (uint32_t)timeOut;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommThreadNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, uint32_t notifyIdx)
+{
+    return HcommThreadNotifyWaitOnThread(thread, notifyIdx, g_notify_timeout);
+}
+
+int32_t HcommThreadResAcquireTimeOut(float timeOut)
+{
+    (void)timeOut;
+    return HCCL_E_NOT_SUPPORT;
+}
+
+/* ---- ordering points ------------------------------------------------------------------------------ */
+
+int32_t HcommFenceOnThread(ThreadHandle thread)
+{
+    return hg_thread_from_handle(thread) ? HCCL_SUCCESS : HCCL_E_PTR;
+}
+
+int32_t HcommChannelFenceOnThread(ThreadHandle thread, ChannelHandle channel)
+{
+    if (!channel) return HCCL_E_PTR;
+    return hg_thread_from_handle(thread) ? HCCL_SUCCESS : HCCL_E_PTR;
+}
+
+int32_t HcommChannelDrainOnThread(ThreadHandle thread, ChannelHandle channel)
+{
+    if (!hg_thread_from_handle(thread)) return HCCL_E_PTR;
+    return channel ? HCCL_SUCCESS : HCCL_E_PTR;
 }
 
 /* ---- memory -------------------------------------------------------------------------------------- */

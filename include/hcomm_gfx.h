@@ -149,6 +149,26 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);
 
 /*
+ * The default notify-wait time-out of the calling host thread and the wait that uses it.  Replace
+ * include/hcomm_primitives.h:559,585 (host adapter cpu_primitives_c_adpt.cc:41-50,1015-1034): a NaN, negative or
+ * larger-than-UINT32_MAX value is HCCL_E_PARA.  HcommThreadResAcquireTimeOut (:567) is not supported on this
+ * path either (cpu_primitives_c_adpt.cc:52-56).
+ */
+int32_t HcommSetNotifyWaitTimeOut(float timeOut);
+int32_t HcommThreadNotifyWaitOnThreadWithDefaultTimeout(ThreadHandle thread, uint32_t notifyIdx);
+int32_t HcommThreadResAcquireTimeOut(float timeOut);
+
+/*
+ * Ordering points.  Replace include/hcomm_primitives.h:534,542,593 (host adapter cpu_primitives_c_adpt.cc:780-808,
+ * 818-823).  A thread is an in-order HIP stream and a simulated peer shares its memory, so everything issued
+ * before such a call is already ordered before everything issued after it: the calls validate their handles and
+ * return.  Inside batch mode the recorded operations keep their order and their dependences anyway.
+ */
+int32_t HcommFenceOnThread(ThreadHandle thread);
+int32_t HcommChannelFenceOnThread(ThreadHandle thread, ChannelHandle channel);
+int32_t HcommChannelDrainOnThread(ThreadHandle thread, ChannelHandle channel);
+
+/*
  * Inter-rank twins of the two local primitives.  Replace include/hcomm_primitives.h:231-246,291-306 (host
  * adapter cpu_primitives_c_adpt.cc:284-318,332-384,490-565).  Same arithmetic with one operand on a peer:
  *   Write        peer dst[0..len) = local src          WriteReduce  peer dst[i] = dst[i] (op) local src[i]
@@ -165,6 +185,11 @@ int32_t HcommWriteReduceOnThread(
 int32_t HcommReadReduceOnThread(
     ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t count, HcommDataType dataType,
     HcommReduceOp reduceOp);
+
+/* The non-blocking spellings of the copy twins (include/hcomm_primitives.h:317-318,370-371): every operation on a
+ * thread is asynchronous here, so they are the same calls. */
+int32_t HcommWriteNbiOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len);
+int32_t HcommReadNbiOnThread(ThreadHandle thread, ChannelHandle channel, void* dst, const void* src, uint64_t len);
 
 /* include/hcomm_primitives.h:77-86 */
 typedef enum {

@@ -122,6 +122,27 @@ def test_notify_argument_checks(rec):
     assert h.HcommThreadNotifyWaitOnThread(rec, 0, 1) == R.E_PARA
 
 
+def test_timeouts_fences_and_non_blocking_twins(rec):
+    """include/hcomm_primitives.h:317-318,370-371,534,542,559,567,585,593 with the host adapter's checks."""
+    nan, CH = float("nan"), 0x77
+    assert h.HcommSetNotifyWaitTimeOut(nan) == R.E_PARA
+    assert h.HcommSetNotifyWaitTimeOut(-1.0) == R.E_PARA
+    assert h.HcommSetNotifyWaitTimeOut(5e9) == R.E_PARA
+    assert h.HcommSetNotifyWaitTimeOut(30.5) == R.SUCCESS
+    assert h.HcommThreadResAcquireTimeOut(1.0) == R.E_NOT_SUPPORT
+    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 0) == R.E_PARA       # the recorder has no notifies
+    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(12345, 0) == R.E_PTR
+    assert h.HcommFenceOnThread(rec) == R.SUCCESS and h.HcommFenceOnThread(12345) == R.E_PTR
+    assert h.HcommChannelFenceOnThread(rec, CH) == R.SUCCESS and h.HcommChannelFenceOnThread(rec, 0) == R.E_PTR
+    assert h.HcommChannelDrainOnThread(rec, CH) == R.SUCCESS and h.HcommChannelDrainOnThread(rec, 0) == R.E_PTR
+    assert h.HcommChannelDrainOnThread(12345, CH) == R.E_PTR
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommWriteNbiOnThread(rec, CH, DST, SRC, 4096) == 0
+    assert h.HcommReadNbiOnThread(rec, CH, DST, SRC, 8192) == 0
+    assert h.HcommWriteNbiOnThread(rec, 0, DST, SRC, 4096) == R.E_PTR
+    assert [(r.kind, r.bytes) for r in h.launch_log(rec)] == [(h.Kernel.COPY, 4096), (h.Kernel.COPY, 8192)]
+
+
 def test_inter_rank_twins_checks_and_launches(rec):
     """HcommWrite/Read[Reduce]OnThread: same arithmetic with a channel argument
     (cpu_primitives_c_adpt.cc:284-318,332-384,490-565)."""
