@@ -342,3 +342,29 @@ def test_plan_from_a_callers_op_list(gpu_thread):
     assert_same(from_dev(d_out[0], a), a + b, dt, "out[0]")
     assert_same(from_dev(d_out[1], a), b + a, dt, "out[1]")
     plan.destroy()
+
+
+def test_randomized_shapes(gpu_thread):
+    """A fixed-seed sample of (algorithm, rank count, ragged element count, type, operation, lowering): every buffer
+    bit-exact against the oracle.  Counts are drawn around the places where the kernels change path: the 16-byte
+    vector, the 16 KiB tile, the 128-byte slice alignment, the small-message thresholds."""
+    rng = np.random.default_rng(20240607)
+    names = sorted(ALGS)
+    interesting = [1, 2, 3, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 4095, 4096, 4097, 8191, 8192,
+                   16383, 16385, 65535, 65537, 131071, 262145]
+    done = 0
+    while done < 250:
+        name = names[rng.integers(len(names))]
+        n = int(rng.integers(1, 17))
+        if name in ("local_reduce", "doubling"):
+            n = 1 << int(rng.integers(0, 5))
+        base = interesting[rng.integers(len(interesting))]
+        count = int(base * rng.integers(1, 4) + rng.integers(0, 3))
+        dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
+        op = ["sum", "max", "min", "prod"][rng.integers(4)]
+        if op == "prod" and dtype == "int16":
+            continue
+        lowering = h.Lowering.FUSED if (name in FUSABLE and rng.integers(2)) else h.Lowering.STEPWISE
+        say("random", done, name, n, count, dtype, op, lowering)
+        run_case(gpu_thread, name, lowering, n, count, dtype, op, seed=done)
+        done += 1

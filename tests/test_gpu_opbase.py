@@ -99,3 +99,24 @@ def test_opbase_fused_leaves_identical_memory(gpu_thread, name, n, count, dtype,
     say("opbase fused", name, n, count, dtype, op, ccl)
     info = run_case(gpu_thread, name, h.Lowering.FUSED, n, count, dtype, op, ccl)
     assert info.movedBytes <= info.algorithmicBytes
+
+
+def test_randomized_opbase_shapes(gpu_thread):
+    """A fixed-seed sample of (algorithm, rank count, element count, type, CCL buffer size, lowering) through the op-base
+    loop: one pass, many chunks, ragged last chunks."""
+    rng = np.random.default_rng(777)
+    names = sorted(ALGS)
+    done = 0
+    while done < 60:
+        name = names[rng.integers(len(names))]
+        n = int(rng.integers(1, 13))
+        if name in ("local_reduce", "doubling"):
+            n = 1 << int(rng.integers(0, 4))
+        count = int(rng.integers(1, 60000))
+        dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
+        op = ["sum", "max", "min"][rng.integers(3)]
+        ccl = int(rng.integers(1, 64)) * 128 * n * 4
+        lowering = h.Lowering.FUSED if (name not in NOT_FUSABLE and rng.integers(2)) else h.Lowering.STEPWISE
+        say("random opbase", done, name, n, count, dtype, op, ccl, lowering)
+        run_case(gpu_thread, name, lowering, n, count, dtype, op, ccl)
+        done += 1
