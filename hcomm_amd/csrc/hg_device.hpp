@@ -1,0 +1,228 @@
+// hg_device.hpp - what the kernel translation units of libhcomm_gfx.so share: element arithmetic, 128-bit
+// accesses with cache hints, the workgroup -> tile numbering and the launch helpers.
+//
+// Element semantics (the reference's "dst = dst (op) src", src/legacy/ascend910/platform/task/
+// dispatcher_common.cc:137-147; CPU witnesses test/ut/stub/llt_hccl_stub.cc:4077-4204 and
+// test/hccl_vm/src/plugin/runner/runner_utils/hccl_task_reduce_process.cc:18-55):
+//   SUM a+b, PROD a*b, MAX (src > dst) ? src : dst, MIN (src < dst) ? src : dst;
+//   integers wrap in two's complement; fp32 is one IEEE operation; fp16 / bf16 widen to fp32, operate,
+//   and round to nearest even back to the storage type after every operation
+//   (test/hccl_vm/src/plugin/runner/ccu_executor/ccu_fp16.h:39-66,102-135); a NaN result of SUM / PROD on a
+//   16-bit type is stored as sign | 0x7e00 (fp16, ccu_fp16.h:121) or sign | 0x7fc0 (bf16, by analogy).
+
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "hg_internal.h"
+
+namespace {
+
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef signed char s8x4 __attribute__((ext_vector_type(4)));
+
+enum { OP_SUM = 0, OP_PROD = 1, OP_MAX = 2, OP_MIN = 3 };
+enum { DT_I8 = 0, DT_I16 = 1, DT_I32 = 2, DT_F16 = 3, DT_F32 = 4, DT_BF16 = 11 };
+
+template <int DT> struct ElemSize { static constexpr uint32_t v = (DT == DT_I8) ? 1u : (DT == DT_I32 || DT == DT_F32) ? 4u : 2u; };
+
+// ---- scalar element operations ----------------------------------------------------------------
+
+template <int OP, typename T> __device__ __forceinline__ T int_op(T d, T s)
+{
+    typedef typename std::make_unsigned<T>::type U;
+    if (OP == OP_SUM) return (T)((U)d + (U)s);
+    if (OP == OP_PROD) return (T)((U)d * (U)s);
+    if (OP == OP_MAX) return (s > d) ? s : d;
+    return (s < d) ? s : d;
+}
+
+__device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+template <int OP> __device__ __forceinline__ uint32_t f32_op(uint32_t d, uint32_t s)
+{
+    const float fd = bits_f32(d), fs = bits_f32(s);
+    if (OP == OP_SUM) return f32_bits(fd + fs);
+    if (OP == OP_PROD) return f32_bits(fd * fs);
+    if (OP == OP_MAX) return (fs > fd) ? s : d;
+    return (fs < fd) ? s : d;
+}
+
+__device__ __forceinline__ float f16_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
+
+__device__ __forceinline__ uint32_t f32_to_f16(float f)
+{
+    if (f != f) return ((f32_bits(f) >> 16) & 0x8000u) | 0x7e00u;
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return bits_f32(h << 16); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16(float f)
+{
+    const uint32_t u = f32_bits(f);
+    if (f != f) return ((u >> 16) & 0x8000u) | 0x7fc0u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// one 16-bit float element held in the low half of a word
+template <int DT, int OP> __device__ __forceinline__ uint32_t half_op(uint32_t d, uint32_t s)
+{
+    const float fd = (DT == DT_F16) ? f16_to_f32(d) : bf16_to_f32(d);
+    const float fs = (DT == DT_F16) ? f16_to_f32(s) : bf16_to_f32(s);
+    if (OP == OP_MAX) return (fs > fd) ? s : d;
+    if (OP == OP_MIN) return (fs < fd) ? s : d;
+    const float r = (OP == OP_SUM) ? fd + fs : fd * fs;
+    return (DT == DT_F16) ? f32_to_f16(r) : f32_to_bf16(r);
+}
+
+// ---- one 32-bit word of packed elements: returns d (op) s, d in the dst role ------------------------
+
+template <int DT, int OP> __device__ __forceinline__ uint32_t word_op(uint32_t d, uint32_t s)
+{
+    if (DT == DT_I32) return (uint32_t)int_op<OP, int32_t>((int32_t)d, (int32_t)s);
+    if (DT == DT_F32) return f32_op<OP>(d, s);
+    if (DT == DT_I16) {
+        const uint32_t lo = (uint16_t)int_op<OP, int16_t>((int16_t)(d & 0xffffu), (int16_t)(s & 0xffffu));
+        const uint32_t hi = (uint16_t)int_op<OP, int16_t>((int16_t)(d >> 16), (int16_t)(s >> 16));
+        return lo | (hi << 16);
+    }
+    if (DT == DT_I8) {
+        uint32_t r = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t e = (uint8_t)int_op<OP, int8_t>((int8_t)(d >> (8 * b)), (int8_t)(s >> (8 * b)));
+            r |= e << (8 * b);
+        }
+        return r;
+    }
+    // fp16 / bf16
+    const uint32_t lo = half_op<DT, OP>(d & 0xffffu, s & 0xffffu);
+    const uint32_t hi = half_op<DT, OP>(d >> 16, s >> 16);
+    return lo | (hi << 16);
+}
+
+template <int DT, int OP> __device__ __forceinline__ u32x4 vec_op(u32x4 d, u32x4 s)
+{
+    u32x4 r;
+    r.x = word_op<DT, OP>(d.x, s.x);
+    r.y = word_op<DT, OP>(d.y, s.y);
+    r.z = word_op<DT, OP>(d.z, s.z);
+    r.w = word_op<DT, OP>(d.w, s.w);
+    return r;
+}
+
+// one element at byte address p, zero-extended into a word / stored from the low bits of a word
+template <uint32_t ES> __device__ __forceinline__ uint32_t ld_elem(const void* p)
+{
+    if (ES == 1) return *(const uint8_t*)p;
+    if (ES == 2) return *(const uint16_t*)p;
+    return *(const uint32_t*)p;
+}
+template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t v)
+{
+    if (ES == 1) *(uint8_t*)p = (uint8_t)v;
+    else if (ES == 2) *(uint16_t*)p = (uint16_t)v;
+    else *(uint32_t*)p = v;
+}
+
+// Cache hints.  A ring step reads what the neighbouring rank's previous step wrote, so plain stores are left
+// to be kept by the memory-side cache while every load is marked non-temporal (each value is read once).
+#ifndef HG_NT_LD_DST
+#define HG_NT_LD_DST 1 /* the operand that is overwritten */
+#endif
+#ifndef HG_NT_LD_SRC
+#define HG_NT_LD_SRC 1 /* the peer's operand */
+#endif
+#ifndef HG_NT_ST
+#define HG_NT_ST 0
+#endif
+#ifndef HG_NT_FOLD_ST
+#define HG_NT_FOLD_ST 1 /* nothing a fold launch stores is read again by it */
+#endif
+template <bool NT> __device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec)
+{
+    if (NT) return __builtin_nontemporal_load((const u32x4*)base + vec);
+    return ((const u32x4*)base)[vec];
+}
+template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec, u32x4 v)
+{
+    if (NT) __builtin_nontemporal_store(v, (u32x4*)base + vec);
+    else ((u32x4*)base)[vec] = v;
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by their index.  REMAP renumbers them so that each XCD walks runs
+// of HG_XCD_RUN consecutive tiles (2 MiB) - or, when the grid does not divide that way, one contiguous eighth of the
+// tiles - instead of every eighth tile.  Measured on the 8 x 128 MiB ring steps (TB/s; plain, runs of 2 / 8 / 32 /
+// 128 tiles, contiguous eighth): copy 6.68, 6.69, 6.65, 6.84, 6.93, 6.87; two-input reduce 6.47, 6.49, 6.53, 6.35,
+// 6.51, 6.17; k-way fold 5.50, 5.44, 5.56, 5.59, 5.15, 4.84.  Only the copy gains beyond run-to-run noise, so only
+// k_copy renumbers.
+#ifndef HG_STREAM_COPY_BYTES
+#define HG_STREAM_COPY_BYTES (256ull << 20) /* the 256 MB memory-side cache */
+#endif
+#ifndef HG_STREAM_REDUCE_BYTES
+#define HG_STREAM_REDUCE_BYTES (256ull << 20)
+#endif
+#ifndef HG_XCD_REMAP_COPY
+#define HG_XCD_REMAP_COPY 1
+#endif
+#ifndef HG_XCD_REMAP
+#define HG_XCD_REMAP 0
+#endif
+#ifndef HG_XCD_RUN
+#define HG_XCD_RUN 128u
+#endif
+template <bool REMAP> __device__ __forceinline__ uint32_t block_id()
+{
+    const uint32_t g = gridDim.x, b = blockIdx.x;
+    if (!REMAP) return b;
+    if ((g % (8u * HG_XCD_RUN)) == 0u) {
+        const uint32_t i = b >> 3;
+        return (i / HG_XCD_RUN) * 8u * HG_XCD_RUN + (b & 7u) * HG_XCD_RUN + i % HG_XCD_RUN;
+    }
+    if ((g & 7u) == 0u) return (b & 7u) * (g >> 3) + (b >> 3);
+    return b;
+}
+
+// segment that owns a tile (uniform across the workgroup; nseg <= 32)
+__device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
+{
+    uint32_t s = 0;
+    while (s + 1 < nseg && tile >= tile_begin[s + 1]) ++s;
+    return s;
+}
+
+template <int DT, int OP> struct VecItem {
+    typedef u32x4 V;
+    static __device__ __forceinline__ V zero() { return V{0u, 0u, 0u, 0u}; }
+    static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ldv<HG_NT_LD_SRC>(p, i); }
+    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stv<HG_NT_FOLD_ST>(p, i, v); }
+    static __device__ __forceinline__ V op(V d, V s) { return vec_op<DT, OP>(d, s); }
+};
+
+template <int DT, int OP> struct ElemItem {
+    typedef uint32_t V;
+    static constexpr uint32_t ES = ElemSize<DT>::v;
+    static __device__ __forceinline__ V zero() { return 0u; }
+    static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ld_elem<ES>(p + i * ES); }
+    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { st_elem<ES>(p + i * ES, v); }
+    static __device__ __forceinline__ V op(V d, V s) { return word_op<DT, OP>(d, s); }
+};
+
+
+int rc(hipError_t e) { return e == hipSuccess ? HCCL_SUCCESS : HCCL_E_RUNTIME; }
+
+#define HG_DISPATCH_DT(dtype, CALL)                   \
+    switch (dtype) {                                  \
+        case DT_I8: return CALL(DT_I8);               \
+        case DT_I16: return CALL(DT_I16);             \
+        case DT_I32: return CALL(DT_I32);             \
+        case DT_F16: return CALL(DT_F16);             \
+        case DT_F32: return CALL(DT_F32);             \
+        case DT_BF16: return CALL(DT_BF16);           \
+        default: return HCCL_E_PARA;                  \
+    }
+
+} // namespace

@@ -1,0 +1,222 @@
+// hg_kernels_tree.hip - the k-way tree fold kernel (recursive halving-doubling, NHR and NB schedules in one launch).
+
+#include "hg_device.hpp"
+
+namespace {
+
+// ---- k-way tree fold (recursive halving) ---------------------------------------------------------
+//
+// K = 2^L block ranks.  For slice c, position q holds block rank c XOR bitrev(q); level l combines position q
+// (dst role) with q + 2^l - exactly the reduce every halving step performs (peer = rank XOR mask, mask from K/2
+// down to 1); each buffer receives the last value the step-wise replay would leave in it, and the root value
+// goes to every output.
+// A block rank with in2 != NULL first absorbs in2 (the odd neighbour folded in before the halving steps).
+
+template <int L> __device__ __forceinline__ constexpr uint32_t bitrev(uint32_t q)
+{
+    uint32_t r = 0;
+    for (int i = 0; i < L; ++i) r |= ((q >> i) & 1u) << (L - 1 - i);
+    return r;
+}
+
+// NU items (128-bit vectors or single elements) per lane, all loads of a lane issued before any of its stores;
+// live[u] guards every access of item u.
+template <class Item, int L, uint32_t NU>
+__device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
+                                                const uint64_t (&idx)[NU])
+{
+    typedef typename Item::V V;
+    constexpr uint32_t K = 1u << L;
+    const uint64_t off = tab.off[s];
+    const uint32_t c = tab.first[s];
+    V x[K][NU];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint8_t* p = (const uint8_t*)tab.in[c ^ bitrev<L>(q)] + off;
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u) x[q][u] = live[u] ? Item::ld(p, idx[u]) : Item::zero();
+    }
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint32_t b = c ^ bitrev<L>(q);
+        if (tab.in2[b]) {
+            const uint8_t* p = (const uint8_t*)tab.in2[b] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) x[q][u] = Item::op(x[q][u], Item::ld(p, idx[u]));
+        }
+    }
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (uint32_t q = 0; q < K; q += (2u << l)) {
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u) x[q][u] = Item::op(x[q][u], x[q + (1u << l)][u]);
+        }
+    }
+    // What the step-wise replay leaves in each input buffer: an even position is overwritten at every level it
+    // takes part in and keeps the last result; an odd position only changes when it absorbed a neighbour.
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint32_t b = c ^ bitrev<L>(q);
+        if ((q & 1u) == 0u || tab.in2[b]) {
+            uint8_t* p = (uint8_t*)tab.in[b] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[q][u]);
+        }
+    }
+    for (uint32_t r = 0; r < tab.nout; ++r) {
+        uint8_t* p = (uint8_t*)tab.out[r] + off;
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u)
+            if (live[u]) Item::st(p, idx[u], x[0][u]);
+    }
+}
+
+// The trees of the nonuniform hierarchical ring and of the nonuniform Bruck schedule: n <= K = 2^L ranks, position
+// q of slice c holds rank c + q (tree == 2) or c - q (tree == 3) mod n, and level l combines position q (dst role,
+// q a multiple of 2^(l+1)) with q + 2^l wherever that position exists - the fold rank (c +- q) performs at step l
+// from rank (c +- q) +- 2^l.  An even position that had a right neighbour keeps the last value it computed; the
+// root goes to every output (allreduce) or to the owner's output (reduce-scatter).
+template <class Item, int L, uint32_t NU>
+__device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
+                                                    const uint64_t (&idx)[NU])
+{
+    typedef typename Item::V V;
+    constexpr uint32_t K = 1u << L;
+    const uint64_t off = tab.off[s];
+    const uint32_t c = tab.first[s];
+    const uint32_t n = tab.nranks;
+    const bool plus = tab.tree == 2u;
+    V x[K][NU];
+    uint32_t b[K];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        b[q] = plus ? c + q : c + n - q;
+        if (b[q] >= n) b[q] -= n;
+        if (q < n) {
+            const uint8_t* p = (const uint8_t*)tab.in[b[q]] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u) x[q][u] = live[u] ? Item::ld(p, idx[u]) : Item::zero();
+        }
+    }
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (uint32_t q = 0; q < K; q += (2u << l))
+            if (q + (1u << l) < n) {
+#pragma unroll
+                for (uint32_t u = 0; u < NU; ++u) x[q][u] = Item::op(x[q][u], x[q + (1u << l)][u]);
+            }
+    }
+#pragma unroll
+    for (uint32_t q = 0; q < K; q += 2)
+        if (q + 1 < n) {
+            uint8_t* p = (uint8_t*)tab.in[b[q]] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[q][u]);
+        }
+    if (tab.out_mode == 1u) {
+        uint8_t* p = (uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s];
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u)
+            if (live[u]) Item::st(p, idx[u], x[0][u]);
+    } else {
+        for (uint32_t r = 0; r < tab.nout; ++r) {
+            uint8_t* p = (uint8_t*)tab.out[r] + off;
+#pragma unroll
+            for (uint32_t u = 0; u < NU; ++u)
+                if (live[u]) Item::st(p, idx[u], x[0][u]);
+        }
+    }
+}
+
+// A lane handles HG_TREE_NU(K) vectors: two while the 2 x K values fit comfortably in registers (K <= 8), else one.
+template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    constexpr uint32_t NU = HG_TREE_NU(1u << L);
+    const uint32_t total = tab.tile_begin[tab.nseg];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * NU) + tid;
+        const uint64_t bytes = tab.bytes[s];
+        const uint64_t nvec = bytes >> 4;
+        uint64_t idx[NU];
+        bool live[NU];
+#pragma unroll
+        for (uint32_t u = 0; u < NU; ++u) {
+            idx[u] = v0 + u * HG_BLOCK;
+            live[u] = idx[u] < nvec;
+        }
+        if (tab.tree == 1u) fold_tree_items<VecItem<DT, OP>, L, NU>(tab, s, live, idx);
+        else fold_tree_items_rot<VecItem<DT, OP>, L, NU>(tab, s, live, idx);
+        if (v0 - tid + HG_BLOCK * NU > nvec) { // the segment's last tile also owns its element tail
+            const uint64_t ti[1] = {(nvec << 4) / ES + tid};
+            const bool tl[1] = {(ti[0] + 1) * ES <= bytes};
+            if (tab.tree == 1u) fold_tree_items<ElemItem<DT, OP>, L, 1>(tab, s, tl, ti);
+            else fold_tree_items_rot<ElemItem<DT, OP>, L, 1>(tab, s, tl, ti);
+        }
+    }
+}
+
+template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+{
+    switch (op) {
+        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        default: return HCCL_E_PARA;
+    }
+    return rc(hipGetLastError());
+}
+
+template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+{
+    switch (tab->k) {
+        case 2: return launch_tree_dt_l<DT, 1>(st, op, tab, blocks);
+        case 4: return launch_tree_dt_l<DT, 2>(st, op, tab, blocks);
+        case 8: return launch_tree_dt_l<DT, 3>(st, op, tab, blocks);
+        case 16: return launch_tree_dt_l<DT, 4>(st, op, tab, blocks);
+        case 32: return launch_tree_dt_l<DT, 5>(st, op, tab, blocks);
+        default: return HCCL_E_PARA;
+    }
+}
+
+} // namespace
+
+// Compiled twice (HG_TREE_PART 0: integer element types, 1: floating-point ones) so that the 120 instances of the
+// kernel build side by side.
+#ifndef HG_TREE_PART
+#define HG_TREE_PART 0
+#endif
+
+#if HG_TREE_PART == 0
+extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks);
+
+extern "C" int hg_launch_tree(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks)
+{
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DT_I8: return launch_tree_dt<DT_I8>(st, op, tab, (uint32_t)blocks);
+        case DT_I16: return launch_tree_dt<DT_I16>(st, op, tab, (uint32_t)blocks);
+        case DT_I32: return launch_tree_dt<DT_I32>(st, op, tab, (uint32_t)blocks);
+        default: return hg_launch_tree_float(stream, dtype, op, tab, blocks);
+    }
+}
+#else
+extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks)
+{
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DT_F16: return launch_tree_dt<DT_F16>(st, op, tab, (uint32_t)blocks);
+        case DT_F32: return launch_tree_dt<DT_F32>(st, op, tab, (uint32_t)blocks);
+        case DT_BF16: return launch_tree_dt<DT_BF16>(st, op, tab, (uint32_t)blocks);
+        default: return HCCL_E_PARA;
+    }
+}
+#endif
