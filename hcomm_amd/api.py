@@ -27,6 +27,7 @@ __all__ = [
     "HcommWriteNbiOnThread", "HcommReadNbiOnThread", "HcommSetNotifyWaitTimeOut",
     "HcommThreadNotifyWaitOnThreadWithDefaultTimeout", "HcommThreadResAcquireTimeOut", "HcommFenceOnThread",
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
+    "HierPlan", "hier_emit", "hier_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -67,7 +68,7 @@ class Alg:
     ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
         REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING, ALLREDUCE_LOCAL_REDUCE, \
         ALLREDUCE_CHUNK_MESH, ALLREDUCE_NHR, REDUCE_SCATTER_NHR, ALLREDUCE_NB, REDUCE_SCATTER_NB, \
-        REDUCE_SCATTER_LOCAL_REDUCE, ALLREDUCE_DOUBLING = range(15)
+        REDUCE_SCATTER_LOCAL_REDUCE, ALLREDUCE_DOUBLING, ALLREDUCE_NHR_ONESHOT = range(16)
 
 
 class Lowering:
@@ -426,4 +427,41 @@ class OpListPlan(Plan):
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+# ---- the ring executor's three-step allreduce over two communicator levels -------------------------------
+
+_hier_emit = _sig("HcommGfxHierEmit", _i32, C.c_int, _u32, _u32, _u64, C.c_int, C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_hier_check = _sig("HcommGfxHierCheck", _i32, C.c_int, _u32, _u32, _u64, C.c_int, C.POINTER(CheckReport))
+_hier_plan = _sig("HcommGfxHierPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
+                  C.c_int, C.POINTER(_vp))
+
+
+def hier_emit(alg1, n_servers, n_local, count, dtype):
+    n = _u64(0)
+    check(_hier_emit(alg1, n_servers, n_local, count, dtype, None, 0, C.byref(n)), "HcommGfxHierEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_hier_emit(alg1, n_servers, n_local, count, dtype, ops, n.value, C.byref(n)), "HcommGfxHierEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def hier_check(alg1, n_servers, n_local, count, dtype):
+    rep = CheckReport()
+    check(_hier_check(alg1, n_servers, n_local, count, dtype, C.byref(rep)), "HcommGfxHierCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class HierPlan(Plan):
+    """HcommGfxHierPlanCreate: ring reduce-scatter inside the servers, alg1 between them, ring all-gather inside."""
+
+    def __init__(self, alg1, n_servers, n_local, in_ptrs, out_ptrs, count, dtype, op):
+        n = n_servers * n_local
+        self._in, self._out = (_vp * n)(*in_ptrs), (_vp * n)(*out_ptrs)
+        p = _vp(0)
+        check(_hier_plan(alg1, n_servers, n_local, self._in, self._out, count, dtype, op, C.byref(p)),
+              "HcommGfxHierPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxHierPlanGetInfo")
         self.info = info

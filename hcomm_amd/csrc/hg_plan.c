@@ -278,6 +278,36 @@ static int fused_rot_tree(HcommGfxPlan* p, int alg, uint32_t n, void* const* in,
     return rc;
 }
 
+/* The one-shot NHR allreduce: one segment, the whole message, on the balanced fold tree rooted at rank 0 - the
+ * positions that absorb a neighbour keep their last partial in their input, as the step-wise replay leaves them. */
+static int fused_oneshot_tree(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t total, int dtype,
+                              int op)
+{
+    if (total == 0) return HCCL_SUCCESS;
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    l->kind = HCOMM_GFX_KERNEL_TREE;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    HgFoldTable* f = &l->tab.fold;
+    f->tree = 2u;
+    f->k = 2;
+    while (f->k < n) f->k <<= 1;
+    f->nranks = n;
+    f->nout = n;
+    f->out_mode = 2u;
+    for (uint32_t r = 0; r < n; ++r) {
+        f->in[r] = in[r];
+        f->out[r] = out[r];
+    }
+    f->nseg = 1;
+    f->bytes[0] = total;
+    hg_finish_fold(l);
+    const int rc = plan_push(l, p);
+    free(l);
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
                        uint64_t stride, int dtype, int op)
 {
@@ -307,6 +337,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_REDUCE_SCATTER_NB:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rot_tree(p, alg, n, in, out, count, stride, dtype, op);
+        case HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_oneshot_tree(p, n, in, out, total, dtype, op);
         default: return HCCL_E_NOT_SUPPORT;
     }
 }
@@ -503,6 +536,27 @@ int32_t HcommGfxPlanCreateFromOps(
     p->info.launches = p->nlaunch;
     *plan = p;
     return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxHierPlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* in, void* const* out, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!in || !out) return HCCL_E_PTR;
+    if (nServers == 0 || nLocal == 0 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(in, nServers * nLocal);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(out, nServers * nLocal);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_hier(&ol, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {in, out, NULL, NULL, NULL};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nServers * nLocal, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
 }
 
 int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n)

@@ -651,6 +651,25 @@ static int sched_allreduce_doubling(HgOpList* l, uint32_t n, uint64_t count, uin
     return HCCL_SUCCESS;
 }
 
+/* AllReduceNHROneshot (temp_all_reduce/all_reduce_nhr_oneshot.cc:26-69): the whole message climbs a binomial tree
+ * to rank 0 and comes back down it.  Up (temp_reduce/reduce_nhr_oneshot.cc:169-236): in round s every rank q that is
+ * a multiple of 2^(s+1) and has a rank q + 2^s above it folds that rank's input into its own input.  Then rank 0
+ * copies its input to its output (temp_broadcast/broadcast_nhr_oneshot.cc:40-46) and the rounds run backwards on the
+ * outputs (:155-205): rank q + 2^s copies rank q's output. */
+static int sched_allreduce_nhr_oneshot(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    uint32_t step = 0;
+    for (uint32_t d = 1; d < n; d <<= 1, ++step)
+        for (uint32_t q = 0; q + d < n; q += 2 * d) CHK(push(l, step, REDUCE, q, IN, 0, q + d, IN, 0, total));
+    CHK(push(l, step++, COPY, 0, OUT, 0, 0, IN, 0, total));
+    uint32_t top = 1;
+    while (top < n) top <<= 1;
+    for (uint32_t d = top >> 1; d >= 1; d >>= 1, ++step)
+        for (uint32_t q = 0; q + d < n; q += 2 * d) CHK(push(l, step, COPY, q + d, OUT, 0, q, OUT, 0, total));
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
@@ -679,6 +698,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
         case HCOMM_GFX_ALG_REDUCE_SCATTER_NB: rc = sched_rs_nb(l, n, count, stride, unit); break;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE: rc = sched_rs_local_reduce(l, n, count, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_DOUBLING: rc = sched_allreduce_doubling(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT: rc = sched_allreduce_nhr_oneshot(l, n, count, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
@@ -801,5 +821,120 @@ int32_t HcommGfxOpBaseMaxCount(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t 
     const uint32_t unit = HcommGfxDataTypeSize(dataType);
     if (unit == 0 || nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     *maxCountPerLoop = hg_opbase_max_count((int)alg, nRanks, cclBytes, unit);
+    return HCCL_SUCCESS;
+}
+
+/* ---- the three-step allreduce of the ring executor (two communicator levels) ------------------------------- */
+
+/* Append `sub` to `l`: ranks through `map`, steps shifted by step0, offsets in the input / output buffers shifted by
+ * base (the templates add baseOffset_ to every slice they address, alg_template_base.cc:53-54).  Only the ops for
+ * which keep() holds. */
+static int append_mapped(HgOpList* l, const HgOpList* sub, const uint32_t* map, uint32_t step0, uint64_t base,
+                         int only_out_to_out, uint32_t* used)
+{
+    for (uint64_t i = 0; i < sub->n; ++i) {
+        const HcommGfxSchedOp* o = &sub->ops[i];
+        if (only_out_to_out && !(o->dstBuf == OUT && o->srcBuf == OUT)) continue;
+        if (o->step + 1 > *used) *used = o->step + 1;
+        CHK(push(l, step0 + o->step, o->kind, map[o->rank], o->dstBuf, o->dstOff + base, map[o->srcRank], o->srcBuf,
+                 o->srcOff + base, o->bytes));
+    }
+    return HCCL_SUCCESS;
+}
+
+/* CollAllReduceRingExecutor::KernelRun (src/legacy/ascend910/algorithm/impl/coll_executor/coll_all_reduce/
+ * coll_all_reduce_ring_executor.cc:94-231) for nServers x nLocal ranks, rank = server * nLocal + local index, one
+ * ring per server:
+ *   1. inside every server, ring reduce-scatter in place on the inputs over the slices of PrepareSliceData
+ *      (:109, alg_template_base.cc:787-820 - the 128-byte-aligned table), MultiRingReduceScatter :134-136;
+ *   2. between the servers, for every local index i, the level-1 allreduce template over segment i of the ranks
+ *      {i, nLocal + i, ...}: input and output ranges of the rank buffers, baseOffset = the segment's offset
+ *      (:156-158, :209-211; segment = local rank, coll_comm_executor.cc:2565-2575);
+ *   3. inside every server, ring all-gather on the outputs (MultiRingAllGather :228-230; input == output there,
+ *      coll_comm_executor.cc:377-379, so the template's own-slice copy does not happen, all_gather_ring.cc:117). */
+int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_RHD && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR &&
+        alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
+        return HCCL_E_PARA; /* the level-1 choices of :164-204 that are built here */
+    HcommGfxSlice seg[HCOMM_GFX_MAX_RANKS];
+    CHK(HcommGfxCalcSlices(count, unit, n_local, seg));
+    uint32_t map[HCOMM_GFX_MAX_RANKS];
+    HgOpList sub;
+    int rc = HCCL_SUCCESS;
+    uint32_t step = 0, used = 0;
+    /* 1 */
+    rc = hg_schedule(&sub, HCOMM_GFX_ALG_REDUCE_SCATTER_RING, n_local, count, count, dtype);
+    if (rc == HCCL_SUCCESS) {
+        for (uint32_t s = 0; s < n_servers && rc == HCCL_SUCCESS; ++s) {
+            for (uint32_t j = 0; j < n_local; ++j) map[j] = s * n_local + j;
+            rc = append_mapped(l, &sub, map, step, 0, 0, &used);
+        }
+        hg_oplist_free(&sub);
+    }
+    step += used;
+    /* 2 */
+    used = 0;
+    /* :171-181: NHR between the servers does not slice messages of up to 256 KiB per device of a server
+     * (NHR_ALLREDUCE_SMALL_SIZE, pub_inc/op_context.h:18) */
+    if (alg1 == HCOMM_GFX_ALG_ALLREDUCE_NHR && count * unit / n_local <= 256u * 1024u) alg1 = HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT;
+    for (uint32_t i = 0; i < n_local && rc == HCCL_SUCCESS; ++i) {
+        for (uint32_t s = 0; s < n_servers; ++s) map[s] = s * n_local + i;
+        rc = hg_schedule(&sub, alg1, n_servers, seg[i].size / unit, seg[i].size / unit, dtype);
+        if (rc != HCCL_SUCCESS) break;
+        rc = append_mapped(l, &sub, map, step, seg[i].offset, 0, &used);
+        hg_oplist_free(&sub);
+    }
+    step += used;
+    /* 3 */
+    used = 0;
+    if (rc == HCCL_SUCCESS) rc = hg_schedule(&sub, HCOMM_GFX_ALG_ALLREDUCE_RING, n_local, count, count, dtype);
+    if (rc == HCCL_SUCCESS) {
+        /* the gather rounds of the ring allreduce are the ops that move output to output; renumber them from 0 */
+        uint32_t first = UINT32_MAX;
+        for (uint64_t i = 0; i < sub.n; ++i)
+            if (sub.ops[i].dstBuf == OUT && sub.ops[i].srcBuf == OUT && sub.ops[i].step < first) first = sub.ops[i].step;
+        for (uint64_t i = 0; i < sub.n; ++i)
+            if (sub.ops[i].dstBuf == OUT && sub.ops[i].srcBuf == OUT) sub.ops[i].step -= first;
+        for (uint32_t s = 0; s < n_servers && rc == HCCL_SUCCESS; ++s) {
+            for (uint32_t j = 0; j < n_local; ++j) map[j] = s * n_local + j;
+            rc = append_mapped(l, &sub, map, step, 0, 1, &used);
+        }
+        hg_oplist_free(&sub);
+    }
+    if (rc != HCCL_SUCCESS) {
+        hg_oplist_free(l);
+        return rc;
+    }
+    /* the list is built level by level and, inside a level, group by group: order it by step, then by rank */
+    for (uint64_t i = 1; i < l->n; ++i) { /* insertion sort, stable */
+        HcommGfxSchedOp x = l->ops[i];
+        uint64_t j = i;
+        while (j > 0 && (l->ops[j - 1].step > x.step || (l->ops[j - 1].step == x.step && l->ops[j - 1].rank > x.rank))) {
+            l->ops[j] = l->ops[j - 1];
+            --j;
+        }
+        l->ops[j] = x;
+    }
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxHierEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_hier(&l, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
     return HCCL_SUCCESS;
 }

@@ -19,6 +19,8 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
  * into the CCL input buffer, run through the template, and copied from the CCL output to the user output. */
 int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 uint64_t hg_opbase_max_count(int alg, uint32_t n, uint64_t ccl_bytes, uint32_t unit);
+/* The ring executor's three-step allreduce over n_servers x n_local ranks with alg1 between the servers. */
+int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype);
 void hg_oplist_free(HgOpList* l);
 /* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);

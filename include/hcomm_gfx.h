@@ -385,7 +385,13 @@ typedef enum {
        temp_all_reduce/all_reduce_doubling.cc:91-128.  Power-of-two rank counts; step s copies the running value
        to the buffer the partner reads (input -> output first, output -> input afterwards) and folds the input of
        rank XOR 2^s into the own output.  The inputs are overwritten.  Step-wise lowering only. */
-    HCOMM_GFX_ALG_ALLREDUCE_DOUBLING = 14
+    HCOMM_GFX_ALG_ALLREDUCE_DOUBLING = 14,
+    /* AllReduceNHROneshot (the inter-server allreduce of messages up to 256 KiB per device, which are not cut into
+       slices): temp_all_reduce/all_reduce_nhr_oneshot.cc:26-69 = ReduceNHROneshot to rank 0
+       (temp_reduce/reduce_nhr_oneshot.cc:169-236, a binomial tree folding input into input) followed by
+       BroadcastNHROneshot (temp_broadcast/broadcast_nhr_oneshot.cc:24-59,155-205: rank 0 copies input -> output,
+       then the tree runs backwards on the outputs).  Any rank count. */
+    HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT = 15
 } HcommGfxAlgorithm;
 
 typedef enum {
@@ -395,7 +401,7 @@ typedef enum {
     /* steps whose data dependences are element-wise are folded into k-way kernels that read every input
        once and store every value the step-wise replay leaves in a buffer (partials included), so the final
        contents of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE.  Available for the ring, mesh,
-       recursive halving-doubling, NHR and NB algorithms; the algorithms that stage through a communication
+       recursive halving-doubling, NHR (sliced and one-shot) and NB algorithms; the algorithms that stage through a communication
        buffer return HCCL_E_NOT_SUPPORT */
     HCOMM_GFX_LOWER_FUSED = 1
 } HcommGfxLowering;
@@ -571,6 +577,24 @@ int32_t HcommGfxOpBasePlanCreate(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* userIn, void* const* userOut,
     void* const* cclIn, void* const* cclOut, void* const* scratch, uint64_t cclBytes, uint64_t count,
     HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+
+/*
+ * The three-step allreduce of the reference's ring executor over two communicator levels
+ * (src/legacy/ascend910/algorithm/impl/coll_executor/coll_all_reduce/coll_all_reduce_ring_executor.cc:94-231):
+ * nServers x nLocal ranks, rank = server * nLocal + local index.  (1) ring reduce-scatter inside every server, in
+ * place on the inputs; (2) for every local index i, level1Alg (HCOMM_GFX_ALG_ALLREDUCE_RING, _RHD, _NHR or _NB) over
+ * segment i of the ranks with that index, from the input to the output buffers; (3) ring all-gather inside every
+ * server on the outputs.  in / out: nServers * nLocal buffers of count elements.  Step-wise lowering.
+ */
+int32_t HcommGfxHierPlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* in, void* const* out, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxHierEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+int32_t HcommGfxHierCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxCheckReport* report);
 
 /*
  * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand

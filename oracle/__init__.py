@@ -17,7 +17,8 @@ SUM, PROD, MAX, MIN = 0, 1, 2, 3
 I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
 ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
     ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING, ALG_ALLREDUCE_LOCAL_REDUCE, ALG_ALLREDUCE_CHUNK_MESH, \
-    ALG_ALLREDUCE_NHR, ALG_RS_NHR, ALG_ALLREDUCE_NB, ALG_RS_NB, ALG_RS_LOCAL_REDUCE, ALG_ALLREDUCE_DOUBLING = range(15)
+    ALG_ALLREDUCE_NHR, ALG_RS_NHR, ALG_ALLREDUCE_NB, ALG_RS_NB, ALG_RS_LOCAL_REDUCE, ALG_ALLREDUCE_DOUBLING, \
+    ALG_ALLREDUCE_NHR_ONESHOT = range(16)
 
 # storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
 NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}
@@ -92,6 +93,11 @@ def lib():
         L.orc_opbase_max_count.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int]
         L.orc_algorithmic_bytes_opbase.restype = C.c_int64
         L.orc_algorithmic_bytes_opbase.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int]
+        L.orc_trace_hier.restype = C.c_int64
+        L.orc_trace_hier.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
+        L.orc_run_hier.restype = C.c_int
+        L.orc_run_hier.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                   C.c_uint64, C.c_int, C.c_int]
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run.restype = C.c_int
@@ -254,3 +260,23 @@ def run_opbase(alg, user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype,
 
 def algorithmic_bytes_opbase(alg, n, count, ccl_bytes, dtype):
     return lib().orc_algorithmic_bytes_opbase(alg, n, count, ccl_bytes, dtype)
+
+
+# ---- the ring executor's three-step allreduce over two communicator levels -------------------------------
+
+def trace_hier(alg1, n_servers, n_local, count, dtype):
+    total = lib().orc_trace_hier(alg1, n_servers, n_local, count, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_hier rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_hier(alg1, n_servers, n_local, count, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_hier(alg1, n_servers, n_local, ins, outs, count, dtype, op):
+    n = len(ins)
+    a = (C.c_void_p * n)(*[x.ctypes.data for x in ins])
+    b = (C.c_void_p * n)(*[x.ctypes.data for x in outs])
+    rc = lib().orc_run_hier(alg1, n_servers, n_local, a, b, count, dtype, op)
+    if rc:
+        raise ValueError("orc_run_hier rc=%d" % rc)

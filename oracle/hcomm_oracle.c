@@ -332,6 +332,11 @@ typedef struct {
 } OrcTrace;
 
 static uint32_t g_step_base = 0; /* added to every emitted step: where the current chunk of an op-base loop starts */
+/* A template running on a sub-communicator: its ranks are positions in g_rank_map, and it addresses the rank buffers
+ * baseOffset_ bytes in (tpl/alg_template_base.cc:53-54). */
+#define B_OUT_ROLE 1u /* roles 0 and 1: the template's input and output memory */
+static const uint32_t* g_rank_map = NULL;
+static uint64_t g_base_off = 0;
 
 static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint32_t dst_buf, uint64_t dst_off,
                  uint32_t src_rank, uint32_t src_buf, uint64_t src_off, uint64_t bytes)
@@ -350,12 +355,12 @@ static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint3
     OrcOp* o = &t->ops[t->n++];
     o->step = g_step_base + step;
     o->kind = kind;
-    o->rank = rank;
+    o->rank = g_rank_map ? g_rank_map[rank] : rank;
     o->dst_buf = dst_buf;
-    o->src_rank = src_rank;
+    o->src_rank = g_rank_map ? g_rank_map[src_rank] : src_rank;
     o->src_buf = src_buf;
-    o->dst_off = dst_off;
-    o->src_off = src_off;
+    o->dst_off = dst_off + (dst_buf <= B_OUT_ROLE ? g_base_off : 0);
+    o->src_off = src_off + (src_buf <= B_OUT_ROLE ? g_base_off : 0);
     o->bytes = bytes;
 }
 
@@ -381,15 +386,21 @@ static void prog_ring_rs(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice*
 }
 
 /* AllGatherRing::RunAsync + RunAllGather for one rank, tpl/temp_all_gather/all_gather_ring.cc:116-121,143-206 */
-static void prog_ring_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t step)
+static void prog_ring_ag_ex(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t step, int two_buffers)
 {
     const uint32_t left = (rank + n - 1) % n;
-    emit(t, step++, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size); /* :116-121 */
+    if (two_buffers) /* inputMem_ != outputMem_, :117 */
+        emit(t, step++, K_COPY, rank, B_OUT, sl[rank].offset, rank, B_IN, sl[rank].offset, sl[rank].size); /* :116-121 */
     uint32_t rx = (rank + n - 1) % n; /* ForwordRank(rank, n, 1), :152 */
     for (uint32_t i = 0; i < n - 1; i++) {
         emit(t, step++, K_COPY, rank, B_OUT, sl[rx].offset, left, B_OUT, sl[rx].offset, sl[rx].size); /* RxVector :34-45 */
         rx = (rx + n - 1) % n; /* :196 */
     }
+}
+
+static void prog_ring_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t step)
+{
+    prog_ring_ag_ex(t, rank, n, sl, step, 1);
 }
 
 static void prog_allreduce_ring(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit, int gather)
@@ -691,6 +702,58 @@ static int prog_allreduce_doubling(OrcTrace* t, uint32_t rank, uint32_t n, uint6
         emit(t, 2 * step + 1, K_REDUCE, rank, B_OUT, 0, neighbor, B_IN, 0, total);       /* :113-121 */
     }
     return 0;
+}
+
+/* ReduceNHROneshot::GetStepInfo, tpl/temp_reduce/reduce_nhr_oneshot.cc:195-227, root 0: whom this rank receives
+ * from in the step (n = nobody). */
+static uint32_t nhr_oneshot_reduce_from(uint32_t step, uint32_t rank, uint32_t n)
+{
+    uint32_t from = n;
+    const uint32_t n_ranks = (n - 1 + (1u << step)) / (1u << (step + 1));
+    const uint32_t delta_root = (rank + n - 0) % n;
+    const uint32_t delta_pair = 1u << step, delta_group = 1u << (step + 1);
+    if (delta_root / delta_group < n_ranks) {
+        if (delta_root % delta_group == 0) from = (rank + delta_pair) % n;
+    }
+    return from;
+}
+
+/* BroadcastNHROneshot::GetStepInfo, tpl/temp_broadcast/broadcast_nhr_oneshot.cc:175-203, root 0 */
+static uint32_t nhr_oneshot_bcast_from(uint32_t step, uint32_t n_steps, uint32_t rank, uint32_t n)
+{
+    uint32_t from = n;
+    const uint32_t n_ranks = (n - 1 + (1u << (n_steps - 1 - step))) / (1u << (n_steps - step));
+    const uint32_t delta_root = (rank + n - 0) % n;
+    const uint32_t delta_pair = 1u << (n_steps - 1 - step), delta_group = 1u << (n_steps - step);
+    if (delta_root / delta_group < n_ranks) {
+        if ((delta_root + delta_pair) % delta_group == 0) from = (rank + n - delta_pair) % n;
+    }
+    return from;
+}
+
+static uint32_t nhr_steps(uint32_t n);
+
+/* AllReduceNHROneshot::RunAsync for one rank, tpl/temp_all_reduce/all_reduce_nhr_oneshot.cc:26-69: the reduce to
+ * rank 0 works on (input, input) with the inline-reduce receive of reduce_nhr_oneshot.cc:96-106 (the left
+ * neighbour's input folded into the own input); the broadcast copies input -> output on the root
+ * (broadcast_nhr_oneshot.cc:40-46) and then output -> output down the tree (:82-104). */
+static void prog_allreduce_nhr_oneshot(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+{
+    const uint64_t total = count * unit;
+    if (n == 1) { /* :34-44 */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
+        return;
+    }
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t from = nhr_oneshot_reduce_from(step, rank, n);
+        if (from != n) emit(t, step, K_REDUCE, rank, B_IN, 0, from, B_IN, 0, total);
+    }
+    if (rank == 0) emit(t, n_steps, K_COPY, rank, B_OUT, 0, rank, B_IN, 0, total);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t from = nhr_oneshot_bcast_from(step, n_steps, rank, n);
+        if (from != n) emit(t, n_steps + 1 + step, K_COPY, rank, B_OUT, 0, from, B_OUT, 0, total);
+    }
 }
 
 /* ---- NHR and NB: per-rank programs --------------------------------------------------------------------- */
@@ -1040,7 +1103,8 @@ enum {
     ORC_ALG_ALLREDUCE_NB = 11,
     ORC_ALG_RS_NB = 12,
     ORC_ALG_RS_LOCAL_REDUCE = 13,
-    ORC_ALG_ALLREDUCE_DOUBLING = 14
+    ORC_ALG_ALLREDUCE_DOUBLING = 14,
+    ORC_ALG_ALLREDUCE_NHR_ONESHOT = 15
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -1103,6 +1167,7 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
             case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, stride, unit); break;
+            case ORC_ALG_ALLREDUCE_NHR_ONESHOT: prog_allreduce_nhr_oneshot(t, r, n, count, unit); break;
             case ORC_ALG_ALLREDUCE_DOUBLING:
                 if (prog_allreduce_doubling(t, r, n, count, unit) != 0) {
                     free(t->ops);
@@ -1243,6 +1308,7 @@ static void run_template(OrcTrace* t, int alg, uint32_t r, uint32_t n, uint64_t 
         case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, count, unit); break;
         case ORC_ALG_RS_LOCAL_REDUCE: prog_rs_local_reduce(t, r, n, count, unit); break;
         case ORC_ALG_ALLREDUCE_DOUBLING: prog_allreduce_doubling(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_NHR_ONESHOT: prog_allreduce_nhr_oneshot(t, r, n, count, unit); break;
         default: break;
     }
 }
@@ -1346,6 +1412,103 @@ int orc_run_opbase(int alg, uint32_t n, void* const* user_in, void* const* user_
     int rc = build_trace_opbase(&t, alg, n, count, ccl_bytes, dtype);
     if (rc) return rc;
     void* const* bufs[5] = {ccl_in, ccl_out, g_scratch, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+/* ---- the ring executor's three-step allreduce over two communicator levels ----------------------------------- */
+
+/* coll_all_reduce_ring_executor.cc:171-181: curSize / deviceNumPerAggregation <= NHR_ALLREDUCE_SMALL_SIZE
+ * (256 KiB, pub_inc/op_context.h:18) selects the one-shot NHR template; the devices of an aggregation are the
+ * n_local ranks of a server here. */
+static int hier_level1_template(int alg1, uint64_t count, uint32_t unit, uint32_t n_local)
+{
+    const uint64_t cur_size = count * unit;
+    if (alg1 == ORC_ALG_ALLREDUCE_NHR && cur_size / n_local <= 256u * 1024u) return ORC_ALG_ALLREDUCE_NHR_ONESHOT;
+    return alg1;
+}
+
+/* CollAllReduceRingExecutor::KernelRun for one rank, exec/coll_all_reduce/coll_all_reduce_ring_executor.cc:94-231,
+ * single ring per server (ringNum == 1, :123-125), buffer-copy mode.  rank = server * n_local + local index. */
+static int prog_hier_allreduce(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                               int dtype, uint32_t level1_steps)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    const uint32_t server = rank / n_local, local = rank % n_local;
+    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+    for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+    for (uint32_t s = 0; s < n_servers; s++) level1[s] = s * n_local + local;
+    OrcSlice seg[ORC_MAX_RANKS];
+    orc_slices_ring(count, unit, n_local, seg);          /* PrepareSliceData, :109 (tpl/alg_template_base.cc:787-820) */
+    /* step 1, :134-136: ReduceScatterRing on (input, input, output-as-scratch) inside the server */
+    g_rank_map = level0;
+    g_step_base = 0;
+    if (n_local > 1) prog_ring_rs(t, local, n_local, seg, NULL);
+    /* step 2, :140-218: level-1 allreduce of the own segment; hdSize / segment from PrepareLevel1CommInfo,
+     * exec/coll_comm_executor.cc:2565-2575 */
+    const uint64_t hd_count = seg[local].size / unit;    /* :146 */
+    g_rank_map = level1;
+    g_base_off = seg[local].offset;                      /* :211 */
+    g_step_base = n_local - 1;
+    run_template(t, hier_level1_template(alg1, count, unit, n_local), server, n_servers, hd_count, unit);
+    g_base_off = 0;
+    /* step 3, :228-230: AllGatherRing on (output, output, input-as-scratch), exec/coll_comm_executor.cc:377-379 */
+    g_rank_map = level0;
+    g_step_base = n_local - 1 + level1_steps;
+    if (n_local > 1) prog_ring_ag_ex(t, local, n_local, seg, 0, 0);
+    g_rank_map = NULL;
+    g_step_base = 0;
+    return 0;
+}
+
+static int build_trace_hier(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (alg1 != ORC_ALG_ALLREDUCE_RING && alg1 != ORC_ALG_ALLREDUCE_RHD && alg1 != ORC_ALG_ALLREDUCE_NHR &&
+        alg1 != ORC_ALG_ALLREDUCE_NB)
+        return -1;
+    /* the ranks run in lock step: the gather starts when the longest level-1 allreduce (the largest segment) is over */
+    OrcSlice seg[ORC_MAX_RANKS];
+    orc_slices_ring(count, unit, n_local, seg);
+    uint32_t level1_steps = 0;
+    for (uint32_t i = 0; i < n_local; i++) {
+        uint32_t st = 0;
+        const int rc = template_steps(hier_level1_template(alg1, count, unit, n_local), n_servers, seg[i].size / unit, dtype, &st);
+        if (rc) return rc;
+        if (st > level1_steps) level1_steps = st;
+    }
+    for (uint32_t r = 0; r < n_servers * n_local; r++) {
+        prog_hier_allreduce(t, alg1, r, n_servers, n_local, count, dtype, level1_steps);
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_hier(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_hier(&t, alg1, n_servers, n_local, count, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_hier(int alg1, uint32_t n_servers, uint32_t n_local, void* const* in, void* const* out, uint64_t count,
+                 int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_hier(&t, alg1, n_servers, n_local, count, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {in, out, NULL, NULL, NULL};
     rc = exec_trace(&t, bufs, dtype, op);
     free(t.ops);
     return rc;

@@ -27,10 +27,11 @@ ALGS = {
     "nb_rs": (h.Alg.REDUCE_SCATTER_NB, oracle.ALG_RS_NB),
     "local_reduce_rs": (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, oracle.ALG_RS_LOCAL_REDUCE),
     "doubling": (h.Alg.ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_DOUBLING),
+    "nhr_oneshot": (h.Alg.ALLREDUCE_NHR_ONESHOT, oracle.ALG_ALLREDUCE_NHR_ONESHOT),
 }
 SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending",
-           "nhr_ar", "nhr_rs", "nb_ar", "nb_rs"}
+           "nhr_ar", "nhr_rs", "nb_ar", "nb_rs", "nhr_oneshot"}
 
 
 def say(*a):
@@ -173,6 +174,14 @@ CASES = [
     ("doubling", 4, 1 << 20, "bf16", "sum"),
     ("doubling", 2, 9, "int8", "min"),
     ("doubling", 1, 100, "int32", "sum"),
+    ("nhr_oneshot", 8, 65536, "bf16", "sum"),       # its use: messages the NHR allreduce does not slice
+    ("nhr_oneshot", 5, 100003, "fp32", "sum"),
+    ("nhr_oneshot", 13, 4099, "fp16", "max"),
+    ("nhr_oneshot", 32, 70001, "int16", "min"),
+    ("nhr_oneshot", 2, 9, "int8", "sum"),
+    ("nhr_oneshot", 3, 1 << 20, "fp32", "prod"),
+    ("nhr_oneshot", 1, 100, "int32", "sum"),
+    ("nhr_oneshot", 6, 0, "fp32", "sum"),
 ]
 
 
@@ -207,7 +216,7 @@ def test_non_associative_inputs_expose_order(gpu_thread):
     """fp32 values for which (a+b)+c != a+(b+c): a replay in any other association order fails here."""
     n, count = 4, 4096
     base = np.array([1e8, 1.0, -1e8, 1.0], np.float32)
-    for alg in ("ring_ar", "rhd_ar", "mesh_oneshot", "nhr_ar", "nb_ar"):
+    for alg in ("ring_ar", "rhd_ar", "mesh_oneshot", "nhr_ar", "nb_ar", "nhr_oneshot"):
         for lowering in ((h.Lowering.STEPWISE, h.Lowering.FUSED) if alg in FUSABLE else (h.Lowering.STEPWISE,)):
             host_in = [np.full(count, base[(r + i) % 4], np.float32) for i, r in enumerate(range(n))]
             for r in range(n):

@@ -17,7 +17,7 @@ ALGS = {
     "nhr_ar": oracle.ALG_ALLREDUCE_NHR, "nb_ar": oracle.ALG_ALLREDUCE_NB, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
     "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "mesh_rs": oracle.ALG_RS_MESH, "ring_rs": oracle.ALG_RS_RING_STANDALONE,
     "nhr_rs": oracle.ALG_RS_NHR, "nb_rs": oracle.ALG_RS_NB, "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE,
-    "doubling": oracle.ALG_ALLREDUCE_DOUBLING,
+    "doubling": oracle.ALG_ALLREDUCE_DOUBLING, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
 }
 SCATTER = {"mesh_rs", "ring_rs", "nhr_rs", "nb_rs", "local_reduce_rs"}
 NOT_FUSABLE = {"chunk_mesh", "local_reduce", "local_reduce_rs", "doubling"}
@@ -40,6 +40,7 @@ CASES = [
     ("local_reduce_rs", 6, 50001, "fp16", "sum", 1 << 17),
     ("ring_ar", 1, 1000, "fp32", "sum", 1024),
     ("doubling", 8, 40009, "fp16", "sum", 1 << 16),
+    ("nhr_oneshot", 5, 40009, "bf16", "sum", 1 << 16),
 ]
 
 

@@ -15,7 +15,8 @@ GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "
 ALG = {"ring_ar": oracle.ALG_ALLREDUCE_RING, "mesh_rs": oracle.ALG_RS_MESH}
 ALLREDUCE = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_ALLREDUCE_RHD, oracle.ALG_ALLREDUCE_MESH_ONESHOT,
              oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
-             oracle.ALG_ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_ALLREDUCE_DOUBLING]
+             oracle.ALG_ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_ALLREDUCE_DOUBLING,
+             oracle.ALG_ALLREDUCE_NHR_ONESHOT]
 POW2_ONLY = (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING)
 SCATTER = [oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
            oracle.ALG_RS_LOCAL_REDUCE]

@@ -17,7 +17,7 @@ ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUC
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
         oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
         oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB,
-        oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING]
+        oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_NHR_ONESHOT]
 POW2_ONLY = (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING)
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
                oracle.ALG_RS_LOCAL_REDUCE)
@@ -418,6 +418,34 @@ def test_doubling_trees_hand_derived(op):
             assert np.array_equal(work[int(r_s)].view(np.uint32), eval_tree(tree, ins, op).view(np.uint32)), (n, r_s)
     with pytest.raises(ValueError):
         oracle.trace(oracle.ALG_ALLREDUCE_DOUBLING, 6, 100, oracle.F32)
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_nhr_oneshot_trees_hand_derived(op):
+    for n_s, want in GOLD["nhr_oneshot_rank_tree"].items():
+        if n_s.startswith("_"):
+            continue
+        n, count = int(n_s), 1003
+        ins = order_sensitive_inputs(n, count, op, seed=120 + n)
+        work = [x.copy() for x in ins]
+        outs = [np.zeros(count, np.float32) for _ in range(n)]
+        oracle.run(oracle.ALG_ALLREDUCE_NHR_ONESHOT, work, outs, count, oracle.F32, op)
+        root = eval_tree(want["out"], ins, op)
+        for r in range(n):
+            assert np.array_equal(outs[r].view(np.uint32), root.view(np.uint32)), (n, r)
+        for r_s, tree in want["in"].items():
+            assert np.array_equal(work[int(r_s)].view(np.uint32), eval_tree(tree, ins, op).view(np.uint32)), (n, r_s)
+        # the trace itself: who receives from whom in every round, up on the inputs and down on the outputs
+        ops = oracle.trace(oracle.ALG_ALLREDUCE_NHR_ONESHOT, n, count, oracle.F32)
+        rounds = len(want["up"])
+        for s, pairs in enumerate(want["up"]):
+            assert sorted([o[2], o[5]] for o in ops if o[0] == s) == pairs
+            assert all(o[1] == 1 and o[3] == 0 and o[6] == 0 and o[8] == count * 4 for o in ops if o[0] == s)
+        assert [o for o in ops if o[0] == rounds] == [(rounds, 0, 0, 1, 0, 0, 0, 0, count * 4)]
+        for s, pairs in enumerate(want["down"]):
+            assert sorted([o[2], o[5]] for o in ops if o[0] == rounds + 1 + s) == pairs
+            assert all(o[1] == 0 and o[3] == 1 and o[6] == 1 for o in ops if o[0] == rounds + 1 + s)
+        assert max(o[0] for o in ops) == 2 * rounds
 
 
 def test_strided_scatter_input_layout():

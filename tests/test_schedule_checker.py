@@ -14,7 +14,8 @@ ALL = [(h.Alg.ALLREDUCE_RING, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_RING, Exp
        (h.Alg.ALLREDUCE_LOCAL_REDUCE, Expect.ALLREDUCE), (h.Alg.ALLREDUCE_CHUNK_MESH, Expect.ALLREDUCE),
        (h.Alg.ALLREDUCE_NHR, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_NHR, Expect.REDUCE_SCATTER_OUT),
        (h.Alg.ALLREDUCE_NB, Expect.ALLREDUCE), (h.Alg.REDUCE_SCATTER_NB, Expect.REDUCE_SCATTER_OUT),
-       (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, Expect.REDUCE_SCATTER_OUT), (h.Alg.ALLREDUCE_DOUBLING, Expect.ALLREDUCE)]
+       (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, Expect.REDUCE_SCATTER_OUT), (h.Alg.ALLREDUCE_DOUBLING, Expect.ALLREDUCE),
+       (h.Alg.ALLREDUCE_NHR_ONESHOT, Expect.ALLREDUCE)]
 DENSE_ONLY = (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE,)
 
 
