@@ -60,6 +60,10 @@ WORKLOADS = {
     # the executors' op-base loop around the ring template: user buffers <-> 200 MiB CCL buffers (the default size)
     "opbase_ring_ar_bf16_n8_128MiB": ("opbase_ring_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "opbase_ring_ar_bf16_n8_512MiB": ("opbase_ring_ar", 8, 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the ring executor's three-step allreduce: 4 servers x 8 ranks, NHR / ring between the servers
+    "hier_nhr_ar_bf16_4x8_128MiB": ("hier_nhr", (4, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "hier_ring_ar_bf16_2x8_128MiB": ("hier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "nhr_oneshot_ar_bf16_n8_256KiB": ("nhr_oneshot", 8, 131072, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
 
@@ -117,12 +121,15 @@ def main():
     ALG = {"ring_ar": h.Alg.ALLREDUCE_RING, "rhd_ar": h.Alg.ALLREDUCE_RHD, "ring_rs_stage": h.Alg.REDUCE_SCATTER_RING,
            "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT, "local_reduce": h.Alg.ALLREDUCE_LOCAL_REDUCE,
            "chunk_mesh": h.Alg.ALLREDUCE_CHUNK_MESH, "nhr": h.Alg.ALLREDUCE_NHR, "nb": h.Alg.ALLREDUCE_NB,
-           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE}
+           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, "nhr_oneshot": h.Alg.ALLREDUCE_NHR_ONESHOT}
     OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
           "min": h.HcommReduceOp.MIN}
     opbase = alg_name.startswith("opbase_")  # the template inside the op-base loop of its executor
     if opbase:
         alg_name = alg_name[len("opbase_"):]
+    hier = None  # (servers, ranks per server): the level-1 template inside the ring executor's three steps
+    if alg_name.startswith("hier_"):
+        alg_name, hier, n = alg_name[len("hier_"):], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
     unit = h.DTYPE_SIZE[dt]
@@ -159,6 +166,8 @@ def main():
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both":
             args.lowering = "stepwise"
+    if hier:
+        args.lowering = "stepwise"  # composed from the step lists of its three levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
     if alg_name in ("local_reduce", "chunk_mesh", "local_reduce_rs") and args.lowering == "both":
@@ -167,6 +176,8 @@ def main():
              h.Kernel.COPY: "k_copy"}
 
     def make_plan(low):
+        if hier:
+            return h.HierPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, count, dt, op)
         if opbase:
             return h.OpBasePlan(alg, low, in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                 [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, scr_ptrs)
@@ -251,19 +262,24 @@ def main():
                 "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT,
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
-                "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE}[alg_name]
+                "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
         host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
-        alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
-                     else oracle.algorithmic_bytes(oalg, n, count, odt))
+        if hier:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_hier(oalg, hier[0], hier[1], count, odt))
+        else:
+            alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
+                         else oracle.algorithmic_bytes(oalg, n, count, odt))
         host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if opbase else None
 
         def cpu_run(ins, outs):
-            if opbase:
+            if hier:
+                oracle.run_hier(oalg, hier[0], hier[1], ins, outs, count, odt, oop)
+            elif opbase:
                 oracle.run_opbase(oalg, ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop, scratch=host_scr)
             else:
                 oracle.run(oalg, ins, outs, count, odt, oop, scratch=host_scr)
@@ -342,7 +358,7 @@ def main():
     h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
-        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, alg_name, opname)
+        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("three-step " if hier else "") + alg_name, opname)
     out = {
         "metric": metric,
         "value": round(res["gbs"], 2),
@@ -359,7 +375,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": opname,
                    "algorithm": alg_name, "values": dist, "lowering": best,
-                   **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {})},
+                   **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {}),
+                   **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": alg_name,
+                       "level0_algorithm": "ring reduce-scatter + ring all-gather"} if hier else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

@@ -1,7 +1,8 @@
 /*
  * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics, of the ring, recursive
- * halving-doubling, mesh, NHR, NB, local-reduce, chunk-mesh and doubling schedules and of the executors' op-base
- * loop around them, used ONLY to check libhcomm_gfx.so.
+ * halving-doubling, mesh, NHR (sliced and one-shot), NB, local-reduce, chunk-mesh and doubling schedules, of the
+ * executors' op-base loop around them and of the ring executor's three-step allreduce, used ONLY to check
+ * libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -42,6 +43,10 @@
  *   recursive doubling .............. per-rank trees and final input contents N = 2, 4, 8 by hand; pinned
  *   op-base loop .................... chunk tables (offsets, sizes, per-slice copies, single-copy case) and
  *                                     maxCountPerLoop values by hand; exact integer results; pinned
+ *   one-shot NHR .................... binomial-tree receive tables, output tree and final input contents
+ *                                     N = 2, 3, 5, 6, 8 by hand; pinned
+ *   three-step allreduce ............ the complete operation list of 2 servers x 2 ranks and the reduction trees
+ *                                     of 2 x 3 by hand; the one-shot threshold; exact integer results; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
