@@ -63,6 +63,10 @@ WORKLOADS = {
     # the ring executor's three-step allreduce: 4 servers x 8 ranks, NHR / ring between the servers
     "hier_nhr_ar_bf16_4x8_128MiB": ("hier_nhr", (4, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "hier_ring_ar_bf16_2x8_128MiB": ("hier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the double-ring executor in op-base mode with DMA reduce: user buffers read and written directly, 200 MiB CCL buffers
+    "dbring_ring_ar_bf16_1x8_128MiB": ("dbring_ring_ar", (1, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "dbring_ring_ar_bf16_1x8_512MiB": ("dbring_ring_ar", (1, 8), 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
+    "dbring_nhr_ar_bf16_2x8_128MiB": ("dbring_nhr", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nhr_oneshot_ar_bf16_n8_256KiB": ("nhr_oneshot", 8, 131072, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
@@ -128,8 +132,10 @@ def main():
     if opbase:
         alg_name = alg_name[len("opbase_"):]
     hier = None  # (servers, ranks per server): the level-1 template inside the ring executor's three steps
-    if alg_name.startswith("hier_"):
-        alg_name, hier, n = alg_name[len("hier_"):], n, n[0] * n[1]
+    dbring = False  # the double-ring executor with DMA reduce instead of the single ring on staged buffers
+    if alg_name.startswith("hier_") or alg_name.startswith("dbring_"):
+        dbring = alg_name.startswith("dbring_")
+        alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
     unit = h.DTYPE_SIZE[dt]
@@ -162,7 +168,7 @@ def main():
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
     scratch_bytes = h.scratch_bytes(alg, n, count, dt)
     d_ccl = None
-    if opbase:
+    if opbase or dbring:
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both":
             args.lowering = "stepwise"
@@ -176,6 +182,9 @@ def main():
              h.Kernel.COPY: "k_copy"}
 
     def make_plan(low):
+        if dbring:
+            return h.DoubleRingPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
+                                    [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if hier:
             return h.HierPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, count, dt, op)
         if opbase:
@@ -269,15 +278,20 @@ def main():
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
         host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
-        if hier:
+        if dbring:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2)
+                            for o in oracle.trace_dbring(oalg, hier[0], hier[1], count, ccl_bytes, odt))
+        elif hier:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_hier(oalg, hier[0], hier[1], count, odt))
         else:
             alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
                          else oracle.algorithmic_bytes(oalg, n, count, odt))
-        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if opbase else None
+        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if (opbase or dbring) else None
 
         def cpu_run(ins, outs):
-            if hier:
+            if dbring:
+                oracle.run_dbring(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
+            elif hier:
                 oracle.run_hier(oalg, hier[0], hier[1], ins, outs, count, odt, oop)
             elif opbase:
                 oracle.run_opbase(oalg, ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop, scratch=host_scr)
@@ -349,7 +363,7 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
-                if opbase:  # what the last chunk left in the CCL buffers
+                if opbase or dbring:  # what the last chunk left in the CCL buffers
                     ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
@@ -358,7 +372,7 @@ def main():
     h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
-        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("three-step " if hier else "") + alg_name, opname)
+        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("double-ring " if dbring else "three-step " if hier else "") + alg_name, opname)
     out = {
         "metric": metric,
         "value": round(res["gbs"], 2),
@@ -377,7 +391,9 @@ def main():
                    "algorithm": alg_name, "values": dist, "lowering": best,
                    **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {}),
                    **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": alg_name,
-                       "level0_algorithm": "ring reduce-scatter + ring all-gather"} if hier else {})},
+                       "level0_algorithm": ("double-ring reduce-scatter + all-gather on user memory (DMA reduce)"
+                                            if dbring else "ring reduce-scatter + ring all-gather")} if hier else {}),
+                   **({"ccl_buffer_bytes": ccl_bytes} if dbring else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

@@ -27,7 +27,7 @@ __all__ = [
     "HcommWriteNbiOnThread", "HcommReadNbiOnThread", "HcommSetNotifyWaitTimeOut",
     "HcommThreadNotifyWaitOnThreadWithDefaultTimeout", "HcommThreadResAcquireTimeOut", "HcommFenceOnThread",
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
-    "HierPlan", "hier_emit", "hier_check",
+    "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -450,6 +450,43 @@ def hier_check(alg1, n_servers, n_local, count, dtype):
     rep = CheckReport()
     check(_hier_check(alg1, n_servers, n_local, count, dtype, C.byref(rep)), "HcommGfxHierCheck")
     return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+_dbring_emit = _sig("HcommGfxDoubleRingEmit", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+                    C.POINTER(_u64))
+_dbring_check = _sig("HcommGfxDoubleRingCheck", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_dbring_plan = _sig("HcommGfxDoubleRingPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                    C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def dbring_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_dbring_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxDoubleRingEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_dbring_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxDoubleRingEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def dbring_check(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_dbring_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxDoubleRingCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class DoubleRingPlan(Plan):
+    """HcommGfxDoubleRingPlanCreate: the double-ring allreduce executor in op-base mode, user buffers read and written
+    directly."""
+
+    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_out, ccl_bytes, count, dtype, op):
+        n = n_servers * n_local
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in, ccl_out)]
+        p = _vp(0)
+        check(_dbring_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3],
+                           ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxDoubleRingPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
 
 
 class HierPlan(Plan):

@@ -842,6 +842,21 @@ static int append_mapped(HgOpList* l, const HgOpList* sub, const uint32_t* map, 
     return HCCL_SUCCESS;
 }
 
+/* Lists built level by level and, inside a level, group by group: order them by step, then by rank, keeping the
+ * order of a rank's operations inside a step (insertion sort, stable; the lists are nearly ordered already). */
+static void order_by_step_rank(HgOpList* l)
+{
+    for (uint64_t i = 1; i < l->n; ++i) {
+        HcommGfxSchedOp x = l->ops[i];
+        uint64_t j = i;
+        while (j > 0 && (l->ops[j - 1].step > x.step || (l->ops[j - 1].step == x.step && l->ops[j - 1].rank > x.rank))) {
+            l->ops[j] = l->ops[j - 1];
+            --j;
+        }
+        l->ops[j] = x;
+    }
+}
+
 /* CollAllReduceRingExecutor::KernelRun (src/legacy/ascend910/algorithm/impl/coll_executor/coll_all_reduce/
  * coll_all_reduce_ring_executor.cc:94-231) for nServers x nLocal ranks, rank = server * nLocal + local index, one
  * ring per server:
@@ -909,16 +924,148 @@ int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local
         hg_oplist_free(l);
         return rc;
     }
-    /* the list is built level by level and, inside a level, group by group: order it by step, then by rank */
-    for (uint64_t i = 1; i < l->n; ++i) { /* insertion sort, stable */
-        HcommGfxSchedOp x = l->ops[i];
-        uint64_t j = i;
-        while (j > 0 && (l->ops[j - 1].step > x.step || (l->ops[j - 1].step == x.step && l->ops[j - 1].rank > x.rank))) {
-            l->ops[j] = l->ops[j - 1];
-            --j;
+    order_by_step_rank(l);
+    return HCCL_SUCCESS;
+}
+
+/* ---- the double-ring allreduce executor in op-base mode --------------------------------------------------------- */
+
+#define UIN HCOMM_GFX_BUF_USER_IN
+#define UOUT HCOMM_GFX_BUF_USER_OUT
+
+/* CollAlignedAllReduceDoubleRingFor91093Executor (coll_executor/coll_all_reduce/
+ * coll_aligned_all_reduce_double_ring_for_910_93_executor.cc; KernelRun of its base,
+ * coll_all_reduce_ring_for_910_93_executor.cc:218-524) with DMA reduce, chunked by the op-base loop
+ * (coll_all_reduce_executor.cc:234-262, no staging copies :305-311, :326-331).
+ *
+ * Every segment of PrepareSliceData is cut in two 128-byte-aligned shares (MutliSegSlicePrepare,
+ * coll_comm_executor.cc:2011-2052); share 0 travels the ring 0 -> 1 -> ... and share 1 the mirrored ring
+ * 0 -> N-1 -> ... (GetRingsOrderByTopoType, :1939-1949).  Written in rank space, with dir = -1 for ring 0 and +1 for
+ * ring 1, every rank r
+ *   reduce-scatter (alg_template/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc:379-412, 640-685):
+ *     first copies the shares of segments r + dir and r + 2 dir from the user input to the CCL input; in step s folds
+ *     the share of segment r + (2 + s) dir of rank r + dir's CCL input into its own and, except in the last step,
+ *     fetches the share of segment r + (3 + s) dir from the user input;
+ *   level 1: the template between the servers on segment r of the CCL input / output buffers;
+ *   all-gather (alg_template/temp_all_gather/aligned_all_gather_double_ring.cc:343-449): in step s copies the share of
+ *     segment r + (1 + s) dir from rank r + dir's CCL output to its own, in the last step straight to the user
+ *     output, and copies the share of segment r + s dir from its CCL output to the user output. */
+static int dbring_build(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                        int dtype)
+{
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
+        return HCCL_E_PARA; /* the level-1 choices of coll_all_reduce_ring_for_910_93_executor.cc:304-351 built here */
+    const uint64_t max_count = ccl_bytes / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint32_t N = n_local;
+    int rc = HCCL_SUCCESS;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    HcommGfxSlice seg[HCOMM_GFX_MAX_RANKS], share[2][HCOMM_GFX_MAX_RANKS];
+    uint32_t map[HCOMM_GFX_MAX_RANKS];
+    for (uint64_t left = count; left > 0 && rc == HCCL_SUCCESS;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        CHK(HcommGfxCalcSlices(cur, unit, N, seg));
+        for (uint32_t i = 0; i < N; ++i) {
+            uint64_t first = ((seg[i].size + 1) / 2 + 127u) / 128u * 128u;
+            if (first > seg[i].size) first = seg[i].size;
+            share[0][i].offset = seg[i].offset;
+            share[0][i].size = first;
+            share[1][i].offset = seg[i].offset + first;
+            share[1][i].size = seg[i].size - first;
         }
-        l->ops[j] = x;
+#define SEG(r, k, dir) (((r) + (uint64_t)N * 4u + (uint64_t)(k) * ((dir) ? 1u : N - 1u)) % N) /* r + k * (+1 | -1) mod N */
+        for (uint32_t srv = 0; srv < n_servers && rc == HCCL_SUCCESS; ++srv) {
+            const uint32_t g0 = srv * N;
+            if (N == 1) { /* OneRankMemcpy of both templates */
+                for (uint32_t ring = 0; ring < 2; ++ring)
+                    CHK(push(l, step, COPY, g0, IN, share[ring][0].offset, g0, UIN, user_off + share[ring][0].offset, share[ring][0].size));
+                continue;
+            }
+            for (uint32_t r = 0; r < N; ++r)
+                for (uint32_t ring = 0; ring < 2; ++ring)
+                    for (uint32_t k = 1; k <= 2; ++k) {
+                        const HcommGfxSlice* x = &share[ring][SEG(r, k, ring)];
+                        CHK(push(l, step, COPY, g0 + r, IN, x->offset, g0 + r, UIN, user_off + x->offset, x->size));
+                    }
+            for (uint32_t s = 0; s + 1 < N; ++s)
+                for (uint32_t r = 0; r < N; ++r)
+                    for (uint32_t ring = 0; ring < 2; ++ring) {
+                        const HcommGfxSlice* x = &share[ring][SEG(r, 2 + s, ring)];
+                        CHK(push(l, step + 1 + s, REDUCE, g0 + r, IN, x->offset, g0 + (uint32_t)SEG(r, 1, ring), IN, x->offset, x->size));
+                        if (s + 2 == N) continue;
+                        x = &share[ring][SEG(r, 3 + s, ring)];
+                        CHK(push(l, step + 1 + s, COPY, g0 + r, IN, x->offset, g0 + r, UIN, user_off + x->offset, x->size));
+                    }
+        }
+        step += N == 1 ? 1 : N;
+        /* level 1 */
+        int alg = alg1;
+        if (alg1 == HCOMM_GFX_ALG_ALLREDUCE_NHR && cur * unit / N <= 256u * 1024u) alg = HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT;
+        uint32_t used = 0;
+        for (uint32_t i = 0; i < N && rc == HCCL_SUCCESS; ++i) {
+            HgOpList sub;
+            for (uint32_t srv = 0; srv < n_servers; ++srv) map[srv] = srv * N + i;
+            rc = hg_schedule(&sub, alg, n_servers, seg[i].size / unit, seg[i].size / unit, dtype);
+            if (rc != HCCL_SUCCESS) break;
+            rc = append_mapped(l, &sub, map, step, seg[i].offset, 0, &used);
+            hg_oplist_free(&sub);
+        }
+        step += used;
+        /* all-gather */
+        for (uint32_t srv = 0; srv < n_servers && rc == HCCL_SUCCESS; ++srv) {
+            const uint32_t g0 = srv * N;
+            if (N == 1) {
+                for (uint32_t ring = 0; ring < 2; ++ring)
+                    CHK(push(l, step, COPY, g0, UOUT, user_off + share[ring][0].offset, g0, OUT, share[ring][0].offset, share[ring][0].size));
+                continue;
+            }
+            for (uint32_t s = 0; s + 1 < N; ++s)
+                for (uint32_t r = 0; r < N; ++r)
+                    for (uint32_t ring = 0; ring < 2; ++ring) {
+                        const HcommGfxSlice* x = &share[ring][SEG(r, 1 + s, ring)];
+                        const int last = s + 2 == N;
+                        CHK(push(l, step + s, COPY, g0 + r, last ? UOUT : OUT, (last ? user_off : 0) + x->offset,
+                                 g0 + (uint32_t)SEG(r, 1, ring), OUT, x->offset, x->size));
+                        x = &share[ring][SEG(r, s, ring)];
+                        CHK(push(l, step + s, COPY, g0 + r, UOUT, user_off + x->offset, g0 + r, OUT, x->offset, x->size));
+                    }
+        }
+#undef SEG
+        step += N == 1 ? 1 : N - 1;
+        user_off += cur * unit;
+        left -= cur;
     }
+    if (rc != HCCL_SUCCESS) return rc;
+    order_by_step_rank(l);
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_dbring(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                       int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const int rc = dbring_build(l, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxDoubleRingEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_dbring(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
     return HCCL_SUCCESS;
 }
 

@@ -597,6 +597,35 @@ int32_t HcommGfxHierCheck(
     HcommGfxCheckReport* report);
 
 /*
+ * The allreduce of the reference's double-ring executor for two-ring servers in op-base mode, where the user buffers
+ * are read and written directly ("DMA reduce") instead of being staged through the CCL buffers
+ * (coll_executor/coll_all_reduce/coll_aligned_all_reduce_double_ring_for_910_93_executor.cc, KernelRun of
+ * coll_all_reduce_ring_for_910_93_executor.cc:218-524, loop of coll_all_reduce_executor.cc:234-262), per chunk of at
+ * most cclBytes / unit elements:
+ *   (1) AlignedReduceScatterDoubleRing inside every server
+ *       (alg_template/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc): every segment is cut in two shares,
+ *       share 0 reduced around the ring 0 -> 1 -> ... and share 1 around the mirrored ring; the CCL input buffer is
+ *       filled slice by slice from the user input just before each slice is needed;
+ *   (2) level1Alg (HCOMM_GFX_ALG_ALLREDUCE_RING, _NHR - one-shot for small chunks - or _NB) between the servers on the
+ *       own segment, CCL input -> CCL output;
+ *   (3) AlignedAllGatherDoubleRing inside every server (alg_template/temp_all_gather/aligned_all_gather_double_ring.cc):
+ *       both shares gathered around their rings in the CCL output buffers, every slice copied on to the user output
+ *       (the last one received lands there directly).
+ * nServers x nLocal ranks, rank = server * nLocal + local index; one super pod.  userIn / userOut: count elements;
+ * cclIn / cclOut: cclBytes each; all 128-byte aligned.  Step-wise lowering.
+ */
+int32_t HcommGfxDoubleRingPlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut,
+    void* const* cclIn, void* const* cclOut, uint64_t cclBytes, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxDoubleRingEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+int32_t HcommGfxDoubleRingCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
  * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand
  * to the dispatcher (HcclD2DMemcpyAsync / HcclReduceAsync, src/legacy/ascend910/platform/task/
  * dispatcher_common.cc:114-147), ordered by step.  buffers[role][rank] gives the device buffer behind each of the

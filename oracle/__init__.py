@@ -98,6 +98,13 @@ def lib():
         L.orc_run_hier.restype = C.c_int
         L.orc_run_hier.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                    C.c_uint64, C.c_int, C.c_int]
+        L.orc_trace_dbring.restype = C.c_int64
+        L.orc_trace_dbring.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.POINTER(OrcOp),
+                                       C.c_uint64]
+        L.orc_run_dbring.restype = C.c_int
+        L.orc_run_dbring.argtypes = [C.c_int, C.c_uint32, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + \
+            [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
+        L.orc_dbring_slices.restype = C.c_int
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run.restype = C.c_int
@@ -280,3 +287,33 @@ def run_hier(alg1, n_servers, n_local, ins, outs, count, dtype, op):
     rc = lib().orc_run_hier(alg1, n_servers, n_local, a, b, count, dtype, op)
     if rc:
         raise ValueError("orc_run_hier rc=%d" % rc)
+
+
+# ---- the double-ring allreduce executor in op-base mode (user memory read and written directly) ----------
+
+def trace_dbring(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    total = lib().orc_trace_dbring(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_dbring rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_dbring(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_dbring(alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype, op):
+    n = len(user_in)
+    arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in b]) for b in (user_in, user_out, ccl_in, ccl_out)]
+    rc = lib().orc_run_dbring(alg1, n_servers, n_local, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
+    if rc:
+        raise ValueError("orc_run_dbring rc=%d" % rc)
+
+
+def dbring_slices(count, dtype, n):
+    """([ring][position] -> (offset, size), [ring][position] -> device) of the double-ring slice preparation."""
+    sl = (OrcSlice * (2 * n))()
+    order = (C.c_uint32 * (2 * n))()
+    rc = lib().orc_dbring_slices(C.c_uint64(count), dtype, C.c_uint32(n), sl, order)
+    if rc:
+        raise ValueError("orc_dbring_slices rc=%d" % rc)
+    return ([[(sl[r * n + i].offset, sl[r * n + i].size) for i in range(n)] for r in range(2)],
+            [[order[r * n + i] for i in range(n)] for r in range(2)])

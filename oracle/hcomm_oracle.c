@@ -342,6 +342,7 @@ static uint32_t g_step_base = 0; /* added to every emitted step: where the curre
 #define B_OUT_ROLE 1u /* roles 0 and 1: the template's input and output memory */
 static const uint32_t* g_rank_map = NULL;
 static uint64_t g_base_off = 0;
+static uint64_t g_user_off = 0; /* where the current chunk of an op-base loop starts in the user buffers (roles 3, 4) */
 
 static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint32_t dst_buf, uint64_t dst_off,
                  uint32_t src_rank, uint32_t src_buf, uint64_t src_off, uint64_t bytes)
@@ -364,8 +365,8 @@ static void emit(OrcTrace* t, uint32_t step, uint32_t kind, uint32_t rank, uint3
     o->dst_buf = dst_buf;
     o->src_rank = g_rank_map ? g_rank_map[src_rank] : src_rank;
     o->src_buf = src_buf;
-    o->dst_off = dst_off + (dst_buf <= B_OUT_ROLE ? g_base_off : 0);
-    o->src_off = src_off + (src_buf <= B_OUT_ROLE ? g_base_off : 0);
+    o->dst_off = dst_off + (dst_buf <= B_OUT_ROLE ? g_base_off : (dst_buf >= 3u ? g_user_off : 0));
+    o->src_off = src_off + (src_buf <= B_OUT_ROLE ? g_base_off : (src_buf >= 3u ? g_user_off : 0));
     o->bytes = bytes;
 }
 
@@ -1517,6 +1518,232 @@ int orc_run_hier(int alg1, uint32_t n_servers, uint32_t n_local, void* const* in
     rc = exec_trace(&t, bufs, dtype, op);
     free(t.ops);
     return rc;
+}
+
+/* ---- the double-ring allreduce executor in op-base mode (user memory read and written directly) -------------- */
+
+typedef struct {
+    OrcSlice slices[2][ORC_MAX_RANKS]; /* multRingsSliceZero: per ring, the slice each ring position owns */
+    uint32_t order[2][ORC_MAX_RANKS];  /* multiRingsOrder */
+    OrcSlice seg[ORC_MAX_RANKS];       /* dataSegsSlice */
+} OrcDoubleRing;
+
+/* The executor's slice preparation for TOPO_TYPE_NP_DOUBLE_RING with every device in the NIC list:
+ * PrepareSliceData (tpl/alg_template_base.cc:787-820), MutliSegSlicePrepare (exec/coll_comm_executor.cc:2011-2052),
+ * GetRingsOrderByTopoType (:1939-1949), PrepareMultiRingSlice (:2094-2163, chunkSize == 1). */
+static void dbring_prepare(OrcDoubleRing* d, uint64_t count, uint32_t unit, uint32_t n)
+{
+    orc_slices_ring(count, unit, n, d->seg);
+    OrcSlice multi_seg[ORC_MAX_RANKS][2];
+    for (uint32_t rank_id = 0; rank_id < n; rank_id++) { /* :2016-2050 */
+        const uint64_t rank_data_size = d->seg[rank_id].size, offset_start = d->seg[rank_id].offset;
+        uint32_t ring_index = 0;
+        if (rank_data_size > 0) {
+            const uint64_t size_temp = (rank_data_size + 2 - 1) / 2;
+            const uint64_t size_per_ring = (size_temp + 127) / 128 * 128;
+            uint64_t residue = rank_data_size;
+            while (residue > 0) {
+                const uint64_t single = size_per_ring < residue ? size_per_ring : residue;
+                multi_seg[rank_id][ring_index].size = single;
+                multi_seg[rank_id][ring_index].offset = offset_start + rank_data_size - residue;
+                ring_index++;
+                residue -= single;
+            }
+        }
+        while (ring_index < 2) {
+            multi_seg[rank_id][ring_index].size = 0;
+            multi_seg[rank_id][ring_index].offset = offset_start;
+            ring_index++;
+        }
+    }
+    for (uint32_t i = 0; i < n; i++) d->order[0][i] = i;                 /* tmpLevel00 = nicList */
+    d->order[1][0] = 0;                                                   /* tmpLevel01: nicList[0], then ring 0 reversed */
+    for (uint32_t i = 1; i < n; i++) d->order[1][i] = d->order[0][n - i];
+    for (uint32_t ring = 0; ring < 2; ring++)
+        for (uint32_t segs_index = 0; segs_index < n; segs_index++)
+            d->slices[ring][segs_index] = multi_seg[d->order[ring][segs_index]][ring]; /* nicPosition == deviceIdx */
+}
+
+/* AlignedReduceScatterDoubleRing::RunAsync for one rank, tpl/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc,
+ * as the allreduce executor prepares it (exec/coll_all_reduce/coll_aligned_all_reduce_double_ring_for_910_93_executor.cc:
+ * 57-63): input and output memory = the CCL input buffer, opInfo->inputAddr = the user input, opInfo->outputAddr = null,
+ * user-memory slices = the ring slices (CalUserMemSlices, exec/coll_comm_executor.cc:2256-2260), one slice per ring
+ * position, inline reduce (:468-488).  Ring 0 (the "sub" ring) receives from rank - 1, ring 1 (the "main" ring) from
+ * rank + 1 (:433-447).  Step 0 of the trace is the template's step -1. */
+static void prog_dbring_rs(OrcTrace* t, uint32_t rank, uint32_t n, const OrcDoubleRing* d)
+{
+    if (n == 1) { /* OneRankMemcpy, :125-163 */
+        for (uint32_t ring = 0; ring < 2; ring++)
+            emit(t, 0, K_COPY, 0, B_IN, d->slices[ring][0].offset, 0, B_UIN, d->slices[ring][0].offset, d->slices[ring][0].size);
+        return;
+    }
+    const uint32_t pre[2] = {(rank + n - 1) % n, (rank + 1) % n};
+    /* RunInitStep, :379-412: the two slices of the first step come from the user input */
+    const uint32_t init0[2] = {(rank + n - 1) % n, (n - rank - 1 + n) % n};
+    const uint32_t init1[2] = {(rank + n - 2) % n, (n - rank - 2 + n) % n};
+    for (uint32_t ring = 0; ring < 2; ring++) {
+        const OrcSlice* s0 = &d->slices[ring][init0[ring]];
+        const OrcSlice* s1 = &d->slices[ring][init1[ring]];
+        emit(t, 0, K_COPY, rank, B_IN, s0->offset, rank, B_UIN, s0->offset, s0->size);
+        emit(t, 0, K_COPY, rank, B_IN, s1->offset, rank, B_UIN, s1->offset, s1->size);
+    }
+    /* RunReduceScatter, :640-685 */
+    uint32_t rx[2] = {(rank + n - 2) % n, (n - rank - 2 + n) % n};
+    uint32_t sub[2] = {(rank + n - 3) % n, (n - rank - 3 + n) % n};
+    for (uint32_t step = 0; step < n - 1; step++) {
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const OrcSlice* rx_slice = &d->slices[ring][rx[ring]];
+            const OrcSlice* ccl_slice = &d->slices[ring][sub[ring]];
+            /* ReducerRun, inline: the neighbour's input memory folded into the own, :476-480 */
+            emit(t, 1 + step, K_REDUCE, rank, B_IN, rx_slice->offset, pre[ring], B_IN, rx_slice->offset, rx_slice->size);
+            /* LocalMemcpy: next step's receive slice from the user input, :503-511, :518-522; none in the last step */
+            if (step != n - 2)
+                emit(t, 1 + step, K_COPY, rank, B_IN, ccl_slice->offset, rank, B_UIN, ccl_slice->offset, ccl_slice->size);
+            rx[ring] = (rx[ring] + n - 1) % n;
+            sub[ring] = (sub[ring] + n - 1) % n;
+        }
+    }
+}
+
+/* AlignedAllGatherDoubleRing::RunAsync for one rank, tpl/temp_all_gather/aligned_all_gather_double_ring.cc, as the
+ * allreduce executor prepares it (coll_aligned_all_reduce_double_ring_for_910_93_executor.cc:112-122): input and output
+ * memory = the CCL output buffer (so the init step copies nothing, :235-237), opInfo->outputAddr = the user output. */
+static void prog_dbring_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcDoubleRing* d)
+{
+    if (n == 1) { /* OneRankMemcpy, :119-153 */
+        for (uint32_t ring = 0; ring < 2; ring++)
+            emit(t, 0, K_COPY, 0, B_UOUT, d->slices[ring][0].offset, 0, B_OUT, d->slices[ring][0].offset, d->slices[ring][0].size);
+        return;
+    }
+    const uint32_t pre[2] = {(rank + n - 1) % n, (rank + 1) % n};
+    uint32_t tx[2] = {rank, (n - rank) % n};                     /* :411-414 */
+    uint32_t rx[2] = {(rank + n - 1) % n, (n - rank - 1 + n) % n};
+    for (uint32_t step = 0; step < n - 1; step++) {
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const OrcSlice* rx_slice = &d->slices[ring][rx[ring]];
+            const OrcSlice* tx_slice = &d->slices[ring][tx[ring]];
+            /* the received slice: into the CCL output, in the last step straight into the user output, :360-374 */
+            emit(t, step, K_COPY, rank, step == n - 2 ? B_UOUT : B_OUT, rx_slice->offset, pre[ring], B_OUT, rx_slice->offset,
+                 rx_slice->size);
+            /* the slice sent in this step also goes to the user output, :376-385 */
+            emit(t, step, K_COPY, rank, B_UOUT, tx_slice->offset, rank, B_OUT, tx_slice->offset, tx_slice->size);
+            tx[ring] = (tx[ring] + n - 1) % n;
+            rx[ring] = (rx[ring] + n - 1) % n;
+        }
+    }
+}
+
+/* CollAllReduceRingFor91093Executor::KernelRun (exec/coll_all_reduce/coll_all_reduce_ring_for_910_93_executor.cc:
+ * 218-524) for one rank and one chunk, TOPO_TYPE_NP_DOUBLE_RING, DMAReduceFlag_ set (op-base mode,
+ * coll_aligned_all_reduce_double_ring_for_910_93_executor.cc:20-24), one super pod (:298). */
+static int prog_dbring_allreduce(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                 int dtype, uint32_t level1_steps, uint32_t step0)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    const uint32_t server = rank / n_local, local = rank % n_local;
+    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+    for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+    for (uint32_t s = 0; s < n_servers; s++) level1[s] = s * n_local + local;
+    OrcDoubleRing d;
+    dbring_prepare(&d, count, unit, n_local);                  /* :229, :242 */
+    const uint32_t rs_steps = n_local == 1 ? 1 : n_local;      /* the init step and n - 1 ring steps */
+    g_rank_map = level0;
+    g_step_base = step0;
+    prog_dbring_rs(t, local, n_local, &d);                     /* :267-270 */
+    /* PrepareLevel1CommInfo on 910_93: segment = local rank, hdSize = both rings' shares of it,
+     * exec/coll_comm_executor.cc:2555-2559 */
+    const uint64_t hd_count = d.seg[local].size / unit;        /* :296 */
+    g_rank_map = level1;
+    g_base_off = d.seg[local].offset;                          /* :299-301, :360 */
+    g_step_base = step0 + rs_steps;
+    run_template(t, hier_level1_template(alg1, count, unit, n_local), server, n_servers, hd_count, unit); /* :338-347 */
+    g_base_off = 0;
+    g_rank_map = level0;
+    g_step_base = step0 + rs_steps + level1_steps;
+    prog_dbring_ag(t, local, n_local, &d);                     /* :519-521 */
+    g_rank_map = NULL;
+    g_step_base = 0;
+    return 0;
+}
+
+static int build_trace_dbring(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                              uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (alg1 != ORC_ALG_ALLREDUCE_RING && alg1 != ORC_ALG_ALLREDUCE_NHR && alg1 != ORC_ALG_ALLREDUCE_NB) return -1; /* :304-351 */
+    const uint64_t max_count = ccl_bytes / unit;               /* CalcLoopMaxCount, exec/coll_all_reduce/coll_all_reduce_executor.cc:129-138 */
+    if (max_count == 0) return -1;
+    /* RunLoop, exec/coll_all_reduce/coll_all_reduce_executor.cc:234-262; no staging copies with DMAReduceFlag_, :305-311, :326-331 */
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        OrcSlice seg[ORC_MAX_RANKS];
+        orc_slices_ring(cur_count, unit, n_local, seg);
+        uint32_t level1_steps = 0;
+        for (uint32_t i = 0; i < n_local; i++) {
+            uint32_t st = 0;
+            const int rc = template_steps(hier_level1_template(alg1, cur_count, unit, n_local), n_servers, seg[i].size / unit, dtype, &st);
+            if (rc) {
+                free(t->ops);
+                return rc;
+            }
+            if (st > level1_steps) level1_steps = st;
+        }
+        g_user_off = user_off;
+        for (uint32_t r = 0; r < n_servers * n_local; r++) prog_dbring_allreduce(t, alg1, r, n_servers, n_local, cur_count, dtype, level1_steps, step0);
+        g_user_off = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        const uint32_t edge = n_local == 1 ? 1 : n_local - 1;
+        step0 += (n_local == 1 ? 1 : n_local) + level1_steps + edge;
+        user_off += cur_count * unit;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_dbring(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes, int dtype,
+                         OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_dbring(int alg1, uint32_t n_servers, uint32_t n_local, void* const* user_in, void* const* user_out,
+                   void* const* ccl_in, void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+/* the double-ring slice tables, for the tests: out[ring * n + position] */
+int orc_dbring_slices(uint64_t count, int dtype, uint32_t n, OrcSlice* out, uint32_t* order)
+{
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n == 0 || n > ORC_MAX_RANKS) return -1;
+    OrcDoubleRing d;
+    dbring_prepare(&d, count, unit, n);
+    for (uint32_t ring = 0; ring < 2; ring++)
+        for (uint32_t i = 0; i < n; i++) {
+            out[ring * n + i] = d.slices[ring][i];
+            order[ring * n + i] = d.order[ring][i];
+        }
+    return 0;
 }
 
 int64_t orc_algorithmic_bytes_opbase(int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
