@@ -55,6 +55,24 @@ static int plan_push(const HgLaunch* l, void* ctx)
     return HCCL_SUCCESS;
 }
 
+static int ranges_meet(const void* a, uint64_t an, const void* b, uint64_t bn)
+{
+    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+    return an && bn && a0 < b0 + bn && b0 < a0 + an;
+}
+
+/* no operation of the group writes what another one reads or writes */
+static int step_is_conflict_free(const HgOp* o, uint64_t n)
+{
+    for (uint64_t a = 0; a < n; ++a)
+        for (uint64_t b = 0; b < n; ++b) {
+            if (a == b) continue;
+            if (ranges_meet(o[a].dst, o[a].bytes, o[b].dst, o[b].bytes) || ranges_meet(o[a].dst, o[a].bytes, o[b].src, o[b].bytes))
+                return 0;
+        }
+    return 1;
+}
+
 /* bufs[role][rank]: the buffer behind each role an op list may name (HCOMM_GFX_NUM_BUFS roles) */
 static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
                      int op)
@@ -74,6 +92,28 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
         o->dst = (char*)bufs[s->dstBuf][s->rank] + s->dstOff;
         o->src = (const char*)bufs[s->srcBuf][s->srcRank] + s->srcOff;
         o->bytes = s->bytes;
+    }
+    /* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the
+     * next slice) would change kernel with every operation: when nothing in the step can observe anything else in it,
+     * run its reduces first and its copies after them, each kind in its original order. */
+    for (uint64_t i = 0; i < n;) {
+        uint64_t j = i;
+        uint64_t reduces = 0;
+        while (j < n && list[j].step == list[i].step) reduces += ops[j++].is_reduce;
+        if (reduces != 0 && reduces != j - i && step_is_conflict_free(ops + i, j - i)) {
+            HgOp* tmp = (HgOp*)malloc((j - i) * sizeof(HgOp));
+            if (!tmp) {
+                free(ops);
+                return HCCL_E_MEMORY;
+            }
+            uint64_t k = 0;
+            for (int want = 1; want >= 0; --want)
+                for (uint64_t q = i; q < j; ++q)
+                    if (ops[q].is_reduce == want) tmp[k++] = ops[q];
+            memcpy(ops + i, tmp, (j - i) * sizeof(HgOp));
+            free(tmp);
+        }
+        i = j;
     }
     int rc = hg_coalesce(ops, n, plan_push, p);
     free(ops);

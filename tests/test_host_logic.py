@@ -420,6 +420,28 @@ def test_plan_from_a_callers_op_list(rec):
     assert empty.info.launches == 0 and empty.run(rec) == 0
 
 
+def test_steps_that_mix_reduces_and_copies_lower_to_one_launch_per_kind(rec):
+    """The double-ring reduce-scatter pairs every reduce with the fetch of the next slice from the user input: a step
+    of 8 ranks x 2 rings is one reduce launch and one copy launch, not 32 alternating ones.  A step whose operations
+    could observe each other keeps its order."""
+    n, count, dt = 8, 1 << 20, DT.FP32
+    bufs = [[DST + (role << 34) + (i << 26) for i in range(n)] for role in range(4)]
+    p = h.DoubleRingPlan(h.Alg.ALLREDUCE_RING, 1, n, bufs[0], bufs[1], bufs[2], bufs[3], 8 << 20, count, dt, OP.SUM)
+    kinds = [l.kind for l in p.launches()]
+    K = h.Kernel
+    assert kinds == [K.COPY] + [K.REDUCE2, K.COPY] * (n - 2) + [K.REDUCE2] + [K.COPY] + [K.COPY] * (n - 1)
+    assert [l.nseg for l in p.launches()][:3] == [32, 16, 16]
+    assert p.run(rec) == 0
+    p.destroy()
+    # copy A -> B, then B += C, then copy B -> D, all in one step: each reads what the one before wrote
+    A, B, C_, D = (DST + (i << 22) for i in range(4))
+    ops = [(0, 0, 0, 0, 1 << 22, 0, 0, 0, 4096), (0, 1, 0, 0, 1 << 22, 0, 0, 2 << 22, 4096),
+           (0, 0, 0, 0, 3 << 22, 0, 0, 1 << 22, 4096)]
+    q = h.OpListPlan(ops, 1, {0: [DST]}, dt, OP.SUM)
+    assert [l.kind for l in q.launches()] == [K.COPY, K.REDUCE2, K.COPY]
+    q.destroy()
+
+
 def test_plan_run_checks(rec):
     i, o = ptrs(2, 4096)
     p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, i, o, 1024, DT.FP32, OP.SUM)
