@@ -1,8 +1,8 @@
 /*
  * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics, of the ring, recursive
  * halving-doubling, mesh, NHR (sliced and one-shot), NB, local-reduce, chunk-mesh and doubling schedules, of the
- * executors' op-base loop around them and of the ring executor's three-step allreduce, used ONLY to check
- * libhcomm_gfx.so.
+ * executors' op-base loop around them, of the ring executor's three-step allreduce and of the double-ring executor
+ * with DMA reduce, used ONLY to check libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -47,6 +47,9 @@
  *                                     N = 2, 3, 5, 6, 8 by hand; pinned
  *   three-step allreduce ............ the complete operation list of 2 servers x 2 ranks and the reduction trees
  *                                     of 2 x 3 by hand; the one-shot threshold; exact integer results; pinned
+ *   double-ring allreduce ........... slice / ring-order tables N = 4, one rank's complete operation list N = 3, the
+ *                                     reduction trees of both shares N = 4, all by hand; exact integer results over
+ *                                     several chunks; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
