@@ -67,6 +67,8 @@ WORKLOADS = {
     "dbring_ring_ar_bf16_1x8_128MiB": ("dbring_ring_ar", (1, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "dbring_ring_ar_bf16_1x8_512MiB": ("dbring_ring_ar", (1, 8), 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
     "dbring_nhr_ar_bf16_2x8_128MiB": ("dbring_nhr", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the order-preserving reduce-scatter executor: plant into the peers' CCL output buffers, fold in rank order
+    "order_preserved_rs_bf16_n8_16MiB": ("order_preserved_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     "nhr_oneshot_ar_bf16_n8_256KiB": ("nhr_oneshot", 8, 131072, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
@@ -137,7 +139,8 @@ def main():
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
-    dt, alg, op = DT[dtname], ALG[alg_name], OP[opname]
+    plant = alg_name == "order_preserved_rs"
+    dt, alg, op = DT[dtname], (None if plant else ALG[alg_name]), OP[opname]
     unit = h.DTYPE_SIZE[dt]
     in_place = alg_name == "ring_rs_stage"
 
@@ -152,7 +155,7 @@ def main():
         return
 
     nbytes = count * unit
-    in_count = n * count if alg_name == "local_reduce_rs" else count  # a scatter's input holds N slices of count
+    in_count = n * count if alg_name in ("local_reduce_rs", "order_preserved_rs") else count  # N slices of count
     pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
     d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
@@ -166,14 +169,14 @@ def main():
 
     in_ptrs = [t.data_ptr() for t in d_in]
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
-    scratch_bytes = h.scratch_bytes(alg, n, count, dt)
+    scratch_bytes = 0 if plant else h.scratch_bytes(alg, n, count, dt)
     d_ccl = None
-    if opbase or dbring:
+    if opbase or dbring or plant:
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both":
             args.lowering = "stepwise"
-    if hier:
-        args.lowering = "stepwise"  # composed from the step lists of its three levels
+    if hier or plant:
+        args.lowering = "stepwise"  # composed from the step lists of its levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
     if alg_name in ("local_reduce", "chunk_mesh", "local_reduce_rs") and args.lowering == "both":
@@ -182,6 +185,8 @@ def main():
              h.Kernel.COPY: "k_copy"}
 
     def make_plan(low):
+        if plant:
+            return h.OrderPreservedPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if dbring:
             return h.DoubleRingPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                     [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
@@ -271,14 +276,17 @@ def main():
                 "ring_rs_stage": oracle.ALG_RS_RING_STAGE, "mesh_oneshot": oracle.ALG_ALLREDUCE_MESH_ONESHOT,
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
-                "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT}[alg_name]
+                "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
+                "order_preserved_rs": None}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
         host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
-        if dbring:
+        if plant:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved(n, count, ccl_bytes, odt))
+        elif dbring:
             alg_bytes = sum(o[8] * (3 if o[1] else 2)
                             for o in oracle.trace_dbring(oalg, hier[0], hier[1], count, ccl_bytes, odt))
         elif hier:
@@ -286,10 +294,12 @@ def main():
         else:
             alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
                          else oracle.algorithmic_bytes(oalg, n, count, odt))
-        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if (opbase or dbring) else None
+        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if (opbase or dbring or plant) else None
 
         def cpu_run(ins, outs):
-            if dbring:
+            if plant:
+                oracle.run_order_preserved(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
+            elif dbring:
                 oracle.run_dbring(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif hier:
                 oracle.run_hier(oalg, hier[0], hier[1], ins, outs, count, odt, oop)
@@ -363,7 +373,7 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
-                if opbase or dbring:  # what the last chunk left in the CCL buffers
+                if opbase or dbring or plant:  # what the last chunk left in the CCL buffers
                     ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
@@ -393,7 +403,7 @@ def main():
                    **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": alg_name,
                        "level0_algorithm": ("double-ring reduce-scatter + all-gather on user memory (DMA reduce)"
                                             if dbring else "ring reduce-scatter + ring all-gather")} if hier else {}),
-                   **({"ccl_buffer_bytes": ccl_bytes} if dbring else {})},
+                   **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant) else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

@@ -28,6 +28,7 @@ __all__ = [
     "HcommThreadNotifyWaitOnThreadWithDefaultTimeout", "HcommThreadResAcquireTimeOut", "HcommFenceOnThread",
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
+    "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -483,6 +484,41 @@ class DoubleRingPlan(Plan):
         p = _vp(0)
         check(_dbring_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3],
                            ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxDoubleRingPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_op_emit = _sig("HcommGfxOrderPreservedEmit", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_op_check = _sig("HcommGfxOrderPreservedCheck", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_op_plan = _sig("HcommGfxOrderPreservedPlanCreate", _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u64,
+                _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def order_preserved_emit(n_ranks, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_op_emit(n_ranks, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxOrderPreservedEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_op_emit(n_ranks, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxOrderPreservedEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def order_preserved_check(n_ranks, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_op_check(n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxOrderPreservedCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class OrderPreservedPlan(Plan):
+    """HcommGfxOrderPreservedPlanCreate: the order-preserving reduce-scatter executor on one server, op-base mode."""
+
+    def __init__(self, user_in, user_out, ccl_out, ccl_bytes, count, dtype, op):
+        n = len(user_in)
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_out)]
+        p = _vp(0)
+        check(_op_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
+              "HcommGfxOrderPreservedPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

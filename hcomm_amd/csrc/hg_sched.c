@@ -1069,6 +1069,71 @@ int32_t HcommGfxDoubleRingEmit(
     return HCCL_SUCCESS;
 }
 
+/* ---- the order-preserving reduce-scatter executor (one server, op-base mode) ------------------------------------- */
+
+/* CollReduceScatterOrderPreservedExecutor (coll_executor/coll_reduce_scatter/
+ * coll_reduce_scatter_order_preserved_executor.cc:181-216, 260-283) around ReduceScatterPlantLocalReduce
+ * (alg_template/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc), chunked by the reduce-scatter loop
+ * (coll_reduce_scatter_executor.cc:149-220, DMA reduce: no staging copies).  Per chunk of c bytes:
+ *   step 0: every rank q plants block p of its user input into slot (p + q) mod N of rank p's CCL output buffer
+ *           (:166-185, :211-240) - so on every rank the slots, read from its own rank number on, hold the
+ *           contributions of ranks 0, 1, 2, ... in that order;
+ *   ceil(log2 N) rounds (:336-407): the contributions h .. min(N, 2h) - 1 are folded onto 0 .. for h = 2^(S-1), .., 1
+ *           - the same tree over RANK order on every rank, which is what "order preserving" means;
+ *   last step: slot p of rank p to its user output (:273-279). */
+static int order_preserved_build(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, uint32_t unit)
+{
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint32_t rounds = ceil_log2(n);
+    const uint64_t stride = count * unit;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        for (uint32_t p = 0; p < n; ++p) /* destination rank; q == p is the rank's own block */
+            for (uint32_t q = 0; q < n; ++q) CHK(push(l, step, COPY, p, OUT, c * ((p + q) % n), q, UIN, user_off + stride * p, c));
+        ++step;
+        for (uint32_t h = 1u << (rounds ? rounds - 1 : 0); rounds && h >= 1; h >>= 1, ++step)
+            for (uint32_t p = 0; p < n; ++p)
+                for (uint32_t j = 0; j + h < (n < 2 * h ? n : 2 * h); ++j)
+                    CHK(push(l, step, REDUCE, p, OUT, c * ((j + p) % n), p, OUT, c * ((h + j + p) % n), c));
+        for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, user_off, p, OUT, c * p, c));
+        ++step;
+        user_off += c;
+        left -= cur;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_order_preserved(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    const int rc = order_preserved_build(l, n, count, ccl_bytes, unit);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved(&l, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 int32_t HcommGfxHierEmit(
     HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
     HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)

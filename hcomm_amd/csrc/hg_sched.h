@@ -25,6 +25,9 @@ int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local
  * buffers of ccl_bytes in between, chunked like the op-base loop. */
 int hg_schedule_dbring(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
                        int dtype);
+/* The order-preserving reduce-scatter executor on one server: all-to-all into the CCL output buffers, a fold tree in
+ * rank order, own slot to the user output; chunked like the reduce-scatter loop. */
+int hg_schedule_order_preserved(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 void hg_oplist_free(HgOpList* l);
 /* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);

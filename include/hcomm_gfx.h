@@ -626,6 +626,27 @@ int32_t HcommGfxDoubleRingCheck(
     HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
+ * The reduce-scatter of the reference's order-preserving executor on one server in op-base mode
+ * (coll_executor/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:181-216, 260-283, around
+ * ReduceScatterPlantLocalReduce, alg_template/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc): per chunk of
+ * at most cclBytes / nRanks (rounded down to 128 bytes) / unit elements, every rank plants block p of its user input
+ * into rank p's CCL output buffer, every rank folds the N blocks it received in RANK order along one fixed tree
+ * (so the result does not depend on which rank computes it), and copies its slot to its user output.
+ * userIn: nRanks * count elements (block p at p * count); userOut: count elements; cclOut: cclBytes; 128-byte
+ * aligned.  nRanks >= 2 (a single rank per module relies on the inter-module stage, which is not built); the
+ * executor's recursive-halving branch for messages up to 32 KiB on 4 or 8 devices (:33-38) is not built either: this
+ * entry point always takes the plant branch.  Step-wise lowering.
+ */
+int32_t HcommGfxOrderPreservedPlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxOrderPreservedEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n);
+int32_t HcommGfxOrderPreservedCheck(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
  * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand
  * to the dispatcher (HcclD2DMemcpyAsync / HcclReduceAsync, src/legacy/ascend910/platform/task/
  * dispatcher_common.cc:114-147), ordered by step.  buffers[role][rank] gives the device buffer behind each of the

@@ -105,6 +105,11 @@ def lib():
         L.orc_run_dbring.argtypes = [C.c_int, C.c_uint32, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + \
             [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
         L.orc_dbring_slices.restype = C.c_int
+        L.orc_trace_order_preserved.restype = C.c_int64
+        L.orc_trace_order_preserved.argtypes = [C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
+        L.orc_run_order_preserved.restype = C.c_int
+        L.orc_run_order_preserved.argtypes = [C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + \
+            [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run.restype = C.c_int
@@ -317,3 +322,22 @@ def dbring_slices(count, dtype, n):
         raise ValueError("orc_dbring_slices rc=%d" % rc)
     return ([[(sl[r * n + i].offset, sl[r * n + i].size) for i in range(n)] for r in range(2)],
             [[order[r * n + i] for i in range(n)] for r in range(2)])
+
+
+# ---- the order-preserving reduce-scatter executor (plant local reduce, one server, op-base mode) ----------
+
+def trace_order_preserved(n, count, ccl_bytes, dtype):
+    total = lib().orc_trace_order_preserved(n, count, ccl_bytes, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_order_preserved rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_order_preserved(n, count, ccl_bytes, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_order_preserved(user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype, op):
+    n = len(user_in)
+    arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in b]) for b in (user_in, user_out, ccl_in, ccl_out)]
+    rc = lib().orc_run_order_preserved(n, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
+    if rc:
+        raise ValueError("orc_run_order_preserved rc=%d" % rc)

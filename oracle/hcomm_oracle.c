@@ -1749,6 +1749,105 @@ int orc_dbring_slices(uint64_t count, int dtype, uint32_t n, OrcSlice* out, uint
     return 0;
 }
 
+/* ---- the order-preserving reduce-scatter executor (one server, op-base mode) ----------------------------------- */
+
+/* ReduceScatterPlantLocalReduce::RunAsync for one rank and one group, tpl/temp_reduce_scatter/
+ * reduce_scatter_plant_local_reduce.cc:106-164, as CollReduceScatterOrderPreservedExecutor::RunReduceScatterLevel0
+ * prepares it for a single module (exec/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:181-216):
+ * every block cur_size bytes, block d of the user input at d * stride bytes, slot d of the CCL output buffer at
+ * d * cur_size, all2allOffset 0, no borrowed space.  Steps: 0 the all-to-all, 1.. the local reduce rounds. */
+static void prog_plant_local_reduce(OrcTrace* t, uint32_t local_rank, uint32_t rank_size, uint64_t cur_size, uint64_t stride)
+{
+    const uint32_t all2all_offset = 0;
+#define CALC_OUTPUT_INDEX(round) ((all2all_offset + (round) + local_rank) % rank_size) /* :90-93 */
+    /* LocalCopy, :166-185 */
+    emit(t, 0, K_COPY, local_rank, B_OUT, cur_size * CALC_OUTPUT_INDEX(local_rank), local_rank, B_UIN, stride * local_rank,
+         cur_size);
+    /* RunAlltoAll, :211-240: block `round` of the own user input planted into rank `round`'s output memory */
+    for (uint32_t round = 0; round < rank_size; round++) {
+        if (round == local_rank) continue;
+        emit(t, 0, K_COPY, round, B_OUT, cur_size * CALC_OUTPUT_INDEX(round), local_rank, B_UIN, stride * round, cur_size);
+    }
+    /* RunLocalReduce, :336-407 */
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < rank_size) reduce_step++; /* ceil(log2(rankSize)) */
+    for (uint32_t round = 0; round < reduce_step; round++) {
+        const uint32_t full = 1u << (reduce_step - round);
+        const uint32_t tail_index = (rank_size < full ? rank_size : full) - 1;
+        const uint32_t head_index = 1u << (reduce_step - round - 1);
+        for (uint32_t offset = 0; offset <= tail_index - head_index; offset++) {
+            const uint32_t input_index = CALC_OUTPUT_INDEX(head_index + offset);
+            const uint32_t output_index = CALC_OUTPUT_INDEX(offset);
+            emit(t, 1 + round, K_REDUCE, local_rank, B_OUT, cur_size * output_index, local_rank, B_OUT, cur_size * input_index,
+                 cur_size);
+        }
+    }
+#undef CALC_OUTPUT_INDEX
+}
+
+/* CollReduceScatterOrderPreservedExecutor::KernelRun for one rank inside CollReduceScatterExecutor::RunLoop
+ * (exec/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:260-283 with DMAReduceFlag_, :19;
+ * exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:149-220): one module, the plant branch. */
+static int build_trace_order_preserved(OrcTrace* t, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    /* one rank per module takes RunReduceScatterLevel0SingleRank (:134-150), which relies on the level-1 stage that a
+     * single module does not have: not restated */
+    if (unit == 0 || n < 2 || n > ORC_MAX_RANKS) return -1;
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit; /* CalcLoopMaxCount, coll_reduce_scatter_executor.cc:124-134 */
+    if (max_count == 0) return -1;
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < n) reduce_step++;
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        const uint64_t cur_size = cur_count * unit;
+        g_user_off = user_off;
+        for (uint32_t r = 0; r < n; r++) {
+            g_step_base = step0;
+            prog_plant_local_reduce(t, r, n, cur_size, count * unit);
+            /* :273-279: the own slot of the scratch (= CCL output) memory to the user output */
+            g_step_base = step0 + 1 + reduce_step;
+            emit(t, 0, K_COPY, r, B_UOUT, 0, r, B_OUT, cur_size * r, cur_size);
+        }
+        g_user_off = 0;
+        g_step_base = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += 2 + reduce_step;
+        user_off += cur_size;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_order_preserved(uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_order_preserved(uint32_t n, void* const* user_in, void* const* user_out, void* const* ccl_in,
+                            void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
 int64_t orc_algorithmic_bytes_opbase(int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
 {
     OrcTrace t;
