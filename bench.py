@@ -62,6 +62,8 @@ WORKLOADS = {
     "opbase_ring_ar_bf16_n8_512MiB": ("opbase_ring_ar", 8, 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
     # the ring executor's three-step allreduce: 4 servers x 8 ranks, NHR / ring between the servers
     "hier_nhr_ar_bf16_4x8_128MiB": ("hier_nhr", (4, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "meshhier_ring_ar_bf16_2x8_128MiB": ("meshhier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "meshhier_ring_ar_bf16_1x8_128MiB": ("meshhier_ring_ar", (1, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "hier_ring_ar_bf16_2x8_128MiB": ("hier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the double-ring executor in op-base mode with DMA reduce: user buffers read and written directly, 200 MiB CCL buffers
     "dbring_ring_ar_bf16_1x8_128MiB": ("dbring_ring_ar", (1, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -135,7 +137,8 @@ def main():
         alg_name = alg_name[len("opbase_"):]
     hier = None  # (servers, ranks per server): the level-1 template inside the ring executor's three steps
     dbring = False  # the double-ring executor with DMA reduce instead of the single ring on staged buffers
-    if alg_name.startswith("hier_") or alg_name.startswith("dbring_"):
+    mesh0 = alg_name.startswith("meshhier_")  # the mesh executor's level 0 instead of the ring executor's
+    if alg_name.startswith("hier_") or alg_name.startswith("dbring_") or mesh0:
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
@@ -191,7 +194,7 @@ def main():
             return h.DoubleRingPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                     [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if hier:
-            return h.HierPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, count, dt, op)
+            return h.HierPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, count, dt, op, mesh=mesh0)
         if opbase:
             return h.OpBasePlan(alg, low, in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                 [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, scr_ptrs)
@@ -290,7 +293,8 @@ def main():
             alg_bytes = sum(o[8] * (3 if o[1] else 2)
                             for o in oracle.trace_dbring(oalg, hier[0], hier[1], count, ccl_bytes, odt))
         elif hier:
-            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_hier(oalg, hier[0], hier[1], count, odt))
+            alg_bytes = sum(o[8] * (3 if o[1] else 2)
+                            for o in oracle.trace_hier(oalg, hier[0], hier[1], count, odt, mesh=mesh0))
         else:
             alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
                          else oracle.algorithmic_bytes(oalg, n, count, odt))
@@ -302,7 +306,7 @@ def main():
             elif dbring:
                 oracle.run_dbring(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif hier:
-                oracle.run_hier(oalg, hier[0], hier[1], ins, outs, count, odt, oop)
+                oracle.run_hier(oalg, hier[0], hier[1], ins, outs, count, odt, oop, mesh=mesh0)
             elif opbase:
                 oracle.run_opbase(oalg, ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop, scratch=host_scr)
             else:
@@ -382,7 +386,7 @@ def main():
     h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
-        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("double-ring " if dbring else "three-step " if hier else "") + alg_name, opname)
+        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("double-ring " if dbring else "mesh three-step " if mesh0 else "three-step " if hier else "") + alg_name, opname)
     out = {
         "metric": metric,
         "value": round(res["gbs"], 2),
@@ -402,7 +406,8 @@ def main():
                    **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {}),
                    **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": alg_name,
                        "level0_algorithm": ("double-ring reduce-scatter + all-gather on user memory (DMA reduce)"
-                                            if dbring else "ring reduce-scatter + ring all-gather")} if hier else {}),
+                                            if dbring else "multi-stream mesh reduce-scatter + mesh all-gather" if mesh0
+                                            else "ring reduce-scatter + ring all-gather")} if hier else {}),
                    **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant) else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),

@@ -437,19 +437,26 @@ _hier_emit = _sig("HcommGfxHierEmit", _i32, C.c_int, _u32, _u32, _u64, C.c_int, 
 _hier_check = _sig("HcommGfxHierCheck", _i32, C.c_int, _u32, _u32, _u64, C.c_int, C.POINTER(CheckReport))
 _hier_plan = _sig("HcommGfxHierPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
                   C.c_int, C.POINTER(_vp))
+_mesh_emit = _sig("HcommGfxMeshHierEmit", _i32, C.c_int, _u32, _u32, _u64, C.c_int, C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_mesh_check = _sig("HcommGfxMeshHierCheck", _i32, C.c_int, _u32, _u32, _u64, C.c_int, C.POINTER(CheckReport))
+_mesh_plan = _sig("HcommGfxMeshHierPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
+                  C.c_int, C.POINTER(_vp))
 
 
-def hier_emit(alg1, n_servers, n_local, count, dtype):
+def hier_emit(alg1, n_servers, n_local, count, dtype, mesh=False):
+    """mesh: the mesh executor's level 0 (HcommGfxMeshHier*) instead of the ring executor's."""
+    f, name = (_mesh_emit, "HcommGfxMeshHierEmit") if mesh else (_hier_emit, "HcommGfxHierEmit")
     n = _u64(0)
-    check(_hier_emit(alg1, n_servers, n_local, count, dtype, None, 0, C.byref(n)), "HcommGfxHierEmit")
+    check(f(alg1, n_servers, n_local, count, dtype, None, 0, C.byref(n)), name)
     ops = (SchedOp * max(n.value, 1))()
-    check(_hier_emit(alg1, n_servers, n_local, count, dtype, ops, n.value, C.byref(n)), "HcommGfxHierEmit")
+    check(f(alg1, n_servers, n_local, count, dtype, ops, n.value, C.byref(n)), name)
     return [ops[i].astuple() for i in range(n.value)]
 
 
-def hier_check(alg1, n_servers, n_local, count, dtype):
+def hier_check(alg1, n_servers, n_local, count, dtype, mesh=False):
     rep = CheckReport()
-    check(_hier_check(alg1, n_servers, n_local, count, dtype, C.byref(rep)), "HcommGfxHierCheck")
+    f, name = (_mesh_check, "HcommGfxMeshHierCheck") if mesh else (_hier_check, "HcommGfxHierCheck")
+    check(f(alg1, n_servers, n_local, count, dtype, C.byref(rep)), name)
     return rep.conflicts, rep.semanticErrors, rep.message.decode()
 
 
@@ -526,14 +533,15 @@ class OrderPreservedPlan(Plan):
 
 
 class HierPlan(Plan):
-    """HcommGfxHierPlanCreate: ring reduce-scatter inside the servers, alg1 between them, ring all-gather inside."""
+    """HcommGfxHierPlanCreate: ring reduce-scatter inside the servers, alg1 between them, ring all-gather inside;
+    mesh=True: HcommGfxMeshHierPlanCreate, the mesh executor's multi-stream reduce-scatter and mesh all-gather."""
 
-    def __init__(self, alg1, n_servers, n_local, in_ptrs, out_ptrs, count, dtype, op):
+    def __init__(self, alg1, n_servers, n_local, in_ptrs, out_ptrs, count, dtype, op, mesh=False):
         n = n_servers * n_local
         self._in, self._out = (_vp * n)(*in_ptrs), (_vp * n)(*out_ptrs)
         p = _vp(0)
-        check(_hier_plan(alg1, n_servers, n_local, self._in, self._out, count, dtype, op, C.byref(p)),
-              "HcommGfxHierPlanCreate")
+        f, name = (_mesh_plan, "HcommGfxMeshHierPlanCreate") if mesh else (_hier_plan, "HcommGfxHierPlanCreate")
+        check(f(alg1, n_servers, n_local, self._in, self._out, count, dtype, op, C.byref(p)), name)
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxHierPlanGetInfo")

@@ -312,7 +312,21 @@ int32_t HcommGfxHierCheck(
 {
     if (!rep) return HCCL_E_PTR;
     HgOpList l;
-    int rc = hg_schedule_hier(&l, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    int rc = hg_schedule_hier(&l, 0, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = HcommGfxOpListCheck(l.ops, l.n, nServers * nLocal, HCOMM_GFX_EXPECT_ALLREDUCE, count, 0,
+                             HcommGfxDataTypeSize(dataType), rep);
+    hg_oplist_free(&l);
+    return rc;
+}
+
+int32_t HcommGfxMeshHierCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxCheckReport* rep)
+{
+    if (!rep) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_hier(&l, 1, (int)level1Alg, nServers, nLocal, count, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     rc = HcommGfxOpListCheck(l.ops, l.n, nServers * nLocal, HCOMM_GFX_EXPECT_ALLREDUCE, count, 0,
                              HcommGfxDataTypeSize(dataType), rep);

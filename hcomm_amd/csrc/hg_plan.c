@@ -591,7 +591,28 @@ int32_t HcommGfxHierPlanCreate(
     if (rc == HCCL_SUCCESS) rc = check_bufs(out, nServers * nLocal);
     if (rc != HCCL_SUCCESS) return rc;
     HgOpList ol;
-    rc = hg_schedule_hier(&ol, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    rc = hg_schedule_hier(&ol, 0, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {in, out, NULL, NULL, NULL};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nServers * nLocal, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
+}
+
+int32_t HcommGfxMeshHierPlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* in, void* const* out, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!in || !out) return HCCL_E_PTR;
+    if (nServers == 0 || nLocal == 0 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(in, nServers * nLocal);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(out, nServers * nLocal);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_hier(&ol, 1, (int)level1Alg, nServers, nLocal, count, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     void* const* bufs[HCOMM_GFX_NUM_BUFS] = {in, out, NULL, NULL, NULL};
     rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nServers * nLocal, bufs, dataType, reduceOp, plan);

@@ -867,7 +867,41 @@ static void order_by_step_rank(HgOpList* l)
  *      (:156-158, :209-211; segment = local rank, coll_comm_executor.cc:2565-2575);
  *   3. inside every server, ring all-gather on the outputs (MultiRingAllGather :228-230; input == output there,
  *      coll_comm_executor.cc:377-379, so the template's own-slice copy does not happen, all_gather_ring.cc:117). */
-int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype)
+/* Level 0 of CollAllReduceMeshExecutor::KernelRun (coll_executor/coll_all_reduce/coll_all_reduce_mesh_executor.cc:
+ * 116-119, 204-228) for one server whose ranks are g0 .. g0 + n - 1:
+ *   reduce-scatter (MultiStreamReduceScatterMesh, coll_comm_executor.cc:1754-1860): segment r is cut into n - 1 pieces
+ *   of ceil(size / (n - 1)) bytes rounded up to 128 (PrepareSliceMeshStreams, alg_template_base.cc:823-865), one per
+ *   stream; in round k = 1 .. n - 1 stream s folds its piece of rank r - 1 - ((k + s - 1) mod (n - 1))'s input into
+ *   rank r's (reduce_scatter_mesh.cc:56-68): every stream meets the peers in the same cyclic order, each starting at
+ *   its own place, so that in every round the n - 1 streams read n - 1 different peers;
+ *   all-gather (AllGatherMesh, all_gather_mesh.cc:66-131, on the outputs): every rank fetches every other rank's
+ *   segment, all at once. */
+static int mesh_level0_rs(HgOpList* l, uint32_t g0, uint32_t n, const HcommGfxSlice* seg, uint32_t step)
+{
+    for (uint32_t k = 1; k < n; ++k)
+        for (uint32_t r = 0; r < n; ++r) {
+            const uint64_t per = ((seg[r].size + (n - 2)) / (n - 1) + 127u) / 128u * 128u;
+            for (uint32_t s = 0; s + 1 < n; ++s) {
+                const uint64_t lo = (uint64_t)s * per < seg[r].size ? (uint64_t)s * per : seg[r].size;
+                const uint64_t len = seg[r].size - lo < per ? seg[r].size - lo : per;
+                const uint32_t src = (r + 2u * n - 1u - ((k + s - 1u) % (n - 1u))) % n;
+                CHK(push(l, step + k - 1, REDUCE, g0 + r, IN, seg[r].offset + lo, g0 + src, IN, seg[r].offset + lo, len));
+            }
+        }
+    return HCCL_SUCCESS;
+}
+
+static int mesh_level0_ag(HgOpList* l, uint32_t g0, uint32_t n, const HcommGfxSlice* seg, uint32_t step)
+{
+    for (uint32_t r = 0; r < n; ++r)
+        for (uint32_t k = 1; k < n; ++k) {
+            const uint32_t peer = (r + n - k) % n;
+            CHK(push(l, step, COPY, g0 + r, OUT, seg[peer].offset, g0 + peer, OUT, seg[peer].offset, seg[peer].size));
+        }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_hier(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype)
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
@@ -882,8 +916,10 @@ int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local
     int rc = HCCL_SUCCESS;
     uint32_t step = 0, used = 0;
     /* 1 */
-    rc = hg_schedule(&sub, HCOMM_GFX_ALG_REDUCE_SCATTER_RING, n_local, count, count, dtype);
-    if (rc == HCCL_SUCCESS) {
+    if (level0_mesh) {
+        for (uint32_t s = 0; s < n_servers && rc == HCCL_SUCCESS; ++s) rc = mesh_level0_rs(l, s * n_local, n_local, seg, step);
+        used = n_local - 1;
+    } else if ((rc = hg_schedule(&sub, HCOMM_GFX_ALG_REDUCE_SCATTER_RING, n_local, count, count, dtype)) == HCCL_SUCCESS) {
         for (uint32_t s = 0; s < n_servers && rc == HCCL_SUCCESS; ++s) {
             for (uint32_t j = 0; j < n_local; ++j) map[j] = s * n_local + j;
             rc = append_mapped(l, &sub, map, step, 0, 0, &used);
@@ -906,8 +942,9 @@ int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local
     step += used;
     /* 3 */
     used = 0;
-    if (rc == HCCL_SUCCESS) rc = hg_schedule(&sub, HCOMM_GFX_ALG_ALLREDUCE_RING, n_local, count, count, dtype);
-    if (rc == HCCL_SUCCESS) {
+    if (level0_mesh) {
+        for (uint32_t s = 0; s < n_servers && rc == HCCL_SUCCESS; ++s) rc = mesh_level0_ag(l, s * n_local, n_local, seg, step);
+    } else if (rc == HCCL_SUCCESS && (rc = hg_schedule(&sub, HCOMM_GFX_ALG_ALLREDUCE_RING, n_local, count, count, dtype)) == HCCL_SUCCESS) {
         /* the gather rounds of the ring allreduce are the ops that move output to output; renumber them from 0 */
         uint32_t first = UINT32_MAX;
         for (uint64_t i = 0; i < sub.n; ++i)
@@ -1140,7 +1177,24 @@ int32_t HcommGfxHierEmit(
 {
     if (!n) return HCCL_E_PTR;
     HgOpList l;
-    int rc = hg_schedule_hier(&l, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    int rc = hg_schedule_hier(&l, 0, (int)level1Alg, nServers, nLocal, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxMeshHierEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_hier(&l, 1, (int)level1Alg, nServers, nLocal, count, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     *n = l.n;
     if (ops) {

@@ -19,8 +19,9 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
  * into the CCL input buffer, run through the template, and copied from the CCL output to the user output. */
 int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 uint64_t hg_opbase_max_count(int alg, uint32_t n, uint64_t ccl_bytes, uint32_t unit);
-/* The ring executor's three-step allreduce over n_servers x n_local ranks with alg1 between the servers. */
-int hg_schedule_hier(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype);
+/* The ring executor's (level0_mesh 0) or the mesh executor's (1) three-step allreduce over n_servers x n_local ranks
+ * with alg1 between the servers. */
+int hg_schedule_hier(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype);
 /* The double-ring allreduce executor in op-base mode with DMA reduce: user buffers read and written directly, CCL
  * buffers of ccl_bytes in between, chunked like the op-base loop. */
 int hg_schedule_dbring(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,

@@ -597,6 +597,24 @@ int32_t HcommGfxHierCheck(
     HcommGfxCheckReport* report);
 
 /*
+ * The same three steps with the mesh executor's level 0
+ * (coll_executor/coll_all_reduce/coll_all_reduce_mesh_executor.cc:88-231, its branch without atomic adds):
+ * (1) MultiStreamReduceScatterMesh inside every server (coll_comm_executor.cc:1754-1860): every segment cut into
+ * nLocal - 1 pieces, piece s folded from the peers in the cyclic order r-1, r-2, ... started at place s, in place on the
+ * inputs; (2) as above; (3) AllGatherMesh inside every server on the outputs (alg_template/temp_all_gather/
+ * all_gather_mesh.cc:66-131), all segments at once.
+ */
+int32_t HcommGfxMeshHierPlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* in, void* const* out, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxMeshHierEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+int32_t HcommGfxMeshHierCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
+    HcommGfxCheckReport* report);
+
+/*
  * The allreduce of the reference's double-ring executor for two-ring servers in op-base mode, where the user buffers
  * are read and written directly ("DMA reduce") instead of being staged through the CCL buffers
  * (coll_executor/coll_all_reduce/coll_aligned_all_reduce_double_ring_for_910_93_executor.cc, KernelRun of

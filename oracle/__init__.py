@@ -94,9 +94,10 @@ def lib():
         L.orc_algorithmic_bytes_opbase.restype = C.c_int64
         L.orc_algorithmic_bytes_opbase.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int]
         L.orc_trace_hier.restype = C.c_int64
-        L.orc_trace_hier.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
+        L.orc_trace_hier.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp),
+                                     C.c_uint64]
         L.orc_run_hier.restype = C.c_int
-        L.orc_run_hier.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+        L.orc_run_hier.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
                                    C.c_uint64, C.c_int, C.c_int]
         L.orc_trace_dbring.restype = C.c_int64
         L.orc_trace_dbring.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.POINTER(OrcOp),
@@ -276,20 +277,21 @@ def algorithmic_bytes_opbase(alg, n, count, ccl_bytes, dtype):
 
 # ---- the ring executor's three-step allreduce over two communicator levels -------------------------------
 
-def trace_hier(alg1, n_servers, n_local, count, dtype):
-    total = lib().orc_trace_hier(alg1, n_servers, n_local, count, dtype, None, 0)
+def trace_hier(alg1, n_servers, n_local, count, dtype, mesh=False):
+    """mesh: the mesh executor's level 0 (multi-stream mesh reduce-scatter, mesh all-gather) instead of the ring's."""
+    total = lib().orc_trace_hier(int(mesh), alg1, n_servers, n_local, count, dtype, None, 0)
     if total < 0:
         raise ValueError("orc_trace_hier rc=%d" % total)
     ops = (OrcOp * max(total, 1))()
-    lib().orc_trace_hier(alg1, n_servers, n_local, count, dtype, ops, total)
+    lib().orc_trace_hier(int(mesh), alg1, n_servers, n_local, count, dtype, ops, total)
     return [ops[i].astuple() for i in range(total)]
 
 
-def run_hier(alg1, n_servers, n_local, ins, outs, count, dtype, op):
+def run_hier(alg1, n_servers, n_local, ins, outs, count, dtype, op, mesh=False):
     n = len(ins)
     a = (C.c_void_p * n)(*[x.ctypes.data for x in ins])
     b = (C.c_void_p * n)(*[x.ctypes.data for x in outs])
-    rc = lib().orc_run_hier(alg1, n_servers, n_local, a, b, count, dtype, op)
+    rc = lib().orc_run_hier(int(mesh), alg1, n_servers, n_local, a, b, count, dtype, op)
     if rc:
         raise ValueError("orc_run_hier rc=%d" % rc)
 

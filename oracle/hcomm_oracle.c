@@ -1430,6 +1430,62 @@ int orc_run_opbase(int alg, uint32_t n, void* const* user_in, void* const* user_
 
 /* ---- the ring executor's three-step allreduce over two communicator levels ----------------------------------- */
 
+/* ExecutorBase::PrepareSliceMeshStreams, tpl/alg_template_base.cc:823-865: every segment cut into stream_count pieces of
+ * ceil(size / stream_count) bytes rounded up to 128; out[stream][rank] */
+static void slices_mesh_streams(const OrcSlice* seg, uint32_t n, uint32_t stream_count, OrcSlice out[][ORC_MAX_RANKS])
+{
+    uint64_t rank_stream_size[ORC_MAX_RANKS], rank_residue[ORC_MAX_RANKS];
+    for (uint32_t rank_id = 0; rank_id < n; rank_id++) {
+        const uint64_t size_per_stream = (seg[rank_id].size + stream_count - 1) / stream_count;
+        rank_stream_size[rank_id] = (size_per_stream + 127) / 128 * 128;
+        rank_residue[rank_id] = seg[rank_id].size;
+    }
+    for (uint32_t stream = 0; stream < stream_count; stream++)
+        for (uint32_t rank_id = 0; rank_id < n; rank_id++) {
+            const uint64_t residue = rank_residue[rank_id];
+            if (residue > 0) {
+                const uint64_t single = rank_stream_size[rank_id] < residue ? rank_stream_size[rank_id] : residue;
+                out[stream][rank_id].offset = seg[rank_id].offset + seg[rank_id].size - residue;
+                out[stream][rank_id].size = single;
+                rank_residue[rank_id] -= single;
+            } else {
+                out[stream][rank_id].offset = seg[rank_id].offset;
+                out[stream][rank_id].size = 0;
+            }
+        }
+}
+
+/* CollCommExecutor::MultiStreamReduceScatterMesh (exec/coll_comm_executor.cc:1754-1860): one ReduceScatterMesh per
+ * stream on that stream's pieces, input memory == output memory (no final copy), each starting its walk through the
+ * default peer order at its stream index (tpl/temp_reduce_scatter/reduce_scatter_mesh.cc:51-68); the streams run side
+ * by side, so round k of all of them is one lock-step step.  Inline reduce (:40-46). */
+static void prog_mesh_rs_streams(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* seg)
+{
+    if (n == 1) return; /* :141-146 with inputMem_ == outputMem_ */
+    static OrcSlice stream_slices[ORC_MAX_RANKS][ORC_MAX_RANKS];
+    slices_mesh_streams(seg, n, n - 1, stream_slices);
+    uint32_t rx_rank_op_order[ORC_MAX_RANKS];
+    for (uint32_t round = 1; round < n; round++) rx_rank_op_order[round - 1] = (rank + n - round) % n; /* ForwardRank */
+    for (uint32_t stream_index = 0; stream_index < n - 1; stream_index++)
+        for (uint32_t round = 1; round < n; round++) {
+            const uint32_t order_index = (round + stream_index - 1) % (n - 1);
+            const uint32_t src_rank = rx_rank_op_order[order_index];
+            const OrcSlice* own = &stream_slices[stream_index][rank];
+            emit(t, round - 1, K_REDUCE, rank, B_IN, own->offset, src_rank, B_IN, own->offset, own->size);
+        }
+}
+
+/* AllGatherMesh::RunAllGather, tpl/temp_all_gather/all_gather_mesh.cc:66-131, prepared with the output memory as both
+ * input and output (exec/coll_all_reduce/coll_all_reduce_mesh_executor.cc:219-222): round r fetches the slice of rank
+ * BackwardRank(rank, r) = rank - r (base/inc/all_gather_mesh_pub.h:33-39) on a stream of its own, all rounds at once. */
+static void prog_mesh_ag(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* seg)
+{
+    for (uint32_t round = 1; round < n; round++) {
+        const uint32_t dst_rank = (rank + n - round) % n;
+        emit(t, 0, K_COPY, rank, B_OUT, seg[dst_rank].offset, dst_rank, B_OUT, seg[dst_rank].offset, seg[dst_rank].size);
+    }
+}
+
 /* coll_all_reduce_ring_executor.cc:171-181: curSize / deviceNumPerAggregation <= NHR_ALLREDUCE_SMALL_SIZE
  * (256 KiB, pub_inc/op_context.h:18) selects the one-shot NHR template; the devices of an aggregation are the
  * n_local ranks of a server here. */
@@ -1442,8 +1498,8 @@ static int hier_level1_template(int alg1, uint64_t count, uint32_t unit, uint32_
 
 /* CollAllReduceRingExecutor::KernelRun for one rank, exec/coll_all_reduce/coll_all_reduce_ring_executor.cc:94-231,
  * single ring per server (ringNum == 1, :123-125), buffer-copy mode.  rank = server * n_local + local index. */
-static int prog_hier_allreduce(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local, uint64_t count,
-                               int dtype, uint32_t level1_steps)
+static int prog_hier_allreduce(OrcTrace* t, int level0_mesh, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local,
+                               uint64_t count, int dtype, uint32_t level1_steps)
 {
     const uint32_t unit = orc_dtype_size(dtype);
     const uint32_t server = rank / n_local, local = rank % n_local;
@@ -1455,7 +1511,8 @@ static int prog_hier_allreduce(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_
     /* step 1, :134-136: ReduceScatterRing on (input, input, output-as-scratch) inside the server */
     g_rank_map = level0;
     g_step_base = 0;
-    if (n_local > 1) prog_ring_rs(t, local, n_local, seg, NULL);
+    if (level0_mesh) prog_mesh_rs_streams(t, local, n_local, seg); /* CollAllReduceMeshExecutor::KernelRun, :116-119 */
+    else if (n_local > 1) prog_ring_rs(t, local, n_local, seg, NULL);
     /* step 2, :140-218: level-1 allreduce of the own segment; hdSize / segment from PrepareLevel1CommInfo,
      * exec/coll_comm_executor.cc:2565-2575 */
     const uint64_t hd_count = seg[local].size / unit;    /* :146 */
@@ -1467,13 +1524,15 @@ static int prog_hier_allreduce(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_
     /* step 3, :228-230: AllGatherRing on (output, output, input-as-scratch), exec/coll_comm_executor.cc:377-379 */
     g_rank_map = level0;
     g_step_base = n_local - 1 + level1_steps;
-    if (n_local > 1) prog_ring_ag_ex(t, local, n_local, seg, 0, 0);
+    if (level0_mesh) prog_mesh_ag(t, local, n_local, seg);         /* CollAllReduceMeshExecutor::KernelRun, :204-228 */
+    else if (n_local > 1) prog_ring_ag_ex(t, local, n_local, seg, 0, 0);
     g_rank_map = NULL;
     g_step_base = 0;
     return 0;
 }
 
-static int build_trace_hier(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype)
+static int build_trace_hier(OrcTrace* t, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                            int dtype)
 {
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
@@ -1492,7 +1551,7 @@ static int build_trace_hier(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t 
         if (st > level1_steps) level1_steps = st;
     }
     for (uint32_t r = 0; r < n_servers * n_local; r++) {
-        prog_hier_allreduce(t, alg1, r, n_servers, n_local, count, dtype, level1_steps);
+        prog_hier_allreduce(t, level0_mesh, alg1, r, n_servers, n_local, count, dtype, level1_steps);
         if (t->oom) {
             free(t->ops);
             return -2;
@@ -1501,10 +1560,11 @@ static int build_trace_hier(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t 
     return sort_trace(t);
 }
 
-int64_t orc_trace_hier(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype, OrcOp* out, uint64_t cap)
+int64_t orc_trace_hier(int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, int dtype, OrcOp* out,
+                       uint64_t cap)
 {
     OrcTrace t;
-    int rc = build_trace_hier(&t, alg1, n_servers, n_local, count, dtype);
+    int rc = build_trace_hier(&t, level0_mesh, alg1, n_servers, n_local, count, dtype);
     if (rc) return rc;
     const uint64_t m = t.n < cap ? t.n : cap;
     if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
@@ -1513,11 +1573,11 @@ int64_t orc_trace_hier(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t 
     return total;
 }
 
-int orc_run_hier(int alg1, uint32_t n_servers, uint32_t n_local, void* const* in, void* const* out, uint64_t count,
-                 int dtype, int op)
+int orc_run_hier(int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, void* const* in, void* const* out,
+                 uint64_t count, int dtype, int op)
 {
     OrcTrace t;
-    int rc = build_trace_hier(&t, alg1, n_servers, n_local, count, dtype);
+    int rc = build_trace_hier(&t, level0_mesh, alg1, n_servers, n_local, count, dtype);
     if (rc) return rc;
     void* const* bufs[5] = {in, out, NULL, NULL, NULL};
     rc = exec_trace(&t, bufs, dtype, op);

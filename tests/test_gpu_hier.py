@@ -37,18 +37,18 @@ def say(*a):
     sys.stdout.flush()
 
 
-def run_case(thread, alg1, ns, nl, count, dtype, op, seed=0):
+def run_case(thread, alg1, ns, nl, count, dtype, op, seed=0, mesh=False):
     dt, o, n = DT[dtype], OPS[op], ns * nl
     host_in = [gen(dt, count, 7000 + seed * 100 + r, "prod" if op == "prod" else "default") for r in range(n)]
     sentinel = gen(dt, count, 997, "wide")
     want_in = [x.copy() for x in host_in]
     want_out = [sentinel.copy() for _ in range(n)]
-    oracle.run_hier(LEVEL1[alg1], ns, nl, want_in, want_out, count, dt, o)
+    oracle.run_hier(LEVEL1[alg1], ns, nl, want_in, want_out, count, dt, o, mesh=mesh)
     d_in = [to_dev(x) for x in host_in]
     d_out = [to_dev(sentinel) for _ in range(n)]
     pad = to_dev(np.zeros(256, np.uint8))
     ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
-    plan = h.HierPlan(LEVEL1[alg1], ns, nl, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+    plan = h.HierPlan(LEVEL1[alg1], ns, nl, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o, mesh=mesh)
     try:
         assert plan.run(thread) == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
@@ -70,6 +70,15 @@ def test_three_step_allreduce_matches_oracle(gpu_thread, alg1, ns, nl, count, dt
     assert info.launches <= 2 * (max(o[0] for o in ops) + 1 if ops else 0)     # about one launch per lock-step step
 
 
+@pytest.mark.parametrize("alg1,ns,nl,count,dtype,op", CASES)
+def test_three_step_allreduce_with_mesh_level0_matches_oracle(gpu_thread, alg1, ns, nl, count, dtype, op):
+    say("mesh hier", alg1, ns, nl, count, dtype, op)
+    info = run_case(gpu_thread, alg1, ns, nl, count, dtype, op, mesh=True)
+    ops = oracle.trace_hier(LEVEL1[alg1], ns, nl, count, DT[dtype], mesh=True)
+    assert info.algorithmicBytes == sum(o[8] * (3 if o[1] else 2) for o in ops)
+    assert info.movedBytes == info.algorithmicBytes
+
+
 def test_randomized_shapes(gpu_thread):
     rng = np.random.default_rng(4242)
     names = sorted(LEVEL1)
@@ -81,5 +90,6 @@ def test_randomized_shapes(gpu_thread):
         count = int(rng.integers(1, 400000))
         dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
         op = ["sum", "max", "min"][rng.integers(3)]
-        say("random hier", i, alg1, ns, nl, count, dtype, op)
-        run_case(gpu_thread, alg1, ns, nl, count, dtype, op, seed=i)
+        mesh = bool(rng.integers(2))
+        say("random hier", i, alg1, ns, nl, count, dtype, op, mesh)
+        run_case(gpu_thread, alg1, ns, nl, count, dtype, op, seed=i, mesh=mesh)

@@ -24,6 +24,36 @@ def test_operation_list_hand_derived():
     assert h.hier_emit(h.Alg.ALLREDUCE_RING, 2, 2, 100, oracle.F32) == want
 
 
+def test_mesh_level0_operation_list_hand_derived():
+    want = [tuple(o) for o in GOLD["mesh_rank0_ops_1x4_fp32_count384"]["ops"]]
+    for gen in (oracle.trace_hier, h.hier_emit):
+        got = [o for o in gen(oracle.ALG_ALLREDUCE_RING, 1, 4, 384, oracle.F32, mesh=True) if o[2] == 0]
+        assert got == want
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_mesh_level0_reduction_trees_hand_derived(op):
+    ins = order_sensitive_inputs(4, 384, op, seed=310)
+    work = [x.copy() for x in ins]
+    outs = [np.zeros(384, np.float32) for _ in range(4)]
+    oracle.run_hier(oracle.ALG_ALLREDUCE_RING, 1, 4, work, outs, 384, oracle.F32, op, mesh=True)
+    for first, cnt, tree in GOLD["mesh_trees_1x4_fp32_count384"]["pieces"]:
+        want = eval_tree(tree, [x[first:first + cnt] for x in ins], op)
+        for r in range(4):
+            assert np.array_equal(outs[r][first:first + cnt].view(np.uint32), want.view(np.uint32)), (first, r)
+
+
+def test_mesh_stream_pieces_hand_derived():
+    """A ragged last segment of 1000 bytes cut for 3 and for 7 streams (the fixture places it at offset 2048)."""
+    c = GOLD["mesh_stream_pieces"]
+    for n, key in ((4, "streams3"), (8, "streams7")):
+        count = next(k for k in range(1, 40000) if oracle.slices_ring(k, 1, n)[n - 1][1] == c["seg"][1])
+        seg = oracle.slices_ring(count, 1, n)[n - 1]
+        for gen in (oracle.trace_hier, h.hier_emit):
+            ops = [o for o in gen(oracle.ALG_ALLREDUCE_RING, 1, n, count, oracle.I8, mesh=True) if o[0] == 0 and o[2] == n - 1]
+            assert [[o[4] - seg[0] + c["seg"][0], o[8]] for o in ops] == c[key], (n, count)
+
+
 @pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
 def test_reduction_trees_hand_derived(op):
     ins = order_sensitive_inputs(6, 192, op, seed=300)
@@ -49,19 +79,21 @@ def test_small_messages_take_the_one_shot_template_between_servers():
         assert len(big) >= nl * ns
 
 
+@pytest.mark.parametrize("mesh", [False, True])
 @pytest.mark.parametrize("alg1", LEVEL1)
-def test_product_generator_equals_oracle_trace_and_passes_the_checker(alg1):
-    for ns, nl in SHAPES:
+def test_product_generator_equals_oracle_trace_and_passes_the_checker(alg1, mesh):
+    for ns, nl in SHAPES + [(1, 2), (1, 32)]:
         for count, dt in ((100003, oracle.F32), (1000, oracle.F16), (7, oracle.I8), (0, oracle.F32),
                           (300007, oracle.I32), (8 * 70000, oracle.F32)):
-            a = oracle.trace_hier(alg1, ns, nl, count, dt)
-            assert a == h.hier_emit(alg1, ns, nl, count, dt), (alg1, ns, nl, count)
-            assert h.hier_check(alg1, ns, nl, count, dt)[:2] == (0, 0), (alg1, ns, nl, count)
+            a = oracle.trace_hier(alg1, ns, nl, count, dt, mesh=mesh)
+            assert a == h.hier_emit(alg1, ns, nl, count, dt, mesh=mesh), (alg1, ns, nl, count)
+            assert h.hier_check(alg1, ns, nl, count, dt, mesh=mesh)[:2] == (0, 0), (alg1, ns, nl, count)
             assert h.oplist_check(a, ns * nl, Expect.ALLREDUCE, count, h.DTYPE_SIZE[dt])[:2] == (0, 0)
 
 
+@pytest.mark.parametrize("mesh", [False, True])
 @pytest.mark.parametrize("alg1", LEVEL1)
-def test_exact_integer_sums(alg1):
+def test_exact_integer_sums(alg1, mesh):
     rng = np.random.default_rng(5)
     for ns, nl in SHAPES:
         n = ns * nl
@@ -69,7 +101,7 @@ def test_exact_integer_sums(alg1):
             ins = [rng.integers(-1000, 1000, count, dtype=np.int32) for _ in range(n)]
             work = [x.copy() for x in ins]
             outs = [np.full(count, -7, np.int32) for _ in range(n)]
-            oracle.run_hier(alg1, ns, nl, work, outs, count, oracle.I32, oracle.SUM)
+            oracle.run_hier(alg1, ns, nl, work, outs, count, oracle.I32, oracle.SUM, mesh=mesh)
             want = np.sum(np.stack(ins).astype(np.int64), axis=0).astype(np.int32)
             for r in range(n):
                 assert np.array_equal(outs[r], want), (alg1, ns, nl, count, r)
