@@ -47,6 +47,8 @@
  *                                     N = 2, 3, 5, 6, 8 by hand; pinned
  *   three-step allreduce ............ the complete operation list of 2 servers x 2 ranks and the reduction trees
  *                                     of 2 x 3 by hand; the one-shot threshold; exact integer results; pinned
+ *   mesh level 0 of the three steps . stream pieces of a ragged segment for 3 and 7 streams, one rank's operation
+ *                                     list and the trees of all 12 pieces N = 4 by hand; pinned
  *   double-ring allreduce ........... slice / ring-order tables N = 4, one rank's complete operation list N = 3, the
  *                                     reduction trees of both shares N = 4, all by hand; exact integer results over
  *                                     several chunks; pinned
