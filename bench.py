@@ -71,6 +71,9 @@ WORKLOADS = {
     "dbring_nhr_ar_bf16_2x8_128MiB": ("dbring_nhr", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving reduce-scatter executor: plant into the peers' CCL output buffers, fold in rank order
     "order_preserved_rs_bf16_n8_16MiB": ("order_preserved_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the ring / mesh reduce-scatter executors over two levels in op-base mode (blocks of 16 MiB, 2 x 8 ranks)
+    "hierrs_ring_rs_bf16_2x8_16MiB": ("hierrs_ring_rs_stage", (2, 8), 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    "meshhierrs_ring_rs_bf16_1x8_16MiB": ("meshhierrs_ring_rs_stage", (1, 8), 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     "nhr_oneshot_ar_bf16_n8_256KiB": ("nhr_oneshot", 8, 131072, "bf16", "sum", "normal(0,1)*1e-3"),
     "mesh_oneshot_fp16_n8_sweep": ("mesh_oneshot", 8, None, "fp16", "sum", "uniform[-1,1)"),
 }
@@ -137,15 +140,16 @@ def main():
         alg_name = alg_name[len("opbase_"):]
     hier = None  # (servers, ranks per server): the level-1 template inside the ring executor's three steps
     dbring = False  # the double-ring executor with DMA reduce instead of the single ring on staged buffers
-    mesh0 = alg_name.startswith("meshhier_")  # the mesh executor's level 0 instead of the ring executor's
-    if alg_name.startswith("hier_") or alg_name.startswith("dbring_") or mesh0:
+    mesh0 = alg_name.startswith("meshhier")  # the mesh executor's level 0 instead of the ring executor's
+    hier_rs = alg_name.startswith("hierrs_") or alg_name.startswith("meshhierrs_")  # the reduce-scatter executors
+    if alg_name.startswith("hier") or alg_name.startswith("dbring_") or mesh0:
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     plant = alg_name == "order_preserved_rs"
     dt, alg, op = DT[dtname], (None if plant else ALG[alg_name]), OP[opname]
     unit = h.DTYPE_SIZE[dt]
-    in_place = alg_name == "ring_rs_stage"
+    in_place = alg_name == "ring_rs_stage" and not hier
 
     stream = torch.cuda.Stream(device=dev)  # default priority
     code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 0)
@@ -158,7 +162,7 @@ def main():
         return
 
     nbytes = count * unit
-    in_count = n * count if alg_name in ("local_reduce_rs", "order_preserved_rs") else count  # N slices of count
+    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs") or hier_rs) else count  # N slices
     pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
     d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
@@ -174,7 +178,7 @@ def main():
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
     scratch_bytes = 0 if plant else h.scratch_bytes(alg, n, count, dt)
     d_ccl = None
-    if opbase or dbring or plant:
+    if opbase or dbring or plant or hier_rs:
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both":
             args.lowering = "stepwise"
@@ -188,6 +192,9 @@ def main():
              h.Kernel.COPY: "k_copy"}
 
     def make_plan(low):
+        if hier_rs:
+            return h.HierReduceScatterPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
+                                           [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, mesh=mesh0)
         if plant:
             return h.OrderPreservedPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if dbring:
@@ -287,7 +294,10 @@ def main():
         host_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
         oracle.lib().orc_set_threads(threads)
         host_scr = [np.zeros(scratch_bytes, np.uint8) for _ in range(n)] if scratch_bytes else None
-        if plant:
+        if hier_rs:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2)
+                            for o in oracle.trace_hier_rs(oalg, hier[0], hier[1], count, ccl_bytes, odt, mesh=mesh0))
+        elif plant:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved(n, count, ccl_bytes, odt))
         elif dbring:
             alg_bytes = sum(o[8] * (3 if o[1] else 2)
@@ -298,10 +308,14 @@ def main():
         else:
             alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
                          else oracle.algorithmic_bytes(oalg, n, count, odt))
-        host_ccl = [[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)] if (opbase or dbring or plant) else None
+        host_ccl = ([[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)]
+                    if (opbase or dbring or plant or hier_rs) else None)
 
         def cpu_run(ins, outs):
-            if plant:
+            if hier_rs:
+                oracle.run_hier_rs(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop,
+                                   mesh=mesh0)
+            elif plant:
                 oracle.run_order_preserved(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif dbring:
                 oracle.run_dbring(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
@@ -377,7 +391,7 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
-                if opbase or dbring or plant:  # what the last chunk left in the CCL buffers
+                if opbase or dbring or plant or hier_rs:  # what the last chunk left in the CCL buffers
                     ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
@@ -408,7 +422,7 @@ def main():
                        "level0_algorithm": ("double-ring reduce-scatter + all-gather on user memory (DMA reduce)"
                                             if dbring else "multi-stream mesh reduce-scatter + mesh all-gather" if mesh0
                                             else "ring reduce-scatter + ring all-gather")} if hier else {}),
-                   **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant) else {})},
+                   **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant or hier_rs) else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

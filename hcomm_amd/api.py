@@ -29,6 +29,7 @@ __all__ = [
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
+    "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -526,6 +527,47 @@ class OrderPreservedPlan(Plan):
         p = _vp(0)
         check(_op_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
               "HcommGfxOrderPreservedPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_hrs_emit = _sig("HcommGfxHierReduceScatterEmit", _i32, _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp),
+                 _u64, C.POINTER(_u64))
+_hrs_check = _sig("HcommGfxHierReduceScatterCheck", _i32, _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+                  C.POINTER(CheckReport))
+_hrs_plan = _sig("HcommGfxHierReduceScatterPlanCreate", _i32, _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                 C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def hier_rs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, mesh=False):
+    n = _u64(0)
+    check(_hrs_emit(int(mesh), alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
+          "HcommGfxHierReduceScatterEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_hrs_emit(int(mesh), alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
+          "HcommGfxHierReduceScatterEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def hier_rs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, mesh=False):
+    rep = CheckReport()
+    check(_hrs_check(int(mesh), alg1, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
+          "HcommGfxHierReduceScatterCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class HierReduceScatterPlan(Plan):
+    """HcommGfxHierReduceScatterPlanCreate: the ring (mesh=False) or mesh reduce-scatter executor over two levels."""
+
+    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_out, ccl_bytes, count, dtype, op,
+                 mesh=False):
+        n = n_servers * n_local
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in, ccl_out)]
+        p = _vp(0)
+        check(_hrs_plan(int(mesh), alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3],
+                        ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxHierReduceScatterPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -843,18 +843,33 @@ static int append_mapped(HgOpList* l, const HgOpList* sub, const uint32_t* map, 
 }
 
 /* Lists built level by level and, inside a level, group by group: order them by step, then by rank, keeping the
- * order of a rank's operations inside a step (insertion sort, stable; the lists are nearly ordered already). */
+ * order of a rank's operations inside a step (bottom-up merge sort, stable; falls back to leaving the list as built
+ * if the scratch array cannot be had, which only costs launches, not correctness of a conflict-free step). */
+static int op_before(const HcommGfxSchedOp* a, const HcommGfxSchedOp* b)
+{
+    return a->step < b->step || (a->step == b->step && a->rank <= b->rank);
+}
+
 static void order_by_step_rank(HgOpList* l)
 {
-    for (uint64_t i = 1; i < l->n; ++i) {
-        HcommGfxSchedOp x = l->ops[i];
-        uint64_t j = i;
-        while (j > 0 && (l->ops[j - 1].step > x.step || (l->ops[j - 1].step == x.step && l->ops[j - 1].rank > x.rank))) {
-            l->ops[j] = l->ops[j - 1];
-            --j;
+    if (l->n < 2) return;
+    HcommGfxSchedOp* tmp = (HcommGfxSchedOp*)malloc(l->n * sizeof(*tmp));
+    if (!tmp) return;
+    HcommGfxSchedOp *src = l->ops, *dst = tmp;
+    for (uint64_t w = 1; w < l->n; w *= 2) {
+        for (uint64_t lo = 0; lo < l->n; lo += 2 * w) {
+            const uint64_t mid = lo + w < l->n ? lo + w : l->n, hi = lo + 2 * w < l->n ? lo + 2 * w : l->n;
+            uint64_t a = lo, b = mid, k = lo;
+            while (a < mid && b < hi) dst[k++] = op_before(&src[a], &src[b]) ? src[a++] : src[b++];
+            while (a < mid) dst[k++] = src[a++];
+            while (b < hi) dst[k++] = src[b++];
         }
-        l->ops[j] = x;
+        HcommGfxSchedOp* t = src;
+        src = dst;
+        dst = t;
     }
+    if (src != l->ops) memcpy(l->ops, src, l->n * sizeof(*tmp));
+    free(tmp);
 }
 
 /* CollAllReduceRingExecutor::KernelRun (src/legacy/ascend910/algorithm/impl/coll_executor/coll_all_reduce/
@@ -909,6 +924,7 @@ int hg_schedule_hier(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers,
     if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_RHD && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR &&
         alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
         return HCCL_E_PARA; /* the level-1 choices of :164-204 that are built here */
+    if (level0_mesh && n_local < 2) return HCCL_E_PARA; /* PrepareSliceMeshStreams refuses zero streams (alg_template_base.cc:832-835) */
     HcommGfxSlice seg[HCOMM_GFX_MAX_RANKS];
     CHK(HcommGfxCalcSlices(count, unit, n_local, seg));
     uint32_t map[HCOMM_GFX_MAX_RANKS];
@@ -1096,6 +1112,128 @@ int32_t HcommGfxDoubleRingEmit(
     if (!n) return HCCL_E_PTR;
     HgOpList l;
     int rc = hg_schedule_dbring(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
+/* ---- the ring and mesh reduce-scatter executors over two communicator levels (op-base mode) --------------------- */
+
+/* CollReduceScatterRingExecutor::KernelRun (coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:
+ * 136-363, single ring, every device with a NIC) and CollReduceScatterMeshExecutor::KernelRun
+ * (coll_reduce_scatter_mesh_executor.cc:131-259, the branch without atomic adds) inside the loop of
+ * CollReduceScatterExecutor (coll_reduce_scatter_executor.cc:149-306, buffer-copy mode) with their own chunk size
+ * cclBytes / (N * unit) (:116-121 / :116-121).  N = n_servers * n_local, rank = server * n_local + local index, block b
+ * of the input belongs to rank b.  Per chunk of c bytes per block:
+ *   0. user input -> CCL input, block by block (one copy when a single chunk takes everything, :262-266);
+ *   1. between the servers, in place on the CCL inputs: reduce-scatter (ring, NHR in slice order, or NB) over the
+ *      n_servers runs of n_local blocks - rank (s, l) ends up with run s summed over the ranks (., l);
+ *   2. inside every server, in place, at base offset = the server's run: ring reduce-scatter over the n_local blocks
+ *      of the run, or the multi-stream mesh reduce-scatter over their pieces;
+ *   3. the rank's own block CCL input -> CCL output (:359 / :255), then CCL output -> user output (:293-298). */
+static int hier_rs_build(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                         uint64_t ccl_bytes, uint32_t unit, int dtype)
+{
+    (void)dtype;
+    const uint32_t n = n_servers * n_local;
+    const uint64_t max_count = ccl_bytes / ((uint64_t)n * unit);
+    if (max_count == 0) return HCCL_E_PARA;
+    uint32_t step = 0, map[HCOMM_GFX_MAX_RANKS];
+    uint64_t user_off = 0;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        /* 0 */
+        for (uint32_t r = 0; r < n; ++r) {
+            if (cur == count) {
+                CHK(push(l, step, COPY, r, IN, 0, r, UIN, 0, c * n));
+                continue;
+            }
+            for (uint32_t b = 0; b < n; ++b) CHK(push(l, step, COPY, r, IN, c * b, r, UIN, user_off + count * unit * b, c));
+        }
+        ++step;
+        /* 1 */
+        if (n_servers > 1) {
+            HgOpList sub;
+            memset(&sub, 0, sizeof(sub));
+            for (uint32_t i = 0; i < n_servers; ++i) {
+                sl[i].offset = c * n_local * i;
+                sl[i].size = c * n_local;
+            }
+            int rc;
+            if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) rc = ring_rs(&sub, n_servers, sl, 0);
+            else if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR) {
+                uint32_t order[HCOMM_GFX_MAX_RANKS];
+                nhr_slice_map(n_servers, 1, order);
+                rc = nhr_rs(&sub, n_servers, sl, order, 0);
+            } else rc = nb_rs(&sub, n_servers, sl);
+            uint32_t used = 0;
+            for (uint32_t i = 0; i < n_local && rc == HCCL_SUCCESS; ++i) {
+                for (uint32_t srv = 0; srv < n_servers; ++srv) map[srv] = srv * n_local + i;
+                rc = append_mapped(l, &sub, map, step, 0, 0, &used);
+            }
+            hg_oplist_free(&sub);
+            CHK(rc);
+            step += used;
+        }
+        /* 2 */
+        for (uint32_t i = 0; i < n_local; ++i) {
+            sl[i].offset = c * i;
+            sl[i].size = c;
+        }
+        if (n_local > 1) {
+            HgOpList sub;
+            memset(&sub, 0, sizeof(sub));
+            int rc = level0_mesh ? mesh_level0_rs(&sub, 0, n_local, sl, 0) : ring_rs(&sub, n_local, sl, 0);
+            uint32_t used = 0;
+            for (uint32_t srv = 0; srv < n_servers && rc == HCCL_SUCCESS; ++srv) {
+                for (uint32_t i = 0; i < n_local; ++i) map[i] = srv * n_local + i;
+                rc = append_mapped(l, &sub, map, step, c * n_local * srv, 0, &used);
+            }
+            hg_oplist_free(&sub);
+            CHK(rc);
+            step += n_local - 1;
+        }
+        /* 3 */
+        for (uint32_t r = 0; r < n; ++r) CHK(push(l, step, COPY, r, OUT, 0, r, IN, c * r, c));
+        ++step;
+        for (uint32_t r = 0; r < n; ++r) CHK(push(l, step, COPY, r, UOUT, user_off, r, OUT, 0, c));
+        ++step;
+        user_off += c;
+        left -= cur;
+    }
+    order_by_step_rank(l);
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                        uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (level0_mesh && n_local < 2) return HCCL_E_PARA; /* PrepareSliceMeshStreams refuses zero streams */
+    if (alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RING && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR &&
+        alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
+        return HCCL_E_PARA;
+    const int rc = hier_rs_build(l, level0_mesh, alg1, n_servers, n_local, count, ccl_bytes, unit, dtype);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxHierReduceScatterEmit(
+    int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_hier_rs(&l, level0Mesh != 0, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     *n = l.n;
     if (ops) {

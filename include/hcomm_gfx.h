@@ -644,6 +644,28 @@ int32_t HcommGfxDoubleRingCheck(
     HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
+ * The reduce-scatter of the reference's ring executor (level0Mesh 0: coll_executor/coll_reduce_scatter/
+ * coll_reduce_scatter_ring_executor.cc:136-363, one ring per server) or mesh executor (level0Mesh 1:
+ * coll_reduce_scatter_mesh_executor.cc:131-259, its branch without atomic adds) over two communicator levels in
+ * op-base mode (loop and staging copies of coll_reduce_scatter_executor.cc:149-306, chunks of at most
+ * cclBytes / (N * unit) elements per block, N = nServers * nLocal, rank = server * nLocal + local index):
+ * user input -> CCL input; level1Alg (HCOMM_GFX_ALG_REDUCE_SCATTER_RING, _NHR or _NB, in place) between the servers over
+ * the nServers runs of nLocal blocks; ring or multi-stream mesh reduce-scatter inside every server over the blocks of
+ * its run; own block -> CCL output -> user output.
+ * userIn: N * count elements (block b at b * count belongs to rank b); userOut: count; cclIn / cclOut: cclBytes.
+ */
+int32_t HcommGfxHierReduceScatterPlanCreate(
+    int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn,
+    void* const* userOut, void* const* cclIn, void* const* cclOut, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxHierReduceScatterEmit(
+    int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+int32_t HcommGfxHierReduceScatterCheck(
+    int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
  * The reduce-scatter of the reference's order-preserving executor on one server in op-base mode
  * (coll_executor/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:181-216, 260-283, around
  * ReduceScatterPlantLocalReduce, alg_template/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc): per chunk of

@@ -1539,6 +1539,7 @@ static int build_trace_hier(OrcTrace* t, int level0_mesh, int alg1, uint32_t n_s
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
     if (unit == 0 || n_servers == 0 || n_local == 0 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (level0_mesh && n_local < 2) return -1; /* streamCount == 0, tpl/alg_template_base.cc:832-835 */
     if (alg1 != ORC_ALG_ALLREDUCE_RING && alg1 != ORC_ALG_ALLREDUCE_RHD && alg1 != ORC_ALG_ALLREDUCE_NHR &&
         alg1 != ORC_ALG_ALLREDUCE_NB)
         return -1;
@@ -1811,6 +1812,138 @@ int orc_dbring_slices(uint64_t count, int dtype, uint32_t n, OrcSlice* out, uint
             order[ring * n + i] = d.order[ring][i];
         }
     return 0;
+}
+
+/* ---- the ring and mesh reduce-scatter executors over two communicator levels, op-base mode ---------------------- */
+
+/* CollReduceScatterRingExecutor::KernelRun (exec/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:136-363, one
+ * ring, every device with a NIC) or CollReduceScatterMeshExecutor::KernelRun (exec/coll_reduce_scatter/
+ * coll_reduce_scatter_mesh_executor.cc:131-259, without atomic adds) for one rank and one chunk, between the copies of
+ * CollReduceScatterExecutor::RunLoopInner (exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:258-298). */
+static void prog_hier_rs(OrcTrace* t, int level0_mesh, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local,
+                         uint64_t total_count, uint64_t cur_count, uint32_t unit, uint32_t step0)
+{
+    const uint32_t n = n_servers * n_local;
+    const uint32_t server = rank / n_local, local = rank % n_local;
+    const uint64_t cur_size = cur_count * unit;
+    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+    for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+    for (uint32_t s = 0; s < n_servers; s++) level1[s] = s * n_local + local;
+    g_rank_map = NULL;
+    g_base_off = 0;
+    g_step_base = step0;
+    /* user input -> CCL input, coll_reduce_scatter_executor.cc:258-276 */
+    if (total_count == cur_count) {
+        emit(t, 0, K_COPY, rank, B_IN, 0, rank, B_UIN, 0, total_count * unit * n);
+    } else {
+        for (uint32_t i = 0; i < n; i++)
+            emit(t, 0, K_COPY, rank, B_IN, cur_size * i, rank, B_UIN, total_count * unit * i, cur_size);
+    }
+    uint32_t step = step0 + 1;
+    /* first: between the servers, :183-247 / :146-205; input memory = scratch of nothing, in place; slices default to
+     * count * unit at i * count * unit (tpl/temp_reduce_scatter/reduce_scatter_ring.cc:140-157, reduce_scatter_nhr.cc:
+     * 57-75, reduce_scatter_nb.cc) with count = inputMem.size() / level1RankSize / unit */
+    if (n_servers > 1) {
+        OrcSlice sl[ORC_MAX_RANKS];
+        const uint64_t ring_size = cur_size * n / n_servers;
+        for (uint32_t i = 0; i < n_servers; i++) {
+            sl[i].size = ring_size;
+            sl[i].offset = (uint64_t)i * ring_size;
+        }
+        g_rank_map = level1;
+        g_step_base = step;
+        if (alg1 == ORC_ALG_RS_RING_STAGE) {
+            prog_ring_rs(t, server, n_servers, sl, NULL);
+            step += n_servers - 1;
+        } else if (alg1 == ORC_ALG_RS_NHR) {
+            uint32_t slice_map[ORC_MAX_RANKS];
+            nhr_rank_mapping(n_servers, 1, slice_map); /* GetRankMapping(rankSize, true), reduce_scatter_nhr.cc:86-88 */
+            prog_nhr_rs(t, server, n_servers, sl, NULL, slice_map, 0);
+            step += nhr_steps(n_servers);
+        } else {
+            prog_nb_rs(t, server, n_servers, sl, NULL);
+            step += nhr_steps(n_servers);
+        }
+    }
+    /* second: inside the server, :249-357 / :207-252, on the server's run of the CCL input at base offset
+     * serverSliceOffset, slices of the output size (ReduceScatterRingSlicePrepare, coll_reduce_scatter_executor.cc:
+     * 491-503 / PrepareReduceScatterSliceData, exec/coll_comm_executor.cc:1906-1919) */
+    const uint64_t server_slice_size = cur_size * n / n_servers;
+    OrcSlice seg[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n_local; i++) {
+        seg[i].size = cur_size;
+        seg[i].offset = cur_size * i;
+    }
+    g_rank_map = level0;
+    g_base_off = server_slice_size * server;
+    g_step_base = step;
+    if (level0_mesh) prog_mesh_rs_streams(t, local, n_local, seg);
+    else if (n_local > 1) prog_ring_rs(t, local, n_local, seg, NULL);
+    step += n_local - 1;
+    g_rank_map = NULL;
+    g_base_off = 0;
+    /* :359 / :255: the own block to the output memory */
+    g_step_base = step;
+    emit(t, 0, K_COPY, rank, B_OUT, 0, rank, B_IN, server_slice_size * server + seg[local].offset, cur_size);
+    /* coll_reduce_scatter_executor.cc:293-298 */
+    g_step_base = step + 1;
+    emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_OUT, 0, cur_size);
+    g_step_base = 0;
+}
+
+static int build_trace_hier_rs(OrcTrace* t, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                               uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n_servers == 0 || n_local == 0 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (level0_mesh && n_local < 2) return -1;
+    if (alg1 != ORC_ALG_RS_RING_STAGE && alg1 != ORC_ALG_RS_NHR && alg1 != ORC_ALG_RS_NB) return -1;
+    const uint32_t n = n_servers * n_local;
+    const uint64_t max_count = ccl_bytes / ((uint64_t)n * unit); /* CalcLoopMaxCount of both executors, :116-121 */
+    if (max_count == 0) return -1;
+    const uint32_t level1_steps = n_servers == 1 ? 0 : (alg1 == ORC_ALG_RS_RING_STAGE ? n_servers - 1 : nhr_steps(n_servers));
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        g_user_off = user_off;
+        for (uint32_t r = 0; r < n; r++) prog_hier_rs(t, level0_mesh, alg1, r, n_servers, n_local, count, cur_count, unit, step0);
+        g_user_off = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += 1 + level1_steps + (n_local - 1) + 2;
+        user_off += cur_count * unit;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_hier_rs(int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                          int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_hier_rs(&t, level0_mesh, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_hier_rs(int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, void* const* user_in,
+                    void* const* user_out, void* const* ccl_in, void* const* ccl_out, uint64_t count, uint64_t ccl_bytes,
+                    int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_hier_rs(&t, level0_mesh, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
 }
 
 /* ---- the order-preserving reduce-scatter executor (one server, op-base mode) ----------------------------------- */

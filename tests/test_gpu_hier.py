@@ -72,6 +72,8 @@ def test_three_step_allreduce_matches_oracle(gpu_thread, alg1, ns, nl, count, dt
 
 @pytest.mark.parametrize("alg1,ns,nl,count,dtype,op", CASES)
 def test_three_step_allreduce_with_mesh_level0_matches_oracle(gpu_thread, alg1, ns, nl, count, dtype, op):
+    if nl < 2:
+        pytest.skip("the mesh executor needs at least two ranks per server")
     say("mesh hier", alg1, ns, nl, count, dtype, op)
     info = run_case(gpu_thread, alg1, ns, nl, count, dtype, op, mesh=True)
     ops = oracle.trace_hier(LEVEL1[alg1], ns, nl, count, DT[dtype], mesh=True)
@@ -90,6 +92,6 @@ def test_randomized_shapes(gpu_thread):
         count = int(rng.integers(1, 400000))
         dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
         op = ["sum", "max", "min"][rng.integers(3)]
-        mesh = bool(rng.integers(2))
+        mesh = bool(rng.integers(2)) and nl >= 2
         say("random hier", i, alg1, ns, nl, count, dtype, op, mesh)
         run_case(gpu_thread, alg1, ns, nl, count, dtype, op, seed=i, mesh=mesh)
