@@ -1,8 +1,9 @@
 /*
  * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics, of the ring, recursive
  * halving-doubling, mesh, NHR (sliced and one-shot), NB, local-reduce, chunk-mesh and doubling schedules, of the
- * executors' op-base loop around them, of the ring executor's three-step allreduce, of the double-ring executor with
- * DMA reduce and of the order-preserving reduce-scatter executor, used ONLY to check libhcomm_gfx.so.
+ * executors' op-base loop around them, of the ring and mesh executors' three-step allreduce and two-level
+ * reduce-scatter, of the double-ring executor with DMA reduce and of the order-preserving reduce-scatter executor, used
+ * ONLY to check libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -52,6 +53,8 @@
  *   double-ring allreduce ........... slice / ring-order tables N = 4, one rank's complete operation list N = 3, the
  *                                     reduction trees of both shares N = 4, all by hand; exact integer results over
  *                                     several chunks; pinned
+ *   two-level reduce-scatter ........ the complete operation list and the reduction trees of 2 x 2, the trees of the
+ *                                     mesh pieces of 1 x 4, a chunk table, by hand; exact integer results; pinned
  *   order-preserving reduce-scatter . the complete operation list N = 3, the rank-order fold trees N = 2..8 and a
  *                                     chunk table by hand; exact integer results over several chunks; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
