@@ -40,26 +40,35 @@ static int ranges_overlap(uint64_t a, uint64_t an, uint64_t b, uint64_t bn) { re
 
 #define MAX_INTERVALS_PER_BUFFER (1u << 20)
 
-/* One rank buffer: intervals [b[i], b[i+1]) with state c[i], i < n; b has n + 1 entries. */
+/* One rank buffer: intervals [b[i], b[i+1]) with state pool[ix[i]], i < n; b has n + 1 entries.  The states live in a
+ * pool and the map orders indices into it, so that cutting an interval moves 4 bytes per interval behind the cut and
+ * not a whole state. */
 typedef struct {
     uint64_t* b;
-    Cell* c;
-    size_t n, cap;
+    uint32_t* ix;
+    Cell* pool;
+    size_t n, cap, pool_n, pool_cap;
 } IMap;
+
+#define CELL(m, i) ((m)->pool[(m)->ix[i]])
 
 static int imap_init(IMap* m, uint64_t extent, uint32_t nranks, int own_rank)
 {
     m->cap = 16;
+    m->pool_cap = 16;
     m->b = (uint64_t*)malloc((m->cap + 1) * sizeof(uint64_t));
-    m->c = (Cell*)calloc(m->cap, sizeof(Cell));
-    if (!m->b || !m->c) return -1;
+    m->ix = (uint32_t*)malloc(m->cap * sizeof(uint32_t));
+    m->pool = (Cell*)calloc(m->pool_cap, sizeof(Cell));
+    if (!m->b || !m->ix || !m->pool) return -1;
     m->n = 1;
+    m->pool_n = 1;
+    m->ix[0] = 0;
     m->b[0] = 0;
     m->b[1] = extent;
-    for (uint32_t k = 0; k < nranks; ++k) m->c[0].delta[k] = NO_DELTA;
+    for (uint32_t k = 0; k < nranks; ++k) m->pool[0].delta[k] = NO_DELTA;
     if (own_rank >= 0) { /* an input holds its own rank's data from the same offset */
-        m->c[0].cnt[own_rank] = 1;
-        m->c[0].delta[own_rank] = 0;
+        m->pool[0].cnt[own_rank] = 1;
+        m->pool[0].delta[own_rank] = 0;
     }
     return 0;
 }
@@ -80,13 +89,22 @@ static long imap_cut(IMap* m, uint64_t v)
         uint64_t* nb = (uint64_t*)realloc(m->b, (cap + 1) * sizeof(uint64_t));
         if (!nb) return -1;
         m->b = nb;
-        Cell* nc = (Cell*)realloc(m->c, cap * sizeof(Cell));
-        if (!nc) return -1;
-        m->c = nc;
+        uint32_t* ni = (uint32_t*)realloc(m->ix, cap * sizeof(uint32_t));
+        if (!ni) return -1;
+        m->ix = ni;
         m->cap = cap;
     }
+    if (m->pool_n == m->pool_cap) {
+        const size_t cap = m->pool_cap * 2;
+        Cell* nc = (Cell*)realloc(m->pool, cap * sizeof(Cell));
+        if (!nc) return -1;
+        m->pool = nc;
+        m->pool_cap = cap;
+    }
     memmove(&m->b[lo + 1], &m->b[lo], (m->n + 1 - lo) * sizeof(uint64_t));
-    memmove(&m->c[lo], &m->c[lo - 1], (m->n - (lo - 1)) * sizeof(Cell));
+    memmove(&m->ix[lo], &m->ix[lo - 1], (m->n - (lo - 1)) * sizeof(uint32_t));
+    m->pool[m->pool_n] = m->pool[m->ix[lo - 1]]; /* the upper half starts as a copy of the interval that was cut */
+    m->ix[lo] = (uint32_t)m->pool_n++;
     m->b[lo] = v;
     m->n++;
     return (long)lo;
@@ -214,9 +232,9 @@ int32_t HcommGfxOpListCheck(
                 tmp_cap = m;
             }
             const int64_t shift = (int64_t)o->srcOff - (int64_t)o->dstOff;
-            memcpy(tmp, &sm->c[s0], m * sizeof(Cell)); /* the value before this operation */
+            for (size_t k = 0; k < m; ++k) tmp[k] = CELL(sm, s0 + k); /* the value before this operation */
             for (size_t k = 0; k < m; ++k) {
-                Cell* d = &dm->c[d0 + k];
+                Cell* d = &CELL(dm, d0 + k);
                 Cell s = tmp[k];
                 for (uint32_t q = 0; q < nRanks; ++q)
                     if (s.cnt[q]) s.delta[q] += shift;
@@ -246,7 +264,7 @@ int32_t HcommGfxOpListCheck(
             break;
         }
         for (size_t iv = (size_t)i0; iv < (size_t)i1; ++iv) {
-            const Cell* c = &m->c[iv];
+            const Cell* c = &CELL(m, iv);
             if (c->bad) report(rep, 0, "result of rank %llu at offset %llu mixes one rank's data from two different offsets (buffer %llu)", r, m->b[iv], res_buf);
             for (uint32_t q = 0; q < nRanks; ++q) {
                 if (c->cnt[q] != 1)
@@ -262,7 +280,8 @@ int32_t HcommGfxOpListCheck(
     if (im)
         for (uint32_t q = 0; q < nbuf; ++q) {
             free(im[q].b);
-            free(im[q].c);
+            free(im[q].ix);
+            free(im[q].pool);
         }
     free(im);
     free(extent);
