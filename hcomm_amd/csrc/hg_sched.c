@@ -1122,6 +1122,40 @@ int32_t HcommGfxDoubleRingEmit(
     return HCCL_SUCCESS;
 }
 
+/* Stand-alone ReduceScatterRecursiveHalvingDoubling (temp_reduce_scatter/reduce_scatter_recursive_hd.cc:29-84) in place
+ * on `bytes` of every rank's input, slices of bytes / n (:86-110, not aligned): the even ranks below 2 (n - B), B the
+ * largest power of two <= n, absorb their odd neighbour's whole input (:112-186); the B survivors halve (block rank b
+ * folds, at distance m = B/2, B/4, .., 1, the group of m block slices that contains its own from block rank b ^ m,
+ * reduce_scatter_halving_doubling.cc:65-92,196-249; a survivor that absorbed a neighbour owns both slices); finally the
+ * absorbed odd ranks fetch their slice from the neighbour (:238-300). */
+static int rhd_rs_inplace(HgOpList* l, uint32_t n, uint64_t bytes)
+{
+    if (n == 1) return HCCL_SUCCESS;
+    const uint32_t block = floor_pow2(n);
+    const uint32_t folded = n - block; /* pairs (2i, 2i + 1), i < folded */
+    const uint64_t per = bytes / n;
+    uint32_t step = 0;
+    if (folded) {
+        for (uint32_t i = 0; i < folded; ++i) CHK(push(l, step, REDUCE, 2 * i, IN, 0, 2 * i + 1, IN, 0, bytes));
+        ++step;
+    }
+    /* block rank b stands for rank real(b) and owns the slices of ranks [first_rank(b), first_rank(b + 1)) */
+#define REAL_OF(b) ((b) < folded ? 2u * (b) : (b) + folded)
+    for (uint32_t m = block / 2; m >= 1; m /= 2, ++step)
+        for (uint32_t b = 0; b < block; ++b) {
+            const uint32_t g = b & ~(m - 1);
+            const uint64_t lo = (uint64_t)REAL_OF(g) * per, hi = (uint64_t)(g + m < block ? REAL_OF(g + m) : n) * per;
+            CHK(push(l, step, REDUCE, REAL_OF(b), IN, lo, REAL_OF(b ^ m), IN, lo, hi - lo));
+        }
+#undef REAL_OF
+    if (folded) {
+        for (uint32_t i = 0; i < folded; ++i)
+            CHK(push(l, step, COPY, 2 * i + 1, IN, (uint64_t)(2 * i + 1) * per, 2 * i, IN, (uint64_t)(2 * i + 1) * per, per));
+        ++step;
+    }
+    return HCCL_SUCCESS;
+}
+
 /* ---- the ring and mesh reduce-scatter executors over two communicator levels (op-base mode) --------------------- */
 
 /* CollReduceScatterRingExecutor::KernelRun (coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:
@@ -1172,7 +1206,8 @@ static int hier_rs_build(HgOpList* l, int level0_mesh, int alg1, uint32_t n_serv
                 uint32_t order[HCOMM_GFX_MAX_RANKS];
                 nhr_slice_map(n_servers, 1, order);
                 rc = nhr_rs(&sub, n_servers, sl, order, 0);
-            } else rc = nb_rs(&sub, n_servers, sl);
+            } else if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_NB) rc = nb_rs(&sub, n_servers, sl);
+            else rc = rhd_rs_inplace(&sub, n_servers, c * n);
             uint32_t used = 0;
             for (uint32_t i = 0; i < n_local && rc == HCCL_SUCCESS; ++i) {
                 for (uint32_t srv = 0; srv < n_servers; ++srv) map[srv] = srv * n_local + i;
@@ -1220,7 +1255,7 @@ int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_serve
     if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (level0_mesh && n_local < 2) return HCCL_E_PARA; /* PrepareSliceMeshStreams refuses zero streams */
     if (alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RING && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR &&
-        alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
+        alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RHD)
         return HCCL_E_PARA;
     const int rc = hier_rs_build(l, level0_mesh, alg1, n_servers, n_local, count, ccl_bytes, unit, dtype);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

@@ -391,7 +391,12 @@ typedef enum {
        (temp_reduce/reduce_nhr_oneshot.cc:169-236, a binomial tree folding input into input) followed by
        BroadcastNHROneshot (temp_broadcast/broadcast_nhr_oneshot.cc:24-59,155-205: rank 0 copies input -> output,
        then the tree runs backwards on the outputs).  Any rank count. */
-    HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT = 15
+    HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT = 15,
+    /* ReduceScatterRecursiveHalvingDoubling (temp_reduce_scatter/reduce_scatter_recursive_hd.cc:29-84), which works in
+       place on slices of total / N bytes: accepted only as the level-1 algorithm of
+       HcommGfxHierReduceScatterPlanCreate / Emit / Check (the executors' default between servers); the flat plan
+       and schedule calls return HCCL_E_PARA for it */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_RHD = 16
 } HcommGfxAlgorithm;
 
 typedef enum {
@@ -649,7 +654,7 @@ int32_t HcommGfxDoubleRingCheck(
  * coll_reduce_scatter_mesh_executor.cc:131-259, its branch without atomic adds) over two communicator levels in
  * op-base mode (loop and staging copies of coll_reduce_scatter_executor.cc:149-306, chunks of at most
  * cclBytes / (N * unit) elements per block, N = nServers * nLocal, rank = server * nLocal + local index):
- * user input -> CCL input; level1Alg (HCOMM_GFX_ALG_REDUCE_SCATTER_RING, _NHR or _NB, in place) between the servers over
+ * user input -> CCL input; level1Alg (HCOMM_GFX_ALG_REDUCE_SCATTER_RING, _NHR, _NB or _RHD, in place) between the servers over
  * the nServers runs of nLocal blocks; ring or multi-stream mesh reduce-scatter inside every server over the blocks of
  * its run; own block -> CCL output -> user output.
  * userIn: N * count elements (block b at b * count belongs to rank b); userOut: count; cclIn / cclOut: cclBytes.

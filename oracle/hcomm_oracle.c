@@ -54,7 +54,8 @@
  *                                     reduction trees of both shares N = 4, all by hand; exact integer results over
  *                                     several chunks; pinned
  *   two-level reduce-scatter ........ the complete operation list and the reduction trees of 2 x 2, the trees of the
- *                                     mesh pieces of 1 x 4, a chunk table, by hand; exact integer results; pinned
+ *                                     mesh pieces of 1 x 4, the recursive halving-doubling trees between 3 and 6
+ *                                     servers, a chunk table, by hand; exact integer results; pinned
  *   order-preserving reduce-scatter . the complete operation list N = 3, the rank-order fold trees N = 2..8 and a
  *                                     chunk table by hand; exact integer results over several chunks; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
@@ -1120,7 +1121,8 @@ enum {
     ORC_ALG_RS_NB = 12,
     ORC_ALG_RS_LOCAL_REDUCE = 13,
     ORC_ALG_ALLREDUCE_DOUBLING = 14,
-    ORC_ALG_ALLREDUCE_NHR_ONESHOT = 15
+    ORC_ALG_ALLREDUCE_NHR_ONESHOT = 15,
+    ORC_ALG_RS_RHD = 16 /* only between the servers of the two-level reduce-scatter */
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -1817,6 +1819,75 @@ int orc_dbring_slices(uint64_t count, int dtype, uint32_t n, OrcSlice* out, uint
     return 0;
 }
 
+/* ReduceScatterRecursiveHalvingDoubling::RunAsync for one rank, tpl/temp_reduce_scatter/reduce_scatter_recursive_hd.cc:
+ * 29-84, on data_bytes of the input memory (count_ elements = rankSize slices): everything happens in the input memory
+ * (the inner template is prepared with it as input and output, :223-225, so its closing copy, tpl/temp_reduce_scatter/
+ * reduce_scatter_halving_doubling.cc:251-254, is a copy onto itself, which the dispatcher drops).  Returns the number of
+ * lock-step steps. */
+static uint32_t prog_rs_recursive_hd(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t data_bytes)
+{
+    if (n == 1) return 0; /* :45-50 with inputMem_ == outputMem_ */
+    /* CalcPartOneSizeAndBlockSize, tpl/recursive_halvingdoubling_base.cc:23-37 */
+    uint32_t round = 0;
+    while ((1u << round) <= n) round++;
+    if (round >= 1) round -= 1;
+    const uint32_t block = 1u << round;
+    const uint32_t part1 = (n - block) * 2;
+    uint32_t step = 0;
+    /* ReduceInPartOne, :112-186: an even rank of part one folds the whole input of its odd neighbour into its own */
+    if (part1 > 0) {
+        if (rank < part1 && rank % 2 == 0) emit(t, step, K_REDUCE, rank, B_IN, 0, rank + 1, B_IN, 0, data_bytes);
+        step++;
+    }
+    /* CalculateSlices, :86-110: per block rank; the first part1 / 2 of them carry two ranks' slices */
+    OrcSlice sl[ORC_MAX_RANKS];
+    const uint64_t bytes_per_slice = data_bytes / n;
+    const uint32_t half_part1 = part1 / 2;
+    uint32_t i = 0;
+    while (i < half_part1) {
+        sl[i].size = 2 * bytes_per_slice;
+        sl[i].offset = (uint64_t)i * 2 * bytes_per_slice;
+        i++;
+    }
+    while (i < block) {
+        sl[i].size = bytes_per_slice;
+        sl[i].offset = (uint64_t)i * bytes_per_slice + (uint64_t)half_part1 * bytes_per_slice;
+        i++;
+    }
+    /* ReduceScatterInBlock, :188-236 */
+    const int idle = (rank < part1 && rank % 2 == 1);
+    uint32_t rib = 0;
+    if (!idle) rib = (rank < part1) ? rank / 2 : rank - part1 / 2;
+#define REAL(b) (((b) < part1 / 2) ? 2 * (b) : (b) + part1 / 2) /* BuildSubLinks, tpl/recursive_halvingdoubling_base.cc:39-62 */
+    uint32_t steps = 0;
+    while ((block >> (steps + 1)) != 0) steps++;
+    for (uint32_t s = 0; s < steps; s++) { /* tpl/temp_reduce_scatter/reduce_scatter_halving_doubling.cc:65-92, 196-249 */
+        if (!idle) {
+            const uint32_t mask = 1u << (steps - s - 1);
+            const uint32_t peer = rib ^ mask;
+            const uint32_t id = rib & (~(mask - 1));
+            uint64_t sz = 0;
+            uint32_t num = mask;
+            while (num > 0) {
+                num--;
+                sz += sl[id + num].size;
+            }
+            emit(t, step, K_REDUCE, rank, B_IN, sl[id].offset, REAL(peer), B_IN, sl[id].offset, sz);
+        }
+        step++;
+    }
+#undef REAL
+    /* ScatterInPartOne, :238-300: the odd rank of part one receives its slice from the even neighbour's input */
+    if (part1 > 0) {
+        if (rank < part1 && rank % 2 == 1) {
+            const uint64_t offset = (uint64_t)rank * bytes_per_slice;
+            emit(t, step, K_COPY, rank, B_IN, offset, rank - 1, B_IN, offset, bytes_per_slice);
+        }
+        step++;
+    }
+    return step;
+}
+
 /* ---- the ring and mesh reduce-scatter executors over two communicator levels, op-base mode ---------------------- */
 
 /* CollReduceScatterRingExecutor::KernelRun (exec/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:136-363, one
@@ -1863,9 +1934,11 @@ static void prog_hier_rs(OrcTrace* t, int level0_mesh, int alg1, uint32_t rank, 
             nhr_rank_mapping(n_servers, 1, slice_map); /* GetRankMapping(rankSize, true), reduce_scatter_nhr.cc:86-88 */
             prog_nhr_rs(t, server, n_servers, sl, NULL, slice_map, 0);
             step += nhr_steps(n_servers);
-        } else {
+        } else if (alg1 == ORC_ALG_RS_NB) {
             prog_nb_rs(t, server, n_servers, sl, NULL);
             step += nhr_steps(n_servers);
+        } else { /* the default branch: recursive halving-doubling over inputMem.size() / unit elements, :236-246 / :193-203 */
+            step += prog_rs_recursive_hd(t, server, n_servers, cur_size * n);
         }
     }
     /* second: inside the server, :249-357 / :207-252, on the server's run of the CCL input at base offset
@@ -1901,11 +1974,17 @@ static int build_trace_hier_rs(OrcTrace* t, int level0_mesh, int alg1, uint32_t 
     const uint32_t unit = orc_dtype_size(dtype);
     if (unit == 0 || n_servers == 0 || n_local == 0 || n_servers * n_local > ORC_MAX_RANKS) return -1;
     if (level0_mesh && n_local < 2) return -1;
-    if (alg1 != ORC_ALG_RS_RING_STAGE && alg1 != ORC_ALG_RS_NHR && alg1 != ORC_ALG_RS_NB) return -1;
+    if (alg1 != ORC_ALG_RS_RING_STAGE && alg1 != ORC_ALG_RS_NHR && alg1 != ORC_ALG_RS_NB && alg1 != ORC_ALG_RS_RHD) return -1;
     const uint32_t n = n_servers * n_local;
     const uint64_t max_count = ccl_bytes / ((uint64_t)n * unit); /* CalcLoopMaxCount of both executors, :116-121 */
     if (max_count == 0) return -1;
-    const uint32_t level1_steps = n_servers == 1 ? 0 : (alg1 == ORC_ALG_RS_RING_STAGE ? n_servers - 1 : nhr_steps(n_servers));
+    uint32_t level1_steps = n_servers == 1 ? 0 : (alg1 == ORC_ALG_RS_RING_STAGE ? n_servers - 1 : nhr_steps(n_servers));
+    if (alg1 == ORC_ALG_RS_RHD && n_servers > 1) {
+        OrcTrace dry;
+        memset(&dry, 0, sizeof(dry));
+        level1_steps = prog_rs_recursive_hd(&dry, 0, n_servers, 0); /* zero-sized operations are not recorded */
+        free(dry.ops);
+    }
     uint32_t step0 = 0;
     uint64_t cur_count = 0, user_off = 0;
     for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {

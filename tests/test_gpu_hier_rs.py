@@ -12,7 +12,7 @@ from util import DT, OPS, assert_same, from_dev, gen, to_dev
 pytestmark = pytest.mark.gpu
 
 LEVEL1 = {"ring": (oracle.ALG_RS_RING_STAGE, h.Alg.REDUCE_SCATTER_RING), "nhr": (oracle.ALG_RS_NHR, h.Alg.REDUCE_SCATTER_NHR),
-          "nb": (oracle.ALG_RS_NB, h.Alg.REDUCE_SCATTER_NB)}
+          "nb": (oracle.ALG_RS_NB, h.Alg.REDUCE_SCATTER_NB), "rhd": (oracle.ALG_RS_RHD, h.Alg.REDUCE_SCATTER_RHD)}
 
 # level 0 (mesh?), level-1 algorithm, servers, ranks per server, elements per block, dtype, op, CCL buffer bytes
 CASES = [
@@ -28,6 +28,9 @@ CASES = [
     (True, "ring", 2, 16, 4099, "fp32", "min", 1 << 20),
     (False, "ring", 4, 8, 9, "int32", "sum", 1 << 16),
     (True, "ring", 2, 4, 0, "fp32", "sum", 4096),
+    (False, "rhd", 6, 2, 70001, "fp32", "sum", 1 << 21),       # recursive halving-doubling between 6 servers
+    (True, "rhd", 4, 4, 30007, "bf16", "sum", 1 << 20),
+    (False, "rhd", 17, 1, 10003, "int32", "max", 1 << 20),
 ]
 
 

@@ -15,8 +15,9 @@ from test_oracle_schedules import eval_tree, order_sensitive_inputs
 
 GOLD = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "schedules_hand_derived.json")))["hier_reduce_scatter"]
 LEVEL1 = {oracle.ALG_RS_RING_STAGE: h.Alg.REDUCE_SCATTER_RING, oracle.ALG_RS_NHR: h.Alg.REDUCE_SCATTER_NHR,
-          oracle.ALG_RS_NB: h.Alg.REDUCE_SCATTER_NB}
-SHAPES = [(1, 8), (1, 2), (1, 3), (2, 4), (3, 5), (4, 8), (2, 2), (2, 1), (1, 1), (5, 3), (1, 16), (2, 16), (8, 4)]
+          oracle.ALG_RS_NB: h.Alg.REDUCE_SCATTER_NB, oracle.ALG_RS_RHD: h.Alg.REDUCE_SCATTER_RHD}
+SHAPES = [(1, 8), (1, 2), (1, 3), (2, 4), (3, 5), (4, 8), (2, 2), (2, 1), (1, 1), (5, 3), (1, 16), (2, 16), (8, 4),
+          (6, 2), (7, 1), (17, 1), (31, 1)]
 CCL_IN, CCL_OUT, UIN, UOUT = 0, 1, 3, 4
 
 
@@ -55,6 +56,23 @@ def test_reduction_trees_hand_derived(op):
     for b, first, cnt, tree in GOLD["trees_1x4_mesh_count96"]["pieces"]:
         want = eval_tree(tree, [x[b * count + first:b * count + first + cnt] for x in ins], op)
         assert np.array_equal(out[b][first:first + cnt].view(np.uint32), want.view(np.uint32)), (b, first)
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_recursive_halving_doubling_between_servers_hand_derived(op):
+    for n_s, trees in GOLD["trees_rhd_between_servers"].items():
+        if n_s.startswith("_"):
+            continue
+        n, count = int(n_s), 33
+        ins = order_sensitive_inputs(n, n * count, op, seed=610 + n)
+        out = run(oracle.ALG_RS_RHD, n, 1, ins, count, 1 << 20, oracle.F32, op, False)
+        for b_s, tree in trees.items():
+            b = int(b_s)
+            want = eval_tree(tree, [x[b * count:(b + 1) * count] for x in ins], op)
+            assert np.array_equal(out[b].view(np.uint32), want.view(np.uint32)), (n, b)
+    for f, a in ((oracle.trace, oracle.ALG_RS_RHD), (h.schedule_emit, h.Alg.REDUCE_SCATTER_RHD)):
+        with pytest.raises((ValueError, h.HcommError)):      # only between the servers of the two-level reduce-scatter
+            f(a, 4, 100, oracle.F32)
 
 
 def test_chunk_table_hand_derived():
