@@ -843,18 +843,17 @@ static int append_mapped(HgOpList* l, const HgOpList* sub, const uint32_t* map, 
 }
 
 /* Lists built level by level and, inside a level, group by group: order them by step, then by rank, keeping the
- * order of a rank's operations inside a step (bottom-up merge sort, stable; falls back to leaving the list as built
- * if the scratch array cannot be had, which only costs launches, not correctness of a conflict-free step). */
+ * order of a rank's operations inside a step (bottom-up merge sort, stable). */
 static int op_before(const HcommGfxSchedOp* a, const HcommGfxSchedOp* b)
 {
     return a->step < b->step || (a->step == b->step && a->rank <= b->rank);
 }
 
-static void order_by_step_rank(HgOpList* l)
+static int order_by_step_rank(HgOpList* l)
 {
-    if (l->n < 2) return;
+    if (l->n < 2) return HCCL_SUCCESS;
     HcommGfxSchedOp* tmp = (HcommGfxSchedOp*)malloc(l->n * sizeof(*tmp));
-    if (!tmp) return;
+    if (!tmp) return HCCL_E_MEMORY;
     HcommGfxSchedOp *src = l->ops, *dst = tmp;
     for (uint64_t w = 1; w < l->n; w *= 2) {
         for (uint64_t lo = 0; lo < l->n; lo += 2 * w) {
@@ -870,6 +869,7 @@ static void order_by_step_rank(HgOpList* l)
     }
     if (src != l->ops) memcpy(l->ops, src, l->n * sizeof(*tmp));
     free(tmp);
+    return HCCL_SUCCESS;
 }
 
 /* CollAllReduceRingExecutor::KernelRun (src/legacy/ascend910/algorithm/impl/coll_executor/coll_all_reduce/
@@ -973,12 +973,9 @@ int hg_schedule_hier(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers,
         }
         hg_oplist_free(&sub);
     }
-    if (rc != HCCL_SUCCESS) {
-        hg_oplist_free(l);
-        return rc;
-    }
-    order_by_step_rank(l);
-    return HCCL_SUCCESS;
+    if (rc == HCCL_SUCCESS) rc = order_by_step_rank(l);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
 }
 
 /* ---- the double-ring allreduce executor in op-base mode --------------------------------------------------------- */
@@ -1092,8 +1089,7 @@ static int dbring_build(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_lo
         left -= cur;
     }
     if (rc != HCCL_SUCCESS) return rc;
-    order_by_step_rank(l);
-    return HCCL_SUCCESS;
+    return order_by_step_rank(l);
 }
 
 int hg_schedule_dbring(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
@@ -1243,8 +1239,7 @@ static int hier_rs_build(HgOpList* l, int level0_mesh, int alg1, uint32_t n_serv
         user_off += c;
         left -= cur;
     }
-    order_by_step_rank(l);
-    return HCCL_SUCCESS;
+    return order_by_step_rank(l);
 }
 
 int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
