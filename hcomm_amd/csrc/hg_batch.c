@@ -160,7 +160,7 @@ static int coalesce_one(Coalescer* c, const HgOp* o)
     HgLaunch* l = c->l;
     const uint32_t kind = kind_of(o);
     const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
-    if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG || conflicts(l, o))) {
+    if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG2 || conflicts(l, o))) {
         hg_finish_seg2(l);
         c->open = 0;
         const int rc = c->emit(l, c->ctx);

@@ -14,7 +14,8 @@
 extern "C" {
 #endif
 
-#define HG_MAX_SEG 32u          /* segments per launch */
+#define HG_MAX_SEG 32u          /* segments per k-way fold launch */
+#define HG_MAX_SEG2 64u         /* segments per copy / two-input reduce launch */
 #define HG_VEC_BYTES 16u        /* one lane moves 128 bits per access */
 #ifndef HG_BLOCK
 #define HG_BLOCK 256u           /* threads per workgroup = 4 wavefronts of 64 */
@@ -31,10 +32,10 @@ extern "C" {
 
 /* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
 typedef struct {
-    void* dst[HG_MAX_SEG];
-    const void* src[HG_MAX_SEG];
-    uint64_t bytes[HG_MAX_SEG];
-    uint32_t tile_begin[HG_MAX_SEG + 1]; /* prefix sum of tiles per segment */
+    void* dst[HG_MAX_SEG2];
+    const void* src[HG_MAX_SEG2];
+    uint64_t bytes[HG_MAX_SEG2];
+    uint32_t tile_begin[HG_MAX_SEG2 + 1]; /* prefix sum of tiles per segment */
     uint32_t nseg;
 } HgSeg2Table;
 

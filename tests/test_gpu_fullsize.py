@@ -199,7 +199,7 @@ def test_nhr_and_nb_int32_full_size_closed_form(gpu_thread, algname, n, count, l
         assert info.launches == 1
     elif algname == "nhr":      # touching slices are merged: one segment or two per rank, one launch per step
         assert info.launches == 2 * steps + 1
-    else:                       # NB keeps its slices apart: a step of 16 ranks x 8 slices needs 4 launches of 32 segments
+    else:                       # NB keeps its slices apart: a step of 16 ranks x 8 slices needs 2 launches of 64 segments
         assert info.launches >= 2 * steps + 1
     for r in range(n):
         assert torch.equal(outs[r], want), "out[%d]" % r

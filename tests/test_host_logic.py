@@ -211,7 +211,7 @@ def test_local_reduce_plan_needs_scratch_and_power_of_two(rec):
     p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i, o, count, DT.FP32, OP.SUM, 0, sc)
     # own copy | 6 gather rounds merged | neighbour reduce | fold + 2 halving rounds | own gather + 7 rounds merged
     kinds = [(r.kind, r.nseg) for r in p.launches()]
-    assert kinds[0] == (h.Kernel.COPY, 32) and sum(ns for k, ns in kinds if k == h.Kernel.COPY) == 8 + 48 + 8 + 56
+    assert kinds[0] == (h.Kernel.COPY, 56) and sum(ns for k, ns in kinds if k == h.Kernel.COPY) == 8 + 48 + 8 + 56
     assert sum(ns for k, ns in kinds if k == h.Kernel.REDUCE2) == 8 + 8 * 3 + 8 * 2 + 8 * 1
     assert p.info.movedBytes == p.info.algorithmicBytes
     p.destroy()
@@ -282,8 +282,8 @@ def test_batch_mode_splits_on_conflict_kind_type_and_capacity(rec):
     assert run([red(A + 4, B + 8)]) == [(K.BYTEWISE, 1)]                          # different misalignment
     small = lambda: h.HcommLocalReduceOnThread(rec, A + 4, B + 4, 1000, DT.FP32, OP.SUM)
     assert run([small]) == [(K.BYTEWISE, 1)]                                      # too small to be worth two launches
-    many = [cp(DST + (2 * i) * mib, DST + (2 * i + 1) * mib) for i in range(70)]
-    assert run(many) == [(K.COPY, 32), (K.COPY, 32), (K.COPY, 6)]                 # 32 segments per launch
+    many = [cp(DST + (2 * i) * mib, DST + (2 * i + 1) * mib) for i in range(134)]
+    assert run(many) == [(K.COPY, 64), (K.COPY, 64), (K.COPY, 6)]                 # 64 segments per launch
 
 
 def test_batch_mode_spans_several_threads(rec):
