@@ -151,16 +151,48 @@ static int conflicts(const HgLaunch* l, const HgOp* o)
 typedef struct {
     HgLaunch* l;
     int open;
+    uint64_t bytes; /* written by the open launch so far */
     HgEmitFn emit;
     void* ctx;
 } Coalescer;
+
+/* A copy launch stops growing once it writes half a GiB.  Measured on the schedules whose copy steps are larger (the 64
+ * plants of the order-preserving reduce-scatter, the gather of the deterministic mesh allreduce: 1 GiB written per
+ * step): two launches of 512 MiB run 1 - 2 % faster than one of 1 GiB, while steps of many small segments (the 56
+ * pieces of a mesh reduce-scatter round) gain 4 % from sharing one launch. */
+#define HG_COPY_LAUNCH_BYTES (512ull << 20)
+
+static uint64_t copy_launch_bytes(void)
+{
+    static uint64_t cap = 0;
+    if (cap == 0) {
+        const char* e = getenv("HCOMM_GFX_COPY_LAUNCH_MIB"); /* experiments; 0 = no limit */
+        cap = e ? (strtoull(e, NULL, 10) ? strtoull(e, NULL, 10) << 20 : UINT64_MAX) : HG_COPY_LAUNCH_BYTES;
+    }
+    return cap;
+}
+
+/* segments a copy / two-input reduce launch may carry: the table's size, or less when HCOMM_GFX_MAX_SEGMENTS says so
+ * (experiments) */
+static uint32_t seg2_cap(void)
+{
+    static uint32_t cap = 0;
+    if (cap == 0) {
+        const char* e = getenv("HCOMM_GFX_MAX_SEGMENTS");
+        const unsigned long v = e ? strtoul(e, NULL, 10) : 0;
+        cap = (v >= 1 && v <= HG_MAX_SEG2) ? (uint32_t)v : HG_MAX_SEG2;
+    }
+    return cap;
+}
 
 static int coalesce_one(Coalescer* c, const HgOp* o)
 {
     HgLaunch* l = c->l;
     const uint32_t kind = kind_of(o);
     const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
-    if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || l->tab.seg2.nseg == HG_MAX_SEG2 || conflicts(l, o))) {
+    const int full = l->tab.seg2.nseg == seg2_cap() ||
+                     (kind == HCOMM_GFX_KERNEL_COPY && c->bytes + o->bytes > copy_launch_bytes());
+    if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || full || conflicts(l, o))) {
         hg_finish_seg2(l);
         c->open = 0;
         const int rc = c->emit(l, c->ctx);
@@ -172,7 +204,9 @@ static int coalesce_one(Coalescer* c, const HgOp* o)
         l->dtype = dt;
         l->op = op;
         c->open = 1;
+        c->bytes = 0;
     }
+    c->bytes += o->bytes;
     HgSeg2Table* t = &l->tab.seg2;
     t->dst[t->nseg] = o->dst;
     t->src[t->nseg] = o->src;
@@ -192,6 +226,7 @@ int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
     c.l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
     if (!c.l) return HCCL_E_MEMORY;
     c.open = 0;
+    c.bytes = 0;
     c.emit = emit;
     c.ctx = ctx;
     int rc = HCCL_SUCCESS;

@@ -190,13 +190,9 @@ template <bool REMAP> __device__ __forceinline__ uint32_t block_id()
 // on the scalar unit; bisection keeps it at 6 probes for the largest table)
 __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
 {
-    uint32_t lo = 0, hi = nseg;
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (tile >= tile_begin[mid]) lo = mid;
-        else hi = mid;
-    }
-    return lo;
+    uint32_t s = 0;
+    while (s + 1 < nseg && tile >= tile_begin[s + 1]) ++s;
+    return s;
 }
 
 template <int DT, int OP> struct VecItem {

@@ -54,7 +54,7 @@ def test_config3_rhd_int32_16_ranks_128MiB(gpu_thread, opname, lowering):
     op = {"sum": oracle.SUM, "max": oracle.MAX, "min": oracle.MIN}[opname]
     info = run_plan(gpu_thread, h.Alg.ALLREDUCE_RHD, lowering, ins, outs, count, oracle.I32, op)
     assert info.algorithmicBytes == 10334765056
-    assert info.launches == (9 if lowering == h.Lowering.STEPWISE else 1)
+    assert info.launches == (10 if lowering == h.Lowering.STEPWISE else 1)   # 9 steps; the last gather (1 GiB) in two launches
     for r in range(n):
         assert torch.equal(outs[r], want), "out[%d]" % r
 
@@ -197,8 +197,8 @@ def test_nhr_and_nb_int32_full_size_closed_form(gpu_thread, algname, n, count, l
     steps = (n - 1).bit_length()
     if lowering == h.Lowering.FUSED:
         assert info.launches == 1
-    elif algname == "nhr":      # touching slices are merged: one segment or two per rank, one launch per step
-        assert info.launches == 2 * steps + 1
+    elif algname == "nhr":      # touching slices are merged: one segment or two per rank, one launch per step (a copy
+        assert 2 * steps + 1 <= info.launches <= 2 * steps + 3   # step that writes more than 512 MiB is cut)
     else:                       # NB keeps its slices apart: a step of 16 ranks x 8 slices needs 2 launches of 64 segments
         assert info.launches >= 2 * steps + 1
     for r in range(n):
