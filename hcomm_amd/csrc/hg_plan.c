@@ -100,7 +100,8 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
         uint64_t j = i;
         uint64_t reduces = 0;
         while (j < n && list[j].step == list[i].step) reduces += ops[j++].is_reduce;
-        if (reduces != 0 && reduces != j - i && step_is_conflict_free(ops + i, j - i)) {
+        /* the pairwise test is quadratic: steps larger than any schedule here produces keep their order */
+        if (reduces != 0 && reduces != j - i && j - i <= 4096 && step_is_conflict_free(ops + i, j - i)) {
             HgOp* tmp = (HgOp*)malloc((j - i) * sizeof(HgOp));
             if (!tmp) {
                 free(ops);
