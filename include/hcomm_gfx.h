@@ -6,11 +6,17 @@
  * name and numeric value, so a caller compiled against the reference headers can bind these symbols
  * unchanged.  Citations are paths relative to the reference tree.
  *
- * Three groups of entry points:
+ * Four groups of entry points:
  *   1. drop-in primitives      - same names, argument meaning and return codes as the reference;
  *   2. HcommGfx* extensions    - k-way fused reduce, stream sync, launch log (no reference counterpart);
- *   3. HcommGfxPlan*           - build once / run many replay of the ring, recursive halving-doubling
- *                                and mesh schedules over N simulated ranks (N pairs of HBM buffers).
+ *   3. HcommGfxPlan*           - build once / run many replay of the templates' schedules (ring, recursive
+ *                                halving-doubling, mesh, NHR, NB, doubling, deterministic local reduce, chunk mesh)
+ *                                over N simulated ranks (N pairs of HBM buffers), with HcommGfxSchedule* to obtain
+ *                                the operation lists and check them symbolically without a GPU;
+ *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
+ *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*: what the reference's executors do
+ *                                around the templates (chunk loops through the CCL buffers, two communicator
+ *                                levels, user memory read and written directly), each as PlanCreate / Emit / Check.
  */
 #ifndef HCOMM_GFX_H
 #define HCOMM_GFX_H
