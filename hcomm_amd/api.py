@@ -30,6 +30,7 @@ __all__ = [
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
+    "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -568,6 +569,42 @@ class HierReduceScatterPlan(Plan):
         p = _vp(0)
         check(_hrs_plan(int(mesh), alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3],
                         ccl_bytes, count, dtype, op, C.byref(p)), "HcommGfxHierReduceScatterPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_dbrs_emit = _sig("HcommGfxDoubleRingReduceScatterEmit", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+                  C.POINTER(_u64))
+_dbrs_check = _sig("HcommGfxDoubleRingReduceScatterCheck", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_dbrs_plan = _sig("HcommGfxDoubleRingReduceScatterPlanCreate", _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                  _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def dbring_rs_emit(n_ranks, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_dbrs_emit(n_ranks, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxDoubleRingReduceScatterEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_dbrs_emit(n_ranks, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxDoubleRingReduceScatterEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def dbring_rs_check(n_ranks, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_dbrs_check(n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxDoubleRingReduceScatterCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class DoubleRingReduceScatterPlan(Plan):
+    """HcommGfxDoubleRingReduceScatterPlanCreate: the double-ring reduce-scatter executor on one server, DMA reduce."""
+
+    def __init__(self, user_in, user_out, ccl_in, ccl_bytes, count, dtype, op):
+        n = len(user_in)
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in)]
+        p = _vp(0)
+        check(_dbrs_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
+              "HcommGfxDoubleRingReduceScatterPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

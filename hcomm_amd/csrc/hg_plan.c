@@ -693,6 +693,28 @@ int32_t HcommGfxHierReduceScatterPlanCreate(
     return rc;
 }
 
+int32_t HcommGfxDoubleRingReduceScatterPlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclIn, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!userIn || !userOut || !cclIn) return HCCL_E_PTR;
+    if (nRanks < 3 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(userIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclIn, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_dbring_rs(&ol, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {cclIn, NULL, NULL, userIn, userOut};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nRanks, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
+}
+
 int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint32_t first, uint32_t n)
 {
     if (!plan || plan->magic != HG_PLAN_MAGIC) return HCCL_E_PTR;

@@ -1274,6 +1274,88 @@ int32_t HcommGfxHierReduceScatterEmit(
     return HCCL_SUCCESS;
 }
 
+/* ---- the double-ring reduce-scatter executor on one server (op-base mode, DMA reduce) ------------------------------ */
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor on a single server (coll_executor/coll_reduce_scatter/
+ * coll_aligned_reduce_scatter_double_ring_for_910_93_executor.cc:22-86; slices and user-memory slices of its base,
+ * coll_reduce_scatter_ring_for_910_93_executor.cc:213-316; template alg_template/temp_reduce_scatter/
+ * aligned_reduce_scatter_double_ring.cc with both user addresses set), chunked by the reduce-scatter loop.  Per chunk of
+ * c bytes per block, with dir = -1 for ring 0 (first shares) and +1 for ring 1 (second shares), every rank r
+ *   step 0: fetches the shares of blocks r + dir and r + 2 dir from its user input into its CCL input;
+ *   step 1 + s, s < N - 2: folds the share of block r + (2 + s) dir of rank r + dir's CCL input into its own and
+ *     fetches the share of block r + (3 + s) dir - which for s = N - 3 is its own block and goes to the user output;
+ *   last step: folds the share of its own block of rank r + dir's CCL input into its user output. */
+static int dbring_rs_build(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, uint32_t unit)
+{
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint64_t stride = count * unit;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        uint64_t first = ((c + 1) / 2 + 127u) / 128u * 128u; /* MutliSegSlicePrepare, coll_comm_executor.cc:2011-2052 */
+        if (first > c) first = c;
+        const uint64_t off[2] = {0, first}, len[2] = {first, c - first};
+#define BLK(r, k, ring) (((r) + (uint64_t)n * 4u + (uint64_t)(k) * ((ring) ? 1u : n - 1u)) % n)
+        for (uint32_t r = 0; r < n; ++r)
+            for (uint32_t ring = 0; ring < 2; ++ring)
+                for (uint32_t k = 1; k <= 2; ++k) {
+                    const uint64_t b = BLK(r, k, ring);
+                    CHK(push(l, step, COPY, r, IN, b * c + off[ring], r, UIN, user_off + b * stride + off[ring], len[ring]));
+                }
+        for (uint32_t s = 0; s + 1 < n; ++s)
+            for (uint32_t r = 0; r < n; ++r)
+                for (uint32_t ring = 0; ring < 2; ++ring) {
+                    const uint64_t b = BLK(r, 2 + s, ring);
+                    const uint32_t peer = (uint32_t)BLK(r, 1, ring);
+                    if (s + 2 == n) {
+                        CHK(push(l, step + 1 + s, REDUCE, r, UOUT, user_off + off[ring], peer, IN, b * c + off[ring], len[ring]));
+                        continue;
+                    }
+                    CHK(push(l, step + 1 + s, REDUCE, r, IN, b * c + off[ring], peer, IN, b * c + off[ring], len[ring]));
+                    const uint64_t nb = BLK(r, 3 + s, ring);
+                    if (s + 3 == n)
+                        CHK(push(l, step + 1 + s, COPY, r, UOUT, user_off + off[ring], r, UIN, user_off + nb * stride + off[ring], len[ring]));
+                    else
+                        CHK(push(l, step + 1 + s, COPY, r, IN, nb * c + off[ring], r, UIN, user_off + nb * stride + off[ring], len[ring]));
+                }
+#undef BLK
+        step += n;
+        user_off += c;
+        left -= cur;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_dbring_rs(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n < 3 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    const int rc = dbring_rs_build(l, n, count, ccl_bytes, unit);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxDoubleRingReduceScatterEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_dbring_rs(&l, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 /* ---- the order-preserving reduce-scatter executor (one server, op-base mode) ------------------------------------- */
 
 /* CollReduceScatterOrderPreservedExecutor (coll_executor/coll_reduce_scatter/

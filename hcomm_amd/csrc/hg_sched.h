@@ -33,6 +33,9 @@ int hg_schedule_order_preserved(HgOpList* l, uint32_t n, uint64_t count, uint64_
  * (in-place ring, NHR or NB reduce-scatter) between the servers first, then the level-0 reduce-scatter inside. */
 int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
                         uint64_t ccl_bytes, int dtype);
+/* The double-ring reduce-scatter executor on one server in op-base mode with DMA reduce: user input read share by share,
+ * the result folded straight into the user output. */
+int hg_schedule_dbring_rs(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 void hg_oplist_free(HgOpList* l);
 /* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);

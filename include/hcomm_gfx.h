@@ -655,6 +655,26 @@ int32_t HcommGfxDoubleRingCheck(
     HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
+ * The reduce-scatter of the reference's double-ring executor on one server in op-base mode with DMA reduce
+ * (coll_executor/coll_reduce_scatter/coll_aligned_reduce_scatter_double_ring_for_910_93_executor.cc:22-86, slices of
+ * coll_reduce_scatter_ring_for_910_93_executor.cc:213-316, AlignedReduceScatterDoubleRing with both user addresses):
+ * per chunk of at most cclBytes / nRanks (rounded down to 128 bytes) / unit elements per block, every block is cut in
+ * two shares that are reduced around two mirrored rings through the CCL input buffers, fetched from the user input just
+ * before they are needed; the last fold of a rank's own block lands in its user output, which the step before filled
+ * with the rank's own share.  userIn: nRanks * count elements (block b at b * count); userOut: count; cclIn: cclBytes.
+ * nRanks >= 3 (the template's two-rank first step, :353-360, leaves the neighbour's share unwritten; the double-ring
+ * servers have more).  The executor's stages between servers and super pods are not built.
+ */
+int32_t HcommGfxDoubleRingReduceScatterPlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclIn, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxDoubleRingReduceScatterEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n);
+int32_t HcommGfxDoubleRingReduceScatterCheck(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
  * The reduce-scatter of the reference's ring executor (level0Mesh 0: coll_executor/coll_reduce_scatter/
  * coll_reduce_scatter_ring_executor.cc:136-363, one ring per server) or mesh executor (level0Mesh 1:
  * coll_reduce_scatter_mesh_executor.cc:131-259, its branch without atomic adds) over two communicator levels in

@@ -1888,6 +1888,135 @@ static uint32_t prog_rs_recursive_hd(OrcTrace* t, uint32_t rank, uint32_t n, uin
     return step;
 }
 
+/* ---- the double-ring reduce-scatter executor on one server, op-base mode with DMA reduce ------------------------- */
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor (exec/coll_reduce_scatter/
+ * coll_aligned_reduce_scatter_double_ring_for_910_93_executor.cc:22-86; KernelRun of its base, exec/coll_reduce_scatter/
+ * coll_reduce_scatter_ring_for_910_93_executor.cc:595-687) for one rank and one chunk on a single server: the slices of
+ * ReduceScatterRingSlicePrepare (exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:491-535: blocks of the output
+ * size, each cut in two shares by PrepareMultiRingSlice), the user-memory slices of CalUserMemDataSegsSlice (:297-313:
+ * block index * count * unit + the ring's first slice offset), and AlignedReduceScatterDoubleRing with both user
+ * addresses set (tpl/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc): the last reduce lands in the user output
+ * at lastStepOffsets_ (:229-238, :452-458), which the step before initialises from the user input (:490-500). */
+static void prog_dbring_rs_user_out(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t cur_size, uint64_t stride_bytes)
+{
+    /* multiStreamSlice / level0DataSegsSlice */
+    OrcSlice seg[ORC_MAX_RANKS], multi_seg[ORC_MAX_RANKS][2], slices[2][ORC_MAX_RANKS], user[2][ORC_MAX_RANKS];
+    uint32_t order[2][ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) {
+        seg[i].size = cur_size;
+        seg[i].offset = cur_size * i;
+    }
+    for (uint32_t rank_id = 0; rank_id < n; rank_id++) { /* MutliSegSlicePrepare, exec/coll_comm_executor.cc:2011-2052 */
+        const uint64_t size_per_ring = ((seg[rank_id].size + 1) / 2 + 127) / 128 * 128;
+        uint64_t residue = seg[rank_id].size;
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const uint64_t single = size_per_ring < residue ? size_per_ring : residue;
+            multi_seg[rank_id][ring].size = single;
+            multi_seg[rank_id][ring].offset = single ? seg[rank_id].offset + seg[rank_id].size - residue : seg[rank_id].offset;
+            residue -= single;
+        }
+    }
+    for (uint32_t i = 0; i < n; i++) order[0][i] = i;
+    order[1][0] = 0;
+    for (uint32_t i = 1; i < n; i++) order[1][i] = order[0][n - i];
+    for (uint32_t ring = 0; ring < 2; ring++)
+        for (uint32_t i = 0; i < n; i++) slices[ring][i] = multi_seg[order[ring][i]][ring];
+    for (uint32_t ring = 0; ring < 2; ring++) /* CalUserMemDataSegsSlice, :297-313 */
+        for (uint32_t i = 0; i < n; i++) {
+            user[ring][i].size = slices[ring][i].size;
+            user[ring][i].offset = (slices[ring][i].offset / cur_size) * stride_bytes + slices[ring][0].offset;
+        }
+    /* SetSlices, :190-240: ringsOrders_ = the positions of each ring's devices in ring 0 = the orders themselves */
+    uint64_t last_step_offset[2];
+    last_step_offset[0] = slices[0][order[0][0]].offset;
+    last_step_offset[1] = slices[1][order[1][rank]].offset - slices[0][order[0][rank]].offset;
+
+    const uint32_t pre[2] = {(rank + n - 1) % n, (rank + 1) % n};
+    const uint32_t init0[2] = {(rank + n - 1) % n, (n - rank - 1 + n) % n};
+    const uint32_t init1[2] = {(rank + n - 2) % n, (n - rank - 2 + n) % n};
+    for (uint32_t ring = 0; ring < 2; ring++) { /* RunInitStep, :379-412 (rankSize > 2) */
+        emit(t, 0, K_COPY, rank, B_IN, slices[ring][init0[ring]].offset, rank, B_UIN, user[ring][init0[ring]].offset,
+             slices[ring][init0[ring]].size);
+        emit(t, 0, K_COPY, rank, B_IN, slices[ring][init1[ring]].offset, rank, B_UIN, user[ring][init1[ring]].offset,
+             slices[ring][init1[ring]].size);
+    }
+    uint32_t rx[2] = {(rank + n - 2) % n, (n - rank - 2 + n) % n};
+    uint32_t sub[2] = {(rank + n - 3) % n, (n - rank - 3 + n) % n};
+    for (uint32_t step = 0; step < n - 1; step++) {
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const OrcSlice* rx_slice = &slices[ring][rx[ring]];
+            const OrcSlice* ccl_slice = &slices[ring][sub[ring]];
+            const OrcSlice* sub_slice = &user[ring][sub[ring]];
+            if (step == n - 2) /* :452-458 */
+                emit(t, 1 + step, K_REDUCE, rank, B_UOUT, last_step_offset[ring], pre[ring], B_IN, rx_slice->offset, rx_slice->size);
+            else
+                emit(t, 1 + step, K_REDUCE, rank, B_IN, rx_slice->offset, pre[ring], B_IN, rx_slice->offset, rx_slice->size);
+            if (step == n - 2) {
+                /* :487-489 */
+            } else if (step == n - 3) { /* :490-500 */
+                emit(t, 1 + step, K_COPY, rank, B_UOUT, last_step_offset[ring], rank, B_UIN, sub_slice->offset, sub_slice->size);
+            } else { /* :501-511 */
+                emit(t, 1 + step, K_COPY, rank, B_IN, ccl_slice->offset, rank, B_UIN, sub_slice->offset, ccl_slice->size);
+            }
+            rx[ring] = (rx[ring] + n - 1) % n;
+            sub[ring] = (sub[ring] + n - 1) % n;
+        }
+    }
+}
+
+static int build_trace_dbring_rs(OrcTrace* t, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    /* two ranks take a first step of their own in the template (:353-360) that does not hold together; the double-ring
+     * topologies have more */
+    if (unit == 0 || n < 3 || n > ORC_MAX_RANKS) return -1;
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit; /* CalcLoopMaxCount, coll_reduce_scatter_ring_for_910_93_executor.cc:167-173 */
+    if (max_count == 0) return -1;
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        g_user_off = user_off;
+        g_step_base = step0;
+        for (uint32_t r = 0; r < n; r++) prog_dbring_rs_user_out(t, r, n, cur_count * unit, count * unit);
+        g_user_off = 0;
+        g_step_base = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += n;
+        user_off += cur_count * unit;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_dbring_rs(uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring_rs(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_dbring_rs(uint32_t n, void* const* user_in, void* const* user_out, void* const* ccl_in, uint64_t count,
+                      uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring_rs(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, NULL, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
 /* ---- the ring and mesh reduce-scatter executors over two communicator levels, op-base mode ---------------------- */
 
 /* CollReduceScatterRingExecutor::KernelRun (exec/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:136-363, one
