@@ -56,6 +56,8 @@
  *   two-level reduce-scatter ........ the complete operation list and the reduction trees of 2 x 2, the trees of the
  *                                     mesh pieces of 1 x 4, the recursive halving-doubling trees between 3 and 6
  *                                     servers, a chunk table, by hand; exact integer results; pinned
+ *   double-ring reduce-scatter ...... one rank's complete operation list N = 3, the trees of both shares N = 4 and a
+ *                                     chunk / share table by hand; exact integer results over several chunks; pinned
  *   order-preserving reduce-scatter . the complete operation list N = 3, the rank-order fold trees N = 2..8 and a
  *                                     chunk table by hand; exact integer results over several chunks; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
