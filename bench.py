@@ -71,6 +71,8 @@ WORKLOADS = {
     "dbring_nhr_ar_bf16_2x8_128MiB": ("dbring_nhr", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving reduce-scatter executor: plant into the peers' CCL output buffers, fold in rank order
     "order_preserved_rs_bf16_n8_16MiB": ("order_preserved_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the order-preserving allreduce executor: plant with a borrowed slot, fold in rank order, mesh all-gather
+    "order_preserved_ar_bf16_n8_128MiB": ("order_preserved_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the double-ring reduce-scatter executor on one server with DMA reduce
     "dbring_rs_bf16_n8_16MiB": ("doublering_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     # the ring / mesh reduce-scatter executors over two levels in op-base mode (blocks of 16 MiB, 2 x 8 ranks)
@@ -148,7 +150,9 @@ def main():
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
-    plant = alg_name in ("order_preserved_rs", "doublering_rs")  # one-server reduce-scatter executors on user memory
+    # one-server executors on user memory (DMA reduce)
+    plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar")
+    opar = alg_name == "order_preserved_ar"
     dbrs = alg_name == "doublering_rs"
     dt, alg, op = DT[dtname], (None if plant else ALG[alg_name]), OP[opname]
     unit = h.DTYPE_SIZE[dt]
@@ -200,6 +204,9 @@ def main():
                                            [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, mesh=mesh0)
         if dbrs:
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
+        if opar:
+            return h.OrderPreservedAllReducePlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
+                                                 [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if plant:
             return h.OrderPreservedPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if dbring:
@@ -292,7 +299,7 @@ def main():
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
                 "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
-                "order_preserved_rs": None, "doublering_rs": None}[alg_name]
+                "order_preserved_rs": None, "doublering_rs": None, "order_preserved_ar": None}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
@@ -304,6 +311,8 @@ def main():
                             for o in oracle.trace_hier_rs(oalg, hier[0], hier[1], count, ccl_bytes, odt, mesh=mesh0))
         elif dbrs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs(n, count, ccl_bytes, odt))
+        elif opar:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved_ar(n, count, ccl_bytes, odt))
         elif plant:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved(n, count, ccl_bytes, odt))
         elif dbring:
@@ -324,6 +333,8 @@ def main():
                                    mesh=mesh0)
             elif dbrs:
                 oracle.run_dbring_rs(ins, outs, host_ccl[0], count, ccl_bytes, odt, oop)
+            elif opar:
+                oracle.run_order_preserved_ar(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif plant:
                 oracle.run_order_preserved(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif dbring:

@@ -29,6 +29,7 @@ __all__ = [
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
+    "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
@@ -528,6 +529,42 @@ class OrderPreservedPlan(Plan):
         p = _vp(0)
         check(_op_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
               "HcommGfxOrderPreservedPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_opar_emit = _sig("HcommGfxOrderPreservedAllReduceEmit", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
+                  C.POINTER(_u64))
+_opar_check = _sig("HcommGfxOrderPreservedAllReduceCheck", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_opar_plan = _sig("HcommGfxOrderPreservedAllReducePlanCreate", _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp),
+                  C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def order_preserved_ar_emit(n_ranks, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_opar_emit(n_ranks, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxOrderPreservedAllReduceEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_opar_emit(n_ranks, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxOrderPreservedAllReduceEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def order_preserved_ar_check(n_ranks, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_opar_check(n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxOrderPreservedAllReduceCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class OrderPreservedAllReducePlan(Plan):
+    """HcommGfxOrderPreservedAllReducePlanCreate: the order-preserving allreduce executor on one server, op-base mode."""
+
+    def __init__(self, user_in, user_out, ccl_in, ccl_out, ccl_bytes, count, dtype, op):
+        n = len(user_in)
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in, ccl_out)]
+        p = _vp(0)
+        check(_opar_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3], ccl_bytes, count, dtype, op,
+                         C.byref(p)), "HcommGfxOrderPreservedAllReducePlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -668,6 +668,29 @@ int32_t HcommGfxOrderPreservedPlanCreate(
     return rc;
 }
 
+int32_t HcommGfxOrderPreservedAllReducePlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclIn, void* const* cclOut,
+    uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!userIn || !userOut || !cclIn || !cclOut) return HCCL_E_PTR;
+    if (nRanks < 2 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(userIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclOut, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_order_preserved_ar(&ol, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {cclIn, cclOut, NULL, userIn, userOut};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nRanks, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
+}
+
 int32_t HcommGfxHierReduceScatterPlanCreate(
     int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn,
     void* const* userOut, void* const* cclIn, void* const* cclOut, uint64_t cclBytes, uint64_t count,

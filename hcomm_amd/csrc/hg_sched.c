@@ -1421,6 +1421,95 @@ int32_t HcommGfxOrderPreservedEmit(
     return HCCL_SUCCESS;
 }
 
+/* ---- the order-preserving allreduce executor (one server, op-base mode) ------------------------------------------- */
+
+/* CollAllReduceOrderPreservedExecutor (coll_executor/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:
+ * 131-193, 248-283, 342-380), chunked by the allreduce loop (coll_all_reduce_executor.cc:129-138, 212-252, DMA reduce:
+ * no staging copies).  Per chunk of c elements: block size B = ceil(c / N) elements rounded up to 128 bytes, block d
+ * = bytes [d * B, min((d + 1) * B, chunk bytes)) - the trailing blocks may be short or empty.
+ *   step 0: every rank q plants block p of its user input into slot (p + q) mod N of rank p's CCL output buffer; the
+ *           last slot of every rank but the last is "borrowed" from the rank's CCL INPUT buffer at p * B, so that the
+ *           N slots of B bytes never reach past the chunk's size (reduce_scatter_plant_local_reduce.cc:168-188, 221-247);
+ *   ceil(log2 N) rounds: the fold tree over rank order of the order-preserving reduce-scatter (:337-414);
+ *   then the mesh all-gather of the N blocks inside the CCL output buffers (all_gather_mesh_atomic.cc:19-69: round r
+ *           reads the block of rank p - r), and the whole chunk from there to the user output (:369-376). */
+static int order_preserved_ar_build(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, uint32_t unit)
+{
+    const uint64_t max_count = ccl_bytes / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint32_t rounds = ceil_log2(n);
+    const uint32_t last = n - 1;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    uint64_t size[HCOMM_GFX_MAX_RANKS];
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        const uint64_t blk = ((cur + n - 1) / n * unit + 127u) / 128u * 128u;
+        for (uint32_t d = 0; d < n; ++d) size[d] = (uint64_t)d * blk >= c ? 0 : (c - d * blk < blk ? c - d * blk : blk);
+        /* the slots of rank p sit at multiples of blk: they fit the buffers whenever they fit the chunk; a tiny
+         * chunk whose rounded-up blocks reach past the CCL buffer is an error in the reference as well (DeviceMem::range
+         * hands back an empty range) */
+        for (uint32_t p = 0; p < n; ++p)
+            if (size[p] && (uint64_t)(p == last ? last : last - 1) * blk + size[p] > ccl_bytes) return HCCL_E_PARA;
+        for (uint32_t p = 0; p < n; ++p)
+            for (uint32_t q = 0; q < n; ++q) {
+                const uint32_t slot = (p + q) % n;
+                if (slot == last && p != last)
+                    CHK(push(l, step, COPY, p, IN, blk * p, q, UIN, user_off + blk * p, size[p]));
+                else
+                    CHK(push(l, step, COPY, p, OUT, blk * slot, q, UIN, user_off + blk * p, size[p]));
+            }
+        ++step;
+        for (uint32_t h = 1u << (rounds - 1); h >= 1; h >>= 1, ++step)
+            for (uint32_t p = 0; p < n; ++p)
+                for (uint32_t j = 0; j + h < (n < 2 * h ? n : 2 * h); ++j) {
+                    const uint32_t to = (j + p) % n, from = (h + j + p) % n;
+                    const int to_in = p != last && to == last, from_in = p != last && from == last;
+                    CHK(push(l, step, REDUCE, p, to_in ? IN : OUT, to_in ? blk * p : blk * to, p, from_in ? IN : OUT,
+                             from_in ? blk * p : blk * from, size[p]));
+                }
+        for (uint32_t p = 0; p < n; ++p)
+            for (uint32_t r = 1; r < n; ++r) {
+                const uint32_t src = (p + n - r) % n;
+                CHK(push(l, step, COPY, p, OUT, blk * src, src, OUT, blk * src, size[src]));
+            }
+        ++step;
+        for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, user_off, p, OUT, 0, c));
+        ++step;
+        user_off += c;
+        left -= cur;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_order_preserved_ar(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    const int rc = order_preserved_ar_build(l, n, count, ccl_bytes, unit);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedAllReduceEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved_ar(&l, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 int32_t HcommGfxHierEmit(
     HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, HcommDataType dataType,
     HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)

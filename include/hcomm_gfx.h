@@ -14,7 +14,7 @@
  *                                over N simulated ranks (N pairs of HBM buffers), with HcommGfxSchedule* to obtain
  *                                the operation lists and check them symbolically without a GPU;
  *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
- *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*: what the reference's executors do
+ *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*: what the reference's executors do
  *                                around the templates (chunk loops through the CCL buffers, two communicator
  *                                levels, user memory read and written directly), each as PlanCreate / Emit / Check.
  */
@@ -715,6 +715,29 @@ int32_t HcommGfxOrderPreservedEmit(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
     uint64_t* n);
 int32_t HcommGfxOrderPreservedCheck(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
+ * The allreduce of the reference's order-preserving executor on one server in op-base mode
+ * (coll_executor/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:131-193, 248-283, 342-380): per chunk of
+ * at most cclBytes / unit elements, cut into N blocks of ceil(chunk / N) elements rounded up to 128 bytes (trailing
+ * blocks short or empty), every rank plants block p of its user input into rank p's CCL buffers - N - 1 slots of
+ * the CCL output buffer plus, on every rank but the last, one slot borrowed from the CCL input buffer
+ * (alg_template/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc:168-188, 221-247) - rank p folds them in
+ * RANK order along the fixed tree of the order-preserving reduce-scatter, the blocks are gathered over the mesh
+ * inside the CCL output buffers (alg_template/temp_all_gather/all_gather_mesh_atomic.cc:19-69) and the chunk is copied
+ * to the user output.  The result is bit-identical on every rank and does not depend on N's factorisation.
+ * userIn, userOut: count elements; cclIn, cclOut: cclBytes; 128-byte aligned.  nRanks >= 2; the inter-module stages
+ * (:208-246, :285-340) are not built.  HCCL_E_PARA when the N - 1 rounded-up slots of a chunk reach past cclBytes
+ * (CCL buffers below about N * N * 128 bytes; the reference's DeviceMem::range refuses them too).  Step-wise lowering.
+ */
+int32_t HcommGfxOrderPreservedAllReducePlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclIn, void* const* cclOut,
+    uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxOrderPreservedAllReduceEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n);
+int32_t HcommGfxOrderPreservedAllReduceCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*

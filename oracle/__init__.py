@@ -111,6 +111,10 @@ def lib():
         L.orc_run_order_preserved.restype = C.c_int
         L.orc_run_order_preserved.argtypes = [C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + \
             [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
+        L.orc_trace_order_preserved_ar.restype = C.c_int64
+        L.orc_trace_order_preserved_ar.argtypes = L.orc_trace_order_preserved.argtypes
+        L.orc_run_order_preserved_ar.restype = C.c_int
+        L.orc_run_order_preserved_ar.argtypes = L.orc_run_order_preserved.argtypes
         L.orc_trace_hier_rs.restype = C.c_int64
         L.orc_trace_hier_rs.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int,
                                         C.POINTER(OrcOp), C.c_uint64]
@@ -353,6 +357,24 @@ def run_order_preserved(user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dt
     rc = lib().orc_run_order_preserved(n, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
     if rc:
         raise ValueError("orc_run_order_preserved rc=%d" % rc)
+
+
+def trace_order_preserved_ar(n, count, ccl_bytes, dtype):
+    """The order-preserving ALLREDUCE executor on one server: plant with borrowed space, mesh all-gather, copy out."""
+    total = lib().orc_trace_order_preserved_ar(n, count, ccl_bytes, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_order_preserved_ar rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_order_preserved_ar(n, count, ccl_bytes, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_order_preserved_ar(user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype, op):
+    n = len(user_in)
+    arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in b]) for b in (user_in, user_out, ccl_in, ccl_out)]
+    rc = lib().orc_run_order_preserved_ar(n, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
+    if rc:
+        raise ValueError("orc_run_order_preserved_ar rc=%d" % rc)
 
 
 # ---- the ring / mesh reduce-scatter executors over two communicator levels, op-base mode -----------------

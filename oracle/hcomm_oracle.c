@@ -2,8 +2,8 @@
  * hcomm_oracle.c - CPU restatement of HCOMM's local copy / reduce semantics, of the ring, recursive
  * halving-doubling, mesh, NHR (sliced and one-shot), NB, local-reduce, chunk-mesh and doubling schedules, of the
  * executors' op-base loop around them, of the ring and mesh executors' three-step allreduce and two-level
- * reduce-scatter, of the double-ring executor with DMA reduce and of the order-preserving reduce-scatter executor, used
- * ONLY to check libhcomm_gfx.so.
+ * reduce-scatter, of the double-ring executor with DMA reduce and of the order-preserving reduce-scatter and allreduce
+ * executors, used ONLY to check libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -60,6 +60,10 @@
  *                                     chunk / share table by hand; exact integer results over several chunks; pinned
  *   order-preserving reduce-scatter . the complete operation list N = 3, the rank-order fold trees N = 2..8 and a
  *                                     chunk table by hand; exact integer results over several chunks; pinned
+ *   order-preserving allreduce ...... the complete operation list N = 3 (blocks of 256, 144 and 0 bytes, both borrowed
+ *                                     slots), a chunk / block table N = 4 by hand; the same rank-order fold trees for
+ *                                     every element N = 2..8; slot and borrowed-slot layout from the definition;
+ *                                     exact integer results over several chunks; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
@@ -2251,6 +2255,149 @@ int orc_run_order_preserved(uint32_t n, void* const* user_in, void* const* user_
 {
     OrcTrace t;
     int rc = build_trace_order_preserved(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+/* ---- the order-preserving allreduce executor (one server, op-base mode) ------------------------------------------ */
+
+/* ReduceScatterPlantLocalReduce::RunAsync for one rank and a single (= last) group whose blocks differ in size and
+ * that borrows space, tpl/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc:105-166 as
+ * CollAllReduceOrderPreservedExecutor::RunReduceScatterLevel0 prepares it for one module
+ * (exec/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:149-193: block d is size[d] bytes at d * stride of the
+ * user input, of the input memory and of the output memory alike; all2allOffset 0; isNeedSpaceBorrow true).
+ * A contribution whose slot is the last one goes to the receiving rank's INPUT memory at that rank's own block
+ * offset instead, on every receiving rank but the last one (:168-188, :190-254, :337-414). */
+static void prog_plant_local_reduce_borrow(OrcTrace* t, uint32_t local_rank, uint32_t rank_size, const uint64_t* size,
+                                           uint64_t stride)
+{
+#define CALC_OUTPUT_INDEX(round) (((round) + local_rank) % rank_size)            /* :94-97, all2allOffset 0 */
+#define IS_LAST_BLOCK(index) ((index) == rank_size - 1)                          /* :103 */
+#define IS_LAST_RANK(r) ((r) == rank_size - 1)                                   /* :101; the one group is the last, :99 */
+    /* LocalCopy, :168-188 */
+    {
+        const uint32_t output_index = CALC_OUTPUT_INDEX(local_rank);
+        if (IS_LAST_BLOCK(output_index) && !IS_LAST_RANK(local_rank))
+            emit(t, 0, K_COPY, local_rank, B_IN, stride * local_rank, local_rank, B_UIN, stride * local_rank, size[local_rank]);
+        else
+            emit(t, 0, K_COPY, local_rank, B_OUT, stride * output_index, local_rank, B_UIN, stride * local_rank,
+                 size[local_rank]);
+    }
+    /* RunAlltoAll, :221-247 */
+    for (uint32_t round = 0; round < rank_size; round++) {
+        if (round == local_rank) continue;
+        const uint32_t output_index = CALC_OUTPUT_INDEX(round);
+        if (IS_LAST_BLOCK(output_index) && !IS_LAST_RANK(round))
+            emit(t, 0, K_COPY, round, B_IN, stride * round, local_rank, B_UIN, stride * round, size[round]);
+        else
+            emit(t, 0, K_COPY, round, B_OUT, stride * output_index, local_rank, B_UIN, stride * round, size[round]);
+    }
+    /* RunLocalReduce, :337-414 */
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < rank_size) reduce_step++;
+    const uint64_t src_offset = stride * local_rank; /* inputOffsets[localRank_], :340 */
+    for (uint32_t round = 0; round < reduce_step; round++) {
+        const uint32_t full = 1u << (reduce_step - round);
+        const uint32_t tail_index = (rank_size < full ? rank_size : full) - 1;
+        const uint32_t head_index = 1u << (reduce_step - round - 1);
+        for (uint32_t offset = 0; offset <= tail_index - head_index; offset++) {
+            const uint32_t input_index = CALC_OUTPUT_INDEX(head_index + offset);
+            const uint32_t output_index = CALC_OUTPUT_INDEX(offset);
+            const int src_borrowed = !IS_LAST_RANK(local_rank) && IS_LAST_BLOCK(input_index);  /* :376-381 */
+            const int dst_borrowed = !IS_LAST_RANK(local_rank) && IS_LAST_BLOCK(output_index); /* :383-388 */
+            emit(t, 1 + round, K_REDUCE, local_rank, dst_borrowed ? B_IN : B_OUT,
+                 dst_borrowed ? src_offset : stride * output_index, local_rank, src_borrowed ? B_IN : B_OUT,
+                 src_borrowed ? src_offset : stride * input_index, size[local_rank]);
+        }
+    }
+#undef CALC_OUTPUT_INDEX
+#undef IS_LAST_BLOCK
+#undef IS_LAST_RANK
+}
+
+/* CollAllReduceOrderPreservedExecutor::KernelRun for every rank inside CollAllReduceExecutor::RunLoop
+ * (exec/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:342-380 with DMAReduceFlag_, :19;
+ * exec/coll_all_reduce/coll_all_reduce_executor.cc:129-138, 212-252): one module. */
+static int build_trace_order_preserved_ar(OrcTrace* t, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    /* one rank per module takes RunReduceScatterLevel0SingleRank (:195-206): not restated */
+    if (unit == 0 || n < 2 || n > ORC_MAX_RANKS) return -1;
+    const uint64_t max_count = ccl_bytes / unit; /* CalcLoopMaxCount, coll_all_reduce_executor.cc:129-138 */
+    if (max_count == 0) return -1;
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < n) reduce_step++;
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        const uint64_t cur_size = cur_count * unit;
+        /* CalcSizePerBlock, :131-136 */
+        uint64_t size_per_block = (cur_count + n - 1) / n * unit;
+        size_per_block = (size_per_block + 127u) / 128u * 128u;
+        /* CalGroupSlices, :138-147 */
+        uint64_t group_size[ORC_MAX_RANKS];
+        uint64_t size_remain = cur_size;
+        for (uint32_t r = 0; r < n; r++) {
+            group_size[r] = size_remain > size_per_block ? size_per_block : size_remain;
+            size_remain -= group_size[r];
+        }
+        /* RunAllGatherLevel0, :256-263 */
+        OrcSlice seg[ORC_MAX_RANKS];
+        for (uint32_t r = 0; r < n; r++) {
+            seg[r].size = group_size[r];
+            seg[r].offset = group_size[r] == 0 ? 0 : r * size_per_block;
+        }
+        g_user_off = user_off;
+        for (uint32_t r = 0; r < n; r++) {
+            g_step_base = step0;
+            prog_plant_local_reduce_borrow(t, r, n, group_size, size_per_block); /* :356 */
+            g_step_base = step0 + 1 + reduce_step;
+            prog_mesh_ag(t, r, n, seg);                                          /* :363, AllGatherMeshAtomic: all_gather_mesh_atomic.cc:19-69, the data movement of AllGatherMesh */
+            g_step_base = step0 + 2 + reduce_step;
+            emit(t, 0, K_COPY, r, B_UOUT, 0, r, B_OUT, 0, cur_size);             /* :369-376 */
+        }
+        g_user_off = 0;
+        g_step_base = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += 3 + reduce_step;
+        user_off += cur_size;
+    }
+    /* DeviceMem::range refuses a range past the end of the CCL buffer (the rounded-up blocks of a tiny buffer) */
+    for (uint64_t i = 0; i < t->n; i++) {
+        const OrcOp* o = &t->ops[i];
+        if ((o->dst_buf <= B_OUT && o->dst_off + o->bytes > ccl_bytes) || (o->src_buf <= B_OUT && o->src_off + o->bytes > ccl_bytes)) {
+            free(t->ops);
+            return -1;
+        }
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_order_preserved_ar(uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_ar(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_order_preserved_ar(uint32_t n, void* const* user_in, void* const* user_out, void* const* ccl_in,
+                               void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_ar(&t, n, count, ccl_bytes, dtype);
     if (rc) return rc;
     void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
     rc = exec_trace(&t, bufs, dtype, op);
