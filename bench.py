@@ -153,6 +153,7 @@ def main():
     # one-server executors on user memory (DMA reduce)
     plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar")
     opar = alg_name == "order_preserved_ar"
+    opfused = alg_name in ("order_preserved_ar", "order_preserved_rs")  # these two also have a single-launch lowering
     dbrs = alg_name == "doublering_rs"
     dt, alg, op = DT[dtname], (None if plant else ALG[alg_name]), OP[opname]
     unit = h.DTYPE_SIZE[dt]
@@ -187,9 +188,9 @@ def main():
     d_ccl = None
     if opbase or dbring or plant or hier_rs:
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
-        if args.lowering == "both":
+        if args.lowering == "both" and not opfused:
             args.lowering = "stepwise"
-    if hier or plant:
+    if hier or (plant and not opfused):
         args.lowering = "stepwise"  # composed from the step lists of its levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
@@ -204,6 +205,8 @@ def main():
                                            [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, mesh=mesh0)
         if dbrs:
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
+        if opfused and low == h.Lowering.FUSED:  # one launch on the user buffers, no CCL buffer
+            return h.OrderPreservedFusedPlan(opar, in_ptrs, out_ptrs, count, dt, op)
         if opar:
             return h.OrderPreservedAllReducePlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                                  [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
@@ -411,7 +414,7 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
-                if opbase or dbring or plant or hier_rs:  # what the last chunk left in the CCL buffers
+                if (opbase or dbring or plant or hier_rs) and not (opfused and name == "fused"):  # what the last chunk left in the CCL buffers
                     ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)

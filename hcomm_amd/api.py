@@ -29,7 +29,7 @@ __all__ = [
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
-    "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check",
+    "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check", "OrderPreservedFusedPlan",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
@@ -565,6 +565,25 @@ class OrderPreservedAllReducePlan(Plan):
         p = _vp(0)
         check(_opar_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3], ccl_bytes, count, dtype, op,
                          C.byref(p)), "HcommGfxOrderPreservedAllReducePlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_opf_plan = _sig("HcommGfxOrderPreservedFusedPlanCreate", _i32, _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
+                 C.c_int, C.POINTER(_vp))
+
+
+class OrderPreservedFusedPlan(Plan):
+    """HcommGfxOrderPreservedFusedPlanCreate: either order-preserving executor as one launch on the user buffers."""
+
+    def __init__(self, all_reduce, user_in, user_out, count, dtype, op):
+        n = len(user_in)
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out)]
+        p = _vp(0)
+        check(_opf_plan(int(all_reduce), n, self._bufs[0], self._bufs[1], count, dtype, op, C.byref(p)),
+              "HcommGfxOrderPreservedFusedPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

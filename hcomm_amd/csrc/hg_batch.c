@@ -97,9 +97,9 @@ void hg_finish_fold(HgLaunch* l)
          * nout outputs */
         uint64_t moved = 0;
         if (t->tree != 1u) {
-            /* truncated rotation trees: nranks leaf reads, one store per even position that has a right neighbour,
-             * and the root to one output or to all of them */
-            const uint64_t n = (uint64_t)t->nranks + t->nranks / 2 + (t->out_mode == 1u ? 1u : t->nout);
+            /* truncated rotation trees: nranks leaf reads, one store per even position that has a right neighbour
+             * (none for the rank-order tree, which only reads its inputs), and the root to one output or to all */
+            const uint64_t n = (uint64_t)t->nranks + (t->tree == 4u ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
             l->moved_bytes = n * bytes;
             l->blocks = hg_grid_blocks(tiles, 0);
             return;

@@ -79,6 +79,9 @@ __device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t
 // q a multiple of 2^(l+1)) with q + 2^l wherever that position exists - the fold rank (c +- q) performs at step l
 // from rank (c +- q) +- 2^l.  An even position that had a right neighbour keeps the last value it computed; the
 // root goes to every output (allreduce) or to the owner's output (reduce-scatter).
+// tree == 4 is the rank-order tree of the order-preserving executors: position q holds rank bitrev(q) where that
+// rank exists, so level l folds rank j + K / 2^(l+1) onto rank j - the contributions K/2 .. onto 0 .., then
+// K/4 .. onto 0 .., down to 1 onto 0; the inputs are only read.
 template <class Item, int L, uint32_t NU>
 __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
                                                     const uint64_t (&idx)[NU])
@@ -89,13 +92,21 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
     const uint32_t c = tab.first[s];
     const uint32_t n = tab.nranks;
     const bool plus = tab.tree == 2u;
+    const bool order = tab.tree == 4u;
     V x[K][NU];
     uint32_t b[K];
+    bool have[K];
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
-        b[q] = plus ? c + q : c + n - q;
-        if (b[q] >= n) b[q] -= n;
-        if (q < n) {
+        if (order) {
+            b[q] = bitrev<L>(q);
+            have[q] = b[q] < n;
+        } else {
+            b[q] = plus ? c + q : c + n - q;
+            if (b[q] >= n) b[q] -= n;
+            have[q] = q < n;
+        }
+        if (have[q]) {
             const uint8_t* p = (const uint8_t*)tab.in[b[q]] + off;
 #pragma unroll
             for (uint32_t u = 0; u < NU; ++u) x[q][u] = live[u] ? Item::ld(p, idx[u]) : Item::zero();
@@ -105,14 +116,14 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
     for (int l = 0; l < L; ++l) {
 #pragma unroll
         for (uint32_t q = 0; q < K; q += (2u << l))
-            if (q + (1u << l) < n) {
+            if (have[q + (1u << l)]) {
 #pragma unroll
                 for (uint32_t u = 0; u < NU; ++u) x[q][u] = Item::op(x[q][u], x[q + (1u << l)][u]);
             }
     }
 #pragma unroll
     for (uint32_t q = 0; q < K; q += 2)
-        if (q + 1 < n) {
+        if (!order && q + 1 < n) {
             uint8_t* p = (uint8_t*)tab.in[b[q]] + off;
 #pragma unroll
             for (uint32_t u = 0; u < NU; ++u)

@@ -691,6 +691,83 @@ int32_t HcommGfxOrderPreservedAllReducePlanCreate(
     return rc;
 }
 
+/* Both order-preserving executors in one launch: the N user inputs are folded in registers along the executors'
+ * rank-order tree (reduce_scatter_plant_local_reduce.cc:337-414: rounds h = 2^(S-1), .., 1 fold contribution h + j
+ * onto contribution j) and the root is written to the user output(s).  No CCL buffer is read or written. */
+int32_t HcommGfxOrderPreservedFusedPlanCreate(
+    int32_t allReduce, uint32_t nRanks, void* const* userIn, void* const* userOut, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (nRanks < 2 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(userIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint64_t block = count * HcommGfxDataTypeSize(dataType);
+    /* the reduce-scatter reads block p of every input at p * block: 128-bit accesses need 16-byte multiples */
+    if (!allReduce && (block & (HG_VEC_BYTES - 1u))) return HCCL_E_NOT_SUPPORT;
+    /* steps and algorithmic bytes are those of the step-wise plan with an unbounded CCL buffer (a single chunk) */
+    HgOpList ol;
+    rc = allReduce ? hg_schedule_order_preserved_ar(&ol, nRanks, count, (uint64_t)1 << 62, (int)dataType)
+                   : hg_schedule_order_preserved(&ol, nRanks, count, (uint64_t)1 << 62, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
+    if (!p) {
+        hg_oplist_free(&ol);
+        return HCCL_E_MEMORY;
+    }
+    p->magic = HG_PLAN_MAGIC;
+    p->graph_wanted = use_graph();
+    p->info.steps = ol.steps;
+    for (uint64_t i = 0; i < ol.n; ++i) p->info.algorithmicBytes += ol.ops[i].bytes * (ol.ops[i].kind ? 3u : 2u);
+    hg_oplist_free(&ol);
+    if (block) {
+        HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+        if (!l) {
+            HcommGfxPlanDestroy(p);
+            return HCCL_E_MEMORY;
+        }
+        l->kind = HCOMM_GFX_KERNEL_TREE;
+        l->dtype = (uint32_t)dataType;
+        l->op = (uint32_t)reduceOp;
+        HgFoldTable* f = &l->tab.fold;
+        f->tree = 4u;
+        f->k = 2;
+        while (f->k < nRanks) f->k <<= 1;
+        f->nranks = nRanks;
+        for (uint32_t r = 0; r < nRanks; ++r) {
+            f->in[r] = userIn[r];
+            f->out[r] = userOut[r];
+        }
+        if (allReduce) {
+            f->nout = nRanks;
+            f->out_mode = 2u;
+            f->nseg = 1;
+            f->bytes[0] = block;
+        } else {
+            f->out_mode = 1u;
+            f->nseg = nRanks;
+            for (uint32_t r = 0; r < nRanks; ++r) {
+                f->off[r] = block * r;
+                f->bytes[r] = block;
+                f->owner[r] = (uint8_t)r;
+            }
+        }
+        hg_finish_fold(l);
+        rc = plan_push(l, p);
+        free(l);
+        if (rc != HCCL_SUCCESS) {
+            HcommGfxPlanDestroy(p);
+            return rc;
+        }
+    }
+    p->info.launches = p->nlaunch;
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
 int32_t HcommGfxHierReduceScatterPlanCreate(
     int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn,
     void* const* userOut, void* const* cclIn, void* const* cclOut, uint64_t cclBytes, uint64_t count,

@@ -14,7 +14,8 @@
  *                                over N simulated ranks (N pairs of HBM buffers), with HcommGfxSchedule* to obtain
  *                                the operation lists and check them symbolically without a GPU;
  *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
- *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*: what the reference's executors do
+ *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*,
+ *                                HcommGfxOrderPreservedFused*: what the reference's executors do
  *                                around the templates (chunk loops through the CCL buffers, two communicator
  *                                levels, user memory read and written directly), each as PlanCreate / Emit / Check.
  */
@@ -739,6 +740,22 @@ int32_t HcommGfxOrderPreservedAllReduceEmit(
     uint64_t* n);
 int32_t HcommGfxOrderPreservedAllReduceCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
+ * The single-launch lowering of the two order-preserving executors (no counterpart in the reference, which has no
+ * device that can read N ranks' memory in one kernel): every element of the result is folded in registers from the
+ * N user inputs along the executors' fixed tree over rank order (reduce_scatter_plant_local_reduce.cc:337-414:
+ * contribution h + j onto contribution j for h = 2^(S-1), .., 1) and written straight to the user output(s).
+ * allReduce == 0: userIn holds nRanks * count elements per rank and rank p's userOut receives block p (the result of
+ * HcommGfxOrderPreservedPlanCreate); allReduce != 0: count elements in and out on every rank (the result of
+ * HcommGfxOrderPreservedAllReducePlanCreate).  The user outputs are bit-identical to those plans' for every data
+ * type and reduce operation; the user inputs are only read; the CCL buffers are not needed and not touched, so there
+ * is no chunk loop.  HCCL_E_NOT_SUPPORT for a reduce-scatter whose block (count * unit bytes) is not a multiple of
+ * 16 bytes: use the step-wise plan.  Buffers 128-byte aligned, nRanks >= 2.
+ */
+int32_t HcommGfxOrderPreservedFusedPlanCreate(
+    int32_t allReduce, uint32_t nRanks, void* const* userIn, void* const* userOut, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
 /*
  * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand

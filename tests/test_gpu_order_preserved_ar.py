@@ -82,3 +82,76 @@ def test_randomized_shapes(gpu_thread):
         ccl = int(rng.integers(64, 2048)) * 512           # at least 32 KiB: the N - 1 rounded-up slots always fit
         say("random order preserved allreduce", i, n, count, dtype, op, ccl)
         run_case(gpu_thread, n, count, dtype, op, ccl, seed=i)
+
+
+# ---- the single-launch lowering: the same user outputs from one kernel that only reads the user inputs ---------------
+
+def run_fused(thread, all_reduce, n, count, dtype, op, seed=0):
+    dt, o = DT[dtype], OPS[op]
+    in_count = count if all_reduce else n * count
+    host_in = [gen(dt, in_count, 13000 + seed * 100 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    sentinel = gen(dt, count, 997, "wide")
+    unit = h.DTYPE_SIZE[dt]
+    ccl = max(4096, -(-count * unit * n // 128) * 128)            # one chunk or several: the result does not depend on it
+    w_in = [x.copy() for x in host_in]
+    w_out = [sentinel.copy() for _ in range(n)]
+    w_ccl = [[np.zeros(ccl, np.uint8) for _ in range(n)] for _ in range(2)]
+    if all_reduce:
+        oracle.run_order_preserved_ar(w_in, w_out, w_ccl[0], w_ccl[1], count, ccl, dt, o)
+    else:
+        oracle.run_order_preserved(w_in, w_out, w_ccl[0], w_ccl[1], count, ccl, dt, o)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    pad = to_dev(np.zeros(256, np.uint8))
+    ptrs = lambda ts: [t.data_ptr() if t.numel() else pad.data_ptr() for t in ts]
+    plan = h.OrderPreservedFusedPlan(all_reduce, ptrs(d_in), ptrs(d_out), count, dt, o)
+    try:
+        assert plan.info.launches == (1 if count else 0)
+        assert plan.run(thread) == 0
+        assert h.HcommGfxThreadSynchronize(thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_out[r], sentinel), w_out[r], dt, "user out[%d]" % r)
+            assert np.array_equal(from_dev(d_in[r], host_in[r]).view(np.uint8), host_in[r].view(np.uint8)), "user in[%d] was written" % r
+    finally:
+        plan.destroy()
+
+
+FUSED_CASES = [
+    (1, 8, 1 << 21, "bf16", "sum"),
+    (1, 8, 300007, "fp32", "sum"),
+    (1, 7, 100003, "fp16", "sum"),
+    (1, 5, 70001, "int8", "max"),
+    (1, 3, 100, "fp32", "prod"),
+    (1, 2, 100003, "fp32", "min"),
+    (1, 16, 4099, "int16", "sum"),
+    (1, 32, 50000, "int32", "sum"),
+    (1, 13, 77777, "bf16", "sum"),
+    (1, 6, 0, "fp32", "sum"),
+    (0, 8, 1 << 18, "bf16", "sum"),
+    (0, 7, 100000, "fp16", "sum"),
+    (0, 5, 70000, "fp32", "prod"),
+    (0, 3, 16, "int8", "max"),
+    (0, 32, 5000, "int32", "sum"),
+    (0, 12, 4104, "int16", "min"),
+]
+
+
+@pytest.mark.parametrize("all_reduce,n,count,dtype,op", FUSED_CASES)
+def test_single_launch_lowering_matches_the_executors_outputs(gpu_thread, all_reduce, n, count, dtype, op):
+    say("order preserved fused", all_reduce, n, count, dtype, op)
+    run_fused(gpu_thread, all_reduce, n, count, dtype, op)
+
+
+def test_single_launch_lowering_randomized(gpu_thread):
+    rng = np.random.default_rng(6363)
+    for i in range(40):
+        all_reduce = int(rng.integers(2))
+        n = int(rng.integers(2, 33))
+        dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
+        unit = h.DTYPE_SIZE[DT[dtype]]
+        count = int(rng.integers(1, 200000))
+        if not all_reduce:
+            count = max(16 // unit, count // 4 // (16 // unit) * (16 // unit))   # blocks of whole 16 bytes
+        op = ["sum", "max", "min"][rng.integers(3)]
+        say("random order preserved fused", i, all_reduce, n, count, dtype, op)
+        run_fused(gpu_thread, all_reduce, n, count, dtype, op, seed=i)

@@ -148,3 +148,52 @@ def test_rejects_bad_arguments():
             f(8, 16, 16, oracle.I8)                      # the 128-byte slots of a 16-byte chunk reach past 16 bytes
         with pytest.raises((ValueError, h.HcommError)):
             f(33, 100, 1 << 20, oracle.F32)
+
+
+# ---- the single-launch lowering of both order-preserving executors --------------------------------------------------
+
+def kernel_tree(n):
+    """The tree the fold kernel's rank-order mode builds: position q of K = 2^L holds rank bitrev(q) if it exists;
+    level l folds position q + 2^l into position q (q a multiple of 2^(l+1)) wherever the former exists."""
+    L = max(1, (n - 1).bit_length())
+    K = 1 << L
+    rev = lambda q: int(format(q, "0%db" % L)[::-1], 2)
+    x = [rev(q) if rev(q) < n else None for q in range(K)]
+    for l in range(L):
+        for q in range(0, K, 2 << l):
+            if x[q + (1 << l)] is not None:
+                x[q] = [x[q], x[q + (1 << l)]]
+    return x[0]
+
+
+def test_fused_kernel_tree_is_the_executors_rank_order_tree():
+    for n_s, tree in TREES.items():
+        assert kernel_tree(int(n_s)) == tree, n_s
+
+
+def test_fused_plan_is_one_tree_launch_on_the_user_buffers():
+    base = 0x7f0000000000
+    for n in (2, 3, 5, 8, 17, 32):
+        uin = [base + r * (1 << 32) for r in range(n)]
+        uout = [base + (64 + r) * (1 << 32) for r in range(n)]
+        for all_reduce, count, dt in ((1, 100003, oracle.F32), (1, 7, oracle.I8), (0, 4096, oracle.BF16), (0, 12, oracle.F32)):
+            unit = h.DTYPE_SIZE[dt]
+            p = h.OrderPreservedFusedPlan(all_reduce, uin, uout, count, dt, oracle.SUM)
+            try:
+                launches = p.launches()
+                assert [l.kind for l in launches] == [h.Kernel.TREE]
+                assert launches[0].nseg == (1 if all_reduce else n)
+                assert launches[0].bytes == count * unit * (1 if all_reduce else n)
+                ops = (oracle.trace_order_preserved_ar if all_reduce else oracle.trace_order_preserved)(n, count, 1 << 40, dt)
+                assert p.info.algorithmicBytes == sum(o[8] * (3 if o[1] else 2) for o in ops)
+                # what the launch itself moves: N reads per element and N (allreduce) or 1 (reduce-scatter) writes
+                assert p.info.movedBytes == launches[0].bytes * (2 * n if all_reduce else n + 1)
+            finally:
+                p.destroy()
+        with pytest.raises(h.HcommError):
+            h.OrderPreservedFusedPlan(0, uin, uout, 3, oracle.F32, oracle.SUM)      # 12-byte blocks: not 16-byte multiples
+        p = h.OrderPreservedFusedPlan(1, uin, uout, 0, oracle.F32, oracle.SUM)
+        assert p.launches() == []
+        p.destroy()
+    with pytest.raises(h.HcommError):
+        h.OrderPreservedFusedPlan(1, [base], [base + 4096], 16, oracle.F32, oracle.SUM)
