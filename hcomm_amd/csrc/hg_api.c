@@ -73,8 +73,9 @@ int hg_reduce_supported(int dtype, int op, int prod_ok)
 {
     if (!hg_dtype_supported(dtype)) return 0;
     if (op == HCOMM_REDUCE_SUM || op == HCOMM_REDUCE_MAX || op == HCOMM_REDUCE_MIN) return 1;
-    /* PROD: collective-level matrix of the reference excludes int16 (param_check.cc:327-343) */
-    if (op == HCOMM_REDUCE_PROD && prod_ok) return dtype != HCOMM_DATA_TYPE_INT16;
+    /* PROD: the collective-level matrix of the reference for 910B / 910_93 excludes int16 and bf16
+     * (HcomCheckReduceDataType, framework/common/src/param_check.cc:327-343) */
+    if (op == HCOMM_REDUCE_PROD && prod_ok) return dtype != HCOMM_DATA_TYPE_INT16 && dtype != HCOMM_DATA_TYPE_BFP16;
     return 0;
 }
 

@@ -295,7 +295,8 @@ int32_t HcommGfxThreadSynchronize(ThreadHandle thread);
  * (the chain of src/legacy/ascend910/algorithm/base/alg_template/temp_all_reduce/all_reduce_mesh_oneshot.cc:94-119)
  * in a single pass that reads each input once.  1 <= k <= HCOMM_GFX_MAX_RANKS.  dst may alias srcs[0].
  * PROD is allowed for the types the reference allows at collective level
- * (src/legacy/ascend910/framework/common/src/param_check.cc:327-343): INT8, INT32, FP16, FP32; and BFP16.
+ * (HcomCheckReduceDataType for 910B / 910_93, src/legacy/ascend910/framework/common/src/param_check.cc:327-343):
+ * INT8, INT32, FP16, FP32 - not INT16, not BFP16.
  */
 int32_t HcommGfxReduceKOnThread(
     ThreadHandle thread, void* dst, const void* const* srcs, uint32_t k, uint64_t count, HcommDataType dataType,
@@ -442,7 +443,7 @@ typedef struct HcommGfxPlan HcommGfxPlan;
  *                   each other or any other rank's buffers).  Algorithms that run in place ignore out.
  *   count         : elements per rank (see the algorithm's note for its exact meaning).
  * Dtypes: INT8, INT16, INT32, FP16, FP32, BFP16.  Ops: SUM, MAX, MIN, and PROD where the reference allows it
- * at collective level (param_check.cc:327-343: not INT16) plus BFP16.
+ * at collective level (param_check.cc:327-343: not INT16, not BFP16).
  * Returns HCCL_SUCCESS and *plan, or an error code and *plan = NULL.  nRanks in [1, HCOMM_GFX_MAX_RANKS].
  * Building a plan allocates nothing on the device and launches nothing.
  */

@@ -371,7 +371,7 @@ def test_randomized_shapes(gpu_thread):
         count = int(base * rng.integers(1, 4) + rng.integers(0, 3))
         dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
         op = ["sum", "max", "min", "prod"][rng.integers(4)]
-        if op == "prod" and dtype == "int16":
+        if op == "prod" and dtype in ("int16", "bf16"):        # the reference refuses these two (param_check.cc:327-343)
             continue
         lowering = h.Lowering.FUSED if (name in FUSABLE and rng.integers(2)) else h.Lowering.STEPWISE
         say("random", done, name, n, count, dtype, op, lowering)

@@ -319,6 +319,8 @@ def test_reduce_k_checks(rec):
     assert f(rec, DST, [SRC, SRC + 4096], 100, DT.FP16, OP.SUM) == R.SUCCESS
     assert f(rec, DST, [SRC], 100, DT.FP32, OP.PROD) == R.SUCCESS            # PROD allowed here
     assert f(rec, DST, [SRC], 100, DT.INT16, OP.PROD) == R.E_PARA            # not for int16 (param_check.cc:327-343)
+    assert f(rec, DST, [SRC], 100, DT.BFP16, OP.PROD) == R.E_PARA            # nor for bf16
+    assert f(rec, DST, [SRC], 100, DT.FP16, OP.PROD) == R.SUCCESS
     assert f(rec, None, [SRC], 100, DT.FP16, OP.SUM) == R.E_PTR
     assert f(rec, DST, [SRC, 0], 100, DT.FP16, OP.SUM) == R.E_PTR
     assert f(rec, DST, [], 100, DT.FP16, OP.SUM) == R.E_PARA
@@ -351,7 +353,10 @@ def test_plan_argument_checks():
         with pytest.raises(h.HcommError) as e:
             mk(**kwargs)
         assert e.value.code == code, kwargs
-    mk(dt=DT.BFP16, op=OP.PROD).destroy()
+    with pytest.raises(h.HcommError) as e:                      # the reference refuses bf16 PROD as well as int16
+        mk(dt=DT.BFP16, op=OP.PROD)
+    assert e.value.code == R.E_PARA
+    mk(dt=DT.FP16, op=OP.PROD).destroy()
     p = mk(alg=h.Alg.ALLREDUCE_RHD, low=h.Lowering.FUSED)
     assert [r.kind for r in p.launches()] == [h.Kernel.TREE]
     p.destroy()
