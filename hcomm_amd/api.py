@@ -30,6 +30,7 @@ __all__ = [
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
     "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check", "OrderPreservedFusedPlan",
+    "OrderPreservedHierAllReducePlan", "order_preserved_hier_ar_emit", "order_preserved_hier_ar_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
@@ -565,6 +566,47 @@ class OrderPreservedAllReducePlan(Plan):
         p = _vp(0)
         check(_opar_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3], ccl_bytes, count, dtype, op,
                          C.byref(p)), "HcommGfxOrderPreservedAllReducePlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_oph_emit = _sig("HcommGfxOrderPreservedHierAllReduceEmit", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+                 C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_oph_check = _sig("HcommGfxOrderPreservedHierAllReduceCheck", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+                  C.POINTER(CheckReport))
+_oph_plan = _sig("HcommGfxOrderPreservedHierAllReducePlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                 C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def order_preserved_hier_ar_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_oph_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
+          "HcommGfxOrderPreservedHierAllReduceEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_oph_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
+          "HcommGfxOrderPreservedHierAllReduceEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def order_preserved_hier_ar_check(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_oph_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
+          "HcommGfxOrderPreservedHierAllReduceCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class OrderPreservedHierAllReducePlan(Plan):
+    """HcommGfxOrderPreservedHierAllReducePlanCreate: the order-preserving allreduce executor over two levels."""
+
+    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_out, ccl_bytes, count, dtype, op):
+        n = n_servers * n_local
+        assert len(user_in) == n
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in, ccl_out)]
+        p = _vp(0)
+        check(_oph_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3], ccl_bytes,
+                        count, dtype, op, C.byref(p)), "HcommGfxOrderPreservedHierAllReducePlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -1483,6 +1483,182 @@ static int order_preserved_ar_build(HgOpList* l, uint32_t n, uint64_t count, uin
     return HCCL_SUCCESS;
 }
 
+/* The same executor over M servers of L devices (rank = server * L + local index; :149-193, 208-246, 285-340 of
+ * coll_all_reduce_order_preserved_executor.cc).  Per chunk, with B the rounded-up block size and block b at b * B:
+ *   step 0 (level 0, all2allOffset 1): inside every server, for every group g (= the blocks g * L .. g * L + L - 1
+ *           that server g will own), rank q plants block g * L + i into rank i's slot (1 + q + i) mod L of the
+ *           group's region of the CCL output buffer; slot L - 1 is borrowed from the CCL input buffer at the block's
+ *           own offset, except on the last device for the last group;
+ *   ceil(log2 L) rounds: every group's contributions folded in device order; the partial lands in slot (1 + i) mod L,
+ *           which is the borrowed place on device L - 2;
+ *   next step (level 1, ReduceScatterPlantLocalReduceCombine, SDMA branch): device i of server c plants its partial
+ *           for block i + d * L into slot (c + d) mod M of device i of server d, slot k being block i + k * L's own
+ *           place in the CCL output buffer - free because the level-0 partials sit one slot further on; the last slot
+ *           of the last device of every server but the last is borrowed again;
+ *   ceil(log2 M) rounds: the partials folded in server order; block i + d * L ends up in its own place;
+ *   mesh all-gather of the server's L blocks, then the all-gather of the M runs of L blocks between the servers
+ *           (ring: M - 1 steps; NB / NHR with the slice order kept: ceil(log2 M) steps), then the chunk to the user
+ *           output. */
+static int order_preserved_ar2_build(HgOpList* l, int alg1, uint32_t n_srv, uint32_t n_loc, uint64_t count,
+                                     uint64_t ccl_bytes, uint32_t unit)
+{
+    const uint64_t max_count = ccl_bytes / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint32_t n = n_srv * n_loc, r0 = ceil_log2(n_loc), r1 = ceil_log2(n_srv);
+    const uint32_t last_loc = n_loc - 1, last_srv = n_srv - 1;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    uint64_t size[HCOMM_GFX_MAX_RANKS];
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        const uint64_t blk = ((cur + n - 1) / n * unit + 127u) / 128u * 128u;
+        for (uint32_t b = 0; b < n; ++b) size[b] = (uint64_t)b * blk >= c ? 0 : (c - b * blk < blk ? c - b * blk : blk);
+#define SRV(s, i) ((s) * n_loc + (i))
+        /* level 0: plants */
+        for (uint32_t s = 0; s < n_srv; ++s)
+            for (uint32_t i = 0; i < n_loc; ++i)     /* destination device */
+                for (uint32_t q = 0; q < n_loc; ++q) /* planting device; per planter the groups in order */
+                    for (uint32_t g = 0; g < n_srv; ++g) {
+                        const uint32_t b = g * n_loc + i, slot = (1 + q + i) % n_loc;
+                        if (slot == last_loc && !(i == last_loc && g == last_srv))
+                            CHK(push(l, step, COPY, SRV(s, i), IN, blk * b, SRV(s, q), UIN, user_off + blk * b, size[b]));
+                        else
+                            CHK(push(l, step, COPY, SRV(s, i), OUT, blk * (g * n_loc + slot), SRV(s, q), UIN,
+                                     user_off + blk * b, size[b]));
+                    }
+        ++step;
+        /* level 0: folds in device order; contribution k of device i sits in slot (1 + k + i) mod L */
+        for (uint32_t h = 1u << (r0 - 1); h >= 1; h >>= 1, ++step)
+            for (uint32_t s = 0; s < n_srv; ++s)
+                for (uint32_t i = 0; i < n_loc; ++i)
+                    for (uint32_t g = 0; g < n_srv; ++g) {
+                        const uint32_t b = g * n_loc + i;
+                        const int may = !(i == last_loc && g == last_srv);
+                        for (uint32_t j = 0; j + h < (n_loc < 2 * h ? n_loc : 2 * h); ++j) {
+                            const uint32_t to = (1 + j + i) % n_loc, from = (1 + h + j + i) % n_loc;
+                            const int to_in = may && to == last_loc, from_in = may && from == last_loc;
+                            CHK(push(l, step, REDUCE, SRV(s, i), to_in ? IN : OUT, to_in ? blk * b : blk * (g * n_loc + to),
+                                     SRV(s, i), from_in ? IN : OUT, from_in ? blk * b : blk * (g * n_loc + from), size[b]));
+                        }
+                    }
+        /* level 1: device i of server c hands its partial for block i + d * L to server d; the own one first */
+        for (uint32_t d = 0; d < n_srv; ++d)
+            for (uint32_t i = 0; i < n_loc; ++i)
+                for (uint32_t c0 = 0; c0 < n_srv; ++c0) {
+                    const uint32_t b = i + d * n_loc, slot = (c0 + d) % n_srv;
+                    const int src_in = i + 2 == n_loc; /* the level-0 partial sits in the borrowed place */
+                    const uint64_t src_off = src_in ? blk * (i + d * n_loc) : blk * ((1 + i) % n_loc + d * n_loc);
+                    if (i == last_loc && slot == last_srv && d != last_srv)
+                        CHK(push(l, step, COPY, SRV(d, i), IN, blk * b, SRV(c0, i), src_in ? IN : OUT, src_off, size[b]));
+                    else
+                        CHK(push(l, step, COPY, SRV(d, i), OUT, blk * (i + slot * n_loc), SRV(c0, i), src_in ? IN : OUT, src_off,
+                                 size[b]));
+                }
+        ++step;
+        /* level 1: folds in server order; contribution k of server d sits in slot (k + d) mod M */
+        for (uint32_t h = 1u << (r1 - 1); h >= 1; h >>= 1, ++step)
+            for (uint32_t d = 0; d < n_srv; ++d)
+                for (uint32_t i = 0; i < n_loc; ++i) {
+                    const uint32_t b = i + d * n_loc;
+                    const int may = i == last_loc && d != last_srv;
+                    for (uint32_t j = 0; j + h < (n_srv < 2 * h ? n_srv : 2 * h); ++j) {
+                        const uint32_t to = (j + d) % n_srv, from = (h + j + d) % n_srv;
+                        const int to_in = may && to == last_srv, from_in = may && from == last_srv;
+                        CHK(push(l, step, REDUCE, SRV(d, i), to_in ? IN : OUT, to_in ? blk * b : blk * (i + to * n_loc), SRV(d, i),
+                                 from_in ? IN : OUT, from_in ? blk * b : blk * (i + from * n_loc), size[b]));
+                    }
+                }
+        /* all-gather inside the servers */
+        for (uint32_t s = 0; s < n_srv; ++s)
+            for (uint32_t i = 0; i < n_loc; ++i)
+                for (uint32_t k = 1; k < n_loc; ++k) {
+                    const uint32_t peer = (i + n_loc - k) % n_loc, b = peer + s * n_loc;
+                    CHK(push(l, step, COPY, SRV(s, i), OUT, blk * b, SRV(s, peer), OUT, blk * b, size[b]));
+                }
+        ++step;
+        /* all-gather of the servers' runs between the servers */
+        uint64_t run[HCOMM_GFX_MAX_RANKS];
+        for (uint32_t d = 0; d < n_srv; ++d) {
+            run[d] = 0;
+            for (uint32_t j = 0; j < n_loc; ++j) run[d] += size[d * n_loc + j];
+        }
+        const uint64_t run_stride = blk * n_loc;
+        if (alg1 == HCOMM_GFX_ALG_ALLREDUCE_RING) {
+            for (uint32_t k = 0; k + 1 < n_srv; ++k, ++step)
+                for (uint32_t s = 0; s < n_srv; ++s)
+                    for (uint32_t i = 0; i < n_loc; ++i) {
+                        const uint32_t d = (s + 2 * n_srv - 1 - k) % n_srv, from = (s + n_srv - 1) % n_srv;
+                        CHK(push(l, step, COPY, SRV(s, i), OUT, run_stride * d, SRV(from, i), OUT, run_stride * d, run[d]));
+                    }
+        } else if (alg1 == HCOMM_GFX_ALG_ALLREDUCE_NB) {
+            for (uint32_t k = 0; k < r1; ++k, ++step) {
+                const uint32_t cnt = (k + 1 == r1 && n_srv != (1u << r1)) ? n_srv - (1u << k) : (1u << k);
+                for (uint32_t s = 0; s < n_srv; ++s)
+                    for (uint32_t i = 0; i < n_loc; ++i)
+                        for (uint32_t j = 0; j < cnt; ++j) {
+                            const uint32_t d = modn((int64_t)s - (1 << k) - j, n_srv), from = modn((int64_t)s - (1 << k), n_srv);
+                            CHK(push(l, step, COPY, SRV(s, i), OUT, run_stride * d, SRV(from, i), OUT, run_stride * d, run[d]));
+                        }
+            }
+        } else {
+            for (uint32_t k = 0; k < r1; ++k, ++step) {
+                const uint32_t delta = 1u << (r1 - 1 - k);
+                const uint32_t cnt = (n_srv - 1 + delta) / (2 * delta);
+                for (uint32_t s = 0; s < n_srv; ++s)
+                    for (uint32_t i = 0; i < n_loc; ++i)
+                        for (uint32_t j = 0; j < cnt; ++j) {
+                            const uint32_t d = modn((int64_t)s - delta - (int64_t)j * 2 * delta, n_srv);
+                            CHK(push(l, step, COPY, SRV(s, i), OUT, run_stride * d, SRV(modn((int64_t)s - delta, n_srv), i), OUT,
+                                     run_stride * d, run[d]));
+                        }
+            }
+        }
+        for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, user_off, p, OUT, 0, c));
+        ++step;
+#undef SRV
+        user_off += c;
+        left -= cur;
+    }
+    for (uint64_t k = 0; k < l->n; ++k) { /* the reference's DeviceMem::range refuses what reaches past a CCL buffer */
+        const HcommGfxSchedOp* o = &l->ops[k];
+        if ((o->dstBuf <= OUT && o->dstOff + o->bytes > ccl_bytes) || (o->srcBuf <= OUT && o->srcOff + o->bytes > ccl_bytes))
+            return HCCL_E_PARA;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_order_preserved_ar2(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                    uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n_servers < 2 || n_local < 2 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
+        return HCCL_E_PARA;
+    int rc = order_preserved_ar2_build(l, alg1, n_servers, n_local, count, ccl_bytes, unit);
+    if (rc == HCCL_SUCCESS) rc = order_by_step_rank(l);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedHierAllReduceEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved_ar2(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule_order_preserved_ar(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
 {
     memset(l, 0, sizeof(*l));

@@ -15,9 +15,10 @@
  *                                the operation lists and check them symbolically without a GPU;
  *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
  *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*,
- *                                HcommGfxOrderPreservedFused*: what the reference's executors do
- *                                around the templates (chunk loops through the CCL buffers, two communicator
- *                                levels, user memory read and written directly), each as PlanCreate / Emit / Check.
+ *                                HcommGfxOrderPreservedHierAllReduce*, HcommGfxOrderPreservedFused*: what the
+ *                                reference's executors do around the templates (chunk loops through the CCL
+ *                                buffers, two communicator levels, user memory read and written directly), each
+ *                                as PlanCreate / Emit / Check.
  */
 #ifndef HCOMM_GFX_H
 #define HCOMM_GFX_H
@@ -741,6 +742,30 @@ int32_t HcommGfxOrderPreservedAllReduceEmit(
     uint64_t* n);
 int32_t HcommGfxOrderPreservedAllReduceCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
+ * The same executor over nServers modules of nLocal devices each (rank = server * nLocal + local index;
+ * coll_all_reduce_order_preserved_executor.cc:149-193, 208-246, 285-340): inside every server the plant template works
+ * on one group of nLocal blocks per server with an all-to-all offset of 1, so that the partial for block b lands one
+ * slot beside b's own place; between the servers ReduceScatterPlantLocalReduceCombine
+ * (alg_template/temp_reduce_scatter/reduce_scatter_plant_local_reduce_combine.cc, SDMA branch) plants the partials
+ * into the blocks' own places and folds them in SERVER order; then the mesh all-gather inside the servers, the
+ * all-gather of the servers' runs between them - level1Alg HCOMM_GFX_ALG_ALLREDUCE_RING, _NB or _NHR selects
+ * AllGatherRing, AllGatherNB or AllGatherNHR (:293-303) - and the copy to the user output.  Every element is
+ * reduced as tree(servers)( tree(devices of server 0), tree(devices of server 1), ... ) with the rank-order tree of
+ * the single-server executor at both levels.  nServers >= 2 and nLocal >= 2 (one device per module takes a branch
+ * of its own, :195-206, which is not built).  Buffers and errors as above.  Step-wise lowering.
+ */
+int32_t HcommGfxOrderPreservedHierAllReducePlanCreate(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut,
+    void* const* cclIn, void* const* cclOut, uint64_t cclBytes, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxOrderPreservedHierAllReduceEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+int32_t HcommGfxOrderPreservedHierAllReduceCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
  * The single-launch lowering of the two order-preserving executors (no counterpart in the reference, which has no

@@ -3,7 +3,7 @@
  * halving-doubling, mesh, NHR (sliced and one-shot), NB, local-reduce, chunk-mesh and doubling schedules, of the
  * executors' op-base loop around them, of the ring and mesh executors' three-step allreduce and two-level
  * reduce-scatter, of the double-ring executor with DMA reduce and of the order-preserving reduce-scatter and allreduce
- * executors, used ONLY to check libhcomm_gfx.so.
+ * executors (the latter on one server and over two levels), used ONLY to check libhcomm_gfx.so.
  *
  * THIS IS TEST INFRASTRUCTURE.  Nothing in the product library links, loads or calls it; only the test
  * suite, the smoke check and the CPU-baseline leg of the benchmark do.
@@ -64,6 +64,10 @@
  *                                     slots), a chunk / block table N = 4 by hand; the same rank-order fold trees for
  *                                     every element N = 2..8; slot and borrowed-slot layout from the definition;
  *                                     exact integer results over several chunks; pinned
+ *   two-level order-preserving allreduce . the complete operation list of 2 x 2 (every borrowed place of both levels)
+ *                                     by hand; reduction trees 2 x 2 .. 3 x 3 composed by hand from the single-level
+ *                                     trees; slot / borrowed-place layout of both levels from the definition; exact
+ *                                     integer results over several chunks, ring / NB / NHR all-gather; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
@@ -2379,6 +2383,241 @@ static int build_trace_order_preserved_ar(OrcTrace* t, uint32_t n, uint64_t coun
         }
     }
     return sort_trace(t);
+}
+
+/* ---- the order-preserving allreduce executor over two communicator levels (op-base mode) -------------------------- */
+
+/* ReduceScatterPlantLocalReduce::RunAsync for one rank of a server and ALL groups, as
+ * CollAllReduceOrderPreservedExecutor::RunReduceScatterLevel0 prepares it for several modules
+ * (exec/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:159-186): group g = the blocks g * L .. g * L + L - 1
+ * (the blocks server g will own), every offset of block b = b * stride, all2allOffset 1 (:176), borrowed space.
+ * The template walks the groups one after the other (tpl/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc:
+ * 132-160: all-to-all of group g on the main and all-to-all streams, its local reduce on the reduce streams); the
+ * groups touch disjoint memory, so step 0 holds every group's all-to-all and steps 1.. every group's reduce rounds. */
+static void prog_plant_groups(OrcTrace* t, uint32_t local_rank, uint32_t rank_size, uint32_t n_groups, const uint64_t* size,
+                              uint64_t stride)
+{
+    const uint32_t all2all_offset = 1;
+#define CALC_OUTPUT_INDEX(round) ((all2all_offset + (round) + local_rank) % rank_size) /* :94-97 */
+#define IS_LAST_BLOCK(index) ((index) == rank_size - 1)                                 /* :103 */
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < rank_size) reduce_step++;
+    for (uint32_t g = 0; g < n_groups; g++) {
+        const uint64_t base = (uint64_t)g * rank_size; /* first block of the group */
+        const int last_group = g == n_groups - 1;      /* :99 */
+        /* LocalCopy, :168-188 */
+        {
+            const uint32_t output_index = CALC_OUTPUT_INDEX(local_rank);
+            if (IS_LAST_BLOCK(output_index) && !(local_rank == rank_size - 1 && last_group))
+                emit(t, 0, K_COPY, local_rank, B_IN, stride * (base + local_rank), local_rank, B_UIN,
+                     stride * (base + local_rank), size[base + local_rank]);
+            else
+                emit(t, 0, K_COPY, local_rank, B_OUT, stride * (base + output_index), local_rank, B_UIN,
+                     stride * (base + local_rank), size[base + local_rank]);
+        }
+        /* RunAlltoAll, :221-247 */
+        for (uint32_t round = 0; round < rank_size; round++) {
+            if (round == local_rank) continue;
+            const uint32_t output_index = CALC_OUTPUT_INDEX(round);
+            if (IS_LAST_BLOCK(output_index) && !(round == rank_size - 1 && last_group))
+                emit(t, 0, K_COPY, round, B_IN, stride * (base + round), local_rank, B_UIN, stride * (base + round),
+                     size[base + round]);
+            else
+                emit(t, 0, K_COPY, round, B_OUT, stride * (base + output_index), local_rank, B_UIN, stride * (base + round),
+                     size[base + round]);
+        }
+        /* RunLocalReduce, :337-414 */
+        const uint64_t src_offset = stride * (base + local_rank); /* inputOffsets[localRank_], :340 */
+        const int may_borrow = !(local_rank == rank_size - 1 && last_group);
+        for (uint32_t round = 0; round < reduce_step; round++) {
+            const uint32_t full = 1u << (reduce_step - round);
+            const uint32_t tail_index = (rank_size < full ? rank_size : full) - 1;
+            const uint32_t head_index = 1u << (reduce_step - round - 1);
+            for (uint32_t offset = 0; offset <= tail_index - head_index; offset++) {
+                const uint32_t input_index = CALC_OUTPUT_INDEX(head_index + offset);
+                const uint32_t output_index = CALC_OUTPUT_INDEX(offset);
+                const int src_borrowed = may_borrow && IS_LAST_BLOCK(input_index);  /* :376-381 */
+                const int dst_borrowed = may_borrow && IS_LAST_BLOCK(output_index); /* :383-388 */
+                emit(t, 1 + round, K_REDUCE, local_rank, dst_borrowed ? B_IN : B_OUT,
+                     dst_borrowed ? src_offset : stride * (base + output_index), local_rank, src_borrowed ? B_IN : B_OUT,
+                     src_borrowed ? src_offset : stride * (base + input_index), size[base + local_rank]);
+            }
+        }
+    }
+#undef CALC_OUTPUT_INDEX
+#undef IS_LAST_BLOCK
+}
+
+/* ReduceScatterPlantLocalReduceCombine::RunAsync for one rank between the servers (links that are not RoCE: the SDMA
+ * branch), tpl/temp_reduce_scatter/reduce_scatter_plant_local_reduce_combine.cc:89-116, prepared by
+ * CollAllReduceOrderPreservedExecutor::RunReduceScatterLevel1 (exec/coll_all_reduce/
+ * coll_all_reduce_order_preserved_executor.cc:208-246).  rank / rank_size: the server index and the number of servers;
+ * in_off[d]: where the level-0 result for server d's block lies, out_off[d]: block (i + d * L) itself.
+ * Step 0: LocalCopy (:118-142) and the all-to-all (:180-209, :211-230); steps 1..: RunLocalReduce (:232-304). */
+static void prog_plant_combine(OrcTrace* t, uint32_t rank, uint32_t rank_size, const uint64_t* size, const uint64_t* in_off,
+                               const uint64_t* out_off, int use_ccl_in, int level0_last_rank)
+{
+#define CALC_OUTPUT_INDEX(round) (((round) + rank) % rank_size) /* :80 */
+#define IS_LAST(x) ((x) == rank_size - 1)                       /* :82-87 */
+    /* userInputOffsets == outputOffsets in this executor (coll_all_reduce_order_preserved_executor.cc:224-227) */
+    for (uint32_t round = 0; round < rank_size; round++) {
+        /* the own block first (LocalCopy), then the peers in ascending order */
+        const uint32_t peer = round == 0 ? rank : (round <= rank ? round - 1 : round);
+        const uint32_t output_index = CALC_OUTPUT_INDEX(peer);
+        const uint32_t src_buf = use_ccl_in ? B_IN : B_OUT;                        /* :125-130, :184-189 */
+        const uint64_t src_off = use_ccl_in ? out_off[peer] : in_off[peer];
+        if (level0_last_rank && IS_LAST(output_index) && !IS_LAST(peer))          /* :132-138, :191-199 */
+            emit(t, 0, K_COPY, peer, B_IN, out_off[peer], rank, src_buf, src_off, size[peer]);
+        else
+            emit(t, 0, K_COPY, peer, B_OUT, out_off[output_index], rank, src_buf, src_off, size[peer]);
+    }
+    uint32_t reduce_step = 0;
+    while ((1u << reduce_step) < rank_size) reduce_step++;
+    for (uint32_t round = 0; round < reduce_step; round++) {
+        const uint32_t full = 1u << (reduce_step - round);
+        const uint32_t tail_index = (rank_size < full ? rank_size : full) - 1;
+        const uint32_t head_index = 1u << (reduce_step - round - 1);
+        for (uint32_t offset = 0; offset <= tail_index - head_index; offset++) {
+            const uint32_t input_index = CALC_OUTPUT_INDEX(head_index + offset);
+            const uint32_t output_index = CALC_OUTPUT_INDEX(offset);
+            const int src_borrowed = level0_last_rank && !IS_LAST(rank) && IS_LAST(input_index);  /* :273-277 */
+            const int dst_borrowed = level0_last_rank && !IS_LAST(rank) && IS_LAST(output_index); /* :279-283 */
+            emit(t, 1 + round, K_REDUCE, rank, dst_borrowed ? B_IN : B_OUT, dst_borrowed ? out_off[rank] : out_off[output_index],
+                 rank, src_borrowed ? B_IN : B_OUT, src_borrowed ? out_off[rank] : out_off[input_index], size[rank]);
+        }
+    }
+#undef CALC_OUTPUT_INDEX
+#undef IS_LAST
+}
+
+static uint32_t ceil_log2_u32(uint32_t n)
+{
+    uint32_t s = 0;
+    while ((1u << s) < n) s++;
+    return s;
+}
+
+/* CollAllReduceOrderPreservedExecutor::KernelRun for every rank of n_servers modules of n_local devices
+ * (exec/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:342-380) inside CollAllReduceExecutor::RunLoop.
+ * alg1 selects the all-gather between the servers (:293-303): ring, NB, else NHR. */
+static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                           uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    /* one device per module takes RunReduceScatterLevel0SingleRank (:195-206): not restated; one module is
+     * build_trace_order_preserved_ar */
+    if (unit == 0 || n_servers < 2 || n_local < 2 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (alg1 != ORC_ALG_ALLREDUCE_RING && alg1 != ORC_ALG_ALLREDUCE_NHR && alg1 != ORC_ALG_ALLREDUCE_NB) return -1;
+    const uint32_t n = n_servers * n_local;
+    const uint64_t max_count = ccl_bytes / unit;
+    if (max_count == 0) return -1;
+    const uint32_t steps0 = ceil_log2_u32(n_local), steps1 = ceil_log2_u32(n_servers);
+    const uint32_t ag1_steps = alg1 == ORC_ALG_ALLREDUCE_RING ? n_servers - 1 : steps1;
+    uint32_t identity[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < ORC_MAX_RANKS; i++) identity[i] = i;
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        const uint64_t cur_size = cur_count * unit;
+        uint64_t spb = (cur_count + n - 1) / n * unit; /* CalcSizePerBlock, :131-136 */
+        spb = (spb + 127u) / 128u * 128u;
+        uint64_t group_size[ORC_MAX_RANKS]; /* CalGroupSlices, :138-147 */
+        uint64_t size_remain = cur_size;
+        for (uint32_t r = 0; r < n; r++) {
+            group_size[r] = size_remain > spb ? spb : size_remain;
+            size_remain -= group_size[r];
+        }
+        g_user_off = user_off;
+        for (uint32_t rank = 0; rank < n; rank++) {
+            const uint32_t server = rank / n_local, local = rank % n_local;
+            uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+            for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+            for (uint32_t d = 0; d < n_servers; d++) level1[d] = d * n_local + local;
+            /* level 0, :356 */
+            g_rank_map = level0;
+            g_step_base = step0;
+            prog_plant_groups(t, local, n_local, n_servers, group_size, spb);
+            /* level 1, :359: RunReduceScatterLevel1 :208-246 */
+            uint64_t size1[ORC_MAX_RANKS], in_off[ORC_MAX_RANKS], out_off[ORC_MAX_RANKS];
+            const uint32_t input_base_index = (1 + local) % n_local; /* :218 */
+            for (uint32_t d = 0; d < n_servers; d++) {
+                in_off[d] = (uint64_t)(input_base_index + d * n_local) * spb;
+                size1[d] = group_size[local + d * n_local];
+                out_off[d] = (uint64_t)(local + d * n_local) * spb;
+            }
+            g_rank_map = level1;
+            g_step_base = step0 + 1 + steps0;
+            prog_plant_combine(t, server, n_servers, size1, in_off, out_off, local == n_local - 2 /* :234-235 */,
+                               local == n_local - 1 /* :239 */);
+            /* all-gather inside the server, :363: RunAllGatherLevel0 :248-283 */
+            OrcSlice seg[ORC_MAX_RANKS];
+            for (uint32_t r = 0; r < n_local; r++) {
+                seg[r].size = group_size[r + server * n_local];
+                seg[r].offset = seg[r].size == 0 ? 0 : (uint64_t)(r + server * n_local) * spb;
+            }
+            g_rank_map = level0;
+            g_step_base = step0 + 2 + steps0 + steps1;
+            prog_mesh_ag(t, local, n_local, seg);
+            /* all-gather between the servers, :366: RunAllGatherLevel1 :285-340 */
+            for (uint32_t d = 0; d < n_servers; d++) {
+                seg[d].size = 0;
+                for (uint32_t j = 0; j < n_local; j++) seg[d].size += group_size[d * n_local + j];
+                seg[d].offset = (uint64_t)d * n_local * spb;
+            }
+            g_rank_map = level1;
+            g_step_base = step0 + 3 + steps0 + steps1;
+            if (alg1 == ORC_ALG_ALLREDUCE_RING) prog_ring_ag_ex(t, server, n_servers, seg, 0, 0);
+            else if (alg1 == ORC_ALG_ALLREDUCE_NB) prog_nb_ag(t, server, n_servers, seg, 0);
+            else prog_nhr_ag(t, server, n_servers, seg, identity, 0, 0); /* stand-alone: order kept, nothing merged */
+            g_rank_map = NULL;
+            g_step_base = step0 + 3 + steps0 + steps1 + ag1_steps;
+            emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_OUT, 0, cur_size); /* :369-376 */
+        }
+        g_user_off = 0;
+        g_step_base = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += 4 + steps0 + steps1 + ag1_steps;
+        user_off += cur_size;
+    }
+    for (uint64_t i = 0; i < t->n; i++) { /* DeviceMem::range refuses a range past the end of the CCL buffer */
+        const OrcOp* o = &t->ops[i];
+        if ((o->dst_buf <= B_OUT && o->dst_off + o->bytes > ccl_bytes) || (o->src_buf <= B_OUT && o->src_off + o->bytes > ccl_bytes)) {
+            free(t->ops);
+            return -1;
+        }
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_order_preserved_ar2(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                                      int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_ar2(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_order_preserved_ar2(int alg1, uint32_t n_servers, uint32_t n_local, void* const* user_in, void* const* user_out,
+                                void* const* ccl_in, void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype,
+                                int op)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_ar2(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
 }
 
 int64_t orc_trace_order_preserved_ar(uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
