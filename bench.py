@@ -80,6 +80,7 @@ WORKLOADS = {
     "dbring_rs_bf16_n8_16MiB": ("doublering_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving allreduce executor over two levels: plant + fold inside the servers, then between them
     "ophier_ring_ar_bf16_2x8_128MiB": ("ophier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
+    "ophierrs_ring_rs_bf16_2x8_8MiB": ("ophierrs_ring_rs_stage", (2, 8), 4194304, "bf16", "sum", "normal(0,1)*1e-3"),
     # the ring / mesh reduce-scatter executors over two levels in op-base mode (blocks of 16 MiB, 2 x 8 ranks)
     "hierrs_ring_rs_bf16_2x8_16MiB": ("hierrs_ring_rs_stage", (2, 8), 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     "meshhierrs_ring_rs_bf16_1x8_16MiB": ("meshhierrs_ring_rs_stage", (1, 8), 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -152,7 +153,8 @@ def main():
     mesh0 = alg_name.startswith("meshhier")  # the mesh executor's level 0 instead of the ring executor's
     hier_rs = alg_name.startswith("hierrs_") or alg_name.startswith("meshhierrs_")  # the reduce-scatter executors
     ophier = alg_name.startswith("ophier_")  # the order-preserving allreduce executor over two levels
-    if alg_name.startswith("hier") or alg_name.startswith("dbring_") or mesh0 or ophier:
+    ophrs = alg_name.startswith("ophierrs_")  # the order-preserving reduce-scatter executor over two levels
+    if alg_name.startswith("hier") or alg_name.startswith("dbring_") or mesh0 or ophier or ophrs:
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
@@ -176,7 +178,7 @@ def main():
         return
 
     nbytes = count * unit
-    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs") or hier_rs) else count
+    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs") or hier_rs or ophrs) else count
     pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
     d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
@@ -192,7 +194,7 @@ def main():
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
     scratch_bytes = 0 if plant else h.scratch_bytes(alg, n, count, dt)
     d_ccl = None
-    if opbase or dbring or plant or hier_rs or ophier:
+    if opbase or dbring or plant or hier_rs or ophier or ophrs:
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both" and not opfused:
             args.lowering = "stepwise"
@@ -218,6 +220,9 @@ def main():
                                                  [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if plant:
             return h.OrderPreservedPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
+        if ophrs:
+            return h.OrderPreservedHierReduceScatterPlan(hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]],
+                                                         ccl_bytes, count, dt, op)
         if ophier:
             return h.OrderPreservedHierAllReducePlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                                      [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
@@ -327,6 +332,9 @@ def main():
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved_ar(n, count, ccl_bytes, odt))
         elif plant:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved(n, count, ccl_bytes, odt))
+        elif ophrs:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2)
+                            for o in oracle.trace_order_preserved_rs2(hier[0], hier[1], count, ccl_bytes, odt))
         elif ophier:
             alg_bytes = sum(o[8] * (3 if o[1] else 2)
                             for o in oracle.trace_order_preserved_ar2(oalg, hier[0], hier[1], count, ccl_bytes, odt))
@@ -340,7 +348,7 @@ def main():
             alg_bytes = (oracle.algorithmic_bytes_opbase(oalg, n, count, ccl_bytes, odt) if opbase
                          else oracle.algorithmic_bytes(oalg, n, count, odt))
         host_ccl = ([[np.zeros(ccl_bytes, np.uint8) for _ in range(n)] for _ in range(2)]
-                    if (opbase or dbring or plant or hier_rs or ophier) else None)
+                    if (opbase or dbring or plant or hier_rs or ophier or ophrs) else None)
 
         def cpu_run(ins, outs):
             if hier_rs:
@@ -352,6 +360,8 @@ def main():
                 oracle.run_order_preserved_ar(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif plant:
                 oracle.run_order_preserved(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
+            elif ophrs:
+                oracle.run_order_preserved_rs2(hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif ophier:
                 oracle.run_order_preserved_ar2(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes,
                                                odt, oop)
@@ -429,7 +439,7 @@ def main():
                 ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
-                if (opbase or dbring or plant or hier_rs or ophier) and not (opfused and name == "fused"):  # what the last chunk left in the CCL buffers
+                if (opbase or dbring or plant or hier_rs or ophier or ophrs) and not (opfused and name == "fused"):  # what the last chunk left in the CCL buffers
                     ok = ok and np.array_equal(d_ccl[0][r].cpu().numpy(), host_ccl[0][r])
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
@@ -438,7 +448,7 @@ def main():
     h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
-        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("order-preserving two-level " if ophier else "double-ring " if dbring else "mesh three-step " if mesh0 else "three-step " if hier else "") + alg_name, opname)
+        metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("order-preserving two-level " if (ophier or ophrs) else "double-ring " if dbring else "mesh three-step " if mesh0 else "three-step " if hier else "") + ("reduce-scatter" if ophrs else "allreduce" if ophier else alg_name), opname)
     out = {
         "metric": metric,
         "value": round(res["gbs"], 2),
@@ -454,14 +464,18 @@ def main():
         "dtype": dtname,
         "data": "synthetic",
         "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": opname,
-                   "algorithm": alg_name, "values": dist, "lowering": best,
+                   "algorithm": ("order_preserved_rs" if ophrs else "order_preserved_ar" if ophier else alg_name),
+                   "values": dist, "lowering": best,
                    **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {}),
-                   **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": alg_name,
-                       "level0_algorithm": ("plant + fold in device order, mesh all-gather (user memory read directly)" if ophier else
+                   **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": ("plant + fold in server order (combine template)" if ophrs else
+                                            "plant + fold in server order (combine template), %s all-gather" % alg_name
+                                            if ophier else alg_name),
+                       "level0_algorithm": ("plant + fold in device order (user memory read directly)" if ophrs else
+                                            "plant + fold in device order, mesh all-gather (user memory read directly)" if ophier else
                                             "double-ring reduce-scatter + all-gather on user memory (DMA reduce)"
                                             if dbring else "multi-stream mesh reduce-scatter + mesh all-gather" if mesh0
                                             else "ring reduce-scatter + ring all-gather")} if hier else {}),
-                   **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant or hier_rs or ophier) else {})},
+                   **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant or hier_rs or ophier or ophrs) else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, best)),

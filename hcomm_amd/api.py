@@ -31,6 +31,7 @@ __all__ = [
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
     "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check", "OrderPreservedFusedPlan",
     "OrderPreservedHierAllReducePlan", "order_preserved_hier_ar_emit", "order_preserved_hier_ar_check",
+    "OrderPreservedHierReduceScatterPlan", "order_preserved_hier_rs_emit", "order_preserved_hier_rs_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
@@ -607,6 +608,47 @@ class OrderPreservedHierAllReducePlan(Plan):
         p = _vp(0)
         check(_oph_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], self._bufs[3], ccl_bytes,
                         count, dtype, op, C.byref(p)), "HcommGfxOrderPreservedHierAllReducePlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_ophrs_emit = _sig("HcommGfxOrderPreservedHierReduceScatterEmit", _i32, _u32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp),
+                   _u64, C.POINTER(_u64))
+_ophrs_check = _sig("HcommGfxOrderPreservedHierReduceScatterCheck", _i32, _u32, _u32, _u64, _u64, C.c_int,
+                    C.POINTER(CheckReport))
+_ophrs_plan = _sig("HcommGfxOrderPreservedHierReduceScatterPlanCreate", _i32, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp),
+                   C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def order_preserved_hier_rs_emit(n_servers, n_local, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_ophrs_emit(n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
+          "HcommGfxOrderPreservedHierReduceScatterEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_ophrs_emit(n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
+          "HcommGfxOrderPreservedHierReduceScatterEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def order_preserved_hier_rs_check(n_servers, n_local, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_ophrs_check(n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
+          "HcommGfxOrderPreservedHierReduceScatterCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class OrderPreservedHierReduceScatterPlan(Plan):
+    """HcommGfxOrderPreservedHierReduceScatterPlanCreate: the order-preserving reduce-scatter executor over two levels."""
+
+    def __init__(self, n_servers, n_local, user_in, user_out, ccl_out, ccl_bytes, count, dtype, op):
+        n = n_servers * n_local
+        assert len(user_in) == n
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_out)]
+        p = _vp(0)
+        check(_ophrs_plan(n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op,
+                          C.byref(p)), "HcommGfxOrderPreservedHierReduceScatterPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

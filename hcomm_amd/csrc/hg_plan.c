@@ -716,6 +716,29 @@ int32_t HcommGfxOrderPreservedHierAllReducePlanCreate(
     return rc;
 }
 
+int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
+    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes,
+    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!userIn || !userOut || !cclOut) return HCCL_E_PTR;
+    if (nServers < 2 || nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    const uint32_t n = nServers * nLocal;
+    int rc = check_bufs(userIn, n);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, n);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclOut, n);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_order_preserved_rs2(&ol, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {NULL, cclOut, NULL, userIn, userOut};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, n, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
+}
+
 /* Both order-preserving executors in one launch: the N user inputs are folded in registers along the executors'
  * rank-order tree (reduce_scatter_plant_local_reduce.cc:337-414: rounds h = 2^(S-1), .., 1 fold contribution h + j
  * onto contribution j) and the root is written to the user output(s).  No CCL buffer is read or written. */

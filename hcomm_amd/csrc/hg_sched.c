@@ -1659,6 +1659,87 @@ int32_t HcommGfxOrderPreservedHierAllReduceEmit(
     return HCCL_SUCCESS;
 }
 
+/* The order-preserving reduce-scatter executor over M servers of L devices (coll_executor/coll_reduce_scatter/
+ * coll_reduce_scatter_order_preserved_executor.cc:171-218, 220-258, 260-283): the two levels of the allreduce executor
+ * above without any borrowed place - every block is one chunk of c bytes, block b of the CCL output buffer at b * c,
+ * of the user input at b * count * unit - and the own block to the user output instead of the all-gathers. */
+static int order_preserved_rs2_build(HgOpList* l, uint32_t n_srv, uint32_t n_loc, uint64_t count, uint64_t ccl_bytes,
+                                     uint32_t unit)
+{
+    const uint32_t n = n_srv * n_loc, r0 = ceil_log2(n_loc), r1 = ceil_log2(n_srv);
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint64_t stride = count * unit;
+    uint32_t step = 0;
+    uint64_t user_off = 0;
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+#define SRV(s, i) ((s) * n_loc + (i))
+        for (uint32_t s = 0; s < n_srv; ++s)
+            for (uint32_t i = 0; i < n_loc; ++i)
+                for (uint32_t q = 0; q < n_loc; ++q)
+                    for (uint32_t g = 0; g < n_srv; ++g)
+                        CHK(push(l, step, COPY, SRV(s, i), OUT, c * (g * n_loc + (1 + q + i) % n_loc), SRV(s, q), UIN,
+                                 user_off + stride * (g * n_loc + i), c));
+        ++step;
+        for (uint32_t h = 1u << (r0 - 1); h >= 1; h >>= 1, ++step)
+            for (uint32_t s = 0; s < n_srv; ++s)
+                for (uint32_t i = 0; i < n_loc; ++i)
+                    for (uint32_t g = 0; g < n_srv; ++g)
+                        for (uint32_t j = 0; j + h < (n_loc < 2 * h ? n_loc : 2 * h); ++j)
+                            CHK(push(l, step, REDUCE, SRV(s, i), OUT, c * (g * n_loc + (1 + j + i) % n_loc), SRV(s, i), OUT,
+                                     c * (g * n_loc + (1 + h + j + i) % n_loc), c));
+        for (uint32_t d = 0; d < n_srv; ++d)
+            for (uint32_t i = 0; i < n_loc; ++i)
+                for (uint32_t c0 = 0; c0 < n_srv; ++c0)
+                    CHK(push(l, step, COPY, SRV(d, i), OUT, c * (i + (c0 + d) % n_srv * n_loc), SRV(c0, i), OUT,
+                             c * ((1 + i) % n_loc + d * n_loc), c));
+        ++step;
+        for (uint32_t h = 1u << (r1 - 1); h >= 1; h >>= 1, ++step)
+            for (uint32_t d = 0; d < n_srv; ++d)
+                for (uint32_t i = 0; i < n_loc; ++i)
+                    for (uint32_t j = 0; j + h < (n_srv < 2 * h ? n_srv : 2 * h); ++j)
+                        CHK(push(l, step, REDUCE, SRV(d, i), OUT, c * (i + (j + d) % n_srv * n_loc), SRV(d, i), OUT,
+                                 c * (i + (h + j + d) % n_srv * n_loc), c));
+        for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, user_off, p, OUT, c * p, c));
+        ++step;
+#undef SRV
+        user_off += c;
+        left -= cur;
+    }
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_order_preserved_rs2(HgOpList* l, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                                    int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || n_servers < 2 || n_local < 2 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    int rc = order_preserved_rs2_build(l, n_servers, n_local, count, ccl_bytes, unit);
+    if (rc == HCCL_SUCCESS) rc = order_by_step_rank(l);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedHierReduceScatterEmit(
+    uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops,
+    uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved_rs2(&l, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 int hg_schedule_order_preserved_ar(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
 {
     memset(l, 0, sizeof(*l));

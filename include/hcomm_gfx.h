@@ -15,7 +15,8 @@
  *                                the operation lists and check them symbolically without a GPU;
  *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
  *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*,
- *                                HcommGfxOrderPreservedHierAllReduce*, HcommGfxOrderPreservedFused*: what the
+ *                                HcommGfxOrderPreservedHierAllReduce*, HcommGfxOrderPreservedHierReduceScatter*,
+ *                                HcommGfxOrderPreservedFused*: what the
  *                                reference's executors do around the templates (chunk loops through the CCL
  *                                buffers, two communicator levels, user memory read and written directly), each
  *                                as PlanCreate / Emit / Check.
@@ -766,6 +767,25 @@ int32_t HcommGfxOrderPreservedHierAllReduceEmit(
 int32_t HcommGfxOrderPreservedHierAllReduceCheck(
     HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
     HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
+ * The order-preserving REDUCE-SCATTER executor over nServers modules of nLocal devices
+ * (coll_executor/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:171-218, 220-258, 260-283): the
+ * two plant levels of the allreduce executor above on blocks of one chunk each (at most cclBytes / N rounded down to
+ * 128 bytes per block), without borrowed places, and rank p's block from the CCL output buffer to its user output.
+ * userIn: N * count elements per rank (block p at p * count); userOut: count elements; cclOut: cclBytes.  Rank p's
+ * result is tree(servers)( tree(devices of server 0), ... ) over the N contributions to block p.
+ * nServers >= 2 and nLocal >= 2.  Step-wise lowering.
+ */
+int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
+    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes,
+    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxOrderPreservedHierReduceScatterEmit(
+    uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops,
+    uint64_t cap, uint64_t* n);
+int32_t HcommGfxOrderPreservedHierReduceScatterCheck(
+    uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes, HcommDataType dataType,
+    HcommGfxCheckReport* report);
 
 /*
  * The single-launch lowering of the two order-preserving executors (no counterpart in the reference, which has no

@@ -68,6 +68,8 @@
  *                                     by hand; reduction trees 2 x 2 .. 3 x 3 composed by hand from the single-level
  *                                     trees; slot / borrowed-place layout of both levels from the definition; exact
  *                                     integer results over several chunks, ring / NB / NHR all-gather; pinned
+ *   two-level order-preserving reduce-scatter . the complete operation list of 2 x 2 by hand; the composed reduction
+ *                                     trees per block; layout from the definition; exact integer results; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
 #include <stdint.h>
@@ -2390,12 +2392,14 @@ static int build_trace_order_preserved_ar(OrcTrace* t, uint32_t n, uint64_t coun
 /* ReduceScatterPlantLocalReduce::RunAsync for one rank of a server and ALL groups, as
  * CollAllReduceOrderPreservedExecutor::RunReduceScatterLevel0 prepares it for several modules
  * (exec/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:159-186): group g = the blocks g * L .. g * L + L - 1
- * (the blocks server g will own), every offset of block b = b * stride, all2allOffset 1 (:176), borrowed space.
+ * (the blocks server g will own), every offset of block b = b * stride, all2allOffset 1 (:176), borrowed space -
+ * and as CollReduceScatterOrderPreservedExecutor::RunReduceScatterLevel0 prepares it (exec/coll_reduce_scatter/
+ * coll_reduce_scatter_order_preserved_executor.cc:185-211): block b of the user input at b * uin_stride, no borrowed space.
  * The template walks the groups one after the other (tpl/temp_reduce_scatter/reduce_scatter_plant_local_reduce.cc:
  * 132-160: all-to-all of group g on the main and all-to-all streams, its local reduce on the reduce streams); the
  * groups touch disjoint memory, so step 0 holds every group's all-to-all and steps 1.. every group's reduce rounds. */
 static void prog_plant_groups(OrcTrace* t, uint32_t local_rank, uint32_t rank_size, uint32_t n_groups, const uint64_t* size,
-                              uint64_t stride)
+                              uint64_t stride, uint64_t uin_stride, int need_space_borrow)
 {
     const uint32_t all2all_offset = 1;
 #define CALC_OUTPUT_INDEX(round) ((all2all_offset + (round) + local_rank) % rank_size) /* :94-97 */
@@ -2408,27 +2412,27 @@ static void prog_plant_groups(OrcTrace* t, uint32_t local_rank, uint32_t rank_si
         /* LocalCopy, :168-188 */
         {
             const uint32_t output_index = CALC_OUTPUT_INDEX(local_rank);
-            if (IS_LAST_BLOCK(output_index) && !(local_rank == rank_size - 1 && last_group))
+            if (need_space_borrow && IS_LAST_BLOCK(output_index) && !(local_rank == rank_size - 1 && last_group))
                 emit(t, 0, K_COPY, local_rank, B_IN, stride * (base + local_rank), local_rank, B_UIN,
-                     stride * (base + local_rank), size[base + local_rank]);
+                     uin_stride * (base + local_rank), size[base + local_rank]);
             else
                 emit(t, 0, K_COPY, local_rank, B_OUT, stride * (base + output_index), local_rank, B_UIN,
-                     stride * (base + local_rank), size[base + local_rank]);
+                     uin_stride * (base + local_rank), size[base + local_rank]);
         }
         /* RunAlltoAll, :221-247 */
         for (uint32_t round = 0; round < rank_size; round++) {
             if (round == local_rank) continue;
             const uint32_t output_index = CALC_OUTPUT_INDEX(round);
-            if (IS_LAST_BLOCK(output_index) && !(round == rank_size - 1 && last_group))
-                emit(t, 0, K_COPY, round, B_IN, stride * (base + round), local_rank, B_UIN, stride * (base + round),
+            if (need_space_borrow && IS_LAST_BLOCK(output_index) && !(round == rank_size - 1 && last_group))
+                emit(t, 0, K_COPY, round, B_IN, stride * (base + round), local_rank, B_UIN, uin_stride * (base + round),
                      size[base + round]);
             else
-                emit(t, 0, K_COPY, round, B_OUT, stride * (base + output_index), local_rank, B_UIN, stride * (base + round),
-                     size[base + round]);
+                emit(t, 0, K_COPY, round, B_OUT, stride * (base + output_index), local_rank, B_UIN,
+                     uin_stride * (base + round), size[base + round]);
         }
         /* RunLocalReduce, :337-414 */
         const uint64_t src_offset = stride * (base + local_rank); /* inputOffsets[localRank_], :340 */
-        const int may_borrow = !(local_rank == rank_size - 1 && last_group);
+        const int may_borrow = need_space_borrow && !(local_rank == rank_size - 1 && last_group);
         for (uint32_t round = 0; round < reduce_step; round++) {
             const uint32_t full = 1u << (reduce_step - round);
             const uint32_t tail_index = (rank_size < full ? rank_size : full) - 1;
@@ -2455,8 +2459,10 @@ static void prog_plant_groups(OrcTrace* t, uint32_t local_rank, uint32_t rank_si
  * in_off[d]: where the level-0 result for server d's block lies, out_off[d]: block (i + d * L) itself.
  * Step 0: LocalCopy (:118-142) and the all-to-all (:180-209, :211-230); steps 1..: RunLocalReduce (:232-304). */
 static void prog_plant_combine(OrcTrace* t, uint32_t rank, uint32_t rank_size, const uint64_t* size, const uint64_t* in_off,
-                               const uint64_t* out_off, int use_ccl_in, int level0_last_rank)
+                               const uint64_t* out_off, int use_ccl_in, int level0_last_rank, int need_space_borrow)
 {
+    use_ccl_in = use_ccl_in && need_space_borrow;             /* every borrowed place is behind isNeedSpaceBorrow_ */
+    level0_last_rank = level0_last_rank && need_space_borrow;
 #define CALC_OUTPUT_INDEX(round) (((round) + rank) % rank_size) /* :80 */
 #define IS_LAST(x) ((x) == rank_size - 1)                       /* :82-87 */
     /* userInputOffsets == outputOffsets in this executor (coll_all_reduce_order_preserved_executor.cc:224-227) */
@@ -2538,7 +2544,7 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
             /* level 0, :356 */
             g_rank_map = level0;
             g_step_base = step0;
-            prog_plant_groups(t, local, n_local, n_servers, group_size, spb);
+            prog_plant_groups(t, local, n_local, n_servers, group_size, spb, spb, 1);
             /* level 1, :359: RunReduceScatterLevel1 :208-246 */
             uint64_t size1[ORC_MAX_RANKS], in_off[ORC_MAX_RANKS], out_off[ORC_MAX_RANKS];
             const uint32_t input_base_index = (1 + local) % n_local; /* :218 */
@@ -2550,7 +2556,7 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
             g_rank_map = level1;
             g_step_base = step0 + 1 + steps0;
             prog_plant_combine(t, server, n_servers, size1, in_off, out_off, local == n_local - 2 /* :234-235 */,
-                               local == n_local - 1 /* :239 */);
+                               local == n_local - 1 /* :239 */, 1);
             /* all-gather inside the server, :363: RunAllGatherLevel0 :248-283 */
             OrcSlice seg[ORC_MAX_RANKS];
             for (uint32_t r = 0; r < n_local; r++) {
@@ -2592,6 +2598,88 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
         }
     }
     return sort_trace(t);
+}
+
+/* CollReduceScatterOrderPreservedExecutor::KernelRun for every rank of n_servers modules of n_local devices
+ * (exec/coll_reduce_scatter/coll_reduce_scatter_order_preserved_executor.cc:260-283: level 0 :171-218, level 1
+ * :220-258 - the Combine template without borrowed space, :248 - own block to the user output :273-279) inside
+ * CollReduceScatterExecutor::RunLoop (exec/coll_reduce_scatter/coll_reduce_scatter_executor.cc:124-134, 149-220). */
+static int build_trace_order_preserved_rs2(OrcTrace* t, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                           uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n_servers < 2 || n_local < 2 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    const uint32_t n = n_servers * n_local;
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
+    if (max_count == 0) return -1;
+    const uint32_t steps0 = ceil_log2_u32(n_local), steps1 = ceil_log2_u32(n_servers);
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        const uint64_t cur_size = cur_count * unit;
+        uint64_t size[ORC_MAX_RANKS];
+        for (uint32_t r = 0; r < n; r++) size[r] = cur_size;
+        g_user_off = user_off;
+        for (uint32_t rank = 0; rank < n; rank++) {
+            const uint32_t server = rank / n_local, local = rank % n_local;
+            uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+            for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+            for (uint32_t d = 0; d < n_servers; d++) level1[d] = d * n_local + local;
+            g_rank_map = level0;
+            g_step_base = step0;
+            prog_plant_groups(t, local, n_local, n_servers, size, cur_size, count * unit, 0); /* :267 */
+            uint64_t in_off[ORC_MAX_RANKS], out_off[ORC_MAX_RANKS];
+            const uint32_t input_base_index = (1 + local) % n_local; /* :231-232 */
+            for (uint32_t d = 0; d < n_servers; d++) {
+                in_off[d] = (uint64_t)(input_base_index + d * n_local) * cur_size;
+                out_off[d] = (uint64_t)(local + d * n_local) * cur_size;
+            }
+            g_rank_map = level1;
+            g_step_base = step0 + 1 + steps0;
+            prog_plant_combine(t, server, n_servers, size, in_off, out_off, local == n_local - 2, local == n_local - 1,
+                               0 /* borrowSpace = level0Ranksize == 1, :248 */); /* :270 */
+            g_rank_map = NULL;
+            g_step_base = step0 + 2 + steps0 + steps1;
+            emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_OUT, cur_size * rank, cur_size); /* :273-279 */
+        }
+        g_user_off = 0;
+        g_step_base = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += 3 + steps0 + steps1;
+        user_off += cur_size;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_order_preserved_rs2(uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes, int dtype,
+                                      OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_rs2(&t, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_order_preserved_rs2(uint32_t n_servers, uint32_t n_local, void* const* user_in, void* const* user_out,
+                                void* const* ccl_in, void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype,
+                                int op)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_rs2(&t, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
 }
 
 int64_t orc_trace_order_preserved_ar2(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
