@@ -161,7 +161,8 @@ def main():
     # one-server executors on user memory (DMA reduce)
     plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar")
     opar = alg_name == "order_preserved_ar"
-    opfused = alg_name in ("order_preserved_ar", "order_preserved_rs")  # these two also have a single-launch lowering
+    # the order-preserving executors also have a single-launch lowering
+    opfused = alg_name in ("order_preserved_ar", "order_preserved_rs") or ophier or ophrs
     dbrs = alg_name == "doublering_rs"
     dt, alg, op = DT[dtname], (None if plant else ALG[alg_name]), OP[opname]
     unit = h.DTYPE_SIZE[dt]
@@ -198,7 +199,7 @@ def main():
         d_ccl = [[torch.zeros(ccl_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] for _ in range(2)]
         if args.lowering == "both" and not opfused:
             args.lowering = "stepwise"
-    if hier or (plant and not opfused):
+    if (hier and not opfused) or (plant and not opfused):
         args.lowering = "stepwise"  # composed from the step lists of its levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
@@ -214,7 +215,7 @@ def main():
         if dbrs:
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
         if opfused and low == h.Lowering.FUSED:  # one launch on the user buffers, no CCL buffer
-            return h.OrderPreservedFusedPlan(opar, in_ptrs, out_ptrs, count, dt, op)
+            return h.OrderPreservedFusedPlan(opar or ophier, in_ptrs, out_ptrs, count, dt, op, n_servers=hier[0] if hier else 1)
         if opar:
             return h.OrderPreservedAllReducePlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                                  [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)

@@ -655,19 +655,20 @@ class OrderPreservedHierReduceScatterPlan(Plan):
         self.info = info
 
 
-_opf_plan = _sig("HcommGfxOrderPreservedFusedPlanCreate", _i32, _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
-                 C.c_int, C.POINTER(_vp))
+_opf_plan = _sig("HcommGfxOrderPreservedFusedPlanCreate", _i32, _i32, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64,
+                 C.c_int, C.c_int, C.POINTER(_vp))
 
 
 class OrderPreservedFusedPlan(Plan):
     """HcommGfxOrderPreservedFusedPlanCreate: either order-preserving executor as one launch on the user buffers."""
 
-    def __init__(self, all_reduce, user_in, user_out, count, dtype, op):
+    def __init__(self, all_reduce, user_in, user_out, count, dtype, op, n_servers=1):
         n = len(user_in)
+        assert n % n_servers == 0
         self._bufs = [(_vp * n)(*b) for b in (user_in, user_out)]
         p = _vp(0)
-        check(_opf_plan(int(all_reduce), n, self._bufs[0], self._bufs[1], count, dtype, op, C.byref(p)),
-              "HcommGfxOrderPreservedFusedPlanCreate")
+        check(_opf_plan(int(all_reduce), n_servers, n // n_servers, self._bufs[0], self._bufs[1], count, dtype, op,
+                        C.byref(p)), "HcommGfxOrderPreservedFusedPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

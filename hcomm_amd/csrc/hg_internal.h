@@ -46,7 +46,8 @@ typedef struct {
  * tree == 1, from in[first[s] XOR bitrev(j)] + off[s] (recursive halving), or, when tree == 2 / 3, from
  * in[(first[s] + j) mod nranks] / in[(first[s] - j) mod nranks] with only nranks <= k positions present (the
  * truncated trees of the nonuniform hierarchical ring / nonuniform Bruck schedules), or, when tree == 4, from
- * in[bitrev(j)] where that rank exists (the rank-order tree of the order-preserving executors; inputs only read).
+ * in[pos[j]] where pos[j] names a rank (the rank-order trees of the order-preserving executors, laid out by the host;
+ * inputs only read).
  */
 typedef struct {
     const void* in[HCOMM_GFX_MAX_RANKS];
@@ -63,12 +64,13 @@ typedef struct {
     uint32_t store_partials; /* store the running value to position j's buffer after fold step j >= 1 */
     uint32_t store_final_first; /* store the final value to position 0's buffer */
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
-    uint32_t tree;           /* 0 chain; binary tree over k = 2^L positions: 1 recursive halving, 2 / 3 rotation + / -, 4 rank order */
+    uint32_t tree;           /* 0 chain; binary tree over k = 2^L positions: 1 recursive halving, 2 / 3 rotation + / -, 4 leaves from pos[] */
     uint32_t nout;           /* tree only: number of out[] entries that receive the result */
     uint32_t ascending;      /* chain only: position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s] */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
+    uint8_t pos[HCOMM_GFX_MAX_RANKS]; /* tree == 4: the rank at leaf position q, or 255 where the tree has a hole */
 } HgFoldTable;
 
 /* Launch geometry decided on the host so that recorder threads can report it without a GPU. */

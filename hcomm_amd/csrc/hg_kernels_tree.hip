@@ -79,9 +79,11 @@ __device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t
 // q a multiple of 2^(l+1)) with q + 2^l wherever that position exists - the fold rank (c +- q) performs at step l
 // from rank (c +- q) +- 2^l.  An even position that had a right neighbour keeps the last value it computed; the
 // root goes to every output (allreduce) or to the owner's output (reduce-scatter).
-// tree == 4 is the rank-order tree of the order-preserving executors: position q holds rank bitrev(q) where that
-// rank exists, so level l folds rank j + K / 2^(l+1) onto rank j - the contributions K/2 .. onto 0 .., then
-// K/4 .. onto 0 .., down to 1 onto 0; the inputs are only read.
+// tree == 4 takes the leaves from tab.pos[] (255 = no leaf): the host lays the rank-order trees of the
+// order-preserving executors out that way - on one server position q holds rank bitrev(q) where that rank exists, so
+// level l folds rank j + K / 2^(l+1) onto rank j (the contributions K/2 .. onto 0 .., then K/4 .. onto 0 .., down to
+// 1 onto 0); over servers x devices the low position bits walk a server's devices like that and the high bits the
+// servers.  A hole's left neighbour always exists; the inputs are only read.
 template <class Item, int L, uint32_t NU>
 __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
                                                     const uint64_t (&idx)[NU])
@@ -99,7 +101,7 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         if (order) {
-            b[q] = bitrev<L>(q);
+            b[q] = tab.pos[q];
             have[q] = b[q] < n;
         } else {
             b[q] = plus ? c + q : c + n - q;

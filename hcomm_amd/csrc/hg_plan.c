@@ -739,27 +739,50 @@ int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
     return rc;
 }
 
-/* Both order-preserving executors in one launch: the N user inputs are folded in registers along the executors'
- * rank-order tree (reduce_scatter_plant_local_reduce.cc:337-414: rounds h = 2^(S-1), .., 1 fold contribution h + j
- * onto contribution j) and the root is written to the user output(s).  No CCL buffer is read or written. */
+/* bit reversal of q inside `bits` bits */
+static uint32_t bitrev_n(uint32_t q, uint32_t bits)
+{
+    uint32_t r = 0;
+    for (uint32_t i = 0; i < bits; ++i) r |= ((q >> i) & 1u) << (bits - 1 - i);
+    return r;
+}
+
+/* The order-preserving executors in one launch: the N user inputs are folded in registers along the executors' tree
+ * and the root is written to the user output(s).  No CCL buffer is read or written.
+ * One server: rounds h = 2^(S-1), .., 1 fold contribution h + j onto contribution j
+ * (reduce_scatter_plant_local_reduce.cc:337-414) - a balanced tree whose leaf q is rank bitrev(q).
+ * Servers x devices: that tree over a server's devices first, then the same shape over the servers
+ * (reduce_scatter_plant_local_reduce_combine.cc:232-304) - leaf q = (server bitrev(high bits), device bitrev(low bits)). */
 int32_t HcommGfxOrderPreservedFusedPlanCreate(
-    int32_t allReduce, uint32_t nRanks, void* const* userIn, void* const* userOut, uint64_t count, HcommDataType dataType,
-    HcommReduceOp reduceOp, HcommGfxPlan** plan)
+    int32_t allReduce, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
 {
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
-    if (nRanks < 2 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (nServers == 0 || nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    const uint32_t nRanks = nServers * nLocal;
     int rc = check_bufs(userIn, nRanks);
     if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, nRanks);
     if (rc != HCCL_SUCCESS) return rc;
+    uint32_t bits_l = 0, bits_s = 0;
+    while ((1u << bits_l) < nLocal) ++bits_l;
+    while ((1u << bits_s) < nServers) ++bits_s;
+    /* the kernel folds at most 32 leaf positions, holes included (5 x 6 ranks would need 8 x 8) */
+    if (bits_l + bits_s > 5u) return HCCL_E_NOT_SUPPORT;
     const uint64_t block = count * HcommGfxDataTypeSize(dataType);
     /* the reduce-scatter reads block p of every input at p * block: 128-bit accesses need 16-byte multiples */
     if (!allReduce && (block & (HG_VEC_BYTES - 1u))) return HCCL_E_NOT_SUPPORT;
     /* steps and algorithmic bytes are those of the step-wise plan with an unbounded CCL buffer (a single chunk) */
     HgOpList ol;
-    rc = allReduce ? hg_schedule_order_preserved_ar(&ol, nRanks, count, (uint64_t)1 << 62, (int)dataType)
-                   : hg_schedule_order_preserved(&ol, nRanks, count, (uint64_t)1 << 62, (int)dataType);
+    const uint64_t unbounded = (uint64_t)1 << 62;
+    if (nServers == 1)
+        rc = allReduce ? hg_schedule_order_preserved_ar(&ol, nRanks, count, unbounded, (int)dataType)
+                       : hg_schedule_order_preserved(&ol, nRanks, count, unbounded, (int)dataType);
+    else
+        rc = allReduce ? hg_schedule_order_preserved_ar2(&ol, HCOMM_GFX_ALG_ALLREDUCE_RING, nServers, nLocal, count, unbounded,
+                                                         (int)dataType)
+                       : hg_schedule_order_preserved_rs2(&ol, nServers, nLocal, count, unbounded, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
     if (!p) {
@@ -782,9 +805,14 @@ int32_t HcommGfxOrderPreservedFusedPlanCreate(
         l->op = (uint32_t)reduceOp;
         HgFoldTable* f = &l->tab.fold;
         f->tree = 4u;
-        f->k = 2;
-        while (f->k < nRanks) f->k <<= 1;
+        f->k = 1u << (bits_l + bits_s);
+        if (f->k < 2) f->k = 2;
         f->nranks = nRanks;
+        memset(f->pos, 255, sizeof(f->pos));
+        for (uint32_t q = 0; q < f->k; ++q) {
+            const uint32_t dev = bitrev_n(q & ((1u << bits_l) - 1u), bits_l), srv = bitrev_n(q >> bits_l, bits_s);
+            if (dev < nLocal && srv < nServers) f->pos[q] = (uint8_t)(srv * nLocal + dev);
+        }
         for (uint32_t r = 0; r < nRanks; ++r) {
             f->in[r] = userIn[r];
             f->out[r] = userOut[r];

@@ -788,20 +788,24 @@ int32_t HcommGfxOrderPreservedHierReduceScatterCheck(
     HcommGfxCheckReport* report);
 
 /*
- * The single-launch lowering of the two order-preserving executors (no counterpart in the reference, which has no
- * device that can read N ranks' memory in one kernel): every element of the result is folded in registers from the
- * N user inputs along the executors' fixed tree over rank order (reduce_scatter_plant_local_reduce.cc:337-414:
- * contribution h + j onto contribution j for h = 2^(S-1), .., 1) and written straight to the user output(s).
- * allReduce == 0: userIn holds nRanks * count elements per rank and rank p's userOut receives block p (the result of
- * HcommGfxOrderPreservedPlanCreate); allReduce != 0: count elements in and out on every rank (the result of
- * HcommGfxOrderPreservedAllReducePlanCreate).  The user outputs are bit-identical to those plans' for every data
+ * The single-launch lowering of the order-preserving executors (no counterpart in the reference, which has no device
+ * that can read N ranks' memory in one kernel): every element of the result is folded in registers from the N user
+ * inputs along the executors' fixed tree - on one server (nServers == 1) the tree over rank order
+ * (reduce_scatter_plant_local_reduce.cc:337-414: contribution h + j onto contribution j for h = 2^(S-1), .., 1); over
+ * nServers x nLocal ranks that tree over every server's devices, then the same shape over the servers
+ * (reduce_scatter_plant_local_reduce_combine.cc:232-304) - and written straight to the user output(s).
+ * allReduce == 0: userIn holds N * count elements per rank and rank p's userOut receives block p (the result of
+ * HcommGfxOrderPreservedPlanCreate / HcommGfxOrderPreservedHierReduceScatterPlanCreate); allReduce != 0: count
+ * elements in and out on every rank (the result of HcommGfxOrderPreservedAllReducePlanCreate /
+ * HcommGfxOrderPreservedHierAllReducePlanCreate).  The user outputs are bit-identical to those plans' for every data
  * type and reduce operation; the user inputs are only read; the CCL buffers are not needed and not touched, so there
  * is no chunk loop.  HCCL_E_NOT_SUPPORT for a reduce-scatter whose block (count * unit bytes) is not a multiple of
- * 16 bytes: use the step-wise plan.  Buffers 128-byte aligned, nRanks >= 2.
+ * 16 bytes, and where ceil_pow2(nServers) * ceil_pow2(nLocal) exceeds 32 (5 x 6, 3 x 9 ...): use the step-wise plan.
+ * Buffers 128-byte aligned, nLocal >= 2.
  */
 int32_t HcommGfxOrderPreservedFusedPlanCreate(
-    int32_t allReduce, uint32_t nRanks, void* const* userIn, void* const* userOut, uint64_t count, HcommDataType dataType,
-    HcommReduceOp reduceOp, HcommGfxPlan** plan);
+    int32_t allReduce, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 
 /*
  * A plan from a caller's own op list - any schedule written as the two operations the reference's templates hand

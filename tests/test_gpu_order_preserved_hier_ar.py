@@ -88,3 +88,78 @@ def test_randomized_shapes(gpu_thread):
         ccl = int(rng.integers(256, 2048)) * 512          # at least 128 KiB: the rounded-up slots always fit
         say("random order preserved two-level allreduce", i, alg, m, l, count, dtype, op, ccl)
         run_case(gpu_thread, alg, m, l, count, dtype, op, ccl, seed=i)
+
+
+# ---- the single-launch lowering over servers x devices: the same user outputs from one kernel ------------------------
+
+def run_fused(thread, all_reduce, m, l, count, dtype, op, seed=0):
+    dt, o, n = DT[dtype], OPS[op], m * l
+    in_count = count if all_reduce else n * count
+    host_in = [gen(dt, in_count, 16000 + seed * 100 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    sentinel = gen(dt, count, 994, "wide")
+    unit = h.DTYPE_SIZE[dt]
+    ccl = max(1 << 17, -(-count * unit * n // 128) * 128)
+    w_in = [x.copy() for x in host_in]
+    w_out = [sentinel.copy() for _ in range(n)]
+    w_ccl = [[np.zeros(ccl, np.uint8) for _ in range(n)] for _ in range(2)]
+    if all_reduce:
+        oracle.run_order_preserved_ar2(oracle.ALG_ALLREDUCE_NHR, m, l, w_in, w_out, w_ccl[0], w_ccl[1], count, ccl, dt, o)
+    else:
+        oracle.run_order_preserved_rs2(m, l, w_in, w_out, w_ccl[0], w_ccl[1], count, ccl, dt, o)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    plan = h.OrderPreservedFusedPlan(all_reduce, [t.data_ptr() for t in d_in], [t.data_ptr() for t in d_out], count, dt, o,
+                                     n_servers=m)
+    try:
+        assert plan.info.launches == 1
+        assert plan.run(thread) == 0
+        assert h.HcommGfxThreadSynchronize(thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_out[r], sentinel), w_out[r], dt, "user out[%d]" % r)
+            assert np.array_equal(from_dev(d_in[r], host_in[r]).view(np.uint8), host_in[r].view(np.uint8)), "user in[%d] was written" % r
+    finally:
+        plan.destroy()
+
+
+FUSED_CASES = [
+    (1, 2, 8, 1 << 20, "bf16", "sum"),
+    (1, 4, 4, 300007, "fp32", "sum"),
+    (1, 3, 5, 100003, "fp16", "sum"),          # 4 x 8 leaf positions, 17 holes
+    (1, 5, 3, 70001, "int8", "max"),
+    (1, 2, 2, 100, "fp32", "prod"),
+    (1, 8, 4, 50000, "int32", "sum"),
+    (1, 7, 3, 4099, "int16", "sum"),
+    (1, 16, 2, 77777, "bf16", "sum"),
+    (1, 2, 16, 33333, "fp32", "min"),
+    (0, 2, 8, 1 << 16, "bf16", "sum"),
+    (0, 4, 4, 100000, "fp32", "sum"),
+    (0, 3, 5, 30000, "fp16", "sum"),
+    (0, 7, 3, 4104, "int16", "sum"),
+    (0, 2, 2, 16, "fp32", "prod"),
+]
+
+
+@pytest.mark.parametrize("all_reduce,m,l,count,dtype,op", FUSED_CASES)
+def test_single_launch_lowering_matches_the_two_level_executors(gpu_thread, all_reduce, m, l, count, dtype, op):
+    say("order preserved two-level fused", all_reduce, m, l, count, dtype, op)
+    run_fused(gpu_thread, all_reduce, m, l, count, dtype, op)
+
+
+def test_single_launch_lowering_randomized(gpu_thread):
+    rng = np.random.default_rng(6666)
+    done = 0
+    while done < 30:
+        all_reduce = int(rng.integers(2))
+        m = int(rng.integers(2, 9))
+        l = int(rng.integers(2, 32 // m + 1))
+        dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
+        unit = h.DTYPE_SIZE[DT[dtype]]
+        count = int(rng.integers(1, 100000))
+        if (m - 1).bit_length() + (l - 1).bit_length() > 5:
+            continue                                          # more than 32 leaf positions: no single-launch plan
+        if not all_reduce:
+            count = max(16 // unit, count // 8 // (16 // unit) * (16 // unit))   # blocks of whole 16 bytes
+        op = ["sum", "max", "min"][rng.integers(3)]
+        say("random order preserved two-level fused", done, all_reduce, m, l, count, dtype, op)
+        run_fused(gpu_thread, all_reduce, m, l, count, dtype, op, seed=done)
+        done += 1

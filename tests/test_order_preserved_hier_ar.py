@@ -159,3 +159,59 @@ def test_rejects_bad_arguments():
                      (oracle.ALG_ALLREDUCE_RHD, 2, 2, 100, 1 << 20, oracle.F32)):
             with pytest.raises((ValueError, h.HcommError)):
                 f(*args)
+
+
+# ---- the single-launch lowering over servers x devices ---------------------------------------------------------------
+
+def kernel_tree_two_level(m, l):
+    """The tree the fold kernel builds from the leaf table the host lays out for m servers of l devices: leaf q holds
+    (server bitrev(high bits), device bitrev(low bits)) where both exist; level k folds position q + 2^k into q."""
+    bl, bs = (l - 1).bit_length(), (m - 1).bit_length()
+    rev = lambda q, bits: int(format(q, "0%db" % bits)[::-1], 2) if bits else 0
+    x = []
+    for q in range(1 << (bl + bs)):
+        dev, srv = rev(q & ((1 << bl) - 1), bl), rev(q >> bl, bs)
+        x.append(srv * l + dev if dev < l and srv < m else None)
+    for k in range(bl + bs):
+        for q in range(0, len(x), 2 << k):
+            if x[q + (1 << k)] is not None:
+                x[q] = [x[q], x[q + (1 << k)]]
+    return x[0]
+
+
+def test_fused_leaf_layout_gives_the_two_level_tree():
+    for key, tree in GOLD["trees"].items():
+        if not key.startswith("_"):
+            m, l = (int(v) for v in key.split("x"))
+            assert kernel_tree_two_level(m, l) == tree, key
+    for m, l in SHAPES + [(1, 2), (1, 5), (1, 8), (1, 32)]:
+        if ((m - 1).bit_length() + (l - 1).bit_length()) <= 5 and m <= 8 and l <= 8:     # hand-derived trees: 2 .. 8
+            want = two_level_tree(m, l) if m > 1 else TREES1[str(l)]
+            assert kernel_tree_two_level(m, l) == want, (m, l)
+
+
+def test_fused_two_level_plan_shape_and_limits():
+    base = 0x7f0000000000
+    for m, l in SHAPES:
+        n = m * l
+        uin = [base + r * (1 << 32) for r in range(n)]
+        uout = [base + (64 + r) * (1 << 32) for r in range(n)]
+        fits = (m - 1).bit_length() + (l - 1).bit_length() <= 5
+        for all_reduce, count in ((1, 100003), (0, 4096)):
+            if not fits:
+                with pytest.raises(h.HcommError) as e:
+                    h.OrderPreservedFusedPlan(all_reduce, uin, uout, count, oracle.F32, oracle.SUM, n_servers=m)
+                assert e.value.code == h.HcclResult.E_NOT_SUPPORT
+                continue
+            p = h.OrderPreservedFusedPlan(all_reduce, uin, uout, count, oracle.F32, oracle.SUM, n_servers=m)
+            try:
+                launches = p.launches()
+                assert [x.kind for x in launches] == [h.Kernel.TREE]
+                assert launches[0].nseg == (1 if all_reduce else n)
+                assert p.info.movedBytes == launches[0].bytes * (2 * n if all_reduce else n + 1)
+                ops = (oracle.trace_order_preserved_ar2(oracle.ALG_ALLREDUCE_RING, m, l, count, 1 << 40, oracle.F32) if all_reduce
+                       else oracle.trace_order_preserved_rs2(m, l, count, 1 << 40, oracle.F32))
+                assert p.info.algorithmicBytes == sum(o[8] * (3 if o[1] else 2) for o in ops)
+            finally:
+                p.destroy()
+    assert not all((m - 1).bit_length() + (l - 1).bit_length() <= 5 for m, l in SHAPES + [(5, 6)])
