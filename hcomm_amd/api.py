@@ -29,6 +29,7 @@ __all__ = [
     "HcommChannelFenceOnThread", "HcommChannelDrainOnThread",
     "HierPlan", "hier_emit", "hier_check", "DoubleRingPlan", "dbring_emit", "dbring_check",
     "OrderPreservedPlan", "order_preserved_emit", "order_preserved_check",
+    "OrderPreservedSmallPlan", "order_preserved_small_emit", "order_preserved_small_check",
     "OrderPreservedAllReducePlan", "order_preserved_ar_emit", "order_preserved_ar_check", "OrderPreservedFusedPlan",
     "OrderPreservedHierAllReducePlan", "order_preserved_hier_ar_emit", "order_preserved_hier_ar_check",
     "OrderPreservedHierReduceScatterPlan", "order_preserved_hier_rs_emit", "order_preserved_hier_rs_check",
@@ -531,6 +532,41 @@ class OrderPreservedPlan(Plan):
         p = _vp(0)
         check(_op_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
               "HcommGfxOrderPreservedPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_ops_emit = _sig("HcommGfxOrderPreservedSmallEmit", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_ops_check = _sig("HcommGfxOrderPreservedSmallCheck", _i32, _u32, _u64, _u64, C.c_int, C.POINTER(CheckReport))
+_ops_plan = _sig("HcommGfxOrderPreservedSmallPlanCreate", _i32, _u32, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _u64,
+                 _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def order_preserved_small_emit(n_ranks, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_ops_emit(n_ranks, count, ccl_bytes, dtype, None, 0, C.byref(n)), "HcommGfxOrderPreservedSmallEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_ops_emit(n_ranks, count, ccl_bytes, dtype, ops, n.value, C.byref(n)), "HcommGfxOrderPreservedSmallEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def order_preserved_small_check(n_ranks, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_ops_check(n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxOrderPreservedSmallCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class OrderPreservedSmallPlan(Plan):
+    """HcommGfxOrderPreservedSmallPlanCreate: the order-preserving reduce-scatter executor's small-message branch."""
+
+    def __init__(self, user_in, user_out, ccl_out, ccl_bytes, count, dtype, op):
+        n = len(user_in)
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_out)]
+        p = _vp(0)
+        check(_ops_plan(n, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op, C.byref(p)),
+              "HcommGfxOrderPreservedSmallPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

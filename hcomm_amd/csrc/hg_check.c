@@ -420,6 +420,19 @@ int32_t HcommGfxOrderPreservedHierReduceScatterCheck(
     return rc;
 }
 
+int32_t HcommGfxOrderPreservedSmallCheck(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* rep)
+{
+    if (!rep) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved_small(&l, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = HcommGfxOpListCheck(l.ops, l.n, nRanks, HCOMM_GFX_EXPECT_REDUCE_SCATTER_USER, count, 0,
+                             HcommGfxDataTypeSize(dataType), rep);
+    hg_oplist_free(&l);
+    return rc;
+}
+
 int32_t HcommGfxHierReduceScatterCheck(
     int32_t level0Mesh, HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
     HcommDataType dataType, HcommGfxCheckReport* rep)

@@ -74,6 +74,13 @@ static int step_is_conflict_free(const HgOp* o, uint64_t n)
 }
 
 /* bufs[role][rank]: the buffer behind each role an op list may name (HCOMM_GFX_NUM_BUFS roles) */
+/* 3 / 2: reduce on / off 16-byte boundaries, 1 / 0: copy on / off them - the kernels the coalescer tells apart */
+static int op_class(const HgOp* o)
+{
+    const int aligned = (((uintptr_t)o->dst | (uintptr_t)o->src) & (HG_VEC_BYTES - 1u)) == 0;
+    return (o->is_reduce ? 2 : 0) + aligned;
+}
+
 static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
                      int op)
 {
@@ -94,23 +101,25 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
         o->bytes = s->bytes;
     }
     /* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the
-     * next slice) would change kernel with every operation: when nothing in the step can observe anything else in it,
-     * run its reduces first and its copies after them, each kind in its original order. */
+     * next slice), or operations on 16-byte boundaries beside others that are not (blocks of odd sizes), would
+     * change kernel with every operation: when nothing in the step can observe anything else in it, run it class by
+     * class - reduces before copies, the 128-bit kernels before the element-wise one - each class in its original
+     * order. */
     for (uint64_t i = 0; i < n;) {
         uint64_t j = i;
-        uint64_t reduces = 0;
-        while (j < n && list[j].step == list[i].step) reduces += ops[j++].is_reduce;
+        uint32_t seen = 0;
+        while (j < n && list[j].step == list[i].step) seen |= 1u << op_class(&ops[j++]);
         /* the pairwise test is quadratic: steps larger than any schedule here produces keep their order */
-        if (reduces != 0 && reduces != j - i && j - i <= 4096 && step_is_conflict_free(ops + i, j - i)) {
+        if ((seen & (seen - 1u)) != 0 && j - i <= 4096 && step_is_conflict_free(ops + i, j - i)) {
             HgOp* tmp = (HgOp*)malloc((j - i) * sizeof(HgOp));
             if (!tmp) {
                 free(ops);
                 return HCCL_E_MEMORY;
             }
             uint64_t k = 0;
-            for (int want = 1; want >= 0; --want)
+            for (int want = 3; want >= 0; --want)
                 for (uint64_t q = i; q < j; ++q)
-                    if (ops[q].is_reduce == want) tmp[k++] = ops[q];
+                    if (op_class(&ops[q]) == want) tmp[k++] = ops[q];
             memcpy(ops + i, tmp, (j - i) * sizeof(HgOp));
             free(tmp);
         }
@@ -712,6 +721,28 @@ int32_t HcommGfxOrderPreservedHierAllReducePlanCreate(
     if (rc != HCCL_SUCCESS) return rc;
     void* const* bufs[HCOMM_GFX_NUM_BUFS] = {cclIn, cclOut, NULL, userIn, userOut};
     rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, n, bufs, dataType, reduceOp, plan);
+    hg_oplist_free(&ol);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedSmallPlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if (!userIn || !userOut || !cclOut) return HCCL_E_PTR;
+    if (nRanks != 4 && nRanks != 8) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(userIn, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(cclOut, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgOpList ol;
+    rc = hg_schedule_order_preserved_small(&ol, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {NULL, cclOut, NULL, userIn, userOut};
+    rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, nRanks, bufs, dataType, reduceOp, plan);
     hg_oplist_free(&ol);
     return rc;
 }

@@ -1421,6 +1421,68 @@ int32_t HcommGfxOrderPreservedEmit(
     return HCCL_SUCCESS;
 }
 
+/* ---- the order-preserving reduce-scatter executor's branch for small messages ----------------------------------- */
+
+/* ReduceScatterHDStage (alg_template/temp_reduce_scatter/reduce_scatter_hd_stage.cc:110-140, 154-185, 205-250), the
+ * branch CollReduceScatterOrderPreservedExecutor takes for at most 32 KiB per rank on one module of 4 or 8 devices in
+ * op-base mode (coll_reduce_scatter_order_preserved_executor.cc:29-38, 141-169).  With T one block in bytes and
+ * H = N / 2:
+ *   step 0: rank p copies the half of its user input that holds block p (H blocks) to the front of its CCL output;
+ *   step 1: rank p ^ H folds the same half of ITS user input into rank p's copy;
+ *   steps 2 ..: for w = H / 2, H / 4, .., 1 rank p folds rank p ^ w's run of w blocks - the run that holds block p,
+ *           at ((p / w) * w mod H) * T - into its own;
+ *   last step: block p, at (p mod H) * T, to the user output.
+ * The fold tree over rank order is the plant branch's; the two operands of a fold swap places from rank to rank. */
+static int order_preserved_small_build(HgOpList* l, uint32_t n, uint64_t total)
+{
+    const uint32_t half = n / 2;
+    uint32_t step = 0;
+    for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, OUT, 0, p, UIN, p >= half ? half * total : 0, half * total));
+    ++step;
+    for (uint32_t p = 0; p < n; ++p)
+        CHK(push(l, step, REDUCE, p, OUT, 0, p ^ half, UIN, p >= half ? half * total : 0, half * total));
+    ++step;
+    for (uint32_t w = half / 2; w >= 1; w /= 2, ++step)
+        for (uint32_t p = 0; p < n; ++p) {
+            const uint64_t off = (uint64_t)(p / w * w % half) * total;
+            CHK(push(l, step, REDUCE, p, OUT, off, p ^ w, OUT, off, w * total));
+        }
+    for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, 0, p, OUT, (uint64_t)(p % half) * total, total));
+    return HCCL_SUCCESS;
+}
+
+int hg_schedule_order_preserved_small(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || (n != 4 && n != 8)) return HCCL_E_PARA;
+    if (count * unit > 32u * 1024u) return HCCL_E_PARA; /* HCCL_SMALL_COUNT_32_KB, alg_template/template_v1_utils.h:64 */
+    /* the template takes the user input's block stride from the chunk (reduce_scatter_hd_stage.cc:156-160): the
+     * executor's loop must not cut the message */
+    if (count > ccl_bytes / n / 128u * 128u / unit) return HCCL_E_PARA;
+    if (count == 0) return HCCL_SUCCESS;
+    const int rc = order_preserved_small_build(l, n, count * unit);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxOrderPreservedSmallEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_order_preserved_small(&l, nRanks, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 /* ---- the order-preserving allreduce executor (one server, op-base mode) ------------------------------------------- */
 
 /* CollAllReduceOrderPreservedExecutor (coll_executor/coll_all_reduce/coll_all_reduce_order_preserved_executor.cc:

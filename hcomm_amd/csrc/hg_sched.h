@@ -30,6 +30,7 @@ int hg_schedule_dbring(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_loc
  * rank order, own slot to the user output; chunked like the reduce-scatter loop. */
 int hg_schedule_order_preserved(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 int hg_schedule_order_preserved_ar(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
+int hg_schedule_order_preserved_small(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
 int hg_schedule_order_preserved_rs2(HgOpList* l, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
                                     int dtype);
 int hg_schedule_order_preserved_ar2(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,

@@ -14,7 +14,8 @@
  *                                over N simulated ranks (N pairs of HBM buffers), with HcommGfxSchedule* to obtain
  *                                the operation lists and check them symbolically without a GPU;
  *   4. executor-level plans    - HcommGfxOpBase*, HcommGfxHier*, HcommGfxMeshHier*, HcommGfxHierReduceScatter*,
- *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedAllReduce*,
+ *                                HcommGfxDoubleRing*, HcommGfxOrderPreserved*, HcommGfxOrderPreservedSmall*,
+ *                                HcommGfxOrderPreservedAllReduce*,
  *                                HcommGfxOrderPreservedHierAllReduce*, HcommGfxOrderPreservedHierReduceScatter*,
  *                                HcommGfxOrderPreservedFused*: what the
  *                                reference's executors do around the templates (chunk loops through the CCL
@@ -709,8 +710,8 @@ int32_t HcommGfxHierReduceScatterCheck(
  * (so the result does not depend on which rank computes it), and copies its slot to its user output.
  * userIn: nRanks * count elements (block p at p * count); userOut: count elements; cclOut: cclBytes; 128-byte
  * aligned.  nRanks >= 2 (a single rank per module relies on the inter-module stage, which is not built); the
- * executor's recursive-halving branch for messages up to 32 KiB on 4 or 8 devices (:33-38) is not built either: this
- * entry point always takes the plant branch.  Step-wise lowering.
+ * executor's recursive-halving branch for messages up to 32 KiB on 4 or 8 devices (:33-38) is
+ * HcommGfxOrderPreservedSmallPlanCreate below: this entry point always takes the plant branch.  Step-wise lowering.
  */
 int32_t HcommGfxOrderPreservedPlanCreate(
     uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes, uint64_t count,
@@ -719,6 +720,26 @@ int32_t HcommGfxOrderPreservedEmit(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
     uint64_t* n);
 int32_t HcommGfxOrderPreservedCheck(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
+
+/*
+ * The branch the same executor takes for small messages (coll_reduce_scatter_order_preserved_executor.cc:29-38:
+ * count * unit <= 32 KiB, one module of 4 or 8 devices, op-base mode): ReduceScatterHDStage
+ * (alg_template/temp_reduce_scatter/reduce_scatter_hd_stage.cc) - every rank copies the half of its user input that
+ * holds its block to its CCL output buffer, the rank N / 2 away folds its own copy of that half in, then log2(N) - 1
+ * halving steps fold the partner's run of blocks, and block p goes to the user output: 2 + log2(N) operations per
+ * rank instead of the plant branch's 2 N.  The fold tree over rank order is the plant branch's, seen from rank p
+ * (every leaf XOR p: the two operands of a fold swap places from rank to rank).
+ * nRanks 4 or 8, count * unit <= 32 KiB, and the message must fit one chunk (count <= cclBytes / nRanks rounded down
+ * to 128 bytes / unit): HCCL_E_PARA otherwise.  Buffers as for HcommGfxOrderPreservedPlanCreate.
+ */
+int32_t HcommGfxOrderPreservedSmallPlanCreate(
+    uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes, uint64_t count,
+    HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+int32_t HcommGfxOrderPreservedSmallEmit(
+    uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap,
+    uint64_t* n);
+int32_t HcommGfxOrderPreservedSmallCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*

@@ -127,6 +127,10 @@ def lib():
         L.orc_run_order_preserved_rs2.restype = C.c_int
         L.orc_run_order_preserved_rs2.argtypes = [C.c_uint32, C.c_uint32] + [C.POINTER(C.c_void_p)] * 4 + \
             [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
+        L.orc_trace_order_preserved_small.restype = C.c_int64
+        L.orc_trace_order_preserved_small.argtypes = L.orc_trace_order_preserved.argtypes
+        L.orc_run_order_preserved_small.restype = C.c_int
+        L.orc_run_order_preserved_small.argtypes = L.orc_run_order_preserved.argtypes
         L.orc_trace_hier_rs.restype = C.c_int64
         L.orc_trace_hier_rs.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int,
                                         C.POINTER(OrcOp), C.c_uint64]
@@ -425,6 +429,24 @@ def run_order_preserved_rs2(n_servers, n_local, user_in, user_out, ccl_in, ccl_o
     rc = lib().orc_run_order_preserved_rs2(n_servers, n_local, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
     if rc:
         raise ValueError("orc_run_order_preserved_rs2 rc=%d" % rc)
+
+
+def trace_order_preserved_small(n, count, ccl_bytes, dtype):
+    """The order-preserving reduce-scatter executor's ReduceScatterHDStage branch (4 or 8 ranks, <= 32 KiB per rank)."""
+    total = lib().orc_trace_order_preserved_small(n, count, ccl_bytes, dtype, None, 0)
+    if total < 0:
+        raise ValueError("orc_trace_order_preserved_small rc=%d" % total)
+    ops = (OrcOp * max(total, 1))()
+    lib().orc_trace_order_preserved_small(n, count, ccl_bytes, dtype, ops, total)
+    return [ops[i].astuple() for i in range(total)]
+
+
+def run_order_preserved_small(user_in, user_out, ccl_in, ccl_out, count, ccl_bytes, dtype, op):
+    n = len(user_in)
+    arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in b]) for b in (user_in, user_out, ccl_in, ccl_out)]
+    rc = lib().orc_run_order_preserved_small(n, arrs[0], arrs[1], arrs[2], arrs[3], count, ccl_bytes, dtype, op)
+    if rc:
+        raise ValueError("orc_run_order_preserved_small rc=%d" % rc)
 
 
 # ---- the ring / mesh reduce-scatter executors over two communicator levels, op-base mode -----------------

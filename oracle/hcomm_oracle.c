@@ -60,6 +60,8 @@
  *                                     chunk / share table by hand; exact integer results over several chunks; pinned
  *   order-preserving reduce-scatter . the complete operation list N = 3, the rank-order fold trees N = 2..8 and a
  *                                     chunk table by hand; exact integer results over several chunks; pinned
+ *   order-preserving small-message branch . the complete operation list N = 4 by hand; per-rank trees N = 4, 8 (the
+ *                                     rank-order tree, leaves XOR p); exact integer results; pinned
  *   order-preserving allreduce ...... the complete operation list N = 3 (blocks of 256, 144 and 0 bytes, both borrowed
  *                                     slots), a chunk / block table N = 4 by hand; the same rank-order fold trees for
  *                                     every element N = 2..8; slot and borrowed-slot layout from the definition;
@@ -2261,6 +2263,96 @@ int orc_run_order_preserved(uint32_t n, void* const* user_in, void* const* user_
 {
     OrcTrace t;
     int rc = build_trace_order_preserved(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
+/* ---- the order-preserving reduce-scatter executor's branch for small messages (ReduceScatterHDStage) -------------- */
+
+/* ReduceScatterHDStage::RunAsync for one rank, tpl/temp_reduce_scatter/reduce_scatter_hd_stage.cc:72-108, as
+ * CollReduceScatterOrderPreservedExecutor::RunReduceScatterLevel0HD prepares it (exec/coll_reduce_scatter/
+ * coll_reduce_scatter_order_preserved_executor.cc:141-169: input memory = CCL input, output memory = the scratch
+ * memory = CCL output in op-base mode, user pointers through opInfo).  total = one block in bytes. */
+static void prog_rs_hd_stage(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t total)
+{
+    uint32_t power = 0;
+    while ((1u << (power + 1)) <= n) power++;
+    const uint32_t half = 1u << (power - 1);
+    /* PrepareSliceData, :110-140 */
+    OrcSlice slice_map[5][ORC_MAX_RANKS];
+    memset(slice_map, 0, sizeof(slice_map));
+    for (uint32_t round = 1; round <= power; round++) {
+        const uint32_t slice_num = n >> round;
+        uint32_t k = 0;
+        for (uint32_t group = 0; group < (1u << round); group++)
+            for (uint32_t c = 0; c < slice_num; c++) {
+                OrcSlice tmp;
+                tmp.size = total * slice_num;
+                const uint64_t offset = total * slice_num * group;
+                if (group == 0 || round == 1) tmp.offset = offset;
+                else tmp.offset = offset >= half * total ? offset - half * total : offset;
+                slice_map[round - 1][k++] = tmp;
+            }
+    }
+    const uint32_t n_steps = power;
+    /* RunReduceScatterStage1st, :154-185: the own half of the user input to the front of the CCL output buffer, the
+     * other half folded into the partner's */
+    emit(t, 0, K_COPY, rank, B_OUT, 0, rank, B_UIN, slice_map[0][rank].offset, slice_map[0][rank].size);
+    {
+        const uint32_t dst_rank = rank ^ (1u << (n_steps - 1));
+        emit(t, 1, K_REDUCE, dst_rank, B_OUT, 0, rank, B_UIN, slice_map[0][dst_rank].offset, slice_map[0][dst_rank].size);
+    }
+    /* RunReduceScatterRead, :205-250 */
+    for (uint32_t step = 1; step < n_steps; step++) {
+        const uint32_t dst_rank = rank ^ (1u << (n_steps - 1 - step));
+        emit(t, 1 + step, K_REDUCE, rank, B_OUT, slice_map[step][rank].offset, dst_rank, B_OUT, slice_map[step][rank].offset,
+             slice_map[step][rank].size);
+    }
+    emit(t, 1 + n_steps, K_COPY, rank, B_UOUT, 0, rank, B_OUT, slice_map[n_steps - 1][rank].offset, total);
+}
+
+/* CollReduceScatterOrderPreservedExecutor::KernelRun on its isUseHDAlg_ branch (exec/coll_reduce_scatter/
+ * coll_reduce_scatter_order_preserved_executor.cc:29-38, 182-183, 273: at most 32 KiB per rank, one module of 4 or 8
+ * devices, op-base mode; the template writes the user output itself).  The template takes the block stride of the
+ * user input from the chunk's count (reduce_scatter_hd_stage.cc:156-160), so the loop of
+ * coll_reduce_scatter_executor.cc:149-220 must not cut the message: refused otherwise. */
+static int build_trace_order_preserved_small(OrcTrace* t, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || (n != 4 && n != 8)) return -1;
+    if (count * unit > 32u * 1024u) return -1;                       /* HCCL_SMALL_COUNT_32_KB, tpl/template_v1_utils.h:64 */
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
+    if (count > max_count) return -1;
+    if (count == 0) return 0;
+    for (uint32_t r = 0; r < n; r++) prog_rs_hd_stage(t, r, n, count * unit);
+    if (t->oom) {
+        free(t->ops);
+        return -2;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_order_preserved_small(uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_small(&t, n, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_order_preserved_small(uint32_t n, void* const* user_in, void* const* user_out, void* const* ccl_in,
+                                  void* const* ccl_out, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_order_preserved_small(&t, n, count, ccl_bytes, dtype);
     if (rc) return rc;
     void* const* bufs[5] = {ccl_in, ccl_out, NULL, user_in, user_out};
     rc = exec_trace(&t, bufs, dtype, op);

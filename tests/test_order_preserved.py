@@ -91,3 +91,75 @@ def test_rejects_bad_arguments():
             f(4, 100, 500, oracle.F32)                   # no 128-byte slot per rank fits the CCL buffer
         with pytest.raises((ValueError, h.HcommError)):
             f(33, 100, 1 << 20, oracle.F32)
+
+
+# ---- the executor's branch for small messages: ReduceScatterHDStage on 4 or 8 ranks -----------------------------------
+
+SMALL = GOLD["small_message_branch"]
+
+
+def xor_leaves(tree, p):
+    return tree ^ p if isinstance(tree, int) else [xor_leaves(tree[0], p), xor_leaves(tree[1], p)]
+
+
+def test_small_branch_operation_list_hand_derived():
+    want = [tuple(o) for o in SMALL["ops_n4_fp32_count4"]]
+    assert oracle.trace_order_preserved_small(4, 4, 1 << 20, oracle.F32) == want
+    assert h.order_preserved_small_emit(4, 4, 1 << 20, oracle.F32) == want
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_small_branch_folds_along_the_rank_order_tree_seen_from_each_rank(op):
+    for n in (4, 8):
+        count = 1000
+        ins = order_sensitive_inputs(n, n * count, op, seed=1300 + n)
+        uin = [x.copy() for x in ins]
+        uout = [np.zeros(count, np.float32) for _ in range(n)]
+        ccl = 1 << 16
+        cin = [np.zeros(1, np.float32) for _ in range(n)]
+        cout = [np.zeros(ccl // 4, np.float32) for _ in range(n)]
+        oracle.run_order_preserved_small(uin, uout, cin, cout, count, ccl, oracle.F32, op)
+        for p in range(n):
+            want = eval_tree(xor_leaves(GOLD["rank_tree"][str(n)], p), [x[p * count:(p + 1) * count] for x in ins], op)
+            assert np.array_equal(uout[p].view(np.uint32), want.view(np.uint32)), (n, p)
+            assert np.array_equal(uin[p].view(np.uint32), ins[p].view(np.uint32))
+
+
+def test_small_branch_product_equals_oracle_and_passes_the_checker():
+    for n in (4, 8):
+        for count, dt in ((1, oracle.F32), (4, oracle.F32), (7, oracle.I8), (8192, oracle.F32), (16384, oracle.F16),
+                          (0, oracle.F32), (32768, oracle.I8), (333, oracle.I16)):
+            a = oracle.trace_order_preserved_small(n, count, 1 << 20, dt)
+            assert a == h.order_preserved_small_emit(n, count, 1 << 20, dt), (n, count)
+            assert h.order_preserved_small_check(n, count, 1 << 20, dt)[:2] == (0, 0), (n, count)
+            assert h.oplist_check(a, n, Expect.REDUCE_SCATTER_USER, count, h.DTYPE_SIZE[dt])[:2] == (0, 0)
+            assert len(a) == (0 if count == 0 else n * (2 + n.bit_length() - 1))
+            for o in a:
+                assert o[3] != UIN and o[6] != UOUT and o[4] + o[8] <= n // 2 * count * h.DTYPE_SIZE[dt] or o[3] == UOUT
+
+
+def test_small_branch_exact_integer_sums():
+    rng = np.random.default_rng(8)
+    for n in (4, 8):
+        for count in (1, 7, 100, 8192):
+            ins = [rng.integers(-1000, 1000, n * count, dtype=np.int32) for _ in range(n)]
+            uin = [x.copy() for x in ins]
+            uout = [np.full(count, -7, np.int32) for _ in range(n)]
+            ccl = n * 32768
+            cin = [np.full(1, -3, np.int32) for _ in range(n)]
+            cout = [np.full(ccl // 4 + 1, -5, np.int32) for _ in range(n)]
+            oracle.run_order_preserved_small(uin, uout, cin, cout, count, ccl, oracle.I32, oracle.SUM)
+            for r in range(n):
+                want = np.sum(np.stack([x[r * count:(r + 1) * count] for x in ins]).astype(np.int64), axis=0).astype(np.int32)
+                assert np.array_equal(uout[r], want), (n, count, r)
+                assert cout[r][-1] == -5 and np.array_equal(uin[r], ins[r])
+                assert np.all(cout[r][n // 2 * count:] == -5)                 # only the first half-message is used
+
+
+def test_small_branch_rejects_what_the_executor_does_not_route_to_it():
+    for f in (oracle.trace_order_preserved_small, h.order_preserved_small_emit):
+        for args in ((2, 100, 1 << 20, oracle.F32), (5, 100, 1 << 20, oracle.F32), (16, 100, 1 << 20, oracle.F32),
+                     (8, 8193, 1 << 20, oracle.F32),          # more than 32 KiB per rank
+                     (8, 1000, 8 * 3968, oracle.F32)):        # the loop would cut the message into chunks
+            with pytest.raises((ValueError, h.HcommError)):
+                f(*args)
