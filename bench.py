@@ -74,6 +74,9 @@ WORKLOADS = {
     "dbring_nhr_ar_bf16_2x8_128MiB": ("dbring_nhr", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving reduce-scatter executor: plant into the peers' CCL output buffers, fold in rank order
     "order_preserved_rs_bf16_n8_16MiB": ("order_preserved_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the same executor at 32 KiB per rank: its plant branch and the branch it takes there (ReduceScatterHDStage)
+    "order_preserved_rs_bf16_n8_32KiB": ("order_preserved_rs", 8, 16384, "bf16", "sum", "normal(0,1)*1e-3"),
+    "order_preserved_small_rs_bf16_n8_32KiB": ("order_preserved_small", 8, 16384, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving allreduce executor: plant with a borrowed slot, fold in rank order, mesh all-gather
     "order_preserved_ar_bf16_n8_128MiB": ("order_preserved_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the double-ring reduce-scatter executor on one server with DMA reduce
@@ -159,7 +162,8 @@ def main():
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     # one-server executors on user memory (DMA reduce)
-    plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar")
+    plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar", "order_preserved_small")
+    opsmall = alg_name == "order_preserved_small"
     opar = alg_name == "order_preserved_ar"
     # the order-preserving executors also have a single-launch lowering
     opfused = alg_name in ("order_preserved_ar", "order_preserved_rs") or ophier or ophrs
@@ -179,7 +183,8 @@ def main():
         return
 
     nbytes = count * unit
-    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs") or hier_rs or ophrs) else count
+    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs", "order_preserved_small")
+                            or hier_rs or ophrs) else count
     pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
     d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
@@ -216,6 +221,8 @@ def main():
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
         if opfused and low == h.Lowering.FUSED:  # one launch on the user buffers, no CCL buffer
             return h.OrderPreservedFusedPlan(opar or ophier, in_ptrs, out_ptrs, count, dt, op, n_servers=hier[0] if hier else 1)
+        if opsmall:
+            return h.OrderPreservedSmallPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
         if opar:
             return h.OrderPreservedAllReducePlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                                  [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op)
@@ -317,7 +324,8 @@ def main():
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
                 "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
-                "order_preserved_rs": None, "doublering_rs": None, "order_preserved_ar": None}[alg_name]
+                "order_preserved_rs": None, "doublering_rs": None, "order_preserved_ar": None,
+                "order_preserved_small": None}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
         host_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
@@ -329,6 +337,8 @@ def main():
                             for o in oracle.trace_hier_rs(oalg, hier[0], hier[1], count, ccl_bytes, odt, mesh=mesh0))
         elif dbrs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs(n, count, ccl_bytes, odt))
+        elif opsmall:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved_small(n, count, ccl_bytes, odt))
         elif opar:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_order_preserved_ar(n, count, ccl_bytes, odt))
         elif plant:
@@ -357,6 +367,8 @@ def main():
                                    mesh=mesh0)
             elif dbrs:
                 oracle.run_dbring_rs(ins, outs, host_ccl[0], count, ccl_bytes, odt, oop)
+            elif opsmall:
+                oracle.run_order_preserved_small(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif opar:
                 oracle.run_order_preserved_ar(ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop)
             elif plant:
