@@ -1,0 +1,170 @@
+/* Exercises every host-side generator, checker and plan builder of libhcomm_gfx on a recorder thread (no GPU): built
+ * with -fsanitize=address,undefined by tests/test_host_sanitizers.py together with the library's C files and
+ * stubs.c in place of the HIP layer.  Valid, boundary and invalid arguments alike; exit status 0 = every call that
+ * reported success produced a consistent plan / list. */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "hcomm_gfx.h"
+
+static void* bufs[5][32];
+static uint64_t plans, emits, checks, bad;
+
+static void run_plan(ThreadHandle th, HcommGfxPlan* p)
+{
+    if (!p) return;
+    ++plans;
+    HcommGfxPlanInfo info;
+    if (HcommGfxPlanGetInfo(p, &info)) ++bad;
+    for (uint32_t i = 0; i < info.launches; ++i) {
+        HcommGfxLaunchRecord r;
+        if (HcommGfxPlanGetLaunch(p, i, &r)) ++bad;
+    }
+    if (HcommGfxPlanRun(p, th)) ++bad;
+    if (info.launches > 1 && HcommGfxPlanRunRange(p, th, 1, info.launches - 1)) ++bad;
+    HcommGfxLaunchLogClear(th);
+    HcommGfxPlanDestroy(p);
+}
+
+static void emit_twice(int32_t (*f)(void*, HcommGfxSchedOp*, uint64_t, uint64_t*), void* ctx)
+{
+    uint64_t n = 0;
+    if (f(ctx, NULL, 0, &n)) return;
+    ++emits;
+    HcommGfxSchedOp* ops = (HcommGfxSchedOp*)malloc((n ? n : 1) * sizeof(*ops));
+    uint64_t m = 0;
+    f(ctx, ops, n / 2, &m); /* a short buffer must not be overrun */
+    f(ctx, ops, n, &m);
+    if (m != n) ++bad;
+    free(ops);
+}
+
+typedef struct { int a, b; uint32_t n, s, l; uint64_t count, ccl; int dt; } Ctx;
+static int32_t e_sched(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxScheduleEmitStrided(x->a, x->n, x->count, x->count + 3, x->dt, o, cap, n); }
+static int32_t e_opbase(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOpBaseEmit(x->a, x->n, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_hier(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return x->b ? HcommGfxMeshHierEmit(x->a, x->s, x->l, x->count, x->dt, o, cap, n) : HcommGfxHierEmit(x->a, x->s, x->l, x->count, x->dt, o, cap, n); }
+static int32_t e_dbring(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingEmit(x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_dbrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingReduceScatterEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_hrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxHierReduceScatterEmit(x->b, x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_oph(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedHierAllReduceEmit(x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_ops(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedSmallEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_ophrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedHierReduceScatterEmit(x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_op(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_opar(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedAllReduceEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
+
+int main(void)
+{
+    for (int k = 0; k < 5; ++k)
+        for (int r = 0; r < 32; ++r) bufs[k][r] = (void*)(uintptr_t)(0x7f0000000000ull + ((uint64_t)(k * 32 + r) << 32));
+    ThreadHandle th;
+    if (HcommGfxRecorderThreadAlloc(&th)) return 2;
+    const uint64_t counts[] = {0, 1, 100, 4097};
+    const uint32_t ns[] = {0, 1, 2, 3, 4, 5, 8, 17, 32, 33};
+    const uint32_t sl[] = {0, 1, 2, 3, 5, 8};
+    const uint64_t ccls[] = {128, 4096, 1 << 20};
+    const int dts[] = {HCOMM_DATA_TYPE_INT8, HCOMM_DATA_TYPE_BFP16, 99};
+    HcommGfxCheckReport rep;
+    HcommGfxPlan* p;
+    for (unsigned ni = 0; ni < 10; ++ni)
+        for (unsigned ci = 0; ci < 4; ++ci)
+            for (unsigned di = 0; di < 3; ++di) {
+                const uint32_t n = ns[ni];
+                Ctx x = {0, 0, n, 0, 0, counts[ci], 0, dts[di]};
+                for (int alg = -1; alg <= 17; ++alg) {
+                    x.a = alg;
+                    emit_twice(e_sched, &x);
+                    if (HcommGfxScheduleCheck(alg, n, x.count, 0, x.dt, &rep) == 0) ++checks;
+                    for (int low = 0; low < 2; ++low) {
+                        p = NULL;
+                        HcommGfxPlanCreateEx(alg, low, n, bufs[0], bufs[1], bufs[2], x.count, 0, x.dt, HCOMM_REDUCE_SUM, &p);
+                        run_plan(th, p);
+                    }
+                    for (unsigned cc = 0; cc < 3; ++cc) {
+                        x.ccl = ccls[cc];
+                        if (n % 4 == 1 || n == 8) {
+                            emit_twice(e_opbase, &x);
+                            if (HcommGfxOpBaseCheck(alg, n, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                            for (int low = 0; low < 2; ++low) {
+                                p = NULL;
+                                HcommGfxOpBasePlanCreate(alg, low, n, bufs[3], bufs[4], bufs[0], bufs[1], bufs[2], x.ccl, x.count, x.dt, HCOMM_REDUCE_MAX, &p);
+                                run_plan(th, p);
+                            }
+                        }
+                    }
+                }
+                for (unsigned cc = 0; cc < 3; ++cc) {
+                    x.ccl = ccls[cc];
+                    emit_twice(e_dbrs, &x);
+                    emit_twice(e_op, &x);
+                    emit_twice(e_ops, &x);
+                    if (HcommGfxOrderPreservedSmallCheck(n, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                    p = NULL; HcommGfxOrderPreservedSmallPlanCreate(n, bufs[3], bufs[4], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_MAX, &p); run_plan(th, p);
+                    emit_twice(e_opar, &x);
+                    if (HcommGfxDoubleRingReduceScatterCheck(n, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                    if (HcommGfxOrderPreservedCheck(n, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                    if (HcommGfxOrderPreservedAllReduceCheck(n, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                    p = NULL; HcommGfxDoubleRingReduceScatterPlanCreate(n, bufs[3], bufs[4], bufs[0], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                    p = NULL; HcommGfxOrderPreservedPlanCreate(n, bufs[3], bufs[4], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_MIN, &p); run_plan(th, p);
+                    p = NULL; HcommGfxOrderPreservedAllReducePlanCreate(n, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                }
+                for (int ar = 0; ar < 2; ++ar) { p = NULL; HcommGfxOrderPreservedFusedPlanCreate(ar, 1, n, bufs[3], bufs[4], x.count, x.dt, HCOMM_REDUCE_PROD, &p); run_plan(th, p); }
+            }
+    /* two-level executors */
+    for (unsigned si = 0; si < 5; ++si)
+        for (unsigned li = 0; li < 5; ++li)
+            for (unsigned ci = 0; ci < 4; ++ci)
+                for (int alg = -1; alg <= 17; ++alg)
+                    for (int mesh = 0; mesh < 2; ++mesh) {
+                        const uint32_t s = sl[si], l = sl[li];
+                        Ctx x = {alg, mesh, s * l, s, l, counts[ci], 0, HCOMM_DATA_TYPE_FP16};
+                        emit_twice(e_hier, &x);
+                        if ((mesh ? HcommGfxMeshHierCheck : HcommGfxHierCheck)(alg, s, l, x.count, x.dt, &rep) == 0) ++checks;
+                        p = NULL;
+                        (mesh ? HcommGfxMeshHierPlanCreate : HcommGfxHierPlanCreate)(alg, s, l, bufs[0], bufs[1], x.count, x.dt, HCOMM_REDUCE_SUM, &p);
+                        run_plan(th, p);
+                        for (unsigned cc = 0; cc < 3; ++cc) {
+                            x.ccl = ccls[cc];
+                            if (x.ccl < 4096 && x.count > 1000) continue;
+                            emit_twice(e_hrs, &x);
+                            if (HcommGfxHierReduceScatterCheck(mesh, alg, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                            p = NULL;
+                            HcommGfxHierReduceScatterPlanCreate(mesh, alg, s, l, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p);
+                            run_plan(th, p);
+                            if (!mesh) {
+                                emit_twice(e_oph, &x);
+                                if (alg == 0) {
+                                    emit_twice(e_ophrs, &x);
+                                    if (HcommGfxOrderPreservedHierReduceScatterCheck(s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                                    p = NULL; HcommGfxOrderPreservedHierReduceScatterPlanCreate(s, l, bufs[3], bufs[4], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                                    for (int ar = 0; ar < 2; ++ar) { p = NULL; HcommGfxOrderPreservedFusedPlanCreate(ar, s, l, bufs[3], bufs[4], x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p); }
+                                }
+                                if (HcommGfxOrderPreservedHierAllReduceCheck(alg, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                                p = NULL;
+                                HcommGfxOrderPreservedHierAllReducePlanCreate(alg, s, l, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p);
+                                run_plan(th, p);
+                                emit_twice(e_dbring, &x);
+                                if (HcommGfxDoubleRingCheck(alg, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                                p = NULL;
+                                HcommGfxDoubleRingPlanCreate(alg, s, l, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p);
+                                run_plan(th, p);
+                            }
+                        }
+                    }
+    /* malformed op lists */
+    HcommGfxSchedOp ops[4];
+    memset(ops, 0, sizeof(ops));
+    ops[0].bytes = 16; ops[1].bytes = 16; ops[1].rank = 40; ops[2].dstBuf = 9; ops[3].step = 0;
+    void* const* bb[5] = {bufs[0], bufs[1], bufs[2], bufs[3], bufs[4]};
+    for (uint64_t k = 0; k <= 4; ++k) {
+        p = NULL;
+        HcommGfxPlanCreateFromOps(ops, k, 2, bb, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM, &p);
+        run_plan(th, p);
+        HcommGfxOpListCheck(ops, k, 2, HCOMM_GFX_EXPECT_ALLREDUCE, 4, 0, 4, &rep);
+    }
+    HcommGfxSlice slc[32];
+    for (uint32_t n = 0; n <= 32; ++n) HcommGfxCalcSlices(100003, 2, n, slc);
+    HcommThreadFree(&th, 1);
+    printf("plans %llu emits %llu checks %llu bad %llu\n", (unsigned long long)plans, (unsigned long long)emits,
+           (unsigned long long)checks, (unsigned long long)bad);
+    return bad ? 1 : 0;
+}
