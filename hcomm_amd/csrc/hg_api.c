@@ -19,13 +19,17 @@ _Static_assert(sizeof(HcommBatchTransferDesc) == 64, "HcommBatchTransferDesc mus
 
 static int g_allow_prod = -1;
 
+/* Settings read from the environment on first use: several host threads may get there at once, every one of them
+ * computes the same value, and the relaxed atomics keep that a defined program. */
 static int allow_prod(void)
 {
-    if (g_allow_prod < 0) {
+    int v = __atomic_load_n(&g_allow_prod, __ATOMIC_RELAXED);
+    if (v < 0) {
         const char* e = getenv("HCOMM_GFX_ALLOW_PROD");
-        g_allow_prod = (e && e[0] == '1') ? 1 : 0;
+        v = (e && e[0] == '1') ? 1 : 0;
+        __atomic_store_n(&g_allow_prod, v, __ATOMIC_RELAXED);
     }
-    return g_allow_prod;
+    return v;
 }
 
 /* thread_local launch context of the calling host thread (cpu_primitives_c_adpt.cc:27) */

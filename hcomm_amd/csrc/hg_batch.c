@@ -13,19 +13,27 @@
 
 #include "hg_host.h"
 
-static uint64_t g_grid_cap = 0;
-static int g_grid_forced = 0;
+/* Settings read from the environment on first use, possibly by several host threads at once: each computes the same
+ * value; relaxed atomics keep that defined.  0 = not read yet. */
+static uint64_t g_grid_cap = 0; /* UINT64_MAX = not set */
 static uint64_t g_small_bytes = 0;
+
+static uint64_t env_once(uint64_t* slot, const char* name, uint64_t unset)
+{
+    uint64_t v = __atomic_load_n(slot, __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv(name);
+        v = e ? strtoull(e, NULL, 10) : 0;
+        if (v == 0) v = unset;
+        __atomic_store_n(slot, v, __ATOMIC_RELAXED);
+    }
+    return v;
+}
 
 uint64_t hg_grid_blocks(uint64_t total_tiles, int capped)
 {
-    if (g_grid_cap == 0) {
-        const char* e = getenv("HCOMM_GFX_GRID_CAP");
-        g_grid_cap = e ? strtoull(e, NULL, 10) : 0;
-        if (g_grid_cap == 0) g_grid_cap = UINT64_MAX; /* not set */
-        else g_grid_forced = 1;
-    }
-    if (g_grid_forced) return total_tiles < g_grid_cap ? total_tiles : g_grid_cap; /* experiments: every kernel */
+    const uint64_t forced = env_once(&g_grid_cap, "HCOMM_GFX_GRID_CAP", UINT64_MAX);
+    if (forced != UINT64_MAX) return total_tiles < forced ? total_tiles : forced; /* experiments: every kernel */
     /* Measured over the benchmark configurations: one tile per workgroup, however many that makes, streams best for
      * the copy and the k-way fold kernels (a 2 GiB copy: 5.84 against 5.38 TB/s with the grid held at 32 workgroups
      * per CU; the fused 16-rank tree: 0.95 against 1.05 ms).  The two-input reduce is the exception: on the ragged
@@ -68,17 +76,13 @@ void hg_finish_fold(HgLaunch* l)
     uint64_t tiles = 0, bytes = 0;
     if (!t->tree) {
         /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
-        if (g_small_bytes == 0) {
-            const char* e = getenv("HCOMM_GFX_SMALL_BYTES");
-            g_small_bytes = e ? strtoull(e, NULL, 10) : 0;
-            if (g_small_bytes == 0) g_small_bytes = 1u << 20;
-        }
+        const uint64_t small_bytes = env_once(&g_small_bytes, "HCOMM_GFX_SMALL_BYTES", 1u << 20);
         uint64_t largest = 0;
         for (uint32_t s = 0; s < t->nseg; ++s)
             if (t->bytes[s] > largest) largest = t->bytes[s];
         /* measured cross-over with 8 ranks: 1 MiB per segment for read-only chains (mesh, k-way reduce), a
          * quarter of that when every position also stores its partial (ring) */
-        const uint64_t limit = t->store_partials ? g_small_bytes / 4 : g_small_bytes;
+        const uint64_t limit = t->store_partials ? small_bytes / 4 : small_bytes;
         t->small = (largest <= limit) ? 1u : 0u;
     }
     const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_TILE_BYTES);
@@ -165,11 +169,13 @@ typedef struct {
 static uint64_t copy_launch_bytes(void)
 {
     static uint64_t cap = 0;
-    if (cap == 0) {
+    uint64_t v = __atomic_load_n(&cap, __ATOMIC_RELAXED);
+    if (v == 0) {
         const char* e = getenv("HCOMM_GFX_COPY_LAUNCH_MIB"); /* experiments; 0 = no limit */
-        cap = e ? (strtoull(e, NULL, 10) ? strtoull(e, NULL, 10) << 20 : UINT64_MAX) : HG_COPY_LAUNCH_BYTES;
+        v = e ? (strtoull(e, NULL, 10) ? strtoull(e, NULL, 10) << 20 : UINT64_MAX) : HG_COPY_LAUNCH_BYTES;
+        __atomic_store_n(&cap, v, __ATOMIC_RELAXED);
     }
-    return cap;
+    return v;
 }
 
 /* segments a copy / two-input reduce launch may carry: the table's size, or less when HCOMM_GFX_MAX_SEGMENTS says so
@@ -177,12 +183,14 @@ static uint64_t copy_launch_bytes(void)
 static uint32_t seg2_cap(void)
 {
     static uint32_t cap = 0;
-    if (cap == 0) {
+    uint32_t c = __atomic_load_n(&cap, __ATOMIC_RELAXED);
+    if (c == 0) {
         const char* e = getenv("HCOMM_GFX_MAX_SEGMENTS");
         const unsigned long v = e ? strtoul(e, NULL, 10) : 0;
-        cap = (v >= 1 && v <= HG_MAX_SEG2) ? (uint32_t)v : HG_MAX_SEG2;
+        c = (v >= 1 && v <= HG_MAX_SEG2) ? (uint32_t)v : HG_MAX_SEG2;
+        __atomic_store_n(&cap, c, __ATOMIC_RELAXED);
     }
-    return cap;
+    return c;
 }
 
 static int coalesce_one(Coalescer* c, const HgOp* o)

@@ -31,13 +31,15 @@ static int g_use_graph = -1;
 
 static int use_graph(void)
 {
-    if (g_use_graph < 0) {
+    int v = __atomic_load_n(&g_use_graph, __ATOMIC_RELAXED); /* first use may come from several host threads */
+    if (v < 0) {
         const char* e = getenv("HCOMM_GFX_GRAPH");
         /* measured on ROCm 7: replaying 15 small kernels as a graph takes 60 us against 54 us launched one by
          * one, so graph replay is opt-in */
-        g_use_graph = (e && e[0] == '1') ? 1 : 0;
+        v = (e && e[0] == '1') ? 1 : 0;
+        __atomic_store_n(&g_use_graph, v, __ATOMIC_RELAXED);
     }
-    return g_use_graph;
+    return v;
 }
 
 static int plan_push(const HgLaunch* l, void* ctx)

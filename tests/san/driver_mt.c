@@ -1,0 +1,57 @@
+/* Eight host threads use the library at once, each with recorder threads of its own: thread registry, batch mode
+ * (per host thread), plan building and replay, launch logs.  Built with -fsanitize=thread by
+ * tests/test_host_sanitizers.py; exit status 0 = every call returned what a single-threaded run returns. */
+#include <pthread.h>
+#include <stdio.h>
+#include <stdint.h>
+#include "hcomm_gfx.h"
+
+static void* worker(void* arg)
+{
+    const uintptr_t id = (uintptr_t)arg;
+    uintptr_t bad = 0;
+    void* bufs[3][8];
+    for (int k = 0; k < 3; ++k)
+        for (int r = 0; r < 8; ++r) bufs[k][r] = (void*)(uintptr_t)(0x7f0000000000ull + ((id * 64 + (uint64_t)k * 8 + r) << 32));
+    for (int it = 0; it < 1000; ++it) {
+        ThreadHandle th[2];
+        if (HcommGfxRecorderThreadAlloc(&th[0]) || HcommGfxRecorderThreadAlloc(&th[1])) { ++bad; continue; }
+        char tag[32];
+        snprintf(tag, sizeof(tag), "w%u_%d", (unsigned)id, it);
+        bad += HcommBatchModeStart(tag) != 0;
+        for (int r = 0; r < 8; ++r) {
+            bad += HcommLocalCopyOnThread(th[0], bufs[1][r], bufs[0][r], 4096) != 0;
+            bad += HcommLocalReduceOnThread(th[0], bufs[1][r], bufs[0][(r + 1) % 8], 1024, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM) != 0;
+        }
+        bad += HcommBatchModeEnd(tag) != 0;
+        HcommGfxLaunchRecord rec[8];
+        uint32_t n = 0;
+        bad += HcommGfxLaunchLogRead(th[0], rec, 8, &n) != 0 || n == 0;
+        HcommGfxPlan* p = NULL;
+        bad += HcommGfxPlanCreate((HcommGfxAlgorithm)(it % 3), HCOMM_GFX_LOWER_STEPWISE, 8, bufs[0], bufs[1], 100003 + it,
+                                  HCOMM_DATA_TYPE_BFP16, HCOMM_REDUCE_MAX, &p) != 0;
+        if (p) {
+            bad += HcommGfxPlanRun(p, th[1]) != 0;
+            bad += HcommGfxPlanDestroy(p) != 0;
+        }
+        bad += HcommGfxLaunchLogRead(th[1], rec, 8, &n) != 0 || n == 0;
+        bad += HcommThreadFree(th, 2) != 0;
+        bad += HcommLocalCopyOnThread(th[0], bufs[1][0], bufs[0][0], 16) == 0; /* a freed handle is refused */
+    }
+    return (void*)bad;
+}
+
+int main(void)
+{
+    pthread_t t[8];
+    uintptr_t bad = 0;
+    for (uintptr_t i = 0; i < 8; ++i)
+        if (pthread_create(&t[i], NULL, worker, (void*)i)) return 2;
+    for (int i = 0; i < 8; ++i) {
+        void* r = NULL;
+        pthread_join(t[i], &r);
+        bad += (uintptr_t)r;
+    }
+    printf("threads 8 bad %lu\n", (unsigned long)bad);
+    return bad ? 1 : 0;
+}

@@ -29,3 +29,21 @@ def test_host_code_is_clean_under_asan_and_ubsan(tmp_path):
     assert " bad 0" in run.stdout and "ERROR" not in run.stderr and "runtime error" not in run.stderr
     plans = int(run.stdout.split("plans")[1].split()[0])
     assert plans > 5000                                              # the walk did reach the plan builders
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no gcc")
+def test_host_code_is_clean_under_tsan_with_eight_host_threads(tmp_path):
+    exe = str(tmp_path / "san_mt")
+    cmd = ["gcc", "-O1", "-g", "-std=c11", "-fsanitize=thread", "-fno-omit-frame-pointer",
+           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    cmd += [os.path.join(CSRC, f) for f in ("hg_api.c", "hg_batch.c", "hg_sched.c", "hg_plan.c", "hg_check.c")]
+    cmd += [os.path.join(SAN, "stubs.c"), os.path.join(SAN, "driver_mt.c"), "-o", exe, "-lpthread", "-lm"]
+    build = subprocess.run(cmd, capture_output=True, text=True)
+    if build.returncode != 0 and "cannot find" in build.stderr:
+        pytest.skip("the sanitizer runtime is not installed")
+    assert build.returncode == 0, build.stderr[-2000:]
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    if "unexpected memory mapping" in run.stderr:                    # ThreadSanitizer cannot place its shadow here
+        pytest.skip("ThreadSanitizer does not run in this environment")
+    assert run.returncode == 0, (run.stdout[-1000:], run.stderr[-3000:])
+    assert "threads 8 bad 0" in run.stdout and "ThreadSanitizer" not in run.stderr
