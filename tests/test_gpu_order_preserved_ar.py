@@ -86,10 +86,10 @@ def test_randomized_shapes(gpu_thread):
 
 # ---- the single-launch lowering: the same user outputs from one kernel that only reads the user inputs ---------------
 
-def run_fused(thread, all_reduce, n, count, dtype, op, seed=0):
+def run_fused(thread, all_reduce, n, count, dtype, op, seed=0, kind=None):
     dt, o = DT[dtype], OPS[op]
     in_count = count if all_reduce else n * count
-    host_in = [gen(dt, in_count, 13000 + seed * 100 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    host_in = [gen(dt, in_count, 13000 + seed * 100 + r, kind or ("prod" if op == "prod" else "default")) for r in range(n)]
     sentinel = gen(dt, count, 997, "wide")
     unit = h.DTYPE_SIZE[dt]
     ccl = max(4096, -(-count * unit * n // 128) * 128)            # one chunk or several: the result does not depend on it
@@ -155,3 +155,13 @@ def test_single_launch_lowering_randomized(gpu_thread):
         op = ["sum", "max", "min"][rng.integers(3)]
         say("random order preserved fused", i, all_reduce, n, count, dtype, op)
         run_fused(gpu_thread, all_reduce, n, count, dtype, op, seed=i)
+
+
+@pytest.mark.parametrize("dtype,op", [("fp16", "sum"), ("fp16", "max"), ("fp16", "min"), ("fp16", "prod"), ("bf16", "sum"),
+                                      ("bf16", "max"), ("bf16", "min"), ("fp32", "max"), ("fp32", "sum")])
+def test_single_launch_lowering_on_every_bit_pattern(gpu_thread, dtype, op):
+    """NaNs, infinities, signed zeros and denormals: MAX / MIN keep the operand in the dst role on a tie or a NaN, so
+    this also pins which side of every fold of the tree is which."""
+    for all_reduce, n, count in ((1, 8, 70000), (1, 5, 70001), (0, 8, 8192), (0, 3, 4096)):
+        say("order preserved fused, wide values", all_reduce, n, count, dtype, op)
+        run_fused(gpu_thread, all_reduce, n, count, dtype, op, seed=77, kind="wide")

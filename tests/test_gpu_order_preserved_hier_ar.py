@@ -92,10 +92,10 @@ def test_randomized_shapes(gpu_thread):
 
 # ---- the single-launch lowering over servers x devices: the same user outputs from one kernel ------------------------
 
-def run_fused(thread, all_reduce, m, l, count, dtype, op, seed=0):
+def run_fused(thread, all_reduce, m, l, count, dtype, op, seed=0, kind=None):
     dt, o, n = DT[dtype], OPS[op], m * l
     in_count = count if all_reduce else n * count
-    host_in = [gen(dt, in_count, 16000 + seed * 100 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    host_in = [gen(dt, in_count, 16000 + seed * 100 + r, kind or ("prod" if op == "prod" else "default")) for r in range(n)]
     sentinel = gen(dt, count, 994, "wide")
     unit = h.DTYPE_SIZE[dt]
     ccl = max(1 << 17, -(-count * unit * n // 128) * 128)
@@ -163,3 +163,13 @@ def test_single_launch_lowering_randomized(gpu_thread):
         say("random order preserved two-level fused", done, all_reduce, m, l, count, dtype, op)
         run_fused(gpu_thread, all_reduce, m, l, count, dtype, op, seed=done)
         done += 1
+
+
+@pytest.mark.parametrize("dtype,op", [("fp16", "sum"), ("fp16", "max"), ("fp16", "min"), ("bf16", "sum"), ("bf16", "max"),
+                                      ("bf16", "min"), ("fp32", "min")])
+def test_single_launch_lowering_on_every_bit_pattern(gpu_thread, dtype, op):
+    """NaNs, infinities, signed zeros and denormals through both levels of the tree: MAX / MIN keep the operand in the
+    dst role on a tie or a NaN, which pins the side of every fold."""
+    for all_reduce, m, l, count in ((1, 2, 8, 70000), (1, 3, 5, 30001), (0, 4, 4, 4096), (0, 2, 3, 8192)):
+        say("order preserved two-level fused, wide values", all_reduce, m, l, count, dtype, op)
+        run_fused(gpu_thread, all_reduce, m, l, count, dtype, op, seed=78, kind="wide")
