@@ -655,7 +655,7 @@ _ophrs_emit = _sig("HcommGfxOrderPreservedHierReduceScatterEmit", _i32, _u32, _u
 _ophrs_check = _sig("HcommGfxOrderPreservedHierReduceScatterCheck", _i32, _u32, _u32, _u64, _u64, C.c_int,
                     C.POINTER(CheckReport))
 _ophrs_plan = _sig("HcommGfxOrderPreservedHierReduceScatterPlanCreate", _i32, _u32, _u32, C.POINTER(_vp), C.POINTER(_vp),
-                   C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+                   C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
 
 
 def order_preserved_hier_rs_emit(n_servers, n_local, count, ccl_bytes, dtype):
@@ -678,13 +678,15 @@ def order_preserved_hier_rs_check(n_servers, n_local, count, ccl_bytes, dtype):
 class OrderPreservedHierReduceScatterPlan(Plan):
     """HcommGfxOrderPreservedHierReduceScatterPlanCreate: the order-preserving reduce-scatter executor over two levels."""
 
-    def __init__(self, n_servers, n_local, user_in, user_out, ccl_out, ccl_bytes, count, dtype, op):
+    def __init__(self, n_servers, n_local, user_in, user_out, ccl_out, ccl_bytes, count, dtype, op, ccl_in=None):
+        """ccl_in is only needed (and used) with one device per server."""
         n = n_servers * n_local
         assert len(user_in) == n
         self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_out)]
+        self._cin = (_vp * n)(*ccl_in) if ccl_in is not None else None
         p = _vp(0)
-        check(_ophrs_plan(n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype, op,
-                          C.byref(p)), "HcommGfxOrderPreservedHierReduceScatterPlanCreate")
+        check(_ophrs_plan(n_servers, n_local, self._bufs[0], self._bufs[1], self._cin, self._bufs[2], ccl_bytes, count,
+                          dtype, op, C.byref(p)), "HcommGfxOrderPreservedHierReduceScatterPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -710,7 +710,7 @@ int32_t HcommGfxOrderPreservedHierAllReducePlanCreate(
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
     if (!userIn || !userOut || !cclIn || !cclOut) return HCCL_E_PTR;
-    if (nServers < 2 || nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (nServers < 2 || nLocal < 1 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
     const uint32_t n = nServers * nLocal;
     int rc = check_bufs(userIn, n);
@@ -750,23 +750,24 @@ int32_t HcommGfxOrderPreservedSmallPlanCreate(
 }
 
 int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
-    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes,
-    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
+    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclIn, void* const* cclOut,
+    uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan)
 {
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
     if (!userIn || !userOut || !cclOut) return HCCL_E_PTR;
-    if (nServers < 2 || nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (nServers < 2 || nLocal < 1 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
     const uint32_t n = nServers * nLocal;
     int rc = check_bufs(userIn, n);
     if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, n);
     if (rc == HCCL_SUCCESS) rc = check_bufs(cclOut, n);
+    if (rc == HCCL_SUCCESS && nLocal == 1) rc = check_bufs(cclIn, n); /* only one device per module stages there */
     if (rc != HCCL_SUCCESS) return rc;
     HgOpList ol;
     rc = hg_schedule_order_preserved_rs2(&ol, nServers, nLocal, count, cclBytes, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
-    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {NULL, cclOut, NULL, userIn, userOut};
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {nLocal == 1 ? cclIn : NULL, cclOut, NULL, userIn, userOut};
     rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, n, bufs, dataType, reduceOp, plan);
     hg_oplist_free(&ol);
     return rc;
@@ -792,7 +793,8 @@ int32_t HcommGfxOrderPreservedFusedPlanCreate(
 {
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
-    if (nServers == 0 || nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (nServers == 0 || nLocal == 0 || (uint64_t)nServers * nLocal < 2 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS)
+        return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
     const uint32_t nRanks = nServers * nLocal;
     int rc = check_bufs(userIn, nRanks);

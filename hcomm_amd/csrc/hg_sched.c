@@ -1577,8 +1577,13 @@ static int order_preserved_ar2_build(HgOpList* l, int alg1, uint32_t n_srv, uint
         const uint64_t blk = ((cur + n - 1) / n * unit + 127u) / 128u * 128u;
         for (uint32_t b = 0; b < n; ++b) size[b] = (uint64_t)b * blk >= c ? 0 : (c - b * blk < blk ? c - b * blk : blk);
 #define SRV(s, i) ((s) * n_loc + (i))
+        const int single = n_loc == 1; /* one device per module: level 0 is a copy of the chunk into the CCL input buffer */
+        if (single) {
+            for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, IN, 0, p, UIN, user_off, c));
+            ++step;
+        }
         /* level 0: plants */
-        for (uint32_t s = 0; s < n_srv; ++s)
+        for (uint32_t s = 0; s < n_srv && !single; ++s)
             for (uint32_t i = 0; i < n_loc; ++i)     /* destination device */
                 for (uint32_t q = 0; q < n_loc; ++q) /* planting device; per planter the groups in order */
                     for (uint32_t g = 0; g < n_srv; ++g) {
@@ -1589,9 +1594,9 @@ static int order_preserved_ar2_build(HgOpList* l, int alg1, uint32_t n_srv, uint
                             CHK(push(l, step, COPY, SRV(s, i), OUT, blk * (g * n_loc + slot), SRV(s, q), UIN,
                                      user_off + blk * b, size[b]));
                     }
-        ++step;
+        if (!single) ++step;
         /* level 0: folds in device order; contribution k of device i sits in slot (1 + k + i) mod L */
-        for (uint32_t h = 1u << (r0 - 1); h >= 1; h >>= 1, ++step)
+        for (uint32_t h = single ? 0 : 1u << (r0 - 1); h >= 1; h >>= 1, ++step)
             for (uint32_t s = 0; s < n_srv; ++s)
                 for (uint32_t i = 0; i < n_loc; ++i)
                     for (uint32_t g = 0; g < n_srv; ++g) {
@@ -1604,20 +1609,26 @@ static int order_preserved_ar2_build(HgOpList* l, int alg1, uint32_t n_srv, uint
                                      SRV(s, i), from_in ? IN : OUT, from_in ? blk * b : blk * (g * n_loc + from), size[b]));
                         }
                     }
-        /* level 1: device i of server c hands its partial for block i + d * L to server d; the own one first */
+        /* level 1: device i of server c hands its partial for block i + d * L to server d.  With one device per module
+         * the partials are the blocks of the chunk in the CCL input buffer, a block that would go to the borrowed place
+         * of its own rank is there already, and the peers' plants come a step after the own ones: one of them may land
+         * where the own block was read from */
         for (uint32_t d = 0; d < n_srv; ++d)
             for (uint32_t i = 0; i < n_loc; ++i)
                 for (uint32_t c0 = 0; c0 < n_srv; ++c0) {
                     const uint32_t b = i + d * n_loc, slot = (c0 + d) % n_srv;
-                    const int src_in = i + 2 == n_loc; /* the level-0 partial sits in the borrowed place */
+                    const int src_in = single || i + 2 == n_loc; /* the level-0 partial sits in the borrowed place */
                     const uint64_t src_off = src_in ? blk * (i + d * n_loc) : blk * ((1 + i) % n_loc + d * n_loc);
-                    if (i == last_loc && slot == last_srv && d != last_srv)
-                        CHK(push(l, step, COPY, SRV(d, i), IN, blk * b, SRV(c0, i), src_in ? IN : OUT, src_off, size[b]));
-                    else
-                        CHK(push(l, step, COPY, SRV(d, i), OUT, blk * (i + slot * n_loc), SRV(c0, i), src_in ? IN : OUT, src_off,
+                    const uint32_t at = step + (single && c0 != d ? 1u : 0u);
+                    if (i == last_loc && slot == last_srv && d != last_srv) {
+                        if (!(single && c0 == d))
+                            CHK(push(l, at, COPY, SRV(d, i), IN, blk * b, SRV(c0, i), src_in ? IN : OUT, src_off, size[b]));
+                    } else {
+                        CHK(push(l, at, COPY, SRV(d, i), OUT, blk * (i + slot * n_loc), SRV(c0, i), src_in ? IN : OUT, src_off,
                                  size[b]));
+                    }
                 }
-        ++step;
+        step += single ? 2 : 1;
         /* level 1: folds in server order; contribution k of server d sits in slot (k + d) mod M */
         for (uint32_t h = 1u << (r1 - 1); h >= 1; h >>= 1, ++step)
             for (uint32_t d = 0; d < n_srv; ++d)
@@ -1638,7 +1649,7 @@ static int order_preserved_ar2_build(HgOpList* l, int alg1, uint32_t n_srv, uint
                     const uint32_t peer = (i + n_loc - k) % n_loc, b = peer + s * n_loc;
                     CHK(push(l, step, COPY, SRV(s, i), OUT, blk * b, SRV(s, peer), OUT, blk * b, size[b]));
                 }
-        ++step;
+        if (!single) ++step;
         /* all-gather of the servers' runs between the servers */
         uint64_t run[HCOMM_GFX_MAX_RANKS];
         for (uint32_t d = 0; d < n_srv; ++d) {
@@ -1695,7 +1706,7 @@ int hg_schedule_order_preserved_ar2(HgOpList* l, int alg1, uint32_t n_servers, u
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 2 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
         return HCCL_E_PARA;
     int rc = order_preserved_ar2_build(l, alg1, n_servers, n_local, count, ccl_bytes, unit);
@@ -1737,6 +1748,39 @@ static int order_preserved_rs2_build(HgOpList* l, uint32_t n_srv, uint32_t n_loc
     for (uint64_t left = count; left > 0;) {
         const uint64_t cur = left > max_count ? max_count : left;
         const uint64_t c = cur * unit;
+        if (n_loc == 1) {
+            /* one device per module (:123-139, :246-252): the N blocks of the chunk to the CCL input buffer; then the
+             * plant stage between the servers WITH the borrowed place - block d's last slot on every rank d but the
+             * last is where the block already lies in the CCL input buffer, so the own plant is dropped there and
+             * the peers' plants follow a step later */
+            const uint32_t last = n - 1;
+            for (uint32_t p = 0; p < n; ++p)
+                for (uint32_t b = 0; b < n; ++b) CHK(push(l, step, COPY, p, IN, c * b, p, UIN, user_off + stride * b, c));
+            ++step;
+            for (uint32_t d = 0; d < n; ++d)
+                for (uint32_t c0 = 0; c0 < n; ++c0) {
+                    const uint32_t slot = (c0 + d) % n;
+                    if (slot == last && d != last) {
+                        if (c0 != d) CHK(push(l, step + 1, COPY, d, IN, c * d, c0, IN, c * d, c));
+                    } else {
+                        CHK(push(l, step + (c0 != d ? 1u : 0u), COPY, d, OUT, c * slot, c0, IN, c * d, c));
+                    }
+                }
+            step += 2;
+            for (uint32_t h = 1u << (r1 - 1); h >= 1; h >>= 1, ++step)
+                for (uint32_t d = 0; d < n; ++d)
+                    for (uint32_t j = 0; j + h < (n < 2 * h ? n : 2 * h); ++j) {
+                        const uint32_t to = (j + d) % n, from = (h + j + d) % n;
+                        const int to_in = d != last && to == last, from_in = d != last && from == last;
+                        CHK(push(l, step, REDUCE, d, to_in ? IN : OUT, to_in ? c * d : c * to, d, from_in ? IN : OUT,
+                                 from_in ? c * d : c * from, c));
+                    }
+            for (uint32_t p = 0; p < n; ++p) CHK(push(l, step, COPY, p, UOUT, user_off, p, OUT, c * p, c));
+            ++step;
+            user_off += c;
+            left -= cur;
+            continue;
+        }
 #define SRV(s, i) ((s) * n_loc + (i))
         for (uint32_t s = 0; s < n_srv; ++s)
             for (uint32_t i = 0; i < n_loc; ++i)
@@ -1778,7 +1822,7 @@ int hg_schedule_order_preserved_rs2(HgOpList* l, uint32_t n_servers, uint32_t n_
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 2 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     int rc = order_preserved_rs2_build(l, n_servers, n_local, count, ccl_bytes, unit);
     if (rc == HCCL_SUCCESS) rc = order_by_step_rank(l);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

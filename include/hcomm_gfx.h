@@ -775,8 +775,9 @@ int32_t HcommGfxOrderPreservedAllReduceCheck(
  * all-gather of the servers' runs between them - level1Alg HCOMM_GFX_ALG_ALLREDUCE_RING, _NB or _NHR selects
  * AllGatherRing, AllGatherNB or AllGatherNHR (:293-303) - and the copy to the user output.  Every element is
  * reduced as tree(servers)( tree(devices of server 0), tree(devices of server 1), ... ) with the rank-order tree of
- * the single-server executor at both levels.  nServers >= 2 and nLocal >= 2 (one device per module takes a branch
- * of its own, :195-206, which is not built).  Buffers and errors as above.  Step-wise lowering.
+ * the single-server executor at both levels.  nServers >= 2; with nLocal == 1 (one device per module, :195-206) level 0
+ * is a copy of the chunk into the CCL input buffer, the stage between the servers reads its blocks from there and
+ * nothing is gathered inside the module.  Buffers and errors as above.  Step-wise lowering.
  */
 int32_t HcommGfxOrderPreservedHierAllReducePlanCreate(
     HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut,
@@ -796,11 +797,13 @@ int32_t HcommGfxOrderPreservedHierAllReduceCheck(
  * 128 bytes per block), without borrowed places, and rank p's block from the CCL output buffer to its user output.
  * userIn: N * count elements per rank (block p at p * count); userOut: count elements; cclOut: cclBytes.  Rank p's
  * result is tree(servers)( tree(devices of server 0), ... ) over the N contributions to block p.
- * nServers >= 2 and nLocal >= 2.  Step-wise lowering.
+ * nServers >= 2.  nLocal == 1 (one device per module, :123-139, :246-252) stages the N blocks in the CCL input buffer
+ * instead of planting inside the server and runs the stage between the servers with the borrowed place: only then is
+ * cclIn used (cclBytes each); it may be NULL otherwise.  Step-wise lowering.
  */
 int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
-    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclOut, uint64_t cclBytes,
-    uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
+    uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, void* const* cclIn, void* const* cclOut,
+    uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp, HcommGfxPlan** plan);
 int32_t HcommGfxOrderPreservedHierReduceScatterEmit(
     uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops,
     uint64_t cap, uint64_t* n);
@@ -822,7 +825,7 @@ int32_t HcommGfxOrderPreservedHierReduceScatterCheck(
  * type and reduce operation; the user inputs are only read; the CCL buffers are not needed and not touched, so there
  * is no chunk loop.  HCCL_E_NOT_SUPPORT for a reduce-scatter whose block (count * unit bytes) is not a multiple of
  * 16 bytes, and where ceil_pow2(nServers) * ceil_pow2(nLocal) exceeds 32 (5 x 6, 3 x 9 ...): use the step-wise plan.
- * Buffers 128-byte aligned, nLocal >= 2.
+ * Buffers 128-byte aligned, at least two ranks.
  */
 int32_t HcommGfxOrderPreservedFusedPlanCreate(
     int32_t allReduce, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut, uint64_t count,

@@ -66,11 +66,11 @@
  *                                     slots), a chunk / block table N = 4 by hand; the same rank-order fold trees for
  *                                     every element N = 2..8; slot and borrowed-slot layout from the definition;
  *                                     exact integer results over several chunks; pinned
- *   two-level order-preserving allreduce . the complete operation list of 2 x 2 (every borrowed place of both levels)
- *                                     by hand; reduction trees 2 x 2 .. 3 x 3 composed by hand from the single-level
+ *   two-level order-preserving allreduce . the complete operation lists of 2 x 2 (every borrowed place of both levels)
+ *                                     and of 3 x 1 (one device per module) by hand; reduction trees 2 x 2 .. 3 x 3 composed by hand from the single-level
  *                                     trees; slot / borrowed-place layout of both levels from the definition; exact
  *                                     integer results over several chunks, ring / NB / NHR all-gather; pinned
- *   two-level order-preserving reduce-scatter . the complete operation list of 2 x 2 by hand; the composed reduction
+ *   two-level order-preserving reduce-scatter . the complete operation lists of 2 x 2 and 3 x 1 by hand; the composed reduction
  *                                     trees per block; layout from the definition; exact integer results; pinned
  *   (every schedule additionally passes the symbolic checker for N = 1..17, 24, 31, 32)
  */
@@ -2551,8 +2551,12 @@ static void prog_plant_groups(OrcTrace* t, uint32_t local_rank, uint32_t rank_si
  * in_off[d]: where the level-0 result for server d's block lies, out_off[d]: block (i + d * L) itself.
  * Step 0: LocalCopy (:118-142) and the all-to-all (:180-209, :211-230); steps 1..: RunLocalReduce (:232-304). */
 static void prog_plant_combine(OrcTrace* t, uint32_t rank, uint32_t rank_size, const uint64_t* size, const uint64_t* in_off,
-                               const uint64_t* out_off, int use_ccl_in, int level0_last_rank, int need_space_borrow)
+                               const uint64_t* out_off, int use_ccl_in, int level0_last_rank, int need_space_borrow,
+                               uint32_t a2a_step)
 {
+    /* a2a_step 0: LocalCopy and the all-to-all share step 0 (nothing a peer writes is read by a LocalCopy); 1: the
+     * peers' writes come a step after the LocalCopies - with one device per module a peer may write the very place
+     * the own block was read from, which the handshake after LocalCopy (:211-220) orders */
     use_ccl_in = use_ccl_in && need_space_borrow;             /* every borrowed place is behind isNeedSpaceBorrow_ */
     level0_last_rank = level0_last_rank && need_space_borrow;
 #define CALC_OUTPUT_INDEX(round) (((round) + rank) % rank_size) /* :80 */
@@ -2564,10 +2568,14 @@ static void prog_plant_combine(OrcTrace* t, uint32_t rank, uint32_t rank_size, c
         const uint32_t output_index = CALC_OUTPUT_INDEX(peer);
         const uint32_t src_buf = use_ccl_in ? B_IN : B_OUT;                        /* :125-130, :184-189 */
         const uint64_t src_off = use_ccl_in ? out_off[peer] : in_off[peer];
-        if (level0_last_rank && IS_LAST(output_index) && !IS_LAST(peer))          /* :132-138, :191-199 */
-            emit(t, 0, K_COPY, peer, B_IN, out_off[peer], rank, src_buf, src_off, size[peer]);
-        else
-            emit(t, 0, K_COPY, peer, B_OUT, out_off[output_index], rank, src_buf, src_off, size[peer]);
+        const uint32_t at = round == 0 ? 0 : a2a_step;
+        if (level0_last_rank && IS_LAST(output_index) && !IS_LAST(peer)) {        /* :132-138, :191-199 */
+            /* a copy onto itself is dropped by the dispatcher (platform/task/dispatcher.cc:495-498) */
+            if (!(peer == rank && src_buf == B_IN && src_off == out_off[peer]))
+                emit(t, at, K_COPY, peer, B_IN, out_off[peer], rank, src_buf, src_off, size[peer]);
+        } else {
+            emit(t, at, K_COPY, peer, B_OUT, out_off[output_index], rank, src_buf, src_off, size[peer]);
+        }
     }
     uint32_t reduce_step = 0;
     while ((1u << reduce_step) < rank_size) reduce_step++;
@@ -2580,7 +2588,7 @@ static void prog_plant_combine(OrcTrace* t, uint32_t rank, uint32_t rank_size, c
             const uint32_t output_index = CALC_OUTPUT_INDEX(offset);
             const int src_borrowed = level0_last_rank && !IS_LAST(rank) && IS_LAST(input_index);  /* :273-277 */
             const int dst_borrowed = level0_last_rank && !IS_LAST(rank) && IS_LAST(output_index); /* :279-283 */
-            emit(t, 1 + round, K_REDUCE, rank, dst_borrowed ? B_IN : B_OUT, dst_borrowed ? out_off[rank] : out_off[output_index],
+            emit(t, 1 + a2a_step + round, K_REDUCE, rank, dst_borrowed ? B_IN : B_OUT, dst_borrowed ? out_off[rank] : out_off[output_index],
                  rank, src_borrowed ? B_IN : B_OUT, src_borrowed ? out_off[rank] : out_off[input_index], size[rank]);
         }
     }
@@ -2603,15 +2611,18 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
 {
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
-    /* one device per module takes RunReduceScatterLevel0SingleRank (:195-206): not restated; one module is
-     * build_trace_order_preserved_ar */
-    if (unit == 0 || n_servers < 2 || n_local < 2 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    /* one module is build_trace_order_preserved_ar */
+    if (unit == 0 || n_servers < 2 || n_local < 1 || n_servers * n_local > ORC_MAX_RANKS) return -1;
     if (alg1 != ORC_ALG_ALLREDUCE_RING && alg1 != ORC_ALG_ALLREDUCE_NHR && alg1 != ORC_ALG_ALLREDUCE_NB) return -1;
     const uint32_t n = n_servers * n_local;
     const uint64_t max_count = ccl_bytes / unit;
     if (max_count == 0) return -1;
     const uint32_t steps0 = ceil_log2_u32(n_local), steps1 = ceil_log2_u32(n_servers);
     const uint32_t ag1_steps = alg1 == ORC_ALG_ALLREDUCE_RING ? n_servers - 1 : steps1;
+    /* one device per module: level 0 is a copy (:151-155), the peers' writes of level 1 come a step after the
+     * LocalCopies, and there is nothing to gather inside the module */
+    const int single = n_local == 1;
+    const uint32_t lvl0_steps = single ? 1 : 1 + steps0, a2a_step = single ? 1 : 0, ag0_steps = single ? 0 : 1;
     uint32_t identity[ORC_MAX_RANKS];
     for (uint32_t i = 0; i < ORC_MAX_RANKS; i++) identity[i] = i;
     uint32_t step0 = 0;
@@ -2636,7 +2647,10 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
             /* level 0, :356 */
             g_rank_map = level0;
             g_step_base = step0;
-            prog_plant_groups(t, local, n_local, n_servers, group_size, spb, spb, 1);
+            if (single) /* RunReduceScatterLevel0SingleRank, :195-206: the chunk to the front of the CCL input buffer */
+                emit(t, 0, K_COPY, local, B_IN, 0, local, B_UIN, 0, cur_size);
+            else
+                prog_plant_groups(t, local, n_local, n_servers, group_size, spb, spb, 1);
             /* level 1, :359: RunReduceScatterLevel1 :208-246 */
             uint64_t size1[ORC_MAX_RANKS], in_off[ORC_MAX_RANKS], out_off[ORC_MAX_RANKS];
             const uint32_t input_base_index = (1 + local) % n_local; /* :218 */
@@ -2646,9 +2660,9 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
                 out_off[d] = (uint64_t)(local + d * n_local) * spb;
             }
             g_rank_map = level1;
-            g_step_base = step0 + 1 + steps0;
-            prog_plant_combine(t, server, n_servers, size1, in_off, out_off, local == n_local - 2 /* :234-235 */,
-                               local == n_local - 1 /* :239 */, 1);
+            g_step_base = step0 + lvl0_steps;
+            prog_plant_combine(t, server, n_servers, size1, in_off, out_off, single || local == n_local - 2 /* :234-235 */,
+                               local == n_local - 1 /* :239 */, 1, a2a_step);
             /* all-gather inside the server, :363: RunAllGatherLevel0 :248-283 */
             OrcSlice seg[ORC_MAX_RANKS];
             for (uint32_t r = 0; r < n_local; r++) {
@@ -2656,7 +2670,7 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
                 seg[r].offset = seg[r].size == 0 ? 0 : (uint64_t)(r + server * n_local) * spb;
             }
             g_rank_map = level0;
-            g_step_base = step0 + 2 + steps0 + steps1;
+            g_step_base = step0 + lvl0_steps + 1 + a2a_step + steps1;
             prog_mesh_ag(t, local, n_local, seg);
             /* all-gather between the servers, :366: RunAllGatherLevel1 :285-340 */
             for (uint32_t d = 0; d < n_servers; d++) {
@@ -2665,12 +2679,12 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
                 seg[d].offset = (uint64_t)d * n_local * spb;
             }
             g_rank_map = level1;
-            g_step_base = step0 + 3 + steps0 + steps1;
+            g_step_base = step0 + lvl0_steps + 1 + a2a_step + steps1 + ag0_steps;
             if (alg1 == ORC_ALG_ALLREDUCE_RING) prog_ring_ag_ex(t, server, n_servers, seg, 0, 0);
             else if (alg1 == ORC_ALG_ALLREDUCE_NB) prog_nb_ag(t, server, n_servers, seg, 0);
             else prog_nhr_ag(t, server, n_servers, seg, identity, 0, 0); /* stand-alone: order kept, nothing merged */
             g_rank_map = NULL;
-            g_step_base = step0 + 3 + steps0 + steps1 + ag1_steps;
+            g_step_base = step0 + lvl0_steps + 1 + a2a_step + steps1 + ag0_steps + ag1_steps;
             emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_OUT, 0, cur_size); /* :369-376 */
         }
         g_user_off = 0;
@@ -2679,7 +2693,7 @@ static int build_trace_order_preserved_ar2(OrcTrace* t, int alg1, uint32_t n_ser
             free(t->ops);
             return -2;
         }
-        step0 += 4 + steps0 + steps1 + ag1_steps;
+        step0 += lvl0_steps + 1 + a2a_step + steps1 + ag0_steps + ag1_steps + 1;
         user_off += cur_size;
     }
     for (uint64_t i = 0; i < t->n; i++) { /* DeviceMem::range refuses a range past the end of the CCL buffer */
@@ -2701,8 +2715,9 @@ static int build_trace_order_preserved_rs2(OrcTrace* t, uint32_t n_servers, uint
 {
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 2 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (unit == 0 || n_servers < 2 || n_local < 1 || n_servers * n_local > ORC_MAX_RANKS) return -1;
     const uint32_t n = n_servers * n_local;
+    const int single = n_local == 1; /* one device per module */
     const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit;
     if (max_count == 0) return -1;
     const uint32_t steps0 = ceil_log2_u32(n_local), steps1 = ceil_log2_u32(n_servers);
@@ -2721,7 +2736,11 @@ static int build_trace_order_preserved_rs2(OrcTrace* t, uint32_t n_servers, uint
             for (uint32_t d = 0; d < n_servers; d++) level1[d] = d * n_local + local;
             g_rank_map = level0;
             g_step_base = step0;
-            prog_plant_groups(t, local, n_local, n_servers, size, cur_size, count * unit, 0); /* :267 */
+            if (single) { /* RunReduceScatterLevel0SingleRank, :123-139: every block to its place in the CCL input buffer */
+                for (uint32_t i = 0; i < n; i++) emit(t, 0, K_COPY, local, B_IN, cur_size * i, local, B_UIN, count * unit * i, cur_size);
+            } else {
+                prog_plant_groups(t, local, n_local, n_servers, size, cur_size, count * unit, 0); /* :267 */
+            }
             uint64_t in_off[ORC_MAX_RANKS], out_off[ORC_MAX_RANKS];
             const uint32_t input_base_index = (1 + local) % n_local; /* :231-232 */
             for (uint32_t d = 0; d < n_servers; d++) {
@@ -2729,11 +2748,11 @@ static int build_trace_order_preserved_rs2(OrcTrace* t, uint32_t n_servers, uint
                 out_off[d] = (uint64_t)(local + d * n_local) * cur_size;
             }
             g_rank_map = level1;
-            g_step_base = step0 + 1 + steps0;
-            prog_plant_combine(t, server, n_servers, size, in_off, out_off, local == n_local - 2, local == n_local - 1,
-                               0 /* borrowSpace = level0Ranksize == 1, :248 */); /* :270 */
+            g_step_base = step0 + (single ? 1 : 1 + steps0);
+            prog_plant_combine(t, server, n_servers, size, in_off, out_off, single || local == n_local - 2 /* :247 */,
+                               local == n_local - 1, single /* borrowSpace = level0Ranksize == 1, :248 */, single ? 1 : 0); /* :270 */
             g_rank_map = NULL;
-            g_step_base = step0 + 2 + steps0 + steps1;
+            g_step_base = step0 + (single ? 3 : 2 + steps0) + steps1;
             emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_OUT, cur_size * rank, cur_size); /* :273-279 */
         }
         g_user_off = 0;
@@ -2742,7 +2761,7 @@ static int build_trace_order_preserved_rs2(OrcTrace* t, uint32_t n_servers, uint
             free(t->ops);
             return -2;
         }
-        step0 += 3 + steps0 + steps1;
+        step0 += (single ? 4 : 3 + steps0) + steps1;
         user_off += cur_size;
     }
     return sort_trace(t);

@@ -135,7 +135,7 @@ int main(void)
                                 if (alg == 0) {
                                     emit_twice(e_ophrs, &x);
                                     if (HcommGfxOrderPreservedHierReduceScatterCheck(s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
-                                    p = NULL; HcommGfxOrderPreservedHierReduceScatterPlanCreate(s, l, bufs[3], bufs[4], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                                    p = NULL; HcommGfxOrderPreservedHierReduceScatterPlanCreate(s, l, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
                                     for (int ar = 0; ar < 2; ++ar) { p = NULL; HcommGfxOrderPreservedFusedPlanCreate(ar, s, l, bufs[3], bufs[4], x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p); }
                                 }
                                 if (HcommGfxOrderPreservedHierAllReduceCheck(alg, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;

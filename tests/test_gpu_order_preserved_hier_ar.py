@@ -28,6 +28,9 @@ CASES = [
     ("nb", 16, 2, 77777, "bf16", "sum", 1 << 20),
     ("ring", 2, 16, 5, "fp32", "sum", 1 << 17),             # one short block, 31 empty ones
     ("nhr", 3, 2, 0, "fp32", "sum", 4096),
+    ("ring", 8, 1, 300007, "fp32", "sum", 1 << 18),        # one device per module: level 0 is a copy into CCL in
+    ("nhr", 5, 1, 100003, "bf16", "sum", 1 << 21),
+    ("nb", 3, 1, 100, "fp32", "max", 1 << 20),
 ]
 
 
@@ -136,6 +139,8 @@ FUSED_CASES = [
     (0, 3, 5, 30000, "fp16", "sum"),
     (0, 7, 3, 4104, "int16", "sum"),
     (0, 2, 2, 16, "fp32", "prod"),
+    (1, 8, 1, 100003, "fp32", "sum"),          # one device per module
+    (0, 5, 1, 4096, "bf16", "sum"),
 ]
 
 

@@ -25,6 +25,9 @@ CASES = [
     (7, 3, 4099, "int16", "sum", 1 << 18),
     (16, 2, 7777, "bf16", "sum", 1 << 20),
     (3, 2, 0, "fp32", "sum", 4096),
+    (8, 1, 100007, "fp32", "sum", 1 << 20),        # one device per module: the blocks are staged in CCL in
+    (5, 1, 30001, "bf16", "sum", 1 << 21),
+    (3, 1, 10, "fp32", "max", 1 << 20),
 ]
 
 
@@ -40,15 +43,17 @@ def run_case(thread, m, l, count, dtype, op, ccl, seed=0):
     junk = np.random.default_rng(19).integers(0, 256, ccl, dtype=np.uint8)
     w_in = [x.copy() for x in host_in]
     w_out = [sentinel.copy() for _ in range(n)]
-    w_cin = [np.zeros(16, np.uint8) for _ in range(n)]
+    w_cin = [junk[::-1].copy() for _ in range(n)]
     w_cout = [junk.copy() for _ in range(n)]
     oracle.run_order_preserved_rs2(m, l, w_in, w_out, w_cin, w_cout, count, ccl, dt, o)
     d_in = [to_dev(x) for x in host_in]
     d_out = [to_dev(sentinel) for _ in range(n)]
+    d_cin = [to_dev(junk[::-1].copy()) for _ in range(n)]
     d_cout = [to_dev(junk) for _ in range(n)]
     pad = to_dev(np.zeros(256, np.uint8))
     ptrs = lambda ts: [t.data_ptr() if t.numel() else pad.data_ptr() for t in ts]
-    plan = h.OrderPreservedHierReduceScatterPlan(m, l, ptrs(d_in), ptrs(d_out), ptrs(d_cout), ccl, count, dt, o)
+    plan = h.OrderPreservedHierReduceScatterPlan(m, l, ptrs(d_in), ptrs(d_out), ptrs(d_cout), ccl, count, dt, o,
+                                                 ccl_in=ptrs(d_cin) if l == 1 else None)
     try:
         assert plan.run(thread) == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
@@ -56,6 +61,7 @@ def run_case(thread, m, l, count, dtype, op, ccl, seed=0):
             assert_same(from_dev(d_out[r], sentinel), w_out[r], dt, "user out[%d]" % r)
             assert np.array_equal(from_dev(d_in[r], host_in[r]).view(np.uint8), host_in[r].view(np.uint8)), "user in[%d] was written" % r
             assert np.array_equal(from_dev(d_cout[r], junk), w_cout[r]), "CCL out[%d]" % r
+            assert np.array_equal(from_dev(d_cin[r], junk), w_cin[r]), "CCL in[%d]" % r
         ops = oracle.trace_order_preserved_rs2(m, l, count, ccl, dt)
         assert plan.info.algorithmicBytes == sum(x[8] * (3 if x[1] else 2) for x in ops)
         return plan.info

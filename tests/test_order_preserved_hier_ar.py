@@ -20,6 +20,7 @@ TREES1 = _G["order_preserved_reduce_scatter"]["rank_tree"]
 CCL_IN, CCL_OUT, UIN, UOUT = 0, 1, 3, 4
 ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NB]
 SHAPES = [(2, 2), (2, 3), (3, 2), (2, 8), (4, 4), (3, 5), (5, 3), (4, 8), (8, 4), (2, 16), (16, 2), (7, 3)]
+SINGLE = [(2, 1), (3, 1), (5, 1), (8, 1), (13, 1), (32, 1)]          # one device per module
 
 
 def compose(tree, leaves):
@@ -41,6 +42,12 @@ def test_operation_list_hand_derived():
     assert h.order_preserved_hier_ar_emit(h.Alg.ALLREDUCE_RING, 2, 2, 100, 1 << 20, oracle.F32) == want
 
 
+def test_operation_list_hand_derived_one_device_per_module():
+    want = [tuple(o) for o in GOLD["ops_3x1_ring_fp32_count100"]["ops"]]
+    assert oracle.trace_order_preserved_ar2(oracle.ALG_ALLREDUCE_RING, 3, 1, 100, 1 << 20, oracle.F32) == want
+    assert h.order_preserved_hier_ar_emit(h.Alg.ALLREDUCE_RING, 3, 1, 100, 1 << 20, oracle.F32) == want
+
+
 def test_hand_composed_trees_are_the_composition_of_the_single_level_trees():
     for key, tree in GOLD["trees"].items():
         if key.startswith("_"):
@@ -52,7 +59,8 @@ def test_hand_composed_trees_are_the_composition_of_the_single_level_trees():
 @pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
 @pytest.mark.parametrize("alg", ALGS)
 def test_every_element_is_folded_devices_first_then_servers_in_rank_order(op, alg):
-    for m, l in ((2, 2), (2, 3), (3, 2), (2, 4), (4, 2), (3, 3), (2, 8), (4, 4), (3, 5), (8, 2), (5, 6)):
+    for m, l in ((2, 2), (2, 3), (3, 2), (2, 4), (4, 2), (3, 3), (2, 8), (4, 4), (3, 5), (8, 2), (5, 6), (2, 1), (3, 1), (5, 1),
+                 (8, 1)):
         n, count = m * l, 80000
         ins = order_sensitive_inputs(n, count, op, seed=900 + n)
         uin = [x.copy() for x in ins]
@@ -61,7 +69,7 @@ def test_every_element_is_folded_devices_first_then_servers_in_rank_order(op, al
         cin = [np.zeros(ccl // 4, np.float32) for _ in range(n)]
         cout = [np.zeros(ccl // 4, np.float32) for _ in range(n)]
         oracle.run_order_preserved_ar2(alg, m, l, uin, uout, cin, cout, count, ccl, oracle.F32, op)
-        tree = GOLD["trees"].get("%dx%d" % (m, l)) or two_level_tree(m, l)
+        tree = TREES1[str(m)] if l == 1 else GOLD["trees"].get("%dx%d" % (m, l)) or two_level_tree(m, l)
         want = eval_tree(tree, ins, op)
         for p in range(n):
             assert np.array_equal(uout[p].view(np.uint32), want.view(np.uint32)), (m, l, p)
@@ -110,7 +118,7 @@ def test_layout_invariants():
 
 def test_product_generator_equals_oracle_trace_and_passes_the_checker():
     refused = 0
-    for m, l in SHAPES:
+    for m, l in SHAPES + SINGLE:
         n = m * l
         for alg in ALGS:
             for count, ccl, dt in ((100, 1 << 20, oracle.F32), (1000, 1 << 20, oracle.F32), (100003, 1 << 18, oracle.F16),
@@ -126,12 +134,12 @@ def test_product_generator_equals_oracle_trace_and_passes_the_checker():
                 assert a == h.order_preserved_hier_ar_emit(alg, m, l, count, ccl, dt), (m, l, alg, count, ccl)
                 assert h.order_preserved_hier_ar_check(alg, m, l, count, ccl, dt)[:2] == (0, 0), (m, l, alg, count, ccl)
                 assert h.oplist_check(a, n, Expect.ALLREDUCE_USER, count, h.DTYPE_SIZE[dt])[:2] == (0, 0)
-    assert 0 < refused <= 3 * len(SHAPES)
+    assert 0 < refused <= 3 * len(SHAPES + SINGLE)
 
 
 def test_exact_integer_sums_and_chunking():
     rng = np.random.default_rng(5)
-    for m, l in SHAPES:
+    for m, l in SHAPES + SINGLE:
         n = m * l
         for alg in ALGS:
             for count, ccl in ((1000, 1 << 20), (100003, 1 << 18), (n * 32, n * 128), (7, 1 << 16), (1, 1 << 16)):
@@ -140,7 +148,11 @@ def test_exact_integer_sums_and_chunking():
                 uout = [np.full(count, -7, np.int32) for _ in range(n)]
                 cin = [np.full(ccl // 4 + 1, -3, np.int32) for _ in range(n)]
                 cout = [np.full(ccl // 4 + 1, -5, np.int32) for _ in range(n)]
-                oracle.run_order_preserved_ar2(alg, m, l, uin, uout, cin, cout, count, ccl, oracle.I32, oracle.SUM)
+                try:
+                    oracle.run_order_preserved_ar2(alg, m, l, uin, uout, cin, cout, count, ccl, oracle.I32, oracle.SUM)
+                except ValueError:                                    # (32 x 1, 128 bytes per rank): the slots do not fit
+                    assert (m, l, count, ccl) == (32, 1, n * 32, n * 128)
+                    continue
                 want = np.sum(np.stack(ins).astype(np.int64), axis=0).astype(np.int32)
                 for r in range(n):
                     assert np.array_equal(uout[r], want), (m, l, alg, count, ccl, r)
@@ -152,7 +164,7 @@ def test_rejects_bad_arguments():
     R = oracle.ALG_ALLREDUCE_RING
     for f in (oracle.trace_order_preserved_ar2, h.order_preserved_hier_ar_emit):
         for args in ((R, 1, 8, 100, 4096, oracle.F32),         # one module: the single-server executor
-                     (R, 8, 1, 100, 4096, oracle.F32),         # one device per module takes a branch that is not built
+                     (R, 8, 0, 100, 4096, oracle.F32),
                      (R, 2, 2, 100, 3, oracle.F32),            # not one element fits the CCL buffer
                      (R, 4, 8, 16, 16, oracle.I8),             # the 128-byte slots reach past 16 bytes
                      (R, 3, 11, 100, 1 << 20, oracle.F32),     # more than 32 ranks
@@ -184,15 +196,15 @@ def test_fused_leaf_layout_gives_the_two_level_tree():
         if not key.startswith("_"):
             m, l = (int(v) for v in key.split("x"))
             assert kernel_tree_two_level(m, l) == tree, key
-    for m, l in SHAPES + [(1, 2), (1, 5), (1, 8), (1, 32)]:
+    for m, l in SHAPES + SINGLE + [(1, 2), (1, 5), (1, 8), (1, 32)]:
         if ((m - 1).bit_length() + (l - 1).bit_length()) <= 5 and m <= 8 and l <= 8:     # hand-derived trees: 2 .. 8
-            want = two_level_tree(m, l) if m > 1 else TREES1[str(l)]
+            want = TREES1[str(m)] if l == 1 else two_level_tree(m, l) if m > 1 else TREES1[str(l)]
             assert kernel_tree_two_level(m, l) == want, (m, l)
 
 
 def test_fused_two_level_plan_shape_and_limits():
     base = 0x7f0000000000
-    for m, l in SHAPES:
+    for m, l in SHAPES + SINGLE:
         n = m * l
         uin = [base + r * (1 << 32) for r in range(n)]
         uout = [base + (64 + r) * (1 << 32) for r in range(n)]
