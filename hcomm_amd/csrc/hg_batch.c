@@ -52,15 +52,9 @@ void hg_finish_seg2(HgLaunch* l)
 {
     HgSeg2Table* t = &l->tab.seg2;
     uint64_t tiles = 0, bytes = 0;
-    /* the bytewise kernel walks elements, not vectors: one "tile" is HG_TILE_VECS elements */
-    uint32_t es = 1;
-    if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE && l->op != 255u) es = HcommGfxDataTypeSize((HcommDataType)l->dtype);
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
-        if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE)
-            tiles += (t->bytes[s] / es + HG_TILE_VECS - 1) / HG_TILE_VECS;
-        else
-            tiles += tiles_of(t->bytes[s]);
+        tiles += tiles_of(t->bytes[s]);
         bytes += t->bytes[s];
     }
     t->tile_begin[t->nseg] = (uint32_t)tiles;
@@ -228,6 +222,15 @@ static int coalesce_one(Coalescer* c, const HgOp* o)
  * extra launch costs more than it saves. */
 #define HG_SPLIT_MIN_BYTES (64u * 1024u)
 
+/* Bytes of `o` that come before the 16-byte boundary both operands reach together; 0 when it is not to be cut. */
+uint64_t hg_split_head(const HgOp* o)
+{
+    const uintptr_t md = (uintptr_t)o->dst & (HG_VEC_BYTES - 1), ms = (uintptr_t)o->src & (HG_VEC_BYTES - 1);
+    const uint32_t es = o->is_reduce ? HcommGfxDataTypeSize((HcommDataType)o->dtype) : 1u;
+    if (md != 0 && md == ms && o->bytes >= HG_SPLIT_MIN_BYTES && es != 0 && md % es == 0) return HG_VEC_BYTES - md;
+    return 0;
+}
+
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
 {
     Coalescer c;
@@ -242,11 +245,10 @@ int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
         const HgOp* o = &ops[i];
         if (o->bytes == 0) continue;                   /* count == 0: nothing to do (dispatcher.cc:719-722) */
         if (!o->is_reduce && o->dst == o->src) continue; /* copy onto itself (dispatcher.cc:495-498) */
-        const uintptr_t md = (uintptr_t)o->dst & (HG_VEC_BYTES - 1), ms = (uintptr_t)o->src & (HG_VEC_BYTES - 1);
-        const uint32_t es = o->is_reduce ? HcommGfxDataTypeSize((HcommDataType)o->dtype) : 1u;
-        if (md != 0 && md == ms && o->bytes >= HG_SPLIT_MIN_BYTES && es != 0 && md % es == 0) {
+        const uint64_t cut = hg_split_head(o);
+        if (cut) {
             HgOp head = *o, body = *o;
-            head.bytes = HG_VEC_BYTES - md;
+            head.bytes = cut;
             body.dst = (char*)o->dst + head.bytes;
             body.src = (const char*)o->src + head.bytes;
             body.bytes = o->bytes - head.bytes;

@@ -57,6 +57,7 @@ HgThread* hg_thread_from_handle(ThreadHandle h);
  * kind / dtype / op share one launch.  Calls emit(launch, ctx) for each; stops at the first error. */
 typedef int (*HgEmitFn)(const HgLaunch* launch, void* ctx);
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
+uint64_t hg_split_head(const HgOp* o); /* bytes before the 16-byte boundary both operands reach together, or 0 */
 
 /* Fill tile_begin / blocks / bytes of a launch whose segment pointers and sizes are set. */
 void hg_finish_seg2(HgLaunch* l);

@@ -79,22 +79,48 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
     }
 }
 
-// ---- element-at-a-time fallback for pointers that are not 16-byte aligned --------------------------------
+// ---- operands that are not on 16-byte boundaries ----------------------------------------------------------
+//
+// The same 16-byte items as k_copy / k_reduce2, counted from the start of the segment (so that an item always holds
+// whole elements), loaded and stored through a type that promises only the element's alignment: the compiler picks
+// the widest access the target allows for it (global memory takes unaligned dwordx4 accesses in the unaligned access
+// mode the HSA ABI runs in; an item that straddles two cache lines costs one extra line).  The bytes after the last
+// whole item go element by element.
+
+template <uint32_t ES> struct UVec;
+template <> struct UVec<1> { typedef u32x4 T __attribute__((aligned(1))); };
+template <> struct UVec<2> { typedef u32x4 T __attribute__((aligned(2))); };
+template <> struct UVec<4> { typedef u32x4 T __attribute__((aligned(4))); };
 
 template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) void k_bytewise(const HgSeg2Table tab)
 {
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
+    typedef typename UVec<ES>::T UV;
     const uint32_t total = tab.tile_begin[tab.nseg];
     for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
-        const uint64_t e0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + threadIdx.x;
-        const uint64_t nelem = tab.bytes[s] / ES;
+        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + threadIdx.x;
+        const uint64_t bytes = tab.bytes[s];
+        const uint64_t nvec = bytes >> 4;
         uint8_t* d = (uint8_t*)tab.dst[s];
         const uint8_t* p = (const uint8_t*)tab.src[s];
+        u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
-            const uint64_t e = e0 + u * HG_BLOCK;
-            if (e < nelem) {
+            const uint64_t v = v0 + u * HG_BLOCK;
+            if (v < nvec) {
+                b[u] = *(const UV*)(p + (v << 4));
+                if (REDUCE) a[u] = *(const UV*)(d + (v << 4));
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) {
+            const uint64_t v = v0 + u * HG_BLOCK;
+            if (v < nvec) *(UV*)(d + (v << 4)) = REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u];
+        }
+        if (v0 - threadIdx.x + HG_TILE_VECS > nvec) { // the segment's one partial tile also owns the bytes after the last item
+            const uint64_t e = (nvec << 4) / ES + threadIdx.x;
+            if ((e + 1) * ES <= bytes) {
                 if (REDUCE) st_elem<ES>(d + e * ES, word_op<DT, OP>(ld_elem<ES>(d + e * ES), ld_elem<ES>(p + e * ES)));
                 else d[e] = p[e];
             }

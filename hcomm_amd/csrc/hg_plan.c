@@ -86,22 +86,43 @@ static int op_class(const HgOp* o)
 static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
                      int op)
 {
-    HgOp* ops = (HgOp*)calloc(n ? n : 1, sizeof(HgOp));
-    if (!ops) return HCCL_E_MEMORY;
+    /* two entries per operation: one whose operands are equally far from a 16-byte boundary is cut, as the coalescer
+     * would cut it, into the few bytes up to that boundary and an aligned rest - here, so that the grouping below sees
+     * the pieces; steps[] carries the step of every entry */
+    HgOp* ops = (HgOp*)calloc(n ? 2 * n : 1, sizeof(HgOp));
+    uint32_t* steps = (uint32_t*)calloc(n ? 2 * n : 1, sizeof(uint32_t));
+    if (!ops || !steps) {
+        free(ops);
+        free(steps);
+        return HCCL_E_MEMORY;
+    }
+    uint64_t m = 0;
     for (uint64_t i = 0; i < n; ++i) {
         const HcommGfxSchedOp* s = &list[i];
-        HgOp* o = &ops[i];
+        HgOp* o = &ops[m];
         o->is_reduce = (uint8_t)s->kind;
         o->dtype = s->kind ? (uint8_t)dtype : 255;
         o->op = s->kind ? (uint8_t)op : 255;
         if (s->dstBuf >= HCOMM_GFX_NUM_BUFS || s->srcBuf >= HCOMM_GFX_NUM_BUFS || !bufs[s->dstBuf] || !bufs[s->srcBuf]) {
             free(ops);
+            free(steps);
             return HCCL_E_PTR;
         }
         o->dst = (char*)bufs[s->dstBuf][s->rank] + s->dstOff;
         o->src = (const char*)bufs[s->srcBuf][s->srcRank] + s->srcOff;
         o->bytes = s->bytes;
+        steps[m++] = s->step;
+        uint64_t head = hg_split_head(o);
+        if (head) {
+            ops[m] = *o;
+            ops[m].dst = (char*)o->dst + head;
+            ops[m].src = (const char*)o->src + head;
+            ops[m].bytes = o->bytes - head;
+            o->bytes = head;
+            steps[m++] = s->step;
+        }
     }
+    n = m;
     /* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the
      * next slice), or operations on 16-byte boundaries beside others that are not (blocks of odd sizes), would
      * change kernel with every operation: when nothing in the step can observe anything else in it, run it class by
@@ -110,12 +131,13 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
     for (uint64_t i = 0; i < n;) {
         uint64_t j = i;
         uint32_t seen = 0;
-        while (j < n && list[j].step == list[i].step) seen |= 1u << op_class(&ops[j++]);
+        while (j < n && steps[j] == steps[i]) seen |= 1u << op_class(&ops[j++]);
         /* the pairwise test is quadratic: steps larger than any schedule here produces keep their order */
         if ((seen & (seen - 1u)) != 0 && j - i <= 4096 && step_is_conflict_free(ops + i, j - i)) {
             HgOp* tmp = (HgOp*)malloc((j - i) * sizeof(HgOp));
             if (!tmp) {
                 free(ops);
+                free(steps);
                 return HCCL_E_MEMORY;
             }
             uint64_t k = 0;
@@ -129,6 +151,7 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
     }
     int rc = hg_coalesce(ops, n, plan_push, p);
     free(ops);
+    free(steps);
     return rc;
 }
 
