@@ -534,7 +534,7 @@ int32_t HcommGfxReduceKOnThread(
     uintptr_t align = (uintptr_t)dst;
     for (uint32_t j = 0; j < k; ++j) align |= (uintptr_t)srcs[j];
     if (align & (HG_VEC_BYTES - 1)) {
-        /* unaligned operands: the same chain as k-1 two-input element-wise launches */
+        /* unaligned operands: the same chain as k-1 two-input launches of the kernel for unaligned operands */
         HgOp o;
         memset(&o, 0, sizeof(o));
         o.dst = dst;

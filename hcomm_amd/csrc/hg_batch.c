@@ -218,7 +218,7 @@ static int coalesce_one(Coalescer* c, const HgOp* o)
 }
 
 /* Both operands equally far from a 16-byte boundary (a rank buffer addressed at an odd element offset): the few
- * bytes up to that boundary go to the element-wise kernel and the rest runs at full width.  Below this size the
+ * bytes up to that boundary go to the kernel for unaligned operands and the rest runs on aligned accesses.  Below this size the
  * extra launch costs more than it saves. */
 #define HG_SPLIT_MIN_BYTES (64u * 1024u)
 

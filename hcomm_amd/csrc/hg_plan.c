@@ -126,7 +126,7 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
     /* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the
      * next slice), or operations on 16-byte boundaries beside others that are not (blocks of odd sizes), would
      * change kernel with every operation: when nothing in the step can observe anything else in it, run it class by
-     * class - reduces before copies, the 128-bit kernels before the element-wise one - each class in its original
+     * class - reduces before copies, the aligned kernels before the one for unaligned operands - each class in its original
      * order. */
     for (uint64_t i = 0; i < n;) {
         uint64_t j = i;

@@ -327,7 +327,7 @@ typedef enum {
     HCOMM_GFX_KERNEL_REDUCE2 = 1,  /* batched dst = dst (op) src */
     HCOMM_GFX_KERNEL_CHAIN = 2,    /* k inputs folded in sequence, optional partial stores, fan-out stores */
     HCOMM_GFX_KERNEL_TREE = 3,     /* k = 2^j inputs folded as a binary tree with partial stores, fan-out */
-    HCOMM_GFX_KERNEL_BYTEWISE = 4  /* element-at-a-time fallback for pointers not 16-byte aligned */
+    HCOMM_GFX_KERNEL_BYTEWISE = 4  /* copy / two-input reduce for pointers off 16-byte boundaries (unaligned 16-byte items) */
 } HcommGfxKernelKind;
 
 /* Copy up to `cap` records of the thread's launch log into `out`; *n receives the total logged. */
