@@ -109,8 +109,8 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
             if (v < nvec) {
-                b[u] = *(const UV*)(p + (v << 4));
-                if (REDUCE) a[u] = *(const UV*)(d + (v << 4));
+                b[u] = __builtin_nontemporal_load((const UV*)(p + (v << 4)));
+                if (REDUCE) a[u] = __builtin_nontemporal_load((const UV*)(d + (v << 4)));
             }
         }
 #pragma unroll
