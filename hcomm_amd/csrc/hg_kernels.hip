@@ -81,11 +81,13 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 
 // ---- operands that are not on 16-byte boundaries ----------------------------------------------------------
 //
-// The same 16-byte items as k_copy / k_reduce2, counted from the start of the segment (so that an item always holds
-// whole elements), loaded and stored through a type that promises only the element's alignment: the compiler picks
-// the widest access the target allows for it (global memory takes unaligned dwordx4 accesses in the unaligned access
-// mode the HSA ABI runs in; an item that straddles two cache lines costs one extra line).  The bytes after the last
-// whole item go element by element.
+// The few elements before dst's next 16-byte boundary go one by one; from there on dst is read and written in
+// aligned 16-byte items like k_copy / k_reduce2 do, and only src - as far from a boundary as it happens to be - is
+// loaded through a type that promises no more than the element's alignment: the compiler picks the widest access
+// the target allows for it (global memory takes unaligned dwordx4 loads in the unaligned access mode the HSA ABI
+// runs in; an item that straddles two cache lines is served from both).  An item holds whole elements because dst
+// and src are element-aligned and the head is a whole number of elements.  The bytes after the last whole item go
+// one by one too; head and tail belong to the tile that holds the end of the items.
 
 template <uint32_t ES> struct UVec;
 template <> struct UVec<1> { typedef u32x4 T __attribute__((aligned(1))); };
@@ -97,32 +99,39 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
     typedef typename UVec<ES>::T UV;
     const uint32_t total = tab.tile_begin[tab.nseg];
+    const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
-        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + threadIdx.x;
         const uint64_t bytes = tab.bytes[s];
-        const uint64_t nvec = bytes >> 4;
-        uint8_t* d = (uint8_t*)tab.dst[s];
-        const uint8_t* p = (const uint8_t*)tab.src[s];
+        uint8_t* d0 = (uint8_t*)tab.dst[s];
+        const uint8_t* p0 = (const uint8_t*)tab.src[s];
+        uint64_t head = (HG_VEC_BYTES - ((uintptr_t)d0 & (HG_VEC_BYTES - 1))) & (HG_VEC_BYTES - 1);
+        if (head > bytes) head = bytes / ES * ES;
+        uint8_t* d = d0 + head;      // on a 16-byte boundary (or past the end of a segment shorter than the head)
+        const uint8_t* p = p0 + head;
+        const uint64_t nvec = (bytes - head) >> 4;
+        const uint64_t vb = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
-            const uint64_t v = v0 + u * HG_BLOCK;
+            const uint64_t v = vb + tid + u * HG_BLOCK;
             if (v < nvec) {
                 b[u] = __builtin_nontemporal_load((const UV*)(p + (v << 4)));
-                if (REDUCE) a[u] = __builtin_nontemporal_load((const UV*)(d + (v << 4)));
+                if (REDUCE) a[u] = ldv<HG_NT_LD_DST>(d, v);
             }
         }
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
-            const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) *(UV*)(d + (v << 4)) = REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u];
+            const uint64_t v = vb + tid + u * HG_BLOCK;
+            if (v < nvec) stv<false>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
         }
-        if (v0 - threadIdx.x + HG_TILE_VECS > nvec) { // the segment's one partial tile also owns the bytes after the last item
-            const uint64_t e = (nvec << 4) / ES + threadIdx.x;
-            if ((e + 1) * ES <= bytes) {
-                if (REDUCE) st_elem<ES>(d + e * ES, word_op<DT, OP>(ld_elem<ES>(d + e * ES), ld_elem<ES>(p + e * ES)));
-                else d[e] = p[e];
+        if (vb <= nvec && vb + HG_TILE_VECS > nvec) { // the one tile that holds the end of the items
+            // fewer than 16 / ES elements before the first item and fewer than that after the last one
+            const uint64_t tail0 = head + (nvec << 4);
+            const uint64_t off = (uint64_t)tid * ES < head ? (uint64_t)tid * ES : tail0 + ((uint64_t)tid * ES - head);
+            if (off + ES <= bytes && (off < head || off >= tail0)) {
+                if (REDUCE) st_elem<ES>(d0 + off, word_op<DT, OP>(ld_elem<ES>(d0 + off), ld_elem<ES>(p0 + off)));
+                else d0[off] = p0[off];
             }
         }
     }
