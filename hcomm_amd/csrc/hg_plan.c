@@ -440,6 +440,7 @@ int32_t HcommGfxScratchBytes(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t co
 {
     if (!bytes) return HCCL_E_PTR;
     if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS || HcommGfxDataTypeSize(dataType) == 0) return HCCL_E_PARA;
+    if (count > HG_MAX_COUNT) return HCCL_E_PARA;
     *bytes = hg_scratch_bytes((int)alg, nRanks, count, (int)dataType);
     return HCCL_SUCCESS;
 }

@@ -20,6 +20,7 @@ int32_t HcommGfxCalcSlices(uint64_t count, uint32_t unitSize, uint32_t n, HcommG
 {
     if (!slices) return HCCL_E_PTR;
     if (unitSize == 0 || n == 0) return HCCL_E_PARA;
+    if (count > ((uint64_t)1 << 62) / unitSize) return HCCL_E_PARA; /* the byte total and its roundings stay in 64 bits */
     /* temp_all_reduce/all_reduce_ring.cc:142-153; RoundUpWithDivisor(0, 128) is 128 (alg_template_base_pub.h:609-616) */
     const uint64_t total = count * unitSize;
     const uint64_t per_raw = (total + (n - 1)) / n;
@@ -675,7 +676,7 @@ int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t strid
     memset(l, 0, sizeof(*l));
     if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (stride == 0) stride = count;
-    if (stride < count) return HCCL_E_PARA;
+    if (stride < count || stride > HG_MAX_COUNT) return HCCL_E_PARA;
     if (stride != count && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_MESH && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE &&
         alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
         return HCCL_E_PARA;
@@ -757,7 +758,7 @@ int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_
     memset(l, 0, sizeof(*l));
     if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) return HCCL_E_PARA;
     const int scatter = is_scatter_alg(alg);
     const uint64_t maxc = hg_opbase_max_count(alg, n, ccl_bytes, unit);
     if (maxc == 0) return scatter ? HCCL_E_INTERNAL : HCCL_E_PARA; /* :213-218 / :163-165 */
@@ -920,7 +921,7 @@ int hg_schedule_hier(HgOpList* l, int level0_mesh, int alg1, uint32_t n_servers,
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_RHD && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR &&
         alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
         return HCCL_E_PARA; /* the level-1 choices of :164-204 that are built here */
@@ -1004,7 +1005,7 @@ static int dbring_build(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_lo
                         int dtype)
 {
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
         return HCCL_E_PARA; /* the level-1 choices of coll_all_reduce_ring_for_910_93_executor.cc:304-351 built here */
     const uint64_t max_count = ccl_bytes / unit;
@@ -1247,7 +1248,7 @@ int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_serve
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers == 0 || n_local == 0 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (level0_mesh && n_local < 2) return HCCL_E_PARA; /* PrepareSliceMeshStreams refuses zero streams */
     if (alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RING && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR &&
         alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RHD)
@@ -1333,7 +1334,7 @@ int hg_schedule_dbring_rs(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n < 3 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n < 3 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     const int rc = dbring_rs_build(l, n, count, ccl_bytes, unit);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
     return rc;
@@ -1398,7 +1399,7 @@ int hg_schedule_order_preserved(HgOpList* l, uint32_t n, uint64_t count, uint64_
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     const int rc = order_preserved_build(l, n, count, ccl_bytes, unit);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
     return rc;
@@ -1455,7 +1456,7 @@ int hg_schedule_order_preserved_small(HgOpList* l, uint32_t n, uint64_t count, u
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || (n != 4 && n != 8)) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || (n != 4 && n != 8)) return HCCL_E_PARA;
     if (count * unit > 32u * 1024u) return HCCL_E_PARA; /* HCCL_SMALL_COUNT_32_KB, alg_template/template_v1_utils.h:64 */
     /* the template takes the user input's block stride from the chunk (reduce_scatter_hd_stage.cc:156-160): the
      * executor's loop must not cut the message */
@@ -1706,7 +1707,7 @@ int hg_schedule_order_preserved_ar2(HgOpList* l, int alg1, uint32_t n_servers, u
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (alg1 != HCOMM_GFX_ALG_ALLREDUCE_RING && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NHR && alg1 != HCOMM_GFX_ALG_ALLREDUCE_NB)
         return HCCL_E_PARA;
     int rc = order_preserved_ar2_build(l, alg1, n_servers, n_local, count, ccl_bytes, unit);
@@ -1822,7 +1823,7 @@ int hg_schedule_order_preserved_rs2(HgOpList* l, uint32_t n_servers, uint32_t n_
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers < 2 || n_local < 1 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     int rc = order_preserved_rs2_build(l, n_servers, n_local, count, ccl_bytes, unit);
     if (rc == HCCL_SUCCESS) rc = order_by_step_rank(l);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
@@ -1850,7 +1851,7 @@ int hg_schedule_order_preserved_ar(HgOpList* l, uint32_t n, uint64_t count, uint
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (unit == 0 || count > HG_MAX_COUNT || n < 2 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     const int rc = order_preserved_ar_build(l, n, count, ccl_bytes, unit);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
     return rc;

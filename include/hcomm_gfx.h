@@ -431,7 +431,9 @@ typedef struct {
  * Slice table of the allreduce templates: total = count * unit; per = roundup(ceil(total / n), 128);
  * slice i takes min(per, what is left) (temp_all_reduce/all_reduce_ring.cc:142-153,
  * alg_template_base.cc:787-820, recursive_halvingdoubling_base.cc:64-94).  Writes n entries.
- * unitSize 0, n 0 or slices NULL -> error.
+ * unitSize 0, n 0 or slices NULL -> error; so is a total beyond 2^62 bytes (HCCL_E_PARA).  Every schedule, plan
+ * and emit entry below refuses counts (and strides) above 2^48 elements per rank the same way, so that no byte
+ * offset derived from a count can wrap.
  */
 int32_t HcommGfxCalcSlices(uint64_t count, uint32_t unitSize, uint32_t n, HcommGfxSlice* slices);
 

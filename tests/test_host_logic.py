@@ -362,6 +362,25 @@ def test_plan_argument_checks():
     p.destroy()
 
 
+def test_counts_whose_byte_offsets_would_leave_64_bits_are_refused():
+    i, o = ptrs(4, 4096)
+    for count in (2**48 + 1, 2**62, 2**64 - 1):
+        for low in (h.Lowering.STEPWISE, h.Lowering.FUSED):
+            with pytest.raises(h.HcommError) as e:
+                h.Plan(h.Alg.ALLREDUCE_RING, low, i, o, count, DT.FP32, OP.SUM)
+            assert e.value.code == R.E_PARA
+        with pytest.raises(h.HcommError) as e:
+            h.schedule_emit(h.Alg.REDUCE_SCATTER_MESH, 4, 16, DT.INT8, stride=count)
+        assert e.value.code == R.E_PARA
+        with pytest.raises(h.HcommError) as e:
+            h.scratch_bytes(h.Alg.ALLREDUCE_CHUNK_MESH, 4, count, DT.INT32)
+        assert e.value.code == R.E_PARA
+    with pytest.raises(h.HcommError) as e:
+        h.calc_slices(2**61, 4, 8)
+    assert e.value.code == R.E_PARA
+    assert sum(sz for _, sz in h.calc_slices(2**60, 4, 8)) == 2**62
+
+
 @pytest.mark.parametrize("name,alg,n,count,dt,launches,algo_bytes,moved_fused", [
     # the five benchmark configurations at full size: launch structure and byte accounting, no memory touched
     ("cfg1", h.Alg.ALLREDUCE_RING, 8, 1048576, DT.FP32, 15, 155189248, 23 * 4194304),
