@@ -96,8 +96,8 @@ void hg_finish_fold(HgLaunch* l)
         uint64_t moved = 0;
         if (t->tree != 1u) {
             /* truncated rotation trees: nranks leaf reads, one store per even position that has a right neighbour
-             * (none for the rank-order tree, which only reads its inputs), and the root to one output or to all */
-            const uint64_t n = (uint64_t)t->nranks + (t->tree == 4u ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
+             * (none for the rank-order trees, which only read their inputs), and the root to one output or to all */
+            const uint64_t n = (uint64_t)t->nranks + (t->tree >= 4u ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
             l->moved_bytes = n * bytes;
             l->blocks = hg_grid_blocks(tiles, 0);
             return;

@@ -47,7 +47,8 @@ typedef struct {
  * in[(first[s] + j) mod nranks] / in[(first[s] - j) mod nranks] with only nranks <= k positions present (the
  * truncated trees of the nonuniform hierarchical ring / nonuniform Bruck schedules), or, when tree == 4, from
  * in[pos[j]] where pos[j] names a rank (the rank-order trees of the order-preserving executors, laid out by the host;
- * inputs only read).
+ * inputs only read), or, when tree == 5, from in[(first[s] - pos[j]) mod nranks] (the deterministic mesh
+ * reduce-scatter's row of receive slots; inputs only read).
  */
 typedef struct {
     const void* in[HCOMM_GFX_MAX_RANKS];
@@ -70,7 +71,7 @@ typedef struct {
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
-    uint8_t pos[HCOMM_GFX_MAX_RANKS]; /* tree == 4: the rank at leaf position q, or 255 where the tree has a hole */
+    uint8_t pos[HCOMM_GFX_MAX_RANKS]; /* tree == 4: the rank at leaf position q (tree == 5: how far below the segment's first rank it lies), or 255 where the tree has a hole */
 } HgFoldTable;
 
 /* Launch geometry decided on the host so that recorder threads can report it without a GPU. */

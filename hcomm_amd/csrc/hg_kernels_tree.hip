@@ -83,7 +83,9 @@ __device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t
 // order-preserving executors out that way - on one server position q holds rank bitrev(q) where that rank exists, so
 // level l folds rank j + K / 2^(l+1) onto rank j (the contributions K/2 .. onto 0 .., then K/4 .. onto 0 .., down to
 // 1 onto 0); over servers x devices the low position bits walk a server's devices like that and the high bits the
-// servers.  A hole's left neighbour always exists; the inputs are only read.
+// servers.  tree == 5 reads tab.pos[] as distances instead: position q of segment s holds rank first[s] - pos[q]
+// (mod n), the row of the deterministic mesh reduce-scatter, whose slot j - 1 is filled by rank d - j.
+// A hole's left neighbour always exists; the inputs are only read.
 template <class Item, int L, uint32_t NU>
 __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
                                                     const uint64_t (&idx)[NU])
@@ -94,7 +96,8 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
     const uint32_t c = tab.first[s];
     const uint32_t n = tab.nranks;
     const bool plus = tab.tree == 2u;
-    const bool order = tab.tree == 4u;
+    const bool order = tab.tree >= 4u;
+    const bool dist = tab.tree == 5u;
     V x[K][NU];
     uint32_t b[K];
     bool have[K];
@@ -103,6 +106,10 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
         if (order) {
             b[q] = tab.pos[q];
             have[q] = b[q] < n;
+            if (dist && have[q]) {
+                b[q] = c + n - b[q];
+                if (b[q] >= n) b[q] -= n;
+            }
         } else {
             b[q] = plus ? c + q : c + n - q;
             if (b[q] >= n) b[q] -= n;

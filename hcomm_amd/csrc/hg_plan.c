@@ -383,6 +383,58 @@ static int fused_oneshot_tree(HcommGfxPlan* p, uint32_t n, void* const* in, void
     return rc;
 }
 
+/* bit reversal of q inside `bits` bits */
+static uint32_t bitrev_n(uint32_t q, uint32_t bits)
+{
+    uint32_t r = 0;
+    for (uint32_t i = 0; i < bits; ++i) r |= ((q >> i) & 1u) << (bits - 1 - i);
+    return r;
+}
+
+/* ReduceScatterLocalReduce as one tree launch on the user buffers.  Destination d's row is V[j] = rank d - j's copy
+ * of slice d; the step-wise replay folds V[a + P] onto V[a] for the tail beyond the largest power of two P <= n and
+ * then V[a + h] onto V[a] for h = P/2 .. 1 (temp_reduce_scatter/reduce_scatter_local_reduce.cc:266-301).  With
+ * leaf position q holding V[bitrev(q)] (a hole where bitrev(q) >= n) level l of the kernel's tree folds exactly
+ * V[j + K / 2^(l+1)] onto V[j].  Only the inputs are read and only out[d] is written: the communication buffers,
+ * which the replay uses for the slots, are not touched. */
+static int fused_rs_local_reduce(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count,
+                                 int dtype, int op)
+{
+    const uint64_t sz = count * HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (sz == 0) return HCCL_SUCCESS;
+    /* slice d is read at d * sz in every input: 128-bit accesses need 16-byte multiples */
+    if (sz & (HG_VEC_BYTES - 1u)) return HCCL_E_NOT_SUPPORT;
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    l->kind = HCOMM_GFX_KERNEL_TREE;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    HgFoldTable* f = &l->tab.fold;
+    uint32_t bits = 1;
+    while ((1u << bits) < n) ++bits;
+    f->tree = 5u;
+    f->k = 1u << bits;
+    f->nranks = n;
+    f->out_mode = 1u;
+    memset(f->pos, 255, sizeof(f->pos));
+    for (uint32_t q = 0; q < f->k; ++q)
+        if (bitrev_n(q, bits) < n) f->pos[q] = (uint8_t)bitrev_n(q, bits);
+    f->nseg = n;
+    for (uint32_t d = 0; d < n; ++d) {
+        f->in[d] = in[d];
+        f->out[d] = out[d];
+        f->off[d] = (uint64_t)d * sz;
+        f->bytes[d] = sz;
+        f->first[d] = (uint8_t)d;
+        f->owner[d] = (uint8_t)d;
+        f->out_off[d] = 0;
+    }
+    hg_finish_fold(l);
+    const int rc = plan_push(l, p);
+    free(l);
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
                        uint64_t stride, int dtype, int op)
 {
@@ -415,6 +467,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_oneshot_tree(p, n, in, out, total, dtype, op);
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_rs_local_reduce(p, n, in, out, count, dtype, op);
         default: return HCCL_E_NOT_SUPPORT;
     }
 }
@@ -465,7 +520,8 @@ int32_t HcommGfxPlanCreateEx(
             if (((uintptr_t)out[r]) & 127u) return HCCL_E_PARA;
         }
     }
-    if (nRanks > 1 && hg_scratch_bytes((int)alg, nRanks, count, (int)dataType) > 0) {
+    /* the single-launch lowerings work on the user buffers alone */
+    if (lowering == HCOMM_GFX_LOWER_STEPWISE && nRanks > 1 && hg_scratch_bytes((int)alg, nRanks, count, (int)dataType) > 0) {
         if (!scratch) return HCCL_E_PTR;
         for (uint32_t r = 0; r < nRanks; ++r) {
             if (!scratch[r]) return HCCL_E_PTR;
@@ -795,14 +851,6 @@ int32_t HcommGfxOrderPreservedHierReduceScatterPlanCreate(
     rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, n, bufs, dataType, reduceOp, plan);
     hg_oplist_free(&ol);
     return rc;
-}
-
-/* bit reversal of q inside `bits` bits */
-static uint32_t bitrev_n(uint32_t q, uint32_t bits)
-{
-    uint32_t r = 0;
-    for (uint32_t i = 0; i < bits; ++i) r |= ((q >> i) & 1u) << (bits - 1 - i);
-    return r;
 }
 
 /* The order-preserving executors in one launch: the N user inputs are folded in registers along the executors' tree

@@ -201,6 +201,50 @@ def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype
     assert moved <= algo
 
 
+@pytest.mark.parametrize("n,count,dtype,op", [
+    (8, 1 << 20, "bf16", "sum"), (7, 100004, "fp32", "sum"), (6, 16384, "fp16", "max"), (5, 70016, "int8", "sum"),
+    (16, 40000, "int32", "min"), (3, 1000, "int16", "sum"), (2, 8, "fp32", "prod"), (1, 100, "fp32", "sum"),
+    (12, 4104, "fp16", "sum"), (31, 4096, "bf16", "max"), (32, 8200, "fp32", "sum"), (4, 0, "fp32", "sum"),
+])
+def test_fused_deterministic_reduce_scatter_on_the_user_buffers(gpu_thread, n, count, dtype, op):
+    """One tree launch in place of the slot writes and halving rounds: the user outputs hold the oracle's bits, the
+    inputs are only read, and no communication buffer is asked for."""
+    say("fused local_reduce_rs", n, count, dtype, op)
+    dt, o = DT[dtype], OPS[op]
+    host_in = [gen(dt, n * count, 7000 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    sentinel = gen(dt, count, 999, "wide")
+    want_in = [x.copy() for x in host_in]
+    want_out = [sentinel.copy() for _ in range(n)]
+    sb = h.scratch_bytes(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, n, count, dt)
+    oracle.run(oracle.ALG_RS_LOCAL_REDUCE, want_in, want_out, count, dt, o,
+               scratch=[np.zeros(sb, np.uint8) for _ in range(n)] if sb else None)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    pad = to_dev(np.zeros(256, np.uint8))
+    ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
+    plan = h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out],
+                  count, dt, o)
+    try:
+        assert plan.info.launches == (1 if count else 0)
+        assert plan.launches()[0].kind == (h.Kernel.TREE if n > 1 else h.Kernel.COPY) if count else True
+        if n > 1:
+            assert plan.info.movedBytes == (n + 1) * n * count * host_in[0].itemsize
+        assert plan.run(gpu_thread) == 0
+        assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_in[r], host_in[r]), host_in[r], dt, "in[%d]" % r)
+            assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+    finally:
+        plan.destroy()
+
+
+def test_fused_deterministic_reduce_scatter_needs_16_byte_slices():
+    with pytest.raises(h.HcommError) as e:
+        h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, [4096 * (r + 1) for r in range(4)],
+               [4096 * (r + 9) for r in range(4)], 100003, DT["fp32"], OPS["sum"])
+    assert e.value.code == h.HcclResult.E_NOT_SUPPORT
+
+
 @pytest.mark.parametrize("alg", SCATTER)
 @pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
 def test_strided_reduce_scatter(gpu_thread, alg, lowering):

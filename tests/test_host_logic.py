@@ -362,6 +362,43 @@ def test_plan_argument_checks():
     p.destroy()
 
 
+def test_fused_deterministic_reduce_scatter_is_one_tree_launch_with_the_hand_derived_trees():
+    """Leaf position q of destination d holds rank d - bitrev(q) where bitrev(q) < n; level l folds position
+    q + 2^l into q.  That tree must be the hand-derived one of the step-wise schedule (tail fold, then halving)."""
+    import json
+    import os
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "schedules_hand_derived.json")))
+    for n_s, trees in gold["rs_local_reduce_rank_tree"].items():
+        if n_s.startswith("_"):
+            continue
+        n = int(n_s)
+        L = max(1, (n - 1).bit_length())
+        K = 1 << L
+        rev = lambda q: int(format(q, "0%db" % L)[::-1], 2)
+        for d_s, tree in trees.items():
+            x = [(int(d_s) - rev(q)) % n if rev(q) < n else None for q in range(K)]
+            for l in range(L):
+                for q in range(0, K, 2 << l):
+                    if x[q + (1 << l)] is not None:
+                        x[q] = [x[q], x[q + (1 << l)]]
+            assert x[0] == tree, (n, d_s)
+    for n in (2, 3, 5, 8, 17, 32):
+        i, o = ptrs(n, 1 << 24)
+        p = h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, i, o, 4096, DT.BFP16, OP.SUM)  # no scratch
+        recs = p.launches()
+        assert [r.kind for r in recs] == [h.Kernel.TREE] and recs[0].nseg == n and recs[0].bytes == n * 8192
+        assert p.info.movedBytes == (n + 1) * n * 8192
+        stepwise_scratch = h.scratch_bytes(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, n, 4096, DT.BFP16)
+        assert stepwise_scratch > 0
+        p.destroy()
+        with pytest.raises(h.HcommError) as e:      # slices that are not 16-byte multiples
+            h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, i, o, 4099, DT.BFP16, OP.SUM)
+        assert e.value.code == R.E_NOT_SUPPORT
+        with pytest.raises(h.HcommError) as e:      # the step-wise replay still needs its communication buffers
+            h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.STEPWISE, i, o, 4096, DT.BFP16, OP.SUM)
+        assert e.value.code == R.E_PTR
+
+
 def test_counts_whose_byte_offsets_would_leave_64_bits_are_refused():
     i, o = ptrs(4, 4096)
     for count in (2**48 + 1, 2**62, 2**64 - 1):
