@@ -210,7 +210,7 @@ def main():
         args.lowering = "stepwise"  # composed from the step lists of its levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
-    if alg_name in ("local_reduce", "chunk_mesh") and args.lowering == "both":
+    if alg_name == "local_reduce" and args.lowering == "both":
         args.lowering = "stepwise"  # this schedule has no fused lowering
     kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
              h.Kernel.COPY: "k_copy", h.Kernel.BYTEWISE: "k_bytewise"}
@@ -301,8 +301,9 @@ def main():
             dom_bytes = sum(launches[i].bytes for i in range(first, first + cnt)) * per_byte // cnt
             dom_moved = dom_bytes
         else:
-            dom_bytes = plan.info.algorithmicBytes  # the single launch is the whole collective
-            dom_moved = plan.info.movedBytes
+            # the launches of the run (one, or one per group of ranks) are the whole collective: per-launch shares
+            dom_bytes = plan.info.algorithmicBytes // cnt
+            dom_moved = plan.info.movedBytes // cnt
         results[name] = {
             "ms_per_step": ms_step,
             "gbs": plan.info.algorithmicBytes / (ms_step * 1e-3) / 1e9,

@@ -67,10 +67,13 @@ typedef struct {
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
     uint32_t tree;           /* 0 chain; binary tree over k = 2^L positions: 1 recursive halving, 2 / 3 rotation + / -, 4 leaves from pos[] */
     uint32_t nout;           /* tree only: number of out[] entries that receive the result */
-    uint32_t ascending;      /* chain only: position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s] */
+    uint32_t ascending;      /* chain only: 1 = position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s];
+                              * 2 = position 0 is first[s], position j >= 1 is first[s] + 1 + (start[s] + j - 1) mod (nranks - 1):
+                              * the other ranks in cyclic order, entered at distance start[s] + 1 */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
+    uint8_t start[HG_MAX_SEG]; /* chain with ascending == 2 only */
     uint8_t pos[HCOMM_GFX_MAX_RANKS]; /* tree == 4: the rank at leaf position q (tree == 5: how far below the segment's first rank it lies), or 255 where the tree has a hole */
 } HgFoldTable;
 

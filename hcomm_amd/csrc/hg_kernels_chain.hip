@@ -14,9 +14,14 @@ namespace {
 
 __device__ __forceinline__ uint32_t fold_rank(const HgFoldTable& t, uint32_t s, uint32_t j)
 {
-    if (t.ascending) {
+    if (t.ascending == 1u) {
         if (j == 0) return t.first[s];
         return (j - 1 < t.first[s]) ? j - 1 : j;
+    }
+    if (t.ascending == 2u) { // the other ranks in cyclic order, entered at distance start[s] + 1
+        if (j == 0) return t.first[s];
+        const uint32_t r = t.first[s] + 1u + (t.start[s] + j - 1u) % (t.nranks - 1u);
+        return r >= t.nranks ? r - t.nranks : r;
     }
     int32_t r = (int32_t)t.first[s] + (int32_t)j * t.stride;
     const int32_t n = (int32_t)t.nranks;

@@ -435,6 +435,54 @@ static int fused_rs_local_reduce(HcommGfxPlan* p, uint32_t n, void* const* in, v
     return rc;
 }
 
+/* AllReduceChunkMesh on the user buffers: sub-chunk q of rank r's slice is the chain in[r], then the peers at
+ * distances q+1, q+2, .., n-1, 1, .., q (temp_all_reduce/all_reduce_chunk_mesh.cc:234-256), the running value in the
+ * dst role; the result goes to every output.  n (n-1) segments, whole ranks' worth per launch.  The communication
+ * buffers, where the replay keeps its copies, are not touched and the inputs are only read. */
+static int fused_chunk_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, int dtype,
+                            int op)
+{
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS], sub[HCOMM_GFX_MAX_RANKS];
+    int rc = HcommGfxCalcSlices(count, unit, n, sl);
+    if (rc != HCCL_SUCCESS) return rc;
+    HgLaunch* l = NULL;
+    for (uint32_t r = 0; r < n && rc == HCCL_SUCCESS; ++r) {
+        if (l && l->tab.fold.nseg + (n - 1) > HG_MAX_SEG) {
+            hg_finish_fold(l);
+            rc = plan_push(l, p);
+            free(l);
+            l = NULL;
+            if (rc != HCCL_SUCCESS) break;
+        }
+        if (!l) {
+            l = new_fold(dtype, op, 1, n, in, out);
+            if (!l) return HCCL_E_MEMORY;
+            l->tab.fold.ascending = 2u;
+            l->tab.fold.out_mode = 2u;
+        }
+        HgFoldTable* f = &l->tab.fold;
+        rc = HcommGfxCalcSlices(sl[r].size / unit, unit, n - 1, sub);
+        for (uint32_t q = 0; q + 1 < n && rc == HCCL_SUCCESS; ++q) {
+            if (sub[q].size == 0) continue;
+            const uint32_t s = f->nseg++;
+            f->off[s] = sl[r].offset + sub[q].offset;
+            f->bytes[s] = sub[q].size;
+            f->first[s] = (uint8_t)r;
+            f->owner[s] = (uint8_t)r;
+            f->start[s] = (uint8_t)q;
+        }
+    }
+    if (l) {
+        if (rc == HCCL_SUCCESS && l->tab.fold.nseg) {
+            hg_finish_fold(l);
+            rc = plan_push(l, p);
+        }
+        free(l);
+    }
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
                        uint64_t stride, int dtype, int op)
 {
@@ -467,6 +515,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_oneshot_tree(p, n, in, out, total, dtype, op);
+        case HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_chunk_mesh(p, n, in, out, count, dtype, op);
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rs_local_reduce(p, n, in, out, count, dtype, op);

@@ -201,34 +201,55 @@ def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype
     assert moved <= algo
 
 
-@pytest.mark.parametrize("n,count,dtype,op", [
-    (8, 1 << 20, "bf16", "sum"), (7, 100004, "fp32", "sum"), (6, 16384, "fp16", "max"), (5, 70016, "int8", "sum"),
-    (16, 40000, "int32", "min"), (3, 1000, "int16", "sum"), (2, 8, "fp32", "prod"), (1, 100, "fp32", "sum"),
-    (12, 4104, "fp16", "sum"), (31, 4096, "bf16", "max"), (32, 8200, "fp32", "sum"), (4, 0, "fp32", "sum"),
-])
-def test_fused_deterministic_reduce_scatter_on_the_user_buffers(gpu_thread, n, count, dtype, op):
-    """One tree launch in place of the slot writes and halving rounds: the user outputs hold the oracle's bits, the
-    inputs are only read, and no communication buffer is asked for."""
-    say("fused local_reduce_rs", n, count, dtype, op)
+USER_BUFFER_FUSED = [
+    # alg, n, count, dtype, op: single-launch lowerings that leave the communication buffers alone
+    ("local_reduce_rs", 8, 1 << 20, "bf16", "sum"), ("local_reduce_rs", 7, 100004, "fp32", "sum"),
+    ("local_reduce_rs", 6, 16384, "fp16", "max"), ("local_reduce_rs", 5, 70016, "int8", "sum"),
+    ("local_reduce_rs", 16, 40000, "int32", "min"), ("local_reduce_rs", 3, 1000, "int16", "sum"),
+    ("local_reduce_rs", 2, 8, "fp32", "prod"), ("local_reduce_rs", 1, 100, "fp32", "sum"),
+    ("local_reduce_rs", 12, 4104, "fp16", "sum"), ("local_reduce_rs", 31, 4096, "bf16", "max"),
+    ("local_reduce_rs", 32, 8200, "fp32", "sum"), ("local_reduce_rs", 4, 0, "fp32", "sum"),
+    ("chunk_mesh", 8, 1 << 20, "bf16", "sum"), ("chunk_mesh", 7, 100003, "fp32", "sum"),
+    ("chunk_mesh", 6, 16385, "fp16", "max"), ("chunk_mesh", 5, 70001, "int8", "sum"),
+    ("chunk_mesh", 16, 400007, "int32", "min"), ("chunk_mesh", 3, 1001, "int16", "sum"),
+    ("chunk_mesh", 2, 9, "fp32", "prod"), ("chunk_mesh", 1, 100, "fp32", "sum"), ("chunk_mesh", 4, 0, "fp32", "sum"),
+    ("chunk_mesh", 12, 77777, "fp16", "sum"), ("chunk_mesh", 31, 300007, "bf16", "max"),
+    ("chunk_mesh", 32, 1 << 20, "fp32", "sum"), ("chunk_mesh", 8, 100, "fp32", "sum"),  # most sub-chunks empty
+]
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", USER_BUFFER_FUSED)
+def test_fused_lowerings_on_the_user_buffers(gpu_thread, alg, n, count, dtype, op):
+    """One tree launch in place of the deterministic reduce-scatter's slot writes and halving rounds, and one chain
+    launch per group of ranks in place of the chunk-mesh allreduce's rounds and gather: the user outputs hold the
+    oracle's bits, the inputs are only read, and no communication buffer is asked for."""
+    say("fused on user buffers", alg, n, count, dtype, op)
     dt, o = DT[dtype], OPS[op]
-    host_in = [gen(dt, n * count, 7000 + r, "prod" if op == "prod" else "default") for r in range(n)]
-    sentinel = gen(dt, count, 999, "wide")
+    in_count, out_count = buffer_counts(alg, n, count)
+    host_in = [gen(dt, in_count, 7000 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    sentinel = gen(dt, out_count, 999, "wide")
     want_in = [x.copy() for x in host_in]
     want_out = [sentinel.copy() for _ in range(n)]
-    sb = h.scratch_bytes(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, n, count, dt)
-    oracle.run(oracle.ALG_RS_LOCAL_REDUCE, want_in, want_out, count, dt, o,
+    sb = h.scratch_bytes(ALGS[alg][0], n, count, dt)
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o,
                scratch=[np.zeros(sb, np.uint8) for _ in range(n)] if sb else None)
     d_in = [to_dev(x) for x in host_in]
     d_out = [to_dev(sentinel) for _ in range(n)]
     pad = to_dev(np.zeros(256, np.uint8))
     ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
-    plan = h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out],
-                  count, dt, o)
+    plan = h.Plan(ALGS[alg][0], h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
     try:
-        assert plan.info.launches == (1 if count else 0)
-        assert plan.launches()[0].kind == (h.Kernel.TREE if n > 1 else h.Kernel.COPY) if count else True
-        if n > 1:
-            assert plan.info.movedBytes == (n + 1) * n * count * host_in[0].itemsize
+        unit = host_in[0].itemsize
+        if alg == "local_reduce_rs":
+            assert plan.info.launches == (1 if count else 0)
+            if n > 1:
+                assert plan.info.movedBytes == (n + 1) * n * count * unit
+        elif n > 1:
+            per_launch = 32 // (n - 1)               # whole ranks' sub-chunks per launch, 32 segments at most
+            assert plan.info.launches <= -(-n // per_launch)
+            assert plan.info.movedBytes == 2 * n * count * unit
+        for rec in plan.launches():
+            assert rec.kind == (h.Kernel.COPY if n == 1 else h.Kernel.TREE if alg == "local_reduce_rs" else h.Kernel.CHAIN)
         assert plan.run(gpu_thread) == 0
         assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
         for r in range(n):

@@ -399,6 +399,22 @@ def test_fused_deterministic_reduce_scatter_is_one_tree_launch_with_the_hand_der
         assert e.value.code == R.E_PTR
 
 
+def test_fused_chunk_mesh_is_chain_launches_over_whole_ranks_sub_chunks():
+    for n, count, launches, nseg in ((2, 1 << 20, 1, [2]), (6, 1 << 20, 1, [30]), (8, 1 << 20, 2, [28, 28]),
+                                     (17, 1 << 22, 9, [32] * 8 + [16]), (32, 1 << 22, 32, [31] * 32), (8, 100, 1, [4])):
+        i, o = ptrs(n, 1 << 26)
+        p = h.Plan(h.Alg.ALLREDUCE_CHUNK_MESH, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM)   # no scratch buffers
+        recs = p.launches()
+        assert [r.kind for r in recs] == [h.Kernel.CHAIN] * launches, n
+        assert [r.nseg for r in recs] == nseg, n
+        assert sum(r.bytes for r in recs) == 4 * count                 # every element of the message folded once
+        assert p.info.movedBytes == 2 * n * 4 * count                  # n reads and n writes per element
+        q = h.Plan(h.Alg.ALLREDUCE_CHUNK_MESH, h.Lowering.STEPWISE, i, o, count, DT.FP32, OP.SUM, 0, ptrs(n, 1 << 26)[0])
+        assert p.info.algorithmicBytes == q.info.algorithmicBytes
+        p.destroy()
+        q.destroy()
+
+
 def test_counts_whose_byte_offsets_would_leave_64_bits_are_refused():
     i, o = ptrs(4, 4096)
     for count in (2**48 + 1, 2**62, 2**64 - 1):
