@@ -210,8 +210,6 @@ def main():
         args.lowering = "stepwise"  # composed from the step lists of its levels
     d_scr = [torch.zeros(scratch_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if scratch_bytes else None
     scr_ptrs = [t.data_ptr() for t in d_scr] if d_scr else None
-    if alg_name == "local_reduce" and args.lowering == "both":
-        args.lowering = "stepwise"  # this schedule has no fused lowering
     kname = {h.Kernel.REDUCE2: "k_reduce2", h.Kernel.CHAIN: "k_fold_chain", h.Kernel.TREE: "k_fold_tree",
              h.Kernel.COPY: "k_copy", h.Kernel.BYTEWISE: "k_bytewise"}
 

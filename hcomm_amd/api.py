@@ -14,7 +14,7 @@ except ImportError:  # a pure C / ctypes caller without torch uses the system ru
     pass
 
 __all__ = [
-    "lib", "LIB_PATH", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
+    "lib", "LIB_PATH", "plan_tree", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
     "LaunchRecord", "PlanInfo", "SchedOp", "Slice", "HcommError", "check",
     "HcommLocalCopyOnThread", "HcommLocalReduceOnThread", "HcommThreadAlloc", "HcommThreadFree",
     "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
@@ -188,6 +188,8 @@ _plan_destroy = _sig("HcommGfxPlanDestroy", _i32, _vp)
 _plan_graph = _sig("HcommGfxPlanSetGraphReplay", _i32, _vp, _i32)
 _plan_info = _sig("HcommGfxPlanGetInfo", _i32, _vp, C.POINTER(PlanInfo))
 _plan_launch = _sig("HcommGfxPlanGetLaunch", _i32, _vp, _u32, C.POINTER(LaunchRecord))
+_plan_tree_segment = _sig("HcommGfxPlanGetTreeSegment", _i32, _vp, _u32, _u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
+                         C.POINTER(_u64), C.POINTER(_u64))
 _sched_emit = _sig("HcommGfxScheduleEmitStrided", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
                    C.POINTER(_u64))
 HcommWriteOnThread = _sig("HcommWriteOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
@@ -366,6 +368,26 @@ class Plan:
             self.destroy()
         except Exception:
             pass
+
+
+def plan_tree(plan, launch, segment, rank_of=None):
+    """(tree, offset, bytes) of one segment of a tree launch of any plan object: the nested [dst, src] lists the
+    kernel's fold pattern makes of the leaf positions (level l folds position q + 2^l onto q, holes skipped); a leaf
+    is the input pointer read there, or rank_of[pointer] when a mapping is given."""
+    k, off, nbytes = _u32(0), _u64(0), _u64(0)
+    check(_plan_tree_segment(plan._p, launch, segment, None, 0, C.byref(k), C.byref(off), C.byref(nbytes)),
+          "HcommGfxPlanGetTreeSegment")
+    leaves = (_vp * k.value)()
+    check(_plan_tree_segment(plan._p, launch, segment, leaves, k.value, C.byref(k), None, None),
+          "HcommGfxPlanGetTreeSegment")
+    x = [None if not v else (rank_of[v] if rank_of is not None else v) for v in leaves]
+    step = 1
+    while step < k.value:
+        for q in range(0, k.value, 2 * step):
+            if x[q + step] is not None:
+                x[q] = [x[q], x[q + step]]
+        step *= 2
+    return x[0], off.value, nbytes.value
 
 
 # ---- the op-base loop around a template ------------------------------------------------------------------

@@ -14,6 +14,7 @@
 extern "C" {
 #endif
 
+#define HG_POS_BYTES 256u      /* leaf-position bytes of a tree launch */
 #define HG_MAX_SEG 32u          /* segments per k-way fold launch */
 #define HG_MAX_SEG2 64u         /* segments per copy / two-input reduce launch */
 #define HG_VEC_BYTES 16u        /* one lane moves 128 bits per access */
@@ -48,7 +49,8 @@ typedef struct {
  * truncated trees of the nonuniform hierarchical ring / nonuniform Bruck schedules), or, when tree == 4, from
  * in[pos[j]] where pos[j] names a rank (the rank-order trees of the order-preserving executors, laid out by the host;
  * inputs only read), or, when tree == 5, from in[(first[s] - pos[j]) mod nranks] (the deterministic mesh
- * reduce-scatter's row of receive slots; inputs only read).
+ * reduce-scatter's row of receive slots; inputs only read), or, when tree == 6, from in[pos[s * k + j]] (any
+ * tree of depth log2 k per segment, laid out by the host from the schedule's own operation list; inputs only read).
  */
 typedef struct {
     const void* in[HCOMM_GFX_MAX_RANKS];
@@ -65,7 +67,7 @@ typedef struct {
     uint32_t store_partials; /* store the running value to position j's buffer after fold step j >= 1 */
     uint32_t store_final_first; /* store the final value to position 0's buffer */
     uint32_t out_mode;       /* 0 none, 1 out[owner[s]] + out_off[s], 2 every out[r] + off[s] */
-    uint32_t tree;           /* 0 chain; binary tree over k = 2^L positions: 1 recursive halving, 2 / 3 rotation + / -, 4 leaves from pos[] */
+    uint32_t tree;           /* 0 chain; binary tree over k = 2^L positions: 1 recursive halving, 2 / 3 rotation + / -, 4 / 5 / 6 leaves from pos[] */
     uint32_t nout;           /* tree only: number of out[] entries that receive the result */
     uint32_t ascending;      /* chain only: 1 = position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s];
                               * 2 = position 0 is first[s], position j >= 1 is first[s] + 1 + (start[s] + j - 1) mod (nranks - 1):
@@ -74,7 +76,10 @@ typedef struct {
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
     uint8_t start[HG_MAX_SEG]; /* chain with ascending == 2 only */
-    uint8_t pos[HCOMM_GFX_MAX_RANKS]; /* tree == 4: the rank at leaf position q (tree == 5: how far below the segment's first rank it lies), or 255 where the tree has a hole */
+    /* tree == 4: the rank at leaf position q (tree == 5: how far below the segment's first rank it lies), or 255 where
+     * the tree has a hole; tree == 6: a table of k entries per segment, segment s at pos[s * k ..], so that every
+     * segment can have a tree of its own shape (nseg * k <= HG_POS_BYTES) */
+    uint8_t pos[HG_POS_BYTES];
 } HgFoldTable;
 
 /* Launch geometry decided on the host so that recorder threads can report it without a GPU. */

@@ -85,6 +85,8 @@ __device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t
 // 1 onto 0); over servers x devices the low position bits walk a server's devices like that and the high bits the
 // servers.  tree == 5 reads tab.pos[] as distances instead: position q of segment s holds rank first[s] - pos[q]
 // (mod n), the row of the deterministic mesh reduce-scatter, whose slot j - 1 is filled by rank d - j.
+// tree == 6 gives every segment a table of its own (tab.pos[s * K + q]): trees of any shape up to depth L, a subtree
+// that is shallower than its span sitting at the span's start with holes behind it.
 // A hole's left neighbour always exists; the inputs are only read.
 template <class Item, int L, uint32_t NU>
 __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint32_t s, const bool (&live)[NU],
@@ -104,7 +106,7 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         if (order) {
-            b[q] = tab.pos[q];
+            b[q] = tab.pos[(tab.tree == 6u ? s * K : 0u) + q];
             have[q] = b[q] < n;
             if (dist && have[q]) {
                 b[q] = c + n - b[q];

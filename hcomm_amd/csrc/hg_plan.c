@@ -483,8 +483,174 @@ static int fused_chunk_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* 
     return rc;
 }
 
-static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, void* const* out, uint64_t count,
-                       uint64_t stride, int dtype, int op)
+/* ---- a schedule's own expression trees as one tree launch ------------------------------------------------------
+ *
+ * The operation list is replayed on symbols: a cell is an exact byte range of one buffer, its value a node - a leaf
+ * (rank, offset: the range of that rank's input) or a fold (dst node, src node).  What ends up in the output cells
+ * are the trees the kernel must evaluate; they are laid out over 2^depth leaf positions so that the kernel's fixed
+ * pattern (level l folds position q + 2^l onto q) walks them with every dst operand on the left.  Lists that write
+ * an input, read a range with other bounds than it was written with, or leave different trees in different ranks'
+ * outputs are refused (HCCL_E_NOT_SUPPORT). */
+typedef struct {
+    uint32_t rank, buf;
+    uint64_t off, bytes;
+    int32_t node;
+} SymCell;
+
+typedef struct {
+    int32_t left, right; /* -1, -1: a leaf */
+    uint32_t rank;
+    uint64_t off;
+} SymNode;
+
+typedef struct {
+    SymCell* cell;
+    SymNode* node;
+    uint32_t ncell, nnode, cap;
+} SymState;
+
+static int32_t sym_find(const SymState* st, uint32_t rank, uint32_t buf, uint64_t off, uint64_t bytes)
+{
+    for (uint32_t i = 0; i < st->ncell; ++i) {
+        const SymCell* c = &st->cell[i];
+        if (c->rank != rank || c->buf != buf) continue;
+        if (c->off == off && c->bytes == bytes) return (int32_t)i;
+        if (c->off < off + bytes && off < c->off + c->bytes) return -2; /* other bounds */
+    }
+    return -1;
+}
+
+static int32_t sym_node(SymState* st, int32_t left, int32_t right, uint32_t rank, uint64_t off)
+{
+    SymNode* n = &st->node[st->nnode];
+    n->left = left;
+    n->right = right;
+    n->rank = rank;
+    n->off = off;
+    return (int32_t)st->nnode++;
+}
+
+static uint32_t sym_depth(const SymState* st, int32_t node)
+{
+    if (st->node[node].left < 0) return 0;
+    const uint32_t a = sym_depth(st, st->node[node].left), b = sym_depth(st, st->node[node].right);
+    return 1u + (a > b ? a : b);
+}
+
+/* node into the span of 2^h positions that starts at q; 0 when a leaf lies at another offset than the segment */
+static int sym_place(const SymState* st, int32_t node, uint8_t* pos, uint32_t q, uint32_t h, uint64_t off)
+{
+    const SymNode* n = &st->node[node];
+    if (n->left < 0) {
+        pos[q] = (uint8_t)n->rank;
+        return n->off == off;
+    }
+    return sym_place(st, n->left, pos, q, h - 1, off) && sym_place(st, n->right, pos, q + (1u << (h - 1)), h - 1, off);
+}
+
+static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, void* const* in, void* const* out, int dtype,
+                            int op)
+{
+    SymState st;
+    memset(&st, 0, sizeof(st));
+    st.cap = (uint32_t)(2 * ol->n + 1);
+    st.cell = (SymCell*)calloc(st.cap, sizeof(SymCell));
+    st.node = (SymNode*)calloc(st.cap, sizeof(SymNode));
+    HgLaunch* l = NULL;
+    int rc = (st.cell && st.node) ? HCCL_SUCCESS : HCCL_E_MEMORY;
+    for (uint64_t i = 0; i < ol->n && rc == HCCL_SUCCESS; ++i) {
+        const HcommGfxSchedOp* o = &ol->ops[i];
+        if (o->bytes == 0) continue;
+        if (o->dstBuf == 0) rc = HCCL_E_NOT_SUPPORT; /* the inputs must stay as they are */
+        int32_t src = sym_find(&st, o->srcRank, o->srcBuf, o->srcOff, o->bytes);
+        if (src == -1 && o->srcBuf == 0) { /* first read of an input range: a leaf */
+            SymCell* c = &st.cell[st.ncell];
+            c->rank = o->srcRank;
+            c->buf = 0;
+            c->off = o->srcOff;
+            c->bytes = o->bytes;
+            c->node = sym_node(&st, -1, -1, o->srcRank, o->srcOff);
+            src = (int32_t)st.ncell++;
+        }
+        int32_t dst = sym_find(&st, o->rank, o->dstBuf, o->dstOff, o->bytes);
+        if (src < 0 || dst == -2 || (dst == -1 && o->kind)) rc = HCCL_E_NOT_SUPPORT;
+        if (rc != HCCL_SUCCESS) break;
+        if (dst == -1) {
+            SymCell* c = &st.cell[st.ncell];
+            c->rank = o->rank;
+            c->buf = o->dstBuf;
+            c->off = o->dstOff;
+            c->bytes = o->bytes;
+            dst = (int32_t)st.ncell++;
+        }
+        st.cell[dst].node = o->kind ? sym_node(&st, st.cell[dst].node, st.cell[src].node, 0, 0) : st.cell[src].node;
+    }
+    /* the output cells of rank 0 are the segments; every other rank must hold the same trees at the same places */
+    uint32_t nseg = 0, depth = 1;
+    for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
+        const SymCell* c = &st.cell[i];
+        if (c->buf != 1) continue;
+        if (c->rank == 0) {
+            ++nseg;
+            const uint32_t d = sym_depth(&st, c->node);
+            if (d > depth) depth = d;
+            for (uint32_t r = 1; r < n; ++r) {
+                const int32_t j = sym_find(&st, r, 1, c->off, c->bytes);
+                if (j < 0 || st.cell[j].node != c->node) rc = HCCL_E_NOT_SUPPORT;
+            }
+        } else if (sym_find(&st, 0, 1, c->off, c->bytes) < 0) {
+            rc = HCCL_E_NOT_SUPPORT;
+        }
+    }
+    if (rc == HCCL_SUCCESS && (1u << depth) > HCOMM_GFX_MAX_RANKS) rc = HCCL_E_NOT_SUPPORT; /* the kernel folds 32 positions at most */
+    const uint32_t k = 1u << depth;
+    const uint32_t per_launch = HG_POS_BYTES / k < HG_MAX_SEG ? HG_POS_BYTES / k : HG_MAX_SEG;
+    for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
+        const SymCell* c = &st.cell[i];
+        if (c->buf != 1 || c->rank != 0) continue;
+        if (!l) {
+            l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+            if (!l) {
+                rc = HCCL_E_MEMORY;
+                break;
+            }
+            l->kind = HCOMM_GFX_KERNEL_TREE;
+            l->dtype = (uint32_t)dtype;
+            l->op = (uint32_t)op;
+            HgFoldTable* f = &l->tab.fold;
+            f->tree = 6u;
+            f->k = k;
+            f->nranks = n;
+            f->nout = n;
+            f->out_mode = 2u;
+            memset(f->pos, 255, sizeof(f->pos));
+            for (uint32_t r = 0; r < n; ++r) {
+                f->in[r] = in[r];
+                f->out[r] = out[r];
+            }
+        }
+        HgFoldTable* f = &l->tab.fold;
+        const uint32_t s = f->nseg++;
+        f->off[s] = c->off;
+        f->bytes[s] = c->bytes;
+        /* 128-bit accesses: a segment must start on a 16-byte boundary of every buffer */
+        if ((c->off & (HG_VEC_BYTES - 1u)) || !sym_place(&st, c->node, f->pos + s * k, 0, depth, c->off)) rc = HCCL_E_NOT_SUPPORT;
+        --nseg;
+        if (rc == HCCL_SUCCESS && (f->nseg == per_launch || nseg == 0)) {
+            hg_finish_fold(l);
+            rc = plan_push(l, p);
+            free(l);
+            l = NULL;
+        }
+    }
+    free(l);
+    free(st.cell);
+    free(st.node);
+    return rc;
+}
+
+static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n, void* const* in, void* const* out,
+                       uint64_t count, uint64_t stride, int dtype, int op)
 {
     const uint64_t total = count * HcommGfxDataTypeSize((HcommDataType)dtype);
     switch (alg) {
@@ -518,6 +684,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, uint32_t n, void* const* in, vo
         case HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_chunk_mesh(p, n, in, out, count, dtype, op);
+        case HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return ol ? fused_from_trees(p, ol, n, in, out, dtype, op) : HCCL_E_NOT_SUPPORT;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rs_local_reduce(p, n, in, out, count, dtype, op);
@@ -595,7 +764,7 @@ int32_t HcommGfxPlanCreateEx(
     if (lowering == HCOMM_GFX_LOWER_STEPWISE)
         rc = lower_stepwise(p, &ol, in, out, scratch, (int)dataType, (int)reduceOp);
     else
-        rc = lower_fused(p, (int)alg, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
+        rc = lower_fused(p, (int)alg, &ol, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
     hg_oplist_free(&ol);
     if (rc != HCCL_SUCCESS) {
         HcommGfxPlanDestroy(p);
@@ -636,6 +805,8 @@ int32_t HcommGfxOpBasePlanCreate(
     const uint64_t maxc = hg_opbase_max_count((int)alg, nRanks, cclBytes, unit);
     const uint64_t chunk = count < maxc ? count : maxc;
     if (nRanks > 1 && chunk > 0 && hg_scratch_bytes((int)alg, nRanks, chunk, (int)dataType) > 0) {
+        /* their single-launch lowerings leave the communication buffers alone, the loop's replay does not */
+        if (lowering == HCOMM_GFX_LOWER_FUSED) return HCCL_E_NOT_SUPPORT;
         rc = check_bufs(scratch, nRanks);
         if (rc != HCCL_SUCCESS) return rc;
     }
@@ -665,7 +836,7 @@ int32_t HcommGfxOpBasePlanCreate(
             uint64_t k = j;
             while (k < ol.n && ol.ops[k].dstBuf != HCOMM_GFX_BUF_USER_OUT) ++k;
             const uint64_t cur = count - done > maxc ? maxc : count - done;
-            if (rc == HCCL_SUCCESS) rc = lower_fused(p, (int)alg, nRanks, cclIn, cclOut, cur, cur, (int)dataType, (int)reduceOp);
+            if (rc == HCCL_SUCCESS) rc = lower_fused(p, (int)alg, NULL, nRanks, cclIn, cclOut, cur, cur, (int)dataType, (int)reduceOp);
             uint64_t m = k;
             while (m < ol.n && ol.ops[m].dstBuf == HCOMM_GFX_BUF_USER_OUT) ++m;
             if (rc == HCCL_SUCCESS) rc = lower_ops(p, &ol.ops[k], m - k, bufs, (int)dataType, (int)reduceOp);
@@ -1135,5 +1306,36 @@ int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaun
     rec->nseg = l->nseg;
     rec->bytes = l->bytes;
     rec->blocks = l->blocks;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanGetTreeSegment(const HcommGfxPlan* plan, uint32_t i, uint32_t segment, const void** leaves,
+                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes)
+{
+    if (!plan || plan->magic != HG_PLAN_MAGIC || !k) return HCCL_E_PTR;
+    if (i >= plan->nlaunch) return HCCL_E_PARA;
+    const HgLaunch* l = &plan->launches[i];
+    const HgFoldTable* f = &l->tab.fold;
+    if (l->kind != HCOMM_GFX_KERNEL_TREE || segment >= f->nseg) return HCCL_E_PARA;
+    *k = f->k;
+    if (offset) *offset = f->off[segment];
+    if (bytes) *bytes = f->bytes[segment];
+    if (!leaves) return HCCL_SUCCESS;
+    if (cap < f->k) return HCCL_E_PARA;
+    const uint32_t n = f->nranks, c = f->first[segment];
+    uint32_t bits = 0;
+    while ((1u << bits) < f->k) ++bits;
+    for (uint32_t q = 0; q < f->k; ++q) {
+        uint32_t b = 255;
+        switch (f->tree) {
+            case 1u: b = c ^ bitrev_n(q, bits); break;
+            case 2u: b = q < n ? (c + q) % n : 255u; break;
+            case 3u: b = q < n ? (c + n - q) % n : 255u; break;
+            case 4u: b = f->pos[q]; break;
+            case 5u: b = f->pos[q] < n ? (c + n - f->pos[q]) % n : 255u; break;
+            default: b = f->pos[segment * f->k + q]; break;
+        }
+        leaves[q] = b < n ? f->in[b] : NULL;
+    }
     return HCCL_SUCCESS;
 }

@@ -511,6 +511,18 @@ int32_t HcommGfxPlanGetInfo(const HcommGfxPlan* plan, HcommGfxPlanInfo* info);
 int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaunchRecord* rec);
 
 /*
+ * The reduction tree launch i (a HCOMM_GFX_KERNEL_TREE launch) evaluates for its segment `segment`, for inspection and
+ * for checking a single-launch lowering against the schedule it stands for without a GPU.  The tree has *k = 2^L leaf
+ * positions; leaves[q] receives the rank buffer (the in[] pointer the plan was built with) read at position q, or NULL
+ * where the tree has a hole; the element at byte *offset + x of every leaf is folded level by level, level l folding
+ * position q + 2^l (src role) onto position q (dst role) for every q that is a multiple of 2^(l+1), holes skipped.
+ * leaves may be NULL to query *k; cap < *k -> HCCL_E_PARA.  No counterpart in the reference: its schedules
+ * are only ever run step by step.
+ */
+int32_t HcommGfxPlanGetTreeSegment(const HcommGfxPlan* plan, uint32_t i, uint32_t segment, const void** leaves,
+                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes);
+
+/*
  * The schedule as the reference's templates emit it, one two-input operation per record, for inspection
  * and for checking a plan against an independent replay.
  */

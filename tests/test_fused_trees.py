@@ -1,0 +1,245 @@
+"""The reduction trees of the single-launch lowerings, read back from the plans, against the expression trees a
+symbolic replay of the ORACLE's operation list leaves in the outputs (a different generator from the product's), and
+against the hand-derived trees of the golden file.  No GPU: plans are built on made-up addresses."""
+import json
+import os
+
+import pytest
+
+import oracle
+import hcomm_amd as h
+from hcomm_amd import HcclResult as R
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "schedules_hand_derived.json")))
+BASE = 0x7f0000000000
+
+
+def ptrs(n):
+    ins = [BASE + r * (1 << 32) for r in range(n)]
+    outs = [BASE + (64 + r) * (1 << 32) for r in range(n)]
+    return ins, outs, {p: r for r, p in enumerate(ins)}
+
+
+def output_trees(ops, n):
+    """{(offset, bytes): tree} of rank 0's output after a symbolic replay; asserts that every rank's output holds the
+    same trees.  A leaf is (rank, input offset); a fold is [dst, src]."""
+    cells = {}
+    for step, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes in ops:
+        if nbytes == 0:
+            continue
+        skey, dkey = (srank, sbuf, soff, nbytes), (rank, dbuf, doff, nbytes)
+        if skey not in cells:
+            assert sbuf == 0, "read of a range that was never written with these bounds"
+            cells[skey] = (srank, soff)
+        assert dbuf != 0 or not kind or dkey in cells or True
+        if kind:
+            if dkey not in cells:
+                assert dbuf == 0
+                cells[dkey] = (rank, doff)
+            cells[dkey] = [cells[dkey], cells[skey]]
+        else:
+            cells[dkey] = cells[skey]
+    per_rank = [{(k[2], k[3]): v for k, v in cells.items() if k[0] == r and k[1] == 1} for r in range(n)]
+    return per_rank
+
+
+def strip(tree, off):
+    """(rank, offset) leaves -> rank, checking that every leaf is read at the segment's own offset."""
+    if isinstance(tree, tuple):
+        assert tree[1] == off
+        return tree[0]
+    return [strip(tree[0], off), strip(tree[1], off)]
+
+
+def plan_segments(plan, rank_of):
+    out = {}
+    for i, rec in enumerate(plan.launches()):
+        assert rec.kind == h.Kernel.TREE
+        for s in range(rec.nseg):
+            tree, off, nbytes = h.plan_tree(plan, i, s, rank_of)
+            out[(off, nbytes)] = tree
+    return out
+
+
+@pytest.mark.parametrize("n", [2, 4, 8, 16])
+@pytest.mark.parametrize("count,dtype", [(1 << 20, oracle.F32), (300007 * 16, oracle.BF16), (16 * 8192 + 40, oracle.I8)])
+def test_deterministic_mesh_allreduce_single_launch_trees_equal_the_replay(n, count, dtype):
+    ins, outs, rank_of = ptrs(n)
+    plan = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, count, dtype, oracle.SUM)
+    try:
+        got = plan_segments(plan, rank_of)
+        per_rank = output_trees(oracle.trace(oracle.ALG_ALLREDUCE_LOCAL_REDUCE, n, count, dtype), n)
+        for r in range(1, n):
+            assert per_rank[r] == per_rank[0]
+        want = {k: strip(v, k[0]) for k, v in per_rank[0].items()}
+        assert got == want
+        unit = h.DTYPE_SIZE[dtype]
+        assert sum(b for _, b in got) == count * unit
+        assert plan.info.movedBytes == 2 * n * count * unit      # n reads and n writes per element, nothing else
+    finally:
+        plan.destroy()
+
+
+def test_deterministic_mesh_allreduce_single_launch_trees_hand_derived():
+    for n_s, trees in GOLD["local_reduce_slice_tree"].items():
+        n = int(n_s)
+        ins, outs, rank_of = ptrs(n)
+        count = n * 4096 * 4 + 5000                              # 16 KiB slots, ragged last slice
+        plan = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, count, oracle.F32, oracle.SUM)
+        got = plan_segments(plan, rank_of)
+        per = h.scratch_bytes(h.Alg.ALLREDUCE_LOCAL_REDUCE, n, count, oracle.F32) // n
+        assert {off // per: t for (off, _), t in got.items()} == {int(d): t for d, t in trees.items()}
+        plan.destroy()
+
+
+def test_deterministic_mesh_allreduce_single_launch_limits():
+    ins, outs, _ = ptrs(32)
+    with pytest.raises(h.HcommError) as e:                       # depth 6: more leaf positions than the kernel folds
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 1 << 22, oracle.F32, oracle.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT
+    ins, outs, _ = ptrs(4)
+    with pytest.raises(h.HcommError) as e:                       # slots of 10 bytes: slices off 16-byte boundaries
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 38, oracle.I8, oracle.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT
+    with pytest.raises(h.HcommError) as e:                       # as the step-wise replay: powers of two only
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins[:3], outs[:3], 4096, oracle.F32, oracle.SUM)
+    assert e.value.code == R.E_PARA
+    p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins[:1], outs[:1], 4096, oracle.F32, oracle.SUM)
+    assert [r.kind for r in p.launches()] == [h.Kernel.COPY]
+    p.destroy()
+    p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 0, oracle.F32, oracle.SUM)
+    assert p.launches() == []
+    p.destroy()
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 6, 7, 8, 12, 16, 17, 31, 32])
+def test_deterministic_mesh_reduce_scatter_single_launch_trees_equal_the_replay(n):
+    ins, outs, rank_of = ptrs(n)
+    count, dtype = 4096, oracle.F32
+    plan = h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, count, dtype, oracle.SUM)
+    try:
+        got = plan_segments(plan, rank_of)
+        per_rank = output_trees(oracle.trace(oracle.ALG_RS_LOCAL_REDUCE, n, count, dtype), n)
+        for d in range(n):
+            assert list(per_rank[d]) == [(0, count * 4)]
+            assert got[(d * count * 4, count * 4)] == strip(per_rank[d][(0, count * 4)], d * count * 4), d
+        if str(n) in GOLD["rs_local_reduce_rank_tree"]:
+            for d_s, tree in GOLD["rs_local_reduce_rank_tree"][str(n)].items():
+                assert got[(int(d_s) * count * 4, count * 4)] == tree
+    finally:
+        plan.destroy()
+
+
+@pytest.mark.parametrize("alg,oalg", [(h.Alg.ALLREDUCE_NHR, oracle.ALG_ALLREDUCE_NHR), (h.Alg.ALLREDUCE_NB, oracle.ALG_ALLREDUCE_NB),
+                                      (h.Alg.ALLREDUCE_NHR_ONESHOT, oracle.ALG_ALLREDUCE_NHR_ONESHOT)])
+@pytest.mark.parametrize("n", [2, 3, 5, 6, 8, 13, 16, 32])
+def test_rotation_tree_launches_equal_the_replay(alg, oalg, n):
+    """The same read-back for the older tree lowerings (their launches also store partials into the inputs, which
+    the replayed outputs do not show; the GPU tests compare those)."""
+    ins, outs, rank_of = ptrs(n)
+    count, dtype = 100003, oracle.F32
+    plan = h.Plan(alg, h.Lowering.FUSED, ins, outs, count, dtype, oracle.SUM)
+    try:
+        got = plan_segments(plan, rank_of)
+        per_rank = output_trees_in_place(oracle.trace(oalg, n, count, dtype), n)
+        for r in range(n):
+            assert merged_runs(per_rank[r]) == merged_runs(got), r
+    finally:
+        plan.destroy()
+
+
+@pytest.mark.parametrize("n", [2, 4, 8, 16, 32])
+def test_halving_tree_launch_equals_the_replay(n):
+    """Recursive halving-doubling on a power-of-two rank count (with other counts the launch first absorbs the odd
+    neighbours, which this read-back does not show; the GPU tests cover them)."""
+    ins, outs, rank_of = ptrs(n)
+    plan = h.Plan(h.Alg.ALLREDUCE_RHD, h.Lowering.FUSED, ins, outs, 100003, oracle.F32, oracle.SUM)
+    try:
+        per_rank = output_trees_in_place(oracle.trace(oracle.ALG_ALLREDUCE_RHD, n, 100003, oracle.F32), n)
+        for r in range(n):
+            assert merged_runs(per_rank[r]) == merged_runs(plan_segments(plan, rank_of)), r
+    finally:
+        plan.destroy()
+
+
+def merged_runs(segments):
+    """[(lo, hi, tree)] with neighbours that hold the same tree joined: independent of how the bytes were cut."""
+    out = []
+    for (off, nbytes), tree in sorted(segments.items()):
+        if out and out[-1][1] == off and out[-1][2] == tree:
+            out[-1] = (out[-1][0], off + nbytes, tree)
+        else:
+            out.append((off, off + nbytes, tree))
+    return out
+
+
+def output_trees_in_place(ops, n):
+    """As output_trees for schedules that reduce inside the input buffers and whose steps run in parallel: reads see
+    the state before the step; ranges are tracked per byte span so that a gather of several slices at once resolves."""
+    state = {}                                                   # (rank, buf) -> sorted list of [lo, hi, tree, lo0]
+    def read(rank, buf, off, nbytes):
+        out, pos = [], off
+        for lo, hi, tree in sorted(state.get((rank, buf), [])):
+            if hi <= off or lo >= off + nbytes:
+                continue
+            assert lo >= pos or lo <= off
+            if lo > pos:
+                assert buf == 0
+                out.append((pos, lo, ("in", rank)))
+            out.append((max(lo, off), min(hi, off + nbytes), tree))
+            pos = min(hi, off + nbytes)
+        if pos < off + nbytes:
+            assert buf == 0, "read of unwritten memory"
+            out.append((pos, off + nbytes, ("in", rank)))
+        return out
+    def write(rank, buf, pieces):
+        cur = state.setdefault((rank, buf), [])
+        for lo, hi, tree in pieces:
+            nxt = []
+            for a, b, t in cur:
+                if b <= lo or a >= hi:
+                    nxt.append((a, b, t))
+                else:
+                    if a < lo:
+                        nxt.append((a, lo, t))
+                    if b > hi:
+                        nxt.append((hi, b, t))
+            nxt.append((lo, hi, tree))
+            cur[:] = nxt
+    by_step = {}
+    for o in ops:
+        by_step.setdefault(o[0], []).append(o)
+    for step in sorted(by_step):
+        pending = []
+        for _, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes in by_step[step]:
+            if nbytes == 0:
+                continue
+            src = read(srank, sbuf, soff, nbytes)
+            if kind:
+                dst = read(rank, dbuf, doff, nbytes)
+                cuts = sorted({p for lo, hi, _ in src for p in (lo - soff, hi - soff)} | {p for lo, hi, _ in dst for p in (lo - doff, hi - doff)})
+                pieces = []
+                for a, b in zip(cuts, cuts[1:]):
+                    s = [t for lo, hi, t in src if lo - soff <= a and b <= hi - soff][0]
+                    d = [t for lo, hi, t in dst if lo - doff <= a and b <= hi - doff][0]
+                    pieces.append((doff + a, doff + b, ("f", d, s, doff - soff)))
+                pending.append((rank, dbuf, pieces))
+            else:
+                pending.append((rank, dbuf, [(lo - soff + doff, hi - soff + doff, ("m", t, doff - soff)) for lo, hi, t in src]))
+        for rank, dbuf, pieces in pending:
+            write(rank, dbuf, pieces)
+    def simplify(t):
+        if t[0] == "in":
+            return t[1]
+        if t[0] == "m":
+            assert t[2] == 0, "a copy between different offsets"
+            return simplify(t[1])
+        assert t[3] == 0
+        return [simplify(t[1]), simplify(t[2])]
+    per_rank = []
+    for r in range(n):
+        merged = {}
+        for lo, hi, t in sorted(state.get((r, 1), [])):
+            merged[(lo, hi - lo)] = simplify(t)
+        per_rank.append(merged)
+    return per_rank

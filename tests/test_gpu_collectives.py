@@ -215,14 +215,20 @@ USER_BUFFER_FUSED = [
     ("chunk_mesh", 2, 9, "fp32", "prod"), ("chunk_mesh", 1, 100, "fp32", "sum"), ("chunk_mesh", 4, 0, "fp32", "sum"),
     ("chunk_mesh", 12, 77777, "fp16", "sum"), ("chunk_mesh", 31, 300007, "bf16", "max"),
     ("chunk_mesh", 32, 1 << 20, "fp32", "sum"), ("chunk_mesh", 8, 100, "fp32", "sum"),  # most sub-chunks empty
+    ("local_reduce", 8, 1 << 20, "bf16", "sum"), ("local_reduce", 4, 100003, "fp32", "sum"),
+    ("local_reduce", 16, 70001 * 16, "fp16", "max"), ("local_reduce", 2, 4099, "int8", "sum"),
+    ("local_reduce", 8, 300007, "int32", "min"), ("local_reduce", 4, 65536, "fp32", "prod"),
+    ("local_reduce", 16, 1 << 20, "bf16", "sum"), ("local_reduce", 8, 8 * 8192 + 24, "int16", "sum"),
+    ("local_reduce", 1, 100, "fp32", "sum"), ("local_reduce", 4, 0, "fp32", "sum"),
 ]
 
 
 @pytest.mark.parametrize("alg,n,count,dtype,op", USER_BUFFER_FUSED)
 def test_fused_lowerings_on_the_user_buffers(gpu_thread, alg, n, count, dtype, op):
-    """One tree launch in place of the deterministic reduce-scatter's slot writes and halving rounds, and one chain
-    launch per group of ranks in place of the chunk-mesh allreduce's rounds and gather: the user outputs hold the
-    oracle's bits, the inputs are only read, and no communication buffer is asked for."""
+    """One tree launch in place of the deterministic reduce-scatter's slot writes and halving rounds, one chain
+    launch per group of ranks in place of the chunk-mesh allreduce's rounds and gather, tree launches laid out from the
+    deterministic allreduce's own operation list: the user outputs hold the oracle's bits, the inputs are only read,
+    and no communication buffer is asked for."""
     say("fused on user buffers", alg, n, count, dtype, op)
     dt, o = DT[dtype], OPS[op]
     in_count, out_count = buffer_counts(alg, n, count)
@@ -245,11 +251,11 @@ def test_fused_lowerings_on_the_user_buffers(gpu_thread, alg, n, count, dtype, o
             if n > 1:
                 assert plan.info.movedBytes == (n + 1) * n * count * unit
         elif n > 1:
-            per_launch = 32 // (n - 1)               # whole ranks' sub-chunks per launch, 32 segments at most
+            per_launch = 32 // (n - 1) if alg == "chunk_mesh" else 8   # segments a launch's tables hold
             assert plan.info.launches <= -(-n // per_launch)
             assert plan.info.movedBytes == 2 * n * count * unit
         for rec in plan.launches():
-            assert rec.kind == (h.Kernel.COPY if n == 1 else h.Kernel.TREE if alg == "local_reduce_rs" else h.Kernel.CHAIN)
+            assert rec.kind == (h.Kernel.COPY if n == 1 else h.Kernel.CHAIN if alg == "chunk_mesh" else h.Kernel.TREE)
         assert plan.run(gpu_thread) == 0
         assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
         for r in range(n):

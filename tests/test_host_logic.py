@@ -206,8 +206,11 @@ def test_local_reduce_plan_needs_scratch_and_power_of_two(rec):
         h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i[:6], o[:6], count, DT.FP32, OP.SUM, 0, sc[:6])
     assert e.value.code == R.E_PARA                                  # 6 ranks
     with pytest.raises(h.HcommError) as e:
-        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM, 0, sc)
-    assert e.value.code == R.E_NOT_SUPPORT
+        h.Plan(h.Alg.ALLREDUCE_DOUBLING, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT                           # no single-launch lowering
+    p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM)   # user buffers only
+    assert [(r.kind, r.nseg) for r in p.launches()] == [(h.Kernel.TREE, 8)]
+    p.destroy()
     p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, i, o, count, DT.FP32, OP.SUM, 0, sc)
     # own copy | 6 gather rounds merged | neighbour reduce | fold + 2 halving rounds | own gather + 7 rounds merged
     kinds = [(r.kind, r.nseg) for r in p.launches()]
