@@ -417,8 +417,14 @@ typedef enum {
     /* steps whose data dependences are element-wise are folded into k-way kernels that read every input
        once and store every value the step-wise replay leaves in a buffer (partials included), so the final
        contents of all 2N buffers are identical to HCOMM_GFX_LOWER_STEPWISE.  Available for the ring, mesh,
-       recursive halving-doubling, NHR (sliced and one-shot) and NB algorithms; the algorithms that stage through a communication
-       buffer return HCCL_E_NOT_SUPPORT */
+       recursive halving-doubling, NHR (sliced and one-shot) and NB algorithms.
+       The three algorithms that stage through a communication buffer (deterministic local-reduce allreduce and
+       reduce-scatter, chunk-mesh allreduce) are lowered onto the in / out buffers alone: every output holds the bits
+       the step-wise replay gives it, the inputs are only read, and no scratch buffers are needed (the argument is
+       ignored).  Limits of these three: the local-reduce reduce-scatter needs count * unit to be a multiple of 16,
+       the local-reduce allreduce needs its slot size (a multiple of 16 KiB, or of 512 bytes for small messages) to
+       keep slices on 16-byte boundaries and at most 16 ranks; otherwise HCCL_E_NOT_SUPPORT.  Inside
+       HcommGfxOpBasePlanCreate they stay step-wise only.  ALLREDUCE_DOUBLING has no fused lowering. */
     HCOMM_GFX_LOWER_FUSED = 1
 } HcommGfxLowering;
 
@@ -602,6 +608,7 @@ int32_t HcommGfxScheduleCheck(
  * userIn / userOut: the caller's buffers (allreduce: count elements each; reduce-scatter: N * count in, count out).
  * cclIn / cclOut: cclBytes each, 128-byte aligned.  scratch: as HcommGfxPlanCreateEx, sized for
  * min(count, maxCountPerLoop) elements.  FUSED lowers the template part of every chunk as HcommGfxPlanCreate would.
+ * (HCCL_E_NOT_SUPPORT for the algorithms that need scratch: the loop's replay defines what those buffers hold).
  */
 int32_t HcommGfxOpBasePlanCreate(
     HcommGfxAlgorithm alg, HcommGfxLowering lowering, uint32_t nRanks, void* const* userIn, void* const* userOut,
