@@ -109,6 +109,30 @@ int main(void)
                 }
                 for (int ar = 0; ar < 2; ++ar) { p = NULL; HcommGfxOrderPreservedFusedPlanCreate(ar, 1, n, bufs[3], bufs[4], x.count, x.dt, HCOMM_REDUCE_PROD, &p); run_plan(th, p); }
             }
+    /* the single-launch lowerings of the three-buffer schedules at sizes that keep their slices on 16-byte
+     * boundaries, with the trees read back */
+    {
+        const uint32_t fn[] = {2, 4, 8, 16, 32};
+        const uint64_t fc[] = {1 << 16, (1 << 18) + 40, 3 << 20};
+        const int fa[] = {HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH, HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE};
+        for (unsigned ni = 0; ni < 5; ++ni)
+            for (unsigned ci = 0; ci < 3; ++ci)
+                for (unsigned ai = 0; ai < 3; ++ai) {
+                    p = NULL;
+                    HcommGfxPlanCreateEx(fa[ai], HCOMM_GFX_LOWER_FUSED, fn[ni], bufs[0], bufs[1], NULL, fc[ci], 0, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM, &p);
+                    HcommGfxPlanInfo info;
+                    if (p && HcommGfxPlanGetInfo(p, &info) == 0)
+                        for (uint32_t i = 0; i < info.launches; ++i)
+                            for (uint32_t sgm = 0; sgm < 40; ++sgm) {
+                                const void* leaves[32];
+                                uint32_t k = 0;
+                                uint64_t off = 0, bytes = 0;
+                                if (HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 32, &k, &off, &bytes) == 0) ++checks;
+                                HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 1, &k, NULL, NULL);
+                            }
+                    run_plan(th, p);
+                }
+    }
     /* two-level executors */
     for (unsigned si = 0; si < 5; ++si)
         for (unsigned li = 0; li < 5; ++li)
