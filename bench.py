@@ -4,7 +4,7 @@
 One "step" is one complete collective over the N simulated ranks (2N HBM buffers).  Inputs are resident in
 HBM before the timed region.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--lowering stepwise|fused|both]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--lowering stepwise|fused|fused_keep_inputs|both]
                     [--no-cpu] [--cpu-threads T]
 
 `value` is algorithmic GB/s of the whole collective - the two-input byte model, 3b per reduce and 2b per copy,
@@ -124,7 +124,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--lowering", default="both", choices=["stepwise", "fused", "both"])
+    ap.add_argument("--lowering", default="both", choices=["stepwise", "fused", "fused_keep_inputs", "both"])
     ap.add_argument("--workload", default="ring_ar_bf16_n8_128MiB", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0 = min(16, cores))")
@@ -245,13 +245,19 @@ def main():
         return h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
 
     lowerings = ["stepwise", "fused"] if args.lowering == "both" else [args.lowering]
+    # a template on the rank buffers themselves also has the fused launches without their stores into the inputs
+    plain_plan = not (hier_rs or dbrs or opfused or opsmall or opar or plant or ophrs or ophier or dbring or hier or opbase)
+    if args.lowering == "both" and plain_plan and not in_place:
+        lowerings.append("fused_keep_inputs")
+    lowering_of = {"stepwise": h.Lowering.STEPWISE, "fused": h.Lowering.FUSED,
+                   "fused_keep_inputs": h.Lowering.FUSED_KEEP_INPUTS}
     results = {}
     for name in lowerings:
-        low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
+        low = lowering_of[name]
         try:
             plan = make_plan(low)
         except h.HcommError as e:  # e.g. the single-launch reduce-scatter needs blocks of whole 16 bytes
-            if name == "fused" and e.code == h.HcclResult.E_NOT_SUPPORT:
+            if name != "stepwise" and e.code == h.HcclResult.E_NOT_SUPPORT:
                 continue
             raise
         launches = plan.launches()
@@ -455,13 +461,16 @@ def main():
         for name in lowerings:
             if name not in results:
                 continue
-            low = h.Lowering.STEPWISE if name == "stepwise" else h.Lowering.FUSED
+            low = lowering_of[name]
             plan = make_plan(low)
             restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
             stream.synchronize()
             for r in range(n):
-                ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
+                if name == "fused_keep_inputs":  # the inputs as they were, not as the replay leaves them
+                    ok = bool(torch.equal(d_in[r], pristine[r]))
+                else:
+                    ok = np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
                 if not in_place:
                     ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
                 if (opbase or dbring or plant or hier_rs or ophier or ophrs) and not (opfused and name == "fused"):  # what the last chunk left in the CCL buffers
@@ -510,6 +519,9 @@ def main():
         "verified_bit_exact_vs_oracle": verified,
         "fused": ({kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in results["fused"].items()}
                   if "fused" in results and best != "fused" else None),
+        "fused_keep_inputs": ({kk: (round(vv, 5) if isinstance(vv, float) else vv)
+                               for kk, vv in results["fused_keep_inputs"].items()}
+                              if "fused_keep_inputs" in results else None),
     }
     print(json.dumps(out))
 

@@ -79,7 +79,7 @@ class Alg:
 
 
 class Lowering:
-    STEPWISE, FUSED = 0, 1
+    STEPWISE, FUSED, FUSED_KEEP_INPUTS = 0, 1, 2
 
 
 class Kernel:

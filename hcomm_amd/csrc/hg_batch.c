@@ -97,15 +97,15 @@ void hg_finish_fold(HgLaunch* l)
         if (t->tree != 1u) {
             /* truncated rotation trees: nranks leaf reads, one store per even position that has a right neighbour
              * (none for the rank-order trees, which only read their inputs), and the root to one output or to all */
-            const uint64_t n = (uint64_t)t->nranks + (t->tree >= 4u ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
+            const uint64_t n = (uint64_t)t->nranks + ((t->tree >= 4u || t->keep_inputs) ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
             l->moved_bytes = n * bytes;
             l->blocks = hg_grid_blocks(tiles, 0);
             return;
         }
         for (uint32_t s = 0; s < t->nseg; ++s) {
-            uint64_t n = t->k + t->k / 2 + t->nout;
+            uint64_t n = t->k + (t->keep_inputs ? 0u : t->k / 2) + t->nout;
             for (uint32_t b = 0; b < t->k; ++b)
-                if (t->in2[b]) n += 1 + (((b ^ t->first[s]) & (t->k / 2)) ? 1 : 0);
+                if (t->in2[b]) n += 1 + ((!t->keep_inputs && ((b ^ t->first[s]) & (t->k / 2))) ? 1 : 0);
             moved += n * t->bytes[s];
         }
         l->moved_bytes = moved;

@@ -72,6 +72,7 @@ typedef struct {
     uint32_t ascending;      /* chain only: 1 = position 0 is first[s], positions 1.. are ranks 0, 1, ... skipping first[s];
                               * 2 = position 0 is first[s], position j >= 1 is first[s] + 1 + (start[s] + j - 1) mod (nranks - 1):
                               * the other ranks in cyclic order, entered at distance start[s] + 1 */
+    uint32_t keep_inputs;    /* tree modes 1 - 3: the partials the step-wise replay leaves in the inputs are not stored */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];

@@ -59,7 +59,7 @@ __device__ __forceinline__ void fold_tree_items(const HgFoldTable& tab, uint32_t
 #pragma unroll
     for (uint32_t q = 0; q < K; ++q) {
         const uint32_t b = c ^ bitrev<L>(q);
-        if ((q & 1u) == 0u || tab.in2[b]) {
+        if (!tab.keep_inputs && ((q & 1u) == 0u || tab.in2[b])) {
             uint8_t* p = (uint8_t*)tab.in[b] + off;
 #pragma unroll
             for (uint32_t u = 0; u < NU; ++u)
@@ -134,7 +134,7 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
     }
 #pragma unroll
     for (uint32_t q = 0; q < K; q += 2)
-        if (!order && q + 1 < n) {
+        if (!order && !tab.keep_inputs && q + 1 < n) {
             uint8_t* p = (uint8_t*)tab.in[b[q]] + off;
 #pragma unroll
             for (uint32_t u = 0; u < NU; ++u)

@@ -694,6 +694,25 @@ static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n,
     }
 }
 
+/* HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS: the launches of the fused lowering with every store into an input dropped */
+static void drop_input_stores(HcommGfxPlan* p)
+{
+    p->info.movedBytes = 0;
+    for (uint32_t i = 0; i < p->nlaunch; ++i) {
+        HgLaunch* l = &p->launches[i];
+        HgFoldTable* f = &l->tab.fold;
+        if (l->kind == HCOMM_GFX_KERNEL_CHAIN) {
+            f->store_partials = 0;
+            f->store_final_first = 0;
+            hg_finish_fold(l);
+        } else if (l->kind == HCOMM_GFX_KERNEL_TREE) {
+            f->keep_inputs = 1;
+            hg_finish_fold(l);
+        }
+        p->info.movedBytes += l->moved_bytes;
+    }
+}
+
 static int in_place(int alg) { return alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING; }
 
 int32_t HcommGfxPlanCreate(
@@ -731,7 +750,10 @@ int32_t HcommGfxPlanCreateEx(
     if (!out && !in_place((int)alg)) return HCCL_E_PTR;
     if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
-    if (lowering != HCOMM_GFX_LOWER_STEPWISE && lowering != HCOMM_GFX_LOWER_FUSED) return HCCL_E_PARA;
+    if (lowering != HCOMM_GFX_LOWER_STEPWISE && lowering != HCOMM_GFX_LOWER_FUSED && lowering != HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS)
+        return HCCL_E_PARA;
+    /* a result that lives in the input cannot leave the input alone */
+    if (lowering == HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS && in_place((int)alg)) return HCCL_E_NOT_SUPPORT;
     for (uint32_t r = 0; r < nRanks; ++r) {
         if (!in[r]) return HCCL_E_PTR;
         if (((uintptr_t)in[r]) & 127u) return HCCL_E_PARA;
@@ -765,6 +787,7 @@ int32_t HcommGfxPlanCreateEx(
         rc = lower_stepwise(p, &ol, in, out, scratch, (int)dataType, (int)reduceOp);
     else
         rc = lower_fused(p, (int)alg, &ol, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
+    if (rc == HCCL_SUCCESS && lowering == HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS) drop_input_stores(p);
     hg_oplist_free(&ol);
     if (rc != HCCL_SUCCESS) {
         HcommGfxPlanDestroy(p);

@@ -425,7 +425,13 @@ typedef enum {
        the local-reduce allreduce needs its slot size (a multiple of 16 KiB, or of 512 bytes for small messages) to
        keep slices on 16-byte boundaries and at most 16 ranks; otherwise HCCL_E_NOT_SUPPORT.  Inside
        HcommGfxOpBasePlanCreate they stay step-wise only.  ALLREDUCE_DOUBLING has no fused lowering. */
-    HCOMM_GFX_LOWER_FUSED = 1
+    HCOMM_GFX_LOWER_FUSED = 1,
+    /* the launches of HCOMM_GFX_LOWER_FUSED without their stores into the inputs: every out[r] holds the same bits,
+       every in[r] is left as the caller filled it (what the collective's caller sees of the reference, which runs
+       its templates on CCL buffers and never writes the send buffer).  One read per input element and one write per
+       output element.  Accepted by HcommGfxPlanCreate / Strided / Ex only; the in-place ring reduce-scatter stage,
+       whose result lives in the input, returns HCCL_E_NOT_SUPPORT. */
+    HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS = 2
 } HcommGfxLowering;
 
 typedef struct {

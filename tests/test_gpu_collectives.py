@@ -272,6 +272,41 @@ def test_fused_deterministic_reduce_scatter_needs_16_byte_slices():
     assert e.value.code == h.HcclResult.E_NOT_SUPPORT
 
 
+KEEP_INPUTS = [c for c in CASES if c[0] in FUSABLE and c[0] != "ring_rs_stage"] + [c for c in USER_BUFFER_FUSED]
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", KEEP_INPUTS)
+def test_fused_lowering_that_keeps_the_inputs(gpu_thread, alg, n, count, dtype, op):
+    """HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS: the outputs hold the oracle's bits, the inputs are exactly what they were,
+    and the launches move one read per input element and one write per output element."""
+    say("keep inputs", alg, n, count, dtype, op)
+    dt, o = DT[dtype], OPS[op]
+    in_count, out_count = buffer_counts(alg, n, count)
+    host_in = [gen(dt, in_count, 8000 + r, "prod" if op == "prod" else "default") for r in range(n)]
+    sentinel = gen(dt, out_count, 999, "wide")
+    want_in = [x.copy() for x in host_in]
+    want_out = [sentinel.copy() for _ in range(n)]
+    sb = h.scratch_bytes(ALGS[alg][0], n, count, dt)
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o,
+               scratch=[np.zeros(sb, np.uint8) for _ in range(n)] if sb else None)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    pad = to_dev(np.zeros(256, np.uint8))
+    ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
+    plan = h.Plan(ALGS[alg][0], h.Lowering.FUSED_KEEP_INPUTS, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+    try:
+        fused = h.Plan(ALGS[alg][0], h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+        assert plan.info.launches == fused.info.launches and plan.info.movedBytes <= fused.info.movedBytes
+        fused.destroy()
+        assert plan.run(gpu_thread) == 0
+        assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_in[r], host_in[r]), host_in[r], dt, "in[%d]" % r)
+            assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+    finally:
+        plan.destroy()
+
+
 @pytest.mark.parametrize("alg", SCATTER)
 @pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
 def test_strided_reduce_scatter(gpu_thread, alg, lowering):

@@ -418,6 +418,28 @@ def test_fused_chunk_mesh_is_chain_launches_over_whole_ranks_sub_chunks():
         q.destroy()
 
 
+def test_keep_inputs_lowering_moves_one_read_per_input_and_one_write_per_output():
+    for alg, n, count, moved in ((h.Alg.ALLREDUCE_RING, 8, 1 << 20, 16), (h.Alg.ALLREDUCE_RHD, 16, 1 << 20, 32),
+                                 (h.Alg.ALLREDUCE_RHD, 6, 1 << 20, 12), (h.Alg.ALLREDUCE_NHR, 7, 7 << 18, 14),
+                                 (h.Alg.ALLREDUCE_NB, 5, 5 << 18, 10), (h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 1 << 20, 72),
+                                 (h.Alg.ALLREDUCE_NHR_ONESHOT, 8, 1 << 20, 16), (h.Alg.ALLREDUCE_LOCAL_REDUCE, 8, 1 << 20, 16)):
+        i, o = ptrs(n, 1 << 24)
+        p = h.Plan(alg, h.Lowering.FUSED_KEEP_INPUTS, i, o, count, DT.FP32, OP.SUM)
+        q = h.Plan(alg, h.Lowering.FUSED, i, o, count, DT.FP32, OP.SUM)
+        assert p.info.movedBytes == moved * count * 4, alg             # (reads + writes) x message bytes
+        assert p.info.movedBytes <= q.info.movedBytes and p.info.algorithmicBytes == q.info.algorithmicBytes
+        assert [(r.kind, r.nseg, r.bytes) for r in p.launches()] == [(r.kind, r.nseg, r.bytes) for r in q.launches()]
+        p.destroy()
+        q.destroy()
+    i, o = ptrs(4, 1 << 20)
+    with pytest.raises(h.HcommError) as e:          # the in-place stage's result lives in the input
+        h.Plan(h.Alg.REDUCE_SCATTER_RING, h.Lowering.FUSED_KEEP_INPUTS, i, None, 4096, DT.FP32, OP.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT
+    with pytest.raises(h.HcommError) as e:
+        h.Plan(h.Alg.ALLREDUCE_RING, 3, i, o, 4096, DT.FP32, OP.SUM)
+    assert e.value.code == R.E_PARA
+
+
 def test_counts_whose_byte_offsets_would_leave_64_bits_are_refused():
     i, o = ptrs(4, 4096)
     for count in (2**48 + 1, 2**62, 2**64 - 1):
