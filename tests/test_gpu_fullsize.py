@@ -205,3 +205,37 @@ def test_nhr_and_nb_int32_full_size_closed_form(gpu_thread, algname, n, count, l
         assert torch.equal(outs[r], want), "out[%d]" % r
     del ins, outs, want
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("algname,lowering", [
+    ("local_reduce", h.Lowering.FUSED), ("chunk_mesh", h.Lowering.FUSED), ("local_reduce_rs", h.Lowering.FUSED),
+    ("ring", h.Lowering.FUSED_KEEP_INPUTS), ("rhd", h.Lowering.FUSED_KEEP_INPUTS), ("nhr", h.Lowering.FUSED_KEEP_INPUTS),
+    ("nb", h.Lowering.FUSED_KEEP_INPUTS), ("mesh_rs", h.Lowering.FUSED_KEEP_INPUTS),
+])
+def test_lowerings_that_only_read_the_inputs_full_size_closed_form(gpu_thread, algname, lowering):
+    """128 MiB of int32 per rank on 8 ranks (reduce-scatters: 8 slices of 16 MiB): every output equals the exact
+    sum, computed independently by torch, and every input is bit for bit what it was."""
+    import torch
+    n = 8
+    scatter = algname in ("local_reduce_rs", "mesh_rs")
+    count = (1 << 22) if scatter else (1 << 25)
+    alg = {"local_reduce": h.Alg.ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": h.Alg.ALLREDUCE_CHUNK_MESH,
+           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, "ring": h.Alg.ALLREDUCE_RING, "rhd": h.Alg.ALLREDUCE_RHD,
+           "nhr": h.Alg.ALLREDUCE_NHR, "nb": h.Alg.ALLREDUCE_NB, "mesh_rs": h.Alg.REDUCE_SCATTER_MESH}[algname]
+    say("read-only lowering, full size", algname, lowering)
+    g = torch.Generator(device="cuda")
+    ins = []
+    for r in range(n):
+        g.manual_seed(900 + r)
+        ins.append(torch.randint(-(1 << 20), (1 << 20) + 1, ((n if scatter else 1) * count,), generator=g, device="cuda",
+                                 dtype=torch.int32))
+    before = [x.clone() for x in ins]
+    want = torch.zeros_like(ins[0])
+    for x in ins:
+        want += x
+    outs = [torch.full((count,), -7, dtype=torch.int32, device="cuda") for _ in range(n)]
+    info = run_plan(gpu_thread, alg, lowering, ins, outs, count, oracle.I32, oracle.SUM)
+    assert info.movedBytes == ((n + 1) * n * count * 4 if scatter else 2 * n * count * 4)
+    for r in range(n):
+        assert torch.equal(ins[r], before[r]), "in[%d]" % r
+        assert torch.equal(outs[r], want[r * count:(r + 1) * count] if scatter else want), "out[%d]" % r
