@@ -189,7 +189,7 @@ _plan_graph = _sig("HcommGfxPlanSetGraphReplay", _i32, _vp, _i32)
 _plan_info = _sig("HcommGfxPlanGetInfo", _i32, _vp, C.POINTER(PlanInfo))
 _plan_launch = _sig("HcommGfxPlanGetLaunch", _i32, _vp, _u32, C.POINTER(LaunchRecord))
 _plan_tree_segment = _sig("HcommGfxPlanGetTreeSegment", _i32, _vp, _u32, _u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
-                         C.POINTER(_u64), C.POINTER(_u64))
+                         C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_i32))
 _sched_emit = _sig("HcommGfxScheduleEmitStrided", _i32, C.c_int, _u32, _u64, _u64, C.c_int, C.POINTER(SchedOp), _u64,
                    C.POINTER(_u64))
 HcommWriteOnThread = _sig("HcommWriteOnThread", _i32, _u64, _u64, _vp, _vp, _u64)
@@ -370,15 +370,15 @@ class Plan:
             pass
 
 
-def plan_tree(plan, launch, segment, rank_of=None):
+def plan_tree(plan, launch, segment, rank_of=None, with_owner=False):
     """(tree, offset, bytes) of one segment of a tree launch of any plan object: the nested [dst, src] lists the
     kernel's fold pattern makes of the leaf positions (level l folds position q + 2^l onto q, holes skipped); a leaf
     is the input pointer read there, or rank_of[pointer] when a mapping is given."""
-    k, off, nbytes = _u32(0), _u64(0), _u64(0)
-    check(_plan_tree_segment(plan._p, launch, segment, None, 0, C.byref(k), C.byref(off), C.byref(nbytes)),
-          "HcommGfxPlanGetTreeSegment")
+    k, off, nbytes, owner = _u32(0), _u64(0), _u64(0), _i32(0)
+    check(_plan_tree_segment(plan._p, launch, segment, None, 0, C.byref(k), C.byref(off), C.byref(nbytes),
+                             C.byref(owner)), "HcommGfxPlanGetTreeSegment")
     leaves = (_vp * k.value)()
-    check(_plan_tree_segment(plan._p, launch, segment, leaves, k.value, C.byref(k), None, None),
+    check(_plan_tree_segment(plan._p, launch, segment, leaves, k.value, C.byref(k), None, None, None),
           "HcommGfxPlanGetTreeSegment")
     x = [None if not v else (rank_of[v] if rank_of is not None else v) for v in leaves]
     step = 1
@@ -387,6 +387,8 @@ def plan_tree(plan, launch, segment, rank_of=None):
             if x[q + step] is not None:
                 x[q] = [x[q], x[q + step]]
         step *= 2
+    if with_owner:  # the rank whose output takes the root, -1 = every rank's
+        return x[0], off.value, nbytes.value, owner.value
     return x[0], off.value, nbytes.value
 
 

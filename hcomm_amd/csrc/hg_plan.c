@@ -488,9 +488,10 @@ static int fused_chunk_mesh(HcommGfxPlan* p, uint32_t n, void* const* in, void* 
  * The operation list is replayed on symbols: a cell is an exact byte range of one buffer, its value a node - a leaf
  * (rank, offset: the range of that rank's input) or a fold (dst node, src node).  What ends up in the output cells
  * are the trees the kernel must evaluate; they are laid out over 2^depth leaf positions so that the kernel's fixed
- * pattern (level l folds position q + 2^l onto q) walks them with every dst operand on the left.  Lists that write
- * an input, read a range with other bounds than it was written with, or leave different trees in different ranks'
- * outputs are refused (HCCL_E_NOT_SUPPORT). */
+ * pattern (level l folds position q + 2^l onto q) walks them with every dst operand on the left.  Lists that read a
+ * range with other bounds than it was written with are refused (HCCL_E_NOT_SUPPORT), and so are lists that write an
+ * input unless the caller asked for the inputs to be left alone (the launch only ever reads the original inputs).
+ * Outputs that hold the same trees in every rank become segments written to all ranks, others one segment each. */
 typedef struct {
     uint32_t rank, buf;
     uint64_t off, bytes;
@@ -549,19 +550,21 @@ static int sym_place(const SymState* st, int32_t node, uint8_t* pos, uint32_t q,
 }
 
 static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, void* const* in, void* const* out, int dtype,
-                            int op)
+                            int op, int inputs_may_change)
 {
     SymState st;
     memset(&st, 0, sizeof(st));
     st.cap = (uint32_t)(2 * ol->n + 1);
-    st.cell = (SymCell*)calloc(st.cap, sizeof(SymCell));
-    st.node = (SymNode*)calloc(st.cap, sizeof(SymNode));
+    st.cell = (SymCell*)calloc(st.cap, sizeof(SymCell));                       /* at most two new cells per operation */
+    st.node = (SymNode*)calloc((size_t)st.cap + ol->n, sizeof(SymNode));       /* and three new nodes */
     HgLaunch* l = NULL;
     int rc = (st.cell && st.node) ? HCCL_SUCCESS : HCCL_E_MEMORY;
     for (uint64_t i = 0; i < ol->n && rc == HCCL_SUCCESS; ++i) {
         const HcommGfxSchedOp* o = &ol->ops[i];
         if (o->bytes == 0) continue;
-        if (o->dstBuf == 0) rc = HCCL_E_NOT_SUPPORT; /* the inputs must stay as they are */
+        /* a list that writes its inputs can only be lowered for a caller who wants them left alone: the launch reads
+         * the original inputs at the leaves and stores nothing into them */
+        if (o->dstBuf == 0 && !inputs_may_change) rc = HCCL_E_NOT_SUPPORT;
         int32_t src = sym_find(&st, o->srcRank, o->srcBuf, o->srcOff, o->bytes);
         if (src == -1 && o->srcBuf == 0) { /* first read of an input range: a leaf */
             SymCell* c = &st.cell[st.ncell];
@@ -573,7 +576,7 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
             src = (int32_t)st.ncell++;
         }
         int32_t dst = sym_find(&st, o->rank, o->dstBuf, o->dstOff, o->bytes);
-        if (src < 0 || dst == -2 || (dst == -1 && o->kind)) rc = HCCL_E_NOT_SUPPORT;
+        if (src < 0 || dst == -2 || (dst == -1 && o->kind && o->dstBuf != 0)) rc = HCCL_E_NOT_SUPPORT;
         if (rc != HCCL_SUCCESS) break;
         if (dst == -1) {
             SymCell* c = &st.cell[st.ncell];
@@ -581,33 +584,39 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
             c->buf = o->dstBuf;
             c->off = o->dstOff;
             c->bytes = o->bytes;
+            if (o->dstBuf == 0) c->node = sym_node(&st, -1, -1, o->rank, o->dstOff); /* an input range folded into */
             dst = (int32_t)st.ncell++;
         }
         st.cell[dst].node = o->kind ? sym_node(&st, st.cell[dst].node, st.cell[src].node, 0, 0) : st.cell[src].node;
     }
-    /* the output cells of rank 0 are the segments; every other rank must hold the same trees at the same places */
-    uint32_t nseg = 0, depth = 1;
+    /* When every rank's output holds the same trees at the same places, the output cells of rank 0 are the segments
+     * and the root goes to all outputs; otherwise (whole-message recursive doubling: every rank folds in an order of
+     * its own) every output cell is a segment with a single destination. */
+    uint32_t nseg = 0, nseg_all = 0, depth = 1;
+    int uniform = 1;
     for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
         const SymCell* c = &st.cell[i];
         if (c->buf != 1) continue;
+        ++nseg_all;
+        const uint32_t d = sym_depth(&st, c->node);
+        if (d > depth) depth = d;
         if (c->rank == 0) {
             ++nseg;
-            const uint32_t d = sym_depth(&st, c->node);
-            if (d > depth) depth = d;
             for (uint32_t r = 1; r < n; ++r) {
                 const int32_t j = sym_find(&st, r, 1, c->off, c->bytes);
-                if (j < 0 || st.cell[j].node != c->node) rc = HCCL_E_NOT_SUPPORT;
+                if (j < 0 || st.cell[j].node != c->node) uniform = 0;
             }
         } else if (sym_find(&st, 0, 1, c->off, c->bytes) < 0) {
-            rc = HCCL_E_NOT_SUPPORT;
+            uniform = 0;
         }
     }
+    if (!uniform) nseg = nseg_all;
     if (rc == HCCL_SUCCESS && (1u << depth) > HCOMM_GFX_MAX_RANKS) rc = HCCL_E_NOT_SUPPORT; /* the kernel folds 32 positions at most */
     const uint32_t k = 1u << depth;
     const uint32_t per_launch = HG_POS_BYTES / k < HG_MAX_SEG ? HG_POS_BYTES / k : HG_MAX_SEG;
     for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
         const SymCell* c = &st.cell[i];
-        if (c->buf != 1 || c->rank != 0) continue;
+        if (c->buf != 1 || (uniform && c->rank != 0)) continue;
         if (!l) {
             l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
             if (!l) {
@@ -621,8 +630,8 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
             f->tree = 6u;
             f->k = k;
             f->nranks = n;
-            f->nout = n;
-            f->out_mode = 2u;
+            f->nout = uniform ? n : 0;
+            f->out_mode = uniform ? 2u : 1u;
             memset(f->pos, 255, sizeof(f->pos));
             for (uint32_t r = 0; r < n; ++r) {
                 f->in[r] = in[r];
@@ -632,6 +641,8 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
         HgFoldTable* f = &l->tab.fold;
         const uint32_t s = f->nseg++;
         f->off[s] = c->off;
+        f->out_off[s] = c->off;
+        f->owner[s] = (uint8_t)c->rank;
         f->bytes[s] = c->bytes;
         /* 128-bit accesses: a segment must start on a 16-byte boundary of every buffer */
         if ((c->off & (HG_VEC_BYTES - 1u)) || !sym_place(&st, c->node, f->pos + s * k, 0, depth, c->off)) rc = HCCL_E_NOT_SUPPORT;
@@ -650,7 +661,7 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
 }
 
 static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n, void* const* in, void* const* out,
-                       uint64_t count, uint64_t stride, int dtype, int op)
+                       uint64_t count, uint64_t stride, int dtype, int op, int keep_inputs)
 {
     const uint64_t total = count * HcommGfxDataTypeSize((HcommDataType)dtype);
     switch (alg) {
@@ -686,7 +697,12 @@ static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n,
             return fused_chunk_mesh(p, n, in, out, count, dtype, op);
         case HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
-            return ol ? fused_from_trees(p, ol, n, in, out, dtype, op) : HCCL_E_NOT_SUPPORT;
+            return ol ? fused_from_trees(p, ol, n, in, out, dtype, op, 0) : HCCL_E_NOT_SUPPORT;
+        case HCOMM_GFX_ALG_ALLREDUCE_DOUBLING:
+            /* its steps copy the running value back into the input for the partner to read, so only the lowering
+             * that promises to leave the inputs alone has a single launch: one tree per rank, root to that rank */
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return (ol && keep_inputs) ? fused_from_trees(p, ol, n, in, out, dtype, op, 1) : HCCL_E_NOT_SUPPORT;
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rs_local_reduce(p, n, in, out, count, dtype, op);
@@ -786,7 +802,8 @@ int32_t HcommGfxPlanCreateEx(
     if (lowering == HCOMM_GFX_LOWER_STEPWISE)
         rc = lower_stepwise(p, &ol, in, out, scratch, (int)dataType, (int)reduceOp);
     else
-        rc = lower_fused(p, (int)alg, &ol, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp);
+        rc = lower_fused(p, (int)alg, &ol, nRanks, in, out, count, strideCount, (int)dataType, (int)reduceOp,
+                         lowering == HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS);
     if (rc == HCCL_SUCCESS && lowering == HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS) drop_input_stores(p);
     hg_oplist_free(&ol);
     if (rc != HCCL_SUCCESS) {
@@ -859,7 +876,7 @@ int32_t HcommGfxOpBasePlanCreate(
             uint64_t k = j;
             while (k < ol.n && ol.ops[k].dstBuf != HCOMM_GFX_BUF_USER_OUT) ++k;
             const uint64_t cur = count - done > maxc ? maxc : count - done;
-            if (rc == HCCL_SUCCESS) rc = lower_fused(p, (int)alg, NULL, nRanks, cclIn, cclOut, cur, cur, (int)dataType, (int)reduceOp);
+            if (rc == HCCL_SUCCESS) rc = lower_fused(p, (int)alg, NULL, nRanks, cclIn, cclOut, cur, cur, (int)dataType, (int)reduceOp, 0);
             uint64_t m = k;
             while (m < ol.n && ol.ops[m].dstBuf == HCOMM_GFX_BUF_USER_OUT) ++m;
             if (rc == HCCL_SUCCESS) rc = lower_ops(p, &ol.ops[k], m - k, bufs, (int)dataType, (int)reduceOp);
@@ -1333,7 +1350,7 @@ int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaun
 }
 
 int32_t HcommGfxPlanGetTreeSegment(const HcommGfxPlan* plan, uint32_t i, uint32_t segment, const void** leaves,
-                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes)
+                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes, int32_t* outRank)
 {
     if (!plan || plan->magic != HG_PLAN_MAGIC || !k) return HCCL_E_PTR;
     if (i >= plan->nlaunch) return HCCL_E_PARA;
@@ -1343,6 +1360,7 @@ int32_t HcommGfxPlanGetTreeSegment(const HcommGfxPlan* plan, uint32_t i, uint32_
     *k = f->k;
     if (offset) *offset = f->off[segment];
     if (bytes) *bytes = f->bytes[segment];
+    if (outRank) *outRank = f->out_mode == 1u ? (int32_t)f->owner[segment] : -1;
     if (!leaves) return HCCL_SUCCESS;
     if (cap < f->k) return HCCL_E_PARA;
     const uint32_t n = f->nranks, c = f->first[segment];

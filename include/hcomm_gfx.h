@@ -424,13 +424,15 @@ typedef enum {
        ignored).  Limits of these three: the local-reduce reduce-scatter needs count * unit to be a multiple of 16,
        the local-reduce allreduce needs its slot size (a multiple of 16 KiB, or of 512 bytes for small messages) to
        keep slices on 16-byte boundaries and at most 16 ranks; otherwise HCCL_E_NOT_SUPPORT.  Inside
-       HcommGfxOpBasePlanCreate they stay step-wise only.  ALLREDUCE_DOUBLING has no fused lowering. */
+       HcommGfxOpBasePlanCreate they stay step-wise only.  ALLREDUCE_DOUBLING, whose steps write the inputs, has
+       none (see HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS). */
     HCOMM_GFX_LOWER_FUSED = 1,
     /* the launches of HCOMM_GFX_LOWER_FUSED without their stores into the inputs: every out[r] holds the same bits,
        every in[r] is left as the caller filled it (what the collective's caller sees of the reference, which runs
        its templates on CCL buffers and never writes the send buffer).  One read per input element and one write per
        output element.  Accepted by HcommGfxPlanCreate / Strided / Ex only; the in-place ring reduce-scatter stage,
-       whose result lives in the input, returns HCCL_E_NOT_SUPPORT. */
+       whose result lives in the input, returns HCCL_E_NOT_SUPPORT.  The only lowering of ALLREDUCE_DOUBLING besides
+       the step-wise one: one tree per rank, root to that rank (N outputs, each from N reads). */
     HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS = 2
 } HcommGfxLowering;
 
@@ -528,11 +530,14 @@ int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaun
  * positions; leaves[q] receives the rank buffer (the in[] pointer the plan was built with) read at position q, or NULL
  * where the tree has a hole; the element at byte *offset + x of every leaf is folded level by level, level l folding
  * position q + 2^l (src role) onto position q (dst role) for every q that is a multiple of 2^(l+1), holes skipped.
- * leaves may be NULL to query *k; cap < *k -> HCCL_E_PARA.  No counterpart in the reference: its schedules
- * are only ever run step by step.
+ * *outRank receives the rank whose output takes the root, or -1 when every rank's output does.
+ * leaves may be NULL to query *k; cap < *k -> HCCL_E_PARA; offset, bytes and outRank may be NULL.  Not reported: the
+ * odd neighbours a recursive halving-doubling launch on a non-power-of-two rank count folds into the even block ranks
+ * before the tree, and the partials a launch stores back into the inputs.  No counterpart in the reference: its
+ * schedules are only ever run step by step.
  */
 int32_t HcommGfxPlanGetTreeSegment(const HcommGfxPlan* plan, uint32_t i, uint32_t segment, const void** leaves,
-                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes);
+                                   uint32_t cap, uint32_t* k, uint64_t* offset, uint64_t* bytes, int32_t* outRank);
 
 /*
  * The schedule as the reference's templates emit it, one two-input operation per record, for inspection

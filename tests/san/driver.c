@@ -114,12 +114,12 @@ int main(void)
     {
         const uint32_t fn[] = {2, 4, 8, 16, 32};
         const uint64_t fc[] = {1 << 16, (1 << 18) + 40, 3 << 20};
-        const int fa[] = {HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH, HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE};
+        const int fa[] = {HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, HCOMM_GFX_ALG_ALLREDUCE_CHUNK_MESH, HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE, HCOMM_GFX_ALG_ALLREDUCE_DOUBLING};
         for (unsigned ni = 0; ni < 5; ++ni)
             for (unsigned ci = 0; ci < 3; ++ci)
-                for (unsigned ai = 0; ai < 3; ++ai) {
+                for (unsigned ai = 0; ai < 4; ++ai) {
                     p = NULL;
-                    HcommGfxPlanCreateEx(fa[ai], HCOMM_GFX_LOWER_FUSED, fn[ni], bufs[0], bufs[1], NULL, fc[ci], 0, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM, &p);
+                    HcommGfxPlanCreateEx(fa[ai], ai == 3 ? HCOMM_GFX_LOWER_FUSED_KEEP_INPUTS : HCOMM_GFX_LOWER_FUSED, fn[ni], bufs[0], bufs[1], NULL, fc[ci], 0, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM, &p);
                     HcommGfxPlanInfo info;
                     if (p && HcommGfxPlanGetInfo(p, &info) == 0)
                         for (uint32_t i = 0; i < info.launches; ++i)
@@ -127,8 +127,8 @@ int main(void)
                                 const void* leaves[32];
                                 uint32_t k = 0;
                                 uint64_t off = 0, bytes = 0;
-                                if (HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 32, &k, &off, &bytes) == 0) ++checks;
-                                HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 1, &k, NULL, NULL);
+                                if (HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 32, &k, &off, &bytes, NULL) == 0) ++checks;
+                                HcommGfxPlanGetTreeSegment(p, i, sgm, leaves, 1, &k, NULL, NULL, NULL);
                             }
                     run_plan(th, p);
                 }

@@ -162,6 +162,39 @@ def test_halving_tree_launch_equals_the_replay(n):
         plan.destroy()
 
 
+@pytest.mark.parametrize("n", [2, 4, 8, 16, 32])
+def test_recursive_doubling_keep_inputs_launch_holds_every_ranks_own_tree(n):
+    """Whole-message recursive doubling: rank r's output is the tree whose position q holds rank r XOR q; the schedule
+    writes the inputs on the way, the single launch (inputs kept) reads only the originals."""
+    ins, outs, rank_of = ptrs(n)
+    count = 25000
+    plan = h.Plan(h.Alg.ALLREDUCE_DOUBLING, h.Lowering.FUSED_KEEP_INPUTS, ins, outs, count, oracle.F32, oracle.SUM)
+    try:
+        per_rank = output_trees_in_place(oracle.trace(oracle.ALG_ALLREDUCE_DOUBLING, n, count, oracle.F32), n)
+        seen = set()
+        for i, rec in enumerate(plan.launches()):
+            assert rec.kind == h.Kernel.TREE
+            for sg in range(rec.nseg):
+                tree, off, nbytes, owner = h.plan_tree(plan, i, sg, rank_of, with_owner=True)
+                assert (off, nbytes) == (0, count * 4) and owner not in seen
+                seen.add(owner)
+                assert per_rank[owner] == {(0, count * 4): tree}, owner
+                x = [owner ^ q for q in range(n)]
+                step = 1
+                while step < n:
+                    for q in range(0, n, 2 * step):
+                        x[q] = [x[q], x[q + step]]
+                    step *= 2
+                assert tree == x[0]
+        assert seen == set(range(n))
+        assert plan.info.movedBytes == (n + 1) * n * count * 4
+    finally:
+        plan.destroy()
+    with pytest.raises(h.HcommError) as e:          # the lowering that reproduces the inputs' final contents has none
+        h.Plan(h.Alg.ALLREDUCE_DOUBLING, h.Lowering.FUSED, ins, outs, count, oracle.F32, oracle.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT
+
+
 def merged_runs(segments):
     """[(lo, hi, tree)] with neighbours that hold the same tree joined: independent of how the bytes were cut."""
     out = []

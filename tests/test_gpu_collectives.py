@@ -272,7 +272,9 @@ def test_fused_deterministic_reduce_scatter_needs_16_byte_slices():
     assert e.value.code == h.HcclResult.E_NOT_SUPPORT
 
 
-KEEP_INPUTS = [c for c in CASES if c[0] in FUSABLE and c[0] != "ring_rs_stage"] + [c for c in USER_BUFFER_FUSED]
+KEEP_INPUTS = ([c for c in CASES if c[0] in FUSABLE and c[0] != "ring_rs_stage"] + [c for c in USER_BUFFER_FUSED]
+               + [c for c in CASES if c[0] == "doubling"]
+               + [("doubling", 32, 70001, "bf16", "sum"), ("doubling", 16, 1 << 18, "fp16", "max"), ("doubling", 2, 3, "fp32", "sum")])
 
 
 @pytest.mark.parametrize("alg,n,count,dtype,op", KEEP_INPUTS)
@@ -295,9 +297,10 @@ def test_fused_lowering_that_keeps_the_inputs(gpu_thread, alg, n, count, dtype, 
     ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
     plan = h.Plan(ALGS[alg][0], h.Lowering.FUSED_KEEP_INPUTS, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
     try:
-        fused = h.Plan(ALGS[alg][0], h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
-        assert plan.info.launches == fused.info.launches and plan.info.movedBytes <= fused.info.movedBytes
-        fused.destroy()
+        if alg != "doubling":   # whose steps write the inputs: no lowering that reproduces them in one launch
+            fused = h.Plan(ALGS[alg][0], h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
+            assert plan.info.launches == fused.info.launches and plan.info.movedBytes <= fused.info.movedBytes
+            fused.destroy()
         assert plan.run(gpu_thread) == 0
         assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
         for r in range(n):
