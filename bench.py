@@ -60,6 +60,8 @@ WORKLOADS = {
     "nhr_ar_bf16_n8_128MiB": ("nhr", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nb_ar_bf16_n8_128MiB": ("nb", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "local_reduce_rs_bf16_n8_16MiB": ("local_reduce_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # whole-message recursive doubling, the small-message allreduce inside a server
+    "doubling_ar_fp16_n8_64KiB": ("doubling", 8, 32768, "fp16", "sum", "uniform[-1,1)"),
     # the executors' op-base loop around the ring template: user buffers <-> 200 MiB CCL buffers (the default size)
     "opbase_ring_ar_bf16_n8_128MiB": ("opbase_ring_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "opbase_ring_ar_bf16_n8_512MiB": ("opbase_ring_ar", 8, 268435456, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -147,7 +149,8 @@ def main():
     ALG = {"ring_ar": h.Alg.ALLREDUCE_RING, "rhd_ar": h.Alg.ALLREDUCE_RHD, "ring_rs_stage": h.Alg.REDUCE_SCATTER_RING,
            "mesh_oneshot": h.Alg.ALLREDUCE_MESH_ONESHOT, "local_reduce": h.Alg.ALLREDUCE_LOCAL_REDUCE,
            "chunk_mesh": h.Alg.ALLREDUCE_CHUNK_MESH, "nhr": h.Alg.ALLREDUCE_NHR, "nb": h.Alg.ALLREDUCE_NB,
-           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, "nhr_oneshot": h.Alg.ALLREDUCE_NHR_ONESHOT}
+           "local_reduce_rs": h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, "nhr_oneshot": h.Alg.ALLREDUCE_NHR_ONESHOT,
+           "doubling": h.Alg.ALLREDUCE_DOUBLING}
     OP = {"sum": h.HcommReduceOp.SUM, "prod": h.HcommReduceOp.PROD, "max": h.HcommReduceOp.MAX,
           "min": h.HcommReduceOp.MIN}
     opbase = alg_name.startswith("opbase_")  # the template inside the op-base loop of its executor
@@ -340,6 +343,7 @@ def main():
                 "local_reduce": oracle.ALG_ALLREDUCE_LOCAL_REDUCE, "chunk_mesh": oracle.ALG_ALLREDUCE_CHUNK_MESH,
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
                 "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
+                "doubling": oracle.ALG_ALLREDUCE_DOUBLING,
                 "order_preserved_rs": None, "doublering_rs": None, "order_preserved_ar": None,
                 "order_preserved_small": None}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
