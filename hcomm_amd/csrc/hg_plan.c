@@ -611,8 +611,8 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
         }
     }
     if (!uniform) nseg = nseg_all;
-    if (rc == HCCL_SUCCESS && (1u << depth) > HCOMM_GFX_MAX_RANKS) rc = HCCL_E_NOT_SUPPORT; /* the kernel folds 32 positions at most */
-    const uint32_t k = 1u << depth;
+    if (rc == HCCL_SUCCESS && depth > 5u) rc = HCCL_E_NOT_SUPPORT; /* the kernel folds 32 = 2^5 positions at most */
+    const uint32_t k = 1u << (depth > 5u ? 5u : depth);
     const uint32_t per_launch = HG_POS_BYTES / k < HG_MAX_SEG ? HG_POS_BYTES / k : HG_MAX_SEG;
     for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
         const SymCell* c = &st.cell[i];
