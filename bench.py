@@ -503,7 +503,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "ranks": n, "elements_per_rank": count, "op": opname,
                    "algorithm": ("order_preserved_rs" if ophrs else "order_preserved_ar" if ophier else alg_name),
-                   "values": dist, "lowering": best,
+                   "values": dist, "seed": "torch generator on the GPU, 1234 + rank", "lowering": best,
                    **({"op_base_loop": True, "ccl_buffer_bytes": ccl_bytes} if opbase else {}),
                    **({"servers": hier[0], "ranks_per_server": hier[1], "level1_algorithm": ("plant + fold in server order (combine template)" if ophrs else
                                             "plant + fold in server order (combine template), %s all-gather" % alg_name
