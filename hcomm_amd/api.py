@@ -14,7 +14,7 @@ except ImportError:  # a pure C / ctypes caller without torch uses the system ru
     pass
 
 __all__ = [
-    "lib", "LIB_PATH", "plan_tree", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
+    "lib", "LIB_PATH", "plan_tree", "OpListKeepInputsPlan", "HcclResult", "HcommReduceOp", "HcommDataType", "CommEngine", "Alg", "Lowering", "Kernel",
     "LaunchRecord", "PlanInfo", "SchedOp", "Slice", "HcommError", "check",
     "HcommLocalCopyOnThread", "HcommLocalReduceOnThread", "HcommThreadAlloc", "HcommThreadFree",
     "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
@@ -455,6 +455,30 @@ class OpListPlan(Plan):
         table = (C.POINTER(_vp) * 5)(*[C.cast(r, C.POINTER(_vp)) if r is not None else None for r in self._rows])
         p = _vp(0)
         check(_plan_from_ops(arr, len(ops), n_ranks, table, dtype, op, C.byref(p)), "HcommGfxPlanCreateFromOps")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
+
+
+_plan_from_ops_keep = _sig("HcommGfxPlanCreateFromOpsKeepInputs", _i32, C.POINTER(SchedOp), _u64, _u32, C.POINTER(_vp),
+                           C.POINTER(_vp), C.c_int, C.c_int, C.POINTER(_vp))
+
+
+class OpListKeepInputsPlan(Plan):
+    """HcommGfxPlanCreateFromOpsKeepInputs: a caller's op list over the roles in / out / communication buffer as
+    tree launches on in_ptrs (only read) and out_ptrs."""
+
+    def __init__(self, ops, in_ptrs, out_ptrs, dtype, op):
+        n = len(in_ptrs)
+        arr = (SchedOp * max(len(ops), 1))()
+        for i, (step, kind, rank, dbuf, doff, srank, sbuf, soff, nbytes) in enumerate(ops):
+            arr[i] = SchedOp(step, kind, rank, dbuf, srank, sbuf, doff, soff, nbytes)
+        self._in = (_vp * n)(*in_ptrs)
+        self._out = (_vp * n)(*out_ptrs)
+        p = _vp(0)
+        check(_plan_from_ops_keep(arr, len(ops), n, self._in, self._out, dtype, op, C.byref(p)),
+              "HcommGfxPlanCreateFromOpsKeepInputs")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

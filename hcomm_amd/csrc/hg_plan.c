@@ -557,38 +557,54 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
     st.cap = (uint32_t)(2 * ol->n + 1);
     st.cell = (SymCell*)calloc(st.cap, sizeof(SymCell));                       /* at most two new cells per operation */
     st.node = (SymNode*)calloc((size_t)st.cap + ol->n, sizeof(SymNode));       /* and three new nodes */
+    int32_t* pend_cell = (int32_t*)calloc(ol->n + 1, sizeof(int32_t));
+    int32_t* pend_node = (int32_t*)calloc(ol->n + 1, sizeof(int32_t));
     HgLaunch* l = NULL;
-    int rc = (st.cell && st.node) ? HCCL_SUCCESS : HCCL_E_MEMORY;
-    for (uint64_t i = 0; i < ol->n && rc == HCCL_SUCCESS; ++i) {
-        const HcommGfxSchedOp* o = &ol->ops[i];
-        if (o->bytes == 0) continue;
-        /* a list that writes its inputs can only be lowered for a caller who wants them left alone: the launch reads
-         * the original inputs at the leaves and stores nothing into them */
-        if (o->dstBuf == 0 && !inputs_may_change) rc = HCCL_E_NOT_SUPPORT;
-        int32_t src = sym_find(&st, o->srcRank, o->srcBuf, o->srcOff, o->bytes);
-        if (src == -1 && o->srcBuf == 0) { /* first read of an input range: a leaf */
-            SymCell* c = &st.cell[st.ncell];
-            c->rank = o->srcRank;
-            c->buf = 0;
-            c->off = o->srcOff;
-            c->bytes = o->bytes;
-            c->node = sym_node(&st, -1, -1, o->srcRank, o->srcOff);
-            src = (int32_t)st.ncell++;
+    int rc = (st.cell && st.node && pend_cell && pend_node) ? HCCL_SUCCESS : HCCL_E_MEMORY;
+    /* the operations of a step act in parallel: all of them read the state the step began with */
+    for (uint64_t i = 0, j; i < ol->n && rc == HCCL_SUCCESS; i = j) {
+        for (j = i; j < ol->n && ol->ops[j].step == ol->ops[i].step && rc == HCCL_SUCCESS; ++j) {
+            const HcommGfxSchedOp* o = &ol->ops[j];
+            pend_cell[j] = -1;
+            if (o->bytes == 0) continue;
+            /* a list that writes its inputs can only be lowered for a caller who wants them left alone: the launch
+             * reads the original inputs at the leaves and stores nothing into them */
+            if (o->dstBuf == 0 && !inputs_may_change) rc = HCCL_E_NOT_SUPPORT;
+            int32_t src = sym_find(&st, o->srcRank, o->srcBuf, o->srcOff, o->bytes);
+            if (src == -1 && o->srcBuf == 0) { /* first read of an input range: a leaf */
+                SymCell* c = &st.cell[st.ncell];
+                c->rank = o->srcRank;
+                c->buf = 0;
+                c->off = o->srcOff;
+                c->bytes = o->bytes;
+                c->node = sym_node(&st, -1, -1, o->srcRank, o->srcOff);
+                src = (int32_t)st.ncell++;
+            }
+            int32_t dst = sym_find(&st, o->rank, o->dstBuf, o->dstOff, o->bytes);
+            if (src < 0 || dst == -2 || st.cell[src].node < 0) rc = HCCL_E_NOT_SUPPORT; /* other bounds, or never written */
+            if (rc != HCCL_SUCCESS) break;
+            if (dst == -1) {
+                SymCell* c = &st.cell[st.ncell];
+                c->rank = o->rank;
+                c->buf = o->dstBuf;
+                c->off = o->dstOff;
+                c->bytes = o->bytes;
+                /* an input range folded into starts as its own leaf; any other range has no value yet */
+                c->node = (o->dstBuf == 0) ? sym_node(&st, -1, -1, o->rank, o->dstOff) : -1;
+                dst = (int32_t)st.ncell++;
+            }
+            if (o->kind && st.cell[dst].node < 0) {
+                rc = HCCL_E_NOT_SUPPORT;
+                break;
+            }
+            pend_cell[j] = dst;
+            pend_node[j] = o->kind ? sym_node(&st, st.cell[dst].node, st.cell[src].node, 0, 0) : st.cell[src].node;
         }
-        int32_t dst = sym_find(&st, o->rank, o->dstBuf, o->dstOff, o->bytes);
-        if (src < 0 || dst == -2 || (dst == -1 && o->kind && o->dstBuf != 0)) rc = HCCL_E_NOT_SUPPORT;
-        if (rc != HCCL_SUCCESS) break;
-        if (dst == -1) {
-            SymCell* c = &st.cell[st.ncell];
-            c->rank = o->rank;
-            c->buf = o->dstBuf;
-            c->off = o->dstOff;
-            c->bytes = o->bytes;
-            if (o->dstBuf == 0) c->node = sym_node(&st, -1, -1, o->rank, o->dstOff); /* an input range folded into */
-            dst = (int32_t)st.ncell++;
-        }
-        st.cell[dst].node = o->kind ? sym_node(&st, st.cell[dst].node, st.cell[src].node, 0, 0) : st.cell[src].node;
+        for (uint64_t t = i; t < j && rc == HCCL_SUCCESS; ++t)
+            if (pend_cell[t] >= 0) st.cell[pend_cell[t]].node = pend_node[t];
     }
+    free(pend_cell);
+    free(pend_node);
     /* When every rank's output holds the same trees at the same places, the output cells of rank 0 are the segments
      * and the root goes to all outputs; otherwise (whole-message recursive doubling: every rank folds in an order of
      * its own) every output cell is a segment with a single destination. */
@@ -598,6 +614,10 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
         const SymCell* c = &st.cell[i];
         if (c->buf != 1) continue;
         ++nseg_all;
+        if (c->node < 0) {
+            rc = HCCL_E_NOT_SUPPORT;
+            break;
+        }
         const uint32_t d = sym_depth(&st, c->node);
         if (d > depth) depth = d;
         if (c->rank == 0) {
@@ -923,6 +943,49 @@ int32_t HcommGfxPlanCreateFromOps(
     p->info.steps = steps;
     for (uint64_t i = 0; i < nOps; ++i) p->info.algorithmicBytes += ops[i].bytes * (ops[i].kind ? 3u : 2u);
     const int rc = lower_ops(p, ops, nOps, buffers, (int)dataType, (int)reduceOp);
+    if (rc != HCCL_SUCCESS) {
+        HcommGfxPlanDestroy(p);
+        return rc;
+    }
+    p->info.launches = p->nlaunch;
+    *plan = p;
+    return HCCL_SUCCESS;
+}
+
+int32_t HcommGfxPlanCreateFromOpsKeepInputs(
+    const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, void* const* in, void* const* out, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan)
+{
+    if (!plan) return HCCL_E_PTR;
+    *plan = NULL;
+    if ((nOps && !ops) || !in || !out) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    int rc = check_bufs(in, nRanks);
+    if (rc == HCCL_SUCCESS) rc = check_bufs(out, nRanks);
+    if (rc != HCCL_SUCCESS) return rc;
+    const uint32_t unit = HcommGfxDataTypeSize(dataType);
+    uint32_t steps = 0;
+    for (uint64_t i = 0; i < nOps; ++i) {
+        const HcommGfxSchedOp* o = &ops[i];
+        /* roles 0, 1, 2 only: the communication buffers exist in the list but not in the launch */
+        if (o->kind > 1 || o->rank >= nRanks || o->srcRank >= nRanks || o->dstBuf > 2u || o->srcBuf > 2u) return HCCL_E_PARA;
+        if (o->kind == 1 && o->bytes % unit) return HCCL_E_PARA;
+        if (i && o->step < ops[i - 1].step) return HCCL_E_PARA;
+        if (o->step + 1 > steps) steps = o->step + 1;
+    }
+    HcommGfxPlan* p = (HcommGfxPlan*)calloc(1, sizeof(*p));
+    if (!p) return HCCL_E_MEMORY;
+    p->magic = HG_PLAN_MAGIC;
+    p->graph_wanted = use_graph();
+    p->info.steps = steps;
+    for (uint64_t i = 0; i < nOps; ++i) p->info.algorithmicBytes += ops[i].bytes * (ops[i].kind ? 3u : 2u);
+    HgOpList ol;
+    memset(&ol, 0, sizeof(ol));
+    ol.ops = (HcommGfxSchedOp*)ops; /* only read */
+    ol.n = nOps;
+    ol.steps = steps;
+    rc = fused_from_trees(p, &ol, nRanks, in, out, (int)dataType, (int)reduceOp, 1);
     if (rc != HCCL_SUCCESS) {
         HcommGfxPlanDestroy(p);
         return rc;

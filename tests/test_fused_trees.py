@@ -195,6 +195,66 @@ def test_recursive_doubling_keep_inputs_launch_holds_every_ranks_own_tree(n):
     assert e.value.code == R.E_NOT_SUPPORT
 
 
+OPLIST_CASES = [
+    # oracle algorithm, ranks: schedules whose trees are at most 5 folds deep and whose ranges keep their bounds
+    (oracle.ALG_ALLREDUCE_RING, 2), (oracle.ALG_ALLREDUCE_RING, 4), (oracle.ALG_ALLREDUCE_RING, 6),
+    (oracle.ALG_ALLREDUCE_MESH_ONESHOT, 3), (oracle.ALG_ALLREDUCE_MESH_ONESHOT, 6), (oracle.ALG_ALLREDUCE_MESH_ASCENDING, 5),
+    (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, 8), (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, 16),
+    (oracle.ALG_ALLREDUCE_DOUBLING, 8), (oracle.ALG_ALLREDUCE_NHR_ONESHOT, 7), (oracle.ALG_ALLREDUCE_NB, 6),
+]
+
+
+@pytest.mark.parametrize("oalg,n", OPLIST_CASES)
+def test_any_op_list_with_shallow_trees_lowers_to_tree_launches(oalg, n):
+    """HcommGfxPlanCreateFromOpsKeepInputs on the oracle's operation lists: the launches' trees are the replay's."""
+    ins, outs, rank_of = ptrs(n)
+    count = 6 * 8192 * 5
+    ops = oracle.trace(oalg, n, count, oracle.F32)
+    plan = h.OpListKeepInputsPlan(ops, ins, outs, oracle.F32, oracle.SUM)
+    try:
+        if oalg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE:     # slots at other offsets than the slices: the exact-cell replay
+            per_rank = [{k: strip(v, k[0]) for k, v in cells.items()} for cells in output_trees(ops, n)]
+        else:
+            per_rank = output_trees_in_place(ops, n)
+        got = [{} for _ in range(n)]
+        for i, rec in enumerate(plan.launches()):
+            assert rec.kind == h.Kernel.TREE
+            for sg in range(rec.nseg):
+                tree, off, nbytes, owner = h.plan_tree(plan, i, sg, rank_of, with_owner=True)
+                for r in (range(n) if owner < 0 else [owner]):
+                    assert (off, nbytes) not in got[r]
+                    got[r][(off, nbytes)] = tree
+        for r in range(n):
+            assert merged_runs(got[r]) == merged_runs(per_rank[r]), r
+    finally:
+        plan.destroy()
+
+
+def test_op_lists_the_tree_lowering_refuses():
+    ins, outs, _ = ptrs(8)
+    for oalg, n in ((oracle.ALG_ALLREDUCE_RING, 8),          # chains of 7 folds
+                    (oracle.ALG_ALLREDUCE_RHD, 8),           # halving steps fold several slices as one range
+                    (oracle.ALG_ALLREDUCE_CHUNK_MESH, 4),    # copies the whole message, then folds sub-chunks of it
+                    (oracle.ALG_RS_MESH, 4)):                # slice r of every input lands at offset 0 of out[r]
+        with pytest.raises(h.HcommError) as e:
+            h.OpListKeepInputsPlan(oracle.trace(oalg, n, 1 << 18, oracle.F32), ins[:n], outs[:n], oracle.F32, oracle.SUM)
+        assert e.value.code == R.E_NOT_SUPPORT, oalg
+    with pytest.raises(h.HcommError) as e:                   # a value read that the list never wrote
+        h.OpListKeepInputsPlan([(0, 0, 0, 1, 0, 1, 2, 0, 4096)], ins[:2], outs[:2], oracle.F32, oracle.SUM)
+    assert e.value.code == R.E_NOT_SUPPORT
+    with pytest.raises(h.HcommError) as e:                   # a user-buffer role of the op-base lists
+        h.OpListKeepInputsPlan([(0, 0, 0, 1, 0, 1, 3, 0, 4096)], ins[:2], outs[:2], oracle.F32, oracle.SUM)
+    assert e.value.code == R.E_PARA
+    # two operations of one step read the state the step began with: a swap through the outputs
+    p = h.OpListKeepInputsPlan([(0, 0, 0, 1, 0, 0, 0, 0, 4096), (0, 0, 1, 1, 0, 1, 0, 0, 4096),
+                                (1, 1, 0, 1, 0, 1, 1, 0, 4096), (1, 1, 1, 1, 0, 0, 1, 0, 4096)], ins[:2], outs[:2],
+                               oracle.F32, oracle.SUM)
+    rank_of = {ins[0]: 0, ins[1]: 1}
+    trees = {h.plan_tree(p, 0, sg, rank_of, with_owner=True)[3]: h.plan_tree(p, 0, sg, rank_of)[0] for sg in range(2)}
+    assert trees == {0: [0, 1], 1: [1, 0]}                   # not [0, [1, 0]]: rank 1's fold reads out[0] of before the step
+    p.destroy()
+
+
 def merged_runs(segments):
     """[(lo, hi, tree)] with neighbours that hold the same tree joined: independent of how the bytes were cut."""
     out = []

@@ -310,6 +310,39 @@ def test_fused_lowering_that_keeps_the_inputs(gpu_thread, alg, n, count, dtype, 
         plan.destroy()
 
 
+@pytest.mark.parametrize("alg,n,count,dtype,op", [
+    ("ring_ar", 6, 100003, "fp32", "sum"), ("ring_ar", 4, 65536, "bf16", "max"), ("ring_ar", 2, 5, "int8", "sum"),
+    ("mesh_oneshot", 6, 4097, "fp16", "sum"), ("mesh_ascending", 5, 100003, "fp32", "sum"),
+    ("local_reduce", 16, 1 << 20, "bf16", "sum"), ("doubling", 8, 2048, "fp16", "sum"),
+    ("nhr_oneshot", 7, 70001, "fp32", "sum"), ("nb_ar", 6, 300007, "int32", "min"),
+])
+def test_op_list_as_tree_launches_that_keep_the_inputs(gpu_thread, alg, n, count, dtype, op):
+    """HcommGfxPlanCreateFromOpsKeepInputs on the oracle's own operation list: outputs as the oracle's replay leaves
+    them, inputs as they were."""
+    say("op list as trees", alg, n, count, dtype, op)
+    dt, o = DT[dtype], OPS[op]
+    host_in = [gen(dt, count, 9000 + r) for r in range(n)]
+    sentinel = gen(dt, count, 999, "wide")
+    want_in = [x.copy() for x in host_in]
+    want_out = [sentinel.copy() for _ in range(n)]
+    sb = h.scratch_bytes(ALGS[alg][0], n, count, dt)
+    oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o,
+               scratch=[np.zeros(sb, np.uint8) for _ in range(n)] if sb else None)
+    d_in = [to_dev(x) for x in host_in]
+    d_out = [to_dev(sentinel) for _ in range(n)]
+    plan = h.OpListKeepInputsPlan(oracle.trace(ALGS[alg][1], n, count, dt), [t.data_ptr() for t in d_in],
+                                  [t.data_ptr() for t in d_out], dt, o)
+    try:
+        assert all(r.kind == h.Kernel.TREE for r in plan.launches())
+        assert plan.run(gpu_thread) == 0
+        assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+        for r in range(n):
+            assert_same(from_dev(d_in[r], host_in[r]), host_in[r], dt, "in[%d]" % r)
+            assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+    finally:
+        plan.destroy()
+
+
 @pytest.mark.parametrize("alg", SCATTER)
 @pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
 def test_strided_reduce_scatter(gpu_thread, alg, lowering):
