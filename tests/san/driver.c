@@ -133,6 +133,23 @@ int main(void)
                     run_plan(th, p);
                 }
     }
+    /* any schedule's own list as tree launches that keep the inputs (most are refused: deep or re-cut trees) */
+    for (int alg = 0; alg <= 17; ++alg)
+        for (uint32_t n = 1; n <= 9; ++n) {
+            uint64_t total = 0;
+            if (HcommGfxScheduleEmit(alg, n, 40960, HCOMM_DATA_TYPE_FP32, NULL, 0, &total) != 0 || total == 0) continue;
+            HcommGfxSchedOp* ops = (HcommGfxSchedOp*)calloc(total, sizeof(*ops));
+            if (!ops) return 2;
+            if (HcommGfxScheduleEmit(alg, n, 40960, HCOMM_DATA_TYPE_FP32, ops, total, &total) == 0) {
+                p = NULL;
+                if (HcommGfxPlanCreateFromOpsKeepInputs(ops, total, n, bufs[0], bufs[1], HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_MAX, &p) == 0) ++checks;
+                run_plan(th, p);
+                p = NULL;
+                HcommGfxPlanCreateFromOpsKeepInputs(ops, total / 2, n, bufs[0], bufs[1], HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_MAX, &p); /* a truncated list */
+                run_plan(th, p);
+            }
+            free(ops);
+        }
     /* two-level executors */
     for (unsigned si = 0; si < 5; ++si)
         for (unsigned li = 0; li < 5; ++li)
