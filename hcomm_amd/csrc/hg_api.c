@@ -286,14 +286,18 @@ int hg_submit(HgThread* t, const HgLaunch* l)
     log_launch(t, l);
     if (t->recorder) return HCCL_SUCCESS;
     switch (l->kind) {
-        case HCOMM_GFX_KERNEL_COPY: return hg_launch_copy(t->stream, &l->tab.seg2, l->blocks);
+        case HCOMM_GFX_KERNEL_COPY:
+            return hg_launch_copy(t->stream, &l->tab.seg2, l->blocks, (int)l->streaming, l->lds_bytes);
         case HCOMM_GFX_KERNEL_REDUCE2:
-            return hg_launch_reduce2(t->stream, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks);
+            return hg_launch_reduce2(t->stream, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks, (int)l->streaming,
+                                     l->lds_bytes);
         case HCOMM_GFX_KERNEL_BYTEWISE:
-            return hg_launch_bytewise(t->stream, l->op != 255u, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks);
+            return hg_launch_bytewise(t->stream, l->op != 255u, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks,
+                                      l->lds_bytes);
         case HCOMM_GFX_KERNEL_CHAIN:
         case HCOMM_GFX_KERNEL_TREE:
-            return hg_launch_fold(t->stream, (int)l->dtype, (int)l->op, (int)l->acc_is_dst, &l->tab.fold, l->blocks);
+            return hg_launch_fold(t->stream, (int)l->dtype, (int)l->op, (int)l->acc_is_dst, &l->tab.fold, l->blocks,
+                                  l->lds_bytes);
         default: return HCCL_E_INTERNAL;
     }
 }

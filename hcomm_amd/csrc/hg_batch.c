@@ -30,20 +30,88 @@ static uint64_t env_once(uint64_t* slot, const char* name, uint64_t unset)
     return v;
 }
 
-uint64_t hg_grid_blocks(uint64_t total_tiles, int capped)
+uint64_t hg_grid_blocks(uint64_t total_tiles)
 {
+    /* One tile per workgroup, however many that makes: measured with the streaming probe, every grid held at a fixed
+     * number of workgroups per CU streams slower (16 x 64 MiB two-input reduce: 5.7 TB/s at 32 per CU, 6.4 without a
+     * limit; copy 5.8 against 6.4).  HCOMM_GFX_GRID_CAP limits the grid for experiments. */
     const uint64_t forced = env_once(&g_grid_cap, "HCOMM_GFX_GRID_CAP", UINT64_MAX);
-    if (forced != UINT64_MAX) return total_tiles < forced ? total_tiles : forced; /* experiments: every kernel */
-    /* Measured over the benchmark configurations: one tile per workgroup, however many that makes, streams best for
-     * the copy and the k-way fold kernels (a 2 GiB copy: 5.84 against 5.38 TB/s with the grid held at 32 workgroups
-     * per CU; the fused 16-rank tree: 0.95 against 1.05 ms).  The two-input reduce is the exception: on the ragged
-     * 7-rank reduce-scatter it loses 6 % without the limit, so it keeps it (its 128 MiB ring step has exactly
-     * 32 workgroups per CU worth of tiles either way). */
-    if (!capped) return total_tiles;
-    int cus = hg_rt_num_cus();
-    if (cus <= 0) cus = 256;
-    const uint64_t cap = (uint64_t)cus * 32u;
-    return total_tiles < cap ? total_tiles : cap;
+    if (forced != UINT64_MAX) return total_tiles < forced ? total_tiles : forced;
+    return total_tiles;
+}
+
+/*
+ * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip; 16 KiB tiles, bf16 SUM,
+ * seeded non-zero data, fractions of 8 TB/s).  Two regimes:
+ *   kept      what the launch writes fits the memory-side cache and a later launch reads it back from there (a ring
+ *             step): plain stores, the overwritten operand loaded plain, XCDs walking runs of 128 tiles.
+ *             8 x 16 MiB ring steps: reduce 0.860 (0.827 with that operand loaded non-temporal and tiles as dealt),
+ *             copy 0.873 with at most five workgroups per CU (0.864 without that bound).
+ *   streaming everything non-temporal and at most three workgroups per CU in flight.  16 x 64 MiB that nothing touched
+ *             recently: reduce 0.823 with runs of 32 tiles (0.795 without the bound, 0.711 with the grid held at 32
+ *             workgroups per CU), copy 0.808 with runs of 128 (0.744 without the bound).
+ * The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
+ * Every figure can be overridden from the environment for experiments.
+ */
+enum {
+    TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE,
+    TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_FOLD,
+    TUNE_N
+};
+static const struct {
+    const char* env;
+    uint64_t dflt;
+} g_tune_def[TUNE_N] = {
+    {"HCOMM_GFX_STREAM_COPY_BYTES", 256ull << 20},   /* the 256 MB memory-side cache */
+    {"HCOMM_GFX_STREAM_REDUCE_BYTES", 256ull << 20},
+    {"HCOMM_GFX_LDS_COPY", 32768},
+    {"HCOMM_GFX_LDS_COPY_STREAM", 53248},
+    {"HCOMM_GFX_LDS_REDUCE", 0},
+    {"HCOMM_GFX_LDS_REDUCE_STREAM", 53248},
+    {"HCOMM_GFX_XCD_RUN_COPY", 128},
+    {"HCOMM_GFX_XCD_RUN_COPY_STREAM", 128},
+    {"HCOMM_GFX_XCD_RUN_REDUCE", 128},
+    {"HCOMM_GFX_XCD_RUN_REDUCE_STREAM", 32},
+    {"HCOMM_GFX_LDS_FOLD", 0},
+};
+static uint64_t g_tune[TUNE_N]; /* value + 1; 0 = not read yet (same relaxed-atomic rule as env_once) */
+
+static uint64_t tune(int i)
+{
+    uint64_t v = __atomic_load_n(&g_tune[i], __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv(g_tune_def[i].env);
+        v = (e && *e ? strtoull(e, NULL, 10) : g_tune_def[i].dflt) + 1u;
+        __atomic_store_n(&g_tune[i], v, __ATOMIC_RELAXED);
+    }
+    return v - 1u;
+}
+
+#define HG_LDS_MAX 65536u /* what a launch may ask for without raising the kernel's limit */
+
+static uint32_t lds_of(int i)
+{
+    const uint64_t v = tune(i);
+    return v > HG_LDS_MAX ? HG_LDS_MAX : (uint32_t)v;
+}
+
+/* Shape of a copy / two-input reduce launch from the bytes it writes; `streaming` < 0 lets the size decide. */
+void hg_shape_seg2(HgLaunch* l, int streaming)
+{
+    HgSeg2Table* t = &l->tab.seg2;
+    if (l->kind == HCOMM_GFX_KERNEL_COPY) {
+        l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_COPY_BYTES));
+        l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_COPY_STREAM : TUNE_LDS_COPY);
+        t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_COPY_STREAM : TUNE_RUN_COPY);
+    } else if (l->kind == HCOMM_GFX_KERNEL_REDUCE2) {
+        l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_REDUCE_BYTES));
+        l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_REDUCE_STREAM : TUNE_LDS_REDUCE);
+        t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_REDUCE_STREAM : TUNE_RUN_REDUCE);
+    } else {
+        l->streaming = 0;
+        l->lds_bytes = 0;
+        t->xcd_run = 0;
+    }
 }
 
 static uint64_t tiles_of(uint64_t bytes) { return (bytes + HG_TILE_BYTES - 1) / HG_TILE_BYTES; }
@@ -61,13 +129,16 @@ void hg_finish_seg2(HgLaunch* l)
     l->nseg = t->nseg;
     l->bytes = bytes;
     l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
-    l->blocks = hg_grid_blocks(tiles, l->kind != HCOMM_GFX_KERNEL_COPY);
+    l->blocks = hg_grid_blocks(tiles);
+    hg_shape_seg2(l, -1);
 }
 
 void hg_finish_fold(HgLaunch* l)
 {
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
+    l->streaming = 0;
+    l->lds_bytes = lds_of(TUNE_LDS_FOLD);
     if (!t->tree) {
         /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
         const uint64_t small_bytes = env_once(&g_small_bytes, "HCOMM_GFX_SMALL_BYTES", 1u << 20);
@@ -99,7 +170,7 @@ void hg_finish_fold(HgLaunch* l)
              * (none for the rank-order trees, which only read their inputs), and the root to one output or to all */
             const uint64_t n = (uint64_t)t->nranks + ((t->tree >= 4u || t->keep_inputs) ? 0u : t->nranks / 2) + (t->out_mode == 1u ? 1u : t->nout);
             l->moved_bytes = n * bytes;
-            l->blocks = hg_grid_blocks(tiles, 0);
+            l->blocks = hg_grid_blocks(tiles);
             return;
         }
         for (uint32_t s = 0; s < t->nseg; ++s) {
@@ -109,7 +180,7 @@ void hg_finish_fold(HgLaunch* l)
             moved += n * t->bytes[s];
         }
         l->moved_bytes = moved;
-        l->blocks = hg_grid_blocks(tiles, 0);
+        l->blocks = hg_grid_blocks(tiles);
         return;
     } else {
         if (t->store_partials) per += t->k - 1;
@@ -118,7 +189,7 @@ void hg_finish_fold(HgLaunch* l)
         if (t->out_mode == 2) per += t->nranks;
     }
     l->moved_bytes = bytes * per;
-    l->blocks = hg_grid_blocks(tiles, 0);
+    l->blocks = hg_grid_blocks(tiles);
 }
 
 static int overlaps(const void* a, uint64_t an, const void* b, uint64_t bn)

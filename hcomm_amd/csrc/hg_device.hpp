@@ -128,19 +128,18 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
     else *(uint32_t*)p = v;
 }
 
-// Cache hints.  A ring step reads what the neighbouring rank's previous step wrote, so plain stores are left
-// to be kept by the memory-side cache while every load is marked non-temporal (each value is read once).
-#ifndef HG_NT_LD_DST
-#define HG_NT_LD_DST 1 /* the operand that is overwritten */
-#endif
+// Cache hints.  Measured with the streaming probe (hg_probe.hip) on 8 x 16 MiB ring steps and on 16 x 64 MiB
+// launches whose operands nothing touched recently:
+//   * a launch whose output the next launch reads back from the memory-side cache (a ring step): peer operand
+//     loaded non-temporal, the operand that is overwritten loaded plain, plain stores;
+//   * a launch that streams (what it writes is more than that cache holds, or nothing reads it soon): every load
+//     and store non-temporal, and no more than three workgroups per CU in flight.
+// Fold launches store non-temporal: nothing they write is read again by the same launch.
 #ifndef HG_NT_LD_SRC
 #define HG_NT_LD_SRC 1 /* the peer's operand */
 #endif
-#ifndef HG_NT_ST
-#define HG_NT_ST 0
-#endif
 #ifndef HG_NT_FOLD_ST
-#define HG_NT_FOLD_ST 1 /* nothing a fold launch stores is read again by it */
+#define HG_NT_FOLD_ST 1
 #endif
 template <bool NT> __device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec)
 {
@@ -153,46 +152,30 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
     else ((u32x4*)base)[vec] = v;
 }
 
-// Workgroups are dealt to the 8 XCDs round-robin by their index.  REMAP renumbers them so that each XCD walks runs
-// of HG_XCD_RUN consecutive tiles (2 MiB) - or, when the grid does not divide that way, one contiguous eighth of the
-// tiles - instead of every eighth tile.  Measured on the 8 x 128 MiB ring steps (TB/s; plain, runs of 2 / 8 / 32 /
-// 128 tiles, contiguous eighth): copy 6.68, 6.69, 6.65, 6.84, 6.93, 6.87; two-input reduce 6.47, 6.49, 6.53, 6.35,
-// 6.51, 6.17; k-way fold 5.50, 5.44, 5.56, 5.59, 5.15, 4.84.  Only the copy gains beyond run-to-run noise, so only
-// k_copy renumbers.
-#ifndef HG_STREAM_COPY_BYTES
-#define HG_STREAM_COPY_BYTES (256ull << 20) /* the 256 MB memory-side cache */
-#endif
-#ifndef HG_STREAM_REDUCE_BYTES
-#define HG_STREAM_REDUCE_BYTES (256ull << 20)
-#endif
-#ifndef HG_XCD_REMAP_COPY
-#define HG_XCD_REMAP_COPY 1
-#endif
-#ifndef HG_XCD_REMAP
-#define HG_XCD_REMAP 0
-#endif
-#ifndef HG_XCD_RUN
-#define HG_XCD_RUN 128u
-#endif
-template <bool REMAP> __device__ __forceinline__ uint32_t block_id()
+// Workgroups are dealt to the 8 XCDs round-robin by their index.  With run > 0 they are renumbered so that each XCD
+// walks runs of `run` consecutive tiles instead of every eighth tile; the workgroups beyond the last whole group of
+// 8 * run keep their numbers.  run == 0: as dealt.
+__device__ __forceinline__ uint32_t block_id(uint32_t run)
 {
     const uint32_t g = gridDim.x, b = blockIdx.x;
-    if (!REMAP) return b;
-    if ((g % (8u * HG_XCD_RUN)) == 0u) {
-        const uint32_t i = b >> 3;
-        return (i / HG_XCD_RUN) * 8u * HG_XCD_RUN + (b & 7u) * HG_XCD_RUN + i % HG_XCD_RUN;
-    }
-    if ((g & 7u) == 0u) return (b & 7u) * (g >> 3) + (b >> 3);
-    return b;
+    if (run == 0u) return b;
+    const uint32_t span = 8u * run;
+    if (b >= g - g % span) return b;
+    const uint32_t i = b >> 3;
+    return (i / run) * span + (b & 7u) * run + i % run;
 }
 
-// segment that owns a tile: the last s with tile_begin[s] <= tile (uniform across the workgroup, so the search runs
-// on the scalar unit; bisection keeps it at 6 probes for the largest table)
+// segment that owns a tile: the last s with tile_begin[s] <= tile (uniform across the workgroup, so the bisection
+// runs on the scalar unit: at most 6 probes for the largest table)
 __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
 {
-    uint32_t s = 0;
-    while (s + 1 < nseg && tile >= tile_begin[s + 1]) ++s;
-    return s;
+    uint32_t lo = 0, hi = nseg; // tile_begin[lo] <= tile < tile_begin[hi]
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (tile >= tile_begin[mid]) lo = mid;
+        else hi = mid;
+    }
+    return lo;
 }
 
 template <int DT, int OP> struct VecItem {

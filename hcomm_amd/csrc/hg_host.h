@@ -29,6 +29,8 @@ typedef struct {
     uint64_t bytes;       /* output bytes covered */
     uint64_t moved_bytes; /* bytes read + written */
     uint32_t nseg;
+    uint32_t streaming;   /* copy / two-input reduce: nothing it writes is expected in the memory-side cache later */
+    uint32_t lds_bytes;   /* dynamic LDS per workgroup: bounds the workgroups per CU, never used as memory */
     union {
         HgSeg2Table seg2;
         HgFoldTable fold;
@@ -59,8 +61,10 @@ typedef int (*HgEmitFn)(const HgLaunch* launch, void* ctx);
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
 uint64_t hg_split_head(const HgOp* o); /* bytes before the 16-byte boundary both operands reach together, or 0 */
 
-/* Fill tile_begin / blocks / bytes of a launch whose segment pointers and sizes are set. */
+/* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment
+ * pointers and sizes are set. */
 void hg_finish_seg2(HgLaunch* l);
+void hg_shape_seg2(HgLaunch* l, int streaming); /* streaming < 0: decided by the bytes the launch writes */
 void hg_finish_fold(HgLaunch* l);
 
 /* Execute (or, on a recorder thread, log) one prepared launch. */

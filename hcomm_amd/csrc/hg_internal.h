@@ -38,6 +38,7 @@ typedef struct {
     uint64_t bytes[HG_MAX_SEG2];
     uint32_t tile_begin[HG_MAX_SEG2 + 1]; /* prefix sum of tiles per segment */
     uint32_t nseg;
+    uint32_t xcd_run; /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
 } HgSeg2Table;
 
 /*
@@ -84,13 +85,15 @@ typedef struct {
 } HgFoldTable;
 
 /* Launch geometry decided on the host so that recorder threads can report it without a GPU. */
-uint64_t hg_grid_blocks(uint64_t total_tiles, int capped);
+uint64_t hg_grid_blocks(uint64_t total_tiles);
 
 /* Launchers.  stream is a hipStream_t.  Return a HcclResult-compatible code. */
-int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks);
-int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks);
-int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks);
-int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks);
+/* streaming: non-temporal stores (and, for the reduce, a non-temporal load of the operand it overwrites);
+ * lds: bytes of dynamic LDS per workgroup, asked for only to bound the workgroups a CU runs at once */
+int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
+int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
+int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, uint32_t lds);
+int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks, uint32_t lds);
 
 /* Thin wrappers over the HIP runtime so that the C files need no HIP headers. */
 int hg_rt_device_count(void);

@@ -11,13 +11,14 @@ namespace {
 
 // ---- batched copy ------------------------------------------------------------------------------
 
-// STREAM: what the launch writes exceeds the memory-side cache, so nothing of it can be found there by the next
-// launch anyway: store with the non-temporal hint (measured on a 2 GiB copy: 6.12 against 5.88 TB/s).
+// STREAM: nothing of what the launch writes will be found in the memory-side cache by a later launch (there is more
+// of it than that cache holds, or nothing reads it soon): store with the non-temporal hint.  The launch's dynamic
+// LDS size is not used as memory: it bounds the workgroups a CU runs at once (hg_launch_lds in hg_batch.c).
 template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP_COPY>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -29,12 +30,12 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM || HG_NT_ST>(d, v0 + u * HG_BLOCK, a[u]);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, a[u]);
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv<STREAM || HG_NT_ST>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+                if (v < nvec) stv<STREAM>(d, v, ldv<HG_NT_LD_SRC>(p, v));
             }
             const uint64_t b = (nvec << 4) + tid; // this tile is the segment's last one: byte tail
             if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
@@ -44,12 +45,14 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 
 // ---- batched dst = dst (op) src -----------------------------------------------------------------
 
+// STREAM as for k_copy; it also decides how the operand that is overwritten is loaded: non-temporal when the launch
+// streams, plain when a later launch is to find the result in the memory-side cache.
 template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2(const HgSeg2Table tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -59,16 +62,16 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
         if (v0 - tid + HG_TILE_VECS <= nvec) {
             u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_DST>(d, v0 + u * HG_BLOCK);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<STREAM>(d, v0 + u * HG_BLOCK);
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM || HG_NT_ST>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv<STREAM || HG_NT_ST>(d, v, vec_op<DT, OP>(ldv<HG_NT_LD_DST>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+                if (v < nvec) stv<STREAM>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -100,7 +103,7 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
     typedef typename UVec<ES>::T UV;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t bytes = tab.bytes[s];
         uint8_t* d0 = (uint8_t*)tab.dst[s];
@@ -117,7 +120,7 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
             const uint64_t v = vb + tid + u * HG_BLOCK;
             if (v < nvec) {
                 b[u] = __builtin_nontemporal_load((const UV*)(p + (v << 4)));
-                if (REDUCE) a[u] = ldv<HG_NT_LD_DST>(d, v);
+                if (REDUCE) a[u] = ldv<true>(d, v);
             }
         }
 #pragma unroll
@@ -139,33 +142,35 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 
 // ---- dispatch -----------------------------------------------------------------------------------
 
-template <int DT, bool STREAM> int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
+template <int DT, bool STREAM>
+int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
 {
+    const dim3 g(blocks), b(HG_BLOCK);
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_reduce2<DT, OP_PROD, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_reduce2<DT, OP_MAX, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_reduce2<DT, OP_MIN, STREAM>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM, STREAM>), g, b, lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_reduce2<DT, OP_PROD, STREAM>), g, b, lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_reduce2<DT, OP_MAX, STREAM>), g, b, lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_reduce2<DT, OP_MIN, STREAM>), g, b, lds, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
 }
 
-template <int DT> int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
+template <int DT>
+int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, int streaming, uint32_t lds)
 {
-    uint64_t bytes = 0; /* what the launch writes */
-    for (uint32_t s = 0; s < tab->nseg; ++s) bytes += tab->bytes[s];
-    if (bytes > HG_STREAM_REDUCE_BYTES) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks);
-    return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks);
+    if (streaming) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks, lds);
+    return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks, lds);
 }
 
-template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks)
+template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
 {
+    const dim3 g(blocks), b(HG_BLOCK);
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_bytewise<DT, OP_SUM, true>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_bytewise<DT, OP_PROD, true>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_bytewise<DT, OP_MAX, true>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_bytewise<DT, OP_MIN, true>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_bytewise<DT, OP_SUM, true>), g, b, lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_bytewise<DT, OP_PROD, true>), g, b, lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_bytewise<DT, OP_MAX, true>), g, b, lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_bytewise<DT, OP_MIN, true>), g, b, lds, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
@@ -176,35 +181,33 @@ template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Tab
 extern "C" {
 
 
-int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks)
+int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-    uint64_t bytes = 0;
-    for (uint32_t s = 0; s < tab->nseg; ++s) bytes += tab->bytes[s];
-    if (bytes > HG_STREAM_COPY_BYTES)
-        hipLaunchKernelGGL(k_copy<true>, dim3((uint32_t)blocks), dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
+    if (streaming)
+        hipLaunchKernelGGL(k_copy<true>, dim3((uint32_t)blocks), dim3(HG_BLOCK), lds, (hipStream_t)stream, *tab);
     else
-        hipLaunchKernelGGL(k_copy<false>, dim3((uint32_t)blocks), dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
+        hipLaunchKernelGGL(k_copy<false>, dim3((uint32_t)blocks), dim3(HG_BLOCK), lds, (hipStream_t)stream, *tab);
     return rc(hipGetLastError());
 }
 
-int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks)
+int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-#define CALL(DT) launch_reduce2_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks)
+#define CALL(DT) launch_reduce2_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, streaming, lds)
     HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
 }
 
-int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks)
+int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
     if (!is_reduce) {
-        hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false>), dim3((uint32_t)blocks), dim3(HG_BLOCK), 0,
+        hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false>), dim3((uint32_t)blocks), dim3(HG_BLOCK), lds,
                            (hipStream_t)stream, *tab);
         return rc(hipGetLastError());
     }
-#define CALL(DT) launch_bytewise_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks)
+#define CALL(DT) launch_bytewise_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, lds)
     HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
 }

@@ -3,7 +3,7 @@
 
 #include "hg_device.hpp"
 
-extern "C" int hg_launch_tree(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks);
+extern "C" int hg_launch_tree(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks, uint32_t lds);
 
 namespace {
 
@@ -97,7 +97,7 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -181,24 +181,24 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     }
 }
 
-template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
     if (tab->small) {
         switch (op) {
-            case OP_SUM: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_SUM, AD>), g, b, 0, st, *tab); break;
-            case OP_PROD: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_PROD, AD>), g, b, 0, st, *tab); break;
-            case OP_MAX: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MAX, AD>), g, b, 0, st, *tab); break;
-            case OP_MIN: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MIN, AD>), g, b, 0, st, *tab); break;
+            case OP_SUM: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_SUM, AD>), g, b, lds, st, *tab); break;
+            case OP_PROD: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_PROD, AD>), g, b, lds, st, *tab); break;
+            case OP_MAX: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MAX, AD>), g, b, lds, st, *tab); break;
+            case OP_MIN: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_MIN, AD>), g, b, lds, st, *tab); break;
             default: return HCCL_E_PARA;
         }
         return rc(hipGetLastError());
     }
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_fold_chain<DT, OP_SUM, AD>), g, b, 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_fold_chain<DT, OP_PROD, AD>), g, b, 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_fold_chain<DT, OP_MAX, AD>), g, b, 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_fold_chain<DT, OP_MIN, AD>), g, b, 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_fold_chain<DT, OP_SUM, AD>), g, b, lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_chain<DT, OP_PROD, AD>), g, b, lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_chain<DT, OP_MAX, AD>), g, b, lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_chain<DT, OP_MIN, AD>), g, b, lds, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
@@ -208,16 +208,16 @@ template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFo
 
 extern "C" {
 
-int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks)
+int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-    if (tab->tree) return hg_launch_tree(stream, dtype, op, tab, blocks);
+    if (tab->tree) return hg_launch_tree(stream, dtype, op, tab, blocks, lds);
     if (acc_is_dst) {
-#define CALL(DT) launch_fold_dt<DT, true>((hipStream_t)stream, op, tab, (uint32_t)blocks)
+#define CALL(DT) launch_fold_dt<DT, true>((hipStream_t)stream, op, tab, (uint32_t)blocks, lds)
         HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
     } else {
-#define CALL(DT) launch_fold_dt<DT, false>((hipStream_t)stream, op, tab, (uint32_t)blocks)
+#define CALL(DT) launch_fold_dt<DT, false>((hipStream_t)stream, op, tab, (uint32_t)blocks, lds)
         HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
     }

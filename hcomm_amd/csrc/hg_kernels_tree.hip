@@ -162,7 +162,7 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     constexpr uint32_t NU = HG_TREE_NU(1u << L);
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id<HG_XCD_REMAP>(); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * NU) + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -185,26 +185,26 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     }
 }
 
-template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L>), dim3(blocks), dim3(HG_BLOCK), 0, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
 }
 
-template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks)
+template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     switch (tab->k) {
-        case 2: return launch_tree_dt_l<DT, 1>(st, op, tab, blocks);
-        case 4: return launch_tree_dt_l<DT, 2>(st, op, tab, blocks);
-        case 8: return launch_tree_dt_l<DT, 3>(st, op, tab, blocks);
-        case 16: return launch_tree_dt_l<DT, 4>(st, op, tab, blocks);
-        case 32: return launch_tree_dt_l<DT, 5>(st, op, tab, blocks);
+        case 2: return launch_tree_dt_l<DT, 1>(st, op, tab, blocks, lds);
+        case 4: return launch_tree_dt_l<DT, 2>(st, op, tab, blocks, lds);
+        case 8: return launch_tree_dt_l<DT, 3>(st, op, tab, blocks, lds);
+        case 16: return launch_tree_dt_l<DT, 4>(st, op, tab, blocks, lds);
+        case 32: return launch_tree_dt_l<DT, 5>(st, op, tab, blocks, lds);
         default: return HCCL_E_PARA;
     }
 }
@@ -218,26 +218,26 @@ template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* 
 #endif
 
 #if HG_TREE_PART == 0
-extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks);
+extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks, uint32_t lds);
 
-extern "C" int hg_launch_tree(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks)
+extern "C" int hg_launch_tree(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks, uint32_t lds)
 {
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case DT_I8: return launch_tree_dt<DT_I8>(st, op, tab, (uint32_t)blocks);
-        case DT_I16: return launch_tree_dt<DT_I16>(st, op, tab, (uint32_t)blocks);
-        case DT_I32: return launch_tree_dt<DT_I32>(st, op, tab, (uint32_t)blocks);
-        default: return hg_launch_tree_float(stream, dtype, op, tab, blocks);
+        case DT_I8: return launch_tree_dt<DT_I8>(st, op, tab, (uint32_t)blocks, lds);
+        case DT_I16: return launch_tree_dt<DT_I16>(st, op, tab, (uint32_t)blocks, lds);
+        case DT_I32: return launch_tree_dt<DT_I32>(st, op, tab, (uint32_t)blocks, lds);
+        default: return hg_launch_tree_float(stream, dtype, op, tab, blocks, lds);
     }
 }
 #else
-extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks)
+extern "C" int hg_launch_tree_float(void* stream, int dtype, int op, const HgFoldTable* tab, uint64_t blocks, uint32_t lds)
 {
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case DT_F16: return launch_tree_dt<DT_F16>(st, op, tab, (uint32_t)blocks);
-        case DT_F32: return launch_tree_dt<DT_F32>(st, op, tab, (uint32_t)blocks);
-        case DT_BF16: return launch_tree_dt<DT_BF16>(st, op, tab, (uint32_t)blocks);
+        case DT_F16: return launch_tree_dt<DT_F16>(st, op, tab, (uint32_t)blocks, lds);
+        case DT_F32: return launch_tree_dt<DT_F32>(st, op, tab, (uint32_t)blocks, lds);
+        case DT_BF16: return launch_tree_dt<DT_BF16>(st, op, tab, (uint32_t)blocks, lds);
         default: return HCCL_E_PARA;
     }
 }

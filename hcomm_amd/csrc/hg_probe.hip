@@ -1,0 +1,464 @@
+// hg_probe.hip - streaming probe for one MI355X: the copy / two-input reduce loops of libhcomm_gfx.so with every
+// launch-shape choice opened up as a parameter, plus read-only and write-only loops that bracket what the memory
+// system gives each access mix.  A stand-alone program (make hg_probe); nothing in the library links it.
+//
+//   hg_probe [file]      one configuration per line of `file` (or stdin): space-separated key=value pairs
+//                        (unknown keys are an error); one JSON line per configuration on stdout.
+//
+// keys (defaults)  kind=reduce|reduce_i32|copy|read|write|triad  (reduce: d = d (op) s in place, bf16 / int32 SUM;
+//                                                      triad: d = a (op) b, three separate streams)
+//                  nseg=16 seg_mib=64    segments per launch and their size: one (dst, src) pair each
+//                  pair=0                which buffer is a segment's src: 0 = a buffer of its own; k > 0 = the buffer of
+//                                        segment (s XOR k), both at the half segment s keeps (the partner pattern of a
+//                                        recursive-halving step; a buffer is then two segments long)
+//                  ring=0                1 = the reduce-scatter steps of a ring over nseg buffers of nseg segments each:
+//                                        launch l is step t = l mod (nseg - 1), segment s folds chunk (s - 2 - t) of
+//                                        buffer s - 1 (written by the launch before) into the same chunk of buffer s
+//                  skew=0                bytes added to the distance between consecutive buffers of the arena
+//                  u=4 block=256         128-bit accesses per lane and operand in flight, lanes per workgroup
+//                  hd=1 hs=1 st=0        cache hint of the dst load, the src load, the store: 0 plain, 1 non-temporal
+//                  pipe=0                1 = grid-stride loop that issues the next tile's loads before this tile's stores
+//                  il=0                  1 = dst and src loads interleaved per access instead of grouped per operand
+//                  wpc=0                 workgroups per CU the grid is capped at (0 = one tile per workgroup)
+//                  lds=0                 bytes of LDS a workgroup asks for (limits how many fit a CU)
+//                  xcd=0 run=128         tile numbering: 0 as dealt, 1 runs of `run` tiles per XCD, 2 a contiguous eighth
+//                  data=random|zeros     buffer contents (two bf16 per word near 1e-3 in magnitude, or all zero)
+//                  reps=10 warm=2 sets=1 timed launches, untimed ones, buffer sets rotated through by the launches
+//
+// kind=lat         one wavefront on XCD `xk` walks a chain of dependent 1 KiB loads (64 lanes x 16 bytes) over the
+//                  pieces p of a 4 GiB arena with p mod `mod` == `cls`, a piece being `gran` bytes (a power of two
+//                  >= 1024): the nanoseconds per load tell how far that class of addresses is from that XCD.
+//                  keys: xk=0 mod=8 cls=0 gran=4096 iters=2000 reps=3
+
+#include "hg_device.hpp"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace {
+
+#define CK(x)                                                                                      \
+    do {                                                                                           \
+        hipError_t e_ = (x);                                                                       \
+        if (e_ != hipSuccess) {                                                                    \
+            fprintf(stderr, "hg_probe: %s failed: %s (line %d)\n", #x, hipGetErrorString(e_), __LINE__); \
+            exit(2);                                                                               \
+        }                                                                                          \
+    } while (0)
+
+enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6 };
+
+struct ProbeTab {
+    void* dst[64];
+    const void* src[64];
+    const void* src2[64]; // triad only
+    uint32_t tiles_per_seg; // every segment has the same whole number of tiles
+    uint32_t nseg;
+    uint32_t xcd, run;
+};
+
+__device__ __forceinline__ uint32_t probe_tile(const ProbeTab& t, uint32_t b, uint32_t g)
+{
+    if (t.xcd == 1u && (g % (8u * t.run)) == 0u) {
+        const uint32_t i = b >> 3;
+        return (i / t.run) * 8u * t.run + (b & 7u) * t.run + i % t.run;
+    }
+    if (t.xcd == 2u && (g & 7u) == 0u) return (b & 7u) * (g >> 3) + (b >> 3);
+    return b;
+}
+
+template <int KIND, uint32_t U, bool HD, bool HS, bool ST, bool IL> struct Tile {
+    u32x4 a[U], b[U];
+    __device__ __forceinline__ void load(const ProbeTab& t, uint32_t tile)
+    {
+        const uint32_t s = tile / t.tiles_per_seg;
+        const uint64_t v0 = (uint64_t)(tile - s * t.tiles_per_seg) * (blockDim.x * U) + threadIdx.x;
+        const void* d = (KIND == K_TRIAD) ? t.src2[s] : t.dst[s];
+        const void* p = t.src[s];
+        if (KIND == K_WRITE) return;
+        if (IL && (KIND == K_REDUCE || KIND == K_REDUCE_I32 || KIND == K_TRIAD)) {
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) {
+                a[u] = ldv<HD>(d, v0 + u * blockDim.x);
+                b[u] = ldv<HS>(p, v0 + u * blockDim.x);
+            }
+            return;
+        }
+        if (KIND == K_REDUCE || KIND == K_REDUCE_I32 || KIND == K_TRIAD) {
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) a[u] = ldv<HD>(d, v0 + u * blockDim.x);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) b[u] = ldv<HS>(p, v0 + u * blockDim.x);
+    }
+    __device__ __forceinline__ void store(const ProbeTab& t, uint32_t tile)
+    {
+        const uint32_t s = tile / t.tiles_per_seg;
+        const uint64_t v0 = (uint64_t)(tile - s * t.tiles_per_seg) * (blockDim.x * U) + threadIdx.x;
+        void* d = t.dst[s];
+        if (KIND == K_READ) { // keeps the loads alive; never true for the data the probe writes
+            u32x4 x = b[0];
+#pragma unroll
+            for (uint32_t u = 1; u < U; ++u) x ^= b[u];
+            if ((x.x ^ x.y ^ x.z ^ x.w) == 0x9e3779b9u && x.x == 0x7f4a7c15u) stv<false>(d, v0, x);
+            return;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            u32x4 r;
+            if (KIND == K_REDUCE || KIND == K_TRIAD) r = vec_op<DT_BF16, OP_SUM>(a[u], b[u]);
+            else if (KIND == K_REDUCE_I32) r = vec_op<DT_I32, OP_SUM>(a[u], b[u]);
+            else if (KIND == K_COPY) r = b[u];
+            else { // write: words that look like the random data the other kinds move
+                const uint32_t x = ((uint32_t)(v0 + u * blockDim.x) * 2654435761u) ^ (tile * 0x85ebca6bu);
+                r = u32x4{(x & 0x807f807fu) | 0x3a003a00u, ((x >> 3) & 0x807f807fu) | 0x3a003a00u,
+                          ((x >> 5) & 0x807f807fu) | 0x3a003a00u, ((x >> 7) & 0x807f807fu) | 0x3a003a00u};
+            }
+            stv<ST>(d, v0 + u * blockDim.x, r);
+        }
+    }
+};
+
+template <int KIND, uint32_t U, bool HD, bool HS, bool ST, bool PIPE, bool IL>
+__global__ __launch_bounds__(1024) void k_probe(const ProbeTab t)
+{
+    extern __shared__ uint8_t lds_pad[]; // only its size matters: it limits the workgroups per CU
+    const uint32_t total = t.tiles_per_seg * t.nseg;
+    const uint32_t g = gridDim.x;
+    if (!PIPE) {
+        for (uint32_t i = blockIdx.x; i < total; i += g) {
+            Tile<KIND, U, HD, HS, ST, IL> x;
+            const uint32_t tile = probe_tile(t, i % g, g) + (i / g) * g;
+            if (tile >= total) continue;
+            x.load(t, tile);
+            x.store(t, tile);
+        }
+        return;
+    }
+    uint32_t i = blockIdx.x;
+    if (i >= total) return;
+    Tile<KIND, U, HD, HS, ST, IL> cur, nxt;
+    cur.load(t, i);
+    for (;;) {
+        const uint32_t n = i + g;
+        const bool more = n < total;
+        if (more) nxt.load(t, n);
+        cur.store(t, i);
+        if (!more) break;
+        cur = nxt;
+        i = n;
+    }
+}
+
+// out[0] += 1 per workgroup that found itself on XCD xk; out[1] = 100 MHz ticks the first such workgroup's chain took
+__global__ __launch_bounds__(64) void k_lat(const uint8_t* base, uint64_t first_piece, uint64_t npieces, uint32_t gran,
+                                            uint32_t mod, uint32_t cls, uint32_t xk, uint32_t iters, unsigned long long* out)
+{
+    const uint32_t xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15u; // HW_REG_XCC_ID, bits 3:0
+    if (xcc != xk) return;
+    unsigned long long mine = 0;
+    if (threadIdx.x == 0) mine = atomicAdd(out, 1ull);
+    mine = __shfl(mine, 0);
+    if (mine != 0) return;
+    const uint32_t cpp = gran >> 10; // 1 KiB chunks per piece
+    uint64_t dep = 0;
+    u32x4 x = {0u, 0u, 0u, 0u};
+    const unsigned long long t0 = wall_clock64();
+    for (uint32_t i = 0; i < iters; ++i) {
+        const uint64_t k = ((uint64_t)i * 7919u) % (npieces * cpp);
+        const uint64_t piece = (first_piece + k / cpp) * mod + cls;
+        const uint8_t* p = base + piece * gran + (k % cpp) * 1024u + threadIdx.x * 16u + dep;
+        x = __builtin_nontemporal_load((const u32x4*)p);
+        dep = (x.x == 0xdeadbeefu && x.y == 0x9e3779b9u) ? 16u : 0u; // never true for the probe's data; ties the chain
+    }
+    const unsigned long long t1 = wall_clock64();
+    if (threadIdx.x == 0) out[1] = t1 - t0;
+    if (dep) out[2] = x.z;
+}
+
+__global__ void k_fill(uint32_t* p, uint64_t nwords, uint32_t seed)
+{
+    for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < nwords; i += (uint64_t)gridDim.x * blockDim.x) {
+        uint32_t x = (uint32_t)i * 2654435761u + seed + (uint32_t)(i >> 32) * 40503u;
+        x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
+        // two bf16 values with magnitudes around 2^-10 and random signs / mantissas
+        const uint32_t lo = (x & 0x807fu) | 0x3a00u | ((x >> 20) & 0x0180u);
+        const uint32_t hi = ((x >> 16) & 0x807fu) | 0x3a00u | ((x >> 9) & 0x0180u);
+        p[i] = lo | (hi << 16);
+    }
+}
+
+struct Cfg {
+    int kind = K_REDUCE;
+    uint32_t nseg = 16, seg_mib = 64, pair = 0, u = 4, block = 256, hd = 1, hs = 1, st = 0, pipe = 0, il = 0, wpc = 0, ring = 0,
+             lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000;
+    uint64_t skew = 0;
+    bool zeros = false;
+    std::string line;
+};
+
+typedef void (*KernelFn)(const ProbeTab);
+
+template <int KIND, uint32_t U, bool HD, bool HS, bool ST> KernelFn pick3(const Cfg& c)
+{
+    if (c.pipe) return c.il ? k_probe<KIND, U, HD, HS, ST, true, true> : k_probe<KIND, U, HD, HS, ST, true, false>;
+    return c.il ? k_probe<KIND, U, HD, HS, ST, false, true> : k_probe<KIND, U, HD, HS, ST, false, false>;
+}
+template <int KIND, uint32_t U> KernelFn pick2(const Cfg& c)
+{
+    const uint32_t h = (c.hd ? 4u : 0u) | (c.hs ? 2u : 0u) | (c.st ? 1u : 0u);
+    switch (h) {
+        case 0: return pick3<KIND, U, false, false, false>(c);
+        case 1: return pick3<KIND, U, false, false, true>(c);
+        case 2: return pick3<KIND, U, false, true, false>(c);
+        case 3: return pick3<KIND, U, false, true, true>(c);
+        case 4: return pick3<KIND, U, true, false, false>(c);
+        case 5: return pick3<KIND, U, true, false, true>(c);
+        case 6: return pick3<KIND, U, true, true, false>(c);
+        default: return pick3<KIND, U, true, true, true>(c);
+    }
+}
+template <int KIND> KernelFn pick1(const Cfg& c)
+{
+    switch (c.u) {
+        case 1: return pick2<KIND, 1>(c);
+        case 2: return pick2<KIND, 2>(c);
+        case 4: return pick2<KIND, 4>(c);
+        case 8: return pick2<KIND, 8>(c);
+        default: return nullptr;
+    }
+}
+KernelFn pick(const Cfg& c)
+{
+    switch (c.kind) {
+        case K_REDUCE: return pick1<K_REDUCE>(c);
+        case K_COPY: return pick1<K_COPY>(c);
+        case K_READ: return pick1<K_READ>(c);
+        case K_WRITE: return pick1<K_WRITE>(c);
+        case K_TRIAD: return pick1<K_TRIAD>(c);
+        case K_REDUCE_I32: return pick1<K_REDUCE_I32>(c);
+        default: return nullptr;
+    }
+}
+
+bool parse(const std::string& line, Cfg& c)
+{
+    c.line = line;
+    size_t i = 0;
+    while (i < line.size()) {
+        while (i < line.size() && (line[i] == ' ' || line[i] == '\t')) ++i;
+        size_t j = i;
+        while (j < line.size() && line[j] != ' ' && line[j] != '\t') ++j;
+        if (j == i) break;
+        const std::string tok = line.substr(i, j - i);
+        i = j;
+        const size_t eq = tok.find('=');
+        if (eq == std::string::npos) return false;
+        const std::string k = tok.substr(0, eq), v = tok.substr(eq + 1);
+        const unsigned long long n = strtoull(v.c_str(), nullptr, 0);
+        if (k == "kind") {
+            if (v == "reduce") c.kind = K_REDUCE;
+            else if (v == "copy") c.kind = K_COPY;
+            else if (v == "read") c.kind = K_READ;
+            else if (v == "write") c.kind = K_WRITE;
+            else if (v == "triad") c.kind = K_TRIAD;
+            else if (v == "reduce_i32") c.kind = K_REDUCE_I32;
+            else if (v == "lat") c.kind = K_LAT;
+            else return false;
+        } else if (k == "data") {
+            if (v == "zeros") c.zeros = true;
+            else if (v == "random") c.zeros = false;
+            else return false;
+        } else if (k == "nseg") c.nseg = (uint32_t)n;
+        else if (k == "seg_mib") c.seg_mib = (uint32_t)n;
+        else if (k == "pair") c.pair = (uint32_t)n;
+        else if (k == "ring") c.ring = (uint32_t)n;
+        else if (k == "skew") c.skew = n;
+        else if (k == "u") c.u = (uint32_t)n;
+        else if (k == "block") c.block = (uint32_t)n;
+        else if (k == "hd") c.hd = (uint32_t)n;
+        else if (k == "hs") c.hs = (uint32_t)n;
+        else if (k == "st") c.st = (uint32_t)n;
+        else if (k == "pipe") c.pipe = (uint32_t)n;
+        else if (k == "il") c.il = (uint32_t)n;
+        else if (k == "wpc") c.wpc = (uint32_t)n;
+        else if (k == "lds") c.lds = (uint32_t)n;
+        else if (k == "xcd") c.xcd = (uint32_t)n;
+        else if (k == "run") c.run = (uint32_t)n;
+        else if (k == "reps") c.reps = (uint32_t)n;
+        else if (k == "warm") c.warm = (uint32_t)n;
+        else if (k == "sets") c.sets = (uint32_t)n;
+        else if (k == "xk") c.xk = (uint32_t)n;
+        else if (k == "mod") c.mod = (uint32_t)n;
+        else if (k == "cls") c.cls = (uint32_t)n;
+        else if (k == "gran") c.gran = (uint32_t)n;
+        else if (k == "iters") c.iters = (uint32_t)n;
+        else return false;
+    }
+    return true;
+}
+
+struct Arena {
+    uint8_t* base = nullptr;
+    uint64_t bytes = 0;
+    bool zeros = true, filled = false;
+};
+
+} // namespace
+
+int main(int argc, char** argv)
+{
+    FILE* in = stdin;
+    if (argc > 1 && !(in = fopen(argv[1], "r"))) {
+        fprintf(stderr, "hg_probe: cannot open %s\n", argv[1]);
+        return 2;
+    }
+    int dev = 0, cus = 0;
+    CK(hipGetDevice(&dev));
+    CK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    hipStream_t st;
+    CK(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    Arena ar;
+    char buf[1024];
+    while (fgets(buf, sizeof buf, in)) {
+        std::string line(buf);
+        while (!line.empty() && (line.back() == '\n' || line.back() == '\r')) line.pop_back();
+        if (line.empty() || line[0] == '#') continue;
+        Cfg c;
+        if (!parse(line, c)) {
+            fprintf(stderr, "hg_probe: bad configuration: %s\n", line.c_str());
+            return 2;
+        }
+        if (c.kind == K_LAT) {
+            const uint64_t arena = 4ull << 30, window = 512ull << 20;
+            if (c.gran < 1024u || (c.gran & (c.gran - 1)) || c.mod == 0 || c.cls >= c.mod || c.xk > 7 || c.iters == 0 ||
+                window / c.gran / c.mod == 0) {
+                fprintf(stderr, "hg_probe: unsupported configuration: %s\n", line.c_str());
+                return 2;
+            }
+            if (arena + 4096 > ar.bytes) {
+                if (ar.base) CK(hipFree(ar.base));
+                CK(hipMalloc((void**)&ar.base, arena + 4096));
+                ar.bytes = arena + 4096;
+                ar.filled = false;
+            }
+            if (!ar.filled) {
+                hipLaunchKernelGGL(k_fill, dim3(8192), dim3(256), 0, 0, (uint32_t*)ar.base, ar.bytes / 4, 12345u);
+                CK(hipDeviceSynchronize());
+                ar.filled = true;
+                ar.zeros = false;
+            }
+            static unsigned long long* out = nullptr;
+            static uint32_t win = 0;
+            if (!out) CK(hipMalloc((void**)&out, 64));
+            unsigned long long host[3];
+            const uint64_t per_win = window / c.gran / c.mod; // pieces of one class in a window
+            double ns_sum = 0, ns_min = 1e30;
+            unsigned long long hits = 0;
+            for (uint32_t r = 0; r < c.reps; ++r, ++win) { // every launch reads a window no recent launch has read
+                CK(hipMemsetAsync(out, 0, 64, st));
+                hipLaunchKernelGGL(k_lat, dim3(64), dim3(64), 0, st, ar.base, (uint64_t)(win % (arena / window)) * per_win, per_win,
+                                   c.gran, c.mod, c.cls, c.xk, c.iters, out);
+                CK(hipMemcpyAsync(host, out, sizeof host, hipMemcpyDeviceToHost, st));
+                CK(hipStreamSynchronize(st));
+                const double ns = (double)host[1] * 10.0 / c.iters;
+                ns_sum += ns;
+                if (ns < ns_min) ns_min = ns;
+                hits = host[0];
+            }
+            printf("{\"cfg\": \"%s\", \"workgroups_on_xcd\": %llu, \"ns_per_load\": %.1f, \"ns_per_load_min\": %.1f}\n", line.c_str(),
+                   hits, ns_sum / c.reps, ns_min);
+            fflush(stdout);
+            continue;
+        }
+        const KernelFn fn = pick(c);
+        const uint64_t seg = (uint64_t)c.seg_mib << 20;
+        const uint64_t tile_bytes = (uint64_t)c.block * c.u * 16u;
+        if (!fn || c.nseg == 0 || c.nseg > 64 || c.block == 0 || c.block > 1024 || (c.block & 63u) || seg % tile_bytes ||
+            c.sets == 0 || (c.ring && ((c.kind != K_REDUCE && c.kind != K_REDUCE_I32 && c.kind != K_COPY) || c.nseg < 3 || c.pair)) || (c.skew & 15u) || c.lds > 160u * 1024u || (c.pair && (c.nseg & (c.nseg - 1)))) {
+            fprintf(stderr, "hg_probe: unsupported configuration: %s\n", line.c_str());
+            return 2;
+        }
+        // Arena: per set, a dst buffer and a src buffer per segment (and a third for triad); with pair > 0 a buffer
+        // is two segments long and segment s folds the half it keeps of buffer (s XOR pair) into its own buffer.
+        const uint64_t buf_bytes = c.ring ? c.nseg * seg : c.pair ? 2 * seg : seg;
+        const uint32_t bufs_per_seg = (c.pair || c.ring) ? 1u : (c.kind == K_TRIAD ? 3u : (c.kind == K_READ || c.kind == K_WRITE) ? 1u : 2u);
+        const uint64_t pitch = buf_bytes + c.skew;
+        const uint64_t need = (uint64_t)(c.ring ? 1u : c.sets) * c.nseg * bufs_per_seg * pitch;
+        if (need > (64ull << 30)) {
+            fprintf(stderr, "hg_probe: configuration needs %llu bytes: %s\n", (unsigned long long)need, line.c_str());
+            return 2;
+        }
+        if (need > ar.bytes) {
+            if (ar.base) CK(hipFree(ar.base));
+            CK(hipMalloc((void**)&ar.base, need));
+            ar.bytes = need;
+            ar.filled = false;
+        }
+        if (!ar.filled || ar.zeros != c.zeros) {
+            if (c.zeros) CK(hipMemset(ar.base, 0, ar.bytes));
+            else hipLaunchKernelGGL(k_fill, dim3(8192), dim3(256), 0, 0, (uint32_t*)ar.base, ar.bytes / 4, 12345u);
+            CK(hipDeviceSynchronize());
+            ar.filled = true;
+            ar.zeros = c.zeros;
+        }
+        if (c.ring) c.sets = c.nseg - 1; // one table per step
+        std::vector<ProbeTab> tabs(c.sets);
+        for (uint32_t k = 0; k < c.sets; ++k) {
+            ProbeTab& t = tabs[k];
+            memset(&t, 0, sizeof t);
+            t.nseg = c.nseg;
+            t.tiles_per_seg = (uint32_t)(seg / tile_bytes);
+            t.xcd = c.xcd;
+            t.run = c.run ? c.run : 1u;
+            uint8_t* set0 = ar.base + (c.ring ? 0 : (uint64_t)k * c.nseg * bufs_per_seg * pitch);
+            for (uint32_t s = 0; s < c.nseg; ++s) {
+                if (c.ring) {
+                    const uint32_t chunk = (s + 2u * c.nseg - 2u - k) % c.nseg;
+                    t.dst[s] = set0 + (uint64_t)s * pitch + chunk * seg;
+                    t.src[s] = set0 + (uint64_t)((s + c.nseg - 1u) % c.nseg) * pitch + chunk * seg;
+                } else if (c.pair) { // the half a rank keeps: the first one where its `pair` bit is clear, else the second
+                    const uint64_t half = (s & c.pair) ? seg : 0;
+                    t.dst[s] = set0 + (uint64_t)s * pitch + half;
+                    t.src[s] = set0 + (uint64_t)(s ^ c.pair) * pitch + half;
+                } else {
+                    t.dst[s] = set0 + (uint64_t)(s * bufs_per_seg) * pitch;
+                    t.src[s] = (bufs_per_seg > 1) ? set0 + (uint64_t)(s * bufs_per_seg + 1) * pitch : t.dst[s];
+                    t.src2[s] = (bufs_per_seg > 2) ? set0 + (uint64_t)(s * bufs_per_seg + 2) * pitch : nullptr;
+                }
+            }
+        }
+        const uint64_t tiles = (uint64_t)tabs[0].tiles_per_seg * c.nseg;
+        uint64_t grid = tiles;
+        if (c.wpc && (uint64_t)c.wpc * cus < grid) grid = (uint64_t)c.wpc * cus;
+        if (c.pipe && !c.wpc) grid = tiles < (uint64_t)cus * 8u ? tiles : (uint64_t)cus * 8u;
+        if (c.lds) CK(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+        uint32_t launch = 0;
+        for (uint32_t i = 0; i < c.warm; ++i, ++launch)
+            hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+        CK(hipGetLastError());
+        CK(hipEventRecord(e0, st));
+        for (uint32_t i = 0; i < c.reps; ++i, ++launch)
+            hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+        CK(hipEventRecord(e1, st));
+        CK(hipStreamSynchronize(st));
+        CK(hipGetLastError());
+        float ms = 0;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        ms /= (float)c.reps;
+        const double per = (c.kind == K_REDUCE || c.kind == K_REDUCE_I32) ? 3.0 : c.kind == K_TRIAD ? 3.0 : c.kind == K_COPY ? 2.0 : 1.0;
+        const double moved = per * (double)seg * c.nseg;
+        printf("{\"cfg\": \"%s\", \"grid\": %llu, \"tile_bytes\": %llu, \"ms\": %.5f, \"moved_bytes\": %.0f, \"gbs\": %.1f, "
+               "\"frac_of_8000\": %.4f}\n",
+               line.c_str(), (unsigned long long)grid, (unsigned long long)tile_bytes, ms, moved, moved / ms / 1e6,
+               moved / ms / 1e6 / 8000.0);
+        fflush(stdout);
+    }
+    return 0;
+}
