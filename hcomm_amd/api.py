@@ -35,6 +35,7 @@ __all__ = [
     "OrderPreservedHierReduceScatterPlan", "order_preserved_hier_rs_emit", "order_preserved_hier_rs_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
+    "HcommGfxAllReduceLocalReduceNoAlloc", "NOALLOC_SCRATCH_BYTES", "NOALLOC_MAX_RANKS",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
@@ -176,6 +177,18 @@ HcommGfxDataTypeSize = _sig("HcommGfxDataTypeSize", _u32, C.c_int)
 _plan_create = _sig("HcommGfxPlanCreateEx", _i32, C.c_int, C.c_int, _u32, C.POINTER(_vp), C.POINTER(_vp),
                     C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
 _scratch_bytes = _sig("HcommGfxScratchBytes", _i32, C.c_int, _u32, _u64, C.c_int, C.POINTER(_u64))
+
+
+_noalloc = _sig("HcommGfxAllReduceLocalReduceNoAlloc", _i32, _u64, _u32, C.POINTER(_vp), C.POINTER(_vp), _u64, C.c_int,
+                C.c_int)
+NOALLOC_SCRATCH_BYTES = 64 << 20
+NOALLOC_MAX_RANKS = 8
+
+
+def HcommGfxAllReduceLocalReduceNoAlloc(thread, in_ptrs, out_ptrs, count, dtype, op):
+    """The deterministic mesh allreduce in one call, on the library's own communication buffers; returns the code."""
+    n = len(in_ptrs)
+    return _noalloc(thread, n, (_vp * n)(*in_ptrs), (_vp * n)(*out_ptrs), count, dtype, op)
 
 
 def scratch_bytes(alg, n_ranks, count, dtype):

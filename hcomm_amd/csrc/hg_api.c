@@ -136,6 +136,12 @@ static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_
     t->owns_stream = owns_stream;
     t->notify_num = notify_num;
     t->log_enabled = 1;
+    if (!recorder) {
+        /* set-up is the place to look up where the library's own array lives on this thread's GPU, so that
+         * HcommGfxAllReduceLocalReduceNoAlloc finds the address ready; a failure here only postpones the lookup */
+        void* unused = NULL;
+        (void)hg_rt_scratch(stream, &unused);
+    }
     if (notify_num) {
         t->notifies = (void**)calloc(notify_num, sizeof(void*));
         if (!t->notifies) {
@@ -264,6 +270,7 @@ static void log_launch(HgThread* t, const HgLaunch* l)
 {
     if (!t->log_enabled || t->log_n >= HG_LOG_MAX) return;
     if (t->log_n == t->log_cap) {
+        if (t->log_fixed) return;
         uint32_t cap = t->log_cap ? t->log_cap * 2 : 64;
         HcommGfxLaunchRecord* p = (HcommGfxLaunchRecord*)realloc(t->log, cap * sizeof(*p));
         if (!p) return;

@@ -302,37 +302,44 @@ uint64_t hg_split_head(const HgOp* o)
     return 0;
 }
 
-int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
+/* One operation into the open launch (closing and emitting it first when the operation cannot join it). */
+static int coalesce_op(Coalescer* c, const HgOp* o)
+{
+    if (o->bytes == 0) return HCCL_SUCCESS;                    /* count == 0: nothing to do (dispatcher.cc:719-722) */
+    if (!o->is_reduce && o->dst == o->src) return HCCL_SUCCESS; /* copy onto itself (dispatcher.cc:495-498) */
+    const uint64_t cut = hg_split_head(o);
+    if (!cut) return coalesce_one(c, o);
+    HgOp head = *o, body = *o;
+    head.bytes = cut;
+    body.dst = (char*)o->dst + head.bytes;
+    body.src = (const char*)o->src + head.bytes;
+    body.bytes = o->bytes - head.bytes;
+    const int rc = coalesce_one(c, &head);
+    return rc == HCCL_SUCCESS ? coalesce_one(c, &body) : rc;
+}
+
+int hg_coalesce_with(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx, HgLaunch* work)
 {
     Coalescer c;
-    c.l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
-    if (!c.l) return HCCL_E_MEMORY;
+    c.l = work;
     c.open = 0;
     c.bytes = 0;
     c.emit = emit;
     c.ctx = ctx;
     int rc = HCCL_SUCCESS;
-    for (uint64_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
-        const HgOp* o = &ops[i];
-        if (o->bytes == 0) continue;                   /* count == 0: nothing to do (dispatcher.cc:719-722) */
-        if (!o->is_reduce && o->dst == o->src) continue; /* copy onto itself (dispatcher.cc:495-498) */
-        const uint64_t cut = hg_split_head(o);
-        if (cut) {
-            HgOp head = *o, body = *o;
-            head.bytes = cut;
-            body.dst = (char*)o->dst + head.bytes;
-            body.src = (const char*)o->src + head.bytes;
-            body.bytes = o->bytes - head.bytes;
-            rc = coalesce_one(&c, &head);
-            if (rc == HCCL_SUCCESS) rc = coalesce_one(&c, &body);
-        } else {
-            rc = coalesce_one(&c, o);
-        }
-    }
+    for (uint64_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) rc = coalesce_op(&c, &ops[i]);
     if (c.open && rc == HCCL_SUCCESS) {
         hg_finish_seg2(c.l);
         rc = emit(c.l, ctx);
     }
-    free(c.l);
+    return rc;
+}
+
+int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx)
+{
+    HgLaunch* work = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!work) return HCCL_E_MEMORY;
+    const int rc = hg_coalesce_with(ops, n, emit, ctx, work);
+    free(work);
     return rc;
 }

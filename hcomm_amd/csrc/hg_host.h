@@ -51,6 +51,7 @@ typedef struct HgThread {
     HcommGfxLaunchRecord* log;
     uint32_t log_n, log_cap;
     int log_enabled;
+    int log_fixed; /* set while a call that must not allocate runs: the log takes what fits and drops the rest */
 } HgThread;
 
 HgThread* hg_thread_from_handle(ThreadHandle h);
@@ -59,6 +60,8 @@ HgThread* hg_thread_from_handle(ThreadHandle h);
  * kind / dtype / op share one launch.  Calls emit(launch, ctx) for each; stops at the first error. */
 typedef int (*HgEmitFn)(const HgLaunch* launch, void* ctx);
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
+/* the same with the launch under construction in storage of the caller's (no allocation) */
+int hg_coalesce_with(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx, HgLaunch* work);
 uint64_t hg_split_head(const HgOp* o); /* bytes before the 16-byte boundary both operands reach together, or 0 */
 
 /* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment

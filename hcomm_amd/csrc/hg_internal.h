@@ -107,6 +107,8 @@ int hg_rt_stream_wait_event(void* stream, void* ev);
 int hg_rt_malloc(void** p, size_t n);
 int hg_rt_free(void* p);
 int hg_rt_num_cus(void);
+/* The library's own per-GPU array of HCOMM_GFX_NOALLOC_SCRATCH_BYTES bytes: its address on the device `stream` belongs to. */
+int hg_rt_scratch(void* stream, void** ptr);
 /* Graph replay of a fixed launch list: capture between begin/end on `stream`, then launch the executable. */
 int hg_rt_stream_is_capturing(void* stream);
 int hg_rt_capture_begin(void* stream);

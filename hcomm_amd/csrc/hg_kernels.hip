@@ -212,6 +212,43 @@ int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgS
 #undef CALL
 }
 
+// ---- device memory of the library's own, for callers that cannot allocate ---------------------------------
+//
+// One array per GPU, held from the moment the code object is loaded there until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; kernels get the address that call returns, per device.
+
+} // extern "C"
+
+static __device__ __align__(256) uint8_t scratch[HCOMM_GFX_NOALLOC_SCRATCH_BYTES];
+
+#define HG_MAX_DEVICES 64
+static void* g_scratch_ptr[HG_MAX_DEVICES]; // device address of `scratch` on each GPU, once asked for
+
+extern "C" {
+
+// Address of the array's copy on the device `stream` belongs to (looked up once per device, with that device
+// current; the calling thread's current device is left as it was).
+int hg_rt_scratch(void* stream, void** ptr)
+{
+    int cur = -1;
+    hipDevice_t sd;
+    *ptr = nullptr;
+    if (hipGetDevice(&cur) != hipSuccess) return HCCL_E_RUNTIME;
+    int dev = cur;
+    if (stream && hipStreamGetDevice((hipStream_t)stream, &sd) == hipSuccess) dev = (int)sd;
+    if (dev < 0 || dev >= HG_MAX_DEVICES) return HCCL_E_RUNTIME;
+    void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        if (dev != cur && hipSetDevice(dev) != hipSuccess) return HCCL_E_RUNTIME;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (dev != cur) (void)hipSetDevice(cur);
+        if (e != hipSuccess || !p) return HCCL_E_RUNTIME;
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+    *ptr = p;
+    return HCCL_SUCCESS;
+}
+
 // ---- HIP runtime wrappers for the C host files -----------------------------------------------------------
 
 int hg_rt_device_count(void)

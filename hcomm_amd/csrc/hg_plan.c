@@ -83,19 +83,13 @@ static int op_class(const HgOp* o)
     return (o->is_reduce ? 2 : 0) + aligned;
 }
 
-static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
-                     int op)
+/* Resolve a schedule's operations into pointers: two entries per operation, because one whose operands are equally far
+ * from a 16-byte boundary is cut, as the coalescer would cut it, into the few bytes up to that boundary and an aligned
+ * rest - here, so that the grouping below sees the pieces; steps[] carries the step of every entry.  ops and steps hold
+ * 2 * n entries; *m receives how many were written. */
+static int resolve_ops(const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype, int op, HgOp* ops,
+                       uint32_t* steps, uint64_t* m_out)
 {
-    /* two entries per operation: one whose operands are equally far from a 16-byte boundary is cut, as the coalescer
-     * would cut it, into the few bytes up to that boundary and an aligned rest - here, so that the grouping below sees
-     * the pieces; steps[] carries the step of every entry */
-    HgOp* ops = (HgOp*)calloc(n ? 2 * n : 1, sizeof(HgOp));
-    uint32_t* steps = (uint32_t*)calloc(n ? 2 * n : 1, sizeof(uint32_t));
-    if (!ops || !steps) {
-        free(ops);
-        free(steps);
-        return HCCL_E_MEMORY;
-    }
     uint64_t m = 0;
     for (uint64_t i = 0; i < n; ++i) {
         const HcommGfxSchedOp* s = &list[i];
@@ -103,11 +97,8 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
         o->is_reduce = (uint8_t)s->kind;
         o->dtype = s->kind ? (uint8_t)dtype : 255;
         o->op = s->kind ? (uint8_t)op : 255;
-        if (s->dstBuf >= HCOMM_GFX_NUM_BUFS || s->srcBuf >= HCOMM_GFX_NUM_BUFS || !bufs[s->dstBuf] || !bufs[s->srcBuf]) {
-            free(ops);
-            free(steps);
+        if (s->dstBuf >= HCOMM_GFX_NUM_BUFS || s->srcBuf >= HCOMM_GFX_NUM_BUFS || !bufs[s->dstBuf] || !bufs[s->srcBuf])
             return HCCL_E_PTR;
-        }
         o->dst = (char*)bufs[s->dstBuf][s->rank] + s->dstOff;
         o->src = (const char*)bufs[s->srcBuf][s->srcRank] + s->srcOff;
         o->bytes = s->bytes;
@@ -122,36 +113,50 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
             steps[m++] = s->step;
         }
     }
-    n = m;
-    /* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the
-     * next slice), or operations on 16-byte boundaries beside others that are not (blocks of odd sizes), would
-     * change kernel with every operation: when nothing in the step can observe anything else in it, run it class by
-     * class - reduces before copies, the aligned kernels before the one for unaligned operands - each class in its original
-     * order. */
+    *m_out = m;
+    return HCCL_SUCCESS;
+}
+
+/* A step that holds both reduces and copies (the double-ring templates pair every reduce with the fetch of the next
+ * slice), or operations on 16-byte boundaries beside others that are not (blocks of odd sizes), would change kernel
+ * with every operation: when nothing in the step can observe anything else in it, run it class by class - reduces
+ * before copies, the aligned kernels before the one for unaligned operands - each class in its original order.
+ * tmp holds as many entries as the largest step that is regrouped (at most HG_REGROUP_MAX). */
+#define HG_REGROUP_MAX 4096u /* the pairwise test is quadratic: steps larger than any schedule here produces keep their order */
+static void regroup_steps(HgOp* ops, const uint32_t* steps, uint64_t n, HgOp* tmp, uint64_t tmp_cap)
+{
     for (uint64_t i = 0; i < n;) {
         uint64_t j = i;
         uint32_t seen = 0;
         while (j < n && steps[j] == steps[i]) seen |= 1u << op_class(&ops[j++]);
-        /* the pairwise test is quadratic: steps larger than any schedule here produces keep their order */
-        if ((seen & (seen - 1u)) != 0 && j - i <= 4096 && step_is_conflict_free(ops + i, j - i)) {
-            HgOp* tmp = (HgOp*)malloc((j - i) * sizeof(HgOp));
-            if (!tmp) {
-                free(ops);
-                free(steps);
-                return HCCL_E_MEMORY;
-            }
+        if ((seen & (seen - 1u)) != 0 && j - i <= HG_REGROUP_MAX && j - i <= tmp_cap && step_is_conflict_free(ops + i, j - i)) {
             uint64_t k = 0;
             for (int want = 3; want >= 0; --want)
                 for (uint64_t q = i; q < j; ++q)
                     if (op_class(&ops[q]) == want) tmp[k++] = ops[q];
             memcpy(ops + i, tmp, (j - i) * sizeof(HgOp));
-            free(tmp);
         }
         i = j;
     }
-    int rc = hg_coalesce(ops, n, plan_push, p);
+}
+
+static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
+                     int op)
+{
+    HgOp* ops = (HgOp*)calloc(n ? 2 * n : 1, sizeof(HgOp));
+    uint32_t* steps = (uint32_t*)calloc(n ? 2 * n : 1, sizeof(uint32_t));
+    const uint64_t tmp_cap = 2 * n < HG_REGROUP_MAX ? 2 * n : HG_REGROUP_MAX;
+    HgOp* tmp = (HgOp*)calloc(tmp_cap ? tmp_cap : 1, sizeof(HgOp));
+    int rc = (ops && steps && tmp) ? HCCL_SUCCESS : HCCL_E_MEMORY;
+    uint64_t m = 0;
+    if (rc == HCCL_SUCCESS) rc = resolve_ops(list, n, bufs, dtype, op, ops, steps, &m);
+    if (rc == HCCL_SUCCESS) {
+        regroup_steps(ops, steps, m, tmp, tmp_cap);
+        rc = hg_coalesce(ops, m, plan_push, p);
+    }
     free(ops);
     free(steps);
+    free(tmp);
     return rc;
 }
 
@@ -832,6 +837,67 @@ int32_t HcommGfxPlanCreateEx(
     }
     p->info.launches = p->nlaunch;
     *plan = p;
+    return HCCL_SUCCESS;
+}
+
+/* ---- the deterministic mesh allreduce for callers that cannot allocate ---------------------------------------- */
+
+#define HG_NOALLOC_MAX_RANKS HCOMM_GFX_NOALLOC_MAX_RANKS
+#define HG_NOALLOC_MAX_OPS (3u * HG_NOALLOC_MAX_RANKS * HG_NOALLOC_MAX_RANKS) /* the schedule has 3 n^2 - 2 n operations */
+
+static int emit_now(const HgLaunch* l, void* ctx) { return hg_submit((HgThread*)ctx, l); }
+
+int32_t HcommGfxAllReduceLocalReduceNoAlloc(
+    ThreadHandle thread, uint32_t nRanks, void* const* in, void* const* out, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp)
+{
+    if (!in || !out) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > HG_NOALLOC_MAX_RANKS) return HCCL_E_PARA;
+    if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
+    if (count > HG_MAX_COUNT) return HCCL_E_PARA;
+    for (uint32_t r = 0; r < nRanks; ++r) {
+        if (!in[r] || !out[r]) return HCCL_E_PTR;
+        if ((((uintptr_t)in[r]) | ((uintptr_t)out[r])) & 127u) return HCCL_E_PARA;
+    }
+    HgThread* t = hg_thread_from_handle(thread);
+    if (!t) return HCCL_E_PTR;
+    /* every rank's communication buffer is a slice of the library's own array on the thread's GPU */
+    uint64_t per_rank = hg_scratch_bytes(HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, nRanks, count, (int)dataType);
+    per_rank = (per_rank + 255u) & ~(uint64_t)255u;
+    if (per_rank > HCOMM_GFX_NOALLOC_SCRATCH_BYTES / nRanks) return HCCL_E_PARA; /* larger than the array: see the header */
+    void* base = NULL;
+    if (t->recorder) {
+        base = (void*)((uintptr_t)1 << 40); /* launches are only logged: any aligned address stands for the array */
+    } else {
+        const int rc = hg_rt_scratch(t->stream, &base);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    void* scratch[HG_NOALLOC_MAX_RANKS];
+    for (uint32_t r = 0; r < nRanks; ++r) scratch[r] = (char*)base + (uint64_t)r * per_rank;
+    HcommGfxSchedOp sched[HG_NOALLOC_MAX_OPS];
+    HgOpList ol;
+    memset(&ol, 0, sizeof(ol));
+    ol.ops = sched;
+    ol.cap = HG_NOALLOC_MAX_OPS;
+    ol.fixed = 1;
+    int rc = hg_schedule_into(&ol, HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, nRanks, count, count, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    /* the plan's own lowering on storage of this call: resolve, regroup the steps that mix kernels, then through the
+     * coalescer, which merges what the ranks do in a step into one launch and submits each launch as soon as the
+     * next operation cannot join it */
+    void* const* bufs[HCOMM_GFX_NUM_BUFS] = {in, out, scratch, NULL, NULL};
+    HgOp ops[2 * HG_NOALLOC_MAX_OPS], tmp[2 * HG_NOALLOC_MAX_OPS];
+    uint32_t steps[2 * HG_NOALLOC_MAX_OPS];
+    uint64_t m = 0;
+    rc = resolve_ops(sched, ol.n, bufs, (int)dataType, (int)reduceOp, ops, steps, &m);
+    if (rc != HCCL_SUCCESS) return rc;
+    regroup_steps(ops, steps, m, tmp, 2 * HG_NOALLOC_MAX_OPS);
+    HgLaunch work;
+    const int log_fixed = t->log_fixed;
+    if (!t->recorder) t->log_fixed = 1; /* the launch log grows by reallocation */
+    rc = hg_coalesce_with(ops, m, emit_now, t, &work);
+    t->log_fixed = log_fixed;
+    if (rc != HCCL_SUCCESS) return rc;
     return HCCL_SUCCESS;
 }
 

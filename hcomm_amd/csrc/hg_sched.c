@@ -36,7 +36,7 @@ int32_t HcommGfxCalcSlices(uint64_t count, uint32_t unitSize, uint32_t n, HcommG
 
 void hg_oplist_free(HgOpList* l)
 {
-    free(l->ops);
+    if (!l->fixed) free(l->ops);
     memset(l, 0, sizeof(*l));
 }
 
@@ -46,6 +46,7 @@ static int push(HgOpList* l, uint32_t step, uint32_t kind, uint32_t rank, uint32
     if (step + 1 > l->steps) l->steps = step + 1;
     if (bytes == 0) return HCCL_SUCCESS; /* zero-size slices produce no work (dispatcher.cc:495-498, 719-722) */
     if (l->n == l->cap) {
+        if (l->fixed) return HCCL_E_INTERNAL;
         uint64_t cap = l->cap ? l->cap * 2 : 256;
         HcommGfxSchedOp* p = (HcommGfxSchedOp*)realloc(l->ops, cap * sizeof(*p));
         if (!p) return HCCL_E_MEMORY;
@@ -674,6 +675,11 @@ static int sched_allreduce_nhr_oneshot(HgOpList* l, uint32_t n, uint64_t count, 
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
 {
     memset(l, 0, sizeof(*l));
+    return hg_schedule_into(l, alg, n, count, stride, dtype);
+}
+
+int hg_schedule_into(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype)
+{
     if (n == 0 || n > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
     if (stride == 0) stride = count;
     if (stride < count || stride > HG_MAX_COUNT) return HCCL_E_PARA;

@@ -10,11 +10,14 @@ typedef struct {
     HcommGfxSchedOp* ops;
     uint64_t n, cap;
     uint32_t steps;
+    int fixed; /* ops is storage of the caller's holding cap entries: never grown, never freed */
 } HgOpList;
 
 /* Fill `l` with the op list of `alg`; the caller releases it with hg_oplist_free. */
 /* stride: elements between consecutive ranks' slices in the input of the scatter algorithms (0 = count). */
 int hg_schedule(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype);
+/* The same into a list the caller has set up (empty, or fixed storage: HCCL_E_INTERNAL when it does not fit). */
+int hg_schedule_into(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t stride, int dtype);
 /* The op-base loop around alg: chunks of at most hg_opbase_max_count elements, each copied from the user input
  * into the CCL input buffer, run through the template, and copied from the CCL output to the user output. */
 int hg_schedule_opbase(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);

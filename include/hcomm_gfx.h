@@ -496,6 +496,27 @@ int32_t HcommGfxScratchBytes(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t co
                              uint64_t* bytes);
 
 /*
+ * The deterministic mesh allreduce (HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, step-wise) submitted to `thread` in one call
+ * that allocates nothing, neither on the device nor on the host.  No counterpart in the reference: it is for callers
+ * that cannot allocate - code under HIP graph capture, serving loops, harnesses that forbid hipMalloc - and so cannot
+ * supply the communication buffers HcommGfxPlanCreateEx asks for.  The ranks' communication buffers are slices of one
+ * array of HCOMM_GFX_NOALLOC_SCRATCH_BYTES bytes that the library keeps on every GPU it is loaded on, from load until
+ * the process ends.  in, out, count, dataType, reduceOp as for HcommGfxPlanCreate; out[r] receives the same bits as
+ * the plan's, and in[r] is only read.
+ *   nRanks      at most HCOMM_GFX_NOALLOC_MAX_RANKS and a rank count the algorithm takes
+ *   size limit  nRanks x (HcommGfxScratchBytes(...) rounded up to 256) must fit the array, else HCCL_E_PARA and nothing
+ *               is launched: 8 ranks -> 8 MiB of communication buffer per rank, i.e. just under 8 MiB per rank buffer
+ * Every call on a GPU uses that GPU's one array: calls that may overlap in time on one GPU (two threads' streams with
+ * no order between them) race on it; calls on one thread's stream are ordered by the stream.  The array keeps the
+ * last call's contents; the schedule writes every byte of it that it later reads, so nothing needs clearing.
+ */
+#define HCOMM_GFX_NOALLOC_SCRATCH_BYTES (64u << 20)
+#define HCOMM_GFX_NOALLOC_MAX_RANKS 8u
+int32_t HcommGfxAllReduceLocalReduceNoAlloc(
+    ThreadHandle thread, uint32_t nRanks, void* const* in, void* const* out, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp);
+
+/*
  * Enqueue every launch of the plan on the thread, in order.  May be called any number of times, from one host
  * thread at a time.  With HCOMM_GFX_GRAPH=1 in the environment a plan of two or more launches is replayed as a
  * HIP graph captured at its first run on the thread's stream (off by default: it measured slower than

@@ -8,6 +8,7 @@ int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, i
 int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, uint32_t l) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)l; return 4; }
 int hg_launch_fold(void* s, int d, int o, int a, const HgFoldTable* t, uint64_t b, uint32_t l) { (void)s; (void)d; (void)o; (void)a; (void)t; (void)b; (void)l; return 4; }
 int hg_rt_device_count(void) { return 0; }
+int hg_rt_scratch(void* s, void** p) { (void)s; *p = NULL; return 4; }
 int hg_rt_stream_create(void** s) { *s = NULL; return 4; }
 int hg_rt_stream_destroy(void* s) { (void)s; return 0; }
 int hg_rt_stream_sync(void* s) { (void)s; return 0; }

@@ -563,3 +563,55 @@ def test_thread_alloc_without_gpu_is_unavailable():
     assert code == R.E_UNAVAIL                                      # fails loudly, no CPU fallback
     code, _ = h.HcommThreadAllocWithStream(0, 0)
     assert code == R.E_UNAVAIL
+
+
+# ---- the entry point for callers that cannot allocate ----------------------------------------------------------
+
+def _launch_tuples(records):
+    return [(r.kind, r.dtype, r.op, r.nseg, r.bytes, r.blocks) for r in records]
+
+
+@pytest.mark.parametrize("n,count,dt", [(8, 1048576 + 37, DT.BFP16), (4, 500001, DT.FP32), (2, 3, DT.FP16), (1, 77, DT.INT8)])
+def test_no_alloc_allreduce_submits_the_plans_launches(rec, n, count, dt):
+    """HcommGfxAllReduceLocalReduceNoAlloc submits exactly the launches of the step-wise plan that is given
+    communication buffers (same kinds, segments, bytes and grids), in the same order."""
+    ins = [0x1000000 * (r + 1) for r in range(n)]
+    outs = [(1 << 36) + 0x1000000 * (r + 1) for r in range(n)]
+    sb = h.scratch_bytes(h.Alg.ALLREDUCE_LOCAL_REDUCE, n, count, dt)
+    scr = [(1 << 38) + ((sb + 255) // 256 * 256) * r for r in range(n)] if sb else None
+    plan = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, ins, outs, count, dt, OP.SUM, 0, scr)
+    want = _launch_tuples(plan.launches())
+    plan.destroy()
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommGfxAllReduceLocalReduceNoAlloc(rec, ins, outs, count, dt, OP.SUM) == R.SUCCESS
+    assert _launch_tuples(h.launch_log(rec)) == want
+
+
+def test_no_alloc_allreduce_checks(rec):
+    f = h.HcommGfxAllReduceLocalReduceNoAlloc
+    ins = [0x1000000 * (r + 1) for r in range(16)]
+    outs = [(1 << 36) + 0x1000000 * (r + 1) for r in range(16)]
+    assert f(rec, ins[:8], outs[:8], 1 << 20, DT.BFP16, OP.SUM) == R.SUCCESS
+    assert f(0, ins[:8], outs[:8], 16, DT.BFP16, OP.SUM) == R.E_PTR                       # no thread
+    assert f(rec, ins[:3] + [None], outs[:4], 16, DT.BFP16, OP.SUM) == R.E_PTR              # a rank without a buffer
+    assert f(rec, ins[:3] + [ins[3] + 64], outs[:4], 16, DT.BFP16, OP.SUM) == R.E_PARA      # not on 128 bytes
+    assert f(rec, ins[:16], outs[:16], 16, DT.BFP16, OP.SUM) == R.E_PARA                    # more ranks than it takes
+    assert f(rec, ins[:8], outs[:8], 16, DT.BFP16, OP.PROD) == R.E_PARA                     # bf16 has no PROD
+    assert f(rec, ins[:8], outs[:8], 16, DT.INT64, OP.SUM) == R.E_PARA
+    # the communication buffers of 8 ranks must fit the library's array: 8 MiB each
+    per_rank = h.NOALLOC_SCRATCH_BYTES // 8
+    fits = per_rank // 2 - 8 * 16384  # bf16 elements; slots are rounded up to 16 KiB
+    assert h.scratch_bytes(h.Alg.ALLREDUCE_LOCAL_REDUCE, 8, fits, DT.BFP16) <= per_rank
+    assert f(rec, ins[:8], outs[:8], fits, DT.BFP16, OP.SUM) == R.SUCCESS
+    h.HcommGfxLaunchLogClear(rec)
+    assert f(rec, ins[:8], outs[:8], per_rank // 2 + 1, DT.BFP16, OP.SUM) == R.E_PARA
+    assert h.launch_log(rec) == []                                                          # refused before any launch
+    # the rank counts the algorithm itself refuses stay refused
+    code3 = f(rec, ins[:3], outs[:3], 100, DT.BFP16, OP.SUM)
+    try:
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.STEPWISE, ins[:3], outs[:3], 100, DT.BFP16, OP.SUM, 0,
+               [(1 << 38) + 0x100000 * r for r in range(3)]).destroy()
+        plan_code = R.SUCCESS
+    except h.HcommError as e:
+        plan_code = e.code
+    assert code3 == plan_code
