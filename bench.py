@@ -27,23 +27,21 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
-# dispatch; FETCH_SIZE scaled by 2.0, the factor that makes k_copy's known 128 MiB read come out right;
-# WRITE_SIZE by 1.0).  Summaries: profiles/k_reduce2_bf16_ring_ar_n8_128MiB.md,
-# profiles/k_fold_chain_bf16_ring_ar_n8_128MiB.md, profiles/k_fold_tree_int32_rhd_ar_n16_128MiB.md,
-# profiles/k_reduce2_bf16_nhr_ar_n8_128MiB.md.
-MEASURED_TRAFFIC = {
-    ("ring_ar_bf16_n8_128MiB", "stepwise"): (131115.7 * 2.0 + 131072.0) * 1024,
-    ("ring_ar_bf16_n8_128MiB", "fused"): (524348.6 * 2.0 + 1966281.4) * 1024,
-    # averages over the launches of the dominant kernel in one collective (they differ in size per step)
-    ("rhd_ar_int32_n16_128MiB_sum", "stepwise"): (491541.9 * 2.0 + 491520.2) * 1024,
-    ("rhd_ar_int32_n16_128MiB_sum", "fused"): (1048645.9 * 2.0 + 3145988.9) * 1024,
-    ("nhr_ar_bf16_n8_128MiB", "stepwise"): (305877.2 * 2.0 + 305834.7) * 1024,
-    ("nhr_ar_bf16_n8_128MiB", "fused"): (524407.5 * 2.0 + 1574742.8) * 1024,
-    # the two plant launches (512 MiB written each) are the dominant kernel's first run of launches
-    ("order_preserved_ar_bf16_n8_128MiB", "stepwise"): (262171.25 * 2.0 + 524392.0) * 1024,
-    ("order_preserved_ar_bf16_n8_128MiB", "fused"): (524395.6 * 2.0 + 1049394.3) * 1024,
-}
+
+
+def measured_traffic(workload, lowering):
+    """L2 <-> fabric bytes per launch of the dominant kernel, from profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE
+    and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain copy of known size.
+    Written by `python -m hcomm_amd.profiling traffic ...` from the counter CSVs; None for what was not profiled."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            e = json.load(f)["entries"].get("%s|%s" % (workload, lowering))
+    except (OSError, ValueError, KeyError):
+        return None
+    if not e:
+        return None
+    return (e["fetch_kib"] * e["fetch_scale"] + e["write_kib"] * e["write_scale"]) * 1024
+
 
 # name: (algorithm, ranks, elements per rank, dtype, op, data distribution)
 WORKLOADS = {
@@ -55,6 +53,7 @@ WORKLOADS = {
     "ring_rs_fp32_prod_n7_100M": ("ring_rs_stage", 7, 100000003, "fp32", "prod", "uniform[0.99,1.01]"),
     "ring_rs_int8_sum_n7_100M": ("ring_rs_stage", 7, 100000003, "int8", "sum", "ints[-8,8]"),
     "mesh_oneshot_fp16_n8_4MiB": ("mesh_oneshot", 8, 2097152, "fp16", "sum", "uniform[-1,1)"),
+    "mesh_oneshot_fp16_n8_4KiB": ("mesh_oneshot", 8, 2048, "fp16", "sum", "uniform[-1,1)"),
     "local_reduce_ar_bf16_n8_128MiB": ("local_reduce", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "chunk_mesh_ar_bf16_n8_128MiB": ("chunk_mesh", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "nhr_ar_bf16_n8_128MiB": ("nhr", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -121,6 +120,11 @@ def make_inputs(torch, dev, n, count, dtname, seed=1234):
     return out
 
 
+# what the default run appends to its line, beside the headline: (workload, steps) of the other BASELINE configs
+CONFIG_LINE = [("ring_ar_fp32_n8_4MiB", 20), ("rhd_ar_int32_n16_128MiB_sum", 10), ("mesh_oneshot_fp16_n8_4KiB", 50),
+               ("mesh_oneshot_fp16_n8_4MiB", 20), ("ring_rs_fp32_prod_n7_100M", 10), ("ring_rs_int8_sum_n7_100M", 10)]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -130,12 +134,13 @@ def main():
     ap.add_argument("--workload", default="ring_ar_bf16_n8_128MiB", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0 = min(16, cores))")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload only: leave out the other configurations and the no-reuse leg")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the N ranks are simulated as HBM buffers on it); "
                  "--gpus %d is not supported" % args.gpus)
 
-    import numpy as np
     import torch
     import hcomm_amd as h
 
@@ -143,6 +148,36 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream(device=dev)  # default priority
+    code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 0)
+    h.check(code, "HcommThreadAllocWithStream")
+    with torch.cuda.stream(stream):  # torch's own work (restoring inputs) is ordered with the library's launches
+        out = run_workload(args, torch, h, dev, stream, thread)
+        if args.workload == "ring_ar_bf16_n8_128MiB" and not args.no_configs:
+            out["roofline"]["no_reuse"] = no_reuse_leg(torch, h, dev, stream, thread, max(args.steps, 20))
+            rows = []
+            for name, steps in CONFIG_LINE:
+                mesh = name.startswith("mesh_oneshot")  # the one-shot's point is its single fused launch: both
+                sub = argparse.Namespace(workload=name, steps=steps, warmup=2, lowering="both" if mesh else "stepwise",
+                                         no_cpu=args.no_cpu, cpu_threads=args.cpu_threads, cpu_seconds=1.0)
+                r = run_workload(sub, torch, h, dev, stream, thread)
+                row = {"workload": name, "ms_per_step": r["ms_per_step"], "gbs": r["value"],
+                       "frac": round(r["value"] / HBM_PEAK_GBS, 4), "launches": r["launches"],
+                       "kernel": r["roofline"]["kernel"], "kernel_ms": r["roofline"]["kernel_ms"],
+                       "kernel_frac": r["roofline"]["frac"], "steps": steps,
+                       "verified": r["verified_bit_exact_vs_oracle"]}
+                if mesh and r.get("fused"):
+                    row["fused_ms_per_step"] = r["fused"]["ms_per_step"]
+                    row["fused_moved_gbs"] = round(r["fused"]["moved_bytes"] / (r["fused"]["ms_per_step"] * 1e-3) / 1e9, 1)
+                rows.append(row)
+            out["configs"] = rows
+    h.HcommThreadFreeWithStream([thread])
+    print(json.dumps(out))
+
+
+def run_workload(args, torch, h, dev, stream, thread):
+    """One workload: timing of every lowering it has, CPU baseline and verification; returns the result line."""
+    import numpy as np
     alg_name, n, count, dtname, opname, dist = WORKLOADS[args.workload]
     DT = {"bf16": h.HcommDataType.BFP16, "fp32": h.HcommDataType.FP32, "fp16": h.HcommDataType.FP16,
           "int32": h.HcommDataType.INT32, "int8": h.HcommDataType.INT8}
@@ -177,15 +212,8 @@ def main():
     unit = h.DTYPE_SIZE[dt]
     in_place = alg_name == "ring_rs_stage" and not hier
 
-    stream = torch.cuda.Stream(device=dev)  # default priority
-    code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 0)
-    h.check(code, "HcommThreadAllocWithStream")
-
     if count is None:
-        out = mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit)
-        h.HcommThreadFreeWithStream([thread])
-        print(json.dumps(out))
-        return
+        return mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit)
 
     nbytes = count * unit
     in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs", "order_preserved_small")
@@ -195,11 +223,12 @@ def main():
     d_out = None if in_place else [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(n)]
 
     def restore():
+        """Inputs as generated, outputs zero; queued on the stream the library launches on (no host wait)."""
         for r in range(n):
             d_in[r].copy_(pristine[r])
-            if d_out is not None:
+        if d_out is not None:
+            for r in range(n):
                 d_out[r].zero_()
-        torch.cuda.synchronize()
 
     in_ptrs = [t.data_ptr() for t in d_in]
     out_ptrs = None if in_place else [t.data_ptr() for t in d_out]
@@ -264,21 +293,34 @@ def main():
                 continue
             raise
         launches = plan.launches()
-        restore()
         for _ in range(args.warmup):
+            restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
         stream.synchronize()
+        # EXACTLY args.steps steps, every one of them on the inputs as generated: the inputs are restored before
+        # each step (outside the timed events), and a step is timed by a pair of HIP events on the launch stream
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in ev:
+            restore()
+            a.record(stream)
+            h.check(plan.run(thread), "HcommGfxPlanRun")
+            b.record(stream)
+        stream.synchronize()
         torch.cuda.synchronize()
+        per_step = sorted(a.elapsed_time(b) for a, b in ev)
+        ms_step = sum(per_step) / args.steps
+        # for comparison: the same number of steps queued back to back with no restore in between, timed by the
+        # host clock (from the second step on they run on what the step before left in the buffers)
+        restore()
+        stream.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             h.check(plan.run(thread), "HcommGfxPlanRun")
         stream.synchronize()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        ms_step = wall * 1e3 / args.steps
+        ms_back_to_back = (time.perf_counter() - t0) * 1e3 / args.steps
 
         # dominant kernel = the kind with the most bytes; its first contiguous run of launches is timed as a
-        # group with HIP events recorded on the stream the kernels run on
+        # group with HIP events recorded on the stream the kernels run on, again on restored inputs
         # (the kernel for unaligned operands comes as a copy and as a reduce: op 255 marks the copies)
         kkey = lambda r: (r.kind, r.op == 255)
         by_kind = {}
@@ -292,6 +334,7 @@ def main():
             cnt += 1
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
         for a, b in ev:
+            restore()
             if first:
                 h.check(plan.run_range(thread, 0, first), "run_range")
             a.record(stream)
@@ -313,6 +356,9 @@ def main():
             dom_moved = plan.info.movedBytes // cnt
         results[name] = {
             "ms_per_step": ms_step,
+            "ms_per_step_min": per_step[0],
+            "ms_per_step_median": per_step[len(per_step) // 2],
+            "ms_per_step_back_to_back": ms_back_to_back,
             "gbs": plan.info.algorithmicBytes / (ms_step * 1e-3) / 1e9,
             "launches": plan.info.launches,
             "algorithmic_bytes": plan.info.algorithmicBytes,
@@ -408,7 +454,8 @@ def main():
                 oracle.run(oalg, ins, outs, count, odt, oop, scratch=host_scr)
 
         passes, cpu_s = 0, 0.0
-        while passes < 1 or (cpu_s < 8.0 and passes < 64):
+        cpu_budget = getattr(args, "cpu_seconds", 8.0)
+        while passes < 1 or (cpu_s < cpu_budget and passes < 64):
             work_in = [x.copy() for x in host_in]  # every pass starts from the pristine inputs (copy not timed)
             t0 = time.perf_counter()
             cpu_run(work_in, host_out)
@@ -416,13 +463,15 @@ def main():
             passes += 1
         host_in = work_in
         # the same schedule on ONE thread (the scalar loop shape of the reference's CPU witnesses), one pass
-        oracle.lib().orc_set_threads(1)
-        one_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
-        one_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
-        t0 = time.perf_counter()
-        cpu_run(one_in, one_out)
-        one_s = time.perf_counter() - t0
-        del one_in, one_out
+        one_s = None
+        if cpu_budget >= 8.0:
+            oracle.lib().orc_set_threads(1)
+            one_in = [p.cpu().numpy().view(npdt).copy() for p in pristine]
+            one_out = [np.zeros(count if not in_place else 1, npdt) for _ in range(n)]
+            t0 = time.perf_counter()
+            cpu_run(one_in, one_out)
+            one_s = time.perf_counter() - t0
+            del one_in, one_out
         model = "unknown"
         try:
             with open("/proc/cpuinfo") as f:
@@ -432,13 +481,13 @@ def main():
         cpu = {"value": round(alg_bytes * passes / cpu_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": "the full workload, %d passes, %.2f s of CPU work in total; OpenMP static over elements"
                          % (passes, cpu_s),
-               "single_thread_value": round(alg_bytes / one_s / 1e9, 2), "cpu_model": model,
+               "single_thread_value": round(alg_bytes / one_s / 1e9, 2) if one_s else None, "cpu_model": model,
                "host_cores": os.cpu_count()}
         # the reference's own CPU reduce loop (VirtualRunTime::MemReduceSum, test/hccl_vm/src/plugin/runner/
         # runner_utils/hccl_task_reduce_process.cc:57-84, compiled from where it lies into oracle/_ref) on one
         # thread, for the element types it has (no bf16 there): dst = dst + src over a bounded sample, 3 bytes
         # of traffic per byte of dst
-        if oracle.have_ref():
+        if oracle.have_ref() and cpu_budget >= 8.0:
             R = oracle.ref()
             rng = np.random.default_rng(7)
             witness = {}
@@ -470,6 +519,7 @@ def main():
             restore()
             h.check(plan.run(thread), "HcommGfxPlanRun")
             stream.synchronize()
+            torch.cuda.synchronize()
             for r in range(n):
                 if name == "fused_keep_inputs":  # the inputs as they were, not as the replay leaves them
                     ok = bool(torch.equal(d_in[r], pristine[r]))
@@ -483,7 +533,6 @@ def main():
                 verified = verified and bool(ok)
             plan.destroy()
 
-    h.HcommThreadFreeWithStream([thread])
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
         metric = "HBM GB/s (%% of peak) for simulated %d-rank %s %s %s" % (n, dtname, ("order-preserving two-level " if (ophier or ophrs) else "double-ring " if dbring else "mesh three-step " if mesh0 else "three-step " if hier else "") + ("reduce-scatter" if ophrs else "allreduce" if ophier else alg_name), opname)
@@ -496,6 +545,13 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(res["ms_per_step"], 5),
+        "ms_per_step_min": round(res["ms_per_step_min"], 5),
+        "ms_per_step_median": round(res["ms_per_step_median"], 5),
+        "ms_per_step_back_to_back": round(res["ms_per_step_back_to_back"], 5),
+        "timing": "every step runs on the inputs as generated (restored before it, outside the timed region) and is "
+                  "timed by a pair of HIP events on the launch stream; ms_per_step is the mean over the steps; "
+                  "ms_per_step_back_to_back is the host clock over the same number of steps queued without restores",
+        "launches": res["launches"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -516,7 +572,10 @@ def main():
                    **({"ccl_buffer_bytes": ccl_bytes} if (dbring or plant or hier_rs or ophier or ophrs) else {})},
         "roofline": {"bound": "hbm", "achieved": round(res["kernel_gbs"], 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(res["kernel_gbs"] / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.workload, best)),
+                     "traffic": measured_traffic(args.workload, best),
+                     "traffic_is": "L2 <-> fabric bytes (FETCH_SIZE / WRITE_SIZE count below the L2): equal to the "
+                                   "algorithmic bytes means no re-reads and no write amplification; how many of them "
+                                   "the memory-side cache served instead of HBM these counters cannot tell",
                      "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
                      "algorithmic_bytes_per_launch": res["kernel_alg_bytes"]},
         "cpu_baseline": cpu,
@@ -527,7 +586,54 @@ def main():
                                for kk, vv in results["fused_keep_inputs"].items()}
                               if "fused_keep_inputs" in results else None),
     }
-    print(json.dumps(out))
+    return out
+
+
+def no_reuse_leg(torch, h, dev, stream, thread, reps):
+    """The two-input reduce on operands that nothing touched recently, through the reference's own primitive API:
+    one batch of HcommLocalReduceOnThread calls = one k_reduce2<bf16,SUM> launch, rotated over buffer sets so that a
+    launch finds nothing of its operands in the 256 MB memory-side cache.
+      ring_step_shape   8 segments of 16 MiB (the headline's launch: 128 MiB written, the variant whose output
+                        the next launch is to find in that cache), 12 sets of 256 MiB -> 3 GiB between two uses
+      streaming_shape   16 segments of 64 MiB (1 GiB written: the variant with non-temporal accesses; the first
+                        halving step of the 16-rank recursive-halving allreduce), 3 sets of 2 GiB"""
+    out = {}
+    for key, nseg, seg_bytes, sets in (("ring_step_shape", 8, 16 << 20, 12), ("streaming_shape", 16, 64 << 20, 3)):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(4321)
+        elems = seg_bytes // 2
+        bufs = []
+        for _ in range(sets):
+            pairs = []
+            for _ in range(nseg):
+                d = (torch.randn(elems, generator=gen, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+                p = (torch.randn(elems, generator=gen, device=dev, dtype=torch.float32) * 1e-3).to(torch.bfloat16)
+                pairs.append((d, p))
+            bufs.append(pairs)
+
+        def launch(k):
+            h.check(h.HcommBatchModeStart(b"no_reuse"), "HcommBatchModeStart")
+            for d, p in bufs[k % sets]:
+                h.check(h.HcommLocalReduceOnThread(thread, d.data_ptr(), p.data_ptr(), elems, h.HcommDataType.BFP16,
+                                                   h.HcommReduceOp.SUM), "HcommLocalReduceOnThread")
+            h.check(h.HcommBatchModeEnd(b"no_reuse"), "HcommBatchModeEnd")
+
+        for k in range(sets):
+            launch(k)
+        stream.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for k, (a, b) in enumerate(ev):
+            a.record(stream)
+            launch(k)
+            b.record(stream)
+        stream.synchronize()
+        ms = sum(a.elapsed_time(b) for a, b in ev) / reps
+        alg = 3 * nseg * seg_bytes
+        out[key] = {"kernel": "k_reduce2<bf16,SUM>", "segments": nseg, "segment_bytes": seg_bytes, "buffer_sets": sets,
+                    "kernel_ms": round(ms, 5), "algorithmic_bytes_per_launch": alg,
+                    "achieved": round(alg / (ms * 1e-3) / 1e9, 2), "frac": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        del bufs
+    return out
 
 
 def mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit):
@@ -536,6 +642,27 @@ def mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit):
     (N launches) is listed beside it."""
     points = []
     reps = max(args.steps, 100)
+    # the floor: what one launch of this library costs in this harness when it moves next to nothing (a 16-byte copy
+    # through HcommLocalCopyOnThread, one workgroup), timed the same two ways as the collectives below
+    tiny = torch.zeros(64, dtype=torch.uint8, device=dev)
+    for _ in range(10):
+        h.HcommLocalCopyOnThread(thread, tiny.data_ptr() + 32, tiny.data_ptr(), 16)
+    stream.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record(stream)
+        h.HcommLocalCopyOnThread(thread, tiny.data_ptr() + 32, tiny.data_ptr(), 16)
+        b.record(stream)
+    stream.synchronize()
+    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in ev)
+    floor_single = round(ts[len(ts) // 2], 2)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record(stream)
+    for _ in range(reps):
+        h.HcommLocalCopyOnThread(thread, tiny.data_ptr() + 32, tiny.data_ptr(), 16)
+    b.record(stream)
+    stream.synchronize()
+    floor_pipelined = round(a.elapsed_time(b) * 1e3 / reps, 2)
     for m in [1 << s for s in range(12, 23)]:
         count = m // unit
         ins = make_inputs(torch, dev, n, count, "fp16")
@@ -574,6 +701,8 @@ def mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit):
             "ms_per_step": top["fused_pipelined_us"] / 1e3, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
             "config": {"workload": args.workload, "ranks": n, "algorithmic_bytes": "N(N+1)M = 72 M"},
+            "launch_floor_us": {"single": floor_single, "pipelined": floor_pipelined,
+                                "what": "a 16-byte HcommLocalCopyOnThread (one workgroup) in the same harness"},
             "sweep": points}
 
 
