@@ -224,6 +224,13 @@ HcommResult HcommThreadFree(const ThreadHandle* threads, uint32_t threadNum)
             ret = HCCL_E_NOT_FOUND;
             continue;
         }
+        /* operations recorded on it by a batch of another host thread are still to be submitted by that thread's
+         * HcommBatchModeEnd: the thread stays until then */
+        const void* owner = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
+        if (owner && owner != (const void*)&g_ctx) {
+            ret = HCCL_E_UNAVAIL;
+            continue;
+        }
         thread_delete(t);
     }
     return ret;
@@ -336,6 +343,8 @@ static int emit_to_thread(const HgLaunch* l, void* ctx) { return hg_submit((HgTh
 static int record_or_run(HgThread* t, const HgOp* o)
 {
     if (!g_ctx.batching) return hg_coalesce(o, 1, emit_to_thread, t);
+    const void* held = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
+    if (held && held != (const void*)&g_ctx) return HCCL_E_UNAVAIL; /* in another host thread's batch */
     if (t->pending_n == t->pending_cap) {
         uint32_t cap = t->pending_cap ? t->pending_cap * 2 : 64;
         HgOp* p = (HgOp*)realloc(t->pending, cap * sizeof(*p));
@@ -343,13 +352,16 @@ static int record_or_run(HgThread* t, const HgOp* o)
         t->pending = p;
         t->pending_cap = cap;
     }
-    t->pending[t->pending_n++] = *o;
-    uint32_t i = 0;
-    while (i < g_ctx.ntouched && g_ctx.touched[i] != t) ++i;
-    if (i == g_ctx.ntouched) {
+    /* the thread joins this host thread's batch before anything is queued on it, so that a refusal leaves nothing
+     * behind for a later, unrelated batch */
+    const void* owner = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
+    if (owner && owner != (const void*)&g_ctx) return HCCL_E_UNAVAIL; /* in another host thread's batch */
+    if (!owner) {
         if (g_ctx.ntouched == HG_TOUCHED_MAX) return HCCL_E_UNAVAIL;
         g_ctx.touched[g_ctx.ntouched++] = t;
+        __atomic_store_n(&t->batch_owner, (const void*)&g_ctx, __ATOMIC_RELEASE);
     }
+    t->pending[t->pending_n++] = *o;
     return HCCL_SUCCESS;
 }
 
@@ -520,6 +532,7 @@ int32_t HcommBatchModeEnd(const char* batchTag)
         if (!t) continue; /* freed inside the batch */
         if (ret == HCCL_SUCCESS) ret = hg_coalesce(t->pending, t->pending_n, emit_to_thread, t);
         t->pending_n = 0;
+        __atomic_store_n(&t->batch_owner, NULL, __ATOMIC_RELEASE);
     }
     g_ctx.ntouched = 0;
     return ret;

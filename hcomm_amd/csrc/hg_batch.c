@@ -55,8 +55,8 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
  */
 enum {
     TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE,
-    TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_FOLD,
-    TUNE_N
+    TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_CHAIN, TUNE_RUN_CHAIN, TUNE_LDS_TREE,
+    TUNE_RUN_TREE, TUNE_N
 };
 static const struct {
     const char* env;
@@ -72,7 +72,14 @@ static const struct {
     {"HCOMM_GFX_XCD_RUN_COPY_STREAM", 128},
     {"HCOMM_GFX_XCD_RUN_REDUCE", 128},
     {"HCOMM_GFX_XCD_RUN_REDUCE_STREAM", 32},
-    {"HCOMM_GFX_LDS_FOLD", 0},
+    /* the k-way folds, measured on their single-launch lowerings.  Tree (16 x 128 MiB int32 recursive halving, 8 x
+     * 128 MiB bf16 NHR): 1.005 -> 0.957 ms and 0.519 -> 0.502 ms with the bound and the runs (inputs kept: 0.785 ->
+     * 0.720, 0.398 -> 0.377).  Chain: neither helps the 8 x 128 MiB ring (0.573 ms either way) and both cost the
+     * cache-resident one-shot mesh (8 x 4 MiB: 37 -> 48 us with runs of 128 tiles), so it keeps tiles as dealt. */
+    {"HCOMM_GFX_LDS_CHAIN", 0},
+    {"HCOMM_GFX_XCD_RUN_CHAIN", 0},
+    {"HCOMM_GFX_LDS_TREE", 53248},
+    {"HCOMM_GFX_XCD_RUN_TREE", 128},
 };
 static uint64_t g_tune[TUNE_N]; /* value + 1; 0 = not read yet (same relaxed-atomic rule as env_once) */
 
@@ -138,7 +145,8 @@ void hg_finish_fold(HgLaunch* l)
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
     l->streaming = 0;
-    l->lds_bytes = lds_of(TUNE_LDS_FOLD);
+    l->lds_bytes = lds_of(t->tree ? TUNE_LDS_TREE : TUNE_LDS_CHAIN);
+    t->xcd_run = (uint32_t)tune(t->tree ? TUNE_RUN_TREE : TUNE_RUN_CHAIN);
     if (!t->tree) {
         /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
         const uint64_t small_bytes = env_once(&g_small_bytes, "HCOMM_GFX_SMALL_BYTES", 1u << 20);

@@ -50,6 +50,9 @@ typedef struct HgThread {
     /* launch log */
     HcommGfxLaunchRecord* log;
     uint32_t log_n, log_cap;
+    /* the host thread's launch context that holds recorded operations of this thread between HcommBatchModeStart and
+     * End (NULL outside a batch); read and written with atomics: another host thread may ask to free the thread */
+    const void* batch_owner;
     int log_enabled;
     int log_fixed; /* set while a call that must not allocate runs: the log takes what fits and drops the rest */
 } HgThread;

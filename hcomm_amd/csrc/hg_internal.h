@@ -75,6 +75,7 @@ typedef struct {
                               * the other ranks in cyclic order, entered at distance start[s] + 1 */
     uint32_t keep_inputs;    /* tree modes 1 - 3: the partials the step-wise replay leaves in the inputs are not stored */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
+    uint32_t xcd_run;        /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
     uint8_t start[HG_MAX_SEG]; /* chain with ascending == 2 only */

@@ -97,7 +97,7 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];

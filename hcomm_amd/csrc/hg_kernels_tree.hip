@@ -162,7 +162,7 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     constexpr uint32_t NU = HG_TREE_NU(1u << L);
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(0u); tile < total; tile += gridDim.x) {
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * NU) + tid;
         const uint64_t bytes = tab.bytes[s];

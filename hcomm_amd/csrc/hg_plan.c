@@ -506,8 +506,11 @@ typedef struct {
 typedef struct {
     int32_t left, right; /* -1, -1: a leaf */
     uint32_t rank;
+    uint32_t depth;      /* folds between this node and its deepest leaf: 0 for a leaf */
     uint64_t off;
 } SymNode;
+
+#define HG_TREE_MAX_DEPTH 5u /* the tree kernel folds 32 = 2^5 leaf positions at most */
 
 typedef struct {
     SymCell* cell;
@@ -533,17 +536,16 @@ static int32_t sym_node(SymState* st, int32_t left, int32_t right, uint32_t rank
     n->right = right;
     n->rank = rank;
     n->off = off;
+    n->depth = 0;
+    if (left >= 0) {
+        const uint32_t a = st->node[left].depth, b = st->node[right].depth;
+        n->depth = 1u + (a > b ? a : b);
+    }
     return (int32_t)st->nnode++;
 }
 
-static uint32_t sym_depth(const SymState* st, int32_t node)
-{
-    if (st->node[node].left < 0) return 0;
-    const uint32_t a = sym_depth(st, st->node[node].left), b = sym_depth(st, st->node[node].right);
-    return 1u + (a > b ? a : b);
-}
-
-/* node into the span of 2^h positions that starts at q; 0 when a leaf lies at another offset than the segment */
+/* node into the span of 2^h positions that starts at q; 0 when a leaf lies at another offset than the segment.
+ * Recursion is as deep as the node, which no caller lets exceed HG_TREE_MAX_DEPTH. */
 static int sym_place(const SymState* st, int32_t node, uint8_t* pos, uint32_t q, uint32_t h, uint64_t off)
 {
     const SymNode* n = &st->node[node];
@@ -564,8 +566,9 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
     st.node = (SymNode*)calloc((size_t)st.cap + ol->n, sizeof(SymNode));       /* and three new nodes */
     int32_t* pend_cell = (int32_t*)calloc(ol->n + 1, sizeof(int32_t));
     int32_t* pend_node = (int32_t*)calloc(ol->n + 1, sizeof(int32_t));
+    uint64_t* written_in = (uint64_t*)calloc(st.cap, sizeof(uint64_t)); /* per cell: 1 + first operation of the step that writes it */
     HgLaunch* l = NULL;
-    int rc = (st.cell && st.node && pend_cell && pend_node) ? HCCL_SUCCESS : HCCL_E_MEMORY;
+    int rc = (st.cell && st.node && pend_cell && pend_node && written_in) ? HCCL_SUCCESS : HCCL_E_MEMORY;
     /* the operations of a step act in parallel: all of them read the state the step began with */
     for (uint64_t i = 0, j; i < ol->n && rc == HCCL_SUCCESS; i = j) {
         for (j = i; j < ol->n && ol->ops[j].step == ol->ops[i].step && rc == HCCL_SUCCESS; ++j) {
@@ -602,14 +605,26 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
                 rc = HCCL_E_NOT_SUPPORT;
                 break;
             }
+            /* "every operation of a step reads the state the step began with" equals the list's replay only while no
+             * operation of the step writes what another one of it reads or writes: refuse the lists where it does not */
+            if (written_in[dst] > i || written_in[src] > i) {
+                rc = HCCL_E_NOT_SUPPORT;
+                break;
+            }
+            written_in[dst] = i + 1;
             pend_cell[j] = dst;
             pend_node[j] = o->kind ? sym_node(&st, st.cell[dst].node, st.cell[src].node, 0, 0) : st.cell[src].node;
+            if (st.node[pend_node[j]].depth > HG_TREE_MAX_DEPTH) { /* deeper than the kernel folds: no point in going on */
+                rc = HCCL_E_NOT_SUPPORT;
+                break;
+            }
         }
         for (uint64_t t = i; t < j && rc == HCCL_SUCCESS; ++t)
             if (pend_cell[t] >= 0) st.cell[pend_cell[t]].node = pend_node[t];
     }
     free(pend_cell);
     free(pend_node);
+    free(written_in);
     /* When every rank's output holds the same trees at the same places, the output cells of rank 0 are the segments
      * and the root goes to all outputs; otherwise (whole-message recursive doubling: every rank folds in an order of
      * its own) every output cell is a segment with a single destination. */
@@ -623,7 +638,7 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
             rc = HCCL_E_NOT_SUPPORT;
             break;
         }
-        const uint32_t d = sym_depth(&st, c->node);
+        const uint32_t d = st.node[c->node].depth;
         if (d > depth) depth = d;
         if (c->rank == 0) {
             ++nseg;
@@ -636,8 +651,8 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
         }
     }
     if (!uniform) nseg = nseg_all;
-    if (rc == HCCL_SUCCESS && depth > 5u) rc = HCCL_E_NOT_SUPPORT; /* the kernel folds 32 = 2^5 positions at most */
-    const uint32_t k = 1u << (depth > 5u ? 5u : depth);
+    if (rc == HCCL_SUCCESS && depth > HG_TREE_MAX_DEPTH) rc = HCCL_E_NOT_SUPPORT;
+    const uint32_t k = 1u << (depth > HG_TREE_MAX_DEPTH ? HG_TREE_MAX_DEPTH : depth);
     const uint32_t per_launch = HG_POS_BYTES / k < HG_MAX_SEG ? HG_POS_BYTES / k : HG_MAX_SEG;
     for (uint32_t i = 0; i < st.ncell && rc == HCCL_SUCCESS; ++i) {
         const SymCell* c = &st.cell[i];

@@ -898,13 +898,14 @@ int32_t HcommGfxPlanCreateFromOps(
 
 /*
  * A caller's own op list over the roles 0 (in), 1 (out) and 2 (communication buffer) as tree launches that keep the
- * inputs: the list is replayed on symbols (the operations of a step all read the state the step began with), and what
- * it leaves in the outputs - per byte range a tree of dst (op) src folds over input ranges - is evaluated in registers
- * from the original inputs.  Every out range the list writes receives the bits the list's replay would give it; in[]
- * is only read and no communication buffer is needed, whatever the list does to them.  HCCL_E_NOT_SUPPORT when a
- * range is read with other bounds than it was written with, when a value is read that the list never wrote, when a
- * tree is deeper than 5 folds, combines ranges at different offsets, or starts off a 16-byte boundary.  ops ordered
- * by step.  No counterpart in the reference.
+ * inputs: the list is replayed on symbols, and what it leaves in the outputs - per byte range a tree of dst (op) src
+ * folds over input ranges - is evaluated in registers from the original inputs.  Every out range the list writes
+ * receives the bits the list's replay would give it; in[] is only read and no communication buffer is needed, whatever
+ * the list does to them.  HCCL_E_NOT_SUPPORT when a range is read with other bounds than it was written with, when a
+ * value is read that the list never wrote, when an operation reads or writes a range that an earlier operation of the
+ * same step writes (the operations of a step must not observe each other: such a step has no single meaning), as
+ * soon as a tree grows deeper than 5 folds, when a tree combines ranges at different offsets or starts off a 16-byte
+ * boundary.  ops ordered by step.  No counterpart in the reference.
  */
 int32_t HcommGfxPlanCreateFromOpsKeepInputs(
     const HcommGfxSchedOp* ops, uint64_t nOps, uint32_t nRanks, void* const* in, void* const* out, HcommDataType dataType,

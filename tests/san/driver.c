@@ -150,6 +150,28 @@ int main(void)
             }
             free(ops);
         }
+    /* lists a caller could write that the tree lowering must refuse at once: a value folded into itself (its tree doubles
+     * with every operation), a chain of a million folds, operations of one step that observe each other */
+    {
+        const uint64_t big = 1000001;
+        HcommGfxSchedOp* ops = (HcommGfxSchedOp*)calloc(big, sizeof(*ops));
+        if (!ops) return 2;
+        for (int variant = 0; variant < 3; ++variant) {
+            const uint64_t total = variant == 0 ? 65 : variant == 1 ? big : 3;
+            memset(ops, 0, total * sizeof(*ops));
+            ops[0].kind = 0; ops[0].dstBuf = 1; ops[0].srcBuf = 0; ops[0].bytes = 4096;       /* out0 = in0 */
+            for (uint64_t i = 1; i < total; ++i) {
+                ops[i].step = variant == 2 ? 1 : (uint32_t)i;                                   /* variant 2: both in step 1 */
+                ops[i].kind = 1; ops[i].dstBuf = 1; ops[i].bytes = 4096;                        /* out0 += ... */
+                ops[i].srcBuf = variant == 0 ? 1 : 0;                                           /* ... out0 / in1 / in1, in2 */
+                ops[i].srcRank = variant == 0 ? 0 : variant == 1 ? 1 : (uint32_t)i;
+            }
+            p = NULL;
+            if (HcommGfxPlanCreateFromOpsKeepInputs(ops, total, 3, bufs[0], bufs[1], HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM, &p) == HCCL_E_NOT_SUPPORT && !p) ++checks;
+            else return 3;
+        }
+        free(ops);
+    }
     /* two-level executors */
     for (unsigned si = 0; si < 5; ++si)
         for (unsigned li = 0; li < 5; ++li)

@@ -1,6 +1,7 @@
 /* Eight host threads use the library at once, each with recorder threads of its own: thread registry, batch mode
  * (per host thread), plan building and replay, launch logs.  Built with -fsanitize=thread by
  * tests/test_host_sanitizers.py; exit status 0 = every call returned what a single-threaded run returns. */
+#define _POSIX_C_SOURCE 200809L
 #include <pthread.h>
 #include <stdio.h>
 #include <stdint.h>
@@ -41,10 +42,57 @@ static void* worker(void* arg)
     return (void*)bad;
 }
 
+/* One host thread records into a recorder thread inside a batch while another host thread tries to free it and to
+ * record into it: both are refused until the batch has ended, and nothing of the refused calls is left queued. */
+static pthread_barrier_t g_bar;
+static ThreadHandle g_shared;
+
+static void* batch_owner(void* arg)
+{
+    (void)arg;
+    uintptr_t bad = 0;
+    bad += HcommGfxRecorderThreadAlloc(&g_shared) != 0;
+    bad += HcommBatchModeStart("owner") != 0;
+    bad += HcommLocalCopyOnThread(g_shared, (void*)0x200000, (const void*)0x100000, 4096) != 0;
+    pthread_barrier_wait(&g_bar); /* the other thread now tries to free and to record */
+    pthread_barrier_wait(&g_bar);
+    bad += HcommBatchModeEnd("owner") != 0;
+    uint32_t n = 0;
+    bad += HcommGfxLaunchLogRead(g_shared, NULL, 0, &n) != 0 || n != 1; /* one launch: the other thread's copy was refused */
+    pthread_barrier_wait(&g_bar); /* after End the other thread may free it */
+    return (void*)bad;
+}
+
+static void* batch_intruder(void* arg)
+{
+    (void)arg;
+    uintptr_t bad = 0;
+    pthread_barrier_wait(&g_bar);
+    bad += HcommThreadFree(&g_shared, 1) != HCCL_E_UNAVAIL;
+    bad += HcommBatchModeStart("intruder") != 0;
+    bad += HcommLocalCopyOnThread(g_shared, (void*)0x400000, (const void*)0x300000, 4096) != HCCL_E_UNAVAIL;
+    bad += HcommBatchModeEnd("intruder") != 0;
+    pthread_barrier_wait(&g_bar);
+    pthread_barrier_wait(&g_bar);
+    bad += HcommThreadFree(&g_shared, 1) != 0;
+    return (void*)bad;
+}
+
 int main(void)
 {
     pthread_t t[8];
     uintptr_t bad = 0;
+    if (pthread_barrier_init(&g_bar, NULL, 2)) return 2;
+    if (pthread_create(&t[0], NULL, batch_owner, NULL) || pthread_create(&t[1], NULL, batch_intruder, NULL)) return 2;
+    for (int i = 0; i < 2; ++i) {
+        void* r = NULL;
+        pthread_join(t[i], &r);
+        bad += (uintptr_t)r;
+    }
+    if (bad) {
+        printf("batch ownership: bad %lu\n", (unsigned long)bad);
+        return 1;
+    }
     for (uintptr_t i = 0; i < 8; ++i)
         if (pthread_create(&t[i], NULL, worker, (void*)i)) return 2;
     for (int i = 0; i < 8; ++i) {

@@ -245,14 +245,38 @@ def test_op_lists_the_tree_lowering_refuses():
     with pytest.raises(h.HcommError) as e:                   # a user-buffer role of the op-base lists
         h.OpListKeepInputsPlan([(0, 0, 0, 1, 0, 1, 3, 0, 4096)], ins[:2], outs[:2], oracle.F32, oracle.SUM)
     assert e.value.code == R.E_PARA
-    # two operations of one step read the state the step began with: a swap through the outputs
-    p = h.OpListKeepInputsPlan([(0, 0, 0, 1, 0, 0, 0, 0, 4096), (0, 0, 1, 1, 0, 1, 0, 0, 4096),
-                                (1, 1, 0, 1, 0, 1, 1, 0, 4096), (1, 1, 1, 1, 0, 0, 1, 0, 4096)], ins[:2], outs[:2],
-                               oracle.F32, oracle.SUM)
-    rank_of = {ins[0]: 0, ins[1]: 1}
-    trees = {h.plan_tree(p, 0, sg, rank_of, with_owner=True)[3]: h.plan_tree(p, 0, sg, rank_of)[0] for sg in range(2)}
-    assert trees == {0: [0, 1], 1: [1, 0]}                   # not [0, [1, 0]]: rank 1's fold reads out[0] of before the step
+    # Operations of one step that observe each other have no single meaning (the step-wise lowering runs them one
+    # after the other, the symbolic replay gives all of them the state the step began with): refused, not guessed.
+    swap = [(0, 0, 0, 1, 0, 0, 0, 0, 4096), (0, 0, 1, 1, 0, 1, 0, 0, 4096),
+            (1, 1, 0, 1, 0, 1, 1, 0, 4096), (1, 1, 1, 1, 0, 0, 1, 0, 4096)]          # out0 += out1 beside out1 += out0
+    twice = [(0, 0, 0, 1, 0, 0, 0, 0, 4096),
+             (1, 1, 0, 1, 0, 1, 0, 0, 4096), (1, 1, 0, 1, 0, 2, 0, 0, 4096)]         # out0 += in1 beside out0 += in2
+    for ops, n in ((swap, 2), (twice, 3)):
+        with pytest.raises(h.HcommError) as e:
+            h.OpListKeepInputsPlan(ops, ins[:n], outs[:n], oracle.F32, oracle.SUM)
+        assert e.value.code == R.E_NOT_SUPPORT
+    # the same two folds in steps of their own are a chain of two: out0 = (in0 + in1) + in2
+    p = h.OpListKeepInputsPlan([twice[0], twice[1], (2,) + twice[2][1:]], ins[:3], outs[:3], oracle.F32, oracle.SUM)
+    rank_of = {ins[r]: r for r in range(3)}
+    assert h.plan_tree(p, 0, 0, rank_of)[0] == [[0, 1], 2]
     p.destroy()
+
+
+def test_deep_or_self_referencing_lists_are_refused_at_once():
+    """Trees deeper than the kernel folds are refused while the list is replayed, not after: a value folded into itself
+    doubles its tree with every operation and a chain grows by one fold per operation, so both lists below would
+    otherwise cost time or stack in proportion to 2^n / n."""
+    import time
+    ins, outs, _ = ptrs(2)
+    first = (0, 0, 0, 1, 0, 0, 0, 0, 4096)                                           # out0 = in0
+    doubling = [first] + [(1 + i, 1, 0, 1, 0, 0, 1, 0, 4096) for i in range(64)]       # out0 += out0, 64 times
+    chain = [first] + [(1 + i, 1, 0, 1, 0, 1, 0, 0, 4096) for i in range(200000)]      # out0 += in1, 200,000 times
+    for ops in (doubling, chain):
+        t0 = time.perf_counter()
+        with pytest.raises(h.HcommError) as e:
+            h.OpListKeepInputsPlan(ops, ins, outs, oracle.F32, oracle.SUM)
+        assert e.value.code == R.E_NOT_SUPPORT
+        assert time.perf_counter() - t0 < 5.0
 
 
 def merged_runs(segments):
