@@ -321,15 +321,45 @@ static int sched_allreduce_chunk_mesh(HgOpList* l, uint32_t n, uint64_t count, u
  * k is the round that maps to w (:225-229), the neighbour d + 1 reduces straight onto d's own copy (:230-247),
  * the slots are folded towards the slot at d's natural offset (:301-364), and everybody fetches that slot
  * (:417-424). */
+/* The block of slots RunLocalReduce halves: 2^floor(log2(n - 1)) of the n - 1 slots (all_reduce_local_reduce.cc:304-305). */
+static uint32_t local_reduce_block(uint32_t n)
+{
+    uint32_t p = 1;
+    while (2u * p <= n - 1u) p *= 2u;
+    return p;
+}
+
+/* Where rank d's folded slice ends up, as a slot index inside d's window: the block starts at slot 0 for the ranks
+ * below the block size and n - block - 1 slots further up for the others (:330), and the halving rounds walk towards
+ * position min(d, or d - block + 1, block - 1) of the block (:328-329, :333-362). */
+static uint32_t local_reduce_result_slot(uint32_t n, uint32_t d)
+{
+    const uint32_t p = local_reduce_block(n);
+    if (d < p) return d;
+    const uint32_t target = d - p + 1u < p - 1u ? d - p + 1u : p - 1u;
+    return n - p - 1u + target;
+}
+
+/* The gather fetches rank d's slice from slot d of d's window, the last rank's from its slot n - 2 (:419-423; the
+ * last rank's window starts one slot up, :102-110).  That is where the folds leave it when n is a power of two, and
+ * when n is 3; for every other rank count some rank's result sits in another slot and the gather would fetch a partial
+ * sum, so those counts are refused (tests/test_local_reduce_any_n.py replays the reference's statements for them). */
+int hg_local_reduce_lands(uint32_t n)
+{
+    for (uint32_t d = 0; d < n; ++d)
+        if (local_reduce_result_slot(n, d) != (d == n - 1u ? n - 2u : d)) return 0;
+    return 1;
+}
+
 static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count, uint32_t unit)
 {
     const uint64_t total = count * unit;
     if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, total); /* :154-163 */
-    if (n & (n - 1)) return HCCL_E_PARA;
+    if (!hg_local_reduce_lands(n)) return HCCL_E_PARA;
     HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
     uint64_t per;
     local_reduce_slices(total, n, unit, sl, &per);
-    const uint32_t half_n = n / 2; /* 2^floor(log2(n-1)) for a power-of-two n */
+    const uint32_t half_n = local_reduce_block(n); /* slots in the block that is halved */
     uint32_t step = 0;
     for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, COPY, d, SCR, sl[d].offset, d, IN, sl[d].offset, sl[d].size));
     ++step;
@@ -346,10 +376,10 @@ static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count,
                 CHK(push(l, step, COPY, d, SCR, base + (uint64_t)w * per, sender, IN, sl[d].offset, sl[d].size));
             }
         }
-    /* fold the n-1 slots: first the slots beyond the power-of-two block onto (or from) the first ones ... */
+    /* fold the n-1 slots: first the n - 1 - block slots beyond the block onto (or from) the first ones (:311-327) ... */
     for (uint32_t d = 0; d < n; ++d) {
         const uint64_t base = (d == n - 1) ? per : 0;
-        for (uint32_t i = 0; i + 1 < half_n; ++i) {
+        for (uint32_t i = 0; i + half_n + 1 < n; ++i) {
             const uint64_t lo = base + (uint64_t)i * per, hi = base + (uint64_t)(half_n + i) * per;
             if (d < half_n) CHK(push(l, step, REDUCE, d, SCR, lo, d, SCR, hi, sl[d].size));
             else CHK(push(l, step, REDUCE, d, SCR, hi, d, SCR, lo, sl[d].size));
@@ -363,7 +393,7 @@ static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count,
         for (uint32_t d = 0; d < n; ++d) {
             const uint64_t base = (d == n - 1) ? per : 0;
             uint32_t target = (d < half_n) ? d : ((d - half_n + 1 < half_n - 1) ? d - half_n + 1 : half_n - 1);
-            uint32_t first = (d < half_n) ? 0 : half_n - 1;
+            uint32_t first = (d < half_n) ? 0 : n - half_n - 1;
             for (uint32_t z = 0; z < q; ++z) { /* replay the earlier rounds' choice of half */
                 const uint32_t h = half_n >> (z + 1);
                 if (target >= h) {

@@ -49,6 +49,8 @@ int hg_schedule_dbring_rs(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_
  * ranks, rounded up to slot sizes) then stays far inside 64 bits.  Larger counts are refused with HCCL_E_PARA. */
 #define HG_MAX_COUNT ((uint64_t)1 << 48)
 void hg_oplist_free(HgOpList* l);
+/* 1 when the deterministic mesh allreduce's folds leave every rank's slice where its gather reads it (n a power of two, or 3). */
+int hg_local_reduce_lands(uint32_t n);
 /* Per-rank communication-buffer bytes alg needs (0 when it stages nothing). */
 uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype);
 

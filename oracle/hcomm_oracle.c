@@ -588,16 +588,34 @@ static void prog_rs_mesh(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count,
  * mesh allreduce.  Three buffers per rank: user input (B_IN), the communication buffer commMemOut (B_SCR) and
  * user output (B_OUT).  An op is recorded under the rank that OWNS the destination; the rank that issues it is
  * the src rank.  Rounds that the reference runs concurrently on sub-streams get one step each.
- * The slot arithmetic of RunLocalReduce leaves the result at the offset the gather reads (:419) only for a
- * power-of-two rank count; other counts are refused. */
-static int prog_allreduce_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit)
+ * RunLocalReduce leaves rank d's result in slot `center` of the block of 2^floor(log2(n-1)) slots it halves (:328-331),
+ * the gather reads slot d, or n - 2 for the last rank (:419 with the last rank's window one slot up, :102-110).  The two
+ * agree for every rank only when n is a power of two or 3 (local_reduce_lands; tests/test_local_reduce_any_n.py replays
+ * the statements for the other counts and finds the gather reading a partial sum), so other counts are refused -
+ * unless as_written is set, which emits the statements as they stand for that test. */
+static int local_reduce_lands(uint32_t n)
+{
+    uint32_t power = 0;
+    while ((2u << power) <= n - 1) power++;
+    const uint32_t rank_power = 1u << power;
+    for (uint32_t d = 0; d < n; ++d) {
+        uint32_t center = d < rank_power ? d : d - rank_power + 1; /* :328-329 */
+        if (center > rank_power - 1) center = rank_power - 1;
+        const uint32_t block = d < rank_power ? 0 : n - rank_power - 1; /* :330 */
+        const uint32_t read = d == n - 1 ? n - 2 : d;                   /* :419 */
+        if (block + center != read) return 0;
+    }
+    return 1;
+}
+
+static int prog_allreduce_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint32_t unit, int as_written)
 {
     const uint64_t total = count * unit;
     if (n == 1) { /* :154-163 */
         emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, total);
         return 0;
     }
-    if (n & (n - 1)) return -1;
+    if (!as_written && !local_reduce_lands(n)) return -1;
     /* PrepareSlice :69-120; the communication buffer is not the user output, so sizeLimit = totalSize (:84-88) */
     OrcSlice sl[ORC_MAX_RANKS], start[ORC_MAX_RANKS];
     const uint64_t ori = (total + n - 1) / n;
@@ -1136,7 +1154,8 @@ enum {
     ORC_ALG_RS_LOCAL_REDUCE = 13,
     ORC_ALG_ALLREDUCE_DOUBLING = 14,
     ORC_ALG_ALLREDUCE_NHR_ONESHOT = 15,
-    ORC_ALG_RS_RHD = 16 /* only between the servers of the two-level reduce-scatter */
+    ORC_ALG_RS_RHD = 16, /* only between the servers of the two-level reduce-scatter */
+    ORC_ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN = 17 /* traces only: the statements for any rank count, right or wrong */
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -1214,7 +1233,8 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
                 prog_rs_local_reduce(t, r, n, count, unit);
                 break;
             case ORC_ALG_ALLREDUCE_LOCAL_REDUCE:
-                if (prog_allreduce_local_reduce(t, r, n, count, unit) != 0) {
+            case ORC_ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN:
+                if (prog_allreduce_local_reduce(t, r, n, count, unit, alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN) != 0) {
                     free(t->ops);
                     return -1;
                 }
@@ -1333,7 +1353,7 @@ static void run_template(OrcTrace* t, int alg, uint32_t r, uint32_t n, uint64_t 
         case ORC_ALG_RS_RING_STANDALONE: prog_rs_ring_standalone(t, r, n, count, count, unit); break;
         case ORC_ALG_ALLREDUCE_MESH_ASCENDING: prog_allreduce_mesh_ascending(t, r, n, count, unit); break;
         case ORC_ALG_ALLREDUCE_CHUNK_MESH: prog_allreduce_chunk_mesh(t, r, n, count, unit); break;
-        case ORC_ALG_ALLREDUCE_LOCAL_REDUCE: prog_allreduce_local_reduce(t, r, n, count, unit); break;
+        case ORC_ALG_ALLREDUCE_LOCAL_REDUCE: prog_allreduce_local_reduce(t, r, n, count, unit, 0); break;
         case ORC_ALG_ALLREDUCE_NHR: prog_allreduce_nhr(t, r, n, count, unit); break;
         case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, count, unit); break;
         case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
@@ -1414,7 +1434,8 @@ static int build_trace_opbase(OrcTrace* t, int alg, uint32_t n, uint64_t count, 
     if (n == 0 || n > ORC_MAX_RANKS || unit == 0 || alg == ORC_ALG_RS_RING_STAGE) return -1;
     const uint64_t max_count = orc_opbase_max_count(alg, n, ccl_bytes, dtype);
     if (max_count == 0) return -1; /* :213-218 / :163-165 */
-    if ((alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE || alg == ORC_ALG_ALLREDUCE_DOUBLING) && (n & (n - 1))) return -1;
+    if (alg == ORC_ALG_ALLREDUCE_DOUBLING && (n & (n - 1))) return -1;
+    if (alg == ORC_ALG_ALLREDUCE_LOCAL_REDUCE && n > 1 && !local_reduce_lands(n)) return -1;
     for (uint32_t r = 0; r < n; r++) {
         const int rc = prog_opbase(t, alg, r, n, count, max_count, dtype);
         if (rc || t->oom) {

@@ -101,8 +101,8 @@ def test_deterministic_mesh_allreduce_single_launch_limits():
     with pytest.raises(h.HcommError) as e:                       # slots of 10 bytes: slices off 16-byte boundaries
         h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 38, oracle.I8, oracle.SUM)
     assert e.value.code == R.E_NOT_SUPPORT
-    with pytest.raises(h.HcommError) as e:                       # as the step-wise replay: powers of two only
-        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins[:3], outs[:3], 4096, oracle.F32, oracle.SUM)
+    with pytest.raises(h.HcommError) as e:                       # as the step-wise replay: rank counts whose folds land
+        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ptrs(5)[0], ptrs(5)[1], 4096, oracle.F32, oracle.SUM)
     assert e.value.code == R.E_PARA
     p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins[:1], outs[:1], 4096, oracle.F32, oracle.SUM)
     assert [r.kind for r in p.launches()] == [h.Kernel.COPY]

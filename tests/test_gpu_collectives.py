@@ -132,6 +132,8 @@ CASES = [
     ("local_reduce", 8, 1001, "int16", "sum"),     # slots fall back to 512-byte / element alignment
     ("local_reduce", 8, 7, "fp32", "sum"),
     ("local_reduce", 1, 100, "fp32", "sum"),
+    ("local_reduce", 3, 100003, "fp32", "sum"),    # the one rank count besides the powers of two whose folds land
+    ("local_reduce", 3, 5, "bf16", "max"),
     ("chunk_mesh", 8, 1 << 20, "bf16", "sum"),
     ("chunk_mesh", 7, 100003, "fp32", "sum"),
     ("chunk_mesh", 3, 4099, "fp16", "max"),
@@ -220,6 +222,7 @@ USER_BUFFER_FUSED = [
     ("local_reduce", 8, 300007, "int32", "min"), ("local_reduce", 4, 65536, "fp32", "prod"),
     ("local_reduce", 16, 1 << 20, "bf16", "sum"), ("local_reduce", 8, 8 * 8192 + 24, "int16", "sum"),
     ("local_reduce", 1, 100, "fp32", "sum"), ("local_reduce", 4, 0, "fp32", "sum"),
+    ("local_reduce", 3, 100003, "fp32", "sum"), ("local_reduce", 3, 3 * 8192 + 8, "fp16", "min"),
 ]
 
 
@@ -509,6 +512,8 @@ def test_randomized_shapes(gpu_thread):
         n = int(rng.integers(1, 17))
         if name in ("local_reduce", "doubling"):
             n = 1 << int(rng.integers(0, 5))
+            if name == "local_reduce" and done % 5 == 0:
+                n = 3
         base = interesting[rng.integers(len(interesting))]
         count = int(base * rng.integers(1, 4) + rng.integers(0, 3))
         dtype = ["int8", "int16", "int32", "fp16", "fp32", "bf16"][rng.integers(6)]
