@@ -76,7 +76,8 @@ class Alg:
     ALLREDUCE_RING, REDUCE_SCATTER_RING, ALLREDUCE_RHD, ALLREDUCE_MESH_ONESHOT, REDUCE_SCATTER_MESH, \
         REDUCE_SCATTER_RING_STANDALONE, ALLREDUCE_MESH_ONESHOT_ASCENDING, ALLREDUCE_LOCAL_REDUCE, \
         ALLREDUCE_CHUNK_MESH, ALLREDUCE_NHR, REDUCE_SCATTER_NHR, ALLREDUCE_NB, REDUCE_SCATTER_NB, \
-        REDUCE_SCATTER_LOCAL_REDUCE, ALLREDUCE_DOUBLING, ALLREDUCE_NHR_ONESHOT, REDUCE_SCATTER_RHD = range(17)
+        REDUCE_SCATTER_LOCAL_REDUCE, ALLREDUCE_DOUBLING, ALLREDUCE_NHR_ONESHOT, REDUCE_SCATTER_RHD, \
+        REDUCE_SCATTER_WINDOW_HALVING = range(18)
 
 
 class Lowering:

@@ -300,7 +300,7 @@ int32_t HcommGfxScheduleCheck(
     if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_IN_PLACE;
     if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_MESH || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE ||
         alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB ||
-        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE)
+        alg == HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING)
         e = HCOMM_GFX_EXPECT_REDUCE_SCATTER_OUT;
     rc = HcommGfxOpListCheck(l.ops, l.n, nRanks, e, count, strideCount, HcommGfxDataTypeSize(dataType), rep);
     hg_oplist_free(&l);

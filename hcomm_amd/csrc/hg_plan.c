@@ -700,6 +700,59 @@ static int fused_from_trees(HcommGfxPlan* p, const HgOpList* ol, uint32_t n, voi
     return rc;
 }
 
+/* Leaf table of the rank-order tree over n_servers x n_local ranks: the low position bits walk a server's devices so
+ * that level l folds device j + 2^(bits - 1 - l) onto device j, the high bits the servers likewise; 255 = no leaf. */
+static uint32_t rank_order_positions(uint32_t n_servers, uint32_t n_local, uint8_t* pos)
+{
+    uint32_t bits_l = 0, bits_s = 0;
+    while ((1u << bits_l) < n_local) ++bits_l;
+    while ((1u << bits_s) < n_servers) ++bits_s;
+    uint32_t k = 1u << (bits_l + bits_s);
+    if (k < 2) k = 2;
+    memset(pos, 255, HG_POS_BYTES);
+    for (uint32_t q = 0; q < k; ++q) {
+        const uint32_t dev = bitrev_n(q & ((1u << bits_l) - 1u), bits_l), srv = bitrev_n(q >> bits_l, bits_s);
+        if (dev < n_local && srv < n_servers) pos[q] = (uint8_t)(srv * n_local + dev);
+    }
+    return k;
+}
+
+/* The AICPU deterministic reduce-scatter in one launch: SelfLocalReduce's folds (the slots beyond the largest power of
+ * two onto the first ones, then halving rounds) are the rank-order tree over the N inputs, slot s holding rank s's
+ * slice; block d of every input at d * stride, root to out[d]. */
+static int fused_window_halving(HcommGfxPlan* p, uint32_t n, void* const* in, void* const* out, uint64_t count, uint64_t stride,
+                                int dtype, int op)
+{
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    const uint64_t block = count * unit;
+    if (block == 0) return HCCL_SUCCESS;
+    if (n > 32u) return HCCL_E_NOT_SUPPORT;
+    /* 128-bit accesses: every block of every input must start on a 16-byte boundary */
+    if ((stride * unit) & (HG_VEC_BYTES - 1u)) return HCCL_E_NOT_SUPPORT;
+    HgLaunch* l = (HgLaunch*)calloc(1, sizeof(HgLaunch));
+    if (!l) return HCCL_E_MEMORY;
+    l->kind = HCOMM_GFX_KERNEL_TREE;
+    l->dtype = (uint32_t)dtype;
+    l->op = (uint32_t)op;
+    HgFoldTable* f = &l->tab.fold;
+    f->tree = 4u;
+    f->k = rank_order_positions(1, n, f->pos);
+    f->nranks = n;
+    f->out_mode = 1u;
+    f->nseg = n;
+    for (uint32_t r = 0; r < n; ++r) {
+        f->in[r] = in[r];
+        f->out[r] = out[r];
+        f->off[r] = stride * unit * r;
+        f->bytes[r] = block;
+        f->owner[r] = (uint8_t)r;
+    }
+    hg_finish_fold(l);
+    const int rc = plan_push(l, p);
+    free(l);
+    return rc;
+}
+
 static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n, void* const* in, void* const* out,
                        uint64_t count, uint64_t stride, int dtype, int op, int keep_inputs)
 {
@@ -746,6 +799,9 @@ static int lower_fused(HcommGfxPlan* p, int alg, const HgOpList* ol, uint32_t n,
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE:
             if (n == 1) return single_copy(p, out[0], in[0], total);
             return fused_rs_local_reduce(p, n, in, out, count, dtype, op);
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING:
+            if (n == 1) return single_copy(p, out[0], in[0], total);
+            return fused_window_halving(p, n, in, out, count, stride, dtype, op);
         default: return HCCL_E_NOT_SUPPORT;
     }
 }
@@ -1318,14 +1374,8 @@ int32_t HcommGfxOrderPreservedFusedPlanCreate(
         l->op = (uint32_t)reduceOp;
         HgFoldTable* f = &l->tab.fold;
         f->tree = 4u;
-        f->k = 1u << (bits_l + bits_s);
-        if (f->k < 2) f->k = 2;
+        f->k = rank_order_positions(nServers, nLocal, f->pos);
         f->nranks = nRanks;
-        memset(f->pos, 255, sizeof(f->pos));
-        for (uint32_t q = 0; q < f->k; ++q) {
-            const uint32_t dev = bitrev_n(q & ((1u << bits_l) - 1u), bits_l), srv = bitrev_n(q >> bits_l, bits_s);
-            if (dev < nLocal && srv < nServers) f->pos[q] = (uint8_t)(srv * nLocal + dev);
-        }
         for (uint32_t r = 0; r < nRanks; ++r) {
             f->in[r] = userIn[r];
             f->out[r] = userOut[r];

@@ -281,6 +281,7 @@ uint64_t hg_scratch_bytes(int alg, uint32_t n, uint64_t count, int dtype)
         }
         return max_off + (uint64_t)(n - 1) * rs_local_reduce_slot(count * unit);
     }
+    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING) return (uint64_t)n * count * unit; /* one slot per rank */
     if (alg != HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE) return 0;
     return (uint64_t)n * local_reduce_slot(count * unit, n, unit);
 }
@@ -416,6 +417,31 @@ static int sched_allreduce_local_reduce(HgOpList* l, uint32_t n, uint64_t count,
             const uint32_t p = modn((int64_t)d - k, n);
             CHK(push(l, step, COPY, d, OUT, sl[p].offset, p, SCR, (uint64_t)p * sl[0].size, sl[p].size));
         }
+    return HCCL_SUCCESS;
+}
+
+/* The AICPU deterministic reduce-scatter (aicpu_kfc/algorithm/aicpu_reduce_scatter.cc:64-118, one pass of its loop):
+ * all N x N slot writes at once (task_orchestrator.cc:80-95, :370-386: rank s's slice d into slot s of rank d's
+ * window), then SelfLocalReduce (:719-755) in every window - the N - P slots beyond the largest power of two P onto
+ * the first ones as one reduce, log2 P rounds that fold the upper half of what is left onto the lower half, one
+ * contiguous reduce each - and window[0, count) to the output (:203-218). */
+static int sched_rs_window_halving(HgOpList* l, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t cur = count * unit;
+    if (n == 1) return push(l, 0, COPY, 0, OUT, 0, 0, IN, 0, cur); /* slot 0 is the result: copied straight through */
+    uint32_t step = 0;
+    for (uint32_t d = 0; d < n; ++d)
+        for (uint32_t s = 0; s < n; ++s) CHK(push(l, step, COPY, d, SCR, (uint64_t)s * cur, s, IN, stride * d * unit, cur));
+    ++step;
+    uint32_t p = 1;
+    while (2u * p <= n) p *= 2u;
+    if (p < n) {
+        for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, REDUCE, d, SCR, 0, d, SCR, (uint64_t)p * cur, (uint64_t)(n - p) * cur));
+    }
+    ++step;
+    for (uint32_t h = p / 2; h >= 1; h /= 2, ++step)
+        for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, REDUCE, d, SCR, 0, d, SCR, (uint64_t)h * cur, (uint64_t)h * cur));
+    for (uint32_t d = 0; d < n; ++d) CHK(push(l, step, COPY, d, OUT, 0, d, SCR, 0, cur));
     return HCCL_SUCCESS;
 }
 
@@ -714,7 +740,8 @@ int hg_schedule_into(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t 
     if (stride == 0) stride = count;
     if (stride < count || stride > HG_MAX_COUNT) return HCCL_E_PARA;
     if (stride != count && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_MESH && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_RING_STANDALONE &&
-        alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
+        alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg != HCOMM_GFX_ALG_REDUCE_SCATTER_NB &&
+        alg != HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING)
         return HCCL_E_PARA;
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
     if (unit == 0) return HCCL_E_PARA;
@@ -736,6 +763,7 @@ int hg_schedule_into(HgOpList* l, int alg, uint32_t n, uint64_t count, uint64_t 
         case HCOMM_GFX_ALG_REDUCE_SCATTER_LOCAL_REDUCE: rc = sched_rs_local_reduce(l, n, count, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_DOUBLING: rc = sched_allreduce_doubling(l, n, count, unit); break;
         case HCOMM_GFX_ALG_ALLREDUCE_NHR_ONESHOT: rc = sched_allreduce_nhr_oneshot(l, n, count, unit); break;
+        case HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING: rc = sched_rs_window_halving(l, n, count, stride, unit); break;
         default: rc = HCCL_E_PARA;
     }
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);

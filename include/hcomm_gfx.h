@@ -407,7 +407,17 @@ typedef enum {
        place on slices of total / N bytes: accepted only as the level-1 algorithm of
        HcommGfxHierReduceScatterPlanCreate / Emit / Check (the executors' default between servers); the flat plan
        and schedule calls return HCCL_E_PARA for it */
-    HCOMM_GFX_ALG_REDUCE_SCATTER_RHD = 16
+    HCOMM_GFX_ALG_REDUCE_SCATTER_RHD = 16,
+    /* The AICPU deterministic reduce-scatter: AicpuReduceScatter::RunDeterministicReduceScatterLocal
+       (src/legacy/ascend910/framework/device/aicpu_kfc/algorithm/aicpu_reduce_scatter.cc:64-118), one pass of its
+       loop.  Every rank writes slice d of its input into slot `own rank` of rank d's window (the third buffer:
+       HcommGfxScratchBytes = N x count x unit), rank d folds its window in place with
+       TaskOrchestrator::SelfLocalReduce (.../task_orchestrator.cc:719-755: the slots beyond the largest power of two
+       onto the first ones in one reduce, then rounds of window[0, h) (op)= window[h, 2h), one contiguous reduce
+       each) and copies window[0, count) to out[d].  count = per-rank OUTPUT count; input slices at i * strideCount
+       (displs, aicpu_reduce_scatter.cc:78-80).  Any rank count.  The fused lowering is one tree launch on the
+       inputs alone (the rank-order tree: level l folds rank j + K / 2^(l+1) onto rank j). */
+    HCOMM_GFX_ALG_REDUCE_SCATTER_WINDOW_HALVING = 17
 } HcommGfxAlgorithm;
 
 typedef enum {

@@ -18,7 +18,7 @@ I8, I16, I32, F16, F32, BF16 = 0, 1, 2, 3, 4, 11
 ALG_ALLREDUCE_RING, ALG_RS_RING_STAGE, ALG_ALLREDUCE_RHD, ALG_ALLREDUCE_MESH_ONESHOT, ALG_RS_MESH, \
     ALG_RS_RING_STANDALONE, ALG_ALLREDUCE_MESH_ASCENDING, ALG_ALLREDUCE_LOCAL_REDUCE, ALG_ALLREDUCE_CHUNK_MESH, \
     ALG_ALLREDUCE_NHR, ALG_RS_NHR, ALG_ALLREDUCE_NB, ALG_RS_NB, ALG_RS_LOCAL_REDUCE, ALG_ALLREDUCE_DOUBLING, \
-    ALG_ALLREDUCE_NHR_ONESHOT, ALG_RS_RHD, ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN = range(18)
+    ALG_ALLREDUCE_NHR_ONESHOT, ALG_RS_RHD, ALG_RS_WINDOW_HALVING, ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN = range(19)
 
 # storage dtype used on the numpy side for each element type (16-bit floats travel as raw uint16)
 NP_STORAGE = {I8: np.int8, I16: np.int16, I32: np.int32, F16: np.uint16, F32: np.float32, BF16: np.uint16}

@@ -699,6 +699,41 @@ static int prog_allreduce_local_reduce(OrcTrace* t, uint32_t rank, uint32_t n, u
     return 0;
 }
 
+/* The AICPU deterministic reduce-scatter for one rank: AicpuReduceScatter::RunDeterministicReduceScatterLocal,
+ * src/legacy/ascend910/framework/device/aicpu_kfc/algorithm/aicpu_reduce_scatter.cc:64-118, one pass of its loop (the
+ * message fits the window: count * unit * n <= windowSize), with TaskOrchestrator's statements
+ * (.../algorithm/task_orchestrator.cc): rank r copies slice r of its send buffer into slot r of its own window
+ * (SelfCpySnd2Win :80-95 with winOffset = rankId * curSize), writes slice d into slot r of every peer d's window
+ * (IpcCpySnd2Win :370-386, one window offset for all peers), folds its window in place (SelfLocalReduce :719-755: the
+ * slots beyond the largest power of two onto the first ones in ONE reduce, then rounds of window[0, h) (op)= window[h, 2h),
+ * each one reduce) and copies window[0, curSize) to its receive buffer (SelfCpyWin2Rcv :203-218).  Slice d of a send
+ * buffer starts at strideLen * d * unit (displs, :78-80).  The window is B_SCR.  An op is recorded under the rank that
+ * owns the destination. */
+static void prog_rs_window_halving(OrcTrace* t, uint32_t rank, uint32_t n, uint64_t count, uint64_t stride, uint32_t unit)
+{
+    const uint64_t cur = count * unit;
+    if (n == 1) { /* nothing to fold: the round trip through the window leaves the input slice in the receive buffer */
+        emit(t, 0, K_COPY, 0, B_OUT, 0, 0, B_IN, 0, cur);
+        return;
+    }
+    uint32_t step = 0;
+    emit(t, step, K_COPY, rank, B_SCR, (uint64_t)rank * cur, rank, B_IN, stride * rank * unit, cur); /* 1. :102-104 */
+    for (uint32_t index = 0; index < n; index++)                                                       /* 3. :109 */
+        if (index != rank) emit(t, step, K_COPY, index, B_SCR, (uint64_t)rank * cur, rank, B_IN, stride * index * unit, cur);
+    step++;
+    uint32_t power = 0;
+    while ((2u << power) <= n) power++; /* floor(log2(rankNum)), :730 */
+    const uint32_t rank_power = 1u << power;
+    if (rank_power < n) /* :732-740 */
+        emit(t, step, K_REDUCE, rank, B_SCR, 0, rank, B_SCR, (uint64_t)rank_power * cur, (uint64_t)(n - rank_power) * cur);
+    step++;
+    for (uint32_t round = 0; round < power; round++) { /* :742-751 */
+        const uint32_t slice_num = rank_power >> (round + 1);
+        emit(t, step++, K_REDUCE, rank, B_SCR, 0, rank, B_SCR, (uint64_t)slice_num * cur, (uint64_t)slice_num * cur);
+    }
+    emit(t, step, K_COPY, rank, B_OUT, 0, rank, B_SCR, 0, cur); /* 6. :115 */
+}
+
 /* AllReduceChunkMesh for one rank, tpl/temp_all_reduce/all_reduce_chunk_mesh.cc:104-345, in the configuration
  * where the communication buffer (B_SCR) is not the user output (the "single operator" branches :186-193,
  * :239-243).  Slices: PrepareSlice :69-102 over n ranks, then each slice again over n-1 sub-chunks (:104-116). */
@@ -1155,7 +1190,8 @@ enum {
     ORC_ALG_ALLREDUCE_DOUBLING = 14,
     ORC_ALG_ALLREDUCE_NHR_ONESHOT = 15,
     ORC_ALG_RS_RHD = 16, /* only between the servers of the two-level reduce-scatter */
-    ORC_ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN = 17 /* traces only: the statements for any rank count, right or wrong */
+    ORC_ALG_RS_WINDOW_HALVING = 17,
+    ORC_ALG_ALLREDUCE_LOCAL_REDUCE_AS_WRITTEN = 18 /* traces only: the statements for any rank count, right or wrong */
 };
 
 static int cmp_ops(const void* a, const void* b)
@@ -1218,6 +1254,7 @@ static int build_trace(OrcTrace* t, int alg, uint32_t n, uint64_t count, int dty
             case ORC_ALG_RS_NHR: prog_rs_nhr(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_NB: prog_allreduce_nb(t, r, n, count, unit); break;
             case ORC_ALG_RS_NB: prog_rs_nb(t, r, n, count, stride, unit); break;
+            case ORC_ALG_RS_WINDOW_HALVING: prog_rs_window_halving(t, r, n, count, stride, unit); break;
             case ORC_ALG_ALLREDUCE_NHR_ONESHOT: prog_allreduce_nhr_oneshot(t, r, n, count, unit); break;
             case ORC_ALG_ALLREDUCE_DOUBLING:
                 if (prog_allreduce_doubling(t, r, n, count, unit) != 0) {

