@@ -144,7 +144,10 @@ static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_
     }
     if (notify_num) {
         t->notifies = (void**)calloc(notify_num, sizeof(void*));
-        if (!t->notifies) {
+        t->notify_pending = (uint64_t*)calloc(notify_num, sizeof(uint64_t));
+        if (!t->notifies || !t->notify_pending) {
+            free(t->notifies);
+            free(t->notify_pending);
             free(t);
             return NULL;
         }
@@ -153,6 +156,7 @@ static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_
                 if (hg_rt_event_create(&t->notifies[i]) != HCCL_SUCCESS) {
                     for (uint32_t j = 0; j < i; ++j) hg_rt_event_destroy(t->notifies[j]);
                     free(t->notifies);
+                    free(t->notify_pending);
                     free(t);
                     return NULL;
                 }
@@ -163,6 +167,7 @@ static HgThread* thread_new(int recorder, void* stream, int owns_stream, uint32_
         if (!recorder)
             for (uint32_t i = 0; i < notify_num; ++i) hg_rt_event_destroy(t->notifies[i]);
         free(t->notifies);
+        free(t->notify_pending);
         free(t);
         return NULL;
     }
@@ -185,6 +190,7 @@ static void thread_delete(HgThread* t)
         }
     }
     free(t->notifies);
+    free(t->notify_pending);
     free(t->pending);
     free(t->log);
     t->magic = 0;
@@ -257,7 +263,7 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
 HcommResult HcommGfxRecorderThreadAlloc(ThreadHandle* thread)
 {
     if (!thread) return HCCL_E_PTR;
-    HgThread* t = thread_new(1, NULL, 0, 0);
+    HgThread* t = thread_new(1, NULL, 0, 2); /* two notify slots: their bookkeeping is host logic, no event behind them */
     if (!t) return HCCL_E_MEMORY;
     *thread = (ThreadHandle)(uintptr_t)t;
     return HCCL_SUCCESS;
@@ -607,8 +613,12 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
     if (!d) return HCCL_E_PTR;
     if (dstNotifyIdx >= d->notify_num) return HCCL_E_PARA;
     if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
-    if (t->recorder || d->recorder) return HCCL_SUCCESS;
-    return hg_rt_event_record(d->notifies[dstNotifyIdx], t->stream);
+    if (!(t->recorder || d->recorder)) {
+        const int rc = hg_rt_event_record(d->notifies[dstNotifyIdx], t->stream);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    __atomic_add_fetch(&d->notify_pending[dstNotifyIdx], 1, __ATOMIC_RELEASE);
+    return HCCL_SUCCESS;
 }
 
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut)
@@ -618,6 +628,14 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     if (!t) return HCCL_E_PTR;
     if (notifyIdx >= t->notify_num) return HCCL_E_PARA;
     if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    /* A wait on a stream can only follow a record that has been issued: the reference's wait would sit until the
+     * record arrives or timeOut runs out; here a wait that finds no record pending is the one that would have run
+     * out of time, whatever timeOut says, and nothing is queued. */
+    uint64_t pending = __atomic_load_n(&t->notify_pending[notifyIdx], __ATOMIC_ACQUIRE);
+    do {
+        if (pending == 0) return HCCL_E_TIMEOUT;
+    } while (!__atomic_compare_exchange_n(&t->notify_pending[notifyIdx], &pending, pending - 1, 0, __ATOMIC_ACQ_REL,
+                                          __ATOMIC_ACQUIRE));
     if (t->recorder) return HCCL_SUCCESS;
     return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
 }

@@ -44,6 +44,7 @@ typedef struct HgThread {
     void* stream;     /* hipStream_t */
     uint32_t notify_num;
     void** notifies;  /* hipEvent_t per slot */
+    uint64_t* notify_pending; /* per slot: records issued that no wait has consumed yet (atomics: recorded by other threads) */
     /* operations recorded in batch mode, in call order */
     HgOp* pending;
     uint32_t pending_n, pending_cap;

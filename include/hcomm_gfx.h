@@ -153,7 +153,11 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
 /*
  * Cross-thread ordering.  Replaces include/hcomm_primitives.h:181,191.  Record marks, on dstThread's
  * notify slot dstNotifyIdx, the point `thread` has reached; Wait makes `thread` wait for the most recent
- * record on its own slot notifyIdx.  timeOut is accepted and ignored (stream-order wait).
+ * record on its own slot notifyIdx.  A notify is a HIP event, so the Record has to be ISSUED (host order) before
+ * the Wait that consumes it: a Wait that finds no unconsumed Record on its slot queues nothing and returns
+ * HCCL_E_TIMEOUT at once - the reference's wait would sit until timeOut ran out - and the timeOut value itself is
+ * not used.  Every Record is consumed by one Wait.  Neither call is available inside batch mode
+ * (HCCL_E_NOT_SUPPORT).
  */
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);

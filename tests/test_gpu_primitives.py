@@ -224,9 +224,11 @@ def test_notify_orders_two_threads(gpu_thread):
         x, y = gen(oracle.I32, count, 1), gen(oracle.I32, count, 2)
         d_x, d_y, d_t = to_dev(x), to_dev(y), to_dev(np.zeros_like(x))
         h.HcommGfxThreadSynchronize(gpu_thread)
+        assert h.HcommThreadNotifyWaitOnThread(tb, 0, 10) == h.HcclResult.E_TIMEOUT   # no record issued yet
         assert h.HcommLocalCopyOnThread(gpu_thread, d_t.data_ptr(), d_x.data_ptr(), count * 4) == 0
         assert h.HcommThreadNotifyRecordOnThread(gpu_thread, tb, 0) == 0
         assert h.HcommThreadNotifyWaitOnThread(tb, 0, 10) == 0
+        assert h.HcommThreadNotifyWaitOnThread(tb, 0, 10) == h.HcclResult.E_TIMEOUT   # that record is consumed
         assert h.HcommLocalReduceOnThread(tb, d_y.data_ptr(), d_t.data_ptr(), count, oracle.I32, oracle.SUM) == 0
         assert h.HcommGfxThreadSynchronize(tb) == 0
         assert_same(from_dev(d_y, y), (x + y), oracle.I32)

@@ -117,9 +117,33 @@ def test_thread_and_memory_argument_checks():
 def test_notify_argument_checks(rec):
     assert h.HcommThreadNotifyRecordOnThread(0, rec, 0) == R.E_PTR
     assert h.HcommThreadNotifyRecordOnThread(rec, 0, 0) == R.E_PTR
-    assert h.HcommThreadNotifyRecordOnThread(rec, rec, 0) == R.E_PARA   # recorder threads own no notifies
+    assert h.HcommThreadNotifyRecordOnThread(rec, rec, 2) == R.E_PARA   # a recorder thread has two notify slots
     assert h.HcommThreadNotifyWaitOnThread(0, 0, 1) == R.E_PTR
-    assert h.HcommThreadNotifyWaitOnThread(rec, 0, 1) == R.E_PARA
+    assert h.HcommThreadNotifyWaitOnThread(rec, 2, 1) == R.E_PARA
+
+
+def test_notify_wait_needs_a_record_issued_before_it(rec):
+    """A notify is an event on a stream: a wait can only follow a record that has been issued.  The wait that finds
+    none is the one the reference would time out on (include/hcomm_primitives.h:191): HCCL_E_TIMEOUT, at once."""
+    code, other = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    try:
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.E_TIMEOUT            # nothing recorded yet
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 0) == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 1, 10) == R.E_TIMEOUT            # the record went to slot 0
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.E_TIMEOUT            # one record, one wait
+        for _ in range(3):
+            assert h.HcommThreadNotifyRecordOnThread(other, rec, 1) == R.SUCCESS
+        for _ in range(3):
+            assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 1) == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 1) == R.E_TIMEOUT
+        assert h.HcommBatchModeStart(b"b") == R.SUCCESS                              # not inside a batch
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 0) == R.E_NOT_SUPPORT
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.E_NOT_SUPPORT
+        assert h.HcommBatchModeEnd(b"b") == R.SUCCESS
+    finally:
+        h.HcommThreadFree([other])
 
 
 def test_timeouts_fences_and_non_blocking_twins(rec):
@@ -130,7 +154,7 @@ def test_timeouts_fences_and_non_blocking_twins(rec):
     assert h.HcommSetNotifyWaitTimeOut(5e9) == R.E_PARA
     assert h.HcommSetNotifyWaitTimeOut(30.5) == R.SUCCESS
     assert h.HcommThreadResAcquireTimeOut(1.0) == R.E_NOT_SUPPORT
-    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 0) == R.E_PARA       # the recorder has no notifies
+    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 2) == R.E_PARA       # the recorder has two notify slots
     assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(12345, 0) == R.E_PTR
     assert h.HcommFenceOnThread(rec) == R.SUCCESS and h.HcommFenceOnThread(12345) == R.E_PTR
     assert h.HcommChannelFenceOnThread(rec, CH) == R.SUCCESS and h.HcommChannelFenceOnThread(rec, 0) == R.E_PTR
