@@ -13,7 +13,7 @@
         profiles/traffic.json under "<workload>|<lowering>" (bench.py reads it for roofline.traffic).  Both counters
         are scaled by what they read for k_copy in the same runs, whose launches read and write a known size:
         fetch_scale = WRITE_SIZE(k_copy) / FETCH_SIZE(k_copy) (a copy reads what it writes, and WRITE_SIZE counts
-        the bytes written one for one), write_scale = 1.
+        the bytes written one for one; 2.0 when the runs hold no k_copy), write_scale = 1.
 """
 import collections
 import csv
@@ -64,10 +64,14 @@ def main(argv):
     elif len(argv) >= 6 and argv[0] == "traffic":
         workload, lowering, sub, fdir, wdir = argv[1:6]
         fetch, write = counters(fdir), counters(wdir)
-        copy_fetch, copy_write = _mean_of(fetch, "k_copy", "FETCH_SIZE"), _mean_of(write, "k_copy", "WRITE_SIZE")
+        if any("k_copy" in k[0] for k in fetch):
+            scale = round(_mean_of(write, "k_copy", "WRITE_SIZE") / _mean_of(fetch, "k_copy", "FETCH_SIZE"), 4)
+            scale_from = "k_copy in the same runs"
+        else:  # a workload without copies: the factor every run that has k_copy gives (2.000 +- 0.002)
+            scale, scale_from = 2.0, "no k_copy in these runs: the factor of the runs that have one"
         entry = {"kernel": sub, "fetch_kib": round(_mean_of(fetch, sub, "FETCH_SIZE"), 1),
                  "write_kib": round(_mean_of(write, sub, "WRITE_SIZE"), 1),
-                 "fetch_scale": round(copy_write / copy_fetch, 4), "write_scale": 1.0,
+                 "fetch_scale": scale, "fetch_scale_from": scale_from, "write_scale": 1.0,
                  "source": argv[6] if len(argv) > 6 else ""}
         path = os.path.join(ROOT, "profiles", "traffic.json")
         try:
