@@ -39,7 +39,9 @@ __all__ = [
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libhcomm_gfx.so")
+# HCOMM_GFX_LIB names another build of the library to bind (a debug build, a build with other compile-time settings)
+LIB_PATH = os.environ.get("HCOMM_GFX_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
+                                                            "libhcomm_gfx.so")
 if not os.path.exists(LIB_PATH):
     raise ImportError(
         "libhcomm_gfx.so is not built (%s); run `python -c 'import __graft_entry__ as g; g.build()'` or "
