@@ -133,6 +133,9 @@ void hg_finish_seg2(HgLaunch* l)
         bytes += t->bytes[s];
     }
     t->tile_begin[t->nseg] = (uint32_t)tiles;
+    t->flat = 1u;
+    for (uint32_t s = 0; s < t->nseg; ++s)
+        if (t->tile_begin[s] != s || t->tile_begin[s + 1] != s + 1u) t->flat = 0u;
     l->nseg = t->nseg;
     l->bytes = bytes;
     l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
@@ -165,6 +168,9 @@ void hg_finish_fold(HgLaunch* l)
         bytes += t->bytes[s];
     }
     t->tile_begin[t->nseg] = (uint32_t)tiles;
+    t->flat = 1u;
+    for (uint32_t s = 0; s < t->nseg; ++s)
+        if (t->tile_begin[s] != s || t->tile_begin[s + 1] != s + 1u) t->flat = 0u;
     l->nseg = t->nseg;
     l->bytes = bytes;
     uint64_t per = t->k; /* reads */

@@ -166,7 +166,8 @@ __device__ __forceinline__ uint32_t block_id(uint32_t run)
 }
 
 // segment that owns a tile: the last s with tile_begin[s] <= tile (uniform across the workgroup, so the bisection
-// runs on the scalar unit: at most 6 probes for the largest table)
+// runs on the scalar unit: at most 6 probes for the largest table).  Every probe is a scalar load that waits for the
+// one before it, so launches whose segments are one tile each (small messages) say so and skip the search.
 __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_t nseg, uint32_t tile)
 {
     uint32_t lo = 0, hi = nseg; // tile_begin[lo] <= tile < tile_begin[hi]
@@ -176,6 +177,11 @@ __device__ __forceinline__ uint32_t find_seg(const uint32_t* tile_begin, uint32_
         else hi = mid;
     }
     return lo;
+}
+
+template <class Table> __device__ __forceinline__ uint32_t seg_of(const Table& tab, uint32_t tile)
+{
+    return tab.flat ? tile : find_seg(tab.tile_begin, tab.nseg, tile);
 }
 
 template <int DT, int OP> struct VecItem {

@@ -39,6 +39,7 @@ typedef struct {
     uint32_t tile_begin[HG_MAX_SEG2 + 1]; /* prefix sum of tiles per segment */
     uint32_t nseg;
     uint32_t xcd_run; /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
+    uint32_t flat;    /* every segment is exactly one tile: tile t belongs to segment t, no search (small messages) */
 } HgSeg2Table;
 
 /*
@@ -76,6 +77,7 @@ typedef struct {
     uint32_t keep_inputs;    /* tree modes 1 - 3: the partials the step-wise replay leaves in the inputs are not stored */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
     uint32_t xcd_run;        /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
+    uint32_t flat;           /* every segment is exactly one tile: tile t belongs to segment t, no search */
     uint8_t first[HG_MAX_SEG];
     uint8_t owner[HG_MAX_SEG];
     uint8_t start[HG_MAX_SEG]; /* chain with ascending == 2 only */

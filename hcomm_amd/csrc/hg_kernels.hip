@@ -19,7 +19,7 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
@@ -53,7 +53,7 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
@@ -104,7 +104,7 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t bytes = tab.bytes[s];
         uint8_t* d0 = (uint8_t*)tab.dst[s];
         const uint8_t* p0 = (const uint8_t*)tab.src[s];

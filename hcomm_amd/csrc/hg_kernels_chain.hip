@@ -98,7 +98,7 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;

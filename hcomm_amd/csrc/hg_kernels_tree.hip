@@ -155,6 +155,64 @@ __device__ __forceinline__ void fold_tree_items_rot(const HgFoldTable& tab, uint
     }
 }
 
+// Per-segment trees (tree == 6) of depth 6: 64 leaf positions are more than a lane holds at once, so the two halves of
+// 32 positions are loaded and folded one after the other - levels 0 .. 4 inside a half are the fixed pattern above -
+// and the last level folds the second half's root onto the first's.
+template <class Item> __device__ __forceinline__ void fold_tree_items_deep(const HgFoldTable& tab, uint32_t s, bool live, uint64_t idx)
+{
+    typedef typename Item::V V;
+    constexpr uint32_t H = 32u;
+    const uint64_t off = tab.off[s];
+    const uint32_t n = tab.nranks;
+    V root[2];
+    bool have_root[2];
+#pragma unroll
+    for (uint32_t half = 0; half < 2u; ++half) {
+        V x[H];
+        bool have[H];
+#pragma unroll
+        for (uint32_t q = 0; q < H; ++q) {
+            const uint32_t b = tab.pos[s * 2u * H + half * H + q];
+            have[q] = b < n;
+            x[q] = Item::zero();
+            if (have[q] && live) x[q] = Item::ld((const uint8_t*)tab.in[b] + off, idx);
+        }
+#pragma unroll
+        for (int l = 0; l < 5; ++l) {
+#pragma unroll
+            for (uint32_t q = 0; q < H; q += (2u << l))
+                if (have[q + (1u << l)]) x[q] = Item::op(x[q], x[q + (1u << l)]);
+        }
+        root[half] = x[0];
+        have_root[half] = have[0];
+    }
+    const V r = have_root[1] ? Item::op(root[0], root[1]) : root[0];
+    if (!live) return;
+    if (tab.out_mode == 1u) {
+        Item::st((uint8_t*)tab.out[tab.owner[s]] + tab.out_off[s], idx, r);
+    } else {
+        for (uint32_t q = 0; q < tab.nout; ++q) Item::st((uint8_t*)tab.out[q] + off, idx, r);
+    }
+}
+
+template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree_deep(const HgFoldTable tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    const uint32_t total = tab.tile_begin[tab.nseg];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
+        const uint32_t s = seg_of(tab, tile);
+        const uint64_t v = (uint64_t)(tile - tab.tile_begin[s]) * HG_BLOCK + tid;
+        const uint64_t bytes = tab.bytes[s];
+        const uint64_t nvec = bytes >> 4;
+        fold_tree_items_deep<VecItem<DT, OP>>(tab, s, v < nvec, v);
+        if (v - tid + HG_BLOCK > nvec) { // the segment's last tile also owns its element tail
+            const uint64_t e = (nvec << 4) / ES + tid;
+            fold_tree_items_deep<ElemItem<DT, OP>>(tab, s, (e + 1) * ES <= bytes, e);
+        }
+    }
+}
+
 // A lane handles HG_TREE_NU(K) vectors: two while the 2 x K values fit comfortably in registers (K <= 8), else one.
 template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
 {
@@ -163,7 +221,7 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
-        const uint32_t s = find_seg(tab.tile_begin, tab.nseg, tile);
+        const uint32_t s = seg_of(tab, tile);
         const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * NU) + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
@@ -197,9 +255,23 @@ template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFo
     return rc(hipGetLastError());
 }
 
+template <int DT> int launch_tree_deep_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
+{
+    if (tab->tree != 6u) return HCCL_E_PARA; /* the only mode whose trees are laid out over 64 positions */
+    switch (op) {
+        case OP_SUM: hipLaunchKernelGGL((k_fold_tree_deep<DT, OP_SUM>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_tree_deep<DT, OP_PROD>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_tree_deep<DT, OP_MAX>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_tree_deep<DT, OP_MIN>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        default: return HCCL_E_PARA;
+    }
+    return rc(hipGetLastError());
+}
+
 template <int DT> int launch_tree_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     switch (tab->k) {
+        case 64: return launch_tree_deep_dt<DT>(st, op, tab, blocks, lds);
         case 2: return launch_tree_dt_l<DT, 1>(st, op, tab, blocks, lds);
         case 4: return launch_tree_dt_l<DT, 2>(st, op, tab, blocks, lds);
         case 8: return launch_tree_dt_l<DT, 3>(st, op, tab, blocks, lds);

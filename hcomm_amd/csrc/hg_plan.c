@@ -510,7 +510,7 @@ typedef struct {
     uint64_t off;
 } SymNode;
 
-#define HG_TREE_MAX_DEPTH 5u /* the tree kernel folds 32 = 2^5 leaf positions at most */
+#define HG_TREE_MAX_DEPTH 6u /* per-segment trees span 64 = 2^6 leaf positions at most (two halves of 32, one after the other) */
 
 typedef struct {
     SymCell* cell;

@@ -61,8 +61,8 @@ def plan_segments(plan, rank_of):
     return out
 
 
-@pytest.mark.parametrize("n", [2, 4, 8, 16])
-@pytest.mark.parametrize("count,dtype", [(1 << 20, oracle.F32), (300007 * 16, oracle.BF16), (16 * 8192 + 40, oracle.I8)])
+@pytest.mark.parametrize("n", [2, 3, 4, 8, 16, 32])
+@pytest.mark.parametrize("count,dtype", [(1 << 20, oracle.F32), (300007 * 16, oracle.BF16), (32 * 16384 + 40, oracle.I8)])
 def test_deterministic_mesh_allreduce_single_launch_trees_equal_the_replay(n, count, dtype):
     ins, outs, rank_of = ptrs(n)
     plan = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, count, dtype, oracle.SUM)
@@ -94,9 +94,10 @@ def test_deterministic_mesh_allreduce_single_launch_trees_hand_derived():
 
 def test_deterministic_mesh_allreduce_single_launch_limits():
     ins, outs, _ = ptrs(32)
-    with pytest.raises(h.HcommError) as e:                       # depth 6: more leaf positions than the kernel folds
-        h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 1 << 22, oracle.F32, oracle.SUM)
-    assert e.value.code == R.E_NOT_SUPPORT
+    # 32 ranks: trees of depth 6 over 64 leaf positions, four segments' tables per launch, so 8 launches for 32 slices
+    p = h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 1 << 22, oracle.F32, oracle.SUM)
+    assert [(r.kind, r.nseg) for r in p.launches()] == [(h.Kernel.TREE, 4)] * 8
+    p.destroy()
     ins, outs, _ = ptrs(4)
     with pytest.raises(h.HcommError) as e:                       # slots of 10 bytes: slices off 16-byte boundaries
         h.Plan(h.Alg.ALLREDUCE_LOCAL_REDUCE, h.Lowering.FUSED, ins, outs, 38, oracle.I8, oracle.SUM)

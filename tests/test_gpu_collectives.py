@@ -237,6 +237,7 @@ USER_BUFFER_FUSED = [
     ("local_reduce", 16, 1 << 20, "bf16", "sum"), ("local_reduce", 8, 8 * 8192 + 24, "int16", "sum"),
     ("local_reduce", 1, 100, "fp32", "sum"), ("local_reduce", 4, 0, "fp32", "sum"),
     ("local_reduce", 3, 100003, "fp32", "sum"), ("local_reduce", 3, 3 * 8192 + 8, "fp16", "min"),
+    ("local_reduce", 32, 1 << 20, "bf16", "sum"), ("local_reduce", 32, 32 * 4096 + 100, "fp32", "max"),  # trees of depth 6
     ("window_rs", 8, 1 << 20, "bf16", "sum"), ("window_rs", 7, 100004, "fp32", "sum"), ("window_rs", 6, 16384, "fp16", "max"),
     ("window_rs", 5, 70016, "int8", "sum"), ("window_rs", 3, 1000, "int16", "sum"), ("window_rs", 2, 8, "fp32", "prod"),
     ("window_rs", 1, 100, "fp32", "sum"), ("window_rs", 12, 4104, "fp16", "sum"), ("window_rs", 31, 4096, "bf16", "max"),
@@ -273,6 +274,8 @@ def test_fused_lowerings_on_the_user_buffers(gpu_thread, alg, n, count, dtype, o
                 assert plan.info.movedBytes == (n + 1) * n * count * unit
         elif n > 1:
             per_launch = 32 // (n - 1) if alg == "chunk_mesh" else 8   # segments a launch's tables hold
+            if alg == "local_reduce" and n > 16:
+                per_launch = 4                                         # trees over 64 leaf positions: 256 table bytes / 64
             assert plan.info.launches <= -(-n // per_launch)
             assert plan.info.movedBytes == 2 * n * count * unit
         for rec in plan.launches():
