@@ -17,6 +17,8 @@ extern "C" {
 #define HG_POS_BYTES 256u      /* leaf-position bytes of a tree launch */
 #define HG_MAX_SEG 32u          /* segments per k-way fold launch */
 #define HG_MAX_SEG2 64u         /* segments per copy / two-input reduce launch */
+#define HG_DIRECT_SEG 8u        /* segments of a chain launch with host-resolved addresses */
+#define HG_DIRECT_K 8u          /* inputs per segment of such a launch */
 #define HG_VEC_BYTES 16u        /* one lane moves 128 bits per access */
 #ifndef HG_BLOCK
 #define HG_BLOCK 256u           /* threads per workgroup = 4 wavefronts of 64 */
@@ -40,6 +42,7 @@ typedef struct {
     uint32_t nseg;
     uint32_t xcd_run; /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
     uint32_t flat;    /* every segment is exactly one tile: tile t belongs to segment t, no search (small messages) */
+    uint32_t direct;  /* > 0: small launch on a two-dimensional grid, y = segment, x = tile of it, this many tiles wide */
 } HgSeg2Table;
 
 /*
@@ -76,6 +79,8 @@ typedef struct {
                               * the other ranks in cyclic order, entered at distance start[s] + 1 */
     uint32_t keep_inputs;    /* tree modes 1 - 3: the partials the step-wise replay leaves in the inputs are not stored */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
+    uint32_t direct;         /* small chain that only reads its inputs, <= HG_DIRECT_K of them in <= HG_DIRECT_SEG segments:
+                              * the launcher resolves every address on the host (one round of kernel-argument reads) */
     uint32_t xcd_run;        /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */
     uint32_t flat;           /* every segment is exactly one tile: tile t belongs to segment t, no search */
     uint8_t first[HG_MAX_SEG];

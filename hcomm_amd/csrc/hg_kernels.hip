@@ -140,12 +140,92 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
     }
 }
 
+// ---- small launches: one round of argument reads ---------------------------------------------------------
+//
+// A launch timed alone is a chain of dependent memory round trips of about a microsecond each: kernel arguments,
+// whatever they index, the data, the stores.  The kernels above find a tile's segment in the table's prefix sums
+// and only then know which pointers to read: two or more rounds of argument reads.  Launches of a few MiB are
+// better off with a two-dimensional grid, y = segment and x = tile of that segment (as wide as the longest
+// segment; workgroups beyond a shorter segment's tiles find nothing to do): every argument a workgroup needs
+// sits at an offset it knows from its own index, so all are read at once.  Same tiles, same arithmetic.
+
+__global__ __launch_bounds__(HG_BLOCK) void k_copy_direct(const HgSeg2Table tab)
+{
+    const uint32_t s = blockIdx.y, tid = threadIdx.x;
+    void* d = tab.dst[s];
+    const void* p = tab.src[s];
+    const uint64_t bytes = tab.bytes[s];
+    const uint64_t nvec = bytes >> 4;
+    const uint64_t v0 = (uint64_t)blockIdx.x * HG_TILE_VECS + tid;
+    if (v0 - tid + HG_TILE_VECS <= nvec) {
+        u32x4 a[HG_UNROLL];
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<false>(d, v0 + u * HG_BLOCK, a[u]);
+    } else {
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) {
+            const uint64_t v = v0 + u * HG_BLOCK;
+            if (v < nvec) stv<false>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+        }
+        if (blockIdx.x == nvec / HG_TILE_VECS) { // the tile the byte tail falls into
+            const uint64_t b = (nvec << 4) + tid;
+            if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
+        }
+    }
+}
+
+template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2_direct(const HgSeg2Table tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    const uint32_t s = blockIdx.y, tid = threadIdx.x;
+    void* d = tab.dst[s];
+    const void* p = tab.src[s];
+    const uint64_t bytes = tab.bytes[s];
+    const uint64_t nvec = bytes >> 4;
+    const uint64_t v0 = (uint64_t)blockIdx.x * HG_TILE_VECS + tid;
+    if (v0 - tid + HG_TILE_VECS <= nvec) {
+        u32x4 a[HG_UNROLL], b[HG_UNROLL];
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<false>(d, v0 + u * HG_BLOCK);
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<false>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+    } else {
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) {
+            const uint64_t v = v0 + u * HG_BLOCK;
+            if (v < nvec) stv<false>(d, v, vec_op<DT, OP>(ldv<false>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+        }
+        if (blockIdx.x == nvec / HG_TILE_VECS) { // the tile the element tail falls into
+            const uint64_t b = (nvec << 4) + (uint64_t)tid * ES;
+            if (b + ES <= bytes) {
+                uint8_t* de = (uint8_t*)d + b;
+                st_elem<ES>(de, word_op<DT, OP>(ld_elem<ES>(de), ld_elem<ES>((const uint8_t*)p + b)));
+            }
+        }
+    }
+}
+
 // ---- dispatch -----------------------------------------------------------------------------------
 
 template <int DT, bool STREAM>
 int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
+    if (tab->direct) {
+        const dim3 g2(tab->direct, tab->nseg);
+        switch (op) {
+            case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM>), g2, b, 0, st, *tab); break;
+            case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD>), g2, b, 0, st, *tab); break;
+            case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX>), g2, b, 0, st, *tab); break;
+            case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN>), g2, b, 0, st, *tab); break;
+            default: return HCCL_E_PARA;
+        }
+        return rc(hipGetLastError());
+    }
     switch (op) {
         case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM, STREAM>), g, b, lds, st, *tab); break;
         case OP_PROD: hipLaunchKernelGGL((k_reduce2<DT, OP_PROD, STREAM>), g, b, lds, st, *tab); break;
@@ -184,6 +264,10 @@ extern "C" {
 int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
+    if (tab->direct) {
+        hipLaunchKernelGGL(k_copy_direct, dim3(tab->direct, tab->nseg), dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
+        return rc(hipGetLastError());
+    }
     if (streaming)
         hipLaunchKernelGGL(k_copy<true>, dim3((uint32_t)blocks), dim3(HG_BLOCK), lds, (hipStream_t)stream, *tab);
     else

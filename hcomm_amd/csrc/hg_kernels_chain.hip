@@ -12,7 +12,7 @@ namespace {
 // Chain: acc = x0; for j = 1..k-1: acc = ACC_IS_DST ? acc (op) xj : xj (op) acc, optionally storing acc into
 // xj's buffer, which reproduces k-1 successive two-input reduces while reading every input once.
 
-__device__ __forceinline__ uint32_t fold_rank(const HgFoldTable& t, uint32_t s, uint32_t j)
+__host__ __device__ __forceinline__ uint32_t fold_rank(const HgFoldTable& t, uint32_t s, uint32_t j)
 {
     if (t.ascending == 1u) {
         if (j == 0) return t.first[s];
@@ -181,9 +181,110 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_small(const HgFoldTable
     }
 }
 
+// ---- k-way chain fold, small messages, addresses resolved by the host ---------------------------------
+//
+// A launch timed alone is a chain of dependent memory round trips: kernel arguments, then whatever they index,
+// then the data, then the stores.  k_fold_chain_small spends three rounds on arguments (the table's scalars, the
+// segment's row, the rank pointers that row selects).  For the common small case (a read-only chain of at most
+// HG_DIRECT_K inputs, at most HG_DIRECT_SEG segments) the launcher resolves every address on the host and the grid
+// is two-dimensional, y = segment, so that everything a workgroup needs sits at an offset it knows from its own
+// index: one round of argument reads.  Same arithmetic, same order, same bits.
+
+struct HgDirectTable {
+    const uint8_t* in[HG_DIRECT_SEG][HG_DIRECT_K]; // position j of segment s
+    uint8_t* out[HG_DIRECT_SEG][HG_DIRECT_K];      // receivers of segment s's result
+    uint32_t bytes[HG_DIRECT_SEG];
+    uint32_t k, nout;
+};
+
+// Positions beyond k repeat position 0's address (a load that is always valid) and are left out of the fold by a
+// select, receivers beyond nout are skipped: no branch sits between the loads, so all of them are in flight at once.
+template <class Item, bool ACC_IS_DST>
+__device__ __forceinline__ void fold_direct(const uint8_t* const (&in)[HG_DIRECT_K], uint8_t* const (&out)[HG_DIRECT_K],
+                                            uint32_t k, uint32_t nout, uint32_t idx)
+{
+    typedef typename Item::V V;
+    V buf[HG_DIRECT_K];
+#pragma unroll
+    for (uint32_t j = 0; j < HG_DIRECT_K; ++j) buf[j] = Item::ld(in[j], idx);
+    V acc = buf[0];
+#pragma unroll
+    for (uint32_t j = 1; j < HG_DIRECT_K; ++j) {
+        const V f = ACC_IS_DST ? Item::op(acc, buf[j]) : Item::op(buf[j], acc);
+        acc = (j < k) ? f : acc;
+    }
+#pragma unroll
+    for (uint32_t r = 0; r < HG_DIRECT_K; ++r)
+        if (r < nout) Item::st(out[r], idx, acc);
+}
+
+template <int DT, int OP, bool ACC_IS_DST>
+__global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_direct(const HgDirectTable tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    const uint32_t s = blockIdx.y, tid = threadIdx.x;
+    // every argument this workgroup needs, read before anything depends on any of them
+    const uint8_t* in[HG_DIRECT_K];
+    uint8_t* out[HG_DIRECT_K];
+#pragma unroll
+    for (uint32_t j = 0; j < HG_DIRECT_K; ++j) {
+        in[j] = tab.in[s][j];
+        out[j] = tab.out[s][j];
+    }
+    const uint32_t bytes = tab.bytes[s], k = tab.k, nout = tab.nout;
+    const uint32_t tiles = (bytes + (uint32_t)HG_TREE_TILE_BYTES - 1u) / (uint32_t)HG_TREE_TILE_BYTES;
+    const uint32_t nvec = bytes >> 4;
+    const uint32_t v = blockIdx.x * HG_BLOCK + tid;
+    // the grid is as wide as the longest segment: workgroups beyond this segment's tiles pass both tests untaken
+    if (v < nvec) fold_direct<VecItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, v);
+    if (blockIdx.x + 1u == tiles) { // the segment's last tile also owns its element tail
+        const uint32_t e = (nvec << 4) / ES + tid;
+        if ((e + 1u) * ES <= bytes) fold_direct<ElemItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, e);
+    }
+}
+
+// whether a small chain launch can take the direct kernel, and its table if so
+bool direct_table(const HgFoldTable& t, HgDirectTable* d, uint32_t* width)
+{
+    if (!t.direct || t.nseg == 0) return false;
+    *width = 0;
+    for (uint32_t s = 0; s < t.nseg; ++s) {
+        if (t.bytes[s] >= (1ull << 31)) return false;
+        const uint32_t tiles = t.tile_begin[s + 1] - t.tile_begin[s];
+        if (tiles > *width) *width = tiles;
+        d->bytes[s] = (uint32_t)t.bytes[s];
+        for (uint32_t j = 0; j < HG_DIRECT_K; ++j) {
+            d->in[s][j] = (const uint8_t*)t.in[fold_rank(t, s, j < t.k ? j : 0u)] + t.off[s];
+            d->out[s][j] = nullptr;
+        }
+        if (t.out_mode == 1u) {
+            d->out[s][0] = (uint8_t*)t.out[t.owner[s]] + t.out_off[s];
+        } else {
+            for (uint32_t r = 0; r < t.nranks; ++r) d->out[s][r] = (uint8_t*)t.out[r] + t.off[s];
+        }
+    }
+    for (uint32_t s = t.nseg; s < HG_DIRECT_SEG; ++s) d->bytes[s] = 0;
+    d->k = t.k;
+    d->nout = t.out_mode == 1u ? 1u : t.nranks;
+    return *width > 0;
+}
+
 template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
+    HgDirectTable direct;
+    uint32_t width = 0;
+    if (direct_table(*tab, &direct, &width)) {
+        const dim3 g2(width, tab->nseg);
+        switch (op) {
+            case OP_SUM: hipLaunchKernelGGL((k_fold_chain_direct<DT, OP_SUM, AD>), g2, b, 0, st, direct); break;
+            case OP_PROD: hipLaunchKernelGGL((k_fold_chain_direct<DT, OP_PROD, AD>), g2, b, 0, st, direct); break;
+            case OP_MAX: hipLaunchKernelGGL((k_fold_chain_direct<DT, OP_MAX, AD>), g2, b, 0, st, direct); break;
+            case OP_MIN: hipLaunchKernelGGL((k_fold_chain_direct<DT, OP_MIN, AD>), g2, b, 0, st, direct); break;
+            default: return HCCL_E_PARA;
+        }
+        return rc(hipGetLastError());
+    }
     if (tab->small) {
         switch (op) {
             case OP_SUM: hipLaunchKernelGGL((k_fold_chain_small<DT, OP_SUM, AD>), g, b, lds, st, *tab); break;
