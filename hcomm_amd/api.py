@@ -20,7 +20,7 @@ __all__ = [
     "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
     "HcommThreadNotifyWaitOnThread", "HcommMemAlloc", "HcommMemFree", "HcommBatchModeStart", "HcommBatchModeEnd",
     "HcommGfxThreadSynchronize", "HcommGfxReduceKOnThread", "HcommGfxRecorderThreadAlloc", "launch_log",
-    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion",
+    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion", "HcommGfxSetDirectLaunches",
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
@@ -271,6 +271,14 @@ def desc_reduce(dst, src, count, dtype, op, read=False):
     r = d.transferInfo.reduce
     r.count, r.dst, r.src, r.reduceOp, r.dataType = count, dst, src, op, dtype
     return d
+
+
+_set_direct = _sig("HcommGfxSetDirectLaunches", C.c_int32, C.c_int32)
+
+
+def HcommGfxSetDirectLaunches(enable):
+    """0: launches shaped from now on stay on the kernels large launches use; 1: the default.  Returns the previous setting."""
+    return int(_set_direct(1 if enable else 0))
 
 
 def HcommGfxVersion():

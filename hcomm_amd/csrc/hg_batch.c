@@ -19,6 +19,7 @@ static uint64_t g_grid_cap = 0; /* UINT64_MAX = not set */
 static uint64_t g_small_bytes = 0;
 static uint64_t g_direct_bytes = 0;
 static uint64_t g_direct_tiles = 0;
+static uint64_t g_direct_tree_bytes = 0;
 
 static uint64_t env_once(uint64_t* slot, const char* name, uint64_t unset)
 {
@@ -30,6 +31,28 @@ static uint64_t env_once(uint64_t* slot, const char* name, uint64_t unset)
         __atomic_store_n(slot, v, __ATOMIC_RELAXED);
     }
     return v;
+}
+
+/* Whether small launches take the kernels that read their arguments in one round (HcommGfxSetDirectLaunches;
+ * HCOMM_GFX_DIRECT=0 in the environment starts with them off). */
+static int g_direct_state = 0; /* 0 not read yet, 1 off, 2 on */
+
+static int direct_on(void)
+{
+    int v = __atomic_load_n(&g_direct_state, __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv("HCOMM_GFX_DIRECT");
+        v = (e && e[0] == '0') ? 1 : 2;
+        __atomic_store_n(&g_direct_state, v, __ATOMIC_RELAXED);
+    }
+    return v == 2;
+}
+
+int32_t HcommGfxSetDirectLaunches(int32_t enable)
+{
+    const int32_t before = direct_on();
+    __atomic_store_n(&g_direct_state, enable ? 2 : 1, __ATOMIC_RELAXED);
+    return before;
 }
 
 uint64_t hg_grid_blocks(uint64_t total_tiles)
@@ -141,7 +164,7 @@ void hg_finish_seg2(HgLaunch* l)
     /* small launches take a two-dimensional grid (one round of kernel-argument reads): at most this many tiles
      * (beyond that the argument reads no longer show) and no more than twice as many workgroups as tiles */
     t->direct = 0u;
-    if (tiles != 0 && tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u) && l->kind != HCOMM_GFX_KERNEL_BYTEWISE) {
+    if (direct_on() && tiles != 0 && tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u) && l->kind != HCOMM_GFX_KERNEL_BYTEWISE) {
         uint32_t w = 0;
         for (uint32_t s = 0; s < t->nseg; ++s) {
             const uint32_t n = t->tile_begin[s + 1] - t->tile_begin[s];
@@ -176,12 +199,19 @@ void hg_finish_fold(HgLaunch* l)
         /* a read-only chain of few inputs and segments runs with host-resolved addresses, which pays up to larger
          * sizes (8 ranks x 4 MiB, everything cache-resident: 32 us against 37.5) */
         const uint64_t direct_bytes = env_once(&g_direct_bytes, "HCOMM_GFX_DIRECT_BYTES", 8u << 20);
-        t->direct = (direct_bytes != 0 && largest <= direct_bytes && !t->store_partials && !t->store_final_first && t->nseg <= HG_DIRECT_SEG &&
+        t->direct = (direct_on() && largest <= direct_bytes && !t->store_partials && !t->store_final_first && t->nseg <= HG_DIRECT_SEG &&
                      t->k >= 1u && t->k <= HG_DIRECT_K &&
                      (t->out_mode == 1u || (t->out_mode == 2u && t->nranks <= HG_DIRECT_K)))
                         ? 1u
                         : 0u;
         if (t->direct) t->small = 1u;
+    } else {
+        /* small trees of up to 16 positions likewise (the launcher still checks what only it can see) */
+        const uint64_t direct_bytes = env_once(&g_direct_tree_bytes, "HCOMM_GFX_DIRECT_TREE_BYTES", 256u << 10);
+        uint64_t largest = 0;
+        for (uint32_t s = 0; s < t->nseg; ++s)
+            if (t->bytes[s] > largest) largest = t->bytes[s];
+        t->direct = (direct_on() && largest <= direct_bytes && t->nseg <= HG_DIRECT_SEG && t->k <= 16u) ? 1u : 0u;
     }
     const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {

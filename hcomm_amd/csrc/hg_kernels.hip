@@ -149,7 +149,26 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 // segment; workgroups beyond a shorter segment's tiles find nothing to do): every argument a workgroup needs
 // sits at an offset it knows from its own index, so all are read at once.  Same tiles, same arithmetic.
 
-__global__ __launch_bounds__(HG_BLOCK) void k_copy_direct(const HgSeg2Table tab)
+// Launches of at most HG_DIRECT_SEG segments pass this table instead of the full one: the runtime copies the kernel
+// arguments on every launch, and 192 bytes cost less there than 1.8 KB.
+struct HgSeg2Few {
+    void* dst[HG_DIRECT_SEG];
+    const void* src[HG_DIRECT_SEG];
+    uint64_t bytes[HG_DIRECT_SEG];
+};
+
+HgSeg2Few few_of(const HgSeg2Table& t)
+{
+    HgSeg2Few f;
+    for (uint32_t s = 0; s < HG_DIRECT_SEG; ++s) {
+        f.dst[s] = s < t.nseg ? t.dst[s] : nullptr;
+        f.src[s] = s < t.nseg ? t.src[s] : nullptr;
+        f.bytes[s] = s < t.nseg ? t.bytes[s] : 0;
+    }
+    return f;
+}
+
+template <class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_copy_direct(const Tab tab)
 {
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
     void* d = tab.dst[s];
@@ -176,7 +195,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_copy_direct(const HgSeg2Table tab)
     }
 }
 
-template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2_direct(const HgSeg2Table tab)
+template <int DT, int OP, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2_direct(const Tab tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
@@ -217,11 +236,22 @@ int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t
     const dim3 g(blocks), b(HG_BLOCK);
     if (tab->direct) {
         const dim3 g2(tab->direct, tab->nseg);
+        if (tab->nseg <= HG_DIRECT_SEG) {
+            const HgSeg2Few few = few_of(*tab);
+            switch (op) {
+                case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM, HgSeg2Few>), g2, b, 0, st, few); break;
+                case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD, HgSeg2Few>), g2, b, 0, st, few); break;
+                case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX, HgSeg2Few>), g2, b, 0, st, few); break;
+                case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN, HgSeg2Few>), g2, b, 0, st, few); break;
+                default: return HCCL_E_PARA;
+            }
+            return rc(hipGetLastError());
+        }
         switch (op) {
-            case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM>), g2, b, 0, st, *tab); break;
-            case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD>), g2, b, 0, st, *tab); break;
-            case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX>), g2, b, 0, st, *tab); break;
-            case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN>), g2, b, 0, st, *tab); break;
+            case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM, HgSeg2Table>), g2, b, 0, st, *tab); break;
+            case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD, HgSeg2Table>), g2, b, 0, st, *tab); break;
+            case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX, HgSeg2Table>), g2, b, 0, st, *tab); break;
+            case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN, HgSeg2Table>), g2, b, 0, st, *tab); break;
             default: return HCCL_E_PARA;
         }
         return rc(hipGetLastError());
@@ -265,7 +295,11 @@ int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int st
 {
     if (blocks == 0) return HCCL_SUCCESS;
     if (tab->direct) {
-        hipLaunchKernelGGL(k_copy_direct, dim3(tab->direct, tab->nseg), dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
+        const dim3 g2(tab->direct, tab->nseg);
+        if (tab->nseg <= HG_DIRECT_SEG)
+            hipLaunchKernelGGL(k_copy_direct<HgSeg2Few>, g2, dim3(HG_BLOCK), 0, (hipStream_t)stream, few_of(*tab));
+        else
+            hipLaunchKernelGGL(k_copy_direct<HgSeg2Table>, g2, dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
         return rc(hipGetLastError());
     }
     if (streaming)

@@ -12,7 +12,7 @@ namespace {
 // goes to every output.
 // A block rank with in2 != NULL first absorbs in2 (the odd neighbour folded in before the halving steps).
 
-template <int L> __device__ __forceinline__ constexpr uint32_t bitrev(uint32_t q)
+template <int L> __host__ __device__ __forceinline__ constexpr uint32_t bitrev(uint32_t q)
 {
     uint32_t r = 0;
     for (int i = 0; i < L; ++i) r |= ((q >> i) & 1u) << (L - 1 - i);
@@ -243,8 +243,153 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     }
 }
 
+// ---- small tree launches with host-resolved addresses --------------------------------------------------------
+//
+// The kernels above read their arguments in rounds that wait for one another (the table's scalars, the segment's
+// row, the leaf table, the rank pointers it selects), about a microsecond each, which is most of what a small
+// launch costs.  For trees of up to 16 positions in up to HG_DIRECT_SEG segments the launcher lays every leaf's
+// address out per segment and the grid is two-dimensional (y = segment, x = tile): one round of argument reads.
+// A hole carries position 0's address (a load that is always valid) and is left out of the fold by a select, so
+// that no branch sits between the loads.  Same tree, same operand roles, same bits.
+
+template <uint32_t K> struct HgTreeDirect {
+    const uint8_t* in[HG_DIRECT_SEG][K]; // leaf position q of segment s (position 0's address where q is a hole)
+    uint8_t* out[HG_DIRECT_SEG][K];      // receivers of segment s's root
+    uint32_t bytes[HG_DIRECT_SEG];
+    uint32_t have[HG_DIRECT_SEG];  // bit q: position q holds a leaf
+    uint32_t store[HG_DIRECT_SEG]; // bit q: position q's last value is stored back to its buffer
+    uint32_t nout;
+};
+
+template <class Item, int L>
+__device__ __forceinline__ void fold_tree_direct(const uint8_t* const (&in)[1u << L], uint8_t* const (&out)[1u << L], uint32_t have,
+                                                 uint32_t store, uint32_t nout, uint32_t idx)
+{
+    typedef typename Item::V V;
+    constexpr uint32_t K = 1u << L;
+    V x[K];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) x[q] = Item::ld(in[q], idx);
+#pragma unroll
+    for (int l = 0; l < L; ++l) {
+#pragma unroll
+        for (uint32_t q = 0; q < K; q += (2u << l)) {
+            const V f = Item::op(x[q], x[q + (1u << l)]);
+            x[q] = ((have >> (q + (1u << l))) & 1u) ? f : x[q];
+        }
+    }
+#pragma unroll
+    for (uint32_t q = 0; q < K; q += 2)
+        if ((store >> q) & 1u) Item::st((uint8_t*)in[q], idx, x[q]);
+#pragma unroll
+    for (uint32_t r = 0; r < K; ++r)
+        if (r < nout) Item::st(out[r], idx, x[0]);
+}
+
+template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree_direct(const HgTreeDirect<(1u << L)> tab)
+{
+    constexpr uint32_t ES = ElemSize<DT>::v;
+    constexpr uint32_t K = 1u << L;
+    const uint32_t s = blockIdx.y, tid = threadIdx.x;
+    // every argument this workgroup needs, read before anything depends on any of them
+    const uint8_t* in[K];
+    uint8_t* out[K];
+#pragma unroll
+    for (uint32_t q = 0; q < K; ++q) {
+        in[q] = tab.in[s][q];
+        out[q] = tab.out[s][q];
+    }
+    const uint32_t bytes = tab.bytes[s], have = tab.have[s], store = tab.store[s], nout = tab.nout;
+    const uint32_t nvec = bytes >> 4;
+    const uint32_t v = blockIdx.x * HG_BLOCK + tid;
+    // the grid is as wide as the longest segment: workgroups beyond this segment's tiles pass both tests untaken
+    if (v < nvec) fold_tree_direct<VecItem<DT, OP>, L>(in, out, have, store, nout, v);
+    if (blockIdx.x == nvec / HG_BLOCK) { // the tile the element tail falls into
+        const uint32_t e = (nvec << 4) / ES + tid;
+        if ((e + 1u) * ES <= bytes) fold_tree_direct<ElemItem<DT, OP>, L>(in, out, have, store, nout, e);
+    }
+}
+
+// The direct table of a tree launch, or false where the launch has something it does not carry (a neighbour
+// absorbed before the tree, more receivers than positions).  Mirrors fold_tree_items / fold_tree_items_rot.
+template <int L> bool tree_direct_table(const HgFoldTable& t, HgTreeDirect<(1u << L)>* d, uint32_t* width)
+{
+    constexpr uint32_t K = 1u << L;
+    const uint32_t n = t.nranks;
+    const bool order = t.tree >= 4u;
+    const uint32_t nout = (t.tree != 1u && t.out_mode == 1u) ? 1u : t.nout;
+    if (nout > K) return false;
+    *width = 0;
+    for (uint32_t s = 0; s < HG_DIRECT_SEG; ++s) {
+        d->bytes[s] = d->have[s] = d->store[s] = 0;
+        for (uint32_t q = 0; q < K; ++q) {
+            d->in[s][q] = nullptr;
+            d->out[s][q] = nullptr;
+        }
+    }
+    for (uint32_t s = 0; s < t.nseg; ++s) {
+        if (t.bytes[s] >= (1ull << 31)) return false;
+        const uint32_t c = t.first[s];
+        const uint64_t off = t.off[s];
+        for (uint32_t q = 0; q < K; ++q) {
+            uint32_t b;
+            bool have;
+            if (t.tree == 1u) {
+                b = c ^ bitrev<L>(q);
+                have = true;
+                if (b >= HCOMM_GFX_MAX_RANKS || t.in2[b]) return false;
+            } else if (order) {
+                b = t.pos[(t.tree == 6u ? s * K : 0u) + q];
+                have = b < n;
+                if (t.tree == 5u && have) {
+                    b = c + n - b;
+                    if (b >= n) b -= n;
+                }
+            } else {
+                b = (t.tree == 2u) ? c + q : c + n - q;
+                if (b >= n) b -= n;
+                have = q < n;
+            }
+            if (have) {
+                d->in[s][q] = (const uint8_t*)t.in[b] + off;
+                d->have[s] |= 1u << q;
+                const bool stored = t.tree == 1u ? !t.keep_inputs : (!order && !t.keep_inputs && q + 1u < n);
+                if ((q & 1u) == 0u && stored) d->store[s] |= 1u << q;
+            }
+        }
+        if (!(d->have[s] & 1u)) return false;
+        for (uint32_t q = 0; q < K; ++q)
+            if (!d->in[s][q]) d->in[s][q] = d->in[s][0];
+        if (t.tree != 1u && t.out_mode == 1u) {
+            d->out[s][0] = (uint8_t*)t.out[t.owner[s]] + t.out_off[s];
+        } else {
+            for (uint32_t r = 0; r < nout; ++r) d->out[s][r] = (uint8_t*)t.out[r] + off;
+        }
+        d->bytes[s] = (uint32_t)t.bytes[s];
+        const uint32_t tiles = (uint32_t)((t.bytes[s] + HG_TREE_TILE_BYTES - 1) / HG_TREE_TILE_BYTES);
+        if (tiles > *width) *width = tiles;
+    }
+    d->nout = nout;
+    return *width > 0;
+}
+
 template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
+    if constexpr (L <= 4) {
+        HgTreeDirect<(1u << L)> direct;
+        uint32_t width = 0;
+        if (tab->direct && tree_direct_table<L>(*tab, &direct, &width)) {
+            const dim3 g2(width, tab->nseg), b(HG_BLOCK);
+            switch (op) {
+                case OP_SUM: hipLaunchKernelGGL((k_fold_tree_direct<DT, OP_SUM, L>), g2, b, 0, st, direct); break;
+                case OP_PROD: hipLaunchKernelGGL((k_fold_tree_direct<DT, OP_PROD, L>), g2, b, 0, st, direct); break;
+                case OP_MAX: hipLaunchKernelGGL((k_fold_tree_direct<DT, OP_MAX, L>), g2, b, 0, st, direct); break;
+                case OP_MIN: hipLaunchKernelGGL((k_fold_tree_direct<DT, OP_MIN, L>), g2, b, 0, st, direct); break;
+                default: return HCCL_E_PARA;
+            }
+            return rc(hipGetLastError());
+        }
+    }
     switch (op) {
         case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
         case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;

@@ -939,6 +939,13 @@ int32_t HcommGfxOpBaseCheck(
     HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType,
     HcommGfxCheckReport* report);
 
+/* No reference counterpart.  Small launches (a few MiB; a fold of at most 16 inputs) run kernels of their own that
+ * read all their arguments at once: addresses resolved on the host, a two-dimensional grid (segment, tile).  Passing
+ * 0 keeps every launch shaped after this call (plans: at creation) on the kernels large launches use, which is how
+ * the tests run those kernels on small and ragged shapes; 1 restores the default.  Returns the previous setting.
+ * HCOMM_GFX_DIRECT=0 in the environment sets the initial value to 0. */
+int32_t HcommGfxSetDirectLaunches(int32_t enable);
+
 /* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */
 const char* HcommGfxVersion(void);
 

@@ -639,3 +639,14 @@ def test_no_alloc_allreduce_checks(rec):
     except h.HcommError as e:
         plan_code = e.code
     assert code3 == plan_code
+
+
+def test_direct_launch_switch_returns_the_previous_setting():
+    before = h.HcommGfxSetDirectLaunches(0)
+    try:
+        assert h.HcommGfxSetDirectLaunches(1) == 0
+        assert h.HcommGfxSetDirectLaunches(5) == 1   # any non-zero value means on
+        assert h.HcommGfxSetDirectLaunches(0) == 1
+    finally:
+        h.HcommGfxSetDirectLaunches(before)
+    assert h.HcommGfxSetDirectLaunches(before) == before
