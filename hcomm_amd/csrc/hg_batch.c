@@ -161,22 +161,34 @@ void hg_finish_seg2(HgLaunch* l)
     t->flat = 1u;
     for (uint32_t s = 0; s < t->nseg; ++s)
         if (t->tile_begin[s] != s || t->tile_begin[s + 1] != s + 1u) t->flat = 0u;
-    /* small launches take a two-dimensional grid (one round of kernel-argument reads): at most this many tiles
-     * (beyond that the argument reads no longer show) and no more than twice as many workgroups as tiles */
-    t->direct = 0u;
-    if (direct_on() && tiles != 0 && tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u) && l->kind != HCOMM_GFX_KERNEL_BYTEWISE) {
-        uint32_t w = 0;
-        for (uint32_t s = 0; s < t->nseg; ++s) {
-            const uint32_t n = t->tile_begin[s + 1] - t->tile_begin[s];
-            if (n > w) w = n;
-        }
-        if ((uint64_t)w * t->nseg <= 2u * tiles) t->direct = w;
-    }
     l->nseg = t->nseg;
     l->bytes = bytes;
     l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
     l->blocks = hg_grid_blocks(tiles);
     hg_shape_seg2(l, -1);
+    /* A two-dimensional grid (segment, tile of it: one round of kernel-argument reads instead of four or five) where
+     * that wastes few workgroups: segments of nearly equal length at any size (at most an eighth more workgroups than
+     * tiles), anything up to HCOMM_GFX_DIRECT_TILES tiles as long as the grid at most doubles.  Launches that small
+     * are latency-bound and take neither the occupancy bound nor the XCD runs. */
+    t->direct = 0u;
+    if (direct_on() && tiles != 0 && l->kind != HCOMM_GFX_KERNEL_BYTEWISE) {
+        const int small = tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u);
+        uint32_t w = 0;
+        for (uint32_t s = 0; s < t->nseg; ++s) {
+            const uint32_t n = t->tile_begin[s + 1] - t->tile_begin[s];
+            if (n > w) w = n;
+        }
+        const uint64_t grid = (uint64_t)w * t->nseg;
+        if (grid <= tiles + tiles / 8u || (small && grid <= 2u * tiles)) {
+            t->direct = w;
+            l->blocks = grid;
+        }
+        if (t->direct && small) {
+            l->streaming = 0;
+            l->lds_bytes = 0;
+            t->xcd_run = 0;
+        }
+    }
 }
 
 void hg_finish_fold(HgLaunch* l)

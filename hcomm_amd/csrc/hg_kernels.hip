@@ -140,21 +140,26 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
     }
 }
 
-// ---- small launches: one round of argument reads ---------------------------------------------------------
+// ---- launches whose segments are (nearly) equally long: one round of argument reads ----------------------------
 //
-// A launch timed alone is a chain of dependent memory round trips of about a microsecond each: kernel arguments,
+// A launch starts with a chain of dependent memory round trips of about a microsecond each: kernel arguments,
 // whatever they index, the data, the stores.  The kernels above find a tile's segment in the table's prefix sums
-// and only then know which pointers to read: two or more rounds of argument reads.  Launches of a few MiB are
-// better off with a two-dimensional grid, y = segment and x = tile of that segment (as wide as the longest
-// segment; workgroups beyond a shorter segment's tiles find nothing to do): every argument a workgroup needs
-// sits at an offset it knows from its own index, so all are read at once.  Same tiles, same arithmetic.
+// and only then know which pointers to read: several rounds of argument reads before the first byte of data is
+// asked for, paid by every launch of a schedule because a launch does not start before the one ahead of it has
+// ended.  When the segments have (nearly) the same number of tiles - the slices of one step of a ring, halving
+// or mesh schedule - the grid is two-dimensional instead, y = segment and x = tile of that segment (as wide as
+// the longest segment; workgroups beyond a shorter segment's tiles find nothing to do): every argument a
+// workgroup needs sits at an offset it knows from its own index, so all are read at once.  Same tiles, same
+// arithmetic, same cache hints; the XCD runs are walked inside a segment's row (the workgroups of a row whose x
+// is equal modulo 8 run on one XCD whatever the row's place in the grid).
 
 // Launches of at most HG_DIRECT_SEG segments pass this table instead of the full one: the runtime copies the kernel
-// arguments on every launch, and 192 bytes cost less there than 1.8 KB.
+// arguments on every launch, and 200 bytes cost less there than 1.8 KB (about a microsecond per launch).
 struct HgSeg2Few {
     void* dst[HG_DIRECT_SEG];
     const void* src[HG_DIRECT_SEG];
     uint64_t bytes[HG_DIRECT_SEG];
+    uint32_t xcd_run;
 };
 
 HgSeg2Few few_of(const HgSeg2Table& t)
@@ -165,60 +170,63 @@ HgSeg2Few few_of(const HgSeg2Table& t)
         f.src[s] = s < t.nseg ? t.src[s] : nullptr;
         f.bytes[s] = s < t.nseg ? t.bytes[s] : 0;
     }
+    f.xcd_run = t.xcd_run;
     return f;
 }
 
-template <class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_copy_direct(const Tab tab)
+template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_copy_rows(const Tab tab)
 {
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
     void* d = tab.dst[s];
     const void* p = tab.src[s];
     const uint64_t bytes = tab.bytes[s];
+    const uint32_t tile = block_id(tab.xcd_run);
     const uint64_t nvec = bytes >> 4;
-    const uint64_t v0 = (uint64_t)blockIdx.x * HG_TILE_VECS + tid;
+    const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {
         u32x4 a[HG_UNROLL];
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<false>(d, v0 + u * HG_BLOCK, a[u]);
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, a[u]);
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stv<false>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+            if (v < nvec) stv<STREAM>(d, v, ldv<HG_NT_LD_SRC>(p, v));
         }
-        if (blockIdx.x == nvec / HG_TILE_VECS) { // the tile the byte tail falls into
+        if (tile == nvec / HG_TILE_VECS) { // the tile the byte tail falls into
             const uint64_t b = (nvec << 4) + tid;
             if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
         }
     }
 }
 
-template <int DT, int OP, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2_direct(const Tab tab)
+template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_reduce2_rows(const Tab tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
     void* d = tab.dst[s];
     const void* p = tab.src[s];
     const uint64_t bytes = tab.bytes[s];
+    const uint32_t tile = block_id(tab.xcd_run);
     const uint64_t nvec = bytes >> 4;
-    const uint64_t v0 = (uint64_t)blockIdx.x * HG_TILE_VECS + tid;
+    const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {
         u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<false>(d, v0 + u * HG_BLOCK);
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<STREAM>(d, v0 + u * HG_BLOCK);
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<false>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stv<false>(d, v, vec_op<DT, OP>(ldv<false>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+            if (v < nvec) stv<STREAM>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
         }
-        if (blockIdx.x == nvec / HG_TILE_VECS) { // the tile the element tail falls into
+        if (tile == nvec / HG_TILE_VECS) { // the tile the element tail falls into
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES;
             if (b + ES <= bytes) {
                 uint8_t* de = (uint8_t*)d + b;
@@ -230,31 +238,28 @@ template <int DT, int OP, class Tab> __global__ __launch_bounds__(HG_BLOCK) void
 
 // ---- dispatch -----------------------------------------------------------------------------------
 
+template <int DT, bool STREAM, class Tab>
+int launch_reduce2_rows(hipStream_t st, int op, const Tab& tab, dim3 g, uint32_t lds)
+{
+    const dim3 b(HG_BLOCK);
+    switch (op) {
+        case OP_SUM: hipLaunchKernelGGL((k_reduce2_rows<DT, OP_SUM, STREAM, Tab>), g, b, lds, st, tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_reduce2_rows<DT, OP_PROD, STREAM, Tab>), g, b, lds, st, tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_reduce2_rows<DT, OP_MAX, STREAM, Tab>), g, b, lds, st, tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_reduce2_rows<DT, OP_MIN, STREAM, Tab>), g, b, lds, st, tab); break;
+        default: return HCCL_E_PARA;
+    }
+    return rc(hipGetLastError());
+}
+
 template <int DT, bool STREAM>
 int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
     if (tab->direct) {
         const dim3 g2(tab->direct, tab->nseg);
-        if (tab->nseg <= HG_DIRECT_SEG) {
-            const HgSeg2Few few = few_of(*tab);
-            switch (op) {
-                case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM, HgSeg2Few>), g2, b, 0, st, few); break;
-                case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD, HgSeg2Few>), g2, b, 0, st, few); break;
-                case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX, HgSeg2Few>), g2, b, 0, st, few); break;
-                case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN, HgSeg2Few>), g2, b, 0, st, few); break;
-                default: return HCCL_E_PARA;
-            }
-            return rc(hipGetLastError());
-        }
-        switch (op) {
-            case OP_SUM: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_SUM, HgSeg2Table>), g2, b, 0, st, *tab); break;
-            case OP_PROD: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_PROD, HgSeg2Table>), g2, b, 0, st, *tab); break;
-            case OP_MAX: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MAX, HgSeg2Table>), g2, b, 0, st, *tab); break;
-            case OP_MIN: hipLaunchKernelGGL((k_reduce2_direct<DT, OP_MIN, HgSeg2Table>), g2, b, 0, st, *tab); break;
-            default: return HCCL_E_PARA;
-        }
-        return rc(hipGetLastError());
+        if (tab->nseg <= HG_DIRECT_SEG) return launch_reduce2_rows<DT, STREAM, HgSeg2Few>(st, op, few_of(*tab), g2, lds);
+        return launch_reduce2_rows<DT, STREAM, HgSeg2Table>(st, op, *tab, g2, lds);
     }
     switch (op) {
         case OP_SUM: hipLaunchKernelGGL((k_reduce2<DT, OP_SUM, STREAM>), g, b, lds, st, *tab); break;
@@ -271,6 +276,21 @@ int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t b
 {
     if (streaming) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks, lds);
     return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks, lds);
+}
+
+template <bool STREAM> int launch_copy_s(hipStream_t st, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
+{
+    const dim3 b(HG_BLOCK);
+    if (tab->direct) {
+        const dim3 g2(tab->direct, tab->nseg);
+        if (tab->nseg <= HG_DIRECT_SEG)
+            hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Few>), g2, b, lds, st, few_of(*tab));
+        else
+            hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Table>), g2, b, lds, st, *tab);
+    } else {
+        hipLaunchKernelGGL(k_copy<STREAM>, dim3(blocks), b, lds, st, *tab);
+    }
+    return rc(hipGetLastError());
 }
 
 template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
@@ -294,19 +314,8 @@ extern "C" {
 int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-    if (tab->direct) {
-        const dim3 g2(tab->direct, tab->nseg);
-        if (tab->nseg <= HG_DIRECT_SEG)
-            hipLaunchKernelGGL(k_copy_direct<HgSeg2Few>, g2, dim3(HG_BLOCK), 0, (hipStream_t)stream, few_of(*tab));
-        else
-            hipLaunchKernelGGL(k_copy_direct<HgSeg2Table>, g2, dim3(HG_BLOCK), 0, (hipStream_t)stream, *tab);
-        return rc(hipGetLastError());
-    }
-    if (streaming)
-        hipLaunchKernelGGL(k_copy<true>, dim3((uint32_t)blocks), dim3(HG_BLOCK), lds, (hipStream_t)stream, *tab);
-    else
-        hipLaunchKernelGGL(k_copy<false>, dim3((uint32_t)blocks), dim3(HG_BLOCK), lds, (hipStream_t)stream, *tab);
-    return rc(hipGetLastError());
+    if (streaming) return launch_copy_s<true>((hipStream_t)stream, tab, (uint32_t)blocks, lds);
+    return launch_copy_s<false>((hipStream_t)stream, tab, (uint32_t)blocks, lds);
 }
 
 int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
