@@ -276,6 +276,16 @@ def run_workload(args, torch, h, dev, stream, thread):
                                 [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, scr_ptrs)
         return h.Plan(alg, low, in_ptrs, out_ptrs, count, dt, op, 0, scr_ptrs)
 
+    def kernel_name(rec):
+        """The kernel a launch record names, as the profiler shows it (template arguments as type and op names)."""
+        copy = rec.op == 255
+        if rec.kind == h.Kernel.BYTEWISE:
+            return "k_bytewise<copy>" if copy else "k_bytewise<%s,%s>" % (dtname, opname.upper())
+        base = kname[rec.kind]
+        if rec.rows:  # the variants that read every address in one round
+            base += "_rows" if rec.kind in (h.Kernel.COPY, h.Kernel.REDUCE2) else "_direct"
+        return base if copy else "%s<%s,%s>" % (base, dtname, opname.upper())
+
     lowerings = ["stepwise", "fused"] if args.lowering == "both" else [args.lowering]
     # a template on the rank buffers themselves also has the fused launches without their stores into the inputs
     plain_plan = not (hier_rs or dbrs or opfused or opsmall or opar or plant or ophrs or ophier or dbring or hier or opbase)
@@ -363,8 +373,7 @@ def run_workload(args, torch, h, dev, stream, thread):
             "launches": plan.info.launches,
             "algorithmic_bytes": plan.info.algorithmicBytes,
             "moved_bytes": plan.info.movedBytes,
-            "kernel": ("k_copy" if dom_kind == h.Kernel.COPY else "k_bytewise<copy>" if dom_is_copy
-                       else "%s<%s,%s>" % (kname[dom_kind], dtname, opname.upper())),
+            "kernel": kernel_name(launches[first]),
             "kernel_ms": dom_ms,
             "kernel_alg_bytes": dom_bytes,
             "kernel_gbs": dom_bytes / (dom_ms * 1e-3) / 1e9,
@@ -591,7 +600,8 @@ def run_workload(args, torch, h, dev, stream, thread):
 
 def no_reuse_leg(torch, h, dev, stream, thread, reps):
     """The two-input reduce on operands that nothing touched recently, through the reference's own primitive API:
-    one batch of HcommLocalReduceOnThread calls = one k_reduce2<bf16,SUM> launch, rotated over buffer sets so that a
+    one batch of HcommLocalReduceOnThread calls = one k_reduce2_rows<bf16,SUM> launch (equally long segments: the
+    two-dimensional grid), rotated over buffer sets so that a
     launch finds nothing of its operands in the 256 MB memory-side cache.
       ring_step_shape   8 segments of 16 MiB (the headline's launch: 128 MiB written, the variant whose output
                         the next launch is to find in that cache), 12 sets of 256 MiB -> 3 GiB between two uses
@@ -629,7 +639,7 @@ def no_reuse_leg(torch, h, dev, stream, thread, reps):
         stream.synchronize()
         ms = sum(a.elapsed_time(b) for a, b in ev) / reps
         alg = 3 * nseg * seg_bytes
-        out[key] = {"kernel": "k_reduce2<bf16,SUM>", "segments": nseg, "segment_bytes": seg_bytes, "buffer_sets": sets,
+        out[key] = {"kernel": "k_reduce2_rows<bf16,SUM>", "segments": nseg, "segment_bytes": seg_bytes, "buffer_sets": sets,
                     "kernel_ms": round(ms, 5), "algorithmic_bytes_per_launch": alg,
                     "achieved": round(alg / (ms * 1e-3) / 1e9, 2), "frac": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
         del bufs

@@ -92,7 +92,7 @@ class Kernel:
 
 class LaunchRecord(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("dtype", C.c_uint32), ("op", C.c_uint32), ("nseg", C.c_uint32),
-                ("bytes", C.c_uint64), ("blocks", C.c_uint64)]
+                ("bytes", C.c_uint64), ("blocks", C.c_uint64), ("rows", C.c_uint32), ("streaming", C.c_uint32)]
 
 
 class PlanInfo(C.Structure):

@@ -297,6 +297,8 @@ static void log_launch(HgThread* t, const HgLaunch* l)
     r->nseg = l->nseg;
     r->bytes = l->bytes;
     r->blocks = l->blocks;
+    r->rows = hg_launch_rows(l);
+    r->streaming = l->streaming;
 }
 
 void hg_log_only(HgThread* t, const HgLaunch* l) { log_launch(t, l); }

@@ -191,6 +191,14 @@ void hg_finish_seg2(HgLaunch* l)
     }
 }
 
+/* what HcommGfxLaunchRecord.rows reports */
+uint32_t hg_launch_rows(const HgLaunch* l)
+{
+    if (l->kind == HCOMM_GFX_KERNEL_COPY || l->kind == HCOMM_GFX_KERNEL_REDUCE2) return l->tab.seg2.direct;
+    if (l->kind == HCOMM_GFX_KERNEL_CHAIN || l->kind == HCOMM_GFX_KERNEL_TREE) return l->tab.fold.direct;
+    return 0;
+}
+
 void hg_finish_fold(HgLaunch* l)
 {
     HgFoldTable* t = &l->tab.fold;
@@ -209,8 +217,8 @@ void hg_finish_fold(HgLaunch* l)
         const uint64_t limit = t->store_partials ? small_bytes / 4 : small_bytes;
         t->small = (largest <= limit) ? 1u : 0u;
         /* a read-only chain of few inputs and segments runs with host-resolved addresses, which pays up to larger
-         * sizes (8 ranks x 4 MiB, everything cache-resident: 32 us against 37.5) */
-        const uint64_t direct_bytes = env_once(&g_direct_bytes, "HCOMM_GFX_DIRECT_BYTES", 8u << 20);
+         * sizes (8 ranks x 4 MiB, everything cache-resident: 31 us against 37; at 16 MiB it no longer does) */
+        const uint64_t direct_bytes = env_once(&g_direct_bytes, "HCOMM_GFX_DIRECT_BYTES", 4u << 20);
         t->direct = (direct_on() && largest <= direct_bytes && !t->store_partials && !t->store_final_first && t->nseg <= HG_DIRECT_SEG &&
                      t->k >= 1u && t->k <= HG_DIRECT_K &&
                      (t->out_mode == 1u || (t->out_mode == 2u && t->nranks <= HG_DIRECT_K)))
@@ -218,12 +226,12 @@ void hg_finish_fold(HgLaunch* l)
                         : 0u;
         if (t->direct) t->small = 1u;
     } else {
-        /* small trees of up to 16 positions likewise (the launcher still checks what only it can see) */
-        const uint64_t direct_bytes = env_once(&g_direct_tree_bytes, "HCOMM_GFX_DIRECT_TREE_BYTES", 256u << 10);
-        uint64_t largest = 0;
-        for (uint32_t s = 0; s < t->nseg; ++s)
-            if (t->bytes[s] > largest) largest = t->bytes[s];
-        t->direct = (direct_on() && largest <= direct_bytes && t->nseg <= HG_DIRECT_SEG && t->k <= 16u) ? 1u : 0u;
+        /* small trees of up to 16 positions likewise (the launcher still checks what only it can see): up to 4 MiB
+         * of output per launch (8 ranks: 16.6 us against 18.1 there, 72 against 68 at 16 MiB) */
+        const uint64_t direct_bytes = env_once(&g_direct_tree_bytes, "HCOMM_GFX_DIRECT_TREE_BYTES", 4u << 20);
+        uint64_t sum = 0;
+        for (uint32_t s = 0; s < t->nseg; ++s) sum += t->bytes[s];
+        t->direct = (direct_on() && sum <= direct_bytes && t->nseg <= HG_DIRECT_SEG && t->k <= 16u) ? 1u : 0u;
     }
     const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {

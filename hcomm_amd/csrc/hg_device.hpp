@@ -155,14 +155,22 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
 // Workgroups are dealt to the 8 XCDs round-robin by their index.  With run > 0 they are renumbered so that each XCD
 // walks runs of `run` consecutive tiles instead of every eighth tile; the workgroups beyond the last whole group of
 // 8 * run keep their numbers.  run == 0: as dealt.
-__device__ __forceinline__ uint32_t block_id(uint32_t run)
+__device__ __forceinline__ uint32_t block_id(uint32_t run, uint32_t g, uint32_t b)
 {
-    const uint32_t g = gridDim.x, b = blockIdx.x;
     if (run == 0u) return b;
     const uint32_t span = 8u * run;
     if (b >= g - g % span) return b;
     const uint32_t i = b >> 3;
     return (i / run) * span + (b & 7u) * run + i % run;
+}
+__device__ __forceinline__ uint32_t block_id(uint32_t run) { return block_id(run, gridDim.x, blockIdx.x); }
+
+// The point by which all the given scalar values must have arrived: the loads that fetch them (kernel arguments, the
+// grid size) are all issued before it and waited for once, instead of each where the compiler first needs its value.
+template <class A, class B, class C, class D, class E>
+__device__ __forceinline__ void arrive_together(A& a, B& b, C& c, D& d, E& e)
+{
+    asm volatile("" : "+s"(a), "+s"(b), "+s"(c), "+s"(d), "+s"(e));
 }
 
 // segment that owns a tile: the last s with tile_begin[s] <= tile (uniform across the workgroup, so the bisection

@@ -71,6 +71,7 @@ uint64_t hg_split_head(const HgOp* o); /* bytes before the 16-byte boundary both
 /* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment
  * pointers and sizes are set. */
 void hg_finish_seg2(HgLaunch* l);
+uint32_t hg_launch_rows(const HgLaunch* l);
 void hg_shape_seg2(HgLaunch* l, int streaming); /* streaming < 0: decided by the bytes the launch writes */
 void hg_finish_fold(HgLaunch* l);
 

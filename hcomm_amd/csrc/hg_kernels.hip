@@ -179,8 +179,10 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
     void* d = tab.dst[s];
     const void* p = tab.src[s];
-    const uint64_t bytes = tab.bytes[s];
-    const uint32_t tile = block_id(tab.xcd_run);
+    uint64_t bytes = tab.bytes[s];
+    uint32_t run = tab.xcd_run, width = gridDim.x;
+    arrive_together(d, p, bytes, run, width); // one round of argument reads
+    const uint32_t tile = block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
     const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {
@@ -208,8 +210,10 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
     const uint32_t s = blockIdx.y, tid = threadIdx.x;
     void* d = tab.dst[s];
     const void* p = tab.src[s];
-    const uint64_t bytes = tab.bytes[s];
-    const uint32_t tile = block_id(tab.xcd_run);
+    uint64_t bytes = tab.bytes[s];
+    uint32_t run = tab.xcd_run, width = gridDim.x;
+    arrive_together(d, p, bytes, run, width); // one round of argument reads
+    const uint32_t tile = block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
     const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {

@@ -1540,6 +1540,8 @@ int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaun
     rec->nseg = l->nseg;
     rec->bytes = l->bytes;
     rec->blocks = l->blocks;
+    rec->rows = hg_launch_rows(l);
+    rec->streaming = l->streaming;
     return HCCL_SUCCESS;
 }
 
