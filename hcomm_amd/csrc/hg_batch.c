@@ -216,12 +216,14 @@ void hg_finish_fold(HgLaunch* l)
          * quarter of that when every position also stores its partial (ring) */
         const uint64_t limit = t->store_partials ? small_bytes / 4 : small_bytes;
         t->small = (largest <= limit) ? 1u : 0u;
-        /* a read-only chain of few inputs and segments runs with host-resolved addresses, which pays up to larger
-         * sizes (8 ranks x 4 MiB, everything cache-resident: 31 us against 37; at 16 MiB it no longer does) */
+        /* a chain of few inputs and segments runs with host-resolved addresses, which pays up to larger sizes
+         * (read-only, 8 ranks x 4 MiB, everything cache-resident: 31 us against 37; at 16 MiB it no longer does; a
+         * sixteenth of that when every position also stores its partial: 8 ranks x 2 MiB 10 us against 14, while
+         * at 4 MiB on operands nothing touched recently the 16 KiB tiles are ahead again) */
         const uint64_t direct_bytes = env_once(&g_direct_bytes, "HCOMM_GFX_DIRECT_BYTES", 4u << 20);
-        t->direct = (direct_on() && largest <= direct_bytes && !t->store_partials && !t->store_final_first && t->nseg <= HG_DIRECT_SEG &&
-                     t->k >= 1u && t->k <= HG_DIRECT_K &&
-                     (t->out_mode == 1u || (t->out_mode == 2u && t->nranks <= HG_DIRECT_K)))
+        const uint64_t direct_limit = t->store_partials ? direct_bytes / 16 : direct_bytes;
+        t->direct = (direct_on() && largest <= direct_limit && t->nseg <= HG_DIRECT_SEG && t->k >= 1u && t->k <= HG_DIRECT_K &&
+                     (t->out_mode <= 1u || (t->out_mode == 2u && t->nranks <= HG_DIRECT_K)))
                         ? 1u
                         : 0u;
         if (t->direct) t->small = 1u;

@@ -195,13 +195,15 @@ struct HgDirectTable {
     uint8_t* out[HG_DIRECT_SEG][HG_DIRECT_K];      // receivers of segment s's result
     uint32_t bytes[HG_DIRECT_SEG];
     uint32_t k, nout;
+    uint32_t store; // bit j >= 1: the running value is stored to position j's buffer after fold step j; bit 0: the
+                    // final value is stored to position 0's buffer
 };
 
 // Positions beyond k repeat position 0's address (a load that is always valid) and are left out of the fold by a
 // select, receivers beyond nout are skipped: no branch sits between the loads, so all of them are in flight at once.
 template <class Item, bool ACC_IS_DST>
 __device__ __forceinline__ void fold_direct(const uint8_t* const (&in)[HG_DIRECT_K], uint8_t* const (&out)[HG_DIRECT_K],
-                                            uint32_t k, uint32_t nout, uint32_t idx)
+                                            uint32_t k, uint32_t nout, uint32_t store, uint32_t idx)
 {
     typedef typename Item::V V;
     V buf[HG_DIRECT_K];
@@ -212,7 +214,9 @@ __device__ __forceinline__ void fold_direct(const uint8_t* const (&in)[HG_DIRECT
     for (uint32_t j = 1; j < HG_DIRECT_K; ++j) {
         const V f = ACC_IS_DST ? Item::op(acc, buf[j]) : Item::op(buf[j], acc);
         acc = (j < k) ? f : acc;
+        if ((store >> j) & 1u) Item::st((uint8_t*)in[j], idx, acc); // set for positions below k only
     }
+    if (store & 1u) Item::st((uint8_t*)in[0], idx, acc);
 #pragma unroll
     for (uint32_t r = 0; r < HG_DIRECT_K; ++r)
         if (r < nout) Item::st(out[r], idx, acc);
@@ -231,22 +235,22 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_direct(const HgDirectTa
         in[j] = tab.in[s][j];
         out[j] = tab.out[s][j];
     }
-    const uint32_t bytes = tab.bytes[s], k = tab.k, nout = tab.nout;
+    const uint32_t bytes = tab.bytes[s], k = tab.k, nout = tab.nout, store = tab.store;
     const uint32_t tiles = (bytes + (uint32_t)HG_TREE_TILE_BYTES - 1u) / (uint32_t)HG_TREE_TILE_BYTES;
     const uint32_t nvec = bytes >> 4;
     const uint32_t v = blockIdx.x * HG_BLOCK + tid;
     // the grid is as wide as the longest segment: workgroups beyond this segment's tiles pass both tests untaken
-    if (v < nvec) fold_direct<VecItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, v);
+    if (v < nvec) fold_direct<VecItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, store, v);
     if (blockIdx.x + 1u == tiles) { // the segment's last tile also owns its element tail
         const uint32_t e = (nvec << 4) / ES + tid;
-        if ((e + 1u) * ES <= bytes) fold_direct<ElemItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, e);
+        if ((e + 1u) * ES <= bytes) fold_direct<ElemItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, store, e);
     }
 }
 
 // whether a small chain launch can take the direct kernel, and its table if so
 bool direct_table(const HgFoldTable& t, HgDirectTable* d, uint32_t* width)
 {
-    if (!t.direct || t.nseg == 0) return false;
+    if (!t.direct || t.nseg == 0 || t.nseg > HG_DIRECT_SEG || t.k == 0 || t.k > HG_DIRECT_K) return false;
     *width = 0;
     for (uint32_t s = 0; s < t.nseg; ++s) {
         if (t.bytes[s] >= (1ull << 31)) return false;
@@ -259,13 +263,15 @@ bool direct_table(const HgFoldTable& t, HgDirectTable* d, uint32_t* width)
         }
         if (t.out_mode == 1u) {
             d->out[s][0] = (uint8_t*)t.out[t.owner[s]] + t.out_off[s];
-        } else {
+        } else if (t.out_mode == 2u) {
+            if (t.nranks > HG_DIRECT_K) return false;
             for (uint32_t r = 0; r < t.nranks; ++r) d->out[s][r] = (uint8_t*)t.out[r] + t.off[s];
         }
     }
     for (uint32_t s = t.nseg; s < HG_DIRECT_SEG; ++s) d->bytes[s] = 0;
     d->k = t.k;
-    d->nout = t.out_mode == 1u ? 1u : t.nranks;
+    d->nout = t.out_mode == 0u ? 0u : t.out_mode == 1u ? 1u : t.nranks;
+    d->store = (t.store_partials ? ((1u << t.k) - 2u) : 0u) | (t.store_final_first ? 1u : 0u);
     return *width > 0;
 }
 
