@@ -235,7 +235,7 @@ void hg_finish_fold(HgLaunch* l)
         for (uint32_t s = 0; s < t->nseg; ++s) sum += t->bytes[s];
         t->direct = (direct_on() && sum <= direct_bytes && t->nseg <= HG_DIRECT_SEG && t->k <= 16u) ? 1u : 0u;
     }
-    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_TILE_BYTES);
+    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_CHAIN_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
         tiles += (t->bytes[s] + tile_bytes - 1) / tile_bytes;

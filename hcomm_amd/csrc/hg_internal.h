@@ -26,6 +26,11 @@ extern "C" {
 #ifndef HG_UNROLL
 #define HG_UNROLL 4u            /* 128-bit accesses in flight per lane and operand */
 #endif
+#ifndef HG_CHAIN_UNROLL
+#define HG_CHAIN_UNROLL 2u      /* the same for the k-way chain fold at bandwidth-bound sizes: 8 KiB tiles (with 8 - 23
+                                 * streams per lane the smaller tile is 4 - 5 % ahead of 16 KiB) */
+#endif
+#define HG_CHAIN_TILE_BYTES ((uint64_t)HG_BLOCK * HG_CHAIN_UNROLL * HG_VEC_BYTES)
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
 #define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree / small-message kernels: one access per lane and input */

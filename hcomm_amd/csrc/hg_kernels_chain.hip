@@ -99,18 +99,18 @@ template <int DT, int OP, bool ACC_IS_DST> __global__ __launch_bounds__(HG_BLOCK
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
-        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
+        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * (HG_BLOCK * HG_CHAIN_UNROLL) + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
-        bool live[HG_UNROLL];
-        uint64_t idx[HG_UNROLL];
-        const bool full = (v0 - tid + HG_TILE_VECS <= nvec);
+        bool live[HG_CHAIN_UNROLL];
+        uint64_t idx[HG_CHAIN_UNROLL];
+        const bool full = (v0 - tid + (HG_BLOCK * HG_CHAIN_UNROLL) <= nvec);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) {
+        for (uint32_t u = 0; u < HG_CHAIN_UNROLL; ++u) {
             idx[u] = v0 + u * HG_BLOCK;
             live[u] = full || idx[u] < nvec;
         }
-        fold_chain_items<VecItem<DT, OP>, ACC_IS_DST, HG_UNROLL>(tab, s, live, idx);
+        fold_chain_items<VecItem<DT, OP>, ACC_IS_DST, HG_CHAIN_UNROLL>(tab, s, live, idx);
         if (!full) { // element tail of the segment, handled by its last tile
             const uint64_t ti[1] = {(nvec << 4) / ES + tid};
             const bool tl[1] = {(ti[0] + 1) * ES <= bytes};

@@ -25,6 +25,13 @@
 //                  data=random|zeros     buffer contents (two bf16 per word near 1e-3 in magnitude, or all zero)
 //                  reps=10 warm=2 sets=1 timed launches, untimed ones, buffer sets rotated through by the launches
 //
+// kind=fold        the k-way chain fold of the single-launch lowerings: per segment 8 inputs in 8 separate buffers are
+//                  folded in sequence (bf16 SUM), the running value optionally stored back to every input but the
+//                  first (part=1, the partials a ring leaves behind), the result to nout outputs.
+//                  keys: nseg seg_mib u(2|4) block hs st lds xcd run skew reps warm sets, and
+//                  depth=1|2|3|7  positions whose loads are in flight ahead of the one being folded
+//                  part=0|1 nout=8
+//
 // kind=lat         one wavefront on XCD `xk` walks a chain of dependent 1 KiB loads (64 lanes x 16 bytes) over the
 //                  pieces p of a 4 GiB arena with p mod `mod` == `cls`, a piece being `gran` bytes (a power of two
 //                  >= 1024): the nanoseconds per load tell how far that class of addresses is from that XCD.
@@ -49,7 +56,7 @@ namespace {
         }                                                                                          \
     } while (0)
 
-enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6 };
+enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6, K_FOLD = 7 };
 
 struct ProbeTab {
     void* dst[64];
@@ -153,6 +160,71 @@ __global__ __launch_bounds__(1024) void k_probe(const ProbeTab t)
     }
 }
 
+// ---- kind=fold ----------------------------------------------------------------------------------------------
+
+struct FoldProbeTab {
+    uint8_t* in[8];  // input j of segment s at in[j] + s * seg_bytes
+    uint8_t* out[8]; // receiver r likewise
+    uint64_t seg_bytes;
+    uint32_t tiles_per_seg, nseg, nout, part, xcd, run;
+};
+
+template <uint32_t U, uint32_t DEPTH, bool HS, bool ST>
+__global__ __launch_bounds__(1024) void k_probe_fold(const FoldProbeTab t)
+{
+    extern __shared__ uint8_t lds_pad[];
+    constexpr uint32_t K = 8;
+    ProbeTab numbering; // only the fields probe_tile reads
+    numbering.xcd = t.xcd;
+    numbering.run = t.run;
+    const uint32_t tile = probe_tile(numbering, blockIdx.x, gridDim.x);
+    const uint32_t s = tile / t.tiles_per_seg;
+    const uint64_t v0 = (uint64_t)(tile - s * t.tiles_per_seg) * (blockDim.x * U) + threadIdx.x;
+    const uint64_t so = (uint64_t)s * t.seg_bytes;
+    u32x4 x[K][U];
+#pragma unroll
+    for (uint32_t j = 0; j <= DEPTH && j < K; ++j)
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) x[j][u] = ldv<HS>(t.in[j] + so, v0 + u * blockDim.x);
+    u32x4 acc[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) acc[u] = x[0][u];
+#pragma unroll
+    for (uint32_t j = 1; j < K; ++j) {
+        if (j + DEPTH < K) {
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) x[j + DEPTH][u] = ldv<HS>(t.in[j + DEPTH] + so, v0 + u * blockDim.x);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) acc[u] = vec_op<DT_BF16, OP_SUM>(x[j][u], acc[u]);
+        if (t.part) {
+#pragma unroll
+            for (uint32_t u = 0; u < U; ++u) stv<ST>(t.in[j] + so, v0 + u * blockDim.x, acc[u]);
+        }
+    }
+    for (uint32_t r = 0; r < t.nout; ++r) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) stv<ST>(t.out[r] + so, v0 + u * blockDim.x, acc[u]);
+    }
+}
+
+typedef void (*FoldFn)(const FoldProbeTab);
+template <uint32_t U, uint32_t DEPTH> FoldFn pick_fold2(uint32_t hs, uint32_t st)
+{
+    if (hs) return st ? k_probe_fold<U, DEPTH, true, true> : k_probe_fold<U, DEPTH, true, false>;
+    return st ? k_probe_fold<U, DEPTH, false, true> : k_probe_fold<U, DEPTH, false, false>;
+}
+template <uint32_t U> FoldFn pick_fold1(uint32_t depth, uint32_t hs, uint32_t st)
+{
+    switch (depth) {
+        case 1: return pick_fold2<U, 1>(hs, st);
+        case 2: return pick_fold2<U, 2>(hs, st);
+        case 3: return pick_fold2<U, 3>(hs, st);
+        case 7: return pick_fold2<U, 7>(hs, st);
+        default: return nullptr;
+    }
+}
+
 // out[0] += 1 per workgroup that found itself on XCD xk; out[1] = 100 MHz ticks the first such workgroup's chain took
 __global__ __launch_bounds__(64) void k_lat(const uint8_t* base, uint64_t first_piece, uint64_t npieces, uint32_t gran,
                                             uint32_t mod, uint32_t cls, uint32_t xk, uint32_t iters, unsigned long long* out)
@@ -194,7 +266,8 @@ __global__ void k_fill(uint32_t* p, uint64_t nwords, uint32_t seed)
 struct Cfg {
     int kind = K_REDUCE;
     uint32_t nseg = 16, seg_mib = 64, pair = 0, u = 4, block = 256, hd = 1, hs = 1, st = 0, pipe = 0, il = 0, wpc = 0, ring = 0,
-             lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000;
+             lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000,
+             depth = 1, part = 0, nout = 8;
     uint64_t skew = 0;
     bool zeros = false;
     std::string line;
@@ -267,6 +340,7 @@ bool parse(const std::string& line, Cfg& c)
             else if (v == "triad") c.kind = K_TRIAD;
             else if (v == "reduce_i32") c.kind = K_REDUCE_I32;
             else if (v == "lat") c.kind = K_LAT;
+            else if (v == "fold") c.kind = K_FOLD;
             else return false;
         } else if (k == "data") {
             if (v == "zeros") c.zeros = true;
@@ -296,6 +370,9 @@ bool parse(const std::string& line, Cfg& c)
         else if (k == "cls") c.cls = (uint32_t)n;
         else if (k == "gran") c.gran = (uint32_t)n;
         else if (k == "iters") c.iters = (uint32_t)n;
+        else if (k == "depth") c.depth = (uint32_t)n;
+        else if (k == "part") c.part = (uint32_t)n;
+        else if (k == "nout") c.nout = (uint32_t)n;
         else return false;
     }
     return true;
@@ -374,6 +451,73 @@ int main(int argc, char** argv)
             }
             printf("{\"cfg\": \"%s\", \"workgroups_on_xcd\": %llu, \"ns_per_load\": %.1f, \"ns_per_load_min\": %.1f}\n", line.c_str(),
                    hits, ns_sum / c.reps, ns_min);
+            fflush(stdout);
+            continue;
+        }
+        if (c.kind == K_FOLD) {
+            const FoldFn ffn = c.u == 2 ? pick_fold1<2>(c.depth, c.hs, c.st) : c.u == 4 ? pick_fold1<4>(c.depth, c.hs, c.st) : nullptr;
+            const uint64_t seg = (uint64_t)c.seg_mib << 20;
+            const uint64_t tile_bytes = (uint64_t)c.block * c.u * 16u;
+            if (!ffn || c.nseg == 0 || c.nseg > 64 || c.block == 0 || c.block > 1024 || (c.block & 63u) || seg % tile_bytes || c.sets == 0 ||
+                c.nout == 0 || c.nout > 8 || c.lds > 160u * 1024u || (c.skew & 15u)) {
+                fprintf(stderr, "hg_probe: unsupported configuration: %s\n", line.c_str());
+                return 2;
+            }
+            const uint64_t buf = (uint64_t)c.nseg * seg;            // one input or output buffer: nseg segments
+            const uint64_t pitch = buf + c.skew;                    // distance between consecutive buffers
+            const uint64_t need = (uint64_t)c.sets * (8u + c.nout) * pitch;
+            if (need > (64ull << 30)) {
+                fprintf(stderr, "hg_probe: configuration needs %llu bytes: %s\n", (unsigned long long)need, line.c_str());
+                return 2;
+            }
+            if (need > ar.bytes) {
+                if (ar.base) CK(hipFree(ar.base));
+                CK(hipMalloc((void**)&ar.base, need));
+                ar.bytes = need;
+                ar.filled = false;
+            }
+            if (!ar.filled || ar.zeros != c.zeros) {
+                if (c.zeros) CK(hipMemset(ar.base, 0, ar.bytes));
+                else hipLaunchKernelGGL(k_fill, dim3(8192), dim3(256), 0, 0, (uint32_t*)ar.base, ar.bytes / 4, 12345u);
+                CK(hipDeviceSynchronize());
+                ar.filled = true;
+                ar.zeros = c.zeros;
+            }
+            std::vector<FoldProbeTab> tabs(c.sets);
+            for (uint32_t k = 0; k < c.sets; ++k) {
+                FoldProbeTab& t = tabs[k];
+                memset(&t, 0, sizeof t);
+                uint8_t* set0 = ar.base + (uint64_t)k * (8u + c.nout) * pitch;
+                for (uint32_t j = 0; j < 8; ++j) t.in[j] = set0 + (uint64_t)j * pitch;
+                for (uint32_t r = 0; r < c.nout; ++r) t.out[r] = set0 + (uint64_t)(8u + r) * pitch;
+                t.seg_bytes = seg;
+                t.tiles_per_seg = (uint32_t)(seg / tile_bytes);
+                t.nseg = c.nseg;
+                t.nout = c.nout;
+                t.part = c.part;
+                t.xcd = c.xcd;
+                t.run = c.run ? c.run : 1u;
+            }
+            const uint64_t grid = (uint64_t)tabs[0].tiles_per_seg * c.nseg;
+            if (c.lds) CK(hipFuncSetAttribute((const void*)ffn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+            uint32_t launch = 0;
+            for (uint32_t i = 0; i < c.warm; ++i, ++launch)
+                hipLaunchKernelGGL(ffn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+            CK(hipGetLastError());
+            CK(hipEventRecord(e0, st));
+            for (uint32_t i = 0; i < c.reps; ++i, ++launch)
+                hipLaunchKernelGGL(ffn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+            CK(hipEventRecord(e1, st));
+            CK(hipStreamSynchronize(st));
+            CK(hipGetLastError());
+            float ms = 0;
+            CK(hipEventElapsedTime(&ms, e0, e1));
+            ms /= (float)c.reps;
+            const double moved = (8.0 + (c.part ? 7.0 : 0.0) + c.nout) * (double)buf;
+            printf("{\"cfg\": \"%s\", \"grid\": %llu, \"tile_bytes\": %llu, \"ms\": %.5f, \"moved_bytes\": %.0f, \"gbs\": %.1f, "
+                   "\"frac_of_8000\": %.4f}\n",
+                   line.c_str(), (unsigned long long)grid, (unsigned long long)tile_bytes, ms, moved, moved / ms / 1e6,
+                   moved / ms / 1e6 / 8000.0);
             fflush(stdout);
             continue;
         }
