@@ -234,6 +234,12 @@ void hg_finish_fold(HgLaunch* l)
         uint64_t sum = 0;
         for (uint32_t s = 0; s < t->nseg; ++s) sum += t->bytes[s];
         t->direct = (direct_on() && sum <= direct_bytes && t->nseg <= HG_DIRECT_SEG && t->k <= 16u) ? 1u : 0u;
+        /* what the host-resolved table does not carry: a neighbour absorbed before the tree (recursive halving on a
+         * rank count that is not a power of two), more receivers than leaf positions */
+        if (t->tree == 1u)
+            for (uint32_t b = 0; b < HCOMM_GFX_MAX_RANKS; ++b)
+                if (t->in2[b]) t->direct = 0u;
+        if (!(t->tree != 1u && t->out_mode == 1u) && t->nout > t->k) t->direct = 0u;
     }
     const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_CHAIN_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {

@@ -650,3 +650,55 @@ def test_direct_launch_switch_returns_the_previous_setting():
     finally:
         h.HcommGfxSetDirectLaunches(before)
     assert h.HcommGfxSetDirectLaunches(before) == before
+
+
+def test_launch_records_name_the_grid_shape():
+    """rows / streaming of HcommGfxLaunchRecord: which kernel variant a launch takes, decided on the host."""
+    K = h.Kernel
+    # 8-rank ring allreduce, 128 MiB per rank: every step is 8 slices of 16 MiB = 1024 tiles each -> a grid of
+    # 1024 x 8, the variant whose output the next step finds cached
+    size = 128 << 20
+    i, o = ptrs(8, size, base=1 << 40)
+    p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, i, o, size // 2, DT.BFP16, OP.SUM)
+    recs = p.launches()
+    assert len(recs) == 15
+    assert all(r.rows == 1024 and r.streaming == 0 and r.blocks == 8 * 1024 for r in recs)
+    p.destroy()
+    # 16-rank recursive halving-doubling: the first halving step writes 16 x 64 MiB = 1 GiB -> streaming, 4096 tiles a row
+    i, o = ptrs(16, size, base=1 << 40)
+    p = h.Plan(h.Alg.ALLREDUCE_RHD, h.Lowering.STEPWISE, i, o, size // 4, DT.INT32, OP.SUM)
+    first = [r for r in p.launches() if r.kind == K.REDUCE2][0]
+    assert (first.rows, first.streaming, first.nseg) == (4096, 1, 16)
+    p.destroy()
+    # small fused launches: addresses resolved on the host
+    i, o = ptrs(8, 4096, base=1 << 40)
+    for alg, kind in ((h.Alg.ALLREDUCE_MESH_ONESHOT, K.CHAIN), (h.Alg.ALLREDUCE_RING, K.CHAIN), (h.Alg.ALLREDUCE_NHR, K.TREE)):
+        p = h.Plan(alg, h.Lowering.FUSED, i, o, 2048, DT.FP16, OP.SUM)
+        assert [(r.kind, r.rows) for r in p.launches()] == [(kind, 1)]
+        p.destroy()
+    # recursive halving on 6 ranks absorbs the odd neighbours before the tree: not a launch the host can resolve
+    i, o = ptrs(6, 6 * 4096, base=1 << 40)
+    p = h.Plan(h.Alg.ALLREDUCE_RHD, h.Lowering.FUSED, i, o, 6 * 1024, DT.FP32, OP.SUM)
+    assert [(r.kind, r.rows) for r in p.launches()] == [(K.TREE, 0)]
+    p.destroy()
+    # segments of very different lengths beyond the small-launch limit keep the one-dimensional grid
+    code, rec = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    h.check(h.HcommBatchModeStart(b"ragged"), "start")
+    base = 1 << 40
+    for k, n in enumerate((16 << 20, 16 << 10, 32 << 20, 4096)):
+        h.check(h.HcommLocalCopyOnThread(rec, base + (2 * k) * (64 << 20), base + (2 * k + 1) * (64 << 20), n), "copy")
+    h.check(h.HcommBatchModeEnd(b"ragged"), "end")
+    log = h.launch_log(rec)
+    assert [(r.kind, r.nseg, r.rows) for r in log] == [(K.COPY, 4, 0)]
+    h.HcommThreadFree([rec])
+    # with the switch off nothing takes a two-dimensional grid
+    before = h.HcommGfxSetDirectLaunches(0)
+    try:
+        i, o = ptrs(8, 4096, base=1 << 40)
+        for low in (h.Lowering.STEPWISE, h.Lowering.FUSED):
+            p = h.Plan(h.Alg.ALLREDUCE_RING, low, i, o, 1024, DT.FP32, OP.SUM)
+            assert all(r.rows == 0 for r in p.launches())
+            p.destroy()
+    finally:
+        h.HcommGfxSetDirectLaunches(before)
