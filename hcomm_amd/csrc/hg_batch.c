@@ -33,8 +33,9 @@ static uint64_t env_once(uint64_t* slot, const char* name, uint64_t unset)
     return v;
 }
 
-/* Whether small launches take the kernels that read their arguments in one round (HcommGfxSetDirectLaunches;
- * HCOMM_GFX_DIRECT=0 in the environment starts with them off). */
+/* Whether launches may take the kernels that read their arguments in one round - the (tile, segment) grids and the
+ * fold launches whose addresses the host resolves (HcommGfxSetDirectLaunches; HCOMM_GFX_DIRECT=0 in the environment
+ * starts with them off). */
 static int g_direct_state = 0; /* 0 not read yet, 1 off, 2 on */
 
 static int direct_on(void)

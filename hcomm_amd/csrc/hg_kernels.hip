@@ -1,8 +1,10 @@
 // hg_kernels.hip - gfx950 kernels of libhcomm_gfx.so and their launchers.
 //
 // Everything here is HBM-bandwidth bound: one lane moves 128 bits per access, a workgroup of 256 lanes
-// keeps HG_UNROLL such accesses per operand in flight, and a launch covers a whole table of segments
-// (all simulated ranks of one schedule step) with a grid-stride loop over 16 KiB tiles.
+// keeps HG_UNROLL such accesses per operand in flight (one 16 KiB tile per workgroup), and a launch covers a whole
+// table of segments (all simulated ranks of one schedule step).  Two grid shapes: one-dimensional over the table's
+// tiles, each workgroup finding its segment in the prefix sums (k_copy, k_reduce2, k_bytewise: any table), and
+// (tile, segment) for tables whose segments are about equally long (k_copy_rows, k_reduce2_rows).
 //
 
 #include "hg_device.hpp"
@@ -13,7 +15,7 @@ namespace {
 
 // STREAM: nothing of what the launch writes will be found in the memory-side cache by a later launch (there is more
 // of it than that cache holds, or nothing reads it soon): store with the non-temporal hint.  The launch's dynamic
-// LDS size is not used as memory: it bounds the workgroups a CU runs at once (hg_launch_lds in hg_batch.c).
+// LDS size is not used as memory: it bounds the workgroups a CU runs at once (hg_shape_seg2 in hg_batch.c).
 template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
