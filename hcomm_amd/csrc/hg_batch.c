@@ -242,7 +242,14 @@ void hg_finish_fold(HgLaunch* l)
                 if (t->in2[b]) t->direct = 0u;
         if (!(t->tree != 1u && t->out_mode == 1u) && t->nout > t->k) t->direct = 0u;
     }
-    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES_K(t->k) : (t->small ? HG_TREE_TILE_BYTES : HG_CHAIN_TILE_BYTES);
+    t->nu = 1u;
+    if (t->tree && (t->k == 4u || t->k == 8u)) {
+        /* 8 KiB tiles unless the launch also stores partials into its inputs (recursive halving and the NHR / NB
+         * rotations when the inputs are not kept) */
+        const int stores_partials = t->tree <= 3u && !t->keep_inputs;
+        t->nu = stores_partials ? 1u : 2u;
+    }
+    const uint64_t tile_bytes = t->tree ? HG_TREE_TILE_BYTES * t->nu : (t->small ? HG_TREE_TILE_BYTES : HG_CHAIN_TILE_BYTES);
     for (uint32_t s = 0; s < t->nseg; ++s) {
         t->tile_begin[s] = (uint32_t)tiles;
         tiles += (t->bytes[s] + tile_bytes - 1) / tile_bytes;

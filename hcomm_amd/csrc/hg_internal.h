@@ -34,9 +34,6 @@ extern "C" {
 #define HG_TILE_VECS (HG_BLOCK * HG_UNROLL)
 #define HG_TILE_BYTES ((uint64_t)HG_TILE_VECS * HG_VEC_BYTES) /* 16 KiB of output per tile */
 #define HG_TREE_TILE_BYTES ((uint64_t)HG_BLOCK * HG_VEC_BYTES) /* tree / small-message kernels: one access per lane and input */
-/* vectors a lane of the tree kernel handles when it folds k values per element, and the tile that makes */
-#define HG_TREE_NU(k) ((k) <= 8u ? 2u : 1u)
-#define HG_TREE_TILE_BYTES_K(k) (HG_TREE_TILE_BYTES * HG_TREE_NU(k))
 
 /* Two-pointer segment table (copy, reduce2, bytewise), passed to the kernel by value. */
 typedef struct {
@@ -84,6 +81,8 @@ typedef struct {
                               * the other ranks in cyclic order, entered at distance start[s] + 1 */
     uint32_t keep_inputs;    /* tree modes 1 - 3: the partials the step-wise replay leaves in the inputs are not stored */
     uint32_t small;          /* chain only: latency-oriented variant (4 KiB tiles, loads issued 8 inputs at a time) */
+    uint32_t nu;             /* tree only: 128-bit vectors per lane, i.e. tiles of 4 or 8 KiB: two for 4 or 8 leaf positions
+                              * (the two sizes compiled both ways) in launches that write little beside their result, else one */
     uint32_t direct;         /* small chain that only reads its inputs, <= HG_DIRECT_K of them in <= HG_DIRECT_SEG segments:
                               * the launcher resolves every address on the host (one round of kernel-argument reads) */
     uint32_t xcd_run;        /* > 0: each XCD walks runs of this many consecutive tiles (block_id in hg_device.hpp) */

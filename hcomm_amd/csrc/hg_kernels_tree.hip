@@ -213,11 +213,12 @@ template <int DT, int OP> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tre
     }
 }
 
-// A lane handles HG_TREE_NU(K) vectors: two while the 2 x K values fit comfortably in registers (K <= 8), else one.
-template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
+// A lane handles NU vectors (tab.nu, chosen by the host): two while the 2 x K values fit comfortably in registers
+// (K <= 8) and the launch writes little beside its result, else one (a launch that also stores the partials into
+// the inputs moves more on 4 KiB tiles: NHR allreduce of 8 x 128 MiB in one launch 0.499 -> 0.463 ms).
+template <int DT, int OP, int L, uint32_t NU> __global__ __launch_bounds__(HG_BLOCK) void k_fold_tree(const HgFoldTable tab)
 {
     constexpr uint32_t ES = ElemSize<DT>::v;
-    constexpr uint32_t NU = HG_TREE_NU(1u << L);
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
@@ -373,6 +374,19 @@ template <int L> bool tree_direct_table(const HgFoldTable& t, HgTreeDirect<(1u <
     return *width > 0;
 }
 
+template <int DT, int L, uint32_t NU>
+int launch_tree_dt_l_nu(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
+{
+    switch (op) {
+        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L, NU>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L, NU>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L, NU>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L, NU>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
+        default: return HCCL_E_PARA;
+    }
+    return rc(hipGetLastError());
+}
+
 template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     if constexpr (L <= 4) {
@@ -390,14 +404,11 @@ template <int DT, int L> int launch_tree_dt_l(hipStream_t st, int op, const HgFo
             return rc(hipGetLastError());
         }
     }
-    switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_fold_tree<DT, OP_SUM, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_fold_tree<DT, OP_PROD, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_fold_tree<DT, OP_MAX, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_fold_tree<DT, OP_MIN, L>), dim3(blocks), dim3(HG_BLOCK), lds, st, *tab); break;
-        default: return HCCL_E_PARA;
+    if constexpr (L == 2 || L == 3) {
+        if (tab->nu == 2u) return launch_tree_dt_l_nu<DT, L, 2>(st, op, tab, blocks, lds);
     }
-    return rc(hipGetLastError());
+    if (tab->nu != 1u) return HCCL_E_INTERNAL;
+    return launch_tree_dt_l_nu<DT, L, 1>(st, op, tab, blocks, lds);
 }
 
 template <int DT> int launch_tree_deep_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
