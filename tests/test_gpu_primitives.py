@@ -309,3 +309,53 @@ def test_more_than_4gib_in_one_call(gpu_thread):
         assert torch.equal(dst[lo:hi], src[lo:hi] * 2), "chunk at %d" % lo
     del src, dst
     torch.cuda.empty_cache()
+
+
+def test_batches_of_nearly_equal_segments(gpu_thread):
+    """Batches whose segments differ a little in length take the (tile, segment) grid, as wide as the longest one:
+    shorter segments leave workgroups with nothing to do, tails fall into different tiles.  A fixed-seed sample of
+    segment counts, lengths around the tile boundaries, types and operations, reduces and copies, every buffer
+    bit-exact against the oracle, and the launch records say which grid a batch took."""
+    rng = np.random.default_rng(77)
+    direct = h.HcommGfxSetDirectLaunches(1)   # the setting this test runs under (the other test module turns it off)
+    h.HcommGfxSetDirectLaunches(direct)
+    names = ["int8", "int16", "int32", "fp16", "fp32", "bf16"]
+    bases = [100, 4096, 16384, 16384 * 3 + 5, 100000, 1 << 20]
+    for case in range(40):
+        nseg = int(rng.choice([1, 2, 3, 8, 9, 17, 64]))
+        dtype = names[rng.integers(len(names))]
+        op = ["sum", "max", "min"][rng.integers(3)]   # PROD is refused by the primitive unless opted in
+        dt, o, unit = DT[dtype], OPS[op], UNIT[DT[dtype]]
+        base = int(bases[rng.integers(len(bases))]) // unit + 1
+        if nseg * base * unit > (48 << 20):
+            base = (48 << 20) // (nseg * unit)
+        counts = [max(1, base - int(rng.integers(0, base // 10 + 2))) for _ in range(nseg)]   # within 10 % of one another
+        is_copy = bool(rng.integers(3) == 0)
+        say("nearly equal", case, nseg, dtype, op, "copy" if is_copy else "reduce", counts[:4])
+        dst = [gen(dt, c, 5000 + 2 * i) for i, c in enumerate(counts)]
+        src = [gen(dt, c, 5001 + 2 * i) for i, c in enumerate(counts)]
+        d_dst, d_src = [to_dev(x) for x in dst], [to_dev(x) for x in src]
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        h.HcommGfxLaunchLogClear(gpu_thread)
+        assert h.HcommBatchModeStart(b"rows") == 0
+        for i, c in enumerate(counts):
+            if is_copy:
+                assert h.HcommLocalCopyOnThread(gpu_thread, d_dst[i].data_ptr(), d_src[i].data_ptr(), c * unit) == 0
+            else:
+                assert h.HcommLocalReduceOnThread(gpu_thread, d_dst[i].data_ptr(), d_src[i].data_ptr(), c, dt, o) == 0
+        assert h.HcommBatchModeEnd(b"rows") == 0
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        log = h.launch_log(gpu_thread)
+        assert len(log) == 1 and log[0].nseg == nseg
+        tiles = [(c * unit + 16383) // 16384 for c in counts]
+        total, grid = sum(tiles), max(tiles) * nseg
+        rows = max(tiles) if direct and (grid <= total + total // 8 or (total <= 512 and grid <= 2 * total)) else 0
+        assert log[0].rows == rows and log[0].blocks == (grid if rows else total)
+        for i in range(nseg):
+            want = dst[i].copy()
+            if is_copy:
+                want = src[i].copy()
+            else:
+                oracle.reduce(want, src[i], dt, o)
+            assert_same(from_dev(d_dst[i], dst[i]), want, dt, "case %d segment %d" % (case, i))
+            assert np.array_equal(from_dev(d_src[i], src[i]), src[i]), "case %d: source %d modified" % (case, i)
