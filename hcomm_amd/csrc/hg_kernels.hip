@@ -144,7 +144,8 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 
 // ---- launches whose segments are (nearly) equally long: one round of argument reads ----------------------------
 //
-// A launch starts with a chain of dependent memory round trips of about a microsecond each: kernel arguments,
+// A launch starts with a chain of dependent memory round trips (a quarter of a microsecond per round of argument
+// reads, measured by hg_probe kind=start; more for the data): kernel arguments,
 // whatever they index, the data, the stores.  The kernels above find a tile's segment in the table's prefix sums
 // and only then know which pointers to read: several rounds of argument reads before the first byte of data is
 // asked for, paid by every launch of a schedule because a launch does not start before the one ahead of it has
@@ -156,7 +157,7 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
 // is equal modulo 8 run on one XCD whatever the row's place in the grid).
 
 // Launches of at most HG_DIRECT_SEG segments pass this table instead of the full one: the runtime copies the kernel
-// arguments on every launch, and 200 bytes cost less there than 1.8 KB (about a microsecond per launch).
+// arguments on every launch, and 200 bytes cost less there than 1.8 KB (half a microsecond to a microsecond per queued launch).
 struct HgSeg2Few {
     void* dst[HG_DIRECT_SEG];
     const void* src[HG_DIRECT_SEG];

@@ -247,7 +247,7 @@ template <int DT, int OP, int L, uint32_t NU> __global__ __launch_bounds__(HG_BL
 // ---- small tree launches with host-resolved addresses --------------------------------------------------------
 //
 // The kernels above read their arguments in rounds that wait for one another (the table's scalars, the segment's
-// row, the leaf table, the rank pointers it selects), about a microsecond each, which is most of what a small
+// row, the leaf table, the rank pointers it selects), a quarter of a microsecond each, which is much of what a small
 // launch costs.  For trees of up to 16 positions in up to HG_DIRECT_SEG segments the launcher lays every leaf's
 // address out per segment and the grid is two-dimensional (y = segment, x = tile): one round of argument reads.
 // A hole carries position 0's address (a load that is always valid) and is left out of the fold by a select, so

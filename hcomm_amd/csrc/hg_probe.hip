@@ -32,6 +32,14 @@
 //                  depth=1|2|3|7  positions whose loads are in flight ahead of the one being folded
 //                  part=0|1 nout=8
 //
+// kind=start       what a launch costs before it streams: one workgroup copies 16 bytes after `rounds` dependent reads of
+//                  its by-value argument table (each read selects the word the next one fetches, a cache line further
+//                  on, the way a kernel walks from a table's scalars to the row and the pointer they select); the
+//                  table is `table` bytes long (256 or 2048: the runtime copies it on every launch).  Reported: the
+//                  median of `reps` launches timed one by one between two events, and the time per launch of `reps`
+//                  launches queued back to back, and the wave's own clock from its first instruction to the arrival of
+//                  the data.   keys: rounds=1..6 table=256|2048 reps=200
+//
 // kind=lat         one wavefront on XCD `xk` walks a chain of dependent 1 KiB loads (64 lanes x 16 bytes) over the
 //                  pieces p of a 4 GiB arena with p mod `mod` == `cls`, a piece being `gran` bytes (a power of two
 //                  >= 1024): the nanoseconds per load tell how far that class of addresses is from that XCD.
@@ -42,6 +50,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -56,7 +65,7 @@ namespace {
         }                                                                                          \
     } while (0)
 
-enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6, K_FOLD = 7 };
+enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6, K_FOLD = 7, K_START = 8 };
 
 struct ProbeTab {
     void* dst[64];
@@ -225,6 +234,30 @@ template <uint32_t U> FoldFn pick_fold1(uint32_t depth, uint32_t hs, uint32_t st
     }
 }
 
+// ---- kind=start ---------------------------------------------------------------------------------------------
+
+template <uint32_t WORDS> struct StartTab {
+    uint32_t next[WORDS]; // next[i]: the word read after word i (16 words = one 64-byte line further on)
+    uint8_t* dst;
+    const uint8_t* src;
+    uint32_t rounds;
+};
+
+template <uint32_t WORDS> __global__ __launch_bounds__(64) void k_probe_start(const StartTab<WORDS> t)
+{
+    const unsigned long long t0 = wall_clock64();
+    uint32_t i = 0;
+    for (uint32_t r = 1; r < t.rounds; ++r) i = t.next[i]; // every read waits for the one before it
+    const uint32_t off = (i == 0xffffffffu) ? 16u : 0u;     // depends on the chain's end; no table word holds that value
+    if (threadIdx.x == 0) {
+        const u32x4 v = *(const u32x4*)(t.src + off);
+        *(u32x4*)(t.dst + off) = v;
+        // 100 MHz ticks from the wave's first instruction to the arrival of the data (v.x keeps the read ahead of the clock)
+        const unsigned long long t1 = wall_clock64() + (v.x == 0xdeadbeefu ? 1u : 0u);
+        *(unsigned long long*)(t.dst + 1024) = t1 - t0;
+    }
+}
+
 // out[0] += 1 per workgroup that found itself on XCD xk; out[1] = 100 MHz ticks the first such workgroup's chain took
 __global__ __launch_bounds__(64) void k_lat(const uint8_t* base, uint64_t first_piece, uint64_t npieces, uint32_t gran,
                                             uint32_t mod, uint32_t cls, uint32_t xk, uint32_t iters, unsigned long long* out)
@@ -267,7 +300,7 @@ struct Cfg {
     int kind = K_REDUCE;
     uint32_t nseg = 16, seg_mib = 64, pair = 0, u = 4, block = 256, hd = 1, hs = 1, st = 0, pipe = 0, il = 0, wpc = 0, ring = 0,
              lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000,
-             depth = 1, part = 0, nout = 8;
+             depth = 1, part = 0, nout = 8, rounds = 1, table = 256;
     uint64_t skew = 0;
     bool zeros = false;
     std::string line;
@@ -341,6 +374,7 @@ bool parse(const std::string& line, Cfg& c)
             else if (v == "reduce_i32") c.kind = K_REDUCE_I32;
             else if (v == "lat") c.kind = K_LAT;
             else if (v == "fold") c.kind = K_FOLD;
+            else if (v == "start") c.kind = K_START;
             else return false;
         } else if (k == "data") {
             if (v == "zeros") c.zeros = true;
@@ -373,6 +407,8 @@ bool parse(const std::string& line, Cfg& c)
         else if (k == "depth") c.depth = (uint32_t)n;
         else if (k == "part") c.part = (uint32_t)n;
         else if (k == "nout") c.nout = (uint32_t)n;
+        else if (k == "rounds") c.rounds = (uint32_t)n;
+        else if (k == "table") c.table = (uint32_t)n;
         else return false;
     }
     return true;
@@ -451,6 +487,55 @@ int main(int argc, char** argv)
             }
             printf("{\"cfg\": \"%s\", \"workgroups_on_xcd\": %llu, \"ns_per_load\": %.1f, \"ns_per_load_min\": %.1f}\n", line.c_str(),
                    hits, ns_sum / c.reps, ns_min);
+            fflush(stdout);
+            continue;
+        }
+        if (c.kind == K_START) {
+            if (c.rounds == 0 || c.rounds > 6 || (c.table != 256 && c.table != 2048) || c.reps == 0) {
+                fprintf(stderr, "hg_probe: unsupported configuration: %s\n", line.c_str());
+                return 2;
+            }
+            static uint8_t* pad = nullptr;
+            if (!pad) {
+                CK(hipMalloc((void**)&pad, 4096));
+                CK(hipMemset(pad, 1, 4096));
+            }
+            StartTab<56> small;   // 256 bytes with the pointers
+            StartTab<504> large;  // 2048 bytes
+            for (uint32_t i = 0; i < 56; ++i) small.next[i] = (i + 16) % 56;
+            for (uint32_t i = 0; i < 504; ++i) large.next[i] = (i + 16) % 504;
+            small.dst = large.dst = pad;
+            small.src = large.src = pad + 2048;
+            small.rounds = large.rounds = c.rounds;
+            auto launch = [&]() {
+                if (c.table == 256) hipLaunchKernelGGL(k_probe_start<56>, dim3(1), dim3(64), 0, st, small);
+                else hipLaunchKernelGGL(k_probe_start<504>, dim3(1), dim3(64), 0, st, large);
+            };
+            for (uint32_t i = 0; i < 20; ++i) launch();
+            CK(hipStreamSynchronize(st));
+            std::vector<float> one(c.reps);
+            std::vector<unsigned long long> ticks(c.reps);
+            for (uint32_t i = 0; i < c.reps; ++i) {
+                CK(hipEventRecord(e0, st));
+                launch();
+                CK(hipEventRecord(e1, st));
+                CK(hipStreamSynchronize(st));
+                CK(hipEventElapsedTime(&one[i], e0, e1));
+                CK(hipMemcpy(&ticks[i], pad + 1024, sizeof ticks[i], hipMemcpyDeviceToHost));
+            }
+            std::sort(one.begin(), one.end());
+            std::sort(ticks.begin(), ticks.end());
+            CK(hipEventRecord(e0, st));
+            for (uint32_t i = 0; i < c.reps; ++i) launch();
+            CK(hipEventRecord(e1, st));
+            CK(hipStreamSynchronize(st));
+            CK(hipGetLastError());
+            float all = 0;
+            CK(hipEventElapsedTime(&all, e0, e1));
+            printf("{\"cfg\": \"%s\", \"alone_us_median\": %.2f, \"alone_us_min\": %.2f, \"queued_us_per_launch\": %.2f, "
+                   "\"in_kernel_us_median\": %.2f, \"in_kernel_us_min\": %.2f}\n",
+                   line.c_str(), one[c.reps / 2] * 1e3, one[0] * 1e3, all * 1e3 / c.reps, (double)ticks[c.reps / 2] * 0.01,
+                   (double)ticks[0] * 0.01);
             fflush(stdout);
             continue;
         }
