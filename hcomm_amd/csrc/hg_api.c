@@ -315,7 +315,7 @@ int hg_submit(HgThread* t, const HgLaunch* l)
                                      l->lds_bytes);
         case HCOMM_GFX_KERNEL_BYTEWISE:
             return hg_launch_bytewise(t->stream, l->op != 255u, (int)l->dtype, (int)l->op, &l->tab.seg2, l->blocks,
-                                      l->lds_bytes);
+                                      (int)l->streaming, l->lds_bytes);
         case HCOMM_GFX_KERNEL_CHAIN:
         case HCOMM_GFX_KERNEL_TREE:
             return hg_launch_fold(t->stream, (int)l->dtype, (int)l->op, (int)l->acc_is_dst, &l->tab.fold, l->blocks,

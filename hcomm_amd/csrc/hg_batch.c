@@ -132,18 +132,16 @@ static uint32_t lds_of(int i)
 void hg_shape_seg2(HgLaunch* l, int streaming)
 {
     HgSeg2Table* t = &l->tab.seg2;
-    if (l->kind == HCOMM_GFX_KERNEL_COPY) {
+    /* the kernel for operands off 16-byte boundaries comes as a copy (op 255) and as a reduce: shaped like them */
+    const int copy = l->kind == HCOMM_GFX_KERNEL_COPY || (l->kind == HCOMM_GFX_KERNEL_BYTEWISE && l->op == 255u);
+    if (copy) {
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_COPY_BYTES));
         l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_COPY_STREAM : TUNE_LDS_COPY);
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_COPY_STREAM : TUNE_RUN_COPY);
-    } else if (l->kind == HCOMM_GFX_KERNEL_REDUCE2) {
+    } else {
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_REDUCE_BYTES));
         l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_REDUCE_STREAM : TUNE_LDS_REDUCE);
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_REDUCE_STREAM : TUNE_RUN_REDUCE);
-    } else {
-        l->streaming = 0;
-        l->lds_bytes = 0;
-        t->xcd_run = 0;
     }
 }
 
@@ -172,8 +170,8 @@ void hg_finish_seg2(HgLaunch* l)
      * tiles), anything up to HCOMM_GFX_DIRECT_TILES tiles as long as the grid at most doubles.  Launches that small
      * are latency-bound and take neither the occupancy bound nor the XCD runs. */
     t->direct = 0u;
+    const int small = tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u);
     if (direct_on() && tiles != 0 && l->kind != HCOMM_GFX_KERNEL_BYTEWISE) {
-        const int small = tiles <= env_once(&g_direct_tiles, "HCOMM_GFX_DIRECT_TILES", 512u);
         uint32_t w = 0;
         for (uint32_t s = 0; s < t->nseg; ++s) {
             const uint32_t n = t->tile_begin[s + 1] - t->tile_begin[s];
@@ -184,11 +182,11 @@ void hg_finish_seg2(HgLaunch* l)
             t->direct = w;
             l->blocks = grid;
         }
-        if (t->direct && small) {
-            l->streaming = 0;
-            l->lds_bytes = 0;
-            t->xcd_run = 0;
-        }
+    }
+    if (small && (t->direct || l->kind == HCOMM_GFX_KERNEL_BYTEWISE)) {
+        l->streaming = 0;
+        l->lds_bytes = 0;
+        t->xcd_run = 0;
     }
 }
 

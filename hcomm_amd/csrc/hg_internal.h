@@ -104,7 +104,8 @@ uint64_t hg_grid_blocks(uint64_t total_tiles);
  * lds: bytes of dynamic LDS per workgroup, asked for only to bound the workgroups a CU runs at once */
 int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
 int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
-int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, uint32_t lds);
+int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming,
+                       uint32_t lds);
 int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks, uint32_t lds);
 
 /* Thin wrappers over the HIP runtime so that the C files need no HIP headers. */

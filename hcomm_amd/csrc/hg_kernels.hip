@@ -99,7 +99,8 @@ template <> struct UVec<1> { typedef u32x4 T __attribute__((aligned(1))); };
 template <> struct UVec<2> { typedef u32x4 T __attribute__((aligned(2))); };
 template <> struct UVec<4> { typedef u32x4 T __attribute__((aligned(4))); };
 
-template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) void k_bytewise(const HgSeg2Table tab)
+// STREAM as for k_copy / k_reduce2.
+template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_bytewise(const HgSeg2Table tab)
 {
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
     typedef typename UVec<ES>::T UV;
@@ -122,13 +123,13 @@ template <int DT, int OP, bool REDUCE> __global__ __launch_bounds__(HG_BLOCK) vo
             const uint64_t v = vb + tid + u * HG_BLOCK;
             if (v < nvec) {
                 b[u] = __builtin_nontemporal_load((const UV*)(p + (v << 4)));
-                if (REDUCE) a[u] = ldv<true>(d, v);
+                if (REDUCE) a[u] = ldv<STREAM>(d, v);
             }
         }
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = vb + tid + u * HG_BLOCK;
-            if (v < nvec) stv<false>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
+            if (v < nvec) stv<STREAM>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
         }
         if (vb <= nvec && vb + HG_TILE_VECS > nvec) { // the one tile that holds the end of the items
             // fewer than 16 / ES elements before the first item and fewer than that after the last one
@@ -300,17 +301,23 @@ template <bool STREAM> int launch_copy_s(hipStream_t st, const HgSeg2Table* tab,
     return rc(hipGetLastError());
 }
 
-template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
+template <int DT, bool STREAM> int launch_bytewise_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
     switch (op) {
-        case OP_SUM: hipLaunchKernelGGL((k_bytewise<DT, OP_SUM, true>), g, b, lds, st, *tab); break;
-        case OP_PROD: hipLaunchKernelGGL((k_bytewise<DT, OP_PROD, true>), g, b, lds, st, *tab); break;
-        case OP_MAX: hipLaunchKernelGGL((k_bytewise<DT, OP_MAX, true>), g, b, lds, st, *tab); break;
-        case OP_MIN: hipLaunchKernelGGL((k_bytewise<DT, OP_MIN, true>), g, b, lds, st, *tab); break;
+        case OP_SUM: hipLaunchKernelGGL((k_bytewise<DT, OP_SUM, true, STREAM>), g, b, lds, st, *tab); break;
+        case OP_PROD: hipLaunchKernelGGL((k_bytewise<DT, OP_PROD, true, STREAM>), g, b, lds, st, *tab); break;
+        case OP_MAX: hipLaunchKernelGGL((k_bytewise<DT, OP_MAX, true, STREAM>), g, b, lds, st, *tab); break;
+        case OP_MIN: hipLaunchKernelGGL((k_bytewise<DT, OP_MIN, true, STREAM>), g, b, lds, st, *tab); break;
         default: return HCCL_E_PARA;
     }
     return rc(hipGetLastError());
+}
+
+template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, int streaming, uint32_t lds)
+{
+    if (streaming) return launch_bytewise_dt_s<DT, true>(st, op, tab, blocks, lds);
+    return launch_bytewise_dt_s<DT, false>(st, op, tab, blocks, lds);
 }
 
 } // namespace
@@ -333,15 +340,17 @@ int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, u
 #undef CALL
 }
 
-int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, uint32_t lds)
+int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming,
+                       uint32_t lds)
 {
     if (blocks == 0) return HCCL_SUCCESS;
     if (!is_reduce) {
-        hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false>), dim3((uint32_t)blocks), dim3(HG_BLOCK), lds,
-                           (hipStream_t)stream, *tab);
+        const dim3 g((uint32_t)blocks), b(HG_BLOCK);
+        if (streaming) hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false, true>), g, b, lds, (hipStream_t)stream, *tab);
+        else hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false, false>), g, b, lds, (hipStream_t)stream, *tab);
         return rc(hipGetLastError());
     }
-#define CALL(DT) launch_bytewise_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, lds)
+#define CALL(DT) launch_bytewise_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, streaming, lds)
     HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
 }

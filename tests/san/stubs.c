@@ -5,7 +5,7 @@
 #include "hg_internal.h"
 int hg_launch_copy(void* s, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)t; (void)b; (void)m; (void)l; return 4; }
 int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)d; (void)o; (void)t; (void)b; (void)m; (void)l; return 4; }
-int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, uint32_t l) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)l; return 4; }
+int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, int st, uint32_t l) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)st; (void)l; return 4; }
 int hg_launch_fold(void* s, int d, int o, int a, const HgFoldTable* t, uint64_t b, uint32_t l) { (void)s; (void)d; (void)o; (void)a; (void)t; (void)b; (void)l; return 4; }
 int hg_rt_device_count(void) { return 0; }
 int hg_rt_scratch(void* s, void** p) { (void)s; *p = NULL; return 4; }
