@@ -278,7 +278,7 @@ bool direct_table(const HgFoldTable& t, HgDirectTable* d, uint32_t* width)
 template <int DT, bool AD> int launch_fold_dt(hipStream_t st, int op, const HgFoldTable* tab, uint32_t blocks, uint32_t lds)
 {
     const dim3 g(blocks), b(HG_BLOCK);
-    HgDirectTable direct;
+    HgDirectTable direct = {};
     uint32_t width = 0;
     if (direct_table(*tab, &direct, &width)) {
         const dim3 g2(width, tab->nseg);
