@@ -224,6 +224,18 @@ int main(void)
         run_plan(th, p);
         HcommGfxOpListCheck(ops, k, 2, HCOMM_GFX_EXPECT_ALLREDUCE, 4, 0, 4, &rep);
     }
+    /* the same plans shaped with the one-round kernels switched off, and on again */
+    for (int on = 0; on <= 1; ++on) {
+        const int32_t before = HcommGfxSetDirectLaunches(on);
+        if (before != !on) ++bad;
+        for (uint32_t n = 1; n <= 9; ++n)
+            for (int alg = 0; alg <= 17; ++alg)
+                for (int low = 0; low <= 2; ++low) {
+                    p = NULL;
+                    HcommGfxPlanCreateEx(alg, low, n, bufs[0], bufs[1], bufs[2], 4099, 0, HCOMM_DATA_TYPE_FP16, HCOMM_REDUCE_SUM, &p);
+                    run_plan(th, p);
+                }
+    }
     HcommGfxSlice slc[32];
     for (uint32_t n = 0; n <= 32; ++n) HcommGfxCalcSlices(100003, 2, n, slc);
     HcommThreadFree(&th, 1);
