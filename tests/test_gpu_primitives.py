@@ -359,3 +359,35 @@ def test_batches_of_nearly_equal_segments(gpu_thread):
                 oracle.reduce(want, src[i], dt, o)
             assert_same(from_dev(d_dst[i], dst[i]), want, dt, "case %d segment %d" % (case, i))
             assert np.array_equal(from_dev(d_src[i], src[i]), src[i]), "case %d: source %d modified" % (case, i)
+
+
+@pytest.mark.parametrize("sizes", [
+    [16384, 32768, 16385, 1, 49152],          # 1, 2, 2, 1, 3 tiles: a grid of 3 x 5 for 9 tiles
+    [1, 1, 1],
+    [16383] * 9 + [5],
+    [65536, 65536 - 16, 65536 + 16, 65535],   # tails in the last tile, one tile further, and a byte short
+    [3 * 16384 + 7] * 64,
+])
+def test_row_grid_leaves_short_segments_alone(gpu_thread, sizes):
+    """Byte copies and int8 sums over segments of hand-picked lengths in one batch: the grid is as wide as the longest
+    segment, so the workgroups past a shorter segment's last tile must touch nothing - every destination is checked
+    together with the 64 guard bytes behind it."""
+    guard = 64
+    rng = np.random.default_rng(len(sizes))
+    for reduce in (False, True):
+        src = [rng.integers(-8, 9, n, dtype=np.int8) for n in sizes]
+        dst = [rng.integers(-8, 9, n + guard, dtype=np.int8) for n in sizes]
+        d_src, d_dst = [to_dev(x) for x in src], [to_dev(x) for x in dst]
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        assert h.HcommBatchModeStart(b"short") == 0
+        for i, n in enumerate(sizes):
+            if reduce:
+                assert h.HcommLocalReduceOnThread(gpu_thread, d_dst[i].data_ptr(), d_src[i].data_ptr(), n, oracle.I8, oracle.SUM) == 0
+            else:
+                assert h.HcommLocalCopyOnThread(gpu_thread, d_dst[i].data_ptr(), d_src[i].data_ptr(), n) == 0
+        assert h.HcommBatchModeEnd(b"short") == 0
+        h.HcommGfxThreadSynchronize(gpu_thread)
+        for i, n in enumerate(sizes):
+            want = dst[i].copy()
+            want[:n] = (dst[i][:n].astype(np.int16) + src[i].astype(np.int16)).astype(np.int8) if reduce else src[i]
+            assert np.array_equal(from_dev(d_dst[i], dst[i]), want), "segment %d of %r (%s)" % (i, sizes[:5], "reduce" if reduce else "copy")
