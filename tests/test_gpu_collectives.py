@@ -61,22 +61,28 @@ def run_case(thread, alg, lowering, n, count, dtype, op, seed=0, kind=None, stri
     junk = np.random.default_rng(5).integers(0, 256, sb, dtype=np.uint8) if sb else None
     want_scr = [junk.copy() for _ in range(n)] if sb else None
     oracle.run(ALGS[alg][1], want_in, want_out, count, dt, o, stride, scratch=want_scr)
-    d_in = [to_dev(x) for x in host_in]
-    d_out = [to_dev(sentinel) for _ in range(n)]
-    d_scr = [to_dev(junk) for _ in range(n)] if sb else None
-    # zero-length tensors have a null data_ptr; give the plan a real (unused) address instead
-    pad = to_dev(np.zeros(256, np.uint8))
-    ptr = lambda t: t.data_ptr() if t.numel() else pad.data_ptr()
-    plan = h.Plan(ALGS[alg][0], lowering, [ptr(t) for t in d_in], [ptr(t) for t in d_out], count, dt, o, stride,
-                  [ptr(t) for t in d_scr] if sb else None)
+    # every device buffer carries 64 guard bytes behind its last element: a kernel that runs past a buffer's end
+    # (a tail handled by the wrong tile, a workgroup of a wider grid that should have found nothing to do) shows there
+    guard = np.arange(64, dtype=np.uint8) ^ 0xA5
+    up = lambda a: to_dev(np.concatenate([np.ascontiguousarray(a).view(np.uint8).ravel(), guard]))
+    body = lambda t, like: t[:like.nbytes].cpu().numpy().view(like.dtype).reshape(like.shape)
+    tail = lambda t, like: t[like.nbytes:].cpu().numpy()
+    d_in = [up(x) for x in host_in]
+    d_out = [up(sentinel) for _ in range(n)]
+    d_scr = [up(junk) for _ in range(n)] if sb else None
+    plan = h.Plan(ALGS[alg][0], lowering, [t.data_ptr() for t in d_in], [t.data_ptr() for t in d_out], count, dt, o, stride,
+                  [t.data_ptr() for t in d_scr] if sb else None)
     try:
         assert plan.run(thread) == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
         for r in range(n):
-            assert_same(from_dev(d_in[r], host_in[r]), want_in[r], dt, "in[%d]" % r)
-            assert_same(from_dev(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+            assert_same(body(d_in[r], host_in[r]), want_in[r], dt, "in[%d]" % r)
+            assert_same(body(d_out[r], sentinel), want_out[r], dt, "out[%d]" % r)
+            assert np.array_equal(tail(d_in[r], host_in[r]), guard), "bytes behind in[%d] written" % r
+            assert np.array_equal(tail(d_out[r], sentinel), guard), "bytes behind out[%d] written" % r
             if sb and lowering == h.Lowering.STEPWISE:  # the communication buffer too (bytes never written keep their junk)
-                assert np.array_equal(d_scr[r].cpu().numpy(), want_scr[r]), "scratch[%d]" % r
+                assert np.array_equal(body(d_scr[r], junk), want_scr[r]), "scratch[%d]" % r
+                assert np.array_equal(tail(d_scr[r], junk), guard), "bytes behind scratch[%d] written" % r
         return plan.info.launches, plan.info.algorithmicBytes, plan.info.movedBytes
     finally:
         plan.destroy()
