@@ -128,18 +128,15 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
     else *(uint32_t*)p = v;
 }
 
-// Cache hints.  Measured with the streaming probe (hg_probe.hip) on 8 x 16 MiB ring steps and on 16 x 64 MiB
-// launches whose operands nothing touched recently:
+// Cache hints of the loads.  Measured with the streaming probe (hg_probe.hip) on 8 x 16 MiB ring steps and on
+// 16 x 64 MiB launches whose operands nothing touched recently:
 //   * a launch whose output the next launch reads back from the memory-side cache (a ring step): peer operand
-//     loaded non-temporal, the operand that is overwritten loaded plain, plain stores;
+//     loaded non-temporal, the operand that is overwritten loaded plain;
 //   * a launch that streams (what it writes is more than that cache holds, or nothing reads it soon): every load
-//     and store non-temporal, and no more than three workgroups per CU in flight.
-// Fold launches store non-temporal: nothing they write is read again by the same launch.
+//     non-temporal, and no more than three workgroups per CU in flight.
+// The stores' policies follow further down.
 #ifndef HG_NT_LD_SRC
 #define HG_NT_LD_SRC 1 /* the peer's operand */
-#endif
-#ifndef HG_NT_FOLD_ST
-#define HG_NT_FOLD_ST 1
 #endif
 template <bool NT> __device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec)
 {
@@ -151,6 +148,32 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
     if (NT) __builtin_nontemporal_store(v, (u32x4*)base + vec);
     else ((u32x4*)base)[vec] = v;
 }
+
+// Store policies.  ST_SC1 carries the sc1 cache-policy bit (device scope) and neither of the other two: measured with
+// the probe's reduce_pol / copy_pol kinds, which spell the bits of every access out (hg_probe_policy.txt), it is the
+// best store for the copy / two-input reduce kernels in every situation (streaming reduce 0.825 -> 0.839 of peak
+// over the non-temporal store, ring-step copy 0.845 -> 0.885 over the plain one).  The language has no 128-bit store
+// of a given scope, so it is written out as the instruction: a vector store like the ones the compiler emits, with
+// one more modifier.  The compiler does not see through the asm, so the two wait states it would put between a
+// 128-bit store and an instruction that overwrites the registers holding its data are part of the asm (without
+// them the next address computation lands in the data of the store before: wrong bytes, found by the probe's check=1).
+enum { ST_PLAIN = 0, ST_NT = 1, ST_SC1 = 2 };
+template <int POL> __device__ __forceinline__ void stp(void* base, uint64_t vec, u32x4 v)
+{
+    u32x4* p = (u32x4*)base + vec;
+    if (POL == ST_SC1) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else if (POL == ST_NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+#ifndef HG_ST_SEG2
+#define HG_ST_SEG2 ST_SC1 /* copy / two-input reduce kernels, kept and streaming variants alike */
+#endif
+#ifndef HG_ST_FOLD
+#define HG_ST_FOLD ST_NT /* the k-way folds at bandwidth-bound sizes (8 - 23 streams a lane): sc1 loses there (tree launches - 8 %) */
+#endif
+#ifndef HG_ST_FOLD_DIRECT
+#define HG_ST_FOLD_DIRECT ST_SC1 /* the small, cache-resident fold launches (mesh allreduce 8 x 4 MiB in one launch: 41.8 -> 37.0 us) */
+#endif
 
 // Workgroups are dealt to the 8 XCDs round-robin by their index.  With run > 0 they are renumbered so that each XCD
 // walks runs of `run` consecutive tiles instead of every eighth tile; the workgroups beyond the last whole group of
@@ -192,11 +215,11 @@ template <class Table> __device__ __forceinline__ uint32_t seg_of(const Table& t
     return tab.flat ? tile : find_seg(tab.tile_begin, tab.nseg, tile);
 }
 
-template <int DT, int OP> struct VecItem {
+template <int DT, int OP, int ST = HG_ST_FOLD> struct VecItem {
     typedef u32x4 V;
     static __device__ __forceinline__ V zero() { return V{0u, 0u, 0u, 0u}; }
     static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ldv<HG_NT_LD_SRC>(p, i); }
-    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stv<HG_NT_FOLD_ST>(p, i, v); }
+    static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stp<ST>(p, i, v); }
     static __device__ __forceinline__ V op(V d, V s) { return vec_op<DT, OP>(d, s); }
 };
 

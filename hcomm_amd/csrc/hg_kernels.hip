@@ -32,12 +32,12 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, a[u]);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, a[u]);
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv<STREAM>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+                if (v < nvec) stp<HG_ST_SEG2>(d, v, ldv<HG_NT_LD_SRC>(p, v));
             }
             const uint64_t b = (nvec << 4) + tid; // this tile is the segment's last one: byte tail
             if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
@@ -68,12 +68,12 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stv<STREAM>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+                if (v < nvec) stp<HG_ST_SEG2>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -129,7 +129,7 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = vb + tid + u * HG_BLOCK;
-            if (v < nvec) stv<STREAM>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
+            if (v < nvec) stp<HG_ST_SEG2>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
         }
         if (vb <= nvec && vb + HG_TILE_VECS > nvec) { // the one tile that holds the end of the items
             // fewer than 16 / ES elements before the first item and fewer than that after the last one
@@ -194,12 +194,12 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, a[u]);
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, a[u]);
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stv<STREAM>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+            if (v < nvec) stp<HG_ST_SEG2>(d, v, ldv<HG_NT_LD_SRC>(p, v));
         }
         if (tile == nvec / HG_TILE_VECS) { // the tile the byte tail falls into
             const uint64_t b = (nvec << 4) + tid;
@@ -227,12 +227,12 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stv<STREAM>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stv<STREAM>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+            if (v < nvec) stp<HG_ST_SEG2>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
         }
         if (tile == nvec / HG_TILE_VECS) { // the tile the element tail falls into
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES;

@@ -32,6 +32,13 @@
 //                  depth=1|2|3|7  positions whose loads are in flight ahead of the one being folded
 //                  part=0|1 nout=8
 //
+// kind=reduce_pol|copy_pol   the reduce / copy loop (u=4, 256 lanes, one tile per workgroup) with the cache-policy bits of
+//                  every access spelled out: pd / pl / ps = policy of the dst load, the src load and the store, a sum of
+//                  1 (sc0), 2 (sc1) and 4 (nt); the compiler's own non-temporal accesses are 4.  Other keys as for reduce.
+//                  check=1 (arenas up to 512 MiB): the same launches once more from freshly filled buffers, and again
+//                  with the compiler's own accesses; "mismatch_bytes" counts where the two arenas differ afterwards
+//                  (check=2: the compiler's kernel both times, which says whether the sequence is reproducible at all).
+//
 // kind=start       what a launch costs before it streams: one workgroup copies 16 bytes after `rounds` dependent reads of
 //                  its by-value argument table (each read selects the word the next one fetches, a cache line further
 //                  on, the way a kernel walks from a table's scalars to the row and the pointer they select); the
@@ -65,7 +72,7 @@ namespace {
         }                                                                                          \
     } while (0)
 
-enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6, K_FOLD = 7, K_START = 8 };
+enum { K_REDUCE = 0, K_COPY = 1, K_READ = 2, K_WRITE = 3, K_TRIAD = 4, K_LAT = 5, K_REDUCE_I32 = 6, K_FOLD = 7, K_START = 8, K_REDUCE_POL = 9, K_COPY_POL = 10 };
 
 struct ProbeTab {
     void* dst[64];
@@ -234,6 +241,82 @@ template <uint32_t U> FoldFn pick_fold1(uint32_t depth, uint32_t hs, uint32_t st
     }
 }
 
+// ---- kind=reduce_pol / copy_pol -----------------------------------------------------------------------------
+
+#define POL_CASES(OP)                                  \
+    switch (pol) {                                     \
+        case 0: OP(""); break;                         \
+        case 1: OP(" sc0"); break;                     \
+        case 2: OP(" sc1"); break;                     \
+        case 3: OP(" sc0 sc1"); break;                 \
+        case 4: OP(" nt"); break;                      \
+        case 5: OP(" sc0 nt"); break;                  \
+        case 6: OP(" sc1 nt"); break;                  \
+        default: OP(" sc0 sc1 nt"); break;             \
+    }
+
+__device__ __forceinline__ u32x4 ld_pol(const void* base, uint64_t vec, uint32_t pol)
+{
+    const u32x4* p = (const u32x4*)base + vec;
+    u32x4 r;
+#define LD(BITS) asm volatile("global_load_dwordx4 %0, %1, off" BITS : "=v"(r) : "v"(p) : "memory")
+    POL_CASES(LD)
+#undef LD
+    return r;
+}
+
+__device__ __forceinline__ void st_pol(void* base, uint64_t vec, u32x4 v, uint32_t pol)
+{
+    u32x4* p = (u32x4*)base + vec;
+    // the two idle cycles stand for the wait states the compiler would put between a 128-bit store and an instruction
+    // that overwrites the registers holding its data: it does not see through the asm to know that one is needed
+#define ST(BITS) asm volatile("global_store_dwordx4 %0, %1, off" BITS "\n\ts_nop 1" : : "v"(p), "v"(v) : "memory")
+    POL_CASES(ST)
+#undef ST
+}
+
+struct PolTab {
+    ProbeTab t;
+    uint32_t pd, pl, ps;
+};
+
+template <bool REDUCE> __global__ __launch_bounds__(256) void k_probe_pol(const PolTab pt)
+{
+    extern __shared__ uint8_t lds_pad[];
+    const ProbeTab& t = pt.t;
+    const uint32_t tile = probe_tile(t, blockIdx.x, gridDim.x);
+    const uint32_t s = tile / t.tiles_per_seg;
+    const uint64_t v0 = (uint64_t)(tile - s * t.tiles_per_seg) * 1024u + threadIdx.x;
+    void* d = t.dst[s];
+    const void* p = t.src[s];
+    u32x4 a0, a1, a2, a3, b0, b1, b2, b3;
+    if (REDUCE) {
+        a0 = ld_pol(d, v0, pt.pd);
+        a1 = ld_pol(d, v0 + 256, pt.pd);
+        a2 = ld_pol(d, v0 + 512, pt.pd);
+        a3 = ld_pol(d, v0 + 768, pt.pd);
+    }
+    b0 = ld_pol(p, v0, pt.pl);
+    b1 = ld_pol(p, v0 + 256, pt.pl);
+    b2 = ld_pol(p, v0 + 512, pt.pl);
+    b3 = ld_pol(p, v0 + 768, pt.pl);
+    // the compiler does not know these are loads: wait for them here, and make every use depend on the wait
+    if (REDUCE)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3));
+    else
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3));
+    if (REDUCE) {
+        b0 = vec_op<DT_BF16, OP_SUM>(a0, b0);
+        b1 = vec_op<DT_BF16, OP_SUM>(a1, b1);
+        b2 = vec_op<DT_BF16, OP_SUM>(a2, b2);
+        b3 = vec_op<DT_BF16, OP_SUM>(a3, b3);
+    }
+    st_pol(d, v0, b0, pt.ps);
+    st_pol(d, v0 + 256, b1, pt.ps);
+    st_pol(d, v0 + 512, b2, pt.ps);
+    st_pol(d, v0 + 768, b3, pt.ps);
+}
+
 // ---- kind=start ---------------------------------------------------------------------------------------------
 
 template <uint32_t WORDS> struct StartTab {
@@ -300,7 +383,7 @@ struct Cfg {
     int kind = K_REDUCE;
     uint32_t nseg = 16, seg_mib = 64, pair = 0, u = 4, block = 256, hd = 1, hs = 1, st = 0, pipe = 0, il = 0, wpc = 0, ring = 0,
              lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000,
-             depth = 1, part = 0, nout = 8, rounds = 1, table = 256;
+             depth = 1, part = 0, nout = 8, rounds = 1, table = 256, pd = 4, pl = 4, ps = 4, check = 0;
     uint64_t skew = 0;
     bool zeros = false;
     std::string line;
@@ -375,6 +458,8 @@ bool parse(const std::string& line, Cfg& c)
             else if (v == "lat") c.kind = K_LAT;
             else if (v == "fold") c.kind = K_FOLD;
             else if (v == "start") c.kind = K_START;
+            else if (v == "reduce_pol") c.kind = K_REDUCE_POL;
+            else if (v == "copy_pol") c.kind = K_COPY_POL;
             else return false;
         } else if (k == "data") {
             if (v == "zeros") c.zeros = true;
@@ -407,6 +492,10 @@ bool parse(const std::string& line, Cfg& c)
         else if (k == "depth") c.depth = (uint32_t)n;
         else if (k == "part") c.part = (uint32_t)n;
         else if (k == "nout") c.nout = (uint32_t)n;
+        else if (k == "pd") c.pd = (uint32_t)n;
+        else if (k == "pl") c.pl = (uint32_t)n;
+        else if (k == "ps") c.ps = (uint32_t)n;
+        else if (k == "check") c.check = (uint32_t)n;
         else if (k == "rounds") c.rounds = (uint32_t)n;
         else if (k == "table") c.table = (uint32_t)n;
         else return false;
@@ -606,6 +695,15 @@ int main(int argc, char** argv)
             fflush(stdout);
             continue;
         }
+        const bool pol = c.kind == K_REDUCE_POL || c.kind == K_COPY_POL; // same buffers and tables as reduce / copy
+        const bool pol_reduce = c.kind == K_REDUCE_POL;
+        if (pol) {
+            if (c.u != 4 || c.block != 256 || c.pipe || c.wpc || c.pd > 7 || c.pl > 7 || c.ps > 7) {
+                fprintf(stderr, "hg_probe: unsupported configuration: %s\n", line.c_str());
+                return 2;
+            }
+            c.kind = pol_reduce ? K_REDUCE : K_COPY;
+        }
         const KernelFn fn = pick(c);
         const uint64_t seg = (uint64_t)c.seg_mib << 20;
         const uint64_t tile_bytes = (uint64_t)c.block * c.u * 16u;
@@ -667,26 +765,64 @@ int main(int argc, char** argv)
         uint64_t grid = tiles;
         if (c.wpc && (uint64_t)c.wpc * cus < grid) grid = (uint64_t)c.wpc * cus;
         if (c.pipe && !c.wpc) grid = tiles < (uint64_t)cus * 8u ? tiles : (uint64_t)cus * 8u;
-        if (c.lds) CK(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+        if (c.lds) {
+            CK(hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+            CK(hipFuncSetAttribute((const void*)k_probe_pol<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+            CK(hipFuncSetAttribute((const void*)k_probe_pol<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
+        }
+        auto launch_one = [&](uint32_t k) {
+            if (!pol) {
+                hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[k]);
+                return;
+            }
+            PolTab pt;
+            pt.t = tabs[k];
+            pt.pd = c.pd;
+            pt.pl = c.pl;
+            pt.ps = c.ps;
+            if (pol_reduce) hipLaunchKernelGGL(k_probe_pol<true>, dim3((uint32_t)grid), dim3(256), c.lds, st, pt);
+            else hipLaunchKernelGGL(k_probe_pol<false>, dim3((uint32_t)grid), dim3(256), c.lds, st, pt);
+        };
         uint32_t launch = 0;
-        for (uint32_t i = 0; i < c.warm; ++i, ++launch)
-            hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+        for (uint32_t i = 0; i < c.warm; ++i, ++launch) launch_one(launch % c.sets);
         CK(hipGetLastError());
         CK(hipEventRecord(e0, st));
-        for (uint32_t i = 0; i < c.reps; ++i, ++launch)
-            hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[launch % c.sets]);
+        for (uint32_t i = 0; i < c.reps; ++i, ++launch) launch_one(launch % c.sets);
         CK(hipEventRecord(e1, st));
         CK(hipStreamSynchronize(st));
         CK(hipGetLastError());
         float ms = 0;
         CK(hipEventElapsedTime(&ms, e0, e1));
         ms /= (float)c.reps;
+        long long mismatch = -1;
+        if (pol && c.check) {
+            if (need > (512ull << 20)) {
+                fprintf(stderr, "hg_probe: check=1 wants an arena of at most 512 MiB: %s\n", line.c_str());
+                return 2;
+            }
+            std::vector<uint8_t> got(need), want(need);
+            for (int pass = 0; pass < 2; ++pass) {
+                hipLaunchKernelGGL(k_fill, dim3(8192), dim3(256), 0, st, (uint32_t*)ar.base, ar.bytes / 4, 12345u);
+                for (uint32_t i = 0; i < c.warm + c.reps; ++i) {
+                    if (pass == 0 && c.check == 1) launch_one(i % c.sets); // check=2: the compiler's kernel both times
+                    else hipLaunchKernelGGL(fn, dim3((uint32_t)grid), dim3(c.block), c.lds, st, tabs[i % c.sets]);
+                }
+                CK(hipStreamSynchronize(st));
+                CK(hipMemcpy(pass == 0 ? got.data() : want.data(), ar.base, need, hipMemcpyDeviceToHost));
+            }
+            mismatch = 0;
+            for (uint64_t i = 0; i < need; ++i) mismatch += got[i] != want[i];
+            hipLaunchKernelGGL(k_fill, dim3(8192), dim3(256), 0, st, (uint32_t*)ar.base, ar.bytes / 4, 12345u);
+            CK(hipStreamSynchronize(st));
+        }
         const double per = (c.kind == K_REDUCE || c.kind == K_REDUCE_I32) ? 3.0 : c.kind == K_TRIAD ? 3.0 : c.kind == K_COPY ? 2.0 : 1.0;
         const double moved = per * (double)seg * c.nseg;
         printf("{\"cfg\": \"%s\", \"grid\": %llu, \"tile_bytes\": %llu, \"ms\": %.5f, \"moved_bytes\": %.0f, \"gbs\": %.1f, "
-               "\"frac_of_8000\": %.4f}\n",
+               "\"frac_of_8000\": %.4f",
                line.c_str(), (unsigned long long)grid, (unsigned long long)tile_bytes, ms, moved, moved / ms / 1e6,
                moved / ms / 1e6 / 8000.0);
+        if (mismatch >= 0) printf(", \"mismatch_bytes\": %lld", mismatch);
+        printf("}\n");
         fflush(stdout);
     }
     return 0;
