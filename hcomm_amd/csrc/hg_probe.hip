@@ -30,7 +30,7 @@
 //                  first (part=1, the partials a ring leaves behind), the result to nout outputs.
 //                  keys: nseg seg_mib u(2|4) block hs st lds xcd run skew reps warm sets, and
 //                  depth=1|2|3|7  positions whose loads are in flight ahead of the one being folded
-//                  part=0|1 nout=8
+//                  part=0|1 nout=8 sp=255 (store policy bits as for reduce_pol's ps; 255 = the compiler's store per st=)
 //
 // kind=reduce_pol|copy_pol   the reduce / copy loop (u=4, 256 lanes, one tile per workgroup) with the cache-policy bits of
 //                  every access spelled out: pd / pl / ps = policy of the dst load, the src load and the store, a sum of
@@ -176,6 +176,40 @@ __global__ __launch_bounds__(1024) void k_probe(const ProbeTab t)
     }
 }
 
+// ---- accesses with their cache-policy bits spelled out (kinds reduce_pol / copy_pol, fold with sp=) ------------
+
+#define POL_CASES(OP)                                  \
+    switch (pol) {                                     \
+        case 0: OP(""); break;                         \
+        case 1: OP(" sc0"); break;                     \
+        case 2: OP(" sc1"); break;                     \
+        case 3: OP(" sc0 sc1"); break;                 \
+        case 4: OP(" nt"); break;                      \
+        case 5: OP(" sc0 nt"); break;                  \
+        case 6: OP(" sc1 nt"); break;                  \
+        default: OP(" sc0 sc1 nt"); break;             \
+    }
+
+__device__ __forceinline__ u32x4 ld_pol(const void* base, uint64_t vec, uint32_t pol)
+{
+    const u32x4* p = (const u32x4*)base + vec;
+    u32x4 r;
+#define LD(BITS) asm volatile("global_load_dwordx4 %0, %1, off" BITS : "=v"(r) : "v"(p) : "memory")
+    POL_CASES(LD)
+#undef LD
+    return r;
+}
+
+__device__ __forceinline__ void st_pol(void* base, uint64_t vec, u32x4 v, uint32_t pol)
+{
+    u32x4* p = (u32x4*)base + vec;
+    // the two idle cycles stand for the wait states the compiler would put between a 128-bit store and an instruction
+    // that overwrites the registers holding its data: it does not see through the asm to know that one is needed
+#define ST(BITS) asm volatile("global_store_dwordx4 %0, %1, off" BITS "\n\ts_nop 1" : : "v"(p), "v"(v) : "memory")
+    POL_CASES(ST)
+#undef ST
+}
+
 // ---- kind=fold ----------------------------------------------------------------------------------------------
 
 struct FoldProbeTab {
@@ -183,6 +217,7 @@ struct FoldProbeTab {
     uint8_t* out[8]; // receiver r likewise
     uint64_t seg_bytes;
     uint32_t tiles_per_seg, nseg, nout, part, xcd, run;
+    uint32_t sp; // store policy bits (1 sc0, 2 sc1, 4 nt), or 255: the compiler's store as the template says
 };
 
 template <uint32_t U, uint32_t DEPTH, bool HS, bool ST>
@@ -215,12 +250,18 @@ __global__ __launch_bounds__(1024) void k_probe_fold(const FoldProbeTab t)
         for (uint32_t u = 0; u < U; ++u) acc[u] = vec_op<DT_BF16, OP_SUM>(x[j][u], acc[u]);
         if (t.part) {
 #pragma unroll
-            for (uint32_t u = 0; u < U; ++u) stv<ST>(t.in[j] + so, v0 + u * blockDim.x, acc[u]);
+            for (uint32_t u = 0; u < U; ++u) {
+                if (t.sp == 255u) stv<ST>(t.in[j] + so, v0 + u * blockDim.x, acc[u]);
+                else st_pol(t.in[j] + so, v0 + u * blockDim.x, acc[u], t.sp);
+            }
         }
     }
     for (uint32_t r = 0; r < t.nout; ++r) {
 #pragma unroll
-        for (uint32_t u = 0; u < U; ++u) stv<ST>(t.out[r] + so, v0 + u * blockDim.x, acc[u]);
+        for (uint32_t u = 0; u < U; ++u) {
+            if (t.sp == 255u) stv<ST>(t.out[r] + so, v0 + u * blockDim.x, acc[u]);
+            else st_pol(t.out[r] + so, v0 + u * blockDim.x, acc[u], t.sp);
+        }
     }
 }
 
@@ -239,40 +280,6 @@ template <uint32_t U> FoldFn pick_fold1(uint32_t depth, uint32_t hs, uint32_t st
         case 7: return pick_fold2<U, 7>(hs, st);
         default: return nullptr;
     }
-}
-
-// ---- kind=reduce_pol / copy_pol -----------------------------------------------------------------------------
-
-#define POL_CASES(OP)                                  \
-    switch (pol) {                                     \
-        case 0: OP(""); break;                         \
-        case 1: OP(" sc0"); break;                     \
-        case 2: OP(" sc1"); break;                     \
-        case 3: OP(" sc0 sc1"); break;                 \
-        case 4: OP(" nt"); break;                      \
-        case 5: OP(" sc0 nt"); break;                  \
-        case 6: OP(" sc1 nt"); break;                  \
-        default: OP(" sc0 sc1 nt"); break;             \
-    }
-
-__device__ __forceinline__ u32x4 ld_pol(const void* base, uint64_t vec, uint32_t pol)
-{
-    const u32x4* p = (const u32x4*)base + vec;
-    u32x4 r;
-#define LD(BITS) asm volatile("global_load_dwordx4 %0, %1, off" BITS : "=v"(r) : "v"(p) : "memory")
-    POL_CASES(LD)
-#undef LD
-    return r;
-}
-
-__device__ __forceinline__ void st_pol(void* base, uint64_t vec, u32x4 v, uint32_t pol)
-{
-    u32x4* p = (u32x4*)base + vec;
-    // the two idle cycles stand for the wait states the compiler would put between a 128-bit store and an instruction
-    // that overwrites the registers holding its data: it does not see through the asm to know that one is needed
-#define ST(BITS) asm volatile("global_store_dwordx4 %0, %1, off" BITS "\n\ts_nop 1" : : "v"(p), "v"(v) : "memory")
-    POL_CASES(ST)
-#undef ST
 }
 
 struct PolTab {
@@ -383,7 +390,7 @@ struct Cfg {
     int kind = K_REDUCE;
     uint32_t nseg = 16, seg_mib = 64, pair = 0, u = 4, block = 256, hd = 1, hs = 1, st = 0, pipe = 0, il = 0, wpc = 0, ring = 0,
              lds = 0, xcd = 0, run = 128, reps = 10, warm = 2, sets = 1, xk = 0, mod = 8, cls = 0, gran = 4096, iters = 2000,
-             depth = 1, part = 0, nout = 8, rounds = 1, table = 256, pd = 4, pl = 4, ps = 4, check = 0;
+             depth = 1, part = 0, nout = 8, rounds = 1, table = 256, pd = 4, pl = 4, ps = 4, check = 0, sp = 255;
     uint64_t skew = 0;
     bool zeros = false;
     std::string line;
@@ -496,6 +503,7 @@ bool parse(const std::string& line, Cfg& c)
         else if (k == "pl") c.pl = (uint32_t)n;
         else if (k == "ps") c.ps = (uint32_t)n;
         else if (k == "check") c.check = (uint32_t)n;
+        else if (k == "sp") c.sp = (uint32_t)n;
         else if (k == "rounds") c.rounds = (uint32_t)n;
         else if (k == "table") c.table = (uint32_t)n;
         else return false;
@@ -671,6 +679,7 @@ int main(int argc, char** argv)
                 t.part = c.part;
                 t.xcd = c.xcd;
                 t.run = c.run ? c.run : 1u;
+                t.sp = c.sp;
             }
             const uint64_t grid = (uint64_t)tabs[0].tiles_per_seg * c.nseg;
             if (c.lds) CK(hipFuncSetAttribute((const void*)ffn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)c.lds));
