@@ -70,13 +70,14 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
  * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip; 16 KiB tiles, bf16 SUM,
  * seeded non-zero data, fractions of 8 TB/s).  Two regimes:
  *   kept      what the launch writes fits the memory-side cache and a later launch reads it back from there (a ring
- *             step): plain stores, the overwritten operand loaded plain, XCDs walking runs of 128 tiles.
+ *             step): the overwritten operand loaded plain, XCDs walking runs of 128 tiles.
  *             8 x 16 MiB ring steps: reduce 0.860 (0.827 with that operand loaded non-temporal and tiles as dealt),
  *             copy 0.873 with at most five workgroups per CU (0.864 without that bound).
- *   streaming everything non-temporal and at most three workgroups per CU in flight.  16 x 64 MiB that nothing touched
+ *   streaming every load non-temporal and at most three workgroups per CU in flight.  16 x 64 MiB that nothing touched
  *             recently: reduce 0.823 with runs of 32 tiles (0.795 without the bound, 0.711 with the grid held at 32
  *             workgroups per CU), copy 0.808 with runs of 128 (0.744 without the bound).
- * The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
+ * (Figures taken with plain / non-temporal stores; both regimes now store with the sc1 policy, which is ahead of either:
+ * hg_device.hpp.)  The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
  * Every figure can be overridden from the environment for experiments.
  */
 enum {

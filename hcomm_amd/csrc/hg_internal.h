@@ -100,7 +100,7 @@ typedef struct {
 uint64_t hg_grid_blocks(uint64_t total_tiles);
 
 /* Launchers.  stream is a hipStream_t.  Return a HcclResult-compatible code. */
-/* streaming: non-temporal stores (and, for the reduce, a non-temporal load of the operand it overwrites);
+/* streaming: the launch shape for output nothing reads back soon (and, for the reduce, a non-temporal load of the operand it overwrites);
  * lds: bytes of dynamic LDS per workgroup, asked for only to bound the workgroups a CU runs at once */
 int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
 int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);

@@ -14,8 +14,10 @@ namespace {
 // ---- batched copy ------------------------------------------------------------------------------
 
 // STREAM: nothing of what the launch writes will be found in the memory-side cache by a later launch (there is more
-// of it than that cache holds, or nothing reads it soon): store with the non-temporal hint.  The launch's dynamic
-// LDS size is not used as memory: it bounds the workgroups a CU runs at once (hg_shape_seg2 in hg_batch.c).
+// of it than that cache holds, or nothing reads it soon).  Since every store of these kernels carries the sc1 policy
+// (stp<HG_ST_SEG2>) the copy's two variants differ in their launch shape only - occupancy bound and XCD runs, set
+// by hg_shape_seg2 in hg_batch.c - and the reduce's also in how the overwritten operand is loaded.  The launch's
+// dynamic LDS size is not used as memory: it bounds the workgroups a CU runs at once.
 template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
 {
     const uint32_t total = tab.tile_begin[tab.nseg];

@@ -327,7 +327,7 @@ typedef struct {
     uint32_t rows;   /* copy / two-input reduce: > 0 = two-dimensional grid of `rows` tiles by nseg segments, every
                         address read in one round (the k_*_rows kernels); 0 = one-dimensional grid over the table's
                         tiles.  Folds: 1 = small launch whose addresses the host resolves (the k_fold_*_direct kernels) */
-    uint32_t streaming; /* copy / two-input reduce: 1 = every access non-temporal */
+    uint32_t streaming; /* copy / two-input reduce: 1 = the variant for output that nothing reads back soon */
 } HcommGfxLaunchRecord;
 
 typedef enum {
