@@ -131,7 +131,7 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = vb + tid + u * HG_BLOCK;
-            if (v < nvec) stp<HG_ST_SEG2>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
+            if (v < nvec) stv<STREAM>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]); // sc1 loses here (0.93 -> 1.00 ms on the odd-block reduce-scatter)
         }
         if (vb <= nvec && vb + HG_TILE_VECS > nvec) { // the one tile that holds the end of the items
             // fewer than 16 / ES elements before the first item and fewer than that after the last one
