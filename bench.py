@@ -84,6 +84,8 @@ WORKLOADS = {
     "order_preserved_ar_bf16_n8_128MiB": ("order_preserved_ar", 8, 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     # the double-ring reduce-scatter executor on one server with DMA reduce
     "dbring_rs_bf16_n8_16MiB": ("doublering_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
+    # the same executor over 2 servers x 8 devices, ring between the servers (blocks of 8 MiB)
+    "dbringhier_ring_rs_bf16_2x8_8MiB": ("doublering_hier_rs", (2, 8), 4194304, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving allreduce executor over two levels: plant + fold inside the servers, then between them
     "ophier_ring_ar_bf16_2x8_128MiB": ("ophier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "ophierrs_ring_rs_bf16_2x8_8MiB": ("ophierrs_ring_rs_stage", (2, 8), 4194304, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -200,9 +202,12 @@ def run_workload(args, torch, h, dev, stream, thread):
     if alg_name.startswith("hier") or alg_name.startswith("dbring_") or mesh0 or ophier or ophrs:
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
+    dbhrs = None  # (servers, ranks per server) of the double-ring reduce-scatter executor over several servers
+    if alg_name == "doublering_hier_rs":
+        dbhrs, n = n, n[0] * n[1]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     # one-server executors on user memory (DMA reduce)
-    plant = alg_name in ("order_preserved_rs", "doublering_rs", "order_preserved_ar", "order_preserved_small")
+    plant = alg_name in ("order_preserved_rs", "doublering_rs", "doublering_hier_rs", "order_preserved_ar", "order_preserved_small")
     opsmall = alg_name == "order_preserved_small"
     opar = alg_name == "order_preserved_ar"
     # the order-preserving executors also have a single-launch lowering
@@ -216,7 +221,8 @@ def run_workload(args, torch, h, dev, stream, thread):
         return mesh_sweep(args, torch, h, dev, stream, thread, n, dt, unit)
 
     nbytes = count * unit
-    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs", "order_preserved_small")
+    in_count = n * count if (alg_name in ("local_reduce_rs", "order_preserved_rs", "doublering_rs", "doublering_hier_rs",
+                                          "order_preserved_small")
                             or hier_rs or ophrs) else count
     pristine = make_inputs(torch, dev, n, in_count, "fp32prod" if opname == "prod" else dtname)
     d_in = [torch.empty(in_count * unit, dtype=torch.uint8, device=dev) for _ in range(n)]
@@ -249,6 +255,9 @@ def run_workload(args, torch, h, dev, stream, thread):
         if hier_rs:
             return h.HierReduceScatterPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                            [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, mesh=mesh0)
+        if dbhrs:
+            return h.DoubleRingHierReduceScatterPlan(h.Alg.REDUCE_SCATTER_RING, dbhrs[0], dbhrs[1], in_ptrs, out_ptrs,
+                                                     [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
         if dbrs:
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
         if opfused and low == h.Lowering.FUSED:  # one launch on the user buffers, no CCL buffer
@@ -399,7 +408,7 @@ def run_workload(args, torch, h, dev, stream, thread):
                 "nhr": oracle.ALG_ALLREDUCE_NHR, "nb": oracle.ALG_ALLREDUCE_NB,
                 "local_reduce_rs": oracle.ALG_RS_LOCAL_REDUCE, "nhr_oneshot": oracle.ALG_ALLREDUCE_NHR_ONESHOT,
                 "doubling": oracle.ALG_ALLREDUCE_DOUBLING,
-                "order_preserved_rs": None, "doublering_rs": None, "order_preserved_ar": None,
+                "order_preserved_rs": None, "doublering_rs": None, "doublering_hier_rs": None, "order_preserved_ar": None,
                 "order_preserved_small": None}[alg_name]
         oop = {"sum": oracle.SUM, "prod": oracle.PROD, "max": oracle.MAX, "min": oracle.MIN}[opname]
         npdt = oracle.NP_STORAGE[odt]
@@ -410,6 +419,9 @@ def run_workload(args, torch, h, dev, stream, thread):
         if hier_rs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2)
                             for o in oracle.trace_hier_rs(oalg, hier[0], hier[1], count, ccl_bytes, odt, mesh=mesh0))
+        elif dbhrs:
+            alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs_servers(
+                oracle.ALG_RS_RING_STAGE, dbhrs[0], dbhrs[1], count, ccl_bytes, odt))
         elif dbrs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs(n, count, ccl_bytes, odt))
         elif opsmall:
@@ -440,6 +452,9 @@ def run_workload(args, torch, h, dev, stream, thread):
             if hier_rs:
                 oracle.run_hier_rs(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop,
                                    mesh=mesh0)
+            elif dbhrs:
+                oracle.run_dbring_rs_servers(oracle.ALG_RS_RING_STAGE, dbhrs[0], dbhrs[1], ins, outs, host_ccl[0], count,
+                                             ccl_bytes, odt, oop)
             elif dbrs:
                 oracle.run_dbring_rs(ins, outs, host_ccl[0], count, ccl_bytes, odt, oop)
             elif opsmall:

@@ -35,6 +35,7 @@ __all__ = [
     "OrderPreservedHierReduceScatterPlan", "order_preserved_hier_rs_emit", "order_preserved_hier_rs_check",
     "HierReduceScatterPlan", "hier_rs_emit", "hier_rs_check",
     "DoubleRingReduceScatterPlan", "dbring_rs_emit", "dbring_rs_check",
+    "DoubleRingHierReduceScatterPlan", "dbring_hier_rs_emit", "dbring_hier_rs_check",
     "HcommGfxAllReduceLocalReduceNoAlloc", "NOALLOC_SCRATCH_BYTES", "NOALLOC_MAX_RANKS",
     "OpBasePlan", "OpListPlan", "opbase_emit", "opbase_check", "opbase_max_count", "BUF_USER_IN", "BUF_USER_OUT",
 ]
@@ -845,6 +846,47 @@ def dbring_rs_check(n_ranks, count, ccl_bytes, dtype):
     rep = CheckReport()
     check(_dbrs_check(n_ranks, count, ccl_bytes, dtype, C.byref(rep)), "HcommGfxDoubleRingReduceScatterCheck")
     return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+_dbhrs_emit = _sig("HcommGfxDoubleRingHierReduceScatterEmit", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+                   C.POINTER(SchedOp), _u64, C.POINTER(_u64))
+_dbhrs_check = _sig("HcommGfxDoubleRingHierReduceScatterCheck", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+                    C.POINTER(CheckReport))
+_dbhrs_plan = _sig("HcommGfxDoubleRingHierReduceScatterPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp),
+                   C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+
+
+def dbring_hier_rs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    n = _u64(0)
+    check(_dbhrs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
+          "HcommGfxDoubleRingHierReduceScatterEmit")
+    ops = (SchedOp * max(n.value, 1))()
+    check(_dbhrs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
+          "HcommGfxDoubleRingHierReduceScatterEmit")
+    return [ops[i].astuple() for i in range(n.value)]
+
+
+def dbring_hier_rs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+    rep = CheckReport()
+    check(_dbhrs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
+          "HcommGfxDoubleRingHierReduceScatterCheck")
+    return rep.conflicts, rep.semanticErrors, rep.message.decode()
+
+
+class DoubleRingHierReduceScatterPlan(Plan):
+    """HcommGfxDoubleRingHierReduceScatterPlanCreate: the double-ring reduce-scatter executor over several servers."""
+
+    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_bytes, count, dtype, op):
+        n = len(user_in)
+        assert n == n_servers * n_local
+        self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in)]
+        p = _vp(0)
+        check(_dbhrs_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype,
+                          op, C.byref(p)), "HcommGfxDoubleRingHierReduceScatterPlanCreate")
+        self._p = p
+        info = PlanInfo()
+        check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")
+        self.info = info
 
 
 class DoubleRingReduceScatterPlan(Plan):

@@ -447,6 +447,20 @@ int32_t HcommGfxHierReduceScatterCheck(
     return rc;
 }
 
+int32_t HcommGfxDoubleRingHierReduceScatterCheck(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxCheckReport* rep)
+{
+    if (!rep) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = HcommGfxOpListCheck(l.ops, l.n, nServers * nLocal, HCOMM_GFX_EXPECT_REDUCE_SCATTER_USER, count, 0,
+                             HcommGfxDataTypeSize(dataType), rep);
+    hg_oplist_free(&l);
+    return rc;
+}
+
 int32_t HcommGfxDoubleRingReduceScatterCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* rep)
 {

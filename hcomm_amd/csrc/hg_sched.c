@@ -1421,6 +1421,126 @@ int32_t HcommGfxDoubleRingReduceScatterEmit(
     return HCCL_SUCCESS;
 }
 
+/* ---- the double-ring reduce-scatter executor over the servers of one super pod (op-base mode, DMA reduce) ---------- */
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor with several servers (KernelRun of its base,
+ * coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:595-812, level2RankSize 1).  With S
+ * servers of N devices, rank = server * N + local index, block g = the output of rank g, per chunk of c bytes per block
+ * and dir = -1 for ring 0 (first shares), +1 for ring 1 (second shares), every rank (s, r):
+ *   step 0: fetches the shares of blocks k * N + (r + dir) and k * N + (r + 2 dir), k = 0 .. S - 1, from its user input
+ *     into its CCL input - every ring position carries S slices, one per server (FillMultiRingSlice :213-233, user
+ *     offsets :297-313; aligned_reduce_scatter_double_ring.cc:305-332);
+ *   step 1 + t, t < N - 1: folds the shares of blocks k * N + (r + (2 + t) dir) of rank (s, r + dir)'s CCL input into
+ *     its own and, except in the last of these steps, fetches those of blocks k * N + (r + (3 + t) dir) (:366-425; the
+ *     user output address is null here, :664-670, so nothing goes to the user output yet);
+ *   then the reduce-scatter between the servers (ring, NHR or NB, :689-746) in place on the CCL input buffers of the
+ *     ranks (0, r) .. (S - 1, r), slice i = block i * N + r (:327-338);
+ *   last: block s * N + r from the CCL input to the user output (:800-808). */
+static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32_t n, uint64_t count, uint64_t ccl_bytes,
+                                   uint32_t unit)
+{
+    const uint32_t total = n_srv * n;
+    const uint64_t max_count = ccl_bytes / total / 128u * 128u / unit; /* CalcLoopMaxCount, :167-173 */
+    if (max_count == 0) return HCCL_E_PARA;
+    const uint64_t stride = count * unit;
+    uint32_t step = 0, map[HCOMM_GFX_MAX_RANKS];
+    uint64_t user_off = 0;
+    HcommGfxSlice sl[HCOMM_GFX_MAX_RANKS];
+    for (uint64_t left = count; left > 0;) {
+        const uint64_t cur = left > max_count ? max_count : left;
+        const uint64_t c = cur * unit;
+        uint64_t first = ((c + 1) / 2 + 127u) / 128u * 128u; /* MutliSegSlicePrepare, coll_comm_executor.cc:2011-2052 */
+        if (first > c) first = c;
+        const uint64_t off[2] = {0, first}, len[2] = {first, c - first};
+#define BLK(r, k, ring) (((r) + (uint64_t)n * 4u + (uint64_t)(k) * ((ring) ? 1u : n - 1u)) % n)
+        for (uint32_t g = 0; g < total; ++g) {
+            const uint32_t r = g % n;
+            for (uint32_t k = 0; k < n_srv; ++k)
+                for (uint32_t ring = 0; ring < 2; ++ring)
+                    for (uint32_t j = 1; j <= 2; ++j) {
+                        const uint64_t b = (uint64_t)k * n + BLK(r, j, ring);
+                        CHK(push(l, step, COPY, g, IN, b * c + off[ring], g, UIN, user_off + b * stride + off[ring], len[ring]));
+                    }
+        }
+        for (uint32_t t = 0; t + 1 < n; ++t)
+            for (uint32_t g = 0; g < total; ++g) {
+                const uint32_t r = g % n, srv = g / n;
+                for (uint32_t ring = 0; ring < 2; ++ring) {
+                    const uint32_t peer = srv * n + (uint32_t)BLK(r, 1, ring);
+                    for (uint32_t k = 0; k < n_srv; ++k) {
+                        const uint64_t b = (uint64_t)k * n + BLK(r, 2 + t, ring);
+                        CHK(push(l, step + 1 + t, REDUCE, g, IN, b * c + off[ring], peer, IN, b * c + off[ring], len[ring]));
+                        if (t + 2 == n) continue;
+                        const uint64_t nb = (uint64_t)k * n + BLK(r, 3 + t, ring);
+                        CHK(push(l, step + 1 + t, COPY, g, IN, nb * c + off[ring], g, UIN, user_off + nb * stride + off[ring], len[ring]));
+                    }
+                }
+            }
+#undef BLK
+        step += n;
+        {
+            HgOpList sub;
+            memset(&sub, 0, sizeof(sub));
+            for (uint32_t i = 0; i < n_srv; ++i) {
+                sl[i].offset = c * n * i;
+                sl[i].size = c;
+            }
+            int rc;
+            if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) rc = ring_rs(&sub, n_srv, sl, 0);
+            else if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_NB) rc = nb_rs(&sub, n_srv, sl);
+            else {
+                uint32_t order[HCOMM_GFX_MAX_RANKS];
+                nhr_slice_map(n_srv, 1, order);
+                rc = nhr_rs(&sub, n_srv, sl, order, 0);
+            }
+            uint32_t used = 0;
+            for (uint32_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
+                for (uint32_t srv = 0; srv < n_srv; ++srv) map[srv] = srv * n + i;
+                rc = append_mapped(l, &sub, map, step, c * i, 0, &used);
+            }
+            hg_oplist_free(&sub);
+            CHK(rc);
+            step += alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_RING ? n_srv - 1 : ceil_log2(n_srv);
+        }
+        for (uint32_t g = 0; g < total; ++g) CHK(push(l, step, COPY, g, UOUT, user_off, g, IN, c * g, c));
+        ++step;
+        user_off += c;
+        left -= cur;
+    }
+    return order_by_step_rank(l);
+}
+
+int hg_schedule_dbring_rs_servers(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                  uint64_t ccl_bytes, int dtype)
+{
+    memset(l, 0, sizeof(*l));
+    const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
+    if (unit == 0 || count > HG_MAX_COUNT || n_servers < 2 || n_local < 3 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS)
+        return HCCL_E_PARA;
+    if (alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RING && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
+        return HCCL_E_PARA;
+    const int rc = dbring_rs_servers_build(l, alg1, n_servers, n_local, count, ccl_bytes, unit);
+    if (rc != HCCL_SUCCESS) hg_oplist_free(l);
+    return rc;
+}
+
+int32_t HcommGfxDoubleRingHierReduceScatterEmit(
+    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
+    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+{
+    if (!n) return HCCL_E_PTR;
+    HgOpList l;
+    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    if (rc != HCCL_SUCCESS) return rc;
+    *n = l.n;
+    if (ops) {
+        const uint64_t m = l.n < cap ? l.n : cap;
+        if (m) memcpy(ops, l.ops, m * sizeof(*ops));
+    }
+    hg_oplist_free(&l);
+    return HCCL_SUCCESS;
+}
+
 /* ---- the order-preserving reduce-scatter executor (one server, op-base mode) ------------------------------------- */
 
 /* CollReduceScatterOrderPreservedExecutor (coll_executor/coll_reduce_scatter/

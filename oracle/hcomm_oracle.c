@@ -2089,6 +2089,191 @@ int orc_run_dbring_rs(uint32_t n, void* const* user_in, void* const* user_out, v
     return rc;
 }
 
+/* ---- the double-ring reduce-scatter executor over servers of one super pod, op-base mode with DMA reduce -------- */
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor with level1RankSize = n_servers > 1 and level2RankSize = 1 for one
+ * rank and one chunk (KernelRun of its base, exec/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:
+ * 595-812):
+ *   level 0: every ring position carries n_servers slices, one per server (FillMultiRingSlice :213-233: the position's
+ *     share + level1Idx * sliceNum * output size), their user-memory twins at block index * count * unit + the ring's
+ *     first slice offset (:297-313), and AlignedReduceScatterDoubleRing runs with the user input address only
+ *     (:664-670: outputAddr = nullptr), so every fold stays in the CCL input buffer
+ *     (tpl/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc: the init step walks the slices of a position,
+ *     :305-332 and :232-249; so does every step, :366-425, :583-590);
+ *   level 1: reduce-scatter between the servers (ring, NHR or NB, :689-746) in place on the CCL input buffer, slice i =
+ *     the block of the i-th server's rank with this local index (CalLevel1DataSegsSlice :327-338);
+ *   last: the own block from the CCL input to the user output (:800-808).
+ * Steps: 0 the init step, 1 .. n_local - 1 the ring steps, then the level-1 steps, then the copy out. */
+static void prog_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local,
+                                   uint64_t cur_size, uint64_t stride_bytes, uint32_t step0)
+{
+    const uint32_t n = n_local, per = n_servers;
+    const uint32_t server = rank / n_local, local = rank % n_local;
+    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
+    for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
+    for (uint32_t s = 0; s < n_servers; s++) level1[s] = s * n_local + local;
+
+    /* multiStreamSlice: ReduceScatterRingSlicePrepare with sliceNum = n_local, as on one server */
+    OrcSlice seg[ORC_MAX_RANKS], multi_seg[ORC_MAX_RANKS][2], ms[2][ORC_MAX_RANKS];
+    uint32_t order[2][ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n; i++) {
+        seg[i].size = cur_size;
+        seg[i].offset = cur_size * i;
+    }
+    for (uint32_t rank_id = 0; rank_id < n; rank_id++) { /* MutliSegSlicePrepare, exec/coll_comm_executor.cc:2011-2052 */
+        const uint64_t size_per_ring = ((seg[rank_id].size + 1) / 2 + 127) / 128 * 128;
+        uint64_t residue = seg[rank_id].size;
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const uint64_t single = size_per_ring < residue ? size_per_ring : residue;
+            multi_seg[rank_id][ring].size = single;
+            multi_seg[rank_id][ring].offset = single ? seg[rank_id].offset + seg[rank_id].size - residue : seg[rank_id].offset;
+            residue -= single;
+        }
+    }
+    for (uint32_t i = 0; i < n; i++) order[0][i] = i;
+    order[1][0] = 0;
+    for (uint32_t i = 1; i < n; i++) order[1][i] = order[0][n - i];
+    for (uint32_t ring = 0; ring < 2; ring++)
+        for (uint32_t i = 0; i < n; i++) ms[ring][i] = multi_seg[order[ring][i]][ring];
+    /* level0DataSegsSlice and multRingsUserMemSlice: index = ring position * n_servers + level1Idx */
+    OrcSlice* ccl[2];
+    OrcSlice* user[2];
+    for (uint32_t ring = 0; ring < 2; ring++) {
+        ccl[ring] = (OrcSlice*)malloc(sizeof(OrcSlice) * n * per);
+        user[ring] = (OrcSlice*)malloc(sizeof(OrcSlice) * n * per);
+        if (!ccl[ring] || !user[ring]) {
+            t->oom = 1;
+            for (uint32_t q = 0; q <= ring; q++) {
+                free(ccl[q]);
+                free(user[q]);
+            }
+            return;
+        }
+        for (uint32_t level0_idx = 0; level0_idx < n; level0_idx++)
+            for (uint32_t level1_idx = 0; level1_idx < per; level1_idx++) {
+                OrcSlice* c = &ccl[ring][level0_idx * per + level1_idx];
+                c->size = ms[ring][level0_idx].size;
+                c->offset = ms[ring][level0_idx].offset + (uint64_t)level1_idx * n * cur_size;
+                OrcSlice* u = &user[ring][level0_idx * per + level1_idx];
+                u->size = c->size;
+                u->offset = (c->offset / cur_size) * stride_bytes + ms[ring][0].offset;
+            }
+    }
+
+    g_rank_map = level0;
+    g_step_base = step0;
+    const uint32_t pre[2] = {(local + n - 1) % n, (local + 1) % n};
+    const uint32_t init0[2] = {(local + n - 1) % n, (n - local - 1 + n) % n};
+    const uint32_t init1[2] = {(local + n - 2) % n, (n - local - 2 + n) % n};
+    for (uint32_t k = 0; k < per; k++)      /* RunInitStep, :305-332 */
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            const uint32_t a = init0[ring] * per + k, b = init1[ring] * per + k;
+            emit(t, 0, K_COPY, local, B_IN, ccl[ring][a].offset, local, B_UIN, user[ring][a].offset, ccl[ring][a].size);
+            emit(t, 0, K_COPY, local, B_IN, ccl[ring][b].offset, local, B_UIN, user[ring][b].offset, ccl[ring][b].size);
+        }
+    uint32_t rx[2] = {(local + n - 2) % n, (n - local - 2 + n) % n};
+    uint32_t sub[2] = {(local + n - 3) % n, (n - local - 3 + n) % n};
+    for (uint32_t step = 0; step < n - 1; step++) { /* RunReduceScatter, :640-685 */
+        for (uint32_t ring = 0; ring < 2; ring++) {
+            for (uint32_t k = 0; k < per; k++) { /* PrepareDeviceMems, :371-425, outputAddr == nullptr */
+                const OrcSlice* rx_slice = &ccl[ring][rx[ring] * per + k];
+                const OrcSlice* ccl_slice = &ccl[ring][sub[ring] * per + k];
+                const OrcSlice* sub_slice = &user[ring][sub[ring] * per + k];
+                emit(t, 1 + step, K_REDUCE, local, B_IN, rx_slice->offset, pre[ring], B_IN, rx_slice->offset, rx_slice->size);
+                if (step != n - 2)
+                    emit(t, 1 + step, K_COPY, local, B_IN, ccl_slice->offset, local, B_UIN, sub_slice->offset, ccl_slice->size);
+            }
+            rx[ring] = (rx[ring] + n - 1) % n;
+            sub[ring] = (sub[ring] + n - 1) % n;
+        }
+    }
+    for (uint32_t ring = 0; ring < 2; ring++) {
+        free(ccl[ring]);
+        free(user[ring]);
+    }
+
+    /* between the servers, :689-746 */
+    OrcSlice sl[ORC_MAX_RANKS];
+    for (uint32_t i = 0; i < n_servers; i++) { /* CalLevel1DataSegsSlice, :327-338 */
+        sl[i].size = cur_size;
+        sl[i].offset = (uint64_t)level1[i] * cur_size;
+    }
+    g_rank_map = level1;
+    g_step_base = step0 + n;
+    uint32_t level1_steps;
+    if (alg1 == ORC_ALG_RS_RING_STAGE) {
+        prog_ring_rs(t, server, n_servers, sl, NULL);
+        level1_steps = n_servers - 1;
+    } else if (alg1 == ORC_ALG_RS_NB) {
+        prog_nb_rs(t, server, n_servers, sl, NULL);
+        level1_steps = nhr_steps(n_servers);
+    } else {
+        uint32_t slice_map[ORC_MAX_RANKS];
+        nhr_rank_mapping(n_servers, 1, slice_map);
+        prog_nhr_rs(t, server, n_servers, sl, NULL, slice_map, 0); /* Prepare(reduceAttr, false), :738 */
+        level1_steps = nhr_steps(n_servers);
+    }
+    g_rank_map = NULL;
+    /* :800-808: CalcSrcMemOffset = userRank * output size */
+    g_step_base = step0 + n + level1_steps;
+    emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_IN, (uint64_t)rank * cur_size, cur_size);
+    g_step_base = 0;
+}
+
+static int build_trace_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                         uint64_t ccl_bytes, int dtype)
+{
+    memset(t, 0, sizeof(*t));
+    const uint32_t unit = orc_dtype_size(dtype);
+    if (unit == 0 || n_servers < 2 || n_local < 3 || n_servers * n_local > ORC_MAX_RANKS) return -1;
+    if (alg1 != ORC_ALG_RS_RING_STAGE && alg1 != ORC_ALG_RS_NHR && alg1 != ORC_ALG_RS_NB) return -1;
+    const uint32_t n = n_servers * n_local;
+    const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit; /* CalcLoopMaxCount, :167-173 */
+    if (max_count == 0) return -1;
+    const uint32_t level1_steps = alg1 == ORC_ALG_RS_RING_STAGE ? n_servers - 1 : nhr_steps(n_servers);
+    uint32_t step0 = 0;
+    uint64_t cur_count = 0, user_off = 0;
+    for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
+        cur_count = count_left > max_count ? max_count : count_left;
+        g_user_off = user_off;
+        for (uint32_t r = 0; r < n; r++)
+            prog_dbring_rs_servers(t, alg1, r, n_servers, n_local, cur_count * unit, count * unit, step0);
+        g_user_off = 0;
+        if (t->oom) {
+            free(t->ops);
+            return -2;
+        }
+        step0 += n_local + level1_steps + 1;
+        user_off += cur_count * unit;
+    }
+    return sort_trace(t);
+}
+
+int64_t orc_trace_dbring_rs_servers(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
+                                    int dtype, OrcOp* out, uint64_t cap)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring_rs_servers(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    const uint64_t m = t.n < cap ? t.n : cap;
+    if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
+    const int64_t total = (int64_t)t.n;
+    free(t.ops);
+    return total;
+}
+
+int orc_run_dbring_rs_servers(int alg1, uint32_t n_servers, uint32_t n_local, void* const* user_in, void* const* user_out,
+                              void* const* ccl_in, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+{
+    OrcTrace t;
+    int rc = build_trace_dbring_rs_servers(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    if (rc) return rc;
+    void* const* bufs[5] = {ccl_in, NULL, NULL, user_in, user_out};
+    rc = exec_trace(&t, bufs, dtype, op);
+    free(t.ops);
+    return rc;
+}
+
 /* ---- the ring and mesh reduce-scatter executors over two communicator levels, op-base mode ---------------------- */
 
 /* CollReduceScatterRingExecutor::KernelRun (exec/coll_reduce_scatter/coll_reduce_scatter_ring_executor.cc:136-363, one
