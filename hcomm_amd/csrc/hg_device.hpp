@@ -168,6 +168,9 @@ template <int POL> __device__ __forceinline__ void stp(void* base, uint64_t vec,
 #ifndef HG_ST_SEG2
 #define HG_ST_SEG2 ST_SC1 /* copy / two-input reduce kernels, kept and streaming variants alike */
 #endif
+#ifndef HG_ST_REDUCE_KEPT
+#define HG_ST_REDUCE_KEPT ST_SC1 /* the kept variant of the two-input reduce; ST_NT there: ring step 59.3 -> 59.9 us, mesh step 15.4 -> 16.3 us */
+#endif
 #ifndef HG_ST_FOLD
 #define HG_ST_FOLD ST_NT /* the k-way folds at bandwidth-bound sizes (8 - 23 streams a lane): sc1 loses there (tree launches - 8 %) */
 #endif

@@ -70,12 +70,12 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stp<HG_ST_SEG2>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+                if (v < nvec) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -229,12 +229,12 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stp<HG_ST_SEG2>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+            if (v < nvec) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
         }
         if (tile == nvec / HG_TILE_VECS) { // the tile the element tail falls into
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES;
