@@ -157,16 +157,20 @@ template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec,
 // one more modifier.  The compiler does not see through the asm, so the two wait states it would put between a
 // 128-bit store and an instruction that overwrites the registers holding its data are part of the asm (without
 // them the next address computation lands in the data of the store before: wrong bytes, found by the probe's check=1).
-enum { ST_PLAIN = 0, ST_NT = 1, ST_SC1 = 2 };
+enum { ST_PLAIN = 0, ST_NT = 1, ST_SC1 = 2, ST_SC1_NT = 3 };
 template <int POL> __device__ __forceinline__ void stp(void* base, uint64_t vec, u32x4 v)
 {
     u32x4* p = (u32x4*)base + vec;
     if (POL == ST_SC1) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else if (POL == ST_SC1_NT) asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
     else if (POL == ST_NT) __builtin_nontemporal_store(v, p);
     else *p = v;
 }
 #ifndef HG_ST_SEG2
 #define HG_ST_SEG2 ST_SC1 /* copy / two-input reduce kernels, kept and streaming variants alike */
+#endif
+#ifndef HG_ST_STREAM
+#define HG_ST_STREAM ST_SC1 /* streaming variants; ST_SC1_NT there: halving-doubling + 0.6 %, the other large workloads - 1 .. - 2 % */
 #endif
 #ifndef HG_ST_REDUCE_KEPT
 #define HG_ST_REDUCE_KEPT ST_SC1 /* the kept variant of the two-input reduce; ST_NT there: ring step 59.3 -> 59.9 us, mesh step 15.4 -> 16.3 us */

@@ -15,7 +15,7 @@ namespace {
 
 // STREAM: nothing of what the launch writes will be found in the memory-side cache by a later launch (there is more
 // of it than that cache holds, or nothing reads it soon).  Since every store of these kernels carries the sc1 policy
-// (stp<HG_ST_SEG2>) the copy's two variants differ in their launch shape only - occupancy bound and XCD runs, set
+// (stp<HG_ST_SEG2> / stp<HG_ST_STREAM>, the same policy today) the copy's two variants differ in their launch shape only - occupancy bound and XCD runs, set
 // by hg_shape_seg2 in hg_batch.c - and the reduce's also in how the overwritten operand is loaded.  The launch's
 // dynamic LDS size is not used as memory: it bounds the workgroups a CU runs at once.
 template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
@@ -34,12 +34,12 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, a[u]);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v0 + u * HG_BLOCK, a[u]);
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stp<HG_ST_SEG2>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+                if (v < nvec) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v, ldv<HG_NT_LD_SRC>(p, v));
             }
             const uint64_t b = (nvec << 4) + tid; // this tile is the segment's last one: byte tail
             if (b < bytes) ((uint8_t*)d)[b] = ((const uint8_t*)p)[b];
@@ -70,12 +70,12 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
                 const uint64_t v = v0 + u * HG_BLOCK;
-                if (v < nvec) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+                if (v < nvec) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
             }
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES; // element tail, fewer than 16 / ES elements
             if (b + ES <= bytes) {
@@ -196,12 +196,12 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<HG_ST_SEG2>(d, v0 + u * HG_BLOCK, a[u]);
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v0 + u * HG_BLOCK, a[u]);
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stp<HG_ST_SEG2>(d, v, ldv<HG_NT_LD_SRC>(p, v));
+            if (v < nvec) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v, ldv<HG_NT_LD_SRC>(p, v));
         }
         if (tile == nvec / HG_TILE_VECS) { // the tile the byte tail falls into
             const uint64_t b = (nvec << 4) + tid;
@@ -229,12 +229,12 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = v0 + u * HG_BLOCK;
-            if (v < nvec) stp<(STREAM ? HG_ST_SEG2 : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
+            if (v < nvec) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v, vec_op<DT, OP>(ldv<STREAM>(d, v), ldv<HG_NT_LD_SRC>(p, v)));
         }
         if (tile == nvec / HG_TILE_VECS) { // the tile the element tail falls into
             const uint64_t b = (nvec << 4) + (uint64_t)tid * ES;
