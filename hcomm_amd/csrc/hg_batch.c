@@ -81,9 +81,9 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
  * Every figure can be overridden from the environment for experiments.
  */
 enum {
-    TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE,
+    TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE, TUNE_LDS_REDUCE_FROM,
     TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_CHAIN, TUNE_RUN_CHAIN, TUNE_LDS_TREE,
-    TUNE_RUN_TREE, TUNE_N
+    TUNE_RUN_TREE, TUNE_LDS_TREE_TABLES, TUNE_N
 };
 static const struct {
     const char* env;
@@ -91,12 +91,16 @@ static const struct {
 } g_tune_def[TUNE_N] = {
     {"HCOMM_GFX_STREAM_COPY_BYTES", 256ull << 20},   /* the 256 MB memory-side cache */
     {"HCOMM_GFX_STREAM_REDUCE_BYTES", 256ull << 20},
-    {"HCOMM_GFX_LDS_COPY", 32768},
-    {"HCOMM_GFX_LDS_COPY_STREAM", 53248},
-    {"HCOMM_GFX_LDS_REDUCE", 0},
+    {"HCOMM_GFX_LDS_COPY", 53248},
+    {"HCOMM_GFX_LDS_COPY_STREAM", 65536},
+    /* kept reduce: at most four workgroups per CU once the launch writes 64 MiB or more (8 x 16 MiB ring steps on
+     * operands nothing touched recently 69.9 -> 67.8 us, the same steps in a ring 60.4 -> 59.9; two-level ring steps of
+     * 256 MiB 112.6 -> 109.7; below that size the bound costs the cache-resident 8 x 4 MiB mesh steps 1 %) */
+    {"HCOMM_GFX_LDS_REDUCE", 40960},
+    {"HCOMM_GFX_LDS_REDUCE_FROM_BYTES", 64ull << 20},
     {"HCOMM_GFX_LDS_REDUCE_STREAM", 53248},
-    {"HCOMM_GFX_XCD_RUN_COPY", 128},
-    {"HCOMM_GFX_XCD_RUN_COPY_STREAM", 128},
+    {"HCOMM_GFX_XCD_RUN_COPY", 64},
+    {"HCOMM_GFX_XCD_RUN_COPY_STREAM", 64},
     {"HCOMM_GFX_XCD_RUN_REDUCE", 128},
     {"HCOMM_GFX_XCD_RUN_REDUCE_STREAM", 32},
     /* the k-way folds, measured on their single-launch lowerings.  Tree (16 x 128 MiB int32 recursive halving, 8 x
@@ -107,6 +111,9 @@ static const struct {
     {"HCOMM_GFX_XCD_RUN_CHAIN", 0},
     {"HCOMM_GFX_LDS_TREE", 53248},
     {"HCOMM_GFX_XCD_RUN_TREE", 128},
+    /* trees read from per-segment tables (the lowering of operation lists): four workgroups per CU (deterministic mesh
+     * allreduce 8 x 128 MiB in one launch 0.383 -> 0.360 ms; the other tree modes lose 1 - 3 % with it) */
+    {"HCOMM_GFX_LDS_TREE_TABLES", 40960},
 };
 static uint64_t g_tune[TUNE_N]; /* value + 1; 0 = not read yet (same relaxed-atomic rule as env_once) */
 
@@ -141,7 +148,7 @@ void hg_shape_seg2(HgLaunch* l, int streaming)
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_COPY_STREAM : TUNE_RUN_COPY);
     } else {
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_REDUCE_BYTES));
-        l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_REDUCE_STREAM : TUNE_LDS_REDUCE);
+        l->lds_bytes = l->streaming ? lds_of(TUNE_LDS_REDUCE_STREAM) : (l->bytes >= tune(TUNE_LDS_REDUCE_FROM) ? lds_of(TUNE_LDS_REDUCE) : 0u);
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_REDUCE_STREAM : TUNE_RUN_REDUCE);
     }
 }
@@ -204,7 +211,7 @@ void hg_finish_fold(HgLaunch* l)
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
     l->streaming = 0;
-    l->lds_bytes = lds_of(t->tree ? TUNE_LDS_TREE : TUNE_LDS_CHAIN);
+    l->lds_bytes = lds_of(t->tree == 6u ? TUNE_LDS_TREE_TABLES : (t->tree ? TUNE_LDS_TREE : TUNE_LDS_CHAIN));
     t->xcd_run = (uint32_t)tune(t->tree ? TUNE_RUN_TREE : TUNE_RUN_CHAIN);
     if (!t->tree) {
         /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
