@@ -67,17 +67,17 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
 }
 
 /*
- * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip; 16 KiB tiles, bf16 SUM,
- * seeded non-zero data, fractions of 8 TB/s).  Two regimes:
+ * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip with hg_probe_shapes.txt:
+ * 16 KiB tiles, bf16 SUM, seeded non-zero data, sc1 stores) and confirmed per workload in the library.  Two regimes:
  *   kept      what the launch writes fits the memory-side cache and a later launch reads it back from there (a ring
- *             step): the overwritten operand loaded plain, XCDs walking runs of 128 tiles.
- *             8 x 16 MiB ring steps: reduce 0.860 (0.827 with that operand loaded non-temporal and tiles as dealt),
- *             copy 0.873 with at most five workgroups per CU (0.864 without that bound).
- *   streaming every load non-temporal and at most three workgroups per CU in flight.  16 x 64 MiB that nothing touched
- *             recently: reduce 0.823 with runs of 32 tiles (0.795 without the bound, 0.711 with the grid held at 32
- *             workgroups per CU), copy 0.808 with runs of 128 (0.744 without the bound).
- * (Figures taken with plain / non-temporal stores; both regimes now store with the sc1 policy, which is ahead of either:
- * hg_device.hpp.)  The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
+ *             step): the overwritten operand loaded plain.  Reduce: XCDs walking runs of 128 tiles, at most four
+ *             workgroups per CU once the launch writes 64 MiB (8 x 16 MiB ring steps on cold operands 69.7 -> 67.9 us,
+ *             inside a ring 60.3 -> 60.2).  Copy: runs of 64 tiles, at most three workgroups per CU (cold 45.0 -> 42.7 us,
+ *             inside a ring 38.0 -> 37.8).
+ *   streaming every load non-temporal.  16 x 64 MiB that nothing touched recently: reduce 477 us with at most three
+ *             workgroups per CU and runs of 32 tiles (499 with runs of 128, 522 with two workgroups), copy 320 us with
+ *             at most two and runs of 64 (331 with three and runs of 128).
+ * The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
  * Every figure can be overridden from the environment for experiments.
  */
 enum {
