@@ -142,9 +142,11 @@ void hg_shape_seg2(HgLaunch* l, int streaming)
     HgSeg2Table* t = &l->tab.seg2;
     /* the kernel for operands off 16-byte boundaries comes as a copy (op 255) and as a reduce: shaped like them */
     const int copy = l->kind == HCOMM_GFX_KERNEL_COPY || (l->kind == HCOMM_GFX_KERNEL_BYTEWISE && l->op == 255u);
-    if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE) {
-        /* its lanes assemble every vector from two loads: it wants more workgroups per CU than the aligned kernels
-         * (order-preserving reduce-scatter on blocks of 16,777,214 bytes: 0.926 ms with these shapes, 0.997 with theirs) */
+    if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE || t->direct == 0u) {
+        /* The kernel for unaligned operands (its lanes assemble every vector from two loads) and the one-dimensional
+         * kernels (ragged tables; a few more rounds of argument reads before the data) want more workgroups per CU than
+         * the row-grid kernels the table above was swept with: order-preserving reduce-scatter on blocks of 16,777,214
+         * bytes 0.926 ms with these shapes, 0.997 with those; a ragged 512 MiB copy launch 170 against 187 us. */
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(copy ? TUNE_STREAM_COPY_BYTES : TUNE_STREAM_REDUCE_BYTES));
         l->lds_bytes = l->streaming ? 53248u : (copy ? 32768u : 0u);
         t->xcd_run = (l->streaming && !copy) ? 32u : 128u;
@@ -180,7 +182,6 @@ void hg_finish_seg2(HgLaunch* l)
     l->bytes = bytes;
     l->moved_bytes = bytes * ((l->op == 255u) ? 2u : 3u);
     l->blocks = hg_grid_blocks(tiles);
-    hg_shape_seg2(l, -1);
     /* A two-dimensional grid (segment, tile of it: one round of kernel-argument reads instead of four or five) where
      * that wastes few workgroups: segments of nearly equal length at any size (at most an eighth more workgroups than
      * tiles), anything up to HCOMM_GFX_DIRECT_TILES tiles as long as the grid at most doubles.  Launches that small
@@ -199,6 +200,7 @@ void hg_finish_seg2(HgLaunch* l)
             l->blocks = grid;
         }
     }
+    hg_shape_seg2(l, -1);
     if (small && (t->direct || l->kind == HCOMM_GFX_KERNEL_BYTEWISE)) {
         l->streaming = 0;
         l->lds_bytes = 0;
