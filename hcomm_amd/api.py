@@ -848,41 +848,43 @@ def dbring_rs_check(n_ranks, count, ccl_bytes, dtype):
     return rep.conflicts, rep.semanticErrors, rep.message.decode()
 
 
-_dbhrs_emit = _sig("HcommGfxDoubleRingHierReduceScatterEmit", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+_dbhrs_emit = _sig("HcommGfxDoubleRingHierReduceScatterEmit", _i32, C.c_int, C.c_int, _u32, _u32, _u32, _u64, _u64, C.c_int,
                    C.POINTER(SchedOp), _u64, C.POINTER(_u64))
-_dbhrs_check = _sig("HcommGfxDoubleRingHierReduceScatterCheck", _i32, C.c_int, _u32, _u32, _u64, _u64, C.c_int,
+_dbhrs_check = _sig("HcommGfxDoubleRingHierReduceScatterCheck", _i32, C.c_int, C.c_int, _u32, _u32, _u32, _u64, _u64, C.c_int,
                     C.POINTER(CheckReport))
-_dbhrs_plan = _sig("HcommGfxDoubleRingHierReduceScatterPlanCreate", _i32, C.c_int, _u32, _u32, C.POINTER(_vp),
+_dbhrs_plan = _sig("HcommGfxDoubleRingHierReduceScatterPlanCreate", _i32, C.c_int, C.c_int, _u32, _u32, _u32, C.POINTER(_vp),
                    C.POINTER(_vp), C.POINTER(_vp), _u64, _u64, C.c_int, C.c_int, C.POINTER(_vp))
+_RS_RING = 1  # HCOMM_GFX_ALG_REDUCE_SCATTER_RING
 
 
-def dbring_hier_rs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+def dbring_hier_rs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, n_pods=1, alg2=_RS_RING):
     n = _u64(0)
-    check(_dbhrs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
+    check(_dbhrs_emit(alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype, None, 0, C.byref(n)),
           "HcommGfxDoubleRingHierReduceScatterEmit")
     ops = (SchedOp * max(n.value, 1))()
-    check(_dbhrs_emit(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
+    check(_dbhrs_emit(alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype, ops, n.value, C.byref(n)),
           "HcommGfxDoubleRingHierReduceScatterEmit")
     return [ops[i].astuple() for i in range(n.value)]
 
 
-def dbring_hier_rs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype):
+def dbring_hier_rs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, n_pods=1, alg2=_RS_RING):
     rep = CheckReport()
-    check(_dbhrs_check(alg1, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
+    check(_dbhrs_check(alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype, C.byref(rep)),
           "HcommGfxDoubleRingHierReduceScatterCheck")
     return rep.conflicts, rep.semanticErrors, rep.message.decode()
 
 
 class DoubleRingHierReduceScatterPlan(Plan):
-    """HcommGfxDoubleRingHierReduceScatterPlanCreate: the double-ring reduce-scatter executor over several servers."""
+    """HcommGfxDoubleRingHierReduceScatterPlanCreate: the double-ring reduce-scatter executor over servers and super pods."""
 
-    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_bytes, count, dtype, op):
+    def __init__(self, alg1, n_servers, n_local, user_in, user_out, ccl_in, ccl_bytes, count, dtype, op, n_pods=1,
+                 alg2=_RS_RING):
         n = len(user_in)
-        assert n == n_servers * n_local
+        assert n == n_pods * n_servers * n_local
         self._bufs = [(_vp * n)(*b) for b in (user_in, user_out, ccl_in)]
         p = _vp(0)
-        check(_dbhrs_plan(alg1, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes, count, dtype,
-                          op, C.byref(p)), "HcommGfxDoubleRingHierReduceScatterPlanCreate")
+        check(_dbhrs_plan(alg1, alg2, n_pods, n_servers, n_local, self._bufs[0], self._bufs[1], self._bufs[2], ccl_bytes,
+                          count, dtype, op, C.byref(p)), "HcommGfxDoubleRingHierReduceScatterPlanCreate")
         self._p = p
         info = PlanInfo()
         check(_plan_info(self._p, C.byref(info)), "HcommGfxPlanGetInfo")

@@ -448,14 +448,14 @@ int32_t HcommGfxHierReduceScatterCheck(
 }
 
 int32_t HcommGfxDoubleRingHierReduceScatterCheck(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
-    HcommDataType dataType, HcommGfxCheckReport* rep)
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal, uint64_t count,
+    uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* rep)
 {
     if (!rep) return HCCL_E_PTR;
     HgOpList l;
-    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, (int)level2Alg, nPods, nServers, nLocal, count, cclBytes, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
-    rc = HcommGfxOpListCheck(l.ops, l.n, nServers * nLocal, HCOMM_GFX_EXPECT_REDUCE_SCATTER_USER, count, 0,
+    rc = HcommGfxOpListCheck(l.ops, l.n, nPods * nServers * nLocal, HCOMM_GFX_EXPECT_REDUCE_SCATTER_USER, count, 0,
                              HcommGfxDataTypeSize(dataType), rep);
     hg_oplist_free(&l);
     return rc;

@@ -1455,22 +1455,24 @@ int32_t HcommGfxDoubleRingReduceScatterPlanCreate(
 }
 
 int32_t HcommGfxDoubleRingHierReduceScatterPlanCreate(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut,
-    void* const* cclIn, uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp,
-    HcommGfxPlan** plan)
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal,
+    void* const* userIn, void* const* userOut, void* const* cclIn, uint64_t cclBytes, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan)
 {
     if (!plan) return HCCL_E_PTR;
     *plan = NULL;
     if (!userIn || !userOut || !cclIn) return HCCL_E_PTR;
-    if (nServers < 2 || nLocal < 3 || (uint64_t)nServers * nLocal > HCOMM_GFX_MAX_RANKS) return HCCL_E_PARA;
+    if (nPods == 0 || nServers == 0 || (uint64_t)nPods * nServers < 2 || nLocal < 3 ||
+        (uint64_t)nPods * nServers * nLocal > HCOMM_GFX_MAX_RANKS)
+        return HCCL_E_PARA;
     if (!hg_reduce_supported((int)dataType, (int)reduceOp, 1)) return HCCL_E_PARA;
-    const uint32_t n = nServers * nLocal;
+    const uint32_t n = nPods * nServers * nLocal;
     int rc = check_bufs(userIn, n);
     if (rc == HCCL_SUCCESS) rc = check_bufs(userOut, n);
     if (rc == HCCL_SUCCESS) rc = check_bufs(cclIn, n);
     if (rc != HCCL_SUCCESS) return rc;
     HgOpList ol;
-    rc = hg_schedule_dbring_rs_servers(&ol, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    rc = hg_schedule_dbring_rs_servers(&ol, (int)level1Alg, (int)level2Alg, nPods, nServers, nLocal, count, cclBytes, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     void* const* bufs[HCOMM_GFX_NUM_BUFS] = {cclIn, NULL, NULL, userIn, userOut};
     rc = HcommGfxPlanCreateFromOps(ol.ops, ol.n, n, bufs, dataType, reduceOp, plan);

@@ -1421,25 +1421,57 @@ int32_t HcommGfxDoubleRingReduceScatterEmit(
     return HCCL_SUCCESS;
 }
 
-/* ---- the double-ring reduce-scatter executor over the servers of one super pod (op-base mode, DMA reduce) ---------- */
+/* ---- the double-ring reduce-scatter executor over servers and super pods (op-base mode, DMA reduce) ---------------- */
 
-/* CollAlignedReduceScatterDoubleRingFor91093Executor with several servers (KernelRun of its base,
- * coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:595-812, level2RankSize 1).  With S
- * servers of N devices, rank = server * N + local index, block g = the output of rank g, per chunk of c bytes per block
- * and dir = -1 for ring 0 (first shares), +1 for ring 1 (second shares), every rank (s, r):
- *   step 0: fetches the shares of blocks k * N + (r + dir) and k * N + (r + 2 dir), k = 0 .. S - 1, from its user input
- *     into its CCL input - every ring position carries S slices, one per server (FillMultiRingSlice :213-233, user
- *     offsets :297-313; aligned_reduce_scatter_double_ring.cc:305-332);
- *   step 1 + t, t < N - 1: folds the shares of blocks k * N + (r + (2 + t) dir) of rank (s, r + dir)'s CCL input into
+/* Append `sub`, a list over the ranks of one communicator level, once per `copies`: operation by operation, copy c shifted
+ * by c * shift bytes (the templates walk the slices of a slice index one after the other: reduce_scatter_ring.cc:221-224,
+ * 242-245, reduce_scatter_nhr.cc:573-579, reduce_scatter_nb.cc:174). */
+static int append_mapped_copies(HgOpList* l, const HgOpList* sub, const uint32_t* map, uint32_t step0, uint64_t base,
+                                uint32_t copies, uint64_t shift)
+{
+    for (uint64_t i = 0; i < sub->n; ++i) {
+        const HcommGfxSchedOp* o = &sub->ops[i];
+        for (uint32_t c = 0; c < copies; ++c)
+            CHK(push(l, step0 + o->step, o->kind, map[o->rank], o->dstBuf, o->dstOff + base + c * shift, map[o->srcRank],
+                     o->srcBuf, o->srcOff + base + c * shift, o->bytes));
+    }
+    return HCCL_SUCCESS;
+}
+
+static int level_rs(HgOpList* sub, int alg, uint32_t n, const HcommGfxSlice* sl)
+{
+    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) return ring_rs(sub, n, sl, 0);
+    if (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB) return nb_rs(sub, n, sl);
+    uint32_t order[HCOMM_GFX_MAX_RANKS];
+    nhr_slice_map(n, 1, order);
+    return nhr_rs(sub, n, sl, order, 0);
+}
+
+static uint32_t level_rs_steps(int alg, uint32_t n)
+{
+    return n < 2 ? 0u : (alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING ? n - 1u : ceil_log2(n));
+}
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor with several servers and super pods (KernelRun of its base,
+ * coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:595-812).  With P pods of S servers of
+ * N devices, rank = (pod * S + server) * N + local index, block g = the output of rank g, per chunk of c bytes per block
+ * and dir = -1 for ring 0 (first shares), +1 for ring 1 (second shares), every rank (p, s, r):
+ *   step 0: fetches the shares of blocks k * N + (r + dir) and k * N + (r + 2 dir), k = 0 .. P * S - 1, from its user
+ *     input into its CCL input - every ring position carries one slice per server of every pod (FillMultiRingSlice
+ *     :213-233, user offsets :297-313; aligned_reduce_scatter_double_ring.cc:305-332);
+ *   step 1 + t, t < N - 1: folds the shares of blocks k * N + (r + (2 + t) dir) of rank (p, s, r + dir)'s CCL input into
  *     its own and, except in the last of these steps, fetches those of blocks k * N + (r + (3 + t) dir) (:366-425; the
  *     user output address is null here, :664-670, so nothing goes to the user output yet);
- *   then the reduce-scatter between the servers (ring, NHR or NB, :689-746) in place on the CCL input buffers of the
- *     ranks (0, r) .. (S - 1, r), slice i = block i * N + r (:327-338);
- *   last: block s * N + r from the CCL input to the user output (:800-808). */
-static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32_t n, uint64_t count, uint64_t ccl_bytes,
-                                   uint32_t unit)
+ *   then (S > 1) the reduce-scatter between the servers of a pod (ring, NHR or NB, :689-746) in place on the CCL input
+ *     buffers of the ranks (p, 0, r) .. (p, S - 1, r): server i's rank owns the blocks (q * S + i) * N + r of every pod q
+ *     (:327-350), walked one after the other wherever the template touches a slice;
+ *   then (P > 1) the one between the pods (:748-797) over the ranks (0, s, r) .. (P - 1, s, r), slice i = block
+ *     (i * S + s) * N + r (:376-382);
+ *   last: the own block from the CCL input to the user output (:800-808). */
+static int dbring_rs_servers_build(HgOpList* l, int alg1, int alg2, uint32_t n_pods, uint32_t n_srv, uint32_t n, uint64_t count,
+                                   uint64_t ccl_bytes, uint32_t unit)
 {
-    const uint32_t total = n_srv * n;
+    const uint32_t groups = n_pods * n_srv, total = groups * n;
     const uint64_t max_count = ccl_bytes / total / 128u * 128u / unit; /* CalcLoopMaxCount, :167-173 */
     if (max_count == 0) return HCCL_E_PARA;
     const uint64_t stride = count * unit;
@@ -1455,7 +1487,7 @@ static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32
 #define BLK(r, k, ring) (((r) + (uint64_t)n * 4u + (uint64_t)(k) * ((ring) ? 1u : n - 1u)) % n)
         for (uint32_t g = 0; g < total; ++g) {
             const uint32_t r = g % n;
-            for (uint32_t k = 0; k < n_srv; ++k)
+            for (uint32_t k = 0; k < groups; ++k)
                 for (uint32_t ring = 0; ring < 2; ++ring)
                     for (uint32_t j = 1; j <= 2; ++j) {
                         const uint64_t b = (uint64_t)k * n + BLK(r, j, ring);
@@ -1464,10 +1496,10 @@ static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32
         }
         for (uint32_t t = 0; t + 1 < n; ++t)
             for (uint32_t g = 0; g < total; ++g) {
-                const uint32_t r = g % n, srv = g / n;
+                const uint32_t r = g % n, grp = g / n;
                 for (uint32_t ring = 0; ring < 2; ++ring) {
-                    const uint32_t peer = srv * n + (uint32_t)BLK(r, 1, ring);
-                    for (uint32_t k = 0; k < n_srv; ++k) {
+                    const uint32_t peer = grp * n + (uint32_t)BLK(r, 1, ring);
+                    for (uint32_t k = 0; k < groups; ++k) {
                         const uint64_t b = (uint64_t)k * n + BLK(r, 2 + t, ring);
                         CHK(push(l, step + 1 + t, REDUCE, g, IN, b * c + off[ring], peer, IN, b * c + off[ring], len[ring]));
                         if (t + 2 == n) continue;
@@ -1478,29 +1510,39 @@ static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32
             }
 #undef BLK
         step += n;
-        {
+        if (n_srv > 1) { /* between the servers of every pod: one list over S ranks, once per (pod, local index) */
             HgOpList sub;
             memset(&sub, 0, sizeof(sub));
             for (uint32_t i = 0; i < n_srv; ++i) {
                 sl[i].offset = c * n * i;
                 sl[i].size = c;
             }
-            int rc;
-            if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_RING) rc = ring_rs(&sub, n_srv, sl, 0);
-            else if (alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_NB) rc = nb_rs(&sub, n_srv, sl);
-            else {
-                uint32_t order[HCOMM_GFX_MAX_RANKS];
-                nhr_slice_map(n_srv, 1, order);
-                rc = nhr_rs(&sub, n_srv, sl, order, 0);
-            }
-            uint32_t used = 0;
-            for (uint32_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
-                for (uint32_t srv = 0; srv < n_srv; ++srv) map[srv] = srv * n + i;
-                rc = append_mapped(l, &sub, map, step, c * i, 0, &used);
-            }
+            int rc = level_rs(&sub, alg1, n_srv, sl);
+            for (uint32_t p = 0; p < n_pods && rc == HCCL_SUCCESS; ++p)
+                for (uint32_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
+                    for (uint32_t srv = 0; srv < n_srv; ++srv) map[srv] = (p * n_srv + srv) * n + i;
+                    rc = append_mapped_copies(l, &sub, map, step, c * i, n_pods, c * n * n_srv);
+                }
             hg_oplist_free(&sub);
             CHK(rc);
-            step += alg1 == HCOMM_GFX_ALG_REDUCE_SCATTER_RING ? n_srv - 1 : ceil_log2(n_srv);
+            step += level_rs_steps(alg1, n_srv);
+        }
+        if (n_pods > 1) { /* between the pods: one list over P ranks, once per (server, local index) */
+            HgOpList sub;
+            memset(&sub, 0, sizeof(sub));
+            for (uint32_t i = 0; i < n_pods; ++i) {
+                sl[i].offset = c * n * n_srv * i;
+                sl[i].size = c;
+            }
+            int rc = level_rs(&sub, alg2, n_pods, sl);
+            for (uint32_t srv = 0; srv < n_srv && rc == HCCL_SUCCESS; ++srv)
+                for (uint32_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
+                    for (uint32_t p = 0; p < n_pods; ++p) map[p] = (p * n_srv + srv) * n + i;
+                    rc = append_mapped_copies(l, &sub, map, step, c * (srv * n + i), 1, 0);
+                }
+            hg_oplist_free(&sub);
+            CHK(rc);
+            step += level_rs_steps(alg2, n_pods);
         }
         for (uint32_t g = 0; g < total; ++g) CHK(push(l, step, COPY, g, UOUT, user_off, g, IN, c * g, c));
         ++step;
@@ -1510,27 +1552,32 @@ static int dbring_rs_servers_build(HgOpList* l, int alg1, uint32_t n_srv, uint32
     return order_by_step_rank(l);
 }
 
-int hg_schedule_dbring_rs_servers(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
-                                  uint64_t ccl_bytes, int dtype)
+static int level_alg_ok(int alg)
+{
+    return alg == HCOMM_GFX_ALG_REDUCE_SCATTER_RING || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NHR || alg == HCOMM_GFX_ALG_REDUCE_SCATTER_NB;
+}
+
+int hg_schedule_dbring_rs_servers(HgOpList* l, int alg1, int alg2, uint32_t n_pods, uint32_t n_servers, uint32_t n_local,
+                                  uint64_t count, uint64_t ccl_bytes, int dtype)
 {
     memset(l, 0, sizeof(*l));
     const uint32_t unit = HcommGfxDataTypeSize((HcommDataType)dtype);
-    if (unit == 0 || count > HG_MAX_COUNT || n_servers < 2 || n_local < 3 || (uint64_t)n_servers * n_local > HCOMM_GFX_MAX_RANKS)
+    if (unit == 0 || count > HG_MAX_COUNT || n_pods == 0 || n_servers == 0 || (uint64_t)n_pods * n_servers < 2 || n_local < 3 ||
+        (uint64_t)n_pods * n_servers * n_local > HCOMM_GFX_MAX_RANKS)
         return HCCL_E_PARA;
-    if (alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_RING && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NHR && alg1 != HCOMM_GFX_ALG_REDUCE_SCATTER_NB)
-        return HCCL_E_PARA;
-    const int rc = dbring_rs_servers_build(l, alg1, n_servers, n_local, count, ccl_bytes, unit);
+    if (!level_alg_ok(alg1) || !level_alg_ok(alg2)) return HCCL_E_PARA;
+    const int rc = dbring_rs_servers_build(l, alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, unit);
     if (rc != HCCL_SUCCESS) hg_oplist_free(l);
     return rc;
 }
 
 int32_t HcommGfxDoubleRingHierReduceScatterEmit(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
-    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal, uint64_t count,
+    uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n)
 {
     if (!n) return HCCL_E_PTR;
     HgOpList l;
-    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, nServers, nLocal, count, cclBytes, (int)dataType);
+    int rc = hg_schedule_dbring_rs_servers(&l, (int)level1Alg, (int)level2Alg, nPods, nServers, nLocal, count, cclBytes, (int)dataType);
     if (rc != HCCL_SUCCESS) return rc;
     *n = l.n;
     if (ops) {

@@ -45,8 +45,8 @@ int hg_schedule_hier_rs(HgOpList* l, int level0_mesh, int alg1, uint32_t n_serve
 /* The double-ring reduce-scatter executor on one server in op-base mode with DMA reduce: user input read share by share,
  * the result folded straight into the user output. */
 int hg_schedule_dbring_rs(HgOpList* l, uint32_t n, uint64_t count, uint64_t ccl_bytes, int dtype);
-int hg_schedule_dbring_rs_servers(HgOpList* l, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
-                                  uint64_t ccl_bytes, int dtype);
+int hg_schedule_dbring_rs_servers(HgOpList* l, int alg1, int alg2, uint32_t n_pods, uint32_t n_servers, uint32_t n_local,
+                                  uint64_t count, uint64_t ccl_bytes, int dtype);
 /* Most elements per rank any schedule accepts: every byte offset a schedule derives from a count (count x unit x
  * ranks, rounded up to slot sizes) then stays far inside 64 bits.  Larger counts are refused with HCCL_E_PARA. */
 #define HG_MAX_COUNT ((uint64_t)1 << 48)

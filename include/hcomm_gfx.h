@@ -739,7 +739,7 @@ int32_t HcommGfxDoubleRingCheck(
  * before they are needed; the last fold of a rank's own block lands in its user output, which the step before filled
  * with the rank's own share.  userIn: nRanks * count elements (block b at b * count); userOut: count; cclIn: cclBytes.
  * nRanks >= 3 (the template's two-rank first step, :353-360, leaves the neighbour's share unwritten; the double-ring
- * servers have more).  Several servers: HcommGfxDoubleRingHierReduceScatter*, below.
+ * servers have more).  Several servers and super pods: HcommGfxDoubleRingHierReduceScatter*, below.
  */
 int32_t HcommGfxDoubleRingReduceScatterPlanCreate(
     uint32_t nRanks, void* const* userIn, void* const* userOut, void* const* cclIn, uint64_t cclBytes, uint64_t count,
@@ -751,30 +751,33 @@ int32_t HcommGfxDoubleRingReduceScatterCheck(
     uint32_t nRanks, uint64_t count, uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
- * The same executor over the nServers >= 2 servers of one super pod, rank = server * nLocal + local index, nLocal >= 3
- * (KernelRun of its base, coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:595-812 with
- * level2RankSize 1), per chunk of at most cclBytes / (nServers * nLocal) (rounded down to 128 bytes) / unit elements per
- * block:
- *   (1) AlignedReduceScatterDoubleRing inside every server with nServers slices per ring position - the two shares of
- *       the blocks of the ranks with one local index, one per server (FillMultiRingSlice :213-233, user-memory slices
- *       :297-313; alg_template/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc:305-332, 366-425) - and only
- *       the user input address set (:664-670), so every fold stays in the CCL input buffers;
- *   (2) level1Alg (HCOMM_GFX_ALG_REDUCE_SCATTER_RING, _NHR or _NB, :689-746) between the servers, in place on the CCL
- *       input buffers of the ranks with one local index, slice i = the block of server i's rank (:327-338);
- *   (3) the own block from the CCL input to the user output (:800-808).
- * userIn: nServers * nLocal * count elements (block b at b * count); userOut: count; cclIn: cclBytes.  The stage between
- * super pods (level2RankSize > 1), the AHC branches and the reduce-scatter-v slices are not built.
+ * The same executor over nPods super pods of nServers servers (more than one between them) of nLocal >= 3 devices,
+ * rank = (pod * nServers + server) * nLocal + local index (KernelRun of its base,
+ * coll_executor/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:595-812), per chunk of at most
+ * cclBytes / ranks (rounded down to 128 bytes) / unit elements per block:
+ *   (1) AlignedReduceScatterDoubleRing inside every server with nPods * nServers slices per ring position - the two
+ *       shares of the blocks of the ranks with one local index, one per server of every pod (FillMultiRingSlice :213-233,
+ *       user-memory slices :297-313; alg_template/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc:305-332,
+ *       366-425) - and only the user input address set (:664-670), so every fold stays in the CCL input buffers;
+ *   (2) nServers > 1: level1Alg (HCOMM_GFX_ALG_REDUCE_SCATTER_RING, _NHR or _NB, :689-746) between the servers of a pod,
+ *       in place on the CCL input buffers of the ranks with one local index; server i's rank owns one slice per pod, the
+ *       block of the rank with its place in that pod (:327-350), and the templates walk the slices of a rank one after
+ *       the other (reduce_scatter_ring.cc:221-224, reduce_scatter_nhr.cc:573-579, reduce_scatter_nb.cc:174);
+ *   (3) nPods > 1: level2Alg (the same three, :748-797) between the pods, slice i = the block of pod i's rank (:376-382);
+ *   (4) the own block from the CCL input to the user output (:800-808).
+ * userIn: ranks * count elements (block b at b * count); userOut: count; cclIn: cclBytes.  The AHC branches and the
+ * reduce-scatter-v slices are not built.
  */
 int32_t HcommGfxDoubleRingHierReduceScatterPlanCreate(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, void* const* userIn, void* const* userOut,
-    void* const* cclIn, uint64_t cclBytes, uint64_t count, HcommDataType dataType, HcommReduceOp reduceOp,
-    HcommGfxPlan** plan);
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal,
+    void* const* userIn, void* const* userOut, void* const* cclIn, uint64_t cclBytes, uint64_t count, HcommDataType dataType,
+    HcommReduceOp reduceOp, HcommGfxPlan** plan);
 int32_t HcommGfxDoubleRingHierReduceScatterEmit(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
-    HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal, uint64_t count,
+    uint64_t cclBytes, HcommDataType dataType, HcommGfxSchedOp* ops, uint64_t cap, uint64_t* n);
 int32_t HcommGfxDoubleRingHierReduceScatterCheck(
-    HcommGfxAlgorithm level1Alg, uint32_t nServers, uint32_t nLocal, uint64_t count, uint64_t cclBytes,
-    HcommDataType dataType, HcommGfxCheckReport* report);
+    HcommGfxAlgorithm level1Alg, HcommGfxAlgorithm level2Alg, uint32_t nPods, uint32_t nServers, uint32_t nLocal, uint64_t count,
+    uint64_t cclBytes, HcommDataType dataType, HcommGfxCheckReport* report);
 
 /*
  * The reduce-scatter of the reference's ring executor (level0Mesh 0: coll_executor/coll_reduce_scatter/

@@ -142,10 +142,10 @@ def lib():
         L.orc_run_dbring_rs.restype = C.c_int
         L.orc_run_dbring_rs.argtypes = [C.c_uint32] + [C.POINTER(C.c_void_p)] * 3 + [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
         L.orc_trace_dbring_rs_servers.restype = C.c_int64
-        L.orc_trace_dbring_rs_servers.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int,
-                                                  C.POINTER(OrcOp), C.c_uint64]
+        L.orc_trace_dbring_rs_servers.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64,
+                                                  C.c_int, C.POINTER(OrcOp), C.c_uint64]
         L.orc_run_dbring_rs_servers.restype = C.c_int
-        L.orc_run_dbring_rs_servers.argtypes = [C.c_int, C.c_uint32, C.c_uint32] + [C.POINTER(C.c_void_p)] * 3 + \
+        L.orc_run_dbring_rs_servers.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_uint32, C.c_uint32] + [C.POINTER(C.c_void_p)] * 3 + \
             [C.c_uint64, C.c_uint64, C.c_int, C.c_int]
         L.orc_trace.restype = C.c_int64
         L.orc_trace.argtypes = [C.c_int, C.c_uint32, C.c_uint64, C.c_int, C.POINTER(OrcOp), C.c_uint64]
@@ -495,21 +495,24 @@ def run_dbring_rs(user_in, user_out, ccl_in, count, ccl_bytes, dtype, op):
         raise ValueError("orc_run_dbring_rs rc=%d" % rc)
 
 
-# ---- the same executor over the servers of one super pod -------------------------------------------------
+# ---- the same executor over servers and super pods ----------------------------------------------------------
 
-def trace_dbring_rs_servers(alg1, n_servers, n_local, count, ccl_bytes, dtype):
-    total = lib().orc_trace_dbring_rs_servers(alg1, n_servers, n_local, count, ccl_bytes, dtype, None, 0)
+def trace_dbring_rs_servers(alg1, n_servers, n_local, count, ccl_bytes, dtype, n_pods=1, alg2=ALG_RS_RING_STAGE):
+    """rank = (pod * n_servers + server) * n_local + local index; alg1 between the servers of a pod, alg2 between pods."""
+    total = lib().orc_trace_dbring_rs_servers(alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype, None, 0)
     if total < 0:
         raise ValueError("orc_trace_dbring_rs_servers rc=%d" % total)
     ops = (OrcOp * max(total, 1))()
-    lib().orc_trace_dbring_rs_servers(alg1, n_servers, n_local, count, ccl_bytes, dtype, ops, total)
+    lib().orc_trace_dbring_rs_servers(alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype, ops, total)
     return [ops[i].astuple() for i in range(total)]
 
 
-def run_dbring_rs_servers(alg1, n_servers, n_local, user_in, user_out, ccl_in, count, ccl_bytes, dtype, op):
+def run_dbring_rs_servers(alg1, n_servers, n_local, user_in, user_out, ccl_in, count, ccl_bytes, dtype, op, n_pods=1,
+                          alg2=ALG_RS_RING_STAGE):
     n = len(user_in)
-    assert n == n_servers * n_local
+    assert n == n_pods * n_servers * n_local
     arrs = [(C.c_void_p * n)(*[x.ctypes.data for x in b]) for b in (user_in, user_out, ccl_in)]
-    rc = lib().orc_run_dbring_rs_servers(alg1, n_servers, n_local, arrs[0], arrs[1], arrs[2], count, ccl_bytes, dtype, op)
+    rc = lib().orc_run_dbring_rs_servers(alg1, alg2, n_pods, n_servers, n_local, arrs[0], arrs[1], arrs[2], count, ccl_bytes,
+                                         dtype, op)
     if rc:
         raise ValueError("orc_run_dbring_rs_servers rc=%d" % rc)

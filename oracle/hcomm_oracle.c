@@ -2089,29 +2089,106 @@ int orc_run_dbring_rs(uint32_t n, void* const* user_in, void* const* user_out, v
     return rc;
 }
 
-/* ---- the double-ring reduce-scatter executor over servers of one super pod, op-base mode with DMA reduce -------- */
+/* ---- the double-ring reduce-scatter executor over servers and super pods, op-base mode with DMA reduce ---------- */
 
-/* CollAlignedReduceScatterDoubleRingFor91093Executor with level1RankSize = n_servers > 1 and level2RankSize = 1 for one
- * rank and one chunk (KernelRun of its base, exec/coll_reduce_scatter/coll_reduce_scatter_ring_for_910_93_executor.cc:
- * 595-812):
- *   level 0: every ring position carries n_servers slices, one per server (FillMultiRingSlice :213-233: the position's
- *     share + level1Idx * sliceNum * output size), their user-memory twins at block index * count * unit + the ring's
- *     first slice offset (:297-313), and AlignedReduceScatterDoubleRing runs with the user input address only
- *     (:664-670: outputAddr = nullptr), so every fold stays in the CCL input buffer
- *     (tpl/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc: the init step walks the slices of a position,
- *     :305-332 and :232-249; so does every step, :366-425, :583-590);
- *   level 1: reduce-scatter between the servers (ring, NHR or NB, :689-746) in place on the CCL input buffer, slice i =
- *     the block of the i-th server's rank with this local index (CalLevel1DataSegsSlice :327-338);
- *   last: the own block from the CCL input to the user output (:800-808).
- * Steps: 0 the init step, 1 .. n_local - 1 the ring steps, then the level-1 steps, then the copy out. */
-static void prog_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t rank, uint32_t n_servers, uint32_t n_local,
-                                   uint64_t cur_size, uint64_t stride_bytes, uint32_t step0)
+/* The level-1 / level-2 templates with `per` slices per rank (the slice vector holds n * per entries, rank i's at
+ * i * per ..): ReduceScatterRing (tpl/temp_reduce_scatter/reduce_scatter_ring.cc:204-304), ReduceScatterNHR
+ * (reduce_scatter_nhr.cc:408-488 with the step table of :552-593) and ReduceScatterNB (reduce_scatter_nb.cc:143-230)
+ * walk the slices of a slice index one after the other wherever the single-slice case touches one slice; input and
+ * output memory are the same, inline reduce, nothing merged. */
+static void prog_ring_rs_multi(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t per)
 {
-    const uint32_t n = n_local, per = n_servers;
-    const uint32_t server = rank / n_local, local = rank % n_local;
-    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS];
-    for (uint32_t j = 0; j < n_local; j++) level0[j] = server * n_local + j;
-    for (uint32_t s = 0; s < n_servers; s++) level1[s] = s * n_local + local;
+    const uint32_t left = (rank + n - 1) % n;
+    uint32_t rx = (rank + n - 2) % n;
+    uint32_t step = 0;
+    for (uint32_t i = 0; i < n - 2; i++) { /* :232-283 */
+        for (uint32_t j = 0; j < per; j++)
+            emit(t, step, K_REDUCE, rank, B_IN, sl[rx * per + j].offset, left, B_IN, sl[rx * per + j].offset, sl[rx * per + j].size);
+        step++;
+        rx = (rx + n - 1) % n;
+    }
+    for (uint32_t j = 0; j < per; j++) /* :288-304 */
+        emit(t, step, K_REDUCE, rank, B_IN, sl[rank * per + j].offset, left, B_IN, sl[rank * per + j].offset, sl[rank * per + j].size);
+}
+
+static void prog_nhr_rs_multi(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t per, const uint32_t* slice_map)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << step;
+        const uint32_t recv_from = (rank + delta_rank) % n;
+        const uint32_t n_slices = (n - 1 + (1u << step)) / (1u << (step + 1));
+        const uint32_t delta_slice = 1u << (step + 1);
+        uint32_t rx_idx = rank;
+        for (uint32_t i = 0; i < n_slices; i++) { /* :570-587 */
+            for (uint32_t j = 0; j < per; j++) {
+                const OrcSlice s = sl[slice_map[rx_idx] * per + j];
+                emit(t, step, K_REDUCE, rank, B_IN, s.offset, recv_from, B_IN, s.offset, s.size);
+            }
+            rx_idx = (rx_idx + n - delta_slice) % n;
+        }
+    }
+}
+
+static void prog_nb_rs_multi(OrcTrace* t, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t per)
+{
+    const uint32_t n_steps = nhr_steps(n);
+    for (uint32_t step = 0; step < n_steps; step++) {
+        const uint32_t delta_rank = 1u << step;
+        const uint32_t recv_from = (n + rank - delta_rank) % n;
+        const uint32_t n_slices = (n - 1 + (1u << step)) / (1u << (step + 1));
+        const uint32_t delta_slice = 1u << (step + 1);
+        uint32_t rx_idx = rank;
+        for (uint32_t i = 0; i < n_slices; i++) {
+            for (uint32_t j = 0; j < per; j++) {
+                const OrcSlice s = sl[rx_idx * per + j];
+                emit(t, step, K_REDUCE, rank, B_IN, s.offset, recv_from, B_IN, s.offset, s.size);
+            }
+            rx_idx = (rx_idx + delta_slice) % n;
+        }
+    }
+}
+
+static uint32_t level_steps(int alg, uint32_t n) { return n < 2 ? 0 : (alg == ORC_ALG_RS_RING_STAGE ? n - 1 : nhr_steps(n)); }
+
+static void prog_level_rs(OrcTrace* t, int alg, uint32_t rank, uint32_t n, const OrcSlice* sl, uint32_t per)
+{
+    if (alg == ORC_ALG_RS_RING_STAGE) {
+        prog_ring_rs_multi(t, rank, n, sl, per);
+    } else if (alg == ORC_ALG_RS_NB) {
+        prog_nb_rs_multi(t, rank, n, sl, per);
+    } else {
+        uint32_t slice_map[ORC_MAX_RANKS];
+        nhr_rank_mapping(n, 1, slice_map);
+        prog_nhr_rs_multi(t, rank, n, sl, per, slice_map); /* Prepare(reduceAttr, false) */
+    }
+}
+
+/* CollAlignedReduceScatterDoubleRingFor91093Executor with level1RankSize = n_servers and level2RankSize = n_pods, more
+ * than one rank between them, for one rank and one chunk (KernelRun of its base, exec/coll_reduce_scatter/
+ * coll_reduce_scatter_ring_for_910_93_executor.cc:595-812); rank = (pod * n_servers + server) * n_local + local index:
+ *   level 0: every ring position carries n_pods * n_servers slices (FillMultiRingSlice :213-233: the position's share
+ *     + level1Idx * sliceNum * output size + level2Idx * sliceNum * level1RankSize * output size, level2Idx the outer
+ *     loop), their user-memory twins at block index * count * unit + the ring's first slice offset (:297-313), and
+ *     AlignedReduceScatterDoubleRing runs with the user input address only (:664-670: outputAddr = nullptr), so every
+ *     fold stays in the CCL input buffer (tpl/temp_reduce_scatter/aligned_reduce_scatter_double_ring.cc: the init step
+ *     walks the slices of a position, :305-332 and :232-249; so does every step, :366-425, :583-590);
+ *   level 1 (n_servers > 1): reduce-scatter between the servers of the pod (ring, NHR or NB, :689-746) in place on the
+ *     CCL input buffer; the i-th server's rank owns one slice per pod, the block of the rank with its place in that pod
+ *     (CalLevel1DataSegsSlice :327-350);
+ *   level 2 (n_pods > 1): reduce-scatter between the pods (:748-797), slice i = the block of the i-th pod's rank with
+ *     this place (CalLevel2DataSegsSlice :376-382);
+ *   last: the own block from the CCL input to the user output (:800-808).
+ * Steps: 0 the init step, 1 .. n_local - 1 the ring steps, then the level-1 steps, the level-2 steps, the copy out. */
+static void prog_dbring_rs_servers(OrcTrace* t, int alg1, int alg2, uint32_t rank, uint32_t n_pods, uint32_t n_servers,
+                                   uint32_t n_local, uint64_t cur_size, uint64_t stride_bytes, uint32_t step0)
+{
+    const uint32_t n = n_local, per = n_servers * n_pods;
+    const uint32_t local = rank % n_local, server = rank / n_local % n_servers, pod = rank / n_local / n_servers;
+    uint32_t level0[ORC_MAX_RANKS], level1[ORC_MAX_RANKS], level2[ORC_MAX_RANKS];
+    for (uint32_t j = 0; j < n_local; j++) level0[j] = (pod * n_servers + server) * n_local + j;
+    for (uint32_t s = 0; s < n_servers; s++) level1[s] = (pod * n_servers + s) * n_local + local;
+    for (uint32_t p = 0; p < n_pods; p++) level2[p] = (p * n_servers + server) * n_local + local;
 
     /* multiStreamSlice: ReduceScatterRingSlicePrepare with sliceNum = n_local, as on one server */
     OrcSlice seg[ORC_MAX_RANKS], multi_seg[ORC_MAX_RANKS][2], ms[2][ORC_MAX_RANKS];
@@ -2135,29 +2212,32 @@ static void prog_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t rank, uint32_
     for (uint32_t i = 1; i < n; i++) order[1][i] = order[0][n - i];
     for (uint32_t ring = 0; ring < 2; ring++)
         for (uint32_t i = 0; i < n; i++) ms[ring][i] = multi_seg[order[ring][i]][ring];
-    /* level0DataSegsSlice and multRingsUserMemSlice: index = ring position * n_servers + level1Idx */
-    OrcSlice* ccl[2];
-    OrcSlice* user[2];
+    /* level0DataSegsSlice and multRingsUserMemSlice: index = ring position * per + level2Idx * n_servers + level1Idx */
+    OrcSlice* ccl[2] = {NULL, NULL};
+    OrcSlice* user[2] = {NULL, NULL};
     for (uint32_t ring = 0; ring < 2; ring++) {
         ccl[ring] = (OrcSlice*)malloc(sizeof(OrcSlice) * n * per);
         user[ring] = (OrcSlice*)malloc(sizeof(OrcSlice) * n * per);
         if (!ccl[ring] || !user[ring]) {
             t->oom = 1;
-            for (uint32_t q = 0; q <= ring; q++) {
+            for (uint32_t q = 0; q < 2; q++) {
                 free(ccl[q]);
                 free(user[q]);
             }
             return;
         }
         for (uint32_t level0_idx = 0; level0_idx < n; level0_idx++)
-            for (uint32_t level1_idx = 0; level1_idx < per; level1_idx++) {
-                OrcSlice* c = &ccl[ring][level0_idx * per + level1_idx];
-                c->size = ms[ring][level0_idx].size;
-                c->offset = ms[ring][level0_idx].offset + (uint64_t)level1_idx * n * cur_size;
-                OrcSlice* u = &user[ring][level0_idx * per + level1_idx];
-                u->size = c->size;
-                u->offset = (c->offset / cur_size) * stride_bytes + ms[ring][0].offset;
-            }
+            for (uint32_t level2_idx = 0; level2_idx < n_pods; level2_idx++)
+                for (uint32_t level1_idx = 0; level1_idx < n_servers; level1_idx++) {
+                    const uint32_t at = level0_idx * per + level2_idx * n_servers + level1_idx;
+                    OrcSlice* c = &ccl[ring][at];
+                    c->size = ms[ring][level0_idx].size;
+                    c->offset = ms[ring][level0_idx].offset + (uint64_t)level1_idx * n * cur_size +
+                                (uint64_t)level2_idx * n * n_servers * cur_size;
+                    OrcSlice* u = &user[ring][at];
+                    u->size = c->size;
+                    u->offset = (c->offset / cur_size) * stride_bytes + ms[ring][0].offset;
+                }
     }
 
     g_rank_map = level0;
@@ -2192,68 +2272,77 @@ static void prog_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t rank, uint32_
         free(user[ring]);
     }
 
-    /* between the servers, :689-746 */
-    OrcSlice sl[ORC_MAX_RANKS];
-    for (uint32_t i = 0; i < n_servers; i++) { /* CalLevel1DataSegsSlice, :327-338 */
-        sl[i].size = cur_size;
-        sl[i].offset = (uint64_t)level1[i] * cur_size;
+    uint32_t step = step0 + n;
+    if (n_servers > 1) { /* between the servers, :689-746 */
+        OrcSlice sl[ORC_MAX_RANKS];
+        const uint32_t ranks_per_pod = n_servers * n_local;
+        for (uint32_t i = 0; i < n_servers; i++) /* CalLevel1DataSegsSlice, :327-350 */
+            for (uint32_t level2_idx = 0; level2_idx < n_pods; level2_idx++) {
+                OrcSlice* x = &sl[i * n_pods + level2_idx];
+                x->size = cur_size;
+                x->offset = n_pods <= 1 ? (uint64_t)level1[i] * cur_size
+                                        : (uint64_t)(level1[i] % ranks_per_pod) * cur_size + (uint64_t)level2_idx * ranks_per_pod * cur_size;
+            }
+        g_rank_map = level1;
+        g_step_base = step;
+        prog_level_rs(t, alg1, server, n_servers, sl, n_pods);
+        step += level_steps(alg1, n_servers);
     }
-    g_rank_map = level1;
-    g_step_base = step0 + n;
-    uint32_t level1_steps;
-    if (alg1 == ORC_ALG_RS_RING_STAGE) {
-        prog_ring_rs(t, server, n_servers, sl, NULL);
-        level1_steps = n_servers - 1;
-    } else if (alg1 == ORC_ALG_RS_NB) {
-        prog_nb_rs(t, server, n_servers, sl, NULL);
-        level1_steps = nhr_steps(n_servers);
-    } else {
-        uint32_t slice_map[ORC_MAX_RANKS];
-        nhr_rank_mapping(n_servers, 1, slice_map);
-        prog_nhr_rs(t, server, n_servers, sl, NULL, slice_map, 0); /* Prepare(reduceAttr, false), :738 */
-        level1_steps = nhr_steps(n_servers);
+    if (n_pods > 1) { /* between the super pods, :748-797 */
+        OrcSlice sl[ORC_MAX_RANKS];
+        for (uint32_t i = 0; i < n_pods; i++) { /* CalLevel2DataSegsSlice, :376-382 */
+            sl[i].size = cur_size;
+            sl[i].offset = (uint64_t)level2[i] * cur_size;
+        }
+        g_rank_map = level2;
+        g_step_base = step;
+        prog_level_rs(t, alg2, pod, n_pods, sl, 1);
+        step += level_steps(alg2, n_pods);
     }
     g_rank_map = NULL;
     /* :800-808: CalcSrcMemOffset = userRank * output size */
-    g_step_base = step0 + n + level1_steps;
+    g_step_base = step;
     emit(t, 0, K_COPY, rank, B_UOUT, 0, rank, B_IN, (uint64_t)rank * cur_size, cur_size);
     g_step_base = 0;
 }
 
-static int build_trace_dbring_rs_servers(OrcTrace* t, int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count,
-                                         uint64_t ccl_bytes, int dtype)
+static int level_alg_ok(int alg) { return alg == ORC_ALG_RS_RING_STAGE || alg == ORC_ALG_RS_NHR || alg == ORC_ALG_RS_NB; }
+
+static int build_trace_dbring_rs_servers(OrcTrace* t, int alg1, int alg2, uint32_t n_pods, uint32_t n_servers, uint32_t n_local,
+                                         uint64_t count, uint64_t ccl_bytes, int dtype)
 {
     memset(t, 0, sizeof(*t));
     const uint32_t unit = orc_dtype_size(dtype);
-    if (unit == 0 || n_servers < 2 || n_local < 3 || n_servers * n_local > ORC_MAX_RANKS) return -1;
-    if (alg1 != ORC_ALG_RS_RING_STAGE && alg1 != ORC_ALG_RS_NHR && alg1 != ORC_ALG_RS_NB) return -1;
-    const uint32_t n = n_servers * n_local;
+    if (unit == 0 || n_pods == 0 || n_servers == 0 || n_pods * n_servers < 2 || n_local < 3 ||
+        (uint64_t)n_pods * n_servers * n_local > ORC_MAX_RANKS)
+        return -1;
+    if (!level_alg_ok(alg1) || !level_alg_ok(alg2)) return -1;
+    const uint32_t n = n_pods * n_servers * n_local;
     const uint64_t max_count = ccl_bytes / n / 128u * 128u / unit; /* CalcLoopMaxCount, :167-173 */
     if (max_count == 0) return -1;
-    const uint32_t level1_steps = alg1 == ORC_ALG_RS_RING_STAGE ? n_servers - 1 : nhr_steps(n_servers);
     uint32_t step0 = 0;
     uint64_t cur_count = 0, user_off = 0;
     for (uint64_t count_left = count; count_left > 0; count_left -= cur_count) {
         cur_count = count_left > max_count ? max_count : count_left;
         g_user_off = user_off;
         for (uint32_t r = 0; r < n; r++)
-            prog_dbring_rs_servers(t, alg1, r, n_servers, n_local, cur_count * unit, count * unit, step0);
+            prog_dbring_rs_servers(t, alg1, alg2, r, n_pods, n_servers, n_local, cur_count * unit, count * unit, step0);
         g_user_off = 0;
         if (t->oom) {
             free(t->ops);
             return -2;
         }
-        step0 += n_local + level1_steps + 1;
+        step0 += n_local + level_steps(alg1, n_servers) + level_steps(alg2, n_pods) + 1;
         user_off += cur_count * unit;
     }
     return sort_trace(t);
 }
 
-int64_t orc_trace_dbring_rs_servers(int alg1, uint32_t n_servers, uint32_t n_local, uint64_t count, uint64_t ccl_bytes,
-                                    int dtype, OrcOp* out, uint64_t cap)
+int64_t orc_trace_dbring_rs_servers(int alg1, int alg2, uint32_t n_pods, uint32_t n_servers, uint32_t n_local, uint64_t count,
+                                    uint64_t ccl_bytes, int dtype, OrcOp* out, uint64_t cap)
 {
     OrcTrace t;
-    int rc = build_trace_dbring_rs_servers(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    int rc = build_trace_dbring_rs_servers(&t, alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype);
     if (rc) return rc;
     const uint64_t m = t.n < cap ? t.n : cap;
     if (out && m) memcpy(out, t.ops, m * sizeof(OrcOp));
@@ -2262,11 +2351,11 @@ int64_t orc_trace_dbring_rs_servers(int alg1, uint32_t n_servers, uint32_t n_loc
     return total;
 }
 
-int orc_run_dbring_rs_servers(int alg1, uint32_t n_servers, uint32_t n_local, void* const* user_in, void* const* user_out,
-                              void* const* ccl_in, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
+int orc_run_dbring_rs_servers(int alg1, int alg2, uint32_t n_pods, uint32_t n_servers, uint32_t n_local, void* const* user_in,
+                              void* const* user_out, void* const* ccl_in, uint64_t count, uint64_t ccl_bytes, int dtype, int op)
 {
     OrcTrace t;
-    int rc = build_trace_dbring_rs_servers(&t, alg1, n_servers, n_local, count, ccl_bytes, dtype);
+    int rc = build_trace_dbring_rs_servers(&t, alg1, alg2, n_pods, n_servers, n_local, count, ccl_bytes, dtype);
     if (rc) return rc;
     void* const* bufs[5] = {ccl_in, NULL, NULL, user_in, user_out};
     rc = exec_trace(&t, bufs, dtype, op);

@@ -45,7 +45,7 @@ static int32_t e_opbase(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) 
 static int32_t e_hier(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return x->b ? HcommGfxMeshHierEmit(x->a, x->s, x->l, x->count, x->dt, o, cap, n) : HcommGfxHierEmit(x->a, x->s, x->l, x->count, x->dt, o, cap, n); }
 static int32_t e_dbring(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingEmit(x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
 static int32_t e_dbrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingReduceScatterEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
-static int32_t e_dbhrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingHierReduceScatterEmit(x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
+static int32_t e_dbhrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxDoubleRingHierReduceScatterEmit(x->a, x->a, x->b + 1, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
 static int32_t e_hrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxHierReduceScatterEmit(x->b, x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
 static int32_t e_oph(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedHierAllReduceEmit(x->a, x->s, x->l, x->count, x->ccl, x->dt, o, cap, n); }
 static int32_t e_ops(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedSmallEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
@@ -196,8 +196,9 @@ int main(void)
                             run_plan(th, p);
                             if (!mesh) {
                                 emit_twice(e_dbhrs, &x);
-                                if (HcommGfxDoubleRingHierReduceScatterCheck(alg, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
-                                p = NULL; HcommGfxDoubleRingHierReduceScatterPlanCreate(alg, s, l, bufs[3], bufs[4], bufs[0], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                                if (HcommGfxDoubleRingHierReduceScatterCheck(alg, alg, 1, s, l, x.count, x.ccl, x.dt, &rep) == 0) ++checks;
+                                p = NULL; HcommGfxDoubleRingHierReduceScatterPlanCreate(alg, alg, 1, s, l, bufs[3], bufs[4], bufs[0], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
+                                if (s * l * 2 <= 32) { p = NULL; HcommGfxDoubleRingHierReduceScatterPlanCreate(alg, HCOMM_GFX_ALG_REDUCE_SCATTER_NHR, 2, s, l, bufs[3], bufs[4], bufs[0], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p); }
                                 emit_twice(e_oph, &x);
                                 if (alg == 0) {
                                     emit_twice(e_ophrs, &x);
