@@ -86,6 +86,8 @@ WORKLOADS = {
     "dbring_rs_bf16_n8_16MiB": ("doublering_rs", 8, 8388608, "bf16", "sum", "normal(0,1)*1e-3"),
     # the same executor over 2 servers x 8 devices, ring between the servers (blocks of 8 MiB)
     "dbringhier_ring_rs_bf16_2x8_8MiB": ("doublering_hier_rs", (2, 8), 4194304, "bf16", "sum", "normal(0,1)*1e-3"),
+    # and over 2 super pods x 2 servers x 8 devices, ring at both levels (blocks of 4 MiB)
+    "dbringhier_ring_rs_bf16_2x2x8_4MiB": ("doublering_hier_rs", (2, 2, 8), 2097152, "bf16", "sum", "normal(0,1)*1e-3"),
     # the order-preserving allreduce executor over two levels: plant + fold inside the servers, then between them
     "ophier_ring_ar_bf16_2x8_128MiB": ("ophier_ring_ar", (2, 8), 67108864, "bf16", "sum", "normal(0,1)*1e-3"),
     "ophierrs_ring_rs_bf16_2x8_8MiB": ("ophierrs_ring_rs_stage", (2, 8), 4194304, "bf16", "sum", "normal(0,1)*1e-3"),
@@ -202,9 +204,10 @@ def run_workload(args, torch, h, dev, stream, thread):
     if alg_name.startswith("hier") or alg_name.startswith("dbring_") or mesh0 or ophier or ophrs:
         dbring = alg_name.startswith("dbring_")
         alg_name, hier, n = alg_name.split("_", 1)[1], n, n[0] * n[1]
-    dbhrs = None  # (servers, ranks per server) of the double-ring reduce-scatter executor over several servers
+    dbhrs = None  # (pods, servers per pod, ranks per server) of the double-ring reduce-scatter executor over several servers
     if alg_name == "doublering_hier_rs":
-        dbhrs, n = n, n[0] * n[1]
+        dbhrs = n if len(n) == 3 else (1,) + tuple(n)
+        n = dbhrs[0] * dbhrs[1] * dbhrs[2]
     ccl_bytes = 200 << 20  # HCCL_CCL_COMM_DEFAULT_BUFFER_SIZE, src/legacy/ascend910/pub_inc/externalinput_pub.h:37
     # one-server executors on user memory (DMA reduce)
     plant = alg_name in ("order_preserved_rs", "doublering_rs", "doublering_hier_rs", "order_preserved_ar", "order_preserved_small")
@@ -256,8 +259,8 @@ def run_workload(args, torch, h, dev, stream, thread):
             return h.HierReduceScatterPlan(alg, hier[0], hier[1], in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]],
                                            [t.data_ptr() for t in d_ccl[1]], ccl_bytes, count, dt, op, mesh=mesh0)
         if dbhrs:
-            return h.DoubleRingHierReduceScatterPlan(h.Alg.REDUCE_SCATTER_RING, dbhrs[0], dbhrs[1], in_ptrs, out_ptrs,
-                                                     [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
+            return h.DoubleRingHierReduceScatterPlan(h.Alg.REDUCE_SCATTER_RING, dbhrs[1], dbhrs[2], in_ptrs, out_ptrs,
+                                                     [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op, n_pods=dbhrs[0])
         if dbrs:
             return h.DoubleRingReduceScatterPlan(in_ptrs, out_ptrs, [t.data_ptr() for t in d_ccl[0]], ccl_bytes, count, dt, op)
         if opfused and low == h.Lowering.FUSED:  # one launch on the user buffers, no CCL buffer
@@ -421,7 +424,7 @@ def run_workload(args, torch, h, dev, stream, thread):
                             for o in oracle.trace_hier_rs(oalg, hier[0], hier[1], count, ccl_bytes, odt, mesh=mesh0))
         elif dbhrs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs_servers(
-                oracle.ALG_RS_RING_STAGE, dbhrs[0], dbhrs[1], count, ccl_bytes, odt))
+                oracle.ALG_RS_RING_STAGE, dbhrs[1], dbhrs[2], count, ccl_bytes, odt, n_pods=dbhrs[0]))
         elif dbrs:
             alg_bytes = sum(o[8] * (3 if o[1] else 2) for o in oracle.trace_dbring_rs(n, count, ccl_bytes, odt))
         elif opsmall:
@@ -453,8 +456,8 @@ def run_workload(args, torch, h, dev, stream, thread):
                 oracle.run_hier_rs(oalg, hier[0], hier[1], ins, outs, host_ccl[0], host_ccl[1], count, ccl_bytes, odt, oop,
                                    mesh=mesh0)
             elif dbhrs:
-                oracle.run_dbring_rs_servers(oracle.ALG_RS_RING_STAGE, dbhrs[0], dbhrs[1], ins, outs, host_ccl[0], count,
-                                             ccl_bytes, odt, oop)
+                oracle.run_dbring_rs_servers(oracle.ALG_RS_RING_STAGE, dbhrs[1], dbhrs[2], ins, outs, host_ccl[0], count,
+                                             ccl_bytes, odt, oop, n_pods=dbhrs[0])
             elif dbrs:
                 oracle.run_dbring_rs(ins, outs, host_ccl[0], count, ccl_bytes, odt, oop)
             elif opsmall:
