@@ -621,10 +621,10 @@ def no_reuse_leg(torch, h, dev, stream, thread, reps):
     one batch of HcommLocalReduceOnThread calls = one k_reduce2_rows<bf16,SUM> launch (equally long segments: the
     two-dimensional grid), rotated over buffer sets so that a
     launch finds nothing of its operands in the 256 MB memory-side cache.
-      ring_step_shape   8 segments of 16 MiB (the headline's launch: 128 MiB written, the variant whose output
-                        the next launch is to find in that cache), 12 sets of 256 MiB -> 3 GiB between two uses
-      streaming_shape   16 segments of 64 MiB (1 GiB written: the variant with non-temporal accesses; the first
-                        halving step of the 16-rank recursive-halving allreduce), 3 sets of 2 GiB"""
+      ring_step_shape   8 segments of 16 MiB (the headline's launch: 128 MiB written), 12 sets of 256 MiB -> 3 GiB
+                        between two uses
+      streaming_shape   16 segments of 64 MiB (1 GiB written: the first halving step of the 16-rank
+                        recursive-halving allreduce), 3 sets of 2 GiB"""
     out = {}
     for key, nseg, seg_bytes, sets in (("ring_step_shape", 8, 16 << 20, 12), ("streaming_shape", 16, 64 << 20, 3)):
         gen = torch.Generator(device=dev)

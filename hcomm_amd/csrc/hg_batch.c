@@ -69,19 +69,22 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
 /*
  * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip with hg_probe_shapes.txt:
  * 16 KiB tiles, bf16 SUM, seeded non-zero data, sc1 stores) and confirmed per workload in the library.  Two regimes:
- *   kept      what the launch writes fits the memory-side cache and a later launch reads it back from there (a ring
- *             step): the overwritten operand loaded plain.  Reduce: XCDs walking runs of 128 tiles, at most four
- *             workgroups per CU once the launch writes 64 MiB (8 x 16 MiB ring steps on cold operands 69.7 -> 67.9 us,
- *             inside a ring 60.3 -> 60.2).  Copy: runs of 64 tiles, at most three workgroups per CU (cold 45.0 -> 42.7 us,
- *             inside a ring 38.0 -> 37.8).
+ *   kept      small enough to stay in the caches until the next launch reads it: the overwritten operand loaded plain,
+ *             as many workgroups per CU as the registers allow (reduce) or at most three (copy, in runs of 64 tiles:
+ *             8 x 16 MiB ring steps on cold operands 45.0 -> 42.7 us, inside a ring 38.0 -> 37.8).
  *   streaming every load non-temporal.  16 x 64 MiB that nothing touched recently: reduce 477 us with at most three
  *             workgroups per CU and runs of 32 tiles (499 with runs of 128, 522 with two workgroups), copy 320 us with
  *             at most two and runs of 64 (331 with three and runs of 128).
+ * A copy streams when it writes more than the 256 MB memory-side cache holds.  A reduce streams from 64 MiB on: with the
+ * sc1 stores its streaming shape is ahead of the kept one on ring steps too, whether or not the step before left the peer
+ * operand in that cache (library, same box: ring allreduce 8 x 128 MiB 0.709 -> 0.705 ms, two-level ring allreduce 2 x 8
+ * 1.457 -> 1.436, order-preserving reduce-scatter 0.787 -> 0.775; at 16 MiB the cache-resident 8 x 4 MiB mesh steps lose
+ * 2 % with it).
  * The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
  * Every figure can be overridden from the environment for experiments.
  */
 enum {
-    TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE, TUNE_LDS_REDUCE_FROM,
+    TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE,
     TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_CHAIN, TUNE_RUN_CHAIN, TUNE_LDS_TREE,
     TUNE_RUN_TREE, TUNE_LDS_TREE_TABLES, TUNE_N
 };
@@ -90,14 +93,10 @@ static const struct {
     uint64_t dflt;
 } g_tune_def[TUNE_N] = {
     {"HCOMM_GFX_STREAM_COPY_BYTES", 256ull << 20},   /* the 256 MB memory-side cache */
-    {"HCOMM_GFX_STREAM_REDUCE_BYTES", 256ull << 20},
+    {"HCOMM_GFX_STREAM_REDUCE_BYTES", 64ull << 20},
     {"HCOMM_GFX_LDS_COPY", 53248},
     {"HCOMM_GFX_LDS_COPY_STREAM", 65536},
-    /* kept reduce: at most four workgroups per CU once the launch writes 64 MiB or more (8 x 16 MiB ring steps on
-     * operands nothing touched recently 69.9 -> 67.8 us, the same steps in a ring 60.4 -> 59.9; two-level ring steps of
-     * 256 MiB 112.6 -> 109.7; below that size the bound costs the cache-resident 8 x 4 MiB mesh steps 1 %) */
-    {"HCOMM_GFX_LDS_REDUCE", 40960},
-    {"HCOMM_GFX_LDS_REDUCE_FROM_BYTES", 64ull << 20},
+    {"HCOMM_GFX_LDS_REDUCE", 0},
     {"HCOMM_GFX_LDS_REDUCE_STREAM", 53248},
     {"HCOMM_GFX_XCD_RUN_COPY", 64},
     {"HCOMM_GFX_XCD_RUN_COPY_STREAM", 64},
@@ -147,7 +146,7 @@ void hg_shape_seg2(HgLaunch* l, int streaming)
          * kernels (ragged tables; a few more rounds of argument reads before the data) want more workgroups per CU than
          * the row-grid kernels the table above was swept with: order-preserving reduce-scatter on blocks of 16,777,214
          * bytes 0.926 ms with these shapes, 0.997 with those; a ragged 512 MiB copy launch 170 against 187 us. */
-        l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(copy ? TUNE_STREAM_COPY_BYTES : TUNE_STREAM_REDUCE_BYTES));
+        l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > (256ull << 20));
         l->lds_bytes = l->streaming ? 53248u : (copy ? 32768u : 0u);
         t->xcd_run = (l->streaming && !copy) ? 32u : 128u;
         return;
@@ -158,7 +157,7 @@ void hg_shape_seg2(HgLaunch* l, int streaming)
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_COPY_STREAM : TUNE_RUN_COPY);
     } else {
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > tune(TUNE_STREAM_REDUCE_BYTES));
-        l->lds_bytes = l->streaming ? lds_of(TUNE_LDS_REDUCE_STREAM) : (l->bytes >= tune(TUNE_LDS_REDUCE_FROM) ? lds_of(TUNE_LDS_REDUCE) : 0u);
+        l->lds_bytes = lds_of(l->streaming ? TUNE_LDS_REDUCE_STREAM : TUNE_LDS_REDUCE);
         t->xcd_run = (uint32_t)tune(l->streaming ? TUNE_RUN_REDUCE_STREAM : TUNE_RUN_REDUCE);
     }
 }
