@@ -13,11 +13,12 @@ namespace {
 
 // ---- batched copy ------------------------------------------------------------------------------
 
-// STREAM: nothing of what the launch writes will be found in the memory-side cache by a later launch (there is more
-// of it than that cache holds, or nothing reads it soon).  Since every store of these kernels carries the sc1 policy
-// (stp<HG_ST_SEG2> / stp<HG_ST_STREAM>, the same policy today) the copy's two variants differ in their launch shape only - occupancy bound and XCD runs, set
-// by hg_shape_seg2 in hg_batch.c - and the reduce's also in how the overwritten operand is loaded.  The launch's
-// dynamic LDS size is not used as memory: it bounds the workgroups a CU runs at once.
+// STREAM: the variant for large launches - a copy that writes more than the memory-side cache holds, a reduce that
+// writes more than 64 MiB (hg_shape_seg2 in hg_batch.c decides, with the measurements behind both figures).  Every
+// store of these kernels carries the sc1 policy (stp<HG_ST_SEG2> / stp<HG_ST_STREAM>, the same policy today), so the
+// copy's two variants differ in their launch shape only - occupancy bound and XCD runs - and the reduce's also in how
+// the overwritten operand is loaded (non-temporal when streaming).  The launch's dynamic LDS size is not used as
+// memory: it bounds the workgroups a CU runs at once.
 template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const HgSeg2Table tab)
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
