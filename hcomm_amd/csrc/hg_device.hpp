@@ -130,10 +130,10 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
 
 // Cache hints of the loads.  Measured with the streaming probe (hg_probe.hip) on 8 x 16 MiB ring steps and on
 // 16 x 64 MiB launches whose operands nothing touched recently:
-//   * a launch whose output the next launch reads back from the memory-side cache (a ring step): peer operand
-//     loaded non-temporal, the operand that is overwritten loaded plain;
-//   * a launch that streams (what it writes is more than that cache holds, or nothing reads it soon): every load
-//     non-temporal, and no more than three workgroups per CU in flight.
+//   * small launches (a reduce that writes up to 64 MiB): peer operand loaded non-temporal, the operand that is
+//     overwritten loaded plain;
+//   * large ones: every load non-temporal, and no more than three workgroups per CU in flight - with the sc1
+//     stores this is ahead on the ring steps too, although the next step reads their output back.
 // The stores' policies follow further down.
 #ifndef HG_NT_LD_SRC
 #define HG_NT_LD_SRC 1 /* the peer's operand */
