@@ -258,3 +258,18 @@ def test_dtype_sizes_match_size_table():
     want = [1, 2, 4, 2, 4, 8, 8, 1, 2, 4, 8, 2, 16, 2, 1, 1, 1, 1]
     assert [oracle.lib().orc_dtype_size(i) for i in range(18)] == want
     assert oracle.lib().orc_dtype_size(255) == 0
+
+
+def test_special_inputs_make_roles_visible():
+    """The inputs do what they are for: on them a MAX / MIN with the operands swapped leaves other bits, in every
+    zone that holds ties or NaNs, for every floating type: what the GPU suite's special-value cases rely on."""
+    for dtype, dt in (("fp32", oracle.F32), ("fp16", oracle.F16), ("bf16", oracle.BF16)):
+        a, b = gen(dt, 6000, 1, "special"), gen(dt, 6000, 132, "special")
+        for o in (oracle.MAX, oracle.MIN):
+            d1, d2 = a.copy(), b.copy()
+            oracle.reduce(d1, b.copy(), dt, o)   # a in the dst role
+            oracle.reduce(d2, a.copy(), dt, o)   # b in the dst role
+            raw = np.uint32 if dt == oracle.F32 else np.uint16
+            differs = d1.view(raw) != d2.view(raw)
+            for zone in (0, 1, 2, 4):
+                assert differs[zone::6].sum() >= 50, (dtype, o, zone)
