@@ -5,10 +5,13 @@
  * hcomm_thread_c_adpt.cc) in names, argument meaning, check order and return codes.  A ThreadHandle is an
  * opaque pointer to a library-owned object, as in the reference (cpu_primitives_c_adpt.cc:66).
  */
+#define _POSIX_C_SOURCE 200809L
 #include <pthread.h>
+#include <sched.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include "hg_host.h"
 
@@ -348,26 +351,38 @@ int32_t HcommGfxLaunchLogClear(ThreadHandle thread)
 
 static int emit_to_thread(const HgLaunch* l, void* ctx) { return hg_submit((HgThread*)ctx, l); }
 
+/* 0 when the calling host thread may submit on `t` now: no batch of another host thread holds operations of it */
+int hg_thread_free_for_caller(const HgThread* t)
+{
+    const void* held = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
+    return (held && held != (const void*)&g_ctx) ? HCCL_E_UNAVAIL : HCCL_SUCCESS;
+}
+
+int hg_caller_is_batching(void) { return g_ctx.batching; }
+
 static int record_or_run(HgThread* t, const HgOp* o)
 {
+    /* a thread that holds recorded operations of another host thread's batch takes nothing from this one, batching
+     * or not: what this call launched would run ahead of what that batch recorded before it */
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     if (!g_ctx.batching) return hg_coalesce(o, 1, emit_to_thread, t);
-    const void* held = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
-    if (held && held != (const void*)&g_ctx) return HCCL_E_UNAVAIL; /* in another host thread's batch */
+    /* The thread joins this host thread's batch before anything is queued on it, so that a refusal leaves nothing
+     * behind for a later, unrelated batch.  The claim is one compare-and-exchange: of two host threads that find the
+     * thread free at the same moment one wins and the other is refused. */
+    if (__atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE) != (const void*)&g_ctx) {
+        if (g_ctx.ntouched == HG_TOUCHED_MAX) return HCCL_E_UNAVAIL;
+        const void* expected = NULL;
+        if (!__atomic_compare_exchange_n(&t->batch_owner, &expected, (const void*)&g_ctx, 0, __ATOMIC_ACQ_REL,
+                                         __ATOMIC_ACQUIRE))
+            return HCCL_E_UNAVAIL;
+        g_ctx.touched[g_ctx.ntouched++] = t;
+    }
     if (t->pending_n == t->pending_cap) {
         uint32_t cap = t->pending_cap ? t->pending_cap * 2 : 64;
         HgOp* p = (HgOp*)realloc(t->pending, cap * sizeof(*p));
-        if (!p) return HCCL_E_MEMORY;
+        if (!p) return HCCL_E_MEMORY; /* the thread stays in the batch (empty, or with what was recorded before) */
         t->pending = p;
         t->pending_cap = cap;
-    }
-    /* the thread joins this host thread's batch before anything is queued on it, so that a refusal leaves nothing
-     * behind for a later, unrelated batch */
-    const void* owner = __atomic_load_n(&t->batch_owner, __ATOMIC_ACQUIRE);
-    if (owner && owner != (const void*)&g_ctx) return HCCL_E_UNAVAIL; /* in another host thread's batch */
-    if (!owner) {
-        if (g_ctx.ntouched == HG_TOUCHED_MAX) return HCCL_E_UNAVAIL;
-        g_ctx.touched[g_ctx.ntouched++] = t;
-        __atomic_store_n(&t->batch_owner, (const void*)&g_ctx, __ATOMIC_RELEASE);
     }
     t->pending[t->pending_n++] = *o;
     return HCCL_SUCCESS;
@@ -509,6 +524,7 @@ int32_t HcommBatchTransferOnThread(
         }
         if (ret == HCCL_SUCCESS && (!o->dst || !o->src)) ret = HCCL_E_PTR;
     }
+    if (ret == HCCL_SUCCESS) ret = hg_thread_free_for_caller(t);
     if (ret == HCCL_SUCCESS) {
         if (g_ctx.batching) {
             for (uint32_t i = 0; i < transferDescNum && ret == HCCL_SUCCESS; ++i) ret = record_or_run(t, &ops[i]);
@@ -561,6 +577,7 @@ int32_t HcommGfxReduceKOnThread(
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     const uint64_t bytes = count * HcommGfxDataTypeSize(dataType);
     if (bytes == 0) return HCCL_SUCCESS;
     uintptr_t align = (uintptr_t)dst;
@@ -623,23 +640,50 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
     return HCCL_SUCCESS;
 }
 
+/* How long a wait whose record has not been issued yet may sit on the host, milliseconds (HCOMM_GFX_NOTIFY_HOST_WAIT_MS;
+ * never longer than the call's own timeOut, which is in seconds). */
+static uint64_t notify_host_wait_ms(void)
+{
+    static uint64_t cached = 0; /* value + 1 */
+    uint64_t v = __atomic_load_n(&cached, __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv("HCOMM_GFX_NOTIFY_HOST_WAIT_MS");
+        v = (e && *e ? strtoull(e, NULL, 10) : 100u) + 1u;
+        __atomic_store_n(&cached, v, __ATOMIC_RELAXED);
+    }
+    return v - 1u;
+}
+
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut)
 {
-    (void)timeOut;
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     if (notifyIdx >= t->notify_num) return HCCL_E_PARA;
     if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
-    /* A wait on a stream can only follow a record that has been issued: the reference's wait would sit until the
-     * record arrives or timeOut runs out; here a wait that finds no record pending is the one that would have run
-     * out of time, whatever timeOut says, and nothing is queued. */
-    uint64_t pending = __atomic_load_n(&t->notify_pending[notifyIdx], __ATOMIC_ACQUIRE);
-    do {
-        if (pending == 0) return HCCL_E_TIMEOUT;
-    } while (!__atomic_compare_exchange_n(&t->notify_pending[notifyIdx], &pending, pending - 1, 0, __ATOMIC_ACQ_REL,
-                                          __ATOMIC_ACQUIRE));
-    if (t->recorder) return HCCL_SUCCESS;
-    return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
+    /* A wait on a stream can only follow a record that has been issued.  The reference queues the wait and lets the
+     * device sit until the record arrives or timeOut runs out (include/hcomm_primitives.h:181-191); here the wait
+     * sits on the HOST until another host thread has issued the record - for at most min(timeOut seconds, the bound
+     * above), so that callers who drive each thread from a host thread of its own need not order the two calls -
+     * and then returns HCCL_E_TIMEOUT with nothing queued. */
+    uint64_t budget_ms = (uint64_t)timeOut * 1000u;
+    if (budget_ms > notify_host_wait_ms()) budget_ms = notify_host_wait_ms();
+    struct timespec t0;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (;;) {
+        uint64_t pending = __atomic_load_n(&t->notify_pending[notifyIdx], __ATOMIC_ACQUIRE);
+        while (pending != 0) {
+            if (__atomic_compare_exchange_n(&t->notify_pending[notifyIdx], &pending, pending - 1, 0, __ATOMIC_ACQ_REL,
+                                            __ATOMIC_ACQUIRE)) {
+                if (t->recorder) return HCCL_SUCCESS;
+                return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
+            }
+        }
+        struct timespec now;
+        clock_gettime(CLOCK_MONOTONIC, &now);
+        const uint64_t waited_ms = (uint64_t)(now.tv_sec - t0.tv_sec) * 1000u + (uint64_t)((now.tv_nsec - t0.tv_nsec) / 1000000);
+        if (waited_ms >= budget_ms) return HCCL_E_TIMEOUT;
+        sched_yield();
+    }
 }
 
 /* default notify-wait time-out of the calling host thread, seconds: NOTIFY_WAIT_TIMEOUT_DEFAULT,

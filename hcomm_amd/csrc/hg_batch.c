@@ -116,12 +116,18 @@ static const struct {
 };
 static uint64_t g_tune[TUNE_N]; /* value + 1; 0 = not read yet (same relaxed-atomic rule as env_once) */
 
+#define HG_XCD_RUN_MAX 65536u /* tiles per XCD run: the kernels compute 8 * run in 32 bits */
+
 static uint64_t tune(int i)
 {
     uint64_t v = __atomic_load_n(&g_tune[i], __ATOMIC_RELAXED);
     if (v == 0) {
         const char* e = getenv(g_tune_def[i].env);
-        v = (e && *e ? strtoull(e, NULL, 10) : g_tune_def[i].dflt) + 1u;
+        v = (e && *e ? strtoull(e, NULL, 10) : g_tune_def[i].dflt);
+        const int is_run = i == TUNE_RUN_COPY || i == TUNE_RUN_COPY_STREAM || i == TUNE_RUN_REDUCE ||
+                           i == TUNE_RUN_REDUCE_STREAM || i == TUNE_RUN_CHAIN || i == TUNE_RUN_TREE;
+        if (is_run && v > HG_XCD_RUN_MAX) v = HG_XCD_RUN_MAX;
+        v += 1u;
         __atomic_store_n(&g_tune[i], v, __ATOMIC_RELAXED);
     }
     return v - 1u;
@@ -380,8 +386,9 @@ static int coalesce_one(Coalescer* c, const HgOp* o)
     HgLaunch* l = c->l;
     const uint32_t kind = kind_of(o);
     const uint32_t dt = o->is_reduce ? o->dtype : 255u, op = o->is_reduce ? o->op : 255u;
-    const int full = l->tab.seg2.nseg == seg2_cap() ||
-                     (kind == HCOMM_GFX_KERNEL_COPY && c->bytes + o->bytes > copy_launch_bytes());
+    /* the work launch holds nothing defined until the first operation opens it */
+    const int full = c->open && (l->tab.seg2.nseg == seg2_cap() ||
+                                 (kind == HCOMM_GFX_KERNEL_COPY && c->bytes + o->bytes > copy_launch_bytes()));
     if (c->open && (l->kind != kind || l->dtype != dt || l->op != op || full || conflicts(l, o))) {
         hg_finish_seg2(l);
         c->open = 0;

@@ -59,6 +59,10 @@ typedef struct HgThread {
 } HgThread;
 
 HgThread* hg_thread_from_handle(ThreadHandle h);
+/* HCCL_SUCCESS, or HCCL_E_UNAVAIL while a batch of ANOTHER host thread holds recorded operations of the thread */
+int hg_thread_free_for_caller(const HgThread* t);
+/* whether the calling host thread is between HcommBatchModeStart and HcommBatchModeEnd */
+int hg_caller_is_batching(void);
 
 /* Turn a list of operations (stream order) into launches: consecutive independent operations of equal
  * kind / dtype / op share one launch.  Calls emit(launch, ctx) for each; stops at the first error. */

@@ -932,6 +932,9 @@ int32_t HcommGfxAllReduceLocalReduceNoAlloc(
     }
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
+    /* its launches are submitted at once: inside a batch they would run ahead of what the batch has recorded */
+    if (hg_caller_is_batching()) return HCCL_E_NOT_SUPPORT;
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     /* every rank's communication buffer is a slice of the library's own array on the thread's GPU */
     uint64_t per_rank = hg_scratch_bytes(HCOMM_GFX_ALG_ALLREDUCE_LOCAL_REDUCE, nRanks, count, (int)dataType);
     per_rank = (per_rank + 255u) & ~(uint64_t)255u;
@@ -1486,6 +1489,9 @@ int32_t HcommGfxPlanRunRange(const HcommGfxPlan* plan, ThreadHandle thread, uint
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     if (first > plan->nlaunch || n > plan->nlaunch - first) return HCCL_E_PARA;
+    /* a plan's launches are submitted at once: inside a batch they would run ahead of what the batch has recorded */
+    if (hg_caller_is_batching()) return HCCL_E_NOT_SUPPORT;
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     for (uint32_t i = first; i < first + n; ++i) {
         int rc = hg_submit(t, &plan->launches[i]);
         if (rc != HCCL_SUCCESS) return rc;

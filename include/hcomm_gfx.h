@@ -153,11 +153,12 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
 /*
  * Cross-thread ordering.  Replaces include/hcomm_primitives.h:181,191.  Record marks, on dstThread's
  * notify slot dstNotifyIdx, the point `thread` has reached; Wait makes `thread` wait for the most recent
- * record on its own slot notifyIdx.  A notify is a HIP event, so the Record has to be ISSUED (host order) before
- * the Wait that consumes it: a Wait that finds no unconsumed Record on its slot queues nothing and returns
- * HCCL_E_TIMEOUT at once - the reference's wait would sit until timeOut ran out - and the timeOut value itself is
- * not used.  Every Record is consumed by one Wait.  Neither call is available inside batch mode
- * (HCCL_E_NOT_SUPPORT).
+ * record on its own slot notifyIdx.  A notify is a HIP event, so the Record has to be ISSUED before the stream can
+ * be told to wait for it: a Wait that finds no unconsumed Record on its slot sits on the host until another host
+ * thread issues one, for at most min(timeOut seconds, HCOMM_GFX_NOTIFY_HOST_WAIT_MS = 100 ms by default), then
+ * queues nothing and returns HCCL_E_TIMEOUT - the reference's wait would sit on the device until timeOut ran out.
+ * Callers that issue both from one host thread issue the Record first.  Every Record is consumed by one Wait.
+ * Neither call is available inside batch mode (HCCL_E_NOT_SUPPORT).
  */
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);
@@ -527,6 +528,9 @@ int32_t HcommGfxScratchBytes(HcommGfxAlgorithm alg, uint32_t nRanks, uint64_t co
  * Every call on a GPU uses that GPU's one array: calls that may overlap in time on one GPU (two threads' streams with
  * no order between them) race on it; calls on one thread's stream are ordered by the stream.  The array keeps the
  * last call's contents; the schedule writes every byte of it that it later reads, so nothing needs clearing.
+ * The launches are submitted at once: between HcommBatchModeStart and HcommBatchModeEnd of the calling host thread
+ * the call returns HCCL_E_NOT_SUPPORT (it would run ahead of what the batch has recorded), and HCCL_E_UNAVAIL while
+ * another host thread's open batch holds operations of `thread`.
  */
 #define HCOMM_GFX_NOALLOC_SCRATCH_BYTES (64u << 20)
 #define HCOMM_GFX_NOALLOC_MAX_RANKS 8u
@@ -539,7 +543,9 @@ int32_t HcommGfxAllReduceLocalReduceNoAlloc(
  * thread at a time.  With HCOMM_GFX_GRAPH=1 in the environment a plan of two or more launches is replayed as a
  * HIP graph captured at its first run on the thread's stream (off by default: it measured slower than
  * launching kernel by kernel); when the caller's stream is itself being captured the launches are always
- * issued individually and become part of the caller's graph.
+ * issued individually and become part of the caller's graph.  Like every call that submits at once it returns
+ * HCCL_E_NOT_SUPPORT inside the calling host thread's own batch and HCCL_E_UNAVAIL while another host thread's open
+ * batch holds operations of `thread`.
  */
 int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread);
 

@@ -108,6 +108,7 @@ int main(void)
                     p = NULL; HcommGfxOrderPreservedPlanCreate(n, bufs[3], bufs[4], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_MIN, &p); run_plan(th, p);
                     p = NULL; HcommGfxOrderPreservedAllReducePlanCreate(n, bufs[3], bufs[4], bufs[0], bufs[1], x.ccl, x.count, x.dt, HCOMM_REDUCE_SUM, &p); run_plan(th, p);
                 }
+                HcommGfxAllReduceLocalReduceNoAlloc(th, n, bufs[0], bufs[1], x.count, x.dt, HCOMM_REDUCE_SUM); /* launches on storage of the call's own */
                 for (int ar = 0; ar < 2; ++ar) { p = NULL; HcommGfxOrderPreservedFusedPlanCreate(ar, 1, n, bufs[3], bufs[4], x.count, x.dt, HCOMM_REDUCE_PROD, &p); run_plan(th, p); }
             }
     /* the single-launch lowerings of the three-buffer schedules at sizes that keep their slices on 16-byte

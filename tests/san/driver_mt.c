@@ -69,6 +69,7 @@ static void* batch_intruder(void* arg)
     uintptr_t bad = 0;
     pthread_barrier_wait(&g_bar);
     bad += HcommThreadFree(&g_shared, 1) != HCCL_E_UNAVAIL;
+    bad += HcommLocalCopyOnThread(g_shared, (void*)0x400000, (const void*)0x300000, 4096) != HCCL_E_UNAVAIL; /* not batching either */
     bad += HcommBatchModeStart("intruder") != 0;
     bad += HcommLocalCopyOnThread(g_shared, (void*)0x400000, (const void*)0x300000, 4096) != HCCL_E_UNAVAIL;
     bad += HcommBatchModeEnd("intruder") != 0;
@@ -78,11 +79,53 @@ static void* batch_intruder(void* arg)
     return (void*)bad;
 }
 
+/* Two host threads open a batch and record into the same free thread at the same moment, 2,000 times over: the claim
+ * is one compare-and-exchange, so exactly one of them is taken each time, and the launch log holds the winner's
+ * operation alone. */
+static ThreadHandle g_raced;
+static int g_race_result[2];
+
+static void* racer(void* arg)
+{
+    const uintptr_t id = (uintptr_t)arg;
+    uintptr_t bad = 0;
+    for (int it = 0; it < 2000; ++it) {
+        if (id == 0) bad += HcommGfxRecorderThreadAlloc(&g_raced) != 0;
+        pthread_barrier_wait(&g_bar);
+        bad += HcommBatchModeStart("race") != 0;
+        g_race_result[id] = HcommLocalCopyOnThread(g_raced, (void*)(0x200000 + (id << 24)), (const void*)(0x100000 + (id << 24)), 4096);
+        pthread_barrier_wait(&g_bar); /* both have tried before either batch ends */
+        bad += HcommBatchModeEnd("race") != 0;
+        pthread_barrier_wait(&g_bar);
+        if (id == 0) {
+            const int won = (g_race_result[0] == 0) + (g_race_result[1] == 0);
+            const int lost = (g_race_result[0] == HCCL_E_UNAVAIL) + (g_race_result[1] == HCCL_E_UNAVAIL);
+            uint32_t n = 0;
+            bad += won != 1 || lost != 1;
+            bad += HcommGfxLaunchLogRead(g_raced, NULL, 0, &n) != 0 || n != 1;
+            bad += HcommThreadFree(&g_raced, 1) != 0;
+        }
+        pthread_barrier_wait(&g_bar);
+    }
+    return (void*)bad;
+}
+
 int main(void)
 {
     pthread_t t[8];
     uintptr_t bad = 0;
     if (pthread_barrier_init(&g_bar, NULL, 2)) return 2;
+    for (uintptr_t i = 0; i < 2; ++i)
+        if (pthread_create(&t[i], NULL, racer, (void*)i)) return 2;
+    for (int i = 0; i < 2; ++i) {
+        void* r = NULL;
+        pthread_join(t[i], &r);
+        bad += (uintptr_t)r;
+    }
+    if (bad) {
+        printf("racing claims: bad %lu\n", (unsigned long)bad);
+        return 1;
+    }
     if (pthread_create(&t[0], NULL, batch_owner, NULL) || pthread_create(&t[1], NULL, batch_intruder, NULL)) return 2;
     for (int i = 0; i < 2; ++i) {
         void* r = NULL;

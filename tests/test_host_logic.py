@@ -146,6 +146,66 @@ def test_notify_wait_needs_a_record_issued_before_it(rec):
         h.HcommThreadFree([other])
 
 
+def test_notify_wait_sits_for_a_record_another_host_thread_issues_late(rec):
+    """Callers that drive each thread from a host thread of its own cannot order a wait after its record: the wait
+    sits on the host (at most min(timeOut, HCOMM_GFX_NOTIFY_HOST_WAIT_MS)) until the record has been issued; a
+    timeOut of 0 seconds does not sit at all."""
+    import threading
+    import time
+    code, other = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    try:
+        t0 = time.perf_counter()
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 0) == R.E_TIMEOUT
+        assert time.perf_counter() - t0 < 0.05
+        late = threading.Timer(0.02, lambda: h.HcommThreadNotifyRecordOnThread(other, rec, 0))
+        late.start()
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.SUCCESS      # ctypes releases the GIL during the call
+        late.join()
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 0) == R.E_TIMEOUT     # that record is consumed
+    finally:
+        h.HcommThreadFree([other])
+
+
+def test_a_thread_in_another_host_threads_batch_takes_nothing(rec):
+    """Between HcommBatchModeStart and End of one host thread, the threads it recorded on refuse every other host
+    thread - batching or not, primitives, k-way reduce, plans and the entry point that allocates nothing alike - and
+    a plan or that entry point is refused inside the caller's own batch, where its launches would run ahead of what
+    the batch recorded (launch_context.cc:139-174: everything between Start and End is submitted at End)."""
+    import threading
+    ins = [0x1000000 * (r + 1) for r in range(4)]
+    outs = [(1 << 36) + 0x1000000 * (r + 1) for r in range(4)]
+    plan = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, ins, outs, 4096, DT.FP32, OP.SUM)
+    seen = {}
+
+    def other_host_thread():
+        seen["copy"] = h.HcommLocalCopyOnThread(rec, DST, SRC, 64)
+        seen["reduce_k"] = h.HcommGfxReduceKOnThread(rec, DST, [SRC, SRC + 4096], 16, DT.FP32, OP.SUM)
+        seen["plan"] = plan.run(rec)
+        seen["no_alloc"] = h.HcommGfxAllReduceLocalReduceNoAlloc(rec, ins, outs, 4096, DT.FP32, OP.SUM)
+        h.HcommBatchModeStart(b"theirs")
+        seen["batched_copy"] = h.HcommLocalCopyOnThread(rec, DST, SRC, 64)
+        seen["end"] = h.HcommBatchModeEnd(b"theirs")
+
+    h.HcommGfxLaunchLogClear(rec)
+    assert h.HcommBatchModeStart(b"mine") == R.SUCCESS
+    try:
+        assert h.HcommLocalCopyOnThread(rec, DST, SRC, 64) == R.SUCCESS       # rec now belongs to this batch
+        assert plan.run(rec) == R.E_NOT_SUPPORT
+        assert h.HcommGfxAllReduceLocalReduceNoAlloc(rec, ins, outs, 4096, DT.FP32, OP.SUM) == R.E_NOT_SUPPORT
+        th = threading.Thread(target=other_host_thread)
+        th.start()
+        th.join()
+        assert seen == {"copy": R.E_UNAVAIL, "reduce_k": R.E_UNAVAIL, "plan": R.E_UNAVAIL, "no_alloc": R.E_UNAVAIL,
+                        "batched_copy": R.E_UNAVAIL, "end": R.SUCCESS}
+        assert h.launch_log(rec) == []                                         # nothing ran ahead of the batch
+    finally:
+        assert h.HcommBatchModeEnd(b"mine") == R.SUCCESS
+    assert len(h.launch_log(rec)) == 1
+    assert plan.run(rec) == R.SUCCESS                                          # free again after End
+    plan.destroy()
+
+
 def test_timeouts_fences_and_non_blocking_twins(rec):
     """include/hcomm_primitives.h:317-318,370-371,534,542,559,567,585,593 with the host adapter's checks."""
     nan, CH = float("nan"), 0x77

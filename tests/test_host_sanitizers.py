@@ -47,3 +47,20 @@ def test_host_code_is_clean_under_tsan_with_eight_host_threads(tmp_path):
         pytest.skip("ThreadSanitizer does not run in this environment")
     assert run.returncode == 0, (run.stdout[-1000:], run.stderr[-3000:])
     assert "threads 8 bad 0" in run.stdout and "ThreadSanitizer" not in run.stderr
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no gcc")
+def test_no_alloc_entry_point_allocates_nothing_on_the_host(tmp_path):
+    """tests/san/driver_noalloc.c: every malloc / calloc / realloc / free the library's host code makes while
+    HcommGfxAllReduceLocalReduceNoAlloc runs on an executing (not a recording) thread is counted through the linker's
+    --wrap; the count must be zero over 120 calls that do reach their launches, and over refused calls."""
+    exe = str(tmp_path / "noalloc_driver")
+    cmd = ["gcc", "-O1", "-g", "-std=c11", "-DHG_STUB_GPU_PRESENT", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    cmd += [os.path.join(CSRC, f) for f in ("hg_api.c", "hg_batch.c", "hg_sched.c", "hg_plan.c", "hg_check.c")]
+    cmd += [os.path.join(SAN, "stubs.c"), os.path.join(SAN, "driver_noalloc.c"), "-o", exe, "-lpthread", "-lm",
+            "-Wl,--wrap=malloc", "-Wl,--wrap=calloc", "-Wl,--wrap=realloc", "-Wl,--wrap=free"]
+    build = subprocess.run(cmd, capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-2000:]
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.stdout, run.stderr[-2000:])
+    assert "calls 120 " in run.stdout and " allocations 0 frees 0 bad 0" in run.stdout, run.stdout
