@@ -266,7 +266,7 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
 HcommResult HcommGfxRecorderThreadAlloc(ThreadHandle* thread)
 {
     if (!thread) return HCCL_E_PTR;
-    HgThread* t = thread_new(1, NULL, 0, 2); /* two notify slots: their bookkeeping is host logic, no event behind them */
+    HgThread* t = thread_new(1, NULL, 0, HCOMM_GFX_MAX_RANKS); /* one notify slot per possible peer: their bookkeeping is host logic, no event behind them */
     if (!t) return HCCL_E_MEMORY;
     *thread = (ThreadHandle)(uintptr_t)t;
     return HCCL_SUCCESS;

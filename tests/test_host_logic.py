@@ -117,9 +117,9 @@ def test_thread_and_memory_argument_checks():
 def test_notify_argument_checks(rec):
     assert h.HcommThreadNotifyRecordOnThread(0, rec, 0) == R.E_PTR
     assert h.HcommThreadNotifyRecordOnThread(rec, 0, 0) == R.E_PTR
-    assert h.HcommThreadNotifyRecordOnThread(rec, rec, 2) == R.E_PARA   # a recorder thread has two notify slots
+    assert h.HcommThreadNotifyRecordOnThread(rec, rec, 32) == R.E_PARA  # a recorder thread has 32 notify slots
     assert h.HcommThreadNotifyWaitOnThread(0, 0, 1) == R.E_PTR
-    assert h.HcommThreadNotifyWaitOnThread(rec, 2, 1) == R.E_PARA
+    assert h.HcommThreadNotifyWaitOnThread(rec, 32, 1) == R.E_PARA
 
 
 def test_notify_wait_needs_a_record_issued_before_it(rec):
@@ -206,6 +206,64 @@ def test_a_thread_in_another_host_threads_batch_takes_nothing(rec):
     plan.destroy()
 
 
+@pytest.mark.parametrize("alg,n,count,dt", [(h.Alg.ALLREDUCE_RING, 8, 1 << 20, DT.BFP16), (h.Alg.ALLREDUCE_RHD, 6, 100003, DT.FP32),
+                                            (h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 2048, DT.FP16), (h.Alg.REDUCE_SCATTER_RING, 7, 1000003, DT.INT8),
+                                            (h.Alg.REDUCE_SCATTER_MESH, 4, 4096, DT.FP16)])
+def test_a_caller_that_batches_each_step_gets_the_plans_launches(rec, alg, n, count, dt):
+    """The reference's own boundary, driven the way its caller drives it (hcomm_amd/csrc/hg_caller.c: one
+    HcommBatchModeStart / End pair per schedule step, every rank's HcommLocalCopy/ReduceOnThread call between them):
+    the launches are those of the step-wise plan - same kernels, segments, bytes and grids, in the same order.  (A plan
+    may do better where two consecutive steps are independent - the own-slice copy and the first gather step of NHR share
+    a launch there - which a caller that ends its batch at every step cannot.)"""
+    from hcomm_amd import caller
+    scatter = alg == h.Alg.REDUCE_SCATTER_MESH
+    i, o = ptrs(n, count * h.DTYPE_SIZE[dt] * (n if scatter else 1), base=1 << 40)
+    plan = h.Plan(alg, h.Lowering.STEPWISE, i, None if alg == h.Alg.REDUCE_SCATTER_RING else o, count, dt, OP.SUM)
+    want = _launch_tuples(plan.launches())
+    plan.destroy()
+    ops = h.schedule_emit(alg, n, count, dt)
+    replay = caller.Replay(ops, {0: i, 1: o}, dt, OP.SUM)
+    h.HcommGfxLaunchLogClear(rec)
+    code, st = replay.run_batched(rec)
+    assert code == R.SUCCESS
+    assert (st.batches, st.calls) == (replay.steps, len(ops))
+    assert _launch_tuples(h.launch_log(rec)) == want
+
+
+def test_a_caller_with_one_thread_per_rank_posts_to_the_peers_it_exchanges_with():
+    """Rank r's calls on thread r, nothing batched: between the steps of a ring every thread waits for the rank it
+    reads (data) and for the rank that read it (acknowledgement) - reduce_scatter_ring.cc:211-217,254-272 - and for
+    nobody else; thread 0 forks and joins the others."""
+    from hcomm_amd import caller
+    n, count, dt = 8, 1 << 16, DT.FP32
+    recs = []
+    for _ in range(n):
+        code, t = h.HcommGfxRecorderThreadAlloc()
+        assert code == 0
+        recs.append(t)
+    try:
+        i, o = ptrs(n, count * 4, base=1 << 40)
+        ops = h.schedule_emit(h.Alg.ALLREDUCE_RING, n, count, dt)
+        code, st = caller.Replay(ops, {0: i, 1: o}, dt, OP.SUM).run_on_threads(recs)
+        assert code == R.SUCCESS
+        steps = 2 * (n - 1) + 1
+        assert (st.batches, st.calls) == (steps, len(ops))
+        # fork and join: n - 1 each.  Step 0 needs nobody.  A reduce-scatter or all-gather step after the first of its
+        # stage: two waits per rank (data from r - 1, acknowledgement from r + 1).  The own-slice copy between the
+        # stages reads no peer (acknowledgement only) and the first all-gather step follows a step in which nobody
+        # read rank r (data only): one wait per rank each.
+        assert st.notifies == 2 * (n - 1) + 2 * n * (steps - 3) + 2 * n
+        for r in range(n):                       # every rank's thread got its own 15 launches, one segment each
+            log = h.launch_log(recs[r])
+            assert len(log) == steps and all(x.nseg == 1 for x in log)
+        # every record was consumed by its wait
+        for r in range(n):
+            for q in range(n):
+                assert h.HcommThreadNotifyWaitOnThread(recs[r], q, 0) == R.E_TIMEOUT
+    finally:
+        h.HcommThreadFree(recs)
+
+
 def test_timeouts_fences_and_non_blocking_twins(rec):
     """include/hcomm_primitives.h:317-318,370-371,534,542,559,567,585,593 with the host adapter's checks."""
     nan, CH = float("nan"), 0x77
@@ -214,7 +272,7 @@ def test_timeouts_fences_and_non_blocking_twins(rec):
     assert h.HcommSetNotifyWaitTimeOut(5e9) == R.E_PARA
     assert h.HcommSetNotifyWaitTimeOut(30.5) == R.SUCCESS
     assert h.HcommThreadResAcquireTimeOut(1.0) == R.E_NOT_SUPPORT
-    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 2) == R.E_PARA       # the recorder has two notify slots
+    assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 32) == R.E_PARA      # the recorder has 32 notify slots
     assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(12345, 0) == R.E_PTR
     assert h.HcommFenceOnThread(rec) == R.SUCCESS and h.HcommFenceOnThread(12345) == R.E_PTR
     assert h.HcommChannelFenceOnThread(rec, CH) == R.SUCCESS and h.HcommChannelFenceOnThread(rec, 0) == R.E_PTR
