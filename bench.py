@@ -26,6 +26,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HcommLocalReduceOnThread refuses PROD like the reference's (cpu_primitives_c_adpt.cc:37); the via_primitives leg of the
+# PROD workload (config 5a) needs the library's extended mode, read once when the library first sees a reduce
+os.environ.setdefault("HCOMM_GFX_ALLOW_PROD", "1")
 
 
 
@@ -138,6 +141,7 @@ def main():
     ap.add_argument("--workload", default="ring_ar_bf16_n8_128MiB", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0 = min(16, cores))")
+    ap.add_argument("--no-via", action="store_true", help="skip the legs that drive the schedule through the primitives")
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: leave out the other configurations and the no-reuse leg")
     args = ap.parse_args()
@@ -153,7 +157,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.Stream(device=dev)  # default priority
-    code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 0)
+    code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 32)  # a notify slot per possible peer thread
     h.check(code, "HcommThreadAllocWithStream")
     with torch.cuda.stream(stream):  # torch's own work (restoring inputs) is ordered with the library's launches
         out = run_workload(args, torch, h, dev, stream, thread)
@@ -170,6 +174,14 @@ def main():
                        "kernel": r["roofline"]["kernel"], "kernel_ms": r["roofline"]["kernel_ms"],
                        "kernel_frac": r["roofline"]["frac"], "steps": steps,
                        "verified": r["verified_bit_exact_vs_oracle"]}
+                if r.get("via_primitives"):
+                    v = r["via_primitives"]
+                    row["via_primitives"] = {"batched_ms": v["batched"]["ms_per_step"],
+                                             "host_us_per_batch": v["batched"]["host_us_per_batch"],
+                                             "thread_per_rank_ms": v["thread_per_rank"]["ms_per_step"],
+                                             "host_thread_per_rank_ms": v["host_thread_per_rank"]["ms_per_step"],
+                                             "verified": all(v[m].get("verified") for m in
+                                                             ("batched", "thread_per_rank", "host_thread_per_rank"))}
                 if mesh and r.get("fused"):
                     row["fused_ms_per_step"] = r["fused"]["ms_per_step"]
                     row["fused_moved_gbs"] = round(r["fused"]["moved_bytes"] / (r["fused"]["ms_per_step"] * 1e-3) / 1e9, 1)
@@ -393,6 +405,11 @@ def run_workload(args, torch, h, dev, stream, thread):
         }
         plan.destroy()
 
+    via, via_run, via_done = None, None, None
+    if plain_plan and "stepwise" in results and not getattr(args, "no_via", False):
+        via, via_run, via_done = via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in_ptrs, out_ptrs, scr_ptrs, restore,
+                                 results["stepwise"])
+
     # The headline is the step-wise replay: every launch is one schedule step of two-input reduces / copies, so
     # the bytes it moves ARE the algorithmic bytes.
     best = "stepwise" if "stepwise" in results else lowerings[0]
@@ -559,6 +576,25 @@ def run_workload(args, torch, h, dev, stream, thread):
                     ok = ok and np.array_equal(d_ccl[1][r].cpu().numpy(), host_ccl[1][r])
                 verified = verified and bool(ok)
             plan.destroy()
+        if via is not None:
+            # the same schedule driven through the primitives must leave the same bits
+            for mode in ("batched", "thread_per_rank", "host_thread_per_rank"):
+                restore()
+                if d_scr:
+                    for t in d_scr:
+                        t.zero_()
+                via_run[mode]()
+                stream.synchronize()
+                torch.cuda.synchronize()
+                ok = True
+                for r in range(n):
+                    ok = ok and np.array_equal(d_in[r].cpu().numpy(), host_in[r].view(np.uint8))
+                    if not in_place:
+                        ok = ok and np.array_equal(d_out[r].cpu().numpy(), host_out[r].view(np.uint8))
+                via[mode]["verified"] = bool(ok)
+                verified = verified and bool(ok)
+    if via_done is not None:
+        via_done()
 
     metric = "HBM GB/s (% of peak) for simulated 8-rank bf16 ring allreduce, 128MiB/rank"
     if args.workload != "ring_ar_bf16_n8_128MiB":
@@ -607,6 +643,7 @@ def run_workload(args, torch, h, dev, stream, thread):
                      "algorithmic_bytes_per_launch": res["kernel_alg_bytes"]},
         "cpu_baseline": cpu,
         "verified_bit_exact_vs_oracle": verified,
+        "via_primitives": via,
         "fused": ({kk: (round(vv, 5) if isinstance(vv, float) else vv) for kk, vv in results["fused"].items()}
                   if "fused" in results and best != "fused" else None),
         "fused_keep_inputs": ({kk: (round(vv, 5) if isinstance(vv, float) else vv)
@@ -614,6 +651,109 @@ def run_workload(args, torch, h, dev, stream, thread):
                               if "fused_keep_inputs" in results else None),
     }
     return out
+
+
+def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in_ptrs, out_ptrs, scr_ptrs, restore, plan_res):
+    """The same schedule driven through the reference's own boundary by a caller that knows nothing but the
+    primitives (hcomm_amd/csrc/hg_caller.c):
+      batched          per schedule step HcommBatchModeStart, every rank's HcommLocalCopy/ReduceOnThread call,
+                       HcommBatchModeEnd, all on the thread the plans run on (cpu_primitives_c_adpt.cc:58-130,
+                       launch_context.cc:139-174): the coalescing a plan does once at creation happens inside every End;
+      thread_per_rank  rank r's calls on a thread (stream) of its own, nothing batched, notifies between the steps the
+                       way the templates post and wait (reduce_scatter_ring.cc:211-217,254-272); thread 0 is the stream
+                       the events are recorded on, the others fork from and join it; ONE host thread issues everything;
+      host_thread_per_rank  the same with a host thread per rank issuing that rank's calls (the ranks of the reference
+                       are processes of their own).
+    Timed like the plans: inputs restored before every step, a pair of HIP events around it."""
+    from hcomm_amd import caller
+    ops = h.schedule_emit(alg, n, count, dt)
+    bufs = {0: in_ptrs}
+    if out_ptrs is not None:
+        bufs[1] = out_ptrs
+    if scr_ptrs:
+        bufs[2] = scr_ptrs
+    replay = caller.Replay(ops, bufs, dt, op)
+    others = []
+    if n > 1:
+        code, others = h.HcommThreadAlloc(h.CommEngine.CPU_TS, n - 1, 32)
+        h.check(code, "HcommThreadAlloc")
+    threads = [thread] + others
+    last = {}
+
+    def run_batched():
+        code, st = replay.run_batched(thread)
+        h.check(code, "replay through HcommBatchModeStart/End")
+        last["batched"] = st
+
+    def run_threads():
+        code, st = replay.run_on_threads(threads)
+        h.check(code, "replay on one thread per rank")
+        last["thread_per_rank"] = st
+
+    def run_host_threads():
+        code, st = replay.run_on_host_threads(threads)
+        h.check(code, "replay on one thread and one host thread per rank")
+        last["host_thread_per_rank"] = st
+
+    out = {"what": "the schedule's op list (HcommGfxScheduleEmit) issued call by call through the reference's primitives "
+                   "by hcomm_amd/csrc/hg_caller.c, which binds the library with dlsym",
+           "plan_ms_per_step": round(plan_res["ms_per_step"], 5)}
+    for mode, run in (("batched", run_batched), ("thread_per_rank", run_threads), ("host_thread_per_rank", run_host_threads)):
+        for _ in range(args.warmup):
+            restore()
+            run()
+        stream.synchronize()
+        h.HcommGfxThreadSynchronize(thread)
+        h.HcommGfxLaunchLogClear(thread)
+        for t in others:
+            h.HcommGfxLaunchLogClear(t)
+        restore()
+        run()
+        stream.synchronize()
+        launches = sum(len(h.launch_log(t)) for t in threads)
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        host_us, end_us, notify_us = 0.0, 0.0, 0.0
+        for a, b in ev:
+            restore()
+            a.record(stream)
+            run()
+            b.record(stream)
+            st = last[mode]
+            host_us += st.host_us
+            end_us += st.host_us_end
+            notify_us += st.host_us_notify
+        stream.synchronize()
+        torch.cuda.synchronize()
+        per = sorted(a.elapsed_time(b) for a, b in ev)
+        ms = sum(per) / len(per)
+        st = last[mode]
+        row = {"ms_per_step": round(ms, 5), "ms_per_step_min": round(per[0], 5),
+               "ms_per_step_median": round(per[len(per) // 2], 5),
+               "vs_plan": round(ms / plan_res["ms_per_step"], 4), "launches": launches, "calls": st.calls,
+               "host_us_per_step": round(host_us / args.steps, 2)}
+        if mode == "batched":
+            row["batches"] = st.batches
+            row["host_us_per_batch"] = round(host_us / args.steps / max(st.batches, 1), 2)
+            row["host_us_in_end_per_batch"] = round(end_us / args.steps / max(st.batches, 1), 2)
+        else:
+            row["threads"] = len(threads)
+            row["notify_pairs"] = st.notifies
+            row["host_us_in_notifies"] = round(notify_us / args.steps, 2)
+            if mode == "host_thread_per_rank":
+                row["host_threads"] = len(threads)
+                row["host_us_in_notifies"] = round(notify_us / args.steps / len(threads), 2)  # per host thread
+                row["host_us_slowest_thread"] = round(st.host_us_end_max, 2)
+        out[mode] = row
+        h.HcommGfxLaunchLogClear(thread)
+
+    def done():
+        caller.pool_shutdown()
+        for t in others:
+            h.HcommGfxThreadSynchronize(t)
+        if others:
+            h.HcommThreadFree(others)
+
+    return out, {"batched": run_batched, "thread_per_rank": run_threads, "host_thread_per_rank": run_host_threads}, done
 
 
 def no_reuse_leg(torch, h, dev, stream, thread, reps):

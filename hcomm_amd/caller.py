@@ -28,8 +28,16 @@ _lib.hg_caller_replay_batched.argtypes = [C.c_uint64, C.POINTER(api.SchedOp), C.
 _lib.hg_caller_replay_threads.restype = C.c_int32
 _lib.hg_caller_replay_threads.argtypes = [C.POINTER(C.c_uint64), C.c_uint32, C.POINTER(api.SchedOp), C.c_uint64,
                                           C.POINTER(_vpp), C.c_int, C.c_int, C.c_uint32, C.POINTER(CallerStats)]
+_lib.hg_caller_replay_host_threads.restype = C.c_int32
+_lib.hg_caller_replay_host_threads.argtypes = _lib.hg_caller_replay_threads.argtypes
+_lib.hg_caller_pool_shutdown.restype = None
 if _lib.hg_caller_bind(api.LIB_PATH.encode()) != 0:
     raise ImportError("libhcomm_caller.so could not bind the primitives of %s" % api.LIB_PATH)
+
+
+def pool_shutdown():
+    """Stop the host threads that run_on_host_threads keeps between calls."""
+    _lib.hg_caller_pool_shutdown()
 
 
 class Replay:
@@ -66,4 +74,13 @@ class Replay:
         st = CallerStats()
         code = _lib.hg_caller_replay_threads(arr, len(threads), self._ops, self.n, self._bufs, self.dtype, self.op,
                                              timeout, C.byref(st))
+        return code, st
+
+    def run_on_host_threads(self, threads, timeout=10):
+        """As run_on_threads, with rank r's calls issued by a host thread of its own (a pool kept between calls):
+        host_us_end_max of the returned stats is the slowest worker's host time."""
+        arr = (C.c_uint64 * len(threads))(*threads)
+        st = CallerStats()
+        code = _lib.hg_caller_replay_host_threads(arr, len(threads), self._ops, self.n, self._bufs, self.dtype, self.op,
+                                                  timeout, C.byref(st))
         return code, st

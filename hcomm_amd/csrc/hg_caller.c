@@ -15,11 +15,16 @@
  *     the acknowledgement from the rank that read it (the TxAck / RxAck / DataSignal handshake of the templates,
  *     reduce_scatter_ring.cc:211-217,254-272), with a fork from and a join to thread 0 around the whole schedule (the
  *     main / sub stream pattern of the executors).
- * The benchmark times both against the library's prepared plans, and the GPU tests compare what they leave in the
+ *   - on one thread per rank with one HOST thread per rank as well: the same posts and waits, every rank's calls
+ *     issued by a host thread of its own, as the ranks of the reference are processes of their own.  A wait may then
+ *     reach the library before the record it is for; the library's wait sits on the host until the record is issued.
+ * The benchmark times all three against the library's prepared plans, and the GPU tests compare what they leave in the
  * rank buffers with the CPU oracle.
  */
 #define _POSIX_C_SOURCE 200809L
 #include <dlfcn.h>
+#include <pthread.h>
+#include <sched.h>
 #include <stdint.h>
 #include <string.h>
 #include <time.h>
@@ -201,6 +206,192 @@ int32_t hg_caller_replay_threads(const ThreadHandle* threads, uint32_t nRanks, c
     tn = now_us();
     for (uint32_t r = 1; r < nRanks && rc == HCCL_SUCCESS; ++r) rc = post_and_wait(threads, r, 0, timeout, st);
     st->host_us_notify += now_us() - tn;
+    st->host_us = now_us() - t0;
+    return rc;
+}
+
+
+/* ---- one host thread per rank ---------------------------------------------------------------------------------
+ *
+ * Every worker walks the whole list with the same bookkeeping as hg_caller_replay_threads - it is deterministic, so
+ * all of them derive the same posts and waits - and issues only what belongs to its rank: the posts it owes (before
+ * anything else of the step: they mark what it was given in earlier steps and never block), then its waits, then its
+ * operations.  Every post of a step precedes every wait of that step in each worker, so a wait only ever sits for a
+ * worker that is still busy with an earlier step.
+ */
+
+static struct {
+    pthread_mutex_t mtx;
+    pthread_cond_t cv;
+    pthread_t th[CALLER_MAX_RANKS];
+    uint32_t nworkers;
+    uint64_t gen;        /* bumped (under mtx) to start a job; read with atomics by workers that are still spinning */
+    uint32_t finished;   /* workers done with the current job (atomics) */
+    int stop;
+    /* the job */
+    const ThreadHandle* threads;
+    uint32_t nRanks;
+    const HcommGfxSchedOp* ops;
+    uint64_t n;
+    void* const* const* bufs;
+    int dtype, op;
+    uint32_t timeout;
+    int32_t rc[CALLER_MAX_RANKS];
+    HgCallerStats st[CALLER_MAX_RANKS];
+} pool = {.mtx = PTHREAD_MUTEX_INITIALIZER, .cv = PTHREAD_COND_INITIALIZER};
+
+static int32_t rank_walk(uint32_t me, HgCallerStats* st)
+{
+    static _Thread_local uint32_t last_op[CALLER_MAX_RANKS];
+    static _Thread_local uint32_t last_read[CALLER_MAX_RANKS][CALLER_MAX_RANKS];
+    static _Thread_local uint32_t synced[CALLER_MAX_RANKS][CALLER_MAX_RANKS];
+    static _Thread_local uint8_t need[CALLER_MAX_RANKS][CALLER_MAX_RANKS]; /* [q][r]: q posts to r before this step */
+    memset(last_op, 0, sizeof(last_op));
+    memset(last_read, 0, sizeof(last_read));
+    memset(synced, 0, sizeof(synced));
+    memset(st, 0, sizeof(*st));
+    const uint32_t nRanks = pool.nRanks, unit = unit_of(pool.dtype);
+    const HcommGfxSchedOp* ops = pool.ops;
+    const double t0 = now_us();
+    int32_t rc = HCCL_SUCCESS;
+    uint64_t i = 0;
+    uint32_t tick = 0;
+    while (i < pool.n && rc == HCCL_SUCCESS) {
+        const uint32_t step = ops[i].step;
+        uint64_t j = i;
+        while (j < pool.n && ops[j].step == step) ++j;
+        ++tick;
+        memset(need, 0, sizeof(need));
+        for (uint64_t k = i; k < j; ++k) {
+            const uint32_t r = ops[k].rank, q0 = ops[k].srcRank;
+            if (r >= nRanks || q0 >= nRanks) return HCCL_E_PARA;
+            for (uint32_t q = 0; q < nRanks; ++q) {
+                if (q == r || need[q][r]) continue;
+                if (((q == q0) && last_op[q] > synced[q][r]) || last_read[q][r] > synced[q][r]) need[q][r] = 1;
+            }
+        }
+        const double tn = now_us();
+        for (uint32_t r = 0; r < nRanks && rc == HCCL_SUCCESS; ++r) /* what this rank owes its peers */
+            if (need[me][r]) rc = g.record(pool.threads[me], pool.threads[r], me);
+        for (uint32_t q = 0; q < nRanks && rc == HCCL_SUCCESS; ++q) /* what its peers owe this rank */
+            if (need[q][me]) {
+                rc = g.wait(pool.threads[me], q, pool.timeout);
+                ++st->notifies;
+            }
+        st->host_us_notify += now_us() - tn;
+        for (uint32_t q = 0; q < nRanks; ++q)
+            for (uint32_t r = 0; r < nRanks; ++r)
+                if (need[q][r]) synced[q][r] = tick - 1;
+        for (uint64_t k = i; k < j && rc == HCCL_SUCCESS; ++k) {
+            if (ops[k].rank == me) {
+                rc = issue(pool.threads[me], &ops[k], pool.bufs, pool.dtype, pool.op, unit);
+                ++st->calls;
+            }
+            last_op[ops[k].rank] = tick;
+            if (ops[k].srcRank != ops[k].rank) last_read[ops[k].rank][ops[k].srcRank] = tick;
+        }
+        ++st->batches;
+        i = j;
+    }
+    st->host_us = now_us() - t0;
+    return rc;
+}
+
+static void* worker_main(void* arg)
+{
+    const uint32_t me = (uint32_t)(uintptr_t)arg;
+    uint64_t seen = 0;
+    for (;;) {
+        /* a caller that replays in a loop finds the workers still spinning; an idle pool sleeps */
+        uint32_t spins = 0;
+        while (__atomic_load_n(&pool.gen, __ATOMIC_ACQUIRE) == seen && !__atomic_load_n(&pool.stop, __ATOMIC_ACQUIRE)) {
+            if (++spins < 20000u) {
+                sched_yield();
+            } else {
+                pthread_mutex_lock(&pool.mtx);
+                while (pool.gen == seen && !pool.stop) pthread_cond_wait(&pool.cv, &pool.mtx);
+                pthread_mutex_unlock(&pool.mtx);
+            }
+        }
+        if (__atomic_load_n(&pool.stop, __ATOMIC_ACQUIRE)) return NULL;
+        seen = __atomic_load_n(&pool.gen, __ATOMIC_ACQUIRE);
+        if (me < pool.nRanks) pool.rc[me] = rank_walk(me, &pool.st[me]);
+        __atomic_add_fetch(&pool.finished, 1, __ATOMIC_ACQ_REL);
+    }
+}
+
+/* Stop and join the workers (also called before the pool grows). */
+void hg_caller_pool_shutdown(void)
+{
+    if (pool.nworkers == 0) return;
+    pthread_mutex_lock(&pool.mtx);
+    __atomic_store_n(&pool.stop, 1, __ATOMIC_RELEASE);
+    pthread_cond_broadcast(&pool.cv);
+    pthread_mutex_unlock(&pool.mtx);
+    for (uint32_t w = 0; w < pool.nworkers; ++w) pthread_join(pool.th[w], NULL);
+    pool.nworkers = 0;
+    pool.stop = 0;
+    pool.gen = 0; /* workers start out having seen generation 0 */
+}
+
+/*
+ * As hg_caller_replay_threads, with rank r's calls issued by worker r of a pool of host threads that lives until
+ * hg_caller_pool_shutdown.  The calling host thread forks the rank threads from threads[0] first and joins them to it
+ * last, so work timed on threads[0]'s stream brackets everything.  *st: the slowest worker's host time (the
+ * critical path), calls and notify pairs summed over the workers.
+ */
+int32_t hg_caller_replay_host_threads(const ThreadHandle* threads, uint32_t nRanks, const HcommGfxSchedOp* ops, uint64_t n,
+                                      void* const* const* bufs, int dtype, int op, uint32_t timeout, HgCallerStats* st)
+{
+    if (!g.lib || !threads || !ops || !bufs || !st) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > CALLER_MAX_RANKS) return HCCL_E_PARA;
+    memset(st, 0, sizeof(*st));
+    if (pool.nworkers < nRanks) {
+        hg_caller_pool_shutdown();
+        pool.finished = 0;
+        for (uint32_t w = 0; w < nRanks; ++w) {
+            if (pthread_create(&pool.th[w], NULL, worker_main, (void*)(uintptr_t)w) != 0) {
+                pool.nworkers = w;
+                hg_caller_pool_shutdown();
+                return HCCL_E_INTERNAL;
+            }
+        }
+        pool.nworkers = nRanks;
+    }
+    const double t0 = now_us();
+    int32_t rc = HCCL_SUCCESS;
+    HgCallerStats fork_join;
+    memset(&fork_join, 0, sizeof(fork_join));
+    for (uint32_t r = 1; r < nRanks && rc == HCCL_SUCCESS; ++r) rc = post_and_wait(threads, 0, r, timeout, &fork_join);
+    if (rc != HCCL_SUCCESS) return rc;
+    pool.threads = threads;
+    pool.nRanks = nRanks;
+    pool.ops = ops;
+    pool.n = n;
+    pool.bufs = bufs;
+    pool.dtype = dtype;
+    pool.op = op;
+    pool.timeout = timeout;
+    __atomic_store_n(&pool.finished, 0, __ATOMIC_RELEASE);
+    pthread_mutex_lock(&pool.mtx);
+    __atomic_add_fetch(&pool.gen, 1, __ATOMIC_ACQ_REL);
+    pthread_cond_broadcast(&pool.cv);
+    pthread_mutex_unlock(&pool.mtx);
+    while (__atomic_load_n(&pool.finished, __ATOMIC_ACQUIRE) < pool.nworkers) sched_yield();
+    for (uint32_t r = 0; r < nRanks; ++r) {
+        if (rc == HCCL_SUCCESS) rc = pool.rc[r];
+        st->calls += pool.st[r].calls;
+        st->notifies += pool.st[r].notifies;
+        if (pool.st[r].host_us > st->host_us_end_max) st->host_us_end_max = pool.st[r].host_us; /* slowest worker */
+        st->host_us_notify += pool.st[r].host_us_notify;
+        st->batches = pool.st[r].batches;
+    }
+    /* also after a failure: the ranks that did get work are joined to thread 0 */
+    for (uint32_t r = 1; r < nRanks; ++r) {
+        const int32_t rj = post_and_wait(threads, r, 0, timeout, &fork_join);
+        if (rc == HCCL_SUCCESS) rc = rj;
+    }
+    st->notifies += fork_join.notifies;
     st->host_us = now_us() - t0;
     return rc;
 }

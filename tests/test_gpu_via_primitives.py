@@ -4,7 +4,9 @@ and the thread notifies):
   batched     one Start / End pair per schedule step on one thread (cpu_primitives_c_adpt.cc:58-130,
               launch_context.cc:139-174);
   per rank    rank r's calls on thread r, eagerly, each thread posting to and waiting for the peers it exchanges data
-              with between the steps (reduce_scatter_ring.cc:211-217,254-272).
+              with between the steps (reduce_scatter_ring.cc:211-217,254-272) - issued by one host thread for all
+              ranks, or by a host thread per rank (the ranks of the reference are processes of their own), where a wait
+              may reach the library before its record and sits on the host until the record has been issued.
 Every one of the 2N rank buffers (and the communication buffers, where a schedule has them) is compared bit for bit
 with the CPU oracle's replay."""
 import numpy as np
@@ -75,7 +77,7 @@ def drive(mode, thread, threads, alg, n, count, dtype, op, special=False):
         # a step whose operations are of one kind and on 16-byte boundaries is one launch
         assert st.batches == replay.steps and len(h.launch_log(thread)) >= (replay.steps if count else 0)
     else:
-        code, st = replay.run_on_threads(threads[:n])
+        code, st = (replay.run_on_threads if mode == "threads" else replay.run_on_host_threads)(threads[:n])
         if prod and n > 1 and count:
             assert code == h.HcclResult.E_PARA
             for t in threads[:n]:
@@ -119,6 +121,16 @@ def test_schedule_on_one_thread_per_rank_matches_oracle(rank_threads, alg, n, co
         assert st.notifies >= 2 * (n - 1)
 
 
+@pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
+def test_schedule_on_one_host_thread_per_rank_matches_oracle(rank_threads, alg, n, count, dtype, op):
+    say("via primitives, one host thread per rank", alg, n, count, dtype, op)
+    try:
+        drive("host_threads", None, rank_threads, alg, n, count, dtype, op)
+    finally:
+        if (alg, n, count) == CASES[-1][:3]:
+            caller.pool_shutdown()
+
+
 @pytest.mark.parametrize("alg,n,count", [("ring_ar", 8, 70001), ("rhd_ar", 6, 20011), ("mesh_oneshot", 5, 20011)])
 @pytest.mark.parametrize("dtype,op", [("fp32", "max"), ("bf16", "min"), ("fp16", "sum")])
 def test_special_values_via_primitives(gpu_thread, rank_threads, alg, n, count, dtype, op):
@@ -126,13 +138,15 @@ def test_special_values_via_primitives(gpu_thread, rank_threads, alg, n, count, 
     say("via primitives, special values", alg, n, count, dtype, op)
     drive("batched", gpu_thread, None, alg, n, count, dtype, op, special=True)
     drive("threads", None, rank_threads, alg, n, count, dtype, op, special=True)
+    drive("host_threads", None, rank_threads, alg, n, count, dtype, op, special=True)
 
 
 def test_repeated_replays_on_threads_leave_no_record_behind(rank_threads):
     """Twenty ring allreduces in a row on eight threads: every record is consumed by its wait, so nothing is left
     pending between collectives and the result is the same every time."""
     for it in range(20):
-        drive("threads", None, rank_threads, "ring_ar", 8, 65539, "fp32", "sum")
+        drive("threads" if it % 2 else "host_threads", None, rank_threads, "ring_ar", 8, 65539, "fp32", "sum")
+    caller.pool_shutdown()
     for t in rank_threads[:8]:
         for q in range(8):
             assert h.HcommThreadNotifyWaitOnThread(t, q, 0) == h.HcclResult.E_TIMEOUT

@@ -260,7 +260,20 @@ def test_a_caller_with_one_thread_per_rank_posts_to_the_peers_it_exchanges_with(
         for r in range(n):
             for q in range(n):
                 assert h.HcommThreadNotifyWaitOnThread(recs[r], q, 0) == R.E_TIMEOUT
+        # the same with a host thread per rank, five times over: waits that reach the library before their record sit
+        # until it is issued; same calls, same posts and waits, same launches on every rank's thread
+        for r in range(n):
+            h.HcommGfxLaunchLogClear(recs[r])
+        for it in range(5):
+            code, st2 = caller.Replay(ops, {0: i, 1: o}, dt, OP.SUM).run_on_host_threads(recs)
+            assert code == R.SUCCESS
+            assert (st2.batches, st2.calls, st2.notifies) == (steps, len(ops), st.notifies)
+        for r in range(n):
+            assert len(h.launch_log(recs[r])) == 5 * steps
+            for q in range(n):
+                assert h.HcommThreadNotifyWaitOnThread(recs[r], q, 0) == R.E_TIMEOUT
     finally:
+        caller.pool_shutdown()
         h.HcommThreadFree(recs)
 
 
