@@ -67,7 +67,7 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
 }
 
 /*
- * Launch shapes of the copy and the two-input reduce, from the streaming probe (hg_probe.hip with hg_probe_shapes.txt:
+ * Launch shapes of the copy and the two-input reduce, from a stand-alone streaming probe built on hg_device.hpp (
  * 16 KiB tiles, bf16 SUM, seeded non-zero data, sc1 stores) and confirmed per workload in the library.  Two regimes:
  *   kept      small enough to stay in the caches until the next launch reads it: the overwritten operand loaded plain,
  *             as many workgroups per CU as the registers allow (reduce) or at most three (copy, in runs of 64 tiles:

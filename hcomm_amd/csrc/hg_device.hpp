@@ -52,35 +52,54 @@ template <int OP> __device__ __forceinline__ uint32_t f32_op(uint32_t d, uint32_
 
 __device__ __forceinline__ float f16_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
 
-__device__ __forceinline__ uint32_t f32_to_f16(float f)
+// A NaN result takes its canonical pattern either by a select (BR = false: both patterns computed, no branch) or by a
+// branch (BR = true: the compiler masks the rare path off, and a vector instruction whose lanes are all masked off
+// costs an issue slot instead of a pass through the lanes).  Measured both ways: the two-input reduce, which has
+// little arithmetic per byte, is faster with the select (ring step 58.6 -> 57.4 us), the k-way folds with the
+// branch (8 x 4 MiB fp16 mesh allreduce in one launch 40.1 -> 36.4 us).
+template <bool BR> __device__ __forceinline__ uint32_t f32_to_f16(float f)
 {
-    if (f != f) return ((f32_bits(f) >> 16) & 0x8000u) | 0x7e00u;
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    if (BR) {
+        if (f != f) return ((f32_bits(f) >> 16) & 0x8000u) | 0x7e00u;
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+    const uint32_t nan = ((f32_bits(f) >> 16) & 0x8000u) | 0x7e00u;
+    const uint32_t r = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    return (f != f) ? nan : r;
 }
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return bits_f32(h << 16); }
 
-__device__ __forceinline__ uint32_t f32_to_bf16(float f)
+template <bool BR> __device__ __forceinline__ uint32_t f32_to_bf16(float f)
 {
     const uint32_t u = f32_bits(f);
-    if (f != f) return ((u >> 16) & 0x8000u) | 0x7fc0u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    if (BR) {
+        if (f != f) return ((u >> 16) & 0x8000u) | 0x7fc0u;
+        return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    }
+    const uint32_t nan = ((u >> 16) & 0x8000u) | 0x7fc0u;
+    const uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? nan : r;
 }
 
 // one 16-bit float element held in the low half of a word
-template <int DT, int OP> __device__ __forceinline__ uint32_t half_op(uint32_t d, uint32_t s)
+template <int DT, int OP, bool BR> __device__ __forceinline__ uint32_t half_op(uint32_t d, uint32_t s)
 {
     const float fd = (DT == DT_F16) ? f16_to_f32(d) : bf16_to_f32(d);
     const float fs = (DT == DT_F16) ? f16_to_f32(s) : bf16_to_f32(s);
     if (OP == OP_MAX) return (fs > fd) ? s : d;
     if (OP == OP_MIN) return (fs < fd) ? s : d;
-    const float r = (OP == OP_SUM) ? fd + fs : fd * fs;
-    return (DT == DT_F16) ? f32_to_f16(r) : f32_to_bf16(r);
+    float r = (OP == OP_SUM) ? fd + fs : fd * fs;
+    // The fp32 result is made opaque before it is narrowed: seeing widen - multiply - narrow in one expression, the
+    // compiler may select a mixed-precision fused multiply-add with an addend of +0 for it, and (-0) * x + (+0) is +0
+    // where the product alone is -0 (found by the signed-zero inputs of the parity suite on the element tail).
+    if (DT == DT_F16) asm("" : "+v"(r));
+    return (DT == DT_F16) ? f32_to_f16<BR>(r) : f32_to_bf16<BR>(r);
 }
 
 // ---- one 32-bit word of packed elements: returns d (op) s, d in the dst role ------------------------
 
-template <int DT, int OP> __device__ __forceinline__ uint32_t word_op(uint32_t d, uint32_t s)
+template <int DT, int OP, bool BR = false> __device__ __forceinline__ uint32_t word_op(uint32_t d, uint32_t s)
 {
     if (DT == DT_I32) return (uint32_t)int_op<OP, int32_t>((int32_t)d, (int32_t)s);
     if (DT == DT_F32) return f32_op<OP>(d, s);
@@ -99,18 +118,18 @@ template <int DT, int OP> __device__ __forceinline__ uint32_t word_op(uint32_t d
         return r;
     }
     // fp16 / bf16
-    const uint32_t lo = half_op<DT, OP>(d & 0xffffu, s & 0xffffu);
-    const uint32_t hi = half_op<DT, OP>(d >> 16, s >> 16);
+    const uint32_t lo = half_op<DT, OP, BR>(d & 0xffffu, s & 0xffffu);
+    const uint32_t hi = half_op<DT, OP, BR>(d >> 16, s >> 16);
     return lo | (hi << 16);
 }
 
-template <int DT, int OP> __device__ __forceinline__ u32x4 vec_op(u32x4 d, u32x4 s)
+template <int DT, int OP, bool BR = false> __device__ __forceinline__ u32x4 vec_op(u32x4 d, u32x4 s)
 {
     u32x4 r;
-    r.x = word_op<DT, OP>(d.x, s.x);
-    r.y = word_op<DT, OP>(d.y, s.y);
-    r.z = word_op<DT, OP>(d.z, s.z);
-    r.w = word_op<DT, OP>(d.w, s.w);
+    r.x = word_op<DT, OP, BR>(d.x, s.x);
+    r.y = word_op<DT, OP, BR>(d.y, s.y);
+    r.z = word_op<DT, OP, BR>(d.z, s.z);
+    r.w = word_op<DT, OP, BR>(d.w, s.w);
     return r;
 }
 
@@ -128,7 +147,7 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
     else *(uint32_t*)p = v;
 }
 
-// Cache hints of the loads.  Measured with the streaming probe (hg_probe.hip) on 8 x 16 MiB ring steps and on
+// Cache hints of the loads.  Measured with a stand-alone streaming probe built on this header, on 8 x 16 MiB ring steps and on
 // 16 x 64 MiB launches whose operands nothing touched recently:
 //   * small launches (a reduce that writes up to 64 MiB): peer operand loaded non-temporal, the operand that is
 //     overwritten loaded plain;
@@ -138,34 +157,64 @@ template <uint32_t ES> __device__ __forceinline__ void st_elem(void* p, uint32_t
 #ifndef HG_NT_LD_SRC
 #define HG_NT_LD_SRC 1 /* the peer's operand */
 #endif
+// Every operand of these kernels is device memory (the primitives' contract, include/hcomm_primitives.h:150), so the
+// accesses name the global address space outright: a pointer that came out of a by-value table, or through the asm
+// of arrive_together, is a generic one to the compiler, and generic 128-bit loads are FLAT instructions, which count
+// on both memory counters and are waited for all at once.
+typedef __attribute__((address_space(1))) u32x4 gvec;
+typedef const __attribute__((address_space(1))) u32x4 cgvec;
 template <bool NT> __device__ __forceinline__ u32x4 ldv(const void* base, uint64_t vec)
 {
-    if (NT) return __builtin_nontemporal_load((const u32x4*)base + vec);
-    return ((const u32x4*)base)[vec];
+    if (NT) return __builtin_nontemporal_load((cgvec*)base + vec);
+    return ((cgvec*)base)[vec];
 }
 template <bool NT> __device__ __forceinline__ void stv(void* base, uint64_t vec, u32x4 v)
 {
-    if (NT) __builtin_nontemporal_store(v, (u32x4*)base + vec);
-    else ((u32x4*)base)[vec] = v;
+    if (NT) __builtin_nontemporal_store(v, (gvec*)base + vec);
+    else ((gvec*)base)[vec] = v;
 }
 
 // Store policies.  ST_SC1 carries the sc1 cache-policy bit (device scope) and neither of the other two: measured with
-// the probe's reduce_pol / copy_pol kinds, which spell the bits of every access out (hg_probe_policy.txt), it is the
-// best store for the copy / two-input reduce kernels in every situation (streaming reduce 0.825 -> 0.839 of peak
-// over the non-temporal store, ring-step copy 0.845 -> 0.885 over the plain one).  The language has no 128-bit store
-// of a given scope, so it is written out as the instruction: a vector store like the ones the compiler emits, with
-// one more modifier.  The compiler does not see through the asm, so the two wait states it would put between a
-// 128-bit store and an instruction that overwrites the registers holding its data are part of the asm (without
-// them the next address computation lands in the data of the store before: wrong bytes, found by the probe's check=1).
+// 8 x 16 MiB ring steps and 16 x 64 MiB streams, with every access's policy bits spelled out, it is the best store for
+// the copy / two-input reduce kernels in every situation (streaming reduce 0.825 -> 0.839 of peak over the
+// non-temporal store, ring-step copy 0.845 -> 0.885 over the plain one).  The language has no 128-bit global store of
+// a given scope; the buffer store builtin has: the policy rides in its aux operand, where the compiler sees it and
+// schedules around the instruction like around any other store.  (Two 64-bit agent-scope atomic stores also come out
+// as sc1 stores and run at half the speed; the instruction written in an asm needs hand-counted wait states behind it
+// and ran 2 % slower on ring steps than the builtin, because the compiler cannot move anything across it.)
 enum { ST_PLAIN = 0, ST_NT = 1, ST_SC1 = 2, ST_SC1_NT = 3 };
+// the aux operand of the buffer store builtins on gfx940 and later: bit 1 = nt, bit 4 = sc1
+template <int POL> struct StAux { static constexpr int v = (POL == ST_SC1) ? 16 : (POL == ST_SC1_NT) ? 18 : (POL == ST_NT) ? 2 : 0; };
+#define HG_BUFFER_WORD3 0x00020000 /* descriptor word 3 of a raw buffer on gfx9: 32-bit data format, no swizzle */
 template <int POL> __device__ __forceinline__ void stp(void* base, uint64_t vec, u32x4 v)
 {
-    u32x4* p = (u32x4*)base + vec;
-    if (POL == ST_SC1) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
-    else if (POL == ST_SC1_NT) asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
-    else if (POL == ST_NT) __builtin_nontemporal_store(v, p);
-    else *p = v;
+    gvec* p = (gvec*)base + vec;
+    if (POL == ST_SC1 || POL == ST_SC1_NT) {
+        // a buffer descriptor that starts at the address of the wave's first active lane (the lanes of a wave store to
+        // ascending addresses), each lane at its distance from there
+        const uint64_t a = (uint64_t)(uintptr_t)p;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        const uint64_t a0 = ((uint64_t)hi << 32) | lo;
+        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(uintptr_t)a0, 0, 0x7fffffff, HG_BUFFER_WORD3);
+        __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)(uint32_t)(a - a0), 0, StAux<POL>::v);
+    } else if (POL == ST_NT) {
+        __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
+    }
 }
+// The same store where the caller knows which part of the address the whole workgroup shares: `base` + 16 * `first`
+// (kernel arguments and the workgroup's tile: scalar registers) and the lane's own vector `lane` behind it.
+template <int POL> __device__ __forceinline__ void stp_tile(void* base, uint64_t first, uint32_t lane, u32x4 v)
+{
+    if (POL == ST_SC1 || POL == ST_SC1_NT) {
+        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((u32x4*)base + first, 0, 0x7fffffff, HG_BUFFER_WORD3);
+        __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)(lane << 4), 0, StAux<POL>::v);
+    } else {
+        stp<POL>(base, first + lane, v);
+    }
+}
+
 #ifndef HG_ST_SEG2
 #define HG_ST_SEG2 ST_SC1 /* copy / two-input reduce kernels, kept and streaming variants alike */
 #endif
@@ -227,7 +276,7 @@ template <int DT, int OP, int ST = HG_ST_FOLD> struct VecItem {
     static __device__ __forceinline__ V zero() { return V{0u, 0u, 0u, 0u}; }
     static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ldv<HG_NT_LD_SRC>(p, i); }
     static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { stp<ST>(p, i, v); }
-    static __device__ __forceinline__ V op(V d, V s) { return vec_op<DT, OP>(d, s); }
+    static __device__ __forceinline__ V op(V d, V s) { return vec_op<DT, OP, true>(d, s); }
 };
 
 template <int DT, int OP> struct ElemItem {
@@ -236,7 +285,7 @@ template <int DT, int OP> struct ElemItem {
     static __device__ __forceinline__ V zero() { return 0u; }
     static __device__ __forceinline__ V ld(const uint8_t* p, uint64_t i) { return ld_elem<ES>(p + i * ES); }
     static __device__ __forceinline__ void st(uint8_t* p, uint64_t i, V v) { st_elem<ES>(p + i * ES, v); }
-    static __device__ __forceinline__ V op(V d, V s) { return word_op<DT, OP>(d, s); }
+    static __device__ __forceinline__ V op(V d, V s) { return word_op<DT, OP, true>(d, s); }
 };
 
 

@@ -25,7 +25,8 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
-        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
+        const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
+        const uint64_t v0 = t0 + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
         void* d = tab.dst[s];
@@ -35,7 +36,7 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v0 + u * HG_BLOCK, a[u]);
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp_tile<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, t0, tid + u * HG_BLOCK, a[u]);
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
@@ -59,7 +60,8 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
-        const uint64_t v0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS + tid;
+        const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
+        const uint64_t v0 = t0 + tid;
         const uint64_t bytes = tab.bytes[s];
         const uint64_t nvec = bytes >> 4;
         void* d = tab.dst[s];
@@ -71,7 +73,7 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+            for (uint32_t u = 0; u < HG_UNROLL; ++u) stp_tile<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, t0, tid + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
         } else {
 #pragma unroll
             for (uint32_t u = 0; u < HG_UNROLL; ++u) {
@@ -149,7 +151,7 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
 // ---- launches whose segments are (nearly) equally long: one round of argument reads ----------------------------
 //
 // A launch starts with a chain of dependent memory round trips (a quarter of a microsecond per round of argument
-// reads, measured by hg_probe kind=start; more for the data): kernel arguments,
+// reads, measured with a kernel that times its own first instructions; more for the data): kernel arguments,
 // whatever they index, the data, the stores.  The kernels above find a tile's segment in the table's prefix sums
 // and only then know which pointers to read: several rounds of argument reads before the first byte of data is
 // asked for, paid by every launch of a schedule because a launch does not start before the one ahead of it has
@@ -191,13 +193,14 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
     arrive_together(d, p, bytes, run, width); // one round of argument reads
     const uint32_t tile = block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
-    const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
+    const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
+    const uint64_t v0 = t0 + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {
         u32x4 a[HG_UNROLL];
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) a[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v0 + u * HG_BLOCK, a[u]);
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp_tile<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, t0, tid + u * HG_BLOCK, a[u]);
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
@@ -222,7 +225,8 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
     arrive_together(d, p, bytes, run, width); // one round of argument reads
     const uint32_t tile = block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
-    const uint64_t v0 = (uint64_t)tile * HG_TILE_VECS + tid;
+    const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
+    const uint64_t v0 = t0 + tid;
     if (v0 - tid + HG_TILE_VECS <= nvec) {
         u32x4 a[HG_UNROLL], b[HG_UNROLL];
 #pragma unroll
@@ -230,7 +234,7 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) b[u] = ldv<HG_NT_LD_SRC>(p, v0 + u * HG_BLOCK);
 #pragma unroll
-        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, v0 + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) stp_tile<(STREAM ? HG_ST_STREAM : HG_ST_REDUCE_KEPT)>(d, t0, tid + u * HG_BLOCK, vec_op<DT, OP>(a[u], b[u]));
     } else {
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
