@@ -765,6 +765,10 @@ def no_reuse_leg(torch, h, dev, stream, thread, reps):
                         between two uses
       streaming_shape   16 segments of 64 MiB (1 GiB written: the first halving step of the 16-rank
                         recursive-halving allreduce), 3 sets of 2 GiB"""
+    import ctypes
+    hip = ctypes.CDLL(os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so"))  # the runtime torch has loaded
+    hip.hipMemcpyAsync.restype = ctypes.c_int
+    hip.hipMemcpyAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
     out = {}
     for key, nseg, seg_bytes, sets in (("ring_step_shape", 8, 16 << 20, 12), ("streaming_shape", 16, 64 << 20, 3)):
         gen = torch.Generator(device=dev)
@@ -786,20 +790,41 @@ def no_reuse_leg(torch, h, dev, stream, thread, reps):
                                                    h.HcommReduceOp.SUM), "HcommLocalReduceOnThread")
             h.check(h.HcommBatchModeEnd(b"no_reuse"), "HcommBatchModeEnd")
 
-        for k in range(sets):
-            launch(k)
-        stream.synchronize()
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-        for k, (a, b) in enumerate(ev):
-            a.record(stream)
-            launch(k)
-            b.record(stream)
-        stream.synchronize()
-        ms = sum(a.elapsed_time(b) for a, b in ev) / reps
-        alg = 3 * nseg * seg_bytes
-        out[key] = {"kernel": "k_reduce2_rows<bf16,SUM>", "segments": nseg, "segment_bytes": seg_bytes, "buffer_sets": sets,
-                    "kernel_ms": round(ms, 5), "algorithmic_bytes_per_launch": alg,
-                    "achieved": round(alg / (ms * 1e-3) / 1e9, 2), "frac": round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        def timed(fn, bytes_per_launch, kernel):
+            for k in range(sets):
+                fn(k)
+            stream.synchronize()
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            for k, (a, b) in enumerate(ev):
+                a.record(stream)
+                fn(k)
+                b.record(stream)
+            stream.synchronize()
+            ms = sum(a.elapsed_time(b) for a, b in ev) / reps
+            return {"kernel": kernel, "kernel_ms": round(ms, 5), "algorithmic_bytes_per_launch": bytes_per_launch,
+                    "achieved": round(bytes_per_launch / (ms * 1e-3) / 1e9, 2),
+                    "frac": round(bytes_per_launch / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+        # the same operands copied (dst = peer, 2 bytes of traffic per byte written) two ways: by the library, one batch of
+        # HcommLocalCopyOnThread calls = one k_copy_rows launch, and by the HIP runtime's own device-to-device copy, one
+        # hipMemcpyAsync per segment - a yardstick that is not this library's code
+        def lib_copy(k):
+            h.check(h.HcommBatchModeStart(b"no_reuse_copy"), "HcommBatchModeStart")
+            for d, p in bufs[k % sets]:
+                h.check(h.HcommLocalCopyOnThread(thread, d.data_ptr(), p.data_ptr(), seg_bytes), "HcommLocalCopyOnThread")
+            h.check(h.HcommBatchModeEnd(b"no_reuse_copy"), "HcommBatchModeEnd")
+
+        def hip_copy(k):
+            for d, p in bufs[k % sets]:
+                rc = hip.hipMemcpyAsync(d.data_ptr(), p.data_ptr(), seg_bytes, 3, stream.cuda_stream)  # 3 = device to device
+                if rc != 0:
+                    raise RuntimeError("hipMemcpyAsync returned %d" % rc)
+
+        row = timed(launch, 3 * nseg * seg_bytes, "k_reduce2_rows<bf16,SUM>")
+        row.update({"segments": nseg, "segment_bytes": seg_bytes, "buffer_sets": sets})
+        row["library_copy"] = timed(lib_copy, 2 * nseg * seg_bytes, "k_copy_rows")
+        row["hip_memcpy_d2d"] = timed(hip_copy, 2 * nseg * seg_bytes, "hipMemcpyAsync, one call per segment")
+        out[key] = row
         del bufs
     return out
 

@@ -83,6 +83,7 @@ uint64_t hg_grid_blocks(uint64_t total_tiles)
  * The bound on workgroups per CU is a dynamic LDS size nobody uses as memory: 160 KiB of LDS per CU / 52 KiB = 3.
  * Every figure can be overridden from the environment for experiments.
  */
+#define HG_TUNE_AUTO (UINT64_MAX - 1u) /* no value from the environment: the launch's own properties decide */
 enum {
     TUNE_STREAM_COPY_BYTES, TUNE_STREAM_REDUCE_BYTES, TUNE_LDS_COPY, TUNE_LDS_COPY_STREAM, TUNE_LDS_REDUCE,
     TUNE_LDS_REDUCE_STREAM, TUNE_RUN_COPY, TUNE_RUN_COPY_STREAM, TUNE_RUN_REDUCE, TUNE_RUN_REDUCE_STREAM, TUNE_LDS_CHAIN, TUNE_RUN_CHAIN, TUNE_LDS_TREE,
@@ -104,10 +105,9 @@ static const struct {
     {"HCOMM_GFX_XCD_RUN_REDUCE_STREAM", 32},
     /* the k-way folds, measured on their single-launch lowerings.  Tree (16 x 128 MiB int32 recursive halving, 8 x
      * 128 MiB bf16 NHR): 1.005 -> 0.957 ms and 0.519 -> 0.502 ms with the bound and the runs (inputs kept: 0.785 ->
-     * 0.720, 0.398 -> 0.377).  Chain: neither helps the 8 x 128 MiB ring (0.573 ms either way) and both cost the
-     * cache-resident one-shot mesh (8 x 4 MiB: 37 -> 48 us with runs of 128 tiles), so it keeps tiles as dealt. */
-    {"HCOMM_GFX_LDS_CHAIN", 0},
-    {"HCOMM_GFX_XCD_RUN_CHAIN", 0},
+     * 0.720, 0.398 -> 0.377).  Chain: decided per launch (chain_shape below) unless the environment names a value. */
+    {"HCOMM_GFX_LDS_CHAIN", HG_TUNE_AUTO},
+    {"HCOMM_GFX_XCD_RUN_CHAIN", HG_TUNE_AUTO},
     {"HCOMM_GFX_LDS_TREE", 53248},
     {"HCOMM_GFX_XCD_RUN_TREE", 128},
     /* trees read from per-segment tables (the lowering of operation lists): four workgroups per CU (deterministic mesh
@@ -115,6 +115,7 @@ static const struct {
     {"HCOMM_GFX_LDS_TREE_TABLES", 40960},
 };
 static uint64_t g_tune[TUNE_N]; /* value + 1; 0 = not read yet (same relaxed-atomic rule as env_once) */
+
 
 #define HG_XCD_RUN_MAX 65536u /* tiles per XCD run: the kernels compute 8 * run in 32 bits */
 
@@ -126,7 +127,7 @@ static uint64_t tune(int i)
         v = (e && *e ? strtoull(e, NULL, 10) : g_tune_def[i].dflt);
         const int is_run = i == TUNE_RUN_COPY || i == TUNE_RUN_COPY_STREAM || i == TUNE_RUN_REDUCE ||
                            i == TUNE_RUN_REDUCE_STREAM || i == TUNE_RUN_CHAIN || i == TUNE_RUN_TREE;
-        if (is_run && v > HG_XCD_RUN_MAX) v = HG_XCD_RUN_MAX;
+        if (is_run && v > HG_XCD_RUN_MAX && v != HG_TUNE_AUTO) v = HG_XCD_RUN_MAX;
         v += 1u;
         __atomic_store_n(&g_tune[i], v, __ATOMIC_RELAXED);
     }
@@ -221,13 +222,66 @@ uint32_t hg_launch_rows(const HgLaunch* l)
     return 0;
 }
 
+/* rank whose buffer a chain reads at position j of segment s (the kernels' fold_rank) */
+static uint32_t chain_rank(const HgFoldTable* t, uint32_t s, uint32_t j)
+{
+    if (t->ascending == 1u) return j == 0 ? t->first[s] : ((j - 1 < t->first[s]) ? j - 1 : j);
+    if (t->ascending == 2u) {
+        if (j == 0) return t->first[s];
+        const uint32_t r = t->first[s] + 1u + (t->start[s] + j - 1u) % (t->nranks - 1u);
+        return r >= t->nranks ? r - t->nranks : r;
+    }
+    int32_t r = ((int32_t)t->first[s] + (int32_t)j * t->stride) % (int32_t)t->nranks;
+    return (uint32_t)(r < 0 ? r + (int32_t)t->nranks : r);
+}
+
+/*
+ * Launch shape of a chain fold.  What a chain launch costs is decided by how much it WRITES: eight read streams alone
+ * run at 0.86 of the bus, a mix goes as reads / 0.86 + writes / w with w = 0.92 for one stream written by few
+ * workgroups per CU in long runs per XCD and 0.65 - 0.78 for eight or fifteen streams written from a full CU, and no
+ * arrangement inside the kernel (phases, tile size, load depth, buffer placement) changes the sum by more than 5 %.
+ * So a launch that does not fit the memory-side cache takes the shape its writes like: 15 writes per 8 reads (the
+ * ring allreduce with its partials) two workgroups per CU in runs of 128 tiles (8 x 128 MiB: 0.566 -> 0.536 ms); 6 per
+ * 7 (the ring reduce-scatter stage) three per CU in runs of 128 (7 x 100,000,003 fp32: 0.922 -> 0.844 ms, and 0.907
+ * with two); 8 per 8 (the allreduce without partials, chunk-mesh) three per CU in runs of 64 (0.380 -> 0.361, 0.387
+ * -> 0.381).  One-byte elements cost four times the arithmetic per byte and want the waves to hide it: four per CU
+ * (int8 reduce-scatter 0.223 -> 0.219 ms, 0.264 with two).  Launches whose operands stay in that cache keep tiles as
+ * dealt and no bound (8 x 4 MiB one-shot mesh: 37 us, 48 with runs).
+ */
+static void chain_shape(HgLaunch* l)
+{
+    HgFoldTable* t = &l->tab.fold;
+    const uint64_t lds = tune(TUNE_LDS_CHAIN), run = tune(TUNE_RUN_CHAIN);
+    uint64_t footprint = 0;
+    for (uint32_t s = 0; s < t->nseg; ++s) {
+        for (uint32_t j = 0; j < t->k; ++j) { /* inputs, each range once however many segments read it */
+            const uint32_t r = chain_rank(t, s, j);
+            int seen = 0;
+            for (uint32_t s2 = 0; s2 < s && !seen; ++s2)
+                if (t->off[s2] == t->off[s])
+                    for (uint32_t j2 = 0; j2 < t->k && !seen; ++j2) seen = chain_rank(t, s2, j2) == r;
+            if (!seen) footprint += t->bytes[s];
+        }
+        footprint += t->bytes[s] * (t->out_mode == 2u ? t->nranks : t->out_mode == 1u ? 1u : 0u);
+    }
+    const int big = footprint > tune(TUNE_STREAM_COPY_BYTES) && !t->small;
+    const uint32_t reads = t->k;
+    const uint32_t writes = (t->store_partials ? t->k - 1u : 0u) + (t->store_final_first ? 1u : 0u) +
+                            (t->out_mode == 2u ? t->nranks : t->out_mode == 1u ? 1u : 0u);
+    const uint32_t bound = HcommGfxDataTypeSize((HcommDataType)l->dtype) == 1u ? 40960u : (2u * writes > 3u * reads ? 65536u : 53248u);
+    l->lds_bytes = lds != HG_TUNE_AUTO ? (lds > HG_LDS_MAX ? HG_LDS_MAX : (uint32_t)lds) : (big ? bound : 0u);
+    t->xcd_run = run != HG_TUNE_AUTO ? (uint32_t)run : (big ? (t->store_partials ? 128u : 64u) : 0u);
+}
+
 void hg_finish_fold(HgLaunch* l)
 {
     HgFoldTable* t = &l->tab.fold;
     uint64_t tiles = 0, bytes = 0;
     l->streaming = 0;
-    l->lds_bytes = lds_of(t->tree == 6u ? TUNE_LDS_TREE_TABLES : (t->tree ? TUNE_LDS_TREE : TUNE_LDS_CHAIN));
-    t->xcd_run = (uint32_t)tune(t->tree ? TUNE_RUN_TREE : TUNE_RUN_CHAIN);
+    if (t->tree) {
+        l->lds_bytes = lds_of(t->tree == 6u ? TUNE_LDS_TREE_TABLES : TUNE_LDS_TREE);
+        t->xcd_run = (uint32_t)tune(TUNE_RUN_TREE);
+    }
     if (!t->tree) {
         /* small messages are latency-bound: below the threshold the chain runs as the grouped-load variant */
         const uint64_t small_bytes = env_once(&g_small_bytes, "HCOMM_GFX_SMALL_BYTES", 1u << 20);
@@ -249,6 +303,7 @@ void hg_finish_fold(HgLaunch* l)
                         ? 1u
                         : 0u;
         if (t->direct) t->small = 1u;
+        chain_shape(l);
     } else {
         /* small trees of up to 16 positions likewise (the launcher still checks what only it can see): up to 4 MiB
          * of output per launch (8 ranks: 16.6 us against 18.1 there, 72 against 68 at 16 MiB) */
