@@ -33,6 +33,12 @@ def test_library_exports_every_declared_symbol():
     for n in sorted(names):
         assert hasattr(h.lib, n), "libhcomm_gfx.so does not export " + n
     assert len(names) >= 27
+    plugin = open(os.path.join(ROOT, "include", "hcomm_gfx_nic_plugin.h")).read()
+    plugin = re.sub(r"/\*.*?\*/", "", plugin, flags=re.S)
+    pnames = set(re.findall(r"\b(HcommNicPlugin\w+)\s*\(", plugin))
+    assert pnames == {"HcommNicPluginGetInfo", "HcommNicPluginCreateEndpoint", "HcommNicPluginCreateChannel"}
+    for n in sorted(pnames):
+        assert hasattr(h.lib, n), "libhcomm_gfx.so does not export " + n
 
 
 def test_enum_values_match_the_reference_headers():
@@ -345,7 +351,7 @@ def test_batch_transfer_descriptors(rec):
     assert h.HcommBatchTransferOnThread(rec, CH, [null]) == R.E_PTR
     assert h.launch_log(rec) == []                     # validated as a whole before anything is enqueued
     import ctypes
-    assert ctypes.sizeof(h.BatchTransferDesc) == 64    # include/hcomm_primitives.h:91-131
+    assert C.sizeof(h.BatchTransferDesc) == 64    # include/hcomm_primitives.h:91-131
 
 
 def test_local_reduce_plan_needs_scratch_and_power_of_two(rec):
@@ -833,3 +839,65 @@ def test_launch_records_name_the_grid_shape():
             p.destroy()
     finally:
         h.HcommGfxSetDirectLaunches(before)
+
+
+# ---- the NIC-plugin face of the library ---------------------------------------------------------------------------
+
+def test_nic_plugin_tables_have_the_references_layout_and_refuse_what_needs_a_network(rec):
+    """hcomm_nic_plugin.h:23-104 as the reference's plugin manager checks it (nic_plugin_manager.cc:61-79,206-270):
+    magic words, versions, sizes, one protocol from the plugins' own range; the data-plane entries run on a thread of
+    this library (a recorder here: launches are logged), everything that needs a network says HCCL_E_NOT_SUPPORT."""
+    from hcomm_amd import nic_plugin as P
+    info = P.get_info()
+    assert (info.header.version, info.header.magicWord, info.header.size) == (1, 0x0fcf0f1f, 112)
+    assert info.name == b"hcomm_gfx" and info.protocolCount == 1 and info.protocols[0] >= 1000
+    assert C.sizeof(P.CommAbiHeader) == 16 and C.sizeof(P.ChannelOps) == 208 and C.sizeof(P.EndpointOps) == 80
+    assert C.sizeof(P.PluginInfo) == 112 and C.sizeof(P.CommMem) == 24
+    assert P.create_endpoint(None)[0] == R.E_PTR
+    code, ep_ctx, ep = P.create_endpoint(P.endpoint_desc())
+    assert code == R.SUCCESS
+    assert (ep.header.version, ep.header.magicWord, ep.header.size) == (1, 0x0fcf0f2f, 80)
+    assert ep.init(ep_ctx) == R.SUCCESS
+    assert ep.getListenPort(ep_ctx, None) == R.E_NOT_SUPPORT
+    assert ep.registerMemory(ep_ctx, None, None, None) == R.E_NOT_SUPPORT
+    assert P.create_channel(None, P.channel_desc(3))[0] == R.E_PTR
+    assert P.create_channel(ep_ctx, None)[0] == R.E_PTR
+    code, ch_ctx, ch = P.create_channel(ep_ctx, P.channel_desc(3))
+    assert code == R.SUCCESS
+    assert (ch.header.version, ch.header.magicWord, ch.header.size) == (1, 0x0fcf0f3f, 208)
+    assert ch.init(ch_ctx) == R.SUCCESS
+    status = C.c_int32(-1)
+    assert ch.getStatus(ch_ctx, C.byref(status)) == R.SUCCESS and status.value == 0
+    # data plane on a thread: the same checks, in the same order, as the primitives
+    h.HcommGfxLaunchLogClear(rec)
+    assert ch.writeReduceOnThread(ch_ctx, rec, None, SRC, 4, DT.FP32, OP.SUM) == R.E_PTR
+    assert ch.writeReduceOnThread(ch_ctx, rec, DST, SRC, 4, DT.INT64, OP.SUM) == R.E_PARA
+    assert ch.writeReduceOnThread(ch_ctx, 0, DST, SRC, 4, DT.FP32, OP.SUM) == R.E_PTR
+    assert ch.writeReduceOnThread(None, rec, DST, SRC, 4, DT.FP32, OP.SUM) == R.E_PTR
+    assert ch.writeReduceOnThread(ch_ctx, rec, DST, SRC, 1 << 20, DT.BFP16, OP.MAX) == R.SUCCESS
+    assert ch.readReduceOnThread(ch_ctx, rec, DST, SRC, 1 << 20, DT.BFP16, OP.MAX) == R.SUCCESS
+    assert ch.writeOnThread(ch_ctx, rec, DST, SRC, 4096) == R.SUCCESS
+    assert ch.readNbiOnThread(ch_ctx, rec, DST, SRC, 4096) == R.SUCCESS
+    descs = (h.BatchTransferDesc * 2)(h.desc_reduce(DST, SRC, 256, DT.FP32, OP.SUM),
+                                      h.desc_reduce(DST + (1 << 24), SRC + (1 << 24), 256, DT.FP32, OP.SUM, read=True))
+    assert ch.batchTransferOnThread(ch_ctx, rec, descs, 2) == R.SUCCESS
+    log = h.launch_log(rec)
+    assert [(r.kind, r.nseg) for r in log] == [(h.Kernel.REDUCE2, 1), (h.Kernel.REDUCE2, 1), (h.Kernel.COPY, 1),
+                                               (h.Kernel.COPY, 1), (h.Kernel.REDUCE2, 2)]
+    # what needs a host-side engine or a remote process
+    assert ch.writeNbi(ch_ctx, DST, SRC, 16) == R.E_NOT_SUPPORT
+    assert ch.readNbi(ch_ctx, DST, SRC, 16) == R.E_NOT_SUPPORT
+    assert ch.writeWithNotifyOnThread(ch_ctx, rec, DST, SRC, 16, 0) == R.E_NOT_SUPPORT
+    assert ch.writeReduceWithNotifyOnThread(ch_ctx, rec, DST, SRC, 4, DT.FP32, OP.SUM, 0) == R.E_NOT_SUPPORT
+    assert ch.notifyRecord(ch_ctx, 0) == R.E_NOT_SUPPORT and ch.notifyWait(ch_ctx, 0, 1) == R.E_NOT_SUPPORT
+    # the channel's own notifies: three of them, each record consumed by one wait
+    assert ch.notifyWaitOnThread(ch_ctx, rec, 0, 1) == R.E_TIMEOUT
+    assert ch.notifyRecordOnThread(ch_ctx, rec, 3) == R.E_PARA
+    assert ch.notifyRecordOnThread(ch_ctx, rec, 2) == R.SUCCESS
+    assert ch.notifyWaitOnThread(ch_ctx, rec, 1, 1) == R.E_TIMEOUT
+    assert ch.notifyWaitOnThreadWithDefaultTimeout(ch_ctx, rec, 2) == R.SUCCESS
+    assert ch.notifyWaitOnThread(ch_ctx, rec, 2, 1) == R.E_TIMEOUT
+    assert ch.fence(ch_ctx) == R.SUCCESS and ch.fenceOnThread(ch_ctx, rec) == R.SUCCESS
+    assert ch.drainOnThread(ch_ctx, rec) == R.SUCCESS and ch.drainOnThread(ch_ctx, 12345) == R.E_PTR
+    assert ch.destroy(ch_ctx) == R.SUCCESS
+    assert ep.destroy(ep_ctx) == R.SUCCESS
