@@ -143,6 +143,9 @@ def main():
     ap.add_argument("--workload", default="ring_ar_bf16_n8_128MiB", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / verification leg")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0 = min(16, cores))")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="ring allreduce bf16 over rank counts x per-rank sizes (both sides of every launch-shape threshold): "
+                         "one JSON line with the dominant kernel's fraction of the HBM roofline per point")
     ap.add_argument("--no-via", action="store_true", help="skip the legs that drive the schedule through the primitives")
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: leave out the other configurations and the no-reuse leg")
@@ -161,6 +164,12 @@ def main():
     stream = torch.cuda.Stream(device=dev)  # default priority
     code, thread = h.HcommThreadAllocWithStream(stream.cuda_stream, 32)  # a notify slot per possible peer thread
     h.check(code, "HcommThreadAllocWithStream")
+    if args.shape_sweep:
+        with torch.cuda.stream(stream):
+            out = shape_sweep(args, torch, h, dev, stream, thread)
+        h.HcommThreadFreeWithStream([thread])
+        print(json.dumps(out))
+        return
     with torch.cuda.stream(stream):  # torch's own work (restoring inputs) is ordered with the library's launches
         out = run_workload(args, torch, h, dev, stream, thread)
         if args.workload == "ring_ar_bf16_n8_128MiB" and not args.no_configs:
@@ -425,6 +434,7 @@ def run_workload(args, torch, h, dev, stream, thread):
             "algorithmic_bytes": plan.info.algorithmicBytes,
             "moved_bytes": plan.info.movedBytes,
             "kernel": kernel_name(launches[first]),
+            "kernel_variant": ("rows" if launches[first].rows else "one-dimensional") + (", streaming" if launches[first].streaming else ""),
             "kernel_ms": dom_ms,
             "kernel_alg_bytes": dom_bytes,
             "kernel_gbs": dom_bytes / (dom_ms * 1e-3) / 1e9,
@@ -677,7 +687,7 @@ def run_workload(args, torch, h, dev, stream, thread):
                      "traffic_is": "L2 <-> fabric bytes (FETCH_SIZE / WRITE_SIZE count below the L2): equal to the "
                                    "algorithmic bytes means no re-reads and no write amplification; how many of them "
                                    "the memory-side cache served instead of HBM these counters cannot tell",
-                     "kernel": res["kernel"], "kernel_ms": round(res["kernel_ms"], 5),
+                     "kernel": res["kernel"], "kernel_variant": res["kernel_variant"], "kernel_ms": round(res["kernel_ms"], 5),
                      "algorithmic_bytes_per_launch": res["kernel_alg_bytes"]},
         "cpu_baseline": cpu,
         "verified_bit_exact_vs_oracle": verified,
@@ -792,6 +802,29 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
             h.HcommThreadFree(others)
 
     return out, {"batched": run_batched, "thread_per_rank": run_threads, "host_thread_per_rank": run_host_threads}, done
+
+
+def shape_sweep(args, torch, h, dev, stream, thread):
+    """Ring allreduce SUM bf16, step-wise, over rank counts and per-rank sizes chosen on both sides of the sizes at which
+    a launch changes shape (a reduce launch of a ring step writes one slice per rank = the per-rank size: streaming from
+    64 MiB on; a copy streams from 256 MiB on).  Per point: time, algorithmic GB/s, and the reduce kernel's fraction of
+    the HBM roofline from HIP events around its launches."""
+    points = []
+    for n in (4, 8, 16, 32):
+        for mib in (32, 63, 65, 128, 255, 257, 512):
+            name = "ring_ar_bf16_n%d_%dMiB" % (n, mib)
+            WORKLOADS[name] = ("ring_ar", n, mib << 19, "bf16", "sum", "normal(0,1)*1e-3")
+            sub = argparse.Namespace(workload=name, steps=max(5, min(args.steps, 10)), warmup=2, lowering="stepwise", no_cpu=True,
+                                     cpu_threads=0, no_via=True)
+            r = run_workload(sub, torch, h, dev, stream, thread)
+            footprint = 2 * n * (mib << 20)
+            points.append({"ranks": n, "mib_per_rank": mib, "ms_per_step": r["ms_per_step"], "gbs": r["value"],
+                           "frac": round(r["value"] / HBM_PEAK_GBS, 4), "kernel": r["roofline"]["kernel"],
+                           "kernel_variant": r["roofline"]["kernel_variant"], "kernel_us": round(r["roofline"]["kernel_ms"] * 1e3, 2),
+                           "kernel_frac": r["roofline"]["frac"], "footprint_mib": footprint >> 20})
+            torch.cuda.empty_cache()
+    return {"metric": "ring allreduce SUM bf16, step-wise: fraction of the HBM roofline over rank counts and per-rank sizes",
+            "unit": "fraction of 8 TB/s", "n_gpus": 1, "points": points}
 
 
 def no_reuse_leg(torch, h, dev, stream, thread, reps):

@@ -240,7 +240,7 @@ __global__ __launch_bounds__(HG_BLOCK) void k_fold_chain_direct(const HgDirectTa
     const uint32_t nvec = bytes >> 4;
     const uint32_t v = blockIdx.x * HG_BLOCK + tid;
     // the grid is as wide as the longest segment: workgroups beyond this segment's tiles pass both tests untaken
-    if (v < nvec) fold_direct<VecItem<DT, OP, HG_ST_FOLD_DIRECT>, ACC_IS_DST>(in, out, k, nout, store, v);
+    if (v < nvec) fold_direct<VecItem<DT, OP, HG_ST_FOLD_DIRECT, false>, ACC_IS_DST>(in, out, k, nout, store, v);
     if (blockIdx.x + 1u == tiles) { // the segment's last tile also owns its element tail
         const uint32_t e = (nvec << 4) / ES + tid;
         if ((e + 1u) * ES <= bytes) fold_direct<ElemItem<DT, OP>, ACC_IS_DST>(in, out, k, nout, store, e);

@@ -304,7 +304,7 @@ template <int DT, int OP, int L> __global__ __launch_bounds__(HG_BLOCK) void k_f
     const uint32_t nvec = bytes >> 4;
     const uint32_t v = blockIdx.x * HG_BLOCK + tid;
     // the grid is as wide as the longest segment: workgroups beyond this segment's tiles pass both tests untaken
-    if (v < nvec) fold_tree_direct<VecItem<DT, OP, HG_ST_FOLD_DIRECT>, L>(in, out, have, store, nout, v);
+    if (v < nvec) fold_tree_direct<VecItem<DT, OP, HG_ST_FOLD_DIRECT, false>, L>(in, out, have, store, nout, v);
     if (blockIdx.x == nvec / HG_BLOCK) { // the tile the element tail falls into
         const uint32_t e = (nvec << 4) / ES + tid;
         if ((e + 1u) * ES <= bytes) fold_tree_direct<ElemItem<DT, OP>, L>(in, out, have, store, nout, e);
