@@ -202,8 +202,8 @@ def main():
                                              "host_us_per_batch": v["batched"]["host_us_per_batch"],
                                              "thread_per_rank_ms": v["thread_per_rank"]["ms_per_step"],
                                              "host_thread_per_rank_ms": v["host_thread_per_rank"]["ms_per_step"],
-                                             "verified": all(v[m].get("verified") for m in
-                                                             ("batched", "thread_per_rank", "host_thread_per_rank"))}
+                                             "thread_per_rank_batched_ms": v["thread_per_rank_batched"]["ms_per_step"],
+                                             "verified": all(v[m].get("verified") for m in VIA_MODES)}
                 for low in ("fused", "fused_keep_inputs"):
                     if r.get(low):
                         row[low + "_ms_per_step"] = r[low]["ms_per_step"]
@@ -626,7 +626,7 @@ def run_workload(args, torch, h, dev, stream, thread):
             plan.destroy()
         if via is not None:
             # the same schedule driven through the primitives must leave the same bits
-            for mode in ("batched", "thread_per_rank", "host_thread_per_rank"):
+            for mode in VIA_MODES:
                 restore()
                 if d_scr:
                     for t in d_scr:
@@ -701,6 +701,9 @@ def run_workload(args, torch, h, dev, stream, thread):
     return out
 
 
+VIA_MODES = ("batched", "thread_per_rank", "host_thread_per_rank", "thread_per_rank_batched")
+
+
 def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in_ptrs, out_ptrs, scr_ptrs, restore, plan_res):
     """The same schedule driven through the reference's own boundary by a caller that knows nothing but the
     primitives (hcomm_amd/csrc/hg_caller.c):
@@ -711,7 +714,10 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
                        way the templates post and wait (reduce_scatter_ring.cc:211-217,254-272); thread 0 is the stream
                        the events are recorded on, the others fork from and join it; ONE host thread issues everything;
       host_thread_per_rank  the same with a host thread per rank issuing that rank's calls (the ranks of the reference
-                       are processes of their own).
+                       are processes of their own);
+      thread_per_rank_batched  the calls of thread_per_rank, posts and waits included, between ONE HcommBatchModeStart /
+                       End pair - the whole collective as one batch over all its threads, what the reference submits as
+                       one task graph (launch_context.cc:16-44); HcommBatchModeEnd resolves the notifies on the host.
     Timed like the plans: inputs restored before every step, a pair of HIP events around it."""
     from hcomm_amd import caller
     ops = h.schedule_emit(alg, n, count, dt)
@@ -743,10 +749,16 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
         h.check(code, "replay on one thread and one host thread per rank")
         last["host_thread_per_rank"] = st
 
+    def run_threads_batched():
+        code, st = replay.run_on_threads_batched(threads)
+        h.check(code, "replay on one thread per rank inside one batch")
+        last["thread_per_rank_batched"] = st
+
     out = {"what": "the schedule's op list (HcommGfxScheduleEmit) issued call by call through the reference's primitives "
                    "by hcomm_amd/csrc/hg_caller.c, which binds the library with dlsym",
            "plan_ms_per_step": round(plan_res["ms_per_step"], 5)}
-    for mode, run in (("batched", run_batched), ("thread_per_rank", run_threads), ("host_thread_per_rank", run_host_threads)):
+    for mode, run in (("batched", run_batched), ("thread_per_rank", run_threads), ("host_thread_per_rank", run_host_threads),
+                      ("thread_per_rank_batched", run_threads_batched)):
         for _ in range(args.warmup):
             restore()
             run()
@@ -791,6 +803,9 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
                 row["host_threads"] = len(threads)
                 row["host_us_in_notifies"] = round(notify_us / args.steps / len(threads), 2)  # per host thread
                 row["host_us_slowest_thread"] = round(st.host_us_end_max, 2)
+            if mode == "thread_per_rank_batched":
+                row["batches"] = 1
+                row["host_us_in_end"] = round(end_us / args.steps, 2)
         out[mode] = row
         h.HcommGfxLaunchLogClear(thread)
 
@@ -801,7 +816,8 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
         if others:
             h.HcommThreadFree(others)
 
-    return out, {"batched": run_batched, "thread_per_rank": run_threads, "host_thread_per_rank": run_host_threads}, done
+    return out, {"batched": run_batched, "thread_per_rank": run_threads, "host_thread_per_rank": run_host_threads,
+                 "thread_per_rank_batched": run_threads_batched}, done
 
 
 def shape_sweep(args, torch, h, dev, stream, thread):

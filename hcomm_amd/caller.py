@@ -30,6 +30,8 @@ _lib.hg_caller_replay_threads.argtypes = [C.POINTER(C.c_uint64), C.c_uint32, C.P
                                           C.POINTER(_vpp), C.c_int, C.c_int, C.c_uint32, C.POINTER(CallerStats)]
 _lib.hg_caller_replay_host_threads.restype = C.c_int32
 _lib.hg_caller_replay_host_threads.argtypes = _lib.hg_caller_replay_threads.argtypes
+_lib.hg_caller_replay_threads_batched.restype = C.c_int32
+_lib.hg_caller_replay_threads_batched.argtypes = _lib.hg_caller_replay_threads.argtypes
 _lib.hg_caller_pool_shutdown.restype = None
 if _lib.hg_caller_bind(api.LIB_PATH.encode()) != 0:
     raise ImportError("libhcomm_caller.so could not bind the primitives of %s" % api.LIB_PATH)
@@ -74,6 +76,15 @@ class Replay:
         st = CallerStats()
         code = _lib.hg_caller_replay_threads(arr, len(threads), self._ops, self.n, self._bufs, self.dtype, self.op,
                                              timeout, C.byref(st))
+        return code, st
+
+    def run_on_threads_batched(self, threads, timeout=10):
+        """The calls of run_on_threads between one HcommBatchModeStart / End pair: the collective as one batch over all
+        its threads.  host_us_end of the returned stats is the time inside HcommBatchModeEnd."""
+        arr = (C.c_uint64 * len(threads))(*threads)
+        st = CallerStats()
+        code = _lib.hg_caller_replay_threads_batched(arr, len(threads), self._ops, self.n, self._bufs, self.dtype,
+                                                     self.op, timeout, C.byref(st))
         return code, st
 
     def run_on_host_threads(self, threads, timeout=10):

@@ -185,12 +185,16 @@ static void thread_delete(HgThread* t)
     for (uint32_t i = 0; i < g_ctx.ntouched; ++i)
         if (g_ctx.touched[i] == t) g_ctx.touched[i] = NULL;
     if (!t->recorder) {
-        for (uint32_t i = 0; i < t->notify_num; ++i)
-            if (t->notifies[i]) hg_rt_event_destroy(t->notifies[i]);
+        /* threads that a batch put behind this one's stream and that have not been used since find it gone: what
+         * they were to wait for is finished before it goes */
+        if (t->led_batch && t->stream && !t->owns_stream) hg_rt_stream_sync(t->stream);
         if (t->owns_stream && t->stream) {
             hg_rt_stream_sync(t->stream);
             hg_rt_stream_destroy(t->stream);
         }
+        for (uint32_t i = 0; i < t->notify_num; ++i)
+            if (t->notifies[i]) hg_rt_event_destroy(t->notifies[i]);
+        if (t->join_ev) hg_rt_event_destroy(t->join_ev);
     }
     free(t->notifies);
     free(t->notify_pending);
@@ -277,6 +281,8 @@ int32_t HcommGfxThreadSynchronize(ThreadHandle thread)
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     if (t->recorder) return HCCL_SUCCESS;
+    const int rc = hg_thread_settle(t);
+    if (rc != HCCL_SUCCESS) return rc;
     return hg_rt_stream_sync(t->stream);
 }
 
@@ -306,10 +312,33 @@ static void log_launch(HgThread* t, const HgLaunch* l)
 
 void hg_log_only(HgThread* t, const HgLaunch* l) { log_launch(t, l); }
 
+/*
+ * A batch that ordered its threads by notifies ran on the stream of its first thread.  Its other threads are put
+ * behind the end of that batch only when they are next given something or synchronised - a wait on every one of
+ * their streams at the end of each batch delayed the batch's own launches by a tenth of its run time - and this is
+ * that moment.  The first thread's event is recorded anew by every such batch it leads: waiting for a later
+ * record than the one meant waits longer, never shorter.  A first thread that is gone by now was synchronised when
+ * it was freed.
+ */
+int hg_thread_settle(HgThread* t)
+{
+    HgThread* lead = t->after;
+    if (!lead) return HCCL_SUCCESS;
+    t->after = NULL;
+    lead = hg_thread_from_handle((ThreadHandle)(uintptr_t)lead);
+    if (!lead || lead == t || t->recorder || lead->recorder || !lead->join_ev) return HCCL_SUCCESS;
+    return hg_rt_stream_wait_event(t->stream, lead->join_ev);
+}
+
 int hg_submit(HgThread* t, const HgLaunch* l)
 {
     log_launch(t, l);
     if (t->recorder) return HCCL_SUCCESS;
+    if (t->after) {
+        const int rc = hg_thread_settle(t);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
+    t->own_work = 1;
     switch (l->kind) {
         case HCOMM_GFX_KERNEL_COPY:
             return hg_launch_copy(t->stream, &l->tab.seg2, l->blocks, (int)l->streaming, l->lds_bytes);
@@ -545,18 +574,185 @@ int32_t HcommBatchModeStart(const char* batchTag)
     return HCCL_SUCCESS;
 }
 
+/*
+ * A batch whose threads order one another by notifies - the reference submits such a batch as one task graph over all
+ * its threads (CommTaskLaunch(threads, threadNum), launch_context.cc:16-44) - is resolved on the host into one list.
+ * Every thread's queue is walked up to its next copy or reduce: records on the way are noted, a wait passes when a
+ * record for its slot has been noted (or was issued before the batch), otherwise the thread sits there.  Of the
+ * copies and reduces now at the head of their threads - none of them ordered after another by any record - those
+ * that can share a launch with the head of the thread that has had the fewest so far are appended to the list, their
+ * threads move on, and so forth.  In a schedule whose ranks post to and wait for one another between steps, one
+ * such round is one step.  The list respects every thread's own order and every record -> wait edge, and the
+ * coalescer keeps apart whatever touches the same memory; it is issued on the stream of the first thread of the
+ * batch, the other threads' streams are ordered after it, and it after them where they had work of their own.  All
+ * ranks of a step thus share one launch although each was given to a thread of its own.
+ * When no thread can move and calls are left, a wait is there that nothing in the batch and no earlier record
+ * satisfies, and this host thread can never satisfy it: HCCL_E_TIMEOUT, and nothing of the batch is submitted.
+ * Records that no wait of the batch consumes stay pending for a later wait, marking the end of the batch.
+ */
+typedef struct {
+    HgThread* t;
+    uint32_t idx;
+} HgSlot;
+
+static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
+{
+    int32_t ret = HCCL_SUCCESS;
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < nt; ++i) {
+        th[i]->batch_cursor = 0;
+        total += th[i]->pending_n;
+    }
+    const uint64_t cap = total ? total : 1;
+    HgOp* sorted = (HgOp*)malloc(cap * sizeof(HgOp));
+    HgSlot* outside = (HgSlot*)malloc(cap * sizeof(HgSlot)); /* records to threads outside the batch */
+    HgSlot* earlier = (HgSlot*)malloc(cap * sizeof(HgSlot)); /* records issued before the batch that its waits consume */
+    uint32_t** count = (uint32_t**)calloc(nt, sizeof(uint32_t*)); /* per thread and slot: unconsumed records of the batch */
+    uint32_t had[HG_TOUCHED_MAX];                                 /* copies and reduces taken from each thread so far */
+    HgThread* main_t = th[0];
+    uint64_t n = 0, nearlier = 0, noutside = 0, done = 0;
+    if (!sorted || !outside || !earlier || !count) ret = HCCL_E_MEMORY;
+    for (uint32_t i = 0; i < nt && ret == HCCL_SUCCESS; ++i) {
+        had[i] = 0;
+        count[i] = (uint32_t*)calloc(th[i]->notify_num ? th[i]->notify_num : 1, sizeof(uint32_t));
+        if (!count[i]) ret = HCCL_E_MEMORY;
+    }
+    while (ret == HCCL_SUCCESS && done < total) {
+        /* every thread up to its next copy or reduce, until no record makes another wait pass */
+        uint64_t moved;
+        do {
+            moved = 0;
+            for (uint32_t i = 0; i < nt; ++i) {
+                HgThread* t = th[i];
+                while (t->batch_cursor < t->pending_n && t->pending[t->batch_cursor].sync != 0) {
+                    const HgOp* o = &t->pending[t->batch_cursor];
+                    if (o->sync == HG_SYNC_RECORD) {
+                        HgThread* d = (HgThread*)o->dst;
+                        uint32_t j = 0;
+                        while (j < nt && th[j] != d) ++j;
+                        if (j < nt) ++count[j][o->idx];
+                        else outside[noutside++] = (HgSlot){d, o->idx};
+                    } else if (count[i][o->idx] > 0) {
+                        --count[i][o->idx];
+                    } else {
+                        /* a record issued before the batch began */
+                        uint64_t pending = __atomic_load_n(&t->notify_pending[o->idx], __ATOMIC_ACQUIRE);
+                        int took = 0;
+                        while (pending != 0 && !took)
+                            took = __atomic_compare_exchange_n(&t->notify_pending[o->idx], &pending, pending - 1, 0,
+                                                               __ATOMIC_ACQ_REL, __ATOMIC_ACQUIRE);
+                        if (!took) break; /* its record is further down another thread's queue, or nowhere */
+                        earlier[nearlier++] = (HgSlot){t, o->idx};
+                    }
+                    ++t->batch_cursor;
+                    ++moved;
+                }
+            }
+            done += moved;
+        } while (moved != 0);
+        /* the thread that is furthest behind names the launch of this round */
+        uint32_t lead = nt;
+        for (uint32_t i = 0; i < nt; ++i) {
+            const HgThread* t = th[i];
+            if (t->batch_cursor < t->pending_n && t->pending[t->batch_cursor].sync == 0 && (lead == nt || had[i] < had[lead])) lead = i;
+        }
+        if (lead == nt) {
+            if (done < total) ret = HCCL_E_TIMEOUT; /* every thread with calls left sits at a wait */
+            break;
+        }
+        const uint32_t key = hg_op_launch_key(&th[lead]->pending[th[lead]->batch_cursor]);
+        for (uint32_t i = 0; i < nt; ++i) {
+            HgThread* t = th[i];
+            if (t->batch_cursor < t->pending_n && t->pending[t->batch_cursor].sync == 0 &&
+                hg_op_launch_key(&t->pending[t->batch_cursor]) == key) {
+                sorted[n++] = t->pending[t->batch_cursor++];
+                ++had[i];
+                ++done;
+            }
+        }
+    }
+    if (ret != HCCL_SUCCESS) {
+        /* nothing is submitted; the earlier records that waits of this batch took are handed back */
+        for (uint64_t k = 0; k < nearlier; ++k)
+            __atomic_add_fetch(&earlier[k].t->notify_pending[earlier[k].idx], 1, __ATOMIC_RELEASE);
+    } else {
+        if (!main_t->recorder) {
+            /* the batch's stream after what the other threads had queued on their own, and after the earlier records */
+            ret = hg_thread_settle(main_t);
+            for (uint32_t i = 1; i < nt && ret == HCCL_SUCCESS; ++i) {
+                HgThread* t = th[i];
+                if (t->recorder) continue;
+                if (t->after != main_t) ret = hg_thread_settle(t); /* behind another batch's first thread: its own stream says so */
+                if (ret != HCCL_SUCCESS || !(t->own_work || !t->owns_stream)) continue;
+                if (!t->join_ev) ret = hg_rt_event_create(&t->join_ev);
+                if (ret == HCCL_SUCCESS) ret = hg_rt_event_record(t->join_ev, t->stream);
+                if (ret == HCCL_SUCCESS) ret = hg_rt_stream_wait_event(main_t->stream, t->join_ev);
+                t->own_work = 0;
+            }
+            for (uint64_t k = 0; k < nearlier && ret == HCCL_SUCCESS; ++k)
+                if (!earlier[k].t->recorder) ret = hg_rt_stream_wait_event(main_t->stream, earlier[k].t->notifies[earlier[k].idx]);
+        }
+        if (ret == HCCL_SUCCESS) ret = hg_coalesce(sorted, n, emit_to_thread, main_t);
+        /* what the batch leaves behind: records nobody in it waited for, and the other threads behind its end */
+        for (uint32_t i = 0; i < nt && ret == HCCL_SUCCESS; ++i)
+            for (uint32_t k = 0; k < th[i]->notify_num && ret == HCCL_SUCCESS; ++k)
+                for (; count[i][k] > 0 && ret == HCCL_SUCCESS; --count[i][k]) {
+                    if (!(main_t->recorder || th[i]->recorder)) ret = hg_rt_event_record(th[i]->notifies[k], main_t->stream);
+                    __atomic_add_fetch(&th[i]->notify_pending[k], 1, __ATOMIC_RELEASE);
+                }
+        for (uint64_t k = 0; k < noutside && ret == HCCL_SUCCESS; ++k) {
+            if (!hg_thread_from_handle((ThreadHandle)(uintptr_t)outside[k].t)) continue; /* freed since the call was recorded */
+            if (!(main_t->recorder || outside[k].t->recorder)) ret = hg_rt_event_record(outside[k].t->notifies[outside[k].idx], main_t->stream);
+            __atomic_add_fetch(&outside[k].t->notify_pending[outside[k].idx], 1, __ATOMIC_RELEASE);
+        }
+        if (!main_t->recorder && nt > 1 && ret == HCCL_SUCCESS) {
+            /* the other threads' own streams go behind the end of the batch when they are next used (hg_thread_settle) */
+            if (!main_t->join_ev) ret = hg_rt_event_create(&main_t->join_ev);
+            if (ret == HCCL_SUCCESS) ret = hg_rt_event_record(main_t->join_ev, main_t->stream);
+            main_t->led_batch = 1;
+            for (uint32_t i = 1; i < nt && ret == HCCL_SUCCESS; ++i) {
+                if (th[i]->recorder) continue;
+                /* a stream of the caller's may be given work the library never sees: it goes behind the batch now */
+                if (th[i]->owns_stream) th[i]->after = main_t;
+                else ret = hg_rt_stream_wait_event(th[i]->stream, main_t->join_ev);
+            }
+        }
+    }
+    for (uint32_t i = 0; i < nt; ++i) {
+        if (count) free(count[i]);
+    }
+    free(count);
+    free(outside);
+    free(earlier);
+    free(sorted);
+    return ret;
+}
+
 int32_t HcommBatchModeEnd(const char* batchTag)
 {
     (void)batchTag;
     if (!g_ctx.batching) return HCCL_E_PARA;
     g_ctx.batching = 0;
     int32_t ret = HCCL_SUCCESS;
+    /* the threads of the batch that are still alive, and whether any of them recorded a notify call */
+    HgThread* th[HG_TOUCHED_MAX];
+    uint32_t nt = 0;
+    int ordered = 0;
     for (uint32_t i = 0; i < g_ctx.ntouched; ++i) {
         HgThread* t = g_ctx.touched[i];
         if (!t) continue; /* freed inside the batch */
-        if (ret == HCCL_SUCCESS) ret = hg_coalesce(t->pending, t->pending_n, emit_to_thread, t);
-        t->pending_n = 0;
-        __atomic_store_n(&t->batch_owner, NULL, __ATOMIC_RELEASE);
+        th[nt++] = t;
+        for (uint32_t k = 0; k < t->pending_n && !ordered; ++k) ordered = t->pending[k].sync != 0;
+    }
+    if (ordered) {
+        ret = batch_end_ordered(th, nt);
+    } else {
+        for (uint32_t i = 0; i < nt; ++i)
+            if (ret == HCCL_SUCCESS) ret = hg_coalesce(th[i]->pending, th[i]->pending_n, emit_to_thread, th[i]);
+    }
+    for (uint32_t i = 0; i < nt; ++i) {
+        th[i]->pending_n = 0;
+        __atomic_store_n(&th[i]->batch_owner, NULL, __ATOMIC_RELEASE);
     }
     g_ctx.ntouched = 0;
     return ret;
@@ -631,9 +827,18 @@ int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThr
     HgThread* d = hg_thread_from_handle(dstThread);
     if (!d) return HCCL_E_PTR;
     if (dstNotifyIdx >= d->notify_num) return HCCL_E_PARA;
-    if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    if (g_ctx.batching) { /* a step of the thread's sequence like any other: resolved by HcommBatchModeEnd */
+        HgOp o;
+        memset(&o, 0, sizeof(o));
+        o.sync = HG_SYNC_RECORD;
+        o.idx = dstNotifyIdx;
+        o.dst = d;
+        return record_or_run(t, &o);
+    }
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     if (!(t->recorder || d->recorder)) {
-        const int rc = hg_rt_event_record(d->notifies[dstNotifyIdx], t->stream);
+        int rc = hg_thread_settle(t);
+        if (rc == HCCL_SUCCESS) rc = hg_rt_event_record(d->notifies[dstNotifyIdx], t->stream);
         if (rc != HCCL_SUCCESS) return rc;
     }
     __atomic_add_fetch(&d->notify_pending[dstNotifyIdx], 1, __ATOMIC_RELEASE);
@@ -659,7 +864,14 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     if (notifyIdx >= t->notify_num) return HCCL_E_PARA;
-    if (g_ctx.batching) return HCCL_E_NOT_SUPPORT;
+    if (g_ctx.batching) {
+        HgOp o;
+        memset(&o, 0, sizeof(o));
+        o.sync = HG_SYNC_WAIT;
+        o.idx = notifyIdx;
+        return record_or_run(t, &o);
+    }
+    if (hg_thread_free_for_caller(t) != HCCL_SUCCESS) return HCCL_E_UNAVAIL;
     /* A wait on a stream can only follow a record that has been issued.  The reference queues the wait and lets the
      * device sit until the record arrives or timeOut runs out (include/hcomm_primitives.h:181-191); here the wait
      * sits on the HOST until another host thread has issued the record - for at most min(timeOut seconds, the bound
@@ -675,6 +887,7 @@ int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, u
             if (__atomic_compare_exchange_n(&t->notify_pending[notifyIdx], &pending, pending - 1, 0, __ATOMIC_ACQ_REL,
                                             __ATOMIC_ACQUIRE)) {
                 if (t->recorder) return HCCL_SUCCESS;
+                t->own_work = 1;
                 return hg_rt_stream_wait_event(t->stream, t->notifies[notifyIdx]);
             }
         }

@@ -384,6 +384,12 @@ static uint32_t kind_of(const HgOp* o)
     return o->is_reduce ? HCOMM_GFX_KERNEL_REDUCE2 : HCOMM_GFX_KERNEL_COPY;
 }
 
+/* Operations with different keys never share a launch. */
+uint32_t hg_op_launch_key(const HgOp* o)
+{
+    return kind_of(o) << 16 | (o->is_reduce ? (uint32_t)o->dtype << 8 | o->op : 0xffffu);
+}
+
 static int conflicts(const HgLaunch* l, const HgOp* o)
 {
     const HgSeg2Table* t = &l->tab.seg2;

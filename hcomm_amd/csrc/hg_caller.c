@@ -153,11 +153,41 @@ static int32_t post_and_wait(const ThreadHandle* threads, uint32_t from, uint32_
  * Work timed on threads[0]'s stream brackets everything: the other threads wait for it first and it waits for them
  * last.
  */
+static int32_t replay_threads(const ThreadHandle* threads, uint32_t nRanks, const HcommGfxSchedOp* ops, uint64_t n,
+                              void* const* const* bufs, int dtype, int op, uint32_t timeout, HgCallerStats* st);
+
 int32_t hg_caller_replay_threads(const ThreadHandle* threads, uint32_t nRanks, const HcommGfxSchedOp* ops, uint64_t n,
                                  void* const* const* bufs, int dtype, int op, uint32_t timeout, HgCallerStats* st)
 {
     if (!g.lib || !threads || !ops || !bufs || !st) return HCCL_E_PTR;
     if (nRanks == 0 || nRanks > CALLER_MAX_RANKS) return HCCL_E_PARA;
+    return replay_threads(threads, nRanks, ops, n, bufs, dtype, op, timeout, st);
+}
+
+/*
+ * The same calls between ONE HcommBatchModeStart / End pair: the whole collective - every rank's operations on its
+ * own thread, every post and wait - is handed over as one batch, the way the reference hands a task graph over all
+ * its threads to CommTaskLaunch at the end of a batch (launch_context.cc:16-44).
+ */
+int32_t hg_caller_replay_threads_batched(const ThreadHandle* threads, uint32_t nRanks, const HcommGfxSchedOp* ops, uint64_t n,
+                                         void* const* const* bufs, int dtype, int op, uint32_t timeout, HgCallerStats* st)
+{
+    if (!g.lib || !threads || !ops || !bufs || !st) return HCCL_E_PTR;
+    if (nRanks == 0 || nRanks > CALLER_MAX_RANKS) return HCCL_E_PARA;
+    const double t0 = now_us();
+    int32_t rc = g.start("collective");
+    if (rc != HCCL_SUCCESS) return rc;
+    rc = replay_threads(threads, nRanks, ops, n, bufs, dtype, op, timeout, st);
+    const double e0 = now_us();
+    const int32_t rc_end = g.end("collective");
+    st->host_us_end = st->host_us_end_max = now_us() - e0;
+    st->host_us = now_us() - t0;
+    return rc != HCCL_SUCCESS ? rc : rc_end;
+}
+
+static int32_t replay_threads(const ThreadHandle* threads, uint32_t nRanks, const HcommGfxSchedOp* ops, uint64_t n,
+                              void* const* const* bufs, int dtype, int op, uint32_t timeout, HgCallerStats* st)
+{
     memset(st, 0, sizeof(*st));
     const uint32_t unit = unit_of(dtype);
     /* in units of "steps issued so far" (1-based); 0 = never */

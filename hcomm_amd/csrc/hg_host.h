@@ -14,6 +14,9 @@ typedef struct {
     uint8_t is_reduce;
     uint8_t dtype; /* HcommDataType (255 for copies) */
     uint8_t op;    /* HcommReduceOp (255 for copies) */
+    uint8_t sync;  /* only in a thread's batch queue: 0 = a copy / reduce, HG_SYNC_RECORD (dst = the HgThread notified),
+                      HG_SYNC_WAIT; never reaches the coalescer */
+    uint32_t idx;  /* notify slot of a record / wait */
     void* dst;
     const void* src;
     uint64_t bytes;
@@ -37,6 +40,9 @@ typedef struct {
     } tab;
 } HgLaunch;
 
+#define HG_SYNC_RECORD 1u
+#define HG_SYNC_WAIT 2u
+
 typedef struct HgThread {
     uint32_t magic;
     int recorder;     /* 1: log launches, never touch the GPU */
@@ -56,9 +62,18 @@ typedef struct HgThread {
     const void* batch_owner;
     int log_enabled;
     int log_fixed; /* set while a call that must not allocate runs: the log takes what fits and drops the rest */
+    /* batches that order several threads by notifies run on one of them: */
+    void* join_ev;      /* hipEvent_t (created on first use) by which this thread's stream and another's are ordered */
+    int own_work;       /* something was submitted on this thread's own stream since it was last joined to another */
+    int led_batch;      /* other threads may still be waiting to be put behind join_ev on this thread's stream */
+    struct HgThread* after; /* first thread of the batch this thread's stream is still to be put behind (hg_thread_settle) */
+    uint32_t batch_cursor; /* next entry of `pending` while HcommBatchModeEnd walks the threads of a batch */
 } HgThread;
 
 HgThread* hg_thread_from_handle(ThreadHandle h);
+/* Puts the thread's stream behind the batch it last took part in on another thread's stream, if that is still due: to be
+ * called before anything is queued on, recorded on or waited for on the thread's stream outside hg_submit. */
+int hg_thread_settle(HgThread* t);
 /* HCCL_SUCCESS, or HCCL_E_UNAVAIL while a batch of ANOTHER host thread holds recorded operations of the thread */
 int hg_thread_free_for_caller(const HgThread* t);
 /* whether the calling host thread is between HcommBatchModeStart and HcommBatchModeEnd */
@@ -70,7 +85,8 @@ typedef int (*HgEmitFn)(const HgLaunch* launch, void* ctx);
 int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
 /* the same with the launch under construction in storage of the caller's (no allocation) */
 int hg_coalesce_with(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx, HgLaunch* work);
-uint64_t hg_split_head(const HgOp* o); /* bytes before the 16-byte boundary both operands reach together, or 0 */
+uint64_t hg_split_head(const HgOp* o);      /* bytes before the 16-byte boundary both operands reach together, or 0 */
+uint32_t hg_op_launch_key(const HgOp* o);   /* operations with different keys never share a launch */
 
 /* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment
  * pointers and sizes are set. */

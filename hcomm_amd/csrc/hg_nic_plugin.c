@@ -210,7 +210,8 @@ static int32_t ch_notify_record(void* ctx, ThreadHandle thread, uint32_t idx)
             const int rc = hg_rt_event_create(&c->notifies[idx]);
             if (rc != HCCL_SUCCESS) return rc;
         }
-        const int rc = hg_rt_event_record(c->notifies[idx], t->stream);
+        int rc = hg_thread_settle(t);
+        if (rc == HCCL_SUCCESS) rc = hg_rt_event_record(c->notifies[idx], t->stream);
         if (rc != HCCL_SUCCESS) return rc;
     }
     __atomic_add_fetch(&c->notify_pending[idx], 1, __ATOMIC_RELEASE);

@@ -1505,6 +1505,10 @@ int32_t HcommGfxPlanRun(const HcommGfxPlan* plan, ThreadHandle thread)
     HgThread* t = hg_thread_from_handle(thread);
     if (!t) return HCCL_E_PTR;
     HcommGfxPlan* p = (HcommGfxPlan*)plan; /* the graph is a cache, not part of the plan's meaning */
+    if (!t->recorder) { /* before anything is captured on or launched into the stream */
+        const int rc = hg_thread_settle(t);
+        if (rc != HCCL_SUCCESS) return rc;
+    }
     if (t->recorder || p->nlaunch < 2 || !p->graph_wanted || p->graph_state < 0 || hg_rt_stream_is_capturing(t->stream))
         return HcommGfxPlanRunRange(plan, thread, 0, plan->nlaunch);
     if (p->graph_state == 1 && p->graph_stream != t->stream) {

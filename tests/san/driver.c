@@ -53,6 +53,72 @@ static int32_t e_ophrs(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) {
 static int32_t e_op(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
 static int32_t e_opar(void* c, HcommGfxSchedOp* o, uint64_t cap, uint64_t* n) { Ctx* x = c; return HcommGfxOrderPreservedAllReduceEmit(x->n, x->count, x->ccl, x->dt, o, cap, n); }
 
+/* Batches whose threads order one another by notifies: rank r's operations on thread r with every thread posting to
+ * and waiting for every other between the steps, all inside one HcommBatchModeStart / End pair; the same with a wait
+ * too many (nothing can satisfy it: HCCL_E_TIMEOUT), with a thread freed in the middle of the batch (likewise: its
+ * records went with it), and with records to threads outside the batch, one of them freed before End. */
+static void ordered_batches(void)
+{
+    enum { N = 6 };
+    ThreadHandle t[N], out[2];
+    for (int r = 0; r < N; ++r) bad += HcommGfxRecorderThreadAlloc(&t[r]) != 0;
+    for (int r = 0; r < 2; ++r) bad += HcommGfxRecorderThreadAlloc(&out[r]) != 0;
+    for (int variant = 0; variant < 4; ++variant)
+        for (int alg = 0; alg <= 17; ++alg) {
+            uint64_t n = 0;
+            if (HcommGfxScheduleEmit(alg, N, 4099, HCOMM_DATA_TYPE_FP32, NULL, 0, &n)) continue;
+            HcommGfxSchedOp* ops = (HcommGfxSchedOp*)malloc((n ? n : 1) * sizeof(*ops));
+            bad += HcommGfxScheduleEmit(alg, N, 4099, HCOMM_DATA_TYPE_FP32, ops, n, &n) != 0;
+            bad += HcommBatchModeStart("ordered") != 0;
+            int freed = 0;
+            for (uint64_t i = 0; i < n;) {
+                uint64_t j = i;
+                while (j < n && ops[j].step == ops[i].step) ++j;
+                for (int r = 0; r < N; ++r)
+                    for (int q = 0; q < N; ++q)
+                        if (q != r && !(freed && (q == N - 1 || r == N - 1))) bad += HcommThreadNotifyRecordOnThread(t[r], t[q], (uint32_t)r) != 0;
+                for (int r = 0; r < N; ++r)
+                    for (int q = 0; q < N; ++q)
+                        if (q != r && !(freed && (q == N - 1 || r == N - 1))) bad += HcommThreadNotifyWaitOnThread(t[r], (uint32_t)q, 10) != 0;
+                for (uint64_t k = i; k < j; ++k) {
+                    if (freed && ops[k].rank == N - 1) continue;
+                    char* d = (char*)bufs[ops[k].dstBuf][ops[k].rank] + ops[k].dstOff;
+                    char* sp = (char*)bufs[ops[k].srcBuf][ops[k].srcRank] + ops[k].srcOff;
+                    bad += (ops[k].kind ? HcommLocalReduceOnThread(t[ops[k].rank], d, sp, ops[k].bytes / 4, HCOMM_DATA_TYPE_FP32, HCOMM_REDUCE_SUM)
+                                        : HcommLocalCopyOnThread(t[ops[k].rank], d, sp, ops[k].bytes)) != 0;
+                }
+                if (variant == 2 && !freed && j < n) { /* a thread of the batch goes away with records still addressed to it */
+                    bad += HcommThreadFree(&t[N - 1], 1) != 0;
+                    freed = 1;
+                }
+                i = j;
+            }
+            if (variant == 1) bad += HcommThreadNotifyWaitOnThread(t[2], 0, 10) != 0; /* one wait too many */
+            if (variant == 3) {
+                bad += HcommThreadNotifyRecordOnThread(t[0], out[0], 3) != 0;
+                bad += HcommThreadNotifyRecordOnThread(t[1], out[1], 4) != 0;
+                bad += HcommThreadFree(&out[1], 1) != 0;
+            }
+            const int32_t rc = HcommBatchModeEnd("ordered");
+            /* a freed thread takes its queued calls with it, records included: the peers' waits for them can never pass */
+            bad += rc != (variant == 1 || freed ? HCCL_E_TIMEOUT : HCCL_SUCCESS);
+            if (variant == 3) {
+                bad += HcommThreadNotifyWaitOnThread(out[0], 3, 0) != 0;
+                bad += HcommGfxRecorderThreadAlloc(&out[1]) != 0;
+            }
+            if (freed) bad += HcommGfxRecorderThreadAlloc(&t[N - 1]) != 0;
+            /* whatever the batch left pending is drained, so that the next one starts clean */
+            for (int r = 0; r < N; ++r)
+                for (uint32_t q = 0; q < N; ++q)
+                    while (HcommThreadNotifyWaitOnThread(t[r], q, 0) == 0) {}
+            for (int r = 0; r < N; ++r) HcommGfxLaunchLogClear(t[r]);
+            free(ops);
+            ++checks;
+        }
+    bad += HcommThreadFree(t, N) != 0;
+    bad += HcommThreadFree(out, 2) != 0;
+}
+
 int main(void)
 {
     for (int k = 0; k < 5; ++k)
@@ -242,6 +308,7 @@ int main(void)
                     run_plan(th, p);
                 }
     }
+    ordered_batches();
     HcommGfxSlice slc[32];
     for (uint32_t n = 0; n <= 32; ++n) HcommGfxCalcSlices(100003, 2, n, slc);
     HcommThreadFree(&th, 1);

@@ -6,7 +6,10 @@ and the thread notifies):
   per rank    rank r's calls on thread r, eagerly, each thread posting to and waiting for the peers it exchanges data
               with between the steps (reduce_scatter_ring.cc:211-217,254-272) - issued by one host thread for all
               ranks, or by a host thread per rank (the ranks of the reference are processes of their own), where a wait
-              may reach the library before its record and sits on the host until the record has been issued.
+              may reach the library before its record and sits on the host until the record has been issued;
+  one batch   the per-rank calls, posts and waits included, between ONE Start / End pair: the collective as one batch
+              over all its threads (launch_context.cc:16-44), which HcommBatchModeEnd turns into the launches of the
+              step-wise plan.
 Every one of the 2N rank buffers (and the communication buffers, where a schedule has them) is compared bit for bit
 with the CPU oracle's replay."""
 import numpy as np
@@ -77,7 +80,9 @@ def drive(mode, thread, threads, alg, n, count, dtype, op, special=False):
         # a step whose operations are of one kind and on 16-byte boundaries is one launch
         assert st.batches == replay.steps and len(h.launch_log(thread)) >= (replay.steps if count else 0)
     else:
-        code, st = (replay.run_on_threads if mode == "threads" else replay.run_on_host_threads)(threads[:n])
+        run = {"threads": replay.run_on_threads, "host_threads": replay.run_on_host_threads,
+               "threads_batched": replay.run_on_threads_batched}[mode]
+        code, st = run(threads[:n])
         if prod and n > 1 and count:
             assert code == h.HcclResult.E_PARA
             for t in threads[:n]:
@@ -131,6 +136,28 @@ def test_schedule_on_one_host_thread_per_rank_matches_oracle(rank_threads, alg, 
             caller.pool_shutdown()
 
 
+@pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
+def test_schedule_as_one_batch_over_a_thread_per_rank_matches_oracle(rank_threads, alg, n, count, dtype, op):
+    say("via primitives, one batch over a thread per rank", alg, n, count, dtype, op)
+    for t in rank_threads[:n]:
+        h.HcommGfxThreadSynchronize(t)
+        h.HcommGfxLaunchLogClear(t)
+    st = drive("threads_batched", None, rank_threads, alg, n, count, dtype, op)
+    if st is None:
+        return
+    # everything was issued on the first thread of the batch, and in no more launches than one Start / End per step gives
+    assert all(not h.launch_log(t) for t in rank_threads[1:n])
+    thread = rank_threads[0]
+    issued = len(h.launch_log(thread))
+    h.HcommGfxLaunchLogClear(thread)
+    drive("batched", thread, None, alg, n, count, dtype, op)
+    assert issued <= len(h.launch_log(thread))
+    if n > 1 and count:   # every record met its wait
+        for t in rank_threads[:n]:
+            for q in range(n):
+                assert h.HcommThreadNotifyWaitOnThread(t, q, 0) == h.HcclResult.E_TIMEOUT
+
+
 @pytest.mark.parametrize("alg,n,count", [("ring_ar", 8, 70001), ("rhd_ar", 6, 20011), ("mesh_oneshot", 5, 20011)])
 @pytest.mark.parametrize("dtype,op", [("fp32", "max"), ("bf16", "min"), ("fp16", "sum")])
 def test_special_values_via_primitives(gpu_thread, rank_threads, alg, n, count, dtype, op):
@@ -139,14 +166,66 @@ def test_special_values_via_primitives(gpu_thread, rank_threads, alg, n, count, 
     drive("batched", gpu_thread, None, alg, n, count, dtype, op, special=True)
     drive("threads", None, rank_threads, alg, n, count, dtype, op, special=True)
     drive("host_threads", None, rank_threads, alg, n, count, dtype, op, special=True)
+    drive("threads_batched", None, rank_threads, alg, n, count, dtype, op, special=True)
 
 
 def test_repeated_replays_on_threads_leave_no_record_behind(rank_threads):
     """Twenty ring allreduces in a row on eight threads: every record is consumed by its wait, so nothing is left
     pending between collectives and the result is the same every time."""
     for it in range(20):
-        drive("threads" if it % 2 else "host_threads", None, rank_threads, "ring_ar", 8, 65539, "fp32", "sum")
+        drive(("threads", "host_threads", "threads_batched")[it % 3], None, rank_threads, "ring_ar", 8, 65539, "fp32", "sum")
     caller.pool_shutdown()
     for t in rank_threads[:8]:
         for q in range(8):
             assert h.HcommThreadNotifyWaitOnThread(t, q, 0) == h.HcclResult.E_TIMEOUT
+
+
+@pytest.mark.parametrize("follow", ["eager_call", "synchronize", "callers_stream"])
+def test_a_batch_with_notifies_is_ordered_with_eager_work_on_its_threads(rank_threads, follow):
+    """The launches of such a batch all go to the stream of its first thread.  What another of its threads was given
+    before the batch (eagerly, on its own stream) is finished before the batch reads it, and what it is given after
+    the batch starts after the batch's last launch: a chain src -> a (eager, thread 1) -> b (batch, thread 1, posts)
+    -> c (batch, thread 0, waits) -> d (after the batch, thread 1) carries src through - whether thread 1 is next
+    given a call of the library, is synchronised, or wraps a stream of the caller's that the caller itself queues
+    the last copy on."""
+    import torch
+    say("via primitives, batch with notifies between eager work", follow)
+    t0, t1 = rank_threads[:2]
+    s1 = None
+    if follow == "callers_stream":
+        s1 = torch.cuda.Stream()
+        code, t1 = h.HcommThreadAllocWithStream(s1.cuda_stream, 4)
+        assert code == 0
+    nbytes = 1 << 27
+    src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda")
+    a, b, c, d = (torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(4))
+    torch.cuda.synchronize()
+    try:
+        for it in range(3):
+            assert h.HcommLocalCopyOnThread(t1, a.data_ptr(), src.data_ptr(), nbytes) == 0
+            assert h.HcommBatchModeStart(b"chain") == 0
+            assert h.HcommThreadNotifyWaitOnThread(t0, 1, 10) == 0
+            assert h.HcommLocalCopyOnThread(t0, c.data_ptr(), b.data_ptr(), nbytes) == 0
+            assert h.HcommLocalCopyOnThread(t1, b.data_ptr(), a.data_ptr(), nbytes) == 0
+            assert h.HcommThreadNotifyRecordOnThread(t1, t0, 1) == 0
+            assert h.HcommBatchModeEnd(b"chain") == 0
+            if follow == "eager_call":
+                assert h.HcommLocalCopyOnThread(t1, d.data_ptr(), c.data_ptr(), nbytes) == 0
+                assert h.HcommGfxThreadSynchronize(t1) == 0
+            elif follow == "synchronize":
+                assert h.HcommGfxThreadSynchronize(t1) == 0      # thread 1's part of the batch is done when this returns
+                d.copy_(c)
+                torch.cuda.synchronize()
+            else:
+                with torch.cuda.stream(s1):
+                    d.copy_(c, non_blocking=True)
+                s1.synchronize()
+            assert torch.equal(d, src), "iteration %d" % it
+            assert h.HcommGfxThreadSynchronize(t0) == 0
+            src.add_(1)
+            for x in (a, b, c, d):
+                x.zero_()
+            torch.cuda.synchronize()
+    finally:
+        if s1 is not None:
+            h.HcommThreadFreeWithStream([t1])

@@ -144,9 +144,100 @@ def test_notify_wait_needs_a_record_issued_before_it(rec):
         for _ in range(3):
             assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 1) == R.SUCCESS
         assert h.HcommThreadNotifyWaitOnThreadWithDefaultTimeout(rec, 1) == R.E_TIMEOUT
-        assert h.HcommBatchModeStart(b"b") == R.SUCCESS                              # not inside a batch
-        assert h.HcommThreadNotifyRecordOnThread(other, rec, 0) == R.E_NOT_SUPPORT
-        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.E_NOT_SUPPORT
+    finally:
+        h.HcommThreadFree([other])
+
+
+def _fake(n, base):
+    return [base + r * (1 << 26) for r in range(n)]
+
+
+@pytest.mark.parametrize("alg,n,count,dt", [
+    (h.Alg.ALLREDUCE_RING, 8, 1 << 20, h.HcommDataType.BFP16),
+    (h.Alg.ALLREDUCE_RHD, 16, 1 << 18, h.HcommDataType.INT32),
+    (h.Alg.ALLREDUCE_RHD, 6, 100003, h.HcommDataType.FP32),
+    (h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 2048, h.HcommDataType.FP16),
+    (h.Alg.ALLREDUCE_NHR, 5, 70001, h.HcommDataType.BFP16),
+    (h.Alg.REDUCE_SCATTER_RING, 7, 1000003, h.HcommDataType.FP32),
+    (h.Alg.REDUCE_SCATTER_MESH, 7, 999, h.HcommDataType.INT32),
+])
+def test_one_batch_over_a_thread_per_rank_with_notifies_is_the_plans_launches(alg, n, count, dt):
+    """The reference hands a batch over ALL its threads, notifies included, to one task graph (launch_context.cc:16-44
+    CommTaskLaunch(threads, threadNum)).  Here HcommBatchModeEnd resolves the records and waits on the host: a
+    collective given as rank r's calls on thread r, posts and waits between the steps, all inside one Start / End
+    pair, comes out as the launches of the step-wise plan - every rank of a step in one launch - on the first
+    thread of the batch, and no record is left pending."""
+    from hcomm_amd import caller
+    recs = [h.HcommGfxRecorderThreadAlloc()[1] for _ in range(n)]
+    try:
+        i, o = _fake(n, 1 << 40), _fake(n, 1 << 41)
+        rp = caller.Replay(h.schedule_emit(alg, n, count, dt), {0: i, 1: o}, dt, 0)
+        code, st = rp.run_on_threads_batched(recs)
+        assert code == 0 and st.notifies >= 2 * (n - 1)
+        plan = h.Plan(alg, h.Lowering.STEPWISE, i, o, count, dt, 0)
+        key = lambda l: (l.kind, l.nseg, l.bytes, l.dtype, l.op)
+        assert [key(l) for l in h.launch_log(recs[0])] == [key(l) for l in plan.launches()]
+        assert all(not h.launch_log(t) for t in recs[1:])
+        for t in recs:
+            for q in range(n):
+                assert h.HcommThreadNotifyWaitOnThread(t, q, 0) == R.E_TIMEOUT
+    finally:
+        h.HcommThreadFree(recs)
+
+
+def test_notifies_inside_a_batch_are_resolved_at_its_end(rec):
+    """Records and waits between HcommBatchModeStart and End are steps of their threads' sequences: End orders the
+    copies and reduces by them.  A wait may come before its record in call order (another thread's record further
+    down); a wait nothing satisfies fails the whole batch with HCCL_E_TIMEOUT and submits nothing; a record no wait
+    of the batch consumes - and one issued before the batch - stay good for a wait outside it."""
+    code, other = h.HcommGfxRecorderThreadAlloc()
+    assert code == 0
+    A, B, C_ = 1 << 40, 1 << 41, 1 << 42
+    try:
+        # other: B <- A, then posts; rec: waits, then C <- B.  Called in the "wrong" order: rec first.
+        assert h.HcommBatchModeStart(b"b") == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 3, 10) == R.SUCCESS
+        assert h.HcommLocalCopyOnThread(rec, C_, B, 8192) == R.SUCCESS
+        assert h.HcommLocalCopyOnThread(other, B, A, 4096) == R.SUCCESS
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 3) == R.SUCCESS
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 4) == R.SUCCESS   # nobody in the batch waits for this one
+        assert h.HcommBatchModeEnd(b"b") == R.SUCCESS
+        log = h.launch_log(rec)                                                # the first thread of the batch issues all
+        # B<-A (4 KiB) before C<-B (8 KiB), and apart: C<-B reads what B<-A writes
+        assert [(l.kind, l.nseg, l.bytes) for l in log] == [(0, 1, 4096), (0, 1, 8192)]
+        assert not h.launch_log(other)
+        assert h.HcommThreadNotifyWaitOnThread(rec, 3, 0) == R.E_TIMEOUT       # consumed inside the batch
+        assert h.HcommThreadNotifyWaitOnThread(rec, 4, 0) == R.SUCCESS         # left over from the batch
+        # a record issued before the batch satisfies a wait inside it
+        h.HcommGfxLaunchLogClear(rec)
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 5) == R.SUCCESS
+        assert h.HcommBatchModeStart(b"b") == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 5, 10) == R.SUCCESS
+        assert h.HcommLocalCopyOnThread(rec, C_, B, 4096) == R.SUCCESS
+        assert h.HcommBatchModeEnd(b"b") == R.SUCCESS
+        assert len(h.launch_log(rec)) == 1
+        assert h.HcommThreadNotifyWaitOnThread(rec, 5, 0) == R.E_TIMEOUT
+        # two threads waiting for each other before either posts: nothing can run
+        h.HcommGfxLaunchLogClear(rec)
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 6) == R.SUCCESS   # an earlier record the failed batch takes ...
+        assert h.HcommBatchModeStart(b"b") == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 6, 10) == R.SUCCESS
+        assert h.HcommLocalCopyOnThread(rec, C_, B, 4096) == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 10) == R.SUCCESS
+        assert h.HcommThreadNotifyRecordOnThread(rec, other, 0) == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(other, 0, 10) == R.SUCCESS
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 0) == R.SUCCESS
+        assert h.HcommBatchModeEnd(b"b") == R.E_TIMEOUT
+        assert not h.launch_log(rec) and not h.launch_log(other)
+        assert h.HcommThreadNotifyWaitOnThread(rec, 6, 0) == R.SUCCESS         # ... and hands back
+        assert h.HcommThreadNotifyWaitOnThread(rec, 0, 0) == R.E_TIMEOUT
+        assert h.HcommThreadNotifyWaitOnThread(other, 0, 0) == R.E_TIMEOUT
+        # the threads are free again
+        assert h.HcommLocalCopyOnThread(other, B, A, 4096) == R.SUCCESS
+        # slot numbers are checked when the call is made
+        assert h.HcommBatchModeStart(b"b") == R.SUCCESS
+        assert h.HcommThreadNotifyWaitOnThread(rec, 32, 10) == R.E_PARA
+        assert h.HcommThreadNotifyRecordOnThread(other, rec, 32) == R.E_PARA
         assert h.HcommBatchModeEnd(b"b") == R.SUCCESS
     finally:
         h.HcommThreadFree([other])
