@@ -158,7 +158,8 @@ HcommResult HcommThreadFreeWithStream(const ThreadHandle* threads, uint32_t thre
  * thread issues one, for at most min(timeOut seconds, HCOMM_GFX_NOTIFY_HOST_WAIT_MS = 100 ms by default), then
  * queues nothing and returns HCCL_E_TIMEOUT - the reference's wait would sit on the device until timeOut ran out.
  * Callers that issue both from one host thread issue the Record first.  Every Record is consumed by one Wait.
- * Neither call is available inside batch mode (HCCL_E_NOT_SUPPORT).
+ * Between HcommBatchModeStart and HcommBatchModeEnd a Record or Wait is queued on its thread like the copies and
+ * reduces around it (slot numbers are still checked at once), and HcommBatchModeEnd resolves them: see there.
  */
 int32_t HcommThreadNotifyRecordOnThread(ThreadHandle thread, ThreadHandle dstThread, uint32_t dstNotifyIdx);
 int32_t HcommThreadNotifyWaitOnThread(ThreadHandle thread, uint32_t notifyIdx, uint32_t timeOut);
@@ -283,6 +284,20 @@ HcommResult HcommMemFree(void* ptr);
  * same kind / type / op into single kernel launches (one launch for all N ranks of a collective step).
  * Two operations are independent when neither writes memory the other reads or writes.
  * Start while already batching, or End without Start -> HCCL_E_PARA.  batchTag may be NULL.
+ *
+ * A BATCH WITH NOTIFIES.  The reference hands a batch to the device as one task graph over ALL the threads it touched,
+ * their notify tasks included (CommTaskLaunch(threads, threadNum), launch_context.cc:16-44).  Here, when any Record or
+ * Wait was queued, HcommBatchModeEnd works out on the host an order of all queued copies and reduces that respects
+ * each thread's own order and every Record -> Wait pair (a Wait may have been called before its Record; a Record
+ * issued BEFORE the batch satisfies a Wait inside it), and issues that one list through the coalescer on the stream
+ * of the FIRST thread the batch touched: operations that different threads perform in the same step of a schedule
+ * share a launch, exactly as if one thread had been given the step between a Start / End pair of its own.  The other
+ * threads' streams are placed behind the end of the batch when they are next given a call or synchronised (a stream
+ * of the caller's, HcommThreadAllocWithStream: at once), and the batch behind whatever they were given before it.
+ * A Wait that neither the batch nor an earlier Record satisfies can never be satisfied - the host thread that would
+ * issue the Record is the one inside HcommBatchModeEnd - so End returns HCCL_E_TIMEOUT at once and submits NOTHING of
+ * the batch; Records the batch took from before it are handed back.  Records that no Wait of the batch consumes
+ * remain for a later Wait, as of the end of the batch.
  */
 int32_t HcommBatchModeStart(const char* batchTag);
 int32_t HcommBatchModeEnd(const char* batchTag);
