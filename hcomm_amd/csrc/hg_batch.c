@@ -148,11 +148,13 @@ void hg_shape_seg2(HgLaunch* l, int streaming)
     HgSeg2Table* t = &l->tab.seg2;
     /* the kernel for operands off 16-byte boundaries comes as a copy (op 255) and as a reduce: shaped like them */
     const int copy = l->kind == HCOMM_GFX_KERNEL_COPY || (l->kind == HCOMM_GFX_KERNEL_BYTEWISE && l->op == 255u);
-    if (l->kind == HCOMM_GFX_KERNEL_BYTEWISE || t->direct == 0u) {
-        /* The kernel for unaligned operands (its lanes assemble every vector from two loads) and the one-dimensional
-         * kernels (ragged tables; a few more rounds of argument reads before the data) want more workgroups per CU than
-         * the row-grid kernels the table above was swept with: order-preserving reduce-scatter on blocks of 16,777,214
-         * bytes 0.926 ms with these shapes, 0.997 with those; a ragged 512 MiB copy launch 170 against 187 us. */
+    const int bytewise = l->kind == HCOMM_GFX_KERNEL_BYTEWISE;
+    if ((bytewise && copy) || (!bytewise && t->direct == 0u)) {
+        /* The copy for unaligned operands and the one-dimensional kernels (ragged tables; a few more rounds of argument
+         * reads before the data) want more workgroups per CU than the row-grid kernels the table above was swept with:
+         * a ragged 512 MiB copy launch 170 against 187 us; the unaligned copy of 56 blocks of 16,777,214 bytes loses
+         * 17 % with two workgroups per CU.  The reduce for unaligned operands reads both operands in aligned vectors
+         * and is shaped like the aligned reduce (order-preserving reduce-scatter on such blocks 0.818 -> 0.788 ms). */
         l->streaming = streaming >= 0 ? (uint32_t)streaming : (l->bytes > (256ull << 20));
         l->lds_bytes = l->streaming ? 53248u : (copy ? 32768u : 0u);
         t->xcd_run = (l->streaming && !copy) ? 32u : 128u;

@@ -92,23 +92,56 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
 // ---- operands that are not on 16-byte boundaries ----------------------------------------------------------
 //
 // The few elements before dst's next 16-byte boundary go one by one; from there on dst is read and written in
-// aligned 16-byte items like k_copy / k_reduce2 do, and only src - as far from a boundary as it happens to be - is
-// loaded through a type that promises no more than the element's alignment: the compiler picks the widest access
-// the target allows for it (global memory takes unaligned dwordx4 loads in the unaligned access mode the HSA ABI
-// runs in; an item that straddles two cache lines is served from both).  An item holds whole elements because dst
-// and src are element-aligned and the head is a whole number of elements.  The bytes after the last whole item go
-// one by one too; head and tail belong to the tile that holds the end of the items.
+// aligned 16-byte items like k_copy / k_reduce2 do.  src - as far from a boundary as it happens to be - is read in
+// ALIGNED 16-byte vectors too: vector v of the 16-byte grid src sits in holds the first bytes of item v, the rest
+// are in vector v + 1 = what the next lane has loaded (the last lane of a wavefront loads it itself), and the two
+// are put together in registers.  (One unaligned 16-byte load per item - global memory takes them in the unaligned
+// access mode the HSA ABI runs in - is served from two cache lines wherever it straddles them and ran at 0.72 of the
+// HBM roofline where this runs at 0.83; reading the five dwords an item touches one by one was slower still.)  An
+// aligned vector that holds one byte of the operand lies inside the operand's pages, so the up to 15 bytes read
+// before its first and after its last byte never fault, and they are never used.  An item holds whole elements
+// because dst and src are element-aligned and the head is a whole number of elements.  The bytes after the last
+// whole item go one by one too; head and tail belong to the tile that holds the end of the items.
 
-template <uint32_t ES> struct UVec;
-template <> struct UVec<1> { typedef u32x4 T __attribute__((aligned(1))); };
-template <> struct UVec<2> { typedef u32x4 T __attribute__((aligned(2))); };
-template <> struct UVec<4> { typedef u32x4 T __attribute__((aligned(4))); };
+// Item v of src, which starts `off` bytes (1 ... 15) behind a 16-byte boundary, out of the two aligned vectors it
+// straddles: bytes off ... off+15 of lo:hi.  `off` is the same for every item of a segment.
+__device__ __forceinline__ u32x4 straddle(const u32x4 lo, const u32x4 hi, uint32_t off)
+{
+    const uint32_t c[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    const uint32_t r = off & 3u;
+    u32x4 o;
+    switch (off >> 2) { // uniform: a scalar branch
+        case 0:
+            o = u32x4{__builtin_amdgcn_alignbyte(c[1], c[0], r), __builtin_amdgcn_alignbyte(c[2], c[1], r),
+                      __builtin_amdgcn_alignbyte(c[3], c[2], r), __builtin_amdgcn_alignbyte(c[4], c[3], r)};
+            break;
+        case 1:
+            o = u32x4{__builtin_amdgcn_alignbyte(c[2], c[1], r), __builtin_amdgcn_alignbyte(c[3], c[2], r),
+                      __builtin_amdgcn_alignbyte(c[4], c[3], r), __builtin_amdgcn_alignbyte(c[5], c[4], r)};
+            break;
+        case 2:
+            o = u32x4{__builtin_amdgcn_alignbyte(c[3], c[2], r), __builtin_amdgcn_alignbyte(c[4], c[3], r),
+                      __builtin_amdgcn_alignbyte(c[5], c[4], r), __builtin_amdgcn_alignbyte(c[6], c[5], r)};
+            break;
+        default:
+            o = u32x4{__builtin_amdgcn_alignbyte(c[4], c[3], r), __builtin_amdgcn_alignbyte(c[5], c[4], r),
+                      __builtin_amdgcn_alignbyte(c[6], c[5], r), __builtin_amdgcn_alignbyte(c[7], c[6], r)};
+            break;
+    }
+    return o;
+}
+
+// The value lane + 1 of the wavefront holds (lane 63: its own).
+__device__ __forceinline__ u32x4 from_next_lane(const u32x4 v)
+{
+    return u32x4{(uint32_t)__shfl_down((int)v.x, 1, 64), (uint32_t)__shfl_down((int)v.y, 1, 64),
+                 (uint32_t)__shfl_down((int)v.z, 1, 64), (uint32_t)__shfl_down((int)v.w, 1, 64)};
+}
 
 // STREAM as for k_copy / k_reduce2.
 template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_bytewise(const HgSeg2Table tab)
 {
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
-    typedef typename UVec<ES>::T UV;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
     for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
@@ -123,18 +156,29 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
         const uint64_t nvec = (bytes - head) >> 4;
         const uint64_t vb = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         u32x4 a[HG_UNROLL], b[HG_UNROLL];
+        const uint32_t skew = (uint32_t)((uintptr_t)p & (HG_VEC_BYTES - 1));
+        const uint8_t* pa = p - skew;                            // the 16-byte grid src sits in
+        const uint64_t nsrc = nvec + (skew != 0 && nvec != 0);  // aligned vectors that hold bytes of the items
+        const bool last_lane = (tid & 63u) == 63u;
+        u32x4 own[HG_UNROLL];
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = vb + tid + u * HG_BLOCK;
-            if (v < nvec) {
-                b[u] = __builtin_nontemporal_load((const UV*)(p + (v << 4)));
-                if (REDUCE) a[u] = ldv<STREAM>(d, v);
-            }
+            b[u] = u32x4{0, 0, 0, 0};
+            own[u] = u32x4{0, 0, 0, 0};
+            if (v < nsrc) b[u] = ldv<true>(pa, v);
+            if (last_lane && v + 1 < nsrc) own[u] = ldv<true>(pa, v + 1);
+            if (REDUCE && v < nvec) a[u] = ldv<STREAM>(d, v);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < HG_UNROLL; ++u) {
+            const u32x4 next = from_next_lane(b[u]); // every lane takes part, whatever it has to do itself
+            if (skew != 0) b[u] = straddle(b[u], last_lane ? own[u] : next, skew);
         }
 #pragma unroll
         for (uint32_t u = 0; u < HG_UNROLL; ++u) {
             const uint64_t v = vb + tid + u * HG_BLOCK;
-            if (v < nvec) stv<STREAM>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]); // sc1 loses here (0.93 -> 1.00 ms on the odd-block reduce-scatter)
+            if (v < nvec) stp<(STREAM ? HG_ST_STREAM : HG_ST_SEG2)>(d, v, REDUCE ? vec_op<DT, OP>(a[u], b[u]) : b[u]);
         }
         if (vb <= nvec && vb + HG_TILE_VECS > nvec) { // the one tile that holds the end of the items
             // fewer than 16 / ES elements before the first item and fewer than that after the last one

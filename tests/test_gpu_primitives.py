@@ -107,6 +107,53 @@ def test_local_reduce_unaligned(gpu_thread, dtype, op, dst_el, src_el):
     assert_same(from_dev(d_a, a), want, dt)
 
 
+@pytest.mark.parametrize("dtype", ["int8", "bf16", "int32"])
+def test_unaligned_operands_every_skew_and_length(gpu_thread, dtype):
+    """The kernel for operands off 16-byte boundaries reads src in aligned vectors and puts every item together from
+    its own and the next lane's: every distance of src from a 16-byte boundary (in whole elements) against several of
+    dst's, for lengths of 0, 1, 2 items, one on either side of a wavefront's 64, of a workgroup's 256 and of a tile's
+    1,024, and a few tiles with a ragged end; copy and reduce in ONE batch each (all segments of a skew in one
+    launch), guard bytes before and behind every destination."""
+    dt = DT[dtype]
+    u = UNIT[dt]
+    items = [0, 1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4099]
+    rng = np.random.default_rng(77)
+    for dst_skew in sorted({0, u, 16 - u, 8}):
+        for src_skew in range(0, 16, u):
+            say("unaligned skews", dtype, dst_skew, src_skew)
+            cases = []
+            for n_items in items:
+                for extra in (0, u, 16 - u):        # bytes beyond the last whole item
+                    nbytes = n_items * 16 + extra + ((16 - dst_skew) % 16 if n_items else 0)
+                    if nbytes == 0:
+                        continue
+                    count = nbytes // u
+                    a, b = gen(dt, count + 64 // u, int(rng.integers(1 << 30))), gen(dt, count + 64 // u, int(rng.integers(1 << 30)))
+                    cases.append((count, a, b, to_dev(a), to_dev(b), to_dev(a)))
+            for reduce in (False, True):
+                assert h.HcommBatchModeStart(b"skews") == 0
+                for count, a, b, d_a, d_b, d_c in cases:
+                    dst = (d_a if reduce else d_c).data_ptr() + 16 + dst_skew
+                    src = d_b.data_ptr() + 16 + src_skew
+                    if reduce:
+                        assert h.HcommLocalReduceOnThread(gpu_thread, dst, src, count, dt, oracle.SUM) == 0
+                    else:
+                        assert h.HcommLocalCopyOnThread(gpu_thread, dst, src, count * u) == 0
+                assert h.HcommBatchModeEnd(b"skews") == 0
+                assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+                for count, a, b, d_a, d_b, d_c in cases:
+                    lo, so = (16 + dst_skew) // u, (16 + src_skew) // u
+                    want = a.copy()
+                    if reduce:
+                        with np.errstate(all="ignore"):
+                            oracle.reduce(want[lo:lo + count], b[so:so + count].copy(), dt, oracle.SUM)
+                    else:
+                        want[lo:lo + count] = b[so:so + count]
+                    got = from_dev(d_a if reduce else d_c, a)
+                    assert_same(got, want, dt, "%s skew %d/%d count %d %s" % (dtype, dst_skew, src_skew, count, "reduce" if reduce else "copy"))
+                    assert np.array_equal(from_dev(d_b, b).view(np.uint8), b.view(np.uint8)), "src modified"
+
+
 def test_local_reduce_dst_equals_src(gpu_thread):
     """The reference's UT passes the same pointer for both operands; the result is x (op) x."""
     a = gen(oracle.F32, 5000, 5)
