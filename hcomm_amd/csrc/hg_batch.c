@@ -49,6 +49,21 @@ static int direct_on(void)
     return v == 2;
 }
 
+/* A copy / two-input reduce launch that writes more than this many bytes takes part in the alternation of directions
+ * (hg_submit): HCOMM_GFX_ALTERNATE_BYTES, 0 = no launch does. */
+uint64_t hg_alternate_bytes(void)
+{
+    static uint64_t cached = 0; /* value + 1 */
+    uint64_t v = __atomic_load_n(&cached, __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv("HCOMM_GFX_ALTERNATE_BYTES");
+        v = (e && *e) ? strtoull(e, NULL, 10) : (128ull << 20);
+        v = (v == 0 || v >= UINT64_MAX - 1u) ? UINT64_MAX : v + 1u; /* 0: nothing is ever larger */
+        __atomic_store_n(&cached, v, __ATOMIC_RELAXED);
+    }
+    return v - 1u;
+}
+
 int32_t HcommGfxSetDirectLaunches(int32_t enable)
 {
     const int32_t before = direct_on();

@@ -65,6 +65,7 @@ typedef struct HgThread {
     /* batches that order several threads by notifies run on one of them: */
     void* join_ev;      /* hipEvent_t (created on first use) by which this thread's stream and another's are ordered */
     int own_work;       /* something was submitted on this thread's own stream since it was last joined to another */
+    int backwards_next[2]; /* the thread's next large reduce [0] / copy [1] launch walks its table from the end (hg_submit) */
     int led_batch;      /* other threads may still be waiting to be put behind join_ev on this thread's stream */
     struct HgThread* after; /* first thread of the batch this thread's stream is still to be put behind (hg_thread_settle) */
     uint32_t batch_cursor; /* next entry of `pending` while HcommBatchModeEnd walks the threads of a batch */
@@ -86,6 +87,7 @@ int hg_coalesce(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx);
 /* the same with the launch under construction in storage of the caller's (no allocation) */
 int hg_coalesce_with(const HgOp* ops, uint64_t n, HgEmitFn emit, void* ctx, HgLaunch* work);
 uint64_t hg_split_head(const HgOp* o);      /* bytes before the 16-byte boundary both operands reach together, or 0 */
+uint64_t hg_alternate_bytes(void);
 uint32_t hg_op_launch_key(const HgOp* o);   /* operations with different keys never share a launch */
 
 /* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment

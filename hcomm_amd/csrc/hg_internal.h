@@ -102,10 +102,11 @@ uint64_t hg_grid_blocks(uint64_t total_tiles);
 /* Launchers.  stream is a hipStream_t.  Return a HcclResult-compatible code. */
 /* streaming: the launch shape for output nothing reads back soon (and, for the reduce, a non-temporal load of the operand it overwrites);
  * lds: bytes of dynamic LDS per workgroup, asked for only to bound the workgroups a CU runs at once */
-int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
-int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds);
+/* backwards: the launch walks its table from the end - last segment first, every segment's last tile first */
+int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds, int backwards);
+int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds, int backwards);
 int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming,
-                       uint32_t lds);
+                       uint32_t lds, int backwards);
 int hg_launch_fold(void* stream, int dtype, int op, int acc_is_dst, const HgFoldTable* tab, uint64_t blocks, uint32_t lds);
 
 /* Thin wrappers over the HIP runtime so that the C files need no HIP headers. */

@@ -11,6 +11,10 @@
 
 namespace {
 
+// Set in a table's xcd_run by the launchers: the launch walks its table from the end - the last segment's last tile
+// goes to the first workgroup (see hg_submit for when and why).  The tiles stay what they are.
+#define HG_BACKWARDS 0x80000000u
+
 // ---- batched copy ------------------------------------------------------------------------------
 
 // STREAM: the variant for large launches - a copy that writes more than the memory-side cache holds, a reduce that
@@ -23,7 +27,8 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
+    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
+        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
         const uint32_t s = seg_of(tab, tile);
         const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         const uint64_t v0 = t0 + tid;
@@ -58,7 +63,8 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
+    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
+        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
         const uint32_t s = seg_of(tab, tile);
         const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         const uint64_t v0 = t0 + tid;
@@ -144,7 +150,8 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t tile = block_id(tab.xcd_run); tile < total; tile += gridDim.x) {
+    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
+        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
         const uint32_t s = seg_of(tab, tile);
         const uint64_t bytes = tab.bytes[s];
         uint8_t* d0 = (uint8_t*)tab.dst[s];
@@ -215,16 +222,30 @@ struct HgSeg2Few {
     uint32_t xcd_run;
 };
 
-HgSeg2Few few_of(const HgSeg2Table& t)
+// `backwards`: the rows in reverse order and the mark that makes a row's workgroups take its tiles from the end.
+HgSeg2Few few_of(const HgSeg2Table& t, bool backwards)
 {
     HgSeg2Few f;
     for (uint32_t s = 0; s < HG_DIRECT_SEG; ++s) {
-        f.dst[s] = s < t.nseg ? t.dst[s] : nullptr;
-        f.src[s] = s < t.nseg ? t.src[s] : nullptr;
-        f.bytes[s] = s < t.nseg ? t.bytes[s] : 0;
+        const uint32_t q = backwards ? t.nseg - 1u - s : s;
+        f.dst[s] = s < t.nseg ? t.dst[q] : nullptr;
+        f.src[s] = s < t.nseg ? t.src[q] : nullptr;
+        f.bytes[s] = s < t.nseg ? t.bytes[q] : 0;
     }
-    f.xcd_run = t.xcd_run;
+    f.xcd_run = t.xcd_run | (backwards ? HG_BACKWARDS : 0u);
     return f;
+}
+
+HgSeg2Table backwards_of(const HgSeg2Table& t)
+{
+    HgSeg2Table r = t;
+    for (uint32_t s = 0; s < t.nseg; ++s) {
+        r.dst[s] = t.dst[t.nseg - 1u - s];
+        r.src[s] = t.src[t.nseg - 1u - s];
+        r.bytes[s] = t.bytes[t.nseg - 1u - s];
+    }
+    r.xcd_run = t.xcd_run | HG_BACKWARDS;
+    return r;
 }
 
 template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_copy_rows(const Tab tab)
@@ -235,7 +256,8 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
     uint64_t bytes = tab.bytes[s];
     uint32_t run = tab.xcd_run, width = gridDim.x;
     arrive_together(d, p, bytes, run, width); // one round of argument reads
-    const uint32_t tile = block_id(run, width, blockIdx.x);
+    uint32_t tile = block_id(run & ~HG_BACKWARDS, width, blockIdx.x);
+    if (run & HG_BACKWARDS) tile = width - 1u - tile; // the launch walks memory from its end (the host has turned the rows round)
     const uint64_t nvec = bytes >> 4;
     const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
     const uint64_t v0 = t0 + tid;
@@ -267,7 +289,8 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
     uint64_t bytes = tab.bytes[s];
     uint32_t run = tab.xcd_run, width = gridDim.x;
     arrive_together(d, p, bytes, run, width); // one round of argument reads
-    const uint32_t tile = block_id(run, width, blockIdx.x);
+    uint32_t tile = block_id(run & ~HG_BACKWARDS, width, blockIdx.x);
+    if (run & HG_BACKWARDS) tile = width - 1u - tile; // the launch walks memory from its end (the host has turned the rows round)
     const uint64_t nvec = bytes >> 4;
     const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
     const uint64_t v0 = t0 + tid;
@@ -312,12 +335,13 @@ int launch_reduce2_rows(hipStream_t st, int op, const Tab& tab, dim3 g, uint32_t
 }
 
 template <int DT, bool STREAM>
-int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
+int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds, bool backwards)
 {
     const dim3 g(blocks), b(HG_BLOCK);
     if (tab->direct) {
         const dim3 g2(tab->direct, tab->nseg);
-        if (tab->nseg <= HG_DIRECT_SEG) return launch_reduce2_rows<DT, STREAM, HgSeg2Few>(st, op, few_of(*tab), g2, lds);
+        if (tab->nseg <= HG_DIRECT_SEG) return launch_reduce2_rows<DT, STREAM, HgSeg2Few>(st, op, few_of(*tab, backwards), g2, lds);
+        if (backwards) return launch_reduce2_rows<DT, STREAM, HgSeg2Table>(st, op, backwards_of(*tab), g2, lds);
         return launch_reduce2_rows<DT, STREAM, HgSeg2Table>(st, op, *tab, g2, lds);
     }
     switch (op) {
@@ -331,19 +355,21 @@ int launch_reduce2_dt_s(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t
 }
 
 template <int DT>
-int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, int streaming, uint32_t lds)
+int launch_reduce2_dt(hipStream_t st, int op, const HgSeg2Table* tab, uint32_t blocks, int streaming, uint32_t lds, bool backwards)
 {
-    if (streaming) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks, lds);
-    return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks, lds);
+    if (streaming) return launch_reduce2_dt_s<DT, true>(st, op, tab, blocks, lds, backwards);
+    return launch_reduce2_dt_s<DT, false>(st, op, tab, blocks, lds, backwards);
 }
 
-template <bool STREAM> int launch_copy_s(hipStream_t st, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds)
+template <bool STREAM> int launch_copy_s(hipStream_t st, const HgSeg2Table* tab, uint32_t blocks, uint32_t lds, bool backwards)
 {
     const dim3 b(HG_BLOCK);
     if (tab->direct) {
         const dim3 g2(tab->direct, tab->nseg);
         if (tab->nseg <= HG_DIRECT_SEG)
-            hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Few>), g2, b, lds, st, few_of(*tab));
+            hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Few>), g2, b, lds, st, few_of(*tab, backwards));
+        else if (backwards)
+            hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Table>), g2, b, lds, st, backwards_of(*tab));
         else
             hipLaunchKernelGGL((k_copy_rows<STREAM, HgSeg2Table>), g2, b, lds, st, *tab);
     } else {
@@ -376,25 +402,43 @@ template <int DT> int launch_bytewise_dt(hipStream_t st, int op, const HgSeg2Tab
 extern "C" {
 
 
-int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
+// The one-dimensional kernels walk the whole table from its last tile when the mark is set; the row grids also need
+// their rows turned round (launch_*_s).
+#define HG_MARK_ONE_DIMENSIONAL(tab, backwards)      \
+    HgSeg2Table marked_;                              \
+    if ((backwards) && !(tab)->direct) {              \
+        marked_ = *(tab);                             \
+        marked_.xcd_run |= HG_BACKWARDS;              \
+        (tab) = &marked_;                             \
+    }
+
+int hg_launch_copy(void* stream, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds, int backwards)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-    if (streaming) return launch_copy_s<true>((hipStream_t)stream, tab, (uint32_t)blocks, lds);
-    return launch_copy_s<false>((hipStream_t)stream, tab, (uint32_t)blocks, lds);
+    HG_MARK_ONE_DIMENSIONAL(tab, backwards)
+    if (streaming) return launch_copy_s<true>((hipStream_t)stream, tab, (uint32_t)blocks, lds, backwards != 0);
+    return launch_copy_s<false>((hipStream_t)stream, tab, (uint32_t)blocks, lds, backwards != 0);
 }
 
-int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds)
+int hg_launch_reduce2(void* stream, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming, uint32_t lds, int backwards)
 {
     if (blocks == 0) return HCCL_SUCCESS;
-#define CALL(DT) launch_reduce2_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, streaming, lds)
+    HG_MARK_ONE_DIMENSIONAL(tab, backwards)
+#define CALL(DT) launch_reduce2_dt<DT>((hipStream_t)stream, op, tab, (uint32_t)blocks, streaming, lds, backwards != 0)
     HG_DISPATCH_DT(dtype, CALL)
 #undef CALL
 }
 
 int hg_launch_bytewise(void* stream, int is_reduce, int dtype, int op, const HgSeg2Table* tab, uint64_t blocks, int streaming,
-                       uint32_t lds)
+                       uint32_t lds, int backwards)
 {
     if (blocks == 0) return HCCL_SUCCESS;
+    HgSeg2Table marked;
+    if (backwards) {
+        marked = *tab;
+        marked.xcd_run |= HG_BACKWARDS;
+        tab = &marked;
+    }
     if (!is_reduce) {
         const dim3 g((uint32_t)blocks), b(HG_BLOCK);
         if (streaming) hipLaunchKernelGGL((k_bytewise<DT_I8, OP_SUM, false, true>), g, b, lds, (hipStream_t)stream, *tab);

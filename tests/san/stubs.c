@@ -9,9 +9,9 @@
 #ifdef HG_STUB_GPU_PRESENT
 unsigned long hg_stub_launches = 0;
 static char stub_scratch[256] __attribute__((aligned(256)));
-int hg_launch_copy(void* s, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)t; (void)b; (void)m; (void)l; ++hg_stub_launches; return 0; }
-int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)d; (void)o; (void)t; (void)b; (void)m; (void)l; ++hg_stub_launches; return 0; }
-int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, int st, uint32_t l) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)st; (void)l; ++hg_stub_launches; return 0; }
+int hg_launch_copy(void* s, const HgSeg2Table* t, uint64_t b, int m, uint32_t l, int w) { (void)s; (void)t; (void)b; (void)m; (void)l; (void)w; ++hg_stub_launches; return 0; }
+int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, int m, uint32_t l, int w) { (void)s; (void)d; (void)o; (void)t; (void)b; (void)m; (void)l; (void)w; ++hg_stub_launches; return 0; }
+int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, int st, uint32_t l, int w) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)st; (void)l; (void)w; ++hg_stub_launches; return 0; }
 int hg_launch_fold(void* s, int d, int o, int a, const HgFoldTable* t, uint64_t b, uint32_t l) { (void)s; (void)d; (void)o; (void)a; (void)t; (void)b; (void)l; ++hg_stub_launches; return 0; }
 int hg_rt_device_count(void) { return 1; }
 int hg_rt_scratch(void* s, void** p) { (void)s; *p = stub_scratch; return 0; } /* an address to do arithmetic on: never dereferenced */
@@ -31,9 +31,9 @@ int hg_rt_capture_end(void* s, void** g) { (void)s; *g = NULL; return 4; }
 int hg_rt_graph_launch(void* g, void* s) { (void)g; (void)s; return 4; }
 int hg_rt_graph_destroy(void* g) { (void)g; return 0; }
 #else
-int hg_launch_copy(void* s, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)t; (void)b; (void)m; (void)l; return 4; }
-int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, int m, uint32_t l) { (void)s; (void)d; (void)o; (void)t; (void)b; (void)m; (void)l; return 4; }
-int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, int st, uint32_t l) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)st; (void)l; return 4; }
+int hg_launch_copy(void* s, const HgSeg2Table* t, uint64_t b, int m, uint32_t l, int w) { (void)s; (void)t; (void)b; (void)m; (void)l; (void)w; return 4; }
+int hg_launch_reduce2(void* s, int d, int o, const HgSeg2Table* t, uint64_t b, int m, uint32_t l, int w) { (void)s; (void)d; (void)o; (void)t; (void)b; (void)m; (void)l; (void)w; return 4; }
+int hg_launch_bytewise(void* s, int r, int d, int o, const HgSeg2Table* t, uint64_t b, int st, uint32_t l, int w) { (void)s; (void)r; (void)d; (void)o; (void)t; (void)b; (void)st; (void)l; (void)w; return 4; }
 int hg_launch_fold(void* s, int d, int o, int a, const HgFoldTable* t, uint64_t b, uint32_t l) { (void)s; (void)d; (void)o; (void)a; (void)t; (void)b; (void)l; return 4; }
 int hg_rt_device_count(void) { return 0; }
 int hg_rt_scratch(void* s, void** p) { (void)s; *p = NULL; return 4; }

@@ -154,6 +154,49 @@ def test_unaligned_operands_every_skew_and_length(gpu_thread, dtype):
                     assert np.array_equal(from_dev(d_b, b).view(np.uint8), b.view(np.uint8)), "src modified"
 
 
+@pytest.mark.parametrize("shape", ["rows_few", "rows_many", "ragged", "unaligned"])
+@pytest.mark.parametrize("reduce", [False, True])
+def test_a_launch_gives_the_same_bytes_in_either_direction(gpu_thread, shape, reduce):
+    """Every other copy / two-input reduce launch of a thread walks its table from the end (the bytes the launch
+    before finished with are the ones the memory-side cache still holds).  The same batch three times in a row
+    therefore runs in both directions: same result each time, for the row grids with the short and the full argument
+    table, the one-dimensional kernels (segments of very different lengths) and the kernel for unaligned operands,
+    with element tails and guard bytes."""
+    dt = DT["bf16"]
+    u = UNIT[dt]
+    counts = {"rows_few": [70001] * 5 + [69999], "rows_many": [33001 + (i % 3) for i in range(20)],
+              "ragged": [5, 300007, 17, 65536, 1000001, 1], "unaligned": [70001, 8191, 300007]}[shape]
+    skew = 1 if shape == "unaligned" else 0
+    say("both directions", shape, reduce)
+    rng = np.random.default_rng(5)
+    bufs = [(gen(dt, c + 32, int(rng.integers(1 << 30))), gen(dt, c + 32, int(rng.integers(1 << 30)))) for c in counts]
+    for attempt in range(3):
+        dev = [(to_dev(a), to_dev(b)) for a, b in bufs]
+        h.HcommGfxLaunchLogClear(gpu_thread)
+        assert h.HcommBatchModeStart(b"dir") == 0
+        for c, (d_a, d_b) in zip(counts, dev):
+            dst, src = d_a.data_ptr() + 16 + skew * u, d_b.data_ptr() + 16 + 3 * skew * u
+            if reduce:
+                assert h.HcommLocalReduceOnThread(gpu_thread, dst, src, c, dt, oracle.SUM) == 0
+            else:
+                assert h.HcommLocalCopyOnThread(gpu_thread, dst, src, c * u) == 0
+        assert h.HcommBatchModeEnd(b"dir") == 0
+        assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
+        log = h.launch_log(gpu_thread)
+        assert len(log) == 1
+        want_kind = h.Kernel.BYTEWISE if skew else (h.Kernel.REDUCE2 if reduce else h.Kernel.COPY)
+        assert log[0].kind == want_kind and bool(log[0].rows) == shape.startswith("rows")
+        for c, (a, b), (d_a, d_b) in zip(counts, bufs, dev):
+            lo, so = 16 // u + skew, 16 // u + 3 * skew
+            want = a.copy()
+            if reduce:
+                with np.errstate(all="ignore"):
+                    oracle.reduce(want[lo:lo + c], b[so:so + c].copy(), dt, oracle.SUM)
+            else:
+                want[lo:lo + c] = b[so:so + c]
+            assert_same(from_dev(d_a, a), want, dt, "%s attempt %d count %d" % (shape, attempt, c))
+
+
 def test_local_reduce_dst_equals_src(gpu_thread):
     """The reference's UT passes the same pointer for both operands; the result is x (op) x."""
     a = gen(oracle.F32, 5000, 5)
