@@ -20,7 +20,7 @@ __all__ = [
     "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
     "HcommThreadNotifyWaitOnThread", "HcommMemAlloc", "HcommMemFree", "HcommBatchModeStart", "HcommBatchModeEnd",
     "HcommGfxThreadSynchronize", "HcommGfxReduceKOnThread", "HcommGfxRecorderThreadAlloc", "launch_log",
-    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion", "HcommGfxSetDirectLaunches",
+    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion", "HcommGfxSetDirectLaunches", "HcommGfxSetAlternateBytes",
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
@@ -93,7 +93,8 @@ class Kernel:
 
 class LaunchRecord(C.Structure):
     _fields_ = [("kind", C.c_uint32), ("dtype", C.c_uint32), ("op", C.c_uint32), ("nseg", C.c_uint32),
-                ("bytes", C.c_uint64), ("blocks", C.c_uint64), ("rows", C.c_uint32), ("streaming", C.c_uint32)]
+                ("bytes", C.c_uint64), ("blocks", C.c_uint64), ("rows", C.c_uint32), ("streaming", C.c_uint32),
+                ("backwards", C.c_uint32), ("reserved", C.c_uint32)]
 
 
 class PlanInfo(C.Structure):
@@ -280,6 +281,14 @@ _set_direct = _sig("HcommGfxSetDirectLaunches", C.c_int32, C.c_int32)
 def HcommGfxSetDirectLaunches(enable):
     """0: launches shaped from now on stay on the kernels large launches use; 1: the default.  Returns the previous setting."""
     return int(_set_direct(1 if enable else 0))
+
+
+_set_alternate = _sig("HcommGfxSetAlternateBytes", C.c_uint64, C.c_uint64)
+
+
+def HcommGfxSetAlternateBytes(nbytes):
+    """Launches that write more than nbytes may walk their table backwards (0 = never); returns the previous value."""
+    return _set_alternate(nbytes)
 
 
 def HcommGfxVersion():

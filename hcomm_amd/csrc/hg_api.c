@@ -288,7 +288,7 @@ int32_t HcommGfxThreadSynchronize(ThreadHandle thread)
 
 /* ---- launch log and submission ---------------------------------------------------------------------- */
 
-static void log_launch(HgThread* t, const HgLaunch* l)
+static void log_launch(HgThread* t, const HgLaunch* l, int backwards)
 {
     if (!t->log_enabled || t->log_n >= HG_LOG_MAX) return;
     if (t->log_n == t->log_cap) {
@@ -308,9 +308,11 @@ static void log_launch(HgThread* t, const HgLaunch* l)
     r->blocks = l->blocks;
     r->rows = hg_launch_rows(l);
     r->streaming = l->streaming;
+    r->backwards = (uint32_t)backwards;
+    r->reserved = 0;
 }
 
-void hg_log_only(HgThread* t, const HgLaunch* l) { log_launch(t, l); }
+void hg_log_only(HgThread* t, const HgLaunch* l) { log_launch(t, l, 0); }
 
 /*
  * A batch that ordered its threads by notifies ran on the stream of its first thread.  Its other threads are put
@@ -330,32 +332,65 @@ int hg_thread_settle(HgThread* t)
     return hg_rt_stream_wait_event(t->stream, lead->join_ev);
 }
 
+/*
+ * Which way a large copy / two-input reduce launch walks its table.  A step of a schedule reads what a step before
+ * it wrote.  When that step wrote more than the memory-side cache keeps, the cache is left with what it wrote LAST -
+ * which a launch walking memory in the same direction reaches last, after its own traffic has displaced it.  So a
+ * launch that reads what one of the thread's last two large launches wrote walks the other way than that launch
+ * did (last segment first, every segment's last tile first: it starts on the bytes still cached); one that reads
+ * nothing of theirs (the first step of a collective, a fetch of fresh data between two folds) walks forwards.
+ * 16-rank halving-doubling allreduce 1.535 -> 1.506 ms, 7-rank ring reduce-scatter in steps of 400 MB 1.107 -> 1.066,
+ * deterministic mesh reduce-scatter 0.737 -> 0.698; the double-ring reduce-scatter over 2 x 8 ranks, whose folds
+ * alternate with fetches as large as they are, is the one loser (1.480 -> 1.496: its folds gain, its fetches lose more).
+ * Results do not depend on it.  Launches that write no more than HCOMM_GFX_ALTERNATE_BYTES (128 MiB) fit the cache
+ * with their operands and are left alone.
+ */
+static int reads_from(const HgLaunch* l, const struct HgWritten* w)
+{
+    const HgSeg2Table* t = &l->tab.seg2;
+    const int reads_dst = l->op != 255u; /* a reduce reads the operand it overwrites */
+    for (uint32_t s = 0; s < t->nseg; ++s) {
+        const uintptr_t p0 = (uintptr_t)t->src[s], d0 = (uintptr_t)t->dst[s];
+        const uint64_t n = t->bytes[s];
+        for (uint32_t q = 0; q < w->n; ++q) {
+            const uintptr_t w0 = (uintptr_t)w->at[q];
+            if (p0 < w0 + w->bytes[q] && w0 < p0 + n) return 1;
+            if (reads_dst && d0 < w0 + w->bytes[q] && w0 < d0 + n) return 1;
+        }
+    }
+    return 0;
+}
+
+static int direction_of(HgThread* t, const HgLaunch* l)
+{
+    if (l->bytes <= hg_alternate_bytes()) return 0;
+    int backwards;
+    if (reads_from(l, &t->written[0])) backwards = !t->written[0].backwards;
+    else if (reads_from(l, &t->written[1])) backwards = !t->written[1].backwards;
+    else backwards = 0;
+    t->written[1] = t->written[0];
+    struct HgWritten* w = &t->written[0];
+    const HgSeg2Table* tab = &l->tab.seg2;
+    w->n = tab->nseg;
+    w->backwards = backwards;
+    for (uint32_t s = 0; s < tab->nseg; ++s) {
+        w->at[s] = tab->dst[s];
+        w->bytes[s] = tab->bytes[s];
+    }
+    return backwards;
+}
+
 int hg_submit(HgThread* t, const HgLaunch* l)
 {
-    log_launch(t, l);
+    const int backwards = (l->kind == HCOMM_GFX_KERNEL_COPY || l->kind == HCOMM_GFX_KERNEL_REDUCE2 || l->kind == HCOMM_GFX_KERNEL_BYTEWISE)
+                              ? direction_of(t, l) : 0;
+    log_launch(t, l, backwards);
     if (t->recorder) return HCCL_SUCCESS;
     if (t->after) {
         const int rc = hg_thread_settle(t);
         if (rc != HCCL_SUCCESS) return rc;
     }
     t->own_work = 1;
-    /* Consecutive launches on a thread are, as a rule, consecutive steps of a schedule: each reads what the one before
-     * wrote.  When a step writes more than the memory-side cache keeps, the cache is left with what was written LAST -
-     * which a launch that walks memory in the same direction reaches last, after its own traffic has displaced it.
-     * So every other one of a thread's large copy / two-input reduce launches walks its table from the end: it starts
-     * on the bytes the launch before finished with (16-rank halving-doubling allreduce 1.540 -> 1.513 ms, 7-rank ring
-     * reduce-scatter of 400 MB steps 1.114 -> 1.066).  Results do not depend on it.  Launches that fit the cache are
-     * left alone: walking backwards hands a tile to another XCD than the step before did, which costs the small
-     * cache-resident steps their L2 hits (8 x 4 MiB mesh steps + 8 %). */
-    int backwards = 0;
-    if ((l->kind == HCOMM_GFX_KERNEL_COPY || l->kind == HCOMM_GFX_KERNEL_REDUCE2 || l->kind == HCOMM_GFX_KERNEL_BYTEWISE) &&
-        l->bytes > hg_alternate_bytes()) {
-        /* copies and reduces alternate each among themselves: where a schedule interleaves the two (a fold, then the
-         * fetch of the next shares), a single alternation would give every fold the same direction */
-        const int which = l->op == 255u;
-        backwards = t->backwards_next[which];
-        t->backwards_next[which] = !t->backwards_next[which];
-    }
     switch (l->kind) {
         case HCOMM_GFX_KERNEL_COPY:
             return hg_launch_copy(t->stream, &l->tab.seg2, l->blocks, (int)l->streaming, l->lds_bytes, backwards);

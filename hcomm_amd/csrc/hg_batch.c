@@ -49,19 +49,28 @@ static int direct_on(void)
     return v == 2;
 }
 
-/* A copy / two-input reduce launch that writes more than this many bytes takes part in the alternation of directions
- * (hg_submit): HCOMM_GFX_ALTERNATE_BYTES, 0 = no launch does. */
+/* A copy / two-input reduce launch that writes more than this many bytes may walk its table backwards (direction_of
+ * in hg_api.c): HCOMM_GFX_ALTERNATE_BYTES, 0 = no launch does. */
+static uint64_t g_alternate = 0; /* 0 = not read yet; else the threshold + 1, UINT64_MAX = never */
+
+static uint64_t alternate_encode(uint64_t bytes) { return (bytes == 0 || bytes >= UINT64_MAX - 1u) ? UINT64_MAX : bytes + 1u; }
+
 uint64_t hg_alternate_bytes(void)
 {
-    static uint64_t cached = 0; /* value + 1 */
-    uint64_t v = __atomic_load_n(&cached, __ATOMIC_RELAXED);
+    uint64_t v = __atomic_load_n(&g_alternate, __ATOMIC_RELAXED);
     if (v == 0) {
         const char* e = getenv("HCOMM_GFX_ALTERNATE_BYTES");
-        v = (e && *e) ? strtoull(e, NULL, 10) : (128ull << 20);
-        v = (v == 0 || v >= UINT64_MAX - 1u) ? UINT64_MAX : v + 1u; /* 0: nothing is ever larger */
-        __atomic_store_n(&cached, v, __ATOMIC_RELAXED);
+        v = alternate_encode((e && *e) ? strtoull(e, NULL, 10) : (128ull << 20));
+        __atomic_store_n(&g_alternate, v, __ATOMIC_RELAXED);
     }
-    return v - 1u;
+    return v - 1u; /* never: UINT64_MAX - 1, which no launch exceeds */
+}
+
+uint64_t HcommGfxSetAlternateBytes(uint64_t bytes)
+{
+    const uint64_t before = hg_alternate_bytes();
+    __atomic_store_n(&g_alternate, alternate_encode(bytes), __ATOMIC_RELAXED);
+    return before == UINT64_MAX - 1u ? 0 : before;
 }
 
 int32_t HcommGfxSetDirectLaunches(int32_t enable)

@@ -297,6 +297,17 @@ __device__ __forceinline__ uint32_t block_id(uint32_t run, uint32_t g, uint32_t 
 }
 __device__ __forceinline__ uint32_t block_id(uint32_t run) { return block_id(run, gridDim.x, blockIdx.x); }
 
+// The same deal walked backwards in time: workgroup b gets the tile that the workgroup which its XCD runs at the
+// mirrored moment gets above - the k-th workgroup of an XCD takes what the k-th from the end would have taken - so a
+// launch starts on the tiles the forward deal ends with, and every tile stays on the XCD the forward deal gives it
+// to.  The few workgroups beyond the last whole group of 8 keep their tiles.
+__device__ __forceinline__ uint32_t block_id_backwards(uint32_t run, uint32_t g, uint32_t b)
+{
+    const uint32_t whole = g & ~7u;
+    if (b >= whole) return block_id(run, g, b);
+    return block_id(run, g, ((whole >> 3) - 1u - (b >> 3)) * 8u + (b & 7u));
+}
+
 // The point by which all the given scalar values must have arrived: the loads that fetch them (kernel arguments, the
 // grid size) are all issued before it and waited for once, instead of each where the compiler first needs its value.
 template <class A, class B, class C, class D, class E>

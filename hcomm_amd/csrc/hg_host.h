@@ -65,7 +65,13 @@ typedef struct HgThread {
     /* batches that order several threads by notifies run on one of them: */
     void* join_ev;      /* hipEvent_t (created on first use) by which this thread's stream and another's are ordered */
     int own_work;       /* something was submitted on this thread's own stream since it was last joined to another */
-    int backwards_next[2]; /* the thread's next large reduce [0] / copy [1] launch walks its table from the end (hg_submit) */
+    /* what the thread's last two large copy / two-input reduce launches wrote, and which way they walked (hg_submit) */
+    struct HgWritten {
+        uint32_t n;
+        int backwards;
+        const void* at[HG_MAX_SEG2];
+        uint64_t bytes[HG_MAX_SEG2];
+    } written[2]; /* [0] the later one */
     int led_batch;      /* other threads may still be waiting to be put behind join_ev on this thread's stream */
     struct HgThread* after; /* first thread of the batch this thread's stream is still to be put behind (hg_thread_settle) */
     uint32_t batch_cursor; /* next entry of `pending` while HcommBatchModeEnd walks the threads of a batch */

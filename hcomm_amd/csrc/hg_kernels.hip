@@ -27,8 +27,9 @@ template <bool STREAM> __global__ __launch_bounds__(HG_BLOCK) void k_copy(const 
 {
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
-        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
+    const uint32_t first = (tab.xcd_run & HG_BACKWARDS) ? block_id_backwards(tab.xcd_run & ~HG_BACKWARDS, gridDim.x, blockIdx.x)
+                                                         : block_id(tab.xcd_run);
+    for (uint32_t tile = first; tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
         const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         const uint64_t v0 = t0 + tid;
@@ -63,8 +64,9 @@ template <int DT, int OP, bool STREAM> __global__ __launch_bounds__(HG_BLOCK) vo
     constexpr uint32_t ES = ElemSize<DT>::v;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
-        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
+    const uint32_t first = (tab.xcd_run & HG_BACKWARDS) ? block_id_backwards(tab.xcd_run & ~HG_BACKWARDS, gridDim.x, blockIdx.x)
+                                                         : block_id(tab.xcd_run);
+    for (uint32_t tile = first; tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
         const uint64_t t0 = (uint64_t)(tile - tab.tile_begin[s]) * HG_TILE_VECS;
         const uint64_t v0 = t0 + tid;
@@ -150,8 +152,9 @@ template <int DT, int OP, bool REDUCE, bool STREAM> __global__ __launch_bounds__
     constexpr uint32_t ES = REDUCE ? ElemSize<DT>::v : 1u;
     const uint32_t total = tab.tile_begin[tab.nseg];
     const uint32_t tid = threadIdx.x;
-    for (uint32_t at = block_id(tab.xcd_run & ~HG_BACKWARDS); at < total; at += gridDim.x) {
-        const uint32_t tile = (tab.xcd_run & HG_BACKWARDS) ? total - 1u - at : at;
+    const uint32_t first = (tab.xcd_run & HG_BACKWARDS) ? block_id_backwards(tab.xcd_run & ~HG_BACKWARDS, gridDim.x, blockIdx.x)
+                                                         : block_id(tab.xcd_run);
+    for (uint32_t tile = first; tile < total; tile += gridDim.x) {
         const uint32_t s = seg_of(tab, tile);
         const uint64_t bytes = tab.bytes[s];
         uint8_t* d0 = (uint8_t*)tab.dst[s];
@@ -256,8 +259,8 @@ template <bool STREAM, class Tab> __global__ __launch_bounds__(HG_BLOCK) void k_
     uint64_t bytes = tab.bytes[s];
     uint32_t run = tab.xcd_run, width = gridDim.x;
     arrive_together(d, p, bytes, run, width); // one round of argument reads
-    uint32_t tile = block_id(run & ~HG_BACKWARDS, width, blockIdx.x);
-    if (run & HG_BACKWARDS) tile = width - 1u - tile; // the launch walks memory from its end (the host has turned the rows round)
+    // HG_BACKWARDS: the launch walks memory from its end (the host has turned the rows round)
+    const uint32_t tile = (run & HG_BACKWARDS) ? block_id_backwards(run & ~HG_BACKWARDS, width, blockIdx.x) : block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
     const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
     const uint64_t v0 = t0 + tid;
@@ -289,8 +292,8 @@ template <int DT, int OP, bool STREAM, class Tab> __global__ __launch_bounds__(H
     uint64_t bytes = tab.bytes[s];
     uint32_t run = tab.xcd_run, width = gridDim.x;
     arrive_together(d, p, bytes, run, width); // one round of argument reads
-    uint32_t tile = block_id(run & ~HG_BACKWARDS, width, blockIdx.x);
-    if (run & HG_BACKWARDS) tile = width - 1u - tile; // the launch walks memory from its end (the host has turned the rows round)
+    // HG_BACKWARDS: the launch walks memory from its end (the host has turned the rows round)
+    const uint32_t tile = (run & HG_BACKWARDS) ? block_id_backwards(run & ~HG_BACKWARDS, width, blockIdx.x) : block_id(run, width, blockIdx.x);
     const uint64_t nvec = bytes >> 4;
     const uint64_t t0 = (uint64_t)tile * HG_TILE_VECS;
     const uint64_t v0 = t0 + tid;

@@ -1578,6 +1578,8 @@ int32_t HcommGfxPlanGetLaunch(const HcommGfxPlan* plan, uint32_t i, HcommGfxLaun
     rec->blocks = l->blocks;
     rec->rows = hg_launch_rows(l);
     rec->streaming = l->streaming;
+    rec->backwards = 0;
+    rec->reserved = 0;
     return HCCL_SUCCESS;
 }
 

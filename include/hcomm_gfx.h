@@ -344,6 +344,9 @@ typedef struct {
                         address read in one round (the k_*_rows kernels); 0 = one-dimensional grid over the table's
                         tiles.  Folds: 1 = small launch whose addresses the host resolves (the k_fold_*_direct kernels) */
     uint32_t streaming; /* copy / two-input reduce: 1 = the variant for output that nothing reads back soon */
+    uint32_t backwards; /* copy / two-input reduce: 1 = the launch walked its table from the end (HcommGfxSetAlternateBytes);
+                           decided when a launch is submitted, so always 0 in what HcommGfxPlanGetLaunch reports */
+    uint32_t reserved;
 } HcommGfxLaunchRecord;
 
 typedef enum {
@@ -999,6 +1002,13 @@ int32_t HcommGfxOpBaseCheck(
  * the tests run those kernels on small and ragged shapes; 1 restores the default.  Returns the previous setting.
  * HCOMM_GFX_DIRECT=0 in the environment sets the initial value to 0. */
 int32_t HcommGfxSetDirectLaunches(int32_t enable);
+
+/* No reference counterpart.  A copy / two-input reduce launch that writes more than `bytes` and reads what one of
+ * its thread's last two such launches wrote walks its table the other way than that launch did (it starts on what
+ * the memory-side cache still holds of it); 0 = no launch ever does.  Returns the previous value; the initial one is
+ * HCOMM_GFX_ALTERNATE_BYTES from the environment, 128 MiB without it.  Results never depend on it; tests lower it
+ * to run both directions on small shapes. */
+uint64_t HcommGfxSetAlternateBytes(uint64_t bytes);
 
 /* Library version string, e.g. "hcomm_gfx 0.1 gfx950". */
 const char* HcommGfxVersion(void);

@@ -157,11 +157,12 @@ def test_unaligned_operands_every_skew_and_length(gpu_thread, dtype):
 @pytest.mark.parametrize("shape", ["rows_few", "rows_many", "ragged", "unaligned"])
 @pytest.mark.parametrize("reduce", [False, True])
 def test_a_launch_gives_the_same_bytes_in_either_direction(gpu_thread, shape, reduce):
-    """Every other copy / two-input reduce launch of a thread walks its table from the end (the bytes the launch
-    before finished with are the ones the memory-side cache still holds).  The same batch three times in a row
-    therefore runs in both directions: same result each time, for the row grids with the short and the full argument
-    table, the one-dimensional kernels (segments of very different lengths) and the kernel for unaligned operands,
-    with element tails and guard bytes."""
+    """A large launch that reads what the launch before it wrote walks its table the other way (it starts on the bytes
+    the memory-side cache still holds).  With the size from which that applies lowered to one byte, a chain of four
+    dependent launches - dst (op)= src four times, or a copy passed on from buffer to buffer - runs forwards, backwards,
+    forwards, backwards: same bytes as the oracle's, for the row grids with the short and the full argument table,
+    the one-dimensional kernels (segments of very different lengths) and the kernel for unaligned operands, with
+    element tails and guard bytes."""
     dt = DT["bf16"]
     u = UNIT[dt]
     counts = {"rows_few": [70001] * 5 + [69999], "rows_many": [33001 + (i % 3) for i in range(20)],
@@ -169,32 +170,49 @@ def test_a_launch_gives_the_same_bytes_in_either_direction(gpu_thread, shape, re
     skew = 1 if shape == "unaligned" else 0
     say("both directions", shape, reduce)
     rng = np.random.default_rng(5)
+    lo, so, lo_c = 16 // u + skew, 16 // u + 3 * skew, 16 // u + 2 * skew   # no two of them equally far from a 16-byte boundary
     bufs = [(gen(dt, c + 32, int(rng.integers(1 << 30))), gen(dt, c + 32, int(rng.integers(1 << 30)))) for c in counts]
-    for attempt in range(3):
-        dev = [(to_dev(a), to_dev(b)) for a, b in bufs]
-        h.HcommGfxLaunchLogClear(gpu_thread)
-        assert h.HcommBatchModeStart(b"dir") == 0
-        for c, (d_a, d_b) in zip(counts, dev):
-            dst, src = d_a.data_ptr() + 16 + skew * u, d_b.data_ptr() + 16 + 3 * skew * u
-            if reduce:
-                assert h.HcommLocalReduceOnThread(gpu_thread, dst, src, c, dt, oracle.SUM) == 0
-            else:
-                assert h.HcommLocalCopyOnThread(gpu_thread, dst, src, c * u) == 0
-        assert h.HcommBatchModeEnd(b"dir") == 0
+    dev = [(to_dev(a), to_dev(b), to_dev(a)) for a, b in bufs]   # dst, src, a second destination for the copy chain
+    before = h.HcommGfxSetAlternateBytes(1)
+    row_grids = h.HcommGfxSetDirectLaunches(1)   # as the caller has set it: this module also runs with them off
+    h.HcommGfxSetDirectLaunches(row_grids)
+    try:
+        for hop in range(4):
+            h.HcommGfxLaunchLogClear(gpu_thread)
+            assert h.HcommBatchModeStart(b"dir") == 0
+            for c, (d_a, d_b, d_c) in zip(counts, dev):
+                if reduce:
+                    assert h.HcommLocalReduceOnThread(gpu_thread, d_a.data_ptr() + lo * u, d_b.data_ptr() + so * u, c, dt,
+                                                      oracle.SUM) == 0
+                else:   # src -> a -> c -> a -> c, every hop reading what the hop before wrote
+                    chain = [(d_b, so), (d_a, lo), (d_c, lo_c), (d_a, lo), (d_c, lo_c)]
+                    (src, s_off), (dst, d_off) = chain[hop], chain[hop + 1]
+                    assert h.HcommLocalCopyOnThread(gpu_thread, dst.data_ptr() + d_off * u, src.data_ptr() + s_off * u,
+                                                    c * u) == 0
+            assert h.HcommBatchModeEnd(b"dir") == 0
+            log = h.launch_log(gpu_thread)
+            assert len(log) == 1
+            want_kind = h.Kernel.BYTEWISE if skew else (h.Kernel.REDUCE2 if reduce else h.Kernel.COPY)
+            assert log[0].kind == want_kind and bool(log[0].rows) == (row_grids and shape.startswith("rows"))
+            if hop == 0:   # forwards, unless the allocator handed out memory a launch of an earlier test wrote to
+                first = log[0].backwards
+            assert log[0].backwards == (first + hop) % 2
         assert h.HcommGfxThreadSynchronize(gpu_thread) == 0
-        log = h.launch_log(gpu_thread)
-        assert len(log) == 1
-        want_kind = h.Kernel.BYTEWISE if skew else (h.Kernel.REDUCE2 if reduce else h.Kernel.COPY)
-        assert log[0].kind == want_kind and bool(log[0].rows) == shape.startswith("rows")
-        for c, (a, b), (d_a, d_b) in zip(counts, bufs, dev):
-            lo, so = 16 // u + skew, 16 // u + 3 * skew
-            want = a.copy()
-            if reduce:
-                with np.errstate(all="ignore"):
+    finally:
+        assert h.HcommGfxSetAlternateBytes(before) == 1
+    for c, (a, b), (d_a, d_b, d_c) in zip(counts, bufs, dev):
+        want = a.copy()
+        if reduce:
+            with np.errstate(all="ignore"):
+                for hop in range(4):
                     oracle.reduce(want[lo:lo + c], b[so:so + c].copy(), dt, oracle.SUM)
-            else:
-                want[lo:lo + c] = b[so:so + c]
-            assert_same(from_dev(d_a, a), want, dt, "%s attempt %d count %d" % (shape, attempt, c))
+            assert_same(from_dev(d_a, a), want, dt, "%s count %d" % (shape, c))
+        else:
+            want[lo:lo + c] = b[so:so + c]
+            assert_same(from_dev(d_a, a), want, dt, "%s count %d, first destination" % (shape, c))
+            want = a.copy()
+            want[lo_c:lo_c + c] = b[so:so + c]
+            assert_same(from_dev(d_c, a), want, dt, "%s count %d, second destination" % (shape, c))
 
 
 def test_local_reduce_dst_equals_src(gpu_thread):

@@ -992,3 +992,41 @@ def test_nic_plugin_tables_have_the_references_layout_and_refuse_what_needs_a_ne
     assert ch.drainOnThread(ch_ctx, rec) == R.SUCCESS and ch.drainOnThread(ch_ctx, 12345) == R.E_PTR
     assert ch.destroy(ch_ctx) == R.SUCCESS
     assert ep.destroy(ep_ctx) == R.SUCCESS
+
+
+def test_direction_of_large_launches_follows_what_they_read(rec):
+    """A copy / two-input reduce launch that writes more than HcommGfxSetAlternateBytes and reads what one of the thread's
+    last two such launches wrote walks the other way than that launch did; one that reads nothing of theirs walks
+    forwards; smaller launches and folds are left alone.  (Recorder thread: the decision is host logic.)"""
+    n, count, dt = 8, 1 << 26, h.HcommDataType.BFP16          # 8 x 128 MiB: every ring step writes exactly 128 MiB
+    i, o = _fake(n, 1 << 40), _fake(n, 1 << 41)
+    plan = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, i, o, count, dt, 0)
+    h.HcommGfxLaunchLogClear(rec)
+    assert plan.run(rec) == 0
+    assert [l.backwards for l in h.launch_log(rec)] == [0] * 15                 # 128 MiB is not MORE than 128 MiB
+    before = h.HcommGfxSetAlternateBytes(1 << 20)
+    try:
+        assert before == 128 << 20
+        h.HcommGfxLaunchLogClear(rec)
+        assert plan.run(rec) == 0
+        # every step reads what the step before wrote - also the first gather copy, which reads the last fold's result
+        assert [l.backwards for l in h.launch_log(rec)] == [s % 2 for s in range(15)]
+        # a fetch of fresh data between two folds walks forwards, and the fold after it against the LATER writer
+        A, B, C_, D, U = (x << 40 for x in (3, 4, 5, 6, 7))
+        h.HcommGfxLaunchLogClear(rec)
+        nbytes = 4 << 20
+        assert h.HcommLocalCopyOnThread(rec, A, U, nbytes) == 0                               # reads nothing recent: forwards
+        assert h.HcommLocalReduceOnThread(rec, B, A, nbytes // 2, dt, 0) == 0                 # reads A: backwards
+        assert h.HcommLocalCopyOnThread(rec, C_, U + nbytes, nbytes) == 0                     # fresh: forwards
+        assert h.HcommLocalReduceOnThread(rec, B, C_, nbytes // 2, dt, 0) == 0                # reads C (forwards) and B (backwards): the later one decides
+        assert h.HcommLocalReduceOnThread(rec, D, A, nbytes // 2, dt, 0) == 0                 # A was written three launches ago: forgotten, forwards
+        assert h.HcommLocalCopyOnThread(rec, A, D, 4096) == 0                                 # small: left alone
+        assert [l.backwards for l in h.launch_log(rec)] == [0, 1, 0, 1, 0, 0]
+        assert h.HcommGfxSetAlternateBytes(0) == 1 << 20                                      # never
+        h.HcommGfxLaunchLogClear(rec)
+        assert plan.run(rec) == 0
+        assert [l.backwards for l in h.launch_log(rec)] == [0] * 15
+        assert h.HcommGfxSetAlternateBytes(1 << 20) == 0
+    finally:
+        h.HcommGfxSetAlternateBytes(before)
+    plan.destroy()
