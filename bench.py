@@ -155,6 +155,8 @@ def main():
                  "--gpus %d is not supported" % args.gpus)
 
     import torch
+    import __graft_entry__
+    __graft_entry__.ensure_built()  # loads what is built; a tree that holds no library yet builds it first
     import hcomm_amd as h
 
     if not torch.cuda.is_available():

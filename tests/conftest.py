@@ -13,11 +13,8 @@ def pytest_configure(config):
 
 
 def _ensure_built():
-    lib = os.path.join(ROOT, "hcomm_amd", "csrc", "libhcomm_gfx.so")
-    orc = os.path.join(ROOT, "oracle", "liboracle.so")
-    if not (os.path.exists(lib) and os.path.exists(orc)):
-        import __graft_entry__ as g
-        g.build()
+    import __graft_entry__ as g
+    g.ensure_built()
 
 
 _ensure_built()
