@@ -20,7 +20,7 @@ __all__ = [
     "HcommThreadAllocWithStream", "HcommThreadFreeWithStream", "HcommThreadNotifyRecordOnThread",
     "HcommThreadNotifyWaitOnThread", "HcommMemAlloc", "HcommMemFree", "HcommBatchModeStart", "HcommBatchModeEnd",
     "HcommGfxThreadSynchronize", "HcommGfxReduceKOnThread", "HcommGfxRecorderThreadAlloc", "launch_log",
-    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion", "HcommGfxSetDirectLaunches", "HcommGfxSetAlternateBytes",
+    "HcommGfxLaunchLogClear", "calc_slices", "HcommGfxDataTypeSize", "Plan", "schedule_emit", "HcommGfxVersion", "HcommGfxSetDirectLaunches", "HcommGfxSetAlternateBytes", "HcommGfxSetPieceBytes",
     "DTYPE_SIZE", "HcommWriteOnThread", "HcommReadOnThread", "HcommWriteReduceOnThread", "HcommReadReduceOnThread",
     "HcommBatchTransferOnThread", "BatchTransferDesc", "TransferType", "desc_copy", "desc_reduce",
     "CheckReport", "Expect", "oplist_check", "schedule_check", "scratch_bytes",
@@ -289,6 +289,15 @@ _set_alternate = _sig("HcommGfxSetAlternateBytes", C.c_uint64, C.c_uint64)
 def HcommGfxSetAlternateBytes(nbytes):
     """Launches that write more than nbytes may walk their table backwards (0 = never); returns the previous value."""
     return _set_alternate(nbytes)
+
+
+_set_piece = _sig("HcommGfxSetPieceBytes", C.c_uint64, C.c_uint64)
+
+
+def HcommGfxSetPieceBytes(nbytes):
+    """Step-wise plans created from now on cut steps that write more than 2 x nbytes into pieces of about nbytes
+    (0 = never); returns the previous value."""
+    return _set_piece(nbytes)
 
 
 def HcommGfxVersion():

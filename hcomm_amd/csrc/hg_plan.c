@@ -140,6 +140,135 @@ static void regroup_steps(HgOp* ops, const uint32_t* steps, uint64_t n, HgOp* tm
     }
 }
 
+/*
+ * Steps that write more than the memory-side cache keeps, cut into pieces that fit it.
+ *
+ * Element i of a collective only ever meets element i of other buffers, so a schedule restricted to a part of every
+ * operation's range is a schedule of its own.  When every two ranges the operations touch are either the same range
+ * or apart - ring, mesh and the other schedules whose operations are whole slices - each operation is cut into the
+ * same P pieces, and the list becomes: all steps on the first piece of every range, then all steps on the second, ...
+ * A step of a piece writes about 128 MiB, so the next step finds the operand it reads in the cache instead of
+ * fetching it from HBM again (7-rank ring reduce-scatter in steps of 400 MB: three pieces).  Same operations on the
+ * same bytes in the same order per byte, hence the same result; schedules that nest ranges (halving-doubling, NHR's
+ * merged runs, the op-base loop's re-cut buffers) stay as they are.  HCOMM_GFX_PIECE_BYTES sets the size aimed at
+ * (0 = never cut).
+ */
+typedef struct {
+    uintptr_t at;
+    uint64_t bytes;
+} HgRange;
+
+static int range_cmp(const void* a, const void* b)
+{
+    const HgRange* x = (const HgRange*)a;
+    const HgRange* y = (const HgRange*)b;
+    if (x->at != y->at) return x->at < y->at ? -1 : 1;
+    return x->bytes < y->bytes ? -1 : (x->bytes > y->bytes);
+}
+
+static uint64_t g_piece_bytes = 0; /* value + 1; 0 = not read yet */
+
+static uint64_t piece_bytes(void)
+{
+    uint64_t v = __atomic_load_n(&g_piece_bytes, __ATOMIC_RELAXED);
+    if (v == 0) {
+        const char* e = getenv("HCOMM_GFX_PIECE_BYTES");
+        v = ((e && *e) ? strtoull(e, NULL, 10) : (128ull << 20));
+        if (v > (1ull << 62)) v = 1ull << 62;
+        v += 1u;
+        __atomic_store_n(&g_piece_bytes, v, __ATOMIC_RELAXED);
+    }
+    return v - 1u;
+}
+
+uint64_t HcommGfxSetPieceBytes(uint64_t bytes)
+{
+    const uint64_t before = piece_bytes();
+    if (bytes > (1ull << 62)) bytes = 1ull << 62;
+    __atomic_store_n(&g_piece_bytes, bytes + 1u, __ATOMIC_RELAXED);
+    return before;
+}
+
+#define HG_PIECES_MAX 16u
+#define HG_PIECE_MIN_PART 8u /* no operation is cut into pieces shorter than an eighth of the size aimed at (16 MiB) */
+#define HG_SPLIT_HEAD_MAX 16u            /* resolve_ops cuts off fewer bytes than this before a 16-byte boundary */
+#define HG_PIECE_ALIGN 128u /* a piece starts as far from a 16-byte (and element) boundary as its operation does */
+
+/* ops[0 .. *m) with steps[]: replaced by the piece-major list when the schedule allows it and has a step large enough
+ * to gain; HCCL_SUCCESS either way, HCCL_E_MEMORY when the larger list cannot be allocated */
+static int cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io)
+{
+    HgOp* ops = *ops_io;
+    const uint32_t* steps = *steps_io;
+    const uint64_t m = *m_io, aim = piece_bytes();
+    if (aim == 0 || m == 0) return HCCL_SUCCESS;
+    uint64_t largest = 0, smallest = UINT64_MAX; /* bytes the largest step writes; the shortest operation of the steps worth cutting */
+    for (uint64_t i = 0; i < m;) {
+        uint64_t written = 0, shortest = UINT64_MAX, j = i;
+        for (; j < m && steps[j] == steps[i]; ++j) {
+            written += ops[j].bytes;
+            if (ops[j].bytes >= HG_SPLIT_HEAD_MAX && ops[j].bytes < shortest) shortest = ops[j].bytes; /* not the few bytes cut off before a boundary */
+        }
+        if (written > largest) largest = written;
+        if (written > 2u * aim && shortest < smallest) smallest = shortest;
+        i = j;
+    }
+    if (largest <= 2u * aim) return HCCL_SUCCESS; /* what such a step leaves in the cache is found by the next as it is */
+    uint64_t pieces = (largest + aim - 1u) / aim;
+    if (pieces > HG_PIECES_MAX) pieces = HG_PIECES_MAX;
+    /* a launch of many short segments streams worse than it gains from the cache (64 pieces of 2 MiB: 0.75 of the
+     * roofline against 0.91 for the whole slices walked against their producer) */
+    const uint64_t shortest_piece = aim / HG_PIECE_MIN_PART ? aim / HG_PIECE_MIN_PART : 1u;
+    if (pieces > smallest / shortest_piece) pieces = smallest / shortest_piece;
+    if (pieces < 2u) return HCCL_SUCCESS;
+    /* every two ranges the same or apart */
+    HgRange* r = (HgRange*)malloc(2u * m * sizeof(HgRange));
+    if (!r) return HCCL_E_MEMORY;
+    for (uint64_t i = 0; i < m; ++i) {
+        r[2u * i] = (HgRange){(uintptr_t)ops[i].dst, ops[i].bytes};
+        r[2u * i + 1u] = (HgRange){(uintptr_t)ops[i].src, ops[i].bytes};
+    }
+    qsort(r, 2u * m, sizeof(HgRange), range_cmp);
+    /* sorted by (start, length): a range that is not a repeat of the one before must start at or behind the furthest
+     * end seen so far */
+    int apart = 1;
+    uintptr_t end = 0;
+    for (uint64_t i = 0; i < 2u * m && apart; ++i) {
+        if (i && r[i].at == r[i - 1u].at && r[i].bytes == r[i - 1u].bytes) continue;
+        if (r[i].at < end) apart = 0;
+        if (r[i].at + r[i].bytes > end) end = r[i].at + r[i].bytes;
+    }
+    free(r);
+    if (!apart) return HCCL_SUCCESS;
+    HgOp* cut = (HgOp*)calloc(m * pieces, sizeof(HgOp));
+    uint32_t* cut_steps = (uint32_t*)calloc(m * pieces, sizeof(uint32_t));
+    if (!cut || !cut_steps) {
+        free(cut);
+        free(cut_steps);
+        return HCCL_E_MEMORY;
+    }
+    const uint32_t nsteps = steps[m - 1u] + 1u; /* steps are numbered in order */
+    uint64_t k = 0;
+    for (uint64_t q = 0; q < pieces; ++q)
+        for (uint64_t i = 0; i < m; ++i) {
+            uint64_t each = (ops[i].bytes + pieces - 1u) / pieces;
+            each = (each + HG_PIECE_ALIGN - 1u) / HG_PIECE_ALIGN * HG_PIECE_ALIGN;
+            const uint64_t from = q * each;
+            if (from >= ops[i].bytes) continue;
+            cut[k] = ops[i];
+            cut[k].dst = (char*)ops[i].dst + from;
+            cut[k].src = (const char*)ops[i].src + from;
+            cut[k].bytes = ops[i].bytes - from < each ? ops[i].bytes - from : each;
+            cut_steps[k++] = (uint32_t)q * nsteps + steps[i];
+        }
+    free(*ops_io);
+    free(*steps_io);
+    *ops_io = cut;
+    *steps_io = cut_steps;
+    *m_io = k;
+    return HCCL_SUCCESS;
+}
+
 static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, void* const* const* bufs, int dtype,
                      int op)
 {
@@ -152,8 +281,9 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
     if (rc == HCCL_SUCCESS) rc = resolve_ops(list, n, bufs, dtype, op, ops, steps, &m);
     if (rc == HCCL_SUCCESS) {
         regroup_steps(ops, steps, m, tmp, tmp_cap);
-        rc = hg_coalesce(ops, m, plan_push, p);
+        rc = cut_into_pieces(&ops, &steps, &m);
     }
+    if (rc == HCCL_SUCCESS) rc = hg_coalesce(ops, m, plan_push, p);
     free(ops);
     free(steps);
     free(tmp);

@@ -1,0 +1,45 @@
+"""Step-wise plans lowered piece by piece (steps that write more than the memory-side cache keeps are run as all steps
+on the first part of every slice, then all steps on the second, ...): with the size aimed at lowered from 128 MiB to a
+few KiB, schedules of every kind at test sizes take that lowering where their operations are whole slices, and all 2N
+buffers (and the communication buffers) still hold what the CPU oracle's replay leaves there, guard bytes included."""
+import pytest
+
+import hcomm_amd as h
+from test_gpu_collectives import ALGS, run_case, say
+from util import DT
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # alg, n, count, dtype, op
+    ("ring_ar", 8, 1000003, "bf16", "sum"),         # ragged last slice
+    ("ring_ar", 5, 400009, "fp32", "max"),
+    ("ring_ar", 3, 1 << 20, "int8", "sum"),
+    ("ring_rs_stage", 7, 1000003, "fp32", "prod"),  # benchmark config 5a, scaled down
+    ("ring_rs_stage", 7, 1000003, "int8", "sum"),
+    ("mesh_oneshot", 8, 300007, "fp16", "sum"),
+    ("mesh_ascending", 5, 300007, "bf16", "min"),
+    ("mesh_rs", 7, 100003, "int32", "sum"),
+    ("ring_rs", 8, 100003, "fp32", "sum"),
+    ("chunk_mesh", 7, 300007, "fp32", "sum"),       # sub-chunks nest inside slices: stays as it is
+    ("rhd_ar", 8, 400009, "int32", "sum"),          # nested ranges: stays as it is
+    ("nhr_ar", 5, 400009, "bf16", "sum"),
+    ("local_reduce", 8, 400009, "fp32", "sum"),
+]
+
+
+@pytest.mark.parametrize("aim", [4096, 65536])
+@pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
+def test_plans_cut_into_pieces_leave_the_oracles_bytes(gpu_thread, alg, n, count, dtype, op, aim):
+    say("pieces", alg, n, count, dtype, op, aim)
+    whole = run_case(gpu_thread, alg, h.Lowering.STEPWISE, n, count, dtype, op, seed=21)
+    before = h.HcommGfxSetPieceBytes(aim)
+    try:
+        cut = run_case(gpu_thread, alg, h.Lowering.STEPWISE, n, count, dtype, op, seed=21)
+    finally:
+        assert h.HcommGfxSetPieceBytes(before) == aim
+    assert cut[1:] == whole[1:]                     # same algorithmic and moved bytes
+    if alg in ("ring_ar", "ring_rs_stage"):   # slices on 128-byte boundaries: every two ranges the same or apart
+        assert cut[0] > whole[0], "expected the piece-wise lowering for %s" % alg
+    if alg in ("rhd_ar", "nhr_ar"):
+        assert cut[0] == whole[0], "%s nests ranges and must keep one launch per step" % alg

@@ -717,7 +717,7 @@ def test_counts_whose_byte_offsets_would_leave_64_bits_are_refused():
     ("cfg2", h.Alg.ALLREDUCE_RING, 8, 67108864, DT.BFP16, 15, 4966055936, 23 * 134217728),
     ("cfg3", h.Alg.ALLREDUCE_RHD, 16, 33554432, DT.INT32, 10, 10334765056, 40 * 134217728),  # last gather: 2 x 512 MiB
     ("cfg4", h.Alg.ALLREDUCE_MESH_ONESHOT, 8, 2097152, DT.FP16, 8, 8 * 23 * 4194304, 72 * 4194304),
-    ("cfg5a", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.FP32, 6, 7200000216, 13 * 400000012),
+    ("cfg5a", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.FP32, 16, 7200000216, 13 * 400000012),  # 3 pieces x 6 steps
     ("cfg5b", h.Alg.REDUCE_SCATTER_RING, 7, 100000003, DT.INT8, 6, 1800000054, 13 * 100000003),
 ])
 def test_plan_structure_of_benchmark_configs(rec, name, alg, n, count, dt, launches, algo_bytes, moved_fused):
@@ -726,8 +726,14 @@ def test_plan_structure_of_benchmark_configs(rec, name, alg, n, count, dt, launc
     op = OP.PROD if name == "cfg5a" else OP.SUM
     p = h.Plan(alg, h.Lowering.STEPWISE, i, o, count, dt, op)
     assert (p.info.launches, p.info.algorithmicBytes, p.info.movedBytes) == (launches, algo_bytes, algo_bytes)
-    # one launch = one step of all ranks; a copy step that writes more than 512 MiB is cut in two
-    assert all(r.nseg == n or (r.kind == h.Kernel.COPY and r.bytes == 512 << 20) for r in p.launches())
+    # one launch = one step of all ranks; a copy step that writes more than 512 MiB is cut in two; steps that write
+    # more than twice what the memory-side cache serves well (cfg5a: 400 MB) run piece by piece, and the last step of
+    # a piece shares its launch with the first step of the next, which touches other memory
+    assert all(r.nseg == n or (r.kind == h.Kernel.COPY and r.bytes == 512 << 20) or (name == "cfg5a" and r.nseg == 2 * n)
+               for r in p.launches())
+    if name == "cfg5a":
+        assert [r.nseg for r in p.launches()] == [7] * 5 + [14] + [7] * 4 + [14] + [7] * 5
+        assert all(r.bytes <= 2 * (128 << 20) for r in p.launches())
     h.HcommGfxLaunchLogClear(rec)
     assert p.run(rec) == 0
     assert [(r.kind, r.nseg, r.bytes) for r in h.launch_log(rec)] == [(r.kind, r.nseg, r.bytes) for r in p.launches()]
@@ -1030,3 +1036,38 @@ def test_direction_of_large_launches_follows_what_they_read(rec):
     finally:
         h.HcommGfxSetAlternateBytes(before)
     plan.destroy()
+
+
+def test_steps_larger_than_the_cache_run_piece_by_piece(rec):
+    """A step-wise plan whose steps write more than 256 MiB, made of operations that are whole slices (any two ranges
+    the same or apart), is lowered piece by piece: all steps on the first part of every slice, then all steps on the
+    second, ... each launch writing about 128 MiB, no piece shorter than 16 MiB.  Schedules with nested ranges
+    (halving-doubling), short slices or smaller steps keep one launch per step; HCOMM_GFX_PIECE_BYTES=0 (a process of
+    its own: read once) keeps every plan that way."""
+    import subprocess
+    import sys
+    key = lambda p: [(l.kind, l.nseg, l.bytes) for l in p.launches()]
+    i, o = _fake(8, 1 << 40), _fake(8, 1 << 41)
+    big = [x * 64 for x in i], [x * 64 for x in o]                      # 4 GiB apart
+    p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, big[0], big[1], 1 << 28, h.HcommDataType.BFP16, 0)   # 8 x 512 MiB
+    assert p.info.launches == 4 * 15 and set(l.bytes for l in p.launches()) == {128 << 20}
+    assert [l.kind for l in p.launches()] == ([1] * 7 + [0] * 8) * 4
+    assert p.info.algorithmicBytes == (3 * 7 + 2 * 8) * (64 << 20) * 8
+    p.destroy()
+    p = h.Plan(h.Alg.ALLREDUCE_RING, h.Lowering.STEPWISE, big[0], big[1], 1 << 27, h.HcommDataType.BFP16, 0)   # steps of 256 MiB: as they are
+    assert p.info.launches == 15
+    p.destroy()
+    i16, o16 = [(1 << 40) + r * (1 << 32) for r in range(16)], [(1 << 44) + r * (1 << 32) for r in range(16)]
+    p = h.Plan(h.Alg.ALLREDUCE_RHD, h.Lowering.STEPWISE, i16, o16, 1 << 25, h.HcommDataType.INT32, 0)            # nested ranges
+    assert p.info.launches == 10
+    p.destroy()
+    scr = [(1 << 52) + r * (1 << 32) for r in range(8)]
+    p = h.Plan(h.Alg.REDUCE_SCATTER_LOCAL_REDUCE, h.Lowering.STEPWISE, big[0], big[1], 1 << 23, h.HcommDataType.BFP16, 0,
+               scratch_ptrs=scr)                                                                                   # 1 GiB steps of 16 MiB slices: too short to cut
+    assert p.info.launches == 5
+    p.destroy()
+    child = ("import sys; sys.path.insert(0, %r); import hcomm_amd as h\n"
+             "i=[(1<<46)+r*(1<<34) for r in range(8)]; o=[(1<<50)+r*(1<<34) for r in range(8)]\n"
+             "p=h.Plan(h.Alg.ALLREDUCE_RING,h.Lowering.STEPWISE,i,o,1<<28,h.HcommDataType.BFP16,0); print(p.info.launches)") % ROOT
+    run = subprocess.run([sys.executable, "-c", child], capture_output=True, text=True, env=dict(os.environ, HCOMM_GFX_PIECE_BYTES="0"))
+    assert run.stdout.split() == ["15"], (run.stdout, run.stderr[-500:])
