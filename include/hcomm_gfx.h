@@ -1010,7 +1010,7 @@ int32_t HcommGfxSetDirectLaunches(int32_t enable);
  * to run both directions on small shapes. */
 uint64_t HcommGfxSetAlternateBytes(uint64_t bytes);
 
-/* No reference counterpart.  A step-wise plan created after this call whose steps write more than 2 x `bytes`, and
+/* No reference counterpart.  A step-wise plan created after this call whose steps write more than 2.5 x `bytes`, and
  * whose operations are whole slices (any two ranges they touch the same or apart), runs piece by piece: all steps on
  * the first part of every slice, then all steps on the second, ... about `bytes` written per launch and no piece
  * shorter than an eighth of that, so that each step finds what the step before wrote in the memory-side cache.

@@ -727,7 +727,7 @@ def test_plan_structure_of_benchmark_configs(rec, name, alg, n, count, dt, launc
     p = h.Plan(alg, h.Lowering.STEPWISE, i, o, count, dt, op)
     assert (p.info.launches, p.info.algorithmicBytes, p.info.movedBytes) == (launches, algo_bytes, algo_bytes)
     # one launch = one step of all ranks; a copy step that writes more than 512 MiB is cut in two; steps that write
-    # more than twice what the memory-side cache serves well (cfg5a: 400 MB) run piece by piece, and the last step of
+    # more than 2.5 times what the memory-side cache serves well (cfg5a: 400 MB) run piece by piece, and the last step of
     # a piece shares its launch with the first step of the next, which touches other memory
     assert all(r.nseg == n or (r.kind == h.Kernel.COPY and r.bytes == 512 << 20) or (name == "cfg5a" and r.nseg == 2 * n)
                for r in p.launches())
@@ -1039,7 +1039,7 @@ def test_direction_of_large_launches_follows_what_they_read(rec):
 
 
 def test_steps_larger_than_the_cache_run_piece_by_piece(rec):
-    """A step-wise plan whose steps write more than 256 MiB, made of operations that are whole slices (any two ranges
+    """A step-wise plan whose steps write more than 320 MiB, made of operations that are whole slices (any two ranges
     the same or apart), is lowered piece by piece: all steps on the first part of every slice, then all steps on the
     second, ... each launch writing about 128 MiB, no piece shorter than 16 MiB.  Schedules with nested ranges
     (halving-doubling), short slices or smaller steps keep one launch per step; HCOMM_GFX_PIECE_BYTES=0 (a process of
