@@ -657,13 +657,15 @@ static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
     }
     const uint64_t cap = total ? total : 1;
     HgOp* sorted = (HgOp*)malloc(cap * sizeof(HgOp));
+    uint32_t* round_of = (uint32_t*)malloc(cap * sizeof(uint32_t)); /* the round each of them was taken in: a schedule's step */
+    uint32_t rounds = 0;
     HgSlot* outside = (HgSlot*)malloc(cap * sizeof(HgSlot)); /* records to threads outside the batch */
     HgSlot* earlier = (HgSlot*)malloc(cap * sizeof(HgSlot)); /* records issued before the batch that its waits consume */
     uint32_t** count = (uint32_t**)calloc(nt, sizeof(uint32_t*)); /* per thread and slot: unconsumed records of the batch */
     uint32_t had[HG_TOUCHED_MAX];                                 /* copies and reduces taken from each thread so far */
     HgThread* main_t = th[0];
     uint64_t n = 0, nearlier = 0, noutside = 0, done = 0;
-    if (!sorted || !outside || !earlier || !count) ret = HCCL_E_MEMORY;
+    if (!sorted || !round_of || !outside || !earlier || !count) ret = HCCL_E_MEMORY;
     for (uint32_t i = 0; i < nt && ret == HCCL_SUCCESS; ++i) {
         had[i] = 0;
         count[i] = (uint32_t*)calloc(th[i]->notify_num ? th[i]->notify_num : 1, sizeof(uint32_t));
@@ -717,11 +719,13 @@ static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
             HgThread* t = th[i];
             if (t->batch_cursor < t->pending_n && t->pending[t->batch_cursor].sync == 0 &&
                 hg_op_launch_key(&t->pending[t->batch_cursor]) == key) {
+                round_of[n] = rounds;
                 sorted[n++] = t->pending[t->batch_cursor++];
                 ++had[i];
                 ++done;
             }
         }
+        ++rounds;
     }
     if (ret != HCCL_SUCCESS) {
         /* nothing is submitted; the earlier records that waits of this batch took are handed back */
@@ -744,6 +748,9 @@ static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
             for (uint64_t k = 0; k < nearlier && ret == HCCL_SUCCESS; ++k)
                 if (!earlier[k].t->recorder) ret = hg_rt_stream_wait_event(main_t->stream, earlier[k].t->notifies[earlier[k].idx]);
         }
+        /* rounds are steps: a collective handed over whole gets the lowering a step-wise plan of it gets, steps larger
+         * than the memory-side cache serves run piece by piece */
+        if (ret == HCCL_SUCCESS) ret = hg_cut_into_pieces(&sorted, &round_of, &n);
         if (ret == HCCL_SUCCESS) ret = hg_coalesce(sorted, n, emit_to_thread, main_t);
         /* what the batch leaves behind: records nobody in it waited for, and the other threads behind its end */
         for (uint32_t i = 0; i < nt && ret == HCCL_SUCCESS; ++i)
@@ -777,6 +784,7 @@ static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
     free(outside);
     free(earlier);
     free(sorted);
+    free(round_of);
     return ret;
 }
 

@@ -196,7 +196,7 @@ uint64_t HcommGfxSetPieceBytes(uint64_t bytes)
 
 /* ops[0 .. *m) with steps[]: replaced by the piece-major list when the schedule allows it and has a step large enough
  * to gain; HCCL_SUCCESS either way, HCCL_E_MEMORY when the larger list cannot be allocated */
-static int cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io)
+int hg_cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io)
 {
     HgOp* ops = *ops_io;
     const uint32_t* steps = *steps_io;
@@ -284,7 +284,7 @@ static int lower_ops(HcommGfxPlan* p, const HcommGfxSchedOp* list, uint64_t n, v
     if (rc == HCCL_SUCCESS) rc = resolve_ops(list, n, bufs, dtype, op, ops, steps, &m);
     if (rc == HCCL_SUCCESS) {
         regroup_steps(ops, steps, m, tmp, tmp_cap);
-        rc = cut_into_pieces(&ops, &steps, &m);
+        rc = hg_cut_into_pieces(&ops, &steps, &m);
     }
     if (rc == HCCL_SUCCESS) rc = hg_coalesce(ops, m, plan_push, p);
     free(ops);

@@ -291,7 +291,8 @@ HcommResult HcommMemFree(void* ptr);
  * each thread's own order and every Record -> Wait pair (a Wait may have been called before its Record; a Record
  * issued BEFORE the batch satisfies a Wait inside it), and issues that one list through the coalescer on the stream
  * of the FIRST thread the batch touched: operations that different threads perform in the same step of a schedule
- * share a launch, exactly as if one thread had been given the step between a Start / End pair of its own.  The other
+ * share a launch, exactly as if one thread had been given the step between a Start / End pair of its own, and steps
+ * that write more than the memory-side cache serves run piece by piece as in a step-wise plan (HcommGfxSetPieceBytes).  The other
  * threads' streams are placed behind the end of the batch when they are next given a call or synchronised (a stream
  * of the caller's, HcommThreadAllocWithStream: at once), and the batch behind whatever they were given before it.
  * A Wait that neither the batch nor an earlier Record satisfies can never be satisfied - the host thread that would

@@ -43,3 +43,30 @@ def test_plans_cut_into_pieces_leave_the_oracles_bytes(gpu_thread, alg, n, count
         assert cut[0] > whole[0], "expected the piece-wise lowering for %s" % alg
     if alg in ("rhd_ar", "nhr_ar"):
         assert cut[0] == whole[0], "%s nests ranges and must keep one launch per step" % alg
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", [("ring_ar", 8, 1000003, "bf16", "sum"), ("ring_rs_stage", 7, 1000003, "int8", "sum"),
+                                                  ("rhd_ar", 6, 100003, "fp32", "sum")])
+def test_a_whole_collective_in_one_batch_is_cut_into_pieces_too(alg, n, count, dtype, op):
+    """The same lowering behind the reference's boundary: a thread per rank, posts and waits, everything inside one
+    HcommBatchModeStart / End pair - End's rounds are the steps it cuts."""
+    from test_gpu_via_primitives import drive
+    say("pieces, one batch over a thread per rank", alg, n, count, dtype, op)
+    code, threads = h.HcommThreadAlloc(h.CommEngine.CPU_TS, n, 16)
+    assert code == 0
+    before = h.HcommGfxSetPieceBytes(8192)
+    try:
+        for t in threads:
+            h.HcommGfxLaunchLogClear(t)
+        drive("threads_batched", None, threads, alg, n, count, dtype, op)
+        cut = len(h.launch_log(threads[0]))
+        h.HcommGfxSetPieceBytes(0)
+        h.HcommGfxLaunchLogClear(threads[0])
+        drive("threads_batched", None, threads, alg, n, count, dtype, op)
+        whole = len(h.launch_log(threads[0]))
+        assert (cut > whole) == (alg != "rhd_ar")
+    finally:
+        h.HcommGfxSetPieceBytes(before)
+        for t in threads:
+            h.HcommGfxThreadSynchronize(t)
+        h.HcommThreadFree(threads)

@@ -1071,3 +1071,25 @@ def test_steps_larger_than_the_cache_run_piece_by_piece(rec):
              "p=h.Plan(h.Alg.ALLREDUCE_RING,h.Lowering.STEPWISE,i,o,1<<28,h.HcommDataType.BFP16,0); print(p.info.launches)") % ROOT
     run = subprocess.run([sys.executable, "-c", child], capture_output=True, text=True, env=dict(os.environ, HCOMM_GFX_PIECE_BYTES="0"))
     assert run.stdout.split() == ["15"], (run.stdout, run.stderr[-500:])
+
+
+def test_a_whole_collective_in_one_batch_is_cut_into_the_plans_pieces():
+    """Benchmark configuration 5a (7 ranks x 100,000,003 fp32, steps of 400 MB) given as a thread per rank with posts
+    and waits inside one batch: HcommBatchModeEnd's rounds are the schedule's steps, so it cuts them into the same
+    three pieces as the step-wise plan and issues the plan's sixteen launches."""
+    from hcomm_amd import caller
+    n, count, dt = 7, 100000003, h.HcommDataType.FP32
+    recs = [h.HcommGfxRecorderThreadAlloc()[1] for _ in range(n)]
+    try:
+        i = [(1 << 40) + r * (1 << 32) for r in range(n)]
+        o = [(1 << 44) + r * (1 << 32) for r in range(n)]
+        rp = caller.Replay(h.schedule_emit(h.Alg.REDUCE_SCATTER_RING, n, count, dt), {0: i, 1: o}, dt, 0)
+        code, st = rp.run_on_threads_batched(recs)
+        assert code == 0
+        plan = h.Plan(h.Alg.REDUCE_SCATTER_RING, h.Lowering.STEPWISE, i, o, count, dt, 0)
+        key = lambda l: (l.kind, l.nseg, l.bytes, l.dtype, l.op)
+        assert [key(l) for l in h.launch_log(recs[0])] == [key(l) for l in plan.launches()]
+        assert plan.info.launches == 16
+        plan.destroy()
+    finally:
+        h.HcommThreadFree(recs)
