@@ -205,6 +205,7 @@ def main():
                                              "thread_per_rank_ms": v["thread_per_rank"]["ms_per_step"],
                                              "host_thread_per_rank_ms": v["host_thread_per_rank"]["ms_per_step"],
                                              "thread_per_rank_batched_ms": v["thread_per_rank_batched"]["ms_per_step"],
+                                             "one_batch_ms": v["one_batch"]["ms_per_step"],
                                              "verified": all(v[m].get("verified") for m in VIA_MODES)}
                 for low in ("fused", "fused_keep_inputs"):
                     if r.get(low):
@@ -703,7 +704,7 @@ def run_workload(args, torch, h, dev, stream, thread):
     return out
 
 
-VIA_MODES = ("batched", "thread_per_rank", "host_thread_per_rank", "thread_per_rank_batched")
+VIA_MODES = ("batched", "thread_per_rank", "host_thread_per_rank", "thread_per_rank_batched", "one_batch")
 
 
 def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in_ptrs, out_ptrs, scr_ptrs, restore, plan_res):
@@ -719,7 +720,8 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
                        are processes of their own);
       thread_per_rank_batched  the calls of thread_per_rank, posts and waits included, between ONE HcommBatchModeStart /
                        End pair - the whole collective as one batch over all its threads, what the reference submits as
-                       one task graph (launch_context.cc:16-44); HcommBatchModeEnd resolves the notifies on the host.
+                       one task graph (launch_context.cc:16-44); HcommBatchModeEnd resolves the notifies on the host;
+      one_batch        every call of the collective between ONE Start / End pair on the one thread.
     Timed like the plans: inputs restored before every step, a pair of HIP events around it."""
     from hcomm_amd import caller
     ops = h.schedule_emit(alg, n, count, dt)
@@ -751,6 +753,11 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
         h.check(code, "replay on one thread and one host thread per rank")
         last["host_thread_per_rank"] = st
 
+    def run_one_batch():
+        code, st = replay.run_one_batch(thread)
+        h.check(code, "replay as one batch on one thread")
+        last["one_batch"] = st
+
     def run_threads_batched():
         code, st = replay.run_on_threads_batched(threads)
         h.check(code, "replay on one thread per rank inside one batch")
@@ -760,7 +767,7 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
                    "by hcomm_amd/csrc/hg_caller.c, which binds the library with dlsym",
            "plan_ms_per_step": round(plan_res["ms_per_step"], 5)}
     for mode, run in (("batched", run_batched), ("thread_per_rank", run_threads), ("host_thread_per_rank", run_host_threads),
-                      ("thread_per_rank_batched", run_threads_batched)):
+                      ("thread_per_rank_batched", run_threads_batched), ("one_batch", run_one_batch)):
         for _ in range(args.warmup):
             restore()
             run()
@@ -793,7 +800,10 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
                "ms_per_step_median": round(per[len(per) // 2], 5),
                "vs_plan": round(ms / plan_res["ms_per_step"], 4), "launches": launches, "calls": st.calls,
                "host_us_per_step": round(host_us / args.steps, 2)}
-        if mode == "batched":
+        if mode == "one_batch":
+            row["batches"] = 1
+            row["host_us_in_end"] = round(end_us / args.steps, 2)
+        elif mode == "batched":
             row["batches"] = st.batches
             row["host_us_per_batch"] = round(host_us / args.steps / max(st.batches, 1), 2)
             row["host_us_in_end_per_batch"] = round(end_us / args.steps / max(st.batches, 1), 2)
@@ -819,7 +829,7 @@ def via_primitives_leg(args, torch, h, stream, thread, alg, n, count, dt, op, in
             h.HcommThreadFree(others)
 
     return out, {"batched": run_batched, "thread_per_rank": run_threads, "host_thread_per_rank": run_host_threads,
-                 "thread_per_rank_batched": run_threads_batched}, done
+                 "thread_per_rank_batched": run_threads_batched, "one_batch": run_one_batch}, done
 
 
 def shape_sweep(args, torch, h, dev, stream, thread):

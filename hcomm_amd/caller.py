@@ -25,6 +25,8 @@ _lib.hg_caller_bind.argtypes = [C.c_char_p]
 _lib.hg_caller_replay_batched.restype = C.c_int32
 _lib.hg_caller_replay_batched.argtypes = [C.c_uint64, C.POINTER(api.SchedOp), C.c_uint64, C.POINTER(_vpp), C.c_int,
                                           C.c_int, C.POINTER(CallerStats)]
+_lib.hg_caller_replay_one_batch.restype = C.c_int32
+_lib.hg_caller_replay_one_batch.argtypes = _lib.hg_caller_replay_batched.argtypes
 _lib.hg_caller_replay_threads.restype = C.c_int32
 _lib.hg_caller_replay_threads.argtypes = [C.POINTER(C.c_uint64), C.c_uint32, C.POINTER(api.SchedOp), C.c_uint64,
                                           C.POINTER(_vpp), C.c_int, C.c_int, C.c_uint32, C.POINTER(CallerStats)]
@@ -67,6 +69,12 @@ class Replay:
         """One HcommBatchModeStart / End pair per step on one thread.  Returns (code, CallerStats)."""
         st = CallerStats()
         code = _lib.hg_caller_replay_batched(thread, self._ops, self.n, self._bufs, self.dtype, self.op, C.byref(st))
+        return code, st
+
+    def run_one_batch(self, thread):
+        """The whole list between ONE HcommBatchModeStart / End pair on one thread.  Returns (code, CallerStats)."""
+        st = CallerStats()
+        code = _lib.hg_caller_replay_one_batch(thread, self._ops, self.n, self._bufs, self.dtype, self.op, C.byref(st))
         return code, st
 
     def run_on_threads(self, threads, timeout=10):

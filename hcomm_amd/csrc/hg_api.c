@@ -788,6 +788,53 @@ static int32_t batch_end_ordered(HgThread** th, uint32_t nt)
     return ret;
 }
 
+/*
+ * A thread's queue of a batch without notifies.  Normally it goes to the coalescer as it is.  When it holds more than
+ * one step's worth of large operations - a whole collective recorded in one batch - its steps are told apart the way
+ * the coalescer would (a call of another kind, or one that touches what the step so far touches, begins a step) and
+ * go through the lowering of a step-wise plan: steps larger than the memory-side cache serves run piece by piece.
+ */
+static int touches(const HgOp* a, const HgOp* b)
+{
+    const uintptr_t ad = (uintptr_t)a->dst, as = (uintptr_t)a->src, bd = (uintptr_t)b->dst, bs = (uintptr_t)b->src;
+    return (ad < bd + b->bytes && bd < ad + a->bytes) || (ad < bs + b->bytes && bs < ad + a->bytes) ||
+           (as < bd + b->bytes && bd < as + a->bytes);
+}
+
+static int32_t end_plain(HgThread* t)
+{
+    const uint64_t aim = hg_piece_bytes();
+    uint64_t bytes = 0;
+    for (uint32_t k = 0; k < t->pending_n; ++k) bytes += t->pending[k].bytes;
+    if (aim == 0 || t->pending_n < 2u || bytes <= aim * 5u) /* fewer than two steps worth cutting */
+        return hg_coalesce(t->pending, t->pending_n, emit_to_thread, t);
+    uint64_t n = t->pending_n;
+    HgOp* ops = (HgOp*)malloc(n * sizeof(HgOp));
+    uint32_t* steps = (uint32_t*)malloc(n * sizeof(uint32_t));
+    if (!ops || !steps) {
+        free(ops);
+        free(steps);
+        return HCCL_E_MEMORY;
+    }
+    memcpy(ops, t->pending, n * sizeof(HgOp));
+    uint32_t step = 0;
+    uint64_t begin = 0;
+    for (uint64_t k = 0; k < n; ++k) {
+        int fresh = k != 0 && hg_op_launch_key(&ops[k]) != hg_op_launch_key(&ops[begin]);
+        for (uint64_t q = begin; q < k && !fresh; ++q) fresh = touches(&ops[k], &ops[q]);
+        if (fresh) {
+            ++step;
+            begin = k;
+        }
+        steps[k] = step;
+    }
+    int32_t ret = hg_cut_into_pieces(&ops, &steps, &n);
+    if (ret == HCCL_SUCCESS) ret = hg_coalesce(ops, n, emit_to_thread, t);
+    free(ops);
+    free(steps);
+    return ret;
+}
+
 int32_t HcommBatchModeEnd(const char* batchTag)
 {
     (void)batchTag;
@@ -808,7 +855,7 @@ int32_t HcommBatchModeEnd(const char* batchTag)
         ret = batch_end_ordered(th, nt);
     } else {
         for (uint32_t i = 0; i < nt; ++i)
-            if (ret == HCCL_SUCCESS) ret = hg_coalesce(th[i]->pending, th[i]->pending_n, emit_to_thread, th[i]);
+            if (ret == HCCL_SUCCESS) ret = end_plain(th[i]);
     }
     for (uint32_t i = 0; i < nt; ++i) {
         th[i]->pending_n = 0;

@@ -135,6 +135,28 @@ int32_t hg_caller_replay_batched(ThreadHandle thread, const HcommGfxSchedOp* ops
     return rc;
 }
 
+/* The whole list between ONE HcommBatchModeStart / End pair on one thread: the collective handed over in one piece. */
+int32_t hg_caller_replay_one_batch(ThreadHandle thread, const HcommGfxSchedOp* ops, uint64_t n, void* const* const* bufs,
+                                   int dtype, int op, HgCallerStats* st)
+{
+    if (!g.lib || !ops || !bufs || !st) return HCCL_E_PTR;
+    memset(st, 0, sizeof(*st));
+    const uint32_t unit = unit_of(dtype);
+    const double t0 = now_us();
+    int32_t rc = g.start("collective");
+    if (rc != HCCL_SUCCESS) return rc;
+    for (uint64_t i = 0; i < n && rc == HCCL_SUCCESS; ++i) {
+        rc = issue(thread, &ops[i], bufs, dtype, op, unit);
+        ++st->calls;
+    }
+    const double e0 = now_us();
+    const int32_t rc_end = g.end("collective");
+    st->host_us_end = st->host_us_end_max = now_us() - e0;
+    st->batches = 1;
+    st->host_us = now_us() - t0;
+    return rc != HCCL_SUCCESS ? rc : rc_end;
+}
+
 static int32_t post_and_wait(const ThreadHandle* threads, uint32_t from, uint32_t to, uint32_t timeout, HgCallerStats* st)
 {
     /* thread `to` keeps one notify slot per peer: slot `from` */

@@ -97,6 +97,7 @@ uint64_t hg_alternate_bytes(void);
 /* ops[0 .. *m) with the step of each (malloc'ed, steps numbered in order): replaced by the piece-major list when the
  * schedule has a step larger than the memory-side cache serves and is made of whole slices (hg_plan.c) */
 int hg_cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io);
+uint64_t hg_piece_bytes(void); /* the size such pieces aim at; 0 = nothing is cut */
 uint32_t hg_op_launch_key(const HgOp* o);   /* operations with different keys never share a launch */
 
 /* Fill tile_begin / blocks / bytes and the launch shape (streaming, lds_bytes, xcd_run) of a launch whose segment

@@ -168,7 +168,7 @@ static int range_cmp(const void* a, const void* b)
 
 static uint64_t g_piece_bytes = 0; /* value + 1; 0 = not read yet */
 
-static uint64_t piece_bytes(void)
+uint64_t hg_piece_bytes(void)
 {
     uint64_t v = __atomic_load_n(&g_piece_bytes, __ATOMIC_RELAXED);
     if (v == 0) {
@@ -183,7 +183,7 @@ static uint64_t piece_bytes(void)
 
 uint64_t HcommGfxSetPieceBytes(uint64_t bytes)
 {
-    const uint64_t before = piece_bytes();
+    const uint64_t before = hg_piece_bytes();
     if (bytes > (1ull << 62)) bytes = 1ull << 62;
     __atomic_store_n(&g_piece_bytes, bytes + 1u, __ATOMIC_RELAXED);
     return before;
@@ -200,7 +200,7 @@ int hg_cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io)
 {
     HgOp* ops = *ops_io;
     const uint32_t* steps = *steps_io;
-    const uint64_t m = *m_io, aim = piece_bytes();
+    const uint64_t m = *m_io, aim = hg_piece_bytes();
     if (aim == 0 || m == 0) return HCCL_SUCCESS;
     uint64_t largest = 0, smallest = UINT64_MAX; /* bytes the largest step writes; the shortest operation of the steps worth cutting */
     for (uint64_t i = 0; i < m;) {
@@ -217,6 +217,7 @@ int hg_cut_into_pieces(HgOp** ops_io, uint32_t** steps_io, uint64_t* m_io)
      * of it in the cache as it is: ring allreduce in steps of 257 MiB 0.905 of the roofline whole, 0.89 in pieces;
      * in steps of 381 MiB 0.845 whole, 0.90 in pieces. */
     if (largest <= aim * 5u / 2u) return HCCL_SUCCESS;
+    if (steps[m - 1u] == steps[0]) return HCCL_SUCCESS; /* one step: nobody follows to find its pieces cached */
     uint64_t pieces = (largest + aim - 1u - aim / 16u) / aim; /* a sixteenth over the size aimed at is not worth a piece more */
     if (pieces > HG_PIECES_MAX) pieces = HG_PIECES_MAX;
     /* a launch of many short segments streams worse than it gains from the cache (64 pieces of 2 MiB: 0.75 of the

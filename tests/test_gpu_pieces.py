@@ -60,11 +60,15 @@ def test_a_whole_collective_in_one_batch_is_cut_into_pieces_too(alg, n, count, d
             h.HcommGfxLaunchLogClear(t)
         drive("threads_batched", None, threads, alg, n, count, dtype, op)
         cut = len(h.launch_log(threads[0]))
+        h.HcommGfxLaunchLogClear(threads[0])
+        drive("one_batch", threads[0], None, alg, n, count, dtype, op)     # the same on one thread, without notifies
+        cut_plain = len(h.launch_log(threads[0]))
         h.HcommGfxSetPieceBytes(0)
         h.HcommGfxLaunchLogClear(threads[0])
         drive("threads_batched", None, threads, alg, n, count, dtype, op)
         whole = len(h.launch_log(threads[0]))
         assert (cut > whole) == (alg != "rhd_ar")
+        assert (cut_plain > whole) == (alg != "rhd_ar")
     finally:
         h.HcommGfxSetPieceBytes(before)
         for t in threads:

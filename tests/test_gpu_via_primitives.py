@@ -68,17 +68,20 @@ def drive(mode, thread, threads, alg, n, count, dtype, op, special=False):
     ops = h.schedule_emit(ALGS[alg][0], n, count, dt)
     replay = caller.Replay(ops, bufs, dt, o)
     prod = op == "prod"   # the primitive refuses PROD like the reference's (cpu_primitives_c_adpt.cc:37) unless told otherwise
-    if mode == "batched":
+    if mode in ("batched", "one_batch"):
         h.HcommGfxThreadSynchronize(thread)
         h.HcommGfxLaunchLogClear(thread)
-        code, st = replay.run_batched(thread)
+        code, st = replay.run_batched(thread) if mode == "batched" else replay.run_one_batch(thread)
         if prod and n > 1 and count:
             assert code == h.HcclResult.E_PARA
             return None
         assert code == 0
         assert h.HcommGfxThreadSynchronize(thread) == 0
         # a step whose operations are of one kind and on 16-byte boundaries is one launch
-        assert st.batches == replay.steps and len(h.launch_log(thread)) >= (replay.steps if count else 0)
+        if mode == "batched":
+            assert st.batches == replay.steps and len(h.launch_log(thread)) >= (replay.steps if count else 0)
+        else:
+            assert st.batches == 1
     else:
         run = {"threads": replay.run_on_threads, "host_threads": replay.run_on_host_threads,
                "threads_batched": replay.run_on_threads_batched}[mode]
@@ -116,6 +119,14 @@ def rank_threads():
 def test_schedule_batched_per_step_matches_oracle(gpu_thread, alg, n, count, dtype, op):
     say("via primitives, batched", alg, n, count, dtype, op)
     drive("batched", gpu_thread, None, alg, n, count, dtype, op)
+
+
+@pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
+def test_schedule_as_one_batch_on_one_thread_matches_oracle(gpu_thread, alg, n, count, dtype, op):
+    """Every call of the collective between ONE Start / End pair on one thread: the coalescer keeps apart what touches
+    the same memory, so the launches come out step by step."""
+    say("via primitives, one batch on one thread", alg, n, count, dtype, op)
+    drive("one_batch", gpu_thread, None, alg, n, count, dtype, op)
 
 
 @pytest.mark.parametrize("alg,n,count,dtype,op", CASES)
@@ -164,6 +175,7 @@ def test_special_values_via_primitives(gpu_thread, rank_threads, alg, n, count, 
     """Signed zeros, NaNs with per-rank payloads, infinities and denormals through both ways of driving the boundary."""
     say("via primitives, special values", alg, n, count, dtype, op)
     drive("batched", gpu_thread, None, alg, n, count, dtype, op, special=True)
+    drive("one_batch", gpu_thread, None, alg, n, count, dtype, op, special=True)
     drive("threads", None, rank_threads, alg, n, count, dtype, op, special=True)
     drive("host_threads", None, rank_threads, alg, n, count, dtype, op, special=True)
     drive("threads_batched", None, rank_threads, alg, n, count, dtype, op, special=True)

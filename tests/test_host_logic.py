@@ -1090,6 +1090,16 @@ def test_a_whole_collective_in_one_batch_is_cut_into_the_plans_pieces():
         key = lambda l: (l.kind, l.nseg, l.bytes, l.dtype, l.op)
         assert [key(l) for l in h.launch_log(recs[0])] == [key(l) for l in plan.launches()]
         assert plan.info.launches == 16
+        # the same without notifies: every call on ONE thread between one Start / End pair - the steps are told
+        # apart by what they touch
+        h.HcommGfxLaunchLogClear(recs[1])
+        code, st = rp.run_one_batch(recs[1])
+        assert code == 0 and st.batches == 1
+        assert [key(l) for l in h.launch_log(recs[1])] == [key(l) for l in plan.launches()]
+        # and a batch per step stays a launch per step: one step alone has nobody to find its pieces cached
+        h.HcommGfxLaunchLogClear(recs[2])
+        code, st = rp.run_batched(recs[2])
+        assert code == 0 and len(h.launch_log(recs[2])) == 6
         plan.destroy()
     finally:
         h.HcommThreadFree(recs)
