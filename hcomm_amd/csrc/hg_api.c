@@ -820,8 +820,11 @@ static int32_t end_plain(HgThread* t)
     uint32_t step = 0;
     uint64_t begin = 0;
     for (uint64_t k = 0; k < n; ++k) {
+        /* The steps only say how much a step writes, i.e. whether cutting pays: the piece-major order is right
+         * whatever they are (two pieces meet only when they are the same piece of the same range, and those keep
+         * their order).  So a very long step is compared with its latest part only, which bounds the work. */
         int fresh = k != 0 && hg_op_launch_key(&ops[k]) != hg_op_launch_key(&ops[begin]);
-        for (uint64_t q = begin; q < k && !fresh; ++q) fresh = touches(&ops[k], &ops[q]);
+        for (uint64_t q = k - begin > 128u ? k - 128u : begin; q < k && !fresh; ++q) fresh = touches(&ops[k], &ops[q]);
         if (fresh) {
             ++step;
             begin = k;
